@@ -1,0 +1,320 @@
+/* myea_hip.h — C ABI of the MI355X (gfx950) training hot path.
+ *
+ * This is the boundary a host-side `Neural_Network` plugs into where the
+ * reference plugs in its CUDA object (`Set__CUDA` / `Initialize__CUDA` /
+ * `Copy__Host_To_Device`, Header_Files/Neural_Network/Data.hpp:3111-3196,
+ * Source_Files/Neural_Network/Neural_Network.cpp:2852-2912).  Every entry point
+ * names the reference member function it replaces.
+ *
+ * Conventions
+ *   - plain C, plain pointers and sizes; no C++/torch types cross this line;
+ *   - every function returns 0 on success or a negative MYEA_E_* code and never
+ *     aborts; myea_hip_last_error() returns the text of the last failure on
+ *     the calling thread (the reference prints and returns `false`);
+ *   - one net = one training stream; calls on one net must come from one host
+ *     thread at a time (the reference has the same rule: its step functions are
+ *     orphaned OpenMP constructs entered by a whole thread team);
+ *   - all arithmetic is IEEE fp32 (`T_ = float`, Common_Library/include/
+ *     Configuration/DTypes.hpp:20-32); indices are 64-bit; masks are bytes.
+ *   - tensors of a layer are row-major [T][batch_size][units] exactly as in the
+ *     reference (Neural_Network__Backward_Pass__OpenMP.cpp:1055-1072);
+ *   - the flat parameter vector keeps the reference order
+ *     [weights | biases | normalisation scales | normalisation shifts]
+ *     (Neural_Network__Compile.cpp:556-665, Neural_Network__Allocate.cpp:2378-2406).
+ */
+#ifndef MYEA_HIP_H
+#define MYEA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- enums: numeric values are the reference's (Common_Library/include/Enums) ---- */
+
+/* Enum_Type_Layer.hpp */
+enum {
+    MYEA_LAYER_NONE = 0,
+    MYEA_LAYER_FULLY_CONNECTED = 4,
+    MYEA_LAYER_LSTM = 8,
+    MYEA_LAYER_RESIDUAL = 10
+};
+
+/* Enum_Type_Networks.hpp */
+enum { MYEA_NETWORK_FEEDFORWARD = 3, MYEA_NETWORK_RECURRENT = 4 };
+
+/* Enum_Type_Activation_Functions.hpp */
+enum {
+    MYEA_AF_NONE = 0, MYEA_AF_COSINE = 1, MYEA_AF_COSINE_SYMMETRIC = 2, MYEA_AF_ELU = 3,
+    MYEA_AF_ELLIOT = 4, MYEA_AF_ELLIOT_SYMMETRIC = 5, MYEA_AF_GAUSSIAN = 6,
+    MYEA_AF_GAUSSIAN_STEPWISE = 7, MYEA_AF_GAUSSIAN_SYMMETRIC = 8, MYEA_AF_ISRU = 9,
+    MYEA_AF_ISRLU = 10, MYEA_AF_LINEAR = 11, MYEA_AF_LINEAR_PIECE = 12,
+    MYEA_AF_LINEAR_PIECE_SYMMETRIC = 13, MYEA_AF_LEAKY_RELU = 14, MYEA_AF_PARAMETRIC_RELU = 15,
+    MYEA_AF_RELU = 16, MYEA_AF_SELU = 17, MYEA_AF_SIGMOID = 18, MYEA_AF_SINE = 19,
+    MYEA_AF_SIGMOID_STEPWISE = 20, MYEA_AF_SINE_SYMMETRIC = 21, MYEA_AF_SOFTMAX = 22,
+    MYEA_AF_TANH = 23, MYEA_AF_TANH_STEPWISE = 24, MYEA_AF_THRESHOLD = 25,
+    MYEA_AF_THRESHOLD_SYMMETRIC = 26, MYEA_AF_LENGTH = 27
+};
+
+/* Enum_Type_Optimizer_Functions.hpp */
+enum {
+    MYEA_OPTIMIZER_NONE = 0, MYEA_OPTIMIZER_ADABOUND = 1, MYEA_OPTIMIZER_ADAM = 2,
+    MYEA_OPTIMIZER_AMSBOUND = 4, MYEA_OPTIMIZER_AMSGRAD = 5, MYEA_OPTIMIZER_GD = 6
+};
+
+/* Enum_Type_Layer_Dropout.hpp */
+enum {
+    MYEA_DROPOUT_NONE = 0, MYEA_DROPOUT_BERNOULLI = 2, MYEA_DROPOUT_BERNOULLI_INVERTED = 3
+};
+
+/* Enum_Type_Layer_Normalization.hpp */
+enum {
+    MYEA_NORMALIZATION_NONE = 0, MYEA_NORMALIZATION_BATCH_NORMALIZATION = 1,
+    MYEA_NORMALIZATION_BATCH_RENORMALIZATION = 2
+};
+
+/* Enum_Type_Loss_Functions.hpp (loss / accuracy) */
+enum {
+    MYEA_LOSS_NONE = 0, MYEA_LOSS_BIT = 1, MYEA_LOSS_CROSS_ENTROPY = 2, MYEA_LOSS_L1 = 3,
+    MYEA_LOSS_L2 = 4, MYEA_LOSS_MAE = 5, MYEA_LOSS_MAPE = 6, MYEA_LOSS_ME = 9, MYEA_LOSS_MSE = 10,
+    MYEA_LOSS_RMSE = 11, MYEA_LOSS_SMAPE = 12
+};
+enum {
+    MYEA_ACCURACY_NONE = 0, MYEA_ACCURACY_CROSS_ENTROPY = 1, MYEA_ACCURACY_DIRECTIONAL = 2,
+    MYEA_ACCURACY_DISTANCE = 3, MYEA_ACCURACY_SIGN = 5
+};
+
+/* Enum_Type_State_Propagation.hpp */
+enum { MYEA_STATE_INFERENCE = 0, MYEA_STATE_TRAINING = 1 };
+
+/* ---- error codes ---- */
+enum {
+    MYEA_OK = 0,
+    MYEA_E_INVALID = -1,      /* bad argument / descriptor */
+    MYEA_E_UNSUPPORTED = -2,  /* layer / activation / optimizer not on this path */
+    MYEA_E_BATCH = -3,        /* batch_size_received > batch_size (Forward_Pass__OpenMP.cpp:33-43) */
+    MYEA_E_STATE = -4,        /* e.g. backward in inference mode (Backward_Pass__OpenMP.cpp:41-51) */
+    MYEA_E_NOMEM = -5,
+    MYEA_E_DEVICE = -6        /* HIP runtime error; text in myea_hip_last_error() */
+};
+
+/* ---- network descriptor ---- */
+
+#define MYEA_MAX_LAYERS 64
+
+/* One entry of `Neural_Network::ptr_array_layers` (struct Layer, Data.hpp:600-760), reduced to the
+ * fields the hot path reads.  The index table is copied from the host `Layer` / `Block_unit` /
+ * `Cell_unit` fields, never recomputed by the device side; myea_net_desc_layout() fills it the
+ * way `Neural_Network::Compile` does for callers that have no host object. */
+typedef struct myea_layer_desc {
+    uint32_t type_layer;               /* MYEA_LAYER_* */
+    uint32_t n_units;                  /* FC: neurons.  LSTM: blocks per direction.  Input layer: inputs. */
+    uint32_t n_cells_per_block;        /* LSTM only, >= 1 (Layer_Parameters::unit_parameters[1]) */
+    uint32_t use_bidirectional;        /* LSTM only */
+    uint32_t type_activation_function; /* FC only; MYEA_AF_* (whole layer, Set__Layer_Activation_Function) */
+    float    activation_steepness;     /* FC only; Set__Layer_Activation_Steepness, default 1 */
+    uint32_t type_dropout;             /* MYEA_DROPOUT_* */
+    float    dropout_values[2];        /* [0] = retention probability */
+    uint32_t type_normalization;       /* MYEA_NORMALIZATION_* */
+    uint32_t use_layer_normalization_before_activation;
+    uint32_t block_depth;              /* residual only: layers inside the block */
+    uint32_t reserved0;
+    /* index table (into the flat parameter / gradient / optimizer vectors, and the mask buffer) */
+    uint64_t first_connection_index;       /* *Layer::ptr_first_connection_index */
+    uint64_t last_connection_index;        /* *Layer::ptr_last_connection_index */
+    uint64_t first_bias_connection_index;  /* Layer::first_bias_connection_index (LSTM: see Prepare__Bias__LSTM) */
+    uint64_t first_normalized_unit_index;  /* offset of the layer's first Normalized_unit in the scale array */
+    uint64_t first_mask_index;             /* offset of Layer::ptr_array__mask__dropout__bernoulli */
+} myea_layer_desc;
+
+typedef struct myea_net_desc {
+    uint32_t type_network;            /* MYEA_NETWORK_* */
+    uint32_t n_layers;                /* input layer + hidden layers + output layer */
+    uint32_t number_recurrent_depth;  /* T, >= 1 */
+    uint32_t batch_size;              /* allocated batch rows (Bmax) */
+    uint64_t total_weights;
+    uint64_t total_bias;
+    uint64_t total_normalized_units;  /* 0 when no layer is normalised (no scale/shift region) */
+    uint64_t total_parameters;        /* weights + bias + 2 * total_normalized_units */
+    uint64_t total_mask_units;        /* bytes in the Bernoulli mask buffer */
+    myea_layer_desc layers[MYEA_MAX_LAYERS];
+} myea_net_desc;
+
+/* Public training fields of `Neural_Network` (Data.hpp:2929-2970) the path reads; defaults are the
+ * reference's (myea_hyper_default()). */
+typedef struct myea_hyper {
+    uint32_t type_optimizer_function;   /* MYEA_OPTIMIZER_* */
+    uint32_t type_loss_function;        /* MYEA_LOSS_* */
+    uint32_t type_accuracy_function;    /* MYEA_ACCURACY_* */
+    uint32_t use_Nesterov;
+    uint32_t use_adam_bias_correction;
+    uint32_t use_clip_gradient;
+    float learning_rate;                /* 0.01 */
+    float learning_rate_final;          /* 0.1   (AdaBound) */
+    float learning_momentum;            /* 0.9 */
+    float learning_gamma;               /* 1e-3  (AdaBound) */
+    float adam_learning_rate;           /* 1e-3 */
+    float adam_beta1;                   /* 0.9 */
+    float adam_beta2;                   /* 0.999 */
+    float adam_epsilon;                 /* 1e-8 */
+    float regularization__weight_decay; /* 0; applied to weights only (mask 1 on weights, 0 elsewhere) */
+    float clip_gradient;                /* 1 */
+    float accuracy_variance;            /* 0.49 */
+    float bit_fail_limit;               /* 0.35 */
+    float normalization_momentum_average;              /* 0.999 */
+    float normalization_epsilon;                       /* 1e-5 */
+    float batch_renormalization_r_correction_maximum;  /* 1 */
+    float batch_renormalization_d_correction_maximum;  /* 0 */
+    float optimizer_time_step;          /* 0; incremented by every update */
+    uint32_t number_time_delays;        /* RNN: first k steps carry no loss */
+} myea_hyper;
+
+/* Loss / accuracy accumulators (ptr_array_loss_values, ptr_array_number_loss,
+ * ptr_array_accuracy_values[0], ptr_array_number_bit_fail; merged as Merge__Post__Training does,
+ * Neural_Network__Merge.cpp:52-98). */
+typedef struct myea_loss_state {
+    double   loss_values;       /* sum of per-output loss terms since the last reset */
+    uint64_t number_loss;       /* number of terms */
+    double   accuracy_value;    /* ptr_array_accuracy_values[0] */
+    uint64_t number_bit_fail;
+} myea_loss_state;
+
+/* kinds for the optimizer-state and tensor taps */
+enum {
+    MYEA_STATE_PREVIOUS_DELTA = 0,       /* ptr_array_previous_delta_parameters */
+    MYEA_STATE_FIRST_MOMENT = 1,         /* ptr_array_previous_biased_first_moment */
+    MYEA_STATE_SECOND_MOMENT = 2,        /* ptr_array_previous_biased_second_moment */
+    MYEA_STATE_SECOND_MOMENT_HAT = 3     /* ptr_array_previous_biased_second_moment_hat */
+};
+enum {
+    MYEA_TENSOR_OUTPUTS = 0,        /* Layer::ptr_array_outputs (post-dropout) [T][Bmax][H] */
+    MYEA_TENSOR_SUMMATIONS = 1,     /* neuron_units->ptr_array_summations */
+    MYEA_TENSOR_ERRORS = 2,         /* neuron_units->ptr_array_errors (delta w.r.t. the summation);
+                                       LSTM: delta of the cell outputs */
+    MYEA_TENSOR_NORM_HATS = 3,      /* normalized_batch_units.ptr_array_values_hats */
+    MYEA_TENSOR_NORM_MEANS = 4,     /* [T][H] batch means */
+    MYEA_TENSOR_NORM_VARIANCES = 5, /* [T][H] batch sqrt(var+eps) */
+    MYEA_TENSOR_NORM_MEANS_AVERAGES = 6,
+    MYEA_TENSOR_NORM_VARIANCES_AVERAGES = 7,
+    /* LSTM taps, [T][Bmax][cells] or [T][Bmax][blocks] */
+    MYEA_TENSOR_LSTM_CELL_INPUT = 16,      /* z  */
+    MYEA_TENSOR_LSTM_CELL_STATE = 17,      /* c  */
+    MYEA_TENSOR_LSTM_INPUT_GATE = 18,      /* i  */
+    MYEA_TENSOR_LSTM_FORGET_GATE = 19,     /* f  */
+    MYEA_TENSOR_LSTM_OUTPUT_GATE = 20,     /* o  */
+    MYEA_TENSOR_LSTM_DELTA_CELL_INPUT = 21,
+    MYEA_TENSOR_LSTM_DELTA_CELL_STATE = 22,
+    MYEA_TENSOR_LSTM_DELTA_INPUT_GATE = 23,
+    MYEA_TENSOR_LSTM_DELTA_FORGET_GATE = 24,
+    MYEA_TENSOR_LSTM_DELTA_OUTPUT_GATE = 25
+};
+
+/* ---- host-side descriptor helpers (no GPU needed) ---- */
+
+/* Defaults of the public training fields, Data.hpp:2929-2970. */
+void myea_hyper_default(myea_hyper *hyper);
+
+/* Fills the index table and the totals of `desc` from type_layer / n_units / n_cells_per_block /
+ * use_bidirectional / block_depth / type_normalization, in the order `Neural_Network::Compile`
+ * assigns them: Prepare__Connections__{FC,LSTM} per layer, then Prepare__Bias__{FC,LSTM} per layer
+ * (Neural_Network__Compile.cpp:556-665, Neural_Network__Prepare_Connections.cpp:20-252), then the
+ * normalised-unit scale/shift region (Neural_Network__Layer_Normalization.cpp:20-78,
+ * Neural_Network__Allocate.cpp:2378-2462) and the mask offsets (Neural_Network.cpp:3948-3962). */
+int myea_net_desc_layout(myea_net_desc *desc);
+
+/* ---- life cycle: replaces Set__CUDA / Initialize__CUDA / Deinitialize__CUDA (Data.hpp:3111-3118) ---- */
+typedef struct myea_hip_net myea_hip_net;
+
+int myea_hip_create(const myea_net_desc *desc, myea_hip_net **out_net);
+int myea_hip_destroy(myea_hip_net *net);
+/* Launch everything on `hip_stream` (a hipStream_t; NULL = the default stream). */
+int myea_hip_set_stream(myea_hip_net *net, void *hip_stream);
+int myea_hip_synchronize(myea_hip_net *net);
+const char *myea_hip_last_error(void);
+
+/* ---- public-field setters: replace the `Set__*` forwarding in Train.cpp:28-90 ---- */
+int myea_hip_set_hyper(myea_hip_net *net, const myea_hyper *hyper);
+int myea_hip_get_hyper(myea_hip_net *net, myea_hyper *hyper);  /* reads back optimizer_time_step */
+/* `type_state_propagation` (Data.hpp, Enum_Type_State_Propagation.hpp) */
+int myea_hip_set_state_propagation(myea_hip_net *net, uint32_t type_state_propagation);
+
+/* ---- parameter / state movement: replace Copy__Parameters__Host_To_Device,
+ *      Copy__Parameters__Device_To_Host, Copy__Optimizer_*__{Host_To_Device,Device_To_Host}
+ *      (Data.hpp:3119-3189) ---- */
+int myea_hip_upload_parameters(myea_hip_net *net, const float *host_parameters, size_t count);
+int myea_hip_download_parameters(myea_hip_net *net, float *host_parameters, size_t count);
+int myea_hip_upload_optimizer_state(myea_hip_net *net, int kind, const float *host, size_t count);
+int myea_hip_download_optimizer_state(myea_hip_net *net, int kind, float *host, size_t count);
+/* `ptr_array_units_mask_dropout_bernoulli` (bool[(sum AF units) * T]), written by the caller between
+ * steps exactly as the reference lets callers write its public mask buffer. */
+int myea_hip_upload_masks(myea_hip_net *net, const uint8_t *host_masks, size_t count);
+/* Clear_Training_Arrays (Train.cpp:93-126) + Clear_Optimizer (Train.cpp:128-263): zero the gradient
+ * vector and all optimizer state, optimizer_time_step = 0. */
+int myea_hip_clear_training_arrays(myea_hip_net *net);
+
+/* ---- the five step entry points ---- */
+
+/* Neural_Network::Forward_Pass (Data.hpp:2896; Neural_Network__Forward_Pass__Loop.cpp:22).
+ * `inputs` is [batch_size_received][T * n_inputs] row-major (the reference's array of per-example
+ * row pointers, flattened); `inputs_on_device` != 0 means it is already resident in HBM. */
+int myea_hip_forward_pass(myea_hip_net *net, size_t batch_size_received, const float *inputs, int inputs_on_device);
+
+/* Neural_Network::Compute__Error (Data.hpp:1033; Neural_Network__Compute__Error__Loop.cpp:79).
+ * `desired_outputs` is [batch_size_received][T * n_outputs] row-major. */
+int myea_hip_compute_error(myea_hip_net *net, size_t batch_size_received, const float *desired_outputs, int desired_on_device);
+
+/* Neural_Network::Backward_Pass (Data.hpp:1709; Neural_Network__Backward_Pass__Loop.cpp:22). */
+int myea_hip_backward_pass(myea_hip_net *net, size_t batch_size_received);
+
+/* Neural_Network::Update_Derivative_Weight (Data.hpp:2199) over layers
+ * [first_layer_index, end_layer_index); the reference's callers pass (layers + 1, last). */
+int myea_hip_update_derivative_weight(myea_hip_net *net, size_t batch_size_received, size_t first_layer_index, size_t end_layer_index);
+
+/* Neural_Network::Update_Parameter (Data.hpp:849; Neural_Network.cpp:4719-4908): clip-by-global-norm
+ * then the fused optimizer; zeroes the gradient. */
+int myea_hip_update_parameter(myea_hip_net *net, size_t batch_size_received, size_t training_size_received);
+
+/* Reset__Loss / the merged loss counters (Neural_Network__Merge.cpp:52-98).  get synchronises. */
+int myea_hip_reset_loss(myea_hip_net *net);
+int myea_hip_get_loss(myea_hip_net *net, myea_loss_state *out_state);
+
+/* ---- debug taps (the reference's data members are public; these read the device copies) ---- */
+int myea_hip_download_gradient(myea_hip_net *net, float *host_gradient, size_t count);
+int myea_hip_upload_gradient(myea_hip_net *net, const float *host_gradient, size_t count);
+int myea_hip_download_tensor(myea_hip_net *net, size_t layer_index, int kind, float *host, size_t count);
+
+/* ---- profiling taps for the benchmark ---- */
+/* When enabled, every dense-contraction (GEMM) launch is bracketed by HIP events on the net's stream;
+ * myea_hip_profile_read() synchronises and returns accumulated launches / milliseconds / FLOPs per
+ * family since the last reset.  family: 0 = forward (NT), 1 = dX (NN), 2 = dW (TN), 3 = optimizer
+ * update (bytes instead of FLOPs). */
+int myea_hip_profile_enable(myea_hip_net *net, int enable);
+int myea_hip_profile_read(myea_hip_net *net, int family, uint64_t *launches, double *milliseconds, double *work);
+
+/* ---- kernel-level entry points on raw device pointers (stream = hipStream_t or NULL) ----
+ * These are the kernels the net-level calls are built from, exported so that each one can be
+ * checked and timed alone. */
+
+/* C[M][N] (ldc) = (accumulate ? C : 0) + op(A) * op(B); fp32 MFMA.
+ *   a_k_contiguous != 0: A is [M][K] with lda;  else A is [K][M] with lda.
+ *   b_k_contiguous != 0: B is [N][K] with ldb;  else B is [K][N] with ldb.
+ * Forward_Pass__FC (a=1,b=1), Backward_Pass__FC (a=1,b=0), Update_Derivative_Weight__FC (a=0,b=0). */
+int myea_hip_gemm_f32(void *stream, int a_k_contiguous, int b_k_contiguous, int accumulate,
+                      size_t M, size_t N, size_t K,
+                      const float *A, size_t lda, const float *B, size_t ldb, float *C, size_t ldc);
+
+/* Fused weight update over [0, count): Update_Parameters__{Adam,AMSGrad,AdaBound} and
+ * Update_Parameter__Gradient_Descent{,_Momentum}, _Nesterov_Accelerated_Gradient.  `hyper` supplies
+ * every scalar; optimizer_time_step is the value *after* the increment.  `gradient_scale` multiplies
+ * the gradient on read (clip-by-norm fused; pass 1).  Unused state pointers may be NULL.
+ * weight decay applies to indices < weight_count. */
+int myea_hip_optimizer_update(void *stream, const myea_hyper *hyper, size_t count, size_t weight_count,
+                              float gradient_scale, float *parameters, float *gradient,
+                              float *state0, float *state1, float *state2);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MYEA_HIP_H */

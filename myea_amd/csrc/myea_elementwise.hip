@@ -1,0 +1,637 @@
+// myea_elementwise.hip — HBM-bound kernels of the training step for gfx950: activations and their
+// derivatives, softmax, dropout column scaling, batch-(re)normalisation forward/backward, bias-gradient
+// column sums, output-layer delta with loss/accuracy accumulation, global-norm clipping and the fused
+// optimizer update.  All of them are coalesced along the unit (fastest) dimension; reductions over the
+// batch are two-stage and deterministic (per-chunk partial sums in a fixed order, no float atomics).
+//
+// NN/ = Neural_Network_Library_Windows/Source_Files/Neural_Network/.
+#include "myea_device_af.h"
+#include "myea_kernels.h"
+
+namespace myea {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int kBlock = 256;
+
+inline unsigned grid_for(size_t n, int per_block, unsigned cap = 65535u * 16u)
+{
+    size_t g = (n + per_block - 1) / per_block;
+    if (g < 1) g = 1;
+    if (g > cap) g = cap;
+    return (unsigned)g;
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// ---- plain elementwise -------------------------------------------------------------------------
+
+__global__ __launch_bounds__(kBlock) void fill_kernel(float *p, size_t n, float v)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) p[i] = v;
+}
+
+// Forward_Pass__FC_AF (NN/Neural_Network__Forward_Pass__OpenMP.cpp:4839-4868) fused with the Bernoulli
+// appliers (:4907-4990) through a per-column multiplier.
+__global__ __launch_bounds__(kBlock) void activation_kernel(int act, size_t n, size_t H, const float *x, float *y, const float *colscale)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        float v = af_fire(act, x[i]);
+        if (colscale) v *= colscale[i % H];
+        y[i] = v;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void colscale_kernel(size_t n, size_t H, float *y, const float *colscale)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) y[i] *= colscale[i % H];
+}
+
+__global__ __launch_bounds__(kBlock) void mask_to_scale_kernel(size_t n, const uint8_t *mask, float on, float *colscale)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) colscale[i] = mask[i] ? on : 0.f;
+}
+
+// Backward_Pass__FC__DF (NN/Neural_Network__Backward_Pass__OpenMP.cpp:1225-1263)
+__global__ __launch_bounds__(kBlock) void activation_derive_kernel(int act, float steep, size_t n, const float *pre, const float *val, const float *dy, float *dx)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
+        dx[i] = dy[i] * af_derive(act, pre[i], steep, val[i]);
+}
+
+// Forward_Pass__FC_AF__Softmax (:4870-4905): one wavefront per row.
+__global__ __launch_bounds__(kBlock) void softmax_kernel(size_t rows, size_t H, const float *x, float *y, const float *colscale)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *xr = x + row * H;
+    float *yr = y + row * H;
+    float mx = -3.402823466e+38f;
+    for (size_t j = lane; j < H; j += 64) mx = fmaxf(mx, xr[j]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (size_t j = lane; j < H; j += 64) { float e = expf(xr[j] - mx); yr[j] = e; sum += e; }
+    sum = 1.f / wave_sum(sum);
+    for (size_t j = lane; j < H; j += 64) { float v = yr[j] * sum; if (colscale) v *= colscale[j]; yr[j] = v; }
+}
+
+// FF/RNN__Assign_Inputs (NN/Neural_Network__Assign_Inputs.cpp:20-204): example rows [T][W] -> [T][Bmax][W]
+__global__ __launch_bounds__(kBlock) void scatter_time_major_kernel(size_t B, size_t T, size_t W, size_t Bmax, const float *src, float *dst)
+{
+    const size_t n = B * T * W;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t w = i % W, bt = i / W, t = bt % T, b = bt / T;
+        dst[(t * Bmax + b) * W + w] = src[i];
+    }
+}
+
+// ---- two-stage column reductions -----------------------------------------------------------------
+// Stage 1: grid (ceil(H/64), S); a workgroup is 64 columns x 4 row lanes and owns rows
+// [y*chunk, (y+1)*chunk).  It writes NV partial sums per column to partial[(y*NV + v)*H + col].
+
+template <int NV, typename F>
+__global__ __launch_bounds__(kBlock) void column_partial_kernel(size_t rows, size_t H, size_t chunk, float *partial, F f)
+{
+    __shared__ float red[NV][4][64];
+    const int c = threadIdx.x & 63, rl = threadIdx.x >> 6;
+    const size_t col = (size_t)blockIdx.x * 64 + c;
+    float acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = 0.f;
+    if (col < H) {
+        const size_t r0 = (size_t)blockIdx.y * chunk, r1 = min(rows, r0 + chunk);
+        for (size_t r = r0 + rl; r < r1; r += 4) f(r, col, acc);
+    }
+#pragma unroll
+    for (int v = 0; v < NV; ++v) red[v][rl][c] = acc[v];
+    __syncthreads();
+    if (rl == 0 && col < H) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+            partial[((size_t)blockIdx.y * NV + v) * H + col] = red[v][0][c] + red[v][1][c] + red[v][2][c] + red[v][3][c];
+    }
+}
+
+inline void split_rows(size_t rows, size_t H, size_t &S, size_t &chunk)
+{
+    // aim at >= 1024 workgroups, at least 32 rows per chunk, at most 64 splits
+    const size_t colblocks = (H + 63) / 64;
+    S = (1024 + colblocks - 1) / colblocks;
+    const size_t max_s = (rows + 31) / 32;
+    if (S > max_s) S = max_s;
+    if (S > 64) S = 64;
+    if (S < 1) S = 1;
+    chunk = (rows + S - 1) / S;
+    S = (rows + chunk - 1) / chunk;
+    if (S < 1) S = 1;
+}
+
+struct SumF {
+    const float *x; size_t H;
+    __device__ void operator()(size_t r, size_t col, float *acc) const { acc[0] += x[r * H + col]; }
+};
+
+__global__ __launch_bounds__(kBlock) void column_sum_final_kernel(size_t H, size_t S, const float *partial, float *out, int accumulate)
+{
+    const size_t col = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (col >= H) return;
+    float s = 0.f;
+    for (size_t y = 0; y < S; ++y) s += partial[y * H + col];
+    out[col] = accumulate ? out[col] + s : s;
+}
+
+// ---- batch normalisation ----------------------------------------------------------------------------
+
+struct BnStatF {
+    const float *x; size_t H;
+    __device__ void operator()(size_t r, size_t col, float *acc) const { float s = x[r * H + col]; acc[0] += s; acc[1] += s * s; }
+};
+
+// Forward_Pass__Batch_Normalization__Training / __Batch_Renormalization__Training, "Average" loop
+// (NN/Neural_Network__Forward_Pass__OpenMP.cpp:4639-4675 and :4756-4813)
+__global__ __launch_bounds__(kBlock) void bn_forward_final_kernel(size_t H, size_t S, size_t rows, const float *partial, BnForwardParams p)
+{
+    const size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (j >= H) return;
+    float sm = 0.f, sv = 0.f;
+    for (size_t y = 0; y < S; ++y) { sm += partial[(y * 2 + 0) * H + j]; sv += partial[(y * 2 + 1) * H + j]; }
+    const float bscale = 1.f / (float)rows;
+    const float mean = sm * bscale;
+    float mavg = p.mean_avg[j];
+    mavg += p.momentum * (mean - mavg);
+    p.mean_avg[j] = mavg;
+    const float var = sqrtf(sv * bscale - mean * mean + p.epsilon);
+    float vavg = p.var_avg[j];
+    vavg += p.momentum * (var - vavg);
+    p.var_avg[j] = vavg;
+    p.mean[j] = mean;
+    p.var[j] = var;
+    if (p.renorm) {
+        const float g = var / vavg, lo = 1.f / p.r_max;
+        p.r_corr[j] = g < lo ? lo : (g > p.r_max ? p.r_max : g);
+        const float d = (mean - mavg) / vavg;
+        p.d_corr[j] = d < -p.d_max ? -p.d_max : (d > p.d_max ? p.d_max : d);
+    }
+}
+
+// "Activation function" loop of the same functions (:4677-4700, :4815-4836)
+__global__ __launch_bounds__(kBlock) void bn_forward_apply_kernel(size_t n, BnForwardParams p)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t j = i % p.H;
+        float s = (p.x[i] - p.mean[j]) / p.var[j];
+        if (p.renorm) s = s * p.r_corr[j] + p.d_corr[j];
+        p.hats[i] = s;
+        p.normalizes[i] = p.scale[j] * s + p.shift[j];
+    }
+}
+
+// Forward_Pass__Batch_Normalization__Inference (:4559-4589)
+__global__ __launch_bounds__(kBlock) void bn_forward_inference_kernel(size_t n, size_t H, const float *x, const float *scale, const float *shift,
+                                                                      const float *mavg, const float *vavg, float *out)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t j = i % H;
+        out[i] = scale[j] * ((x[i] - mavg[j]) / vavg[j]) + shift[j];
+    }
+}
+
+// Backward_Pass__Batch_Normalization / __Batch_Renormalization, first loop
+// (NN/Neural_Network__Backward_Pass__OpenMP.cpp:1385-1413, :1627-1655)
+struct BnBackF {
+    BnBackwardParams p;
+    __device__ void operator()(size_t r, size_t col, float *acc) const
+    {
+        const size_t k = r * p.H + col;
+        float e = p.dy[k];
+        const float vb = p.var[col], rc = p.renorm ? p.r_corr[col] : 1.f;
+        acc[0] += e * p.hats[k];
+        acc[1] += e;
+        e *= p.scale[col];
+        acc[2] += e * (-rc / vb);
+        acc[3] += e * (p.x[k] - p.mean[col]) * (-rc / (vb * vb));
+    }
+};
+
+// reduction of the partials: dscale/dshift accumulate into the gradient vector, dmean/dvar go to scratch
+__global__ __launch_bounds__(kBlock) void bn_backward_final_kernel(size_t H, size_t S, const float *partial, float *dscale, float *dshift, float *dmean_dvar)
+{
+    const size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (j >= H) return;
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    for (size_t y = 0; y < S; ++y) {
+        a0 += partial[(y * 4 + 0) * H + j];
+        a1 += partial[(y * 4 + 1) * H + j];
+        a2 += partial[(y * 4 + 2) * H + j];
+        a3 += partial[(y * 4 + 3) * H + j];
+    }
+    dscale[j] += a0;
+    dshift[j] += a1;
+    dmean_dvar[j] = a2;
+    dmean_dvar[H + j] = a3;
+}
+
+// last loop (:1437-1466, :1679-1708)
+__global__ __launch_bounds__(kBlock) void bn_backward_apply_kernel(size_t n, BnBackwardParams p, const float *dmean_dvar)
+{
+    const float bsz = (float)p.rows, bscale = 1.f / (float)p.rows;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t j = i % p.H;
+        const float vb = p.var[j], rc = p.renorm ? p.r_corr[j] : 1.f;
+        float e = p.dy[i] * p.scale[j];
+        e *= rc / vb;
+        e += dmean_dvar[p.H + j] * ((p.x[i] - p.mean[j]) / (bsz * vb));
+        e += dmean_dvar[j] * bscale;
+        p.dx[i] = e;
+    }
+}
+
+// ---- output-layer delta, loss and accuracy -------------------------------------------------------------
+// FF__Compute__Error (NN/Neural_Network__Compute__Error__OpenMP.cpp:22-141), RNN__Compute__Error
+// (NN/Neural_Network__Recurrent_Compute__Error__OpenMP.cpp:22-159), Update_Error
+// (NN/Neural_Network__Compute__Error__Loop.cpp:20-77).  One wavefront per (t, example) row.
+
+__device__ __forceinline__ float sign_f(float v) { return v > 0.f ? 1.f : (v < 0.f ? -1.f : 0.f); }
+
+__global__ __launch_bounds__(kBlock) void compute_error_kernel(ErrorParams p)
+{
+    const int lane = threadIdx.x & 63;
+    const size_t nrows = (p.T - p.first_t) * p.B;
+    const size_t rid = (size_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (rid >= nrows) return;
+    const size_t t = p.first_t + rid / p.B, b = rid % p.B;
+    const size_t off = (t * p.Bmax + b) * p.H;
+    const float *y = p.values + off, *pre = p.pre + off;
+    const float *d = p.desired + (b * p.T + t) * p.H;
+    float *err = p.errors + off;
+
+    float loss = 0.f, cnt = 0.f, acc = 0.f, bits = 0.f;
+    // cross-entropy accuracy: first index whose target is 1, last index reaching the maximum (">=")
+    if (p.accuracy == MYEA_ACCURACY_CROSS_ENTROPY) {
+        unsigned want = 0xffffffffu; float mx = -3.402823466e+38f; unsigned got = 0;
+        for (size_t j = lane; j < p.H; j += 64) {
+            if (d[j] == 1.f && (unsigned)j < want) want = (unsigned)j;
+            if (y[j] >= mx) { mx = y[j]; got = (unsigned)j; }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const unsigned w2 = __shfl_xor(want, o, 64);
+            const float m2 = __shfl_xor(mx, o, 64);
+            const unsigned g2 = __shfl_xor(got, o, 64);
+            want = min(want, w2);
+            if (m2 > mx || (m2 == mx && g2 > got)) { mx = m2; got = g2; }
+        }
+        if (want == 0xffffffffu) want = (unsigned)p.H;
+        if (lane == 0) acc += (want == got) ? 1.f : 0.f;
+    }
+    for (size_t j = lane; j < p.H; j += 64) {
+        const float yo = y[j], de = d[j], diff = yo - de;
+        float e = 0.f; bool counted = true;
+        switch (p.loss) {
+        case MYEA_LOSS_ME:
+        case MYEA_LOSS_L1: e = diff; break;
+        case MYEA_LOSS_MAE: e = fabsf(diff); break;
+        case MYEA_LOSS_L2:
+        case MYEA_LOSS_MSE:
+        case MYEA_LOSS_RMSE: e = diff * diff; break;
+        case MYEA_LOSS_MAPE: { float q = yo != 0.f ? yo : fmaxf(yo, 1e-6f); e = fabsf(diff / q); break; }
+        case MYEA_LOSS_SMAPE: e = fabsf(diff) / (fabsf(de) + fabsf(yo)); break;
+        case MYEA_LOSS_CROSS_ENTROPY: {
+            float q = yo != 0.f ? yo : fmaxf(yo, 1e-6f);
+            e = (p.H == 1) ? -(de * logf(q) + (1.f - de) * logf(1.f - q)) : -(de * logf(q));
+            break;
+        }
+        case MYEA_LOSS_BIT: counted = false; if (fabsf(diff) >= p.bit_fail_limit) bits += 1.f; break;
+        default: counted = false; break;
+        }
+        if (counted) { loss += e; cnt += 1.f; }
+        switch (p.accuracy) {
+        case MYEA_ACCURACY_DISTANCE: if (fabsf(diff) <= p.accuracy_variance) acc += 1.f; break;
+        case MYEA_ACCURACY_DIRECTIONAL: acc += 1.f; break;
+        case MYEA_ACCURACY_SIGN:
+            if (sign_f(de) == sign_f(yo) || (sign_f(de) == 0.f && yo >= -1.192092896e-07f && yo <= 1.192092896e-07f)) acc += 1.f;
+            break;
+        default: break;
+        }
+        const float q = p.rnn_pre_quirk ? pre[0] : pre[j];
+        err[j] = af_derive(p.act, q, p.steep, yo) * diff;
+    }
+    loss = wave_sum(loss); cnt = wave_sum(cnt); acc = wave_sum(acc); bits = wave_sum(bits);
+    if (lane == 0) {
+        if (cnt != 0.f) { atomicAdd(&p.loss_acc[0], (double)loss); atomicAdd(&p.loss_acc[1], (double)cnt); }
+        if (acc != 0.f) atomicAdd(&p.loss_acc[2], (double)acc);
+        if (bits != 0.f) atomicAdd(&p.loss_acc[3], (double)bits);
+    }
+}
+
+// ---- global-norm clipping and the fused optimizer update -------------------------------------------------
+
+// Euclidean_Norm (NN/Neural_Network__Regularization__Max_Norm_Constraints.cpp:48-140), sum-of-squares part
+__global__ __launch_bounds__(kBlock) void sum_squares_partial_kernel(size_t n, const float *g, float *partials)
+{
+    __shared__ float red[kBlock / 64];
+    float s = 0.f;
+    const size_t n4 = n / 4;
+    const f32x4 *g4 = reinterpret_cast<const f32x4 *>(g);
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += (size_t)gridDim.x * kBlock) {
+        const f32x4 v = g4[i];
+        s += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) { const float v = g[n4 * 4 + threadIdx.x]; s += v * v; }
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) partials[blockIdx.x] = red[0] + red[1] + red[2] + red[3];
+}
+
+__global__ __launch_bounds__(kBlock) void sum_squares_final_kernel(unsigned nparts, const float *partials, float *out)
+{
+    __shared__ float red[kBlock / 64];
+    float s = 0.f;
+    for (unsigned i = threadIdx.x; i < nparts; i += kBlock) s += partials[i];
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) out[0] = red[0] + red[1] + red[2] + red[3];
+}
+
+struct UpdateDev {
+    size_t n, n_weights;
+    float *w, *g, *s0, *s1, *s2;
+    float lr, mu, lr_t, beta1, beta2, eps, lower, upper, wd;
+    const float *norm_sq;
+    float clip, grad_scale;
+};
+
+// One element of Update_Parameters__Adam (NN/Neural_Network__Adam.cpp:43-97), __AMSGrad
+// (NN/Neural_Network__AMSGrad.cpp:43-105), __AdaBound (NN/Neural_Network__AdaBound.cpp:43-110),
+// Update_Parameter__Gradient_Descent (NN/Neural_Network__Gradient_Descent.cpp:84-120), __Momentum
+// (NN/Neural_Network__Gradient_Descent_Momentum.cpp:22-62), Nesterov
+// (NN/Neural_Network__Nesterov_Accelerated_Gradient.cpp:22-64; sign of the lr*g term as written there).
+// KIND: 0 GD, 1 momentum, 2 Nesterov, 3 Adam, 4 AMSGrad, 5 AdaBound.
+template <int KIND, bool WD>
+__device__ __forceinline__ void update_one(const UpdateDev &p, float gs, float &w, float g, float &a, float &b, float &c, bool is_weight)
+{
+    g *= gs;
+    float step;
+    if (KIND == 0) {
+        step = p.lr * g;
+    } else if (KIND == 1) {
+        a = p.lr * g + p.mu * a;
+        step = a;
+    } else if (KIND == 2) {
+        a = p.lr * g + p.mu * a;
+        step = p.mu * a - p.lr * g;
+    } else {
+        a = p.beta1 * a + (1.f - p.beta1) * g;
+        b = p.beta2 * b + (1.f - p.beta2) * g * g;
+        if (KIND == 3) step = p.lr_t * a / (sqrtf(b) + p.eps);
+        else if (KIND == 4) { c = fmaxf(c, b); step = p.lr_t * a / (sqrtf(c) + p.eps); }
+        else { float r = p.lr_t / (sqrtf(b) + p.eps); r = r < p.lower ? p.lower : (r > p.upper ? p.upper : r); step = r * a; }
+    }
+    if (WD) step += (is_weight ? 1.f : 0.f) * p.wd * w;
+    w -= step;
+}
+
+template <int KIND, bool WD>
+__global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
+{
+    float gs = p.grad_scale;
+    if (p.norm_sq) {  // Clip_Gradient: scale when norm >= clip (NN/Neural_Network__Clip_Gradient.cpp:81-94)
+        const float norm = sqrtf(p.norm_sq[0]);
+        if (norm >= p.clip) gs = p.clip / norm;
+    }
+    constexpr bool kA = KIND >= 1, kB = KIND >= 3, kC = KIND == 4;
+    const size_t n4 = p.n / 4;
+    f32x4 *w4 = reinterpret_cast<f32x4 *>(p.w), *g4 = reinterpret_cast<f32x4 *>(p.g);
+    f32x4 *a4 = reinterpret_cast<f32x4 *>(p.s0), *b4 = reinterpret_cast<f32x4 *>(p.s1), *c4 = reinterpret_cast<f32x4 *>(p.s2);
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += (size_t)gridDim.x * kBlock) {
+        const f32x4 wv = w4[i], gv = g4[i];
+        f32x4 av = {0.f, 0.f, 0.f, 0.f}, bv = av, cv = av;
+        if (kA) av = a4[i];
+        if (kB) bv = b4[i];
+        if (kC) cv = c4[i];
+        float w[4], a[4], b[4], c[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            w[e] = wv[e]; a[e] = av[e]; b[e] = bv[e]; c[e] = cv[e];
+            update_one<KIND, WD>(p, gs, w[e], gv[e], a[e], b[e], c[e], i * 4 + e < p.n_weights);
+        }
+        w4[i] = f32x4{w[0], w[1], w[2], w[3]};
+        if (kA) a4[i] = f32x4{a[0], a[1], a[2], a[3]};
+        if (kB) b4[i] = f32x4{b[0], b[1], b[2], b[3]};
+        if (kC) c4[i] = f32x4{c[0], c[1], c[2], c[3]};
+        g4[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (p.n & 3)) {
+        const size_t i = n4 * 4 + threadIdx.x;
+        float w = p.w[i], a = kA ? p.s0[i] : 0.f, b = kB ? p.s1[i] : 0.f, c = kC ? p.s2[i] : 0.f;
+        update_one<KIND, WD>(p, gs, w, p.g[i], a, b, c, i < p.n_weights);
+        p.w[i] = w;
+        if (kA) p.s0[i] = a;
+        if (kB) p.s1[i] = b;
+        if (kC) p.s2[i] = c;
+        p.g[i] = 0.f;
+    }
+}
+
+template <int KIND>
+int launch_update_kind(hipStream_t s, const UpdateDev &d, bool wd)
+{
+    const unsigned grid = grid_for(d.n / 4 + 1, kBlock, 256u * 16u);
+    if (wd) hipLaunchKernelGGL((update_kernel<KIND, true>), dim3(grid), dim3(kBlock), 0, s, d);
+    else hipLaunchKernelGGL((update_kernel<KIND, false>), dim3(grid), dim3(kBlock), 0, s, d);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+}  // namespace
+
+// ---- launchers ----------------------------------------------------------------------------------------
+
+int launch_fill(hipStream_t s, float *p, size_t n, float v)
+{
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(fill_kernel, dim3(grid_for(n, kBlock, 4096)), dim3(kBlock), 0, s, p, n, v);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_activation(hipStream_t s, int act, size_t rows, size_t H, const float *x, float *y, const float *colscale)
+{
+    const size_t n = rows * H;
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(activation_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, act, n, H, x, y, colscale);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_softmax(hipStream_t s, size_t rows, size_t H, const float *x, float *y, const float *colscale)
+{
+    if (rows == 0 || H == 0) return MYEA_OK;
+    hipLaunchKernelGGL(softmax_kernel, dim3(grid_for(rows, kBlock / 64)), dim3(kBlock), 0, s, rows, H, x, y, colscale);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_activation_derive(hipStream_t s, int act, float steep, size_t n, const float *pre, const float *val, const float *dy, float *dx)
+{
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(activation_derive_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, act, steep, n, pre, val, dy, dx);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_colscale(hipStream_t s, size_t rows, size_t H, float *y, const float *colscale)
+{
+    const size_t n = rows * H;
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(colscale_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, n, H, y, colscale);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_mask_to_scale(hipStream_t s, size_t n, const uint8_t *mask, float on, float *colscale)
+{
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(mask_to_scale_kernel, dim3(grid_for(n, kBlock, 4096)), dim3(kBlock), 0, s, n, mask, on, colscale);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+// scratch: 64 * H floats at most (S <= 64 row splits)
+int launch_column_sum(hipStream_t s, size_t rows, size_t H, const float *x, float *out, int accumulate, float *scratch)
+{
+    if (H == 0) return MYEA_OK;
+    if (rows == 0) { if (!accumulate) return launch_fill(s, out, H, 0.f); return MYEA_OK; }
+    size_t S, chunk;
+    split_rows(rows, H, S, chunk);
+    SumF f{x, H};
+    hipLaunchKernelGGL((column_partial_kernel<1, SumF>), dim3((unsigned)((H + 63) / 64), (unsigned)S), dim3(kBlock), 0, s, rows, H, chunk, scratch, f);
+    MYEA_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, kBlock)), dim3(kBlock), 0, s, H, S, scratch, out, accumulate);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_bn_forward_training(hipStream_t s, const BnForwardParams &p, float *scratch)
+{
+    if (p.H == 0 || p.rows == 0) return MYEA_OK;
+    size_t S, chunk;
+    split_rows(p.rows, p.H, S, chunk);
+    BnStatF f{p.x, p.H};
+    hipLaunchKernelGGL((column_partial_kernel<2, BnStatF>), dim3((unsigned)((p.H + 63) / 64), (unsigned)S), dim3(kBlock), 0, s, p.rows, p.H, chunk, scratch, f);
+    MYEA_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(bn_forward_final_kernel, dim3(grid_for(p.H, kBlock)), dim3(kBlock), 0, s, p.H, S, p.rows, scratch, p);
+    MYEA_HIP_TRY(hipGetLastError());
+    const size_t n = p.rows * p.H;
+    hipLaunchKernelGGL(bn_forward_apply_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, n, p);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_bn_forward_inference(hipStream_t s, size_t rows, size_t H, const float *x, const float *scale, const float *shift,
+                                const float *mean_avg, const float *var_avg, float *normalizes)
+{
+    const size_t n = rows * H;
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(bn_forward_inference_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, n, H, x, scale, shift, mean_avg, var_avg, normalizes);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_bn_backward(hipStream_t s, const BnBackwardParams &p, float *scratch)
+{
+    if (p.H == 0 || p.rows == 0) return MYEA_OK;
+    size_t S, chunk;
+    split_rows(p.rows, p.H, S, chunk);
+    BnBackF f{p};
+    float *dmean_dvar = scratch;            // 2 * H
+    float *partial = scratch + 2 * p.H;     // S * 4 * H
+    hipLaunchKernelGGL((column_partial_kernel<4, BnBackF>), dim3((unsigned)((p.H + 63) / 64), (unsigned)S), dim3(kBlock), 0, s, p.rows, p.H, chunk, partial, f);
+    MYEA_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(bn_backward_final_kernel, dim3(grid_for(p.H, kBlock)), dim3(kBlock), 0, s, p.H, S, partial, p.dscale, p.dshift, dmean_dvar);
+    MYEA_HIP_TRY(hipGetLastError());
+    const size_t n = p.rows * p.H;
+    hipLaunchKernelGGL(bn_backward_apply_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, n, p, dmean_dvar);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_compute_error(hipStream_t s, const ErrorParams &p)
+{
+    if (p.T <= p.first_t || p.B == 0 || p.H == 0) return MYEA_OK;
+    const size_t nrows = (p.T - p.first_t) * p.B;
+    hipLaunchKernelGGL(compute_error_kernel, dim3(grid_for(nrows, kBlock / 64)), dim3(kBlock), 0, s, p);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_scatter_time_major(hipStream_t s, size_t B, size_t T, size_t W, size_t Bmax, const float *src, float *dst)
+{
+    const size_t n = B * T * W;
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(scatter_time_major_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, B, T, W, Bmax, src, dst);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_sum_squares(hipStream_t s, size_t n, const float *g, float *partials, float *out_sum)
+{
+    const unsigned nparts = grid_for(n / 4 + 1, kBlock, 1024);
+    hipLaunchKernelGGL(sum_squares_partial_kernel, dim3(nparts), dim3(kBlock), 0, s, n, g, partials);
+    MYEA_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(sum_squares_final_kernel, dim3(1), dim3(kBlock), 0, s, nparts, partials, out_sum);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_update(hipStream_t s, const UpdateParams &p)
+{
+    if (p.n == 0) return MYEA_OK;
+    UpdateDev d;
+    d.n = p.n; d.n_weights = p.n_weights;
+    d.w = p.w; d.g = p.g; d.s0 = p.s0; d.s1 = p.s1; d.s2 = p.s2;
+    d.lr = p.lr; d.mu = p.mu; d.lr_t = p.lr_t; d.beta1 = p.beta1; d.beta2 = p.beta2; d.eps = p.eps;
+    d.lower = p.lower; d.upper = p.upper; d.wd = p.wd;
+    d.norm_sq = p.norm_sq; d.clip = p.clip; d.grad_scale = p.grad_scale;
+    const bool wd = p.wd != 0.f;
+    auto need = [&](float *ptr, const char *name) { if (!ptr) { set_last_error("optimizer update: %s state is null", name); return false; } return true; };
+    // the vector path needs 16-byte aligned bases
+    auto al = [](const void *q) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (!al(p.w) || !al(p.g) || !al(p.s0) || !al(p.s1) || !al(p.s2)) { set_last_error("optimizer update: vectors must be 16-byte aligned"); return MYEA_E_INVALID; }
+    switch (p.optimizer) {
+    case MYEA_OPTIMIZER_GD:
+        if (p.variant == 0) return launch_update_kind<0>(s, d, wd);
+        if (!need(p.s0, "previous delta")) return MYEA_E_INVALID;
+        return p.variant == 1 ? launch_update_kind<1>(s, d, wd) : launch_update_kind<2>(s, d, wd);
+    case MYEA_OPTIMIZER_ADAM:
+        if (!need(p.s0, "first moment") || !need(p.s1, "second moment")) return MYEA_E_INVALID;
+        return launch_update_kind<3>(s, d, wd);
+    case MYEA_OPTIMIZER_AMSGRAD:
+        if (!need(p.s0, "first moment") || !need(p.s1, "second moment") || !need(p.s2, "second moment hat")) return MYEA_E_INVALID;
+        return launch_update_kind<4>(s, d, wd);
+    case MYEA_OPTIMIZER_ADABOUND:
+        if (!need(p.s0, "first moment") || !need(p.s1, "second moment")) return MYEA_E_INVALID;
+        return launch_update_kind<5>(s, d, wd);
+    default:
+        set_last_error("optimizer %d is not on this path", p.optimizer);
+        return MYEA_E_UNSUPPORTED;
+    }
+}
+
+}  // namespace myea

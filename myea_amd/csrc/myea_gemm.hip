@@ -1,0 +1,350 @@
+// myea_gemm.hip — FP32 MFMA dense contraction for gfx950 (CDNA4), LDS-staged.
+//
+// One kernel template covers the three contractions of the fully-connected and LSTM path:
+//   forward  Y  = X W^T          (A k-contiguous, B k-contiguous)   Forward_Pass__FC,
+//            Neural_Network__Forward_Pass__OpenMP.cpp:4517-4557
+//   backward dX = delta W        (A k-contiguous, B n-contiguous)   Backward_Pass__FC, Neural_Network__Backward_Pass__OpenMP.cpp:1044-1082
+//   weights  dW += delta^T X     (A m-contiguous, B n-contiguous)   Update_Derivative_Weight__FC,
+//            Neural_Network__Update_Derivative_Weight__OpenMP.cpp:178-216
+//
+// Tiling: a workgroup of 256 lanes (4 wavefronts, 2 x 2) owns a BM x BN tile of C; each wavefront owns
+// (BM/2) x (BN/2) as TM x TN accumulators of v_mfma_f32_32x32x2_f32 (16 VGPRs each).  The K loop moves
+// BK = 32 columns per step: global -> registers (128-bit loads, issued before the MFMA block of the
+// current step) -> LDS (double buffered, one barrier per step).  Operands keep their global
+// orientation in LDS, so no transposes are needed:
+//   k-contiguous operand : LDS [rows][BK + 4]   fragment = one ds_read_b128 per 4 MFMA k-steps
+//   mn-contiguous operand: LDS [BK][rows + 8]   fragment = conflict-free ds_read_b32 per k
+// Inside a group of 8 k's, MFMA step j of lane-half h consumes k = 4h + j for BOTH operands, which is
+// what makes the two layouts interchangeable.
+//
+// Accumulator layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
+//   C[(r / 4) * 8 + (l / 32) * 4 + (r % 4)][l % 32].
+#include "myea_device_af.h"
+#include "myea_kernels.h"
+
+namespace myea {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kBK = 32;
+constexpr int kPadK = 4;   // k-contiguous LDS rows: BK + 4 floats (144 B, keeps 16 B alignment)
+constexpr int kPadMN = 8;  // mn-contiguous LDS rows: rows + 8 floats
+
+template <int ROWS, bool KC>
+struct TileShape {
+    static constexpr int kLd = KC ? (kBK + kPadK) : (ROWS + kPadMN);
+    static constexpr int kFloats = KC ? ROWS * kLd : kBK * kLd;
+    static constexpr int kVec = ROWS * kBK / 4;            // float4 per tile
+    static constexpr int kPasses = kVec / kThreads;        // float4 per thread
+    static_assert(kVec % kThreads == 0, "tile must be a multiple of the workgroup");
+};
+
+// Global -> register -> LDS mover for one operand tile (ROWS x BK).
+template <int ROWS, bool KC, bool VEC>
+struct TileMover {
+    using S = TileShape<ROWS, KC>;
+    f32x4 reg[S::kPasses];
+
+    // base: operand origin; ld: leading dimension; row0: first row (m or n) of the tile;
+    // extent: M or N; k0: first k of the step; K: total depth.
+    __device__ __forceinline__ void load(const float *__restrict__ base, long ld, int row0, int extent, int k0, int K)
+    {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int p = 0; p < S::kPasses; ++p) {
+            int row, k;
+            if (KC) {
+                constexpr int vec_per_row = kBK / 4;
+                constexpr int rows_per_pass = kThreads / vec_per_row;
+                row = t / vec_per_row + p * rows_per_pass;
+                k = (t % vec_per_row) * 4;
+            } else {
+                constexpr int vec_per_k = ROWS / 4;
+                constexpr int k_per_pass = kThreads / vec_per_k;
+                k = t / vec_per_k + p * k_per_pass;
+                row = (t % vec_per_k) * 4;
+            }
+            const int gr = row0 + row, gk = k0 + k;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (KC) {
+                const float *src = base + (long)gr * ld + gk;
+                if (VEC) {
+                    if (gr < extent && gk < K) v = *reinterpret_cast<const f32x4 *>(src);
+                } else if (gr < extent) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (gk + e < K) v[e] = src[e];
+                }
+            } else {
+                const float *src = base + (long)gk * ld + gr;
+                if (VEC) {
+                    if (gk < K && gr < extent) v = *reinterpret_cast<const f32x4 *>(src);
+                } else if (gk < K) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (gr + e < extent) v[e] = src[e];
+                }
+            }
+            reg[p] = v;
+        }
+    }
+
+    __device__ __forceinline__ void store(float *lds) const
+    {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int p = 0; p < S::kPasses; ++p) {
+            int idx;
+            if (KC) {
+                constexpr int vec_per_row = kBK / 4;
+                constexpr int rows_per_pass = kThreads / vec_per_row;
+                idx = (t / vec_per_row + p * rows_per_pass) * S::kLd + (t % vec_per_row) * 4;
+            } else {
+                constexpr int vec_per_k = ROWS / 4;
+                constexpr int k_per_pass = kThreads / vec_per_k;
+                idx = (t / vec_per_k + p * k_per_pass) * S::kLd + (t % vec_per_k) * 4;
+            }
+            *reinterpret_cast<f32x4 *>(lds + idx) = reg[p];
+        }
+    }
+};
+
+// Fragment of one 32-row MFMA operand tile for a group of 8 k's: frag[j] feeds MFMA step j.
+template <int ROWS, bool KC>
+__device__ __forceinline__ f32x4 read_fragment(const float *lds, int tile_row, int kgroup, int lane32, int half)
+{
+    using S = TileShape<ROWS, KC>;
+    if (KC) {
+        return *reinterpret_cast<const f32x4 *>(lds + (tile_row + lane32) * S::kLd + kgroup * 8 + half * 4);
+    } else {
+        f32x4 v;
+        const float *src = lds + (kgroup * 8 + half * 4) * S::kLd + tile_row + lane32;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = src[j * S::kLd];
+        return v;
+    }
+}
+
+struct GemmDev {
+    const float *A, *B;
+    float *C;
+    int M, N, K;
+    long lda, ldb, ldc;
+    int accumulate, epilogue;
+    const float *bias;
+    float *aux_out;
+    const float *colscale;
+    const float *pre, *val;
+    int act;
+    float steep;
+    int nbm, nbn;
+};
+
+template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
+__global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
+{
+    constexpr int TM = BM / 64, TN = BN / 64;  // 32x32 accumulators per wavefront along m / n
+    using SA = TileShape<BM, A_KC>;
+    using SB = TileShape<BN, B_KC>;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    constexpr int kStage = SA::kFloats + SB::kFloats;  // one LDS stage = A tile then B tile
+
+    // Workgroup -> tile.  Consecutive workgroup ids land on different XCDs (8 of them, each with its own
+    // L2), so give every XCD a contiguous run of tile ids, and walk tiles in bands of 8 m-tiles so that a
+    // run shares its B columns and a small set of A rows.
+    const int nblocks = p.nbm * p.nbn;
+    int pid = blockIdx.x;
+    if ((nblocks & 7) == 0) pid = (pid & 7) * (nblocks >> 3) + (pid >> 3);
+    constexpr int kBand = 8;
+    const int band = pid / (kBand * p.nbn);
+    const int band_first = band * kBand;
+    const int band_rows = min(p.nbm - band_first, kBand);
+    const int in_band = pid - band * kBand * p.nbn;
+    const int m0 = (band_first + in_band % band_rows) * BM;
+    const int n0 = (in_band / band_rows) * BN;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane32 = lane & 31, half = lane >> 5;
+    const int wave_m = (wave >> 1) * (BM / 2), wave_n = (wave & 1) * (BN / 2);
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    TileMover<BM, A_KC, VEC> moveA;
+    TileMover<BN, B_KC, VEC> moveB;
+    const int nk = (p.K + kBK - 1) / kBK;
+
+    moveA.load(p.A, p.lda, m0, p.M, 0, p.K);
+    moveB.load(p.B, p.ldb, n0, p.N, 0, p.K);
+    moveA.store(smem);
+    moveB.store(smem + SA::kFloats);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < nk;
+        if (more) {
+            moveA.load(p.A, p.lda, m0, p.M, (kt + 1) * kBK, p.K);
+            moveB.load(p.B, p.ldb, n0, p.N, (kt + 1) * kBK, p.K);
+        }
+        const float *la = smem + cur * kStage, *lb = la + SA::kFloats;
+#pragma unroll
+        for (int g = 0; g < kBK / 8; ++g) {
+            f32x4 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = read_fragment<BM, A_KC>(la, wave_m + i * 32, g, lane32, half);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = read_fragment<BN, B_KC>(lb, wave_n + j * 32, g, lane32, half);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            moveA.store(smem + (cur ^ 1) * kStage);
+            moveB.store(smem + (cur ^ 1) * kStage + SA::kFloats);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue.  A lane owns one column of each accumulator, so per-column operands are read once.
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wave_n + j * 32 + lane32;
+        if (col >= p.N) continue;
+        float bias = 0.f, cs = 1.f;
+        if (p.epilogue == EPI_FC_FORWARD) {
+            if (p.bias) bias = p.bias[col];
+            if (p.colscale) cs = p.colscale[col];
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wave_m + i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+                if (row >= p.M) continue;
+                const long o = (long)row * p.ldc + col;
+                float v = acc[i][j][r];
+                if (p.epilogue == EPI_FC_FORWARD) {
+                    v += bias;
+                    p.C[o] = v;
+                    if (p.aux_out) p.aux_out[o] = af_fire_fused(p.act, v) * cs;
+                } else if (p.epilogue == EPI_FC_DERIVE) {
+                    p.C[o] = v * af_derive_fused(p.act, p.pre[o], p.steep, p.val[o]);
+                } else {
+                    if (p.accumulate) v += p.C[o];
+                    p.C[o] = v;
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
+int launch_one(hipStream_t stream, GemmDev d)
+{
+    using SA = TileShape<BM, A_KC>;
+    using SB = TileShape<BN, B_KC>;
+    constexpr size_t lds_bytes = 2 * (SA::kFloats + SB::kFloats) * sizeof(float);
+    auto kern = gemm_f32_mfma_kernel<BM, BN, A_KC, B_KC, VEC>;
+    static bool attr_done = false;  // per instantiation
+    if (!attr_done) {
+        MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        attr_done = true;
+    }
+    d.nbm = (d.M + BM - 1) / BM;
+    d.nbn = (d.N + BN - 1) / BN;
+    const long nblocks = (long)d.nbm * d.nbn;
+    if (nblocks <= 0 || nblocks > 0x7fffffffL) { set_last_error("gemm: grid of %ld workgroups out of range", nblocks); return MYEA_E_INVALID; }
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(kThreads), lds_bytes, stream, d);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+template <int BM, int BN>
+int launch_layout_vec(hipStream_t stream, const GemmDev &d, bool a_kc, bool b_kc)
+{
+    if (a_kc && b_kc) return launch_one<BM, BN, true, true, true>(stream, d);
+    if (a_kc && !b_kc) return launch_one<BM, BN, true, false, true>(stream, d);
+    return launch_one<BM, BN, false, false, true>(stream, d);
+}
+
+// guarded scalar loads, any alignment, any layout: the general (slow) path
+int launch_layout_scalar(hipStream_t stream, const GemmDev &d, bool a_kc, bool b_kc)
+{
+    if (a_kc && b_kc) return launch_one<64, 64, true, true, false>(stream, d);
+    if (a_kc && !b_kc) return launch_one<64, 64, true, false, false>(stream, d);
+    if (!a_kc && !b_kc) return launch_one<64, 64, false, false, false>(stream, d);
+    return launch_one<64, 64, false, true, false>(stream, d);
+}
+
+}  // namespace
+
+bool gemm_can_fuse_activation(int act)
+{
+    return act == MYEA_AF_LINEAR || act == MYEA_AF_RELU || act == MYEA_AF_LEAKY_RELU || act == MYEA_AF_PARAMETRIC_RELU ||
+           act == MYEA_AF_TANH || act == MYEA_AF_SIGMOID;
+}
+
+int launch_gemm(hipStream_t stream, const GemmParams &p)
+{
+    if (p.M <= 0 || p.N <= 0 || p.K < 0) { set_last_error("gemm: bad shape M=%d N=%d K=%d", p.M, p.N, p.K); return MYEA_E_INVALID; }
+    if (!p.A || !p.B || !p.C) { set_last_error("gemm: null operand"); return MYEA_E_INVALID; }
+    const long a_min = p.a_k_contiguous ? p.K : p.M, b_min = p.b_k_contiguous ? p.K : p.N;
+    if (p.lda < a_min || p.ldb < b_min || p.ldc < p.N) { set_last_error("gemm: leading dimension smaller than the row length"); return MYEA_E_INVALID; }
+    if (p.epilogue == EPI_FC_DERIVE && (!p.pre || !p.val)) { set_last_error("gemm: derive epilogue without pre/val"); return MYEA_E_INVALID; }
+    if (p.epilogue == EPI_FC_DERIVE && !gemm_can_fuse_activation(p.act)) { set_last_error("gemm: activation %d cannot be fused", p.act); return MYEA_E_INVALID; }
+    if (p.epilogue == EPI_FC_FORWARD && p.aux_out && !gemm_can_fuse_activation(p.act)) { set_last_error("gemm: activation %d cannot be fused", p.act); return MYEA_E_INVALID; }
+
+    GemmDev d;
+    d.A = p.A; d.B = p.B; d.C = p.C;
+    d.M = p.M; d.N = p.N; d.K = p.K;
+    d.lda = p.lda; d.ldb = p.ldb; d.ldc = p.ldc;
+    d.accumulate = p.accumulate; d.epilogue = p.epilogue;
+    d.bias = p.bias; d.aux_out = p.aux_out; d.colscale = p.colscale;
+    d.pre = p.pre; d.val = p.val; d.act = p.act; d.steep = p.steep;
+    d.nbm = d.nbn = 0;
+
+    // 128-bit global loads need 16-byte aligned rows; otherwise fall back to guarded scalar loads.
+    auto aligned = [](const float *ptr, long ld, long contiguous_extent) {
+        return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0 && (ld & 3) == 0 && (contiguous_extent & 3) == 0;
+    };
+    const bool vec = aligned(p.A, p.lda, p.a_k_contiguous ? p.K : p.M) && aligned(p.B, p.ldb, p.b_k_contiguous ? p.K : p.N);
+    const bool a_kc = p.a_k_contiguous != 0, b_kc = p.b_k_contiguous != 0;
+
+    if (!vec || (!a_kc && b_kc)) return launch_layout_scalar(stream, d, a_kc, b_kc);
+    // Tile choice: 128 x 128 when that still yields at least two workgroups per CU (256 CUs), else
+    // 64-row tiles to keep the chip filled for short-M / short-N problems.
+    const long tiles_128 = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
+    if (tiles_128 >= 512) return launch_layout_vec<128, 128>(stream, d, a_kc, b_kc);
+    if (p.M <= p.N) return launch_layout_vec<64, 128>(stream, d, a_kc, b_kc);
+    return launch_layout_vec<128, 64>(stream, d, a_kc, b_kc);
+}
+
+}  // namespace myea
+
+extern "C" int myea_hip_gemm_f32(void *stream, int a_k_contiguous, int b_k_contiguous, int accumulate, size_t M, size_t N, size_t K,
+                                 const float *A, size_t lda, const float *B, size_t ldb, float *C, size_t ldc)
+{
+    if (M > 0x7fffffffu || N > 0x7fffffffu || K > 0x7fffffffu) { myea::set_last_error("gemm: dimension too large"); return MYEA_E_INVALID; }
+    myea::GemmParams p{};
+    p.A = A; p.B = B; p.C = C;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    p.lda = (long)lda; p.ldb = (long)ldb; p.ldc = (long)ldc;
+    p.a_k_contiguous = a_k_contiguous; p.b_k_contiguous = b_k_contiguous;
+    p.accumulate = accumulate;
+    p.epilogue = myea::EPI_NONE;
+    return myea::launch_gemm(static_cast<hipStream_t>(stream), p);
+}

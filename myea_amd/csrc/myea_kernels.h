@@ -1,0 +1,124 @@
+// myea_kernels.h — internal launch interface between the net driver and the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/myea_hip.h"
+
+namespace myea {
+
+// ---- error plumbing -------------------------------------------------------------------------
+void set_last_error(const char *fmt, ...);
+int hip_fail(hipError_t e, const char *what);
+
+#define MYEA_HIP_TRY(expr)                                             \
+    do {                                                               \
+        hipError_t e__ = (expr);                                       \
+        if (e__ != hipSuccess) return ::myea::hip_fail(e__, #expr);    \
+    } while (0)
+
+// ---- dense contraction ------------------------------------------------------------------------
+enum GemmEpilogue : int {
+    EPI_NONE = 0,        // C = acc (+ C when accumulate)
+    EPI_FC_FORWARD = 1,  // C = acc + bias[n]; aux_out = AF(C) * colscale[n] when act != MYEA_AF_NONE
+    EPI_FC_DERIVE = 2    // C = acc * AF'(pre[m][n], steep, val[m][n])
+};
+
+struct GemmParams {
+    const float *A, *B;
+    float *C;
+    int M, N, K;
+    long lda, ldb, ldc;
+    int a_k_contiguous, b_k_contiguous;
+    int accumulate;
+    int epilogue;
+    const float *bias;      // EPI_FC_FORWARD, may be null
+    float *aux_out;         // EPI_FC_FORWARD, [M][ldc], may be null
+    const float *colscale;  // EPI_FC_FORWARD, [N] multiplier (dropout), may be null
+    const float *pre;       // EPI_FC_DERIVE, [M][ldc]
+    const float *val;       // EPI_FC_DERIVE, [M][ldc]
+    int act;
+    float steep;
+};
+
+int launch_gemm(hipStream_t stream, const GemmParams &p);
+// activations the FC_FORWARD / FC_DERIVE epilogues can apply (the others run as a separate kernel)
+bool gemm_can_fuse_activation(int act);
+
+// ---- elementwise / reduction kernels ------------------------------------------------------------
+// rows are the leading dimension everywhere: element (r, j) at base[r * H + j].
+
+// y = AF(x) * colscale[j]  (colscale may be null); x and y may alias.
+int launch_activation(hipStream_t s, int act, size_t rows, size_t H, const float *x, float *y, const float *colscale);
+// row softmax (max-subtracted) then * colscale
+int launch_softmax(hipStream_t s, size_t rows, size_t H, const float *x, float *y, const float *colscale);
+// dx = dy * AF'(pre, steep, val)
+int launch_activation_derive(hipStream_t s, int act, float steep, size_t n, const float *pre, const float *val, const float *dy, float *dx);
+// y[r][j] *= colscale[j]
+int launch_colscale(hipStream_t s, size_t rows, size_t H, float *y, const float *colscale);
+// colscale[j] = mask[j] ? on : 0   (training) over n entries
+int launch_mask_to_scale(hipStream_t s, size_t n, const uint8_t *mask, float on, float *colscale);
+// out[j] (+)= sum_r x[r][j]; scratch >= 64 * H floats
+int launch_column_sum(hipStream_t s, size_t rows, size_t H, const float *x, float *out, int accumulate, float *scratch);
+
+// batch-normalisation forward (training): statistics, running averages, r/d corrections, hats, normalizes
+struct BnForwardParams {
+    size_t rows, H;
+    const float *x;
+    const float *scale, *shift;
+    float *mean, *var, *mean_avg, *var_avg, *r_corr, *d_corr;
+    float *hats, *normalizes;
+    float epsilon, momentum, r_max, d_max;
+    int renorm;
+};
+int launch_bn_forward_training(hipStream_t s, const BnForwardParams &p, float *scratch /* >= 128 * H floats */);
+int launch_bn_forward_inference(hipStream_t s, size_t rows, size_t H, const float *x, const float *scale, const float *shift,
+                                const float *mean_avg, const float *var_avg, float *normalizes);
+struct BnBackwardParams {
+    size_t rows, H;
+    const float *x, *hats, *dy;
+    const float *mean, *var, *scale, *r_corr;
+    float *dscale, *dshift;  // accumulated (+=) into the gradient vector
+    float *dx;
+    int renorm;
+};
+int launch_bn_backward(hipStream_t s, const BnBackwardParams &p, float *scratch /* >= 258 * H floats */);
+
+// output-layer delta + loss / accuracy accumulation
+struct ErrorParams {
+    size_t B, T, H, Bmax;
+    const float *values, *pre;   // [T][Bmax][H]
+    const float *desired;        // [B][T][H]
+    float *errors;               // [T][Bmax][H]
+    int act;
+    float steep;
+    int loss, accuracy;
+    float accuracy_variance, bit_fail_limit;
+    size_t first_t;              // number_time_delays
+    int rnn_pre_quirk;           // RNN head: every unit reads the first unit's pre-activation
+    double *loss_acc;            // [0]=loss sum [1]=count [2]=accuracy [3]=bit fails
+};
+int launch_compute_error(hipStream_t s, const ErrorParams &p);
+
+// [B][T][W] (example rows) -> [T][Bmax][W]
+int launch_scatter_time_major(hipStream_t s, size_t B, size_t T, size_t W, size_t Bmax, const float *src, float *dst);
+
+// optimizer
+int launch_sum_squares(hipStream_t s, size_t n, const float *g, float *partials /* >= 1024 */, float *out_sum);
+struct UpdateParams {
+    int optimizer;       // MYEA_OPTIMIZER_*
+    int variant;         // GD: 0 plain, 1 momentum, 2 nesterov
+    size_t n, n_weights;
+    float *w, *g, *s0, *s1, *s2;
+    float lr, mu, lr_t, beta1, beta2, eps, lower, upper, wd;
+    const float *norm_sq;  // device scalar: sum of squares of g, or null (no clipping)
+    float clip;
+    float grad_scale;      // host-side multiplier (used when norm_sq is null)
+};
+int launch_update(hipStream_t s, const UpdateParams &p);
+
+int launch_fill(hipStream_t s, float *p, size_t n, float v);
+
+}  // namespace myea

@@ -1,0 +1,83 @@
+// myea_net.h — the device-resident network object behind the C ABI (internal).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <vector>
+
+#include "../../include/myea_hip.h"
+
+namespace myea {
+
+struct LstmLayer;  // myea_lstm.hip
+
+struct DevLayer {
+    size_t H = 0;  // *Layer::ptr_number_outputs
+    // [T][Bmax][H]
+    float *summations = nullptr, *values = nullptr, *hats = nullptr, *normalizes = nullptr, *neuron_errors = nullptr;
+    // [T][H]
+    float *means = nullptr, *variances = nullptr, *means_averages = nullptr, *variances_averages = nullptr;
+    float *r_corrections = nullptr, *d_corrections = nullptr;
+    float *colscale = nullptr;  // dropout multiplier per (t, unit)
+    LstmLayer *lstm = nullptr;
+};
+
+constexpr int kProfFamilies = 4;
+struct ProfEvent {
+    hipEvent_t start = nullptr, stop = nullptr;
+    int family = 0;
+    double work = 0;
+};
+
+bool layer_uses_norm(const myea_layer_desc &l);
+bool layer_uses_bias(const myea_layer_desc &l);
+
+struct Net {
+    myea_net_desc d{};
+    myea_hyper h{};
+    uint32_t state = MYEA_STATE_INFERENCE;
+    hipStream_t stream = nullptr;
+    float *parameters = nullptr, *gradient = nullptr, *opt[4] = {nullptr, nullptr, nullptr, nullptr};
+    uint8_t *masks = nullptr;
+    std::vector<DevLayer> L;
+    float *tmp1 = nullptr, *tmp2 = nullptr, *scratch = nullptr, *stage_in = nullptr, *stage_out = nullptr;
+    double *loss_acc = nullptr;
+
+    bool profiling = false, open_event = false;
+    std::vector<ProfEvent> pending, free_events;
+    uint64_t prof_launches[kProfFamilies] = {0, 0, 0, 0};
+    double prof_ms[kProfFamilies] = {0, 0, 0, 0}, prof_work[kProfFamilies] = {0, 0, 0, 0};
+
+    ~Net();
+    int create(const myea_net_desc &desc);
+
+    float *layer_outputs(size_t li);
+    float *scale_ptr(float *base, size_t li);
+    float *shift_ptr(float *base, size_t li);
+    void prof_begin(int family);
+    void prof_end(double work);
+
+    int refresh_colscale(size_t li, bool *active);
+    int forward_fc_layer(size_t li, size_t B);
+    int bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training);
+    int bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx);
+    int backward_into_fc_layer(size_t li, size_t B);
+
+    int forward_pass(size_t B, const float *inputs, int on_device);
+    int compute_error(size_t B, const float *desired, int on_device);
+    int backward_pass(size_t B);
+    int update_derivative_weight(size_t B, size_t first, size_t end);
+    int update_parameter(size_t B, size_t training_size);
+
+    // LSTM-with-peephole layers (myea_lstm.hip)
+    int lstm_create_layer(size_t li);
+    void lstm_destroy_layer(DevLayer &o);
+    int lstm_parameters_changed();
+    int lstm_forward_layer(size_t li, size_t B);
+    int lstm_backward_into_layer(size_t li, size_t B);  // delta of layer li from an LSTM consumer li + 1
+    int lstm_backward_layer(size_t li, size_t B);       // BPTT inside LSTM layer li
+    int lstm_update_derivative_weight(size_t li, size_t B);
+    const float *lstm_tensor(size_t li, int kind, size_t *count);
+};
+
+}  // namespace myea

@@ -1,0 +1,741 @@
+// myea_net.hip — the device-resident network behind the C ABI: buffers, the five step entry points and
+// the movement of parameters / optimizer state.  Host code only; the kernels live in myea_gemm.hip and
+// myea_elementwise.hip (and myea_lstm.hip).
+//
+// NN/ = Neural_Network_Library_Windows/Source_Files/Neural_Network/ of the reference.
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "myea_kernels.h"
+#include "myea_net.h"
+
+namespace myea {
+
+// ---- error plumbing ---------------------------------------------------------------------------------
+static thread_local char g_last_error[512] = "";
+
+void set_last_error(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char *what)
+{
+    set_last_error("HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+    return MYEA_E_DEVICE;
+}
+
+// ---- small helpers ------------------------------------------------------------------------------------
+static int dev_alloc(float **p, size_t count)
+{
+    *p = nullptr;
+    void *q = nullptr;
+    hipError_t e = hipMalloc(&q, (count ? count : 1) * sizeof(float));
+    if (e != hipSuccess) { hip_fail(e, "hipMalloc"); return MYEA_E_NOMEM; }
+    *p = static_cast<float *>(q);
+    return MYEA_OK;
+}
+
+#define MYEA_TRY(expr)                 \
+    do {                               \
+        int rc__ = (expr);             \
+        if (rc__ != MYEA_OK) return rc__; \
+    } while (0)
+
+bool layer_uses_norm(const myea_layer_desc &l) { return l.type_normalization != MYEA_NORMALIZATION_NONE; }
+bool layer_uses_bias(const myea_layer_desc &l) { return !layer_uses_norm(l); }  // Layer::Use__Bias, Data.hpp:736
+
+float *Net::layer_outputs(size_t li)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    if (li != 0 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED && layer_uses_norm(l) && !l.use_layer_normalization_before_activation) return o.normalizes;
+    return o.values;
+}
+
+float *Net::scale_ptr(float *base, size_t li) { return base + d.total_weights + d.total_bias + d.layers[li].first_normalized_unit_index; }
+float *Net::shift_ptr(float *base, size_t li) { return scale_ptr(base, li) + d.total_normalized_units; }
+
+// ---- profiling ------------------------------------------------------------------------------------------
+void Net::prof_begin(int family)
+{
+    if (!profiling) return;
+    ProfEvent ev;
+    ev.family = family;
+    if (!free_events.empty()) { ev = free_events.back(); free_events.pop_back(); ev.family = family; }
+    else if (hipEventCreate(&ev.start) != hipSuccess || hipEventCreate(&ev.stop) != hipSuccess) return;
+    hipEventRecord(ev.start, stream);
+    pending.push_back(ev);
+    open_event = true;
+}
+
+void Net::prof_end(double work)
+{
+    if (!profiling || !open_event) return;
+    ProfEvent &ev = pending.back();
+    ev.work = work;
+    hipEventRecord(ev.stop, stream);
+    open_event = false;
+}
+
+static int check_desc(const myea_net_desc &d)
+{
+    if (d.n_layers < 2 || d.n_layers > MYEA_MAX_LAYERS) { set_last_error("descriptor: %u layers (need 2..%d)", d.n_layers, MYEA_MAX_LAYERS); return MYEA_E_INVALID; }
+    if (d.batch_size == 0 || d.number_recurrent_depth == 0) { set_last_error("descriptor: batch_size and number_recurrent_depth must be >= 1"); return MYEA_E_INVALID; }
+    if (d.total_parameters != d.total_weights + d.total_bias + 2 * d.total_normalized_units) { set_last_error("descriptor: total_parameters inconsistent"); return MYEA_E_INVALID; }
+    if (d.layers[0].type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("descriptor: the input layer must be a fully-connected (unit) layer"); return MYEA_E_INVALID; }
+    for (uint32_t li = 0; li < d.n_layers; ++li) {
+        const myea_layer_desc &l = d.layers[li];
+        if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED && l.type_layer != MYEA_LAYER_LSTM) {
+            set_last_error("layer %u: type %u is not on this path", li, l.type_layer);
+            return MYEA_E_UNSUPPORTED;
+        }
+        if (l.n_units == 0) { set_last_error("layer %u: no units", li); return MYEA_E_INVALID; }
+        if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_BERNOULLI && l.type_dropout != MYEA_DROPOUT_BERNOULLI_INVERTED) {
+            set_last_error("layer %u: dropout type %u is not on this path", li, l.type_dropout);
+            return MYEA_E_UNSUPPORTED;
+        }
+        if (l.type_normalization > MYEA_NORMALIZATION_BATCH_RENORMALIZATION) { set_last_error("layer %u: normalization type %u is not on this path", li, l.type_normalization); return MYEA_E_UNSUPPORTED; }
+        if (l.type_layer == MYEA_LAYER_FULLY_CONNECTED && li > 0) {
+            if (l.type_activation_function == MYEA_AF_NONE || l.type_activation_function >= MYEA_AF_LENGTH) { set_last_error("layer %u: activation %u invalid", li, l.type_activation_function); return MYEA_E_INVALID; }
+            const size_t fan_in = (d.layers[li - 1].type_layer == MYEA_LAYER_LSTM) ? (size_t)d.layers[li - 1].n_units * d.layers[li - 1].n_cells_per_block : d.layers[li - 1].n_units;
+            if (l.first_connection_index + fan_in * l.n_units > d.total_weights) { set_last_error("layer %u: weight slice leaves the weight region", li); return MYEA_E_INVALID; }
+            if (layer_uses_bias(l) && l.first_bias_connection_index + l.n_units > d.total_weights + d.total_bias) { set_last_error("layer %u: bias slice leaves the bias region", li); return MYEA_E_INVALID; }
+            if (layer_uses_norm(l) && l.first_normalized_unit_index + l.n_units > d.total_normalized_units) { set_last_error("layer %u: scale/shift slice leaves its region", li); return MYEA_E_INVALID; }
+        }
+        if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_layer == MYEA_LAYER_FULLY_CONNECTED &&
+            l.first_mask_index + (uint64_t)l.n_units * d.number_recurrent_depth > d.total_mask_units) { set_last_error("layer %u: mask slice leaves the mask buffer", li); return MYEA_E_INVALID; }
+    }
+    return MYEA_OK;
+}
+
+int Net::create(const myea_net_desc &desc)
+{
+    MYEA_TRY(check_desc(desc));
+    d = desc;
+    myea_hyper_default(&h);
+    const size_t P = d.total_parameters, T = d.number_recurrent_depth, B = d.batch_size;
+    MYEA_TRY(dev_alloc(&parameters, P));
+    MYEA_TRY(dev_alloc(&gradient, P));
+    for (int k = 0; k < 4; ++k) MYEA_TRY(dev_alloc(&opt[k], P));
+    MYEA_HIP_TRY(hipMemset(parameters, 0, P * sizeof(float)));
+    MYEA_HIP_TRY(hipMemset(gradient, 0, P * sizeof(float)));
+    for (int k = 0; k < 4; ++k) MYEA_HIP_TRY(hipMemset(opt[k], 0, P * sizeof(float)));
+    if (d.total_normalized_units) MYEA_TRY(launch_fill(0, parameters + d.total_weights + d.total_bias, d.total_normalized_units, 1.f));
+    {
+        void *q = nullptr;
+        MYEA_HIP_TRY(hipMalloc(&q, d.total_mask_units ? d.total_mask_units : 1));
+        masks = static_cast<uint8_t *>(q);
+        MYEA_HIP_TRY(hipMemset(masks, 1, d.total_mask_units ? d.total_mask_units : 1));  // all true, NN/Neural_Network__Allocate.cpp:386-410
+    }
+    size_t max_h = 0;
+    L.resize(d.n_layers);
+    for (size_t li = 0; li < d.n_layers; ++li) {
+        const myea_layer_desc &l = d.layers[li];
+        DevLayer &o = L[li];
+        o.H = (l.type_layer == MYEA_LAYER_LSTM) ? (size_t)l.n_units * l.n_cells_per_block : l.n_units;
+        if (o.H > max_h) max_h = o.H;
+        const size_t sz = T * B * o.H;
+        MYEA_TRY(dev_alloc(&o.values, sz));
+        MYEA_HIP_TRY(hipMemset(o.values, 0, sz * sizeof(float)));
+        if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(dev_alloc(&o.colscale, T * o.H));
+        if (li == 0) continue;
+        if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_create_layer(li)); continue; }
+        MYEA_TRY(dev_alloc(&o.summations, sz));
+        MYEA_TRY(dev_alloc(&o.neuron_errors, sz));
+        MYEA_HIP_TRY(hipMemset(o.summations, 0, sz * sizeof(float)));
+        MYEA_HIP_TRY(hipMemset(o.neuron_errors, 0, sz * sizeof(float)));
+        if (layer_uses_norm(l)) {
+            MYEA_TRY(dev_alloc(&o.hats, sz));
+            MYEA_TRY(dev_alloc(&o.normalizes, sz));
+            MYEA_HIP_TRY(hipMemset(o.hats, 0, sz * sizeof(float)));
+            MYEA_HIP_TRY(hipMemset(o.normalizes, 0, sz * sizeof(float)));
+            float **small[] = {&o.means, &o.variances, &o.means_averages, &o.variances_averages, &o.r_corrections, &o.d_corrections};
+            for (float **s : small) { MYEA_TRY(dev_alloc(s, T * o.H)); MYEA_HIP_TRY(hipMemset(*s, 0, T * o.H * sizeof(float))); }
+            MYEA_TRY(launch_fill(0, o.variances_averages, T * o.H, 1.f));  // NN/Neural_Network__Allocate.cpp:2612-2615
+        }
+    }
+    MYEA_TRY(dev_alloc(&tmp1, T * B * max_h));
+    MYEA_TRY(dev_alloc(&tmp2, T * B * max_h));
+    MYEA_TRY(dev_alloc(&scratch, 258 * max_h + 2048));
+    MYEA_TRY(dev_alloc(&stage_in, T * B * L[0].H));
+    MYEA_TRY(dev_alloc(&stage_out, T * B * L[d.n_layers - 1].H));
+    {
+        void *q = nullptr;
+        MYEA_HIP_TRY(hipMalloc(&q, 4 * sizeof(double)));
+        loss_acc = static_cast<double *>(q);
+        MYEA_HIP_TRY(hipMemset(loss_acc, 0, 4 * sizeof(double)));
+    }
+    MYEA_HIP_TRY(hipDeviceSynchronize());
+    return MYEA_OK;
+}
+
+Net::~Net()
+{
+    auto fr = [](void *p) { if (p) (void)hipFree(p); };
+    fr(parameters); fr(gradient);
+    for (int k = 0; k < 4; ++k) fr(opt[k]);
+    fr(masks);
+    for (DevLayer &o : L) {
+        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.colscale);
+        fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
+        lstm_destroy_layer(o);
+    }
+    fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc);
+    for (ProfEvent &e : pending) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
+    for (ProfEvent &e : free_events) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
+}
+
+// ---- dropout column multipliers ---------------------------------------------------------------------------
+// Training: Bernoulli -> mask ? 1 : 0; inverted -> mask ? 1/keep : 0 (NN/Neural_Network__Forward_Pass__OpenMP.cpp:
+// 628-647, 4907-4966).  Inference: Bernoulli scales by keep (:4968-4990); inverted does nothing.
+int Net::refresh_colscale(size_t li, bool *active)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    *active = false;
+    if (l.type_dropout == MYEA_DROPOUT_NONE || !o.colscale) return MYEA_OK;
+    const size_t n = (size_t)d.number_recurrent_depth * o.H;
+    if (state == MYEA_STATE_TRAINING) {
+        float on = 1.f;
+        if (l.type_dropout == MYEA_DROPOUT_BERNOULLI_INVERTED) on = l.dropout_values[0] == 0.f ? 0.f : 1.f / l.dropout_values[0];
+        MYEA_TRY(launch_mask_to_scale(stream, n, masks + l.first_mask_index, on, o.colscale));
+        *active = true;
+    } else if (l.type_dropout == MYEA_DROPOUT_BERNOULLI) {
+        MYEA_TRY(launch_fill(stream, o.colscale, n, l.dropout_values[0]));
+        *active = true;
+    }
+    return MYEA_OK;
+}
+
+// ---- forward ----------------------------------------------------------------------------------------------
+// Forward_Pass__FC (layer driver), NN/Neural_Network__Forward_Pass__OpenMP.cpp:256-698:
+// GEMM -> bias -> [BN before] -> activation / softmax -> [BN after] -> dropout.
+int Net::forward_fc_layer(size_t li, size_t B)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, In = L[li - 1].H, H = o.H;
+    const float *x = layer_outputs(li - 1);
+    const bool norm = layer_uses_norm(l), before = l.use_layer_normalization_before_activation != 0;
+    const bool softmax = l.type_activation_function == MYEA_AF_SOFTMAX;
+    const bool training = state >= MYEA_STATE_TRAINING;
+    bool drop = false;
+    MYEA_TRY(refresh_colscale(li, &drop));
+    // all time steps in one launch when the rows are contiguous and nothing is per time step
+    const bool per_t = T > 1 && (B != Bmax || norm || drop);
+    const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
+    for (size_t c = 0; c < chunks; ++c) {
+        const size_t roff = c * Bmax;  // first row of the chunk
+        const float *cs = drop ? o.colscale + c * H : nullptr;
+        GemmParams g{};
+        g.A = x + roff * In; g.lda = (long)In; g.a_k_contiguous = 1;
+        g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 1;
+        g.C = o.summations + roff * H; g.ldc = (long)H;
+        g.M = (int)rows; g.N = (int)H; g.K = (int)In;
+        g.epilogue = EPI_FC_FORWARD;
+        g.bias = layer_uses_bias(l) ? parameters + l.first_bias_connection_index : nullptr;
+        g.act = (int)l.type_activation_function;
+        const bool fuse_af = !softmax && !(norm && before) && gemm_can_fuse_activation((int)l.type_activation_function);
+        g.aux_out = fuse_af ? o.values + roff * H : nullptr;
+        g.colscale = (fuse_af && !norm) ? cs : nullptr;
+        prof_begin(0);
+        MYEA_TRY(launch_gemm(stream, g));
+        prof_end(2.0 * (double)rows * (double)H * (double)In);
+
+        const float *cur = o.summations + roff * H;
+        if (norm && before) {
+            MYEA_TRY(bn_forward(li, c, rows, cur, training));
+            cur = o.normalizes + roff * H;
+        }
+        if (softmax) MYEA_TRY(launch_softmax(stream, rows, H, cur, o.values + roff * H, norm ? nullptr : cs));
+        else if (!fuse_af) MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, rows, H, cur, o.values + roff * H, cs));
+        if (norm && !before) {
+            MYEA_TRY(bn_forward(li, c, rows, o.values + roff * H, training));
+            if (cs) MYEA_TRY(launch_colscale(stream, rows, H, o.normalizes + roff * H, cs));
+        }
+    }
+    return MYEA_OK;
+}
+
+int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    const size_t H = o.H, roff = t * d.batch_size;
+    if (!training) {
+        return launch_bn_forward_inference(stream, rows, H, x, scale_ptr(parameters, li), shift_ptr(parameters, li),
+                                           o.means_averages + t * H, o.variances_averages + t * H, o.normalizes + roff * H);
+    }
+    BnForwardParams p{};
+    p.rows = rows; p.H = H; p.x = x;
+    p.scale = scale_ptr(parameters, li); p.shift = shift_ptr(parameters, li);
+    p.mean = o.means + t * H; p.var = o.variances + t * H;
+    p.mean_avg = o.means_averages + t * H; p.var_avg = o.variances_averages + t * H;
+    p.r_corr = o.r_corrections + t * H; p.d_corr = o.d_corrections + t * H;
+    p.hats = o.hats + roff * H; p.normalizes = o.normalizes + roff * H;
+    p.epsilon = h.normalization_epsilon; p.momentum = h.normalization_momentum_average;
+    p.r_max = h.batch_renormalization_r_correction_maximum; p.d_max = h.batch_renormalization_d_correction_maximum;
+    p.renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    return launch_bn_forward_training(stream, p, scratch);
+}
+
+// FF__Forward_Pass_Batch (NN/Neural_Network__Forward_Pass__OpenMP.cpp:24-120) / RNN__Forward_Pass_Batch
+// (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:24-130): assign inputs, then layer by layer.
+int Net::forward_pass(size_t B, const float *inputs, int on_device)
+{
+    if (!inputs) { set_last_error("Forward_Pass: null inputs"); return MYEA_E_INVALID; }
+    if (B == 0 || B > d.batch_size) { set_last_error("Forward_Pass: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
+    const size_t T = d.number_recurrent_depth, In = L[0].H, Bmax = d.batch_size;
+    const size_t n = B * T * In;
+    if (T == 1) {
+        MYEA_HIP_TRY(hipMemcpyAsync(L[0].values, inputs, n * sizeof(float), on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, stream));
+    } else {
+        const float *src = inputs;
+        if (!on_device) {
+            MYEA_HIP_TRY(hipMemcpyAsync(stage_in, inputs, n * sizeof(float), hipMemcpyHostToDevice, stream));
+            src = stage_in;
+        }
+        MYEA_TRY(launch_scatter_time_major(stream, B, T, In, Bmax, src, L[0].values));
+    }
+    bool drop = false;
+    MYEA_TRY(refresh_colscale(0, &drop));
+    if (drop) {
+        for (size_t t = 0; t < T; ++t) MYEA_TRY(launch_colscale(stream, B, In, L[0].values + t * Bmax * In, L[0].colscale + t * In));
+    }
+    for (size_t li = 1; li < d.n_layers; ++li) {
+        if (d.layers[li].type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(forward_fc_layer(li, B));
+        else MYEA_TRY(lstm_forward_layer(li, B));
+    }
+    return MYEA_OK;
+}
+
+// ---- Compute__Error -------------------------------------------------------------------------------------------
+int Net::compute_error(size_t B, const float *desired, int on_device)
+{
+    if (!desired) { set_last_error("Compute__Error: null desired outputs"); return MYEA_E_INVALID; }
+    if (B == 0 || B > d.batch_size) { set_last_error("Compute__Error: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
+    const size_t lo = d.n_layers - 1, T = d.number_recurrent_depth;
+    const myea_layer_desc &l = d.layers[lo];
+    if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("Compute__Error: the output layer must be fully connected"); return MYEA_E_UNSUPPORTED; }
+    DevLayer &o = L[lo];
+    const float *dsrc = desired;
+    if (!on_device) {
+        MYEA_HIP_TRY(hipMemcpyAsync(stage_out, desired, B * T * o.H * sizeof(float), hipMemcpyHostToDevice, stream));
+        dsrc = stage_out;
+    }
+    ErrorParams p{};
+    p.B = B; p.T = T; p.H = o.H; p.Bmax = d.batch_size;
+    p.values = o.values;
+    p.pre = (layer_uses_norm(l) && l.use_layer_normalization_before_activation) ? o.normalizes : o.summations;
+    p.desired = dsrc;
+    p.errors = o.neuron_errors;  // AF errors are copied to the neuron errors unchanged (:136-139)
+    p.act = (int)l.type_activation_function; p.steep = l.activation_steepness;
+    p.loss = (int)h.type_loss_function; p.accuracy = (int)h.type_accuracy_function;
+    p.accuracy_variance = h.accuracy_variance; p.bit_fail_limit = h.bit_fail_limit;
+    p.first_t = T > 1 ? h.number_time_delays : 0;
+    p.rnn_pre_quirk = T > 1;
+    p.loss_acc = loss_acc;
+    return launch_compute_error(stream, p);
+}
+
+// ---- backward ---------------------------------------------------------------------------------------------------
+// FF__Backward_Pass_Batch (NN/Neural_Network__Backward_Pass__OpenMP.cpp:24-155): for every layer below the
+// output layer, dX = delta_next * W_next (Backward_Pass__FC, :1044-1082) and then
+// Backward_Pass__Gradient__FC (:544-709): [BN after] -> act' -> [BN before].  The act' multiply is fused
+// into the dX contraction's epilogue whenever it directly follows it.
+int Net::backward_into_fc_layer(size_t li, size_t B)
+{
+    const size_t gi = li + 1;
+    const myea_layer_desc &l = d.layers[li], &next = d.layers[gi];
+    DevLayer &o = L[li], &on = L[gi];
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, H = o.H, Out = on.H;
+    const bool norm = layer_uses_norm(l), before = l.use_layer_normalization_before_activation != 0;
+    const bool per_t = T > 1 && (B != Bmax || norm);
+    const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
+    if (next.type_layer != MYEA_LAYER_FULLY_CONNECTED) return lstm_backward_into_layer(li, B);
+    for (size_t c = 0; c < chunks; ++c) {
+        const size_t roff = c * Bmax;
+        GemmParams g{};
+        g.A = on.neuron_errors + roff * Out; g.lda = (long)Out; g.a_k_contiguous = 1;
+        g.B = parameters + next.first_connection_index; g.ldb = (long)H; g.b_k_contiguous = 0;
+        g.M = (int)rows; g.N = (int)H; g.K = (int)Out;
+        g.ldc = (long)H;
+        g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
+        const bool fuse = gemm_can_fuse_activation(g.act);
+        if (!norm) {
+            g.C = (fuse ? o.neuron_errors : tmp1) + roff * H;
+            g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.summations + roff * H; g.val = o.values + roff * H;
+        } else if (before) {
+            g.C = tmp1 + roff * H;
+            g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.normalizes + roff * H; g.val = o.values + roff * H;
+        } else {
+            g.C = tmp1 + roff * H;
+            g.epilogue = EPI_NONE;
+        }
+        prof_begin(1);
+        MYEA_TRY(launch_gemm(stream, g));
+        prof_end(2.0 * (double)rows * (double)H * (double)Out);
+        if (!fuse && !(norm && !before)) {  // act' as its own kernel (Backward_Pass__FC__DF)
+            MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, rows * H, g.pre, g.val, tmp1 + roff * H, (norm ? tmp1 : o.neuron_errors) + roff * H));
+        }
+        if (norm && before) {
+            MYEA_TRY(bn_backward(li, c, rows, o.summations + roff * H, tmp1 + roff * H, o.neuron_errors + roff * H));
+        } else if (norm) {
+            MYEA_TRY(bn_backward(li, c, rows, o.values + roff * H, tmp1 + roff * H, tmp2 + roff * H));
+            MYEA_TRY(launch_activation_derive(stream, (int)l.type_activation_function, l.activation_steepness, rows * H,
+                                              o.summations + roff * H, o.values + roff * H, tmp2 + roff * H, o.neuron_errors + roff * H));
+        }
+    }
+    return MYEA_OK;
+}
+
+int Net::bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    const size_t H = o.H, roff = t * d.batch_size;
+    BnBackwardParams p{};
+    p.rows = rows; p.H = H; p.x = x; p.hats = o.hats + roff * H; p.dy = dy;
+    p.mean = o.means + t * H; p.var = o.variances + t * H; p.scale = scale_ptr(parameters, li); p.r_corr = o.r_corrections + t * H;
+    p.dscale = scale_ptr(gradient, li); p.dshift = shift_ptr(gradient, li);
+    p.dx = dx;
+    p.renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    return launch_bn_backward(stream, p, scratch);
+}
+
+int Net::backward_pass(size_t B)
+{
+    if (B == 0 || B > d.batch_size) { set_last_error("Backward_Pass: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
+    if (state != MYEA_STATE_TRAINING) { set_last_error("Backward_Pass: can not back propagate gradient in inference mode"); return MYEA_E_STATE; }
+    for (size_t gi = d.n_layers - 1; gi >= 2; --gi) {
+        const size_t li = gi - 1;
+        if (d.layers[li].type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(backward_into_fc_layer(li, B));
+        else MYEA_TRY(lstm_backward_layer(li, B));
+    }
+    return MYEA_OK;
+}
+
+// ---- Update_Derivative_Weight -----------------------------------------------------------------------------------
+// FF__Update_Derivative_Weight_Batch (NN/Neural_Network__Update_Derivative_Weight__OpenMP.cpp:24-59):
+// dW += delta^T X (:178-216) with X = the previous layer's post-dropout outputs, db += column sums (:218-242).
+int Net::update_derivative_weight(size_t B, size_t first, size_t end)
+{
+    if (first < 1 || end > d.n_layers || first > end) { set_last_error("Update_Derivative_Weight: layer range [%zu, %zu) invalid", first, end); return MYEA_E_INVALID; }
+    if (B == 0 || B > d.batch_size) { set_last_error("Update_Derivative_Weight: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
+    for (size_t li = first; li < end; ++li) {
+        const myea_layer_desc &l = d.layers[li];
+        if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_update_derivative_weight(li, B)); continue; }
+        DevLayer &o = L[li];
+        const size_t In = L[li - 1].H, H = o.H;
+        const float *x = layer_outputs(li - 1);
+        const bool per_t = T > 1 && B != Bmax;
+        const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
+        for (size_t c = 0; c < chunks; ++c) {
+            const size_t roff = c * Bmax;
+            GemmParams g{};
+            g.A = o.neuron_errors + roff * H; g.lda = (long)H; g.a_k_contiguous = 0;
+            g.B = x + roff * In; g.ldb = (long)In; g.b_k_contiguous = 0;
+            g.C = gradient + l.first_connection_index; g.ldc = (long)In;
+            g.M = (int)H; g.N = (int)In; g.K = (int)rows;
+            g.accumulate = 1; g.epilogue = EPI_NONE;
+            prof_begin(2);
+            MYEA_TRY(launch_gemm(stream, g));
+            prof_end(2.0 * (double)rows * (double)H * (double)In);
+            if (layer_uses_bias(l)) MYEA_TRY(launch_column_sum(stream, rows, H, o.neuron_errors + roff * H, gradient + l.first_bias_connection_index, 1, scratch));
+        }
+    }
+    return MYEA_OK;
+}
+
+// ---- Update_Parameter ------------------------------------------------------------------------------------------------
+// Update_Parameter__OpenMP (NN/Neural_Network.cpp:4727-4828): [merge: one accumulator here] -> clip by global norm
+// over all P (NN/Neural_Network__Clip_Gradient.cpp:81-94) -> optimizer.  The clip scale is applied inside the
+// optimizer's gradient read instead of a separate pass over the gradient.
+int Net::update_parameter(size_t B, size_t training_size)
+{
+    (void)B; (void)training_size;
+    UpdateParams p{};
+    p.optimizer = (int)h.type_optimizer_function;
+    p.n = d.total_parameters; p.n_weights = d.total_weights;
+    p.w = parameters; p.g = gradient;
+    p.grad_scale = 1.f;
+    p.wd = h.regularization__weight_decay;
+    if (h.use_clip_gradient) {
+        MYEA_TRY(launch_sum_squares(stream, p.n, gradient, scratch + 16, scratch));
+        p.norm_sq = scratch;
+        p.clip = h.clip_gradient;
+    }
+    h.optimizer_time_step += 1.f;
+    const float ts = h.optimizer_time_step;
+    double bytes_per_param = 16;
+    switch (h.type_optimizer_function) {
+    case MYEA_OPTIMIZER_GD:
+        p.lr = h.learning_rate; p.mu = h.learning_momentum;
+        p.variant = h.learning_momentum != 0.f ? (h.use_Nesterov ? 2 : 1) : 0;
+        p.s0 = opt[MYEA_STATE_PREVIOUS_DELTA];
+        bytes_per_param = p.variant ? 24 : 16;
+        break;
+    case MYEA_OPTIMIZER_ADAM:
+    case MYEA_OPTIMIZER_AMSGRAD:
+    case MYEA_OPTIMIZER_ADABOUND:
+        p.beta1 = h.adam_beta1; p.beta2 = h.adam_beta2; p.eps = h.adam_epsilon;
+        p.lr_t = h.use_adam_bias_correction
+                     ? (float)(h.adam_learning_rate * std::sqrt(1.0 - std::pow((double)h.adam_beta2, (double)ts)) / (1.0 - std::pow((double)h.adam_beta1, (double)ts)))
+                     : h.adam_learning_rate;
+        p.lower = h.learning_rate_final * (1.f - 1.f / (h.learning_gamma * ts + 1.f));
+        p.upper = h.learning_rate_final * (1.f + 1.f / (h.learning_gamma * ts));
+        p.s0 = opt[MYEA_STATE_FIRST_MOMENT]; p.s1 = opt[MYEA_STATE_SECOND_MOMENT]; p.s2 = opt[MYEA_STATE_SECOND_MOMENT_HAT];
+        bytes_per_param = h.type_optimizer_function == MYEA_OPTIMIZER_AMSGRAD ? 40 : 32;
+        break;
+    default:
+        h.optimizer_time_step -= 1.f;
+        set_last_error("Update_Parameter: optimizer %u is not on this path", h.type_optimizer_function);
+        return MYEA_E_UNSUPPORTED;
+    }
+    prof_begin(3);
+    const int rc = launch_update(stream, p);
+    prof_end(bytes_per_param * (double)p.n);
+    return rc;
+}
+
+}  // namespace myea
+
+// =====================================================================================================================
+// C ABI
+// =====================================================================================================================
+using myea::Net;
+
+struct myea_hip_net { Net net; };
+
+#define NET_OR_FAIL(n)                                             \
+    do {                                                           \
+        if (!(n)) { myea::set_last_error("null network handle"); return MYEA_E_INVALID; } \
+    } while (0)
+
+extern "C" {
+
+const char *myea_hip_last_error(void) { return myea::g_last_error; }
+
+int myea_hip_create(const myea_net_desc *desc, myea_hip_net **out)
+{
+    if (!desc || !out) { myea::set_last_error("myea_hip_create: null argument"); return MYEA_E_INVALID; }
+    *out = nullptr;
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) { myea::set_last_error("myea_hip_create: no HIP device"); return MYEA_E_DEVICE; }
+    myea_hip_net *n = new (std::nothrow) myea_hip_net();
+    if (!n) return MYEA_E_NOMEM;
+    const int rc = n->net.create(*desc);
+    if (rc != MYEA_OK) { delete n; return rc; }
+    *out = n;
+    return MYEA_OK;
+}
+
+int myea_hip_destroy(myea_hip_net *n)
+{
+    if (!n) return MYEA_OK;
+    (void)hipStreamSynchronize(n->net.stream);
+    delete n;
+    return MYEA_OK;
+}
+
+int myea_hip_set_stream(myea_hip_net *n, void *s) { NET_OR_FAIL(n); n->net.stream = static_cast<hipStream_t>(s); return MYEA_OK; }
+int myea_hip_synchronize(myea_hip_net *n) { NET_OR_FAIL(n); MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream)); return MYEA_OK; }
+
+int myea_hip_set_hyper(myea_hip_net *n, const myea_hyper *h)
+{
+    NET_OR_FAIL(n);
+    if (!h) { myea::set_last_error("set_hyper: null"); return MYEA_E_INVALID; }
+    n->net.h = *h;
+    return MYEA_OK;
+}
+int myea_hip_get_hyper(myea_hip_net *n, myea_hyper *h)
+{
+    NET_OR_FAIL(n);
+    if (!h) { myea::set_last_error("get_hyper: null"); return MYEA_E_INVALID; }
+    *h = n->net.h;
+    return MYEA_OK;
+}
+int myea_hip_set_state_propagation(myea_hip_net *n, uint32_t s)
+{
+    NET_OR_FAIL(n);
+    if (s > MYEA_STATE_TRAINING) { myea::set_last_error("state propagation %u is not on this path", s); return MYEA_E_UNSUPPORTED; }
+    n->net.state = s;
+    return MYEA_OK;
+}
+
+static int copy_vec(myea_hip_net *n, float *dev, float *host_out, const float *host_in, size_t count, const char *what)
+{
+    if (count > n->net.d.total_parameters) { myea::set_last_error("%s: count %zu > total_parameters %llu", what, count, (unsigned long long)n->net.d.total_parameters); return MYEA_E_INVALID; }
+    if (host_in) MYEA_HIP_TRY(hipMemcpyAsync(dev, host_in, count * sizeof(float), hipMemcpyHostToDevice, n->net.stream));
+    else MYEA_HIP_TRY(hipMemcpyAsync(host_out, dev, count * sizeof(float), hipMemcpyDeviceToHost, n->net.stream));
+    MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
+    return MYEA_OK;
+}
+
+int myea_hip_upload_parameters(myea_hip_net *n, const float *p, size_t c)
+{
+    NET_OR_FAIL(n);
+    if (!p) { myea::set_last_error("upload_parameters: null"); return MYEA_E_INVALID; }
+    const int rc = copy_vec(n, n->net.parameters, nullptr, p, c, "upload_parameters");
+    if (rc == MYEA_OK) return n->net.lstm_parameters_changed();
+    return rc;
+}
+int myea_hip_download_parameters(myea_hip_net *n, float *p, size_t c)
+{
+    NET_OR_FAIL(n);
+    if (!p) { myea::set_last_error("download_parameters: null"); return MYEA_E_INVALID; }
+    return copy_vec(n, n->net.parameters, p, nullptr, c, "download_parameters");
+}
+int myea_hip_upload_optimizer_state(myea_hip_net *n, int kind, const float *p, size_t c)
+{
+    NET_OR_FAIL(n);
+    if (kind < 0 || kind > 3 || !p) { myea::set_last_error("upload_optimizer_state: bad kind %d or null", kind); return MYEA_E_INVALID; }
+    return copy_vec(n, n->net.opt[kind], nullptr, p, c, "upload_optimizer_state");
+}
+int myea_hip_download_optimizer_state(myea_hip_net *n, int kind, float *p, size_t c)
+{
+    NET_OR_FAIL(n);
+    if (kind < 0 || kind > 3 || !p) { myea::set_last_error("download_optimizer_state: bad kind %d or null", kind); return MYEA_E_INVALID; }
+    return copy_vec(n, n->net.opt[kind], p, nullptr, c, "download_optimizer_state");
+}
+int myea_hip_upload_masks(myea_hip_net *n, const uint8_t *m, size_t c)
+{
+    NET_OR_FAIL(n);
+    if (!m || c > n->net.d.total_mask_units) { myea::set_last_error("upload_masks: null or count %zu > %llu", c, (unsigned long long)n->net.d.total_mask_units); return MYEA_E_INVALID; }
+    MYEA_HIP_TRY(hipMemcpyAsync(n->net.masks, m, c, hipMemcpyHostToDevice, n->net.stream));
+    MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
+    return MYEA_OK;
+}
+int myea_hip_clear_training_arrays(myea_hip_net *n)
+{
+    NET_OR_FAIL(n);
+    const size_t bytes = n->net.d.total_parameters * sizeof(float);
+    MYEA_HIP_TRY(hipMemsetAsync(n->net.gradient, 0, bytes, n->net.stream));
+    for (int k = 0; k < 4; ++k) MYEA_HIP_TRY(hipMemsetAsync(n->net.opt[k], 0, bytes, n->net.stream));
+    n->net.h.optimizer_time_step = 0.f;
+    return MYEA_OK;
+}
+
+int myea_hip_forward_pass(myea_hip_net *n, size_t B, const float *x, int dev) { NET_OR_FAIL(n); return n->net.forward_pass(B, x, dev); }
+int myea_hip_compute_error(myea_hip_net *n, size_t B, const float *y, int dev) { NET_OR_FAIL(n); return n->net.compute_error(B, y, dev); }
+int myea_hip_backward_pass(myea_hip_net *n, size_t B) { NET_OR_FAIL(n); return n->net.backward_pass(B); }
+int myea_hip_update_derivative_weight(myea_hip_net *n, size_t B, size_t first, size_t end) { NET_OR_FAIL(n); return n->net.update_derivative_weight(B, first, end); }
+int myea_hip_update_parameter(myea_hip_net *n, size_t B, size_t ts) { NET_OR_FAIL(n); return n->net.update_parameter(B, ts); }
+
+int myea_hip_reset_loss(myea_hip_net *n)
+{
+    NET_OR_FAIL(n);
+    MYEA_HIP_TRY(hipMemsetAsync(n->net.loss_acc, 0, 4 * sizeof(double), n->net.stream));
+    return MYEA_OK;
+}
+int myea_hip_get_loss(myea_hip_net *n, myea_loss_state *s)
+{
+    NET_OR_FAIL(n);
+    if (!s) { myea::set_last_error("get_loss: null"); return MYEA_E_INVALID; }
+    double v[4];
+    MYEA_HIP_TRY(hipMemcpyAsync(v, n->net.loss_acc, sizeof(v), hipMemcpyDeviceToHost, n->net.stream));
+    MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
+    s->loss_values = v[0]; s->number_loss = (uint64_t)v[1]; s->accuracy_value = v[2]; s->number_bit_fail = (uint64_t)v[3];
+    return MYEA_OK;
+}
+
+int myea_hip_download_gradient(myea_hip_net *n, float *g, size_t c)
+{
+    NET_OR_FAIL(n);
+    if (!g) { myea::set_last_error("download_gradient: null"); return MYEA_E_INVALID; }
+    return copy_vec(n, n->net.gradient, g, nullptr, c, "download_gradient");
+}
+int myea_hip_upload_gradient(myea_hip_net *n, const float *g, size_t c)
+{
+    NET_OR_FAIL(n);
+    if (!g) { myea::set_last_error("upload_gradient: null"); return MYEA_E_INVALID; }
+    return copy_vec(n, n->net.gradient, nullptr, g, c, "upload_gradient");
+}
+
+int myea_hip_download_tensor(myea_hip_net *n, size_t li, int kind, float *host, size_t count)
+{
+    NET_OR_FAIL(n);
+    if (!host || li >= n->net.d.n_layers) { myea::set_last_error("download_tensor: null or layer %zu out of range", li); return MYEA_E_INVALID; }
+    myea::DevLayer &o = n->net.L[li];
+    const size_t T = n->net.d.number_recurrent_depth, full = T * n->net.d.batch_size * o.H, th = T * o.H;
+    const float *p = nullptr;
+    size_t c = full;
+    switch (kind) {
+    case MYEA_TENSOR_OUTPUTS: p = n->net.layer_outputs(li); break;
+    case MYEA_TENSOR_SUMMATIONS: p = o.summations; break;
+    case MYEA_TENSOR_ERRORS: p = o.neuron_errors; break;
+    case MYEA_TENSOR_NORM_HATS: p = o.hats; break;
+    case MYEA_TENSOR_NORM_MEANS: p = o.means; c = th; break;
+    case MYEA_TENSOR_NORM_VARIANCES: p = o.variances; c = th; break;
+    case MYEA_TENSOR_NORM_MEANS_AVERAGES: p = o.means_averages; c = th; break;
+    case MYEA_TENSOR_NORM_VARIANCES_AVERAGES: p = o.variances_averages; c = th; break;
+    default: p = n->net.lstm_tensor(li, kind, &c); break;
+    }
+    if (!p) { myea::set_last_error("download_tensor: layer %zu has no tensor of kind %d", li, kind); return MYEA_E_INVALID; }
+    if (count > c) { myea::set_last_error("download_tensor: count %zu > tensor length %zu", count, c); return MYEA_E_INVALID; }
+    MYEA_HIP_TRY(hipMemcpyAsync(host, p, count * sizeof(float), hipMemcpyDeviceToHost, n->net.stream));
+    MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
+    return MYEA_OK;
+}
+
+int myea_hip_profile_enable(myea_hip_net *n, int enable)
+{
+    NET_OR_FAIL(n);
+    n->net.profiling = enable != 0;
+    return MYEA_OK;
+}
+
+int myea_hip_profile_read(myea_hip_net *n, int family, uint64_t *launches, double *ms, double *work)
+{
+    NET_OR_FAIL(n);
+    if (family < 0 || family >= myea::kProfFamilies) { myea::set_last_error("profile_read: family %d", family); return MYEA_E_INVALID; }
+    MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
+    for (myea::ProfEvent &e : n->net.pending) {
+        float t = 0.f;
+        if (hipEventElapsedTime(&t, e.start, e.stop) == hipSuccess) {
+            n->net.prof_ms[e.family] += t;
+            n->net.prof_work[e.family] += e.work;
+            n->net.prof_launches[e.family] += 1;
+        }
+        n->net.free_events.push_back(e);
+    }
+    n->net.pending.clear();
+    if (launches) *launches = n->net.prof_launches[family];
+    if (ms) *ms = n->net.prof_ms[family];
+    if (work) *work = n->net.prof_work[family];
+    n->net.prof_launches[family] = 0; n->net.prof_ms[family] = 0; n->net.prof_work[family] = 0;
+    return MYEA_OK;
+}
+
+int myea_hip_optimizer_update(void *stream, const myea_hyper *h, size_t count, size_t weight_count, float gradient_scale,
+                              float *parameters, float *gradient, float *state0, float *state1, float *state2)
+{
+    if (!h || !parameters || !gradient) { myea::set_last_error("optimizer_update: null argument"); return MYEA_E_INVALID; }
+    myea::UpdateParams p{};
+    p.optimizer = (int)h->type_optimizer_function;
+    p.n = count; p.n_weights = weight_count;
+    p.w = parameters; p.g = gradient; p.s0 = state0; p.s1 = state1; p.s2 = state2;
+    p.grad_scale = gradient_scale;
+    p.wd = h->regularization__weight_decay;
+    const float ts = h->optimizer_time_step;
+    p.lr = h->learning_rate; p.mu = h->learning_momentum;
+    p.variant = h->learning_momentum != 0.f ? (h->use_Nesterov ? 2 : 1) : 0;
+    p.beta1 = h->adam_beta1; p.beta2 = h->adam_beta2; p.eps = h->adam_epsilon;
+    p.lr_t = h->use_adam_bias_correction
+                 ? (float)(h->adam_learning_rate * std::sqrt(1.0 - std::pow((double)h->adam_beta2, (double)ts)) / (1.0 - std::pow((double)h->adam_beta1, (double)ts)))
+                 : h->adam_learning_rate;
+    p.lower = h->learning_rate_final * (1.f - 1.f / (h->learning_gamma * ts + 1.f));
+    p.upper = h->learning_rate_final * (1.f + 1.f / (h->learning_gamma * ts));
+    return myea::launch_update(static_cast<hipStream_t>(stream), p);
+}
+
+}  // extern "C"

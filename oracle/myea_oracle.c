@@ -1,0 +1,812 @@
+/* myea_oracle.c — CPU restatement of the reference's training step.  TEST INFRASTRUCTURE ONLY:
+ * only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load this.
+ *
+ * Each function follows the reference file:line named above it.  Abbreviations:
+ *   NN/  = Neural_Network_Library_Windows/Source_Files/Neural_Network/
+ *   NNH/ = Neural_Network_Library_Windows/Header_Files/Neural_Network/
+ *
+ * The reference itself cannot be built in this image (every translation unit includes
+ * Header_Files/stdafx.hpp -> <Eigen/QR>, Configuration.hpp -> <boost/assert.hpp>,
+ * Dataset_Manager.hpp -> <systemd/sd-bus.h>; none of the three is installed or vendored), and it
+ * ships no tests, golden vectors or fixtures.  This restatement is therefore pinned by what the
+ * mathematics fixes — see tests/test_oracle_*.py: automatic differentiation of an independent
+ * float64 forward model, closed forms, brute force on tiny shapes and invariants.
+ * Parts of the behaviour that are reference quirks rather than mathematics (listed at each
+ * function) are pinned only by reading: "parity unpinned" for
+ *   - the LSTM bias index overrun (Prepare__Bias__LSTM),
+ *   - the RNN head `pre` pointer quirk (RNN__Compute__Error).
+ *
+ * Summation order is the serial order of the reference's __Loop variants; the __OpenMP variants
+ * differ only in the order of the per-thread partial sums.
+ */
+#include "myea_oracle.h"
+
+#include <float.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+typedef struct olayer {
+    size_t H;            /* *ptr_number_outputs */
+    size_t norm_units;   /* number of Normalized_unit owned by the layer */
+    /* [T][Bmax][H] */
+    float *summations, *values, *hats, *normalizes;
+    float *neuron_errors, *af_errors, *norm_errors;
+    /* [T][H] */
+    float *means, *variances, *means_averages, *variances_averages, *r_corrections, *d_corrections;
+    float *derivatives_means, *derivatives_variances;
+    /* LSTM, [T][Bmax][C] or [T][Bmax][K] per direction d (index d*...) */
+    struct olstm *lstm;
+} olayer;
+
+struct myea_oracle_net {
+    myea_net_desc d;
+    myea_hyper h;
+    uint32_t state;
+    int threads;
+    float *parameters, *gradient, *opt[4];
+    uint8_t *masks;
+    olayer L[MYEA_MAX_LAYERS];
+    myea_loss_state loss;
+};
+
+/* ------------------------------------------------------------------------------------------- */
+/* activation functions: NNH/Activation_Functions.hpp:17-184 (AF_FIRE; forward ignores steepness) */
+
+static float af_linear_seg(float v1, float r1, float v2, float r2, float s) { return (((r2 - r1) * (s - v1)) / (v2 - v1)) + r1; }
+
+static float af_stepwise(float v1, float v2, float v3, float v4, float v5, float v6,
+                         float r1, float r2, float r3, float r4, float r5, float r6,
+                         float mn, float mx, float s)
+{
+    return s < v5 ? (s < v3 ? (s < v2 ? (s < v1 ? mn : af_linear_seg(v1, r1, v2, r2, s)) : af_linear_seg(v2, r2, v3, r3, s))
+                            : (s < v4 ? af_linear_seg(v3, r3, v4, r4, s) : af_linear_seg(v4, r4, v5, r5, s)))
+                  : (s < v6 ? af_linear_seg(v5, r5, v6, r6, s) : mx);
+}
+
+#define SELU_ALPHA 1.6732632423543772848170429916717f
+#define SELU_SCALE 1.0507009873554804934193349852946f
+
+float myea_oracle_activation(uint32_t type, float s)
+{
+    switch (type) {
+    case MYEA_AF_LINEAR: return s;
+    case MYEA_AF_LINEAR_PIECE: return s < 0.f ? 0.f : (s > 1.f ? 1.f : s);
+    case MYEA_AF_LINEAR_PIECE_SYMMETRIC: return s < -1.f ? -1.f : (s > 1.f ? 1.f : s);
+    case MYEA_AF_SIGMOID: return 1.f / (1.f + expf(-s));                      /* AF_SIGMOID_real */
+    case MYEA_AF_TANH: return 2.f / (1.f + expf(-2.f * s)) - 1.f;             /* AF_TANH_real (not tanhf) */
+    case MYEA_AF_SIGMOID_STEPWISE:
+        return af_stepwise(-2.64665246009826660156f, -1.47221946716308593750f, -5.49306154251098632812e-01f,
+                           5.49306154251098632812e-01f, 1.47221934795379638672f, 2.64665293693542480469f,
+                           4.99999988824129104614e-03f, 5.00000007450580596924e-02f, 2.5e-01f, 7.5e-01f,
+                           9.49999988079071044922e-01f, 9.95000004768371582031e-01f, 0.f, 1.f, s);
+    case MYEA_AF_TANH_STEPWISE:
+        return af_stepwise(-2.64665293693542480469f, -1.47221934795379638672f, -5.49306154251098632812e-01f,
+                           5.49306154251098632812e-01f, 1.47221934795379638672f, 2.64665293693542480469f,
+                           -9.90000009536743164062e-01f, -8.99999976158142089844e-01f, -5.0e-01f, 5.0e-01f,
+                           8.99999976158142089844e-01f, 9.90000009536743164062e-01f, -1.f, 1.f, s);
+    case MYEA_AF_THRESHOLD: return s < 0.f ? 0.f : 1.f;
+    case MYEA_AF_THRESHOLD_SYMMETRIC: return s < 0.f ? -1.f : 1.f;
+    case MYEA_AF_GAUSSIAN: return expf(-s * s);
+    case MYEA_AF_GAUSSIAN_SYMMETRIC: return expf(-s * s) * 2.f - 1.f;
+    case MYEA_AF_GAUSSIAN_STEPWISE: return 0.f;
+    case MYEA_AF_ELLIOT: return (s / 2.f) / (1.f + fabsf(s)) + 0.5f;
+    case MYEA_AF_ELLIOT_SYMMETRIC: return s / (1.f + fabsf(s));
+    case MYEA_AF_SINE: return sinf(s) / 2.f + 0.5f;
+    case MYEA_AF_SINE_SYMMETRIC: return sinf(s);
+    case MYEA_AF_COSINE: return cosf(s) / 2.f + 0.5f;
+    case MYEA_AF_COSINE_SYMMETRIC: return cosf(s);
+    case MYEA_AF_ISRU: return s * (1.f / sqrtf(1.f + 1.f * s * s));
+    case MYEA_AF_ISRLU: return s < 0.f ? s * (1.f / sqrtf(1.f + 1.f * s * s)) : s;
+    case MYEA_AF_ELU: return s < 0.f ? 1.f * (expf(s) - 1.f) : s;
+    case MYEA_AF_SELU: return SELU_SCALE * (s <= 0.f ? SELU_ALPHA * expf(s) - SELU_ALPHA : s);
+    case MYEA_AF_RELU: return s < 0.f ? 0.f : s;
+    case MYEA_AF_LEAKY_RELU: return s < 0.f ? 0.01f * s : s;
+    case MYEA_AF_PARAMETRIC_RELU: return s < 0.f ? 0.01f * s : s;
+    case MYEA_AF_SOFTMAX: return expf(s);
+    default: return s; /* AF_FIRE default: leaves the value untouched */
+    }
+}
+
+/* Activation_Function_Derive: NN/Neural_Network.cpp:3157-3201 + the *_derive macros. */
+float myea_oracle_activation_derive(uint32_t type, float q, float st, float v)
+{
+    switch (type) {
+    case MYEA_AF_COSINE: return st * -sinf(st * q) / 2.f;
+    case MYEA_AF_COSINE_SYMMETRIC: return st * -sinf(st * q);
+    case MYEA_AF_ELU: return q < 0.f ? st * 1.f * v : st;
+    case MYEA_AF_ELLIOT: return st * 1.f / (2.f * (1.f + fabsf(q)) * (1.f + fabsf(q)));
+    case MYEA_AF_ELLIOT_SYMMETRIC: return st * 1.f / ((1.f + fabsf(q)) * (1.f + fabsf(q)));
+    case MYEA_AF_GAUSSIAN: return -2.f * q * v * st * st;
+    case MYEA_AF_GAUSSIAN_SYMMETRIC: return -2.f * q * (v + 1.f) * st * st;
+    case MYEA_AF_ISRU: { float r = v / q; return st * (r * r * r); }
+    case MYEA_AF_ISRLU: { float r = v / q; return q < 0.f ? st * (r * r * r) : st; }
+    case MYEA_AF_LINEAR:
+    case MYEA_AF_LINEAR_PIECE:
+    case MYEA_AF_LINEAR_PIECE_SYMMETRIC: return st;
+    case MYEA_AF_LEAKY_RELU: return q < 0.f ? st * 0.01f : st;
+    case MYEA_AF_PARAMETRIC_RELU: return q < 0.f ? st * 0.01f : st;
+    case MYEA_AF_RELU: return q < 0.f ? 0.f : st;          /* 1 at q == 0 */
+    case MYEA_AF_SELU: return SELU_SCALE * (q <= 0.f ? st * (v + SELU_ALPHA) : st);
+    case MYEA_AF_SIGMOID:
+    case MYEA_AF_SIGMOID_STEPWISE: return st * v * (1.f - v);
+    case MYEA_AF_SINE: return st * cosf(st * q) / 2.f;
+    case MYEA_AF_SINE_SYMMETRIC: return st * cosf(st * q);
+    case MYEA_AF_TANH:
+    case MYEA_AF_TANH_STEPWISE: return st * (1.f - v * v);
+    case MYEA_AF_SOFTMAX: return st;                       /* cross-entropy shortcut */
+    default: return v;
+    }
+}
+
+/* ------------------------------------------------------------------------------------------- */
+/* helpers */
+
+static int layer_uses_norm(const myea_layer_desc *l) { return l->type_normalization != MYEA_NORMALIZATION_NONE; }
+static int layer_uses_bias(const myea_layer_desc *l) { return !layer_uses_norm(l); } /* NNH/Data.hpp:736 */
+
+static float *zalloc(size_t n) { return (float *)calloc(n ? n : 1, sizeof(float)); }
+
+/* Layer::ptr_array_outputs, NN/Neural_Network__Ordered.cpp:78-389 (non-residual group). */
+static float *layer_outputs(myea_oracle_net *n, size_t li)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    if (li == 0) return o->values;
+    if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (layer_uses_norm(l) && !l->use_layer_normalization_before_activation) return o->normalizes;
+        return o->values;
+    }
+    return o->values; /* LSTM: cell outputs live in values */
+}
+
+/* Layer::ptr_array_derivative_outputs */
+static float *layer_derivative_outputs(myea_oracle_net *n, size_t li)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (layer_uses_norm(l) && !l->use_layer_normalization_before_activation) return o->norm_errors;
+        return o->af_errors;
+    }
+    return o->af_errors; /* LSTM: ptr_delta_cell_output */
+}
+
+static float *scale_ptr(myea_oracle_net *n, float *base, size_t li)
+{
+    return base + n->d.total_weights + n->d.total_bias + n->d.layers[li].first_normalized_unit_index;
+}
+static float *shift_ptr(myea_oracle_net *n, float *base, size_t li)
+{
+    return scale_ptr(n, base, li) + n->d.total_normalized_units;
+}
+
+/* ------------------------------------------------------------------------------------------- */
+/* life cycle */
+
+static size_t layer_width(const myea_layer_desc *l)
+{
+    if (l->type_layer == MYEA_LAYER_LSTM) return (size_t)l->n_units * l->n_cells_per_block;
+    return l->n_units;
+}
+
+int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
+{
+    if (!desc || !out || desc->n_layers < 2 || desc->n_layers > MYEA_MAX_LAYERS) return MYEA_E_INVALID;
+    myea_oracle_net *n = (myea_oracle_net *)calloc(1, sizeof(*n));
+    if (!n) return MYEA_E_NOMEM;
+    n->d = *desc;
+    myea_hyper_default(&n->h);
+    n->threads = 1;
+    size_t P = desc->total_parameters, T = desc->number_recurrent_depth, B = desc->batch_size;
+    n->parameters = zalloc(P);
+    n->gradient = zalloc(P);
+    for (int k = 0; k < 4; ++k) n->opt[k] = zalloc(P);
+    n->masks = (uint8_t *)malloc(desc->total_mask_units ? desc->total_mask_units : 1);
+    memset(n->masks, 1, desc->total_mask_units ? desc->total_mask_units : 1); /* NN/Neural_Network__Allocate.cpp:386-410: all true */
+    /* scales start at 1, shifts at 0 (NN/Neural_Network__Allocate.cpp:2395-2401 and the scale fill) */
+    for (size_t i = 0; i < desc->total_normalized_units; ++i) n->parameters[desc->total_weights + desc->total_bias + i] = 1.f;
+    for (size_t li = 0; li < desc->n_layers; ++li) {
+        const myea_layer_desc *l = &desc->layers[li];
+        olayer *o = &n->L[li];
+        o->H = layer_width(l);
+        if (l->type_layer == MYEA_LAYER_RESIDUAL || l->type_layer == MYEA_LAYER_LSTM) { free(n); return MYEA_E_UNSUPPORTED; }
+        size_t sz = T * B * o->H;
+        o->values = zalloc(sz);
+        if (li == 0) continue;
+        o->summations = zalloc(sz);
+        o->neuron_errors = zalloc(sz);
+        o->af_errors = zalloc(sz);
+        if (layer_uses_norm(l)) {
+            o->hats = zalloc(sz);
+            o->normalizes = zalloc(sz);
+            o->norm_errors = zalloc(sz);
+            o->means = zalloc(T * o->H);
+            o->variances = zalloc(T * o->H);
+            o->means_averages = zalloc(T * o->H);
+            o->variances_averages = zalloc(T * o->H);
+            for (size_t i = 0; i < T * o->H; ++i) o->variances_averages[i] = 1.f; /* NN/Neural_Network__Allocate.cpp:2612-2615 */
+            o->r_corrections = zalloc(T * o->H);
+            o->d_corrections = zalloc(T * o->H);
+            o->derivatives_means = zalloc(T * o->H);
+            o->derivatives_variances = zalloc(T * o->H);
+        }
+    }
+    *out = n;
+    return MYEA_OK;
+}
+
+int myea_oracle_destroy(myea_oracle_net *n)
+{
+    if (!n) return MYEA_OK;
+    free(n->parameters); free(n->gradient);
+    for (int k = 0; k < 4; ++k) free(n->opt[k]);
+    free(n->masks);
+    for (size_t li = 0; li < n->d.n_layers; ++li) {
+        olayer *o = &n->L[li];
+        free(o->summations); free(o->values); free(o->hats); free(o->normalizes);
+        free(o->neuron_errors); free(o->af_errors); free(o->norm_errors);
+        free(o->means); free(o->variances); free(o->means_averages); free(o->variances_averages);
+        free(o->r_corrections); free(o->d_corrections); free(o->derivatives_means); free(o->derivatives_variances);
+    }
+    free(n);
+    return MYEA_OK;
+}
+
+int myea_oracle_set_hyper(myea_oracle_net *n, const myea_hyper *h) { if (!n || !h) return MYEA_E_INVALID; n->h = *h; return MYEA_OK; }
+int myea_oracle_get_hyper(myea_oracle_net *n, myea_hyper *h) { if (!n || !h) return MYEA_E_INVALID; *h = n->h; return MYEA_OK; }
+int myea_oracle_set_state_propagation(myea_oracle_net *n, uint32_t s) { if (!n) return MYEA_E_INVALID; n->state = s; return MYEA_OK; }
+int myea_oracle_set_threads(myea_oracle_net *n, int t) { if (!n || t < 1) return MYEA_E_INVALID; n->threads = t; return MYEA_OK; }
+float *myea_oracle_parameters(myea_oracle_net *n) { return n->parameters; }
+float *myea_oracle_gradient(myea_oracle_net *n) { return n->gradient; }
+float *myea_oracle_optimizer_state(myea_oracle_net *n, int k) { return (k >= 0 && k < 4) ? n->opt[k] : NULL; }
+uint8_t *myea_oracle_masks(myea_oracle_net *n) { return n->masks; }
+
+/* Clear_Training_Arrays NN/Train.cpp:93-126, Clear_Optimizer NN/Train.cpp:128-263 */
+int myea_oracle_clear_training_arrays(myea_oracle_net *n)
+{
+    size_t P = n->d.total_parameters;
+    memset(n->gradient, 0, P * sizeof(float));
+    for (int k = 0; k < 4; ++k) memset(n->opt[k], 0, P * sizeof(float));
+    n->h.optimizer_time_step = 0.f;
+    return MYEA_OK;
+}
+
+/* ------------------------------------------------------------------------------------------- */
+/* forward pieces */
+
+/* Forward_Pass__FC: NN/Neural_Network__Forward_Pass__OpenMP.cpp:4517-4557 */
+static void fwd_fc(myea_oracle_net *n, size_t t, size_t B, size_t In, size_t Out, const float *x, const float *w, float *y)
+{
+    size_t Bmax = n->d.batch_size;
+    const float *xt = x + Bmax * In * t;
+    float *yt = y + Bmax * Out * t;
+    long b;
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+    for (b = 0; b < (long)B; ++b) {
+        const float *xi = xt + (size_t)b * In;
+        float *yo = yt + (size_t)b * Out;
+        for (size_t o = 0; o < Out; ++o) {
+            const float *wr = w + o * In;
+            float s = 0.f;
+            for (size_t i = 0; i < In; ++i) s += xi[i] * wr[i];
+            yo[o] = s;
+        }
+    }
+}
+
+/* Forward_Pass__Bias: NN/Neural_Network__Forward_Pass__OpenMP.cpp:4494-4515 */
+static void fwd_bias(myea_oracle_net *n, size_t t, size_t B, size_t Out, const float *bias, float *y)
+{
+    float *yt = y + n->d.batch_size * Out * t;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t o = 0; o < Out; ++o) yt[b * Out + o] += bias[o];
+}
+
+/* Forward_Pass__Batch_Normalization__Training: NN/Neural_Network__Forward_Pass__OpenMP.cpp:4591-4701
+ * Forward_Pass__Batch_Renormalization__Training: :4703-4837.
+ * `variances` receives sqrt(var + eps) (:4675). */
+static void fwd_bn_training(myea_oracle_net *n, int renorm, size_t t, size_t B, size_t H, const float *x,
+                            const float *scale, const float *shift, olayer *o)
+{
+    size_t Bmax = n->d.batch_size;
+    const float *xt = x + Bmax * H * t;
+    float *mean = o->means + t * H, *var = o->variances + t * H;
+    float *mavg = o->means_averages + t * H, *vavg = o->variances_averages + t * H;
+    float *rc = o->r_corrections + t * H, *dc = o->d_corrections + t * H;
+    float *hat = o->hats + Bmax * H * t, *nor = o->normalizes + Bmax * H * t;
+    float bscale = 1.f / (float)B, eps = n->h.normalization_epsilon, mom = n->h.normalization_momentum_average;
+    float rmax = n->h.batch_renormalization_r_correction_maximum, dmax = n->h.batch_renormalization_d_correction_maximum;
+    for (size_t j = 0; j < H; ++j) { mean[j] = 0.f; var[j] = 0.f; } /* MEMSET at the start of the pass, :54-66 */
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) { float s = xt[b * H + j]; mean[j] += s; var[j] += s * s; }
+    for (size_t j = 0; j < H; ++j) {
+        mean[j] *= bscale;
+        mavg[j] += mom * (mean[j] - mavg[j]);
+        var[j] = sqrtf(var[j] * bscale - mean[j] * mean[j] + eps);
+        vavg[j] += mom * (var[j] - vavg[j]);
+        if (renorm) {
+            float g = var[j] / vavg[j], lo = 1.f / rmax;
+            rc[j] = g < lo ? lo : (g > rmax ? rmax : g);
+            float dd = (mean[j] - mavg[j]) / vavg[j];
+            dc[j] = dd < -dmax ? -dmax : (dd > dmax ? dmax : dd);
+        }
+    }
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            float s = xt[b * H + j];
+            if (renorm) s = (s - mean[j]) / var[j] * rc[j] + dc[j];
+            else s = (s - mean[j]) / var[j];
+            hat[b * H + j] = s;
+            nor[b * H + j] = scale[j] * s + shift[j];
+        }
+}
+
+/* Forward_Pass__Batch_Normalization__Inference: NN/Neural_Network__Forward_Pass__OpenMP.cpp:4559-4589 */
+static void fwd_bn_inference(myea_oracle_net *n, size_t t, size_t B, size_t H, const float *x, const float *scale, const float *shift, olayer *o)
+{
+    size_t Bmax = n->d.batch_size;
+    const float *xt = x + Bmax * H * t;
+    float *nor = o->normalizes + Bmax * H * t;
+    const float *mavg = o->means_averages + t * H, *vavg = o->variances_averages + t * H;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) nor[b * H + j] = scale[j] * ((xt[b * H + j] - mavg[j]) / vavg[j]) + shift[j];
+}
+
+/* Forward_Pass__FC_AF: :4839-4868; Forward_Pass__FC_AF__Softmax: :4870-4905 */
+static void fwd_af(myea_oracle_net *n, size_t t, size_t B, size_t H, uint32_t type, const float *x, float *y)
+{
+    size_t off = n->d.batch_size * H * t;
+    for (size_t b = 0; b < B; ++b) {
+        const float *xi = x + off + b * H;
+        float *yo = y + off + b * H;
+        if (type == MYEA_AF_SOFTMAX) {
+            float mx = -FLT_MAX, sum = 0.f;
+            for (size_t j = 0; j < H; ++j) mx = mx > xi[j] ? mx : xi[j];
+            for (size_t j = 0; j < H; ++j) sum += yo[j] = expf(xi[j] - mx);
+            sum = 1.f / sum;
+            for (size_t j = 0; j < H; ++j) yo[j] *= sum;
+        } else {
+            for (size_t j = 0; j < H; ++j) yo[j] = myea_oracle_activation(type, xi[j]);
+        }
+    }
+}
+
+/* Forward_Pass__Dropout__Bernoulli__{Training,Inverted,Inference}: :4907-4990.
+ * mask is per (t, unit), shared by every example. */
+static void fwd_dropout(myea_oracle_net *n, const myea_layer_desc *l, size_t t, size_t B, size_t H, float *v)
+{
+    size_t off = n->d.batch_size * H * t;
+    const uint8_t *m = n->masks + l->first_mask_index + t * H;
+    if (n->state == MYEA_STATE_TRAINING) {
+        if (l->type_dropout == MYEA_DROPOUT_BERNOULLI) {
+            for (size_t b = 0; b < B; ++b)
+                for (size_t j = 0; j < H; ++j) if (!m[j]) v[off + b * H + j] = 0.f;
+        } else if (l->type_dropout == MYEA_DROPOUT_BERNOULLI_INVERTED) {
+            float inv = l->dropout_values[0] == 0.f ? 0.f : 1.f / l->dropout_values[0];
+            for (size_t b = 0; b < B; ++b)
+                for (size_t j = 0; j < H; ++j) { if (m[j]) v[off + b * H + j] *= inv; else v[off + b * H + j] = 0.f; }
+        }
+    } else if (l->type_dropout == MYEA_DROPOUT_BERNOULLI) {
+        for (size_t b = 0; b < B; ++b)
+            for (size_t j = 0; j < H; ++j) v[off + b * H + j] *= l->dropout_values[0];
+    }
+}
+
+/* Forward_Pass__FC (layer driver): NN/Neural_Network__Forward_Pass__OpenMP.cpp:256-698.
+ * order: GEMM -> bias -> [BN before] -> activation / softmax -> [BN after] -> dropout. */
+static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    size_t In = n->L[li - 1].H, H = o->H;
+    const float *x = layer_outputs(n, li - 1);
+    int training = n->state >= MYEA_STATE_TRAINING;
+    int renorm = l->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    fwd_fc(n, t, B, In, H, x, n->parameters + l->first_connection_index, o->summations);
+    if (layer_uses_bias(l)) fwd_bias(n, t, B, H, n->parameters + l->first_bias_connection_index, o->summations);
+    const float *cur = o->summations;
+    if (layer_uses_norm(l) && l->use_layer_normalization_before_activation) {
+        if (training) fwd_bn_training(n, renorm, t, B, H, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
+        else fwd_bn_inference(n, t, B, H, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
+        cur = o->normalizes;
+    }
+    fwd_af(n, t, B, H, l->type_activation_function, cur, o->values);
+    float *out = o->values;
+    if (layer_uses_norm(l) && !l->use_layer_normalization_before_activation) {
+        if (training) fwd_bn_training(n, renorm, t, B, H, o->values, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
+        else fwd_bn_inference(n, t, B, H, o->values, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
+        out = o->normalizes;
+    }
+    fwd_dropout(n, l, t, B, H, out);
+}
+
+/* FF__Forward_Pass_Batch: NN/Neural_Network__Forward_Pass__OpenMP.cpp:24-120;
+ * RNN__Forward_Pass_Batch: NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:24-130 (layer-major,
+ * every layer loops over t); FF/RNN__Assign_Inputs: NN/Neural_Network__Assign_Inputs.cpp:20-204
+ * (example rows are [T][In]; scattered into [T][Bmax][In]; input-layer dropout applied in place). */
+int myea_oracle_forward_pass(myea_oracle_net *n, size_t B, const float *inputs)
+{
+    if (!n || !inputs) return MYEA_E_INVALID;
+    size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, In = n->L[0].H;
+    if (B > Bmax) return MYEA_E_BATCH;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t t = 0; t < T; ++t)
+            memcpy(n->L[0].values + Bmax * In * t + b * In, inputs + b * T * In + t * In, In * sizeof(float));
+    for (size_t t = 0; t < T; ++t) fwd_dropout(n, &n->d.layers[0], t, B, In, n->L[0].values);
+    for (size_t li = 1; li < n->d.n_layers; ++li) {
+        const myea_layer_desc *l = &n->d.layers[li];
+        if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+            for (size_t t = 0; t < T; ++t) fwd_fc_layer(n, li, t, B);
+        } else return MYEA_E_UNSUPPORTED;
+    }
+    return MYEA_OK;
+}
+
+/* ------------------------------------------------------------------------------------------- */
+/* Compute__Error */
+
+/* Update_Error: NN/Neural_Network__Compute__Error__Loop.cpp:20-77 */
+static void update_error(myea_oracle_net *n, float observed, float desired, float error)
+{
+    float e;
+    switch (n->h.type_loss_function) {
+    case MYEA_LOSS_ME:
+    case MYEA_LOSS_L1: e = error; break;
+    case MYEA_LOSS_MAE: e = fabsf(error); break;
+    case MYEA_LOSS_L2:
+    case MYEA_LOSS_MSE:
+    case MYEA_LOSS_RMSE: e = error * error; break;
+    case MYEA_LOSS_MAPE:
+        e = observed != 0.f ? observed : (observed > 1e-6f ? observed : 1e-6f);
+        e = fabsf(error / e);
+        break;
+    case MYEA_LOSS_SMAPE: e = fabsf(error) / (fabsf(desired) + fabsf(observed)); break;
+    case MYEA_LOSS_CROSS_ENTROPY: {
+        size_t n_out = n->L[n->d.n_layers - 1].H;
+        e = observed != 0.f ? observed : (observed > 1e-6f ? observed : 1e-6f);
+        if (n_out == 1) e = -(desired * logf(e) + (1.f - desired) * logf(1.f - e));
+        else e = -(desired * logf(e));
+        break;
+    }
+    case MYEA_LOSS_BIT:
+        if (fabsf(error) >= n->h.bit_fail_limit) ++n->loss.number_bit_fail;
+        return;
+    default: return;
+    }
+    n->loss.loss_values += e;
+    ++n->loss.number_loss;
+}
+
+static float sign_f(float v) { return v > 0.f ? 1.f : (v < 0.f ? -1.f : 0.f); }
+
+/* FF__Compute__Error: NN/Neural_Network__Compute__Error__OpenMP.cpp:22-141.
+ * RNN__Compute__Error: NN/Neural_Network__Recurrent_Compute__Error__OpenMP.cpp:22-159 — same per
+ * t >= number_time_delays; its per-unit loop does not advance the pre-activation pointer (:97-99),
+ * so every unit of an example sees the first unit's pre-activation.  Only activations whose derivative
+ * ignores the pre-activation (linear, tanh, sigmoid, softmax) are unaffected; this restatement
+ * reproduces the quirk.
+ * delta = Activation_Function_Derive(type, pre, steepness, y) * (y - desired); no 1/B, no factor 2. */
+int myea_oracle_compute_error(myea_oracle_net *n, size_t B, const float *desired)
+{
+    if (!n || !desired) return MYEA_E_INVALID;
+    size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth;
+    if (B > Bmax) return MYEA_E_BATCH;
+    size_t lo = n->d.n_layers - 1;
+    const myea_layer_desc *l = &n->d.layers[lo];
+    olayer *o = &n->L[lo];
+    size_t H = o->H;
+    const float *pre_af = (layer_uses_norm(l) && l->use_layer_normalization_before_activation) ? o->normalizes : o->summations;
+    int rnn = T > 1;
+    for (size_t t = rnn ? n->h.number_time_delays : 0; t < T; ++t) {
+        size_t off = Bmax * H * t;
+        for (size_t b = 0; b < B; ++b) {
+            const float *y = o->values + off + b * H;
+            const float *d = desired + b * T * H + t * H;
+            const float *pre = pre_af + off + b * H;
+            float *err = o->af_errors + off + b * H;
+            if (n->h.type_accuracy_function == MYEA_ACCURACY_CROSS_ENTROPY) {
+                size_t want = 0, got = 0;
+                for (want = 0; want < H; ++want) if (d[want] == 1.f) break;
+                float mx = -FLT_MAX;
+                for (size_t j = 0; j < H; ++j) if (y[j] >= mx) { got = j; mx = y[j]; }
+                n->loss.accuracy_value += (double)(want == got);
+            }
+            for (size_t j = 0; j < H; ++j) {
+                float diff = y[j] - d[j];
+                update_error(n, y[j], d[j], diff);
+                switch (n->h.type_accuracy_function) {
+                case MYEA_ACCURACY_DISTANCE: if (fabsf(diff) <= n->h.accuracy_variance) n->loss.accuracy_value += 1.0; break;
+                case MYEA_ACCURACY_DIRECTIONAL: n->loss.accuracy_value += 1.0; break;
+                case MYEA_ACCURACY_SIGN:
+                    if (sign_f(d[j]) == sign_f(y[j]) || (sign_f(d[j]) == 0.f && y[j] >= -FLT_EPSILON && y[j] <= FLT_EPSILON)) n->loss.accuracy_value += 1.0;
+                    break;
+                default: break;
+                }
+                float q = rnn ? pre[0] : pre[j];
+                err[j] = myea_oracle_activation_derive(l->type_activation_function, q, l->activation_steepness, y[j]) * diff;
+            }
+        }
+    }
+    /* MEMCPY AF errors -> neuron errors over batch_size * T * H (:136-139) */
+    memcpy(o->neuron_errors, o->af_errors, T * Bmax * H * sizeof(float));
+    return MYEA_OK;
+}
+
+/* ------------------------------------------------------------------------------------------- */
+/* backward pieces */
+
+/* Backward_Pass__FC (7-arg): NN/Neural_Network__Backward_Pass__OpenMP.cpp:1044-1082.
+ * dst[b][i] += sum_o delta[b][o] * W[o][i]; dst is pre-zeroed by the driver. */
+static void bwd_fc(myea_oracle_net *n, size_t t, size_t B, size_t Out, size_t In, const float *delta, const float *w, float *dst)
+{
+    size_t Bmax = n->d.batch_size;
+    const float *dt = delta + Bmax * Out * t;
+    float *xt = dst + Bmax * In * t;
+    long b;
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+    for (b = 0; b < (long)B; ++b) {
+        const float *di = dt + (size_t)b * Out;
+        float *xo = xt + (size_t)b * In;
+        for (size_t o = 0; o < Out; ++o) {
+            float e = di[o];
+            const float *wr = w + o * In;
+            for (size_t i = 0; i < In; ++i) xo[i] += e * wr[i];
+        }
+    }
+}
+
+/* Backward_Pass__FC__DF: :1225-1263 */
+static void bwd_df(myea_oracle_net *n, size_t t, size_t B, size_t H, uint32_t type, float steep,
+                   const float *pre, const float *val, const float *dy, float *dx)
+{
+    size_t off = n->d.batch_size * H * t;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            size_t k = off + b * H + j;
+            dx[k] = dy[k] * myea_oracle_activation_derive(type, pre[k], steep, val[k]);
+        }
+}
+
+/* Backward_Pass__Batch_Normalization: :1346-1467; Backward_Pass__Batch_Renormalization: :1586-1709.
+ * dScale / dShift accumulate into the gradient vector at the scale / shift slots. */
+static void bwd_bn(myea_oracle_net *n, int renorm, size_t li, size_t t, size_t B, size_t H,
+                   const float *x, const float *dy, float *dx)
+{
+    olayer *o = &n->L[li];
+    size_t Bmax = n->d.batch_size, off = Bmax * H * t;
+    const float *mean = o->means + t * H, *var = o->variances + t * H, *rc = o->r_corrections + t * H;
+    const float *scale = scale_ptr(n, n->parameters, li);
+    float *dscale = scale_ptr(n, n->gradient, li), *dshift = shift_ptr(n, n->gradient, li);
+    float *dmean = o->derivatives_means + t * H, *dvar = o->derivatives_variances + t * H;
+    float bscale = 1.f / (float)B;
+    for (size_t j = 0; j < H; ++j) { dmean[j] = 0.f; dvar[j] = 0.f; } /* MEMSET at the start of the pass, :54-68 */
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            size_t k = off + b * H + j;
+            float e = dy[k], vb = var[j], r = renorm ? rc[j] : 1.f;
+            dscale[j] += e * o->hats[k];
+            dshift[j] += e;
+            e *= scale[j];
+            dmean[j] += e * (-r / vb);
+            dvar[j] += e * (x[k] - mean[j]) * (-r / (vb * vb));
+            dx[k] = e;
+        }
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            size_t k = off + b * H + j;
+            float e = dx[k], vb = var[j], r = renorm ? rc[j] : 1.f;
+            e *= r / vb;
+            e += dvar[j] * ((x[k] - mean[j]) / ((float)B * vb));
+            e += dmean[j] * bscale;
+            dx[k] = e;
+        }
+}
+
+/* Backward_Pass__Gradient__FC: :544-709 — [BN after] -> act' -> [BN before] -> copy to neuron errors */
+static void bwd_gradient_fc(myea_oracle_net *n, size_t li, size_t t, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    size_t H = o->H, Bmax = n->d.batch_size;
+    int renorm = l->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    int before = l->use_layer_normalization_before_activation;
+    const float *cur = layer_derivative_outputs(n, li);
+    if (layer_uses_norm(l) && !before) {
+        bwd_bn(n, renorm, li, t, B, H, o->values /* pre_normalization */, cur, o->norm_errors);
+        cur = o->norm_errors;
+    }
+    const float *pre_af = (layer_uses_norm(l) && before) ? o->normalizes : o->summations;
+    bwd_df(n, t, B, H, l->type_activation_function, l->activation_steepness, pre_af, o->values, cur, o->af_errors);
+    cur = o->af_errors;
+    if (layer_uses_norm(l) && before) {
+        bwd_bn(n, renorm, li, t, B, H, o->summations /* pre_normalization */, cur, o->norm_errors);
+        cur = o->norm_errors;
+    }
+    memcpy(o->neuron_errors + Bmax * H * t, cur + Bmax * H * t, Bmax * H * sizeof(float));
+}
+
+/* FF__Backward_Pass_Batch: NN/Neural_Network__Backward_Pass__OpenMP.cpp:24-155.
+ * RNN__Backward_Pass_Batch: NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:24-181 (FC
+ * consumers iterate t descending).  The input layer's delta is never computed. */
+int myea_oracle_backward_pass(myea_oracle_net *n, size_t B)
+{
+    if (!n) return MYEA_E_INVALID;
+    if (B > n->d.batch_size) return MYEA_E_BATCH;
+    if (n->state != MYEA_STATE_TRAINING) return MYEA_E_STATE;
+    size_t T = n->d.number_recurrent_depth, Bmax = n->d.batch_size;
+    for (size_t gi = n->d.n_layers - 1; gi >= 2; --gi) {
+        size_t li = gi - 1; /* previous_connected_layers[0] */
+        const myea_layer_desc *next = &n->d.layers[gi];
+        olayer *o = &n->L[li];
+        float *dst = layer_derivative_outputs(n, li);
+        memset(dst, 0, T * Bmax * o->H * sizeof(float));
+        if (next->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+            for (size_t tt = T; tt-- > 0;)
+                bwd_fc(n, tt, B, n->L[gi].H, o->H, n->L[gi].neuron_errors, n->parameters + next->first_connection_index, dst);
+        } else return MYEA_E_UNSUPPORTED;
+        if (n->d.layers[li].type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+            for (size_t tt = T; tt-- > 0;) bwd_gradient_fc(n, li, tt, B);
+        } else return MYEA_E_UNSUPPORTED;
+    }
+    return MYEA_OK;
+}
+
+/* ------------------------------------------------------------------------------------------- */
+/* Update_Derivative_Weight */
+
+/* Update_Derivative_Weight__FC (7-arg): NN/Neural_Network__Update_Derivative_Weight__OpenMP.cpp:178-216;
+ * Update_Derivative_Weight__Bias: :218-242.  dW += delta^T X; db += column sums. */
+static void dw_fc(myea_oracle_net *n, size_t t, size_t B, size_t In, size_t Out, const float *x, const float *delta, float *dw)
+{
+    size_t Bmax = n->d.batch_size;
+    const float *xt = x + Bmax * In * t, *dt = delta + Bmax * Out * t;
+    long o;
+    /* parallel over output rows: same per-element summation order as the serial loop */
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+    for (o = 0; o < (long)Out; ++o) {
+        float *row = dw + (size_t)o * In;
+        for (size_t b = 0; b < B; ++b) {
+            float e = dt[b * Out + (size_t)o];
+            const float *xi = xt + b * In;
+            for (size_t i = 0; i < In; ++i) row[i] += e * xi[i];
+        }
+    }
+}
+
+static void dw_bias(myea_oracle_net *n, size_t t, size_t B, size_t Out, const float *delta, float *db)
+{
+    const float *dt = delta + n->d.batch_size * Out * t;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t o = 0; o < Out; ++o) db[o] += dt[b * Out + o];
+}
+
+/* FF__Update_Derivative_Weight_Batch: :24-59; RNN variant:
+ * NN/Neural_Network__Recurrent_Update_Derivative_Weight__OpenMP.cpp:24-166 (per layer, t ascending).
+ * X is Layer::ptr_array_pre_summations = the previous layer's (post-dropout) outputs. */
+int myea_oracle_update_derivative_weight(myea_oracle_net *n, size_t B, size_t first, size_t end)
+{
+    if (!n || first < 1 || end > n->d.n_layers || first > end) return MYEA_E_INVALID;
+    if (B > n->d.batch_size) return MYEA_E_BATCH;
+    size_t T = n->d.number_recurrent_depth;
+    for (size_t li = first; li < end; ++li) {
+        const myea_layer_desc *l = &n->d.layers[li];
+        if (l->type_layer == MYEA_LAYER_RESIDUAL) continue;
+        if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_UNSUPPORTED;
+        olayer *o = &n->L[li];
+        const float *x = layer_outputs(n, li - 1);
+        for (size_t t = 0; t < T; ++t) {
+            dw_fc(n, t, B, n->L[li - 1].H, o->H, x, o->neuron_errors, n->gradient + l->first_connection_index);
+            if (layer_uses_bias(l)) dw_bias(n, t, B, o->H, o->neuron_errors, n->gradient + l->first_bias_connection_index);
+        }
+    }
+    return MYEA_OK;
+}
+
+/* ------------------------------------------------------------------------------------------- */
+/* Update_Parameter: NN/Neural_Network.cpp:4719-4908 (merge is a no-op with one accumulator) */
+
+/* Euclidean_Norm (Clip_Gradient): NN/Neural_Network__Regularization__Max_Norm_Constraints.cpp:48-140,
+ * NN/Neural_Network__Clip_Gradient.cpp:81-94.  One global norm over all P; scale when norm >= clip. */
+static void clip_gradient(myea_oracle_net *n)
+{
+    size_t P = n->d.total_parameters;
+    float norms = 0.f;
+    for (size_t i = 0; i < P; ++i) norms += n->gradient[i] * n->gradient[i];
+    norms = sqrtf(norms);
+    if (norms >= n->h.clip_gradient) {
+        float s = n->h.clip_gradient / norms;
+        for (size_t i = 0; i < P; ++i) n->gradient[i] *= s;
+    }
+}
+
+static float clipf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+int myea_oracle_update_parameter(myea_oracle_net *n, size_t B, size_t training_size)
+{
+    (void)B; (void)training_size; /* only used by normalised weight decay, which is off by default */
+    if (!n) return MYEA_E_INVALID;
+    size_t P = n->d.total_parameters, W = n->d.total_weights;
+    myea_hyper *h = &n->h;
+    float *g = n->gradient, *w = n->parameters;
+    if (h->use_clip_gradient) clip_gradient(n);
+    h->optimizer_time_step += 1.f;
+    float wd = h->regularization__weight_decay;
+    switch (h->type_optimizer_function) {
+    case MYEA_OPTIMIZER_GD: {
+        /* NN/Neural_Network__Gradient_Descent.cpp:22-159, NN/Neural_Network__Gradient_Descent_Momentum.cpp:22-62,
+         * NN/Neural_Network__Nesterov_Accelerated_Gradient.cpp:22-64 */
+        float lr = h->learning_rate, mu = h->learning_momentum;
+        float *dprev = n->opt[MYEA_STATE_PREVIOUS_DELTA];
+        for (size_t i = 0; i < P; ++i) {
+            float reg = (wd != 0.f) ? (i < W ? 1.f : 0.f) * wd * w[i] : 0.f;
+            if (mu == 0.f) {
+                if (wd != 0.f) w[i] -= lr * g[i] + reg; else w[i] -= lr * g[i];
+            } else if (!h->use_Nesterov) {
+                float d = dprev[i] = lr * g[i] + mu * dprev[i];
+                if (wd != 0.f) w[i] -= d + reg; else w[i] -= d;
+            } else {
+                float d = dprev[i] = lr * g[i] + mu * dprev[i];
+                if (wd != 0.f) w[i] -= mu * d - lr * g[i] + reg; else w[i] -= mu * d - lr * g[i]; /* sign as written, :48,59 */
+            }
+            g[i] = 0.f;
+        }
+        break;
+    }
+    case MYEA_OPTIMIZER_ADAM:
+    case MYEA_OPTIMIZER_AMSGRAD:
+    case MYEA_OPTIMIZER_ADABOUND: {
+        /* NN/Neural_Network__Adam.cpp:43-97, NN/Neural_Network__AMSGrad.cpp:43-105, NN/Neural_Network__AdaBound.cpp:43-110 */
+        float lr = h->adam_learning_rate, b1 = h->adam_beta1, b2 = h->adam_beta2, eps = h->adam_epsilon, ts = h->optimizer_time_step;
+        float lr_t = h->use_adam_bias_correction ? (float)(lr * sqrt(1.0 - pow(b2, ts)) / (1.0 - pow(b1, ts))) : lr;
+        float lo = h->learning_rate_final * (1.f - 1.f / (h->learning_gamma * ts + 1.f));
+        float hi = h->learning_rate_final * (1.f + 1.f / (h->learning_gamma * ts));
+        float *m = n->opt[MYEA_STATE_FIRST_MOMENT], *v = n->opt[MYEA_STATE_SECOND_MOMENT], *vh = n->opt[MYEA_STATE_SECOND_MOMENT_HAT];
+        for (size_t i = 0; i < P; ++i) {
+            float gi = g[i];
+            float mi = m[i] = b1 * m[i] + (1.f - b1) * gi;
+            float vi = v[i] = b2 * v[i] + (1.f - b2) * gi * gi;
+            float reg = (wd != 0.f) ? (i < W ? 1.f : 0.f) * wd * w[i] : 0.f;
+            float step;
+            if (h->type_optimizer_function == MYEA_OPTIMIZER_ADAM) step = lr_t * mi / (sqrtf(vi) + eps);
+            else if (h->type_optimizer_function == MYEA_OPTIMIZER_AMSGRAD) {
+                float hh = vh[i] = vh[i] > vi ? vh[i] : vi;
+                step = lr_t * mi / (sqrtf(hh) + eps);
+            } else step = clipf(lr_t / (sqrtf(vi) + eps), lo, hi) * mi;
+            if (wd != 0.f) w[i] -= step + reg; else w[i] -= step;
+            g[i] = 0.f;
+        }
+        break;
+    }
+    default: return MYEA_E_UNSUPPORTED;
+    }
+    return MYEA_OK;
+}
+
+int myea_oracle_reset_loss(myea_oracle_net *n) { if (!n) return MYEA_E_INVALID; memset(&n->loss, 0, sizeof(n->loss)); return MYEA_OK; }
+int myea_oracle_get_loss(myea_oracle_net *n, myea_loss_state *s) { if (!n || !s) return MYEA_E_INVALID; *s = n->loss; return MYEA_OK; }
+
+const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t *count)
+{
+    if (!n || li >= n->d.n_layers) return NULL;
+    olayer *o = &n->L[li];
+    size_t T = n->d.number_recurrent_depth, full = T * n->d.batch_size * o->H, th = T * o->H;
+    const float *p = NULL; size_t c = full;
+    switch (kind) {
+    case MYEA_TENSOR_OUTPUTS: p = layer_outputs(n, li); break;
+    case MYEA_TENSOR_SUMMATIONS: p = o->summations; break;
+    case MYEA_TENSOR_ERRORS: p = o->neuron_errors; break;
+    case MYEA_TENSOR_NORM_HATS: p = o->hats; break;
+    case MYEA_TENSOR_NORM_MEANS: p = o->means; c = th; break;
+    case MYEA_TENSOR_NORM_VARIANCES: p = o->variances; c = th; break;
+    case MYEA_TENSOR_NORM_MEANS_AVERAGES: p = o->means_averages; c = th; break;
+    case MYEA_TENSOR_NORM_VARIANCES_AVERAGES: p = o->variances_averages; c = th; break;
+    default: break;
+    }
+    if (count) *count = p ? c : 0;
+    return p;
+}

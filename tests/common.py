@@ -1,0 +1,70 @@
+"""Shared builders for the parity tests: seeded synthetic nets and data in the reference's layouts."""
+import ctypes as C
+
+import numpy as np
+
+from myea_amd import binding as mb
+from tests.oracle_lib import load_oracle
+
+
+def oracle_desc(layers, batch_size, recurrent_depth=1):
+    """make_desc through the oracle build of the layout code (no HIP library needed on CPU)."""
+    return mb.make_desc(layers, batch_size, recurrent_depth, lib=load_oracle())
+
+
+def oracle_hyper(**kw):
+    return mb.default_hyper(lib=load_oracle(), **kw)
+
+
+def glorot_parameters(desc, seed, bias_range=0.1):
+    """Glorot-uniform weights per FC layer written into the flat vector; small random biases so that the
+    bias path is exercised; scales near 1, shifts near 0 for normalised layers."""
+    rng = np.random.default_rng(seed)
+    w = np.zeros(desc.total_parameters, dtype=np.float32)
+    widths = []
+    for i in range(desc.n_layers):
+        l = desc.layers[i]
+        widths.append(l.n_units * (l.n_cells_per_block if l.type_layer == mb.LAYER_LSTM else 1))
+    for i in range(1, desc.n_layers):
+        l = desc.layers[i]
+        fan_in, fan_out = widths[i - 1], widths[i]
+        n = l.last_connection_index - l.first_connection_index
+        r = np.sqrt(6.0 / (fan_in + fan_out))
+        w[l.first_connection_index:l.last_connection_index] = rng.uniform(-r, r, n).astype(np.float32)
+    nb = desc.total_bias
+    w[desc.total_weights:desc.total_weights + nb] = rng.uniform(-bias_range, bias_range, nb).astype(np.float32)
+    tn = desc.total_normalized_units
+    if tn:
+        base = desc.total_weights + desc.total_bias
+        w[base:base + tn] = rng.uniform(0.5, 1.5, tn).astype(np.float32)
+        w[base + tn:base + 2 * tn] = rng.uniform(-0.2, 0.2, tn).astype(np.float32)
+    return w
+
+
+def one_hot(labels, n):
+    y = np.zeros((len(labels), n), dtype=np.float32)
+    y[np.arange(len(labels)), labels] = 1.0
+    return y
+
+
+def run_step(net, B, X, Y, training_size=None, update=True):
+    """the 4-call loop of Dataset::Train_Batch_BP (Neural_Network/Dataset.cpp:645-658) + Update_Parameter"""
+    net.Forward_Pass(B, X)
+    net.Compute__Error(B, Y)
+    net.Backward_Pass(B)
+    net.Update_Derivative_Weight(B, 1, net.desc.n_layers)
+    if update:
+        net.Update_Parameter(B, training_size or B)
+
+
+def assert_close(a, b, rel=1e-4, abs_=1e-5, what=""):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    assert a.shape == b.shape, (what, a.shape, b.shape)
+    err = np.abs(a - b)
+    tol = abs_ + rel * np.abs(b)
+    bad = err > tol
+    if bad.any():
+        i = int(np.argmax(err - tol))
+        raise AssertionError("%s: %d / %d out of tolerance; worst at %d: got %.9g want %.9g (err %.3g, tol %.3g)"
+                             % (what, int(bad.sum()), a.size, i, a.flat[i], b.flat[i], err.flat[i], tol.flat[i]))
