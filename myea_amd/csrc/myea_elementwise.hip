@@ -103,15 +103,18 @@ __global__ __launch_bounds__(kBlock) void scatter_time_major_kernel(size_t B, si
 // Stage 1: grid (ceil(H/64), S); a workgroup is 64 columns x 4 row lanes and owns rows
 // [y*chunk, (y+1)*chunk).  It writes NV partial sums per column to partial[(y*NV + v)*H + col].
 
+// Per-lane accumulation is in fp64 (the kernels are HBM-bound, the adds are free): sums like
+// E[x^2] - mean^2 lose most of their digits when |mean| >> sigma, and the fp32 result should then be the
+// correctly rounded one rather than depend on the summation order.
 template <int NV, typename F>
 __global__ __launch_bounds__(kBlock) void column_partial_kernel(size_t rows, size_t H, size_t chunk, float *partial, F f)
 {
-    __shared__ float red[NV][4][64];
+    __shared__ double red[NV][4][64];
     const int c = threadIdx.x & 63, rl = threadIdx.x >> 6;
     const size_t col = (size_t)blockIdx.x * 64 + c;
-    float acc[NV];
+    double acc[NV];
 #pragma unroll
-    for (int v = 0; v < NV; ++v) acc[v] = 0.f;
+    for (int v = 0; v < NV; ++v) acc[v] = 0.0;
     if (col < H) {
         const size_t r0 = (size_t)blockIdx.y * chunk, r1 = min(rows, r0 + chunk);
         for (size_t r = r0 + rl; r < r1; r += 4) f(r, col, acc);
@@ -122,7 +125,7 @@ __global__ __launch_bounds__(kBlock) void column_partial_kernel(size_t rows, siz
     if (rl == 0 && col < H) {
 #pragma unroll
         for (int v = 0; v < NV; ++v)
-            partial[((size_t)blockIdx.y * NV + v) * H + col] = red[v][0][c] + red[v][1][c] + red[v][2][c] + red[v][3][c];
+            partial[((size_t)blockIdx.y * NV + v) * H + col] = (float)(red[v][0][c] + red[v][1][c] + red[v][2][c] + red[v][3][c]);
     }
 }
 
@@ -142,23 +145,23 @@ inline void split_rows(size_t rows, size_t H, size_t &S, size_t &chunk)
 
 struct SumF {
     const float *x; size_t H;
-    __device__ void operator()(size_t r, size_t col, float *acc) const { acc[0] += x[r * H + col]; }
+    __device__ void operator()(size_t r, size_t col, double *acc) const { acc[0] += x[r * H + col]; }
 };
 
 __global__ __launch_bounds__(kBlock) void column_sum_final_kernel(size_t H, size_t S, const float *partial, float *out, int accumulate)
 {
     const size_t col = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (col >= H) return;
-    float s = 0.f;
+    double s = 0.0;
     for (size_t y = 0; y < S; ++y) s += partial[y * H + col];
-    out[col] = accumulate ? out[col] + s : s;
+    out[col] = accumulate ? out[col] + (float)s : (float)s;
 }
 
 // ---- batch normalisation ----------------------------------------------------------------------------
 
 struct BnStatF {
     const float *x; size_t H;
-    __device__ void operator()(size_t r, size_t col, float *acc) const { float s = x[r * H + col]; acc[0] += s; acc[1] += s * s; }
+    __device__ void operator()(size_t r, size_t col, double *acc) const { const double s = x[r * H + col]; acc[0] += s; acc[1] += s * s; }
 };
 
 // Forward_Pass__Batch_Normalization__Training / __Batch_Renormalization__Training, "Average" loop
@@ -167,8 +170,9 @@ __global__ __launch_bounds__(kBlock) void bn_forward_final_kernel(size_t H, size
 {
     const size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (j >= H) return;
-    float sm = 0.f, sv = 0.f;
-    for (size_t y = 0; y < S; ++y) { sm += partial[(y * 2 + 0) * H + j]; sv += partial[(y * 2 + 1) * H + j]; }
+    double smd = 0.0, svd = 0.0;
+    for (size_t y = 0; y < S; ++y) { smd += partial[(y * 2 + 0) * H + j]; svd += partial[(y * 2 + 1) * H + j]; }
+    const float sm = (float)smd, sv = (float)svd;
     const float bscale = 1.f / (float)rows;
     const float mean = sm * bscale;
     float mavg = p.mean_avg[j];
@@ -214,7 +218,7 @@ __global__ __launch_bounds__(kBlock) void bn_forward_inference_kernel(size_t n, 
 // (NN/Neural_Network__Backward_Pass__OpenMP.cpp:1385-1413, :1627-1655)
 struct BnBackF {
     BnBackwardParams p;
-    __device__ void operator()(size_t r, size_t col, float *acc) const
+    __device__ void operator()(size_t r, size_t col, double *acc) const
     {
         const size_t k = r * p.H + col;
         float e = p.dy[k];
@@ -232,17 +236,17 @@ __global__ __launch_bounds__(kBlock) void bn_backward_final_kernel(size_t H, siz
 {
     const size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (j >= H) return;
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
     for (size_t y = 0; y < S; ++y) {
         a0 += partial[(y * 4 + 0) * H + j];
         a1 += partial[(y * 4 + 1) * H + j];
         a2 += partial[(y * 4 + 2) * H + j];
         a3 += partial[(y * 4 + 3) * H + j];
     }
-    dscale[j] += a0;
-    dshift[j] += a1;
-    dmean_dvar[j] = a2;
-    dmean_dvar[H + j] = a3;
+    dscale[j] += (float)a0;
+    dshift[j] += (float)a1;
+    dmean_dvar[j] = (float)a2;
+    dmean_dvar[H + j] = (float)a3;
 }
 
 // last loop (:1437-1466, :1679-1708)
