@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the training hot path on one MI355X.
+
+One "step" = Forward_Pass + Compute__Error + Backward_Pass + Update_Derivative_Weight + Update_Parameter on one
+batch of synthetic data already resident in HBM.  Default workload: BASELINE config 2, the deep fully-connected
+stack 4096-4096-4096-4096-4096-1000 (ReLU, softmax + cross-entropy, Adam) at batch 1024, fp32.
+
+Prints ONE JSON line (see README / DESIGN).  `roofline` covers the dominant kernel family — the FP32 MFMA
+contractions (forward X W^T, dX = delta W, dW += delta^T X): algorithmic FLOPs of all their launches in the
+timed region over their summed HIP-event durations on the stream they run on.  `cpu_baseline` times the CPU
+restatement of the reference (oracle/, OpenMP) on this host on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
+PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+
+WORKLOADS = {
+    # BASELINE.json configs[1]
+    "fc4096x4_b1024_adam": dict(
+        layers=[dict(units=4096)] + [dict(units=4096, activation="RELU")] * 4 + [dict(units=1000, activation="SOFTMAX")],
+        batch=1024, head="SOFTMAX", optimizer="ADAM", loss="CROSS_ENTROPY", data="normal", hyper={}),
+    # BASELINE.json configs[0] (the reference's own CPU-sized case)
+    "mlp784_256_10_b128_sgd": dict(
+        layers=[dict(units=784), dict(units=256, activation="TANH"), dict(units=10, activation="SIGMOID")],
+        batch=128, head="SIGMOID", optimizer="GD", loss="MSE", data="uniform", hyper=dict(learning_rate=0.01, learning_momentum=0.9)),
+    # BASELINE.json configs[3] (input width 2048)
+    "fc2048x8_bn_relu_dropout_b512_nesterov": dict(
+        layers=[dict(units=2048)] + [dict(units=2048, activation="RELU", normalization="BATCH_NORMALIZATION", norm_before=True,
+                                          dropout="BERNOULLI_INVERTED", keep=0.5)] * 8 + [dict(units=100, activation="SOFTMAX")],
+        batch=512, head="SOFTMAX", optimizer="GD", loss="CROSS_ENTROPY", data="normal",
+        hyper=dict(learning_rate=0.01, learning_momentum=0.9, use_Nesterov=1)),
+}
+
+
+def gemm_flops_per_step(layers, batch):
+    """2*M*N*K of forward, dX (layers 2..) and dW."""
+    w = [l["units"] for l in layers]
+    fwd = sum(2.0 * batch * w[i] * w[i - 1] for i in range(1, len(w)))
+    dx = sum(2.0 * batch * w[i] * w[i - 1] for i in range(2, len(w)))
+    return fwd + dx + fwd
+
+
+def make_inputs(np, wl, seed):
+    rng = np.random.default_rng(seed)
+    B, n_in, n_out = wl["batch"], wl["layers"][0]["units"], wl["layers"][-1]["units"]
+    X = (rng.normal(0, 1, (B, n_in)) if wl["data"] == "normal" else rng.uniform(0, 1, (B, n_in))).astype(np.float32)
+    Y = np.zeros((B, n_out), dtype=np.float32)
+    Y[np.arange(B), rng.integers(0, n_out, B)] = 1.0
+    return X, Y
+
+
+def cpu_baseline(wl, sample_rows, threads):
+    """The oracle (a port of the reference's CPU path) on `sample_rows` examples of the same network: forward +
+    error + backward + dW are timed on the sample and scaled to the full batch; the weight update is timed over the
+    full parameter vector; samples/s = batch / (t_sample * batch / sample_rows + t_update)."""
+    import numpy as np
+    from myea_amd import binding as mb
+    from tests.common import glorot_parameters
+    from tests.oracle_lib import OracleNetwork, load_oracle
+    lib = load_oracle()
+    desc = mb.make_desc(wl["layers"], sample_rows, lib=lib)
+    h = mb.default_hyper(lib=lib, type_optimizer_function=mb.OPTIMIZER[wl["optimizer"]], type_loss_function=mb.LOSS[wl["loss"]], **wl["hyper"])
+    net = OracleNetwork(desc, h, threads=threads)
+    net.set_state_propagation(mb.STATE_TRAINING)
+    net.upload_parameters(glorot_parameters(desc, 2))
+    if desc.total_mask_units:
+        net.upload_masks((np.random.default_rng(4).uniform(0, 1, desc.total_mask_units) < 0.5).astype(np.uint8))
+    X, Y = make_inputs(np, dict(wl, batch=sample_rows), 2)
+    t_sample, t_update, reps = 0.0, 0.0, 0
+    while reps < 1 or (t_sample + t_update < 10.0 and reps < 8):   # about 10-30 s of CPU work
+        t0 = time.perf_counter()
+        net.Forward_Pass(sample_rows, X)
+        net.Compute__Error(sample_rows, Y)
+        net.Backward_Pass(sample_rows)
+        net.Update_Derivative_Weight(sample_rows)
+        t1 = time.perf_counter()
+        net.Update_Parameter(sample_rows, sample_rows)
+        t2 = time.perf_counter()
+        t_sample += t1 - t0
+        t_update += t2 - t1
+        reps += 1
+    t_sample /= reps
+    t_update /= reps
+    t_step = t_sample * wl["batch"] / sample_rows + t_update
+    return dict(value=wl["batch"] / t_step, unit="samples/s", cores=threads, kind="port",
+                sample="%d of %d examples through the full-width network (%.2f s per pass, %d passes) scaled to the batch, plus the full weight update (%.2f s)"
+                       % (sample_rows, wl["batch"], t_sample, reps, t_update))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="fc4096x4_b1024_adam", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-rows", type=int, default=0, help="examples in the CPU sample (default: sized for ~20 s)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); no multi-GPU path exists")
+
+    import numpy as np
+    import torch
+    from myea_amd import binding as mb
+    from tests.common import glorot_parameters
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    wl = WORKLOADS[args.workload]
+    B = wl["batch"]
+    desc = mb.make_desc(wl["layers"], B)
+    h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER[wl["optimizer"]], type_loss_function=mb.LOSS[wl["loss"]], **wl["hyper"])
+    net = mb.HipNetwork(desc, h)
+    net.set_stream(torch.cuda.current_stream().cuda_stream)
+    net.set_state_propagation(mb.STATE_TRAINING)
+    net.upload_parameters(glorot_parameters(desc, 2))
+    net.Clear_Training_Arrays()
+    if desc.total_mask_units:
+        net.upload_masks((np.random.default_rng(4).uniform(0, 1, desc.total_mask_units) < 0.5).astype(np.uint8))
+    X, Y = make_inputs(np, wl, 2)
+    xd, yd = torch.from_numpy(X).cuda(), torch.from_numpy(Y).cuda()   # inputs resident in HBM before the timed region
+
+    def step():
+        net.Forward_Pass(B, xd, on_device=True)
+        net.Compute__Error(B, yd, on_device=True)
+        net.Backward_Pass(B)
+        net.Update_Derivative_Weight(B)
+        net.Update_Parameter(B, B)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    net.profile_enable(True)
+    for f in range(4):
+        net.profile_read(f)            # drop anything recorded so far
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    fam = {name: net.profile_read(i) for i, name in enumerate(("forward", "dx", "dw", "update"))}
+    net.profile_enable(False)
+    loss = net.get_loss()
+
+    g_launch = sum(fam[k][0] for k in ("forward", "dx", "dw"))
+    g_ms = sum(fam[k][1] for k in ("forward", "dx", "dw"))
+    g_flop = sum(fam[k][2] for k in ("forward", "dx", "dw"))
+    achieved = g_flop / (g_ms * 1e-3) / 1e12 if g_ms > 0 else 0.0
+    kernels = {}
+    for k in ("forward", "dx", "dw"):
+        n, ms, work = fam[k]
+        kernels["gemm_" + k] = dict(launches=n, avg_ms=ms / max(n, 1), tflops=work / max(ms * 1e-3, 1e-12) / 1e12,
+                                    frac_mfma_peak=work / max(ms * 1e-3, 1e-12) / 1e12 / PEAK_FP32_MFMA_TFLOPS)
+    n, ms, work = fam["update"]
+    kernels["optimizer_update"] = dict(launches=n, avg_ms=ms / max(n, 1), gbs=work / max(ms * 1e-3, 1e-12) / 1e9,
+                                       frac_hbm_peak=work / max(ms * 1e-3, 1e-12) / 1e9 / PEAK_HBM_GBS)
+
+    out = {
+        "metric": "train samples/s (fwd+bwd+Adam) FC-4096x4 & LSTM-512; % FP32 MFMA/HBM peak",
+        "value": B / (ms_per_step * 1e-3),
+        "unit": "samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "batch": B, "layers": [l["units"] for l in wl["layers"]],
+                   "optimizer": wl["optimizer"], "parameters": int(desc.total_parameters),
+                   "gemm_flops_per_step": gemm_flops_per_step(wl["layers"], B)},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                     "kernel": "gemm_f32_mfma_kernel (forward + dX + dW launches)", "launches": g_launch,
+                     "avg_launch_ms": g_ms / max(g_launch, 1), "flops_per_launch": g_flop / max(g_launch, 1),
+                     "gemm_ms_per_step": g_ms / args.steps},
+        "kernels": kernels,
+        "loss_per_output": loss.loss_values / max(loss.number_loss, 1),
+    }
+    if not args.no_cpu_baseline:
+        threads = min(16, os.cpu_count() or 1)
+        rows = args.cpu_sample_rows
+        if rows <= 0:
+            # sized from the layer widths for ~20 s at ~15 GFLOP/s per thread (gcc -O2 vectorises the inner loops)
+            flop_per_row = gemm_flops_per_step(wl["layers"], 1)
+            rows = int(max(4, min(B, 20.0 * threads * 15.0e9 / flop_per_row)))
+            rows = max(threads, rows - rows % threads)
+        out["cpu_baseline"] = cpu_baseline(wl, rows, threads)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

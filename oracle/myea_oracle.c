@@ -742,8 +742,11 @@ int myea_oracle_update_parameter(myea_oracle_net *n, size_t B, size_t training_s
          * NN/Neural_Network__Nesterov_Accelerated_Gradient.cpp:22-64 */
         float lr = h->learning_rate, mu = h->learning_momentum;
         float *dprev = n->opt[MYEA_STATE_PREVIOUS_DELTA];
-        for (size_t i = 0; i < P; ++i) {
-            float reg = (wd != 0.f) ? (i < W ? 1.f : 0.f) * wd * w[i] : 0.f;
+        long i;
+        /* elementwise: the thread split does not change any result (the reference's __OpenMP variants do the same) */
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+        for (i = 0; i < (long)P; ++i) {
+            float reg = (wd != 0.f) ? ((size_t)i < W ? 1.f : 0.f) * wd * w[i] : 0.f;
             if (mu == 0.f) {
                 if (wd != 0.f) w[i] -= lr * g[i] + reg; else w[i] -= lr * g[i];
             } else if (!h->use_Nesterov) {
@@ -766,11 +769,13 @@ int myea_oracle_update_parameter(myea_oracle_net *n, size_t B, size_t training_s
         float lo = h->learning_rate_final * (1.f - 1.f / (h->learning_gamma * ts + 1.f));
         float hi = h->learning_rate_final * (1.f + 1.f / (h->learning_gamma * ts));
         float *m = n->opt[MYEA_STATE_FIRST_MOMENT], *v = n->opt[MYEA_STATE_SECOND_MOMENT], *vh = n->opt[MYEA_STATE_SECOND_MOMENT_HAT];
-        for (size_t i = 0; i < P; ++i) {
+        long i;
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+        for (i = 0; i < (long)P; ++i) {
             float gi = g[i];
             float mi = m[i] = b1 * m[i] + (1.f - b1) * gi;
             float vi = v[i] = b2 * v[i] + (1.f - b2) * gi * gi;
-            float reg = (wd != 0.f) ? (i < W ? 1.f : 0.f) * wd * w[i] : 0.f;
+            float reg = (wd != 0.f) ? ((size_t)i < W ? 1.f : 0.f) * wd * w[i] : 0.f;
             float step;
             if (h->type_optimizer_function == MYEA_OPTIMIZER_ADAM) step = lr_t * mi / (sqrtf(vi) + eps);
             else if (h->type_optimizer_function == MYEA_OPTIMIZER_AMSGRAD) {
