@@ -423,7 +423,10 @@ __global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
     const size_t n4 = p.n / 4;
     f32x4 *w4 = reinterpret_cast<f32x4 *>(p.w), *g4 = reinterpret_cast<f32x4 *>(p.g);
     f32x4 *a4 = reinterpret_cast<f32x4 *>(p.s0), *b4 = reinterpret_cast<f32x4 *>(p.s1), *c4 = reinterpret_cast<f32x4 *>(p.s2);
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += (size_t)gridDim.x * kBlock) {
+    // One 128-bit element per lane and no loop: every vector is streamed exactly once, so the stores bypass
+    // the caches (non-temporal) and a grid of n/1024 workgroups keeps enough requests in flight for HBM.
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n4) {
         const f32x4 wv = w4[i], gv = g4[i];
         f32x4 av = {0.f, 0.f, 0.f, 0.f}, bv = av, cv = av;
         if (kA) av = a4[i];
@@ -435,11 +438,11 @@ __global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
             w[e] = wv[e]; a[e] = av[e]; b[e] = bv[e]; c[e] = cv[e];
             update_one<KIND, WD>(p, gs, w[e], gv[e], a[e], b[e], c[e], i * 4 + e < p.n_weights);
         }
-        w4[i] = f32x4{w[0], w[1], w[2], w[3]};
-        if (kA) a4[i] = f32x4{a[0], a[1], a[2], a[3]};
-        if (kB) b4[i] = f32x4{b[0], b[1], b[2], b[3]};
-        if (kC) c4[i] = f32x4{c[0], c[1], c[2], c[3]};
-        g4[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        __builtin_nontemporal_store(f32x4{w[0], w[1], w[2], w[3]}, &w4[i]);
+        if (kA) __builtin_nontemporal_store(f32x4{a[0], a[1], a[2], a[3]}, &a4[i]);
+        if (kB) __builtin_nontemporal_store(f32x4{b[0], b[1], b[2], b[3]}, &b4[i]);
+        if (kC) __builtin_nontemporal_store(f32x4{c[0], c[1], c[2], c[3]}, &c4[i]);
+        __builtin_nontemporal_store(f32x4{0.f, 0.f, 0.f, 0.f}, &g4[i]);
     }
     if (blockIdx.x == 0 && threadIdx.x < (p.n & 3)) {
         const size_t i = n4 * 4 + threadIdx.x;
@@ -456,7 +459,7 @@ __global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
 template <int KIND>
 int launch_update_kind(hipStream_t s, const UpdateDev &d, bool wd)
 {
-    const unsigned grid = grid_for(d.n / 4 + 1, kBlock, 256u * 16u);
+    const unsigned grid = grid_for(d.n / 4 + 1, kBlock, 0x7fffffffu);
     if (wd) hipLaunchKernelGGL((update_kernel<KIND, true>), dim3(grid), dim3(kBlock), 0, s, d);
     else hipLaunchKernelGGL((update_kernel<KIND, false>), dim3(grid), dim3(kBlock), 0, s, d);
     MYEA_HIP_TRY(hipGetLastError());

@@ -30,6 +30,16 @@
 #include <omp.h>
 #endif
 
+/* LSTM-with-peephole layer state, one direction.  Cell tensors are [T][Bmax][C], block tensors [T][Bmax][K]
+ * (NNH/Data.hpp:2985-3016: ptr_array_cells_* / ptr_array_blocks_*). */
+typedef struct olstm {
+    size_t K, cpb, C, In;   /* blocks, cells per block, cells, fan-in */
+    size_t per_block;       /* parameters of one block */
+    float *sum_in_z, *sum_rec_z, *sum_z, *z, *c, *ca;          /* cells */
+    float *sum_in_i, *sum_in_f, *sum_in_o, *sum_rec_i, *sum_rec_f, *sum_rec_o, *sum_i, *sum_f, *sum_o, *gi, *gf, *go; /* blocks */
+    float *dz, *dc, *di, *df, *dgo;                              /* deltas */
+} olstm;
+
 typedef struct olayer {
     size_t H;            /* *ptr_number_outputs */
     size_t norm_units;   /* number of Normalized_unit owned by the layer */
@@ -214,10 +224,29 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
         const myea_layer_desc *l = &desc->layers[li];
         olayer *o = &n->L[li];
         o->H = layer_width(l);
-        if (l->type_layer == MYEA_LAYER_RESIDUAL || l->type_layer == MYEA_LAYER_LSTM) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (l->type_layer == MYEA_LAYER_RESIDUAL) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (l->type_layer == MYEA_LAYER_LSTM && (l->use_bidirectional || layer_uses_norm(l) || l->type_dropout != MYEA_DROPOUT_NONE)) { free(n); return MYEA_E_UNSUPPORTED; }
         size_t sz = T * B * o->H;
         o->values = zalloc(sz);
         if (li == 0) continue;
+        if (l->type_layer == MYEA_LAYER_LSTM) {
+            /* the bias vectors are read at first_bias_connection_index + [0, C + 3K): with the index as the reference
+             * leaves it they run C entries past the layer's own slice; past the end of the bias region the reference
+             * reads and writes outside its parameter array, which nothing here reproduces */
+            if (l->first_bias_connection_index + (size_t)l->n_units * l->n_cells_per_block + 3u * l->n_units > desc->total_weights + desc->total_bias) { free(n); return MYEA_E_INVALID; }
+            olstm *q = (olstm *)calloc(1, sizeof(olstm));
+            q->K = l->n_units; q->cpb = l->n_cells_per_block; q->C = q->K * q->cpb; q->In = n->L[li - 1].H;
+            q->per_block = q->cpb * (q->In + q->C) + 3 * q->In + 3 * q->C + 3 * q->cpb;
+            size_t sc = T * B * q->C, sk = T * B * q->K;
+            float **cells[] = {&q->sum_in_z, &q->sum_rec_z, &q->sum_z, &q->z, &q->c, &q->ca, &q->dz, &q->dc};
+            float **blocks[] = {&q->sum_in_i, &q->sum_in_f, &q->sum_in_o, &q->sum_rec_i, &q->sum_rec_f, &q->sum_rec_o, &q->sum_i, &q->sum_f, &q->sum_o,
+                                &q->gi, &q->gf, &q->go, &q->di, &q->df, &q->dgo};
+            for (size_t a = 0; a < sizeof(cells) / sizeof(cells[0]); ++a) *cells[a] = zalloc(sc);
+            for (size_t a = 0; a < sizeof(blocks) / sizeof(blocks[0]); ++a) *blocks[a] = zalloc(sk);
+            o->lstm = q;
+            o->af_errors = zalloc(sz);  /* ptr_delta_cell_output */
+            continue;
+        }
         o->summations = zalloc(sz);
         o->neuron_errors = zalloc(sz);
         o->af_errors = zalloc(sz);
@@ -252,6 +281,13 @@ int myea_oracle_destroy(myea_oracle_net *n)
         free(o->neuron_errors); free(o->af_errors); free(o->norm_errors);
         free(o->means); free(o->variances); free(o->means_averages); free(o->variances_averages);
         free(o->r_corrections); free(o->d_corrections); free(o->derivatives_means); free(o->derivatives_variances);
+        if (o->lstm) {
+            olstm *q = o->lstm;
+            float *all[] = {q->sum_in_z, q->sum_rec_z, q->sum_z, q->z, q->c, q->ca, q->dz, q->dc, q->sum_in_i, q->sum_in_f, q->sum_in_o, q->sum_rec_i,
+                            q->sum_rec_f, q->sum_rec_o, q->sum_i, q->sum_f, q->sum_o, q->gi, q->gf, q->go, q->di, q->df, q->dgo};
+            for (size_t a = 0; a < sizeof(all) / sizeof(all[0]); ++a) free(all[a]);
+            free(q);
+        }
     }
     free(n);
     return MYEA_OK;
@@ -425,6 +461,250 @@ static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
     fwd_dropout(n, l, t, B, H, out);
 }
 
+
+/* ------------------------------------------------------------------------------------------- */
+/* LSTM with peepholes (one direction, time ascending) */
+
+/* parameter offsets inside the layer's slice, NN/Neural_Network__Prepare_Connections.cpp:82-222: per block
+ * [z_in(In) | z_rec(C)] x cells, i_in, f_in, o_in (In each), i_rec, f_rec, o_rec (C each), peep_i, peep_f, peep_o (cpb each) */
+static size_t lstm_block_base(const myea_layer_desc *l, const olstm *q, size_t k) { return l->first_connection_index + k * q->per_block; }
+static size_t lstm_z_in(const myea_layer_desc *l, const olstm *q, size_t k, size_t j) { return lstm_block_base(l, q, k) + j * (q->In + q->C); }
+static size_t lstm_z_rec(const myea_layer_desc *l, const olstm *q, size_t k, size_t j) { return lstm_z_in(l, q, k, j) + q->In; }
+static size_t lstm_gate_in(const myea_layer_desc *l, const olstm *q, size_t k, int g) { return lstm_block_base(l, q, k) + q->cpb * (q->In + q->C) + (size_t)g * q->In; }
+static size_t lstm_gate_rec(const myea_layer_desc *l, const olstm *q, size_t k, int g) { return lstm_gate_in(l, q, k, 3) + (size_t)g * q->C; }
+static size_t lstm_peep(const myea_layer_desc *l, const olstm *q, size_t k, int g) { return lstm_gate_rec(l, q, k, 3) + (size_t)g * q->cpb; }
+
+static float sigmoid_f(float s) { return 1.f / (1.f + expf(-s)); }
+static float tanh_f(float s) { return 2.f / (1.f + expf(-2.f * s)) - 1.f; }
+
+/* Forward_Pass__LSTM (NN/Neural_Network__Forward_Pass__OpenMP.cpp:1769-2340), training and inference alike without
+ * normalisation / zoneout: Gates_CIFO (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:859-1040) ->
+ * Gates_CIF_AF_State (:1042-1191) -> States_AF (:1547-1582) -> Output (:1351-1418).
+ * First step: no recurrent sums, no forget gate, no input-gate peephole, c = i * z; the output gate peeps at c[t].
+ * Bias vectors sit at first_bias_connection_index + {0, C, C + K, C + 2K} (the field as Prepare__Bias__LSTM leaves it). */
+static void fwd_lstm_step(myea_oracle_net *n, size_t li, size_t t, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    olstm *q = o->lstm;
+    size_t Bmax = n->d.batch_size, K = q->K, C = q->C, cpb = q->cpb, In = q->In;
+    const float *x = layer_outputs(n, li - 1), *w = n->parameters;
+    const float *bz = w + l->first_bias_connection_index, *bi = bz + C, *bf = bi + K, *bo = bf + K;
+    int first = t == 0;
+    long b;
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+    for (b = 0; b < (long)B; ++b) {
+        size_t kb = (size_t)b * K + Bmax * K * t, cb = (size_t)b * C + Bmax * C * t, cp = (size_t)b * C + Bmax * C * (t - 1);
+        const float *xi = x + (size_t)b * In + Bmax * In * t;
+        const float *hp = first ? NULL : o->values + cp;
+        for (size_t k = 0; k < K; ++k) {
+            for (size_t j = 0; j < cpb; ++j) {
+                size_t c = k * cpb + j;
+                const float *wi = w + lstm_z_in(l, q, k, j), *wr = w + lstm_z_rec(l, q, k, j);
+                float s = 0.f;
+                for (size_t a = 0; a < In; ++a) s += xi[a] * wi[a];
+                q->sum_in_z[cb + c] = s;
+                if (!first) { s = 0.f; for (size_t a = 0; a < C; ++a) s += hp[a] * wr[a]; q->sum_rec_z[cb + c] = s; }
+            }
+            float si = 0.f, sf = 0.f, so = 0.f;
+            const float *wi = w + lstm_gate_in(l, q, k, 0), *wf = w + lstm_gate_in(l, q, k, 1), *wo = w + lstm_gate_in(l, q, k, 2);
+            for (size_t a = 0; a < In; ++a) { si += xi[a] * wi[a]; sf += xi[a] * wf[a]; so += xi[a] * wo[a]; }
+            q->sum_in_i[kb + k] = si; q->sum_in_f[kb + k] = sf; q->sum_in_o[kb + k] = so;
+            if (!first) {
+                si = sf = so = 0.f;
+                wi = w + lstm_gate_rec(l, q, k, 0); wf = w + lstm_gate_rec(l, q, k, 1); wo = w + lstm_gate_rec(l, q, k, 2);
+                for (size_t a = 0; a < C; ++a) { si += hp[a] * wi[a]; sf += hp[a] * wf[a]; so += hp[a] * wo[a]; }
+                q->sum_rec_i[kb + k] = si; q->sum_rec_f[kb + k] = sf; q->sum_rec_o[kb + k] = so;
+            }
+        }
+        /* Gates_CIF_AF_State */
+        for (size_t k = 0; k < K; ++k) {
+            const float *pi = w + lstm_peep(l, q, k, 0), *pf = w + lstm_peep(l, q, k, 1);
+            if (!first) {
+                float si = q->sum_in_i[kb + k] + q->sum_rec_i[kb + k] + bi[k];
+                float sf = q->sum_in_f[kb + k] + q->sum_rec_f[kb + k] + bf[k];
+                for (size_t j = 0; j < cpb; ++j) { si += q->c[cp + k * cpb + j] * pi[j]; sf += q->c[cp + k * cpb + j] * pf[j]; }
+                q->sum_i[kb + k] = si; q->sum_f[kb + k] = sf;
+                q->gi[kb + k] = sigmoid_f(si); q->gf[kb + k] = sigmoid_f(sf);
+            } else {
+                float si = q->sum_in_i[kb + k] + bi[k];
+                q->sum_i[kb + k] = si;
+                q->gi[kb + k] = sigmoid_f(si);
+            }
+            for (size_t j = 0; j < cpb; ++j) {
+                size_t c = k * cpb + j;
+                float sz = first ? q->sum_in_z[cb + c] + bz[c] : q->sum_in_z[cb + c] + q->sum_rec_z[cb + c] + bz[c];
+                q->sum_z[cb + c] = sz;
+                q->z[cb + c] = tanh_f(sz);
+                q->c[cb + c] = first ? q->z[cb + c] * q->gi[kb + k] : q->z[cb + c] * q->gi[kb + k] + q->gf[kb + k] * q->c[cp + c];
+            }
+        }
+        /* States_AF */
+        for (size_t c = 0; c < C; ++c) q->ca[cb + c] = tanh_f(q->c[cb + c]);
+        /* Output: the recurrent sum of the first step is never written by the reference and stays 0 */
+        for (size_t k = 0; k < K; ++k) {
+            const float *po = w + lstm_peep(l, q, k, 2);
+            float so = q->sum_in_o[kb + k] + (first ? 0.f : q->sum_rec_o[kb + k]) + bo[k];
+            for (size_t j = 0; j < cpb; ++j) so += q->c[cb + k * cpb + j] * po[j];
+            q->sum_o[kb + k] = so;
+            q->go[kb + k] = sigmoid_f(so);
+            for (size_t j = 0; j < cpb; ++j) o->values[cb + k * cpb + j] = q->ca[cb + k * cpb + j] * q->go[kb + k];
+        }
+    }
+}
+
+/* Backward_Pass__LSTM (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:1024-1120): delta to the layer below,
+ * dst[t][b][:] += dz_c Wz_in[c][:] + di_k Wi_in[k][:] + df_k Wf_in[k][:] + do_k Wo_in[k][:] */
+static void bwd_lstm_to_previous(myea_oracle_net *n, size_t gi, size_t t, size_t B, float *dst)
+{
+    const myea_layer_desc *l = &n->d.layers[gi];
+    olstm *q = n->L[gi].lstm;
+    size_t Bmax = n->d.batch_size, K = q->K, C = q->C, cpb = q->cpb, In = q->In;
+    const float *w = n->parameters;
+    long b;
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+    for (b = 0; b < (long)B; ++b) {
+        size_t kb = (size_t)b * K + Bmax * K * t, cb = (size_t)b * C + Bmax * C * t;
+        float *dx = dst + (size_t)b * In + Bmax * In * t;
+        for (size_t k = 0; k < K; ++k) {
+            for (size_t j = 0; j < cpb; ++j) {
+                float e = q->dz[cb + k * cpb + j];
+                const float *wr = w + lstm_z_in(l, q, k, j);
+                for (size_t a = In; a--;) dx[a] += e * wr[a];
+            }
+            const float *d3[3] = {q->di, q->df, q->dgo};
+            for (int g = 0; g < 3; ++g) {
+                float e = d3[g][kb + k];
+                const float *wr = w + lstm_gate_in(l, q, k, g);
+                for (size_t a = In; a--;) dx[a] += e * wr[a];
+            }
+        }
+    }
+}
+
+/* Recurrent__Backward_Pass__Gradient__LSTM (:440-862) for one time step, t descending:
+ * Backward_Pass__LSTM_Derivative__Output (:1130-1273), __Cell_State_AF (:1275-1327), __Gates_CIF_AF_State (:1329-1604). */
+static void bwd_lstm_step(myea_oracle_net *n, size_t li, size_t t, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    olstm *q = o->lstm;
+    size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, K = q->K, C = q->C, cpb = q->cpb;
+    const float *w = n->parameters;
+    int last = t == T - 1, first = t == 0;
+    long b;
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+    for (b = 0; b < (long)B; ++b) {
+        size_t kb = (size_t)b * K + Bmax * K * t, cb = (size_t)b * C + Bmax * C * t;
+        size_t kn = (size_t)b * K + Bmax * K * (t + 1), cn = (size_t)b * C + Bmax * C * (t + 1), cp = (size_t)b * C + Bmax * C * (t - 1);
+        float *dh = o->af_errors + cb;
+        if (!last) { /* recurrent delta from t + 1 */
+            for (size_t c = 0; c < C; ++c) {
+                float e = q->dz[cn + c];
+                const float *wr = w + lstm_z_rec(l, q, c / cpb, c % cpb);
+                for (size_t a = 0; a < C; ++a) dh[a] += e * wr[a];
+            }
+            for (size_t k = 0; k < K; ++k) {
+                float ei = q->di[kn + k], ef = q->df[kn + k], eo = q->dgo[kn + k];
+                const float *wi = w + lstm_gate_rec(l, q, k, 0), *wf = w + lstm_gate_rec(l, q, k, 1), *wo = w + lstm_gate_rec(l, q, k, 2);
+                for (size_t a = C; a--;) { float e = ei * wi[a]; e += ef * wf[a]; e += eo * wo[a]; dh[a] += e; }
+            }
+        }
+        for (size_t k = 0; k < K; ++k) { /* output gate */
+            float e = 0.f;
+            for (size_t j = 0; j < cpb; ++j) e += dh[k * cpb + j] * q->ca[cb + k * cpb + j];
+            float a = q->go[kb + k];
+            q->dgo[kb + k] = (1.f * a * (1.f - a)) * e;
+        }
+        for (size_t k = 0; k < K; ++k) /* cell state through tanh, on the stored activation */
+            for (size_t j = 0; j < cpb; ++j) {
+                size_t c = k * cpb + j;
+                q->dc[cb + c] = dh[c] * q->go[kb + k] * (1.f * (1.f - q->ca[cb + c] * q->ca[cb + c]));
+            }
+        if (first && last) continue; /* T == 1: no branch of Gates_CIF_AF_State matches */
+        for (size_t k = 0; k < K; ++k) {
+            const float *pi = w + lstm_peep(l, q, k, 0), *pf = w + lstm_peep(l, q, k, 1), *po = w + lstm_peep(l, q, k, 2);
+            float gi_ = q->gi[kb + k], ddo = q->dgo[kb + k];
+            for (size_t j = 0; j < cpb; ++j) {
+                size_t c = k * cpb + j;
+                float e = q->dc[cb + c];
+                e += po[j] * ddo;
+                if (!last) {
+                    e += pi[j] * q->di[kn + k];
+                    e += pf[j] * q->df[kn + k];
+                    e += q->dc[cn + c] * q->gf[kn + k];
+                }
+                q->dc[cb + c] = e;
+                q->dz[cb + c] = e * gi_ * (1.f * (1.f - q->z[cb + c] * q->z[cb + c]));
+            }
+            float ei = 0.f, ef = 0.f;
+            for (size_t j = 0; j < cpb; ++j) {
+                size_t c = k * cpb + j;
+                ei += q->dc[cb + c] * q->z[cb + c];
+                if (!first) ef += q->dc[cb + c] * q->c[cp + c];
+            }
+            q->di[kb + k] = ei * (1.f * gi_ * (1.f - gi_));
+            if (!first) { float f = q->gf[kb + k]; q->df[kb + k] = ef * (1.f * f * (1.f - f)); } /* df[0] is never written */
+        }
+    }
+}
+
+/* Recurrent__Update_Derivative_Weight__LSTM (NN/Neural_Network__Recurrent_Update_Derivative_Weight__OpenMP.cpp:492-728)
+ * and __LSTM__Bias (:730-776). */
+static void dw_lstm(myea_oracle_net *n, size_t li, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    olstm *q = o->lstm;
+    size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, K = q->K, C = q->C, cpb = q->cpb, In = q->In;
+    const float *x = layer_outputs(n, li - 1);
+    float *g = n->gradient;
+    long kk;
+    /* parallel over blocks: every parameter belongs to one block, so the per-parameter summation order (b, then t)
+     * is the serial one */
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+    for (kk = 0; kk < (long)K; ++kk) {
+        size_t k = (size_t)kk;
+        for (size_t b = 0; b < B; ++b)
+            for (size_t t = 0; t < T; ++t) {
+                int last = t == T - 1;
+                size_t kb = b * K + Bmax * K * t, cb = b * C + Bmax * C * t, kn = b * K + Bmax * K * (t + 1), cn = b * C + Bmax * C * (t + 1);
+                const float *xi = x + b * In + Bmax * In * t, *h = o->values + cb;
+                for (size_t j = 0; j < cpb; ++j) {
+                    size_t c = k * cpb + j;
+                    float e = q->dz[cb + c];
+                    float *gw = g + lstm_z_in(l, q, k, j);
+                    for (size_t a = 0; a < In; ++a) gw[a] += e * xi[a];
+                    if (!last) {
+                        e = q->dz[cn + c];
+                        gw = g + lstm_z_rec(l, q, k, j);
+                        for (size_t a = 0; a < C; ++a) gw[a] += e * h[a];
+                    }
+                }
+                float ei = q->di[kb + k], ef = q->df[kb + k], eo = q->dgo[kb + k];
+                float *gi_ = g + lstm_gate_in(l, q, k, 0), *gf_ = g + lstm_gate_in(l, q, k, 1), *go_ = g + lstm_gate_in(l, q, k, 2);
+                for (size_t a = 0; a < In; ++a) { gi_[a] += ei * xi[a]; gf_[a] += ef * xi[a]; go_[a] += eo * xi[a]; }
+                float *pi = g + lstm_peep(l, q, k, 0), *pf = g + lstm_peep(l, q, k, 1), *po = g + lstm_peep(l, q, k, 2);
+                if (!last) {
+                    ei = q->di[kn + k]; ef = q->df[kn + k];
+                    for (size_t j = 0; j < cpb; ++j) { float cs = q->c[cb + k * cpb + j]; pi[j] += ei * cs; pf[j] += ef * cs; po[j] += eo * cs; }
+                    eo = q->dgo[kn + k];
+                    gi_ = g + lstm_gate_rec(l, q, k, 0); gf_ = g + lstm_gate_rec(l, q, k, 1); go_ = g + lstm_gate_rec(l, q, k, 2);
+                    for (size_t a = 0; a < C; ++a) { gi_[a] += ei * h[a]; gf_[a] += ef * h[a]; go_[a] += eo * h[a]; }
+                } else {
+                    for (size_t j = 0; j < cpb; ++j) po[j] += eo * q->c[cb + k * cpb + j];
+                }
+            }
+    }
+    float *bz = g + l->first_bias_connection_index, *bi = bz + C, *bf = bi + K, *bo = bf + K;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t t = 0; t < T; ++t) {
+            size_t kb = b * K + Bmax * K * t, cb = b * C + Bmax * C * t;
+            for (size_t c = 0; c < C; ++c) bz[c] += q->dz[cb + c];
+            for (size_t k = 0; k < K; ++k) { bi[k] += q->di[kb + k]; bf[k] += q->df[kb + k]; bo[k] += q->dgo[kb + k]; }
+        }
+}
+
 /* FF__Forward_Pass_Batch: NN/Neural_Network__Forward_Pass__OpenMP.cpp:24-120;
  * RNN__Forward_Pass_Batch: NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:24-130 (layer-major,
  * every layer loops over t); FF/RNN__Assign_Inputs: NN/Neural_Network__Assign_Inputs.cpp:20-204
@@ -442,6 +722,8 @@ int myea_oracle_forward_pass(myea_oracle_net *n, size_t B, const float *inputs)
         const myea_layer_desc *l = &n->d.layers[li];
         if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             for (size_t t = 0; t < T; ++t) fwd_fc_layer(n, li, t, B);
+        } else if (l->type_layer == MYEA_LAYER_LSTM) {
+            for (size_t t = 0; t < T; ++t) fwd_lstm_step(n, li, t, B);
         } else return MYEA_E_UNSUPPORTED;
     }
     return MYEA_OK;
@@ -521,7 +803,10 @@ int myea_oracle_compute_error(myea_oracle_net *n, size_t B, const float *desired
                 update_error(n, y[j], d[j], diff);
                 switch (n->h.type_accuracy_function) {
                 case MYEA_ACCURACY_DISTANCE: if (fabsf(diff) <= n->h.accuracy_variance) n->loss.accuracy_value += 1.0; break;
-                case MYEA_ACCURACY_DIRECTIONAL: n->loss.accuracy_value += 1.0; break;
+                case MYEA_ACCURACY_DIRECTIONAL:
+                    /* RNN: direction of change against the previous target (NN/Neural_Network__Recurrent_Compute__Error__OpenMP.cpp:115-120) */
+                    if (!rnn || t == 0 || sign_f(d[j] - (d - H)[j]) == sign_f(y[j] - (d - H)[j])) n->loss.accuracy_value += 1.0;
+                    break;
                 case MYEA_ACCURACY_SIGN:
                     if (sign_f(d[j]) == sign_f(y[j]) || (sign_f(d[j]) == 0.f && y[j] >= -FLT_EPSILON && y[j] <= FLT_EPSILON)) n->loss.accuracy_value += 1.0;
                     break;
@@ -648,9 +933,13 @@ int myea_oracle_backward_pass(myea_oracle_net *n, size_t B)
         if (next->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             for (size_t tt = T; tt-- > 0;)
                 bwd_fc(n, tt, B, n->L[gi].H, o->H, n->L[gi].neuron_errors, n->parameters + next->first_connection_index, dst);
+        } else if (next->type_layer == MYEA_LAYER_LSTM) {
+            for (size_t tt = 0; tt < T; ++tt) bwd_lstm_to_previous(n, gi, tt, B, dst);
         } else return MYEA_E_UNSUPPORTED;
         if (n->d.layers[li].type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             for (size_t tt = T; tt-- > 0;) bwd_gradient_fc(n, li, tt, B);
+        } else if (n->d.layers[li].type_layer == MYEA_LAYER_LSTM) {
+            for (size_t tt = T; tt-- > 0;) bwd_lstm_step(n, li, tt, B);
         } else return MYEA_E_UNSUPPORTED;
     }
     return MYEA_OK;
@@ -696,6 +985,7 @@ int myea_oracle_update_derivative_weight(myea_oracle_net *n, size_t B, size_t fi
     for (size_t li = first; li < end; ++li) {
         const myea_layer_desc *l = &n->d.layers[li];
         if (l->type_layer == MYEA_LAYER_RESIDUAL) continue;
+        if (l->type_layer == MYEA_LAYER_LSTM) { dw_lstm(n, li, B); continue; }
         if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_UNSUPPORTED;
         olayer *o = &n->L[li];
         const float *x = layer_outputs(n, li - 1);
@@ -811,6 +1101,24 @@ const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t 
     case MYEA_TENSOR_NORM_MEANS_AVERAGES: p = o->means_averages; c = th; break;
     case MYEA_TENSOR_NORM_VARIANCES_AVERAGES: p = o->variances_averages; c = th; break;
     default: break;
+    }
+    if (o->lstm) {
+        olstm *q = o->lstm;
+        size_t cc = T * n->d.batch_size * q->C, kk = T * n->d.batch_size * q->K;
+        switch (kind) {
+        case MYEA_TENSOR_ERRORS: p = o->af_errors; c = cc; break;
+        case MYEA_TENSOR_LSTM_CELL_INPUT: p = q->z; c = cc; break;
+        case MYEA_TENSOR_LSTM_CELL_STATE: p = q->c; c = cc; break;
+        case MYEA_TENSOR_LSTM_INPUT_GATE: p = q->gi; c = kk; break;
+        case MYEA_TENSOR_LSTM_FORGET_GATE: p = q->gf; c = kk; break;
+        case MYEA_TENSOR_LSTM_OUTPUT_GATE: p = q->go; c = kk; break;
+        case MYEA_TENSOR_LSTM_DELTA_CELL_INPUT: p = q->dz; c = cc; break;
+        case MYEA_TENSOR_LSTM_DELTA_CELL_STATE: p = q->dc; c = cc; break;
+        case MYEA_TENSOR_LSTM_DELTA_INPUT_GATE: p = q->di; c = kk; break;
+        case MYEA_TENSOR_LSTM_DELTA_FORGET_GATE: p = q->df; c = kk; break;
+        case MYEA_TENSOR_LSTM_DELTA_OUTPUT_GATE: p = q->dgo; c = kk; break;
+        default: break;
+        }
     }
     if (count) *count = p ? c : 0;
     return p;
