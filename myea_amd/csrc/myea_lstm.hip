@@ -1,16 +1,495 @@
-// myea_lstm.hip — LSTM-with-peephole layers (placeholder until the BPTT kernels land).
+// myea_lstm.hip — LSTM-with-peephole layers on gfx950: forward, BPTT and weight gradients.
+//
+// MI355X-first structure.  The reference keeps the gate weights interleaved per block inside the flat parameter
+// vector (Prepare__Connections__LSTM, Neural_Network__Prepare_Connections.cpp:82-222) and walks them with scalar
+// dot products per example.  Here the flat vector stays the source of truth (upload / download / optimizer run
+// on it unchanged) and a packed device copy feeds the MFMA contractions:
+//     Win  [G][In],  Wrec [G][C],  peep [3][C],   rows ordered  z (C cells) | i (K) | f (K) | o (K),  G = C + 3K
+// refreshed by one gather kernel whenever the parameters change.  With that order the four bias vectors are one
+// contiguous [G] slice of the flat vector at Layer::first_bias_connection_index, exactly where the reference reads
+// them.  Per layer:
+//   forward   one contraction over all time steps for the input sums  (T*B x G x In),
+//             per step one contraction h[t-1] Wrec^T accumulated onto them and one fused gate kernel;
+//   backward  per step one contraction dG[t+1] Wrec accumulated onto dh[t] and one fused gate-delta kernel,
+//             then ONE contraction dG Win for the layer below;
+//   weights   two contractions dG^T X (K = T*B) and dG[1..]^T h[..T-2] into packed scratch + scatter-add into the
+//             flat gradient, a column reduction for the three peephole vectors, a column sum for the biases.
+//
+// NN/ = Neural_Network_Library_Windows/Source_Files/Neural_Network/.
+#include "myea_device_af.h"
 #include "myea_kernels.h"
 #include "myea_net.h"
+#include "myea_reduce.h"
 
 namespace myea {
 
-int Net::lstm_create_layer(size_t li) { set_last_error("layer %zu: LSTM layers are not built yet", li); return MYEA_E_UNSUPPORTED; }
-void Net::lstm_destroy_layer(DevLayer &) {}
-int Net::lstm_parameters_changed() { return MYEA_OK; }
-int Net::lstm_forward_layer(size_t li, size_t) { set_last_error("layer %zu: LSTM forward not built", li); return MYEA_E_UNSUPPORTED; }
-int Net::lstm_backward_into_layer(size_t li, size_t) { set_last_error("layer %zu: LSTM backward not built", li); return MYEA_E_UNSUPPORTED; }
-int Net::lstm_backward_layer(size_t li, size_t) { set_last_error("layer %zu: LSTM backward not built", li); return MYEA_E_UNSUPPORTED; }
-int Net::lstm_update_derivative_weight(size_t li, size_t) { set_last_error("layer %zu: LSTM dW not built", li); return MYEA_E_UNSUPPORTED; }
-const float *Net::lstm_tensor(size_t, int, size_t *count) { if (count) *count = 0; return nullptr; }
+struct LstmLayer {
+    size_t K = 0, cpb = 0, C = 0, G = 0, In = 0, per_block = 0, base = 0;
+    float *Win = nullptr, *Wrec = nullptr, *peep = nullptr;      // packed parameters
+    float *gWin = nullptr, *gWrec = nullptr;                     // packed gradient scratch
+    float *acts = nullptr;  // [T][Bmax][G]: pre-activation sums, overwritten in place by z | i | f | o
+    float *c = nullptr, *ca = nullptr;                           // [T][Bmax][C] cell state and tanh(cell state)
+    float *dG = nullptr;    // [T][Bmax][G] deltas dz | di | df | do
+    float *dc = nullptr;    // [T][Bmax][C]
+};
+
+namespace {
+
+#define MYEA_TRY(expr)                    \
+    do {                                  \
+        int rc__ = (expr);                \
+        if (rc__ != MYEA_OK) return rc__; \
+    } while (0)
+
+struct LstmGeom {
+    size_t K, cpb, C, G, In, per_block, base;
+};
+
+// flat index of packed element (row r of Win / Wrec, column a), NN/Neural_Network__Prepare_Connections.cpp:123-217
+__device__ __forceinline__ size_t flat_index(const LstmGeom &g, size_t r, size_t a, bool recurrent)
+{
+    if (r < g.C) {
+        const size_t k = r / g.cpb, j = r % g.cpb;
+        return g.base + k * g.per_block + j * (g.In + g.C) + (recurrent ? g.In + a : a);
+    }
+    const size_t gate = (r - g.C) / g.K, k = (r - g.C) % g.K;
+    const size_t gates0 = g.base + k * g.per_block + g.cpb * (g.In + g.C);
+    return recurrent ? gates0 + 3 * g.In + gate * g.C + a : gates0 + gate * g.In + a;
+}
+__device__ __forceinline__ size_t peep_index(const LstmGeom &g, size_t gate, size_t c)
+{
+    const size_t k = c / g.cpb, j = c % g.cpb;
+    return g.base + k * g.per_block + g.cpb * (g.In + g.C) + 3 * g.In + 3 * g.C + gate * g.cpb + j;
+}
+
+__global__ __launch_bounds__(kBlock) void lstm_gather_kernel(LstmGeom g, const float *flat, float *Win, float *Wrec, float *peep)
+{
+    const size_t n_in = g.G * g.In, n_rec = g.G * g.C, n_peep = 3 * g.C, n = n_in + n_rec + n_peep;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        if (i < n_in) Win[i] = flat[flat_index(g, i / g.In, i % g.In, false)];
+        else if (i < n_in + n_rec) { const size_t q = i - n_in; Wrec[q] = flat[flat_index(g, q / g.C, q % g.C, true)]; }
+        else { const size_t q = i - n_in - n_rec; peep[q] = flat[peep_index(g, q / g.C, q % g.C)]; }
+    }
+}
+
+// flat gradient += packed gradient (every flat slot is owned by exactly one packed element: no atomics)
+__global__ __launch_bounds__(kBlock) void lstm_scatter_add_kernel(LstmGeom g, float *flat, const float *gWin, const float *gWrec, int with_rec)
+{
+    const size_t n_in = g.G * g.In, n_rec = with_rec ? g.G * g.C : 0, n = n_in + n_rec;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        if (i < n_in) flat[flat_index(g, i / g.In, i % g.In, false)] += gWin[i];
+        else { const size_t q = i - n_in; flat[flat_index(g, q / g.C, q % g.C, true)] += gWrec[q]; }
+    }
+}
+
+__device__ __forceinline__ float sigmoid_f(float s) { return 1.f / (1.f + expf(-s)); }
+__device__ __forceinline__ float tanh_f(float s) { return 2.f / (1.f + expf(-2.f * s)) - 1.f; }  // AF_TANH_real
+
+// One lane per (example, block).  Forward_Pass__LSTM__Gates_CIF_AF_State (NN/Neural_Network__Recurrent_Forward_Pass__
+// OpenMP.cpp:1042-1191), __States_AF (:1547-1582), __Output (:1351-1418).  `acts` holds input + recurrent sums on
+// entry (the contraction accumulated them) and the activations on exit.  First step: no forget gate, no input-gate
+// peephole, c = i z; the output gate peeps at c[t].
+__global__ __launch_bounds__(kBlock) void lstm_forward_step_kernel(LstmGeom g, size_t B, int first, const float *bias, const float *peep,
+                                                                   float *acts, const float *c_prev, float *c, float *ca, float *h)
+{
+    const size_t n = B * g.K;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < n; idx += (size_t)gridDim.x * kBlock) {
+        const size_t b = idx / g.K, k = idx % g.K;
+        float *row = acts + b * g.G;
+        const size_t cell0 = b * g.C + k * g.cpb;
+        const float *pi = peep + k * g.cpb, *pf = peep + g.C + k * g.cpb, *po = peep + 2 * g.C + k * g.cpb;
+        float si = row[g.C + k] + bias[g.C + k];
+        float gi, gf = 0.f;
+        if (!first) {
+            float sf = row[g.C + g.K + k] + bias[g.C + g.K + k];
+            for (size_t j = 0; j < g.cpb; ++j) { const float cp = c_prev[cell0 + j]; si += cp * pi[j]; sf += cp * pf[j]; }
+            gf = sigmoid_f(sf);
+        }
+        gi = sigmoid_f(si);
+        row[g.C + k] = gi;
+        row[g.C + g.K + k] = gf;
+        float so = row[g.C + 2 * g.K + k] + bias[g.C + 2 * g.K + k];
+        for (size_t j = 0; j < g.cpb; ++j) {
+            const size_t cc = k * g.cpb + j;
+            const float z = tanh_f(row[cc] + bias[cc]);
+            row[cc] = z;
+            const float cs = first ? z * gi : z * gi + gf * c_prev[cell0 + j];
+            c[cell0 + j] = cs;
+            ca[cell0 + j] = tanh_f(cs);
+            so += cs * po[j];
+        }
+        const float go = sigmoid_f(so);
+        row[g.C + 2 * g.K + k] = go;
+        for (size_t j = 0; j < g.cpb; ++j) h[cell0 + j] = ca[cell0 + j] * go;
+    }
+}
+
+// One lane per (example, block).  Backward_Pass__LSTM_Derivative__Output (elementwise part, NN/Neural_Network__
+// Recurrent_Backward_Pass__OpenMP.cpp:1228-1240), __Cell_State_AF (:1275-1327), __Gates_CIF_AF_State (:1329-1604).
+// dh[t] already holds the delta from the layers above plus the recurrent term dG[t+1] Wrec.
+//   mode 0: T == 1            (no gate deltas are computed: no branch of the reference matches)
+//   mode 1: last step, T > 1  (only the output-gate peephole term; delta i and delta f computed)
+//   mode 2: middle step       (all future terms)
+//   mode 3: first step, T > 1 (all future terms; delta f is not written)
+__global__ __launch_bounds__(kBlock) void lstm_backward_step_kernel(LstmGeom g, size_t B, int mode, const float *peep, const float *acts,
+                                                                    const float *acts_next, const float *c_prev, const float *ca,
+                                                                    const float *dh, float *dG, const float *dG_next, float *dc,
+                                                                    const float *dc_next)
+{
+    const size_t n = B * g.K;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < n; idx += (size_t)gridDim.x * kBlock) {
+        const size_t b = idx / g.K, k = idx % g.K;
+        const float *row = acts + b * g.G;
+        float *drow = dG + b * g.G;
+        const size_t cell0 = b * g.C + k * g.cpb;
+        const float gi = row[g.C + k], gf = row[g.C + g.K + k], go = row[g.C + 2 * g.K + k];
+        float eo = 0.f;
+        for (size_t j = 0; j < g.cpb; ++j) eo += dh[cell0 + j] * ca[cell0 + j];
+        const float ddo = go * (1.f - go) * eo;
+        drow[g.C + 2 * g.K + k] = ddo;
+        if (mode == 0) {
+            for (size_t j = 0; j < g.cpb; ++j) {
+                const float a = ca[cell0 + j];
+                dc[cell0 + j] = dh[cell0 + j] * go * (1.f - a * a);
+                drow[k * g.cpb + j] = 0.f;
+            }
+            drow[g.C + k] = 0.f;
+            drow[g.C + g.K + k] = 0.f;
+            continue;
+        }
+        const bool future = mode >= 2;
+        float di_n = 0.f, df_n = 0.f, f_n = 0.f;
+        if (future) {
+            di_n = dG_next[b * g.G + g.C + k];
+            df_n = dG_next[b * g.G + g.C + g.K + k];
+            f_n = acts_next[b * g.G + g.C + g.K + k];
+        }
+        const float *pi = peep + k * g.cpb, *pf = peep + g.C + k * g.cpb, *po = peep + 2 * g.C + k * g.cpb;
+        float ei = 0.f, ef = 0.f;
+        for (size_t j = 0; j < g.cpb; ++j) {
+            const float a = ca[cell0 + j], z = row[k * g.cpb + j];
+            float e = dh[cell0 + j] * go * (1.f - a * a);
+            e += po[j] * ddo;
+            if (future) {
+                e += pi[j] * di_n;
+                e += pf[j] * df_n;
+                e += dc_next[cell0 + j] * f_n;
+            }
+            dc[cell0 + j] = e;
+            drow[k * g.cpb + j] = e * gi * (1.f - z * z);
+            ei += e * z;
+            if (mode != 3) ef += e * c_prev[cell0 + j];
+        }
+        drow[g.C + k] = ei * (gi * (1.f - gi));
+        drow[g.C + g.K + k] = mode != 3 ? ef * (gf * (1.f - gf)) : 0.f;
+    }
+}
+
+// peephole gradients (NN/Neural_Network__Recurrent_Update_Derivative_Weight__OpenMP.cpp:603-625,673-683):
+//   dp_i += di[t+1] c[t], dp_f += df[t+1] c[t] for t < T-1;  dp_o += do[t] c[t] for all t.
+// rows of the reduction are (t, b) pairs; columns are cells.
+struct PeepF {
+    LstmGeom g;
+    size_t B, Bmax, T;
+    const float *c, *dG;
+    __device__ void operator()(size_t r, size_t col, double *acc) const
+    {
+        const size_t t = r / B, b = r % B, k = col / g.cpb;
+        const size_t row = t * Bmax + b;
+        const float cs = c[row * g.C + col];
+        acc[2] += dG[row * g.G + g.C + 2 * g.K + k] * cs;
+        if (t + 1 < T) {
+            const size_t nrow = (t + 1) * Bmax + b;
+            acc[0] += dG[nrow * g.G + g.C + k] * cs;
+            acc[1] += dG[nrow * g.G + g.C + g.K + k] * cs;
+        }
+    }
+};
+
+__global__ __launch_bounds__(kBlock) void lstm_peep_final_kernel(LstmGeom g, size_t S, const float *partial, float *flat_gradient)
+{
+    const size_t c = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (c >= g.C) return;
+    for (size_t gate = 0; gate < 3; ++gate) {
+        double s = 0.0;
+        for (size_t y = 0; y < S; ++y) s += partial[(y * 3 + gate) * g.C + c];
+        flat_gradient[peep_index(g, gate, c)] += (float)s;
+    }
+}
+
+// column sums over (t, b) rows of a [T][Bmax][W] tensor when B < Bmax (rows are not contiguous)
+struct StridedSumF {
+    size_t B, Bmax, W;
+    const float *x;
+    __device__ void operator()(size_t r, size_t col, double *acc) const { acc[0] += x[((r / B) * Bmax + r % B) * W + col]; }
+};
+__global__ __launch_bounds__(kBlock) void lstm_colsum_final_kernel(size_t H, size_t S, const float *partial, float *out)
+{
+    const size_t col = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (col >= H) return;
+    double s = 0.0;
+    for (size_t y = 0; y < S; ++y) s += partial[y * H + col];
+    out[col] += (float)s;
+}
+
+int dev_alloc_zero(float **p, size_t count)
+{
+    void *q = nullptr;
+    const size_t bytes = (count ? count : 1) * sizeof(float);
+    hipError_t e = hipMalloc(&q, bytes);
+    if (e != hipSuccess) { hip_fail(e, "hipMalloc"); return MYEA_E_NOMEM; }
+    e = hipMemset(q, 0, bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipMemset");
+    *p = static_cast<float *>(q);
+    return MYEA_OK;
+}
+
+LstmGeom geom_of(const LstmLayer &q) { return LstmGeom{q.K, q.cpb, q.C, q.G, q.In, q.per_block, q.base}; }
+
+}  // namespace
+
+int Net::lstm_create_layer(size_t li)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    if (l.use_bidirectional) { set_last_error("layer %zu: bidirectional LSTM is not on this path", li); return MYEA_E_UNSUPPORTED; }
+    if (layer_uses_norm(l)) { set_last_error("layer %zu: normalisation inside an LSTM layer is not on this path", li); return MYEA_E_UNSUPPORTED; }
+    if (l.type_dropout != MYEA_DROPOUT_NONE) { set_last_error("layer %zu: dropout on an LSTM layer is not on this path", li); return MYEA_E_UNSUPPORTED; }
+    if (l.n_cells_per_block == 0) { set_last_error("layer %zu: LSTM needs at least one cell per block", li); return MYEA_E_INVALID; }
+    LstmLayer *q = new LstmLayer();
+    o.lstm = q;
+    q->K = l.n_units; q->cpb = l.n_cells_per_block; q->C = q->K * q->cpb; q->G = q->C + 3 * q->K; q->In = L[li - 1].H;
+    q->per_block = q->cpb * (q->In + q->C) + 3 * q->In + 3 * q->C + 3 * q->cpb;
+    q->base = l.first_connection_index;
+    if (q->base + q->K * q->per_block > d.total_weights) { set_last_error("layer %zu: LSTM weight slice leaves the weight region", li); return MYEA_E_INVALID; }
+    // The four bias vectors are read at first_bias_connection_index + [0, G).  With the index as Prepare__Bias__LSTM
+    // leaves it they reach C entries into the following layers' bias slots; beyond the bias region the reference would
+    // read and write outside its parameter array, which is refused here.
+    if (l.first_bias_connection_index < d.total_weights || l.first_bias_connection_index + q->G > d.total_weights + d.total_bias) {
+        set_last_error("layer %zu: LSTM bias slice [%llu, +%zu) leaves the bias region", li, (unsigned long long)l.first_bias_connection_index, q->G);
+        return MYEA_E_INVALID;
+    }
+    const size_t T = d.number_recurrent_depth, B = d.batch_size;
+    MYEA_TRY(dev_alloc_zero(&q->Win, q->G * q->In));
+    MYEA_TRY(dev_alloc_zero(&q->Wrec, q->G * q->C));
+    MYEA_TRY(dev_alloc_zero(&q->peep, 3 * q->C));
+    MYEA_TRY(dev_alloc_zero(&q->gWin, q->G * q->In));
+    MYEA_TRY(dev_alloc_zero(&q->gWrec, q->G * q->C));
+    MYEA_TRY(dev_alloc_zero(&q->acts, T * B * q->G));
+    MYEA_TRY(dev_alloc_zero(&q->c, T * B * q->C));
+    MYEA_TRY(dev_alloc_zero(&q->ca, T * B * q->C));
+    MYEA_TRY(dev_alloc_zero(&q->dG, T * B * q->G));
+    MYEA_TRY(dev_alloc_zero(&q->dc, T * B * q->C));
+    MYEA_TRY(dev_alloc_zero(&o.neuron_errors, T * B * q->C));  // delta of the cell outputs (ptr_delta_cell_output)
+    return MYEA_OK;
+}
+
+void Net::lstm_destroy_layer(DevLayer &o)
+{
+    if (!o.lstm) return;
+    LstmLayer *q = o.lstm;
+    float *all[] = {q->Win, q->Wrec, q->peep, q->gWin, q->gWrec, q->acts, q->c, q->ca, q->dG, q->dc};
+    for (float *p : all) if (p) (void)hipFree(p);
+    delete q;
+    o.lstm = nullptr;
+}
+
+size_t Net::lstm_scratch_floats() const
+{
+    size_t need = 0;
+    for (const DevLayer &o : L)
+        if (o.lstm) { const size_t n = 64 * 3 * o.lstm->C + 64 * o.lstm->G; if (n > need) need = n; }
+    return need;
+}
+
+// packed copies <- flat vector; called after every parameter upload and every optimizer update
+int Net::lstm_parameters_changed()
+{
+    for (size_t li = 1; li < L.size(); ++li) {
+        LstmLayer *q = L[li].lstm;
+        if (!q) continue;
+        const size_t n = q->G * (q->In + q->C) + 3 * q->C;
+        hipLaunchKernelGGL(lstm_gather_kernel, dim3(grid_for(n, kBlock, 4096)), dim3(kBlock), 0, stream, geom_of(*q), parameters, q->Win, q->Wrec, q->peep);
+        MYEA_HIP_TRY(hipGetLastError());
+    }
+    return MYEA_OK;
+}
+
+// Recurrent__Forward_Pass__LSTM (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:448-471), time ascending.
+int Net::lstm_forward_layer(size_t li, size_t B)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    LstmLayer &q = *o.lstm;
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
+    const float *x = layer_outputs(li - 1);
+    const float *bias = parameters + l.first_bias_connection_index;
+    // input sums of every time step in one contraction when the rows are contiguous
+    const bool per_t = T > 1 && B != Bmax;
+    const size_t chunks = per_t ? T : 1, rows = per_t ? B : T * B;
+    for (size_t c = 0; c < chunks; ++c) {
+        GemmParams g{};
+        g.A = x + c * Bmax * q.In; g.lda = (long)q.In; g.a_k_contiguous = 1;
+        g.B = q.Win; g.ldb = (long)q.In; g.b_k_contiguous = 1;
+        g.C = q.acts + c * Bmax * q.G; g.ldc = (long)q.G;
+        g.M = (int)rows; g.N = (int)q.G; g.K = (int)q.In;
+        prof_begin(0);
+        MYEA_TRY(launch_gemm(stream, g));
+        prof_end(2.0 * (double)rows * (double)q.G * (double)q.In);
+    }
+    const LstmGeom geom = geom_of(q);
+    for (size_t t = 0; t < T; ++t) {
+        float *acts_t = q.acts + t * Bmax * q.G;
+        if (t > 0) {
+            GemmParams g{};
+            g.A = o.values + (t - 1) * Bmax * q.C; g.lda = (long)q.C; g.a_k_contiguous = 1;
+            g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 1;
+            g.C = acts_t; g.ldc = (long)q.G; g.accumulate = 1;
+            g.M = (int)B; g.N = (int)q.G; g.K = (int)q.C;
+            prof_begin(0);
+            MYEA_TRY(launch_gemm(stream, g));
+            prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
+        }
+        hipLaunchKernelGGL(lstm_forward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, (int)(t == 0), bias, q.peep,
+                           acts_t, t ? q.c + (t - 1) * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, o.values + t * Bmax * q.C);
+        MYEA_HIP_TRY(hipGetLastError());
+    }
+    return MYEA_OK;
+}
+
+// Recurrent__Backward_Pass__Gradient__LSTM (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:440-862), time
+// descending; o.neuron_errors (= delta of the cell outputs) already holds what the layers above sent down.
+int Net::lstm_backward_layer(size_t li, size_t B)
+{
+    DevLayer &o = L[li];
+    LstmLayer &q = *o.lstm;
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
+    const LstmGeom geom = geom_of(q);
+    for (size_t t = T; t-- > 0;) {
+        float *dh_t = o.neuron_errors + t * Bmax * q.C;
+        const bool last = t == T - 1, first = t == 0;
+        if (!last) {  // Backward_Pass__LSTM_Derivative__Output, recurrent part (:1174-1226)
+            GemmParams g{};
+            g.A = q.dG + (t + 1) * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 1;
+            g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 0;
+            g.C = dh_t; g.ldc = (long)q.C; g.accumulate = 1;
+            g.M = (int)B; g.N = (int)q.C; g.K = (int)q.G;
+            prof_begin(1);
+            MYEA_TRY(launch_gemm(stream, g));
+            prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
+        }
+        const int mode = (first && last) ? 0 : (last ? 1 : (first ? 3 : 2));
+        hipLaunchKernelGGL(lstm_backward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, mode, q.peep,
+                           q.acts + t * Bmax * q.G, last ? nullptr : q.acts + (t + 1) * Bmax * q.G, first ? nullptr : q.c + (t - 1) * Bmax * q.C,
+                           q.ca + t * Bmax * q.C, dh_t, q.dG + t * Bmax * q.G, last ? nullptr : q.dG + (t + 1) * Bmax * q.G,
+                           q.dc + t * Bmax * q.C, last ? nullptr : q.dc + (t + 1) * Bmax * q.C);
+        MYEA_HIP_TRY(hipGetLastError());
+    }
+    return MYEA_OK;
+}
+
+// the operands of "delta of the layer below = dG Win" (Backward_Pass__LSTM, :1024-1120), handed to the shared driver
+void Net::lstm_delta_source(size_t gi, const float **delta, size_t *width, const float **weights)
+{
+    LstmLayer &q = *L[gi].lstm;
+    *delta = q.dG;
+    *width = q.G;
+    *weights = q.Win;
+}
+
+// Recurrent__Update_Derivative_Weight__LSTM (NN/Neural_Network__Recurrent_Update_Derivative_Weight__OpenMP.cpp:492-728)
+// and __LSTM__Bias (:730-776).
+int Net::lstm_update_derivative_weight(size_t li, size_t B)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    LstmLayer &q = *o.lstm;
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
+    const float *x = layer_outputs(li - 1);
+    const LstmGeom geom = geom_of(q);
+    const bool per_t = T > 1 && B != Bmax;
+    // input weights: dG^T X over every (t, b)
+    {
+        const size_t chunks = per_t ? T : 1, rows = per_t ? B : T * B;
+        for (size_t c = 0; c < chunks; ++c) {
+            GemmParams g{};
+            g.A = q.dG + c * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
+            g.B = x + c * Bmax * q.In; g.ldb = (long)q.In; g.b_k_contiguous = 0;
+            g.C = q.gWin; g.ldc = (long)q.In; g.accumulate = c > 0;
+            g.M = (int)q.G; g.N = (int)q.In; g.K = (int)rows;
+            prof_begin(2);
+            MYEA_TRY(launch_gemm(stream, g));
+            prof_end(2.0 * (double)rows * (double)q.G * (double)q.In);
+        }
+    }
+    // recurrent weights: dG[t+1]^T h[t] for t < T-1
+    const bool with_rec = T > 1;
+    if (with_rec) {
+        const size_t chunks = per_t ? T - 1 : 1, rows = per_t ? B : (T - 1) * B;
+        for (size_t c = 0; c < chunks; ++c) {
+            GemmParams g{};
+            g.A = q.dG + (c + 1) * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
+            g.B = o.values + c * Bmax * q.C; g.ldb = (long)q.C; g.b_k_contiguous = 0;
+            g.C = q.gWrec; g.ldc = (long)q.C; g.accumulate = c > 0;
+            g.M = (int)q.G; g.N = (int)q.C; g.K = (int)rows;
+            prof_begin(2);
+            MYEA_TRY(launch_gemm(stream, g));
+            prof_end(2.0 * (double)rows * (double)q.G * (double)q.C);
+        }
+    }
+    hipLaunchKernelGGL(lstm_scatter_add_kernel, dim3(grid_for(q.G * (q.In + q.C), kBlock, 4096)), dim3(kBlock), 0, stream, geom, gradient, q.gWin, q.gWrec,
+                       (int)with_rec);
+    MYEA_HIP_TRY(hipGetLastError());
+    // peepholes
+    {
+        size_t S, chunk;
+        split_rows(T * B, q.C, S, chunk);
+        PeepF f{geom, B, Bmax, T, q.c, q.dG};
+        hipLaunchKernelGGL((column_partial_kernel<3, PeepF>), dim3((unsigned)((q.C + 63) / 64), (unsigned)S), dim3(kBlock), 0, stream, T * B, q.C, chunk, scratch, f);
+        MYEA_HIP_TRY(hipGetLastError());
+        hipLaunchKernelGGL(lstm_peep_final_kernel, dim3(grid_for(q.C, kBlock)), dim3(kBlock), 0, stream, geom, S, scratch, gradient);
+        MYEA_HIP_TRY(hipGetLastError());
+    }
+    // the four bias vectors: one contiguous [G] slice in the order z | i | f | o
+    {
+        size_t S, chunk;
+        split_rows(T * B, q.G, S, chunk);
+        StridedSumF f{B, Bmax, q.G, q.dG};
+        hipLaunchKernelGGL((column_partial_kernel<1, StridedSumF>), dim3((unsigned)((q.G + 63) / 64), (unsigned)S), dim3(kBlock), 0, stream, T * B, q.G, chunk, scratch, f);
+        MYEA_HIP_TRY(hipGetLastError());
+        hipLaunchKernelGGL(lstm_colsum_final_kernel, dim3(grid_for(q.G, kBlock)), dim3(kBlock), 0, stream, q.G, S, scratch, gradient + l.first_bias_connection_index);
+        MYEA_HIP_TRY(hipGetLastError());
+    }
+    return MYEA_OK;
+}
+
+const float *Net::lstm_tensor(size_t li, int kind, size_t *count)
+{
+    if (count) *count = 0;
+    LstmLayer *q = L[li].lstm;
+    if (!q) return nullptr;
+    // The device keeps gate tensors packed as rows of [G]; taps are served from small staging copies.
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, rows = T * Bmax;
+    const float *src = nullptr;
+    size_t width = 0, offset = 0, ld = 0;
+    switch (kind) {
+    case MYEA_TENSOR_LSTM_CELL_STATE: if (count) *count = rows * q->C; return q->c;
+    case MYEA_TENSOR_LSTM_DELTA_CELL_STATE: if (count) *count = rows * q->C; return q->dc;
+    case MYEA_TENSOR_LSTM_CELL_INPUT: src = q->acts; width = q->C; offset = 0; break;
+    case MYEA_TENSOR_LSTM_INPUT_GATE: src = q->acts; width = q->K; offset = q->C; break;
+    case MYEA_TENSOR_LSTM_FORGET_GATE: src = q->acts; width = q->K; offset = q->C + q->K; break;
+    case MYEA_TENSOR_LSTM_OUTPUT_GATE: src = q->acts; width = q->K; offset = q->C + 2 * q->K; break;
+    case MYEA_TENSOR_LSTM_DELTA_CELL_INPUT: src = q->dG; width = q->C; offset = 0; break;
+    case MYEA_TENSOR_LSTM_DELTA_INPUT_GATE: src = q->dG; width = q->K; offset = q->C; break;
+    case MYEA_TENSOR_LSTM_DELTA_FORGET_GATE: src = q->dG; width = q->K; offset = q->C + q->K; break;
+    case MYEA_TENSOR_LSTM_DELTA_OUTPUT_GATE: src = q->dG; width = q->K; offset = q->C + 2 * q->K; break;
+    default: return nullptr;
+    }
+    ld = q->G;
+    // strided copy of the column band into tmp1 (large enough: rows * max width)
+    if (hipMemcpy2DAsync(tmp1, width * sizeof(float), src + offset, ld * sizeof(float), width * sizeof(float), rows, hipMemcpyDeviceToDevice, stream) != hipSuccess) return nullptr;
+    if (count) *count = rows * width;
+    return tmp1;
+}
 
 }  // namespace myea

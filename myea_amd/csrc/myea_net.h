@@ -61,7 +61,7 @@ struct Net {
     int forward_fc_layer(size_t li, size_t B);
     int bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training);
     int bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx);
-    int backward_into_fc_layer(size_t li, size_t B);
+    int backward_into_layer(size_t li, size_t B);
 
     int forward_pass(size_t B, const float *inputs, int on_device);
     int compute_error(size_t B, const float *desired, int on_device);
@@ -74,8 +74,10 @@ struct Net {
     void lstm_destroy_layer(DevLayer &o);
     int lstm_parameters_changed();
     int lstm_forward_layer(size_t li, size_t B);
-    int lstm_backward_into_layer(size_t li, size_t B);  // delta of layer li from an LSTM consumer li + 1
     int lstm_backward_layer(size_t li, size_t B);       // BPTT inside LSTM layer li
+    // delta / weight operands an LSTM consumer gi offers to the layer below: delta [T][Bmax][width], weights [width][fan-in]
+    void lstm_delta_source(size_t gi, const float **delta, size_t *width, const float **weights);
+    size_t lstm_scratch_floats() const;
     int lstm_update_derivative_weight(size_t li, size_t B);
     const float *lstm_tensor(size_t li, int kind, size_t *count);
 };

@@ -164,7 +164,11 @@ int Net::create(const myea_net_desc &desc)
     }
     MYEA_TRY(dev_alloc(&tmp1, T * B * max_h));
     MYEA_TRY(dev_alloc(&tmp2, T * B * max_h));
-    MYEA_TRY(dev_alloc(&scratch, 258 * max_h + 2048));
+    {
+        size_t need = 258 * max_h + 2048;
+        if (lstm_scratch_floats() > need) need = lstm_scratch_floats();
+        MYEA_TRY(dev_alloc(&scratch, need));
+    }
     MYEA_TRY(dev_alloc(&stage_in, T * B * L[0].H));
     MYEA_TRY(dev_alloc(&stage_out, T * B * L[d.n_layers - 1].H));
     {
@@ -351,23 +355,35 @@ int Net::compute_error(size_t B, const float *desired, int on_device)
 // output layer, dX = delta_next * W_next (Backward_Pass__FC, :1044-1082) and then
 // Backward_Pass__Gradient__FC (:544-709): [BN after] -> act' -> [BN before].  The act' multiply is fused
 // into the dX contraction's epilogue whenever it directly follows it.
-int Net::backward_into_fc_layer(size_t li, size_t B)
+int Net::backward_into_layer(size_t li, size_t B)
 {
     const size_t gi = li + 1;
     const myea_layer_desc &l = d.layers[li], &next = d.layers[gi];
     DevLayer &o = L[li], &on = L[gi];
-    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, H = o.H, Out = on.H;
-    const bool norm = layer_uses_norm(l), before = l.use_layer_normalization_before_activation != 0;
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, H = o.H;
+    // what the consumer hands down: delta [T][Bmax][Out] and weights [Out][H]
+    const float *delta = on.neuron_errors, *weights = parameters + next.first_connection_index;
+    size_t Out = on.H;
+    if (next.type_layer == MYEA_LAYER_LSTM) lstm_delta_source(gi, &delta, &Out, &weights);
+    const bool is_fc = l.type_layer == MYEA_LAYER_FULLY_CONNECTED;
+    const bool norm = is_fc && layer_uses_norm(l), before = l.use_layer_normalization_before_activation != 0;
     const bool per_t = T > 1 && (B != Bmax || norm);
     const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
-    if (next.type_layer != MYEA_LAYER_FULLY_CONNECTED) return lstm_backward_into_layer(li, B);
     for (size_t c = 0; c < chunks; ++c) {
         const size_t roff = c * Bmax;
         GemmParams g{};
-        g.A = on.neuron_errors + roff * Out; g.lda = (long)Out; g.a_k_contiguous = 1;
-        g.B = parameters + next.first_connection_index; g.ldb = (long)H; g.b_k_contiguous = 0;
+        g.A = delta + roff * Out; g.lda = (long)Out; g.a_k_contiguous = 1;
+        g.B = weights; g.ldb = (long)H; g.b_k_contiguous = 0;
         g.M = (int)rows; g.N = (int)H; g.K = (int)Out;
         g.ldc = (long)H;
+        if (!is_fc) {  // an LSTM layer receives the plain delta of its cell outputs; BPTT follows
+            g.C = o.neuron_errors + roff * H;
+            g.epilogue = EPI_NONE;
+            prof_begin(1);
+            MYEA_TRY(launch_gemm(stream, g));
+            prof_end(2.0 * (double)rows * (double)H * (double)Out);
+            continue;
+        }
         g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
         const bool fuse = gemm_can_fuse_activation(g.act);
         if (!norm) {
@@ -417,8 +433,8 @@ int Net::backward_pass(size_t B)
     if (state != MYEA_STATE_TRAINING) { set_last_error("Backward_Pass: can not back propagate gradient in inference mode"); return MYEA_E_STATE; }
     for (size_t gi = d.n_layers - 1; gi >= 2; --gi) {
         const size_t li = gi - 1;
-        if (d.layers[li].type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(backward_into_fc_layer(li, B));
-        else MYEA_TRY(lstm_backward_layer(li, B));
+        MYEA_TRY(backward_into_layer(li, B));
+        if (d.layers[li].type_layer == MYEA_LAYER_LSTM) MYEA_TRY(lstm_backward_layer(li, B));
     }
     return MYEA_OK;
 }
@@ -504,7 +520,8 @@ int Net::update_parameter(size_t B, size_t training_size)
     prof_begin(3);
     const int rc = launch_update(stream, p);
     prof_end(bytes_per_param * (double)p.n);
-    return rc;
+    if (rc != MYEA_OK) return rc;
+    return lstm_parameters_changed();  // refresh the packed gate matrices
 }
 
 }  // namespace myea
