@@ -20,6 +20,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per contraction launch (mean over the launches of one step) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of this script, scaled by what the same counters read for copies of known size (FETCH_SIZE x2, WRITE_SIZE x1);
+# the per-kernel figures are in profiles/hbm_traffic__*__pmc.txt.  None where no counter run has been made.
+PMC_TRAFFIC_BYTES_PER_GEMM_LAUNCH = {"fc4096x4_b1024_adam": 2930703 * 1024 / 14}
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
@@ -28,6 +32,10 @@ WORKLOADS = {
     "fc4096x4_b1024_adam": dict(
         layers=[dict(units=4096)] + [dict(units=4096, activation="RELU")] * 4 + [dict(units=1000, activation="SOFTMAX")],
         batch=1024, head="SOFTMAX", optimizer="ADAM", loss="CROSS_ENTROPY", data="normal", hyper={}),
+    # BASELINE.json configs[2]: 2 x LSTM-512 with peepholes, input 128, T = 64, batch 256, linear FC-512 head, MSE, AMSGrad
+    "lstm512x2_t64_b256_amsgrad": dict(
+        layers=[dict(units=128), dict(type="lstm", units=512), dict(type="lstm", units=512), dict(units=512, activation="LINEAR")],
+        batch=256, depth=64, head="LINEAR", optimizer="AMSGRAD", loss="MSE", data="normal", hyper={}),
     # BASELINE.json configs[0] (the reference's own CPU-sized case)
     "mlp784_256_10_b128_sgd": dict(
         layers=[dict(units=784), dict(units=256, activation="TANH"), dict(units=10, activation="SIGMOID")],
@@ -41,18 +49,31 @@ WORKLOADS = {
 }
 
 
-def gemm_flops_per_step(layers, batch):
-    """2*M*N*K of forward, dX (layers 2..) and dW."""
-    w = [l["units"] for l in layers]
-    fwd = sum(2.0 * batch * w[i] * w[i - 1] for i in range(1, len(w)))
-    dx = sum(2.0 * batch * w[i] * w[i - 1] for i in range(2, len(w)))
+def gemm_flops_per_step(layers, batch, depth=1):
+    """2*M*N*K of forward, dX (layers 2..) and dW; LSTM layers: 4 gate rows per cell, input contraction at every
+    step, recurrent contraction at T-1 steps."""
+    w = [l["units"] * l.get("cells_per_block", 1) for l in layers]
+    fwd = dx = 0.0
+    for i in range(1, len(w)):
+        if layers[i].get("type") == "lstm":
+            gates = w[i] + 3 * layers[i]["units"]
+            f_in, f_rec = 2.0 * batch * depth * gates * w[i - 1], 2.0 * batch * (depth - 1) * gates * w[i]
+            fwd += f_in + f_rec
+            dx += f_rec + (f_in if i >= 2 else 0.0)
+        else:
+            f = 2.0 * batch * depth * w[i] * w[i - 1]
+            fwd += f
+            dx += f if i >= 2 else 0.0
     return fwd + dx + fwd
 
 
 def make_inputs(np, wl, seed):
     rng = np.random.default_rng(seed)
-    B, n_in, n_out = wl["batch"], wl["layers"][0]["units"], wl["layers"][-1]["units"]
+    T = wl.get("depth", 1)
+    B, n_in, n_out = wl["batch"], wl["layers"][0]["units"] * T, wl["layers"][-1]["units"]
     X = (rng.normal(0, 1, (B, n_in)) if wl["data"] == "normal" else rng.uniform(0, 1, (B, n_in))).astype(np.float32)
+    if wl["loss"] == "MSE" and T > 1:
+        return X, rng.normal(0, 1, (B, T * n_out)).astype(np.float32)
     Y = np.zeros((B, n_out), dtype=np.float32)
     Y[np.arange(B), rng.integers(0, n_out, B)] = 1.0
     return X, Y
@@ -67,7 +88,7 @@ def cpu_baseline(wl, sample_rows, threads):
     from tests.common import glorot_parameters
     from tests.oracle_lib import OracleNetwork, load_oracle
     lib = load_oracle()
-    desc = mb.make_desc(wl["layers"], sample_rows, lib=lib)
+    desc = mb.make_desc(wl["layers"], sample_rows, wl.get("depth", 1), lib=lib)
     h = mb.default_hyper(lib=lib, type_optimizer_function=mb.OPTIMIZER[wl["optimizer"]], type_loss_function=mb.LOSS[wl["loss"]], **wl["hyper"])
     net = OracleNetwork(desc, h, threads=threads)
     net.set_state_propagation(mb.STATE_TRAINING)
@@ -117,7 +138,7 @@ def main():
         sys.exit("bench.py: no GPU visible")
     wl = WORKLOADS[args.workload]
     B = wl["batch"]
-    desc = mb.make_desc(wl["layers"], B)
+    desc = mb.make_desc(wl["layers"], B, wl.get("depth", 1))
     h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER[wl["optimizer"]], type_loss_function=mb.LOSS[wl["loss"]], **wl["hyper"])
     net = mb.HipNetwork(desc, h)
     net.set_stream(torch.cuda.current_stream().cuda_stream)
@@ -171,11 +192,12 @@ def main():
         "unit": "samples/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": args.workload, "batch": B, "layers": [l["units"] for l in wl["layers"]],
+        "config": {"workload": args.workload, "batch": B, "sequence_length": wl.get("depth", 1),
+                   "layers": [("lstm%d" if l.get("type") == "lstm" else "fc%d") % l["units"] for l in wl["layers"]],
                    "optimizer": wl["optimizer"], "parameters": int(desc.total_parameters),
-                   "gemm_flops_per_step": gemm_flops_per_step(wl["layers"], B)},
+                   "gemm_flops_per_step": gemm_flops_per_step(wl["layers"], B, wl.get("depth", 1))},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": PMC_TRAFFIC_BYTES_PER_GEMM_LAUNCH.get(args.workload),
                      "kernel": "gemm_f32_mfma_kernel (forward + dX + dW launches)", "launches": g_launch,
                      "avg_launch_ms": g_ms / max(g_launch, 1), "flops_per_launch": g_flop / max(g_launch, 1),
                      "gemm_ms_per_step": g_ms / args.steps},
@@ -187,7 +209,7 @@ def main():
         rows = args.cpu_sample_rows
         if rows <= 0:
             # sized from the layer widths for ~20 s at ~15 GFLOP/s per thread (gcc -O2 vectorises the inner loops)
-            flop_per_row = gemm_flops_per_step(wl["layers"], 1)
+            flop_per_row = gemm_flops_per_step(wl["layers"], 1, wl.get("depth", 1))
             rows = int(max(4, min(B, 20.0 * threads * 15.0e9 / flop_per_row)))
             rows = max(threads, rows - rows % threads)
         out["cpu_baseline"] = cpu_baseline(wl, rows, threads)

@@ -1,0 +1,275 @@
+// myea_nn_hip.hpp — header-only C++ host adaptor over the C ABI of include/myea_hip.h.
+//
+// `Neural_Network_HIP` mirrors the part of the reference's `class Neural_Network`
+// (Header_Files/Neural_Network/Data.hpp:760-3294) that sits on the training hot path: same method names, same
+// argument meaning (batch_size_received, arrays of per-example row pointers, layer indices), same error behaviour
+// (`bool` setters that print and return false; `void` step functions that print and return), same public training
+// fields.  A host program written against the reference (see Neural_Network_Launcher_Windows/Source_Files/debug.cpp:
+// 481-1555 for the call order) switches to the MI355X path by swapping the class.
+//
+// Everything here is host code; the device work happens behind myea_hip_*.
+#pragma once
+
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "myea_hip.h"
+
+namespace MyEA_HIP {
+
+typedef float T_;  // COMPILE_FLOAT (Common_Library/include/Configuration/DTypes.hpp:20-32)
+
+// Header_Files/Neural_Network/Data.hpp:56-80
+struct Layer_Parameters {
+    bool use_bidirectional = false;
+    unsigned int type_layer = MYEA_LAYER_NONE;  // MYEA_LAYER_*
+    // [0] FC: neurons, LSTM: blocks, RESIDUAL: block depth.  [1] LSTM: cells per block.
+    size_t unit_parameters[5u] = {0};
+};
+
+class Neural_Network_HIP {
+public:
+    // ---- public training fields, defaults of Data.hpp:2929-2970 ----
+    T_ learning_rate = 0.01f, learning_rate_final = 0.1f, learning_momentum = 0.9f, learning_gamma = 1e-3f;
+    T_ adam_learning_rate = 0.001f, adam_beta1 = 0.9f, adam_beta2 = 0.999f, adam_epsilon = 1e-8f;
+    T_ regularization__weight_decay = 0.f, clip_gradient = 1.f, accuracy_variance = 0.49f, bit_fail_limit = 0.35f;
+    T_ normalization_momentum_average = 0.999f, normalization_epsilon = 1e-5f;
+    T_ batch_renormalization_r_correction_maximum = 1.f, batch_renormalization_d_correction_maximum = 0.f;
+    bool use_Nesterov = false, use_adam_bias_correction = true, use_clip_gradient = false;
+    unsigned int type_optimizer_function = MYEA_OPTIMIZER_NONE, type_loss_function = MYEA_LOSS_NONE;
+    unsigned int type_accuracy_function = MYEA_ACCURACY_DISTANCE;
+    unsigned int type_state_propagation = MYEA_STATE_INFERENCE;
+    size_t number_time_delays = 0, number_recurrent_depth = 1, batch_size = 1;
+    size_t total_parameters = 0, total_weights = 0, total_bias = 0;
+    // public host copies, written by the caller like the reference's members and pushed with the Copy__* calls
+    T_ *ptr_array_parameters = nullptr;                      // [total_parameters]
+    bool *ptr_array_units_mask_dropout_bernoulli = nullptr;  // [(sum of AF units) * T], all true after Compile
+
+    Neural_Network_HIP() { std::memset(&desc_, 0, sizeof(desc_)); }
+    ~Neural_Network_HIP() { Deallocate(); }
+    Neural_Network_HIP(const Neural_Network_HIP &) = delete;
+    Neural_Network_HIP &operator=(const Neural_Network_HIP &) = delete;
+
+    // Neural_Network::Compile (Data.hpp:2531; Neural_Network__Compile.cpp:426).  maximum_allowable_memory is accepted
+    // for signature compatibility; device memory is sized from the descriptor.
+    bool Compile(size_t number_layers, size_t number_recurrent_depth_received, unsigned int type_network,
+                 Layer_Parameters const *ptr_array_layers, size_t maximum_allowable_memory = 0)
+    {
+        (void)maximum_allowable_memory;
+        if (number_layers < 2 || number_layers > MYEA_MAX_LAYERS || ptr_array_layers == nullptr) return Fail("Compile", "bad layer count");
+        if (number_recurrent_depth_received == 0) return Fail("Compile", "recurrent depth can not be zero");
+        Deallocate();
+        std::memset(&desc_, 0, sizeof(desc_));
+        desc_.type_network = type_network;
+        desc_.n_layers = (uint32_t)number_layers;
+        desc_.number_recurrent_depth = (uint32_t)number_recurrent_depth_received;
+        desc_.batch_size = (uint32_t)batch_size;
+        number_recurrent_depth = number_recurrent_depth_received;
+        for (size_t i = 0; i < number_layers; ++i) {
+            myea_layer_desc &l = desc_.layers[i];
+            l.type_layer = ptr_array_layers[i].type_layer;
+            l.use_bidirectional = ptr_array_layers[i].use_bidirectional;
+            l.n_units = (uint32_t)ptr_array_layers[i].unit_parameters[0];
+            l.n_cells_per_block = l.type_layer == MYEA_LAYER_LSTM ? (uint32_t)ptr_array_layers[i].unit_parameters[1] : 0;
+            if (l.type_layer == MYEA_LAYER_RESIDUAL) { l.block_depth = l.n_units; l.n_units = 0; }
+            // Compile's defaults: FC layers start as sigmoid with steepness 1 (Neural_Network__Compile.cpp:572-590)
+            l.type_activation_function = (i > 0 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) ? MYEA_AF_SIGMOID : MYEA_AF_NONE;
+            l.activation_steepness = 1.f;
+            l.use_layer_normalization_before_activation = 1;
+            l.dropout_values[0] = 1.f;
+        }
+        return Relayout("Compile");
+    }
+
+    bool Set__Layer_Activation_Function(size_t index_layer, unsigned int type_activation_function)
+    {
+        if (!CheckLayer("Set__Layer_Activation_Function", index_layer)) return false;
+        if (type_activation_function == MYEA_AF_NONE || type_activation_function >= MYEA_AF_LENGTH) return Fail("Set__Layer_Activation_Function", "activation function out of range");
+        desc_.layers[index_layer].type_activation_function = type_activation_function;
+        return Dirty();
+    }
+    bool Set__Layer_Activation_Steepness(size_t index_layer, T_ activation_steepness)
+    {
+        if (!CheckLayer("Set__Layer_Activation_Steepness", index_layer)) return false;
+        desc_.layers[index_layer].activation_steepness = activation_steepness;
+        return Dirty();
+    }
+    // Data.hpp:2697; `use_layer_normalization_before_activation` is a public Layer field in the reference
+    bool Set__Layer_Normalization(size_t index_layer, unsigned int type_layer_normalization, bool use_layer_normalization_before_activation = true)
+    {
+        if (!CheckLayer("Set__Layer_Normalization", index_layer)) return false;
+        desc_.layers[index_layer].type_normalization = type_layer_normalization;
+        desc_.layers[index_layer].use_layer_normalization_before_activation = use_layer_normalization_before_activation;
+        return Relayout("Set__Layer_Normalization");
+    }
+    // Data.hpp:2667; value_dropout[0] = retention probability
+    bool Set__Dropout(size_t index_layer, unsigned int type_layer_dropout, T_ const value_dropout[], bool scale_weights = true)
+    {
+        (void)scale_weights;
+        if (index_layer >= desc_.n_layers) return Fail("Set__Dropout", "layer index overflow");
+        if (value_dropout == nullptr || value_dropout[0] < 0.f || value_dropout[0] > 1.f) return Fail("Set__Dropout", "retention probability out of [0, 1]");
+        desc_.layers[index_layer].type_dropout = type_layer_dropout;
+        desc_.layers[index_layer].dropout_values[0] = value_dropout[0];
+        return Dirty();
+    }
+    void Set__Loss_Function(unsigned int f) { type_loss_function = f; }
+    void Set__Accuracy_Function(unsigned int f) { type_accuracy_function = f; }
+    void Set__Optimizer_Function(unsigned int f) { type_optimizer_function = f; }
+    void Set__Clip_Gradient(bool use) { use_clip_gradient = use; }
+    bool Set__Clip_Gradient(T_ value) { clip_gradient = value; return true; }
+    bool Set__Accurancy_Variance(T_ v) { accuracy_variance = v; return true; }
+    bool Set__Number_Time_Delays(size_t n) { if (n > number_recurrent_depth) return Fail("Set__Number_Time_Delays", "time delays exceed the recurrent depth"); number_time_delays = n; return true; }
+    bool Set__Normalization_Momentum_Average(T_ v) { normalization_momentum_average = v; return true; }
+    bool Set__Normalization_Epsilon(T_ v) { normalization_epsilon = v; return true; }
+    bool Set__Batch_Renormalization_r_Correction_Maximum(T_ v) { batch_renormalization_r_correction_maximum = v; return true; }
+    bool Set__Batch_Renormalization_d_Correction_Maximum(T_ v) { batch_renormalization_d_correction_maximum = v; return true; }
+
+    // Data.hpp:2559
+    bool Update__Batch_Size(size_t desired_batch_size, bool force_update = false)
+    {
+        (void)force_update;
+        if (desired_batch_size == 0) return Fail("Update__Batch_Size", "batch size can not be zero");
+        batch_size = desired_batch_size;
+        desc_.batch_size = (uint32_t)desired_batch_size;
+        return Dirty();
+    }
+
+    // The seam where the reference has Set__CUDA (Data.hpp:3116): creates the device object from the current
+    // descriptor and uploads parameters and masks.
+    bool Set__HIP(bool use_hip)
+    {
+        if (!use_hip) { if (net_) { myea_hip_destroy(net_); net_ = nullptr; } return true; }
+        if (net_) { myea_hip_destroy(net_); net_ = nullptr; }
+        if (myea_hip_create(&desc_, &net_) != MYEA_OK) return Fail("Set__HIP", myea_hip_last_error());
+        return Copy__Parameters__Host_To_Device() && Copy__Dropout_Mask__Host_To_Device();
+    }
+    bool Use__HIP() const { return net_ != nullptr; }
+
+    // Data.hpp:3119-3189
+    bool Copy__Parameters__Host_To_Device() { return Need("Copy__Parameters__Host_To_Device") && Ok("Copy__Parameters__Host_To_Device", myea_hip_upload_parameters(net_, ptr_array_parameters, total_parameters)); }
+    bool Copy__Parameters__Device_To_Host() { return Need("Copy__Parameters__Device_To_Host") && Ok("Copy__Parameters__Device_To_Host", myea_hip_download_parameters(net_, ptr_array_parameters, total_parameters)); }
+    bool Copy__Optimizer__Device_To_Host(int kind, T_ *dst) { return Need("Copy__Optimizer__Device_To_Host") && Ok("Copy__Optimizer__Device_To_Host", myea_hip_download_optimizer_state(net_, kind, dst, total_parameters)); }
+    bool Copy__Optimizer__Host_To_Device(int kind, T_ const *src) { return Need("Copy__Optimizer__Host_To_Device") && Ok("Copy__Optimizer__Host_To_Device", myea_hip_upload_optimizer_state(net_, kind, src, total_parameters)); }
+    bool Copy__Derivatives_Parameters__Device_To_Host(T_ *dst) { return Need("Copy__Derivatives_Parameters__Device_To_Host") && Ok("Copy__Derivatives_Parameters__Device_To_Host", myea_hip_download_gradient(net_, dst, total_parameters)); }
+    bool Copy__Dropout_Mask__Host_To_Device()
+    {
+        if (!Need("Copy__Dropout_Mask__Host_To_Device")) return false;
+        std::vector<uint8_t> bytes(desc_.total_mask_units);
+        for (size_t i = 0; i < bytes.size(); ++i) bytes[i] = ptr_array_units_mask_dropout_bernoulli[i] ? 1 : 0;
+        return Ok("Copy__Dropout_Mask__Host_To_Device", myea_hip_upload_masks(net_, bytes.data(), bytes.size()));
+    }
+
+    // Train.cpp:93-263
+    void Clear_Training_Arrays() { if (Need("Clear_Training_Arrays")) Ok("Clear_Training_Arrays", myea_hip_clear_training_arrays(net_)); }
+    void Reset__Loss() { if (Need("Reset__Loss")) Ok("Reset__Loss", myea_hip_reset_loss(net_)); }
+
+    // ---- the five step entry points (Data.hpp:2896, 1033, 1709, 2199, 849) ----
+    void Forward_Pass(size_t batch_size_received, T_ const *const *ptr_array_inputs)
+    {
+        if (!Need("Forward_Pass") || !PushFields("Forward_Pass")) return;
+        const size_t row = (size_t)desc_.layers[0].n_units * desc_.number_recurrent_depth;
+        if (!Flatten("Forward_Pass", batch_size_received, ptr_array_inputs, row)) return;
+        Ok("Forward_Pass", myea_hip_forward_pass(net_, batch_size_received, rows_.data(), 0));
+    }
+    void Compute__Error(size_t batch_size_received, T_ const *const *ptr_array_desireds_outputs)
+    {
+        if (!Need("Compute__Error") || !PushFields("Compute__Error")) return;
+        const size_t row = (size_t)desc_.layers[desc_.n_layers - 1].n_units * desc_.number_recurrent_depth;
+        if (!Flatten("Compute__Error", batch_size_received, ptr_array_desireds_outputs, row)) return;
+        Ok("Compute__Error", myea_hip_compute_error(net_, batch_size_received, rows_.data(), 0));
+    }
+    void Backward_Pass(size_t batch_size_received) { if (Need("Backward_Pass") && PushFields("Backward_Pass")) Ok("Backward_Pass", myea_hip_backward_pass(net_, batch_size_received)); }
+    // the reference's callers pass (ptr_array_layers + 1, ptr_last_layer); here as layer indices
+    void Update_Derivative_Weight(size_t batch_size_received, size_t first_layer_index = 1, size_t end_layer_index = 0)
+    {
+        if (!Need("Update_Derivative_Weight")) return;
+        Ok("Update_Derivative_Weight", myea_hip_update_derivative_weight(net_, batch_size_received, first_layer_index, end_layer_index ? end_layer_index : desc_.n_layers));
+    }
+    void Update_Parameter(size_t batch_size_received, size_t training_size_received)
+    {
+        if (!Need("Update_Parameter") || !PushFields("Update_Parameter")) return;
+        Ok("Update_Parameter", myea_hip_update_parameter(net_, batch_size_received, training_size_received));
+        myea_hyper h;
+        if (myea_hip_get_hyper(net_, &h) == MYEA_OK) optimizer_time_step = h.optimizer_time_step;
+    }
+    T_ optimizer_time_step = 0.f;
+
+    // merged loss counters (Neural_Network__Merge.cpp:52-98); mean of the accumulated per-output terms
+    T_ Get__Loss()
+    {
+        myea_loss_state s;
+        if (!Need("Get__Loss") || !Ok("Get__Loss", myea_hip_get_loss(net_, &s)) || s.number_loss == 0) return 0.f;
+        return (T_)(s.loss_values / (double)s.number_loss);
+    }
+    bool Get__Loss_State(myea_loss_state *out) { return Need("Get__Loss_State") && Ok("Get__Loss_State", myea_hip_get_loss(net_, out)); }
+
+    myea_net_desc const &Get__Descriptor() const { return desc_; }
+    myea_hip_net *Get__Device_Handle() { return net_; }
+
+private:
+    myea_net_desc desc_;
+    myea_hip_net *net_ = nullptr;
+    std::vector<T_> rows_;
+
+    static bool Fail(const char *fn, const char *what) { std::printf("%s: ERROR: %s.\n", fn, what); return false; }
+    bool Ok(const char *fn, int rc) { if (rc != MYEA_OK) { Fail(fn, myea_hip_last_error()); return false; } return true; }
+    bool Need(const char *fn) const { if (!net_) { Fail(fn, "the device object is not initialised (Set__HIP)"); return false; } return true; }
+    bool CheckLayer(const char *fn, size_t i) const
+    {
+        if (i == 0 || i >= desc_.n_layers) return Fail(fn, "layer index overflow");
+        return true;
+    }
+    // a structural change after Set__HIP needs a new device object, as a changed Layer does in the reference's CUDA path
+    bool Dirty() { if (net_) { myea_hip_destroy(net_); net_ = nullptr; } return true; }
+    void Deallocate()
+    {
+        if (net_) { myea_hip_destroy(net_); net_ = nullptr; }
+        delete[] ptr_array_parameters; ptr_array_parameters = nullptr;
+        delete[] ptr_array_units_mask_dropout_bernoulli; ptr_array_units_mask_dropout_bernoulli = nullptr;
+    }
+    bool Relayout(const char *fn)
+    {
+        Dirty();
+        const size_t old_p = total_parameters;
+        T_ *old = ptr_array_parameters;
+        if (myea_net_desc_layout(&desc_) != MYEA_OK) return Fail(fn, "the layer list is not valid on this path");
+        total_parameters = desc_.total_parameters; total_weights = desc_.total_weights; total_bias = desc_.total_bias;
+        ptr_array_parameters = new T_[total_parameters ? total_parameters : 1]();
+        if (old) std::memcpy(ptr_array_parameters, old, sizeof(T_) * (old_p < total_parameters ? old_p : total_parameters));
+        // scales start at one (Allocate__Parameter__Normalization), shifts at zero
+        if (desc_.total_normalized_units && old_p <= desc_.total_weights + desc_.total_bias)
+            for (size_t i = 0; i < desc_.total_normalized_units; ++i) ptr_array_parameters[desc_.total_weights + desc_.total_bias + i] = 1.f;
+        delete[] old;
+        delete[] ptr_array_units_mask_dropout_bernoulli;
+        ptr_array_units_mask_dropout_bernoulli = new bool[desc_.total_mask_units ? desc_.total_mask_units : 1];
+        for (size_t i = 0; i < desc_.total_mask_units; ++i) ptr_array_units_mask_dropout_bernoulli[i] = true;
+        return true;
+    }
+    bool PushFields(const char *fn)
+    {
+        myea_hyper h;
+        if (myea_hip_get_hyper(net_, &h) != MYEA_OK) return Fail(fn, myea_hip_last_error());
+        h.type_optimizer_function = type_optimizer_function; h.type_loss_function = type_loss_function; h.type_accuracy_function = type_accuracy_function;
+        h.use_Nesterov = use_Nesterov; h.use_adam_bias_correction = use_adam_bias_correction; h.use_clip_gradient = use_clip_gradient;
+        h.learning_rate = learning_rate; h.learning_rate_final = learning_rate_final; h.learning_momentum = learning_momentum; h.learning_gamma = learning_gamma;
+        h.adam_learning_rate = adam_learning_rate; h.adam_beta1 = adam_beta1; h.adam_beta2 = adam_beta2; h.adam_epsilon = adam_epsilon;
+        h.regularization__weight_decay = regularization__weight_decay; h.clip_gradient = clip_gradient; h.accuracy_variance = accuracy_variance;
+        h.bit_fail_limit = bit_fail_limit; h.normalization_momentum_average = normalization_momentum_average; h.normalization_epsilon = normalization_epsilon;
+        h.batch_renormalization_r_correction_maximum = batch_renormalization_r_correction_maximum;
+        h.batch_renormalization_d_correction_maximum = batch_renormalization_d_correction_maximum;
+        h.number_time_delays = (uint32_t)number_time_delays;
+        if (myea_hip_set_hyper(net_, &h) != MYEA_OK) return Fail(fn, myea_hip_last_error());
+        return Ok(fn, myea_hip_set_state_propagation(net_, type_state_propagation));
+    }
+    bool Flatten(const char *fn, size_t B, T_ const *const *rows, size_t row)
+    {
+        if (rows == nullptr) return Fail(fn, "null row pointer array");
+        if (B > desc_.batch_size) { std::printf("%s: ERROR: Overflow of memory. Unable to process %zu examples out of %u allocated.\n", fn, B, desc_.batch_size); return false; }
+        rows_.resize(B * row);
+        for (size_t b = 0; b < B; ++b) std::memcpy(rows_.data() + b * row, rows[b], row * sizeof(T_));
+        return true;
+    }
+};
+
+}  // namespace MyEA_HIP

@@ -207,72 +207,77 @@ __device__ __forceinline__ float sign_f(float v) { return v > 0.f ? 1.f : (v < 0
 
 __global__ __launch_bounds__(kBlock) void compute_error_kernel(ErrorParams p)
 {
-    const int lane = threadIdx.x & 63;
+    __shared__ float red[4][kBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const size_t nrows = (p.T - p.first_t) * p.B;
-    const size_t rid = (size_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-    if (rid >= nrows) return;
-    const size_t t = p.first_t + rid / p.B, b = rid % p.B;
-    const size_t off = (t * p.Bmax + b) * p.H;
-    const float *y = p.values + off, *pre = p.pre + off;
-    const float *d = p.desired + (b * p.T + t) * p.H;
-    float *err = p.errors + off;
-
     float loss = 0.f, cnt = 0.f, acc = 0.f, bits = 0.f;
-    // cross-entropy accuracy: first index whose target is 1, last index reaching the maximum (">=")
-    if (p.accuracy == MYEA_ACCURACY_CROSS_ENTROPY) {
-        unsigned want = 0xffffffffu; float mx = -3.402823466e+38f; unsigned got = 0;
-        for (size_t j = lane; j < p.H; j += 64) {
-            if (d[j] == 1.f && (unsigned)j < want) want = (unsigned)j;
-            if (y[j] >= mx) { mx = y[j]; got = (unsigned)j; }
-        }
+    // wavefronts stride over the rows and keep their sums in registers: one set of fp64 atomics per workgroup
+    for (size_t rid = (size_t)blockIdx.x * (kBlock / 64) + wave; rid < nrows; rid += (size_t)gridDim.x * (kBlock / 64)) {
+        const size_t t = p.first_t + rid / p.B, b = rid % p.B;
+        const size_t off = (t * p.Bmax + b) * p.H;
+        const float *y = p.values + off, *pre = p.pre + off;
+        const float *d = p.desired + (b * p.T + t) * p.H;
+        float *err = p.errors + off;
+        // cross-entropy accuracy: first index whose target is 1, last index reaching the maximum (">=")
+        if (p.accuracy == MYEA_ACCURACY_CROSS_ENTROPY) {
+            unsigned want = 0xffffffffu; float mx = -3.402823466e+38f; unsigned got = 0;
+            for (size_t j = lane; j < p.H; j += 64) {
+                if (d[j] == 1.f && (unsigned)j < want) want = (unsigned)j;
+                if (y[j] >= mx) { mx = y[j]; got = (unsigned)j; }
+            }
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const unsigned w2 = __shfl_xor(want, o, 64);
-            const float m2 = __shfl_xor(mx, o, 64);
-            const unsigned g2 = __shfl_xor(got, o, 64);
-            want = min(want, w2);
-            if (m2 > mx || (m2 == mx && g2 > got)) { mx = m2; got = g2; }
+            for (int o = 32; o > 0; o >>= 1) {
+                const unsigned w2 = __shfl_xor(want, o, 64);
+                const float m2 = __shfl_xor(mx, o, 64);
+                const unsigned g2 = __shfl_xor(got, o, 64);
+                want = min(want, w2);
+                if (m2 > mx || (m2 == mx && g2 > got)) { mx = m2; got = g2; }
+            }
+            if (want == 0xffffffffu) want = (unsigned)p.H;
+            if (lane == 0) acc += (want == got) ? 1.f : 0.f;
         }
-        if (want == 0xffffffffu) want = (unsigned)p.H;
-        if (lane == 0) acc += (want == got) ? 1.f : 0.f;
-    }
-    for (size_t j = lane; j < p.H; j += 64) {
-        const float yo = y[j], de = d[j], diff = yo - de;
-        float e = 0.f; bool counted = true;
-        switch (p.loss) {
-        case MYEA_LOSS_ME:
-        case MYEA_LOSS_L1: e = diff; break;
-        case MYEA_LOSS_MAE: e = fabsf(diff); break;
-        case MYEA_LOSS_L2:
-        case MYEA_LOSS_MSE:
-        case MYEA_LOSS_RMSE: e = diff * diff; break;
-        case MYEA_LOSS_MAPE: { float q = yo != 0.f ? yo : fmaxf(yo, 1e-6f); e = fabsf(diff / q); break; }
-        case MYEA_LOSS_SMAPE: e = fabsf(diff) / (fabsf(de) + fabsf(yo)); break;
-        case MYEA_LOSS_CROSS_ENTROPY: {
-            float q = yo != 0.f ? yo : fmaxf(yo, 1e-6f);
-            e = (p.H == 1) ? -(de * logf(q) + (1.f - de) * logf(1.f - q)) : -(de * logf(q));
-            break;
+        for (size_t j = lane; j < p.H; j += 64) {
+            const float yo = y[j], de = d[j], diff = yo - de;
+            float e = 0.f; bool counted = true;
+            switch (p.loss) {
+            case MYEA_LOSS_ME:
+            case MYEA_LOSS_L1: e = diff; break;
+            case MYEA_LOSS_MAE: e = fabsf(diff); break;
+            case MYEA_LOSS_L2:
+            case MYEA_LOSS_MSE:
+            case MYEA_LOSS_RMSE: e = diff * diff; break;
+            case MYEA_LOSS_MAPE: { float q = yo != 0.f ? yo : fmaxf(yo, 1e-6f); e = fabsf(diff / q); break; }
+            case MYEA_LOSS_SMAPE: e = fabsf(diff) / (fabsf(de) + fabsf(yo)); break;
+            case MYEA_LOSS_CROSS_ENTROPY: {
+                float q = yo != 0.f ? yo : fmaxf(yo, 1e-6f);
+                e = (p.H == 1) ? -(de * logf(q) + (1.f - de) * logf(1.f - q)) : -(de * logf(q));
+                break;
+            }
+            case MYEA_LOSS_BIT: counted = false; if (fabsf(diff) >= p.bit_fail_limit) bits += 1.f; break;
+            default: counted = false; break;
+            }
+            if (counted) { loss += e; cnt += 1.f; }
+            switch (p.accuracy) {
+            case MYEA_ACCURACY_DISTANCE: if (fabsf(diff) <= p.accuracy_variance) acc += 1.f; break;
+            case MYEA_ACCURACY_DIRECTIONAL:
+                // RNN: direction of change against the previous target (Recurrent_Compute__Error__OpenMP.cpp:115-120)
+                if (!p.rnn_pre_quirk || t == 0 || sign_f(de - d[(long)j - (long)p.H]) == sign_f(yo - d[(long)j - (long)p.H])) acc += 1.f;
+                break;
+            case MYEA_ACCURACY_SIGN:
+                if (sign_f(de) == sign_f(yo) || (sign_f(de) == 0.f && yo >= -1.192092896e-07f && yo <= 1.192092896e-07f)) acc += 1.f;
+                break;
+            default: break;
+            }
+            const float q = p.rnn_pre_quirk ? pre[0] : pre[j];
+            err[j] = af_derive(p.act, q, p.steep, yo) * diff;
         }
-        case MYEA_LOSS_BIT: counted = false; if (fabsf(diff) >= p.bit_fail_limit) bits += 1.f; break;
-        default: counted = false; break;
-        }
-        if (counted) { loss += e; cnt += 1.f; }
-        switch (p.accuracy) {
-        case MYEA_ACCURACY_DISTANCE: if (fabsf(diff) <= p.accuracy_variance) acc += 1.f; break;
-        case MYEA_ACCURACY_DIRECTIONAL: acc += 1.f; break;
-        case MYEA_ACCURACY_SIGN:
-            if (sign_f(de) == sign_f(yo) || (sign_f(de) == 0.f && yo >= -1.192092896e-07f && yo <= 1.192092896e-07f)) acc += 1.f;
-            break;
-        default: break;
-        }
-        const float q = p.rnn_pre_quirk ? pre[0] : pre[j];
-        err[j] = af_derive(p.act, q, p.steep, yo) * diff;
     }
     loss = wave_sum(loss); cnt = wave_sum(cnt); acc = wave_sum(acc); bits = wave_sum(bits);
-    if (lane == 0) {
-        if (cnt != 0.f) { atomicAdd(&p.loss_acc[0], (double)loss); atomicAdd(&p.loss_acc[1], (double)cnt); }
-        if (acc != 0.f) atomicAdd(&p.loss_acc[2], (double)acc);
-        if (bits != 0.f) atomicAdd(&p.loss_acc[3], (double)bits);
+    if (lane == 0) { red[0][wave] = loss; red[1][wave] = cnt; red[2][wave] = acc; red[3][wave] = bits; }
+    __syncthreads();
+    if (threadIdx.x < 4) {
+        const float v = red[threadIdx.x][0] + red[threadIdx.x][1] + red[threadIdx.x][2] + red[threadIdx.x][3];
+        if (v != 0.f) atomicAdd(&p.loss_acc[threadIdx.x], (double)v);
     }
 }
 
@@ -517,7 +522,7 @@ int launch_compute_error(hipStream_t s, const ErrorParams &p)
 {
     if (p.T <= p.first_t || p.B == 0 || p.H == 0) return MYEA_OK;
     const size_t nrows = (p.T - p.first_t) * p.B;
-    hipLaunchKernelGGL(compute_error_kernel, dim3(grid_for(nrows, kBlock / 64)), dim3(kBlock), 0, s, p);
+    hipLaunchKernelGGL(compute_error_kernel, dim3(grid_for(nrows, kBlock / 64, 1024)), dim3(kBlock), 0, s, p);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

@@ -142,6 +142,8 @@ struct GemmDev {
     int act;
     float steep;
     int nbm, nbn;
+    int ksplit, kchunk;   // split-K: number of slabs and k's per slab (multiple of BK); slab s writes C + s * slab
+    long slab;
 };
 
 template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
@@ -157,8 +159,10 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
     // L2), so give every XCD a contiguous run of tile ids, and walk tiles in bands of 8 m-tiles so that a
     // run shares its B columns and a small set of A rows.
     const int nblocks = p.nbm * p.nbn;
-    int pid = blockIdx.x;
+    const int split = blockIdx.x / nblocks;   // split-K slab of this workgroup
+    int pid = blockIdx.x - split * nblocks;
     if ((nblocks & 7) == 0) pid = (pid & 7) * (nblocks >> 3) + (pid >> 3);
+    const int k_begin = split * p.kchunk, k_end = min(p.K, k_begin + p.kchunk);
     constexpr int kBand = 8;
     const int band = pid / (kBand * p.nbn);
     const int band_first = band * kBand;
@@ -181,10 +185,10 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
 
     TileMover<BM, A_KC, VEC> moveA;
     TileMover<BN, B_KC, VEC> moveB;
-    const int nk = (p.K + kBK - 1) / kBK;
+    const int nk = (k_end - k_begin + kBK - 1) / kBK;
 
-    moveA.load(p.A, p.lda, m0, p.M, 0, p.K);
-    moveB.load(p.B, p.ldb, n0, p.N, 0, p.K);
+    moveA.load(p.A, p.lda, m0, p.M, k_begin, k_end);
+    moveB.load(p.B, p.ldb, n0, p.N, k_begin, k_end);
     moveA.store(smem);
     moveB.store(smem + SA::kFloats);
     __syncthreads();
@@ -193,8 +197,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
         const int cur = kt & 1;
         const bool more = kt + 1 < nk;
         if (more) {
-            moveA.load(p.A, p.lda, m0, p.M, (kt + 1) * kBK, p.K);
-            moveB.load(p.B, p.ldb, n0, p.N, (kt + 1) * kBK, p.K);
+            moveA.load(p.A, p.lda, m0, p.M, k_begin + (kt + 1) * kBK, k_end);
+            moveB.load(p.B, p.ldb, n0, p.N, k_begin + (kt + 1) * kBK, k_end);
         }
         const float *la = smem + cur * kStage, *lb = la + SA::kFloats;
 #pragma unroll
@@ -235,7 +239,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wave_m + i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
                 if (row >= p.M) continue;
-                const long o = (long)row * p.ldc + col;
+                const long o = (long)row * p.ldc + col + (long)split * p.slab;
                 float v = acc[i][j][r];
                 if (p.epilogue == EPI_FC_FORWARD) {
                     v += bias;
@@ -266,7 +270,7 @@ int launch_one(hipStream_t stream, GemmDev d)
     }
     d.nbm = (d.M + BM - 1) / BM;
     d.nbn = (d.N + BN - 1) / BN;
-    const long nblocks = (long)d.nbm * d.nbn;
+    const long nblocks = (long)d.nbm * d.nbn * d.ksplit;
     if (nblocks <= 0 || nblocks > 0x7fffffffL) { set_last_error("gemm: grid of %ld workgroups out of range", nblocks); return MYEA_E_INVALID; }
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(kThreads), lds_bytes, stream, d);
     MYEA_HIP_TRY(hipGetLastError());
@@ -281,6 +285,14 @@ int launch_layout_vec(hipStream_t stream, const GemmDev &d, bool a_kc, bool b_kc
     return launch_one<BM, BN, false, false, true>(stream, d);
 }
 
+// short-M, short-N problems (the per-time-step recurrent contractions): 64 x 64 tiles
+int launch_layout_vec_small(hipStream_t stream, const GemmDev &d, bool a_kc, bool b_kc)
+{
+    if (a_kc && b_kc) return launch_one<64, 64, true, true, true>(stream, d);
+    if (a_kc && !b_kc) return launch_one<64, 64, true, false, true>(stream, d);
+    return launch_one<64, 64, false, false, true>(stream, d);
+}
+
 // guarded scalar loads, any alignment, any layout: the general (slow) path
 int launch_layout_scalar(hipStream_t stream, const GemmDev &d, bool a_kc, bool b_kc)
 {
@@ -291,6 +303,23 @@ int launch_layout_scalar(hipStream_t stream, const GemmDev &d, bool a_kc, bool b
 }
 
 }  // namespace
+
+// Number of K slabs for a short contraction so that the launch reaches about one workgroup per CU with 64 x 64 tiles
+// (each slab at least 128 k's deep); 1 when the plain launch already fills the chip.
+int gemm_split_k(int M, int N, int K)
+{
+    const long tiles_128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (tiles_128 * 2 >= 256) return 1;
+    const long tiles_64 = (long)((M + 63) / 64) * ((N + 63) / 64);
+    long want = (256 + tiles_64 - 1) / tiles_64;
+    const long max_by_k = K / 128 > 0 ? K / 128 : 1;
+    if (want > max_by_k) want = max_by_k;
+    if (want > 16) want = 16;
+    if (want < 1) want = 1;
+    // the launcher rounds the chunk up to a multiple of 32: return the slab count that rounding produces
+    const int chunk = (int)(((K + want - 1) / want + kBK - 1) / kBK * kBK);
+    return (K + chunk - 1) / chunk;
+}
 
 bool gemm_can_fuse_activation(int act)
 {
@@ -316,6 +345,15 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     d.bias = p.bias; d.aux_out = p.aux_out; d.colscale = p.colscale;
     d.pre = p.pre; d.val = p.val; d.act = p.act; d.steep = p.steep;
     d.nbm = d.nbn = 0;
+    d.ksplit = 1; d.kchunk = p.K > 0 ? p.K : 1; d.slab = 0;
+    if (p.split_k > 1) {
+        if (p.epilogue != EPI_NONE || p.accumulate) { set_last_error("gemm: split-K writes plain partial slabs"); return MYEA_E_INVALID; }
+        const int chunk = ((p.K + p.split_k - 1) / p.split_k + kBK - 1) / kBK * kBK;
+        d.kchunk = chunk;
+        d.ksplit = (p.K + chunk - 1) / chunk;
+        d.slab = p.split_k_slab;
+        if (d.ksplit != p.split_k) { set_last_error("gemm: split-K count %d does not divide K=%d into %d-wide chunks; use gemm_split_k()", p.split_k, p.K, chunk); return MYEA_E_INVALID; }
+    }
 
     // 128-bit global loads need 16-byte aligned rows; otherwise fall back to guarded scalar loads.
     auto aligned = [](const float *ptr, long ld, long contiguous_extent) {
@@ -329,6 +367,7 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     // 64-row tiles to keep the chip filled for short-M / short-N problems.
     const long tiles_128 = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
     if (tiles_128 >= 512) return launch_layout_vec<128, 128>(stream, d, a_kc, b_kc);
+    if (tiles_128 * 2 * d.ksplit < 256) return launch_layout_vec_small(stream, d, a_kc, b_kc);
     if (p.M <= p.N) return launch_layout_vec<64, 128>(stream, d, a_kc, b_kc);
     return launch_layout_vec<128, 64>(stream, d, a_kc, b_kc);
 }

@@ -41,8 +41,13 @@ struct GemmParams {
     const float *val;       // EPI_FC_DERIVE, [M][ldc]
     int act;
     float steep;
+    // split-K (deterministic): slab s of the K range writes its partial product to C + s * split_k_slab; the consumer
+    // sums the slabs in order.  Requires EPI_NONE and accumulate == 0.  0 / 1 = off.
+    int split_k;
+    long split_k_slab;
 };
 
+int gemm_split_k(int M, int N, int K);
 int launch_gemm(hipStream_t stream, const GemmParams &p);
 // activations the FC_FORWARD / FC_DERIVE epilogues can apply (the others run as a separate kernel)
 bool gemm_can_fuse_activation(int act);

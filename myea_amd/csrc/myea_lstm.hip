@@ -31,6 +31,7 @@ struct LstmLayer {
     float *c = nullptr, *ca = nullptr;                           // [T][Bmax][C] cell state and tanh(cell state)
     float *dG = nullptr;    // [T][Bmax][G] deltas dz | di | df | do
     float *dc = nullptr;    // [T][Bmax][C]
+    float *part = nullptr;  // split-K slabs of the per-step recurrent contractions, 16 x [Bmax][G]
 };
 
 namespace {
@@ -40,6 +41,8 @@ namespace {
         int rc__ = (expr);                \
         if (rc__ != MYEA_OK) return rc__; \
     } while (0)
+
+constexpr size_t kMaxSlabs = 16;
 
 struct LstmGeom {
     size_t K, cpb, C, G, In, per_block, base;
@@ -73,12 +76,21 @@ __global__ __launch_bounds__(kBlock) void lstm_gather_kernel(LstmGeom g, const f
 }
 
 // flat gradient += packed gradient (every flat slot is owned by exactly one packed element: no atomics)
-__global__ __launch_bounds__(kBlock) void lstm_scatter_add_kernel(LstmGeom g, float *flat, const float *gWin, const float *gWrec, int with_rec)
+// gWin / gWrec hold s_in / s_rec split-K slabs, summed in slab order.
+__global__ __launch_bounds__(kBlock) void lstm_scatter_add_kernel(LstmGeom g, float *flat, const float *gWin, int s_in, const float *gWrec, int s_rec)
 {
-    const size_t n_in = g.G * g.In, n_rec = with_rec ? g.G * g.C : 0, n = n_in + n_rec;
+    const size_t n_in = g.G * g.In, n_rec = s_rec > 0 ? g.G * g.C : 0, n = n_in + n_rec;
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-        if (i < n_in) flat[flat_index(g, i / g.In, i % g.In, false)] += gWin[i];
-        else { const size_t q = i - n_in; flat[flat_index(g, q / g.C, q % g.C, true)] += gWrec[q]; }
+        if (i < n_in) {
+            float v = 0.f;
+            for (int s = 0; s < s_in; ++s) v += gWin[(size_t)s * n_in + i];
+            flat[flat_index(g, i / g.In, i % g.In, false)] += v;
+        } else {
+            const size_t q = i - n_in;
+            float v = 0.f;
+            for (int s = 0; s < s_rec; ++s) v += gWrec[(size_t)s * n_rec + q];
+            flat[flat_index(g, q / g.C, q % g.C, true)] += v;
+        }
     }
 }
 
@@ -89,13 +101,22 @@ __device__ __forceinline__ float tanh_f(float s) { return 2.f / (1.f + expf(-2.f
 // OpenMP.cpp:1042-1191), __States_AF (:1547-1582), __Output (:1351-1418).  `acts` holds input + recurrent sums on
 // entry (the contraction accumulated them) and the activations on exit.  First step: no forget gate, no input-gate
 // peephole, c = i z; the output gate peeps at c[t].
+// `part` holds `nparts` slabs [B][G] of the recurrent contraction h[t-1] Wrec^T (split along K), summed here in order.
 __global__ __launch_bounds__(kBlock) void lstm_forward_step_kernel(LstmGeom g, size_t B, int first, const float *bias, const float *peep,
-                                                                   float *acts, const float *c_prev, float *c, float *ca, float *h)
+                                                                   float *acts, const float *c_prev, float *c, float *ca, float *h,
+                                                                   const float *part, int nparts)
 {
     const size_t n = B * g.K;
     for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < n; idx += (size_t)gridDim.x * kBlock) {
         const size_t b = idx / g.K, k = idx % g.K;
         float *row = acts + b * g.G;
+        for (int s = 0; s < nparts; ++s) {   // recurrent sums join the input sums
+            const float *pr = part + ((size_t)s * B + b) * g.G;
+            row[g.C + k] += pr[g.C + k];
+            row[g.C + g.K + k] += pr[g.C + g.K + k];
+            row[g.C + 2 * g.K + k] += pr[g.C + 2 * g.K + k];
+            for (size_t j = 0; j < g.cpb; ++j) row[k * g.cpb + j] += pr[k * g.cpb + j];
+        }
         const size_t cell0 = b * g.C + k * g.cpb;
         const float *pi = peep + k * g.cpb, *pf = peep + g.C + k * g.cpb, *po = peep + 2 * g.C + k * g.cpb;
         float si = row[g.C + k] + bias[g.C + k];
@@ -133,8 +154,8 @@ __global__ __launch_bounds__(kBlock) void lstm_forward_step_kernel(LstmGeom g, s
 //   mode 3: first step, T > 1 (all future terms; delta f is not written)
 __global__ __launch_bounds__(kBlock) void lstm_backward_step_kernel(LstmGeom g, size_t B, int mode, const float *peep, const float *acts,
                                                                     const float *acts_next, const float *c_prev, const float *ca,
-                                                                    const float *dh, float *dG, const float *dG_next, float *dc,
-                                                                    const float *dc_next)
+                                                                    float *dh, float *dG, const float *dG_next, float *dc,
+                                                                    const float *dc_next, const float *part, int nparts)
 {
     const size_t n = B * g.K;
     for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < n; idx += (size_t)gridDim.x * kBlock) {
@@ -142,6 +163,13 @@ __global__ __launch_bounds__(kBlock) void lstm_backward_step_kernel(LstmGeom g, 
         const float *row = acts + b * g.G;
         float *drow = dG + b * g.G;
         const size_t cell0 = b * g.C + k * g.cpb;
+        if (nparts > 0) {   // recurrent delta dG[t+1] Wrec (slabs along K) joins the delta from the layers above
+            for (size_t j = 0; j < g.cpb; ++j) {
+                float v = dh[cell0 + j];
+                for (int s = 0; s < nparts; ++s) v += part[((size_t)s * B + b) * g.C + k * g.cpb + j];
+                dh[cell0 + j] = v;
+            }
+        }
         const float gi = row[g.C + k], gf = row[g.C + g.K + k], go = row[g.C + 2 * g.K + k];
         float eo = 0.f;
         for (size_t j = 0; j < g.cpb; ++j) eo += dh[cell0 + j] * ca[cell0 + j];
@@ -273,13 +301,14 @@ int Net::lstm_create_layer(size_t li)
     MYEA_TRY(dev_alloc_zero(&q->Win, q->G * q->In));
     MYEA_TRY(dev_alloc_zero(&q->Wrec, q->G * q->C));
     MYEA_TRY(dev_alloc_zero(&q->peep, 3 * q->C));
-    MYEA_TRY(dev_alloc_zero(&q->gWin, q->G * q->In));
-    MYEA_TRY(dev_alloc_zero(&q->gWrec, q->G * q->C));
+    MYEA_TRY(dev_alloc_zero(&q->gWin, kMaxSlabs * q->G * q->In));   // split-K slabs of the weight-gradient contractions
+    MYEA_TRY(dev_alloc_zero(&q->gWrec, kMaxSlabs * q->G * q->C));
     MYEA_TRY(dev_alloc_zero(&q->acts, T * B * q->G));
     MYEA_TRY(dev_alloc_zero(&q->c, T * B * q->C));
     MYEA_TRY(dev_alloc_zero(&q->ca, T * B * q->C));
     MYEA_TRY(dev_alloc_zero(&q->dG, T * B * q->G));
     MYEA_TRY(dev_alloc_zero(&q->dc, T * B * q->C));
+    MYEA_TRY(dev_alloc_zero(&q->part, 16 * B * q->G));
     MYEA_TRY(dev_alloc_zero(&o.neuron_errors, T * B * q->C));  // delta of the cell outputs (ptr_delta_cell_output)
     return MYEA_OK;
 }
@@ -288,7 +317,7 @@ void Net::lstm_destroy_layer(DevLayer &o)
 {
     if (!o.lstm) return;
     LstmLayer *q = o.lstm;
-    float *all[] = {q->Win, q->Wrec, q->peep, q->gWin, q->gWrec, q->acts, q->c, q->ca, q->dG, q->dc};
+    float *all[] = {q->Win, q->Wrec, q->peep, q->gWin, q->gWrec, q->acts, q->c, q->ca, q->dG, q->dc, q->part};
     for (float *p : all) if (p) (void)hipFree(p);
     delete q;
     o.lstm = nullptr;
@@ -340,18 +369,22 @@ int Net::lstm_forward_layer(size_t li, size_t B)
     const LstmGeom geom = geom_of(q);
     for (size_t t = 0; t < T; ++t) {
         float *acts_t = q.acts + t * Bmax * q.G;
+        int nparts = 0;
         if (t > 0) {
             GemmParams g{};
             g.A = o.values + (t - 1) * Bmax * q.C; g.lda = (long)q.C; g.a_k_contiguous = 1;
             g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 1;
-            g.C = acts_t; g.ldc = (long)q.G; g.accumulate = 1;
+            g.C = q.part; g.ldc = (long)q.G;
             g.M = (int)B; g.N = (int)q.G; g.K = (int)q.C;
+            nparts = gemm_split_k(g.M, g.N, g.K);
+            g.split_k = nparts; g.split_k_slab = (long)(B * q.G);
             prof_begin(0);
             MYEA_TRY(launch_gemm(stream, g));
             prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
         }
         hipLaunchKernelGGL(lstm_forward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, (int)(t == 0), bias, q.peep,
-                           acts_t, t ? q.c + (t - 1) * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, o.values + t * Bmax * q.C);
+                           acts_t, t ? q.c + (t - 1) * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, o.values + t * Bmax * q.C,
+                           q.part, nparts);
         MYEA_HIP_TRY(hipGetLastError());
     }
     return MYEA_OK;
@@ -368,12 +401,15 @@ int Net::lstm_backward_layer(size_t li, size_t B)
     for (size_t t = T; t-- > 0;) {
         float *dh_t = o.neuron_errors + t * Bmax * q.C;
         const bool last = t == T - 1, first = t == 0;
+        int nparts = 0;
         if (!last) {  // Backward_Pass__LSTM_Derivative__Output, recurrent part (:1174-1226)
             GemmParams g{};
             g.A = q.dG + (t + 1) * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 1;
             g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 0;
-            g.C = dh_t; g.ldc = (long)q.C; g.accumulate = 1;
+            g.C = q.part; g.ldc = (long)q.C;
             g.M = (int)B; g.N = (int)q.C; g.K = (int)q.G;
+            nparts = gemm_split_k(g.M, g.N, g.K);
+            g.split_k = nparts; g.split_k_slab = (long)(B * q.C);
             prof_begin(1);
             MYEA_TRY(launch_gemm(stream, g));
             prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
@@ -382,7 +418,7 @@ int Net::lstm_backward_layer(size_t li, size_t B)
         hipLaunchKernelGGL(lstm_backward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, mode, q.peep,
                            q.acts + t * Bmax * q.G, last ? nullptr : q.acts + (t + 1) * Bmax * q.G, first ? nullptr : q.c + (t - 1) * Bmax * q.C,
                            q.ca + t * Bmax * q.C, dh_t, q.dG + t * Bmax * q.G, last ? nullptr : q.dG + (t + 1) * Bmax * q.G,
-                           q.dc + t * Bmax * q.C, last ? nullptr : q.dc + (t + 1) * Bmax * q.C);
+                           q.dc + t * Bmax * q.C, last ? nullptr : q.dc + (t + 1) * Bmax * q.C, q.part, nparts);
         MYEA_HIP_TRY(hipGetLastError());
     }
     return MYEA_OK;
@@ -408,37 +444,61 @@ int Net::lstm_update_derivative_weight(size_t li, size_t B)
     const float *x = layer_outputs(li - 1);
     const LstmGeom geom = geom_of(q);
     const bool per_t = T > 1 && B != Bmax;
-    // input weights: dG^T X over every (t, b)
-    {
-        const size_t chunks = per_t ? T : 1, rows = per_t ? B : T * B;
-        for (size_t c = 0; c < chunks; ++c) {
+    // input weights: dG^T X over every (t, b).  M x N is small and K = T*B is long: split K into slabs so that the
+    // launch fills the chip; the scatter kernel sums the slabs in order.
+    int s_in = 1, s_rec = 0;
+    if (!per_t) {
+        const size_t rows = T * B;
+        GemmParams g{};
+        g.A = q.dG; g.lda = (long)q.G; g.a_k_contiguous = 0;
+        g.B = x; g.ldb = (long)q.In; g.b_k_contiguous = 0;
+        g.C = q.gWin; g.ldc = (long)q.In;
+        g.M = (int)q.G; g.N = (int)q.In; g.K = (int)rows;
+        s_in = gemm_split_k(g.M, g.N, g.K);
+        g.split_k = s_in; g.split_k_slab = (long)(q.G * q.In);
+        prof_begin(2);
+        MYEA_TRY(launch_gemm(stream, g));
+        prof_end(2.0 * (double)rows * (double)q.G * (double)q.In);
+    } else {
+        for (size_t c = 0; c < T; ++c) {
             GemmParams g{};
             g.A = q.dG + c * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
             g.B = x + c * Bmax * q.In; g.ldb = (long)q.In; g.b_k_contiguous = 0;
             g.C = q.gWin; g.ldc = (long)q.In; g.accumulate = c > 0;
-            g.M = (int)q.G; g.N = (int)q.In; g.K = (int)rows;
+            g.M = (int)q.G; g.N = (int)q.In; g.K = (int)B;
             prof_begin(2);
             MYEA_TRY(launch_gemm(stream, g));
-            prof_end(2.0 * (double)rows * (double)q.G * (double)q.In);
+            prof_end(2.0 * (double)B * (double)q.G * (double)q.In);
         }
     }
     // recurrent weights: dG[t+1]^T h[t] for t < T-1
-    const bool with_rec = T > 1;
-    if (with_rec) {
-        const size_t chunks = per_t ? T - 1 : 1, rows = per_t ? B : (T - 1) * B;
-        for (size_t c = 0; c < chunks; ++c) {
+    if (T > 1 && !per_t) {
+        const size_t rows = (T - 1) * B;
+        GemmParams g{};
+        g.A = q.dG + Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
+        g.B = o.values; g.ldb = (long)q.C; g.b_k_contiguous = 0;
+        g.C = q.gWrec; g.ldc = (long)q.C;
+        g.M = (int)q.G; g.N = (int)q.C; g.K = (int)rows;
+        s_rec = gemm_split_k(g.M, g.N, g.K);
+        g.split_k = s_rec; g.split_k_slab = (long)(q.G * q.C);
+        prof_begin(2);
+        MYEA_TRY(launch_gemm(stream, g));
+        prof_end(2.0 * (double)rows * (double)q.G * (double)q.C);
+    } else if (T > 1) {
+        s_rec = 1;
+        for (size_t c = 0; c + 1 < T; ++c) {
             GemmParams g{};
             g.A = q.dG + (c + 1) * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
             g.B = o.values + c * Bmax * q.C; g.ldb = (long)q.C; g.b_k_contiguous = 0;
             g.C = q.gWrec; g.ldc = (long)q.C; g.accumulate = c > 0;
-            g.M = (int)q.G; g.N = (int)q.C; g.K = (int)rows;
+            g.M = (int)q.G; g.N = (int)q.C; g.K = (int)B;
             prof_begin(2);
             MYEA_TRY(launch_gemm(stream, g));
-            prof_end(2.0 * (double)rows * (double)q.G * (double)q.C);
+            prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
         }
     }
-    hipLaunchKernelGGL(lstm_scatter_add_kernel, dim3(grid_for(q.G * (q.In + q.C), kBlock, 4096)), dim3(kBlock), 0, stream, geom, gradient, q.gWin, q.gWrec,
-                       (int)with_rec);
+    hipLaunchKernelGGL(lstm_scatter_add_kernel, dim3(grid_for(q.G * (q.In + q.C), kBlock, 4096)), dim3(kBlock), 0, stream, geom, gradient, q.gWin, s_in,
+                       q.gWrec, s_rec);
     MYEA_HIP_TRY(hipGetLastError());
     // peepholes
     {

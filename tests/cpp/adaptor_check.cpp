@@ -1,0 +1,97 @@
+// adaptor_check.cpp — drives the C++ adaptor `Neural_Network_HIP` exactly as a host program drives the reference's
+// `Neural_Network` (Compile -> Set__* -> Set__HIP -> the 4-call step loop + Update_Parameter, cf.
+// Neural_Network_Launcher_Windows/Source_Files/debug.cpp:481-1555 and Neural_Network/Dataset.cpp:645-658).
+// usage: adaptor_check <dir> <kind>   reads <dir>/{w,x,y,mask}.bin, writes <dir>/{params,grad}.bin and prints the loss.
+#include <cstdio>
+#include <cstdlib>
+#include <string>
+#include <vector>
+
+#include "../../include/myea_nn_hip.hpp"
+
+using namespace MyEA_HIP;
+
+static std::vector<float> read_f32(const std::string &path)
+{
+    FILE *f = std::fopen(path.c_str(), "rb");
+    if (!f) { std::printf("can not open %s\n", path.c_str()); std::exit(2); }
+    std::fseek(f, 0, SEEK_END);
+    long n = std::ftell(f);
+    std::fseek(f, 0, SEEK_SET);
+    std::vector<float> v(n / 4);
+    if (std::fread(v.data(), 4, v.size(), f) != v.size()) std::exit(2);
+    std::fclose(f);
+    return v;
+}
+static void write_f32(const std::string &path, const float *p, size_t n)
+{
+    FILE *f = std::fopen(path.c_str(), "wb");
+    std::fwrite(p, 4, n, f);
+    std::fclose(f);
+}
+
+int main(int argc, char **argv)
+{
+    if (argc < 3) return 2;
+    const std::string dir = argv[1], kind = argv[2];
+    Neural_Network_HIP nn;
+    size_t B, T, n_in, n_out, steps = 3;
+    if (kind == "mlp") {  // FC 20 -> 32 (BN before, ReLU, inverted dropout .5) -> 24 tanh -> 6 softmax, Nesterov
+        B = 16; T = 1; n_in = 20; n_out = 6;
+        Layer_Parameters layers[4];
+        for (auto &l : layers) l.type_layer = MYEA_LAYER_FULLY_CONNECTED;
+        layers[0].unit_parameters[0] = 20; layers[1].unit_parameters[0] = 32; layers[2].unit_parameters[0] = 24; layers[3].unit_parameters[0] = 6;
+        if (!nn.Update__Batch_Size(B)) return 1;
+        if (!nn.Compile(4, T, MYEA_NETWORK_FEEDFORWARD, layers)) return 1;
+        T_ keep[2] = {0.5f, 0.f};
+        if (!nn.Set__Layer_Activation_Function(1, MYEA_AF_RELU) || !nn.Set__Layer_Activation_Function(2, MYEA_AF_TANH) ||
+            !nn.Set__Layer_Activation_Function(3, MYEA_AF_SOFTMAX) || !nn.Set__Layer_Normalization(1, MYEA_NORMALIZATION_BATCH_NORMALIZATION, true) ||
+            !nn.Set__Dropout(1, MYEA_DROPOUT_BERNOULLI_INVERTED, keep)) return 1;
+        nn.Set__Loss_Function(MYEA_LOSS_CROSS_ENTROPY);
+        nn.Set__Accuracy_Function(MYEA_ACCURACY_CROSS_ENTROPY);
+        nn.Set__Optimizer_Function(MYEA_OPTIMIZER_GD);
+        nn.use_Nesterov = true;
+    } else {  // LSTM 8 -> 2 x LSTM-12 -> FC-12 linear, AMSGrad, clip 1.0
+        B = 6; T = 5; n_in = 8; n_out = 12;
+        Layer_Parameters layers[4];
+        layers[0].type_layer = MYEA_LAYER_FULLY_CONNECTED; layers[0].unit_parameters[0] = 8;
+        layers[1].type_layer = MYEA_LAYER_LSTM; layers[1].unit_parameters[0] = 12; layers[1].unit_parameters[1] = 1;
+        layers[2].type_layer = MYEA_LAYER_LSTM; layers[2].unit_parameters[0] = 6; layers[2].unit_parameters[1] = 2;
+        layers[3].type_layer = MYEA_LAYER_FULLY_CONNECTED; layers[3].unit_parameters[0] = 12;
+        if (!nn.Update__Batch_Size(B)) return 1;
+        if (!nn.Compile(4, T, MYEA_NETWORK_RECURRENT, layers)) return 1;
+        if (!nn.Set__Layer_Activation_Function(3, MYEA_AF_LINEAR)) return 1;
+        nn.Set__Loss_Function(MYEA_LOSS_MSE);
+        nn.Set__Optimizer_Function(MYEA_OPTIMIZER_AMSGRAD);
+        nn.Set__Clip_Gradient(true);
+        nn.Set__Clip_Gradient(1.0f);
+    }
+    std::vector<float> w = read_f32(dir + "/w.bin"), x = read_f32(dir + "/x.bin"), y = read_f32(dir + "/y.bin"), m = read_f32(dir + "/mask.bin");
+    if (w.size() != nn.total_parameters) { std::printf("parameter count %zu != %zu\n", w.size(), nn.total_parameters); return 1; }
+    for (size_t i = 0; i < w.size(); ++i) nn.ptr_array_parameters[i] = w[i];
+    for (size_t i = 0; i < m.size() && i < nn.Get__Descriptor().total_mask_units; ++i) nn.ptr_array_units_mask_dropout_bernoulli[i] = m[i] != 0.f;
+    if (!nn.Set__HIP(true)) return 1;
+    nn.type_state_propagation = MYEA_STATE_TRAINING;
+    nn.Clear_Training_Arrays();
+    std::vector<const float *> xr(B), yr(B);
+    for (size_t b = 0; b < B; ++b) { xr[b] = x.data() + b * T * n_in; yr[b] = y.data() + b * T * n_out; }
+    std::vector<float> grad(nn.total_parameters);
+    for (size_t s = 0; s < steps; ++s) {
+        nn.Reset__Loss();
+        nn.Forward_Pass(B, xr.data());
+        nn.Compute__Error(B, yr.data());
+        nn.Backward_Pass(B);
+        nn.Update_Derivative_Weight(B);
+        if (s + 1 == steps && !nn.Copy__Derivatives_Parameters__Device_To_Host(grad.data())) return 1;
+        std::printf("step %zu loss %.9g\n", s, (double)nn.Get__Loss());
+        nn.Update_Parameter(B, B);
+    }
+    if (!nn.Copy__Parameters__Device_To_Host()) return 1;
+    write_f32(dir + "/params.bin", nn.ptr_array_parameters, nn.total_parameters);
+    write_f32(dir + "/grad.bin", grad.data(), grad.size());
+    // error behaviour: a batch larger than the allocated one prints and returns, leaving the network usable
+    std::vector<const float *> big(B + 1, x.data());
+    nn.Forward_Pass(B + 1, big.data());
+    std::printf("time step %.1f\n", (double)nn.optimizer_time_step);
+    return 0;
+}
