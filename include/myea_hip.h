@@ -198,6 +198,9 @@ enum {
     MYEA_TENSOR_NORM_VARIANCES = 5, /* [T][H] batch sqrt(var+eps) */
     MYEA_TENSOR_NORM_MEANS_AVERAGES = 6,
     MYEA_TENSOR_NORM_VARIANCES_AVERAGES = 7,
+    MYEA_TENSOR_INPUT_SIDE_ERRORS = 8,  /* member of a residual block: delta reduced to the layer's input side
+                                           [Bmax][fan-in] (AF_unit errors, or the normalised units' errors when
+                                           the member is normalised); absent for an un-normalised first member */
     /* LSTM taps, [T][Bmax][cells] or [T][Bmax][blocks] */
     MYEA_TENSOR_LSTM_CELL_INPUT = 16,      /* z  */
     MYEA_TENSOR_LSTM_CELL_STATE = 17,      /* c  */
@@ -223,6 +226,16 @@ void myea_hyper_default(myea_hyper *hyper);
  * normalised-unit scale/shift region (Neural_Network__Layer_Normalization.cpp:20-78,
  * Neural_Network__Allocate.cpp:2378-2462) and the mask offsets (Neural_Network.cpp:3948-3962). */
 int myea_net_desc_layout(myea_net_desc *desc);
+
+/* Layer::previous_connected_layers[0] as Organize__Previous_Layers_Connected (Neural_Network.cpp:20-57)
+ * assigns it: the layer before, except that the first layer after a residual block connects to the
+ * block's residual layer and the first layer inside a block to the layer the residual layer connects
+ * to (the shortcut source).  0 for li == 0 or out of range. */
+uint32_t myea_net_desc_previous_layer(const myea_net_desc *desc, uint32_t layer_index);
+
+/* *Layer::ptr_number_outputs: FC neurons; LSTM blocks x cells per block; residual = max(shortcut
+ * source width, width of the block's last layer) (Neural_Network__Compile.cpp:79,272-281). */
+uint64_t myea_net_desc_number_outputs(const myea_net_desc *desc, uint32_t layer_index);
 
 /* ---- life cycle: replaces Set__CUDA / Initialize__CUDA / Deinitialize__CUDA (Data.hpp:3111-3118) ---- */
 typedef struct myea_hip_net myea_hip_net;

@@ -30,7 +30,7 @@ ACCURACY = dict(NONE=0, CROSS_ENTROPY=1, DIRECTIONAL=2, DISTANCE=3, SIGN=5)
 STATE_INFERENCE, STATE_TRAINING = 0, 1
 OPT_STATE = dict(PREVIOUS_DELTA=0, FIRST_MOMENT=1, SECOND_MOMENT=2, SECOND_MOMENT_HAT=3)
 TENSOR = dict(OUTPUTS=0, SUMMATIONS=1, ERRORS=2, NORM_HATS=3, NORM_MEANS=4, NORM_VARIANCES=5,
-              NORM_MEANS_AVERAGES=6, NORM_VARIANCES_AVERAGES=7,
+              NORM_MEANS_AVERAGES=6, NORM_VARIANCES_AVERAGES=7, INPUT_SIDE_ERRORS=8,
               LSTM_CELL_INPUT=16, LSTM_CELL_STATE=17, LSTM_INPUT_GATE=18, LSTM_FORGET_GATE=19,
               LSTM_OUTPUT_GATE=20, LSTM_DELTA_CELL_INPUT=21, LSTM_DELTA_CELL_STATE=22,
               LSTM_DELTA_INPUT_GATE=23, LSTM_DELTA_FORGET_GATE=24, LSTM_DELTA_OUTPUT_GATE=25)
@@ -82,7 +82,7 @@ class LossState(C.Structure):
 
 # every symbol include/myea_hip.h declares
 ABI_SYMBOLS = [
-    "myea_hyper_default", "myea_net_desc_layout", "myea_hip_create", "myea_hip_destroy", "myea_hip_set_stream",
+    "myea_hyper_default", "myea_net_desc_layout", "myea_net_desc_previous_layer", "myea_net_desc_number_outputs", "myea_hip_create", "myea_hip_destroy", "myea_hip_set_stream",
     "myea_hip_synchronize", "myea_hip_last_error", "myea_hip_set_hyper", "myea_hip_get_hyper",
     "myea_hip_set_state_propagation", "myea_hip_upload_parameters", "myea_hip_download_parameters",
     "myea_hip_upload_optimizer_state", "myea_hip_download_optimizer_state", "myea_hip_upload_masks",
@@ -107,6 +107,10 @@ def load_library(path=LIB_PATH):
     lib.myea_hyper_default.argtypes = [P(Hyper)]
     lib.myea_hyper_default.restype = None
     lib.myea_net_desc_layout.argtypes = [P(NetDesc)]
+    lib.myea_net_desc_previous_layer.argtypes = [P(NetDesc), u32]
+    lib.myea_net_desc_previous_layer.restype = u32
+    lib.myea_net_desc_number_outputs.argtypes = [P(NetDesc), u32]
+    lib.myea_net_desc_number_outputs.restype = C.c_uint64
     lib.myea_hip_create.argtypes = [P(NetDesc), P(vp)]
     lib.myea_hip_destroy.argtypes = [vp]
     lib.myea_hip_set_stream.argtypes = [vp, vp]

@@ -442,6 +442,35 @@ int launch_activation_derive(hipStream_t s, int act, float steep, size_t n, cons
     return MYEA_OK;
 }
 
+// Forward_Pass__Zero_Padded_Identity (NN/Neural_Network__Forward_Pass__OpenMP.cpp:5158-5240) and
+// Backward_Pass__Residual (NN/Neural_Network__Backward_Pass__OpenMP.cpp:1155-1215) as one shifted add.
+__global__ void padded_add_kernel(size_t n, size_t wo, const float *__restrict__ a, size_t wa, long sa,
+                                  const float *__restrict__ b, size_t wb, long sb, float *__restrict__ out)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / wo;
+        const long j = (long)(i - r * wo);
+        float v = 0.f;
+        const long ja = j + sa;
+        if (ja >= 0 && ja < (long)wa) v = a[r * wa + (size_t)ja];
+        if (b) {
+            const long jb = j + sb;
+            if (jb >= 0 && jb < (long)wb) v += b[r * wb + (size_t)jb];
+        }
+        out[i] = v;
+    }
+}
+
+int launch_padded_add(hipStream_t s, size_t rows, size_t wo, const float *a, size_t wa, long sa,
+                      const float *b, size_t wb, long sb, float *out)
+{
+    const size_t n = rows * wo;
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(padded_add_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, n, wo, a, wa, sa, b, wb, sb, out);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
 int launch_colscale(hipStream_t s, size_t rows, size_t H, float *y, const float *colscale)
 {
     const size_t n = rows * H;

@@ -141,6 +141,8 @@ struct GemmDev {
     const float *pre, *val;
     int act;
     float steep;
+    const float *addend;
+    long ld_addend;
     int nbm, nbn;
     int ksplit, kchunk;   // split-K: number of slabs and k's per slab (multiple of BK); slab s writes C + s * slab
     long slab;
@@ -241,6 +243,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
                 if (row >= p.M) continue;
                 const long o = (long)row * p.ldc + col + (long)split * p.slab;
                 float v = acc[i][j][r];
+                if (p.addend) v += p.addend[(long)row * p.ld_addend + col];
                 if (p.epilogue == EPI_FC_FORWARD) {
                     v += bias;
                     p.C[o] = v;
@@ -344,10 +347,12 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     d.accumulate = p.accumulate; d.epilogue = p.epilogue;
     d.bias = p.bias; d.aux_out = p.aux_out; d.colscale = p.colscale;
     d.pre = p.pre; d.val = p.val; d.act = p.act; d.steep = p.steep;
+    d.addend = p.addend; d.ld_addend = p.ld_addend;
+    if (p.addend && (p.epilogue == EPI_FC_FORWARD || p.ld_addend < p.N)) { set_last_error("gemm: addend needs EPI_NONE / EPI_FC_DERIVE and ld_addend >= N"); return MYEA_E_INVALID; }
     d.nbm = d.nbn = 0;
     d.ksplit = 1; d.kchunk = p.K > 0 ? p.K : 1; d.slab = 0;
     if (p.split_k > 1) {
-        if (p.epilogue != EPI_NONE || p.accumulate) { set_last_error("gemm: split-K writes plain partial slabs"); return MYEA_E_INVALID; }
+        if (p.epilogue != EPI_NONE || p.accumulate || p.addend) { set_last_error("gemm: split-K writes plain partial slabs"); return MYEA_E_INVALID; }
         const int chunk = ((p.K + p.split_k - 1) / p.split_k + kBK - 1) / kBK * kBK;
         d.kchunk = chunk;
         d.ksplit = (p.K + chunk - 1) / chunk;

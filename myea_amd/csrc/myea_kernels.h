@@ -41,6 +41,10 @@ struct GemmParams {
     const float *val;       // EPI_FC_DERIVE, [M][ldc]
     int act;
     float steep;
+    // EPI_NONE / EPI_FC_DERIVE: addend[row * ld_addend + col] joins the product before the epilogue (the shortcut
+    // gradient of a residual block arriving at the same destination); may be null
+    const float *addend;
+    long ld_addend;
     // split-K (deterministic): slab s of the K range writes its partial product to C + s * split_k_slab; the consumer
     // sums the slabs in order.  Requires EPI_NONE and accumulate == 0.  0 / 1 = off.
     int split_k;
@@ -55,6 +59,11 @@ bool gemm_can_fuse_activation(int act);
 // ---- elementwise / reduction kernels ------------------------------------------------------------
 // rows are the leading dimension everywhere: element (r, j) at base[r * H + j].
 
+// out[r][j] = A[r][j + sa] + B[r][j + sb] for j in [0, wo), where an operand contributes zero outside its own width
+// (wa, wb) and B may be null: the zero-padded identity shortcut (narrower operand shifted by -padding) and its gradient
+// (wider operand cropped at +padding).  out may alias neither operand unless the shifts are zero.
+int launch_padded_add(hipStream_t s, size_t rows, size_t wo, const float *a, size_t wa, long sa,
+                      const float *b, size_t wb, long sb, float *out);
 // y = AF(x) * colscale[j]  (colscale may be null); x and y may alias.
 int launch_activation(hipStream_t s, int act, size_t rows, size_t H, const float *x, float *y, const float *colscale);
 // row softmax (max-subtracted) then * colscale

@@ -39,29 +39,49 @@ void myea_hyper_default(myea_hyper *h)
     h->number_time_delays = 0;
 }
 
-/* *Layer::ptr_number_outputs: FC = neurons; LSTM = blocks * cells per direction
- * (NN/Neural_Network__Compile.cpp:79); residual = width of the block's last layer. */
-static uint64_t number_outputs(const myea_net_desc *d, uint32_t li)
+/* Index of the residual layer whose block contains layer li, or 0 when li is outside every block
+ * (layer 0 is the input layer and never a residual layer).  Blocks do not nest here. */
+static uint32_t enclosing_block(const myea_net_desc *d, uint32_t li)
 {
+    for (uint32_t r = 1; r < li; ++r) {
+        const myea_layer_desc *l = &d->layers[r];
+        if (l->type_layer == MYEA_LAYER_RESIDUAL && li <= r + l->block_depth) return r;
+    }
+    return 0;
+}
+
+/* previous_connected_layers[0] (Organize__Previous_Layers_Connected, NN/Neural_Network.cpp:20-57): the layer
+ * before; the first layer after a residual block connects to the block's residual layer; the first layer inside a
+ * block connects to what the residual layer itself connects to (the shortcut source). */
+uint32_t myea_net_desc_previous_layer(const myea_net_desc *d, uint32_t li)
+{
+    if (!d || li == 0 || li >= d->n_layers) return 0;
+    uint32_t before = li - 1;
+    if (d->layers[before].type_layer == MYEA_LAYER_RESIDUAL) return myea_net_desc_previous_layer(d, before);
+    uint32_t r = enclosing_block(d, before);
+    if (r != 0 && before == r + d->layers[r].block_depth && enclosing_block(d, li) != r) return r;
+    return before;
+}
+
+/* *Layer::ptr_number_outputs: FC = neurons; LSTM = blocks * cells per direction
+ * (NN/Neural_Network__Compile.cpp:79); residual = the wider of the shortcut source and the block's last layer
+ * (Assign__Post__Layer, NN/Neural_Network__Compile.cpp:272-281). */
+uint64_t myea_net_desc_number_outputs(const myea_net_desc *d, uint32_t li)
+{
+    if (!d || li >= d->n_layers) return 0;
     const myea_layer_desc *l = &d->layers[li];
     switch (l->type_layer) {
     case MYEA_LAYER_LSTM: return (uint64_t)l->n_units * l->n_cells_per_block;
-    case MYEA_LAYER_RESIDUAL: return number_outputs(d, li + l->block_depth);
+    case MYEA_LAYER_RESIDUAL: {
+        uint64_t a = myea_net_desc_number_outputs(d, myea_net_desc_previous_layer(d, li));
+        uint64_t b = myea_net_desc_number_outputs(d, li + l->block_depth);
+        return a > b ? a : b;
+    }
     default: return l->n_units;
     }
 }
-
-/* previous_connected_layers[0] for a sequential stack: the layer before, except that the first layer
- * after a residual block connects to the block's unit (NN/Neural_Network__Ordered.cpp, Order__Layers__Connection). */
-static uint32_t previous_layer(const myea_net_desc *d, uint32_t li)
-{
-    /* walk back: if li-1 is the last layer inside a residual block, the producer is that block's layer */
-    for (uint32_t r = 0; r + 1 < li; ++r) {
-        const myea_layer_desc *l = &d->layers[r];
-        if (l->type_layer == MYEA_LAYER_RESIDUAL && r + l->block_depth == li - 1) return r;
-    }
-    return li - 1;
-}
+#define number_outputs myea_net_desc_number_outputs
+#define previous_layer myea_net_desc_previous_layer
 
 int myea_net_desc_layout(myea_net_desc *d)
 {
@@ -79,6 +99,16 @@ int myea_net_desc_layout(myea_net_desc *d)
         if (l->type_normalization != MYEA_NORMALIZATION_NONE) any_norm = 1;
     }
     if (d->layers[0].type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_INVALID;
+    /* residual blocks: depth >= 1, wholly inside the stack, followed by at least one layer, fully-connected
+     * members only, no block inside a block */
+    for (uint32_t li = 1; li < d->n_layers; ++li) {
+        const myea_layer_desc *l = &d->layers[li];
+        if (l->type_layer != MYEA_LAYER_RESIDUAL) continue;
+        if (l->block_depth == 0 || (uint64_t)li + l->block_depth + 1 >= d->n_layers) return MYEA_E_INVALID;
+        for (uint32_t k = 1; k <= l->block_depth; ++k)
+            if (d->layers[li + k].type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_UNSUPPORTED;
+        li += l->block_depth;
+    }
 
     /* weights: Prepare__Connections__FC / __LSTM, NN/Neural_Network__Prepare_Connections.cpp:20-222 */
     for (uint32_t li = 1; li < d->n_layers; ++li) {
@@ -126,17 +156,26 @@ int myea_net_desc_layout(myea_net_desc *d)
         if (l->type_layer == MYEA_LAYER_LSTM) {
             uint64_t dirs = l->use_bidirectional ? 2u : 1u;
             total_norm += 3u * (uint64_t)l->n_units * l->n_cells_per_block * dirs + 6u * (uint64_t)l->n_units * dirs;
+        } else if (l->type_layer == MYEA_LAYER_RESIDUAL) {
+            total_norm += number_outputs(d, li + l->block_depth);   /* Prepare__Normalized__Layer, :60-67 */
+        } else if (enclosing_block(d, li) != 0) {
+            total_norm += number_outputs(d, previous_layer(d, li)); /* Prepare__Normalized__Residual_Layer: fan-in wide */
         } else {
             total_norm += number_outputs(d, li);
         }
     }
     /* Bernoulli masks: (AF units of the layer) * T per layer, in layer order
-     * (Reset__Parameter__Mask_Dropout, NN/Neural_Network.cpp:3948-3962); LSTM layers own no AF unit. */
+     * (Reset__Parameter__Mask_Dropout, NN/Neural_Network.cpp:3948-3962); LSTM and residual layers own no AF unit. */
     uint64_t total_mask = 0;
     for (uint32_t li = 0; li < d->n_layers; ++li) {
         myea_layer_desc *l = &d->layers[li];
         l->first_mask_index = total_mask;
-        if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) total_mask += (uint64_t)l->n_units * d->number_recurrent_depth;
+        if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED) continue;
+        uint32_t r = li ? enclosing_block(d, li) : 0;
+        /* inside a block the activation units sit on the layer's input side: none for the block's first layer, fan-in
+         * many for the others (Assign__Post__Residual_Layer, NN/Neural_Network__Compile.cpp:378-384) */
+        uint64_t af_units = r == 0 ? l->n_units : (li == r + 1 ? 0 : number_outputs(d, previous_layer(d, li)));
+        total_mask += af_units * d->number_recurrent_depth;
     }
     d->total_weights = total_weights;
     d->total_bias = total_bias;

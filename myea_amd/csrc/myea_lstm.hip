@@ -286,7 +286,7 @@ int Net::lstm_create_layer(size_t li)
     if (l.n_cells_per_block == 0) { set_last_error("layer %zu: LSTM needs at least one cell per block", li); return MYEA_E_INVALID; }
     LstmLayer *q = new LstmLayer();
     o.lstm = q;
-    q->K = l.n_units; q->cpb = l.n_cells_per_block; q->C = q->K * q->cpb; q->G = q->C + 3 * q->K; q->In = L[li - 1].H;
+    q->K = l.n_units; q->cpb = l.n_cells_per_block; q->C = q->K * q->cpb; q->G = q->C + 3 * q->K; q->In = L[li].In;
     q->per_block = q->cpb * (q->In + q->C) + 3 * q->In + 3 * q->C + 3 * q->cpb;
     q->base = l.first_connection_index;
     if (q->base + q->K * q->per_block > d.total_weights) { set_last_error("layer %zu: LSTM weight slice leaves the weight region", li); return MYEA_E_INVALID; }
@@ -351,7 +351,7 @@ int Net::lstm_forward_layer(size_t li, size_t B)
     DevLayer &o = L[li];
     LstmLayer &q = *o.lstm;
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
-    const float *x = layer_outputs(li - 1);
+    const float *x = layer_outputs(L[li].prev);
     const float *bias = parameters + l.first_bias_connection_index;
     // input sums of every time step in one contraction when the rows are contiguous
     const bool per_t = T > 1 && B != Bmax;
@@ -441,7 +441,7 @@ int Net::lstm_update_derivative_weight(size_t li, size_t B)
     DevLayer &o = L[li];
     LstmLayer &q = *o.lstm;
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
-    const float *x = layer_outputs(li - 1);
+    const float *x = layer_outputs(L[li].prev);
     const LstmGeom geom = geom_of(q);
     const bool per_t = T > 1 && B != Bmax;
     // input weights: dG^T X over every (t, b).  M x N is small and K = T*B is long: split K into slabs so that the

@@ -13,9 +13,19 @@ struct LstmLayer;  // myea_lstm.hip
 
 struct DevLayer {
     size_t H = 0;  // *Layer::ptr_number_outputs
-    // [T][Bmax][H]
+    // connections (Organize__Previous_Layers_Connected / Organize__Layer__Group, NN/Neural_Network.cpp:20-125)
+    size_t prev = 0;  // previous_connected_layers[0]
+    int group = 0;    // 0 outside a residual block, 1 first member of a block, 2 other members
+    size_t In = 0;    // width of the producer
+    // width of the activation-unit tensors (values, colscale) and of the normalised-unit tensors: H outside a block;
+    // a block member carries both on its input side (In wide, no activation units on the first member); a residual
+    // layer keeps its basic units in values / neuron_errors (H wide) and normalises the block's last member (NH wide)
+    size_t AH = 0, NH = 0;
+    size_t pad = 0;   // residual layer: column offset of the narrower shortcut operand (pooling_values[2])
+    // [T][Bmax][H] (summations, neuron_errors), [T][Bmax][AH] (values), [T][Bmax][NH] (hats, normalizes)
     float *summations = nullptr, *values = nullptr, *hats = nullptr, *normalizes = nullptr, *neuron_errors = nullptr;
-    // [T][H]
+    float *in_errors = nullptr;  // normalised first member of a block: delta reduced to its input side [Bmax][In]
+    // [T][NH]
     float *means = nullptr, *variances = nullptr, *means_averages = nullptr, *variances_averages = nullptr;
     float *r_corrections = nullptr, *d_corrections = nullptr;
     float *colscale = nullptr;  // dropout multiplier per (t, unit)
@@ -62,6 +72,8 @@ struct Net {
     int bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training);
     int bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx);
     int backward_into_layer(size_t li, size_t B);
+    int forward_residual_block(size_t ri, size_t B);
+    int backward_residual_block(size_t ri, size_t B);
 
     int forward_pass(size_t B, const float *inputs, int on_device);
     int compute_error(size_t B, const float *desired, int on_device);

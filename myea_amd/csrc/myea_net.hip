@@ -56,8 +56,11 @@ float *Net::layer_outputs(size_t li)
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
-    if (li != 0 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED && layer_uses_norm(l) && !l.use_layer_normalization_before_activation) return o.normalizes;
-    return o.values;
+    if (li != 0 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (o.group) return o.summations;  // residual group: the member's output is its summation (NN/Neural_Network__Ordered.cpp:96-141)
+        if (layer_uses_norm(l) && !l.use_layer_normalization_before_activation) return o.normalizes;
+    }
+    return o.values;  // LSTM: cell outputs; residual layer: its basic units' values
 }
 
 float *Net::scale_ptr(float *base, size_t li) { return base + d.total_weights + d.total_bias + d.layers[li].first_normalized_unit_index; }
@@ -91,11 +94,36 @@ static int check_desc(const myea_net_desc &d)
     if (d.batch_size == 0 || d.number_recurrent_depth == 0) { set_last_error("descriptor: batch_size and number_recurrent_depth must be >= 1"); return MYEA_E_INVALID; }
     if (d.total_parameters != d.total_weights + d.total_bias + 2 * d.total_normalized_units) { set_last_error("descriptor: total_parameters inconsistent"); return MYEA_E_INVALID; }
     if (d.layers[0].type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("descriptor: the input layer must be a fully-connected (unit) layer"); return MYEA_E_INVALID; }
+    // residual blocks: members are the block_depth fully-connected layers after the residual layer, a consumer follows
+    bool any_residual = false, any_lstm = false;
+    uint32_t block_end = 0;  // index of the last member of the block being walked, 0 outside
+    std::vector<int> group(d.n_layers, 0);
     for (uint32_t li = 0; li < d.n_layers; ++li) {
         const myea_layer_desc &l = d.layers[li];
-        if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED && l.type_layer != MYEA_LAYER_LSTM) {
+        if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED && l.type_layer != MYEA_LAYER_LSTM && l.type_layer != MYEA_LAYER_RESIDUAL) {
             set_last_error("layer %u: type %u is not on this path", li, l.type_layer);
             return MYEA_E_UNSUPPORTED;
+        }
+        if (block_end != 0) {
+            if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("layer %u: only fully-connected layers may sit inside a residual block", li); return MYEA_E_UNSUPPORTED; }
+            group[li] = (d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) ? 1 : 2;
+            if (li == block_end) block_end = 0;
+        } else if (l.type_layer == MYEA_LAYER_RESIDUAL) {
+            if (l.block_depth == 0 || (uint64_t)li + l.block_depth + 1 >= d.n_layers) { set_last_error("layer %u: residual block of depth %u does not fit in front of a consumer", li, l.block_depth); return MYEA_E_INVALID; }
+            if (l.type_dropout != MYEA_DROPOUT_NONE) { set_last_error("layer %u: block-level dropout (ShakeDrop) is not on this path", li); return MYEA_E_UNSUPPORTED; }
+            any_residual = true;
+            block_end = li + l.block_depth;
+        }
+        if (l.type_layer == MYEA_LAYER_LSTM) any_lstm = true;
+    }
+    if (any_residual && (any_lstm || d.number_recurrent_depth != 1)) { set_last_error("descriptor: residual blocks are on this path for feed-forward stacks only"); return MYEA_E_UNSUPPORTED; }
+    for (uint32_t li = 0; li < d.n_layers; ++li) {
+        const myea_layer_desc &l = d.layers[li];
+        if (l.type_layer == MYEA_LAYER_RESIDUAL) {
+            const uint64_t nh = myea_net_desc_number_outputs(&d, li + l.block_depth);
+            if (layer_uses_norm(l) && l.first_normalized_unit_index + nh > d.total_normalized_units) { set_last_error("layer %u: scale/shift slice leaves its region", li); return MYEA_E_INVALID; }
+            if (l.type_normalization > MYEA_NORMALIZATION_BATCH_RENORMALIZATION) { set_last_error("layer %u: normalization type %u is not on this path", li, l.type_normalization); return MYEA_E_UNSUPPORTED; }
+            continue;
         }
         if (l.n_units == 0) { set_last_error("layer %u: no units", li); return MYEA_E_INVALID; }
         if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_BERNOULLI && l.type_dropout != MYEA_DROPOUT_BERNOULLI_INVERTED) {
@@ -104,13 +132,18 @@ static int check_desc(const myea_net_desc &d)
         }
         if (l.type_normalization > MYEA_NORMALIZATION_BATCH_RENORMALIZATION) { set_last_error("layer %u: normalization type %u is not on this path", li, l.type_normalization); return MYEA_E_UNSUPPORTED; }
         if (l.type_layer == MYEA_LAYER_FULLY_CONNECTED && li > 0) {
-            if (l.type_activation_function == MYEA_AF_NONE || l.type_activation_function >= MYEA_AF_LENGTH) { set_last_error("layer %u: activation %u invalid", li, l.type_activation_function); return MYEA_E_INVALID; }
-            const size_t fan_in = (d.layers[li - 1].type_layer == MYEA_LAYER_LSTM) ? (size_t)d.layers[li - 1].n_units * d.layers[li - 1].n_cells_per_block : d.layers[li - 1].n_units;
+            const bool has_af = group[li] != 1;
+            if (has_af && (l.type_activation_function == MYEA_AF_NONE || l.type_activation_function >= MYEA_AF_LENGTH)) { set_last_error("layer %u: activation %u invalid", li, l.type_activation_function); return MYEA_E_INVALID; }
+            if (group[li] == 2 && l.type_activation_function == MYEA_AF_SOFTMAX) { set_last_error("layer %u: softmax belongs to the output layer only", li); return MYEA_E_UNSUPPORTED; }
+            const size_t fan_in = (size_t)myea_net_desc_number_outputs(&d, myea_net_desc_previous_layer(&d, li));
+            const size_t units_af = group[li] == 0 ? l.n_units : (group[li] == 1 ? 0 : fan_in), units_norm = group[li] == 0 ? l.n_units : fan_in;
             if (l.first_connection_index + fan_in * l.n_units > d.total_weights) { set_last_error("layer %u: weight slice leaves the weight region", li); return MYEA_E_INVALID; }
             if (layer_uses_bias(l) && l.first_bias_connection_index + l.n_units > d.total_weights + d.total_bias) { set_last_error("layer %u: bias slice leaves the bias region", li); return MYEA_E_INVALID; }
-            if (layer_uses_norm(l) && l.first_normalized_unit_index + l.n_units > d.total_normalized_units) { set_last_error("layer %u: scale/shift slice leaves its region", li); return MYEA_E_INVALID; }
+            if (layer_uses_norm(l) && l.first_normalized_unit_index + units_norm > d.total_normalized_units) { set_last_error("layer %u: scale/shift slice leaves its region", li); return MYEA_E_INVALID; }
+            if (l.type_dropout != MYEA_DROPOUT_NONE && l.first_mask_index + (uint64_t)units_af * d.number_recurrent_depth > d.total_mask_units) { set_last_error("layer %u: mask slice leaves the mask buffer", li); return MYEA_E_INVALID; }
+            if (l.type_dropout != MYEA_DROPOUT_NONE && group[li] == 1) { set_last_error("layer %u: the first layer of a residual block has no activation unit to drop", li); return MYEA_E_INVALID; }
         }
-        if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_layer == MYEA_LAYER_FULLY_CONNECTED &&
+        if (li == 0 && l.type_dropout != MYEA_DROPOUT_NONE &&
             l.first_mask_index + (uint64_t)l.n_units * d.number_recurrent_depth > d.total_mask_units) { set_last_error("layer %u: mask slice leaves the mask buffer", li); return MYEA_E_INVALID; }
     }
     return MYEA_OK;
@@ -140,26 +173,47 @@ int Net::create(const myea_net_desc &desc)
     for (size_t li = 0; li < d.n_layers; ++li) {
         const myea_layer_desc &l = d.layers[li];
         DevLayer &o = L[li];
-        o.H = (l.type_layer == MYEA_LAYER_LSTM) ? (size_t)l.n_units * l.n_cells_per_block : l.n_units;
+        o.H = (size_t)myea_net_desc_number_outputs(&d, (uint32_t)li);
+        o.prev = myea_net_desc_previous_layer(&d, (uint32_t)li);
+        o.In = li ? (size_t)myea_net_desc_number_outputs(&d, (uint32_t)o.prev) : 0;
+        o.group = 0;
+        if (li > 1 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+            if (d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) o.group = 1;
+            else if (L[li - 1].group != 0 && o.prev == li - 1) o.group = 2;  // the first layer after a block connects to the residual layer
+        }
+        if (l.type_layer == MYEA_LAYER_RESIDUAL) {
+            o.NH = (size_t)myea_net_desc_number_outputs(&d, (uint32_t)(li + l.block_depth));
+            o.AH = o.H;
+            o.pad = ((o.In > o.NH ? o.In - o.NH : o.NH - o.In) + 1) / 2;  // Assign__Post__Layer, NN/Neural_Network__Compile.cpp:277
+        } else {
+            o.AH = o.group == 0 ? o.H : (o.group == 1 ? 0 : o.In);
+            o.NH = o.group == 0 ? o.H : o.In;
+        }
         if (o.H > max_h) max_h = o.H;
-        const size_t sz = T * B * o.H;
-        MYEA_TRY(dev_alloc(&o.values, sz));
-        MYEA_HIP_TRY(hipMemset(o.values, 0, sz * sizeof(float)));
-        if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(dev_alloc(&o.colscale, T * o.H));
+        const size_t sz = T * B * o.H, sa = T * B * o.AH, sn = T * B * o.NH;
+        MYEA_TRY(dev_alloc(&o.values, sa));
+        MYEA_HIP_TRY(hipMemset(o.values, 0, (sa ? sa : 1) * sizeof(float)));
+        if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(dev_alloc(&o.colscale, T * o.AH));
         if (li == 0) continue;
         if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_create_layer(li)); continue; }
-        MYEA_TRY(dev_alloc(&o.summations, sz));
-        MYEA_TRY(dev_alloc(&o.neuron_errors, sz));
-        MYEA_HIP_TRY(hipMemset(o.summations, 0, sz * sizeof(float)));
+        if (l.type_layer != MYEA_LAYER_RESIDUAL) {
+            MYEA_TRY(dev_alloc(&o.summations, sz));
+            MYEA_HIP_TRY(hipMemset(o.summations, 0, sz * sizeof(float)));
+        }
+        MYEA_TRY(dev_alloc(&o.neuron_errors, sz));  // residual layer: its basic units' errors
         MYEA_HIP_TRY(hipMemset(o.neuron_errors, 0, sz * sizeof(float)));
         if (layer_uses_norm(l)) {
-            MYEA_TRY(dev_alloc(&o.hats, sz));
-            MYEA_TRY(dev_alloc(&o.normalizes, sz));
-            MYEA_HIP_TRY(hipMemset(o.hats, 0, sz * sizeof(float)));
-            MYEA_HIP_TRY(hipMemset(o.normalizes, 0, sz * sizeof(float)));
+            MYEA_TRY(dev_alloc(&o.hats, sn));
+            MYEA_TRY(dev_alloc(&o.normalizes, sn));
+            MYEA_HIP_TRY(hipMemset(o.hats, 0, sn * sizeof(float)));
+            MYEA_HIP_TRY(hipMemset(o.normalizes, 0, sn * sizeof(float)));
+            if (o.group == 1) {
+                MYEA_TRY(dev_alloc(&o.in_errors, sn));
+                MYEA_HIP_TRY(hipMemset(o.in_errors, 0, sn * sizeof(float)));
+            }
             float **small[] = {&o.means, &o.variances, &o.means_averages, &o.variances_averages, &o.r_corrections, &o.d_corrections};
-            for (float **s : small) { MYEA_TRY(dev_alloc(s, T * o.H)); MYEA_HIP_TRY(hipMemset(*s, 0, T * o.H * sizeof(float))); }
-            MYEA_TRY(launch_fill(0, o.variances_averages, T * o.H, 1.f));  // NN/Neural_Network__Allocate.cpp:2612-2615
+            for (float **s : small) { MYEA_TRY(dev_alloc(s, T * o.NH)); MYEA_HIP_TRY(hipMemset(*s, 0, T * o.NH * sizeof(float))); }
+            MYEA_TRY(launch_fill(0, o.variances_averages, T * o.NH, 1.f));  // NN/Neural_Network__Allocate.cpp:2612-2615
         }
     }
     MYEA_TRY(dev_alloc(&tmp1, T * B * max_h));
@@ -188,7 +242,7 @@ Net::~Net()
     for (int k = 0; k < 4; ++k) fr(opt[k]);
     fr(masks);
     for (DevLayer &o : L) {
-        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.colscale);
+        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale);
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
@@ -206,7 +260,7 @@ int Net::refresh_colscale(size_t li, bool *active)
     DevLayer &o = L[li];
     *active = false;
     if (l.type_dropout == MYEA_DROPOUT_NONE || !o.colscale) return MYEA_OK;
-    const size_t n = (size_t)d.number_recurrent_depth * o.H;
+    const size_t n = (size_t)d.number_recurrent_depth * o.AH;
     if (state == MYEA_STATE_TRAINING) {
         float on = 1.f;
         if (l.type_dropout == MYEA_DROPOUT_BERNOULLI_INVERTED) on = l.dropout_values[0] == 0.f ? 0.f : 1.f / l.dropout_values[0];
@@ -226,8 +280,8 @@ int Net::forward_fc_layer(size_t li, size_t B)
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
-    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, In = L[li - 1].H, H = o.H;
-    const float *x = layer_outputs(li - 1);
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, In = o.In, H = o.H;
+    const float *x = layer_outputs(o.prev);
     const bool norm = layer_uses_norm(l), before = l.use_layer_normalization_before_activation != 0;
     const bool softmax = l.type_activation_function == MYEA_AF_SOFTMAX;
     const bool training = state >= MYEA_STATE_TRAINING;
@@ -273,7 +327,7 @@ int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool train
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
-    const size_t H = o.H, roff = t * d.batch_size;
+    const size_t H = o.NH, roff = t * d.batch_size;
     if (!training) {
         return launch_bn_forward_inference(stream, rows, H, x, scale_ptr(parameters, li), shift_ptr(parameters, li),
                                            o.means_averages + t * H, o.variances_averages + t * H, o.normalizes + roff * H);
@@ -316,9 +370,75 @@ int Net::forward_pass(size_t B, const float *inputs, int on_device)
     }
     for (size_t li = 1; li < d.n_layers; ++li) {
         if (d.layers[li].type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(forward_fc_layer(li, B));
-        else MYEA_TRY(lstm_forward_layer(li, B));
+        else if (d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) {
+            MYEA_TRY(forward_residual_block(li, B));
+            li += d.layers[li].block_depth;  // the walk resumes after the block's last member
+        } else MYEA_TRY(lstm_forward_layer(li, B));
     }
     return MYEA_OK;
+}
+
+// Forward_Pass__Residual (NN/Neural_Network__Forward_Pass__OpenMP.cpp:3861-3997) over pre-activation members
+// (Forward_Pass__Residual__FC, :4039-4433): on the member's INPUT [BN] -> (not the first member: activation -> dropout),
+// then weights and bias; the member's output is its summation.  The activation (+ dropout) of member m+1 is applied by
+// the epilogue of member m's contraction whenever nothing (a normalisation) sits between them.  After the last
+// member: [block-level BN], then the zero-padded identity shortcut (:5158-5240).
+int Net::forward_residual_block(size_t ri, size_t B)
+{
+    const myea_layer_desc &r = d.layers[ri];
+    const size_t last = ri + r.block_depth;
+    const bool training = state >= MYEA_STATE_TRAINING;
+    bool values_ready = false;  // the member's activation values were written by the previous contraction
+    for (size_t m = ri + 1; m <= last; ++m) {
+        const myea_layer_desc &l = d.layers[m];
+        DevLayer &o = L[m];
+        const size_t In = o.In, H = o.H;
+        const float *cur = layer_outputs(o.prev);
+        if (layer_uses_norm(l)) {
+            MYEA_TRY(bn_forward(m, 0, B, cur, training));
+            cur = o.normalizes;
+        }
+        if (o.group == 2) {
+            if (!values_ready) {
+                bool drop = false;
+                MYEA_TRY(refresh_colscale(m, &drop));
+                MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, B, In, cur, o.values, drop ? o.colscale : nullptr));
+            }
+            cur = o.values;
+        }
+        GemmParams g{};
+        g.A = cur; g.lda = (long)In; g.a_k_contiguous = 1;
+        g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 1;
+        g.C = o.summations; g.ldc = (long)H;
+        g.M = (int)B; g.N = (int)H; g.K = (int)In;
+        g.epilogue = EPI_FC_FORWARD;
+        g.bias = layer_uses_bias(l) ? parameters + l.first_bias_connection_index : nullptr;
+        values_ready = false;
+        if (m < last) {
+            const myea_layer_desc &nx = d.layers[m + 1];
+            if (!layer_uses_norm(nx) && gemm_can_fuse_activation((int)nx.type_activation_function)) {
+                bool drop = false;
+                MYEA_TRY(refresh_colscale(m + 1, &drop));
+                g.act = (int)nx.type_activation_function;
+                g.aux_out = L[m + 1].values;
+                g.colscale = drop ? L[m + 1].colscale : nullptr;
+                values_ready = true;
+            }
+        }
+        prof_begin(0);
+        MYEA_TRY(launch_gemm(stream, g));
+        prof_end(2.0 * (double)B * (double)H * (double)In);
+    }
+    DevLayer &o = L[ri];
+    const float *blk = L[last].summations;
+    if (layer_uses_norm(r)) {
+        MYEA_TRY(bn_forward(ri, 0, B, blk, training));
+        blk = o.normalizes;
+    }
+    const float *src = layer_outputs(o.prev);
+    const size_t na = o.In, nb = o.NH;
+    if (na >= nb) return launch_padded_add(stream, B, o.H, src, na, 0, blk, nb, -(long)o.pad, o.values);
+    return launch_padded_add(stream, B, o.H, blk, nb, 0, src, na, -(long)o.pad, o.values);
 }
 
 // ---- Compute__Error -------------------------------------------------------------------------------------------
@@ -357,10 +477,29 @@ int Net::compute_error(size_t B, const float *desired, int on_device)
 // into the dX contraction's epilogue whenever it directly follows it.
 int Net::backward_into_layer(size_t li, size_t B)
 {
-    const size_t gi = li + 1;
-    const myea_layer_desc &l = d.layers[li], &next = d.layers[gi];
-    DevLayer &o = L[li], &on = L[gi];
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, H = o.H;
+    // next_connected_layers (Organize__Next_Layers_Connected, NN/Neural_Network.cpp:59-102): the layer after this one (after
+    // this block, for a residual layer); when that is a residual layer, its shortcut AND its block's first member consume
+    // this layer.  The shortcut's share (Backward_Pass__Residual, NN/Neural_Network__Backward_Pass__OpenMP.cpp:1155-1215:
+    // the residual layer's errors, cropped at the padding offset) joins the contraction as its addend.
+    size_t gi = l.type_layer == MYEA_LAYER_RESIDUAL ? li + l.block_depth + 1 : li + 1;
+    const float *addend = nullptr, *identity = nullptr;
+    const DevLayer *shortcut = nullptr;
+    long ld_addend = 0, crop = 0;
+    bool have_gemm = true;
+    if (d.layers[gi].type_layer == MYEA_LAYER_RESIDUAL) {
+        shortcut = &L[gi];
+        crop = shortcut->H > H ? (long)shortcut->pad : 0;
+        addend = shortcut->neuron_errors + crop;
+        ld_addend = (long)shortcut->H;
+        gi += 1;
+        // a normalised first member hands down its normalisation errors (Backward_Pass__Residual__FC, :454-534)
+        if (layer_uses_norm(d.layers[gi])) { have_gemm = false; identity = L[gi].in_errors; }
+    }
+    const myea_layer_desc &next = d.layers[gi];
+    DevLayer &on = L[gi];
     // what the consumer hands down: delta [T][Bmax][Out] and weights [Out][H]
     const float *delta = on.neuron_errors, *weights = parameters + next.first_connection_index;
     size_t Out = on.H;
@@ -376,16 +515,18 @@ int Net::backward_into_layer(size_t li, size_t B)
         g.B = weights; g.ldb = (long)H; g.b_k_contiguous = 0;
         g.M = (int)rows; g.N = (int)H; g.K = (int)Out;
         g.ldc = (long)H;
-        if (!is_fc) {  // an LSTM layer receives the plain delta of its cell outputs; BPTT follows
+        g.addend = addend; g.ld_addend = ld_addend;
+        if (!is_fc) {  // an LSTM layer receives the plain delta of its cell outputs (BPTT follows), a residual layer that of its units
             g.C = o.neuron_errors + roff * H;
             g.epilogue = EPI_NONE;
+            if (!have_gemm) { MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors, shortcut->H, crop, identity, H, 0, g.C)); continue; }
             prof_begin(1);
             MYEA_TRY(launch_gemm(stream, g));
             prof_end(2.0 * (double)rows * (double)H * (double)Out);
             continue;
         }
         g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
-        const bool fuse = gemm_can_fuse_activation(g.act);
+        const bool fuse = have_gemm && gemm_can_fuse_activation(g.act);
         if (!norm) {
             g.C = (fuse ? o.neuron_errors : tmp1) + roff * H;
             g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.summations + roff * H; g.val = o.values + roff * H;
@@ -396,9 +537,13 @@ int Net::backward_into_layer(size_t li, size_t B)
             g.C = tmp1 + roff * H;
             g.epilogue = EPI_NONE;
         }
-        prof_begin(1);
-        MYEA_TRY(launch_gemm(stream, g));
-        prof_end(2.0 * (double)rows * (double)H * (double)Out);
+        if (have_gemm) {
+            prof_begin(1);
+            MYEA_TRY(launch_gemm(stream, g));
+            prof_end(2.0 * (double)rows * (double)H * (double)Out);
+        } else {
+            MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors, shortcut->H, crop, identity, H, 0, g.C));
+        }
         if (!fuse && !(norm && !before)) {  // act' as its own kernel (Backward_Pass__FC__DF)
             MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, rows * H, g.pre, g.val, tmp1 + roff * H, (norm ? tmp1 : o.neuron_errors) + roff * H));
         }
@@ -413,11 +558,61 @@ int Net::backward_into_layer(size_t li, size_t B)
     return MYEA_OK;
 }
 
+// Backward_Pass__Gradient__Residual (NN/Neural_Network__Backward_Pass__OpenMP.cpp:711-950) with
+// Backward_Pass__Residual__Block (:351-452) and Backward_Pass__Residual__FC (:454-534), members from the last to the first.
+// The last member's delta is the residual layer's errors (cropped to its width), through the block-level BN backward when
+// there is one.  A member reduces its delta to its input side: dX = delta * W, times act' of its input-side activation,
+// through its BN backward; that result IS the delta of the member before it (the reference copies it there), so it is
+// written straight into that member's buffer.  A normalised first member keeps its input-side errors for the shortcut
+// source; an un-normalised one contributes delta * W there directly (backward_into_layer).
+int Net::backward_residual_block(size_t ri, size_t B)
+{
+    const myea_layer_desc &r = d.layers[ri];
+    DevLayer &ro = L[ri];
+    const size_t last = ri + r.block_depth;
+    const long crop = ro.H > ro.NH ? (long)ro.pad : 0;
+    if (layer_uses_norm(r)) {
+        MYEA_TRY(launch_padded_add(stream, B, ro.NH, ro.neuron_errors, ro.H, crop, nullptr, 0, 0, tmp1));
+        MYEA_TRY(bn_backward(ri, 0, B, L[last].summations, tmp1, L[last].neuron_errors));
+    } else {
+        MYEA_TRY(launch_padded_add(stream, B, ro.NH, ro.neuron_errors, ro.H, crop, nullptr, 0, 0, L[last].neuron_errors));
+    }
+    for (size_t m = last; m > ri; --m) {
+        const myea_layer_desc &l = d.layers[m];
+        DevLayer &o = L[m];
+        const bool norm = layer_uses_norm(l);
+        if (o.group == 1 && !norm) break;
+        const size_t In = o.In, H = o.H;
+        float *dst = o.group == 2 ? L[m - 1].neuron_errors : o.in_errors;
+        const float *prev_out = layer_outputs(o.prev);
+        GemmParams g{};
+        g.A = o.neuron_errors; g.lda = (long)H; g.a_k_contiguous = 1;
+        g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 0;
+        g.C = norm ? tmp1 : dst; g.ldc = (long)In;
+        g.M = (int)B; g.N = (int)In; g.K = (int)H;
+        g.epilogue = EPI_NONE;
+        bool derive_pending = false;
+        if (o.group == 2) {
+            g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
+            g.pre = norm ? o.normalizes : prev_out;   // Layer::ptr_array_pre_activation_functions
+            g.val = o.values;
+            if (gemm_can_fuse_activation(g.act)) g.epilogue = EPI_FC_DERIVE;
+            else derive_pending = true;
+        }
+        prof_begin(1);
+        MYEA_TRY(launch_gemm(stream, g));
+        prof_end(2.0 * (double)B * (double)H * (double)In);
+        if (derive_pending) MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, B * In, g.pre, g.val, g.C, g.C));
+        if (norm) MYEA_TRY(bn_backward(m, 0, B, prev_out, tmp1, dst));
+    }
+    return MYEA_OK;
+}
+
 int Net::bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx)
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
-    const size_t H = o.H, roff = t * d.batch_size;
+    const size_t H = o.NH, roff = t * d.batch_size;
     BnBackwardParams p{};
     p.rows = rows; p.H = H; p.x = x; p.hats = o.hats + roff * H; p.dy = dy;
     p.mean = o.means + t * H; p.var = o.variances + t * H; p.scale = scale_ptr(parameters, li); p.r_corr = o.r_corrections + t * H;
@@ -431,10 +626,16 @@ int Net::backward_pass(size_t B)
 {
     if (B == 0 || B > d.batch_size) { set_last_error("Backward_Pass: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
     if (state != MYEA_STATE_TRAINING) { set_last_error("Backward_Pass: can not back propagate gradient in inference mode"); return MYEA_E_STATE; }
-    for (size_t gi = d.n_layers - 1; gi >= 2; --gi) {
-        const size_t li = gi - 1;
+    // the walk of FF__Backward_Pass_Batch: from a consumer gi to its producer li = previous_connected_layers[0]; once a
+    // residual layer's block is done it resumes from the residual layer itself (:117-120)
+    for (size_t gi = d.n_layers - 1; gi != 1; --gi) {
+        const size_t li = L[gi].prev;
         MYEA_TRY(backward_into_layer(li, B));
         if (d.layers[li].type_layer == MYEA_LAYER_LSTM) MYEA_TRY(lstm_backward_layer(li, B));
+        else if (d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) {
+            MYEA_TRY(backward_residual_block(li, B));
+            gi = li + 1;
+        }
     }
     return MYEA_OK;
 }
@@ -450,9 +651,13 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
     for (size_t li = first; li < end; ++li) {
         const myea_layer_desc &l = d.layers[li];
         if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_update_derivative_weight(li, B)); continue; }
+        if (l.type_layer == MYEA_LAYER_RESIDUAL) continue;  // owns no connection (:31-36)
         DevLayer &o = L[li];
-        const size_t In = L[li - 1].H, H = o.H;
-        const float *x = layer_outputs(li - 1);
+        const size_t In = o.In, H = o.H;
+        // Layer::ptr_array_pre_summations: the operand the weights were applied to (NN/Neural_Network__Ordered.cpp:96-141)
+        const float *x = layer_outputs(o.prev);
+        if (o.group == 2) x = o.values;
+        else if (o.group == 1 && layer_uses_norm(l)) x = o.normalizes;
         const bool per_t = T > 1 && B != Bmax;
         const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
         for (size_t c = 0; c < chunks; ++c) {
@@ -683,14 +888,19 @@ int myea_hip_download_tensor(myea_hip_net *n, size_t li, int kind, float *host, 
     NET_OR_FAIL(n);
     if (!host || li >= n->net.d.n_layers) { myea::set_last_error("download_tensor: null or layer %zu out of range", li); return MYEA_E_INVALID; }
     myea::DevLayer &o = n->net.L[li];
-    const size_t T = n->net.d.number_recurrent_depth, full = T * n->net.d.batch_size * o.H, th = T * o.H;
+    const size_t T = n->net.d.number_recurrent_depth, full = T * n->net.d.batch_size * o.H, th = T * o.NH;
     const float *p = nullptr;
     size_t c = full;
     switch (kind) {
     case MYEA_TENSOR_OUTPUTS: p = n->net.layer_outputs(li); break;
     case MYEA_TENSOR_SUMMATIONS: p = o.summations; break;
     case MYEA_TENSOR_ERRORS: p = o.neuron_errors; break;
-    case MYEA_TENSOR_NORM_HATS: p = o.hats; break;
+    case MYEA_TENSOR_NORM_HATS: p = o.hats; c = T * n->net.d.batch_size * o.NH; break;
+    case MYEA_TENSOR_INPUT_SIDE_ERRORS:
+        if (o.group == 2) p = n->net.L[li - 1].neuron_errors;
+        else if (o.group == 1) p = o.in_errors;
+        c = T * n->net.d.batch_size * o.In;
+        break;
     case MYEA_TENSOR_NORM_MEANS: p = o.means; c = th; break;
     case MYEA_TENSOR_NORM_VARIANCES: p = o.variances; c = th; break;
     case MYEA_TENSOR_NORM_MEANS_AVERAGES: p = o.means_averages; c = th; break;

@@ -43,10 +43,18 @@ typedef struct olstm {
 typedef struct olayer {
     size_t H;            /* *ptr_number_outputs */
     size_t norm_units;   /* number of Normalized_unit owned by the layer */
-    /* [T][Bmax][H] */
+    /* topology (Organize__Previous_Layers_Connected / Organize__Layer__Group, NN/Neural_Network.cpp:20-125) */
+    size_t prev;         /* previous_connected_layers[0] */
+    int group;           /* 0 outside a residual block, 1 first layer of a block, 2 other layers of a block */
+    size_t In;           /* *previous_connected_layers[0]->ptr_number_outputs */
+    size_t AH, NH;       /* width of the AF-unit tensors (values, af_errors) and of the normalised-unit tensors:
+                            H outside a block; inside a block they sit on the input side and are In wide; a residual
+                            layer has basic units (H wide, kept in values / af_errors) and NH = the block's last width */
+    size_t pad;          /* residual layer: pooling_values[2], the zero-padding offset of the narrower operand */
+    /* [T][Bmax][H] (summations, neuron_errors), [T][Bmax][AH] (values, af_errors), [T][Bmax][NH] (hats, normalizes, norm_errors) */
     float *summations, *values, *hats, *normalizes;
     float *neuron_errors, *af_errors, *norm_errors;
-    /* [T][H] */
+    /* [T][NH] */
     float *means, *variances, *means_averages, *variances_averages, *r_corrections, *d_corrections;
     float *derivatives_means, *derivatives_variances;
     /* LSTM, [T][Bmax][C] or [T][Bmax][K] per direction d (index d*...) */
@@ -168,10 +176,11 @@ static float *layer_outputs(myea_oracle_net *n, size_t li)
     olayer *o = &n->L[li];
     if (li == 0) return o->values;
     if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (o->group) return o->summations; /* residual group: NN/Neural_Network__Ordered.cpp:96-141 */
         if (layer_uses_norm(l) && !l->use_layer_normalization_before_activation) return o->normalizes;
         return o->values;
     }
-    return o->values; /* LSTM: cell outputs live in values */
+    return o->values; /* LSTM: cell outputs live in values; residual layer: basic units' values (:360-366) */
 }
 
 /* Layer::ptr_array_derivative_outputs */
@@ -180,10 +189,11 @@ static float *layer_derivative_outputs(myea_oracle_net *n, size_t li)
     const myea_layer_desc *l = &n->d.layers[li];
     olayer *o = &n->L[li];
     if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (o->group) return o->neuron_errors;
         if (layer_uses_norm(l) && !l->use_layer_normalization_before_activation) return o->norm_errors;
         return o->af_errors;
     }
-    return o->af_errors; /* LSTM: ptr_delta_cell_output */
+    return o->af_errors; /* LSTM: ptr_delta_cell_output; residual layer: basic units' errors */
 }
 
 static float *scale_ptr(myea_oracle_net *n, float *base, size_t li)
@@ -220,14 +230,49 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
     memset(n->masks, 1, desc->total_mask_units ? desc->total_mask_units : 1); /* NN/Neural_Network__Allocate.cpp:386-410: all true */
     /* scales start at 1, shifts at 0 (NN/Neural_Network__Allocate.cpp:2395-2401 and the scale fill) */
     for (size_t i = 0; i < desc->total_normalized_units; ++i) n->parameters[desc->total_weights + desc->total_bias + i] = 1.f;
+    /* connections, walked with the same running state as Order__Layers__Connection (NN/Neural_Network__Ordered.cpp:20-68):
+     * `block` is the residual layer whose members are being visited, `seen` how many of them have been */
+    {
+        size_t block = 0, seen = 0;
+        for (size_t li = 0; li < desc->n_layers; ++li) {
+            const myea_layer_desc *l = &desc->layers[li];
+            olayer *o = &n->L[li];
+            o->group = 0;
+            if (li == 0) { o->prev = 0; o->H = l->n_units; if (l->type_layer == MYEA_LAYER_RESIDUAL) { free(n); return MYEA_E_INVALID; } continue; }
+            if (block != 0 && seen == desc->layers[block].block_depth) { o->prev = block; block = 0; seen = 0; } /* first layer after the block */
+            else {
+                o->prev = li - 1;
+                if (desc->layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) o->prev = n->L[li - 1].prev;
+                if (block != 0) { o->group = seen == 0 ? 1 : 2; ++seen; }
+            }
+            if (l->type_layer == MYEA_LAYER_RESIDUAL) {
+                if (block != 0 || T != 1 || l->block_depth == 0 || li + l->block_depth + 1 >= desc->n_layers || l->type_dropout != MYEA_DROPOUT_NONE) { free(n); return MYEA_E_UNSUPPORTED; }
+                block = li; seen = 0;
+            }
+        }
+        /* widths: a residual layer is as wide as the wider of its shortcut source and its block's last layer
+         * (Assign__Post__Layer, NN/Neural_Network__Compile.cpp:272-281); its members' widths are known up front */
+        for (size_t li = 0; li < desc->n_layers; ++li) {
+            const myea_layer_desc *l = &desc->layers[li];
+            olayer *o = &n->L[li];
+            if (l->type_layer == MYEA_LAYER_RESIDUAL) {
+                size_t a = n->L[o->prev].H, b = layer_width(&desc->layers[li + l->block_depth]);
+                o->H = a > b ? a : b;
+                o->pad = ((a > b ? a - b : b - a) + 1) / 2;
+                o->NH = b;
+            } else o->H = layer_width(l);
+            o->In = li ? n->L[o->prev].H : 0;
+            if (l->type_layer != MYEA_LAYER_RESIDUAL) { o->AH = o->group ? (o->group == 1 ? 0 : o->In) : o->H; o->NH = o->group ? o->In : o->H; }
+            else o->AH = o->H;
+        }
+    }
     for (size_t li = 0; li < desc->n_layers; ++li) {
         const myea_layer_desc *l = &desc->layers[li];
         olayer *o = &n->L[li];
-        o->H = layer_width(l);
-        if (l->type_layer == MYEA_LAYER_RESIDUAL) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED) { free(n); return MYEA_E_UNSUPPORTED; }
         if (l->type_layer == MYEA_LAYER_LSTM && (l->use_bidirectional || layer_uses_norm(l) || l->type_dropout != MYEA_DROPOUT_NONE)) { free(n); return MYEA_E_UNSUPPORTED; }
         size_t sz = T * B * o->H;
-        o->values = zalloc(sz);
+        o->values = zalloc(T * B * o->AH);
         if (li == 0) continue;
         if (l->type_layer == MYEA_LAYER_LSTM) {
             /* the bias vectors are read at first_bias_connection_index + [0, C + 3K): with the index as the reference
@@ -235,7 +280,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
              * reads and writes outside its parameter array, which nothing here reproduces */
             if (l->first_bias_connection_index + (size_t)l->n_units * l->n_cells_per_block + 3u * l->n_units > desc->total_weights + desc->total_bias) { free(n); return MYEA_E_INVALID; }
             olstm *q = (olstm *)calloc(1, sizeof(olstm));
-            q->K = l->n_units; q->cpb = l->n_cells_per_block; q->C = q->K * q->cpb; q->In = n->L[li - 1].H;
+            q->K = l->n_units; q->cpb = l->n_cells_per_block; q->C = q->K * q->cpb; q->In = o->In;
             q->per_block = q->cpb * (q->In + q->C) + 3 * q->In + 3 * q->C + 3 * q->cpb;
             size_t sc = T * B * q->C, sk = T * B * q->K;
             float **cells[] = {&q->sum_in_z, &q->sum_rec_z, &q->sum_z, &q->z, &q->c, &q->ca, &q->dz, &q->dc};
@@ -247,22 +292,25 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
             o->af_errors = zalloc(sz);  /* ptr_delta_cell_output */
             continue;
         }
-        o->summations = zalloc(sz);
-        o->neuron_errors = zalloc(sz);
-        o->af_errors = zalloc(sz);
+        o->af_errors = zalloc(T * B * o->AH);
+        if (l->type_layer != MYEA_LAYER_RESIDUAL) {
+            o->summations = zalloc(sz);
+            o->neuron_errors = zalloc(sz);
+        }
         if (layer_uses_norm(l)) {
-            o->hats = zalloc(sz);
-            o->normalizes = zalloc(sz);
-            o->norm_errors = zalloc(sz);
-            o->means = zalloc(T * o->H);
-            o->variances = zalloc(T * o->H);
-            o->means_averages = zalloc(T * o->H);
-            o->variances_averages = zalloc(T * o->H);
-            for (size_t i = 0; i < T * o->H; ++i) o->variances_averages[i] = 1.f; /* NN/Neural_Network__Allocate.cpp:2612-2615 */
-            o->r_corrections = zalloc(T * o->H);
-            o->d_corrections = zalloc(T * o->H);
-            o->derivatives_means = zalloc(T * o->H);
-            o->derivatives_variances = zalloc(T * o->H);
+            size_t sn = T * B * o->NH, tn = T * o->NH;
+            o->hats = zalloc(sn);
+            o->normalizes = zalloc(sn);
+            o->norm_errors = zalloc(sn);
+            o->means = zalloc(tn);
+            o->variances = zalloc(tn);
+            o->means_averages = zalloc(tn);
+            o->variances_averages = zalloc(tn);
+            for (size_t i = 0; i < tn; ++i) o->variances_averages[i] = 1.f; /* NN/Neural_Network__Allocate.cpp:2612-2615 */
+            o->r_corrections = zalloc(tn);
+            o->d_corrections = zalloc(tn);
+            o->derivatives_means = zalloc(tn);
+            o->derivatives_variances = zalloc(tn);
         }
     }
     *out = n;
@@ -439,8 +487,8 @@ static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
 {
     const myea_layer_desc *l = &n->d.layers[li];
     olayer *o = &n->L[li];
-    size_t In = n->L[li - 1].H, H = o->H;
-    const float *x = layer_outputs(n, li - 1);
+    size_t In = o->In, H = o->H;
+    const float *x = layer_outputs(n, o->prev);
     int training = n->state >= MYEA_STATE_TRAINING;
     int renorm = l->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
     fwd_fc(n, t, B, In, H, x, n->parameters + l->first_connection_index, o->summations);
@@ -461,6 +509,65 @@ static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
     fwd_dropout(n, l, t, B, H, out);
 }
 
+/* Forward_Pass__Residual__FC: NN/Neural_Network__Forward_Pass__OpenMP.cpp:4039-4433.  Pre-activation order on the
+ * layer's INPUT (fan-in wide): [BN] -> (not for the block's first layer: activation -> dropout) -> weights -> bias.
+ * The layer's output is its summation. */
+static void fwd_residual_fc_layer(myea_oracle_net *n, size_t li, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    size_t In = o->In, H = o->H;
+    const float *cur = layer_outputs(n, o->prev);
+    int training = n->state >= MYEA_STATE_TRAINING;
+    int renorm = l->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    if (layer_uses_norm(l)) {
+        if (training) fwd_bn_training(n, renorm, 0, B, In, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
+        else fwd_bn_inference(n, 0, B, In, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
+        cur = o->normalizes;
+    }
+    if (o->group == 2) {
+        fwd_af(n, 0, B, In, l->type_activation_function, cur, o->values);
+        fwd_dropout(n, l, 0, B, In, o->values);
+        cur = o->values;
+    }
+    fwd_fc(n, 0, B, In, H, cur, n->parameters + l->first_connection_index, o->summations);
+    if (layer_uses_bias(l)) fwd_bias(n, 0, B, H, n->parameters + l->first_bias_connection_index, o->summations);
+}
+
+/* Forward_Pass__Residual: :3861-3997 (block members, then [block-level BN] on the last member's output, then the
+ * shortcut); Forward_Pass__Zero_Padded_Identity: :5158-5240 (A = shortcut source, B = block output; the narrower one is
+ * added into the wider one at offset `padding`). */
+static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t B)
+{
+    const myea_layer_desc *r = &n->d.layers[ri];
+    olayer *o = &n->L[ri];
+    size_t last = ri + r->block_depth, Bmax = n->d.batch_size; (void)Bmax;
+    for (size_t li = ri + 1; li <= last; ++li) fwd_residual_fc_layer(n, li, B);
+    const float *blk = layer_outputs(n, last);
+    size_t nb = n->L[last].H, na = n->L[o->prev].H;
+    if (layer_uses_norm(r)) {
+        int renorm = r->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+        if (n->state >= MYEA_STATE_TRAINING) fwd_bn_training(n, renorm, 0, B, nb, blk, scale_ptr(n, n->parameters, ri), shift_ptr(n, n->parameters, ri), o);
+        else fwd_bn_inference(n, 0, B, nb, blk, scale_ptr(n, n->parameters, ri), shift_ptr(n, n->parameters, ri), o);
+        blk = o->normalizes;
+    }
+    const float *a = layer_outputs(n, o->prev);
+    for (size_t b = 0; b < B; ++b) {
+        const float *ar = a + b * na, *br = blk + b * nb;
+        if (o->pad == 0) {
+            float *y = o->values + b * na;
+            for (size_t j = 0; j < na; ++j) y[j] = ar[j] + br[j];
+        } else if (na > nb) {
+            float *y = o->values + b * na;
+            for (size_t j = 0; j < na; ++j) y[j] = ar[j];
+            for (size_t j = 0; j < nb; ++j) y[j + o->pad] += br[j];
+        } else {
+            float *y = o->values + b * nb;
+            for (size_t j = 0; j < nb; ++j) y[j] = br[j];
+            for (size_t j = 0; j < na; ++j) y[j + o->pad] += ar[j];
+        }
+    }
+}
 
 /* ------------------------------------------------------------------------------------------- */
 /* LSTM with peepholes (one direction, time ascending) */
@@ -488,7 +595,7 @@ static void fwd_lstm_step(myea_oracle_net *n, size_t li, size_t t, size_t B)
     olayer *o = &n->L[li];
     olstm *q = o->lstm;
     size_t Bmax = n->d.batch_size, K = q->K, C = q->C, cpb = q->cpb, In = q->In;
-    const float *x = layer_outputs(n, li - 1), *w = n->parameters;
+    const float *x = layer_outputs(n, n->L[li].prev), *w = n->parameters;
     const float *bz = w + l->first_bias_connection_index, *bi = bz + C, *bf = bi + K, *bo = bf + K;
     int first = t == 0;
     long b;
@@ -657,7 +764,7 @@ static void dw_lstm(myea_oracle_net *n, size_t li, size_t B)
     olayer *o = &n->L[li];
     olstm *q = o->lstm;
     size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, K = q->K, C = q->C, cpb = q->cpb, In = q->In;
-    const float *x = layer_outputs(n, li - 1);
+    const float *x = layer_outputs(n, n->L[li].prev);
     float *g = n->gradient;
     long kk;
     /* parallel over blocks: every parameter belongs to one block, so the per-parameter summation order (b, then t)
@@ -724,6 +831,9 @@ int myea_oracle_forward_pass(myea_oracle_net *n, size_t B, const float *inputs)
             for (size_t t = 0; t < T; ++t) fwd_fc_layer(n, li, t, B);
         } else if (l->type_layer == MYEA_LAYER_LSTM) {
             for (size_t t = 0; t < T; ++t) fwd_lstm_step(n, li, t, B);
+        } else if (l->type_layer == MYEA_LAYER_RESIDUAL) {
+            fwd_residual_block(n, li, B);
+            li += l->block_depth; /* the iterator is left on the block's last member, :3884-3885 */
         } else return MYEA_E_UNSUPPORTED;
     }
     return MYEA_OK;
@@ -915,31 +1025,133 @@ static void bwd_gradient_fc(myea_oracle_net *n, size_t li, size_t t, size_t B)
     memcpy(o->neuron_errors + Bmax * H * t, cur + Bmax * H * t, Bmax * H * sizeof(float));
 }
 
+/* Backward_Pass__Residual (7-arg): NN/Neural_Network__Backward_Pass__OpenMP.cpp:1155-1215.  Shortcut gradient:
+ * dst (width D) += the residual layer's errors (width R >= D), cropped at `pad` when R > D. */
+static void bwd_residual_shortcut(myea_oracle_net *n, size_t B, size_t R, size_t D, size_t pad, const float *err, float *dst)
+{
+    (void)n;
+    for (size_t b = 0; b < B; ++b) {
+        const float *e = err + b * R;
+        float *d = dst + b * D;
+        if (R == D) for (size_t j = 0; j < R; ++j) d[j] += e[j];
+        else if (R > D) for (size_t j = 0; j < D; ++j) d[j] += e[j + pad];
+        else for (size_t j = 0; j < R; ++j) d[j + pad] += e[j];
+    }
+}
+
+/* Backward_Pass__Residual__FC: :454-534 - what a block member hands to its producer.  A member that is not the block's
+ * first layer has already reduced its delta to its input side (Backward_Pass__Gradient__Residual__FC), so the producer
+ * receives a COPY of those errors; the block's first layer ADDS (its producer also receives the shortcut): its
+ * normalisation errors when it is normalised, delta * W otherwise. */
+static void bwd_residual_fc_to_previous(myea_oracle_net *n, size_t gi, size_t B, float *dst)
+{
+    const myea_layer_desc *g = &n->d.layers[gi];
+    olayer *q = &n->L[gi];
+    size_t Bmax = n->d.batch_size, D = q->In;
+    if (q->group == 2) memcpy(dst, layer_uses_norm(g) ? q->norm_errors : q->af_errors, Bmax * D * sizeof(float));
+    else if (layer_uses_norm(g)) {
+        for (size_t b = 0; b < B; ++b)
+            for (size_t j = 0; j < D; ++j) dst[b * D + j] += q->norm_errors[b * D + j]; /* Backward_Pass__Identity, :1084-1108 */
+    } else bwd_fc(n, 0, B, q->H, D, q->neuron_errors, n->parameters + g->first_connection_index, dst);
+}
+
+/* Backward_Pass__Gradient__Residual__FC: :822-950 - delta of the summation -> input side: dX = delta * W into the
+ * activation errors (block's first layer: into the normalisation errors, or nothing when it is not normalised),
+ * then act' on the input-side activation, then [BN backward] over the fan-in wide normalised units. */
+static void bwd_gradient_residual_fc(myea_oracle_net *n, size_t li, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    size_t In = o->In, Bmax = n->d.batch_size;
+    int renorm = l->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    float *din;
+    if (o->group == 2) din = o->af_errors;
+    else if (layer_uses_norm(l)) din = o->norm_errors;
+    else return;
+    memset(din, 0, Bmax * In * sizeof(float));
+    bwd_fc(n, 0, B, o->H, In, o->neuron_errors, n->parameters + l->first_connection_index, din);
+    const float *prev_out = layer_outputs(n, o->prev);
+    if (o->group == 2) {
+        const float *pre_af = layer_uses_norm(l) ? o->normalizes : prev_out; /* ptr_array_pre_activation_functions */
+        bwd_df(n, 0, B, In, l->type_activation_function, l->activation_steepness, pre_af, o->values, din, o->af_errors);
+    }
+    if (layer_uses_norm(l)) bwd_bn(n, renorm, li, 0, B, In, prev_out /* ptr_array_pre_normalization */, din, o->norm_errors);
+}
+
+/* Backward_Pass__Residual__Block: :351-452 - the residual layer's errors reach the block's last member through the
+ * (cropped) shortcut add, then [block-level BN backward], copied into the member's delta. */
+static void bwd_residual_block_to_last(myea_oracle_net *n, size_t ri, size_t B, float *dst)
+{
+    const myea_layer_desc *r = &n->d.layers[ri];
+    olayer *o = &n->L[ri];
+    size_t D = o->NH, Bmax = n->d.batch_size;
+    float *tmp = dst;
+    if (layer_uses_norm(r)) { tmp = o->norm_errors; memset(tmp, 0, Bmax * D * sizeof(float)); }
+    bwd_residual_shortcut(n, B, o->H, D, o->pad, o->af_errors, tmp);
+    if (layer_uses_norm(r)) {
+        int renorm = r->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+        bwd_bn(n, renorm, ri, 0, B, D, layer_outputs(n, ri + r->block_depth), tmp, o->norm_errors);
+        memcpy(dst, o->norm_errors, Bmax * D * sizeof(float));
+    }
+}
+
+/* Backward_Pass__Gradient__Residual: :711-729 with Backward_Pass__Gradient__Residual__Layer :731-820 - members from the
+ * last to the first: zero the member's delta, pull it from its consumer, reduce it to the input side. */
+static void bwd_gradient_residual(myea_oracle_net *n, size_t ri, size_t B)
+{
+    const myea_layer_desc *r = &n->d.layers[ri];
+    size_t Bmax = n->d.batch_size, last = ri + r->block_depth;
+    for (size_t li = last; li > ri; --li) {
+        olayer *o = &n->L[li];
+        memset(o->neuron_errors, 0, Bmax * o->H * sizeof(float));
+        if (li == last) bwd_residual_block_to_last(n, ri, B, o->neuron_errors);
+        else bwd_residual_fc_to_previous(n, li + 1, B, o->neuron_errors);
+        bwd_gradient_residual_fc(n, li, B);
+    }
+}
+
 /* FF__Backward_Pass_Batch: NN/Neural_Network__Backward_Pass__OpenMP.cpp:24-155.
  * RNN__Backward_Pass_Batch: NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:24-181 (FC
- * consumers iterate t descending).  The input layer's delta is never computed. */
+ * consumers iterate t descending).  The input layer's delta is never computed.  The walk goes from consumer
+ * `gi` to its producer `li = previous_connected_layers[0]`; a producer collects from every consumer in
+ * next_connected_layers (a layer in front of a residual block feeds the shortcut AND the block's first member);
+ * after a residual layer's block has been processed the walk resumes from the residual layer itself (:117-120). */
 int myea_oracle_backward_pass(myea_oracle_net *n, size_t B)
 {
     if (!n) return MYEA_E_INVALID;
     if (B > n->d.batch_size) return MYEA_E_BATCH;
     if (n->state != MYEA_STATE_TRAINING) return MYEA_E_STATE;
     size_t T = n->d.number_recurrent_depth, Bmax = n->d.batch_size;
-    for (size_t gi = n->d.n_layers - 1; gi >= 2; --gi) {
-        size_t li = gi - 1; /* previous_connected_layers[0] */
-        const myea_layer_desc *next = &n->d.layers[gi];
+    for (size_t gi = n->d.n_layers - 1; gi != 1; --gi) {
+        size_t li = n->L[gi].prev;
+        const myea_layer_desc *cur = &n->d.layers[li];
         olayer *o = &n->L[li];
         float *dst = layer_derivative_outputs(n, li);
         memset(dst, 0, T * Bmax * o->H * sizeof(float));
-        if (next->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
-            for (size_t tt = T; tt-- > 0;)
-                bwd_fc(n, tt, B, n->L[gi].H, o->H, n->L[gi].neuron_errors, n->parameters + next->first_connection_index, dst);
-        } else if (next->type_layer == MYEA_LAYER_LSTM) {
-            for (size_t tt = 0; tt < T; ++tt) bwd_lstm_to_previous(n, gi, tt, B, dst);
-        } else return MYEA_E_UNSUPPORTED;
-        if (n->d.layers[li].type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        /* next_connected_layers (Organize__Next_Layers_Connected, NN/Neural_Network.cpp:59-102) */
+        size_t consumers[2], nc = 0;
+        consumers[nc++] = cur->type_layer == MYEA_LAYER_RESIDUAL ? li + cur->block_depth + 1 : li + 1;
+        if (n->d.layers[consumers[0]].type_layer == MYEA_LAYER_RESIDUAL) consumers[nc++] = consumers[0] + 1;
+        for (size_t c = 0; c < nc; ++c) {
+            size_t ci = consumers[c];
+            const myea_layer_desc *next = &n->d.layers[ci];
+            if (next->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+                if (n->L[ci].group) bwd_residual_fc_to_previous(n, ci, B, dst);
+                else for (size_t tt = T; tt-- > 0;)
+                    bwd_fc(n, tt, B, n->L[ci].H, o->H, n->L[ci].neuron_errors, n->parameters + next->first_connection_index, dst);
+            } else if (next->type_layer == MYEA_LAYER_LSTM) {
+                for (size_t tt = 0; tt < T; ++tt) bwd_lstm_to_previous(n, ci, tt, B, dst);
+            } else if (next->type_layer == MYEA_LAYER_RESIDUAL) {
+                bwd_residual_shortcut(n, B, n->L[ci].H, o->H, n->L[ci].pad, n->L[ci].af_errors, dst);
+            } else return MYEA_E_UNSUPPORTED;
+        }
+        if (cur->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             for (size_t tt = T; tt-- > 0;) bwd_gradient_fc(n, li, tt, B);
-        } else if (n->d.layers[li].type_layer == MYEA_LAYER_LSTM) {
+        } else if (cur->type_layer == MYEA_LAYER_LSTM) {
             for (size_t tt = T; tt-- > 0;) bwd_lstm_step(n, li, tt, B);
+        } else if (cur->type_layer == MYEA_LAYER_RESIDUAL) {
+            bwd_gradient_residual(n, li, B);
+            gi = li + 1;
         } else return MYEA_E_UNSUPPORTED;
     }
     return MYEA_OK;
@@ -988,9 +1200,14 @@ int myea_oracle_update_derivative_weight(myea_oracle_net *n, size_t B, size_t fi
         if (l->type_layer == MYEA_LAYER_LSTM) { dw_lstm(n, li, B); continue; }
         if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_UNSUPPORTED;
         olayer *o = &n->L[li];
-        const float *x = layer_outputs(n, li - 1);
+        /* Layer::ptr_array_pre_summations (NN/Neural_Network__Ordered.cpp:96-141): inside a residual block the operand
+         * the weights were applied to - the layer's own activation values, or for the block's first layer its normalised
+         * input / the shortcut source's output */
+        const float *x = layer_outputs(n, o->prev);
+        if (o->group == 2) x = o->values;
+        else if (o->group == 1 && layer_uses_norm(l)) x = o->normalizes;
         for (size_t t = 0; t < T; ++t) {
-            dw_fc(n, t, B, n->L[li - 1].H, o->H, x, o->neuron_errors, n->gradient + l->first_connection_index);
+            dw_fc(n, t, B, o->In, o->H, x, o->neuron_errors, n->gradient + l->first_connection_index);
             if (layer_uses_bias(l)) dw_bias(n, t, B, o->H, o->neuron_errors, n->gradient + l->first_bias_connection_index);
         }
     }
@@ -1089,13 +1306,18 @@ const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t 
 {
     if (!n || li >= n->d.n_layers) return NULL;
     olayer *o = &n->L[li];
-    size_t T = n->d.number_recurrent_depth, full = T * n->d.batch_size * o->H, th = T * o->H;
+    size_t T = n->d.number_recurrent_depth, full = T * n->d.batch_size * o->H, th = T * o->NH;
     const float *p = NULL; size_t c = full;
     switch (kind) {
     case MYEA_TENSOR_OUTPUTS: p = layer_outputs(n, li); break;
     case MYEA_TENSOR_SUMMATIONS: p = o->summations; break;
-    case MYEA_TENSOR_ERRORS: p = o->neuron_errors; break;
-    case MYEA_TENSOR_NORM_HATS: p = o->hats; break;
+    case MYEA_TENSOR_ERRORS: p = n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL ? o->af_errors : o->neuron_errors; break;
+    case MYEA_TENSOR_NORM_HATS: p = o->hats; c = T * n->d.batch_size * o->NH; break;
+    case MYEA_TENSOR_INPUT_SIDE_ERRORS:
+        if (o->group == 2) p = layer_uses_norm(&n->d.layers[li]) ? o->norm_errors : o->af_errors;
+        else if (o->group == 1 && layer_uses_norm(&n->d.layers[li])) p = o->norm_errors;
+        c = T * n->d.batch_size * o->In;
+        break;
     case MYEA_TENSOR_NORM_MEANS: p = o->means; c = th; break;
     case MYEA_TENSOR_NORM_VARIANCES: p = o->variances; c = th; break;
     case MYEA_TENSOR_NORM_MEANS_AVERAGES: p = o->means_averages; c = th; break;

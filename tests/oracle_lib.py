@@ -20,6 +20,10 @@ def load_oracle():
     lib = C.CDLL(ORACLE_PATH)
     P, sz, vp, i32 = C.POINTER, C.c_size_t, C.c_void_p, C.c_int
     lib.myea_oracle_create.argtypes = [P(mb.NetDesc), P(vp)]
+    lib.myea_net_desc_previous_layer.argtypes = [P(mb.NetDesc), C.c_uint32]
+    lib.myea_net_desc_previous_layer.restype = C.c_uint32
+    lib.myea_net_desc_number_outputs.argtypes = [P(mb.NetDesc), C.c_uint32]
+    lib.myea_net_desc_number_outputs.restype = C.c_uint64
     lib.myea_oracle_destroy.argtypes = [vp]
     lib.myea_oracle_set_hyper.argtypes = [vp, P(mb.Hyper)]
     lib.myea_oracle_get_hyper.argtypes = [vp, P(mb.Hyper)]
