@@ -211,7 +211,9 @@ enum {
     MYEA_TENSOR_LSTM_DELTA_CELL_STATE = 22,
     MYEA_TENSOR_LSTM_DELTA_INPUT_GATE = 23,
     MYEA_TENSOR_LSTM_DELTA_FORGET_GATE = 24,
-    MYEA_TENSOR_LSTM_DELTA_OUTPUT_GATE = 25
+    MYEA_TENSOR_LSTM_DELTA_OUTPUT_GATE = 25,
+    MYEA_TENSOR_LSTM_CELL_OUTPUT = 26,     /* h of one direction (OUTPUTS is the layer's output: the sum of both) */
+    MYEA_TENSOR_DIRECTION_BACKWARD = 0x100 /* OR-ed onto an LSTM kind: the time-reversed direction of a bidirectional layer */
 };
 
 /* ---- host-side descriptor helpers (no GPU needed) ---- */

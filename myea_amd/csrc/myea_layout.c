@@ -138,7 +138,12 @@ int myea_net_desc_layout(myea_net_desc *d)
         } else {
             uint64_t dirs = l->use_bidirectional ? 2u : 1u;
             uint64_t cells = (uint64_t)l->n_units * l->n_cells_per_block * dirs, blocks = (uint64_t)l->n_units * dirs;
-            l->first_bias_connection_index = total_weights + total_bias + cells;
+            /* one direction: the field as the reference leaves it.  Two directions: the reference splits
+             * [first, last) in halves before either is assigned (Allocate__Bidirectional__Layers runs ahead of
+             * Prepare__Bias__LSTM, NN/Neural_Network__Compile.cpp:542 vs :665) and overlays the directions' buffers, so
+             * there is no working behaviour to follow; here direction d owns the contiguous [z | i | f | o] vectors at
+             * first_bias_connection_index + d * (cells + 3 * blocks) per direction, starting at the slice's start. */
+            l->first_bias_connection_index = total_weights + total_bias + (l->use_bidirectional ? 0u : cells);
             total_bias += cells + 3u * blocks;
         }
     }

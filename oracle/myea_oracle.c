@@ -33,8 +33,11 @@
 /* LSTM-with-peephole layer state, one direction.  Cell tensors are [T][Bmax][C], block tensors [T][Bmax][K]
  * (NNH/Data.hpp:2985-3016: ptr_array_cells_* / ptr_array_blocks_*). */
 typedef struct olstm {
-    size_t K, cpb, C, In;   /* blocks, cells per block, cells, fan-in */
+    size_t K, cpb, C, In;   /* blocks, cells per block, cells, fan-in (per direction) */
     size_t per_block;       /* parameters of one block */
+    size_t base, bias;      /* flat index of the direction's first block and of its bias vectors z | i | f | o */
+    int reverse;            /* the direction walks time from T-1 down to 0 */
+    float *h, *dh;          /* cell outputs and their delta [T][Bmax][C]: the layer's own buffers for a one-direction layer */
     float *sum_in_z, *sum_rec_z, *sum_z, *z, *c, *ca;          /* cells */
     float *sum_in_i, *sum_in_f, *sum_in_o, *sum_rec_i, *sum_rec_f, *sum_rec_o, *sum_i, *sum_f, *sum_o, *gi, *gf, *go; /* blocks */
     float *dz, *dc, *di, *df, *dgo;                              /* deltas */
@@ -270,7 +273,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
         const myea_layer_desc *l = &desc->layers[li];
         olayer *o = &n->L[li];
         if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED) { free(n); return MYEA_E_UNSUPPORTED; }
-        if (l->type_layer == MYEA_LAYER_LSTM && (l->use_bidirectional || layer_uses_norm(l) || l->type_dropout != MYEA_DROPOUT_NONE)) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (l->type_layer == MYEA_LAYER_LSTM && (layer_uses_norm(l) || l->type_dropout != MYEA_DROPOUT_NONE)) { free(n); return MYEA_E_UNSUPPORTED; }
         size_t sz = T * B * o->H;
         o->values = zalloc(T * B * o->AH);
         if (li == 0) continue;
@@ -278,18 +281,27 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
             /* the bias vectors are read at first_bias_connection_index + [0, C + 3K): with the index as the reference
              * leaves it they run C entries past the layer's own slice; past the end of the bias region the reference
              * reads and writes outside its parameter array, which nothing here reproduces */
-            if (l->first_bias_connection_index + (size_t)l->n_units * l->n_cells_per_block + 3u * l->n_units > desc->total_weights + desc->total_bias) { free(n); return MYEA_E_INVALID; }
-            olstm *q = (olstm *)calloc(1, sizeof(olstm));
-            q->K = l->n_units; q->cpb = l->n_cells_per_block; q->C = q->K * q->cpb; q->In = o->In;
-            q->per_block = q->cpb * (q->In + q->C) + 3 * q->In + 3 * q->C + 3 * q->cpb;
-            size_t sc = T * B * q->C, sk = T * B * q->K;
-            float **cells[] = {&q->sum_in_z, &q->sum_rec_z, &q->sum_z, &q->z, &q->c, &q->ca, &q->dz, &q->dc};
-            float **blocks[] = {&q->sum_in_i, &q->sum_in_f, &q->sum_in_o, &q->sum_rec_i, &q->sum_rec_f, &q->sum_rec_o, &q->sum_i, &q->sum_f, &q->sum_o,
-                                &q->gi, &q->gf, &q->go, &q->di, &q->df, &q->dgo};
-            for (size_t a = 0; a < sizeof(cells) / sizeof(cells[0]); ++a) *cells[a] = zalloc(sc);
-            for (size_t a = 0; a < sizeof(blocks) / sizeof(blocks[0]); ++a) *blocks[a] = zalloc(sk);
-            o->lstm = q;
+            if (l->first_bias_connection_index + (l->use_bidirectional ? 2u : 1u) * ((size_t)l->n_units * l->n_cells_per_block + 3u * l->n_units) > desc->total_weights + desc->total_bias) { free(n); return MYEA_E_INVALID; }
+            size_t dirs = l->use_bidirectional ? 2 : 1;
+            olstm *qq = (olstm *)calloc(2, sizeof(olstm));
             o->af_errors = zalloc(sz);  /* ptr_delta_cell_output */
+            for (size_t dir = 0; dir < dirs; ++dir) {
+                olstm *q = &qq[dir];
+                q->K = l->n_units; q->cpb = l->n_cells_per_block; q->C = q->K * q->cpb; q->In = o->In;
+                q->per_block = q->cpb * (q->In + q->C) + 3 * q->In + 3 * q->C + 3 * q->cpb;
+                q->base = l->first_connection_index + dir * q->K * q->per_block;
+                q->bias = l->first_bias_connection_index + dir * (q->C + 3 * q->K);
+                q->reverse = (int)dir;
+                size_t sc = T * B * q->C, sk = T * B * q->K;
+                float **cells[] = {&q->sum_in_z, &q->sum_rec_z, &q->sum_z, &q->z, &q->c, &q->ca, &q->dz, &q->dc};
+                float **blocks[] = {&q->sum_in_i, &q->sum_in_f, &q->sum_in_o, &q->sum_rec_i, &q->sum_rec_f, &q->sum_rec_o, &q->sum_i, &q->sum_f, &q->sum_o,
+                                    &q->gi, &q->gf, &q->go, &q->di, &q->df, &q->dgo};
+                for (size_t a = 0; a < sizeof(cells) / sizeof(cells[0]); ++a) *cells[a] = zalloc(sc);
+                for (size_t a = 0; a < sizeof(blocks) / sizeof(blocks[0]); ++a) *blocks[a] = zalloc(sk);
+                if (dirs == 2) { q->h = zalloc(sc); q->dh = zalloc(sc); }
+                else { q->h = o->values; q->dh = o->af_errors; }
+            }
+            o->lstm = qq;
             continue;
         }
         o->af_errors = zalloc(T * B * o->AH);
@@ -330,11 +342,15 @@ int myea_oracle_destroy(myea_oracle_net *n)
         free(o->means); free(o->variances); free(o->means_averages); free(o->variances_averages);
         free(o->r_corrections); free(o->d_corrections); free(o->derivatives_means); free(o->derivatives_variances);
         if (o->lstm) {
-            olstm *q = o->lstm;
-            float *all[] = {q->sum_in_z, q->sum_rec_z, q->sum_z, q->z, q->c, q->ca, q->dz, q->dc, q->sum_in_i, q->sum_in_f, q->sum_in_o, q->sum_rec_i,
-                            q->sum_rec_f, q->sum_rec_o, q->sum_i, q->sum_f, q->sum_o, q->gi, q->gf, q->go, q->di, q->df, q->dgo};
-            for (size_t a = 0; a < sizeof(all) / sizeof(all[0]); ++a) free(all[a]);
-            free(q);
+            for (int dir = 0; dir < 2; ++dir) {
+                olstm *q = &o->lstm[dir];
+                float *all[] = {q->sum_in_z, q->sum_rec_z, q->sum_z, q->z, q->c, q->ca, q->dz, q->dc, q->sum_in_i, q->sum_in_f, q->sum_in_o, q->sum_rec_i,
+                                q->sum_rec_f, q->sum_rec_o, q->sum_i, q->sum_f, q->sum_o, q->gi, q->gf, q->go, q->di, q->df, q->dgo};
+                for (size_t a = 0; a < sizeof(all) / sizeof(all[0]); ++a) free(all[a]);
+                if (q->h != o->values) free(q->h);
+                if (q->dh != o->af_errors) free(q->dh);
+            }
+            free(o->lstm);
         }
     }
     free(n);
@@ -574,7 +590,7 @@ static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t B)
 
 /* parameter offsets inside the layer's slice, NN/Neural_Network__Prepare_Connections.cpp:82-222: per block
  * [z_in(In) | z_rec(C)] x cells, i_in, f_in, o_in (In each), i_rec, f_rec, o_rec (C each), peep_i, peep_f, peep_o (cpb each) */
-static size_t lstm_block_base(const myea_layer_desc *l, const olstm *q, size_t k) { return l->first_connection_index + k * q->per_block; }
+static size_t lstm_block_base(const myea_layer_desc *l, const olstm *q, size_t k) { (void)l; return q->base + k * q->per_block; }
 static size_t lstm_z_in(const myea_layer_desc *l, const olstm *q, size_t k, size_t j) { return lstm_block_base(l, q, k) + j * (q->In + q->C); }
 static size_t lstm_z_rec(const myea_layer_desc *l, const olstm *q, size_t k, size_t j) { return lstm_z_in(l, q, k, j) + q->In; }
 static size_t lstm_gate_in(const myea_layer_desc *l, const olstm *q, size_t k, int g) { return lstm_block_base(l, q, k) + q->cpb * (q->In + q->C) + (size_t)g * q->In; }
@@ -589,21 +605,24 @@ static float tanh_f(float s) { return 2.f / (1.f + expf(-2.f * s)) - 1.f; }
  * Gates_CIF_AF_State (:1042-1191) -> States_AF (:1547-1582) -> Output (:1351-1418).
  * First step: no recurrent sums, no forget gate, no input-gate peephole, c = i * z; the output gate peeps at c[t].
  * Bias vectors sit at first_bias_connection_index + {0, C, C + K, C + 2K} (the field as Prepare__Bias__LSTM leaves it). */
-static void fwd_lstm_step(myea_oracle_net *n, size_t li, size_t t, size_t B)
+static void fwd_lstm_step(myea_oracle_net *n, size_t li, int dir, size_t t, size_t B)
 {
     const myea_layer_desc *l = &n->d.layers[li];
     olayer *o = &n->L[li];
-    olstm *q = o->lstm;
+    olstm *q = &o->lstm[dir];
     size_t Bmax = n->d.batch_size, K = q->K, C = q->C, cpb = q->cpb, In = q->In;
     const float *x = layer_outputs(n, n->L[li].prev), *w = n->parameters;
-    const float *bz = w + l->first_bias_connection_index, *bi = bz + C, *bf = bi + K, *bo = bf + K;
-    int first = t == 0;
+    const float *bz = w + q->bias, *bi = bz + C, *bf = bi + K, *bo = bf + K;
+    /* the step processed before this one: t - 1, or t + 1 for the direction that walks time backwards
+     * (tmp_time_step_reverse_direction, NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:456-461) */
+    size_t tp = q->reverse ? t + 1 : t - 1;
+    int first = q->reverse ? t == n->d.number_recurrent_depth - 1 : t == 0;
     long b;
 #pragma omp parallel for schedule(static) num_threads(n->threads)
     for (b = 0; b < (long)B; ++b) {
-        size_t kb = (size_t)b * K + Bmax * K * t, cb = (size_t)b * C + Bmax * C * t, cp = (size_t)b * C + Bmax * C * (t - 1);
+        size_t kb = (size_t)b * K + Bmax * K * t, cb = (size_t)b * C + Bmax * C * t, cp = (size_t)b * C + Bmax * C * tp;
         const float *xi = x + (size_t)b * In + Bmax * In * t;
-        const float *hp = first ? NULL : o->values + cp;
+        const float *hp = first ? NULL : q->h + cp;
         for (size_t k = 0; k < K; ++k) {
             for (size_t j = 0; j < cpb; ++j) {
                 size_t c = k * cpb + j;
@@ -655,17 +674,17 @@ static void fwd_lstm_step(myea_oracle_net *n, size_t li, size_t t, size_t B)
             for (size_t j = 0; j < cpb; ++j) so += q->c[cb + k * cpb + j] * po[j];
             q->sum_o[kb + k] = so;
             q->go[kb + k] = sigmoid_f(so);
-            for (size_t j = 0; j < cpb; ++j) o->values[cb + k * cpb + j] = q->ca[cb + k * cpb + j] * q->go[kb + k];
+            for (size_t j = 0; j < cpb; ++j) q->h[cb + k * cpb + j] = q->ca[cb + k * cpb + j] * q->go[kb + k];
         }
     }
 }
 
 /* Backward_Pass__LSTM (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:1024-1120): delta to the layer below,
  * dst[t][b][:] += dz_c Wz_in[c][:] + di_k Wi_in[k][:] + df_k Wf_in[k][:] + do_k Wo_in[k][:] */
-static void bwd_lstm_to_previous(myea_oracle_net *n, size_t gi, size_t t, size_t B, float *dst)
+static void bwd_lstm_to_previous_dir(myea_oracle_net *n, size_t gi, int dir, size_t t, size_t B, float *dst)
 {
     const myea_layer_desc *l = &n->d.layers[gi];
-    olstm *q = n->L[gi].lstm;
+    olstm *q = &n->L[gi].lstm[dir];
     size_t Bmax = n->d.batch_size, K = q->K, C = q->C, cpb = q->cpb, In = q->In;
     const float *w = n->parameters;
     long b;
@@ -689,22 +708,30 @@ static void bwd_lstm_to_previous(myea_oracle_net *n, size_t gi, size_t t, size_t
     }
 }
 
+static void bwd_lstm_to_previous(myea_oracle_net *n, size_t gi, size_t t, size_t B, float *dst)
+{
+    bwd_lstm_to_previous_dir(n, gi, 0, t, B, dst);
+    if (n->d.layers[gi].use_bidirectional) bwd_lstm_to_previous_dir(n, gi, 1, t, B, dst);
+}
+
 /* Recurrent__Backward_Pass__Gradient__LSTM (:440-862) for one time step, t descending:
  * Backward_Pass__LSTM_Derivative__Output (:1130-1273), __Cell_State_AF (:1275-1327), __Gates_CIF_AF_State (:1329-1604). */
-static void bwd_lstm_step(myea_oracle_net *n, size_t li, size_t t, size_t B)
+static void bwd_lstm_step(myea_oracle_net *n, size_t li, int dir, size_t t, size_t B)
 {
     const myea_layer_desc *l = &n->d.layers[li];
     olayer *o = &n->L[li];
-    olstm *q = o->lstm;
+    olstm *q = &o->lstm[dir];
     size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, K = q->K, C = q->C, cpb = q->cpb;
     const float *w = n->parameters;
-    int last = t == T - 1, first = t == 0;
+    /* "next" / "previous" in the direction's own processing order */
+    size_t tn = q->reverse ? t - 1 : t + 1, tp = q->reverse ? t + 1 : t - 1;
+    int last = q->reverse ? t == 0 : t == T - 1, first = q->reverse ? t == T - 1 : t == 0;
     long b;
 #pragma omp parallel for schedule(static) num_threads(n->threads)
     for (b = 0; b < (long)B; ++b) {
         size_t kb = (size_t)b * K + Bmax * K * t, cb = (size_t)b * C + Bmax * C * t;
-        size_t kn = (size_t)b * K + Bmax * K * (t + 1), cn = (size_t)b * C + Bmax * C * (t + 1), cp = (size_t)b * C + Bmax * C * (t - 1);
-        float *dh = o->af_errors + cb;
+        size_t kn = (size_t)b * K + Bmax * K * tn, cn = (size_t)b * C + Bmax * C * tn, cp = (size_t)b * C + Bmax * C * tp;
+        float *dh = q->dh + cb;
         if (!last) { /* recurrent delta from t + 1 */
             for (size_t c = 0; c < C; ++c) {
                 float e = q->dz[cn + c];
@@ -758,11 +785,11 @@ static void bwd_lstm_step(myea_oracle_net *n, size_t li, size_t t, size_t B)
 
 /* Recurrent__Update_Derivative_Weight__LSTM (NN/Neural_Network__Recurrent_Update_Derivative_Weight__OpenMP.cpp:492-728)
  * and __LSTM__Bias (:730-776). */
-static void dw_lstm(myea_oracle_net *n, size_t li, size_t B)
+static void dw_lstm_dir(myea_oracle_net *n, size_t li, int dir, size_t B)
 {
     const myea_layer_desc *l = &n->d.layers[li];
     olayer *o = &n->L[li];
-    olstm *q = o->lstm;
+    olstm *q = &o->lstm[dir];
     size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, K = q->K, C = q->C, cpb = q->cpb, In = q->In;
     const float *x = layer_outputs(n, n->L[li].prev);
     float *g = n->gradient;
@@ -774,9 +801,10 @@ static void dw_lstm(myea_oracle_net *n, size_t li, size_t B)
         size_t k = (size_t)kk;
         for (size_t b = 0; b < B; ++b)
             for (size_t t = 0; t < T; ++t) {
-                int last = t == T - 1;
-                size_t kb = b * K + Bmax * K * t, cb = b * C + Bmax * C * t, kn = b * K + Bmax * K * (t + 1), cn = b * C + Bmax * C * (t + 1);
-                const float *xi = x + b * In + Bmax * In * t, *h = o->values + cb;
+                int last = q->reverse ? t == 0 : t == T - 1;
+                size_t tn = q->reverse ? t - 1 : t + 1;
+                size_t kb = b * K + Bmax * K * t, cb = b * C + Bmax * C * t, kn = b * K + Bmax * K * tn, cn = b * C + Bmax * C * tn;
+                const float *xi = x + b * In + Bmax * In * t, *h = q->h + cb;
                 for (size_t j = 0; j < cpb; ++j) {
                     size_t c = k * cpb + j;
                     float e = q->dz[cb + c];
@@ -803,13 +831,46 @@ static void dw_lstm(myea_oracle_net *n, size_t li, size_t B)
                 }
             }
     }
-    float *bz = g + l->first_bias_connection_index, *bi = bz + C, *bf = bi + K, *bo = bf + K;
+    float *bz = g + q->bias, *bi = bz + C, *bf = bi + K, *bo = bf + K;
     for (size_t b = 0; b < B; ++b)
         for (size_t t = 0; t < T; ++t) {
             size_t kb = b * K + Bmax * K * t, cb = b * C + Bmax * C * t;
             for (size_t c = 0; c < C; ++c) bz[c] += q->dz[cb + c];
             for (size_t k = 0; k < K; ++k) { bi[k] += q->di[kb + k]; bf[k] += q->df[kb + k]; bo[k] += q->dgo[kb + k]; }
         }
+}
+
+static void dw_lstm(myea_oracle_net *n, size_t li, size_t B)
+{
+    dw_lstm_dir(n, li, 0, B);
+    if (n->d.layers[li].use_bidirectional) dw_lstm_dir(n, li, 1, B);
+}
+
+/* A layer with two directions (contract of this library; the reference's own two-direction path overlays the
+ * directions' buffers and cannot be followed): each direction is the one-direction recurrence above over its own blocks,
+ * the second one walking time backwards; the layer's output is the SUM of the two cell outputs (the layer keeps the
+ * width of one direction, NN/Neural_Network__Compile.cpp:79) and both directions receive the same delta from above
+ * (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:144-156). */
+static void fwd_lstm_layer(myea_oracle_net *n, size_t li, size_t B)
+{
+    olayer *o = &n->L[li];
+    size_t T = n->d.number_recurrent_depth, dirs = n->d.layers[li].use_bidirectional ? 2 : 1;
+    for (size_t dir = 0; dir < dirs; ++dir)
+        for (size_t s = 0; s < T; ++s) fwd_lstm_step(n, li, (int)dir, dir ? T - 1 - s : s, B);
+    if (dirs == 2) {
+        size_t cnt = T * n->d.batch_size * o->H;
+        for (size_t i = 0; i < cnt; ++i) o->values[i] = o->lstm[0].h[i] + o->lstm[1].h[i];
+    }
+}
+
+static void bwd_lstm_layer(myea_oracle_net *n, size_t li, size_t B)
+{
+    olayer *o = &n->L[li];
+    size_t T = n->d.number_recurrent_depth, dirs = n->d.layers[li].use_bidirectional ? 2 : 1;
+    for (size_t dir = 0; dir < dirs; ++dir) {
+        if (dirs == 2) memcpy(o->lstm[dir].dh, o->af_errors, T * n->d.batch_size * o->H * sizeof(float));
+        for (size_t s = T; s-- > 0;) bwd_lstm_step(n, li, (int)dir, dir ? T - 1 - s : s, B);
+    }
 }
 
 /* FF__Forward_Pass_Batch: NN/Neural_Network__Forward_Pass__OpenMP.cpp:24-120;
@@ -830,7 +891,7 @@ int myea_oracle_forward_pass(myea_oracle_net *n, size_t B, const float *inputs)
         if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             for (size_t t = 0; t < T; ++t) fwd_fc_layer(n, li, t, B);
         } else if (l->type_layer == MYEA_LAYER_LSTM) {
-            for (size_t t = 0; t < T; ++t) fwd_lstm_step(n, li, t, B);
+            fwd_lstm_layer(n, li, B);
         } else if (l->type_layer == MYEA_LAYER_RESIDUAL) {
             fwd_residual_block(n, li, B);
             li += l->block_depth; /* the iterator is left on the block's last member, :3884-3885 */
@@ -1148,7 +1209,7 @@ int myea_oracle_backward_pass(myea_oracle_net *n, size_t B)
         if (cur->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             for (size_t tt = T; tt-- > 0;) bwd_gradient_fc(n, li, tt, B);
         } else if (cur->type_layer == MYEA_LAYER_LSTM) {
-            for (size_t tt = T; tt-- > 0;) bwd_lstm_step(n, li, tt, B);
+            bwd_lstm_layer(n, li, B);
         } else if (cur->type_layer == MYEA_LAYER_RESIDUAL) {
             bwd_gradient_residual(n, li, B);
             gi = li + 1;
@@ -1325,10 +1386,14 @@ const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t 
     default: break;
     }
     if (o->lstm) {
-        olstm *q = o->lstm;
+        int backward = (kind & MYEA_TENSOR_DIRECTION_BACKWARD) != 0;
+        if (backward && !n->d.layers[li].use_bidirectional) { if (count) *count = 0; return NULL; }
+        olstm *q = &o->lstm[backward];
+        kind &= ~MYEA_TENSOR_DIRECTION_BACKWARD;
         size_t cc = T * n->d.batch_size * q->C, kk = T * n->d.batch_size * q->K;
         switch (kind) {
-        case MYEA_TENSOR_ERRORS: p = o->af_errors; c = cc; break;
+        case MYEA_TENSOR_LSTM_CELL_OUTPUT: p = q->h; c = cc; break;
+        case MYEA_TENSOR_ERRORS: p = q->dh; c = cc; break;
         case MYEA_TENSOR_LSTM_CELL_INPUT: p = q->z; c = cc; break;
         case MYEA_TENSOR_LSTM_CELL_STATE: p = q->c; c = cc; break;
         case MYEA_TENSOR_LSTM_INPUT_GATE: p = q->gi; c = kk; break;
