@@ -213,6 +213,8 @@ enum {
     MYEA_TENSOR_LSTM_DELTA_FORGET_GATE = 24,
     MYEA_TENSOR_LSTM_DELTA_OUTPUT_GATE = 25,
     MYEA_TENSOR_LSTM_CELL_OUTPUT = 26,     /* h of one direction (OUTPUTS is the layer's output: the sum of both) */
+    MYEA_TENSOR_LSTM_DELTA_CELL_OUTPUT = 27, /* delta of h of one direction incl. its recurrent terms (ERRORS of a
+                                              bidirectional layer is the delta of the summed output, from above only) */
     MYEA_TENSOR_DIRECTION_BACKWARD = 0x100 /* OR-ed onto an LSTM kind: the time-reversed direction of a bidirectional layer */
 };
 

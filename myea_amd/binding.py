@@ -33,7 +33,7 @@ TENSOR = dict(OUTPUTS=0, SUMMATIONS=1, ERRORS=2, NORM_HATS=3, NORM_MEANS=4, NORM
               NORM_MEANS_AVERAGES=6, NORM_VARIANCES_AVERAGES=7, INPUT_SIDE_ERRORS=8,
               LSTM_CELL_INPUT=16, LSTM_CELL_STATE=17, LSTM_INPUT_GATE=18, LSTM_FORGET_GATE=19,
               LSTM_OUTPUT_GATE=20, LSTM_DELTA_CELL_INPUT=21, LSTM_DELTA_CELL_STATE=22,
-              LSTM_DELTA_INPUT_GATE=23, LSTM_DELTA_FORGET_GATE=24, LSTM_DELTA_OUTPUT_GATE=25, LSTM_CELL_OUTPUT=26,
+              LSTM_DELTA_INPUT_GATE=23, LSTM_DELTA_FORGET_GATE=24, LSTM_DELTA_OUTPUT_GATE=25, LSTM_CELL_OUTPUT=26, LSTM_DELTA_CELL_OUTPUT=27,
               DIRECTION_BACKWARD=0x100)
 E_INVALID, E_UNSUPPORTED, E_BATCH, E_STATE, E_NOMEM, E_DEVICE = -1, -2, -3, -4, -5, -6
 

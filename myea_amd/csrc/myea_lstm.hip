@@ -25,6 +25,10 @@ namespace myea {
 
 struct LstmLayer {
     size_t K = 0, cpb = 0, C = 0, G = 0, In = 0, per_block = 0, base = 0;
+    size_t bias = 0;        // flat index of the direction's bias vectors z | i | f | o
+    bool reverse = false;   // second direction of a bidirectional layer: walks time from T-1 down to 0
+    bool own_h = false;     // bidirectional: h / dh are the direction's own buffers; else the layer's values / neuron_errors
+    float *h = nullptr, *dh = nullptr;                           // [T][Bmax][C] cell outputs and their delta
     float *Win = nullptr, *Wrec = nullptr, *peep = nullptr;      // packed parameters
     float *gWin = nullptr, *gWrec = nullptr;                     // packed gradient scratch
     float *acts = nullptr;  // [T][Bmax][G]: pre-activation sums, overwritten in place by z | i | f | o
@@ -220,14 +224,15 @@ struct PeepF {
     LstmGeom g;
     size_t B, Bmax, T;
     const float *c, *dG;
+    int reverse;   // the step processed after t is t - 1
     __device__ void operator()(size_t r, size_t col, double *acc) const
     {
         const size_t t = r / B, b = r % B, k = col / g.cpb;
         const size_t row = t * Bmax + b;
         const float cs = c[row * g.C + col];
         acc[2] += dG[row * g.G + g.C + 2 * g.K + k] * cs;
-        if (t + 1 < T) {
-            const size_t nrow = (t + 1) * Bmax + b;
+        if (reverse ? t > 0 : t + 1 < T) {
+            const size_t nrow = (reverse ? t - 1 : t + 1) * Bmax + b;
             acc[0] += dG[nrow * g.G + g.C + k] * cs;
             acc[1] += dG[nrow * g.G + g.C + g.K + k] * cs;
         }
@@ -280,47 +285,61 @@ int Net::lstm_create_layer(size_t li)
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
-    if (l.use_bidirectional) { set_last_error("layer %zu: bidirectional LSTM is not on this path", li); return MYEA_E_UNSUPPORTED; }
     if (layer_uses_norm(l)) { set_last_error("layer %zu: normalisation inside an LSTM layer is not on this path", li); return MYEA_E_UNSUPPORTED; }
     if (l.type_dropout != MYEA_DROPOUT_NONE) { set_last_error("layer %zu: dropout on an LSTM layer is not on this path", li); return MYEA_E_UNSUPPORTED; }
     if (l.n_cells_per_block == 0) { set_last_error("layer %zu: LSTM needs at least one cell per block", li); return MYEA_E_INVALID; }
-    LstmLayer *q = new LstmLayer();
-    o.lstm = q;
-    q->K = l.n_units; q->cpb = l.n_cells_per_block; q->C = q->K * q->cpb; q->G = q->C + 3 * q->K; q->In = L[li].In;
-    q->per_block = q->cpb * (q->In + q->C) + 3 * q->In + 3 * q->C + 3 * q->cpb;
-    q->base = l.first_connection_index;
-    if (q->base + q->K * q->per_block > d.total_weights) { set_last_error("layer %zu: LSTM weight slice leaves the weight region", li); return MYEA_E_INVALID; }
-    // The four bias vectors are read at first_bias_connection_index + [0, G).  With the index as Prepare__Bias__LSTM
-    // leaves it they reach C entries into the following layers' bias slots; beyond the bias region the reference would
-    // read and write outside its parameter array, which is refused here.
-    if (l.first_bias_connection_index < d.total_weights || l.first_bias_connection_index + q->G > d.total_weights + d.total_bias) {
-        set_last_error("layer %zu: LSTM bias slice [%llu, +%zu) leaves the bias region", li, (unsigned long long)l.first_bias_connection_index, q->G);
-        return MYEA_E_INVALID;
-    }
     const size_t T = d.number_recurrent_depth, B = d.batch_size;
-    MYEA_TRY(dev_alloc_zero(&q->Win, q->G * q->In));
-    MYEA_TRY(dev_alloc_zero(&q->Wrec, q->G * q->C));
-    MYEA_TRY(dev_alloc_zero(&q->peep, 3 * q->C));
-    MYEA_TRY(dev_alloc_zero(&q->gWin, kMaxSlabs * q->G * q->In));   // split-K slabs of the weight-gradient contractions
-    MYEA_TRY(dev_alloc_zero(&q->gWrec, kMaxSlabs * q->G * q->C));
-    MYEA_TRY(dev_alloc_zero(&q->acts, T * B * q->G));
-    MYEA_TRY(dev_alloc_zero(&q->c, T * B * q->C));
-    MYEA_TRY(dev_alloc_zero(&q->ca, T * B * q->C));
-    MYEA_TRY(dev_alloc_zero(&q->dG, T * B * q->G));
-    MYEA_TRY(dev_alloc_zero(&q->dc, T * B * q->C));
-    MYEA_TRY(dev_alloc_zero(&q->part, 16 * B * q->G));
-    MYEA_TRY(dev_alloc_zero(&o.neuron_errors, T * B * q->C));  // delta of the cell outputs (ptr_delta_cell_output)
+    const size_t dirs = l.use_bidirectional ? 2 : 1;
+    MYEA_TRY(dev_alloc_zero(&o.neuron_errors, T * B * (size_t)l.n_units * l.n_cells_per_block));  // delta of the layer's output (ptr_delta_cell_output)
+    // Two directions (contract of this library: the reference overlays its two directions' buffers and has no behaviour to
+    // follow): direction 1 owns the second half of the layer's blocks and the second [G] slice of its biases and walks time
+    // backwards; the layer's output is the sum of both cell outputs and both receive the same delta from above.
+    for (size_t dir = 0; dir < dirs; ++dir) {
+        LstmLayer *q = new LstmLayer();
+        (dir ? o.lstm2 : o.lstm) = q;
+        q->K = l.n_units; q->cpb = l.n_cells_per_block; q->C = q->K * q->cpb; q->G = q->C + 3 * q->K; q->In = L[li].In;
+        q->per_block = q->cpb * (q->In + q->C) + 3 * q->In + 3 * q->C + 3 * q->cpb;
+        q->base = l.first_connection_index + dir * q->K * q->per_block;
+        q->bias = l.first_bias_connection_index + dir * q->G;
+        q->reverse = dir == 1;
+        q->own_h = dirs == 2;
+        if (q->base + q->K * q->per_block > d.total_weights) { set_last_error("layer %zu: LSTM weight slice leaves the weight region", li); return MYEA_E_INVALID; }
+        // The four bias vectors are read at bias + [0, G).  With the index as Prepare__Bias__LSTM leaves it (one direction)
+        // they reach C entries into the following layers' bias slots; beyond the bias region the reference would read and
+        // write outside its parameter array, which is refused here.
+        if (q->bias < d.total_weights || q->bias + q->G > d.total_weights + d.total_bias) {
+            set_last_error("layer %zu: LSTM bias slice [%zu, +%zu) leaves the bias region", li, q->bias, q->G);
+            return MYEA_E_INVALID;
+        }
+        MYEA_TRY(dev_alloc_zero(&q->Win, q->G * q->In));
+        MYEA_TRY(dev_alloc_zero(&q->Wrec, q->G * q->C));
+        MYEA_TRY(dev_alloc_zero(&q->peep, 3 * q->C));
+        MYEA_TRY(dev_alloc_zero(&q->gWin, kMaxSlabs * q->G * q->In));   // split-K slabs of the weight-gradient contractions
+        MYEA_TRY(dev_alloc_zero(&q->gWrec, kMaxSlabs * q->G * q->C));
+        MYEA_TRY(dev_alloc_zero(&q->acts, T * B * q->G));
+        MYEA_TRY(dev_alloc_zero(&q->c, T * B * q->C));
+        MYEA_TRY(dev_alloc_zero(&q->ca, T * B * q->C));
+        MYEA_TRY(dev_alloc_zero(&q->dG, T * B * q->G));
+        MYEA_TRY(dev_alloc_zero(&q->dc, T * B * q->C));
+        MYEA_TRY(dev_alloc_zero(&q->part, 16 * B * q->G));
+        if (q->own_h) {
+            MYEA_TRY(dev_alloc_zero(&q->h, T * B * q->C));
+            MYEA_TRY(dev_alloc_zero(&q->dh, T * B * q->C));
+        } else { q->h = o.values; q->dh = o.neuron_errors; }
+    }
     return MYEA_OK;
 }
 
 void Net::lstm_destroy_layer(DevLayer &o)
 {
-    if (!o.lstm) return;
-    LstmLayer *q = o.lstm;
-    float *all[] = {q->Win, q->Wrec, q->peep, q->gWin, q->gWrec, q->acts, q->c, q->ca, q->dG, q->dc, q->part};
-    for (float *p : all) if (p) (void)hipFree(p);
-    delete q;
-    o.lstm = nullptr;
+    for (LstmLayer **slot : {&o.lstm, &o.lstm2}) {
+        LstmLayer *q = *slot;
+        if (!q) continue;
+        float *all[] = {q->Win, q->Wrec, q->peep, q->gWin, q->gWrec, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr};
+        for (float *p : all) if (p) (void)hipFree(p);
+        delete q;
+        *slot = nullptr;
+    }
 }
 
 size_t Net::lstm_scratch_floats() const
@@ -335,24 +354,23 @@ size_t Net::lstm_scratch_floats() const
 int Net::lstm_parameters_changed()
 {
     for (size_t li = 1; li < L.size(); ++li) {
-        LstmLayer *q = L[li].lstm;
-        if (!q) continue;
-        const size_t n = q->G * (q->In + q->C) + 3 * q->C;
-        hipLaunchKernelGGL(lstm_gather_kernel, dim3(grid_for(n, kBlock, 4096)), dim3(kBlock), 0, stream, geom_of(*q), parameters, q->Win, q->Wrec, q->peep);
-        MYEA_HIP_TRY(hipGetLastError());
+        for (LstmLayer *q : {L[li].lstm, L[li].lstm2}) {
+            if (!q) continue;
+            const size_t n = q->G * (q->In + q->C) + 3 * q->C;
+            hipLaunchKernelGGL(lstm_gather_kernel, dim3(grid_for(n, kBlock, 4096)), dim3(kBlock), 0, stream, geom_of(*q), parameters, q->Win, q->Wrec, q->peep);
+            MYEA_HIP_TRY(hipGetLastError());
+        }
     }
     return MYEA_OK;
 }
 
-// Recurrent__Forward_Pass__LSTM (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:448-471), time ascending.
-int Net::lstm_forward_layer(size_t li, size_t B)
+// Recurrent__Forward_Pass__LSTM (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:448-471): time ascending, or
+// descending for the second direction (the "previous" step is then t + 1, :456-461).
+int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
 {
-    const myea_layer_desc &l = d.layers[li];
-    DevLayer &o = L[li];
-    LstmLayer &q = *o.lstm;
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
     const float *x = layer_outputs(L[li].prev);
-    const float *bias = parameters + l.first_bias_connection_index;
+    const float *bias = parameters + q.bias;
     // input sums of every time step in one contraction when the rows are contiguous
     const bool per_t = T > 1 && B != Bmax;
     const size_t chunks = per_t ? T : 1, rows = per_t ? B : T * B;
@@ -367,12 +385,13 @@ int Net::lstm_forward_layer(size_t li, size_t B)
         prof_end(2.0 * (double)rows * (double)q.G * (double)q.In);
     }
     const LstmGeom geom = geom_of(q);
-    for (size_t t = 0; t < T; ++t) {
+    for (size_t s = 0; s < T; ++s) {
+        const size_t t = q.reverse ? T - 1 - s : s, tp = q.reverse ? t + 1 : t - 1;  // tp: the step processed before t
         float *acts_t = q.acts + t * Bmax * q.G;
         int nparts = 0;
-        if (t > 0) {
+        if (s > 0) {
             GemmParams g{};
-            g.A = o.values + (t - 1) * Bmax * q.C; g.lda = (long)q.C; g.a_k_contiguous = 1;
+            g.A = q.h + tp * Bmax * q.C; g.lda = (long)q.C; g.a_k_contiguous = 1;
             g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 1;
             g.C = q.part; g.ldc = (long)q.G;
             g.M = (int)B; g.N = (int)q.G; g.K = (int)q.C;
@@ -382,29 +401,41 @@ int Net::lstm_forward_layer(size_t li, size_t B)
             MYEA_TRY(launch_gemm(stream, g));
             prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
         }
-        hipLaunchKernelGGL(lstm_forward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, (int)(t == 0), bias, q.peep,
-                           acts_t, t ? q.c + (t - 1) * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, o.values + t * Bmax * q.C,
+        hipLaunchKernelGGL(lstm_forward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, (int)(s == 0), bias, q.peep,
+                           acts_t, s ? q.c + tp * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, q.h + t * Bmax * q.C,
                            q.part, nparts);
         MYEA_HIP_TRY(hipGetLastError());
     }
     return MYEA_OK;
 }
 
-// Recurrent__Backward_Pass__Gradient__LSTM (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:440-862), time
-// descending; o.neuron_errors (= delta of the cell outputs) already holds what the layers above sent down.
-int Net::lstm_backward_layer(size_t li, size_t B)
+int Net::lstm_forward_layer(size_t li, size_t B)
 {
     DevLayer &o = L[li];
-    LstmLayer &q = *o.lstm;
+    MYEA_TRY(lstm_forward_direction(li, *o.lstm, B));
+    if (o.lstm2) {
+        MYEA_TRY(lstm_forward_direction(li, *o.lstm2, B));
+        const size_t rows = (size_t)d.number_recurrent_depth * d.batch_size;
+        MYEA_TRY(launch_padded_add(stream, rows, o.H, o.lstm->h, o.H, 0, o.lstm2->h, o.H, 0, o.values));  // output = h_forward + h_backward
+    }
+    return MYEA_OK;
+}
+
+// Recurrent__Backward_Pass__Gradient__LSTM (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:440-862), time
+// descending; o.neuron_errors (= delta of the cell outputs) already holds what the layers above sent down.
+int Net::lstm_backward_direction(LstmLayer &q, size_t B)
+{
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
     const LstmGeom geom = geom_of(q);
-    for (size_t t = T; t-- > 0;) {
-        float *dh_t = o.neuron_errors + t * Bmax * q.C;
-        const bool last = t == T - 1, first = t == 0;
+    for (size_t s = T; s-- > 0;) {
+        // tn / tp: the steps processed after / before t in the direction's own order
+        const size_t t = q.reverse ? T - 1 - s : s, tn = q.reverse ? t - 1 : t + 1, tp = q.reverse ? t + 1 : t - 1;
+        float *dh_t = q.dh + t * Bmax * q.C;
+        const bool last = s == T - 1, first = s == 0;
         int nparts = 0;
         if (!last) {  // Backward_Pass__LSTM_Derivative__Output, recurrent part (:1174-1226)
             GemmParams g{};
-            g.A = q.dG + (t + 1) * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 1;
+            g.A = q.dG + tn * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 1;
             g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 0;
             g.C = q.part; g.ldc = (long)q.C;
             g.M = (int)B; g.N = (int)q.C; g.K = (int)q.G;
@@ -416,18 +447,30 @@ int Net::lstm_backward_layer(size_t li, size_t B)
         }
         const int mode = (first && last) ? 0 : (last ? 1 : (first ? 3 : 2));
         hipLaunchKernelGGL(lstm_backward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, mode, q.peep,
-                           q.acts + t * Bmax * q.G, last ? nullptr : q.acts + (t + 1) * Bmax * q.G, first ? nullptr : q.c + (t - 1) * Bmax * q.C,
-                           q.ca + t * Bmax * q.C, dh_t, q.dG + t * Bmax * q.G, last ? nullptr : q.dG + (t + 1) * Bmax * q.G,
-                           q.dc + t * Bmax * q.C, last ? nullptr : q.dc + (t + 1) * Bmax * q.C, q.part, nparts);
+                           q.acts + t * Bmax * q.G, last ? nullptr : q.acts + tn * Bmax * q.G, first ? nullptr : q.c + tp * Bmax * q.C,
+                           q.ca + t * Bmax * q.C, dh_t, q.dG + t * Bmax * q.G, last ? nullptr : q.dG + tn * Bmax * q.G,
+                           q.dc + t * Bmax * q.C, last ? nullptr : q.dc + tn * Bmax * q.C, q.part, nparts);
         MYEA_HIP_TRY(hipGetLastError());
     }
     return MYEA_OK;
 }
 
-// the operands of "delta of the layer below = dG Win" (Backward_Pass__LSTM, :1024-1120), handed to the shared driver
-void Net::lstm_delta_source(size_t gi, const float **delta, size_t *width, const float **weights)
+int Net::lstm_backward_layer(size_t li, size_t B)
 {
-    LstmLayer &q = *L[gi].lstm;
+    DevLayer &o = L[li];
+    for (LstmLayer *q : {o.lstm, o.lstm2}) {
+        if (!q) continue;
+        if (q->own_h)  // both directions start from the same delta of the layer's output
+            MYEA_HIP_TRY(hipMemcpyAsync(q->dh, o.neuron_errors, (size_t)d.number_recurrent_depth * d.batch_size * q->C * sizeof(float), hipMemcpyDeviceToDevice, stream));
+        MYEA_TRY(lstm_backward_direction(*q, B));
+    }
+    return MYEA_OK;
+}
+
+// the operands of "delta of the layer below = dG Win" (Backward_Pass__LSTM, :1024-1120), handed to the shared driver
+void Net::lstm_delta_source(size_t gi, int direction, const float **delta, size_t *width, const float **weights)
+{
+    LstmLayer &q = direction ? *L[gi].lstm2 : *L[gi].lstm;
     *delta = q.dG;
     *width = q.G;
     *weights = q.Win;
@@ -437,9 +480,13 @@ void Net::lstm_delta_source(size_t gi, const float **delta, size_t *width, const
 // and __LSTM__Bias (:730-776).
 int Net::lstm_update_derivative_weight(size_t li, size_t B)
 {
-    const myea_layer_desc &l = d.layers[li];
-    DevLayer &o = L[li];
-    LstmLayer &q = *o.lstm;
+    MYEA_TRY(lstm_update_derivative_weight_direction(li, *L[li].lstm, B));
+    if (L[li].lstm2) MYEA_TRY(lstm_update_derivative_weight_direction(li, *L[li].lstm2, B));
+    return MYEA_OK;
+}
+
+int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t B)
+{
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
     const float *x = layer_outputs(L[li].prev);
     const LstmGeom geom = geom_of(q);
@@ -471,12 +518,13 @@ int Net::lstm_update_derivative_weight(size_t li, size_t B)
             prof_end(2.0 * (double)B * (double)q.G * (double)q.In);
         }
     }
-    // recurrent weights: dG[t+1]^T h[t] for t < T-1
+    // recurrent weights: dG[t+1]^T h[t] for t < T-1 (second direction: dG[t]^T h[t+1]); both operand ranges are contiguous
+    const size_t dg_shift = q.reverse ? 0 : 1, h_shift = q.reverse ? 1 : 0;
     if (T > 1 && !per_t) {
         const size_t rows = (T - 1) * B;
         GemmParams g{};
-        g.A = q.dG + Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
-        g.B = o.values; g.ldb = (long)q.C; g.b_k_contiguous = 0;
+        g.A = q.dG + dg_shift * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
+        g.B = q.h + h_shift * Bmax * q.C; g.ldb = (long)q.C; g.b_k_contiguous = 0;
         g.C = q.gWrec; g.ldc = (long)q.C;
         g.M = (int)q.G; g.N = (int)q.C; g.K = (int)rows;
         s_rec = gemm_split_k(g.M, g.N, g.K);
@@ -488,8 +536,8 @@ int Net::lstm_update_derivative_weight(size_t li, size_t B)
         s_rec = 1;
         for (size_t c = 0; c + 1 < T; ++c) {
             GemmParams g{};
-            g.A = q.dG + (c + 1) * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
-            g.B = o.values + c * Bmax * q.C; g.ldb = (long)q.C; g.b_k_contiguous = 0;
+            g.A = q.dG + (c + dg_shift) * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
+            g.B = q.h + (c + h_shift) * Bmax * q.C; g.ldb = (long)q.C; g.b_k_contiguous = 0;
             g.C = q.gWrec; g.ldc = (long)q.C; g.accumulate = c > 0;
             g.M = (int)q.G; g.N = (int)q.C; g.K = (int)B;
             prof_begin(2);
@@ -504,7 +552,7 @@ int Net::lstm_update_derivative_weight(size_t li, size_t B)
     {
         size_t S, chunk;
         split_rows(T * B, q.C, S, chunk);
-        PeepF f{geom, B, Bmax, T, q.c, q.dG};
+        PeepF f{geom, B, Bmax, T, q.c, q.dG, q.reverse ? 1 : 0};
         hipLaunchKernelGGL((column_partial_kernel<3, PeepF>), dim3((unsigned)((q.C + 63) / 64), (unsigned)S), dim3(kBlock), 0, stream, T * B, q.C, chunk, scratch, f);
         MYEA_HIP_TRY(hipGetLastError());
         hipLaunchKernelGGL(lstm_peep_final_kernel, dim3(grid_for(q.C, kBlock)), dim3(kBlock), 0, stream, geom, S, scratch, gradient);
@@ -517,7 +565,7 @@ int Net::lstm_update_derivative_weight(size_t li, size_t B)
         StridedSumF f{B, Bmax, q.G, q.dG};
         hipLaunchKernelGGL((column_partial_kernel<1, StridedSumF>), dim3((unsigned)((q.G + 63) / 64), (unsigned)S), dim3(kBlock), 0, stream, T * B, q.G, chunk, scratch, f);
         MYEA_HIP_TRY(hipGetLastError());
-        hipLaunchKernelGGL(lstm_colsum_final_kernel, dim3(grid_for(q.G, kBlock)), dim3(kBlock), 0, stream, q.G, S, scratch, gradient + l.first_bias_connection_index);
+        hipLaunchKernelGGL(lstm_colsum_final_kernel, dim3(grid_for(q.G, kBlock)), dim3(kBlock), 0, stream, q.G, S, scratch, gradient + q.bias);
         MYEA_HIP_TRY(hipGetLastError());
     }
     return MYEA_OK;
@@ -526,13 +574,17 @@ int Net::lstm_update_derivative_weight(size_t li, size_t B)
 const float *Net::lstm_tensor(size_t li, int kind, size_t *count)
 {
     if (count) *count = 0;
-    LstmLayer *q = L[li].lstm;
+    const bool backward = (kind & MYEA_TENSOR_DIRECTION_BACKWARD) != 0;
+    kind &= ~MYEA_TENSOR_DIRECTION_BACKWARD;
+    LstmLayer *q = backward ? L[li].lstm2 : L[li].lstm;
     if (!q) return nullptr;
     // The device keeps gate tensors packed as rows of [G]; taps are served from small staging copies.
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, rows = T * Bmax;
     const float *src = nullptr;
     size_t width = 0, offset = 0, ld = 0;
     switch (kind) {
+    case MYEA_TENSOR_LSTM_CELL_OUTPUT: if (count) *count = rows * q->C; return q->h;
+    case MYEA_TENSOR_LSTM_DELTA_CELL_OUTPUT: if (count) *count = rows * q->C; return q->dh;
     case MYEA_TENSOR_LSTM_CELL_STATE: if (count) *count = rows * q->C; return q->c;
     case MYEA_TENSOR_LSTM_DELTA_CELL_STATE: if (count) *count = rows * q->C; return q->dc;
     case MYEA_TENSOR_LSTM_CELL_INPUT: src = q->acts; width = q->C; offset = 0; break;

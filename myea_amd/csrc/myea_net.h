@@ -29,7 +29,7 @@ struct DevLayer {
     float *means = nullptr, *variances = nullptr, *means_averages = nullptr, *variances_averages = nullptr;
     float *r_corrections = nullptr, *d_corrections = nullptr;
     float *colscale = nullptr;  // dropout multiplier per (t, unit)
-    LstmLayer *lstm = nullptr;
+    LstmLayer *lstm = nullptr, *lstm2 = nullptr;  // lstm2: the time-reversed direction of a bidirectional layer
 };
 
 constexpr int kProfFamilies = 4;
@@ -88,7 +88,10 @@ struct Net {
     int lstm_forward_layer(size_t li, size_t B);
     int lstm_backward_layer(size_t li, size_t B);       // BPTT inside LSTM layer li
     // delta / weight operands an LSTM consumer gi offers to the layer below: delta [T][Bmax][width], weights [width][fan-in]
-    void lstm_delta_source(size_t gi, const float **delta, size_t *width, const float **weights);
+    void lstm_delta_source(size_t gi, int direction, const float **delta, size_t *width, const float **weights);
+    int lstm_forward_direction(size_t li, LstmLayer &q, size_t B);
+    int lstm_backward_direction(LstmLayer &q, size_t B);
+    int lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t B);
     size_t lstm_scratch_floats() const;
     int lstm_update_derivative_weight(size_t li, size_t B);
     const float *lstm_tensor(size_t li, int kind, size_t *count);

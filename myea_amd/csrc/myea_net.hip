@@ -503,7 +503,8 @@ int Net::backward_into_layer(size_t li, size_t B)
     // what the consumer hands down: delta [T][Bmax][Out] and weights [Out][H]
     const float *delta = on.neuron_errors, *weights = parameters + next.first_connection_index;
     size_t Out = on.H;
-    if (next.type_layer == MYEA_LAYER_LSTM) lstm_delta_source(gi, &delta, &Out, &weights);
+    if (next.type_layer == MYEA_LAYER_LSTM) lstm_delta_source(gi, 0, &delta, &Out, &weights);
+    const bool second_direction = next.type_layer == MYEA_LAYER_LSTM && on.lstm2 != nullptr;
     const bool is_fc = l.type_layer == MYEA_LAYER_FULLY_CONNECTED;
     const bool norm = is_fc && layer_uses_norm(l), before = l.use_layer_normalization_before_activation != 0;
     const bool per_t = T > 1 && (B != Bmax || norm);
@@ -516,6 +517,18 @@ int Net::backward_into_layer(size_t li, size_t B)
         g.M = (int)rows; g.N = (int)H; g.K = (int)Out;
         g.ldc = (long)H;
         g.addend = addend; g.ld_addend = ld_addend;
+        if (second_direction) {  // the time-reversed direction's share dG2 Win2 first; it joins the main contraction as its addend
+            const float *delta2, *weights2;
+            size_t out2;
+            lstm_delta_source(gi, 1, &delta2, &out2, &weights2);
+            GemmParams g2 = g;
+            g2.A = delta2 + roff * out2; g2.lda = (long)out2; g2.B = weights2; g2.K = (int)out2;
+            g2.C = tmp2 + roff * H; g2.epilogue = EPI_NONE; g2.addend = nullptr;
+            prof_begin(1);
+            MYEA_TRY(launch_gemm(stream, g2));
+            prof_end(2.0 * (double)rows * (double)H * (double)out2);
+            g.addend = tmp2 + roff * H; g.ld_addend = (long)H;
+        }
         if (!is_fc) {  // an LSTM layer receives the plain delta of its cell outputs (BPTT follows), a residual layer that of its units
             g.C = o.neuron_errors + roff * H;
             g.epilogue = EPI_NONE;

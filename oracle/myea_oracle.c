@@ -1393,7 +1393,8 @@ const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t 
         size_t cc = T * n->d.batch_size * q->C, kk = T * n->d.batch_size * q->K;
         switch (kind) {
         case MYEA_TENSOR_LSTM_CELL_OUTPUT: p = q->h; c = cc; break;
-        case MYEA_TENSOR_ERRORS: p = q->dh; c = cc; break;
+        case MYEA_TENSOR_ERRORS: p = o->af_errors; c = cc; break;
+        case MYEA_TENSOR_LSTM_DELTA_CELL_OUTPUT: p = q->dh; c = cc; break;
         case MYEA_TENSOR_LSTM_CELL_INPUT: p = q->z; c = cc; break;
         case MYEA_TENSOR_LSTM_CELL_STATE: p = q->c; c = cc; break;
         case MYEA_TENSOR_LSTM_INPUT_GATE: p = q->gi; c = kk; break;

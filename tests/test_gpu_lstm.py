@@ -119,7 +119,7 @@ def test_lstm_error_paths():
         mb.HipNetwork(mb.make_desc([dict(units=3), dict(type="lstm", units=6), dict(units=2, activation="LINEAR")], 2, 3))
     assert e.value.code == mb.E_INVALID and "bias" in str(e.value)
     with pytest.raises(mb.MyeaError) as e:
-        mb.HipNetwork(mb.make_desc([dict(units=3), dict(type="lstm", units=2, bidirectional=True), dict(units=8, activation="LINEAR")], 2, 3))
+        mb.HipNetwork(mb.make_desc([dict(units=3), dict(type="lstm", units=2, normalization="BATCH_NORMALIZATION"), dict(units=8, activation="LINEAR")], 2, 3))
     assert e.value.code == mb.E_UNSUPPORTED
 
 
