@@ -46,24 +46,46 @@ WORKLOADS = {
                                           dropout="BERNOULLI_INVERTED", keep=0.5)] * 8 + [dict(units=100, activation="SOFTMAX")],
         batch=512, head="SOFTMAX", optimizer="GD", loss="CROSS_ENTROPY", data="normal",
         hyper=dict(learning_rate=0.01, learning_momentum=0.9, use_Nesterov=1)),
+    # BASELINE.json configs[4]: bidirectional LSTM with peepholes, input 256, 1024 cells per direction, T = 512, batch 64,
+    # per-step 32-class softmax + cross-entropy, clip at norm 1, AdaBound
+    "bilstm1024_t512_b64_adabound": dict(
+        layers=[dict(units=256), dict(type="lstm", units=1024, bidirectional=True), dict(units=32, activation="SOFTMAX")],
+        batch=64, depth=512, head="SOFTMAX", optimizer="ADABOUND", loss="CROSS_ENTROPY", data="uniform_pm1",
+        hyper=dict(use_clip_gradient=1, clip_gradient=1.0)),
+    # configs[3] as residual blocks: 4 blocks of 2 pre-activation members [BN -> ReLU -> inverted dropout -> FC 2048]
+    "resfc2048x8_bn_relu_dropout_b512_nesterov": dict(
+        layers=[dict(units=2048), dict(units=2048, activation="RELU")]
+               + sum(([dict(type="residual", block_depth=2),
+                       dict(units=2048, activation="RELU", normalization="BATCH_NORMALIZATION"),
+                       dict(units=2048, activation="RELU", normalization="BATCH_NORMALIZATION", dropout="BERNOULLI_INVERTED", keep=0.5)]
+                      for _ in range(4)), [])
+               + [dict(units=100, activation="SOFTMAX")],
+        batch=512, head="SOFTMAX", optimizer="GD", loss="CROSS_ENTROPY", data="normal",
+        hyper=dict(learning_rate=0.01, learning_momentum=0.9, use_Nesterov=1)),
 }
 
 
 def gemm_flops_per_step(layers, batch, depth=1):
     """2*M*N*K of forward, dX (layers 2..) and dW; LSTM layers: 4 gate rows per cell, input contraction at every
     step, recurrent contraction at T-1 steps."""
-    w = [l["units"] * l.get("cells_per_block", 1) for l in layers]
+    w = [l.get("units", 0) * l.get("cells_per_block", 1) for l in layers]
     fwd = dx = 0.0
+    prev = 0   # index of the producer (residual layers own no weights and keep the block's width here: equal widths)
     for i in range(1, len(w)):
+        if layers[i].get("type") == "residual":
+            w[i] = w[prev]
+            continue
         if layers[i].get("type") == "lstm":
+            dirs = 2 if layers[i].get("bidirectional") else 1
             gates = w[i] + 3 * layers[i]["units"]
-            f_in, f_rec = 2.0 * batch * depth * gates * w[i - 1], 2.0 * batch * (depth - 1) * gates * w[i]
+            f_in, f_rec = 2.0 * dirs * batch * depth * gates * w[prev], 2.0 * dirs * batch * (depth - 1) * gates * w[i]
             fwd += f_in + f_rec
             dx += f_rec + (f_in if i >= 2 else 0.0)
         else:
-            f = 2.0 * batch * depth * w[i] * w[i - 1]
+            f = 2.0 * batch * depth * w[i] * w[prev]
             fwd += f
             dx += f if i >= 2 else 0.0
+        prev = i
     return fwd + dx + fwd
 
 
@@ -71,9 +93,14 @@ def make_inputs(np, wl, seed):
     rng = np.random.default_rng(seed)
     T = wl.get("depth", 1)
     B, n_in, n_out = wl["batch"], wl["layers"][0]["units"] * T, wl["layers"][-1]["units"]
-    X = (rng.normal(0, 1, (B, n_in)) if wl["data"] == "normal" else rng.uniform(0, 1, (B, n_in))).astype(np.float32)
+    X = (rng.normal(0, 1, (B, n_in)) if wl["data"] == "normal" else
+         rng.uniform(-1, 1, (B, n_in)) if wl["data"] == "uniform_pm1" else rng.uniform(0, 1, (B, n_in))).astype(np.float32)
     if wl["loss"] == "MSE" and T > 1:
         return X, rng.normal(0, 1, (B, T * n_out)).astype(np.float32)
+    if T > 1:   # one label per time step
+        Y = np.zeros((B, T, n_out), dtype=np.float32)
+        np.put_along_axis(Y, rng.integers(0, n_out, (B, T))[..., None], 1.0, axis=2)
+        return X, Y.reshape(B, T * n_out)
     Y = np.zeros((B, n_out), dtype=np.float32)
     Y[np.arange(B), rng.integers(0, n_out, B)] = 1.0
     return X, Y
@@ -193,7 +220,8 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": args.workload, "batch": B, "sequence_length": wl.get("depth", 1),
-                   "layers": [("lstm%d" if l.get("type") == "lstm" else "fc%d") % l["units"] for l in wl["layers"]],
+                   "layers": ["res%d" % l["block_depth"] if l.get("type") == "residual" else
+                              ("bilstm%d" if l.get("bidirectional") else "lstm%d" if l.get("type") == "lstm" else "fc%d") % l["units"] for l in wl["layers"]],
                    "optimizer": wl["optimizer"], "parameters": int(desc.total_parameters),
                    "gemm_flops_per_step": gemm_flops_per_step(wl["layers"], B, wl.get("depth", 1))},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
