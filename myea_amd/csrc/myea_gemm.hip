@@ -9,11 +9,17 @@
 //
 // Tiling: a workgroup of 256 lanes (4 wavefronts, 2 x 2) owns a BM x BN tile of C; each wavefront owns
 // (BM/2) x (BN/2) as TM x TN accumulators of v_mfma_f32_32x32x2_f32 (16 VGPRs each).  The K loop moves
-// BK = 32 columns per step: global -> registers (128-bit loads, issued before the MFMA block of the
-// current step) -> LDS (double buffered, one barrier per step).  Operands keep their global
-// orientation in LDS, so no transposes are needed:
+// BK = 32 columns per step through LDS stages with one barrier per step; the fragments of the next 8 k's are read from
+// LDS while the MFMAs of the current 8 issue.  General path (any alignment): global -> registers (guarded scalar loads,
+// issued before the MFMA block of the current step) -> LDS, two stages.  Operands keep their global orientation in LDS,
+// so no transposes are needed:
 //   k-contiguous operand : LDS [rows][BK + 4]   fragment = one ds_read_b128 per 4 MFMA k-steps
 //   mn-contiguous operand: LDS [BK][rows + 8]   fragment = conflict-free ds_read_b32 per k
+// When the operands are 16-byte aligned the tiles do not pass through registers at all: global_load_lds_dwordx4 writes
+// 1 KiB per wavefront instruction straight into LDS (lane l lands at base + 16 l), which rules out per-row padding, so
+//   k-contiguous operand : LDS [rows][BK], the 16-byte chunk c of row r stored at chunk c ^ ((r >> 1) & 7)
+//   mn-contiguous operand: LDS [BK][rows] in 1 KiB pieces, each padded so that k and k + 4 sit 32 banks apart
+// both again conflict-free for the fragment reads.
 // Inside a group of 8 k's, MFMA step j of lane-half h consumes k = 4h + j for BOTH operands, which is
 // what makes the two layouts interchangeable.
 //
@@ -43,15 +49,22 @@ struct TileShape {
     static_assert(kVec % kThreads == 0, "tile must be a multiple of the workgroup");
 };
 
-// Global -> register -> LDS mover for one operand tile (ROWS x BK).
-template <int ROWS, bool KC, bool VEC>
+// Global -> register -> LDS mover for one operand tile (ROWS x BK): guarded scalar loads, any alignment (the general,
+// slower path; aligned operands take the direct path below).
+template <int ROWS, bool KC>
 struct TileMover {
     using S = TileShape<ROWS, KC>;
     f32x4 reg[S::kPasses];
+    const float *base; long ld; int row0, extent;
 
-    // base: operand origin; ld: leading dimension; row0: first row (m or n) of the tile;
-    // extent: M or N; k0: first k of the step; K: total depth.
-    __device__ __forceinline__ void load(const float *__restrict__ base, long ld, int row0, int extent, int k0, int K)
+    // base: operand origin; ld: leading dimension; row0: first row (m or n) of the tile; extent: M or N
+    __device__ __forceinline__ void init(const float *__restrict__ base_, long ld_, int row0_, int extent_, int)
+    {
+        base = base_; ld = ld_; row0 = row0_; extent = extent_;
+    }
+
+    // k0: first k of the step; K: end of the k range
+    __device__ __forceinline__ void load(int k0, int K)
     {
         const int t = threadIdx.x;
 #pragma unroll
@@ -72,18 +85,14 @@ struct TileMover {
             f32x4 v = {0.f, 0.f, 0.f, 0.f};
             if (KC) {
                 const float *src = base + (long)gr * ld + gk;
-                if (VEC) {
-                    if (gr < extent && gk < K) v = *reinterpret_cast<const f32x4 *>(src);
-                } else if (gr < extent) {
+                if (gr < extent) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         if (gk + e < K) v[e] = src[e];
                 }
             } else {
                 const float *src = base + (long)gk * ld + gr;
-                if (VEC) {
-                    if (gk < K && gr < extent) v = *reinterpret_cast<const f32x4 *>(src);
-                } else if (gk < K) {
+                if (gk < K) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         if (gr + e < extent) v[e] = src[e];
@@ -92,6 +101,11 @@ struct TileMover {
             reg[p] = v;
         }
     }
+
+    __device__ __forceinline__ void fill(float *, int k0, int K) { load(k0, K); }
+    __device__ __forceinline__ void commit(float *tile) const { store(tile); }
+    template <int N>
+    static __device__ __forceinline__ void wait() {}
 
     __device__ __forceinline__ void store(float *lds) const
     {
@@ -129,6 +143,108 @@ __device__ __forceinline__ f32x4 read_fragment(const float *lds, int tile_row, i
     }
 }
 
+// ---- direct global -> LDS path (16-byte aligned operands) --------------------------------------------------------
+template <int ROWS, bool KC>
+struct DirectShape {
+    static constexpr int kPieces = ROWS * kBK * 4 / 1024;          // wavefront-wide 1 KiB pieces per tile
+    static constexpr int kPerWave = kPieces / 4;
+    static constexpr int kRowsPerPiece = KC ? 8 : 256 / ROWS;      // tile rows (KC) or k rows (MN) per piece
+    static constexpr int kPiecePad = KC ? 0 : (ROWS == 128 ? 16 : 32);
+    static constexpr int kPieceFloats = 256 + kPiecePad;
+    static constexpr int kFloats = kPieces * kPieceFloats;
+    static_assert(ROWS == 64 || ROWS == 128, "tile rows");
+};
+
+template <int ROWS, bool KC>
+struct DirectMover {
+    using S = DirectShape<ROWS, KC>;
+    const float *ptr[S::kPerWave];
+    int kofs[S::kPerWave];      // k of the lane's 16 bytes inside the K step (for the predicated last step)
+    long step;
+
+    __device__ __forceinline__ void init(const float *__restrict__ base, long ld, int row0, int extent, int k0)
+    {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+        for (int q = 0; q < S::kPerWave; ++q) {
+            const int piece = wave * S::kPerWave + q;
+            if (KC) {
+                const int row = piece * 8 + (lane >> 3);
+                const int c = (lane & 7) ^ ((row >> 1) & 7);
+                ptr[q] = base + (long)min(row0 + row, extent - 1) * ld + k0 + c * 4;
+                kofs[q] = c * 4;
+            } else {
+                const int k = piece * S::kRowsPerPiece + (lane * 4) / ROWS, col = (lane * 4) % ROWS;
+                ptr[q] = base + (long)(k0 + k) * ld + min(row0 + col, extent - 4);
+                kofs[q] = k;
+            }
+        }
+        step = KC ? (long)kBK : (long)kBK * ld;
+    }
+
+    // Starts filling `tile` (LDS) with the K step that begins at k0; K is the end of the k range.
+    __device__ __forceinline__ void fill(float *tile, int k0, int K)
+    {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        if (k0 + kBK <= K) {
+#pragma unroll
+            for (int q = 0; q < S::kPerWave; ++q) {
+                float *dst = tile + (wave * S::kPerWave + q) * S::kPieceFloats;   // wave-uniform
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)ptr[q],
+                                                 (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+                ptr[q] += step;
+            }
+        } else {   // last, partial step: through registers, zero filled along k
+#pragma unroll
+            for (int q = 0; q < S::kPerWave; ++q) {
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (k0 + kofs[q] < K) v = *reinterpret_cast<const f32x4 *>(ptr[q]);
+                *reinterpret_cast<f32x4 *>(tile + (wave * S::kPerWave + q) * S::kPieceFloats + lane * 4) = v;
+            }
+        }
+    }
+    __device__ __forceinline__ void commit(float *) const {}
+    // the direct loads count on vmcnt; they must have landed before the barrier that publishes the stage
+    // n = number of younger loads that may stay in flight (those of the step after next)
+    template <int N>
+    static __device__ __forceinline__ void wait() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }   // vmcnt(N)
+};
+
+template <int ROWS, bool KC>
+__device__ __forceinline__ f32x4 read_fragment_direct(const float *lds, int tile_row, int kgroup, int lane32, int half)
+{
+    using S = DirectShape<ROWS, KC>;
+    if (KC) {
+        const int row = tile_row + lane32;
+        const int slot = (kgroup * 2 + half) ^ ((row >> 1) & 7);
+        return *reinterpret_cast<const f32x4 *>(lds + row * kBK + slot * 4);
+    } else {
+        f32x4 v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = kgroup * 8 + half * 4 + j;
+            v[j] = lds[(k / S::kRowsPerPiece) * S::kPieceFloats + (k % S::kRowsPerPiece) * ROWS + tile_row + lane32];
+        }
+        return v;
+    }
+}
+
+// data path of one operand: how a tile gets into LDS and how fragments come out of it
+template <int ROWS, bool KC, bool VEC>
+struct OperandPath {
+    using Mover = TileMover<ROWS, KC>;
+    static constexpr int kFloats = TileShape<ROWS, KC>::kFloats;
+    static constexpr int kLoads = 0;
+    static __device__ __forceinline__ f32x4 frag(const float *lds, int tile_row, int g, int lane32, int half) { return read_fragment<ROWS, KC>(lds, tile_row, g, lane32, half); }
+};
+template <int ROWS, bool KC>
+struct OperandPath<ROWS, KC, true> {
+    using Mover = DirectMover<ROWS, KC>;
+    static constexpr int kFloats = DirectShape<ROWS, KC>::kFloats;
+    static constexpr int kLoads = DirectShape<ROWS, KC>::kPerWave;   // vmcnt events per wavefront per K step
+    static __device__ __forceinline__ f32x4 frag(const float *lds, int tile_row, int g, int lane32, int half) { return read_fragment_direct<ROWS, KC>(lds, tile_row, g, lane32, half); }
+};
+
 struct GemmDev {
     const float *A, *B;
     float *C;
@@ -152,10 +268,10 @@ template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
 __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
 {
     constexpr int TM = BM / 64, TN = BN / 64;  // 32x32 accumulators per wavefront along m / n
-    using SA = TileShape<BM, A_KC>;
-    using SB = TileShape<BN, B_KC>;
+    using PA = OperandPath<BM, A_KC, VEC>;
+    using PB = OperandPath<BN, B_KC, VEC>;
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    constexpr int kStage = SA::kFloats + SB::kFloats;  // one LDS stage = A tile then B tile
+    constexpr int kStage = PA::kFloats + PB::kFloats;  // one LDS stage = A tile then B tile
 
     // Workgroup -> tile.  Consecutive workgroup ids land on different XCDs (8 of them, each with its own
     // L2), so give every XCD a contiguous run of tile ids, and walk tiles in bands of 8 m-tiles so that a
@@ -185,44 +301,74 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    TileMover<BM, A_KC, VEC> moveA;
-    TileMover<BN, B_KC, VEC> moveB;
+    typename PA::Mover moveA;
+    typename PB::Mover moveB;
     const int nk = (k_end - k_begin + kBK - 1) / kBK;
+    // LDS stages.  Register path: 2 (the next step's tile waits in registers).  Direct path: 3 - the loads of step
+    // kt + 2 are issued while step kt computes, so a load has two steps of compute to hide behind and only the loads of
+    // step kt + 1 must have landed (vmcnt(loads of one step)) at the barrier.
+    constexpr int NS = (VEC && BM * BN < 128 * 128) ? 3 : 2;   // 128 x 128 keeps two stages so that two workgroups fit a CU
+    constexpr int kInFlight = PA::kLoads + PB::kLoads;
 
-    moveA.load(p.A, p.lda, m0, p.M, k_begin, k_end);
-    moveB.load(p.B, p.ldb, n0, p.N, k_begin, k_end);
-    moveA.store(smem);
-    moveB.store(smem + SA::kFloats);
+    moveA.init(p.A, p.lda, m0, p.M, k_begin);
+    moveB.init(p.B, p.ldb, n0, p.N, k_begin);
+    moveA.fill(smem, k_begin, k_end);
+    moveB.fill(smem + PA::kFloats, k_begin, k_end);
+    moveA.commit(smem);
+    moveB.commit(smem + PA::kFloats);
+    if (NS == 3 && nk > 1) {
+        moveA.fill(smem + kStage, k_begin + kBK, k_end);
+        moveB.fill(smem + kStage + PA::kFloats, k_begin + kBK, k_end);
+        PA::Mover::template wait<kInFlight>();
+    } else {
+        PA::Mover::template wait<0>();
+    }
     __syncthreads();
 
+    int cur = 0;   // stage holding step kt
     for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < nk;
-        if (more) {
-            moveA.load(p.A, p.lda, m0, p.M, k_begin + (kt + 1) * kBK, k_end);
-            moveB.load(p.B, p.ldb, n0, p.N, k_begin + (kt + 1) * kBK, k_end);
+        const int ahead = NS - 1;                       // how many steps ahead the fill runs
+        const bool more = kt + ahead < nk;
+        int nxt = cur + ahead; if (nxt >= NS) nxt -= NS;
+        float *next = smem + nxt * kStage;
+        if (more) {   // that stage was last read before the previous barrier
+            moveA.fill(next, k_begin + (kt + ahead) * kBK, k_end);
+            moveB.fill(next + PA::kFloats, k_begin + (kt + ahead) * kBK, k_end);
         }
-        const float *la = smem + cur * kStage, *lb = la + SA::kFloats;
+        const float *la = smem + cur * kStage, *lb = la + PA::kFloats;
+        // Fragments are double buffered in registers: the LDS reads of group g + 1 are in flight while the MFMAs of
+        // group g issue, so that a wavefront does not sit out the LDS latency between groups.
+        f32x4 fa[2][TM], fb[2][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[0][i] = PA::frag(la, wave_m + i * 32, 0, lane32, half);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[0][j] = PB::frag(lb, wave_n + j * 32, 0, lane32, half);
 #pragma unroll
         for (int g = 0; g < kBK / 8; ++g) {
-            f32x4 fa[TM], fb[TN];
+            const int cb = g & 1, nb = cb ^ 1;
+            if (g + 1 < kBK / 8) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = read_fragment<BM, A_KC>(la, wave_m + i * 32, g, lane32, half);
+                for (int i = 0; i < TM; ++i) fa[nb][i] = PA::frag(la, wave_m + i * 32, g + 1, lane32, half);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fb[j] = read_fragment<BN, B_KC>(lb, wave_n + j * 32, g, lane32, half);
+                for (int j = 0; j < TN; ++j) fb[nb][j] = PB::frag(lb, wave_n + j * 32, g + 1, lane32, half);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of this group's MFMAs (the scheduler sinks it otherwise)
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][i][s], fb[cb][j][s], acc[i][j], 0, 0, 0);
         }
         if (more) {
-            moveA.store(smem + (cur ^ 1) * kStage);
-            moveB.store(smem + (cur ^ 1) * kStage + SA::kFloats);
+            moveA.commit(next);
+            moveB.commit(next + PA::kFloats);
         }
+        if (NS == 3 && more) PA::Mover::template wait<kInFlight>();
+        else PA::Mover::template wait<0>();
         __syncthreads();
+        cur = cur + 1 == NS ? 0 : cur + 1;
     }
 
     // Epilogue.  A lane owns one column of each accumulator, so per-column operands are read once.
@@ -262,9 +408,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
 template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
 int launch_one(hipStream_t stream, GemmDev d)
 {
-    using SA = TileShape<BM, A_KC>;
-    using SB = TileShape<BN, B_KC>;
-    constexpr size_t lds_bytes = 2 * (SA::kFloats + SB::kFloats) * sizeof(float);
+    constexpr size_t lds_bytes = ((VEC && BM * BN < 128 * 128) ? 3 : 2) * (OperandPath<BM, A_KC, VEC>::kFloats + OperandPath<BN, B_KC, VEC>::kFloats) * sizeof(float);
     auto kern = gemm_f32_mfma_kernel<BM, BN, A_KC, B_KC, VEC>;
     static bool attr_done = false;  // per instantiation
     if (!attr_done) {
