@@ -266,6 +266,14 @@ int myea_hip_upload_optimizer_state(myea_hip_net *net, int kind, const float *ho
 int myea_hip_download_optimizer_state(myea_hip_net *net, int kind, float *host, size_t count);
 /* `ptr_array_units_mask_dropout_bernoulli` (bool[(sum AF units) * T]), written by the caller between
  * steps exactly as the reference lets callers write its public mask buffer. */
+/* Per-unit activation functions and steepnesses of one fully-connected layer: AF_unit::ptr_type_activation_function /
+ * ptr_activation_steepness are per-unit arrays in the reference (Data.hpp, struct AF_unit; read per unit by
+ * Forward_Pass__FC_AF and Backward_Pass__FC__DF, Neural_Network__Forward_Pass__OpenMP.cpp:4839-4868,
+ * Neural_Network__Backward_Pass__OpenMP.cpp:1225-1263); its setters fill them uniformly, direct writes may not.
+ * `count` = the layer's activation units (its width; inside a residual block: its fan-in).  Either array may be NULL
+ * (keep the layer-wide value).  Softmax stays a layer-wide choice.  Call with both NULL to return to the layer-wide values. */
+int myea_hip_set_unit_activations(myea_hip_net *net, size_t layer_index, const uint32_t *host_types, const float *host_steepness, size_t count);
+
 int myea_hip_upload_masks(myea_hip_net *net, const uint8_t *host_masks, size_t count);
 /* Clear_Training_Arrays (Train.cpp:93-126) + Clear_Optimizer (Train.cpp:128-263): zero the gradient
  * vector and all optimizer state, optimizer_time_step = 0. */

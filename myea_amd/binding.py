@@ -86,7 +86,7 @@ ABI_SYMBOLS = [
     "myea_hyper_default", "myea_net_desc_layout", "myea_net_desc_previous_layer", "myea_net_desc_number_outputs", "myea_hip_create", "myea_hip_destroy", "myea_hip_set_stream",
     "myea_hip_synchronize", "myea_hip_last_error", "myea_hip_set_hyper", "myea_hip_get_hyper",
     "myea_hip_set_state_propagation", "myea_hip_upload_parameters", "myea_hip_download_parameters",
-    "myea_hip_upload_optimizer_state", "myea_hip_download_optimizer_state", "myea_hip_upload_masks",
+    "myea_hip_upload_optimizer_state", "myea_hip_download_optimizer_state", "myea_hip_upload_masks", "myea_hip_set_unit_activations",
     "myea_hip_clear_training_arrays", "myea_hip_forward_pass", "myea_hip_compute_error", "myea_hip_backward_pass",
     "myea_hip_update_derivative_weight", "myea_hip_update_parameter", "myea_hip_reset_loss", "myea_hip_get_loss",
     "myea_hip_download_gradient", "myea_hip_upload_gradient", "myea_hip_download_tensor",
@@ -127,6 +127,7 @@ def load_library(path=LIB_PATH):
     lib.myea_hip_upload_optimizer_state.argtypes = [vp, i32, vp, sz]
     lib.myea_hip_download_optimizer_state.argtypes = [vp, i32, vp, sz]
     lib.myea_hip_upload_masks.argtypes = [vp, vp, sz]
+    lib.myea_hip_set_unit_activations.argtypes = [vp, sz, vp, vp, sz]
     lib.myea_hip_clear_training_arrays.argtypes = [vp]
     lib.myea_hip_forward_pass.argtypes = [vp, sz, vp, i32]
     lib.myea_hip_compute_error.argtypes = [vp, sz, vp, i32]
@@ -259,6 +260,12 @@ class HipNetwork:
         out = np.empty(self.desc.total_parameters, dtype=np.float32)
         self._check(self.lib.myea_hip_download_optimizer_state(self.handle, kind, _ptr(out), out.size))
         return out
+
+    def set_unit_activations(self, layer, types=None, steepness=None):
+        t = None if types is None else np.ascontiguousarray(types, dtype=np.uint32)
+        st = None if steepness is None else np.ascontiguousarray(steepness, dtype=np.float32)
+        n = len(t) if t is not None else (len(st) if st is not None else 0)
+        self._check(self.lib.myea_hip_set_unit_activations(self.handle, layer, _ptr(t), _ptr(st), n))
 
     def upload_masks(self, m):
         m = np.ascontiguousarray(m, dtype=np.uint8)

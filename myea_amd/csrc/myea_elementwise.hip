@@ -24,10 +24,10 @@ __global__ __launch_bounds__(kBlock) void fill_kernel(float *p, size_t n, float 
 
 // Forward_Pass__FC_AF (NN/Neural_Network__Forward_Pass__OpenMP.cpp:4839-4868) fused with the Bernoulli
 // appliers (:4907-4990) through a per-column multiplier.
-__global__ __launch_bounds__(kBlock) void activation_kernel(int act, size_t n, size_t H, const float *x, float *y, const float *colscale)
+__global__ __launch_bounds__(kBlock) void activation_kernel(int act, const int *unit_act, size_t n, size_t H, const float *x, float *y, const float *colscale)
 {
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-        float v = af_fire(act, x[i]);
+        float v = af_fire(unit_act ? unit_act[i % H] : act, x[i]);
         if (colscale) v *= colscale[i % H];
         y[i] = v;
     }
@@ -44,10 +44,11 @@ __global__ __launch_bounds__(kBlock) void mask_to_scale_kernel(size_t n, const u
 }
 
 // Backward_Pass__FC__DF (NN/Neural_Network__Backward_Pass__OpenMP.cpp:1225-1263)
-__global__ __launch_bounds__(kBlock) void activation_derive_kernel(int act, float steep, size_t n, const float *pre, const float *val, const float *dy, float *dx)
+__global__ __launch_bounds__(kBlock) void activation_derive_kernel(int act, float steep, const int *unit_act, const float *unit_steep, size_t H, size_t n,
+                                                                   const float *pre, const float *val, const float *dy, float *dx)
 {
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
-        dx[i] = dy[i] * af_derive(act, pre[i], steep, val[i]);
+        dx[i] = dy[i] * af_derive(unit_act ? unit_act[i % H] : act, pre[i], unit_steep ? unit_steep[i % H] : steep, val[i]);
 }
 
 // Forward_Pass__FC_AF__Softmax (:4870-4905): one wavefront per row.
@@ -269,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void compute_error_kernel(ErrorParams p)
             default: break;
             }
             const float q = p.rnn_pre_quirk ? pre[0] : pre[j];
-            err[j] = af_derive(p.act, q, p.steep, yo) * diff;
+            err[j] = af_derive(p.unit_act ? p.unit_act[j] : p.act, q, p.unit_steep ? p.unit_steep[j] : p.steep, yo) * diff;
         }
     }
     loss = wave_sum(loss); cnt = wave_sum(cnt); acc = wave_sum(acc); bits = wave_sum(bits);
@@ -417,11 +418,11 @@ int launch_fill(hipStream_t s, float *p, size_t n, float v)
     return MYEA_OK;
 }
 
-int launch_activation(hipStream_t s, int act, size_t rows, size_t H, const float *x, float *y, const float *colscale)
+int launch_activation(hipStream_t s, int act, size_t rows, size_t H, const float *x, float *y, const float *colscale, const int *unit_act)
 {
     const size_t n = rows * H;
     if (n == 0) return MYEA_OK;
-    hipLaunchKernelGGL(activation_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, act, n, H, x, y, colscale);
+    hipLaunchKernelGGL(activation_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, act, unit_act, n, H, x, y, colscale);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
@@ -434,10 +435,12 @@ int launch_softmax(hipStream_t s, size_t rows, size_t H, const float *x, float *
     return MYEA_OK;
 }
 
-int launch_activation_derive(hipStream_t s, int act, float steep, size_t n, const float *pre, const float *val, const float *dy, float *dx)
+int launch_activation_derive(hipStream_t s, int act, float steep, size_t n, const float *pre, const float *val, const float *dy, float *dx,
+                             const int *unit_act, const float *unit_steep, size_t H)
 {
     if (n == 0) return MYEA_OK;
-    hipLaunchKernelGGL(activation_derive_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, act, steep, n, pre, val, dy, dx);
+    if ((unit_act || unit_steep) && H == 0) { set_last_error("activation derive: per-unit arrays need the row width"); return MYEA_E_INVALID; }
+    hipLaunchKernelGGL(activation_derive_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, act, steep, unit_act, unit_steep, H ? H : 1, n, pre, val, dy, dx);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

@@ -65,11 +65,13 @@ bool gemm_can_fuse_activation(int act);
 int launch_padded_add(hipStream_t s, size_t rows, size_t wo, const float *a, size_t wa, long sa,
                       const float *b, size_t wb, long sb, float *out);
 // y = AF(x) * colscale[j]  (colscale may be null); x and y may alias.
-int launch_activation(hipStream_t s, int act, size_t rows, size_t H, const float *x, float *y, const float *colscale);
+int launch_activation(hipStream_t s, int act, size_t rows, size_t H, const float *x, float *y, const float *colscale, const int *unit_act = nullptr);
 // row softmax (max-subtracted) then * colscale
 int launch_softmax(hipStream_t s, size_t rows, size_t H, const float *x, float *y, const float *colscale);
 // dx = dy * AF'(pre, steep, val)
-int launch_activation_derive(hipStream_t s, int act, float steep, size_t n, const float *pre, const float *val, const float *dy, float *dx);
+// unit_act / unit_steep: optional per-column arrays [H] (element i belongs to column i % H)
+int launch_activation_derive(hipStream_t s, int act, float steep, size_t n, const float *pre, const float *val, const float *dy, float *dx,
+                             const int *unit_act = nullptr, const float *unit_steep = nullptr, size_t H = 0);
 // y[r][j] *= colscale[j]
 int launch_colscale(hipStream_t s, size_t rows, size_t H, float *y, const float *colscale);
 // colscale[j] = mask[j] ? on : 0   (training) over n entries
@@ -108,6 +110,8 @@ struct ErrorParams {
     float *errors;               // [T][Bmax][H]
     int act;
     float steep;
+    const int *unit_act;       // optional per-unit activation types [H]
+    const float *unit_steep;   // optional per-unit steepnesses [H]
     int loss, accuracy;
     float accuracy_variance, bit_fail_limit;
     size_t first_t;              // number_time_delays

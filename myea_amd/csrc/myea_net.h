@@ -29,6 +29,8 @@ struct DevLayer {
     float *means = nullptr, *variances = nullptr, *means_averages = nullptr, *variances_averages = nullptr;
     float *r_corrections = nullptr, *d_corrections = nullptr;
     float *colscale = nullptr;  // dropout multiplier per (t, unit)
+    int *unit_act = nullptr;    // per-unit activation types [AH], null = layer-wide
+    float *unit_steep = nullptr;  // per-unit steepnesses [AH], null = layer-wide
     LstmLayer *lstm = nullptr, *lstm2 = nullptr;  // lstm2: the time-reversed direction of a bidirectional layer
 };
 
@@ -80,6 +82,7 @@ struct Net {
     int backward_pass(size_t B);
     int update_derivative_weight(size_t B, size_t first, size_t end);
     int update_parameter(size_t B, size_t training_size);
+    int set_unit_activations(size_t li, const uint32_t *types, const float *steep, size_t count);
 
     // LSTM-with-peephole layers (myea_lstm.hip)
     int lstm_create_layer(size_t li);

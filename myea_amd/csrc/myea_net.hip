@@ -242,7 +242,7 @@ Net::~Net()
     for (int k = 0; k < 4; ++k) fr(opt[k]);
     fr(masks);
     for (DevLayer &o : L) {
-        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale);
+        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep);
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
@@ -301,7 +301,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
         g.epilogue = EPI_FC_FORWARD;
         g.bias = layer_uses_bias(l) ? parameters + l.first_bias_connection_index : nullptr;
         g.act = (int)l.type_activation_function;
-        const bool fuse_af = !softmax && !(norm && before) && gemm_can_fuse_activation((int)l.type_activation_function);
+        const bool fuse_af = !softmax && !(norm && before) && !o.unit_act && gemm_can_fuse_activation((int)l.type_activation_function);
         g.aux_out = fuse_af ? o.values + roff * H : nullptr;
         g.colscale = (fuse_af && !norm) ? cs : nullptr;
         prof_begin(0);
@@ -314,7 +314,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
             cur = o.normalizes + roff * H;
         }
         if (softmax) MYEA_TRY(launch_softmax(stream, rows, H, cur, o.values + roff * H, norm ? nullptr : cs));
-        else if (!fuse_af) MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, rows, H, cur, o.values + roff * H, cs));
+        else if (!fuse_af) MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, rows, H, cur, o.values + roff * H, cs, o.unit_act));
         if (norm && !before) {
             MYEA_TRY(bn_forward(li, c, rows, o.values + roff * H, training));
             if (cs) MYEA_TRY(launch_colscale(stream, rows, H, o.normalizes + roff * H, cs));
@@ -402,7 +402,7 @@ int Net::forward_residual_block(size_t ri, size_t B)
             if (!values_ready) {
                 bool drop = false;
                 MYEA_TRY(refresh_colscale(m, &drop));
-                MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, B, In, cur, o.values, drop ? o.colscale : nullptr));
+                MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, B, In, cur, o.values, drop ? o.colscale : nullptr, o.unit_act));
             }
             cur = o.values;
         }
@@ -416,7 +416,7 @@ int Net::forward_residual_block(size_t ri, size_t B)
         values_ready = false;
         if (m < last) {
             const myea_layer_desc &nx = d.layers[m + 1];
-            if (!layer_uses_norm(nx) && gemm_can_fuse_activation((int)nx.type_activation_function)) {
+            if (!layer_uses_norm(nx) && !L[m + 1].unit_act && gemm_can_fuse_activation((int)nx.type_activation_function)) {
                 bool drop = false;
                 MYEA_TRY(refresh_colscale(m + 1, &drop));
                 g.act = (int)nx.type_activation_function;
@@ -462,6 +462,7 @@ int Net::compute_error(size_t B, const float *desired, int on_device)
     p.desired = dsrc;
     p.errors = o.neuron_errors;  // AF errors are copied to the neuron errors unchanged (:136-139)
     p.act = (int)l.type_activation_function; p.steep = l.activation_steepness;
+    p.unit_act = o.unit_act; p.unit_steep = o.unit_steep;
     p.loss = (int)h.type_loss_function; p.accuracy = (int)h.type_accuracy_function;
     p.accuracy_variance = h.accuracy_variance; p.bit_fail_limit = h.bit_fail_limit;
     p.first_t = T > 1 ? h.number_time_delays : 0;
@@ -539,7 +540,7 @@ int Net::backward_into_layer(size_t li, size_t B)
             continue;
         }
         g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
-        const bool fuse = have_gemm && gemm_can_fuse_activation(g.act);
+        const bool fuse = have_gemm && !o.unit_act && !o.unit_steep && gemm_can_fuse_activation(g.act);
         if (!norm) {
             g.C = (fuse ? o.neuron_errors : tmp1) + roff * H;
             g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.summations + roff * H; g.val = o.values + roff * H;
@@ -558,14 +559,15 @@ int Net::backward_into_layer(size_t li, size_t B)
             MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors, shortcut->H, crop, identity, H, 0, g.C));
         }
         if (!fuse && !(norm && !before)) {  // act' as its own kernel (Backward_Pass__FC__DF)
-            MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, rows * H, g.pre, g.val, tmp1 + roff * H, (norm ? tmp1 : o.neuron_errors) + roff * H));
+            MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, rows * H, g.pre, g.val, tmp1 + roff * H, (norm ? tmp1 : o.neuron_errors) + roff * H,
+                                              o.unit_act, o.unit_steep, H));
         }
         if (norm && before) {
             MYEA_TRY(bn_backward(li, c, rows, o.summations + roff * H, tmp1 + roff * H, o.neuron_errors + roff * H));
         } else if (norm) {
             MYEA_TRY(bn_backward(li, c, rows, o.values + roff * H, tmp1 + roff * H, tmp2 + roff * H));
             MYEA_TRY(launch_activation_derive(stream, (int)l.type_activation_function, l.activation_steepness, rows * H,
-                                              o.summations + roff * H, o.values + roff * H, tmp2 + roff * H, o.neuron_errors + roff * H));
+                                              o.summations + roff * H, o.values + roff * H, tmp2 + roff * H, o.neuron_errors + roff * H, o.unit_act, o.unit_steep, H));
         }
     }
     return MYEA_OK;
@@ -609,13 +611,13 @@ int Net::backward_residual_block(size_t ri, size_t B)
             g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
             g.pre = norm ? o.normalizes : prev_out;   // Layer::ptr_array_pre_activation_functions
             g.val = o.values;
-            if (gemm_can_fuse_activation(g.act)) g.epilogue = EPI_FC_DERIVE;
+            if (!o.unit_act && !o.unit_steep && gemm_can_fuse_activation(g.act)) g.epilogue = EPI_FC_DERIVE;
             else derive_pending = true;
         }
         prof_begin(1);
         MYEA_TRY(launch_gemm(stream, g));
         prof_end(2.0 * (double)B * (double)H * (double)In);
-        if (derive_pending) MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, B * In, g.pre, g.val, g.C, g.C));
+        if (derive_pending) MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, B * In, g.pre, g.val, g.C, g.C, o.unit_act, o.unit_steep, In));
         if (norm) MYEA_TRY(bn_backward(m, 0, B, prev_out, tmp1, dst));
     }
     return MYEA_OK;
@@ -686,6 +688,33 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
             prof_end(2.0 * (double)rows * (double)H * (double)In);
             if (layer_uses_bias(l)) MYEA_TRY(launch_column_sum(stream, rows, H, o.neuron_errors + roff * H, gradient + l.first_bias_connection_index, 1, scratch));
         }
+    }
+    return MYEA_OK;
+}
+
+// Per-unit activation arrays (struct AF_unit: ptr_type_activation_function / ptr_activation_steepness).  With them the
+// activation can no longer ride in a contraction's epilogue; it runs as its own kernel reading the arrays per column.
+int Net::set_unit_activations(size_t li, const uint32_t *types, const float *steep, size_t count)
+{
+    if (li == 0 || li >= d.n_layers || d.layers[li].type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("set_unit_activations: layer %zu is not a fully-connected hidden / output layer", li); return MYEA_E_INVALID; }
+    DevLayer &o = L[li];
+    if (d.layers[li].type_activation_function == MYEA_AF_SOFTMAX) { set_last_error("set_unit_activations: layer %zu is a softmax layer", li); return MYEA_E_INVALID; }
+    if ((types || steep) && count != o.AH) { set_last_error("set_unit_activations: layer %zu has %zu activation units, got %zu", li, o.AH, count); return MYEA_E_INVALID; }
+    if (types)
+        for (size_t j = 0; j < count; ++j)
+            if (types[j] == MYEA_AF_NONE || types[j] >= MYEA_AF_LENGTH || types[j] == MYEA_AF_SOFTMAX) { set_last_error("set_unit_activations: unit %zu: activation %u invalid", j, types[j]); return MYEA_E_INVALID; }
+    MYEA_HIP_TRY(hipStreamSynchronize(stream));
+    if (o.unit_act) { (void)hipFree(o.unit_act); o.unit_act = nullptr; }
+    if (o.unit_steep) { (void)hipFree(o.unit_steep); o.unit_steep = nullptr; }
+    if (types) {
+        void *q = nullptr;
+        MYEA_HIP_TRY(hipMalloc(&q, count * sizeof(int)));
+        o.unit_act = static_cast<int *>(q);
+        MYEA_HIP_TRY(hipMemcpy(o.unit_act, types, count * sizeof(int), hipMemcpyHostToDevice));
+    }
+    if (steep) {
+        MYEA_TRY(dev_alloc(&o.unit_steep, count));
+        MYEA_HIP_TRY(hipMemcpy(o.unit_steep, steep, count * sizeof(float), hipMemcpyHostToDevice));
     }
     return MYEA_OK;
 }
@@ -842,6 +871,12 @@ int myea_hip_download_optimizer_state(myea_hip_net *n, int kind, float *p, size_
     if (kind < 0 || kind > 3 || !p) { myea::set_last_error("download_optimizer_state: bad kind %d or null", kind); return MYEA_E_INVALID; }
     return copy_vec(n, n->net.opt[kind], p, nullptr, c, "download_optimizer_state");
 }
+int myea_hip_set_unit_activations(myea_hip_net *n, size_t li, const uint32_t *types, const float *steep, size_t count)
+{
+    NET_OR_FAIL(n);
+    return n->net.set_unit_activations(li, types, steep, count);
+}
+
 int myea_hip_upload_masks(myea_hip_net *n, const uint8_t *m, size_t c)
 {
     NET_OR_FAIL(n);

@@ -60,7 +60,9 @@ typedef struct olayer {
     /* [T][NH] */
     float *means, *variances, *means_averages, *variances_averages, *r_corrections, *d_corrections;
     float *derivatives_means, *derivatives_variances;
-    /* LSTM, [T][Bmax][C] or [T][Bmax][K] per direction d (index d*...) */
+    /* per-unit activation types / steepnesses (AF_unit arrays), NULL = the layer-wide value; AH entries */
+    uint32_t *unit_af; float *unit_steep;
+    /* LSTM: one olstm per direction */
     struct olstm *lstm;
 } olayer;
 
@@ -341,6 +343,7 @@ int myea_oracle_destroy(myea_oracle_net *n)
         free(o->neuron_errors); free(o->af_errors); free(o->norm_errors);
         free(o->means); free(o->variances); free(o->means_averages); free(o->variances_averages);
         free(o->r_corrections); free(o->d_corrections); free(o->derivatives_means); free(o->derivatives_variances);
+        free(o->unit_af); free(o->unit_steep);
         if (o->lstm) {
             for (int dir = 0; dir < 2; ++dir) {
                 olstm *q = &o->lstm[dir];
@@ -360,6 +363,20 @@ int myea_oracle_destroy(myea_oracle_net *n)
 int myea_oracle_set_hyper(myea_oracle_net *n, const myea_hyper *h) { if (!n || !h) return MYEA_E_INVALID; n->h = *h; return MYEA_OK; }
 int myea_oracle_get_hyper(myea_oracle_net *n, myea_hyper *h) { if (!n || !h) return MYEA_E_INVALID; *h = n->h; return MYEA_OK; }
 int myea_oracle_set_state_propagation(myea_oracle_net *n, uint32_t s) { if (!n) return MYEA_E_INVALID; n->state = s; return MYEA_OK; }
+/* AF_unit::ptr_type_activation_function / ptr_activation_steepness as per-unit arrays (NNH/Data.hpp, struct AF_unit) */
+int myea_oracle_set_unit_activations(myea_oracle_net *n, size_t li, const uint32_t *types, const float *steep, size_t count)
+{
+    if (!n || li == 0 || li >= n->d.n_layers || n->d.layers[li].type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_INVALID;
+    olayer *o = &n->L[li];
+    if (((types || steep) && count != o->AH) || n->d.layers[li].type_activation_function == MYEA_AF_SOFTMAX) return MYEA_E_INVALID;
+    free(o->unit_af); free(o->unit_steep); o->unit_af = NULL; o->unit_steep = NULL;
+    if (types) {
+        for (size_t j = 0; j < count; ++j) if (types[j] == MYEA_AF_NONE || types[j] >= MYEA_AF_LENGTH || types[j] == MYEA_AF_SOFTMAX) return MYEA_E_INVALID;
+        o->unit_af = (uint32_t *)malloc(count * sizeof(uint32_t)); memcpy(o->unit_af, types, count * sizeof(uint32_t));
+    }
+    if (steep) { o->unit_steep = (float *)malloc(count * sizeof(float)); memcpy(o->unit_steep, steep, count * sizeof(float)); }
+    return MYEA_OK;
+}
 int myea_oracle_set_threads(myea_oracle_net *n, int t) { if (!n || t < 1) return MYEA_E_INVALID; n->threads = t; return MYEA_OK; }
 float *myea_oracle_parameters(myea_oracle_net *n) { return n->parameters; }
 float *myea_oracle_gradient(myea_oracle_net *n) { return n->gradient; }
@@ -458,7 +475,7 @@ static void fwd_bn_inference(myea_oracle_net *n, size_t t, size_t B, size_t H, c
 }
 
 /* Forward_Pass__FC_AF: :4839-4868; Forward_Pass__FC_AF__Softmax: :4870-4905 */
-static void fwd_af(myea_oracle_net *n, size_t t, size_t B, size_t H, uint32_t type, const float *x, float *y)
+static void fwd_af(myea_oracle_net *n, size_t t, size_t B, size_t H, uint32_t type, const uint32_t *unit_type, const float *x, float *y)
 {
     size_t off = n->d.batch_size * H * t;
     for (size_t b = 0; b < B; ++b) {
@@ -471,7 +488,7 @@ static void fwd_af(myea_oracle_net *n, size_t t, size_t B, size_t H, uint32_t ty
             sum = 1.f / sum;
             for (size_t j = 0; j < H; ++j) yo[j] *= sum;
         } else {
-            for (size_t j = 0; j < H; ++j) yo[j] = myea_oracle_activation(type, xi[j]);
+            for (size_t j = 0; j < H; ++j) yo[j] = myea_oracle_activation(unit_type ? unit_type[j] : type, xi[j]);
         }
     }
 }
@@ -515,7 +532,7 @@ static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
         else fwd_bn_inference(n, t, B, H, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
         cur = o->normalizes;
     }
-    fwd_af(n, t, B, H, l->type_activation_function, cur, o->values);
+    fwd_af(n, t, B, H, l->type_activation_function, o->unit_af, cur, o->values);
     float *out = o->values;
     if (layer_uses_norm(l) && !l->use_layer_normalization_before_activation) {
         if (training) fwd_bn_training(n, renorm, t, B, H, o->values, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
@@ -542,7 +559,7 @@ static void fwd_residual_fc_layer(myea_oracle_net *n, size_t li, size_t B)
         cur = o->normalizes;
     }
     if (o->group == 2) {
-        fwd_af(n, 0, B, In, l->type_activation_function, cur, o->values);
+        fwd_af(n, 0, B, In, l->type_activation_function, o->unit_af, cur, o->values);
         fwd_dropout(n, l, 0, B, In, o->values);
         cur = o->values;
     }
@@ -984,7 +1001,7 @@ int myea_oracle_compute_error(myea_oracle_net *n, size_t B, const float *desired
                 default: break;
                 }
                 float q = rnn ? pre[0] : pre[j];
-                err[j] = myea_oracle_activation_derive(l->type_activation_function, q, l->activation_steepness, y[j]) * diff;
+                err[j] = myea_oracle_activation_derive(o->unit_af ? o->unit_af[j] : l->type_activation_function, q, o->unit_steep ? o->unit_steep[j] : l->activation_steepness, y[j]) * diff;
             }
         }
     }
@@ -1017,14 +1034,14 @@ static void bwd_fc(myea_oracle_net *n, size_t t, size_t B, size_t Out, size_t In
 }
 
 /* Backward_Pass__FC__DF: :1225-1263 */
-static void bwd_df(myea_oracle_net *n, size_t t, size_t B, size_t H, uint32_t type, float steep,
+static void bwd_df(myea_oracle_net *n, size_t t, size_t B, size_t H, uint32_t type, float steep, const uint32_t *unit_type, const float *unit_steep,
                    const float *pre, const float *val, const float *dy, float *dx)
 {
     size_t off = n->d.batch_size * H * t;
     for (size_t b = 0; b < B; ++b)
         for (size_t j = 0; j < H; ++j) {
             size_t k = off + b * H + j;
-            dx[k] = dy[k] * myea_oracle_activation_derive(type, pre[k], steep, val[k]);
+            dx[k] = dy[k] * myea_oracle_activation_derive(unit_type ? unit_type[j] : type, pre[k], unit_steep ? unit_steep[j] : steep, val[k]);
         }
 }
 
@@ -1077,7 +1094,7 @@ static void bwd_gradient_fc(myea_oracle_net *n, size_t li, size_t t, size_t B)
         cur = o->norm_errors;
     }
     const float *pre_af = (layer_uses_norm(l) && before) ? o->normalizes : o->summations;
-    bwd_df(n, t, B, H, l->type_activation_function, l->activation_steepness, pre_af, o->values, cur, o->af_errors);
+    bwd_df(n, t, B, H, l->type_activation_function, l->activation_steepness, o->unit_af, o->unit_steep, pre_af, o->values, cur, o->af_errors);
     cur = o->af_errors;
     if (layer_uses_norm(l) && before) {
         bwd_bn(n, renorm, li, t, B, H, o->summations /* pre_normalization */, cur, o->norm_errors);
@@ -1134,7 +1151,7 @@ static void bwd_gradient_residual_fc(myea_oracle_net *n, size_t li, size_t B)
     const float *prev_out = layer_outputs(n, o->prev);
     if (o->group == 2) {
         const float *pre_af = layer_uses_norm(l) ? o->normalizes : prev_out; /* ptr_array_pre_activation_functions */
-        bwd_df(n, 0, B, In, l->type_activation_function, l->activation_steepness, pre_af, o->values, din, o->af_errors);
+        bwd_df(n, 0, B, In, l->type_activation_function, l->activation_steepness, o->unit_af, o->unit_steep, pre_af, o->values, din, o->af_errors);
     }
     if (layer_uses_norm(l)) bwd_bn(n, renorm, li, 0, B, In, prev_out /* ptr_array_pre_normalization */, din, o->norm_errors);
 }

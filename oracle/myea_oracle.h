@@ -24,6 +24,7 @@ int myea_oracle_get_hyper(myea_oracle_net *net, myea_hyper *hyper);
 int myea_oracle_set_state_propagation(myea_oracle_net *net, uint32_t type_state_propagation);
 /* number of OpenMP threads used by the batch loops (1 = the reference's __Loop variants). */
 int myea_oracle_set_threads(myea_oracle_net *net, int threads);
+int myea_oracle_set_unit_activations(myea_oracle_net *net, size_t layer_index, const uint32_t *types, const float *steepness, size_t count);
 
 /* direct pointers to the flat vectors (the reference's data members are public) */
 float *myea_oracle_parameters(myea_oracle_net *net);

@@ -29,6 +29,7 @@ def load_oracle():
     lib.myea_oracle_get_hyper.argtypes = [vp, P(mb.Hyper)]
     lib.myea_oracle_set_state_propagation.argtypes = [vp, C.c_uint32]
     lib.myea_oracle_set_threads.argtypes = [vp, i32]
+    lib.myea_oracle_set_unit_activations.argtypes = [vp, C.c_size_t, vp, vp, C.c_size_t]
     for name in ("myea_oracle_parameters", "myea_oracle_gradient"):
         getattr(lib, name).argtypes = [vp]
         getattr(lib, name).restype = P(C.c_float)
@@ -113,6 +114,14 @@ class OracleNetwork:
 
     def download_optimizer_state(self, kind):
         return self._view(self.lib.myea_oracle_optimizer_state(self.handle, kind), self.desc.total_parameters).copy()
+
+    def set_unit_activations(self, layer, types=None, steepness=None):
+        t = None if types is None else np.ascontiguousarray(types, dtype=np.uint32)
+        st = None if steepness is None else np.ascontiguousarray(steepness, dtype=np.float32)
+        n = len(t) if t is not None else (len(st) if st is not None else 0)
+        self._keep = (t, st)
+        self._check(self.lib.myea_oracle_set_unit_activations(self.handle, layer, None if t is None else t.ctypes.data_as(C.c_void_p),
+                                                              None if st is None else st.ctypes.data_as(C.c_void_p), n))
 
     def upload_masks(self, m):
         m = np.asarray(m, dtype=np.uint8)
