@@ -61,7 +61,8 @@ enum {
 /* Enum_Type_Optimizer_Functions.hpp */
 enum {
     MYEA_OPTIMIZER_NONE = 0, MYEA_OPTIMIZER_ADABOUND = 1, MYEA_OPTIMIZER_ADAM = 2,
-    MYEA_OPTIMIZER_AMSBOUND = 4, MYEA_OPTIMIZER_AMSGRAD = 5, MYEA_OPTIMIZER_GD = 6
+    MYEA_OPTIMIZER_AMSBOUND = 4, MYEA_OPTIMIZER_AMSGRAD = 5, MYEA_OPTIMIZER_GD = 6,
+    MYEA_OPTIMIZER_IRPROP_PLUS = 8, MYEA_OPTIMIZER_NOSADAM = 9
 };
 
 /* Enum_Type_Layer_Dropout.hpp */
@@ -169,6 +170,30 @@ typedef struct myea_hyper {
     float batch_renormalization_d_correction_maximum;  /* 0 */
     float optimizer_time_step;          /* 0; incremented by every update */
     uint32_t number_time_delays;        /* RNN: first k steps carry no loss */
+    /* weight decay normalisation (Normalized_Weight_Decay, Train.cpp:285-286): wd * sqrt(B / (N_train * epoch_time_step)) */
+    uint32_t use_normalized_weight_decay;   /* 1 */
+    float epoch_time_step;                  /* 1; the caller's epoch loop increments it (Dataset.cpp:7660) */
+    /* NosAdam (Neural_Network__NosAdam.cpp) */
+    float adam_gamma;                       /* 0.1 */
+    float adam_previous_beta2;              /* 0; running sum of t^-gamma */
+    /* iRPROP+ (Neural_Network__iRPROP_plus.cpp); the caller's loop maintains the two losses (Dataset.cpp:575-579) */
+    float rprop_increase_factor;            /* 1.2 */
+    float rprop_decrease_factor;            /* 0.5 */
+    float rprop_delta_min;                  /* 1e-6 */
+    float rprop_delta_max;                  /* 50 */
+    float rprop_delta_zero;                 /* 0.1: initial step, written by clear_training_arrays */
+    float loss_rprop;                       /* FLT_MAX */
+    float previous_loss_rprop;              /* FLT_MAX */
+    /* max-norm constraint on every neuron's incoming weight vector after the update
+     * (Neural_Network__Regularization__Max_Norm_Constraints.cpp:140-529); 0 = off */
+    float regularization__max_norm_constraints;
+    /* warm restarts (Warm_Restarts_Decay, Train.cpp:266-283) */
+    uint32_t use_Warm_Restarts;             /* 0 */
+    float warm_restarts_decay_learning_rate;    /* 1 */
+    float warm_restarts_maximum_learning_rate;  /* 1 */
+    float warm_restarts_minimum_learning_rate;  /* 1e-7 */
+    float warm_restarts_T_i;                    /* 1 */
+    float warm_restarts_multiplier;             /* 2 */
 } myea_hyper;
 
 /* Loss / accuracy accumulators (ptr_array_loss_values, ptr_array_number_loss,
@@ -186,8 +211,11 @@ enum {
     MYEA_STATE_PREVIOUS_DELTA = 0,       /* ptr_array_previous_delta_parameters */
     MYEA_STATE_FIRST_MOMENT = 1,         /* ptr_array_previous_biased_first_moment */
     MYEA_STATE_SECOND_MOMENT = 2,        /* ptr_array_previous_biased_second_moment */
-    MYEA_STATE_SECOND_MOMENT_HAT = 3     /* ptr_array_previous_biased_second_moment_hat */
+    MYEA_STATE_SECOND_MOMENT_HAT = 3,    /* ptr_array_previous_biased_second_moment_hat */
+    MYEA_STATE_PREVIOUS_STEPS = 4,       /* ptr_array_previous_steps (iRPROP) */
+    MYEA_STATE_PREVIOUS_DERIVATIVES = 5  /* ptr_array_previous_derivatives_parameters (iRPROP) */
 };
+#define MYEA_STATE_KINDS 6
 enum {
     MYEA_TENSOR_OUTPUTS = 0,        /* Layer::ptr_array_outputs (post-dropout) [T][Bmax][H] */
     MYEA_TENSOR_SUMMATIONS = 1,     /* neuron_units->ptr_array_summations */

@@ -11,6 +11,7 @@
 #pragma once
 
 #include <cstdio>
+#include <cfloat>
 #include <cstring>
 #include <vector>
 
@@ -37,6 +38,15 @@ public:
     T_ normalization_momentum_average = 0.999f, normalization_epsilon = 1e-5f;
     T_ batch_renormalization_r_correction_maximum = 1.f, batch_renormalization_d_correction_maximum = 0.f;
     bool use_Nesterov = false, use_adam_bias_correction = true, use_clip_gradient = false;
+    bool use_normalized_weight_decay = true, use_Warm_Restarts = false;
+    T_ adam_gamma = 0.1f, regularization__max_norm_constraints = 0.f;
+    T_ rprop_increase_factor = 1.2f, rprop_decrease_factor = 0.5f, rprop_delta_min = 1e-6f, rprop_delta_max = 50.f, rprop_delta_zero = 0.1f;
+    T_ warm_restarts_decay_learning_rate = 1.f, warm_restarts_minimum_learning_rate = 1e-7f, warm_restarts_multiplier = 2.f;
+    // written by the caller's epoch loop and by the library (Clear_Optimizer, Warm_Restarts_Decay, the NosAdam step):
+    // pushed before and read back after every call that may change them
+    T_ optimizer_time_step = 0.f, epoch_time_step = 1.f, adam_previous_beta2 = 0.f;
+    T_ loss_rprop = FLT_MAX, previous_loss_rprop = FLT_MAX;
+    T_ warm_restarts_maximum_learning_rate = 1.f, warm_restarts_T_i = 1.f;
     unsigned int type_optimizer_function = MYEA_OPTIMIZER_NONE, type_loss_function = MYEA_LOSS_NONE;
     unsigned int type_accuracy_function = MYEA_ACCURACY_DISTANCE;
     unsigned int type_state_propagation = MYEA_STATE_INFERENCE;
@@ -161,7 +171,11 @@ public:
     }
 
     // Train.cpp:93-263
-    void Clear_Training_Arrays() { if (Need("Clear_Training_Arrays")) Ok("Clear_Training_Arrays", myea_hip_clear_training_arrays(net_)); }
+    void Clear_Training_Arrays()
+    {
+        if (!Need("Clear_Training_Arrays") || !PushFields("Clear_Training_Arrays")) return;
+        if (Ok("Clear_Training_Arrays", myea_hip_clear_training_arrays(net_))) PullState();
+    }
     void Reset__Loss() { if (Need("Reset__Loss")) Ok("Reset__Loss", myea_hip_reset_loss(net_)); }
 
     // ---- the five step entry points (Data.hpp:2896, 1033, 1709, 2199, 849) ----
@@ -190,10 +204,8 @@ public:
     {
         if (!Need("Update_Parameter") || !PushFields("Update_Parameter")) return;
         Ok("Update_Parameter", myea_hip_update_parameter(net_, batch_size_received, training_size_received));
-        myea_hyper h;
-        if (myea_hip_get_hyper(net_, &h) == MYEA_OK) optimizer_time_step = h.optimizer_time_step;
+        PullState();
     }
-    T_ optimizer_time_step = 0.f;
 
     // merged loss counters (Neural_Network__Merge.cpp:52-98); mean of the accumulated per-output terms
     T_ Get__Loss()
@@ -246,6 +258,14 @@ private:
         for (size_t i = 0; i < desc_.total_mask_units; ++i) ptr_array_units_mask_dropout_bernoulli[i] = true;
         return true;
     }
+    void PullState()
+    {
+        myea_hyper h;
+        if (myea_hip_get_hyper(net_, &h) != MYEA_OK) return;
+        optimizer_time_step = h.optimizer_time_step; epoch_time_step = h.epoch_time_step; adam_previous_beta2 = h.adam_previous_beta2;
+        loss_rprop = h.loss_rprop; previous_loss_rprop = h.previous_loss_rprop;
+        warm_restarts_maximum_learning_rate = h.warm_restarts_maximum_learning_rate; warm_restarts_T_i = h.warm_restarts_T_i;
+    }
     bool PushFields(const char *fn)
     {
         myea_hyper h;
@@ -259,6 +279,15 @@ private:
         h.batch_renormalization_r_correction_maximum = batch_renormalization_r_correction_maximum;
         h.batch_renormalization_d_correction_maximum = batch_renormalization_d_correction_maximum;
         h.number_time_delays = (uint32_t)number_time_delays;
+        h.use_normalized_weight_decay = use_normalized_weight_decay; h.use_Warm_Restarts = use_Warm_Restarts;
+        h.adam_gamma = adam_gamma; h.regularization__max_norm_constraints = regularization__max_norm_constraints;
+        h.rprop_increase_factor = rprop_increase_factor; h.rprop_decrease_factor = rprop_decrease_factor;
+        h.rprop_delta_min = rprop_delta_min; h.rprop_delta_max = rprop_delta_max; h.rprop_delta_zero = rprop_delta_zero;
+        h.warm_restarts_decay_learning_rate = warm_restarts_decay_learning_rate;
+        h.warm_restarts_minimum_learning_rate = warm_restarts_minimum_learning_rate; h.warm_restarts_multiplier = warm_restarts_multiplier;
+        h.optimizer_time_step = optimizer_time_step; h.epoch_time_step = epoch_time_step; h.adam_previous_beta2 = adam_previous_beta2;
+        h.loss_rprop = loss_rprop; h.previous_loss_rprop = previous_loss_rprop;
+        h.warm_restarts_maximum_learning_rate = warm_restarts_maximum_learning_rate; h.warm_restarts_T_i = warm_restarts_T_i;
         if (myea_hip_set_hyper(net_, &h) != MYEA_OK) return Fail(fn, myea_hip_last_error());
         return Ok(fn, myea_hip_set_state_propagation(net_, type_state_propagation));
     }

@@ -22,13 +22,13 @@ AF = dict(NONE=0, COSINE=1, COSINE_SYMMETRIC=2, ELU=3, ELLIOT=4, ELLIOT_SYMMETRI
           LINEAR_PIECE_SYMMETRIC=13, LEAKY_RELU=14, PARAMETRIC_RELU=15, RELU=16, SELU=17, SIGMOID=18,
           SINE=19, SIGMOID_STEPWISE=20, SINE_SYMMETRIC=21, SOFTMAX=22, TANH=23, TANH_STEPWISE=24,
           THRESHOLD=25, THRESHOLD_SYMMETRIC=26)
-OPTIMIZER = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6)
+OPTIMIZER = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP_PLUS=8, NOSADAM=9)
 DROPOUT = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
 NORMALIZATION = dict(NONE=0, BATCH_NORMALIZATION=1, BATCH_RENORMALIZATION=2)
 LOSS = dict(NONE=0, BIT=1, CROSS_ENTROPY=2, L1=3, L2=4, MAE=5, MAPE=6, ME=9, MSE=10, RMSE=11, SMAPE=12)
 ACCURACY = dict(NONE=0, CROSS_ENTROPY=1, DIRECTIONAL=2, DISTANCE=3, SIGN=5)
 STATE_INFERENCE, STATE_TRAINING = 0, 1
-OPT_STATE = dict(PREVIOUS_DELTA=0, FIRST_MOMENT=1, SECOND_MOMENT=2, SECOND_MOMENT_HAT=3)
+OPT_STATE = dict(PREVIOUS_DELTA=0, FIRST_MOMENT=1, SECOND_MOMENT=2, SECOND_MOMENT_HAT=3, PREVIOUS_STEPS=4, PREVIOUS_DERIVATIVES=5)
 TENSOR = dict(OUTPUTS=0, SUMMATIONS=1, ERRORS=2, NORM_HATS=3, NORM_MEANS=4, NORM_VARIANCES=5,
               NORM_MEANS_AVERAGES=6, NORM_VARIANCES_AVERAGES=7, INPUT_SIDE_ERRORS=8,
               LSTM_CELL_INPUT=16, LSTM_CELL_STATE=17, LSTM_INPUT_GATE=18, LSTM_FORGET_GATE=19,
@@ -73,6 +73,14 @@ class Hyper(C.Structure):
         ("batch_renormalization_r_correction_maximum", C.c_float),
         ("batch_renormalization_d_correction_maximum", C.c_float),
         ("optimizer_time_step", C.c_float), ("number_time_delays", C.c_uint32),
+        ("use_normalized_weight_decay", C.c_uint32), ("epoch_time_step", C.c_float),
+        ("adam_gamma", C.c_float), ("adam_previous_beta2", C.c_float),
+        ("rprop_increase_factor", C.c_float), ("rprop_decrease_factor", C.c_float), ("rprop_delta_min", C.c_float),
+        ("rprop_delta_max", C.c_float), ("rprop_delta_zero", C.c_float), ("loss_rprop", C.c_float),
+        ("previous_loss_rprop", C.c_float), ("regularization__max_norm_constraints", C.c_float),
+        ("use_Warm_Restarts", C.c_uint32), ("warm_restarts_decay_learning_rate", C.c_float),
+        ("warm_restarts_maximum_learning_rate", C.c_float), ("warm_restarts_minimum_learning_rate", C.c_float),
+        ("warm_restarts_T_i", C.c_float), ("warm_restarts_multiplier", C.c_float),
     ]
 
 

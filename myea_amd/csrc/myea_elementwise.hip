@@ -326,12 +326,34 @@ struct UpdateDev {
 // Update_Parameter__Gradient_Descent (NN/Neural_Network__Gradient_Descent.cpp:84-120), __Momentum
 // (NN/Neural_Network__Gradient_Descent_Momentum.cpp:22-62), Nesterov
 // (NN/Neural_Network__Nesterov_Accelerated_Gradient.cpp:22-64; sign of the lr*g term as written there).
-// KIND: 0 GD, 1 momentum, 2 Nesterov, 3 Adam, 4 AMSGrad, 5 AdaBound.
+// __AMSBound (NN/Neural_Network__AMSBound.cpp:43-110), iRPROP+ (NN/Neural_Network__iRPROP_plus.cpp:28-117).
+// NosAdam (NN/Neural_Network__NosAdam.cpp:43-100) is KIND 3 with the host's beta2 at time t.
+// KIND: 0 GD, 1 momentum, 2 Nesterov, 3 Adam, 4 AMSGrad, 5 AdaBound, 6 AMSBound,
+//       7 iRPROP+ (a = previous delta, b = previous step, c = previous slope; lr / mu = increase / decrease factor,
+//         lower / upper = smallest / largest step, beta1 != 0 when the loss got worse).
 template <int KIND, bool WD>
 __device__ __forceinline__ void update_one(const UpdateDev &p, float gs, float &w, float g, float &a, float &b, float &c, bool is_weight)
 {
     g *= gs;
     float step;
+    if (KIND == 7) {
+        const float sg = g > 0.f ? 1.f : (g < 0.f ? -1.f : 0.f), same = c * g;
+        if (same > 0.f) {
+            b = fminf(b * p.lr, p.upper);
+            a = -sg * b;
+            w += a;
+            c = g;
+        } else if (same < 0.f) {
+            b = fmaxf(b * p.mu, p.lower);
+            if (p.beta1 != 0.f) w -= a;
+            c = 0.f;
+        } else {
+            a = -sg * b;
+            w += a;
+            c = g;
+        }
+        return;
+    }
     if (KIND == 0) {
         step = p.lr * g;
     } else if (KIND == 1) {
@@ -345,7 +367,12 @@ __device__ __forceinline__ void update_one(const UpdateDev &p, float gs, float &
         b = p.beta2 * b + (1.f - p.beta2) * g * g;
         if (KIND == 3) step = p.lr_t * a / (sqrtf(b) + p.eps);
         else if (KIND == 4) { c = fmaxf(c, b); step = p.lr_t * a / (sqrtf(c) + p.eps); }
-        else { float r = p.lr_t / (sqrtf(b) + p.eps); r = r < p.lower ? p.lower : (r > p.upper ? p.upper : r); step = r * a; }
+        else {
+            if (KIND == 6) c = fmaxf(c, b);
+            float r = p.lr_t / (sqrtf(KIND == 6 ? c : b) + p.eps);
+            r = r < p.lower ? p.lower : (r > p.upper ? p.upper : r);
+            step = r * a;
+        }
     }
     if (WD) step += (is_weight ? 1.f : 0.f) * p.wd * w;
     w -= step;
@@ -359,7 +386,7 @@ __global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
         const float norm = sqrtf(p.norm_sq[0]);
         if (norm >= p.clip) gs = p.clip / norm;
     }
-    constexpr bool kA = KIND >= 1, kB = KIND >= 3, kC = KIND == 4;
+    constexpr bool kA = KIND >= 1, kB = KIND >= 3, kC = KIND == 4 || KIND >= 6;
     const size_t n4 = p.n / 4;
     f32x4 *w4 = reinterpret_cast<f32x4 *>(p.w), *g4 = reinterpret_cast<f32x4 *>(p.g);
     f32x4 *a4 = reinterpret_cast<f32x4 *>(p.s0), *b4 = reinterpret_cast<f32x4 *>(p.s1), *c4 = reinterpret_cast<f32x4 *>(p.s2);
@@ -393,6 +420,45 @@ __global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
         if (kB) p.s1[i] = b;
         if (kC) p.s2[i] = c;
         p.g[i] = 0.f;
+    }
+}
+
+// Euclidean_Norm (NN/Neural_Network__Regularization__Max_Norm_Constraints.cpp:48-137): a weight segment whose norm is at
+// or above max_norm is rescaled to max_norm.  GROUP threads (one wave, or the whole workgroup) own one segment.
+template <int GROUP>
+__global__ __launch_bounds__(kBlock) void max_norm_kernel(size_t nseg, const unsigned long long *__restrict__ first, const unsigned *__restrict__ len,
+                                                          float max_norm, float *w)
+{
+    constexpr int kPerBlock = kBlock / GROUP;
+    __shared__ float red[kBlock / 64];
+    const size_t seg = (size_t)blockIdx.x * kPerBlock + threadIdx.x / GROUP;
+    const unsigned lane = threadIdx.x % GROUP;
+    const bool live = seg < nseg;
+    float *v = live ? w + first[seg] : nullptr;
+    const unsigned L = live ? len[seg] : 0u;
+    const bool vec = ((reinterpret_cast<uintptr_t>(v) | ((uintptr_t)L * 4u)) & 15u) == 0;
+    float s = 0.f;
+    if (vec) {
+        const f32x4 *v4 = reinterpret_cast<const f32x4 *>(v);
+        for (unsigned i = lane; i < L / 4; i += GROUP) { const f32x4 x = v4[i]; s += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3]; }
+    } else {
+        for (unsigned i = lane; i < L; i += GROUP) s += v[i] * v[i];
+    }
+    s = wave_sum(s);
+    if (GROUP > 64) {
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+        __syncthreads();
+        s = red[0] + red[1] + red[2] + red[3];
+    }
+    const float norm = sqrtf(s);
+    if (norm >= max_norm) {
+        const float r = max_norm / norm;
+        if (vec) {
+            f32x4 *v4 = reinterpret_cast<f32x4 *>(v);
+            for (unsigned i = lane; i < L / 4; i += GROUP) { f32x4 x = v4[i]; x[0] *= r; x[1] *= r; x[2] *= r; x[3] *= r; v4[i] = x; }
+        } else {
+            for (unsigned i = lane; i < L; i += GROUP) v[i] *= r;
+        }
     }
 }
 
@@ -578,6 +644,16 @@ int launch_sum_squares(hipStream_t s, size_t n, const float *g, float *partials,
     return MYEA_OK;
 }
 
+int launch_max_norm(hipStream_t s, size_t nseg, const unsigned long long *first, const unsigned *len, unsigned longest, float max_norm, float *w)
+{
+    if (nseg == 0) return MYEA_OK;
+    if (!first || !len || !w) { set_last_error("max-norm: null segment table"); return MYEA_E_INVALID; }
+    if (longest > 1024) hipLaunchKernelGGL((max_norm_kernel<kBlock>), dim3(grid_for(nseg, 1, 0x7fffffffu)), dim3(kBlock), 0, s, nseg, first, len, max_norm, w);
+    else hipLaunchKernelGGL((max_norm_kernel<64>), dim3(grid_for(nseg, kBlock / 64, 0x7fffffffu)), dim3(kBlock), 0, s, nseg, first, len, max_norm, w);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
 int launch_update(hipStream_t s, const UpdateParams &p)
 {
     if (p.n == 0) return MYEA_OK;
@@ -606,6 +682,15 @@ int launch_update(hipStream_t s, const UpdateParams &p)
     case MYEA_OPTIMIZER_ADABOUND:
         if (!need(p.s0, "first moment") || !need(p.s1, "second moment")) return MYEA_E_INVALID;
         return launch_update_kind<5>(s, d, wd);
+    case MYEA_OPTIMIZER_AMSBOUND:
+        if (!need(p.s0, "first moment") || !need(p.s1, "second moment") || !need(p.s2, "second moment hat")) return MYEA_E_INVALID;
+        return launch_update_kind<6>(s, d, wd);
+    case MYEA_OPTIMIZER_NOSADAM:
+        if (!need(p.s0, "first moment") || !need(p.s1, "second moment")) return MYEA_E_INVALID;
+        return launch_update_kind<3>(s, d, wd);
+    case MYEA_OPTIMIZER_IRPROP_PLUS:
+        if (!need(p.s0, "previous delta") || !need(p.s1, "previous steps") || !need(p.s2, "previous slopes")) return MYEA_E_INVALID;
+        return launch_update_kind<7>(s, d, false);
     default:
         set_last_error("optimizer %d is not on this path", p.optimizer);
         return MYEA_E_UNSUPPORTED;

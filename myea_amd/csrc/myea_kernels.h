@@ -136,6 +136,9 @@ struct UpdateParams {
     float grad_scale;      // host-side multiplier (used when norm_sq is null)
 };
 int launch_update(hipStream_t s, const UpdateParams &p);
+// every segment w[first[i] .. first[i] + len[i]) whose Euclidean norm is >= max_norm is scaled onto that norm;
+// `longest` = the largest len (picks one wave or one workgroup per segment)
+int launch_max_norm(hipStream_t s, size_t nseg, const unsigned long long *first, const unsigned *len, unsigned longest, float max_norm, float *w);
 
 int launch_fill(hipStream_t s, float *p, size_t n, float v);
 

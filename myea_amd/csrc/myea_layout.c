@@ -6,6 +6,7 @@
  */
 #include "../../include/myea_hip.h"
 
+#include <float.h>
 #include <string.h>
 
 /* Public training fields: Header_Files/Neural_Network/Data.hpp:2929-2970. */
@@ -37,6 +38,24 @@ void myea_hyper_default(myea_hyper *h)
     h->batch_renormalization_d_correction_maximum = 0.f;
     h->optimizer_time_step = 0.f;
     h->number_time_delays = 0;
+    h->use_normalized_weight_decay = 1;
+    h->epoch_time_step = 1.f;
+    h->adam_gamma = 0.1f;
+    h->adam_previous_beta2 = 0.f;
+    h->rprop_increase_factor = 1.2f;
+    h->rprop_decrease_factor = 0.5f;
+    h->rprop_delta_min = 1e-6f;
+    h->rprop_delta_max = 50.f;
+    h->rprop_delta_zero = 0.1f;
+    h->loss_rprop = FLT_MAX;
+    h->previous_loss_rprop = FLT_MAX;
+    h->regularization__max_norm_constraints = 0.f;
+    h->use_Warm_Restarts = 0;
+    h->warm_restarts_decay_learning_rate = 1.f;
+    h->warm_restarts_maximum_learning_rate = 1.f;
+    h->warm_restarts_minimum_learning_rate = 1e-7f;
+    h->warm_restarts_T_i = 1.f;
+    h->warm_restarts_multiplier = 2.f;
 }
 
 /* Index of the residual layer whose block contains layer li, or 0 when li is outside every block

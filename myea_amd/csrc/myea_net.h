@@ -49,8 +49,13 @@ struct Net {
     myea_hyper h{};
     uint32_t state = MYEA_STATE_INFERENCE;
     hipStream_t stream = nullptr;
-    float *parameters = nullptr, *gradient = nullptr, *opt[4] = {nullptr, nullptr, nullptr, nullptr};
+    float *parameters = nullptr, *gradient = nullptr, *opt[MYEA_STATE_KINDS] = {};
     uint8_t *masks = nullptr;
+    // max-norm constraint: weight segments (one per neuron / per LSTM gate vector), built on first use
+    unsigned long long *seg_first = nullptr;
+    unsigned *seg_len = nullptr;
+    size_t n_segments = 0;
+    unsigned longest_segment = 0;
     std::vector<DevLayer> L;
     float *tmp1 = nullptr, *tmp2 = nullptr, *scratch = nullptr, *stage_in = nullptr, *stage_out = nullptr;
     double *loss_acc = nullptr;
@@ -62,6 +67,9 @@ struct Net {
 
     ~Net();
     int create(const myea_net_desc &desc);
+    int clear_optimizer();
+    int build_max_norm_segments();
+    float warm_restarts_decay(int *rc);
 
     float *layer_outputs(size_t li);
     float *scale_ptr(float *base, size_t li);

@@ -3,6 +3,8 @@
 // myea_elementwise.hip (and myea_lstm.hip).
 //
 // NN/ = Neural_Network_Library_Windows/Source_Files/Neural_Network/ of the reference.
+#include <algorithm>
+#include <cfloat>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -74,7 +76,7 @@ void Net::prof_begin(int family)
     ev.family = family;
     if (!free_events.empty()) { ev = free_events.back(); free_events.pop_back(); ev.family = family; }
     else if (hipEventCreate(&ev.start) != hipSuccess || hipEventCreate(&ev.stop) != hipSuccess) return;
-    hipEventRecord(ev.start, stream);
+    (void)hipEventRecord(ev.start, stream);
     pending.push_back(ev);
     open_event = true;
 }
@@ -84,7 +86,7 @@ void Net::prof_end(double work)
     if (!profiling || !open_event) return;
     ProfEvent &ev = pending.back();
     ev.work = work;
-    hipEventRecord(ev.stop, stream);
+    (void)hipEventRecord(ev.stop, stream);
     open_event = false;
 }
 
@@ -157,10 +159,11 @@ int Net::create(const myea_net_desc &desc)
     const size_t P = d.total_parameters, T = d.number_recurrent_depth, B = d.batch_size;
     MYEA_TRY(dev_alloc(&parameters, P));
     MYEA_TRY(dev_alloc(&gradient, P));
-    for (int k = 0; k < 4; ++k) MYEA_TRY(dev_alloc(&opt[k], P));
+    for (int k = 0; k < MYEA_STATE_KINDS; ++k) MYEA_TRY(dev_alloc(&opt[k], P));
     MYEA_HIP_TRY(hipMemset(parameters, 0, P * sizeof(float)));
     MYEA_HIP_TRY(hipMemset(gradient, 0, P * sizeof(float)));
-    for (int k = 0; k < 4; ++k) MYEA_HIP_TRY(hipMemset(opt[k], 0, P * sizeof(float)));
+    for (int k = 0; k < MYEA_STATE_KINDS; ++k) MYEA_HIP_TRY(hipMemset(opt[k], 0, P * sizeof(float)));
+    MYEA_TRY(launch_fill(0, opt[MYEA_STATE_PREVIOUS_STEPS], P, h.rprop_delta_zero));
     if (d.total_normalized_units) MYEA_TRY(launch_fill(0, parameters + d.total_weights + d.total_bias, d.total_normalized_units, 1.f));
     {
         void *q = nullptr;
@@ -239,7 +242,8 @@ Net::~Net()
 {
     auto fr = [](void *p) { if (p) (void)hipFree(p); };
     fr(parameters); fr(gradient);
-    for (int k = 0; k < 4; ++k) fr(opt[k]);
+    for (int k = 0; k < MYEA_STATE_KINDS; ++k) fr(opt[k]);
+    fr(seg_first); fr(seg_len);
     fr(masks);
     for (DevLayer &o : L) {
         fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep);
@@ -723,51 +727,163 @@ int Net::set_unit_activations(size_t li, const uint32_t *types, const float *ste
 // Update_Parameter__OpenMP (NN/Neural_Network.cpp:4727-4828): [merge: one accumulator here] -> clip by global norm
 // over all P (NN/Neural_Network__Clip_Gradient.cpp:81-94) -> optimizer.  The clip scale is applied inside the
 // optimizer's gradient read instead of a separate pass over the gradient.
+// Clear_Optimizer (NN/Train.cpp:128-263): state vectors to zero (iRPROP steps to rprop_delta_zero, its two losses to the
+// largest float, NosAdam's running sum to 0), optimizer_time_step = 0, epoch_time_step = 1.
+int Net::clear_optimizer()
+{
+    const size_t P = d.total_parameters;
+    for (int k = 0; k < MYEA_STATE_KINDS; ++k)
+        if (k != MYEA_STATE_PREVIOUS_STEPS) MYEA_HIP_TRY(hipMemsetAsync(opt[k], 0, P * sizeof(float), stream));
+    MYEA_TRY(launch_fill(stream, opt[MYEA_STATE_PREVIOUS_STEPS], P, h.rprop_delta_zero));
+    h.loss_rprop = FLT_MAX;
+    h.previous_loss_rprop = FLT_MAX;
+    h.adam_previous_beta2 = 0.f;
+    h.optimizer_time_step = 0.f;
+    h.epoch_time_step = 1.f;
+    return MYEA_OK;
+}
+
+// Warm_Restarts_Decay (NN/Train.cpp:266-283): cosine-annealed rate from the step count before this update; at the end of
+// a cycle the optimizer is cleared, the cycle lengthens and its maximum rate decays.
+float Net::warm_restarts_decay(int *rc)
+{
+    const float lr = h.warm_restarts_minimum_learning_rate
+                     + 0.5f * (h.warm_restarts_maximum_learning_rate - h.warm_restarts_minimum_learning_rate)
+                           * (1.f + std::cos(h.optimizer_time_step / h.warm_restarts_T_i * 3.14159265358979323846f));
+    *rc = MYEA_OK;
+    if (h.optimizer_time_step >= h.warm_restarts_T_i) {
+        *rc = clear_optimizer();
+        h.warm_restarts_T_i *= h.warm_restarts_multiplier;
+        h.warm_restarts_maximum_learning_rate = std::max(h.warm_restarts_maximum_learning_rate * h.warm_restarts_decay_learning_rate,
+                                                         h.warm_restarts_minimum_learning_rate);
+    }
+    return lr;
+}
+
+// The vectors Update_Weight_Regularization__Max_Norm_Constraints walks with (0, total_weights)
+// (NN/Neural_Network__Regularization__Max_Norm_Constraints.cpp:147-332): one per fully-connected neuron (hidden and output
+// layers); per LSTM block the cell-input feed-forward / recurrent vectors of each cell, then the three gates' feed-forward,
+// recurrent and peephole vectors.  The LSTM tests are `first index > start`: a vector at flat index 0 is skipped.
+int Net::build_max_norm_segments()
+{
+    if (seg_first) return MYEA_OK;
+    std::vector<unsigned long long> first;
+    std::vector<unsigned> len;
+    for (size_t li = 1; li < d.n_layers; ++li) {
+        const myea_layer_desc &l = d.layers[li];
+        const size_t In = L[li].In;
+        if (l.type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+            for (size_t o = 0; o < L[li].H; ++o) { first.push_back(l.first_connection_index + o * In); len.push_back((unsigned)In); }
+        } else if (l.type_layer == MYEA_LAYER_LSTM) {
+            const size_t K = l.n_units, cpb = l.n_cells_per_block, C = K * cpb;
+            const size_t per_block = cpb * (In + C) + 3 * In + 3 * C + 3 * cpb;
+            const size_t blocks = l.use_bidirectional ? 2 * K : K;
+            for (size_t k = 0; k < blocks; ++k) {
+                size_t at = l.first_connection_index + k * per_block;
+                auto push = [&](size_t n) { if (at != 0 && n != 0) { first.push_back(at); len.push_back((unsigned)n); } at += n; };
+                for (size_t j = 0; j < cpb; ++j) { push(In); push(C); }
+                for (int g = 0; g < 3; ++g) push(In);
+                for (int g = 0; g < 3; ++g) push(C);
+                for (int g = 0; g < 3; ++g) push(cpb);
+            }
+        }
+    }
+    n_segments = first.size();
+    longest_segment = 0;
+    for (unsigned v : len) longest_segment = std::max(longest_segment, v);
+    void *q = nullptr;
+    MYEA_HIP_TRY(hipMalloc(&q, std::max<size_t>(1, n_segments) * sizeof(unsigned long long)));
+    seg_first = static_cast<unsigned long long *>(q);
+    MYEA_HIP_TRY(hipMalloc(&q, std::max<size_t>(1, n_segments) * sizeof(unsigned)));
+    seg_len = static_cast<unsigned *>(q);
+    if (n_segments) {
+        MYEA_HIP_TRY(hipMemcpy(seg_first, first.data(), n_segments * sizeof(unsigned long long), hipMemcpyHostToDevice));
+        MYEA_HIP_TRY(hipMemcpy(seg_len, len.data(), n_segments * sizeof(unsigned), hipMemcpyHostToDevice));
+    }
+    return MYEA_OK;
+}
+
+// Update_Parameter (NN/Neural_Network.cpp:4722-4911).  The L1 / L2 gradient terms are called there with (batch size, 0,
+// total weights) where the callee expects (start, end, batch size) - both loops are empty
+// (NN/Neural_Network__Regularization__L1.cpp:98-128), so they add nothing here either.
 int Net::update_parameter(size_t B, size_t training_size)
 {
-    (void)B; (void)training_size;
+    const uint32_t kind = h.type_optimizer_function;
+    switch (kind) {
+    case MYEA_OPTIMIZER_GD: case MYEA_OPTIMIZER_ADAM: case MYEA_OPTIMIZER_AMSGRAD: case MYEA_OPTIMIZER_ADABOUND:
+    case MYEA_OPTIMIZER_AMSBOUND: case MYEA_OPTIMIZER_NOSADAM: case MYEA_OPTIMIZER_IRPROP_PLUS: break;
+    default:
+        set_last_error("Update_Parameter: optimizer %u is not on this path", kind);
+        return MYEA_E_UNSUPPORTED;
+    }
+    if (training_size == 0 && h.use_normalized_weight_decay && h.regularization__weight_decay != 0.f) {
+        set_last_error("Update_Parameter: normalized weight decay needs the training-set size");
+        return MYEA_E_INVALID;
+    }
     UpdateParams p{};
-    p.optimizer = (int)h.type_optimizer_function;
+    p.optimizer = (int)kind;
     p.n = d.total_parameters; p.n_weights = d.total_weights;
     p.w = parameters; p.g = gradient;
     p.grad_scale = 1.f;
-    p.wd = h.regularization__weight_decay;
     if (h.use_clip_gradient) {
         MYEA_TRY(launch_sum_squares(stream, p.n, gradient, scratch + 16, scratch));
         p.norm_sq = scratch;
         p.clip = h.clip_gradient;
     }
-    h.optimizer_time_step += 1.f;
+    const bool rprop = kind == MYEA_OPTIMIZER_IRPROP_PLUS, gd = kind == MYEA_OPTIMIZER_GD;
+    float scale = 1.f;
+    if (h.use_Warm_Restarts && !rprop) {
+        int rc = MYEA_OK;
+        scale = warm_restarts_decay(&rc) / (gd ? h.learning_rate : h.adam_learning_rate);
+        if (rc != MYEA_OK) return rc;
+    }
+    if (!rprop) h.optimizer_time_step += 1.f;
     const float ts = h.optimizer_time_step;
+    // Normalized_Weight_Decay (NN/Train.cpp:285-286); only the gradient-descent family scales it by the warm-restart factor
+    p.wd = h.use_normalized_weight_decay
+               ? h.regularization__weight_decay * std::sqrt((float)B / ((float)training_size * h.epoch_time_step))
+               : h.regularization__weight_decay;
+    if (h.regularization__weight_decay == 0.f) p.wd = 0.f;
     double bytes_per_param = 16;
-    switch (h.type_optimizer_function) {
-    case MYEA_OPTIMIZER_GD:
-        p.lr = h.learning_rate; p.mu = h.learning_momentum;
+    if (gd) {
+        p.lr = scale * h.learning_rate; p.mu = h.learning_momentum;
+        p.wd *= scale;
         p.variant = h.learning_momentum != 0.f ? (h.use_Nesterov ? 2 : 1) : 0;
         p.s0 = opt[MYEA_STATE_PREVIOUS_DELTA];
         bytes_per_param = p.variant ? 24 : 16;
-        break;
-    case MYEA_OPTIMIZER_ADAM:
-    case MYEA_OPTIMIZER_AMSGRAD:
-    case MYEA_OPTIMIZER_ADABOUND:
+    } else if (rprop) {
+        p.lr = h.rprop_increase_factor; p.mu = h.rprop_decrease_factor;
+        p.lower = h.rprop_delta_min; p.upper = h.rprop_delta_max;
+        p.beta1 = h.loss_rprop > h.previous_loss_rprop ? 1.f : 0.f;
+        p.wd = 0.f;
+        p.s0 = opt[MYEA_STATE_PREVIOUS_DELTA]; p.s1 = opt[MYEA_STATE_PREVIOUS_STEPS]; p.s2 = opt[MYEA_STATE_PREVIOUS_DERIVATIVES];
+        bytes_per_param = 40;
+    } else {
+        const float lr = scale * h.adam_learning_rate;
         p.beta1 = h.adam_beta1; p.beta2 = h.adam_beta2; p.eps = h.adam_epsilon;
         p.lr_t = h.use_adam_bias_correction
-                     ? (float)(h.adam_learning_rate * std::sqrt(1.0 - std::pow((double)h.adam_beta2, (double)ts)) / (1.0 - std::pow((double)h.adam_beta1, (double)ts)))
-                     : h.adam_learning_rate;
-        p.lower = h.learning_rate_final * (1.f - 1.f / (h.learning_gamma * ts + 1.f));
-        p.upper = h.learning_rate_final * (1.f + 1.f / (h.learning_gamma * ts));
+                     ? (float)(lr * std::sqrt(1.0 - std::pow((double)h.adam_beta2, (double)ts)) / (1.0 - std::pow((double)h.adam_beta1, (double)ts)))
+                     : lr;
+        p.lower = scale * h.learning_rate_final * (1.f - 1.f / (h.learning_gamma * ts + 1.f));
+        p.upper = scale * h.learning_rate_final * (1.f + 1.f / (h.learning_gamma * ts));
+        if (kind == MYEA_OPTIMIZER_NOSADAM) {
+            // the second moment decays with beta2_t = S / (S + t^-gamma), S the sum of the earlier t^-gamma; the bias
+            // correction above keeps the plain beta2 (NN/Neural_Network__NosAdam.cpp:57-70)
+            const float pg = std::pow(ts, -h.adam_gamma);
+            p.beta2 = h.adam_previous_beta2 / (h.adam_previous_beta2 + pg);
+            h.adam_previous_beta2 += pg;
+        }
         p.s0 = opt[MYEA_STATE_FIRST_MOMENT]; p.s1 = opt[MYEA_STATE_SECOND_MOMENT]; p.s2 = opt[MYEA_STATE_SECOND_MOMENT_HAT];
-        bytes_per_param = h.type_optimizer_function == MYEA_OPTIMIZER_AMSGRAD ? 40 : 32;
-        break;
-    default:
-        h.optimizer_time_step -= 1.f;
-        set_last_error("Update_Parameter: optimizer %u is not on this path", h.type_optimizer_function);
-        return MYEA_E_UNSUPPORTED;
+        bytes_per_param = (kind == MYEA_OPTIMIZER_AMSGRAD || kind == MYEA_OPTIMIZER_AMSBOUND) ? 40 : 32;
     }
     prof_begin(3);
     const int rc = launch_update(stream, p);
     prof_end(bytes_per_param * (double)p.n);
     if (rc != MYEA_OK) return rc;
+    if (h.regularization__max_norm_constraints != 0.f) {
+        MYEA_TRY(build_max_norm_segments());
+        MYEA_TRY(launch_max_norm(stream, n_segments, seg_first, seg_len, longest_segment, h.regularization__max_norm_constraints, parameters));
+    }
     return lstm_parameters_changed();  // refresh the packed gate matrices
 }
 
@@ -819,6 +935,8 @@ int myea_hip_set_hyper(myea_hip_net *n, const myea_hyper *h)
     NET_OR_FAIL(n);
     if (!h) { myea::set_last_error("set_hyper: null"); return MYEA_E_INVALID; }
     n->net.h = *h;
+    // the constraint's segment table is built here so that the step itself never allocates
+    if (h->regularization__max_norm_constraints != 0.f) return n->net.build_max_norm_segments();
     return MYEA_OK;
 }
 int myea_hip_get_hyper(myea_hip_net *n, myea_hyper *h)
@@ -862,13 +980,13 @@ int myea_hip_download_parameters(myea_hip_net *n, float *p, size_t c)
 int myea_hip_upload_optimizer_state(myea_hip_net *n, int kind, const float *p, size_t c)
 {
     NET_OR_FAIL(n);
-    if (kind < 0 || kind > 3 || !p) { myea::set_last_error("upload_optimizer_state: bad kind %d or null", kind); return MYEA_E_INVALID; }
+    if (kind < 0 || kind >= MYEA_STATE_KINDS || !p) { myea::set_last_error("upload_optimizer_state: bad kind %d or null", kind); return MYEA_E_INVALID; }
     return copy_vec(n, n->net.opt[kind], nullptr, p, c, "upload_optimizer_state");
 }
 int myea_hip_download_optimizer_state(myea_hip_net *n, int kind, float *p, size_t c)
 {
     NET_OR_FAIL(n);
-    if (kind < 0 || kind > 3 || !p) { myea::set_last_error("download_optimizer_state: bad kind %d or null", kind); return MYEA_E_INVALID; }
+    if (kind < 0 || kind >= MYEA_STATE_KINDS || !p) { myea::set_last_error("download_optimizer_state: bad kind %d or null", kind); return MYEA_E_INVALID; }
     return copy_vec(n, n->net.opt[kind], p, nullptr, c, "download_optimizer_state");
 }
 int myea_hip_set_unit_activations(myea_hip_net *n, size_t li, const uint32_t *types, const float *steep, size_t count)
@@ -890,9 +1008,7 @@ int myea_hip_clear_training_arrays(myea_hip_net *n)
     NET_OR_FAIL(n);
     const size_t bytes = n->net.d.total_parameters * sizeof(float);
     MYEA_HIP_TRY(hipMemsetAsync(n->net.gradient, 0, bytes, n->net.stream));
-    for (int k = 0; k < 4; ++k) MYEA_HIP_TRY(hipMemsetAsync(n->net.opt[k], 0, bytes, n->net.stream));
-    n->net.h.optimizer_time_step = 0.f;
-    return MYEA_OK;
+    return n->net.clear_optimizer();
 }
 
 int myea_hip_forward_pass(myea_hip_net *n, size_t B, const float *x, int dev) { NET_OR_FAIL(n); return n->net.forward_pass(B, x, dev); }

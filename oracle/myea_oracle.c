@@ -71,7 +71,7 @@ struct myea_oracle_net {
     myea_hyper h;
     uint32_t state;
     int threads;
-    float *parameters, *gradient, *opt[4];
+    float *parameters, *gradient, *opt[MYEA_STATE_KINDS];
     uint8_t *masks;
     olayer L[MYEA_MAX_LAYERS];
     myea_loss_state loss;
@@ -230,7 +230,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
     size_t P = desc->total_parameters, T = desc->number_recurrent_depth, B = desc->batch_size;
     n->parameters = zalloc(P);
     n->gradient = zalloc(P);
-    for (int k = 0; k < 4; ++k) n->opt[k] = zalloc(P);
+    for (int k = 0; k < MYEA_STATE_KINDS; ++k) n->opt[k] = zalloc(P);
     n->masks = (uint8_t *)malloc(desc->total_mask_units ? desc->total_mask_units : 1);
     memset(n->masks, 1, desc->total_mask_units ? desc->total_mask_units : 1); /* NN/Neural_Network__Allocate.cpp:386-410: all true */
     /* scales start at 1, shifts at 0 (NN/Neural_Network__Allocate.cpp:2395-2401 and the scale fill) */
@@ -335,7 +335,7 @@ int myea_oracle_destroy(myea_oracle_net *n)
 {
     if (!n) return MYEA_OK;
     free(n->parameters); free(n->gradient);
-    for (int k = 0; k < 4; ++k) free(n->opt[k]);
+    for (int k = 0; k < MYEA_STATE_KINDS; ++k) free(n->opt[k]);
     free(n->masks);
     for (size_t li = 0; li < n->d.n_layers; ++li) {
         olayer *o = &n->L[li];
@@ -380,16 +380,29 @@ int myea_oracle_set_unit_activations(myea_oracle_net *n, size_t li, const uint32
 int myea_oracle_set_threads(myea_oracle_net *n, int t) { if (!n || t < 1) return MYEA_E_INVALID; n->threads = t; return MYEA_OK; }
 float *myea_oracle_parameters(myea_oracle_net *n) { return n->parameters; }
 float *myea_oracle_gradient(myea_oracle_net *n) { return n->gradient; }
-float *myea_oracle_optimizer_state(myea_oracle_net *n, int k) { return (k >= 0 && k < 4) ? n->opt[k] : NULL; }
+float *myea_oracle_optimizer_state(myea_oracle_net *n, int k) { return (k >= 0 && k < MYEA_STATE_KINDS) ? n->opt[k] : NULL; }
 uint8_t *myea_oracle_masks(myea_oracle_net *n) { return n->masks; }
 
-/* Clear_Training_Arrays NN/Train.cpp:93-126, Clear_Optimizer NN/Train.cpp:128-263 */
+/* Clear_Optimizer NN/Train.cpp:128-263: state vectors to zero (iRPROP steps to rprop_delta_zero, its two losses to the
+ * largest float, NosAdam's running beta2 sum to 0), optimizer_time_step = 0, epoch_time_step = 1 */
+static void clear_optimizer(myea_oracle_net *n)
+{
+    size_t P = n->d.total_parameters;
+    for (int k = 0; k < MYEA_STATE_KINDS; ++k) memset(n->opt[k], 0, P * sizeof(float));
+    for (size_t i = 0; i < P; ++i) n->opt[MYEA_STATE_PREVIOUS_STEPS][i] = n->h.rprop_delta_zero;
+    n->h.loss_rprop = FLT_MAX;
+    n->h.previous_loss_rprop = FLT_MAX;
+    n->h.adam_previous_beta2 = 0.f;
+    n->h.optimizer_time_step = 0.f;
+    n->h.epoch_time_step = 1.f;
+}
+
+/* Clear_Training_Arrays NN/Train.cpp:93-126 */
 int myea_oracle_clear_training_arrays(myea_oracle_net *n)
 {
     size_t P = n->d.total_parameters;
     memset(n->gradient, 0, P * sizeof(float));
-    for (int k = 0; k < 4; ++k) memset(n->opt[k], 0, P * sizeof(float));
-    n->h.optimizer_time_step = 0.f;
+    clear_optimizer(n);
     return MYEA_OK;
 }
 
@@ -1311,21 +1324,91 @@ static void clip_gradient(myea_oracle_net *n)
 
 static float clipf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
+/* Warm_Restarts_Decay NN/Train.cpp:266-283: cosine-annealed rate from the step count BEFORE this update; at the end of a
+ * cycle the optimizer is cleared, the cycle lengthens and its maximum rate decays */
+static float warm_restarts_decay(myea_oracle_net *n)
+{
+    myea_hyper *h = &n->h;
+    float lr = h->warm_restarts_minimum_learning_rate + 0.5f * (h->warm_restarts_maximum_learning_rate - h->warm_restarts_minimum_learning_rate)
+                   * (1.f + cosf(h->optimizer_time_step / h->warm_restarts_T_i * 3.14159265358979323846f));
+    if (h->optimizer_time_step >= h->warm_restarts_T_i) {
+        clear_optimizer(n);
+        h->warm_restarts_T_i *= h->warm_restarts_multiplier;
+        h->warm_restarts_maximum_learning_rate *= h->warm_restarts_decay_learning_rate;
+        if (h->warm_restarts_maximum_learning_rate < h->warm_restarts_minimum_learning_rate) h->warm_restarts_maximum_learning_rate = h->warm_restarts_minimum_learning_rate;
+    }
+    return lr;
+}
+
+/* Euclidean_Norm NN/Neural_Network__Regularization__Max_Norm_Constraints.cpp:48-82 */
+static void max_norm_vector(float *v, size_t n, float max_norm)
+{
+    float s = 0.f;
+    for (size_t i = 0; i < n; ++i) s += v[i] * v[i];
+    s = sqrtf(s);
+    if (s >= max_norm) { float r = max_norm / s; for (size_t i = 0; i < n; ++i) v[i] *= r; }
+}
+
+/* Update_Weight_Regularization__Max_Norm_Constraints NN/Neural_Network__Regularization__Max_Norm_Constraints.cpp:140-529 with
+ * (start, end) = (0, total_weights): every fully-connected neuron's incoming weight vector (hidden and output layers) is
+ * rescaled onto the ball of radius max_norm; for an LSTM block the same is done per weight segment (per cell: cell-input
+ * feed-forward and recurrent; per block: the three gates' feed-forward, recurrent and peephole vectors).  The LSTM tests
+ * are `first index > start`, so a segment that begins at flat index 0 is left alone (:184, :197, ... as written). */
+static void max_norm_segment(myea_oracle_net *n, size_t first, size_t len, int strict)
+{
+    if (strict && first == 0) return;
+    max_norm_vector(n->parameters + first, len, n->h.regularization__max_norm_constraints);
+}
+
+static int max_norm_constraints(myea_oracle_net *n)
+{
+    for (size_t li = 1; li < n->d.n_layers; ++li) {
+        const myea_layer_desc *l = &n->d.layers[li];
+        if (l->type_layer == MYEA_LAYER_RESIDUAL) continue;
+        if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+            for (size_t o = 0; o < n->L[li].H; ++o) max_norm_segment(n, l->first_connection_index + o * n->L[li].In, n->L[li].In, 0);
+        } else if (l->type_layer == MYEA_LAYER_LSTM) {
+            for (int dir = 0; dir < (l->use_bidirectional ? 2 : 1); ++dir) {
+                const olstm *q = &n->L[li].lstm[dir];
+                for (size_t k = 0; k < q->K; ++k) {
+                    for (size_t j = 0; j < q->cpb; ++j) {
+                        max_norm_segment(n, lstm_z_in(l, q, k, j), q->In, 1);
+                        max_norm_segment(n, lstm_z_rec(l, q, k, j), q->C, 1);
+                    }
+                    for (int g = 0; g < 3; ++g) max_norm_segment(n, lstm_gate_in(l, q, k, g), q->In, 1);
+                    for (int g = 0; g < 3; ++g) max_norm_segment(n, lstm_gate_rec(l, q, k, g), q->C, 1);
+                    for (int g = 0; g < 3; ++g) max_norm_segment(n, lstm_peep(l, q, k, g), q->cpb, 1);
+                }
+            }
+        } else return MYEA_E_UNSUPPORTED;
+    }
+    return MYEA_OK;
+}
+
 int myea_oracle_update_parameter(myea_oracle_net *n, size_t B, size_t training_size)
 {
-    (void)B; (void)training_size; /* only used by normalised weight decay, which is off by default */
     if (!n) return MYEA_E_INVALID;
     size_t P = n->d.total_parameters, W = n->d.total_weights;
     myea_hyper *h = &n->h;
     float *g = n->gradient, *w = n->parameters;
+    /* the L1 / L2 gradient terms are called with (batch size, 0, total weights) where the callee expects (start, end, batch
+     * size): both loops are empty, the terms never reach the gradient (NN/Neural_Network.cpp:4729-4740 against
+     * NN/Neural_Network__Regularization__L1.cpp:98-128) - nothing to do here */
     if (h->use_clip_gradient) clip_gradient(n);
-    h->optimizer_time_step += 1.f;
-    float wd = h->regularization__weight_decay;
+    int adam_type = h->type_optimizer_function != MYEA_OPTIMIZER_GD && h->type_optimizer_function != MYEA_OPTIMIZER_IRPROP_PLUS;
+    float scale = 1.f;
+    if (h->use_Warm_Restarts && h->type_optimizer_function != MYEA_OPTIMIZER_IRPROP_PLUS)
+        scale = warm_restarts_decay(n) / (adam_type ? h->adam_learning_rate : h->learning_rate);
+    if (h->type_optimizer_function != MYEA_OPTIMIZER_IRPROP_PLUS) h->optimizer_time_step += 1.f;
+    /* Normalized_Weight_Decay NN/Train.cpp:285-286 */
+    float wd = h->use_normalized_weight_decay ? h->regularization__weight_decay * sqrtf((float)B / ((float)training_size * h->epoch_time_step)) : h->regularization__weight_decay;
+    if (h->regularization__weight_decay == 0.f) wd = 0.f;   /* keeps a call without a training-set size well defined */
     switch (h->type_optimizer_function) {
     case MYEA_OPTIMIZER_GD: {
         /* NN/Neural_Network__Gradient_Descent.cpp:22-159, NN/Neural_Network__Gradient_Descent_Momentum.cpp:22-62,
          * NN/Neural_Network__Nesterov_Accelerated_Gradient.cpp:22-64 */
-        float lr = h->learning_rate, mu = h->learning_momentum;
+        float lr = scale * h->learning_rate, mu = h->learning_momentum;
+        wd *= scale;
         float *dprev = n->opt[MYEA_STATE_PREVIOUS_DELTA];
         long i;
         /* elementwise: the thread split does not change any result (the reference's __OpenMP variants do the same) */
@@ -1347,33 +1430,76 @@ int myea_oracle_update_parameter(myea_oracle_net *n, size_t B, size_t training_s
     }
     case MYEA_OPTIMIZER_ADAM:
     case MYEA_OPTIMIZER_AMSGRAD:
-    case MYEA_OPTIMIZER_ADABOUND: {
-        /* NN/Neural_Network__Adam.cpp:43-97, NN/Neural_Network__AMSGrad.cpp:43-105, NN/Neural_Network__AdaBound.cpp:43-110 */
-        float lr = h->adam_learning_rate, b1 = h->adam_beta1, b2 = h->adam_beta2, eps = h->adam_epsilon, ts = h->optimizer_time_step;
+    case MYEA_OPTIMIZER_ADABOUND:
+    case MYEA_OPTIMIZER_AMSBOUND:
+    case MYEA_OPTIMIZER_NOSADAM: {
+        /* NN/Neural_Network__Adam.cpp:43-97, NN/Neural_Network__AMSGrad.cpp:43-105, NN/Neural_Network__AdaBound.cpp:43-110,
+         * NN/Neural_Network__AMSBound.cpp:43-110, NN/Neural_Network__NosAdam.cpp:43-100 */
+        uint32_t kind = h->type_optimizer_function;
+        float lr = scale * h->adam_learning_rate, b1 = h->adam_beta1, b2 = h->adam_beta2, eps = h->adam_epsilon, ts = h->optimizer_time_step;
         float lr_t = h->use_adam_bias_correction ? (float)(lr * sqrt(1.0 - pow(b2, ts)) / (1.0 - pow(b1, ts))) : lr;
-        float lo = h->learning_rate_final * (1.f - 1.f / (h->learning_gamma * ts + 1.f));
-        float hi = h->learning_rate_final * (1.f + 1.f / (h->learning_gamma * ts));
+        float lo = scale * h->learning_rate_final * (1.f - 1.f / (h->learning_gamma * ts + 1.f));
+        float hi = scale * h->learning_rate_final * (1.f + 1.f / (h->learning_gamma * ts));
+        float b2v = b2;   /* the decay applied to the second moment */
+        if (kind == MYEA_OPTIMIZER_NOSADAM) {
+            float pg = powf(ts, -h->adam_gamma);
+            b2v = h->adam_previous_beta2 / (h->adam_previous_beta2 + pg);
+            h->adam_previous_beta2 += pg;
+        }
         float *m = n->opt[MYEA_STATE_FIRST_MOMENT], *v = n->opt[MYEA_STATE_SECOND_MOMENT], *vh = n->opt[MYEA_STATE_SECOND_MOMENT_HAT];
         long i;
 #pragma omp parallel for schedule(static) num_threads(n->threads)
         for (i = 0; i < (long)P; ++i) {
             float gi = g[i];
             float mi = m[i] = b1 * m[i] + (1.f - b1) * gi;
-            float vi = v[i] = b2 * v[i] + (1.f - b2) * gi * gi;
+            float vi = v[i] = b2v * v[i] + (1.f - b2v) * gi * gi;
             float reg = (wd != 0.f) ? ((size_t)i < W ? 1.f : 0.f) * wd * w[i] : 0.f;
             float step;
-            if (h->type_optimizer_function == MYEA_OPTIMIZER_ADAM) step = lr_t * mi / (sqrtf(vi) + eps);
-            else if (h->type_optimizer_function == MYEA_OPTIMIZER_AMSGRAD) {
+            if (kind == MYEA_OPTIMIZER_ADAM || kind == MYEA_OPTIMIZER_NOSADAM) step = lr_t * mi / (sqrtf(vi) + eps);
+            else if (kind == MYEA_OPTIMIZER_AMSGRAD) {
                 float hh = vh[i] = vh[i] > vi ? vh[i] : vi;
                 step = lr_t * mi / (sqrtf(hh) + eps);
+            } else if (kind == MYEA_OPTIMIZER_AMSBOUND) {
+                float hh = vh[i] = vh[i] > vi ? vh[i] : vi;
+                step = clipf(lr_t / (sqrtf(hh) + eps), lo, hi) * mi;
             } else step = clipf(lr_t / (sqrtf(vi) + eps), lo, hi) * mi;
             if (wd != 0.f) w[i] -= step + reg; else w[i] -= step;
             g[i] = 0.f;
         }
         break;
     }
-    default: return MYEA_E_UNSUPPORTED;
+    case MYEA_OPTIMIZER_IRPROP_PLUS: {
+        /* NN/Neural_Network__iRPROP_plus.cpp:28-117: sign-based steps; a sign change shrinks the step, takes the last weight change
+         * back when the loss got worse, and forgets the slope */
+        int worse = h->loss_rprop > h->previous_loss_rprop;
+        float *dprev = n->opt[MYEA_STATE_PREVIOUS_DELTA], *st = n->opt[MYEA_STATE_PREVIOUS_STEPS], *gp = n->opt[MYEA_STATE_PREVIOUS_DERIVATIVES];
+        for (size_t i = 0; i < P; ++i) {
+            float gi = g[i], s = gp[i] * gi;
+            if (s > 0.f) {
+                float d = st[i] * h->rprop_increase_factor;
+                st[i] = d = d < h->rprop_delta_max ? d : h->rprop_delta_max;
+                dprev[i] = -sign_f(gi) * d;
+                w[i] += dprev[i];
+                gp[i] = gi;
+            } else if (s < 0.f) {
+                float d = st[i] * h->rprop_decrease_factor;
+                st[i] = d > h->rprop_delta_min ? d : h->rprop_delta_min;
+                if (worse) w[i] -= dprev[i];
+                gp[i] = 0.f;
+            } else {
+                dprev[i] = -sign_f(gi) * st[i];
+                w[i] += dprev[i];
+                gp[i] = gi;
+            }
+            g[i] = 0.f;
+        }
+        break;
     }
+    default:
+        h->optimizer_time_step -= 1.f;
+        return MYEA_E_UNSUPPORTED;
+    }
+    if (h->regularization__max_norm_constraints != 0.f) return max_norm_constraints(n);
     return MYEA_OK;
 }
 
