@@ -84,7 +84,7 @@ enum {
 };
 enum {
     MYEA_ACCURACY_NONE = 0, MYEA_ACCURACY_CROSS_ENTROPY = 1, MYEA_ACCURACY_DIRECTIONAL = 2,
-    MYEA_ACCURACY_DISTANCE = 3, MYEA_ACCURACY_SIGN = 5
+    MYEA_ACCURACY_DISTANCE = 3, MYEA_ACCURACY_R = 4, MYEA_ACCURACY_SIGN = 5
 };
 
 /* Enum_Type_State_Propagation.hpp */
@@ -197,13 +197,17 @@ typedef struct myea_hyper {
 } myea_hyper;
 
 /* Loss / accuracy accumulators (ptr_array_loss_values, ptr_array_number_loss,
- * ptr_array_accuracy_values[0], ptr_array_number_bit_fail; merged as Merge__Post__Training does,
+ * ptr_array_accuracy_values[0..4], ptr_array_number_bit_fail; merged as Merge__Post__Training does,
  * Neural_Network__Merge.cpp:52-98). */
 typedef struct myea_loss_state {
     double   loss_values;       /* sum of per-output loss terms since the last reset */
     uint64_t number_loss;       /* number of terms */
-    double   accuracy_value;    /* ptr_array_accuracy_values[0] */
+    double   accuracy_value;    /* ptr_array_accuracy_values[0]: hits; with the R accuracy the sum of the desired values */
     uint64_t number_bit_fail;
+    /* R accuracy only (Pearson correlation over every output entry): ptr_array_accuracy_values[1..4] =
+     * sum of the predicted values; then, from Compute__Accuracy__R, the numerator sum (d - mean_d)(y - mean_y)
+     * and the two denominators sum (d - mean_d)^2, sum (y - mean_y)^2 */
+    double   accuracy_r[4];
 } myea_loss_state;
 
 /* kinds for the optimizer-state and tensor taps */
@@ -328,6 +332,34 @@ int myea_hip_update_derivative_weight(myea_hip_net *net, size_t batch_size_recei
 /* Neural_Network::Update_Parameter (Data.hpp:849; Neural_Network.cpp:4719-4908): clip-by-global-norm
  * then the fused optimizer; zeroes the gradient. */
 int myea_hip_update_parameter(myea_hip_net *net, size_t batch_size_received, size_t training_size_received);
+
+/* Neural_Network::Compute__Loss (Neural_Network__Compute__Loss__Loop.cpp:22-140, Neural_Network__Recurrent_Compute__Loss__Loop.cpp:20-140):
+ * the evaluation twin of Compute__Error - the same loss and accuracy accumulation over the output layer's values, no
+ * delta is written.  Used after a Forward_Pass in the inference state by Dataset::Testing (Dataset.cpp:7829-7860). */
+int myea_hip_compute_loss(myea_hip_net *net, size_t batch_size_received, const float *desired_outputs, int desired_on_device);
+
+/* Neural_Network::Compute__Accuracy__R (Neural_Network__Compute__R__Loop.cpp:22-90, Neural_Network__Recurrent_Compute__R__Loop.cpp):
+ * second pass of the R accuracy.  The reference divides its two running sums by the number of entries in place
+ * (Dataset::Measure_Accuracy, Dataset.cpp:7712-7713) and reads them back as the means; here the caller passes the
+ * means (from myea_hip_get_loss) and the call adds to accuracy_r[1..3]. */
+int myea_hip_compute_accuracy_r(myea_hip_net *net, size_t batch_size_received, const float *desired_outputs, int desired_on_device,
+                                float desired_mean, float predicted_mean);
+
+/* Device-side replacement of Dataset_Mini_Batch::Increment_Mini_Batch (Dataset__Mini_Batch.cpp:290-314), which
+ * re-points an array of row pointers at the shuffled examples: copies rows `index[0..B)` of a dataset resident in
+ * HBM ([examples][row_floats], fp32) into the contiguous batch `device_batch` ([B][row_floats]), ready to be
+ * handed to forward_pass / compute_error / compute_loss with on_device = 1.  `index` is a host array, or a device
+ * array when `index_on_device` != 0 (a whole epoch's permutation uploaded once).  No bound check on device
+ * indices; host indices are checked against `dataset_examples`. */
+int myea_hip_gather_examples(myea_hip_net *net, float *device_batch, const float *device_dataset, size_t dataset_examples,
+                             size_t row_floats, const uint64_t *index, int index_on_device, size_t batch_size_received);
+
+/* Device memory for a dataset kept in HBM (the reference's Dataset<T> keeps one host allocation per side and an array of
+ * row pointers into it, Dataset.cpp `Allocate`; its CUDA twin copies both to the device, Dataset_Manager.cu).  `floats`
+ * fp32 values, filled from `host` when that is not NULL.  The pointer is a plain device address: valid as `inputs` /
+ * `desired_outputs` with on_device = 1 and as the source or destination of myea_hip_gather_examples. */
+int myea_hip_device_buffer_create(size_t floats, const float *host, float **out_device);
+int myea_hip_device_buffer_destroy(float *device);
 
 /* Reset__Loss / the merged loss counters (Neural_Network__Merge.cpp:52-98).  get synchronises. */
 int myea_hip_reset_loss(myea_hip_net *net);

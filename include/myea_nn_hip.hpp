@@ -12,6 +12,7 @@
 
 #include <cstdio>
 #include <cfloat>
+#include <cmath>
 #include <cstring>
 #include <vector>
 
@@ -207,12 +208,94 @@ public:
         PullState();
     }
 
-    // merged loss counters (Neural_Network__Merge.cpp:52-98); mean of the accumulated per-output terms
-    T_ Get__Loss()
+    // Compute__Loss (Neural_Network__Compute__Loss__Loop.cpp:22): loss / accuracy of the last forward pass, no delta
+    void Compute__Loss(size_t batch_size_received, T_ const *const *ptr_array_desireds_outputs)
+    {
+        if (!Need("Compute__Loss") || !PushFields("Compute__Loss")) return;
+        const size_t row = (size_t)desc_.layers[desc_.n_layers - 1].n_units * desc_.number_recurrent_depth;
+        if (!Flatten("Compute__Loss", batch_size_received, ptr_array_desireds_outputs, row)) return;
+        Ok("Compute__Loss", myea_hip_compute_loss(net_, batch_size_received, rows_.data(), 0));
+    }
+    // Compute__Accuracy__R (Neural_Network__Compute__R__Loop.cpp:22): the means are ptr_array_accuracy_values[0] / [1],
+    // which Dataset::Measure_Accuracy has divided by the number of entries (R_Means)
+    void Compute__Accuracy__R(size_t batch_size_received, T_ const *const *ptr_array_desireds_outputs)
+    {
+        if (!Need("Compute__Accuracy__R") || !PushFields("Compute__Accuracy__R")) return;
+        const size_t row = (size_t)desc_.layers[desc_.n_layers - 1].n_units * desc_.number_recurrent_depth;
+        if (!Flatten("Compute__Accuracy__R", batch_size_received, ptr_array_desireds_outputs, row)) return;
+        Ok("Compute__Accuracy__R", myea_hip_compute_accuracy_r(net_, batch_size_received, rows_.data(), 0, r_mean_desired_, r_mean_predicted_));
+    }
+    // device-resident variants: [batch][T * width] rows already in HBM (a dataset kept on the GPU)
+    void Forward_Pass__Device(size_t B, T_ const *dev) { if (Need("Forward_Pass") && PushFields("Forward_Pass")) Ok("Forward_Pass", myea_hip_forward_pass(net_, B, dev, 1)); }
+    void Compute__Error__Device(size_t B, T_ const *dev) { if (Need("Compute__Error") && PushFields("Compute__Error")) Ok("Compute__Error", myea_hip_compute_error(net_, B, dev, 1)); }
+    void Compute__Loss__Device(size_t B, T_ const *dev) { if (Need("Compute__Loss") && PushFields("Compute__Loss")) Ok("Compute__Loss", myea_hip_compute_loss(net_, B, dev, 1)); }
+    void Compute__Accuracy__R__Device(size_t B, T_ const *dev)
+    { if (Need("Compute__Accuracy__R") && PushFields("Compute__Accuracy__R")) Ok("Compute__Accuracy__R", myea_hip_compute_accuracy_r(net_, B, dev, 1, r_mean_desired_, r_mean_predicted_)); }
+    // the in-place division of the two running sums in Dataset::Measure_Accuracy (Dataset.cpp:7712-7713)
+    void R_Means(size_t number_entries)
     {
         myea_loss_state s;
-        if (!Need("Get__Loss") || !Ok("Get__Loss", myea_hip_get_loss(net_, &s)) || s.number_loss == 0) return 0.f;
-        return (T_)(s.loss_values / (double)s.number_loss);
+        if (!Get__Loss_State(&s) || number_entries == 0) return;
+        r_mean_desired_ = (T_)(s.accuracy_value / (double)number_entries);
+        r_mean_predicted_ = (T_)(s.accuracy_r[0] / (double)number_entries);
+    }
+
+    // Get__Loss (Neural_Network__Loss.cpp:103-214) / Get__Accuracy (Neural_Network__Accuracy.cpp:88-113); dataset kinds as
+    // Enum_Type_Dataset.hpp: 0 none (read the counters), 1 testing, 2 training, 3 validation (the stored values)
+    enum { TYPE_DATASET_NONE = 0, TYPE_DATASET_TESTING = 1, TYPE_DATASET_TRAINING = 2, TYPE_DATASET_VALIDATION = 3 };
+    T_ loss_training = FLT_MAX, loss_validating = FLT_MAX, loss_testing = FLT_MAX;
+    T_ accuracy_training = 0.f, accuracy_validating = 0.f, accuracy_testing = 0.f;
+    size_t number_accuracy_trial = 0;
+    size_t Get__Output_Size() const { return desc_.layers[desc_.n_layers - 1].n_units; }
+    T_ Get__Loss(unsigned int type_dataset = TYPE_DATASET_NONE)
+    {
+        switch (type_dataset) {
+        case TYPE_DATASET_TRAINING: return loss_training;
+        case TYPE_DATASET_VALIDATION: return loss_validating;
+        case TYPE_DATASET_TESTING: return loss_testing;
+        case TYPE_DATASET_NONE: break;
+        default: return 1.f;
+        }
+        myea_loss_state s;
+        if (!Get__Loss_State(&s)) return 1.f;
+        const double n = (double)s.number_loss;
+        switch (type_loss_function) {
+        case MYEA_LOSS_L1: case MYEA_LOSS_L2: return (T_)s.loss_values;
+        case MYEA_LOSS_ME: case MYEA_LOSS_MAE: case MYEA_LOSS_MSE: case MYEA_LOSS_MAPE: case MYEA_LOSS_SMAPE:
+            return s.number_loss ? (T_)(s.loss_values / n) : 1.f;
+        case MYEA_LOSS_RMSE: return s.number_loss ? (T_)std::sqrt(s.loss_values / n) : 1.f;
+        case MYEA_LOSS_CROSS_ENTROPY: return s.number_loss ? (T_)(s.loss_values / (double)(s.number_loss / Get__Output_Size())) : FLT_MAX;
+        case MYEA_LOSS_BIT: return (T_)s.number_bit_fail;
+        default: return 1.f;
+        }
+    }
+    T_ Get__Accuracy(unsigned int type_dataset = TYPE_DATASET_NONE)
+    {
+        switch (type_dataset) {
+        case TYPE_DATASET_TRAINING: return accuracy_training;
+        case TYPE_DATASET_VALIDATION: return accuracy_validating;
+        case TYPE_DATASET_TESTING: return accuracy_testing;
+        case TYPE_DATASET_NONE: break;
+        default: return 0.f;
+        }
+        myea_loss_state s;
+        if (!Get__Loss_State(&s)) return 0.f;
+        if (type_accuracy_function == MYEA_ACCURACY_R) {
+            const double den = s.accuracy_r[2] * s.accuracy_r[3];
+            const double r = den == 0.0 ? 0.0 : s.accuracy_r[1] / (std::sqrt(s.accuracy_r[2]) * std::sqrt(s.accuracy_r[3]));
+            return (T_)(r < -1.0 ? -1.0 : (r > 1.0 ? 1.0 : r));
+        }
+        return number_accuracy_trial == 0 ? 0.f : (T_)(s.accuracy_value / (double)number_accuracy_trial * 100.0);
+    }
+    void Set__Loss(unsigned int type_dataset, T_ v)
+    {
+        if (type_dataset == TYPE_DATASET_TRAINING) loss_training = v; else if (type_dataset == TYPE_DATASET_VALIDATION) loss_validating = v;
+        else if (type_dataset == TYPE_DATASET_TESTING) loss_testing = v; else std::printf("Set__Loss: ERROR: Loss type (%u) is not managed in the switch.\n", type_dataset);
+    }
+    void Set__Accuracy(unsigned int type_dataset, T_ v)
+    {
+        if (type_dataset == TYPE_DATASET_TRAINING) accuracy_training = v; else if (type_dataset == TYPE_DATASET_VALIDATION) accuracy_validating = v;
+        else if (type_dataset == TYPE_DATASET_TESTING) accuracy_testing = v; else std::printf("Set__Accuracy: ERROR: Accuracy type (%u) is not managed in the switch.\n", type_dataset);
     }
     bool Get__Loss_State(myea_loss_state *out) { return Need("Get__Loss_State") && Ok("Get__Loss_State", myea_hip_get_loss(net_, out)); }
 
@@ -223,6 +306,7 @@ private:
     myea_net_desc desc_;
     myea_hip_net *net_ = nullptr;
     std::vector<T_> rows_;
+    T_ r_mean_desired_ = 0.f, r_mean_predicted_ = 0.f;
 
     static bool Fail(const char *fn, const char *what) { std::printf("%s: ERROR: %s.\n", fn, what); return false; }
     bool Ok(const char *fn, int rc) { if (rc != MYEA_OK) { Fail(fn, myea_hip_last_error()); return false; } return true; }

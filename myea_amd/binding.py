@@ -26,7 +26,7 @@ OPTIMIZER = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP
 DROPOUT = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
 NORMALIZATION = dict(NONE=0, BATCH_NORMALIZATION=1, BATCH_RENORMALIZATION=2)
 LOSS = dict(NONE=0, BIT=1, CROSS_ENTROPY=2, L1=3, L2=4, MAE=5, MAPE=6, ME=9, MSE=10, RMSE=11, SMAPE=12)
-ACCURACY = dict(NONE=0, CROSS_ENTROPY=1, DIRECTIONAL=2, DISTANCE=3, SIGN=5)
+ACCURACY = dict(NONE=0, CROSS_ENTROPY=1, DIRECTIONAL=2, DISTANCE=3, R=4, SIGN=5)
 STATE_INFERENCE, STATE_TRAINING = 0, 1
 OPT_STATE = dict(PREVIOUS_DELTA=0, FIRST_MOMENT=1, SECOND_MOMENT=2, SECOND_MOMENT_HAT=3, PREVIOUS_STEPS=4, PREVIOUS_DERIVATIVES=5)
 TENSOR = dict(OUTPUTS=0, SUMMATIONS=1, ERRORS=2, NORM_HATS=3, NORM_MEANS=4, NORM_VARIANCES=5,
@@ -86,7 +86,7 @@ class Hyper(C.Structure):
 
 class LossState(C.Structure):
     _fields_ = [("loss_values", C.c_double), ("number_loss", C.c_uint64), ("accuracy_value", C.c_double),
-                ("number_bit_fail", C.c_uint64)]
+                ("number_bit_fail", C.c_uint64), ("accuracy_r", C.c_double * 4)]
 
 
 # every symbol include/myea_hip.h declares
@@ -95,6 +95,7 @@ ABI_SYMBOLS = [
     "myea_hip_synchronize", "myea_hip_last_error", "myea_hip_set_hyper", "myea_hip_get_hyper",
     "myea_hip_set_state_propagation", "myea_hip_upload_parameters", "myea_hip_download_parameters",
     "myea_hip_upload_optimizer_state", "myea_hip_download_optimizer_state", "myea_hip_upload_masks", "myea_hip_set_unit_activations",
+    "myea_hip_compute_loss", "myea_hip_compute_accuracy_r", "myea_hip_gather_examples", "myea_hip_device_buffer_create", "myea_hip_device_buffer_destroy",
     "myea_hip_clear_training_arrays", "myea_hip_forward_pass", "myea_hip_compute_error", "myea_hip_backward_pass",
     "myea_hip_update_derivative_weight", "myea_hip_update_parameter", "myea_hip_reset_loss", "myea_hip_get_loss",
     "myea_hip_download_gradient", "myea_hip_upload_gradient", "myea_hip_download_tensor",
@@ -144,6 +145,11 @@ def load_library(path=LIB_PATH):
     lib.myea_hip_update_parameter.argtypes = [vp, sz, sz]
     lib.myea_hip_reset_loss.argtypes = [vp]
     lib.myea_hip_get_loss.argtypes = [vp, P(LossState)]
+    lib.myea_hip_compute_loss.argtypes = [vp, sz, vp, i32]
+    lib.myea_hip_compute_accuracy_r.argtypes = [vp, sz, vp, i32, C.c_float, C.c_float]
+    lib.myea_hip_gather_examples.argtypes = [vp, vp, vp, sz, sz, vp, i32, sz]
+    lib.myea_hip_device_buffer_create.argtypes = [sz, vp, P(vp)]
+    lib.myea_hip_device_buffer_destroy.argtypes = [vp]
     lib.myea_hip_download_tensor.argtypes = [vp, sz, i32, vp, sz]
     lib.myea_hip_profile_enable.argtypes = [vp, i32]
     lib.myea_hip_profile_read.argtypes = [vp, i32, P(C.c_uint64), P(C.c_double), P(C.c_double)]
@@ -305,6 +311,23 @@ class HipNetwork:
         if isinstance(desired, np.ndarray):
             desired = np.ascontiguousarray(desired, dtype=np.float32)
         self._check(self.lib.myea_hip_compute_error(self.handle, batch_size, _ptr(desired), int(on_device)))
+
+    def Compute__Loss(self, batch_size, desired, on_device=False):
+        if isinstance(desired, np.ndarray):
+            desired = np.ascontiguousarray(desired, dtype=np.float32)
+        self._check(self.lib.myea_hip_compute_loss(self.handle, batch_size, _ptr(desired), int(on_device)))
+
+    def Compute__Accuracy__R(self, batch_size, desired, desired_mean, predicted_mean, on_device=False):
+        if isinstance(desired, np.ndarray):
+            desired = np.ascontiguousarray(desired, dtype=np.float32)
+        self._check(self.lib.myea_hip_compute_accuracy_r(self.handle, batch_size, _ptr(desired), int(on_device), desired_mean, predicted_mean))
+
+    def gather_examples(self, device_batch, device_dataset, dataset_examples, row_floats, index, batch_size, index_on_device=False):
+        """device_batch / device_dataset: device pointers (int or an object with data_ptr()); index: uint64 array (host) or device pointer"""
+        if isinstance(index, np.ndarray):
+            index = np.ascontiguousarray(index, dtype=np.uint64)
+        self._check(self.lib.myea_hip_gather_examples(self.handle, _ptr(device_batch), _ptr(device_dataset), dataset_examples, row_floats,
+                                                      _ptr(index), int(index_on_device), batch_size))
 
     def Backward_Pass(self, batch_size): self._check(self.lib.myea_hip_backward_pass(self.handle, batch_size))
 

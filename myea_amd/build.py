@@ -40,11 +40,12 @@ def build(verbose=False):
         _run(["gcc", "-O2", "-fPIC", "-std=c11", "-Wall", "-c", os.path.join(CSRC, src), "-o", obj])
         objs.append(obj)
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
-    # the C++ adaptor's check program (host code only; links the C ABI)
+    # the C++ adaptor's check programs (host code only; link the C ABI)
     root = os.path.dirname(HERE)
-    _run(["g++", "-O2", "-std=c++17", "-Wall", os.path.join(root, "tests", "cpp", "adaptor_check.cpp"), "-o",
-          os.path.join(root, "tests", "cpp", "adaptor_check"), "-L" + CSRC, "-lmyea_hip", "-Wl,-rpath," + CSRC,
-          "-Wl,-rpath,$ORIGIN/../../myea_amd/csrc"])
+    for name in ("adaptor_check", "dataset_check"):
+        _run(["g++", "-O2", "-std=c++17", "-Wall", os.path.join(root, "tests", "cpp", name + ".cpp"), "-o",
+              os.path.join(root, "tests", "cpp", name), "-L" + CSRC, "-lmyea_hip", "-Wl,-rpath," + CSRC,
+              "-Wl,-rpath,$ORIGIN/../../myea_amd/csrc"])
     return LIB
 
 

@@ -208,10 +208,10 @@ __device__ __forceinline__ float sign_f(float v) { return v > 0.f ? 1.f : (v < 0
 
 __global__ __launch_bounds__(kBlock) void compute_error_kernel(ErrorParams p)
 {
-    __shared__ float red[4][kBlock / 64];
+    __shared__ float red[5][kBlock / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const size_t nrows = (p.T - p.first_t) * p.B;
-    float loss = 0.f, cnt = 0.f, acc = 0.f, bits = 0.f;
+    float loss = 0.f, cnt = 0.f, acc = 0.f, bits = 0.f, sum_y = 0.f;
     // wavefronts stride over the rows and keep their sums in registers: one set of fp64 atomics per workgroup
     for (size_t rid = (size_t)blockIdx.x * (kBlock / 64) + wave; rid < nrows; rid += (size_t)gridDim.x * (kBlock / 64)) {
         const size_t t = p.first_t + rid / p.B, b = rid % p.B;
@@ -267,18 +267,66 @@ __global__ __launch_bounds__(kBlock) void compute_error_kernel(ErrorParams p)
             case MYEA_ACCURACY_SIGN:
                 if (sign_f(de) == sign_f(yo) || (sign_f(de) == 0.f && yo >= -1.192092896e-07f && yo <= 1.192092896e-07f)) acc += 1.f;
                 break;
+            case MYEA_ACCURACY_R: acc += de; sum_y += yo; break;  // running sums of the desired and the predicted values
             default: break;
             }
+            if (!p.write_delta) continue;  // Compute__Loss: the same accumulation, no delta
             const float q = p.rnn_pre_quirk ? pre[0] : pre[j];
             err[j] = af_derive(p.unit_act ? p.unit_act[j] : p.act, q, p.unit_steep ? p.unit_steep[j] : p.steep, yo) * diff;
         }
     }
-    loss = wave_sum(loss); cnt = wave_sum(cnt); acc = wave_sum(acc); bits = wave_sum(bits);
-    if (lane == 0) { red[0][wave] = loss; red[1][wave] = cnt; red[2][wave] = acc; red[3][wave] = bits; }
+    loss = wave_sum(loss); cnt = wave_sum(cnt); acc = wave_sum(acc); bits = wave_sum(bits); sum_y = wave_sum(sum_y);
+    if (lane == 0) { red[0][wave] = loss; red[1][wave] = cnt; red[2][wave] = acc; red[3][wave] = bits; red[4][wave] = sum_y; }
     __syncthreads();
-    if (threadIdx.x < 4) {
+    if (threadIdx.x < 5) {
         const float v = red[threadIdx.x][0] + red[threadIdx.x][1] + red[threadIdx.x][2] + red[threadIdx.x][3];
         if (v != 0.f) atomicAdd(&p.loss_acc[threadIdx.x], (double)v);
+    }
+}
+
+// FF / RNN__Compute__Accuracy__R (NN/Neural_Network__Compute__R__Loop.cpp:38-90, NN/Neural_Network__Recurrent_Compute__R__Loop.cpp:20-75):
+// numerator and the two denominators of the Pearson correlation into loss_acc[5..7]
+__global__ __launch_bounds__(kBlock) void accuracy_r_kernel(ErrorParams p, float mean_d, float mean_y)
+{
+    __shared__ float red[3][kBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t nrows = (p.T - p.first_t) * p.B;
+    float num = 0.f, den_d = 0.f, den_y = 0.f;
+    for (size_t rid = (size_t)blockIdx.x * (kBlock / 64) + wave; rid < nrows; rid += (size_t)gridDim.x * (kBlock / 64)) {
+        const size_t t = p.first_t + rid / p.B, b = rid % p.B;
+        const float *y = p.values + (t * p.Bmax + b) * p.H, *d = p.desired + (b * p.T + t) * p.H;
+        for (size_t j = lane; j < p.H; j += 64) {
+            const float dd = d[j] - mean_d, dy = y[j] - mean_y;
+            num += dd * dy; den_d += dd * dd; den_y += dy * dy;
+        }
+    }
+    num = wave_sum(num); den_d = wave_sum(den_d); den_y = wave_sum(den_y);
+    if (lane == 0) { red[0][wave] = num; red[1][wave] = den_d; red[2][wave] = den_y; }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        const float v = red[threadIdx.x][0] + red[threadIdx.x][1] + red[threadIdx.x][2] + red[threadIdx.x][3];
+        if (v != 0.f) atomicAdd(&p.loss_acc[5 + threadIdx.x], (double)v);
+    }
+}
+
+// rows index[0..B) of a resident dataset -> one contiguous batch (Dataset_Mini_Batch::Increment_Mini_Batch,
+// NN/Dataset__Mini_Batch.cpp:290-314, re-points row pointers; here the rows are copied on the device)
+__global__ __launch_bounds__(kBlock) void gather_rows_kernel(size_t B, size_t row_floats, const unsigned long long *__restrict__ index,
+                                                             const float *__restrict__ src, float *__restrict__ dst)
+{
+    const bool vec = (row_floats & 3) == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
+    if (vec) {
+        const size_t r4 = row_floats / 4, n = B * r4;
+        for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+            const size_t b = i / r4, j = i - b * r4;
+            reinterpret_cast<f32x4 *>(dst)[i] = reinterpret_cast<const f32x4 *>(src + index[b] * row_floats)[j];
+        }
+    } else {
+        const size_t n = B * row_floats;
+        for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+            const size_t b = i / row_floats, j = i - b * row_floats;
+            dst[i] = src[index[b] * row_floats + j];
+        }
     }
 }
 
@@ -621,6 +669,23 @@ int launch_compute_error(hipStream_t s, const ErrorParams &p)
     if (p.T <= p.first_t || p.B == 0 || p.H == 0) return MYEA_OK;
     const size_t nrows = (p.T - p.first_t) * p.B;
     hipLaunchKernelGGL(compute_error_kernel, dim3(grid_for(nrows, kBlock / 64, 1024)), dim3(kBlock), 0, s, p);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_accuracy_r(hipStream_t s, const ErrorParams &p, float desired_mean, float predicted_mean)
+{
+    if (p.T <= p.first_t || p.B == 0 || p.H == 0) return MYEA_OK;
+    const size_t nrows = (p.T - p.first_t) * p.B;
+    hipLaunchKernelGGL(accuracy_r_kernel, dim3(grid_for(nrows, kBlock / 64, 1024)), dim3(kBlock), 0, s, p, desired_mean, predicted_mean);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_gather_rows(hipStream_t s, size_t B, size_t row_floats, const unsigned long long *index, const float *src, float *dst)
+{
+    if (B == 0 || row_floats == 0) return MYEA_OK;
+    hipLaunchKernelGGL(gather_rows_kernel, dim3(grid_for(B * row_floats / 4 + 1, kBlock, 8192)), dim3(kBlock), 0, s, B, row_floats, index, src, dst);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

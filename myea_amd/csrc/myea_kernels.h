@@ -116,9 +116,13 @@ struct ErrorParams {
     float accuracy_variance, bit_fail_limit;
     size_t first_t;              // number_time_delays
     int rnn_pre_quirk;           // RNN head: every unit reads the first unit's pre-activation
-    double *loss_acc;            // [0]=loss sum [1]=count [2]=accuracy [3]=bit fails
+    double *loss_acc;            // [0]=loss sum [1]=count [2]=accuracy (R: sum desired) [3]=bit fails [4]=R: sum predicted
+                                 // [5..7]=R: numerator, desired / predicted denominators
+    int write_delta;             // 0 = Compute__Loss (accumulate only)
 };
 int launch_compute_error(hipStream_t s, const ErrorParams &p);
+int launch_accuracy_r(hipStream_t s, const ErrorParams &p, float desired_mean, float predicted_mean);
+int launch_gather_rows(hipStream_t s, size_t B, size_t row_floats, const unsigned long long *index, const float *src, float *dst);
 
 // [B][T][W] (example rows) -> [T][Bmax][W]
 int launch_scatter_time_major(hipStream_t s, size_t B, size_t T, size_t W, size_t Bmax, const float *src, float *dst);

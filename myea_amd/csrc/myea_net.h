@@ -58,7 +58,8 @@ struct Net {
     unsigned longest_segment = 0;
     std::vector<DevLayer> L;
     float *tmp1 = nullptr, *tmp2 = nullptr, *scratch = nullptr, *stage_in = nullptr, *stage_out = nullptr;
-    double *loss_acc = nullptr;
+    double *loss_acc = nullptr;                  // 8 doubles, see ErrorParams::loss_acc
+    unsigned long long *index_stage = nullptr;   // [Bmax] example indices of a gathered batch
 
     bool profiling = false, open_event = false;
     std::vector<ProfEvent> pending, free_events;
@@ -68,6 +69,10 @@ struct Net {
     ~Net();
     int create(const myea_net_desc &desc);
     int clear_optimizer();
+    int output_error_params(size_t B, const float *desired, int on_device, const char *fn, ErrorParams *p);
+    int compute_loss(size_t B, const float *desired, int on_device);
+    int compute_accuracy_r(size_t B, const float *desired, int on_device, float desired_mean, float predicted_mean);
+    int gather_examples(float *dst, const float *src, size_t examples, size_t row_floats, const uint64_t *index, int index_on_device, size_t B);
     int build_max_norm_segments();
     float warm_restarts_decay(int *rc);
 

@@ -230,9 +230,11 @@ int Net::create(const myea_net_desc &desc)
     MYEA_TRY(dev_alloc(&stage_out, T * B * L[d.n_layers - 1].H));
     {
         void *q = nullptr;
-        MYEA_HIP_TRY(hipMalloc(&q, 4 * sizeof(double)));
+        MYEA_HIP_TRY(hipMalloc(&q, 8 * sizeof(double)));
         loss_acc = static_cast<double *>(q);
-        MYEA_HIP_TRY(hipMemset(loss_acc, 0, 4 * sizeof(double)));
+        MYEA_HIP_TRY(hipMemset(loss_acc, 0, 8 * sizeof(double)));
+        MYEA_HIP_TRY(hipMalloc(&q, B * sizeof(unsigned long long)));
+        index_stage = static_cast<unsigned long long *>(q);
     }
     MYEA_HIP_TRY(hipDeviceSynchronize());
     return MYEA_OK;
@@ -250,7 +252,7 @@ Net::~Net()
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
-    fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc);
+    fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc); fr(index_stage);
     for (ProfEvent &e : pending) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
     for (ProfEvent &e : free_events) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
 }
@@ -446,13 +448,14 @@ int Net::forward_residual_block(size_t ri, size_t B)
 }
 
 // ---- Compute__Error -------------------------------------------------------------------------------------------
-int Net::compute_error(size_t B, const float *desired, int on_device)
+// what Compute__Error, Compute__Loss and Compute__Accuracy__R share: the output layer's tensors and the staged targets
+int Net::output_error_params(size_t B, const float *desired, int on_device, const char *fn, ErrorParams *out)
 {
-    if (!desired) { set_last_error("Compute__Error: null desired outputs"); return MYEA_E_INVALID; }
-    if (B == 0 || B > d.batch_size) { set_last_error("Compute__Error: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
+    if (!desired) { set_last_error("%s: null desired outputs", fn); return MYEA_E_INVALID; }
+    if (B == 0 || B > d.batch_size) { set_last_error("%s: batch size (%zu) > maximum batch size (%u)", fn, B, d.batch_size); return MYEA_E_BATCH; }
     const size_t lo = d.n_layers - 1, T = d.number_recurrent_depth;
     const myea_layer_desc &l = d.layers[lo];
-    if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("Compute__Error: the output layer must be fully connected"); return MYEA_E_UNSUPPORTED; }
+    if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("%s: the output layer must be fully connected", fn); return MYEA_E_UNSUPPORTED; }
     DevLayer &o = L[lo];
     const float *dsrc = desired;
     if (!on_device) {
@@ -472,7 +475,46 @@ int Net::compute_error(size_t B, const float *desired, int on_device)
     p.first_t = T > 1 ? h.number_time_delays : 0;
     p.rnn_pre_quirk = T > 1;
     p.loss_acc = loss_acc;
+    p.write_delta = 1;
+    *out = p;
+    return MYEA_OK;
+}
+
+int Net::compute_error(size_t B, const float *desired, int on_device)
+{
+    ErrorParams p;
+    MYEA_TRY(output_error_params(B, desired, on_device, "Compute__Error", &p));
     return launch_compute_error(stream, p);
+}
+
+// Compute__Loss (NN/Neural_Network__Compute__Loss__Loop.cpp:22-140): loss and accuracy of the values the last forward pass left
+int Net::compute_loss(size_t B, const float *desired, int on_device)
+{
+    ErrorParams p;
+    MYEA_TRY(output_error_params(B, desired, on_device, "Compute__Loss", &p));
+    p.write_delta = 0;
+    return launch_compute_error(stream, p);
+}
+
+int Net::compute_accuracy_r(size_t B, const float *desired, int on_device, float desired_mean, float predicted_mean)
+{
+    ErrorParams p;
+    MYEA_TRY(output_error_params(B, desired, on_device, "Compute__Accuracy__R", &p));
+    return launch_accuracy_r(stream, p, desired_mean, predicted_mean);
+}
+
+int Net::gather_examples(float *dst, const float *src, size_t examples, size_t row_floats, const uint64_t *index, int index_on_device, size_t B)
+{
+    if (!dst || !src || !index) { set_last_error("gather_examples: null argument"); return MYEA_E_INVALID; }
+    const unsigned long long *dindex = reinterpret_cast<const unsigned long long *>(index);
+    if (!index_on_device) {
+        if (B > d.batch_size) { set_last_error("gather_examples: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
+        for (size_t b = 0; b < B; ++b)
+            if (index[b] >= examples) { set_last_error("gather_examples: index[%zu] = %llu outside the %zu examples", b, (unsigned long long)index[b], examples); return MYEA_E_INVALID; }
+        MYEA_HIP_TRY(hipMemcpyAsync(index_stage, index, B * sizeof(unsigned long long), hipMemcpyHostToDevice, stream));
+        dindex = index_stage;
+    }
+    return launch_gather_rows(stream, B, row_floats, dindex, src, dst);
 }
 
 // ---- backward ---------------------------------------------------------------------------------------------------
@@ -1013,6 +1055,31 @@ int myea_hip_clear_training_arrays(myea_hip_net *n)
 
 int myea_hip_forward_pass(myea_hip_net *n, size_t B, const float *x, int dev) { NET_OR_FAIL(n); return n->net.forward_pass(B, x, dev); }
 int myea_hip_compute_error(myea_hip_net *n, size_t B, const float *y, int dev) { NET_OR_FAIL(n); return n->net.compute_error(B, y, dev); }
+int myea_hip_compute_loss(myea_hip_net *n, size_t B, const float *y, int dev) { NET_OR_FAIL(n); return n->net.compute_loss(B, y, dev); }
+int myea_hip_compute_accuracy_r(myea_hip_net *n, size_t B, const float *y, int dev, float mean_d, float mean_y) { NET_OR_FAIL(n); return n->net.compute_accuracy_r(B, y, dev, mean_d, mean_y); }
+int myea_hip_gather_examples(myea_hip_net *n, float *dst, const float *src, size_t examples, size_t row_floats, const uint64_t *index, int index_on_device, size_t B)
+{
+    NET_OR_FAIL(n);
+    return n->net.gather_examples(dst, src, examples, row_floats, index, index_on_device, B);
+}
+int myea_hip_device_buffer_create(size_t floats, const float *host, float **out)
+{
+    if (!out || floats == 0) { myea::set_last_error("device_buffer_create: null or empty"); return MYEA_E_INVALID; }
+    *out = nullptr;
+    void *q = nullptr;
+    if (hipMalloc(&q, floats * sizeof(float)) != hipSuccess) { (void)hipGetLastError(); myea::set_last_error("device_buffer_create: out of device memory (%zu floats)", floats); return MYEA_E_NOMEM; }
+    if (host) {
+        const hipError_t e = hipMemcpy(q, host, floats * sizeof(float), hipMemcpyHostToDevice);
+        if (e != hipSuccess) { (void)hipFree(q); myea::set_last_error("device_buffer_create: %s", hipGetErrorString(e)); return MYEA_E_DEVICE; }
+    }
+    *out = static_cast<float *>(q);
+    return MYEA_OK;
+}
+int myea_hip_device_buffer_destroy(float *device)
+{
+    if (device) MYEA_HIP_TRY(hipFree(device));
+    return MYEA_OK;
+}
 int myea_hip_backward_pass(myea_hip_net *n, size_t B) { NET_OR_FAIL(n); return n->net.backward_pass(B); }
 int myea_hip_update_derivative_weight(myea_hip_net *n, size_t B, size_t first, size_t end) { NET_OR_FAIL(n); return n->net.update_derivative_weight(B, first, end); }
 int myea_hip_update_parameter(myea_hip_net *n, size_t B, size_t ts) { NET_OR_FAIL(n); return n->net.update_parameter(B, ts); }
@@ -1020,17 +1087,18 @@ int myea_hip_update_parameter(myea_hip_net *n, size_t B, size_t ts) { NET_OR_FAI
 int myea_hip_reset_loss(myea_hip_net *n)
 {
     NET_OR_FAIL(n);
-    MYEA_HIP_TRY(hipMemsetAsync(n->net.loss_acc, 0, 4 * sizeof(double), n->net.stream));
+    MYEA_HIP_TRY(hipMemsetAsync(n->net.loss_acc, 0, 8 * sizeof(double), n->net.stream));
     return MYEA_OK;
 }
 int myea_hip_get_loss(myea_hip_net *n, myea_loss_state *s)
 {
     NET_OR_FAIL(n);
     if (!s) { myea::set_last_error("get_loss: null"); return MYEA_E_INVALID; }
-    double v[4];
+    double v[8];
     MYEA_HIP_TRY(hipMemcpyAsync(v, n->net.loss_acc, sizeof(v), hipMemcpyDeviceToHost, n->net.stream));
     MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
     s->loss_values = v[0]; s->number_loss = (uint64_t)v[1]; s->accuracy_value = v[2]; s->number_bit_fail = (uint64_t)v[3];
+    for (int k = 0; k < 4; ++k) s->accuracy_r[k] = v[4 + k];
     return MYEA_OK;
 }
 

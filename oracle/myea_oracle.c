@@ -974,7 +974,7 @@ static float sign_f(float v) { return v > 0.f ? 1.f : (v < 0.f ? -1.f : 0.f); }
  * ignores the pre-activation (linear, tanh, sigmoid, softmax) are unaffected; this restatement
  * reproduces the quirk.
  * delta = Activation_Function_Derive(type, pre, steepness, y) * (y - desired); no 1/B, no factor 2. */
-int myea_oracle_compute_error(myea_oracle_net *n, size_t B, const float *desired)
+static int compute_error_or_loss(myea_oracle_net *n, size_t B, const float *desired, int write_delta)
 {
     if (!n || !desired) return MYEA_E_INVALID;
     size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth;
@@ -1011,15 +1011,47 @@ int myea_oracle_compute_error(myea_oracle_net *n, size_t B, const float *desired
                 case MYEA_ACCURACY_SIGN:
                     if (sign_f(d[j]) == sign_f(y[j]) || (sign_f(d[j]) == 0.f && y[j] >= -FLT_EPSILON && y[j] <= FLT_EPSILON)) n->loss.accuracy_value += 1.0;
                     break;
+                case MYEA_ACCURACY_R: /* running sums; the means are taken by the caller (NN/Neural_Network__Compute__Error__Loop.cpp:173-176) */
+                    n->loss.accuracy_value += d[j];
+                    n->loss.accuracy_r[0] += y[j];
+                    break;
                 default: break;
                 }
+                if (!write_delta) continue;
                 float q = rnn ? pre[0] : pre[j];
                 err[j] = myea_oracle_activation_derive(o->unit_af ? o->unit_af[j] : l->type_activation_function, q, o->unit_steep ? o->unit_steep[j] : l->activation_steepness, y[j]) * diff;
             }
         }
     }
     /* MEMCPY AF errors -> neuron errors over batch_size * T * H (:136-139) */
-    memcpy(o->neuron_errors, o->af_errors, T * Bmax * H * sizeof(float));
+    if (write_delta) memcpy(o->neuron_errors, o->af_errors, T * Bmax * H * sizeof(float));
+    return MYEA_OK;
+}
+
+int myea_oracle_compute_error(myea_oracle_net *n, size_t B, const float *desired) { return compute_error_or_loss(n, B, desired, 1); }
+
+/* FF__Compute__Loss / RNN__Compute__Loss (NN/Neural_Network__Compute__Loss__Loop.cpp:39-140,
+ * NN/Neural_Network__Recurrent_Compute__Loss__Loop.cpp:20-140): the same accumulation, no delta */
+int myea_oracle_compute_loss(myea_oracle_net *n, size_t B, const float *desired) { return compute_error_or_loss(n, B, desired, 0); }
+
+/* FF / RNN__Compute__Accuracy__R (NN/Neural_Network__Compute__R__Loop.cpp:38-90, NN/Neural_Network__Recurrent_Compute__R__Loop.cpp:20-75) */
+int myea_oracle_compute_accuracy_r(myea_oracle_net *n, size_t B, const float *desired, float desired_mean, float predicted_mean)
+{
+    if (!n || !desired) return MYEA_E_INVALID;
+    size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth;
+    if (B > Bmax) return MYEA_E_BATCH;
+    olayer *o = &n->L[n->d.n_layers - 1];
+    size_t H = o->H;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t t = T > 1 ? n->h.number_time_delays : 0; t < T; ++t) {
+            const float *y = o->values + Bmax * H * t + b * H, *d = desired + b * T * H + t * H;
+            for (size_t j = 0; j < H; ++j) {
+                float dd = d[j] - desired_mean, dy = y[j] - predicted_mean;
+                n->loss.accuracy_r[1] += dd * dy;
+                n->loss.accuracy_r[2] += dd * dd;
+                n->loss.accuracy_r[3] += dy * dy;
+            }
+        }
     return MYEA_OK;
 }
 

@@ -35,6 +35,8 @@ int myea_oracle_clear_training_arrays(myea_oracle_net *net);
 
 int myea_oracle_forward_pass(myea_oracle_net *net, size_t batch_size_received, const float *inputs);
 int myea_oracle_compute_error(myea_oracle_net *net, size_t batch_size_received, const float *desired_outputs);
+int myea_oracle_compute_loss(myea_oracle_net *net, size_t batch_size_received, const float *desired_outputs);
+int myea_oracle_compute_accuracy_r(myea_oracle_net *net, size_t batch_size_received, const float *desired_outputs, float desired_mean, float predicted_mean);
 int myea_oracle_backward_pass(myea_oracle_net *net, size_t batch_size_received);
 int myea_oracle_update_derivative_weight(myea_oracle_net *net, size_t batch_size_received, size_t first_layer_index, size_t end_layer_index);
 int myea_oracle_update_parameter(myea_oracle_net *net, size_t batch_size_received, size_t training_size_received);

@@ -40,6 +40,8 @@ def load_oracle():
     lib.myea_oracle_clear_training_arrays.argtypes = [vp]
     lib.myea_oracle_forward_pass.argtypes = [vp, sz, vp]
     lib.myea_oracle_compute_error.argtypes = [vp, sz, vp]
+    lib.myea_oracle_compute_loss.argtypes = [vp, sz, vp]
+    lib.myea_oracle_compute_accuracy_r.argtypes = [vp, sz, vp, C.c_float, C.c_float]
     lib.myea_oracle_backward_pass.argtypes = [vp, sz]
     lib.myea_oracle_update_derivative_weight.argtypes = [vp, sz, sz, sz]
     lib.myea_oracle_update_parameter.argtypes = [vp, sz, sz]
@@ -144,6 +146,14 @@ class OracleNetwork:
     def Compute__Error(self, batch_size, desired, on_device=False):
         y = np.ascontiguousarray(desired, dtype=np.float32)
         self._check(self.lib.myea_oracle_compute_error(self.handle, batch_size, C.c_void_p(y.ctypes.data)))
+
+    def Compute__Loss(self, batch_size, desired, on_device=False):
+        y = np.ascontiguousarray(desired, dtype=np.float32)
+        self._check(self.lib.myea_oracle_compute_loss(self.handle, batch_size, C.c_void_p(y.ctypes.data)))
+
+    def Compute__Accuracy__R(self, batch_size, desired, desired_mean, predicted_mean, on_device=False):
+        y = np.ascontiguousarray(desired, dtype=np.float32)
+        self._check(self.lib.myea_oracle_compute_accuracy_r(self.handle, batch_size, C.c_void_p(y.ctypes.data), desired_mean, predicted_mean))
 
     def Backward_Pass(self, batch_size): self._check(self.lib.myea_oracle_backward_pass(self.handle, batch_size))
 

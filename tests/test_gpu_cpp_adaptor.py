@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from myea_amd import binding as mb
+from myea_amd.dataset import get_loss
 from tests.common import assert_close, glorot_parameters, one_hot, run_step
 from tests.oracle_lib import OracleNetwork
 
@@ -31,8 +32,7 @@ def _run(tmp_path, kind, specs, B, T, hyper, X, Y, masks, seed):
         cpu.Reset__Loss()
         run_step(cpu, B, X, Y, update=False)
         g = cpu.download_gradient()
-        st = cpu.get_loss()
-        losses.append(st.loss_values / st.number_loss)
+        losses.append(get_loss(cpu, specs[-1]["units"]))
         cpu.Update_Parameter(B, B)
     got_losses = [float(l.split()[-1]) for l in out.stdout.splitlines() if l.startswith("step ")]
     assert got_losses == pytest.approx(losses, rel=1e-4)
