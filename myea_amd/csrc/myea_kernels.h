@@ -146,4 +146,35 @@ int launch_max_norm(hipStream_t s, size_t nseg, const unsigned long long *first,
 
 int launch_fill(hipStream_t s, float *p, size_t n, float v);
 
+// ---- fused LSTM time step (one cell per block, C % 32 == 0) ---------------------------------------------------
+// all tensors are the rows of ONE time step: [B][C] (stride C) or [B][4C] gate rows z | i | f | o (stride 4C)
+struct LstmFusedForward {
+    size_t B, C;
+    const float *h_prev;   // [B][C]   cell outputs of the step processed before this one
+    const float *Wrec;     // [4C][C]  packed recurrent weights, rows z | i | f | o
+    const float *bias;     // [4C]
+    const float *peep;     // [3][C]   input / forget / output gate peepholes
+    float *acts;           // [B][4C]  in: input sums; out: the activations z, i, f, o
+    const float *c_prev;   // [B][C]
+    float *c, *ca, *h;     // [B][C]   cell state, tanh(cell state), cell output
+};
+struct LstmFusedBackward {
+    size_t B, C;
+    int first_step;           // the sequence's first step: no forget-gate delta
+    const float *dG_next;     // [B][4C] gate deltas of the step processed after this one
+    const float *WrecT;       // [C][4C] transposed packed recurrent weights
+    const float *peep;        // [3][C]
+    const float *acts, *acts_next;   // [B][4C]
+    const float *c_prev;      // [B][C], unused on the first step
+    const float *ca;          // [B][C]
+    float *dh;                // [B][C]  in: delta from the layers above; out: plus the recurrent term
+    float *dG;                // [B][4C] out
+    float *dc;                // [B][C]  out
+    const float *dc_next;     // [B][C]
+};
+bool lstm_fused_supported(size_t C, size_t cells_per_block);
+int launch_lstm_fused_forward(hipStream_t s, const LstmFusedForward &p);
+int launch_lstm_fused_backward(hipStream_t s, const LstmFusedBackward &p);
+int launch_transpose(hipStream_t s, size_t rows, size_t cols, const float *src, float *dst);
+
 }  // namespace myea

@@ -16,6 +16,8 @@
 //             flat gradient, a column reduction for the three peephole vectors, a column sum for the biases.
 //
 // NN/ = Neural_Network_Library_Windows/Source_Files/Neural_Network/.
+#include <cstdlib>
+
 #include "myea_device_af.h"
 #include "myea_kernels.h"
 #include "myea_net.h"
@@ -30,6 +32,8 @@ struct LstmLayer {
     bool own_h = false;     // bidirectional: h / dh are the direction's own buffers; else the layer's values / neuron_errors
     float *h = nullptr, *dh = nullptr;                           // [T][Bmax][C] cell outputs and their delta
     float *Win = nullptr, *Wrec = nullptr, *peep = nullptr;      // packed parameters
+    float *WrecT = nullptr; // [C][G] transposed Wrec for the fused backward step; null when the fused step is not used
+    bool fused = false;     // one launch per time step (myea_lstm_fused.hip) instead of contraction + gate kernel
     float *gWin = nullptr, *gWrec = nullptr;                     // packed gradient scratch
     float *acts = nullptr;  // [T][Bmax][G]: pre-activation sums, overwritten in place by z | i | f | o
     float *c = nullptr, *ca = nullptr;                           // [T][Bmax][C] cell state and tanh(cell state)
@@ -279,6 +283,13 @@ int dev_alloc_zero(float **p, size_t count)
 
 LstmGeom geom_of(const LstmLayer &q) { return LstmGeom{q.K, q.cpb, q.C, q.G, q.In, q.per_block, q.base}; }
 
+// MYEA_LSTM_FUSED=0 in the environment keeps every layer on the generic path (contraction + gate kernel per step)
+bool fused_lstm_disabled()
+{
+    const char *e = std::getenv("MYEA_LSTM_FUSED");
+    return e && e[0] == '0';
+}
+
 }  // namespace
 
 int Net::lstm_create_layer(size_t li)
@@ -314,6 +325,8 @@ int Net::lstm_create_layer(size_t li)
         MYEA_TRY(dev_alloc_zero(&q->Win, q->G * q->In));
         MYEA_TRY(dev_alloc_zero(&q->Wrec, q->G * q->C));
         MYEA_TRY(dev_alloc_zero(&q->peep, 3 * q->C));
+        q->fused = lstm_fused_supported(q->C, q->cpb) && !fused_lstm_disabled();
+        if (q->fused) MYEA_TRY(dev_alloc_zero(&q->WrecT, q->C * q->G));
         MYEA_TRY(dev_alloc_zero(&q->gWin, kMaxSlabs * q->G * q->In));   // split-K slabs of the weight-gradient contractions
         MYEA_TRY(dev_alloc_zero(&q->gWrec, kMaxSlabs * q->G * q->C));
         MYEA_TRY(dev_alloc_zero(&q->acts, T * B * q->G));
@@ -335,7 +348,7 @@ void Net::lstm_destroy_layer(DevLayer &o)
     for (LstmLayer **slot : {&o.lstm, &o.lstm2}) {
         LstmLayer *q = *slot;
         if (!q) continue;
-        float *all[] = {q->Win, q->Wrec, q->peep, q->gWin, q->gWrec, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr};
+        float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin, q->gWrec, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr};
         for (float *p : all) if (p) (void)hipFree(p);
         delete q;
         *slot = nullptr;
@@ -359,6 +372,7 @@ int Net::lstm_parameters_changed()
             const size_t n = q->G * (q->In + q->C) + 3 * q->C;
             hipLaunchKernelGGL(lstm_gather_kernel, dim3(grid_for(n, kBlock, 4096)), dim3(kBlock), 0, stream, geom_of(*q), parameters, q->Win, q->Wrec, q->peep);
             MYEA_HIP_TRY(hipGetLastError());
+            if (q->WrecT) MYEA_TRY(launch_transpose(stream, q->G, q->C, q->Wrec, q->WrecT));
         }
     }
     return MYEA_OK;
@@ -389,6 +403,17 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
         const size_t t = q.reverse ? T - 1 - s : s, tp = q.reverse ? t + 1 : t - 1;  // tp: the step processed before t
         float *acts_t = q.acts + t * Bmax * q.G;
         int nparts = 0;
+        if (s > 0 && q.fused) {   // recurrent contraction and gate math of the step in one launch
+            LstmFusedForward f{};
+            f.B = B; f.C = q.C;
+            f.h_prev = q.h + tp * Bmax * q.C; f.Wrec = q.Wrec; f.bias = bias; f.peep = q.peep;
+            f.acts = acts_t; f.c_prev = q.c + tp * Bmax * q.C;
+            f.c = q.c + t * Bmax * q.C; f.ca = q.ca + t * Bmax * q.C; f.h = q.h + t * Bmax * q.C;
+            prof_begin(0);
+            MYEA_TRY(launch_lstm_fused_forward(stream, f));
+            prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
+            continue;
+        }
         if (s > 0) {
             GemmParams g{};
             g.A = q.h + tp * Bmax * q.C; g.lda = (long)q.C; g.a_k_contiguous = 1;
@@ -433,6 +458,18 @@ int Net::lstm_backward_direction(LstmLayer &q, size_t B)
         float *dh_t = q.dh + t * Bmax * q.C;
         const bool last = s == T - 1, first = s == 0;
         int nparts = 0;
+        if (!last && q.fused) {   // dh[t] += dG[tn] Wrec and the gate deltas of step t in one launch
+            LstmFusedBackward f{};
+            f.B = B; f.C = q.C; f.first_step = first;
+            f.dG_next = q.dG + tn * Bmax * q.G; f.WrecT = q.WrecT; f.peep = q.peep;
+            f.acts = q.acts + t * Bmax * q.G; f.acts_next = q.acts + tn * Bmax * q.G;
+            f.c_prev = first ? nullptr : q.c + tp * Bmax * q.C; f.ca = q.ca + t * Bmax * q.C;
+            f.dh = dh_t; f.dG = q.dG + t * Bmax * q.G; f.dc = q.dc + t * Bmax * q.C; f.dc_next = q.dc + tn * Bmax * q.C;
+            prof_begin(1);
+            MYEA_TRY(launch_lstm_fused_backward(stream, f));
+            prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
+            continue;
+        }
         if (!last) {  // Backward_Pass__LSTM_Derivative__Output, recurrent part (:1174-1226)
             GemmParams g{};
             g.A = q.dG + tn * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 1;

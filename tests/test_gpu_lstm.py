@@ -60,6 +60,12 @@ CASES = [
     ("single-step", [dict(units=3), dict(type="lstm", units=5), dict(units=6, activation="LINEAR")], 1, 4, 4),
     ("two-steps", [dict(units=3), dict(type="lstm", units=4), dict(units=5, activation="LINEAR")], 2, 7, 7),
     ("unfused-activation-below", [dict(units=8), dict(units=12, activation="ELU"), dict(type="lstm", units=12), dict(units=12, activation="LINEAR")], 4, 8, 8),
+    # one cell per block and a multiple of 32 cells: the one-launch-per-step kernels (k groups per wavefront 1, 3, 5; ragged rows)
+    ("fused-step-32-cells", [dict(units=9), dict(type="lstm", units=32), dict(units=32, activation="LINEAR")], 5, 7, 7),
+    ("fused-step-96-cells-partial-batch", [dict(units=20), dict(type="lstm", units=96), dict(units=96, activation="TANH")], 4, 37, 40),
+    ("fused-step-160-cells-two-steps", [dict(units=6), dict(type="lstm", units=160), dict(units=160, activation="LINEAR")], 2, 33, 33),
+    ("fused-step-stacked-on-generic", [dict(units=10), dict(type="lstm", units=24), dict(type="lstm", units=64), dict(type="lstm", units=32),
+                                       dict(units=32, activation="LINEAR")], 3, 12, 16),
 ]
 
 
@@ -90,6 +96,39 @@ def test_lstm_parity_three_amsgrad_steps(name, specs, T, B, Bmax):
     for kind in (1, 2, 3):
         a, b = gpu.download_optimizer_state(kind), cpu.download_optimizer_state(kind)
         assert_close(a, b, REL, ABS, what="optimizer state %d" % kind)
+
+
+def test_fused_time_step_matches_the_generic_path_on_the_gpu():
+    """the same step through one launch per time step and through contraction + gate kernel per step (MYEA_LSTM_FUSED=0)"""
+    T, B, Bmax = 7, 70, 72
+    specs = [dict(units=24), dict(type="lstm", units=128), dict(type="lstm", units=64), dict(units=64, activation="LINEAR")]
+    desc = mb.make_desc(specs, Bmax, T)
+    h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["ADAM"], type_loss_function=mb.LOSS["MSE"])
+    w = glorot_parameters(desc, 8, bias_range=0.3)
+    rng = np.random.default_rng(8)
+    X = rng.normal(0, 1, (B, T * 24)).astype(np.float32)
+    Y = rng.normal(0, 1, (B, T * 64)).astype(np.float32)
+    nets = []
+    for flag in ("1", "0"):
+        os.environ["MYEA_LSTM_FUSED"] = flag
+        try:
+            n = mb.HipNetwork(desc, h)
+        finally:
+            del os.environ["MYEA_LSTM_FUSED"]
+        n.set_state_propagation(mb.STATE_TRAINING)
+        n.upload_parameters(w)
+        n.Clear_Training_Arrays()
+        n.Reset__Loss()
+        run_step(n, B, X, Y, update=False)
+        nets.append(n)
+    fused, generic = nets
+    for li in (1, 2):
+        for kind in ["OUTPUTS", "ERRORS"] + LSTM_TAPS:
+            a = fused.download_tensor(li, mb.TENSOR[kind], T * Bmax * _width(desc.layers[li]))
+            b = generic.download_tensor(li, mb.TENSOR[kind], T * Bmax * _width(desc.layers[li]))
+            assert_close(_rows(a, T, Bmax, B, _width(desc.layers[li])), _rows(b, T, Bmax, B, _width(desc.layers[li])), REL, ABS, what="layer %d %s" % (li, kind))
+    assert_close(fused.download_gradient(), generic.download_gradient(), REL, ABS, what="gradient")
+    assert fused.get_loss().loss_values == pytest.approx(generic.get_loss().loss_values, rel=1e-5)
 
 
 def test_lstm_softmax_head_cross_entropy_clip_and_adabound():
