@@ -709,6 +709,31 @@ int launch_sum_squares(hipStream_t s, size_t n, const float *g, float *partials,
     return MYEA_OK;
 }
 
+// dst[i] += slab 0 [i] + slab 1 [i] + ... (in slab order): the second half of a deterministic split-K contraction
+__global__ __launch_bounds__(kBlock) void slab_sum_add_kernel(size_t n, int nslab, const float *__restrict__ slabs, float *__restrict__ dst)
+{
+    const size_t n4 = n / 4;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += (size_t)gridDim.x * kBlock) {
+        f32x4 v = reinterpret_cast<const f32x4 *>(slabs)[i];
+        for (int s = 1; s < nslab; ++s) {
+            const f32x4 w = reinterpret_cast<const f32x4 *>(slabs + (size_t)s * n)[i];
+            v[0] += w[0]; v[1] += w[1]; v[2] += w[2]; v[3] += w[3];
+        }
+        f32x4 d = reinterpret_cast<f32x4 *>(dst)[i];
+        d[0] += v[0]; d[1] += v[1]; d[2] += v[2]; d[3] += v[3];
+        reinterpret_cast<f32x4 *>(dst)[i] = d;
+    }
+}
+
+int launch_slab_sum_add(hipStream_t s, size_t n, int nslab, const float *slabs, float *dst)
+{
+    if (n == 0 || nslab <= 0) return MYEA_OK;
+    if ((n & 3) || (reinterpret_cast<uintptr_t>(slabs) & 15u) || (reinterpret_cast<uintptr_t>(dst) & 15u)) { set_last_error("slab sum: operands must be 16-byte aligned multiples of 4"); return MYEA_E_INVALID; }
+    hipLaunchKernelGGL(slab_sum_add_kernel, dim3(grid_for(n / 4, kBlock, 8192)), dim3(kBlock), 0, s, n, nslab, slabs, dst);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
 int launch_max_norm(hipStream_t s, size_t nseg, const unsigned long long *first, const unsigned *len, unsigned longest, float max_norm, float *w)
 {
     if (nseg == 0) return MYEA_OK;

@@ -451,16 +451,24 @@ int launch_layout_scalar(hipStream_t stream, const GemmDev &d, bool a_kc, bool b
 
 }  // namespace
 
-// Number of K slabs for a short contraction so that the launch reaches about one workgroup per CU with 64 x 64 tiles
-// (each slab at least 128 k's deep); 1 when the plain launch already fills the chip.
+// Number of K slabs for a contraction whose M x N alone does not fill the chip; 1 when the plain launch already does.
+// Short k: about one workgroup per CU with 64 x 64 tiles, each slab at least 128 k's deep.
 int gemm_split_k(int M, int N, int K)
 {
     const long tiles_128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     if (tiles_128 * 2 >= 256) return 1;
-    const long tiles_64 = (long)((M + 63) / 64) * ((N + 63) / 64);
-    long want = (256 + tiles_64 - 1) / tiles_64;
-    const long max_by_k = K / 128 > 0 ? K / 128 : 1;
-    if (want > max_by_k) want = max_by_k;
+    long want;
+    if (K >= 4096) {
+        // long k (weight gradients over T x batch rows): enough slabs for ~1000 workgroups of 128 x 64, each slab at least
+        // 1024 k's deep - the larger tile's operand reuse is worth more than the pass over the slabs that sums them
+        want = (512 + tiles_128 - 1) / tiles_128;
+        if (want > K / 1024) want = K / 1024;
+    } else {
+        const long tiles_64 = (long)((M + 63) / 64) * ((N + 63) / 64);
+        want = (256 + tiles_64 - 1) / tiles_64;
+        const long max_by_k = K / 128 > 0 ? K / 128 : 1;
+        if (want > max_by_k) want = max_by_k;
+    }
     if (want > 16) want = 16;
     if (want < 1) want = 1;
     // the launcher rounds the chunk up to a multiple of 32: return the slab count that rounding produces

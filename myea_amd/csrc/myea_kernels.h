@@ -145,6 +145,8 @@ int launch_update(hipStream_t s, const UpdateParams &p);
 int launch_max_norm(hipStream_t s, size_t nseg, const unsigned long long *first, const unsigned *len, unsigned longest, float max_norm, float *w);
 
 int launch_fill(hipStream_t s, float *p, size_t n, float v);
+// dst[0..n) += sum over the nslab slabs of n floats each, in slab order (n % 4 == 0, 16-byte aligned)
+int launch_slab_sum_add(hipStream_t s, size_t n, int nslab, const float *slabs, float *dst);
 
 // ---- fused LSTM time step (one cell per block, C % 32 == 0) ---------------------------------------------------
 // all tensors are the rows of ONE time step: [B][C] (stride C) or [B][4C] gate rows z | i | f | o (stride 4C)

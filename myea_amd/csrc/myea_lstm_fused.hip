@@ -107,6 +107,20 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
     constexpr int kStage = (32 + 64) * 32;           // floats: A tile 32 x 32, then B tile 64 x 32
     float *stage0 = smem + wave * kFwdStages * kStage;
 
+    // what the gate math of this lane's two (example, cell) pairs reads does not depend on the contraction: fetch it now
+    float e_in[2][4], e_bias[2][4], e_peep[2][3], e_cp[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int pair = threadIdx.x + q * kThreads, row = pair >> 4, cell = pair & 15;
+        const int b = min(r0 + row, B - 1), k = c0 + cell;
+        const float *arow = p.acts + (size_t)b * 4 * C;
+#pragma unroll
+        for (int gate = 0; gate < 4; ++gate) { e_in[q][gate] = arow[gate * C + k]; e_bias[q][gate] = p.bias[gate * C + k]; }
+#pragma unroll
+        for (int gate = 0; gate < 3; ++gate) e_peep[q][gate] = p.peep[gate * C + k];
+        e_cp[q] = p.c_prev[(size_t)b * C + k];
+    }
+
     f32x16 acc0, acc1;
 #pragma unroll
     for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
@@ -129,15 +143,24 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
                 wait_loads<0>();
             }
             const float *la = cur, *lb = cur + 32 * 32;
+            // fragments of k group kg + 1 are read while the MFMAs of group kg issue
+            f32x4 fa[2], fb0[2], fb1[2];
+            fa[0] = WaveTile<32>::chunk(la, lane32, half);
+            fb0[0] = WaveTile<64>::chunk(lb, lane32, half);
+            fb1[0] = WaveTile<64>::chunk(lb, 32 + lane32, half);
 #pragma unroll
             for (int kg = 0; kg < 4; ++kg) {
-                const f32x4 a = WaveTile<32>::chunk(la, lane32, kg * 2 + half);
-                const f32x4 b0 = WaveTile<64>::chunk(lb, lane32, kg * 2 + half);
-                const f32x4 b1 = WaveTile<64>::chunk(lb, 32 + lane32, kg * 2 + half);
+                const int cb = kg & 1, nb = cb ^ 1;
+                if (kg + 1 < 4) {
+                    fa[nb] = WaveTile<32>::chunk(la, lane32, (kg + 1) * 2 + half);
+                    fb0[nb] = WaveTile<64>::chunk(lb, lane32, (kg + 1) * 2 + half);
+                    fb1[nb] = WaveTile<64>::chunk(lb, 32 + lane32, (kg + 1) * 2 + half);
+                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
-                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b0[s], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b1[s], acc1, 0, 0, 0);
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][s], fb0[cb][s], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][s], fb1[cb][s], acc1, 0, 0, 0);
                 }
             }
         }
@@ -169,16 +192,16 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
         const int k = c0 + cell;
         float *arow = p.acts + (size_t)b * 4 * C;
         const size_t ci = (size_t)b * C + k;
-        const float cp = p.c_prev[ci];
-        float si = arow[C + k] + rec[1] + p.bias[C + k];
-        float sf = arow[2 * C + k] + rec[2] + p.bias[2 * C + k];
-        si += cp * p.peep[k];
-        sf += cp * p.peep[C + k];
+        const float cp = e_cp[q];
+        float si = e_in[q][1] + rec[1] + e_bias[q][1];
+        float sf = e_in[q][2] + rec[2] + e_bias[q][2];
+        si += cp * e_peep[q][0];
+        sf += cp * e_peep[q][1];
         const float gi = sigmoid_f(si), gf = sigmoid_f(sf);
-        const float z = tanh_f(arow[k] + rec[0] + p.bias[k]);
+        const float z = tanh_f(e_in[q][0] + rec[0] + e_bias[q][0]);
         const float cs = z * gi + gf * cp;
         const float a = tanh_f(cs);
-        const float so = arow[3 * C + k] + rec[3] + p.bias[3 * C + k] + cs * p.peep[2 * C + k];
+        const float so = e_in[q][3] + rec[3] + e_bias[q][3] + cs * e_peep[q][2];
         const float go = sigmoid_f(so);
         arow[k] = z; arow[C + k] = gi; arow[2 * C + k] = gf; arow[3 * C + k] = go;
         p.c[ci] = cs; p.ca[ci] = a; p.h[ci] = a * go;
@@ -206,6 +229,24 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_backward_kernel(LstmFused
     constexpr int kStage = (32 + 16) * 32;   // floats: A tile 32 x 32 (rows of dG[t']), then B tile 16 x 32 (rows of WrecT)
     float *stage0 = smem + wave * kBwdStages * kStage;
 
+    // operands of the gate math of this lane's two (example, cell) pairs, fetched ahead of the contraction
+    float e_dh[2], e_act[2][4], e_ca[2], e_din[2], e_dfn[2], e_fn[2], e_peep[2][3], e_dcn[2], e_cp[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int pair = threadIdx.x + q * kThreads, row = pair >> 4, cell = pair & 15;
+        const int b = min(r0 + row, B - 1), k = c0 + cell;
+        const size_t ci = (size_t)b * C + k, gi_ = (size_t)b * G;
+        e_dh[q] = p.dh[ci];
+#pragma unroll
+        for (int gate = 0; gate < 4; ++gate) e_act[q][gate] = p.acts[gi_ + gate * C + k];
+        e_ca[q] = p.ca[ci];
+        e_din[q] = p.dG_next[gi_ + C + k]; e_dfn[q] = p.dG_next[gi_ + 2 * C + k]; e_fn[q] = p.acts_next[gi_ + 2 * C + k];
+#pragma unroll
+        for (int gate = 0; gate < 3; ++gate) e_peep[q][gate] = p.peep[gate * C + k];
+        e_dcn[q] = p.dc_next[ci];
+        e_cp[q] = p.first_step ? 0.f : p.c_prev[ci];
+    }
+
     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
     WaveTile<32> ta;
     WaveTile<16> tb;
@@ -230,17 +271,20 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_backward_kernel(LstmFused
             wait_loads<0>();
         }
         const float *la = cur, *lb = cur + 32 * 32;
+        f32x4 fa0[2], fa1[2], fb[2];
 #pragma unroll
         for (int kg = 0; kg < 2; ++kg) {
-            const f32x4 a0 = WaveTile<32>::chunk(la, lane16, kg * 4 + quad);
-            const f32x4 a1 = WaveTile<32>::chunk(la, 16 + lane16, kg * 4 + quad);
-            const f32x4 b = WaveTile<16>::chunk(lb, lane16, kg * 4 + quad);
+            fa0[kg] = WaveTile<32>::chunk(la, lane16, kg * 4 + quad);
+            fa1[kg] = WaveTile<32>::chunk(la, 16 + lane16, kg * 4 + quad);
+            fb[kg] = WaveTile<16>::chunk(lb, lane16, kg * 4 + quad);
+        }
+#pragma unroll
+        for (int kg = 0; kg < 2; ++kg)
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[s], b[s], acc0, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[s], b[s], acc1, 0, 0, 0);
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(fa0[kg][s], fb[kg][s], acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(fa1[kg][s], fb[kg][s], acc1, 0, 0, 0);
             }
-        }
     }
     __syncthreads();   // every wavefront is done with its stages: the partial tiles reuse the memory
     float *part = smem;
@@ -261,24 +305,22 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_backward_kernel(LstmFused
         for (int w = 0; w < 4; ++w) rec += part[(w * 32 + row) * kBwdStride + cell];
         const int k = c0 + cell;
         const size_t ci = (size_t)b * C + k, gi_ = (size_t)b * G;
-        const float dh = p.dh[ci] + rec;
+        const float dh = e_dh[q] + rec;
         p.dh[ci] = dh;
-        const float *arow = p.acts + gi_;
         float *drow = p.dG + gi_;
-        const float z = arow[k], gi = arow[C + k], gf = arow[2 * C + k], go = arow[3 * C + k];
-        const float a = p.ca[ci];
+        const float z = e_act[q][0], gi = e_act[q][1], gf = e_act[q][2], go = e_act[q][3];
+        const float a = e_ca[q];
         const float ddo = go * (1.f - go) * (dh * a);
         drow[3 * C + k] = ddo;
-        const float di_n = p.dG_next[gi_ + C + k], df_n = p.dG_next[gi_ + 2 * C + k], f_n = p.acts_next[gi_ + 2 * C + k];
         float e = dh * go * (1.f - a * a);
-        e += p.peep[2 * C + k] * ddo;
-        e += p.peep[k] * di_n;
-        e += p.peep[C + k] * df_n;
-        e += p.dc_next[ci] * f_n;
+        e += e_peep[q][2] * ddo;
+        e += e_peep[q][0] * e_din[q];
+        e += e_peep[q][1] * e_dfn[q];
+        e += e_dcn[q] * e_fn[q];
         p.dc[ci] = e;
         drow[k] = e * gi * (1.f - z * z);
         drow[C + k] = (e * z) * (gi * (1.f - gi));
-        drow[2 * C + k] = p.first_step ? 0.f : (e * p.c_prev[ci]) * (gf * (1.f - gf));
+        drow[2 * C + k] = p.first_step ? 0.f : (e * e_cp[q]) * (gf * (1.f - gf));
     }
 }
 

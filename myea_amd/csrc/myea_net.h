@@ -58,6 +58,7 @@ struct Net {
     unsigned longest_segment = 0;
     std::vector<DevLayer> L;
     float *tmp1 = nullptr, *tmp2 = nullptr, *scratch = nullptr, *stage_in = nullptr, *stage_out = nullptr;
+    float *dw_slabs = nullptr;   // split-K slabs of a fully-connected weight gradient whose M x N is small and k long
     double *loss_acc = nullptr;                  // 8 doubles, see ErrorParams::loss_acc
     unsigned long long *index_stage = nullptr;   // [Bmax] example indices of a gathered batch
 

@@ -151,6 +151,8 @@ static int check_desc(const myea_net_desc &d)
     return MYEA_OK;
 }
 
+static int fc_dw_slabs(size_t H, size_t In, size_t rows, size_t first_connection_index);
+
 int Net::create(const myea_net_desc &desc)
 {
     MYEA_TRY(check_desc(desc));
@@ -226,6 +228,15 @@ int Net::create(const myea_net_desc &desc)
         if (lstm_scratch_floats() > need) need = lstm_scratch_floats();
         MYEA_TRY(dev_alloc(&scratch, need));
     }
+    {   // weight gradients of narrow layers over long T x batch row ranges run as split-K contractions into slabs
+        size_t need = 0;
+        for (size_t li = 1; li < d.n_layers; ++li) {
+            if (d.layers[li].type_layer != MYEA_LAYER_FULLY_CONNECTED) continue;
+            const int slabs = fc_dw_slabs(L[li].H, L[li].In, T * B, d.layers[li].first_connection_index);
+            if (slabs > 1) need = std::max(need, (size_t)slabs * L[li].H * L[li].In);
+        }
+        if (need) MYEA_TRY(dev_alloc(&dw_slabs, need));
+    }
     MYEA_TRY(dev_alloc(&stage_in, T * B * L[0].H));
     MYEA_TRY(dev_alloc(&stage_out, T * B * L[d.n_layers - 1].H));
     {
@@ -252,7 +263,7 @@ Net::~Net()
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
-    fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc); fr(index_stage);
+    fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc); fr(index_stage); fr(dw_slabs);
     for (ProfEvent &e : pending) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
     for (ProfEvent &e : free_events) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
 }
@@ -704,6 +715,13 @@ int Net::backward_pass(size_t B)
 // ---- Update_Derivative_Weight -----------------------------------------------------------------------------------
 // FF__Update_Derivative_Weight_Batch (NN/Neural_Network__Update_Derivative_Weight__OpenMP.cpp:24-59):
 // dW += delta^T X (:178-216) with X = the previous layer's post-dropout outputs, db += column sums (:218-242).
+// slabs of the split-K form of a fully-connected layer's weight gradient; 1 = the plain accumulating contraction
+static int fc_dw_slabs(size_t H, size_t In, size_t rows, size_t first_connection_index)
+{
+    if (((H * In) & 3) || (first_connection_index & 3) || rows > 0x7fffffffu) return 1;   // the slab sum works on aligned quads
+    return gemm_split_k((int)H, (int)In, (int)rows);
+}
+
 int Net::update_derivative_weight(size_t B, size_t first, size_t end)
 {
     if (first < 1 || end > d.n_layers || first > end) { set_last_error("Update_Derivative_Weight: layer range [%zu, %zu) invalid", first, end); return MYEA_E_INVALID; }
@@ -729,8 +747,11 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
             g.C = gradient + l.first_connection_index; g.ldc = (long)In;
             g.M = (int)H; g.N = (int)In; g.K = (int)rows;
             g.accumulate = 1; g.epilogue = EPI_NONE;
+            const int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
+            if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
             prof_begin(2);
             MYEA_TRY(launch_gemm(stream, g));
+            if (slabs > 1) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
             prof_end(2.0 * (double)rows * (double)H * (double)In);
             if (layer_uses_bias(l)) MYEA_TRY(launch_column_sum(stream, rows, H, o.neuron_errors + roff * H, gradient + l.first_bias_connection_index, 1, scratch));
         }
