@@ -38,7 +38,9 @@ extern "C" {
 enum {
     MYEA_LAYER_NONE = 0,
     MYEA_LAYER_FULLY_CONNECTED = 4,
+    MYEA_LAYER_AVERAGE_POOLING = 1,
     MYEA_LAYER_LSTM = 8,
+    MYEA_LAYER_MAX_POOLING = 9,
     MYEA_LAYER_RESIDUAL = 10
 };
 
@@ -121,7 +123,10 @@ typedef struct myea_layer_desc {
     uint32_t type_normalization;       /* MYEA_NORMALIZATION_* */
     uint32_t use_layer_normalization_before_activation;
     uint32_t block_depth;              /* residual only: layers inside the block */
-    uint32_t reserved0;
+    /* pooling layers only (Layer::pooling_values, Assign__Layer NN/Neural_Network__Compile.cpp:51-58): kernel size,
+     * stride, padding, dilation, ceil mode.  n_units of a pooling layer is an OUTPUT of myea_net_desc_layout
+     * (Assign__Post__Layer :250-271). */
+    uint32_t pooling_values[5];
     /* index table (into the flat parameter / gradient / optimizer vectors, and the mask buffer) */
     uint64_t first_connection_index;       /* *Layer::ptr_first_connection_index */
     uint64_t last_connection_index;        /* *Layer::ptr_last_connection_index */

@@ -27,6 +27,7 @@ struct Layer_Parameters {
     bool use_bidirectional = false;
     unsigned int type_layer = MYEA_LAYER_NONE;  // MYEA_LAYER_*
     // [0] FC: neurons, LSTM: blocks, RESIDUAL: block depth.  [1] LSTM: cells per block.
+    // pooling layers: [0] kernel size, [1] stride, [2] padding, [3] dilation, [4] ceil mode.
     size_t unit_parameters[5u] = {0};
 };
 
@@ -84,6 +85,11 @@ public:
             l.n_units = (uint32_t)ptr_array_layers[i].unit_parameters[0];
             l.n_cells_per_block = l.type_layer == MYEA_LAYER_LSTM ? (uint32_t)ptr_array_layers[i].unit_parameters[1] : 0;
             if (l.type_layer == MYEA_LAYER_RESIDUAL) { l.block_depth = l.n_units; l.n_units = 0; }
+            if (l.type_layer == MYEA_LAYER_AVERAGE_POOLING || l.type_layer == MYEA_LAYER_MAX_POOLING) {
+                // kernel size, stride, padding, dilation, ceil mode (Assign__Layer, Neural_Network__Compile.cpp:51-58); the width follows
+                for (int k = 0; k < 5; ++k) l.pooling_values[k] = (uint32_t)ptr_array_layers[i].unit_parameters[k];
+                l.n_units = 0;
+            }
             // Compile's defaults: FC layers start as sigmoid with steepness 1 (Neural_Network__Compile.cpp:572-590)
             l.type_activation_function = (i > 0 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) ? MYEA_AF_SIGMOID : MYEA_AF_NONE;
             l.activation_steepness = 1.f;

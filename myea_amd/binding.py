@@ -16,6 +16,7 @@ MAX_LAYERS = 64
 
 # ---- enum values (Common_Library/include/Enums of the reference) ----
 LAYER_FULLY_CONNECTED, LAYER_LSTM, LAYER_RESIDUAL = 4, 8, 10
+LAYER_AVERAGE_POOLING, LAYER_MAX_POOLING = 1, 9
 NETWORK_FEEDFORWARD, NETWORK_RECURRENT = 3, 4
 AF = dict(NONE=0, COSINE=1, COSINE_SYMMETRIC=2, ELU=3, ELLIOT=4, ELLIOT_SYMMETRIC=5, GAUSSIAN=6,
           GAUSSIAN_STEPWISE=7, GAUSSIAN_SYMMETRIC=8, ISRU=9, ISRLU=10, LINEAR=11, LINEAR_PIECE=12,
@@ -44,7 +45,7 @@ class LayerDesc(C.Structure):
         ("use_bidirectional", C.c_uint32), ("type_activation_function", C.c_uint32),
         ("activation_steepness", C.c_float), ("type_dropout", C.c_uint32), ("dropout_values", C.c_float * 2),
         ("type_normalization", C.c_uint32), ("use_layer_normalization_before_activation", C.c_uint32),
-        ("block_depth", C.c_uint32), ("reserved0", C.c_uint32),
+        ("block_depth", C.c_uint32), ("pooling_values", C.c_uint32 * 5),
         ("first_connection_index", C.c_uint64), ("last_connection_index", C.c_uint64),
         ("first_bias_connection_index", C.c_uint64), ("first_normalized_unit_index", C.c_uint64),
         ("first_mask_index", C.c_uint64),
@@ -184,7 +185,11 @@ def make_desc(layers, batch_size, recurrent_depth=1, network=None, lib=None):
     for i, spec in enumerate(layers):
         l = d.layers[i]
         kind = spec.get("type", "fc")
-        l.type_layer = {"fc": LAYER_FULLY_CONNECTED, "lstm": LAYER_LSTM, "residual": LAYER_RESIDUAL}[kind]
+        l.type_layer = {"fc": LAYER_FULLY_CONNECTED, "lstm": LAYER_LSTM, "residual": LAYER_RESIDUAL,
+                        "average_pooling": LAYER_AVERAGE_POOLING, "max_pooling": LAYER_MAX_POOLING}[kind]
+        if kind.endswith("pooling"):   # units is computed by the layout
+            for k, name in enumerate(("kernel", "stride", "padding", "dilation", "ceil_mode")):
+                l.pooling_values[k] = int(spec.get(name, 1 if name in ("stride", "dilation") else 0))
         l.n_units = spec.get("units", 0)
         l.n_cells_per_block = spec.get("cells_per_block", 1 if kind == "lstm" else 0)
         l.use_bidirectional = int(spec.get("bidirectional", False))

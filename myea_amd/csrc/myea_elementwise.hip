@@ -709,6 +709,79 @@ int launch_sum_squares(hipStream_t s, size_t n, const float *g, float *partials,
     return MYEA_OK;
 }
 
+// Forward_Pass__Average_Pooling / __Max_Pooling (NN/Neural_Network__Forward_Pass__Loop.cpp:4537-4583, 5070-5135).  Window positions
+// are padded coordinates p = j stride + k dilation; the input occupies [padding, padding + In).  Average: padding adds 0, the
+// divisor is always the kernel size.  Max: a padded position stands for 0; the first maximum's position is kept.
+__global__ __launch_bounds__(kBlock) void pool_forward_kernel(PoolParams p, const float *__restrict__ x, float *__restrict__ y, unsigned *__restrict__ index)
+{
+    const size_t n = p.rows * p.H;
+    const float scale = 1.f / (float)p.kernel;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t r = i / p.H, j = i - r * p.H;
+        const float *xr = x + r * p.In;
+        if (!p.is_max) {
+            float s = 0.f;
+            for (unsigned k = 0; k < p.kernel; ++k) {
+                const size_t pos = j * p.stride + (size_t)k * p.dilation;
+                if (pos < p.padding || pos >= p.In + p.padding) continue;
+                s += xr[pos - p.padding];
+            }
+            y[i] = s * scale;
+        } else {
+            size_t at = 0; float mx = -3.402823466e+38f;
+            for (unsigned k = 0; k < p.kernel; ++k) {
+                const size_t pos = j * p.stride + (size_t)k * p.dilation;
+                if (pos < p.padding || pos >= p.In + p.padding) { if (mx < 0.f) { at = pos; mx = 0.f; } }
+                else { const float v = xr[pos - p.padding]; if (mx < v) { at = pos; mx = v; } }
+            }
+            index[i] = (unsigned)at;
+            y[i] = mx;
+        }
+    }
+}
+
+// Backward_Pass__Average_Pooling / __Max_Pooling (NN/Neural_Network__Backward_Pass__Loop.cpp:1004-1049, 1139-1181) as a gather: an input
+// position collects from the windows that contain it, in ascending window order (the order the reference's scatter adds them).
+__global__ __launch_bounds__(kBlock) void pool_backward_kernel(PoolParams p, const float *__restrict__ dy, const unsigned *__restrict__ index, float *__restrict__ dx)
+{
+    const size_t n = p.rows * p.In;
+    const float scale = 1.f / (float)p.kernel;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t r = i / p.In, c = i - r * p.In;
+        const size_t pos = c + p.padding;
+        float v = 0.f;
+        for (unsigned kk = p.kernel; kk-- > 0;) {
+            const size_t off = (size_t)kk * p.dilation;
+            if (off > pos) continue;
+            const size_t q = pos - off;
+            if (q % p.stride) continue;
+            const size_t j = q / p.stride;
+            if (j >= p.H) continue;
+            if (!p.is_max) v += dy[r * p.H + j] * scale;
+            else if (index[r * p.H + j] == (unsigned)pos) v += dy[r * p.H + j];
+        }
+        dx[i] = v;
+    }
+}
+
+int launch_pool_forward(hipStream_t s, const PoolParams &p, const float *x, float *y, unsigned *index)
+{
+    if (p.rows == 0 || p.H == 0) return MYEA_OK;
+    if (p.kernel == 0 || p.stride == 0 || !x || !y || (p.is_max && !index)) { set_last_error("pooling forward: bad parameters"); return MYEA_E_INVALID; }
+    hipLaunchKernelGGL(pool_forward_kernel, dim3(grid_for(p.rows * p.H, kBlock, 8192)), dim3(kBlock), 0, s, p, x, y, index);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_pool_backward(hipStream_t s, const PoolParams &p, const float *dy, const unsigned *index, float *dx)
+{
+    if (p.rows == 0 || p.In == 0) return MYEA_OK;
+    if (p.kernel == 0 || p.stride == 0 || !dy || !dx || (p.is_max && !index)) { set_last_error("pooling backward: bad parameters"); return MYEA_E_INVALID; }
+    hipLaunchKernelGGL(pool_backward_kernel, dim3(grid_for(p.rows * p.In, kBlock, 8192)), dim3(kBlock), 0, s, p, dy, index, dx);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
 // dst[i] += slab 0 [i] + slab 1 [i] + ... (in slab order): the second half of a deterministic split-K contraction
 __global__ __launch_bounds__(kBlock) void slab_sum_add_kernel(size_t n, int nslab, const float *__restrict__ slabs, float *__restrict__ dst)
 {

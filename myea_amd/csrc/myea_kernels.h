@@ -145,6 +145,17 @@ int launch_update(hipStream_t s, const UpdateParams &p);
 int launch_max_norm(hipStream_t s, size_t nseg, const unsigned long long *first, const unsigned *len, unsigned longest, float max_norm, float *w);
 
 int launch_fill(hipStream_t s, float *p, size_t n, float v);
+
+// ---- pooling over the feature axis (average / max), rows = (time step, example) pairs --------------------------
+struct PoolParams {
+    size_t rows, In, H;                       // input and output width
+    unsigned kernel, stride, padding, dilation;
+    int is_max;
+};
+// y [rows][H] <- x [rows][In]; index [rows][H] (max only): padded position of the window's first maximum
+int launch_pool_forward(hipStream_t s, const PoolParams &p, const float *x, float *y, unsigned *index);
+// dx [rows][In] <- dy [rows][H] (overwrites dx)
+int launch_pool_backward(hipStream_t s, const PoolParams &p, const float *dy, const unsigned *index, float *dx);
 // dst[0..n) += sum over the nslab slabs of n floats each, in slab order (n % 4 == 0, 16-byte aligned)
 int launch_slab_sum_add(hipStream_t s, size_t n, int nslab, const float *slabs, float *dst);
 

@@ -7,6 +7,7 @@
 #include "../../include/myea_hip.h"
 
 #include <float.h>
+#include <math.h>
 #include <string.h>
 
 /* Public training fields: Header_Files/Neural_Network/Data.hpp:2929-2970. */
@@ -102,6 +103,8 @@ uint64_t myea_net_desc_number_outputs(const myea_net_desc *d, uint32_t li)
 #define number_outputs myea_net_desc_number_outputs
 #define previous_layer myea_net_desc_previous_layer
 
+static int is_pooling(const myea_layer_desc *l) { return l->type_layer == MYEA_LAYER_AVERAGE_POOLING || l->type_layer == MYEA_LAYER_MAX_POOLING; }
+
 int myea_net_desc_layout(myea_net_desc *d)
 {
     if (!d || d->n_layers < 2 || d->n_layers > MYEA_MAX_LAYERS) return MYEA_E_INVALID;
@@ -111,13 +114,30 @@ int myea_net_desc_layout(myea_net_desc *d)
 
     for (uint32_t li = 0; li < d->n_layers; ++li) {
         myea_layer_desc *l = &d->layers[li];
-        if (l->n_units == 0 && l->type_layer != MYEA_LAYER_RESIDUAL) return MYEA_E_INVALID;
+        const int pooling = is_pooling(l);
+        if (l->n_units == 0 && l->type_layer != MYEA_LAYER_RESIDUAL && !pooling) return MYEA_E_INVALID;
         if (l->type_layer == MYEA_LAYER_LSTM && l->n_cells_per_block == 0) return MYEA_E_INVALID;
         if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED && l->type_layer != MYEA_LAYER_LSTM &&
-            l->type_layer != MYEA_LAYER_RESIDUAL) return MYEA_E_UNSUPPORTED;
+            l->type_layer != MYEA_LAYER_RESIDUAL && !pooling) return MYEA_E_UNSUPPORTED;
+        if (pooling && (l->pooling_values[0] == 0 || l->pooling_values[1] == 0 || li == 0 || li + 1 == d->n_layers)) return MYEA_E_INVALID;
         if (l->type_normalization != MYEA_NORMALIZATION_NONE) any_norm = 1;
     }
-    if (d->layers[0].type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_INVALID;
+    if (d->layers[0].type_layer != MYEA_LAYER_FULLY_CONNECTED || d->layers[d->n_layers - 1].type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_INVALID;
+    /* widths of the pooling layers, in layer order (Assign__Post__Layer, NN/Neural_Network__Compile.cpp:250-271):
+     * average: floor or ceil((In + 2 padding - kernel) / stride + 1) - the dilation is not in the formula;
+     * max:     floor or ceil((In + 2 padding - dilation (kernel - 1) - 1) / stride + 1) */
+    for (uint32_t li = 1; li < d->n_layers; ++li) {
+        myea_layer_desc *l = &d->layers[li];
+        if (!is_pooling(l)) continue;
+        if (enclosing_block(d, li) != 0) return MYEA_E_UNSUPPORTED;
+        const double in = (double)number_outputs(d, previous_layer(d, li));
+        const double kernel = l->pooling_values[0], stride = l->pooling_values[1], padding = l->pooling_values[2], dilation = l->pooling_values[3];
+        const double span = l->type_layer == MYEA_LAYER_AVERAGE_POOLING ? in + 2.0 * padding - kernel : in + 2.0 * padding - dilation * (kernel - 1.0) - 1.0;
+        if (span < 0.0) return MYEA_E_INVALID;
+        const double out = l->pooling_values[4] == 0 ? floor(span / stride + 1.0) : ceil(span / stride + 1.0);
+        if (out < 1.0 || out > 4294967295.0) return MYEA_E_INVALID;
+        l->n_units = (uint32_t)out;
+    }
     /* residual blocks: depth >= 1, wholly inside the stack, followed by at least one layer, fully-connected
      * members only, no block inside a block */
     for (uint32_t li = 1; li < d->n_layers; ++li) {
@@ -132,7 +152,7 @@ int myea_net_desc_layout(myea_net_desc *d)
     /* weights: Prepare__Connections__FC / __LSTM, NN/Neural_Network__Prepare_Connections.cpp:20-222 */
     for (uint32_t li = 1; li < d->n_layers; ++li) {
         myea_layer_desc *l = &d->layers[li];
-        if (l->type_layer == MYEA_LAYER_RESIDUAL) { l->first_connection_index = l->last_connection_index = total_weights; continue; }
+        if (l->type_layer == MYEA_LAYER_RESIDUAL || is_pooling(l)) { l->first_connection_index = l->last_connection_index = total_weights; continue; }
         uint64_t fan_in = number_outputs(d, previous_layer(d, li));
         l->first_connection_index = total_weights;
         if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
@@ -150,7 +170,7 @@ int myea_net_desc_layout(myea_net_desc *d)
      * overwrites the first at :240); the kernels use the field as stored. */
     for (uint32_t li = 1; li < d->n_layers; ++li) {
         myea_layer_desc *l = &d->layers[li];
-        if (l->type_layer == MYEA_LAYER_RESIDUAL) { l->first_bias_connection_index = total_weights + total_bias; continue; }
+        if (l->type_layer == MYEA_LAYER_RESIDUAL || is_pooling(l)) { l->first_bias_connection_index = total_weights + total_bias; continue; }
         if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             l->first_bias_connection_index = total_weights + total_bias;
             total_bias += l->n_units;
@@ -180,6 +200,8 @@ int myea_net_desc_layout(myea_net_desc *d)
         if (l->type_layer == MYEA_LAYER_LSTM) {
             uint64_t dirs = l->use_bidirectional ? 2u : 1u;
             total_norm += 3u * (uint64_t)l->n_units * l->n_cells_per_block * dirs + 6u * (uint64_t)l->n_units * dirs;
+        } else if (is_pooling(l)) {
+            /* pooling layers own none (Prepare__Normalized__Layer, NN/Neural_Network__Layer_Normalization.cpp:44-45) */
         } else if (l->type_layer == MYEA_LAYER_RESIDUAL) {
             total_norm += number_outputs(d, li + l->block_depth);   /* Prepare__Normalized__Layer, :60-67 */
         } else if (enclosing_block(d, li) != 0) {

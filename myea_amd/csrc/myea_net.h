@@ -29,6 +29,7 @@ struct DevLayer {
     float *means = nullptr, *variances = nullptr, *means_averages = nullptr, *variances_averages = nullptr;
     float *r_corrections = nullptr, *d_corrections = nullptr;
     float *colscale = nullptr;  // dropout multiplier per (t, unit)
+    unsigned *pool_index = nullptr;  // max pooling: padded position each output took its value from [T][Bmax][H]
     int *unit_act = nullptr;    // per-unit activation types [AH], null = layer-wide
     float *unit_steep = nullptr;  // per-unit steepnesses [AH], null = layer-wide
     LstmLayer *lstm = nullptr, *lstm2 = nullptr;  // lstm2: the time-reversed direction of a bidirectional layer
@@ -41,6 +42,7 @@ struct ProfEvent {
     double work = 0;
 };
 
+bool layer_is_pooling(const myea_layer_desc &l);
 bool layer_uses_norm(const myea_layer_desc &l);
 bool layer_uses_bias(const myea_layer_desc &l);
 
@@ -70,6 +72,8 @@ struct Net {
     ~Net();
     int create(const myea_net_desc &desc);
     int clear_optimizer();
+    PoolParams pool_params(size_t li, size_t rows) const;
+    int forward_pool_layer(size_t li, size_t B);
     int output_error_params(size_t B, const float *desired, int on_device, const char *fn, ErrorParams *p);
     int compute_loss(size_t B, const float *desired, int on_device);
     int compute_accuracy_r(size_t B, const float *desired, int on_device, float desired_mean, float predicted_mean);

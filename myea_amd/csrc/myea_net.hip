@@ -51,6 +51,7 @@ static int dev_alloc(float **p, size_t count)
         if (rc__ != MYEA_OK) return rc__; \
     } while (0)
 
+bool layer_is_pooling(const myea_layer_desc &l) { return l.type_layer == MYEA_LAYER_AVERAGE_POOLING || l.type_layer == MYEA_LAYER_MAX_POOLING; }
 bool layer_uses_norm(const myea_layer_desc &l) { return l.type_normalization != MYEA_NORMALIZATION_NONE; }
 bool layer_uses_bias(const myea_layer_desc &l) { return !layer_uses_norm(l); }  // Layer::Use__Bias, Data.hpp:736
 
@@ -97,14 +98,31 @@ static int check_desc(const myea_net_desc &d)
     if (d.total_parameters != d.total_weights + d.total_bias + 2 * d.total_normalized_units) { set_last_error("descriptor: total_parameters inconsistent"); return MYEA_E_INVALID; }
     if (d.layers[0].type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("descriptor: the input layer must be a fully-connected (unit) layer"); return MYEA_E_INVALID; }
     // residual blocks: members are the block_depth fully-connected layers after the residual layer, a consumer follows
-    bool any_residual = false, any_lstm = false;
+    bool any_residual = false, any_lstm = false, any_pool = false;
     uint32_t block_end = 0;  // index of the last member of the block being walked, 0 outside
     std::vector<int> group(d.n_layers, 0);
     for (uint32_t li = 0; li < d.n_layers; ++li) {
         const myea_layer_desc &l = d.layers[li];
-        if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED && l.type_layer != MYEA_LAYER_LSTM && l.type_layer != MYEA_LAYER_RESIDUAL) {
+        if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED && l.type_layer != MYEA_LAYER_LSTM && l.type_layer != MYEA_LAYER_RESIDUAL && !layer_is_pooling(l)) {
             set_last_error("layer %u: type %u is not on this path", li, l.type_layer);
             return MYEA_E_UNSUPPORTED;
+        }
+        if (layer_is_pooling(l)) {
+            // between fully-connected / pooling layers of a stack without blocks around it; the width must be the one
+            // Assign__Post__Layer computes (NN/Neural_Network__Compile.cpp:250-271) - the kernels index with it
+            any_pool = true;
+            if (li == 0 || li + 1 >= d.n_layers || block_end != 0) { set_last_error("layer %u: a pooling layer sits between the input and the output layer, outside residual blocks", li); return MYEA_E_UNSUPPORTED; }
+            const myea_layer_desc &pl = d.layers[li - 1], &nl = d.layers[li + 1];
+            if ((pl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(pl)) || (nl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(nl))) {
+                set_last_error("layer %u: pooling layers connect to fully-connected or pooling layers on this path", li);
+                return MYEA_E_UNSUPPORTED;
+            }
+            const double in = (double)myea_net_desc_number_outputs(&d, li - 1), k = l.pooling_values[0], st = l.pooling_values[1], pad = l.pooling_values[2], dil = l.pooling_values[3];
+            if (k < 1 || st < 1) { set_last_error("layer %u: pooling kernel and stride must be >= 1", li); return MYEA_E_INVALID; }
+            const double span = l.type_layer == MYEA_LAYER_AVERAGE_POOLING ? in + 2 * pad - k : in + 2 * pad - dil * (k - 1) - 1;
+            const double out = span < 0 ? 0 : (l.pooling_values[4] == 0 ? std::floor(span / st + 1.0) : std::ceil(span / st + 1.0));
+            if (out < 1 || (double)l.n_units != out) { set_last_error("layer %u: pooling width %u does not follow from its parameters (%.0f)", li, l.n_units, out); return MYEA_E_INVALID; }
+            if (l.type_dropout != MYEA_DROPOUT_NONE || l.type_normalization != MYEA_NORMALIZATION_NONE) { set_last_error("layer %u: a pooling layer carries no dropout or normalization", li); return MYEA_E_UNSUPPORTED; }
         }
         if (block_end != 0) {
             if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("layer %u: only fully-connected layers may sit inside a residual block", li); return MYEA_E_UNSUPPORTED; }
@@ -118,6 +136,7 @@ static int check_desc(const myea_net_desc &d)
         }
         if (l.type_layer == MYEA_LAYER_LSTM) any_lstm = true;
     }
+    if (any_pool && any_lstm) { set_last_error("descriptor: pooling layers are on this path for stacks without LSTM layers"); return MYEA_E_UNSUPPORTED; }
     if (any_residual && (any_lstm || d.number_recurrent_depth != 1)) { set_last_error("descriptor: residual blocks are on this path for feed-forward stacks only"); return MYEA_E_UNSUPPORTED; }
     for (uint32_t li = 0; li < d.n_layers; ++li) {
         const myea_layer_desc &l = d.layers[li];
@@ -128,6 +147,7 @@ static int check_desc(const myea_net_desc &d)
             continue;
         }
         if (l.n_units == 0) { set_last_error("layer %u: no units", li); return MYEA_E_INVALID; }
+        if (layer_is_pooling(l)) continue;
         if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_BERNOULLI && l.type_dropout != MYEA_DROPOUT_BERNOULLI_INVERTED) {
             set_last_error("layer %u: dropout type %u is not on this path", li, l.type_dropout);
             return MYEA_E_UNSUPPORTED;
@@ -201,7 +221,13 @@ int Net::create(const myea_net_desc &desc)
         if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(dev_alloc(&o.colscale, T * o.AH));
         if (li == 0) continue;
         if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_create_layer(li)); continue; }
-        if (l.type_layer != MYEA_LAYER_RESIDUAL) {
+        if (l.type_layer == MYEA_LAYER_MAX_POOLING) {
+            void *q = nullptr;
+            MYEA_HIP_TRY(hipMalloc(&q, (sz ? sz : 1) * sizeof(unsigned)));
+            o.pool_index = static_cast<unsigned *>(q);
+            MYEA_HIP_TRY(hipMemset(o.pool_index, 0, (sz ? sz : 1) * sizeof(unsigned)));
+        }
+        if (l.type_layer != MYEA_LAYER_RESIDUAL && !layer_is_pooling(l)) {
             MYEA_TRY(dev_alloc(&o.summations, sz));
             MYEA_HIP_TRY(hipMemset(o.summations, 0, sz * sizeof(float)));
         }
@@ -259,7 +285,7 @@ Net::~Net()
     fr(seg_first); fr(seg_len);
     fr(masks);
     for (DevLayer &o : L) {
-        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep);
+        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index);
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
@@ -387,10 +413,35 @@ int Net::forward_pass(size_t B, const float *inputs, int on_device)
     }
     for (size_t li = 1; li < d.n_layers; ++li) {
         if (d.layers[li].type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(forward_fc_layer(li, B));
+        else if (layer_is_pooling(d.layers[li])) MYEA_TRY(forward_pool_layer(li, B));
         else if (d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) {
             MYEA_TRY(forward_residual_block(li, B));
             li += d.layers[li].block_depth;  // the walk resumes after the block's last member
         } else MYEA_TRY(lstm_forward_layer(li, B));
+    }
+    return MYEA_OK;
+}
+
+PoolParams Net::pool_params(size_t li, size_t rows) const
+{
+    const myea_layer_desc &l = d.layers[li];
+    PoolParams p{};
+    p.rows = rows; p.In = L[li].In; p.H = L[li].H;
+    p.kernel = l.pooling_values[0]; p.stride = l.pooling_values[1]; p.padding = l.pooling_values[2]; p.dilation = l.pooling_values[3];
+    p.is_max = l.type_layer == MYEA_LAYER_MAX_POOLING;
+    return p;
+}
+
+int Net::forward_pool_layer(size_t li, size_t B)
+{
+    DevLayer &o = L[li];
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
+    const float *x = layer_outputs(o.prev);
+    const bool per_t = T > 1 && B != Bmax;
+    const size_t chunks = per_t ? T : 1, rows = per_t ? B : T * B;
+    for (size_t c = 0; c < chunks; ++c) {
+        const size_t roff = c * Bmax;
+        MYEA_TRY(launch_pool_forward(stream, pool_params(li, rows), x + roff * o.In, o.values + roff * o.H, o.pool_index ? o.pool_index + roff * o.H : nullptr));
     }
     return MYEA_OK;
 }
@@ -558,6 +609,9 @@ int Net::backward_into_layer(size_t li, size_t B)
     }
     const myea_layer_desc &next = d.layers[gi];
     DevLayer &on = L[gi];
+    // a pooling consumer hands its errors down through its windows instead of a contraction
+    const bool pool_consumer = layer_is_pooling(next);
+    if (pool_consumer) have_gemm = false;
     // what the consumer hands down: delta [T][Bmax][Out] and weights [Out][H]
     const float *delta = on.neuron_errors, *weights = parameters + next.first_connection_index;
     size_t Out = on.H;
@@ -590,6 +644,7 @@ int Net::backward_into_layer(size_t li, size_t B)
         if (!is_fc) {  // an LSTM layer receives the plain delta of its cell outputs (BPTT follows), a residual layer that of its units
             g.C = o.neuron_errors + roff * H;
             g.epilogue = EPI_NONE;
+            if (pool_consumer) { MYEA_TRY(launch_pool_backward(stream, pool_params(gi, rows), on.neuron_errors + roff * on.H, on.pool_index ? on.pool_index + roff * on.H : nullptr, g.C)); continue; }
             if (!have_gemm) { MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors, shortcut->H, crop, identity, H, 0, g.C)); continue; }
             prof_begin(1);
             MYEA_TRY(launch_gemm(stream, g));
@@ -612,6 +667,8 @@ int Net::backward_into_layer(size_t li, size_t B)
             prof_begin(1);
             MYEA_TRY(launch_gemm(stream, g));
             prof_end(2.0 * (double)rows * (double)H * (double)Out);
+        } else if (pool_consumer) {
+            MYEA_TRY(launch_pool_backward(stream, pool_params(gi, rows), on.neuron_errors + roff * on.H, on.pool_index ? on.pool_index + roff * on.H : nullptr, g.C));
         } else {
             MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors, shortcut->H, crop, identity, H, 0, g.C));
         }
@@ -730,7 +787,7 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
     for (size_t li = first; li < end; ++li) {
         const myea_layer_desc &l = d.layers[li];
         if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_update_derivative_weight(li, B)); continue; }
-        if (l.type_layer == MYEA_LAYER_RESIDUAL) continue;  // owns no connection (:31-36)
+        if (l.type_layer == MYEA_LAYER_RESIDUAL || layer_is_pooling(l)) continue;  // own no connection (:31-36)
         DevLayer &o = L[li];
         const size_t In = o.In, H = o.H;
         // Layer::ptr_array_pre_summations: the operand the weights were applied to (NN/Neural_Network__Ordered.cpp:96-141)

@@ -64,6 +64,8 @@ typedef struct olayer {
     uint32_t *unit_af; float *unit_steep;
     /* LSTM: one olstm per direction */
     struct olstm *lstm;
+    /* max pooling: Basic_indice_unit::ptr_array_indices, the (padded) position each output took its value from [T][Bmax][H] */
+    uint32_t *pool_index;
 } olayer;
 
 struct myea_oracle_net {
@@ -213,6 +215,8 @@ static float *shift_ptr(myea_oracle_net *n, float *base, size_t li)
 /* ------------------------------------------------------------------------------------------- */
 /* life cycle */
 
+static int is_pooling(const myea_layer_desc *l) { return l->type_layer == MYEA_LAYER_AVERAGE_POOLING || l->type_layer == MYEA_LAYER_MAX_POOLING; }
+
 static size_t layer_width(const myea_layer_desc *l)
 {
     if (l->type_layer == MYEA_LAYER_LSTM) return (size_t)l->n_units * l->n_cells_per_block;
@@ -307,6 +311,10 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
             continue;
         }
         o->af_errors = zalloc(T * B * o->AH);
+        if (is_pooling(l)) {   /* basic (indice) units: values and errors only */
+            if (l->type_layer == MYEA_LAYER_MAX_POOLING) o->pool_index = (uint32_t *)calloc(sz ? sz : 1, sizeof(uint32_t));
+            continue;
+        }
         if (l->type_layer != MYEA_LAYER_RESIDUAL) {
             o->summations = zalloc(sz);
             o->neuron_errors = zalloc(sz);
@@ -343,6 +351,7 @@ int myea_oracle_destroy(myea_oracle_net *n)
         free(o->neuron_errors); free(o->af_errors); free(o->norm_errors);
         free(o->means); free(o->variances); free(o->means_averages); free(o->variances_averages);
         free(o->r_corrections); free(o->d_corrections); free(o->derivatives_means); free(o->derivatives_variances);
+        free(o->pool_index);
         free(o->unit_af); free(o->unit_steep);
         if (o->lstm) {
             for (int dir = 0; dir < 2; ++dir) {
@@ -907,6 +916,68 @@ static void bwd_lstm_layer(myea_oracle_net *n, size_t li, size_t B)
  * RNN__Forward_Pass_Batch: NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:24-130 (layer-major,
  * every layer loops over t); FF/RNN__Assign_Inputs: NN/Neural_Network__Assign_Inputs.cpp:20-204
  * (example rows are [T][In]; scattered into [T][Bmax][In]; input-layer dropout applied in place). */
+/* Forward_Pass__Average_Pooling / __Max_Pooling (NN/Neural_Network__Forward_Pass__Loop.cpp:4537-4583, 5070-5135): windows over the
+ * feature axis of one example; positions are counted in the padded coordinate p = output * stride + k * dilation, the input
+ * sits at [padding, padding + In).  Average: padding contributes 0 and the divisor is always the kernel size.  Max: a padded
+ * position stands for the value 0; the index kept for the backward pass is the padded coordinate of the first maximum. */
+static void fwd_pooling(myea_oracle_net *n, size_t li, size_t t, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    size_t Bmax = n->d.batch_size, In = o->In, H = o->H;
+    size_t kernel = l->pooling_values[0], stride = l->pooling_values[1], padding = l->pooling_values[2], dilation = l->pooling_values[3];
+    const float *x = layer_outputs(n, o->prev) + Bmax * In * t;
+    float *y = o->values + Bmax * H * t;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            if (l->type_layer == MYEA_LAYER_AVERAGE_POOLING) {
+                float s = 0.f;
+                for (size_t k = 0; k < kernel; ++k) {
+                    size_t p = j * stride + k * dilation;
+                    if (p < padding || p >= In + padding) continue;
+                    s += x[b * In + p - padding];
+                }
+                y[b * H + j] = s * (1.f / (float)kernel);
+            } else {
+                size_t at = 0; float mx = -FLT_MAX;
+                for (size_t k = 0; k < kernel; ++k) {
+                    size_t p = j * stride + k * dilation;
+                    if (p < padding || p >= In + padding) { if (mx < 0.f) { at = p; mx = 0.f; } }
+                    else if (mx < x[b * In + p - padding]) { at = p; mx = x[b * In + p - padding]; }
+                }
+                o->pool_index[Bmax * H * t + b * H + j] = (uint32_t)at;
+                y[b * H + j] = mx;
+            }
+        }
+}
+
+/* Backward_Pass__Average_Pooling / __Max_Pooling (NN/Neural_Network__Backward_Pass__Loop.cpp:1004-1049, 1139-1181): the pooling layer
+ * ci hands its errors down to `dst` (the previous layer's derivative outputs, In wide), added in place */
+static void bwd_pooling_to_previous(myea_oracle_net *n, size_t ci, size_t t, size_t B, float *dst)
+{
+    const myea_layer_desc *l = &n->d.layers[ci];
+    olayer *o = &n->L[ci];
+    size_t Bmax = n->d.batch_size, In = o->In, H = o->H;
+    size_t kernel = l->pooling_values[0], stride = l->pooling_values[1], padding = l->pooling_values[2], dilation = l->pooling_values[3];
+    const float *dy = o->af_errors + Bmax * H * t;
+    float *dx = dst + Bmax * In * t;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            if (l->type_layer == MYEA_LAYER_AVERAGE_POOLING) {
+                float e = dy[b * H + j] * (1.f / (float)kernel);
+                for (size_t k = 0; k < kernel; ++k) {
+                    size_t p = j * stride + k * dilation;
+                    if (p < padding || p >= In + padding) continue;
+                    dx[b * In + p - padding] += e;
+                }
+            } else {
+                size_t p = o->pool_index[Bmax * H * t + b * H + j];
+                if (p < padding || p >= In + padding) continue;
+                dx[b * In + p - padding] += dy[b * H + j];
+            }
+        }
+}
+
 int myea_oracle_forward_pass(myea_oracle_net *n, size_t B, const float *inputs)
 {
     if (!n || !inputs) return MYEA_E_INVALID;
@@ -925,6 +996,8 @@ int myea_oracle_forward_pass(myea_oracle_net *n, size_t B, const float *inputs)
         } else if (l->type_layer == MYEA_LAYER_RESIDUAL) {
             fwd_residual_block(n, li, B);
             li += l->block_depth; /* the iterator is left on the block's last member, :3884-3885 */
+        } else if (is_pooling(l)) {
+            for (size_t t = 0; t < T; ++t) fwd_pooling(n, li, t, B);
         } else return MYEA_E_UNSUPPORTED;
     }
     return MYEA_OK;
@@ -1266,6 +1339,8 @@ int myea_oracle_backward_pass(myea_oracle_net *n, size_t B)
                 for (size_t tt = 0; tt < T; ++tt) bwd_lstm_to_previous(n, ci, tt, B, dst);
             } else if (next->type_layer == MYEA_LAYER_RESIDUAL) {
                 bwd_residual_shortcut(n, B, n->L[ci].H, o->H, n->L[ci].pad, n->L[ci].af_errors, dst);
+            } else if (is_pooling(next)) {
+                for (size_t tt = 0; tt < T; ++tt) bwd_pooling_to_previous(n, ci, tt, B, dst);
             } else return MYEA_E_UNSUPPORTED;
         }
         if (cur->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
@@ -1275,6 +1350,8 @@ int myea_oracle_backward_pass(myea_oracle_net *n, size_t B)
         } else if (cur->type_layer == MYEA_LAYER_RESIDUAL) {
             bwd_gradient_residual(n, li, B);
             gi = li + 1;
+        } else if (is_pooling(cur)) {
+            /* a pooling layer has no gradient of its own (NN/Neural_Network__Backward_Pass__Loop.cpp:184-185) */
         } else return MYEA_E_UNSUPPORTED;
     }
     return MYEA_OK;
@@ -1319,7 +1396,7 @@ int myea_oracle_update_derivative_weight(myea_oracle_net *n, size_t B, size_t fi
     size_t T = n->d.number_recurrent_depth;
     for (size_t li = first; li < end; ++li) {
         const myea_layer_desc *l = &n->d.layers[li];
-        if (l->type_layer == MYEA_LAYER_RESIDUAL) continue;
+        if (l->type_layer == MYEA_LAYER_RESIDUAL || is_pooling(l)) continue;
         if (l->type_layer == MYEA_LAYER_LSTM) { dw_lstm(n, li, B); continue; }
         if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_UNSUPPORTED;
         olayer *o = &n->L[li];
@@ -1396,7 +1473,7 @@ static int max_norm_constraints(myea_oracle_net *n)
 {
     for (size_t li = 1; li < n->d.n_layers; ++li) {
         const myea_layer_desc *l = &n->d.layers[li];
-        if (l->type_layer == MYEA_LAYER_RESIDUAL) continue;
+        if (l->type_layer == MYEA_LAYER_RESIDUAL || is_pooling(l)) continue;
         if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             for (size_t o = 0; o < n->L[li].H; ++o) max_norm_segment(n, l->first_connection_index + o * n->L[li].In, n->L[li].In, 0);
         } else if (l->type_layer == MYEA_LAYER_LSTM) {
@@ -1547,7 +1624,7 @@ const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t 
     switch (kind) {
     case MYEA_TENSOR_OUTPUTS: p = layer_outputs(n, li); break;
     case MYEA_TENSOR_SUMMATIONS: p = o->summations; break;
-    case MYEA_TENSOR_ERRORS: p = n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL ? o->af_errors : o->neuron_errors; break;
+    case MYEA_TENSOR_ERRORS: p = (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL || is_pooling(&n->d.layers[li])) ? o->af_errors : o->neuron_errors; break;
     case MYEA_TENSOR_NORM_HATS: p = o->hats; c = T * n->d.batch_size * o->NH; break;
     case MYEA_TENSOR_INPUT_SIDE_ERRORS:
         if (o->group == 2) p = layer_uses_norm(&n->d.layers[li]) ? o->norm_errors : o->af_errors;
