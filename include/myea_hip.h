@@ -69,7 +69,8 @@ enum {
 
 /* Enum_Type_Layer_Dropout.hpp */
 enum {
-    MYEA_DROPOUT_NONE = 0, MYEA_DROPOUT_BERNOULLI = 2, MYEA_DROPOUT_BERNOULLI_INVERTED = 3
+    MYEA_DROPOUT_NONE = 0, MYEA_DROPOUT_BERNOULLI = 2, MYEA_DROPOUT_BERNOULLI_INVERTED = 3,
+    MYEA_DROPOUT_ZONEOUT = 7   /* LSTM layers only: dropout_values[0] / [1] = zoneout probability of the cell state / the cell output */
 };
 
 /* Enum_Type_Layer_Normalization.hpp */
@@ -312,6 +313,14 @@ int myea_hip_download_optimizer_state(myea_hip_net *net, int kind, float *host, 
 int myea_hip_set_unit_activations(myea_hip_net *net, size_t layer_index, const uint32_t *host_types, const float *host_steepness, size_t count);
 
 int myea_hip_upload_masks(myea_hip_net *net, const uint8_t *host_masks, size_t count);
+/* Zoneout masks of the LSTM layers, drawn by the caller as Dropout_Zoneout() does (Neural_Network__Dropout__Zoneout__Loop.cpp:57-87)
+ * and laid out as ptr_array_cell_units_mask_dropout_zoneout (Reset__Parameters__Cell_Unit__Mask_Dropout, Neural_Network.cpp:3964-3995):
+ * first the cell-STATE masks, per LSTM layer in layer order [T][cells of the layer], then - at offset T x (cells of all LSTM
+ * layers) - the cell-OUTPUT masks in the same arrangement.  1 = update the unit, 0 = keep its previous value (0 on a sequence's
+ * first step).  One mask per (time step, cell), shared by the batch.  `count` = 2 x T x total cells; all 1 after create.  The
+ * masks act in the training state only (Neural_Network__Forward_Pass__Loop.cpp:2088-2092); the backward pass does not read them,
+ * as in the reference. */
+int myea_hip_upload_zoneout_masks(myea_hip_net *net, const uint8_t *host_masks, size_t count);
 /* Clear_Training_Arrays (Train.cpp:93-126) + Clear_Optimizer (Train.cpp:128-263): zero the gradient
  * vector and all optimizer state, optimizer_time_step = 0. */
 int myea_hip_clear_training_arrays(myea_hip_net *net);

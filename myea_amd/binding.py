@@ -24,7 +24,7 @@ AF = dict(NONE=0, COSINE=1, COSINE_SYMMETRIC=2, ELU=3, ELLIOT=4, ELLIOT_SYMMETRI
           SINE=19, SIGMOID_STEPWISE=20, SINE_SYMMETRIC=21, SOFTMAX=22, TANH=23, TANH_STEPWISE=24,
           THRESHOLD=25, THRESHOLD_SYMMETRIC=26)
 OPTIMIZER = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP_PLUS=8, NOSADAM=9)
-DROPOUT = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3)
+DROPOUT = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3, ZONEOUT=7)
 NORMALIZATION = dict(NONE=0, BATCH_NORMALIZATION=1, BATCH_RENORMALIZATION=2)
 LOSS = dict(NONE=0, BIT=1, CROSS_ENTROPY=2, L1=3, L2=4, MAE=5, MAPE=6, ME=9, MSE=10, RMSE=11, SMAPE=12)
 ACCURACY = dict(NONE=0, CROSS_ENTROPY=1, DIRECTIONAL=2, DISTANCE=3, R=4, SIGN=5)
@@ -96,7 +96,7 @@ ABI_SYMBOLS = [
     "myea_hip_synchronize", "myea_hip_last_error", "myea_hip_set_hyper", "myea_hip_get_hyper",
     "myea_hip_set_state_propagation", "myea_hip_upload_parameters", "myea_hip_download_parameters",
     "myea_hip_upload_optimizer_state", "myea_hip_download_optimizer_state", "myea_hip_upload_masks", "myea_hip_set_unit_activations",
-    "myea_hip_compute_loss", "myea_hip_compute_accuracy_r", "myea_hip_gather_examples", "myea_hip_device_buffer_create", "myea_hip_device_buffer_destroy",
+    "myea_hip_upload_zoneout_masks", "myea_hip_compute_loss", "myea_hip_compute_accuracy_r", "myea_hip_gather_examples", "myea_hip_device_buffer_create", "myea_hip_device_buffer_destroy",
     "myea_hip_clear_training_arrays", "myea_hip_forward_pass", "myea_hip_compute_error", "myea_hip_backward_pass",
     "myea_hip_update_derivative_weight", "myea_hip_update_parameter", "myea_hip_reset_loss", "myea_hip_get_loss",
     "myea_hip_download_gradient", "myea_hip_upload_gradient", "myea_hip_download_tensor",
@@ -146,6 +146,7 @@ def load_library(path=LIB_PATH):
     lib.myea_hip_update_parameter.argtypes = [vp, sz, sz]
     lib.myea_hip_reset_loss.argtypes = [vp]
     lib.myea_hip_get_loss.argtypes = [vp, P(LossState)]
+    lib.myea_hip_upload_zoneout_masks.argtypes = [vp, vp, sz]
     lib.myea_hip_compute_loss.argtypes = [vp, sz, vp, i32]
     lib.myea_hip_compute_accuracy_r.argtypes = [vp, sz, vp, i32, C.c_float, C.c_float]
     lib.myea_hip_gather_examples.argtypes = [vp, vp, vp, sz, sz, vp, i32, sz]
@@ -197,6 +198,7 @@ def make_desc(layers, batch_size, recurrent_depth=1, network=None, lib=None):
         l.activation_steepness = spec.get("steepness", 1.0)
         l.type_dropout = DROPOUT[spec.get("dropout", "NONE")]
         l.dropout_values[0] = spec.get("keep", 1.0)
+        l.dropout_values[1] = spec.get("keep_output", 0.0)
         l.type_normalization = NORMALIZATION[spec.get("normalization", "NONE")]
         l.use_layer_normalization_before_activation = int(spec.get("norm_before", True))
         l.block_depth = spec.get("block_depth", 0)
@@ -303,6 +305,10 @@ class HipNetwork:
         out = np.empty(count, dtype=np.float32)
         self._check(self.lib.myea_hip_download_tensor(self.handle, layer, kind, _ptr(out), out.size))
         return out
+
+    def upload_zoneout_masks(self, m):
+        m = np.ascontiguousarray(m, dtype=np.uint8)
+        self._check(self.lib.myea_hip_upload_zoneout_masks(self.handle, _ptr(m), m.size))
 
     def Clear_Training_Arrays(self): self._check(self.lib.myea_hip_clear_training_arrays(self.handle))
 

@@ -170,6 +170,7 @@ struct LstmFusedForward {
     float *acts;           // [B][4C]  in: input sums; out: the activations z, i, f, o
     const float *c_prev;   // [B][C]
     float *c, *ca, *h;     // [B][C]   cell state, tanh(cell state), cell output
+    const uint8_t *zone_state, *zone_output;   // [C] zoneout masks of this time step (1 = update), or null
 };
 struct LstmFusedBackward {
     size_t B, C;

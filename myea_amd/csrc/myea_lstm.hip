@@ -33,6 +33,8 @@ struct LstmLayer {
     float *h = nullptr, *dh = nullptr;                           // [T][Bmax][C] cell outputs and their delta
     float *Win = nullptr, *Wrec = nullptr, *peep = nullptr;      // packed parameters
     float *WrecT = nullptr; // [C][G] transposed Wrec for the fused backward step; null when the fused step is not used
+    const uint8_t *zone_state = nullptr, *zone_output = nullptr;   // zoneout masks [T][zone_stride], this direction's cells from 0
+    size_t zone_stride = 0;
     bool fused = false;     // one launch per time step (myea_lstm_fused.hip) instead of contraction + gate kernel
     float *gWin = nullptr, *gWrec = nullptr;                     // packed gradient scratch
     float *acts = nullptr;  // [T][Bmax][G]: pre-activation sums, overwritten in place by z | i | f | o
@@ -112,7 +114,8 @@ __device__ __forceinline__ float tanh_f(float s) { return 2.f / (1.f + expf(-2.f
 // `part` holds `nparts` slabs [B][G] of the recurrent contraction h[t-1] Wrec^T (split along K), summed here in order.
 __global__ __launch_bounds__(kBlock) void lstm_forward_step_kernel(LstmGeom g, size_t B, int first, const float *bias, const float *peep,
                                                                    float *acts, const float *c_prev, float *c, float *ca, float *h,
-                                                                   const float *part, int nparts)
+                                                                   const float *part, int nparts, const float *h_prev,
+                                                                   const uint8_t *zone_state, const uint8_t *zone_output)
 {
     const size_t n = B * g.K;
     for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < n; idx += (size_t)gridDim.x * kBlock) {
@@ -142,14 +145,22 @@ __global__ __launch_bounds__(kBlock) void lstm_forward_step_kernel(LstmGeom g, s
             const size_t cc = k * g.cpb + j;
             const float z = tanh_f(row[cc] + bias[cc]);
             row[cc] = z;
-            const float cs = first ? z * gi : z * gi + gf * c_prev[cell0 + j];
+            float cs = first ? z * gi : z * gi + gf * c_prev[cell0 + j];
+            // zoneout of the cell state: a masked-out cell keeps its previous state, 0 on the first step
+            // (Forward_Pass__LSTM__Gates_CIF_AF_State__Zoneout, NN/Neural_Network__Recurrent_Forward_Pass__Loop.cpp:1285-1288, 1331-1334)
+            if (zone_state && !zone_state[cc]) cs = first ? 0.f : c_prev[cell0 + j];
             c[cell0 + j] = cs;
             ca[cell0 + j] = tanh_f(cs);
             so += cs * po[j];
         }
         const float go = sigmoid_f(so);
         row[g.C + 2 * g.K + k] = go;
-        for (size_t j = 0; j < g.cpb; ++j) h[cell0 + j] = ca[cell0 + j] * go;
+        for (size_t j = 0; j < g.cpb; ++j) {
+            float hv = ca[cell0 + j] * go;
+            // zoneout of the cell output (Forward_Pass__LSTM__Output__Zoneout, :1475-1478, 1520-1523)
+            if (zone_output && !zone_output[k * g.cpb + j]) hv = first ? 0.f : h_prev[cell0 + j];
+            h[cell0 + j] = hv;
+        }
     }
 }
 
@@ -297,7 +308,7 @@ int Net::lstm_create_layer(size_t li)
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
     if (layer_uses_norm(l)) { set_last_error("layer %zu: normalisation inside an LSTM layer is not on this path", li); return MYEA_E_UNSUPPORTED; }
-    if (l.type_dropout != MYEA_DROPOUT_NONE) { set_last_error("layer %zu: dropout on an LSTM layer is not on this path", li); return MYEA_E_UNSUPPORTED; }
+    if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_ZONEOUT) { set_last_error("layer %zu: dropout type %u on an LSTM layer is not on this path", li, l.type_dropout); return MYEA_E_UNSUPPORTED; }
     if (l.n_cells_per_block == 0) { set_last_error("layer %zu: LSTM needs at least one cell per block", li); return MYEA_E_INVALID; }
     const size_t T = d.number_recurrent_depth, B = d.batch_size;
     const size_t dirs = l.use_bidirectional ? 2 : 1;
@@ -314,6 +325,16 @@ int Net::lstm_create_layer(size_t li)
         q->bias = l.first_bias_connection_index + dir * q->G;
         q->reverse = dir == 1;
         q->own_h = dirs == 2;
+        if (l.type_dropout == MYEA_DROPOUT_ZONEOUT) {
+            // ptr_array_cell_units_mask_dropout_zoneout (Reset__Parameters__Cell_Unit__Mask_Dropout, NN/Neural_Network.cpp:3964-3995):
+            // per LSTM layer [T][cells of the layer], cell-state masks first, cell-output masks T x (all cells) further on
+            size_t before = 0;
+            for (size_t lj = 1; lj < li; ++lj)
+                if (d.layers[lj].type_layer == MYEA_LAYER_LSTM) before += (size_t)d.layers[lj].n_units * d.layers[lj].n_cells_per_block * (d.layers[lj].use_bidirectional ? 2 : 1);
+            q->zone_stride = q->C * dirs;
+            q->zone_state = zoneout_masks + T * before + dir * q->C;
+            q->zone_output = q->zone_state + zoneout_count / 2;
+        }
         if (q->base + q->K * q->per_block > d.total_weights) { set_last_error("layer %zu: LSTM weight slice leaves the weight region", li); return MYEA_E_INVALID; }
         // The four bias vectors are read at bias + [0, G).  With the index as Prepare__Bias__LSTM leaves it (one direction)
         // they reach C entries into the following layers' bias slots; beyond the bias region the reference would read and
@@ -402,6 +423,9 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
     for (size_t s = 0; s < T; ++s) {
         const size_t t = q.reverse ? T - 1 - s : s, tp = q.reverse ? t + 1 : t - 1;  // tp: the step processed before t
         float *acts_t = q.acts + t * Bmax * q.G;
+        // zoneout acts strictly in the training state (NN/Neural_Network__Forward_Pass__Loop.cpp:2088-2092)
+        const bool zone = q.zone_state != nullptr && state == MYEA_STATE_TRAINING;
+        const uint8_t *zs = zone ? q.zone_state + t * q.zone_stride : nullptr, *zo = zone ? q.zone_output + t * q.zone_stride : nullptr;
         int nparts = 0;
         if (s > 0 && q.fused) {   // recurrent contraction and gate math of the step in one launch
             LstmFusedForward f{};
@@ -409,6 +433,7 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
             f.h_prev = q.h + tp * Bmax * q.C; f.Wrec = q.Wrec; f.bias = bias; f.peep = q.peep;
             f.acts = acts_t; f.c_prev = q.c + tp * Bmax * q.C;
             f.c = q.c + t * Bmax * q.C; f.ca = q.ca + t * Bmax * q.C; f.h = q.h + t * Bmax * q.C;
+            f.zone_state = zs; f.zone_output = zo;
             prof_begin(0);
             MYEA_TRY(launch_lstm_fused_forward(stream, f));
             prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
@@ -428,7 +453,7 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
         }
         hipLaunchKernelGGL(lstm_forward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, (int)(s == 0), bias, q.peep,
                            acts_t, s ? q.c + tp * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, q.h + t * Bmax * q.C,
-                           q.part, nparts);
+                           q.part, nparts, s ? q.h + tp * Bmax * q.C : nullptr, zs, zo);
         MYEA_HIP_TRY(hipGetLastError());
     }
     return MYEA_OK;

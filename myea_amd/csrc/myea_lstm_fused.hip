@@ -199,12 +199,15 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
         sf += cp * e_peep[q][1];
         const float gi = sigmoid_f(si), gf = sigmoid_f(sf);
         const float z = tanh_f(e_in[q][0] + rec[0] + e_bias[q][0]);
-        const float cs = z * gi + gf * cp;
+        float cs = z * gi + gf * cp;
+        if (p.zone_state && !p.zone_state[k]) cs = cp;   // zoned-out cell state: keep the previous one
         const float a = tanh_f(cs);
         const float so = e_in[q][3] + rec[3] + e_bias[q][3] + cs * e_peep[q][2];
         const float go = sigmoid_f(so);
         arow[k] = z; arow[C + k] = gi; arow[2 * C + k] = gf; arow[3 * C + k] = go;
-        p.c[ci] = cs; p.ca[ci] = a; p.h[ci] = a * go;
+        float hv = a * go;
+        if (p.zone_output && !p.zone_output[k]) hv = p.h_prev[ci];   // zoned-out cell output
+        p.c[ci] = cs; p.ca[ci] = a; p.h[ci] = hv;
     }
 }
 

@@ -53,6 +53,8 @@ struct Net {
     hipStream_t stream = nullptr;
     float *parameters = nullptr, *gradient = nullptr, *opt[MYEA_STATE_KINDS] = {};
     uint8_t *masks = nullptr;
+    uint8_t *zoneout_masks = nullptr;   // [state | output] halves, per LSTM layer [T][cells]
+    size_t zoneout_count = 0;
     // max-norm constraint: weight segments (one per neuron / per LSTM gate vector), built on first use
     unsigned long long *seg_first = nullptr;
     unsigned *seg_len = nullptr;

@@ -148,7 +148,9 @@ static int check_desc(const myea_net_desc &d)
         }
         if (l.n_units == 0) { set_last_error("layer %u: no units", li); return MYEA_E_INVALID; }
         if (layer_is_pooling(l)) continue;
-        if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_BERNOULLI && l.type_dropout != MYEA_DROPOUT_BERNOULLI_INVERTED) {
+        if (l.type_dropout == MYEA_DROPOUT_ZONEOUT && l.type_layer == MYEA_LAYER_LSTM) {
+            // masks per (time step, cell), uploaded with myea_hip_upload_zoneout_masks
+        } else if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_BERNOULLI && l.type_dropout != MYEA_DROPOUT_BERNOULLI_INVERTED) {
             set_last_error("layer %u: dropout type %u is not on this path", li, l.type_dropout);
             return MYEA_E_UNSUPPORTED;
         }
@@ -192,6 +194,13 @@ int Net::create(const myea_net_desc &desc)
         MYEA_HIP_TRY(hipMalloc(&q, d.total_mask_units ? d.total_mask_units : 1));
         masks = static_cast<uint8_t *>(q);
         MYEA_HIP_TRY(hipMemset(masks, 1, d.total_mask_units ? d.total_mask_units : 1));  // all true, NN/Neural_Network__Allocate.cpp:386-410
+        size_t cells = 0;
+        for (size_t li = 1; li < d.n_layers; ++li)
+            if (d.layers[li].type_layer == MYEA_LAYER_LSTM) cells += (size_t)d.layers[li].n_units * d.layers[li].n_cells_per_block * (d.layers[li].use_bidirectional ? 2 : 1);
+        zoneout_count = 2 * T * cells;
+        MYEA_HIP_TRY(hipMalloc(&q, zoneout_count ? zoneout_count : 1));
+        zoneout_masks = static_cast<uint8_t *>(q);
+        MYEA_HIP_TRY(hipMemset(zoneout_masks, 1, zoneout_count ? zoneout_count : 1));  // all true, NN/Neural_Network__Allocate.cpp:1209-1211
     }
     size_t max_h = 0;
     L.resize(d.n_layers);
@@ -283,7 +292,7 @@ Net::~Net()
     fr(parameters); fr(gradient);
     for (int k = 0; k < MYEA_STATE_KINDS; ++k) fr(opt[k]);
     fr(seg_first); fr(seg_len);
-    fr(masks);
+    fr(masks); fr(zoneout_masks);
     for (DevLayer &o : L) {
         fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index);
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
@@ -1120,6 +1129,15 @@ int myea_hip_upload_masks(myea_hip_net *n, const uint8_t *m, size_t c)
     NET_OR_FAIL(n);
     if (!m || c > n->net.d.total_mask_units) { myea::set_last_error("upload_masks: null or count %zu > %llu", c, (unsigned long long)n->net.d.total_mask_units); return MYEA_E_INVALID; }
     MYEA_HIP_TRY(hipMemcpyAsync(n->net.masks, m, c, hipMemcpyHostToDevice, n->net.stream));
+    MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
+    return MYEA_OK;
+}
+int myea_hip_upload_zoneout_masks(myea_hip_net *n, const uint8_t *m, size_t c)
+{
+    NET_OR_FAIL(n);
+    if (!m || c != n->net.zoneout_count) { myea::set_last_error("upload_zoneout_masks: null or count %zu != %zu (2 x T x cells of the LSTM layers)", c, n->net.zoneout_count); return MYEA_E_INVALID; }
+    if (c == 0) return MYEA_OK;
+    MYEA_HIP_TRY(hipMemcpyAsync(n->net.zoneout_masks, m, c, hipMemcpyHostToDevice, n->net.stream));
     MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
     return MYEA_OK;
 }

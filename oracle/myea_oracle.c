@@ -37,6 +37,8 @@ typedef struct olstm {
     size_t per_block;       /* parameters of one block */
     size_t base, bias;      /* flat index of the direction's first block and of its bias vectors z | i | f | o */
     int reverse;            /* the direction walks time from T-1 down to 0 */
+    const uint8_t *zone_state, *zone_output;   /* zoneout masks of the direction: [T][zone_stride], this direction's cells first at 0 */
+    size_t zone_stride;
     float *h, *dh;          /* cell outputs and their delta [T][Bmax][C]: the layer's own buffers for a one-direction layer */
     float *sum_in_z, *sum_rec_z, *sum_z, *z, *c, *ca;          /* cells */
     float *sum_in_i, *sum_in_f, *sum_in_o, *sum_rec_i, *sum_rec_f, *sum_rec_o, *sum_i, *sum_f, *sum_o, *gi, *gf, *go; /* blocks */
@@ -75,6 +77,7 @@ struct myea_oracle_net {
     int threads;
     float *parameters, *gradient, *opt[MYEA_STATE_KINDS];
     uint8_t *masks;
+    uint8_t *zoneout; size_t zoneout_count;   /* ptr_array_cell_units_mask_dropout_zoneout: state half, then output half */
     olayer L[MYEA_MAX_LAYERS];
     myea_loss_state loss;
 };
@@ -275,11 +278,18 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
             else o->AH = o->H;
         }
     }
+    size_t total_cells = 0, zone_at = 0;
+    for (size_t li = 0; li < desc->n_layers; ++li)
+        if (desc->layers[li].type_layer == MYEA_LAYER_LSTM) total_cells += (size_t)desc->layers[li].n_units * desc->layers[li].n_cells_per_block * (desc->layers[li].use_bidirectional ? 2 : 1);
+    n->zoneout_count = 2 * T * total_cells;
+    n->zoneout = (uint8_t *)malloc(n->zoneout_count ? n->zoneout_count : 1);
+    memset(n->zoneout, 1, n->zoneout_count ? n->zoneout_count : 1);
     for (size_t li = 0; li < desc->n_layers; ++li) {
         const myea_layer_desc *l = &desc->layers[li];
         olayer *o = &n->L[li];
         if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED) { free(n); return MYEA_E_UNSUPPORTED; }
-        if (l->type_layer == MYEA_LAYER_LSTM && (layer_uses_norm(l) || l->type_dropout != MYEA_DROPOUT_NONE)) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (l->type_layer == MYEA_LAYER_LSTM && (layer_uses_norm(l) || (l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_ZONEOUT))) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (l->type_layer != MYEA_LAYER_LSTM && l->type_dropout == MYEA_DROPOUT_ZONEOUT) { free(n); return MYEA_E_UNSUPPORTED; }
         size_t sz = T * B * o->H;
         o->values = zalloc(T * B * o->AH);
         if (li == 0) continue;
@@ -298,6 +308,9 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
                 q->base = l->first_connection_index + dir * q->K * q->per_block;
                 q->bias = l->first_bias_connection_index + dir * (q->C + 3 * q->K);
                 q->reverse = (int)dir;
+                q->zone_stride = q->C * dirs;
+                q->zone_state = n->zoneout + zone_at + dir * q->C;
+                q->zone_output = q->zone_state + T * total_cells;
                 size_t sc = T * B * q->C, sk = T * B * q->K;
                 float **cells[] = {&q->sum_in_z, &q->sum_rec_z, &q->sum_z, &q->z, &q->c, &q->ca, &q->dz, &q->dc};
                 float **blocks[] = {&q->sum_in_i, &q->sum_in_f, &q->sum_in_o, &q->sum_rec_i, &q->sum_rec_f, &q->sum_rec_o, &q->sum_i, &q->sum_f, &q->sum_o,
@@ -308,6 +321,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
                 else { q->h = o->values; q->dh = o->af_errors; }
             }
             o->lstm = qq;
+            zone_at += T * qq[0].zone_stride;
             continue;
         }
         o->af_errors = zalloc(T * B * o->AH);
@@ -344,7 +358,7 @@ int myea_oracle_destroy(myea_oracle_net *n)
     if (!n) return MYEA_OK;
     free(n->parameters); free(n->gradient);
     for (int k = 0; k < MYEA_STATE_KINDS; ++k) free(n->opt[k]);
-    free(n->masks);
+    free(n->masks); free(n->zoneout);
     for (size_t li = 0; li < n->d.n_layers; ++li) {
         olayer *o = &n->L[li];
         free(o->summations); free(o->values); free(o->hats); free(o->normalizes);
@@ -390,6 +404,7 @@ int myea_oracle_set_threads(myea_oracle_net *n, int t) { if (!n || t < 1) return
 float *myea_oracle_parameters(myea_oracle_net *n) { return n->parameters; }
 float *myea_oracle_gradient(myea_oracle_net *n) { return n->gradient; }
 float *myea_oracle_optimizer_state(myea_oracle_net *n, int k) { return (k >= 0 && k < MYEA_STATE_KINDS) ? n->opt[k] : NULL; }
+uint8_t *myea_oracle_zoneout_masks(myea_oracle_net *n, size_t *count) { if (count) *count = n->zoneout_count; return n->zoneout; }
 uint8_t *myea_oracle_masks(myea_oracle_net *n) { return n->masks; }
 
 /* Clear_Optimizer NN/Train.cpp:128-263: state vectors to zero (iRPROP steps to rprop_delta_zero, its two losses to the
@@ -656,6 +671,8 @@ static void fwd_lstm_step(myea_oracle_net *n, size_t li, int dir, size_t t, size
      * (tmp_time_step_reverse_direction, NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:456-461) */
     size_t tp = q->reverse ? t + 1 : t - 1;
     int first = q->reverse ? t == n->d.number_recurrent_depth - 1 : t == 0;
+    /* strictly in the training state (NN/Neural_Network__Forward_Pass__Loop.cpp:2088-2092) */
+    int zone = l->type_dropout == MYEA_DROPOUT_ZONEOUT && n->state == MYEA_STATE_TRAINING;
     long b;
 #pragma omp parallel for schedule(static) num_threads(n->threads)
     for (b = 0; b < (long)B; ++b) {
@@ -702,6 +719,8 @@ static void fwd_lstm_step(myea_oracle_net *n, size_t li, int dir, size_t t, size
                 q->sum_z[cb + c] = sz;
                 q->z[cb + c] = tanh_f(sz);
                 q->c[cb + c] = first ? q->z[cb + c] * q->gi[kb + k] : q->z[cb + c] * q->gi[kb + k] + q->gf[kb + k] * q->c[cp + c];
+                /* zoneout of the cell state (Forward_Pass__LSTM__Gates_CIF_AF_State__Zoneout, :1285-1288, :1331-1334) */
+                if (zone && !q->zone_state[t * q->zone_stride + c]) q->c[cb + c] = first ? 0.f : q->c[cp + c];
             }
         }
         /* States_AF */
@@ -713,7 +732,12 @@ static void fwd_lstm_step(myea_oracle_net *n, size_t li, int dir, size_t t, size
             for (size_t j = 0; j < cpb; ++j) so += q->c[cb + k * cpb + j] * po[j];
             q->sum_o[kb + k] = so;
             q->go[kb + k] = sigmoid_f(so);
-            for (size_t j = 0; j < cpb; ++j) q->h[cb + k * cpb + j] = q->ca[cb + k * cpb + j] * q->go[kb + k];
+            for (size_t j = 0; j < cpb; ++j) {
+                size_t c = k * cpb + j;
+                q->h[cb + c] = q->ca[cb + c] * q->go[kb + k];
+                /* zoneout of the cell output (Forward_Pass__LSTM__Output__Zoneout, :1475-1478, :1520-1523) */
+                if (zone && !q->zone_output[t * q->zone_stride + c]) q->h[cb + c] = first ? 0.f : q->h[cp + c];
+            }
         }
     }
 }

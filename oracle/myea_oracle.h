@@ -31,6 +31,7 @@ float *myea_oracle_parameters(myea_oracle_net *net);
 float *myea_oracle_gradient(myea_oracle_net *net);
 float *myea_oracle_optimizer_state(myea_oracle_net *net, int kind);
 uint8_t *myea_oracle_masks(myea_oracle_net *net);
+uint8_t *myea_oracle_zoneout_masks(myea_oracle_net *net, size_t *count);
 int myea_oracle_clear_training_arrays(myea_oracle_net *net);
 
 int myea_oracle_forward_pass(myea_oracle_net *net, size_t batch_size_received, const float *inputs);

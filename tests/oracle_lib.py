@@ -37,6 +37,8 @@ def load_oracle():
     lib.myea_oracle_optimizer_state.restype = P(C.c_float)
     lib.myea_oracle_masks.argtypes = [vp]
     lib.myea_oracle_masks.restype = P(C.c_uint8)
+    lib.myea_oracle_zoneout_masks.argtypes = [vp, P(sz)]
+    lib.myea_oracle_zoneout_masks.restype = P(C.c_uint8)
     lib.myea_oracle_clear_training_arrays.argtypes = [vp]
     lib.myea_oracle_forward_pass.argtypes = [vp, sz, vp]
     lib.myea_oracle_compute_error.argtypes = [vp, sz, vp]
@@ -128,6 +130,13 @@ class OracleNetwork:
     def upload_masks(self, m):
         m = np.asarray(m, dtype=np.uint8)
         self._view(self.lib.myea_oracle_masks(self.handle), self.desc.total_mask_units, np.uint8)[: len(m)] = m
+
+    def upload_zoneout_masks(self, m):
+        m = np.asarray(m, dtype=np.uint8)
+        n = C.c_size_t()
+        p = self.lib.myea_oracle_zoneout_masks(self.handle, C.byref(n))
+        assert len(m) == n.value, "zoneout mask count %d != %d" % (len(m), n.value)
+        self._view(p, n.value, np.uint8)[:] = m
 
     def download_tensor(self, layer, kind, count=None):
         n = C.c_size_t()

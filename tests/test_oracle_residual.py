@@ -2,6 +2,8 @@
 shortcut) without the reference build: the descriptor layout against hand-counted offsets, the forward/backward
 against automatic differentiation of an independent float64 model, and a block that computes zero against the same
 stack without the block.  CPU only."""
+import zlib
+
 import numpy as np
 import pytest
 import torch
@@ -227,7 +229,7 @@ CASES = {
 def test_residual_forward_and_gradients_match_float64_autograd(name):
     specs, B = CASES[name]
     desc = oracle_desc(specs, B)
-    rng = np.random.default_rng(abs(hash(name)) % 1000)
+    rng = np.random.default_rng(zlib.crc32(name.encode()) % 1000)   # str hashes change from process to process
     w = glorot_parameters(desc, 11, bias_range=0.3)
     X = rng.normal(0, 1, (B, specs[0]["units"])).astype(np.float32)
     n_out = specs[-1]["units"]
@@ -249,7 +251,8 @@ def test_residual_forward_and_gradients_match_float64_autograd(name):
         got_v = net.download_tensor(key, mb.TENSOR["OUTPUTS"]).reshape(B, width)
         assert_close(got_v, t.detach().numpy(), 3e-5, 3e-6, "values of layer %d" % key)
         got_e = net.download_tensor(key, mb.TENSOR[kind]).reshape(B, width)
-        assert_close(got_e, t.grad.numpy(), 3e-4, 3e-6, "delta of layer %d" % key)
+        # fp32 against float64: entries that are small differences of O(1) terms carry the terms' rounding
+        assert_close(got_e, t.grad.numpy(), 3e-4, 1e-5, "delta of layer %d" % key)
     assert_close(net.download_gradient(), model.flat.grad.numpy(), 3e-4, 3e-5, "gradient")
 
 
