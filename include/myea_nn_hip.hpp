@@ -128,6 +128,7 @@ public:
         if (value_dropout == nullptr || value_dropout[0] < 0.f || value_dropout[0] > 1.f) return Fail("Set__Dropout", "retention probability out of [0, 1]");
         desc_.layers[index_layer].type_dropout = type_layer_dropout;
         desc_.layers[index_layer].dropout_values[0] = value_dropout[0];
+        if (type_layer_dropout == MYEA_DROPOUT_ZONEOUT) desc_.layers[index_layer].dropout_values[1] = value_dropout[1];   // cell-output probability
         return Dirty();
     }
     void Set__Loss_Function(unsigned int f) { type_loss_function = f; }
@@ -169,6 +170,15 @@ public:
     bool Copy__Optimizer__Device_To_Host(int kind, T_ *dst) { return Need("Copy__Optimizer__Device_To_Host") && Ok("Copy__Optimizer__Device_To_Host", myea_hip_download_optimizer_state(net_, kind, dst, total_parameters)); }
     bool Copy__Optimizer__Host_To_Device(int kind, T_ const *src) { return Need("Copy__Optimizer__Host_To_Device") && Ok("Copy__Optimizer__Host_To_Device", myea_hip_upload_optimizer_state(net_, kind, src, total_parameters)); }
     bool Copy__Derivatives_Parameters__Device_To_Host(T_ *dst) { return Need("Copy__Derivatives_Parameters__Device_To_Host") && Ok("Copy__Derivatives_Parameters__Device_To_Host", myea_hip_download_gradient(net_, dst, total_parameters)); }
+    // zoneout masks as the caller's Dropout_Zoneout() leaves them in ptr_array_cell_units_mask_dropout_zoneout:
+    // [state | output] halves, per LSTM layer [T][cells] (Neural_Network.cpp:3964-3995); `count` = 2 x T x total cells
+    bool Copy__Zoneout_Mask__Host_To_Device(bool const *ptr_array_cell_units_mask_dropout_zoneout, size_t count)
+    {
+        if (!Need("Copy__Zoneout_Mask__Host_To_Device")) return false;
+        std::vector<uint8_t> bytes(count);
+        for (size_t i = 0; i < count; ++i) bytes[i] = ptr_array_cell_units_mask_dropout_zoneout[i] ? 1 : 0;
+        return Ok("Copy__Zoneout_Mask__Host_To_Device", myea_hip_upload_zoneout_masks(net_, bytes.data(), bytes.size()));
+    }
     bool Copy__Dropout_Mask__Host_To_Device()
     {
         if (!Need("Copy__Dropout_Mask__Host_To_Device")) return false;
