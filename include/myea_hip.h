@@ -38,6 +38,7 @@ extern "C" {
 enum {
     MYEA_LAYER_NONE = 0,
     MYEA_LAYER_FULLY_CONNECTED = 4,
+    MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT = 5,  /* h[t] = AF(W x[t] + b + u * h[t-1]), one self weight per unit */
     MYEA_LAYER_AVERAGE_POOLING = 1,
     MYEA_LAYER_LSTM = 8,
     MYEA_LAYER_MAX_POOLING = 9,
@@ -128,6 +129,12 @@ typedef struct myea_layer_desc {
      * stride, padding, dilation, ceil mode.  n_units of a pooling layer is an OUTPUT of myea_net_desc_layout
      * (Assign__Post__Layer :250-271). */
     uint32_t pooling_values[5];
+    /* independently recurrent layers only: the clip applied to the self weights after every update, no clip when both
+     * are 0 (Layer::constraint_recurrent_weight_{lower,upper}_bound,
+     * NN/Neural_Network__Regularization__Constraint_Recurrent_Weight.cpp:317-333; Compile gives the layer the bounds of
+     * Compute__Regularization__Constraint_Recurrent_Weight__Default, :33-75) */
+    float    constraint_recurrent_weight_lower_bound;
+    float    constraint_recurrent_weight_upper_bound;
     /* index table (into the flat parameter / gradient / optimizer vectors, and the mask buffer) */
     uint64_t first_connection_index;       /* *Layer::ptr_first_connection_index */
     uint64_t last_connection_index;        /* *Layer::ptr_last_connection_index */

@@ -90,8 +90,13 @@ public:
                 for (int k = 0; k < 5; ++k) l.pooling_values[k] = (uint32_t)ptr_array_layers[i].unit_parameters[k];
                 l.n_units = 0;
             }
-            // Compile's defaults: FC layers start as sigmoid with steepness 1 (Neural_Network__Compile.cpp:572-590)
+            // Compile's defaults: FC layers start as sigmoid with steepness 1 (Neural_Network__Compile.cpp:572-590),
+            // independently recurrent layers as rectifiers with the default clip of their self weights (:593-627)
             l.type_activation_function = (i > 0 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) ? MYEA_AF_SIGMOID : MYEA_AF_NONE;
+            if (l.type_layer == MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT) {
+                l.type_activation_function = MYEA_AF_RELU;
+                Compute__Regularization__Constraint_Recurrent_Weight__Default(i, &l.constraint_recurrent_weight_lower_bound, &l.constraint_recurrent_weight_upper_bound);
+            }
             l.activation_steepness = 1.f;
             l.use_layer_normalization_before_activation = 1;
             l.dropout_values[0] = 1.f;
@@ -103,8 +108,53 @@ public:
     {
         if (!CheckLayer("Set__Layer_Activation_Function", index_layer)) return false;
         if (type_activation_function == MYEA_AF_NONE || type_activation_function >= MYEA_AF_LENGTH) return Fail("Set__Layer_Activation_Function", "activation function out of range");
+        // a layer still on the default clip of its self weights follows the new activation's default (Train.cpp:538-640)
+        const bool follows = Check__Use__Regularization__Constraint_Recurrent_Weight__Default(index_layer);
         desc_.layers[index_layer].type_activation_function = type_activation_function;
+        if (follows) Set__Regularization__Constraint_Recurrent_Weight__Default(index_layer);
         return Dirty();
+    }
+    // Compute__Regularization__Constraint_Recurrent_Weight__Default
+    // (Neural_Network__Regularization__Constraint_Recurrent_Weight.cpp:33-75): +-MAG^(1/T) with MAG = clip_gradient kept in
+    // [2, 10]; for the symmetric activations MAG is first divided by 0.9^(T/10)
+    void Compute__Regularization__Constraint_Recurrent_Weight__Default(size_t index_layer, T_ *lower_bound, T_ *upper_bound) const
+    {
+        const T_ MAG = clip_gradient < 2.f ? 2.f : (clip_gradient > 10.f ? 10.f : clip_gradient), T = (T_)number_recurrent_depth;
+        T_ bound;
+        switch (desc_.layers[index_layer].type_activation_function) {
+        case MYEA_AF_COSINE_SYMMETRIC: case MYEA_AF_ELLIOT_SYMMETRIC: case MYEA_AF_GAUSSIAN_SYMMETRIC: case MYEA_AF_LINEAR_PIECE_SYMMETRIC:
+        case MYEA_AF_SINE_SYMMETRIC: case MYEA_AF_TANH: case MYEA_AF_TANH_STEPWISE: case MYEA_AF_THRESHOLD_SYMMETRIC:
+            bound = std::pow(MAG / std::pow(0.9f, T / 10.f), 1.f / T);
+            break;
+        default: bound = std::pow(MAG, 1.f / T); break;
+        }
+        *lower_bound = -bound; *upper_bound = bound;
+    }
+    bool Check__Use__Regularization__Constraint_Recurrent_Weight__Default(size_t index_layer) const
+    {
+        if (index_layer >= desc_.n_layers || desc_.layers[index_layer].type_layer != MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT) return false;
+        T_ lo, hi;
+        Compute__Regularization__Constraint_Recurrent_Weight__Default(index_layer, &lo, &hi);
+        const myea_layer_desc &l = desc_.layers[index_layer];
+        return std::fabs(l.constraint_recurrent_weight_lower_bound - lo) <= 1e-8 && std::fabs(l.constraint_recurrent_weight_upper_bound - hi) <= 1e-8;
+    }
+    // Set__Regularization__Constraint_Recurrent_Weight (:143-229): recurrent hidden layers only, lower <= upper
+    bool Set__Regularization__Constraint_Recurrent_Weight(size_t index_layer, T_ lower_bound, T_ upper_bound)
+    {
+        if (!CheckLayer("Set__Regularization__Constraint_Recurrent_Weight", index_layer)) return false;
+        if (index_layer + 1 == desc_.n_layers) return Fail("Set__Regularization__Constraint_Recurrent_Weight", "layer received as argument is the output layer");
+        if (desc_.layers[index_layer].type_layer != MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT) return Fail("Set__Regularization__Constraint_Recurrent_Weight", "can not constrain the recurrent weight of this type of layer");
+        if (lower_bound > upper_bound) return Fail("Set__Regularization__Constraint_Recurrent_Weight", "lower bound greater than upper bound");
+        desc_.layers[index_layer].constraint_recurrent_weight_lower_bound = lower_bound;
+        desc_.layers[index_layer].constraint_recurrent_weight_upper_bound = upper_bound;
+        return Dirty();
+    }
+    bool Set__Regularization__Constraint_Recurrent_Weight__Default(size_t index_layer)
+    {
+        if (!CheckLayer("Set__Regularization__Constraint_Recurrent_Weight__Default", index_layer)) return false;
+        T_ lo, hi;
+        Compute__Regularization__Constraint_Recurrent_Weight__Default(index_layer, &lo, &hi);
+        return Set__Regularization__Constraint_Recurrent_Weight(index_layer, lo, hi);
     }
     bool Set__Layer_Activation_Steepness(size_t index_layer, T_ activation_steepness)
     {
@@ -135,7 +185,16 @@ public:
     void Set__Accuracy_Function(unsigned int f) { type_accuracy_function = f; }
     void Set__Optimizer_Function(unsigned int f) { type_optimizer_function = f; }
     void Set__Clip_Gradient(bool use) { use_clip_gradient = use; }
-    bool Set__Clip_Gradient(T_ value) { clip_gradient = value; return true; }
+    // Set__Clip_Gradient (Neural_Network__Clip_Gradient.cpp:20-80): layers on the default clip of their self weights follow
+    bool Set__Clip_Gradient(T_ value)
+    {
+        bool follows[MYEA_MAX_LAYERS];
+        for (size_t i = 0; i < desc_.n_layers; ++i) follows[i] = Check__Use__Regularization__Constraint_Recurrent_Weight__Default(i);
+        clip_gradient = value;
+        for (size_t i = 0; i < desc_.n_layers; ++i)
+            if (follows[i] && !Set__Regularization__Constraint_Recurrent_Weight__Default(i)) return false;
+        return true;
+    }
     bool Set__Accurancy_Variance(T_ v) { accuracy_variance = v; return true; }
     bool Set__Number_Time_Delays(size_t n) { if (n > number_recurrent_depth) return Fail("Set__Number_Time_Delays", "time delays exceed the recurrent depth"); number_time_delays = n; return true; }
     bool Set__Normalization_Momentum_Average(T_ v) { normalization_momentum_average = v; return true; }

@@ -17,6 +17,7 @@ MAX_LAYERS = 64
 # ---- enum values (Common_Library/include/Enums of the reference) ----
 LAYER_FULLY_CONNECTED, LAYER_LSTM, LAYER_RESIDUAL = 4, 8, 10
 LAYER_AVERAGE_POOLING, LAYER_MAX_POOLING = 1, 9
+LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT = 5
 NETWORK_FEEDFORWARD, NETWORK_RECURRENT = 3, 4
 AF = dict(NONE=0, COSINE=1, COSINE_SYMMETRIC=2, ELU=3, ELLIOT=4, ELLIOT_SYMMETRIC=5, GAUSSIAN=6,
           GAUSSIAN_STEPWISE=7, GAUSSIAN_SYMMETRIC=8, ISRU=9, ISRLU=10, LINEAR=11, LINEAR_PIECE=12,
@@ -46,6 +47,7 @@ class LayerDesc(C.Structure):
         ("activation_steepness", C.c_float), ("type_dropout", C.c_uint32), ("dropout_values", C.c_float * 2),
         ("type_normalization", C.c_uint32), ("use_layer_normalization_before_activation", C.c_uint32),
         ("block_depth", C.c_uint32), ("pooling_values", C.c_uint32 * 5),
+        ("constraint_recurrent_weight_lower_bound", C.c_float), ("constraint_recurrent_weight_upper_bound", C.c_float),
         ("first_connection_index", C.c_uint64), ("last_connection_index", C.c_uint64),
         ("first_bias_connection_index", C.c_uint64), ("first_normalized_unit_index", C.c_uint64),
         ("first_mask_index", C.c_uint64),
@@ -174,9 +176,29 @@ def default_hyper(lib=None, **overrides):
     return h
 
 
+# Activation_Function__To__Class_Activation_Function (NN/Train.cpp:453-500): the functions of the symmetric class
+_SYMMETRIC_AF = ("COSINE_SYMMETRIC", "ELLIOT_SYMMETRIC", "GAUSSIAN_SYMMETRIC", "LINEAR_PIECE_SYMMETRIC", "SINE_SYMMETRIC",
+                 "TANH", "TANH_STEPWISE", "THRESHOLD_SYMMETRIC")
+
+
+def constraint_recurrent_weight_default(activation, recurrent_depth, clip_gradient=1.0):
+    """Compute__Regularization__Constraint_Recurrent_Weight__Default
+    (NN/Neural_Network__Regularization__Constraint_Recurrent_Weight.cpp:33-75): the bounds Compile gives an
+    independently recurrent layer, in the reference's float arithmetic."""
+    f = np.float32
+    mag = f(min(max(f(clip_gradient), f(2)), f(10)))
+    T = f(recurrent_depth)
+    if activation in _SYMMETRIC_AF:
+        hi = np.power(f(mag / np.power(f(0.9), f(T / f(10)), dtype=f)), f(f(1) / T), dtype=f)
+    else:
+        hi = np.power(mag, f(f(1) / T), dtype=f)
+    return float(-hi), float(hi)
+
+
 def make_desc(layers, batch_size, recurrent_depth=1, network=None, lib=None):
-    """layers: list of dicts (first = input layer).  Keys: units, type ('fc'|'lstm'), cells_per_block,
-    bidirectional, activation (name), steepness, dropout (name), keep, normalization (name), norm_before."""
+    """layers: list of dicts (first = input layer).  Keys: units, type ('fc'|'ind_rnn'|'lstm'|...), cells_per_block,
+    bidirectional, activation (name), steepness, dropout (name), keep, normalization (name), norm_before,
+    recurrent_bounds ((lower, upper) clip of an ind_rnn layer's self weights; default: the reference's)."""
     lib = lib or load_library()
     d = NetDesc()
     d.n_layers = len(layers)
@@ -186,7 +208,7 @@ def make_desc(layers, batch_size, recurrent_depth=1, network=None, lib=None):
     for i, spec in enumerate(layers):
         l = d.layers[i]
         kind = spec.get("type", "fc")
-        l.type_layer = {"fc": LAYER_FULLY_CONNECTED, "lstm": LAYER_LSTM, "residual": LAYER_RESIDUAL,
+        l.type_layer = {"fc": LAYER_FULLY_CONNECTED, "ind_rnn": LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT, "lstm": LAYER_LSTM, "residual": LAYER_RESIDUAL,
                         "average_pooling": LAYER_AVERAGE_POOLING, "max_pooling": LAYER_MAX_POOLING}[kind]
         if kind.endswith("pooling"):   # units is computed by the layout
             for k, name in enumerate(("kernel", "stride", "padding", "dilation", "ceil_mode")):
@@ -194,7 +216,10 @@ def make_desc(layers, batch_size, recurrent_depth=1, network=None, lib=None):
         l.n_units = spec.get("units", 0)
         l.n_cells_per_block = spec.get("cells_per_block", 1 if kind == "lstm" else 0)
         l.use_bidirectional = int(spec.get("bidirectional", False))
-        l.type_activation_function = AF[spec.get("activation", "SIGMOID")] if (kind == "fc" and i > 0) else 0
+        l.type_activation_function = AF[spec.get("activation", "SIGMOID")] if (kind in ("fc", "ind_rnn") and i > 0) else 0
+        if kind == "ind_rnn":
+            lo, hi = spec.get("recurrent_bounds") or constraint_recurrent_weight_default(spec.get("activation", "SIGMOID"), recurrent_depth)
+            l.constraint_recurrent_weight_lower_bound, l.constraint_recurrent_weight_upper_bound = lo, hi
         l.activation_steepness = spec.get("steepness", 1.0)
         l.type_dropout = DROPOUT[spec.get("dropout", "NONE")]
         l.dropout_values[0] = spec.get("keep", 1.0)

@@ -51,6 +51,76 @@ __global__ __launch_bounds__(kBlock) void activation_derive_kernel(int act, floa
         dx[i] = dy[i] * af_derive(unit_act ? unit_act[i % H] : act, pre[i], unit_steep ? unit_steep[i % H] : steep, val[i]);
 }
 
+// Independently recurrent layer, the whole sequence in one launch: a thread owns one (example, unit) pair and walks the
+// time steps with the previous activation in a register, so the T dependent steps cost one pass over the tensors.
+// Forward_Pass__FC_Ind_RNN (NN/Neural_Network__Recurrent_Forward_Pass__Loop.cpp:813-866): pre_AF[t] = input[t] + u * AF[t-1]
+// (a copy at t = 0), then Forward_Pass__FC_AF and, for an un-normalised layer, the Bernoulli applier in place on AF - the
+// value the next time step reads.
+__global__ __launch_bounds__(kBlock) void ind_rnn_forward_kernel(IndRnnParams p)
+{
+    const size_t n = p.B * p.H, step = p.Bmax * p.H;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t j = i % p.H;
+        const float u = p.u[j];
+        const int act = p.unit_act ? p.unit_act[j] : p.act;
+        float h = 0.f;
+        size_t k = i;
+#pragma unroll 4
+        for (size_t t = 0; t < p.T; ++t, k += step) {
+            float pre = p.in[k];
+            if (t) pre = __fadd_rn(pre, __fmul_rn(u, h));
+            p.pre_afs[k] = pre;
+            h = af_fire(act, pre);
+            if (p.colscale) h *= p.colscale[t * p.H + j];
+            p.afs[k] = h;
+        }
+    }
+}
+
+// Backward_Pass__FC__DF_Ind_RNN (NN/Neural_Network__Backward_Pass__Loop.cpp:1296-1390), time steps from the last to the
+// first: errors = dY AF'(t); dAF(t) = errors + u AF'(t) dAF(t+1), without the second term at the last step.
+__global__ __launch_bounds__(kBlock) void ind_rnn_backward_kernel(IndRnnParams p)
+{
+    const size_t n = p.B * p.H, step = p.Bmax * p.H;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t j = i % p.H;
+        const float u = p.u[j], steep = p.unit_steep ? p.unit_steep[j] : p.steep;
+        const int act = p.unit_act ? p.unit_act[j] : p.act;
+        float next = 0.f;
+        size_t k = i + (p.T - 1) * step;
+#pragma unroll 4
+        for (size_t t = p.T; t-- > 0; k -= step) {
+            const float daf = af_derive(act, p.pre_afs[k], steep, p.afs[k]);
+            const float e = __fmul_rn(p.dy[k], daf);
+            const float r = (t + 1 == p.T) ? e : __fadd_rn(e, __fmul_rn(__fmul_rn(u, daf), next));
+            p.dafs[k] = r;
+            next = r;
+            if (t == 0) break;
+        }
+    }
+}
+
+// Update_Derivative_Weight__FC_Ind_RNN (NN/Neural_Network__Recurrent_Update_Derivative_Weight__Loop.cpp:461-483) summed over
+// the time steps 1 .. T-1: du[j] += sum_{t, b} AF[t-1][b][j] dAF[t][b][j].  Row r of the reduction is (t = r / B, b = r % B).
+struct IndRnnDotF {
+    const float *afs, *dafs; size_t H, B, Bmax;
+    __device__ void operator()(size_t r, size_t col, double *acc) const
+    {
+        const size_t t = r / B, b = r % B;
+        acc[0] += (double)afs[(t * Bmax + b) * H + col] * (double)dafs[((t + 1) * Bmax + b) * H + col];
+    }
+};
+
+// Update_Weight_Regularization__Constraint_Recurrent_Weight__FC_Ind_RNN
+// (NN/Neural_Network__Regularization__Constraint_Recurrent_Weight.cpp:317-333)
+__global__ __launch_bounds__(kBlock) void clip_range_kernel(size_t n, float *w, float lo, float hi)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const float v = w[i];
+        w[i] = v < lo ? lo : (v > hi ? hi : v);
+    }
+}
+
 // Forward_Pass__FC_AF__Softmax (:4870-4905): one wavefront per row.
 __global__ __launch_bounds__(kBlock) void softmax_kernel(size_t rows, size_t H, const float *x, float *y, const float *colscale)
 {
@@ -616,6 +686,45 @@ int launch_column_sum(hipStream_t s, size_t rows, size_t H, const float *x, floa
     hipLaunchKernelGGL((column_partial_kernel<1, SumF>), dim3((unsigned)((H + 63) / 64), (unsigned)S), dim3(kBlock), 0, s, rows, H, chunk, scratch, f);
     MYEA_HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, kBlock)), dim3(kBlock), 0, s, H, S, scratch, out, accumulate);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_ind_rnn_forward(hipStream_t s, const IndRnnParams &p)
+{
+    if (p.B * p.H == 0 || p.T == 0) return MYEA_OK;
+    hipLaunchKernelGGL(ind_rnn_forward_kernel, dim3(grid_for(p.B * p.H, kBlock)), dim3(kBlock), 0, s, p);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_ind_rnn_backward(hipStream_t s, const IndRnnParams &p)
+{
+    if (p.B * p.H == 0 || p.T == 0) return MYEA_OK;
+    hipLaunchKernelGGL(ind_rnn_backward_kernel, dim3(grid_for(p.B * p.H, kBlock)), dim3(kBlock), 0, s, p);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+// scratch: 64 * H floats at most
+int launch_ind_rnn_self_weight_gradient(hipStream_t s, size_t T, size_t B, size_t Bmax, size_t H, const float *afs, const float *dafs, float *du, float *scratch)
+{
+    if (H == 0 || B == 0 || T < 2) return MYEA_OK;
+    const size_t rows = (T - 1) * B;
+    size_t S, chunk;
+    split_rows(rows, H, S, chunk);
+    IndRnnDotF f{afs, dafs, H, B, Bmax};
+    hipLaunchKernelGGL((column_partial_kernel<1, IndRnnDotF>), dim3((unsigned)((H + 63) / 64), (unsigned)S), dim3(kBlock), 0, s, rows, H, chunk, scratch, f);
+    MYEA_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, kBlock)), dim3(kBlock), 0, s, H, S, scratch, du, 1);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_clip_range(hipStream_t s, size_t n, float *w, float lo, float hi)
+{
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(clip_range_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, n, w, lo, hi);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

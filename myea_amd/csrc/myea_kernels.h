@@ -124,6 +124,25 @@ int launch_compute_error(hipStream_t s, const ErrorParams &p);
 int launch_accuracy_r(hipStream_t s, const ErrorParams &p, float desired_mean, float predicted_mean);
 int launch_gather_rows(hipStream_t s, size_t B, size_t row_floats, const unsigned long long *index, const float *src, float *dst);
 
+// Independently recurrent layer over the whole sequence: tensors are [T][Bmax][H], the first B rows of a time step in use.
+struct IndRnnParams {
+    size_t T, B, Bmax, H;
+    const float *u;            // self weights [H]
+    int act; float steep;      // layer-wide activation / steepness
+    const int *unit_act;       // optional per-unit activation types [H]
+    const float *unit_steep;   // optional per-unit steepnesses [H]
+    const float *in;           // forward: summations or their normalisation
+    float *pre_afs, *afs;      // forward: written; backward: read
+    const float *colscale;     // forward: optional dropout multiplier [T][H] applied in place on the activations
+    const float *dy;           // backward: delta of the layer's activations
+    float *dafs;               // backward: delta of the pre-activations (the recurrence runs through it)
+};
+int launch_ind_rnn_forward(hipStream_t s, const IndRnnParams &p);
+int launch_ind_rnn_backward(hipStream_t s, const IndRnnParams &p);
+// du[j] += sum over t >= 1 and the batch of AF[t-1] dAF[t]; scratch: 64 * H floats
+int launch_ind_rnn_self_weight_gradient(hipStream_t s, size_t T, size_t B, size_t Bmax, size_t H, const float *afs, const float *dafs, float *du, float *scratch);
+int launch_clip_range(hipStream_t s, size_t n, float *w, float lo, float hi);
+
 // [B][T][W] (example rows) -> [T][Bmax][W]
 int launch_scatter_time_major(hipStream_t s, size_t B, size_t T, size_t W, size_t Bmax, const float *src, float *dst);
 

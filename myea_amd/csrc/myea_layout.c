@@ -104,6 +104,9 @@ uint64_t myea_net_desc_number_outputs(const myea_net_desc *d, uint32_t li)
 #define previous_layer myea_net_desc_previous_layer
 
 static int is_pooling(const myea_layer_desc *l) { return l->type_layer == MYEA_LAYER_AVERAGE_POOLING || l->type_layer == MYEA_LAYER_MAX_POOLING; }
+static int is_ind_rnn(const myea_layer_desc *l) { return l->type_layer == MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT; }
+/* neuron units + activation units: fully-connected and independently recurrent layers */
+static int is_dense(const myea_layer_desc *l) { return l->type_layer == MYEA_LAYER_FULLY_CONNECTED || is_ind_rnn(l); }
 
 int myea_net_desc_layout(myea_net_desc *d)
 {
@@ -117,8 +120,8 @@ int myea_net_desc_layout(myea_net_desc *d)
         const int pooling = is_pooling(l);
         if (l->n_units == 0 && l->type_layer != MYEA_LAYER_RESIDUAL && !pooling) return MYEA_E_INVALID;
         if (l->type_layer == MYEA_LAYER_LSTM && l->n_cells_per_block == 0) return MYEA_E_INVALID;
-        if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED && l->type_layer != MYEA_LAYER_LSTM &&
-            l->type_layer != MYEA_LAYER_RESIDUAL && !pooling) return MYEA_E_UNSUPPORTED;
+        if (!is_dense(l) && l->type_layer != MYEA_LAYER_LSTM && l->type_layer != MYEA_LAYER_RESIDUAL && !pooling) return MYEA_E_UNSUPPORTED;
+        if (is_ind_rnn(l) && (li == 0 || li + 1 == d->n_layers)) return MYEA_E_INVALID;
         if (pooling && (l->pooling_values[0] == 0 || l->pooling_values[1] == 0 || li == 0 || li + 1 == d->n_layers)) return MYEA_E_INVALID;
         if (l->type_normalization != MYEA_NORMALIZATION_NONE) any_norm = 1;
     }
@@ -149,14 +152,15 @@ int myea_net_desc_layout(myea_net_desc *d)
         li += l->block_depth;
     }
 
-    /* weights: Prepare__Connections__FC / __LSTM, NN/Neural_Network__Prepare_Connections.cpp:20-222 */
+    /* weights: Prepare__Connections__FC / __FC_Ind_RNN / __LSTM, NN/Neural_Network__Prepare_Connections.cpp:20-222.
+     * An independently recurrent layer's self weights (one per unit) follow its [units][fan-in] matrix (:45-77). */
     for (uint32_t li = 1; li < d->n_layers; ++li) {
         myea_layer_desc *l = &d->layers[li];
         if (l->type_layer == MYEA_LAYER_RESIDUAL || is_pooling(l)) { l->first_connection_index = l->last_connection_index = total_weights; continue; }
         uint64_t fan_in = number_outputs(d, previous_layer(d, li));
         l->first_connection_index = total_weights;
-        if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
-            total_weights += fan_in * l->n_units;
+        if (is_dense(l)) {
+            total_weights += fan_in * l->n_units + (is_ind_rnn(l) ? l->n_units : 0u);
         } else { /* LSTM */
             uint64_t dirs = l->use_bidirectional ? 2u : 1u;
             uint64_t cpb = l->n_cells_per_block, cells_per_layer = (uint64_t)l->n_units * cpb;
@@ -171,7 +175,7 @@ int myea_net_desc_layout(myea_net_desc *d)
     for (uint32_t li = 1; li < d->n_layers; ++li) {
         myea_layer_desc *l = &d->layers[li];
         if (l->type_layer == MYEA_LAYER_RESIDUAL || is_pooling(l)) { l->first_bias_connection_index = total_weights + total_bias; continue; }
-        if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (is_dense(l)) {
             l->first_bias_connection_index = total_weights + total_bias;
             total_bias += l->n_units;
         } else {
@@ -216,7 +220,7 @@ int myea_net_desc_layout(myea_net_desc *d)
     for (uint32_t li = 0; li < d->n_layers; ++li) {
         myea_layer_desc *l = &d->layers[li];
         l->first_mask_index = total_mask;
-        if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED) continue;
+        if (!is_dense(l)) continue;   /* AF_unit and AF_Ind_recurrent_unit alike, :3959-3960 */
         uint32_t r = li ? enclosing_block(d, li) : 0;
         /* inside a block the activation units sit on the layer's input side: none for the block's first layer, fan-in
          * many for the others (Assign__Post__Residual_Layer, NN/Neural_Network__Compile.cpp:378-384) */

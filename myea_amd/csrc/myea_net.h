@@ -30,6 +30,9 @@ struct DevLayer {
     float *r_corrections = nullptr, *d_corrections = nullptr;
     float *colscale = nullptr;  // dropout multiplier per (t, unit)
     unsigned *pool_index = nullptr;  // max pooling: padded position each output took its value from [T][Bmax][H]
+    // independently recurrent layer: pre-activations [T][Bmax][H]; the delta of the pre-activations lives in neuron_errors
+    // unless a normalisation sits between the summation and the activation (then in dafs_own)
+    float *pre_afs = nullptr, *dafs_own = nullptr;
     int *unit_act = nullptr;    // per-unit activation types [AH], null = layer-wide
     float *unit_steep = nullptr;  // per-unit steepnesses [AH], null = layer-wide
     LstmLayer *lstm = nullptr, *lstm2 = nullptr;  // lstm2: the time-reversed direction of a bidirectional layer
@@ -43,6 +46,8 @@ struct ProfEvent {
 };
 
 bool layer_is_pooling(const myea_layer_desc &l);
+bool layer_is_ind_rnn(const myea_layer_desc &l);
+bool layer_is_dense(const myea_layer_desc &l);
 bool layer_uses_norm(const myea_layer_desc &l);
 bool layer_uses_bias(const myea_layer_desc &l);
 

@@ -52,6 +52,9 @@ static int dev_alloc(float **p, size_t count)
     } while (0)
 
 bool layer_is_pooling(const myea_layer_desc &l) { return l.type_layer == MYEA_LAYER_AVERAGE_POOLING || l.type_layer == MYEA_LAYER_MAX_POOLING; }
+bool layer_is_ind_rnn(const myea_layer_desc &l) { return l.type_layer == MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT; }
+// layers made of neuron units and activation units
+bool layer_is_dense(const myea_layer_desc &l) { return l.type_layer == MYEA_LAYER_FULLY_CONNECTED || layer_is_ind_rnn(l); }
 bool layer_uses_norm(const myea_layer_desc &l) { return l.type_normalization != MYEA_NORMALIZATION_NONE; }
 bool layer_uses_bias(const myea_layer_desc &l) { return !layer_uses_norm(l); }  // Layer::Use__Bias, Data.hpp:736
 
@@ -59,7 +62,7 @@ float *Net::layer_outputs(size_t li)
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
-    if (li != 0 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+    if (li != 0 && layer_is_dense(l)) {
         if (o.group) return o.summations;  // residual group: the member's output is its summation (NN/Neural_Network__Ordered.cpp:96-141)
         if (layer_uses_norm(l) && !l.use_layer_normalization_before_activation) return o.normalizes;
     }
@@ -103,9 +106,14 @@ static int check_desc(const myea_net_desc &d)
     std::vector<int> group(d.n_layers, 0);
     for (uint32_t li = 0; li < d.n_layers; ++li) {
         const myea_layer_desc &l = d.layers[li];
-        if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED && l.type_layer != MYEA_LAYER_LSTM && l.type_layer != MYEA_LAYER_RESIDUAL && !layer_is_pooling(l)) {
+        if (!layer_is_dense(l) && l.type_layer != MYEA_LAYER_LSTM && l.type_layer != MYEA_LAYER_RESIDUAL && !layer_is_pooling(l)) {
             set_last_error("layer %u: type %u is not on this path", li, l.type_layer);
             return MYEA_E_UNSUPPORTED;
+        }
+        if (layer_is_ind_rnn(l)) {
+            if (li == 0 || li + 1 >= d.n_layers) { set_last_error("layer %u: an independently recurrent layer is a hidden layer", li); return MYEA_E_INVALID; }
+            if (l.type_activation_function == MYEA_AF_SOFTMAX) { set_last_error("layer %u: softmax belongs to the output layer only", li); return MYEA_E_UNSUPPORTED; }
+            if (l.constraint_recurrent_weight_lower_bound > l.constraint_recurrent_weight_upper_bound) { set_last_error("layer %u: recurrent weight bounds out of order", li); return MYEA_E_INVALID; }
         }
         if (layer_is_pooling(l)) {
             // between fully-connected / pooling layers of a stack without blocks around it; the width must be the one
@@ -155,13 +163,13 @@ static int check_desc(const myea_net_desc &d)
             return MYEA_E_UNSUPPORTED;
         }
         if (l.type_normalization > MYEA_NORMALIZATION_BATCH_RENORMALIZATION) { set_last_error("layer %u: normalization type %u is not on this path", li, l.type_normalization); return MYEA_E_UNSUPPORTED; }
-        if (l.type_layer == MYEA_LAYER_FULLY_CONNECTED && li > 0) {
+        if (layer_is_dense(l) && li > 0) {
             const bool has_af = group[li] != 1;
             if (has_af && (l.type_activation_function == MYEA_AF_NONE || l.type_activation_function >= MYEA_AF_LENGTH)) { set_last_error("layer %u: activation %u invalid", li, l.type_activation_function); return MYEA_E_INVALID; }
             if (group[li] == 2 && l.type_activation_function == MYEA_AF_SOFTMAX) { set_last_error("layer %u: softmax belongs to the output layer only", li); return MYEA_E_UNSUPPORTED; }
             const size_t fan_in = (size_t)myea_net_desc_number_outputs(&d, myea_net_desc_previous_layer(&d, li));
             const size_t units_af = group[li] == 0 ? l.n_units : (group[li] == 1 ? 0 : fan_in), units_norm = group[li] == 0 ? l.n_units : fan_in;
-            if (l.first_connection_index + fan_in * l.n_units > d.total_weights) { set_last_error("layer %u: weight slice leaves the weight region", li); return MYEA_E_INVALID; }
+            if (l.first_connection_index + fan_in * l.n_units + (layer_is_ind_rnn(l) ? l.n_units : 0u) > d.total_weights) { set_last_error("layer %u: weight slice leaves the weight region", li); return MYEA_E_INVALID; }
             if (layer_uses_bias(l) && l.first_bias_connection_index + l.n_units > d.total_weights + d.total_bias) { set_last_error("layer %u: bias slice leaves the bias region", li); return MYEA_E_INVALID; }
             if (layer_uses_norm(l) && l.first_normalized_unit_index + units_norm > d.total_normalized_units) { set_last_error("layer %u: scale/shift slice leaves its region", li); return MYEA_E_INVALID; }
             if (l.type_dropout != MYEA_DROPOUT_NONE && l.first_mask_index + (uint64_t)units_af * d.number_recurrent_depth > d.total_mask_units) { set_last_error("layer %u: mask slice leaves the mask buffer", li); return MYEA_E_INVALID; }
@@ -227,7 +235,7 @@ int Net::create(const myea_net_desc &desc)
         const size_t sz = T * B * o.H, sa = T * B * o.AH, sn = T * B * o.NH;
         MYEA_TRY(dev_alloc(&o.values, sa));
         MYEA_HIP_TRY(hipMemset(o.values, 0, (sa ? sa : 1) * sizeof(float)));
-        if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(dev_alloc(&o.colscale, T * o.AH));
+        if (l.type_dropout != MYEA_DROPOUT_NONE && layer_is_dense(l)) MYEA_TRY(dev_alloc(&o.colscale, T * o.AH));
         if (li == 0) continue;
         if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_create_layer(li)); continue; }
         if (l.type_layer == MYEA_LAYER_MAX_POOLING) {
@@ -242,6 +250,15 @@ int Net::create(const myea_net_desc &desc)
         }
         MYEA_TRY(dev_alloc(&o.neuron_errors, sz));  // residual layer: its basic units' errors
         MYEA_HIP_TRY(hipMemset(o.neuron_errors, 0, sz * sizeof(float)));
+        if (layer_is_ind_rnn(l)) {
+            MYEA_TRY(dev_alloc(&o.pre_afs, sz));
+            MYEA_HIP_TRY(hipMemset(o.pre_afs, 0, sz * sizeof(float)));
+            // the delta of the pre-activations IS the neuron errors unless a normalisation sits between the two
+            if (layer_uses_norm(l) && l.use_layer_normalization_before_activation) {
+                MYEA_TRY(dev_alloc(&o.dafs_own, sz));
+                MYEA_HIP_TRY(hipMemset(o.dafs_own, 0, sz * sizeof(float)));
+            }
+        }
         if (layer_uses_norm(l)) {
             MYEA_TRY(dev_alloc(&o.hats, sn));
             MYEA_TRY(dev_alloc(&o.normalizes, sn));
@@ -266,7 +283,7 @@ int Net::create(const myea_net_desc &desc)
     {   // weight gradients of narrow layers over long T x batch row ranges run as split-K contractions into slabs
         size_t need = 0;
         for (size_t li = 1; li < d.n_layers; ++li) {
-            if (d.layers[li].type_layer != MYEA_LAYER_FULLY_CONNECTED) continue;
+            if (!layer_is_dense(d.layers[li])) continue;
             const int slabs = fc_dw_slabs(L[li].H, L[li].In, T * B, d.layers[li].first_connection_index);
             if (slabs > 1) need = std::max(need, (size_t)slabs * L[li].H * L[li].In);
         }
@@ -294,7 +311,7 @@ Net::~Net()
     fr(seg_first); fr(seg_len);
     fr(masks); fr(zoneout_masks);
     for (DevLayer &o : L) {
-        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index);
+        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index); fr(o.pre_afs); fr(o.dafs_own);
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
@@ -337,10 +354,11 @@ int Net::forward_fc_layer(size_t li, size_t B)
     const bool norm = layer_uses_norm(l), before = l.use_layer_normalization_before_activation != 0;
     const bool softmax = l.type_activation_function == MYEA_AF_SOFTMAX;
     const bool training = state >= MYEA_STATE_TRAINING;
+    const bool ind = layer_is_ind_rnn(l);
     bool drop = false;
     MYEA_TRY(refresh_colscale(li, &drop));
     // all time steps in one launch when the rows are contiguous and nothing is per time step
-    const bool per_t = T > 1 && (B != Bmax || norm || drop);
+    const bool per_t = T > 1 && (B != Bmax || norm || (drop && !ind));
     const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
     for (size_t c = 0; c < chunks; ++c) {
         const size_t roff = c * Bmax;  // first row of the chunk
@@ -353,7 +371,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
         g.epilogue = EPI_FC_FORWARD;
         g.bias = layer_uses_bias(l) ? parameters + l.first_bias_connection_index : nullptr;
         g.act = (int)l.type_activation_function;
-        const bool fuse_af = !softmax && !(norm && before) && !o.unit_act && gemm_can_fuse_activation((int)l.type_activation_function);
+        const bool fuse_af = !ind && !softmax && !(norm && before) && !o.unit_act && gemm_can_fuse_activation((int)l.type_activation_function);
         g.aux_out = fuse_af ? o.values + roff * H : nullptr;
         g.colscale = (fuse_af && !norm) ? cs : nullptr;
         prof_begin(0);
@@ -365,11 +383,31 @@ int Net::forward_fc_layer(size_t li, size_t B)
             MYEA_TRY(bn_forward(li, c, rows, cur, training));
             cur = o.normalizes + roff * H;
         }
+        if (ind) continue;   // the recurrence and the activation follow for the whole sequence
         if (softmax) MYEA_TRY(launch_softmax(stream, rows, H, cur, o.values + roff * H, norm ? nullptr : cs));
         else if (!fuse_af) MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, rows, H, cur, o.values + roff * H, cs, o.unit_act));
         if (norm && !before) {
             MYEA_TRY(bn_forward(li, c, rows, o.values + roff * H, training));
             if (cs) MYEA_TRY(launch_colscale(stream, rows, H, o.normalizes + roff * H, cs));
+        }
+    }
+    if (ind) {
+        // Forward_Pass__FC_Ind_RNN + Forward_Pass__FC_AF (NN/Neural_Network__Forward_Pass__Loop.cpp:434-470): the dropout of an
+        // un-normalised layer works in place on the activations the next time step reads, so it rides in the same kernel
+        const bool after = norm && !before;
+        IndRnnParams p{};
+        p.T = T; p.B = B; p.Bmax = Bmax; p.H = H;
+        p.u = parameters + l.first_connection_index + H * In;
+        p.act = (int)l.type_activation_function; p.unit_act = o.unit_act;
+        p.in = (norm && before) ? o.normalizes : o.summations;
+        p.pre_afs = o.pre_afs; p.afs = o.values;
+        p.colscale = (drop && !after) ? o.colscale : nullptr;
+        MYEA_TRY(launch_ind_rnn_forward(stream, p));
+        if (after) {
+            for (size_t t = 0; t < T; ++t) {
+                MYEA_TRY(bn_forward(li, t, B, o.values + t * Bmax * H, training));
+                if (drop) MYEA_TRY(launch_colscale(stream, B, H, o.normalizes + t * Bmax * H, o.colscale + t * H));
+            }
         }
     }
     return MYEA_OK;
@@ -421,7 +459,7 @@ int Net::forward_pass(size_t B, const float *inputs, int on_device)
         for (size_t t = 0; t < T; ++t) MYEA_TRY(launch_colscale(stream, B, In, L[0].values + t * Bmax * In, L[0].colscale + t * In));
     }
     for (size_t li = 1; li < d.n_layers; ++li) {
-        if (d.layers[li].type_layer == MYEA_LAYER_FULLY_CONNECTED) MYEA_TRY(forward_fc_layer(li, B));
+        if (layer_is_dense(d.layers[li])) MYEA_TRY(forward_fc_layer(li, B));
         else if (layer_is_pooling(d.layers[li])) MYEA_TRY(forward_pool_layer(li, B));
         else if (d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) {
             MYEA_TRY(forward_residual_block(li, B));
@@ -626,7 +664,7 @@ int Net::backward_into_layer(size_t li, size_t B)
     size_t Out = on.H;
     if (next.type_layer == MYEA_LAYER_LSTM) lstm_delta_source(gi, 0, &delta, &Out, &weights);
     const bool second_direction = next.type_layer == MYEA_LAYER_LSTM && on.lstm2 != nullptr;
-    const bool is_fc = l.type_layer == MYEA_LAYER_FULLY_CONNECTED;
+    const bool is_fc = layer_is_dense(l), ind = layer_is_ind_rnn(l);
     const bool norm = is_fc && layer_uses_norm(l), before = l.use_layer_normalization_before_activation != 0;
     const bool per_t = T > 1 && (B != Bmax || norm);
     const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
@@ -661,8 +699,11 @@ int Net::backward_into_layer(size_t li, size_t B)
             continue;
         }
         g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
-        const bool fuse = have_gemm && !o.unit_act && !o.unit_steep && gemm_can_fuse_activation(g.act);
-        if (!norm) {
+        const bool fuse = !ind && have_gemm && !o.unit_act && !o.unit_steep && gemm_can_fuse_activation(g.act);
+        if (ind) {
+            g.C = tmp1 + roff * H;
+            g.epilogue = EPI_NONE;
+        } else if (!norm) {
             g.C = (fuse ? o.neuron_errors : tmp1) + roff * H;
             g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.summations + roff * H; g.val = o.values + roff * H;
         } else if (before) {
@@ -681,6 +722,10 @@ int Net::backward_into_layer(size_t li, size_t B)
         } else {
             MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors, shortcut->H, crop, identity, H, 0, g.C));
         }
+        if (ind) {   // the recurrence follows for the whole sequence
+            if (norm && !before) MYEA_TRY(bn_backward(li, c, rows, o.values + roff * H, tmp1 + roff * H, tmp2 + roff * H));
+            continue;
+        }
         if (!fuse && !(norm && !before)) {  // act' as its own kernel (Backward_Pass__FC__DF)
             MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, rows * H, g.pre, g.val, tmp1 + roff * H, (norm ? tmp1 : o.neuron_errors) + roff * H,
                                               o.unit_act, o.unit_steep, H));
@@ -692,6 +737,19 @@ int Net::backward_into_layer(size_t li, size_t B)
             MYEA_TRY(launch_activation_derive(stream, (int)l.type_activation_function, l.activation_steepness, rows * H,
                                               o.summations + roff * H, o.values + roff * H, tmp2 + roff * H, o.neuron_errors + roff * H, o.unit_act, o.unit_steep, H));
         }
+    }
+    if (ind) {
+        // Backward_Pass__FC__DF_Ind_RNN for all time steps, then the normalisation in front of the activation, per time step
+        IndRnnParams p{};
+        p.T = T; p.B = B; p.Bmax = Bmax; p.H = H;
+        p.u = parameters + l.first_connection_index + H * o.In;
+        p.act = (int)l.type_activation_function; p.steep = l.activation_steepness; p.unit_act = o.unit_act; p.unit_steep = o.unit_steep;
+        p.pre_afs = o.pre_afs; p.afs = o.values;
+        p.dy = (norm && !before) ? tmp2 : tmp1;
+        p.dafs = o.dafs_own ? o.dafs_own : o.neuron_errors;
+        MYEA_TRY(launch_ind_rnn_backward(stream, p));
+        if (norm && before)
+            for (size_t t = T; t-- > 0;) MYEA_TRY(bn_backward(li, t, B, o.summations + t * Bmax * H, o.dafs_own + t * Bmax * H, o.neuron_errors + t * Bmax * H));
     }
     return MYEA_OK;
 }
@@ -821,6 +879,9 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
             prof_end(2.0 * (double)rows * (double)H * (double)In);
             if (layer_uses_bias(l)) MYEA_TRY(launch_column_sum(stream, rows, H, o.neuron_errors + roff * H, gradient + l.first_bias_connection_index, 1, scratch));
         }
+        if (layer_is_ind_rnn(l))
+            MYEA_TRY(launch_ind_rnn_self_weight_gradient(stream, T, B, Bmax, H, o.values, o.dafs_own ? o.dafs_own : o.neuron_errors,
+                                                         gradient + l.first_connection_index + H * In, scratch));
     }
     return MYEA_OK;
 }
@@ -829,7 +890,7 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
 // activation can no longer ride in a contraction's epilogue; it runs as its own kernel reading the arrays per column.
 int Net::set_unit_activations(size_t li, const uint32_t *types, const float *steep, size_t count)
 {
-    if (li == 0 || li >= d.n_layers || d.layers[li].type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("set_unit_activations: layer %zu is not a fully-connected hidden / output layer", li); return MYEA_E_INVALID; }
+    if (li == 0 || li >= d.n_layers || !layer_is_dense(d.layers[li])) { set_last_error("set_unit_activations: layer %zu is not a fully-connected hidden / output layer", li); return MYEA_E_INVALID; }
     DevLayer &o = L[li];
     if (d.layers[li].type_activation_function == MYEA_AF_SOFTMAX) { set_last_error("set_unit_activations: layer %zu is a softmax layer", li); return MYEA_E_INVALID; }
     if ((types || steep) && count != o.AH) { set_last_error("set_unit_activations: layer %zu has %zu activation units, got %zu", li, o.AH, count); return MYEA_E_INVALID; }
@@ -901,7 +962,7 @@ int Net::build_max_norm_segments()
     for (size_t li = 1; li < d.n_layers; ++li) {
         const myea_layer_desc &l = d.layers[li];
         const size_t In = L[li].In;
-        if (l.type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (layer_is_dense(l)) {   // neuron units; an independently recurrent layer's self weights are not among them
             for (size_t o = 0; o < L[li].H; ++o) { first.push_back(l.first_connection_index + o * In); len.push_back((unsigned)In); }
         } else if (l.type_layer == MYEA_LAYER_LSTM) {
             const size_t K = l.n_units, cpb = l.n_cells_per_block, C = K * cpb;
@@ -1012,6 +1073,14 @@ int Net::update_parameter(size_t B, size_t training_size)
     if (h.regularization__max_norm_constraints != 0.f) {
         MYEA_TRY(build_max_norm_segments());
         MYEA_TRY(launch_max_norm(stream, n_segments, seg_first, seg_len, longest_segment, h.regularization__max_norm_constraints, parameters));
+    }
+    // Update_Weight_Regularization__Constraint_Recurrent_Weight (NN/Neural_Network__Regularization__Constraint_Recurrent_Weight.cpp:
+    // 289-333): the self weights of the independently recurrent hidden layers clipped to their bounds
+    for (size_t li = 1; li + 1 < d.n_layers; ++li) {
+        const myea_layer_desc &l = d.layers[li];
+        if (!layer_is_ind_rnn(l) || (l.constraint_recurrent_weight_lower_bound == 0.f && l.constraint_recurrent_weight_upper_bound == 0.f)) continue;
+        MYEA_TRY(launch_clip_range(stream, L[li].H, parameters + l.first_connection_index + L[li].H * L[li].In,
+                                   l.constraint_recurrent_weight_lower_bound, l.constraint_recurrent_weight_upper_bound));
     }
     return lstm_parameters_changed();  // refresh the packed gate matrices
 }

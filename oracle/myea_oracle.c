@@ -68,6 +68,9 @@ typedef struct olayer {
     struct olstm *lstm;
     /* max pooling: Basic_indice_unit::ptr_array_indices, the (padded) position each output took its value from [T][Bmax][H] */
     uint32_t *pool_index;
+    /* independently recurrent layer: AF_Ind_recurrent_unit::ptr_array_pre_AFs and ::ptr_array_dAFs [T][Bmax][H]
+     * (its ptr_array_AFs are `values`, its ptr_array_errors `af_errors`) */
+    float *pre_afs, *dafs;
 } olayer;
 
 struct myea_oracle_net {
@@ -175,6 +178,9 @@ float myea_oracle_activation_derive(uint32_t type, float q, float st, float v)
 /* helpers */
 
 static int layer_uses_norm(const myea_layer_desc *l) { return l->type_normalization != MYEA_NORMALIZATION_NONE; }
+static int is_ind_rnn(const myea_layer_desc *l) { return l->type_layer == MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT; }
+/* layers made of neuron units and activation units */
+static int is_dense(const myea_layer_desc *l) { return l->type_layer == MYEA_LAYER_FULLY_CONNECTED || is_ind_rnn(l); }
 static int layer_uses_bias(const myea_layer_desc *l) { return !layer_uses_norm(l); } /* NNH/Data.hpp:736 */
 
 static float *zalloc(size_t n) { return (float *)calloc(n ? n : 1, sizeof(float)); }
@@ -185,7 +191,7 @@ static float *layer_outputs(myea_oracle_net *n, size_t li)
     const myea_layer_desc *l = &n->d.layers[li];
     olayer *o = &n->L[li];
     if (li == 0) return o->values;
-    if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+    if (is_dense(l)) {
         if (o->group) return o->summations; /* residual group: NN/Neural_Network__Ordered.cpp:96-141 */
         if (layer_uses_norm(l) && !l->use_layer_normalization_before_activation) return o->normalizes;
         return o->values;
@@ -198,7 +204,7 @@ static float *layer_derivative_outputs(myea_oracle_net *n, size_t li)
 {
     const myea_layer_desc *l = &n->d.layers[li];
     olayer *o = &n->L[li];
-    if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+    if (is_dense(l)) {
         if (o->group) return o->neuron_errors;
         if (layer_uses_norm(l) && !l->use_layer_normalization_before_activation) return o->norm_errors;
         return o->af_errors;
@@ -290,6 +296,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
         if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED) { free(n); return MYEA_E_UNSUPPORTED; }
         if (l->type_layer == MYEA_LAYER_LSTM && (layer_uses_norm(l) || (l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_ZONEOUT))) { free(n); return MYEA_E_UNSUPPORTED; }
         if (l->type_layer != MYEA_LAYER_LSTM && l->type_dropout == MYEA_DROPOUT_ZONEOUT) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (is_ind_rnn(l) && l->type_activation_function == MYEA_AF_SOFTMAX) { free(n); return MYEA_E_UNSUPPORTED; }
         size_t sz = T * B * o->H;
         o->values = zalloc(T * B * o->AH);
         if (li == 0) continue;
@@ -333,6 +340,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
             o->summations = zalloc(sz);
             o->neuron_errors = zalloc(sz);
         }
+        if (is_ind_rnn(l)) { o->pre_afs = zalloc(sz); o->dafs = zalloc(sz); }
         if (layer_uses_norm(l)) {
             size_t sn = T * B * o->NH, tn = T * o->NH;
             o->hats = zalloc(sn);
@@ -365,7 +373,7 @@ int myea_oracle_destroy(myea_oracle_net *n)
         free(o->neuron_errors); free(o->af_errors); free(o->norm_errors);
         free(o->means); free(o->variances); free(o->means_averages); free(o->variances_averages);
         free(o->r_corrections); free(o->d_corrections); free(o->derivatives_means); free(o->derivatives_variances);
-        free(o->pool_index);
+        free(o->pool_index); free(o->pre_afs); free(o->dafs);
         free(o->unit_af); free(o->unit_steep);
         if (o->lstm) {
             for (int dir = 0; dir < 2; ++dir) {
@@ -389,7 +397,7 @@ int myea_oracle_set_state_propagation(myea_oracle_net *n, uint32_t s) { if (!n) 
 /* AF_unit::ptr_type_activation_function / ptr_activation_steepness as per-unit arrays (NNH/Data.hpp, struct AF_unit) */
 int myea_oracle_set_unit_activations(myea_oracle_net *n, size_t li, const uint32_t *types, const float *steep, size_t count)
 {
-    if (!n || li == 0 || li >= n->d.n_layers || n->d.layers[li].type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_INVALID;
+    if (!n || li == 0 || li >= n->d.n_layers || !is_dense(&n->d.layers[li])) return MYEA_E_INVALID;
     olayer *o = &n->L[li];
     if (((types || steep) && count != o->AH) || n->d.layers[li].type_activation_function == MYEA_AF_SOFTMAX) return MYEA_E_INVALID;
     free(o->unit_af); free(o->unit_steep); o->unit_af = NULL; o->unit_steep = NULL;
@@ -551,8 +559,22 @@ static void fwd_dropout(myea_oracle_net *n, const myea_layer_desc *l, size_t t, 
     }
 }
 
-/* Forward_Pass__FC (layer driver): NN/Neural_Network__Forward_Pass__OpenMP.cpp:256-698.
- * order: GEMM -> bias -> [BN before] -> activation / softmax -> [BN after] -> dropout. */
+/* Forward_Pass__FC_Ind_RNN (NN/Neural_Network__Recurrent_Forward_Pass__Loop.cpp:813-866): pre_AF[t] = input[t] + u * AF[t-1],
+ * a plain copy at the first time step.  AF[t-1] is what the previous time step left in the array: after an un-normalised
+ * layer's dropout, which works in place on it. */
+static void fwd_ind_rnn(myea_oracle_net *n, size_t t, size_t B, size_t H, const float *u, const float *afs, const float *in, float *pre_afs)
+{
+    size_t Bmax = n->d.batch_size, off = Bmax * H * t, prev = t ? Bmax * H * (t - 1) : 0;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            size_t k = off + b * H + j;
+            pre_afs[k] = t ? in[k] + u[j] * afs[prev + b * H + j] : in[k];
+        }
+}
+
+/* Forward_Pass__FC (layer driver): NN/Neural_Network__Forward_Pass__OpenMP.cpp:256-698 (the serial build's
+ * NN/Neural_Network__Forward_Pass__Loop.cpp:350-790 carries the independently recurrent branch).
+ * order: GEMM -> bias -> [BN before] -> [+ u * AF[t-1]] -> activation / softmax -> [BN after] -> dropout. */
 static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
 {
     const myea_layer_desc *l = &n->d.layers[li];
@@ -568,6 +590,10 @@ static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
         if (training) fwd_bn_training(n, renorm, t, B, H, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
         else fwd_bn_inference(n, t, B, H, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
         cur = o->normalizes;
+    }
+    if (is_ind_rnn(l)) {
+        fwd_ind_rnn(n, t, B, H, n->parameters + l->first_connection_index + H * In, o->values, cur, o->pre_afs);
+        cur = o->pre_afs;
     }
     fwd_af(n, t, B, H, l->type_activation_function, o->unit_af, cur, o->values);
     float *out = o->values;
@@ -1013,7 +1039,7 @@ int myea_oracle_forward_pass(myea_oracle_net *n, size_t B, const float *inputs)
     for (size_t t = 0; t < T; ++t) fwd_dropout(n, &n->d.layers[0], t, B, In, n->L[0].values);
     for (size_t li = 1; li < n->d.n_layers; ++li) {
         const myea_layer_desc *l = &n->d.layers[li];
-        if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (is_dense(l)) {
             for (size_t t = 0; t < T; ++t) fwd_fc_layer(n, li, t, B);
         } else if (l->type_layer == MYEA_LAYER_LSTM) {
             fwd_lstm_layer(n, li, B);
@@ -1187,6 +1213,23 @@ static void bwd_df(myea_oracle_net *n, size_t t, size_t B, size_t H, uint32_t ty
         }
 }
 
+/* Backward_Pass__FC__DF_Ind_RNN (NN/Neural_Network__Backward_Pass__Loop.cpp:1296-1390): errors = dY * AF'(t);
+ * dAF(t) = errors + u * AF'(t) * dAF(t+1), without the second term at the last time step.  dAF is what the layer hands on
+ * (to its normalisation, its neuron errors and the self-weight gradient). */
+static void bwd_df_ind_rnn(myea_oracle_net *n, size_t t, size_t B, size_t H, const float *u, uint32_t type, float steep, const uint32_t *unit_type,
+                           const float *unit_steep, const float *pre, const float *val, const float *dy, float *dafs, float *errors)
+{
+    size_t Bmax = n->d.batch_size, off = Bmax * H * t, next = Bmax * H * (t + 1);
+    int last = t + 1 == n->d.number_recurrent_depth;
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            size_t k = off + b * H + j;
+            float daf = myea_oracle_activation_derive(unit_type ? unit_type[j] : type, pre[k], unit_steep ? unit_steep[j] : steep, val[k]);
+            errors[k] = dy[k] * daf;
+            dafs[k] = last ? errors[k] : errors[k] + u[j] * daf * dafs[next + b * H + j];
+        }
+}
+
 /* Backward_Pass__Batch_Normalization: :1346-1467; Backward_Pass__Batch_Renormalization: :1586-1709.
  * dScale / dShift accumulate into the gradient vector at the scale / shift slots. */
 static void bwd_bn(myea_oracle_net *n, int renorm, size_t li, size_t t, size_t B, size_t H,
@@ -1236,8 +1279,14 @@ static void bwd_gradient_fc(myea_oracle_net *n, size_t li, size_t t, size_t B)
         cur = o->norm_errors;
     }
     const float *pre_af = (layer_uses_norm(l) && before) ? o->normalizes : o->summations;
-    bwd_df(n, t, B, H, l->type_activation_function, l->activation_steepness, o->unit_af, o->unit_steep, pre_af, o->values, cur, o->af_errors);
-    cur = o->af_errors;
+    if (is_ind_rnn(l)) {
+        bwd_df_ind_rnn(n, t, B, H, n->parameters + l->first_connection_index + H * o->In, l->type_activation_function, l->activation_steepness,
+                       o->unit_af, o->unit_steep, o->pre_afs, o->values, cur, o->dafs, o->af_errors);
+        cur = o->dafs;
+    } else {
+        bwd_df(n, t, B, H, l->type_activation_function, l->activation_steepness, o->unit_af, o->unit_steep, pre_af, o->values, cur, o->af_errors);
+        cur = o->af_errors;
+    }
     if (layer_uses_norm(l) && before) {
         bwd_bn(n, renorm, li, t, B, H, o->summations /* pre_normalization */, cur, o->norm_errors);
         cur = o->norm_errors;
@@ -1355,7 +1404,7 @@ int myea_oracle_backward_pass(myea_oracle_net *n, size_t B)
         for (size_t c = 0; c < nc; ++c) {
             size_t ci = consumers[c];
             const myea_layer_desc *next = &n->d.layers[ci];
-            if (next->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+            if (is_dense(next)) {
                 if (n->L[ci].group) bwd_residual_fc_to_previous(n, ci, B, dst);
                 else for (size_t tt = T; tt-- > 0;)
                     bwd_fc(n, tt, B, n->L[ci].H, o->H, n->L[ci].neuron_errors, n->parameters + next->first_connection_index, dst);
@@ -1367,7 +1416,7 @@ int myea_oracle_backward_pass(myea_oracle_net *n, size_t B)
                 for (size_t tt = 0; tt < T; ++tt) bwd_pooling_to_previous(n, ci, tt, B, dst);
             } else return MYEA_E_UNSUPPORTED;
         }
-        if (cur->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (is_dense(cur)) {
             for (size_t tt = T; tt-- > 0;) bwd_gradient_fc(n, li, tt, B);
         } else if (cur->type_layer == MYEA_LAYER_LSTM) {
             bwd_lstm_layer(n, li, B);
@@ -1422,7 +1471,7 @@ int myea_oracle_update_derivative_weight(myea_oracle_net *n, size_t B, size_t fi
         const myea_layer_desc *l = &n->d.layers[li];
         if (l->type_layer == MYEA_LAYER_RESIDUAL || is_pooling(l)) continue;
         if (l->type_layer == MYEA_LAYER_LSTM) { dw_lstm(n, li, B); continue; }
-        if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_UNSUPPORTED;
+        if (!is_dense(l)) return MYEA_E_UNSUPPORTED;
         olayer *o = &n->L[li];
         /* Layer::ptr_array_pre_summations (NN/Neural_Network__Ordered.cpp:96-141): inside a residual block the operand
          * the weights were applied to - the layer's own activation values, or for the block's first layer its normalised
@@ -1433,6 +1482,14 @@ int myea_oracle_update_derivative_weight(myea_oracle_net *n, size_t B, size_t fi
         for (size_t t = 0; t < T; ++t) {
             dw_fc(n, t, B, o->In, o->H, x, o->neuron_errors, n->gradient + l->first_connection_index);
             if (layer_uses_bias(l)) dw_bias(n, t, B, o->H, o->neuron_errors, n->gradient + l->first_bias_connection_index);
+            /* Update_Derivative_Weight__FC_Ind_RNN (NN/Neural_Network__Recurrent_Update_Derivative_Weight__Loop.cpp:461-483),
+             * from the second time step on: du += AF[t-1] * dAF[t] */
+            if (t != 0 && is_ind_rnn(l)) {
+                size_t Bmax = n->d.batch_size, H = o->H;
+                float *du = n->gradient + l->first_connection_index + H * o->In;
+                for (size_t b = 0; b < B; ++b)
+                    for (size_t j = 0; j < H; ++j) du[j] += o->values[Bmax * H * (t - 1) + b * H + j] * o->dafs[Bmax * H * t + b * H + j];
+            }
         }
     }
     return MYEA_OK;
@@ -1498,7 +1555,7 @@ static int max_norm_constraints(myea_oracle_net *n)
     for (size_t li = 1; li < n->d.n_layers; ++li) {
         const myea_layer_desc *l = &n->d.layers[li];
         if (l->type_layer == MYEA_LAYER_RESIDUAL || is_pooling(l)) continue;
-        if (l->type_layer == MYEA_LAYER_FULLY_CONNECTED) {
+        if (is_dense(l)) {   /* neuron units: an independently recurrent layer's self weights are not among them */
             for (size_t o = 0; o < n->L[li].H; ++o) max_norm_segment(n, l->first_connection_index + o * n->L[li].In, n->L[li].In, 0);
         } else if (l->type_layer == MYEA_LAYER_LSTM) {
             for (int dir = 0; dir < (l->use_bidirectional ? 2 : 1); ++dir) {
@@ -1632,7 +1689,15 @@ int myea_oracle_update_parameter(myea_oracle_net *n, size_t B, size_t training_s
         h->optimizer_time_step -= 1.f;
         return MYEA_E_UNSUPPORTED;
     }
-    if (h->regularization__max_norm_constraints != 0.f) return max_norm_constraints(n);
+    if (h->regularization__max_norm_constraints != 0.f) { int rc = max_norm_constraints(n); if (rc != MYEA_OK) return rc; }
+    /* Update_Weight_Regularization__Constraint_Recurrent_Weight (NN/Neural_Network__Regularization__Constraint_Recurrent_Weight.cpp:
+     * 289-333): hidden layers only; the self weights of an independently recurrent layer clipped to its bounds */
+    for (size_t li = 1; li + 1 < n->d.n_layers; ++li) {
+        const myea_layer_desc *l = &n->d.layers[li];
+        if (!is_ind_rnn(l) || (l->constraint_recurrent_weight_lower_bound == 0.f && l->constraint_recurrent_weight_upper_bound == 0.f)) continue;
+        float *u = n->parameters + l->first_connection_index + n->L[li].H * n->L[li].In;
+        for (size_t j = 0; j < n->L[li].H; ++j) u[j] = clipf(u[j], l->constraint_recurrent_weight_lower_bound, l->constraint_recurrent_weight_upper_bound);
+    }
     return MYEA_OK;
 }
 

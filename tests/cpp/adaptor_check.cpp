@@ -2,6 +2,7 @@
 // `Neural_Network` (Compile -> Set__* -> Set__HIP -> the 4-call step loop + Update_Parameter, cf.
 // Neural_Network_Launcher_Windows/Source_Files/debug.cpp:481-1555 and Neural_Network/Dataset.cpp:645-658).
 // usage: adaptor_check <dir> <kind>   reads <dir>/{w,x,y,mask}.bin, writes <dir>/{params,grad}.bin and prints the loss.
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <string>
@@ -51,6 +52,27 @@ int main(int argc, char **argv)
         nn.Set__Accuracy_Function(MYEA_ACCURACY_CROSS_ENTROPY);
         nn.Set__Optimizer_Function(MYEA_OPTIMIZER_GD);
         nn.use_Nesterov = true;
+    } else if (kind == "indrnn") {  // 8 -> IndRNN-16 (default: ReLU) -> IndRNN-12 tanh, clip [-0.5, 0.75] -> FC-4 linear, GD
+        B = 6; T = 5; n_in = 8; n_out = 4;
+        Layer_Parameters layers[4];
+        for (auto &l : layers) l.type_layer = MYEA_LAYER_FULLY_CONNECTED;
+        layers[1].type_layer = layers[2].type_layer = MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT;
+        layers[0].unit_parameters[0] = 8; layers[1].unit_parameters[0] = 16; layers[2].unit_parameters[0] = 12; layers[3].unit_parameters[0] = 4;
+        if (!nn.Update__Batch_Size(B)) return 1;
+        if (!nn.Compile(4, T, MYEA_NETWORK_RECURRENT, layers)) return 1;
+        // Compile's default bounds: +-2^(1/T) for the rectifier; a layer on its default follows the activation and the clip value
+        if (!nn.Check__Use__Regularization__Constraint_Recurrent_Weight__Default(1) || nn.Check__Use__Regularization__Constraint_Recurrent_Weight__Default(3)) return 1;
+        if (std::fabs(nn.Get__Descriptor().layers[1].constraint_recurrent_weight_upper_bound - std::pow(2.f, 1.f / 5.f)) > 1e-6f) return 1;
+        if (!nn.Set__Layer_Activation_Function(2, MYEA_AF_TANH) || !nn.Check__Use__Regularization__Constraint_Recurrent_Weight__Default(2)) return 1;
+        if (std::fabs(nn.Get__Descriptor().layers[2].constraint_recurrent_weight_upper_bound - std::pow(2.f / std::pow(0.9f, 0.5f), 1.f / 5.f)) > 1e-6f) return 1;
+        if (!nn.Set__Clip_Gradient(3.0f)) return 1;
+        if (std::fabs(nn.Get__Descriptor().layers[1].constraint_recurrent_weight_upper_bound - std::pow(3.f, 1.f / 5.f)) > 1e-6f) return 1;
+        if (!nn.Set__Regularization__Constraint_Recurrent_Weight(2, -0.5f, 0.75f) || nn.Set__Regularization__Constraint_Recurrent_Weight(3, -1.f, 1.f) ||
+            nn.Set__Regularization__Constraint_Recurrent_Weight(2, 1.f, -1.f)) return 1;
+        if (!nn.Set__Clip_Gradient(1.0f) || nn.Get__Descriptor().layers[2].constraint_recurrent_weight_upper_bound != 0.75f) return 1;
+        if (!nn.Set__Layer_Activation_Function(3, MYEA_AF_LINEAR)) return 1;
+        nn.Set__Loss_Function(MYEA_LOSS_MSE);
+        nn.Set__Optimizer_Function(MYEA_OPTIMIZER_GD);
     } else {  // LSTM 8 -> 2 x LSTM-12 -> FC-12 linear, AMSGrad, clip 1.0
         B = 6; T = 5; n_in = 8; n_out = 12;
         Layer_Parameters layers[4];

@@ -69,3 +69,22 @@ def test_adaptor_lstm_amsgrad_clip(tmp_path):
     # three AMSGrad steps without re-synchronisation: entries driven by rounding-noise gradients may move by up to lr per step
     close = np.abs(got.astype(np.float64) - want) <= 1e-5 + 1e-4 * np.abs(want)
     assert close.mean() > 0.99 and np.max(np.abs(got.astype(np.float64) - want)) <= 3 * 2.1e-3
+
+
+def test_adaptor_ind_rnn_default_bounds_and_clip(tmp_path):
+    """Compile's defaults for independently recurrent layers (rectifier, bounds that follow the activation and the clip value
+    until they are set by hand) are asserted inside the host program; the training steps against the oracle here"""
+    specs = [dict(units=8), dict(type="ind_rnn", units=16, activation="RELU"), dict(type="ind_rnn", units=12, activation="TANH", recurrent_bounds=(-0.5, 0.75)),
+             dict(units=4, activation="LINEAR")]
+    B, T = 6, 5
+    rng = np.random.default_rng(3)
+    X = rng.normal(0, 1, (B, T * 8)).astype(np.float32)
+    Y = rng.normal(0, 1, (B, T * 4)).astype(np.float32)
+    desc = mb.make_desc(specs, B, T)
+    masks = np.ones(desc.total_mask_units, dtype=np.uint8)
+    hyper = dict(type_optimizer_function=mb.OPTIMIZER["GD"], type_loss_function=mb.LOSS["MSE"])
+    got, want, _ = _run(tmp_path, "indrnn", specs, B, T, hyper, X, Y, masks, seed=3)
+    assert_close(got, want, 1e-4, 1e-5, what="parameters")
+    l = desc.layers[2]
+    u = got[l.last_connection_index - 12:l.last_connection_index]
+    assert u.min() >= -0.5 and u.max() <= 0.75
