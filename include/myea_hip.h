@@ -135,6 +135,12 @@ typedef struct myea_layer_desc {
      * Compute__Regularization__Constraint_Recurrent_Weight__Default, :33-75) */
     float    constraint_recurrent_weight_lower_bound;
     float    constraint_recurrent_weight_upper_bound;
+    /* k-sparse filter on the layer's outputs (hidden fully-connected layers, also inside residual blocks): after the dropout
+     * only the k_sparsity largest values of an example's row stay, the others become 0; at inference
+     * size_t(alpha_sparsity * k_sparsity) stay.  0 = no filter (Layer::k_sparsity / ::alpha_sparsity, Data.hpp:733-734;
+     * Sparse_K_Filter, NN/Neural_Network__K_Sparse.cpp:268-339; the backward pass does not look at the filter). */
+    uint32_t k_sparsity;
+    float    alpha_sparsity;
     /* index table (into the flat parameter / gradient / optimizer vectors, and the mask buffer) */
     uint64_t first_connection_index;       /* *Layer::ptr_first_connection_index */
     uint64_t last_connection_index;        /* *Layer::ptr_last_connection_index */

@@ -100,6 +100,7 @@ public:
             l.activation_steepness = 1.f;
             l.use_layer_normalization_before_activation = 1;
             l.dropout_values[0] = 1.f;
+            l.alpha_sparsity = 1.f;   // Data.hpp:734
         }
         return Relayout("Compile");
     }
@@ -179,6 +180,28 @@ public:
         desc_.layers[index_layer].type_dropout = type_layer_dropout;
         desc_.layers[index_layer].dropout_values[0] = value_dropout[0];
         if (type_layer_dropout == MYEA_DROPOUT_ZONEOUT) desc_.layers[index_layer].dropout_values[1] = value_dropout[1];   // cell-output probability
+        return Dirty();
+    }
+    // Set__K_Sparsity / Set__Alpha_Sparsity (Neural_Network__K_Sparse.cpp:21-190): hidden layers; size_t(k * alpha) may not
+    // exceed the layer's width
+    bool Set__K_Sparsity(size_t index_layer, size_t k_sparsity)
+    {
+        if (!CheckLayer("Set__K_Sparsity", index_layer)) return false;
+        if (index_layer + 1 == desc_.n_layers) return Fail("Set__K_Sparsity", "layer received as argument is the output layer");
+        myea_layer_desc &l = desc_.layers[index_layer];
+        if (l.k_sparsity == k_sparsity) return true;
+        if ((size_t)((T_)k_sparsity * l.alpha_sparsity) > (size_t)myea_net_desc_number_outputs(&desc_, (uint32_t)index_layer)) return Fail("Set__K_Sparsity", "k-sparse can not be greater than the number of outputs");
+        l.k_sparsity = (uint32_t)k_sparsity;
+        return Dirty();
+    }
+    bool Set__Alpha_Sparsity(size_t index_layer, T_ alpha_sparsity)
+    {
+        if (!CheckLayer("Set__Alpha_Sparsity", index_layer)) return false;
+        if (index_layer + 1 == desc_.n_layers) return Fail("Set__Alpha_Sparsity", "layer received as argument is the output layer");
+        if (alpha_sparsity < 0.f) return Fail("Set__Alpha_Sparsity", "alpha k-sparse can not be less than zero");
+        myea_layer_desc &l = desc_.layers[index_layer];
+        if ((size_t)((T_)l.k_sparsity * alpha_sparsity) > (size_t)myea_net_desc_number_outputs(&desc_, (uint32_t)index_layer)) return Fail("Set__Alpha_Sparsity", "k-sparse can not be greater than the number of outputs");
+        l.alpha_sparsity = alpha_sparsity;
         return Dirty();
     }
     void Set__Loss_Function(unsigned int f) { type_loss_function = f; }

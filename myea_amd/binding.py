@@ -48,6 +48,7 @@ class LayerDesc(C.Structure):
         ("type_normalization", C.c_uint32), ("use_layer_normalization_before_activation", C.c_uint32),
         ("block_depth", C.c_uint32), ("pooling_values", C.c_uint32 * 5),
         ("constraint_recurrent_weight_lower_bound", C.c_float), ("constraint_recurrent_weight_upper_bound", C.c_float),
+        ("k_sparsity", C.c_uint32), ("alpha_sparsity", C.c_float),
         ("first_connection_index", C.c_uint64), ("last_connection_index", C.c_uint64),
         ("first_bias_connection_index", C.c_uint64), ("first_normalized_unit_index", C.c_uint64),
         ("first_mask_index", C.c_uint64),
@@ -198,7 +199,8 @@ def constraint_recurrent_weight_default(activation, recurrent_depth, clip_gradie
 def make_desc(layers, batch_size, recurrent_depth=1, network=None, lib=None):
     """layers: list of dicts (first = input layer).  Keys: units, type ('fc'|'ind_rnn'|'lstm'|...), cells_per_block,
     bidirectional, activation (name), steepness, dropout (name), keep, normalization (name), norm_before,
-    recurrent_bounds ((lower, upper) clip of an ind_rnn layer's self weights; default: the reference's)."""
+    recurrent_bounds ((lower, upper) clip of an ind_rnn layer's self weights; default: the reference's),
+    k_sparsity / alpha_sparsity (k-sparse filter on a hidden fc layer's outputs)."""
     lib = lib or load_library()
     d = NetDesc()
     d.n_layers = len(layers)
@@ -227,6 +229,8 @@ def make_desc(layers, batch_size, recurrent_depth=1, network=None, lib=None):
         l.type_normalization = NORMALIZATION[spec.get("normalization", "NONE")]
         l.use_layer_normalization_before_activation = int(spec.get("norm_before", True))
         l.block_depth = spec.get("block_depth", 0)
+        l.k_sparsity = spec.get("k_sparsity", 0)
+        l.alpha_sparsity = spec.get("alpha_sparsity", 1.0)
     rc = lib.myea_net_desc_layout(C.byref(d))
     if rc != 0:
         raise ValueError("myea_net_desc_layout failed with %d" % rc)

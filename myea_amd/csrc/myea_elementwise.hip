@@ -121,6 +121,66 @@ __global__ __launch_bounds__(kBlock) void clip_range_kernel(size_t n, float *w, 
     }
 }
 
+// Sparse_K_Filter (NN/Neural_Network__K_Sparse.cpp:268-339): per row the k largest values stay, the others become 0; among
+// equal values at the cut the lower indices stay.  One workgroup per row: a 4-pass radix select over order-preserving keys
+// finds the k-th largest key and how many entries equal to it stay, then one ordered pass writes the zeros.
+__device__ __forceinline__ unsigned k_sparse_key(float f)
+{
+    const unsigned u = __float_as_uint(f + 0.f);   // -0 and +0 are one value
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__global__ __launch_bounds__(kBlock) void k_sparse_kernel(size_t rows, size_t H, unsigned k, float *x)
+{
+    __shared__ unsigned hist[256];
+    __shared__ unsigned s_bin, s_need, wave_cnt[kBlock / 64];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    for (size_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        float *r = x + row * H;
+        unsigned prefix = 0, mask = 0, need = k;
+        for (int shift = 24; shift >= 0; shift -= 8) {
+            hist[tid] = 0;
+            __syncthreads();
+            for (size_t j = tid; j < H; j += kBlock) {
+                const unsigned key = k_sparse_key(r[j]);
+                if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+            }
+            __syncthreads();
+            if (tid == 0) {
+                unsigned acc = 0;
+                int b = 255;
+                for (; b > 0; --b) {
+                    if (acc + hist[b] >= need) break;
+                    acc += hist[b];
+                }
+                s_bin = (unsigned)b; s_need = need - acc;
+            }
+            __syncthreads();
+            prefix |= s_bin << shift; mask |= 255u << shift; need = s_need;
+            __syncthreads();
+        }
+        // prefix is the k-th largest key; `need` entries equal to it stay, in index order
+        unsigned base = 0;
+        for (size_t j0 = 0; j0 < H; j0 += kBlock) {
+            const size_t j = j0 + tid;
+            const bool valid = j < H;
+            const unsigned key = valid ? k_sparse_key(r[j]) : 0u;
+            const bool eq = valid && key == prefix;
+            const unsigned long long ballot = __ballot(eq);
+            const unsigned rank = (unsigned)__popcll(ballot & ((1ull << lane) - 1ull));
+            if (lane == 0) wave_cnt[w] = (unsigned)__popcll(ballot);
+            __syncthreads();
+            unsigned before = 0, total = 0;
+#pragma unroll
+            for (int q = 0; q < kBlock / 64; ++q) { if (q < w) before += wave_cnt[q]; total += wave_cnt[q]; }
+            const bool keep = key > prefix || (eq && base + before + rank < need);
+            if (valid && !keep) r[j] = 0.f;
+            base += total;
+            __syncthreads();
+        }
+    }
+}
+
 // Forward_Pass__FC_AF__Softmax (:4870-4905): one wavefront per row.
 __global__ __launch_bounds__(kBlock) void softmax_kernel(size_t rows, size_t H, const float *x, float *y, const float *colscale)
 {
@@ -686,6 +746,15 @@ int launch_column_sum(hipStream_t s, size_t rows, size_t H, const float *x, floa
     hipLaunchKernelGGL((column_partial_kernel<1, SumF>), dim3((unsigned)((H + 63) / 64), (unsigned)S), dim3(kBlock), 0, s, rows, H, chunk, scratch, f);
     MYEA_HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, kBlock)), dim3(kBlock), 0, s, H, S, scratch, out, accumulate);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_k_sparse(hipStream_t s, size_t rows, size_t H, size_t k, float *x)
+{
+    if (rows == 0 || k >= H) return MYEA_OK;   // k == width: nothing to filter (:288)
+    if (k == 0) { set_last_error("k-sparse filter: k is 0"); return MYEA_E_INVALID; }
+    hipLaunchKernelGGL(k_sparse_kernel, dim3(grid_for(rows, 1)), dim3(kBlock), 0, s, rows, H, (unsigned)k, x);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

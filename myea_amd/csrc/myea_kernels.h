@@ -124,6 +124,9 @@ int launch_compute_error(hipStream_t s, const ErrorParams &p);
 int launch_accuracy_r(hipStream_t s, const ErrorParams &p, float desired_mean, float predicted_mean);
 int launch_gather_rows(hipStream_t s, size_t B, size_t row_floats, const unsigned long long *index, const float *src, float *dst);
 
+// per row of x [rows][H]: the k largest values stay, the others become 0 (ties at the cut: the lower indices stay)
+int launch_k_sparse(hipStream_t s, size_t rows, size_t H, size_t k, float *x);
+
 // Independently recurrent layer over the whole sequence: tensors are [T][Bmax][H], the first B rows of a time step in use.
 struct IndRnnParams {
     size_t T, B, Bmax, H;

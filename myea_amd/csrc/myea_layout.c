@@ -122,6 +122,14 @@ int myea_net_desc_layout(myea_net_desc *d)
         if (l->type_layer == MYEA_LAYER_LSTM && l->n_cells_per_block == 0) return MYEA_E_INVALID;
         if (!is_dense(l) && l->type_layer != MYEA_LAYER_LSTM && l->type_layer != MYEA_LAYER_RESIDUAL && !pooling) return MYEA_E_UNSUPPORTED;
         if (is_ind_rnn(l) && (li == 0 || li + 1 == d->n_layers)) return MYEA_E_INVALID;
+        if (l->k_sparsity != 0) {
+            /* Set__K_Sparsity / Set__Alpha_Sparsity (NN/Neural_Network__K_Sparse.cpp:38-190): hidden layers, alpha >= 0,
+             * size_t(k * alpha) <= width.  Here also k <= width and at least one value kept at inference (the reference
+             * reads its pair array's first slot whatever k is). */
+            const float scaled = (float)l->k_sparsity * l->alpha_sparsity;
+            if (li == 0 || li + 1 == d->n_layers || l->type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_UNSUPPORTED;
+            if (l->k_sparsity > l->n_units || !(l->alpha_sparsity >= 0.f) || !(scaled >= 1.f) || (uint64_t)scaled > l->n_units) return MYEA_E_INVALID;
+        }
         if (pooling && (l->pooling_values[0] == 0 || l->pooling_values[1] == 0 || li == 0 || li + 1 == d->n_layers)) return MYEA_E_INVALID;
         if (l->type_normalization != MYEA_NORMALIZATION_NONE) any_norm = 1;
     }
@@ -148,7 +156,7 @@ int myea_net_desc_layout(myea_net_desc *d)
         if (l->type_layer != MYEA_LAYER_RESIDUAL) continue;
         if (l->block_depth == 0 || (uint64_t)li + l->block_depth + 1 >= d->n_layers) return MYEA_E_INVALID;
         for (uint32_t k = 1; k <= l->block_depth; ++k)
-            if (d->layers[li + k].type_layer != MYEA_LAYER_FULLY_CONNECTED) return MYEA_E_UNSUPPORTED;
+            if (d->layers[li + k].type_layer != MYEA_LAYER_FULLY_CONNECTED || d->layers[li + k].k_sparsity != 0) return MYEA_E_UNSUPPORTED;
         li += l->block_depth;
     }
 

@@ -110,6 +110,11 @@ static int check_desc(const myea_net_desc &d)
             set_last_error("layer %u: type %u is not on this path", li, l.type_layer);
             return MYEA_E_UNSUPPORTED;
         }
+        if (l.k_sparsity != 0) {
+            const float scaled = (float)l.k_sparsity * l.alpha_sparsity;
+            if (li == 0 || li + 1 >= d.n_layers || l.type_layer != MYEA_LAYER_FULLY_CONNECTED || block_end != 0) { set_last_error("layer %u: the k-sparse filter is on this path for hidden fully-connected layers outside residual blocks", li); return MYEA_E_UNSUPPORTED; }
+            if (l.k_sparsity > l.n_units || !(l.alpha_sparsity >= 0.f) || !(scaled >= 1.f) || (uint64_t)scaled > l.n_units) { set_last_error("layer %u: k-sparse filter: k %u, alpha %g do not fit %u units", li, l.k_sparsity, (double)l.alpha_sparsity, l.n_units); return MYEA_E_INVALID; }
+        }
         if (layer_is_ind_rnn(l)) {
             if (li == 0 || li + 1 >= d.n_layers) { set_last_error("layer %u: an independently recurrent layer is a hidden layer", li); return MYEA_E_INVALID; }
             if (l.type_activation_function == MYEA_AF_SOFTMAX) { set_last_error("layer %u: softmax belongs to the output layer only", li); return MYEA_E_UNSUPPORTED; }
@@ -389,6 +394,12 @@ int Net::forward_fc_layer(size_t li, size_t B)
         if (norm && !before) {
             MYEA_TRY(bn_forward(li, c, rows, o.values + roff * H, training));
             if (cs) MYEA_TRY(launch_colscale(stream, rows, H, o.normalizes + roff * H, cs));
+        }
+        // k-Sparse, after the dropout (NN/Neural_Network__Forward_Pass__Loop.cpp:752-790): k values stay strictly in the
+        // training state, size_t(alpha k) otherwise
+        if (l.k_sparsity != 0) {
+            const size_t k = state == MYEA_STATE_TRAINING ? (size_t)l.k_sparsity : (size_t)(l.alpha_sparsity * (float)l.k_sparsity);
+            MYEA_TRY(launch_k_sparse(stream, rows, H, k, ((norm && !before) ? o.normalizes : o.values) + roff * H));
         }
     }
     if (ind) {

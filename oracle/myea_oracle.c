@@ -559,6 +559,42 @@ static void fwd_dropout(myea_oracle_net *n, const myea_layer_desc *l, size_t t, 
     }
 }
 
+/* Sparse_K_Filter (NN/Neural_Network__K_Sparse.cpp:268-339): per example, the k largest values of the row stay where they
+ * are and the others become 0.  The reference keeps a sorted array of (index, value) pairs seeded with the first k entries
+ * and lets a later entry replace the smallest pair only when it is strictly greater; which of several EQUAL smallest pairs
+ * goes is left to std::sort's unspecified order of equal keys.  Restated with that choice fixed: among equal values the
+ * lower index stays.  Rows without equal values at the cut are unaffected by the choice. */
+static void fwd_k_sparse(myea_oracle_net *n, size_t t, size_t B, size_t H, size_t k, float *v)
+{
+    if (k >= H) return;
+    size_t off = n->d.batch_size * H * t;
+    size_t *idx = (size_t *)malloc((k ? k : 1) * sizeof(size_t));
+    float *val = (float *)malloc((k ? k : 1) * sizeof(float));
+    for (size_t b = 0; b < B; ++b) {
+        float *row = v + off + b * H;
+        size_t kept = 0;
+        /* pairs ascending by (value, then index descending): slot 0 is the one to go - the smallest value, and among equal
+         * values the highest index */
+        for (size_t j = 0; j < H; ++j) {
+            if (kept == k) {
+                if (!(val[0] < row[j])) continue;   /* strictly greater only */
+                /* drop slot 0 */
+                for (size_t s = 1; s < kept; ++s) { val[s - 1] = val[s]; idx[s - 1] = idx[s]; }
+                --kept;
+            }
+            /* insert (j, row[j]); j is the highest index so far, so among equal values it goes in front */
+            size_t at = 0;
+            while (at < kept && val[at] < row[j]) ++at;
+            for (size_t s = kept; s > at; --s) { val[s] = val[s - 1]; idx[s] = idx[s - 1]; }
+            val[at] = row[j]; idx[at] = j;
+            ++kept;
+        }
+        memset(row, 0, H * sizeof(float));
+        for (size_t s = 0; s < kept; ++s) row[idx[s]] = val[s];
+    }
+    free(idx); free(val);
+}
+
 /* Forward_Pass__FC_Ind_RNN (NN/Neural_Network__Recurrent_Forward_Pass__Loop.cpp:813-866): pre_AF[t] = input[t] + u * AF[t-1],
  * a plain copy at the first time step.  AF[t-1] is what the previous time step left in the array: after an un-normalised
  * layer's dropout, which works in place on it. */
@@ -603,6 +639,10 @@ static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
         out = o->normalizes;
     }
     fwd_dropout(n, l, t, B, H, out);
+    /* k-Sparse, after the dropout (NN/Neural_Network__Forward_Pass__Loop.cpp:752-790): k values stay strictly in the
+     * training state, size_t(alpha * k) otherwise */
+    if (l->k_sparsity != 0)
+        fwd_k_sparse(n, t, B, H, n->state == MYEA_STATE_TRAINING ? (size_t)l->k_sparsity : (size_t)(l->alpha_sparsity * (float)l->k_sparsity), out);
 }
 
 /* Forward_Pass__Residual__FC: NN/Neural_Network__Forward_Pass__OpenMP.cpp:4039-4433.  Pre-activation order on the

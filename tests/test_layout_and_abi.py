@@ -95,4 +95,4 @@ def test_struct_sizes_match_the_header():
     """ctypes mirrors are laid out as the C structs (checked through the layout function writing the far end)"""
     d = oracle_desc([dict(units=3)] + [dict(units=2, activation="TANH")] * 63, 1)
     assert d.n_layers == 64 and d.layers[63].first_bias_connection_index == d.total_weights + 2 * 62
-    assert C.sizeof(mb.LayerDesc) == 120 and C.sizeof(mb.Hyper) == 42 * 4 and C.sizeof(mb.LossState) == 64
+    assert C.sizeof(mb.LayerDesc) == 128 and C.sizeof(mb.Hyper) == 42 * 4 and C.sizeof(mb.LossState) == 64
