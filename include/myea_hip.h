@@ -71,6 +71,8 @@ enum {
 /* Enum_Type_Layer_Dropout.hpp */
 enum {
     MYEA_DROPOUT_NONE = 0, MYEA_DROPOUT_BERNOULLI = 2, MYEA_DROPOUT_BERNOULLI_INVERTED = 3,
+    MYEA_DROPOUT_GAUSSIAN = 4, /* training state: y *= N(1, dropout_values[0]) per (example, unit); dropout_values[0] = p / (1 - p) */
+    MYEA_DROPOUT_UOUT = 6,     /* training state: y += y * U(-dropout_values[0], dropout_values[0]) per (example, unit) */
     MYEA_DROPOUT_ZONEOUT = 7   /* LSTM layers only: dropout_values[0] / [1] = zoneout probability of the cell state / the cell output */
 };
 
@@ -253,6 +255,7 @@ enum {
                                            [Bmax][fan-in] (AF_unit errors, or the normalised units' errors when
                                            the member is normalised); absent for an un-normalised first member */
     /* LSTM taps, [T][Bmax][cells] or [T][Bmax][blocks] */
+    MYEA_TENSOR_DROPOUT_NOISE = 9,      /* Gaussian / Uout dropout: the draws the last training-state forward pass used [T][Bmax][H] */
     MYEA_TENSOR_LSTM_CELL_INPUT = 16,      /* z  */
     MYEA_TENSOR_LSTM_CELL_STATE = 17,      /* c  */
     MYEA_TENSOR_LSTM_INPUT_GATE = 18,      /* i  */
@@ -334,6 +337,18 @@ int myea_hip_upload_masks(myea_hip_net *net, const uint8_t *host_masks, size_t c
  * masks act in the training state only (Neural_Network__Forward_Pass__Loop.cpp:2088-2092); the backward pass does not read them,
  * as in the reference. */
 int myea_hip_upload_zoneout_masks(myea_hip_net *net, const uint8_t *host_masks, size_t count);
+/* Gaussian / Uout dropout (Forward_Pass__Dropout__Gaussian / __Uout, Neural_Network__Forward_Pass__Loop.cpp:4993-5014, 5047-5068)
+ * draw one random number per (time step, example, unit) inside the forward pass, strictly in the training state, from the
+ * network's host generators (std::mt19937 behind std::normal_distribution / uniform_real_distribution); the backward pass never
+ * sees the draws.  Two sources here:
+ *  - default: a counter-based device generator (Philox 4x32-10; normal draws by Box-Muller) keyed by
+ *    myea_hip_set_dropout_seed() and advanced by every training-state forward pass - same distributions, another stream;
+ *  - myea_hip_upload_dropout_noise(): the caller's own draws for one layer, [T][Bmax][H] floats (`count` = T x batch_size x
+ *    width), used by every following forward pass until the call is repeated with NULL / 0.  A caller that draws with the
+ *    reference's generators in the reference's order gets the reference's numbers.
+ * Either way MYEA_TENSOR_DROPOUT_NOISE reads back what the last forward pass used. */
+int myea_hip_set_dropout_seed(myea_hip_net *net, uint64_t seed);
+int myea_hip_upload_dropout_noise(myea_hip_net *net, size_t layer_index, const float *noise, size_t count, int noise_on_device);
 /* Clear_Training_Arrays (Train.cpp:93-126) + Clear_Optimizer (Train.cpp:128-263): zero the gradient
  * vector and all optimizer state, optimizer_time_step = 0. */
 int myea_hip_clear_training_arrays(myea_hip_net *net);

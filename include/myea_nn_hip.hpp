@@ -179,6 +179,9 @@ public:
         if (value_dropout == nullptr || value_dropout[0] < 0.f || value_dropout[0] > 1.f) return Fail("Set__Dropout", "retention probability out of [0, 1]");
         desc_.layers[index_layer].type_dropout = type_layer_dropout;
         desc_.layers[index_layer].dropout_values[0] = value_dropout[0];
+        // Set__Dropout_Gaussian keeps p / (1 - p), the spread of the multiplicative noise (Neural_Network__Dropout.cpp:509-565)
+        if (type_layer_dropout == MYEA_DROPOUT_GAUSSIAN)
+            desc_.layers[index_layer].dropout_values[0] = value_dropout[0] == 1.f ? 0.f : (T_)((double)value_dropout[0] / (1.0 - (double)value_dropout[0]));
         if (type_layer_dropout == MYEA_DROPOUT_ZONEOUT) desc_.layers[index_layer].dropout_values[1] = value_dropout[1];   // cell-output probability
         return Dirty();
     }

@@ -25,14 +25,14 @@ AF = dict(NONE=0, COSINE=1, COSINE_SYMMETRIC=2, ELU=3, ELLIOT=4, ELLIOT_SYMMETRI
           SINE=19, SIGMOID_STEPWISE=20, SINE_SYMMETRIC=21, SOFTMAX=22, TANH=23, TANH_STEPWISE=24,
           THRESHOLD=25, THRESHOLD_SYMMETRIC=26)
 OPTIMIZER = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP_PLUS=8, NOSADAM=9)
-DROPOUT = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3, ZONEOUT=7)
+DROPOUT = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3, GAUSSIAN=4, UOUT=6, ZONEOUT=7)
 NORMALIZATION = dict(NONE=0, BATCH_NORMALIZATION=1, BATCH_RENORMALIZATION=2)
 LOSS = dict(NONE=0, BIT=1, CROSS_ENTROPY=2, L1=3, L2=4, MAE=5, MAPE=6, ME=9, MSE=10, RMSE=11, SMAPE=12)
 ACCURACY = dict(NONE=0, CROSS_ENTROPY=1, DIRECTIONAL=2, DISTANCE=3, R=4, SIGN=5)
 STATE_INFERENCE, STATE_TRAINING = 0, 1
 OPT_STATE = dict(PREVIOUS_DELTA=0, FIRST_MOMENT=1, SECOND_MOMENT=2, SECOND_MOMENT_HAT=3, PREVIOUS_STEPS=4, PREVIOUS_DERIVATIVES=5)
 TENSOR = dict(OUTPUTS=0, SUMMATIONS=1, ERRORS=2, NORM_HATS=3, NORM_MEANS=4, NORM_VARIANCES=5,
-              NORM_MEANS_AVERAGES=6, NORM_VARIANCES_AVERAGES=7, INPUT_SIDE_ERRORS=8,
+              NORM_MEANS_AVERAGES=6, NORM_VARIANCES_AVERAGES=7, INPUT_SIDE_ERRORS=8, DROPOUT_NOISE=9,
               LSTM_CELL_INPUT=16, LSTM_CELL_STATE=17, LSTM_INPUT_GATE=18, LSTM_FORGET_GATE=19,
               LSTM_OUTPUT_GATE=20, LSTM_DELTA_CELL_INPUT=21, LSTM_DELTA_CELL_STATE=22,
               LSTM_DELTA_INPUT_GATE=23, LSTM_DELTA_FORGET_GATE=24, LSTM_DELTA_OUTPUT_GATE=25, LSTM_CELL_OUTPUT=26, LSTM_DELTA_CELL_OUTPUT=27,
@@ -99,7 +99,7 @@ ABI_SYMBOLS = [
     "myea_hip_synchronize", "myea_hip_last_error", "myea_hip_set_hyper", "myea_hip_get_hyper",
     "myea_hip_set_state_propagation", "myea_hip_upload_parameters", "myea_hip_download_parameters",
     "myea_hip_upload_optimizer_state", "myea_hip_download_optimizer_state", "myea_hip_upload_masks", "myea_hip_set_unit_activations",
-    "myea_hip_upload_zoneout_masks", "myea_hip_compute_loss", "myea_hip_compute_accuracy_r", "myea_hip_gather_examples", "myea_hip_device_buffer_create", "myea_hip_device_buffer_destroy",
+    "myea_hip_upload_zoneout_masks", "myea_hip_set_dropout_seed", "myea_hip_upload_dropout_noise", "myea_hip_compute_loss", "myea_hip_compute_accuracy_r", "myea_hip_gather_examples", "myea_hip_device_buffer_create", "myea_hip_device_buffer_destroy",
     "myea_hip_clear_training_arrays", "myea_hip_forward_pass", "myea_hip_compute_error", "myea_hip_backward_pass",
     "myea_hip_update_derivative_weight", "myea_hip_update_parameter", "myea_hip_reset_loss", "myea_hip_get_loss",
     "myea_hip_download_gradient", "myea_hip_upload_gradient", "myea_hip_download_tensor",
@@ -150,6 +150,8 @@ def load_library(path=LIB_PATH):
     lib.myea_hip_reset_loss.argtypes = [vp]
     lib.myea_hip_get_loss.argtypes = [vp, P(LossState)]
     lib.myea_hip_upload_zoneout_masks.argtypes = [vp, vp, sz]
+    lib.myea_hip_set_dropout_seed.argtypes = [vp, C.c_uint64]
+    lib.myea_hip_upload_dropout_noise.argtypes = [vp, sz, vp, sz, i32]
     lib.myea_hip_compute_loss.argtypes = [vp, sz, vp, i32]
     lib.myea_hip_compute_accuracy_r.argtypes = [vp, sz, vp, i32, C.c_float, C.c_float]
     lib.myea_hip_gather_examples.argtypes = [vp, vp, vp, sz, sz, vp, i32, sz]
@@ -330,10 +332,27 @@ class HipNetwork:
         g = np.ascontiguousarray(g, dtype=np.float32)
         self._check(self.lib.myea_hip_upload_gradient(self.handle, _ptr(g), g.size))
 
-    def download_tensor(self, layer, kind, count):
+    def download_tensor(self, layer, kind, count=None):
+        if count is None:   # a [T][batch_size][width] tensor of the layer, whole
+            count = self.desc.number_recurrent_depth * self.desc.batch_size * self.lib.myea_net_desc_number_outputs(C.byref(self.desc), layer)
         out = np.empty(count, dtype=np.float32)
         self._check(self.lib.myea_hip_download_tensor(self.handle, layer, kind, _ptr(out), out.size))
         return out
+
+    def set_dropout_seed(self, seed):
+        self._check(self.lib.myea_hip_set_dropout_seed(self.handle, seed))
+
+    def upload_dropout_noise(self, layer, noise, on_device=False):
+        """[T][batch_size][width] draws for a Gaussian / Uout layer; None returns the layer to the device generator"""
+        if noise is None:
+            self._check(self.lib.myea_hip_upload_dropout_noise(self.handle, layer, None, 0, 0))
+            return
+        if isinstance(noise, np.ndarray):
+            noise = np.ascontiguousarray(noise, dtype=np.float32)
+            count = noise.size
+        else:
+            count = noise.numel()
+        self._check(self.lib.myea_hip_upload_dropout_noise(self.handle, layer, _ptr(noise), count, int(on_device)))
 
     def upload_zoneout_masks(self, m):
         m = np.ascontiguousarray(m, dtype=np.uint8)

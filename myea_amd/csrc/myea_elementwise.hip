@@ -121,6 +121,60 @@ __global__ __launch_bounds__(kBlock) void clip_range_kernel(size_t n, float *w, 
     }
 }
 
+// Gaussian / Uout dropout (Forward_Pass__Dropout__Gaussian / __Uout, NN/Neural_Network__Forward_Pass__Loop.cpp:4993-5014,
+// 5047-5068).  The draws come from a tensor: either the caller's own or the output of the counter-based generator below.
+// Philox 4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11): counter = (element index / 4 lo, hi,
+// stream lo, stream hi), key = the seed's two halves; four 32-bit outputs per counter value.
+__device__ __forceinline__ void philox4x32_10(unsigned c0, unsigned c1, unsigned c2, unsigned c3, unsigned k0, unsigned k1, unsigned out[4])
+{
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const unsigned long long p0 = 0xD2511F53ull * c0, p1 = 0xCD9E8D57ull * c2;
+        const unsigned n0 = (unsigned)(p1 >> 32) ^ c1 ^ k0, n1 = (unsigned)p1, n2 = (unsigned)(p0 >> 32) ^ c3 ^ k1, n3 = (unsigned)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+// normal: mean + sd * N(0,1) by Box-Muller on two uniforms in (0, 1]; uniform: lo + (hi - lo) * U[0, 1)
+__global__ __launch_bounds__(kBlock) void dropout_noise_kernel(size_t n, float *noise, int normal, float a, float b, unsigned long long seed, unsigned long long stream)
+{
+    const size_t quads = (n + 3) / 4;
+    for (size_t q = (size_t)blockIdx.x * kBlock + threadIdx.x; q < quads; q += (size_t)gridDim.x * kBlock) {
+        unsigned r[4];
+        philox4x32_10((unsigned)q, (unsigned)(q >> 32), (unsigned)stream, (unsigned)(stream >> 32), (unsigned)seed, (unsigned)(seed >> 32), r);
+        float v[4];
+        if (normal) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const float u1 = ((float)(r[2 * h] >> 8) + 1.f) * (1.f / 16777216.f);   // (0, 1]
+                const float u2 = (float)(r[2 * h + 1] >> 8) * (1.f / 16777216.f);       // [0, 1)
+                const float rad = sqrtf(-2.f * logf(u1));
+                float sn, cs;
+                sincosf(6.283185307179586f * u2, &sn, &cs);
+                v[2 * h] = a + b * rad * cs;
+                v[2 * h + 1] = a + b * rad * sn;
+            }
+        } else {
+#pragma unroll
+            for (int h = 0; h < 4; ++h) v[h] = a + (b - a) * ((float)(r[h] >> 8) * (1.f / 16777216.f));
+        }
+#pragma unroll
+        for (int h = 0; h < 4; ++h)
+            if (q * 4 + h < n) noise[q * 4 + h] = v[h];
+    }
+}
+
+// gaussian: y *= noise; uout: y += y * noise
+__global__ __launch_bounds__(kBlock) void dropout_noise_apply_kernel(size_t n, float *y, const float *noise, int uout)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const float v = y[i], g = noise[i];
+        y[i] = uout ? __fadd_rn(v, __fmul_rn(v, g)) : v * g;
+    }
+}
+
 // Sparse_K_Filter (NN/Neural_Network__K_Sparse.cpp:268-339): per row the k largest values stay, the others become 0; among
 // equal values at the cut the lower indices stay.  One workgroup per row: a 4-pass radix select over order-preserving keys
 // finds the k-th largest key and how many entries equal to it stay, then one ordered pass writes the zeros.
@@ -746,6 +800,22 @@ int launch_column_sum(hipStream_t s, size_t rows, size_t H, const float *x, floa
     hipLaunchKernelGGL((column_partial_kernel<1, SumF>), dim3((unsigned)((H + 63) / 64), (unsigned)S), dim3(kBlock), 0, s, rows, H, chunk, scratch, f);
     MYEA_HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, kBlock)), dim3(kBlock), 0, s, H, S, scratch, out, accumulate);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_dropout_noise(hipStream_t s, size_t n, float *noise, int normal, float a, float b, unsigned long long seed, unsigned long long stream_id)
+{
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(dropout_noise_kernel, dim3(grid_for((n + 3) / 4, kBlock)), dim3(kBlock), 0, s, n, noise, normal, a, b, seed, stream_id);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_dropout_noise_apply(hipStream_t s, size_t n, float *y, const float *noise, int uout)
+{
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(dropout_noise_apply_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, n, y, noise, uout);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

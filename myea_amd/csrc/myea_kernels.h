@@ -124,6 +124,12 @@ int launch_compute_error(hipStream_t s, const ErrorParams &p);
 int launch_accuracy_r(hipStream_t s, const ErrorParams &p, float desired_mean, float predicted_mean);
 int launch_gather_rows(hipStream_t s, size_t B, size_t row_floats, const unsigned long long *index, const float *src, float *dst);
 
+// Gaussian / Uout dropout draws: noise[i] = a + b * N(0,1) (normal) or uniform in [a, b); counter-based, reproducible from
+// (seed, stream_id, i)
+int launch_dropout_noise(hipStream_t s, size_t n, float *noise, int normal, float a, float b, unsigned long long seed, unsigned long long stream_id);
+// y *= noise (Gaussian) or y += y * noise (Uout)
+int launch_dropout_noise_apply(hipStream_t s, size_t n, float *y, const float *noise, int uout);
+
 // per row of x [rows][H]: the k largest values stay, the others become 0 (ties at the cut: the lower indices stay)
 int launch_k_sparse(hipStream_t s, size_t rows, size_t H, size_t k, float *x);
 

@@ -33,6 +33,9 @@ struct DevLayer {
     // independently recurrent layer: pre-activations [T][Bmax][H]; the delta of the pre-activations lives in neuron_errors
     // unless a normalisation sits between the summation and the activation (then in dafs_own)
     float *pre_afs = nullptr, *dafs_own = nullptr;
+    // Gaussian / Uout dropout: the draws of the forward pass [T][Bmax][H]; noise_uploaded: the caller's own, kept as they are
+    float *noise = nullptr;
+    bool noise_uploaded = false;
     int *unit_act = nullptr;    // per-unit activation types [AH], null = layer-wide
     float *unit_steep = nullptr;  // per-unit steepnesses [AH], null = layer-wide
     LstmLayer *lstm = nullptr, *lstm2 = nullptr;  // lstm2: the time-reversed direction of a bidirectional layer
@@ -48,6 +51,8 @@ struct ProfEvent {
 bool layer_is_pooling(const myea_layer_desc &l);
 bool layer_is_ind_rnn(const myea_layer_desc &l);
 bool layer_is_dense(const myea_layer_desc &l);
+bool layer_uses_mask_dropout(const myea_layer_desc &l);
+bool layer_uses_noise_dropout(const myea_layer_desc &l);
 bool layer_uses_norm(const myea_layer_desc &l);
 bool layer_uses_bias(const myea_layer_desc &l);
 
@@ -58,6 +63,7 @@ struct Net {
     hipStream_t stream = nullptr;
     float *parameters = nullptr, *gradient = nullptr, *opt[MYEA_STATE_KINDS] = {};
     uint8_t *masks = nullptr;
+    unsigned long long dropout_seed = 0x9E3779B97F4A7C15ull, dropout_stream = 0;   // device generator: key and the next stream id
     uint8_t *zoneout_masks = nullptr;   // [state | output] halves, per LSTM layer [T][cells]
     size_t zoneout_count = 0;
     // max-norm constraint: weight segments (one per neuron / per LSTM gate vector), built on first use

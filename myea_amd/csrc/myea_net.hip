@@ -55,6 +55,8 @@ bool layer_is_pooling(const myea_layer_desc &l) { return l.type_layer == MYEA_LA
 bool layer_is_ind_rnn(const myea_layer_desc &l) { return l.type_layer == MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT; }
 // layers made of neuron units and activation units
 bool layer_is_dense(const myea_layer_desc &l) { return l.type_layer == MYEA_LAYER_FULLY_CONNECTED || layer_is_ind_rnn(l); }
+bool layer_uses_mask_dropout(const myea_layer_desc &l) { return l.type_dropout == MYEA_DROPOUT_BERNOULLI || l.type_dropout == MYEA_DROPOUT_BERNOULLI_INVERTED; }
+bool layer_uses_noise_dropout(const myea_layer_desc &l) { return l.type_dropout == MYEA_DROPOUT_GAUSSIAN || l.type_dropout == MYEA_DROPOUT_UOUT; }
 bool layer_uses_norm(const myea_layer_desc &l) { return l.type_normalization != MYEA_NORMALIZATION_NONE; }
 bool layer_uses_bias(const myea_layer_desc &l) { return !layer_uses_norm(l); }  // Layer::Use__Bias, Data.hpp:736
 
@@ -163,7 +165,11 @@ static int check_desc(const myea_net_desc &d)
         if (layer_is_pooling(l)) continue;
         if (l.type_dropout == MYEA_DROPOUT_ZONEOUT && l.type_layer == MYEA_LAYER_LSTM) {
             // masks per (time step, cell), uploaded with myea_hip_upload_zoneout_masks
-        } else if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_BERNOULLI && l.type_dropout != MYEA_DROPOUT_BERNOULLI_INVERTED) {
+        } else if (layer_uses_noise_dropout(l)) {
+            // one draw per (time step, example, unit): hidden / output fully-connected layers outside residual blocks
+            if (li == 0 || l.type_layer != MYEA_LAYER_FULLY_CONNECTED || group[li] != 0) { set_last_error("layer %u: Gaussian / Uout dropout is on this path for fully-connected layers outside residual blocks", li); return MYEA_E_UNSUPPORTED; }
+            if (!(l.dropout_values[0] >= 0.f)) { set_last_error("layer %u: dropout value %g", li, (double)l.dropout_values[0]); return MYEA_E_INVALID; }
+        } else if (l.type_dropout != MYEA_DROPOUT_NONE && !layer_uses_mask_dropout(l)) {
             set_last_error("layer %u: dropout type %u is not on this path", li, l.type_dropout);
             return MYEA_E_UNSUPPORTED;
         }
@@ -240,7 +246,11 @@ int Net::create(const myea_net_desc &desc)
         const size_t sz = T * B * o.H, sa = T * B * o.AH, sn = T * B * o.NH;
         MYEA_TRY(dev_alloc(&o.values, sa));
         MYEA_HIP_TRY(hipMemset(o.values, 0, (sa ? sa : 1) * sizeof(float)));
-        if (l.type_dropout != MYEA_DROPOUT_NONE && layer_is_dense(l)) MYEA_TRY(dev_alloc(&o.colscale, T * o.AH));
+        if (layer_uses_mask_dropout(l) && layer_is_dense(l)) MYEA_TRY(dev_alloc(&o.colscale, T * o.AH));
+        if (layer_uses_noise_dropout(l)) {
+            MYEA_TRY(dev_alloc(&o.noise, sz));
+            MYEA_TRY(launch_fill(0, o.noise, sz, l.type_dropout == MYEA_DROPOUT_GAUSSIAN ? 1.f : 0.f));   // neutral until a pass draws
+        }
         if (li == 0) continue;
         if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_create_layer(li)); continue; }
         if (l.type_layer == MYEA_LAYER_MAX_POOLING) {
@@ -316,7 +326,7 @@ Net::~Net()
     fr(seg_first); fr(seg_len);
     fr(masks); fr(zoneout_masks);
     for (DevLayer &o : L) {
-        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index); fr(o.pre_afs); fr(o.dafs_own);
+        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index); fr(o.pre_afs); fr(o.dafs_own); fr(o.noise);
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
@@ -333,7 +343,7 @@ int Net::refresh_colscale(size_t li, bool *active)
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
     *active = false;
-    if (l.type_dropout == MYEA_DROPOUT_NONE || !o.colscale) return MYEA_OK;
+    if (!layer_uses_mask_dropout(l) || !o.colscale) return MYEA_OK;
     const size_t n = (size_t)d.number_recurrent_depth * o.AH;
     if (state == MYEA_STATE_TRAINING) {
         float on = 1.f;
@@ -394,6 +404,14 @@ int Net::forward_fc_layer(size_t li, size_t B)
         if (norm && !before) {
             MYEA_TRY(bn_forward(li, c, rows, o.values + roff * H, training));
             if (cs) MYEA_TRY(launch_colscale(stream, rows, H, o.normalizes + roff * H, cs));
+        }
+        // Gaussian / Uout dropout on the layer's outputs, strictly in the training state (:716-750)
+        if (o.noise && state == MYEA_STATE_TRAINING) {
+            if (c == 0 && !o.noise_uploaded) {   // fresh draws for the whole sequence, one stream id per (pass, layer)
+                const bool normal = l.type_dropout == MYEA_DROPOUT_GAUSSIAN;
+                MYEA_TRY(launch_dropout_noise(stream, T * Bmax * H, o.noise, normal ? 1 : 0, normal ? 1.f : -l.dropout_values[0], l.dropout_values[0], dropout_seed, dropout_stream++));
+            }
+            MYEA_TRY(launch_dropout_noise_apply(stream, rows * H, ((norm && !before) ? o.normalizes : o.values) + roff * H, o.noise + roff * H, l.type_dropout == MYEA_DROPOUT_UOUT));
         }
         // k-Sparse, after the dropout (NN/Neural_Network__Forward_Pass__Loop.cpp:752-790): k values stay strictly in the
         // training state, size_t(alpha k) otherwise
@@ -1221,6 +1239,26 @@ int myea_hip_upload_zoneout_masks(myea_hip_net *n, const uint8_t *m, size_t c)
     MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
     return MYEA_OK;
 }
+int myea_hip_set_dropout_seed(myea_hip_net *n, uint64_t seed)
+{
+    NET_OR_FAIL(n);
+    n->net.dropout_seed = seed;
+    n->net.dropout_stream = 0;
+    return MYEA_OK;
+}
+int myea_hip_upload_dropout_noise(myea_hip_net *n, size_t li, const float *noise, size_t count, int on_device)
+{
+    NET_OR_FAIL(n);
+    if (li >= n->net.d.n_layers || !n->net.L[li].noise) { myea::set_last_error("upload_dropout_noise: layer %zu has no Gaussian / Uout dropout", li); return MYEA_E_INVALID; }
+    myea::DevLayer &o = n->net.L[li];
+    if (!noise && count == 0) { o.noise_uploaded = false; return MYEA_OK; }   // back to the device generator
+    const size_t want = (size_t)n->net.d.number_recurrent_depth * n->net.d.batch_size * o.H;
+    if (!noise || count != want) { myea::set_last_error("upload_dropout_noise: null or count %zu != %zu (T x batch_size x width)", count, want); return MYEA_E_INVALID; }
+    MYEA_HIP_TRY(hipMemcpyAsync(o.noise, noise, count * sizeof(float), on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, n->net.stream));
+    MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
+    o.noise_uploaded = true;
+    return MYEA_OK;
+}
 int myea_hip_clear_training_arrays(myea_hip_net *n)
 {
     NET_OR_FAIL(n);
@@ -1304,6 +1342,7 @@ int myea_hip_download_tensor(myea_hip_net *n, size_t li, int kind, float *host, 
     case MYEA_TENSOR_SUMMATIONS: p = o.summations; break;
     case MYEA_TENSOR_ERRORS: p = o.neuron_errors; break;
     case MYEA_TENSOR_NORM_HATS: p = o.hats; c = T * n->net.d.batch_size * o.NH; break;
+    case MYEA_TENSOR_DROPOUT_NOISE: p = o.noise; break;
     case MYEA_TENSOR_INPUT_SIDE_ERRORS:
         if (o.group == 2) p = n->net.L[li - 1].neuron_errors;
         else if (o.group == 1) p = o.in_errors;

@@ -71,6 +71,9 @@ typedef struct olayer {
     /* independently recurrent layer: AF_Ind_recurrent_unit::ptr_array_pre_AFs and ::ptr_array_dAFs [T][Bmax][H]
      * (its ptr_array_AFs are `values`, its ptr_array_errors `af_errors`) */
     float *pre_afs, *dafs;
+    /* Gaussian / Uout dropout: the draws of the forward pass [T][Bmax][H], supplied by the test (the reference draws them from
+     * its host generators inside the pass); all-neutral after create */
+    float *noise;
 } olayer;
 
 struct myea_oracle_net {
@@ -341,6 +344,11 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
             o->neuron_errors = zalloc(sz);
         }
         if (is_ind_rnn(l)) { o->pre_afs = zalloc(sz); o->dafs = zalloc(sz); }
+        if (l->type_dropout == MYEA_DROPOUT_GAUSSIAN || l->type_dropout == MYEA_DROPOUT_UOUT) {
+            if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED || o->group) { free(n); return MYEA_E_UNSUPPORTED; }
+            o->noise = zalloc(sz);
+            if (l->type_dropout == MYEA_DROPOUT_GAUSSIAN) for (size_t i = 0; i < sz; ++i) o->noise[i] = 1.f;
+        }
         if (layer_uses_norm(l)) {
             size_t sn = T * B * o->NH, tn = T * o->NH;
             o->hats = zalloc(sn);
@@ -373,7 +381,7 @@ int myea_oracle_destroy(myea_oracle_net *n)
         free(o->neuron_errors); free(o->af_errors); free(o->norm_errors);
         free(o->means); free(o->variances); free(o->means_averages); free(o->variances_averages);
         free(o->r_corrections); free(o->d_corrections); free(o->derivatives_means); free(o->derivatives_variances);
-        free(o->pool_index); free(o->pre_afs); free(o->dafs);
+        free(o->pool_index); free(o->pre_afs); free(o->dafs); free(o->noise);
         free(o->unit_af); free(o->unit_steep);
         if (o->lstm) {
             for (int dir = 0; dir < 2; ++dir) {
@@ -412,6 +420,12 @@ int myea_oracle_set_threads(myea_oracle_net *n, int t) { if (!n || t < 1) return
 float *myea_oracle_parameters(myea_oracle_net *n) { return n->parameters; }
 float *myea_oracle_gradient(myea_oracle_net *n) { return n->gradient; }
 float *myea_oracle_optimizer_state(myea_oracle_net *n, int k) { return (k >= 0 && k < MYEA_STATE_KINDS) ? n->opt[k] : NULL; }
+float *myea_oracle_dropout_noise(myea_oracle_net *n, size_t li, size_t *count)
+{
+    if (!n || li >= n->d.n_layers || !n->L[li].noise) { if (count) *count = 0; return NULL; }
+    if (count) *count = (size_t)n->d.number_recurrent_depth * n->d.batch_size * n->L[li].H;
+    return n->L[li].noise;
+}
 uint8_t *myea_oracle_zoneout_masks(myea_oracle_net *n, size_t *count) { if (count) *count = n->zoneout_count; return n->zoneout; }
 uint8_t *myea_oracle_masks(myea_oracle_net *n) { return n->masks; }
 
@@ -543,6 +557,7 @@ static void fwd_af(myea_oracle_net *n, size_t t, size_t B, size_t H, uint32_t ty
 static void fwd_dropout(myea_oracle_net *n, const myea_layer_desc *l, size_t t, size_t B, size_t H, float *v)
 {
     size_t off = n->d.batch_size * H * t;
+    const float *li_noise = n->L[l - n->d.layers].noise;
     const uint8_t *m = n->masks + l->first_mask_index + t * H;
     if (n->state == MYEA_STATE_TRAINING) {
         if (l->type_dropout == MYEA_DROPOUT_BERNOULLI) {
@@ -556,6 +571,18 @@ static void fwd_dropout(myea_oracle_net *n, const myea_layer_desc *l, size_t t, 
     } else if (l->type_dropout == MYEA_DROPOUT_BERNOULLI) {
         for (size_t b = 0; b < B; ++b)
             for (size_t j = 0; j < H; ++j) v[off + b * H + j] *= l->dropout_values[0];
+    }
+    /* Forward_Pass__Dropout__Gaussian (NN/Neural_Network__Forward_Pass__Loop.cpp:4993-5014): v *= N(1, dropout_values[0]);
+     * Forward_Pass__Dropout__Uout (:5047-5068): v += v * U(-dropout_values[0], +dropout_values[0]); strictly in the training
+     * state, one draw per (example, unit), example-major - here read from the supplied tensor */
+    if (n->state == MYEA_STATE_TRAINING && li_noise) {
+        if (l->type_dropout == MYEA_DROPOUT_GAUSSIAN) {
+            for (size_t b = 0; b < B; ++b)
+                for (size_t j = 0; j < H; ++j) v[off + b * H + j] *= li_noise[off + b * H + j];
+        } else if (l->type_dropout == MYEA_DROPOUT_UOUT) {
+            for (size_t b = 0; b < B; ++b)
+                for (size_t j = 0; j < H; ++j) v[off + b * H + j] += v[off + b * H + j] * li_noise[off + b * H + j];
+        }
     }
 }
 
@@ -1755,6 +1782,7 @@ const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t 
     case MYEA_TENSOR_SUMMATIONS: p = o->summations; break;
     case MYEA_TENSOR_ERRORS: p = (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL || is_pooling(&n->d.layers[li])) ? o->af_errors : o->neuron_errors; break;
     case MYEA_TENSOR_NORM_HATS: p = o->hats; c = T * n->d.batch_size * o->NH; break;
+    case MYEA_TENSOR_DROPOUT_NOISE: p = o->noise; break;
     case MYEA_TENSOR_INPUT_SIDE_ERRORS:
         if (o->group == 2) p = layer_uses_norm(&n->d.layers[li]) ? o->norm_errors : o->af_errors;
         else if (o->group == 1 && layer_uses_norm(&n->d.layers[li])) p = o->norm_errors;

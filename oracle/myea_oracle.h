@@ -32,6 +32,8 @@ float *myea_oracle_gradient(myea_oracle_net *net);
 float *myea_oracle_optimizer_state(myea_oracle_net *net, int kind);
 uint8_t *myea_oracle_masks(myea_oracle_net *net);
 uint8_t *myea_oracle_zoneout_masks(myea_oracle_net *net, size_t *count);
+/* Gaussian / Uout dropout draws of layer `li`, [T][Bmax][H]; NULL when the layer has no such dropout */
+float *myea_oracle_dropout_noise(myea_oracle_net *net, size_t li, size_t *count);
 int myea_oracle_clear_training_arrays(myea_oracle_net *net);
 
 int myea_oracle_forward_pass(myea_oracle_net *net, size_t batch_size_received, const float *inputs);

@@ -39,6 +39,8 @@ def load_oracle():
     lib.myea_oracle_masks.restype = P(C.c_uint8)
     lib.myea_oracle_zoneout_masks.argtypes = [vp, P(sz)]
     lib.myea_oracle_zoneout_masks.restype = P(C.c_uint8)
+    lib.myea_oracle_dropout_noise.argtypes = [vp, sz, P(sz)]
+    lib.myea_oracle_dropout_noise.restype = P(C.c_float)
     lib.myea_oracle_clear_training_arrays.argtypes = [vp]
     lib.myea_oracle_forward_pass.argtypes = [vp, sz, vp]
     lib.myea_oracle_compute_error.argtypes = [vp, sz, vp]
@@ -130,6 +132,13 @@ class OracleNetwork:
     def upload_masks(self, m):
         m = np.asarray(m, dtype=np.uint8)
         self._view(self.lib.myea_oracle_masks(self.handle), self.desc.total_mask_units, np.uint8)[: len(m)] = m
+
+    def upload_dropout_noise(self, layer, noise):
+        n = C.c_size_t()
+        p = self.lib.myea_oracle_dropout_noise(self.handle, layer, C.byref(n))
+        noise = np.asarray(noise, dtype=np.float32).ravel()
+        assert p and len(noise) == n.value, "dropout noise count %d != %d" % (len(noise), n.value)
+        self._view(p, n.value)[:] = noise
 
     def upload_zoneout_masks(self, m):
         m = np.asarray(m, dtype=np.uint8)
