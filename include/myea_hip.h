@@ -72,6 +72,9 @@ enum {
 enum {
     MYEA_DROPOUT_NONE = 0, MYEA_DROPOUT_BERNOULLI = 2, MYEA_DROPOUT_BERNOULLI_INVERTED = 3,
     MYEA_DROPOUT_GAUSSIAN = 4, /* training state: y *= N(1, dropout_values[0]) per (example, unit); dropout_values[0] = p / (1 - p) */
+    MYEA_DROPOUT_SHAKEDROP = 5, /* residual layers only: with probability dropout_values[0] an example's block output is multiplied,
+                                  * value by value, by U(-1, 1) draws going forward and its delta by U(0, 1) draws going back;
+                                  * outside the training state the block output is scaled by 1 - dropout_values[0] */
     MYEA_DROPOUT_UOUT = 6,     /* training state: y += y * U(-dropout_values[0], dropout_values[0]) per (example, unit) */
     MYEA_DROPOUT_ZONEOUT = 7   /* LSTM layers only: dropout_values[0] / [1] = zoneout probability of the cell state / the cell output */
 };
@@ -346,7 +349,11 @@ int myea_hip_upload_zoneout_masks(myea_hip_net *net, const uint8_t *host_masks, 
  *  - myea_hip_upload_dropout_noise(): the caller's own draws for one layer, [T][Bmax][H] floats (`count` = T x batch_size x
  *    width), used by every following forward pass until the call is repeated with NULL / 0.  A caller that draws with the
  *    reference's generators in the reference's order gets the reference's numbers.
- * Either way MYEA_TENSOR_DROPOUT_NOISE reads back what the last forward pass used. */
+ * Either way MYEA_TENSOR_DROPOUT_NOISE reads back what the last forward pass used.
+ * ShakeDrop on a residual layer (Forward_Pass__Dropout__ShakeDrop :5016-5045, Backward_Pass__Dropout__ShakeDrop
+ * Neural_Network__Backward_Pass__Loop.cpp:1050-1078) uses the same two sources; its tensor is
+ * [batch_size masks as 0 / 1][batch_size x width forward draws][batch_size x width backward draws] with `width` the block's
+ * last layer's, `count` = batch_size x (1 + 2 x width).  The device generator draws all three in the forward pass. */
 int myea_hip_set_dropout_seed(myea_hip_net *net, uint64_t seed);
 int myea_hip_upload_dropout_noise(myea_hip_net *net, size_t layer_index, const float *noise, size_t count, int noise_on_device);
 /* Clear_Training_Arrays (Train.cpp:93-126) + Clear_Optimizer (Train.cpp:128-263): zero the gradient

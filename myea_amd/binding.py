@@ -25,7 +25,7 @@ AF = dict(NONE=0, COSINE=1, COSINE_SYMMETRIC=2, ELU=3, ELLIOT=4, ELLIOT_SYMMETRI
           SINE=19, SIGMOID_STEPWISE=20, SINE_SYMMETRIC=21, SOFTMAX=22, TANH=23, TANH_STEPWISE=24,
           THRESHOLD=25, THRESHOLD_SYMMETRIC=26)
 OPTIMIZER = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP_PLUS=8, NOSADAM=9)
-DROPOUT = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3, GAUSSIAN=4, UOUT=6, ZONEOUT=7)
+DROPOUT = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3, GAUSSIAN=4, SHAKEDROP=5, UOUT=6, ZONEOUT=7)
 NORMALIZATION = dict(NONE=0, BATCH_NORMALIZATION=1, BATCH_RENORMALIZATION=2)
 LOSS = dict(NONE=0, BIT=1, CROSS_ENTROPY=2, L1=3, L2=4, MAE=5, MAPE=6, ME=9, MSE=10, RMSE=11, SMAPE=12)
 ACCURACY = dict(NONE=0, CROSS_ENTROPY=1, DIRECTIONAL=2, DISTANCE=3, R=4, SIGN=5)

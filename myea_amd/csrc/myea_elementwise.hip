@@ -175,6 +175,24 @@ __global__ __launch_bounds__(kBlock) void dropout_noise_apply_kernel(size_t n, f
     }
 }
 
+// ShakeDrop (Forward_Pass__Dropout__ShakeDrop NN/Neural_Network__Forward_Pass__Loop.cpp:5016-5045, Backward_Pass__Dropout__ShakeDrop
+// NN/Neural_Network__Backward_Pass__Loop.cpp:1050-1078): rows whose mask is set are multiplied value by value by their draws;
+// without a mask every value is multiplied by `constant` (the inference scaling).
+__global__ __launch_bounds__(kBlock) void shakedrop_apply_kernel(size_t rows, size_t W, float *x, const float *mask, const float *draws, float constant)
+{
+    const size_t n = rows * W;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        if (!mask) x[i] *= constant;
+        else if (mask[i / W] != 0.f) x[i] *= draws[i];
+    }
+}
+
+// uniform draws in [0, 1) to a Bernoulli(p) mask held as 0 / 1
+__global__ __launch_bounds__(kBlock) void threshold_kernel(size_t n, float *x, float p)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) x[i] = x[i] < p ? 1.f : 0.f;
+}
+
 // Sparse_K_Filter (NN/Neural_Network__K_Sparse.cpp:268-339): per row the k largest values stay, the others become 0; among
 // equal values at the cut the lower indices stay.  One workgroup per row: a 4-pass radix select over order-preserving keys
 // finds the k-th largest key and how many entries equal to it stay, then one ordered pass writes the zeros.
@@ -816,6 +834,22 @@ int launch_dropout_noise_apply(hipStream_t s, size_t n, float *y, const float *n
 {
     if (n == 0) return MYEA_OK;
     hipLaunchKernelGGL(dropout_noise_apply_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, n, y, noise, uout);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_shakedrop_apply(hipStream_t s, size_t rows, size_t W, float *x, const float *mask, const float *draws, float constant)
+{
+    if (rows * W == 0) return MYEA_OK;
+    hipLaunchKernelGGL(shakedrop_apply_kernel, dim3(grid_for(rows * W, kBlock)), dim3(kBlock), 0, s, rows, W, x, mask, draws, constant);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_threshold(hipStream_t s, size_t n, float *x, float p)
+{
+    if (n == 0) return MYEA_OK;
+    hipLaunchKernelGGL(threshold_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, n, x, p);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

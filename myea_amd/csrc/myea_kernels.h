@@ -130,6 +130,11 @@ int launch_dropout_noise(hipStream_t s, size_t n, float *noise, int normal, floa
 // y *= noise (Gaussian) or y += y * noise (Uout)
 int launch_dropout_noise_apply(hipStream_t s, size_t n, float *y, const float *noise, int uout);
 
+// ShakeDrop: x[r][j] *= draws[r][j] where mask[r] is set; with a null mask x *= constant
+int launch_shakedrop_apply(hipStream_t s, size_t rows, size_t W, float *x, const float *mask, const float *draws, float constant);
+// x[i] = x[i] < p ? 1 : 0
+int launch_threshold(hipStream_t s, size_t n, float *x, float p);
+
 // per row of x [rows][H]: the k largest values stay, the others become 0 (ties at the cut: the lower indices stay)
 int launch_k_sparse(hipStream_t s, size_t rows, size_t H, size_t k, float *x);
 

@@ -145,7 +145,8 @@ static int check_desc(const myea_net_desc &d)
             if (li == block_end) block_end = 0;
         } else if (l.type_layer == MYEA_LAYER_RESIDUAL) {
             if (l.block_depth == 0 || (uint64_t)li + l.block_depth + 1 >= d.n_layers) { set_last_error("layer %u: residual block of depth %u does not fit in front of a consumer", li, l.block_depth); return MYEA_E_INVALID; }
-            if (l.type_dropout != MYEA_DROPOUT_NONE) { set_last_error("layer %u: block-level dropout (ShakeDrop) is not on this path", li); return MYEA_E_UNSUPPORTED; }
+            if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_SHAKEDROP) { set_last_error("layer %u: a residual layer's dropout is ShakeDrop or none", li); return MYEA_E_UNSUPPORTED; }
+            if (l.type_dropout == MYEA_DROPOUT_SHAKEDROP && !(l.dropout_values[0] >= 0.f && l.dropout_values[0] <= 1.f)) { set_last_error("layer %u: ShakeDrop probability %g", li, (double)l.dropout_values[0]); return MYEA_E_INVALID; }
             any_residual = true;
             block_end = li + l.block_depth;
         }
@@ -247,6 +248,10 @@ int Net::create(const myea_net_desc &desc)
         MYEA_TRY(dev_alloc(&o.values, sa));
         MYEA_HIP_TRY(hipMemset(o.values, 0, (sa ? sa : 1) * sizeof(float)));
         if (layer_uses_mask_dropout(l) && layer_is_dense(l)) MYEA_TRY(dev_alloc(&o.colscale, T * o.AH));
+        if (l.type_layer == MYEA_LAYER_RESIDUAL && l.type_dropout == MYEA_DROPOUT_SHAKEDROP) {   // [masks][forward draws][backward draws]
+            MYEA_TRY(dev_alloc(&o.noise, B + 2 * B * o.NH));
+            MYEA_HIP_TRY(hipMemset(o.noise, 0, (B + 2 * B * o.NH) * sizeof(float)));
+        }
         if (layer_uses_noise_dropout(l)) {
             MYEA_TRY(dev_alloc(&o.noise, sz));
             MYEA_TRY(launch_fill(0, o.noise, sz, l.type_dropout == MYEA_DROPOUT_GAUSSIAN ? 1.f : 0.f));   // neutral until a pass draws
@@ -579,6 +584,22 @@ int Net::forward_residual_block(size_t ri, size_t B)
         MYEA_TRY(bn_forward(ri, 0, B, blk, training));
         blk = o.normalizes;
     }
+    // ShakeDrop on the block's output, in place (NN/Neural_Network__Forward_Pass__Loop.cpp:4053-4078)
+    if (r.type_dropout == MYEA_DROPOUT_SHAKEDROP) {
+        const size_t Bmax = d.batch_size, W = o.NH;
+        float *out = const_cast<float *>(blk);
+        if (state == MYEA_STATE_TRAINING) {
+            if (!o.noise_uploaded) {   // masks, forward and backward draws of this pass
+                MYEA_TRY(launch_dropout_noise(stream, Bmax, o.noise, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
+                MYEA_TRY(launch_threshold(stream, Bmax, o.noise, r.dropout_values[0]));
+                MYEA_TRY(launch_dropout_noise(stream, Bmax * W, o.noise + Bmax, 0, -1.f, 1.f, dropout_seed, dropout_stream++));
+                MYEA_TRY(launch_dropout_noise(stream, Bmax * W, o.noise + Bmax + Bmax * W, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
+            }
+            MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, o.noise, o.noise + Bmax, 1.f));
+        } else {
+            MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, nullptr, nullptr, 1.f - r.dropout_values[0]));
+        }
+    }
     const float *src = layer_outputs(o.prev);
     const size_t na = o.In, nb = o.NH;
     if (na >= nb) return launch_padded_add(stream, B, o.H, src, na, 0, blk, nb, -(long)o.pad, o.values);
@@ -796,11 +817,16 @@ int Net::backward_residual_block(size_t ri, size_t B)
     DevLayer &ro = L[ri];
     const size_t last = ri + r.block_depth;
     const long crop = ro.H > ro.NH ? (long)ro.pad : 0;
+    // the perturbed examples' deltas times the backward draws (NN/Neural_Network__Backward_Pass__Loop.cpp:433-443)
+    const bool shake = r.type_dropout == MYEA_DROPOUT_SHAKEDROP;
+    const float *beta = shake ? ro.noise + d.batch_size + d.batch_size * ro.NH : nullptr;
     if (layer_uses_norm(r)) {
         MYEA_TRY(launch_padded_add(stream, B, ro.NH, ro.neuron_errors, ro.H, crop, nullptr, 0, 0, tmp1));
+        if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, tmp1, ro.noise, beta, 1.f));
         MYEA_TRY(bn_backward(ri, 0, B, L[last].summations, tmp1, L[last].neuron_errors));
     } else {
         MYEA_TRY(launch_padded_add(stream, B, ro.NH, ro.neuron_errors, ro.H, crop, nullptr, 0, 0, L[last].neuron_errors));
+        if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, L[last].neuron_errors, ro.noise, beta, 1.f));
     }
     for (size_t m = last; m > ri; --m) {
         const myea_layer_desc &l = d.layers[m];
@@ -1252,8 +1278,9 @@ int myea_hip_upload_dropout_noise(myea_hip_net *n, size_t li, const float *noise
     if (li >= n->net.d.n_layers || !n->net.L[li].noise) { myea::set_last_error("upload_dropout_noise: layer %zu has no Gaussian / Uout dropout", li); return MYEA_E_INVALID; }
     myea::DevLayer &o = n->net.L[li];
     if (!noise && count == 0) { o.noise_uploaded = false; return MYEA_OK; }   // back to the device generator
-    const size_t want = (size_t)n->net.d.number_recurrent_depth * n->net.d.batch_size * o.H;
-    if (!noise || count != want) { myea::set_last_error("upload_dropout_noise: null or count %zu != %zu (T x batch_size x width)", count, want); return MYEA_E_INVALID; }
+    const bool shake = n->net.d.layers[li].type_layer == MYEA_LAYER_RESIDUAL;
+    const size_t want = shake ? (size_t)n->net.d.batch_size * (1 + 2 * o.NH) : (size_t)n->net.d.number_recurrent_depth * n->net.d.batch_size * o.H;
+    if (!noise || count != want) { myea::set_last_error("upload_dropout_noise: null or count %zu != %zu (%s)", count, want, shake ? "batch_size x (1 + 2 x block width)" : "T x batch_size x width"); return MYEA_E_INVALID; }
     MYEA_HIP_TRY(hipMemcpyAsync(o.noise, noise, count * sizeof(float), on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, n->net.stream));
     MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
     o.noise_uploaded = true;
@@ -1342,7 +1369,7 @@ int myea_hip_download_tensor(myea_hip_net *n, size_t li, int kind, float *host, 
     case MYEA_TENSOR_SUMMATIONS: p = o.summations; break;
     case MYEA_TENSOR_ERRORS: p = o.neuron_errors; break;
     case MYEA_TENSOR_NORM_HATS: p = o.hats; c = T * n->net.d.batch_size * o.NH; break;
-    case MYEA_TENSOR_DROPOUT_NOISE: p = o.noise; break;
+    case MYEA_TENSOR_DROPOUT_NOISE: p = o.noise; if (n->net.d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) c = n->net.d.batch_size * (1 + 2 * o.NH); break;
     case MYEA_TENSOR_INPUT_SIDE_ERRORS:
         if (o.group == 2) p = n->net.L[li - 1].neuron_errors;
         else if (o.group == 1) p = o.in_errors;

@@ -267,7 +267,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
                 if (block != 0) { o->group = seen == 0 ? 1 : 2; ++seen; }
             }
             if (l->type_layer == MYEA_LAYER_RESIDUAL) {
-                if (block != 0 || T != 1 || l->block_depth == 0 || li + l->block_depth + 1 >= desc->n_layers || l->type_dropout != MYEA_DROPOUT_NONE) { free(n); return MYEA_E_UNSUPPORTED; }
+                if (block != 0 || T != 1 || l->block_depth == 0 || li + l->block_depth + 1 >= desc->n_layers || (l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_SHAKEDROP)) { free(n); return MYEA_E_UNSUPPORTED; }
                 block = li; seen = 0;
             }
         }
@@ -344,6 +344,8 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
             o->neuron_errors = zalloc(sz);
         }
         if (is_ind_rnn(l)) { o->pre_afs = zalloc(sz); o->dafs = zalloc(sz); }
+        if (l->type_layer == MYEA_LAYER_RESIDUAL && l->type_dropout == MYEA_DROPOUT_SHAKEDROP) o->noise = zalloc(B + 2 * B * o->NH);   /* all masks false */
+        if (l->type_layer != MYEA_LAYER_RESIDUAL && l->type_dropout == MYEA_DROPOUT_SHAKEDROP) { free(n); return MYEA_E_UNSUPPORTED; }
         if (l->type_dropout == MYEA_DROPOUT_GAUSSIAN || l->type_dropout == MYEA_DROPOUT_UOUT) {
             if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED || o->group) { free(n); return MYEA_E_UNSUPPORTED; }
             o->noise = zalloc(sz);
@@ -423,6 +425,7 @@ float *myea_oracle_optimizer_state(myea_oracle_net *n, int k) { return (k >= 0 &
 float *myea_oracle_dropout_noise(myea_oracle_net *n, size_t li, size_t *count)
 {
     if (!n || li >= n->d.n_layers || !n->L[li].noise) { if (count) *count = 0; return NULL; }
+    if (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) { if (count) *count = (size_t)n->d.batch_size * (1 + 2 * n->L[li].NH); return n->L[li].noise; }
     if (count) *count = (size_t)n->d.number_recurrent_depth * n->d.batch_size * n->L[li].H;
     return n->L[li].noise;
 }
@@ -704,15 +707,27 @@ static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t B)
 {
     const myea_layer_desc *r = &n->d.layers[ri];
     olayer *o = &n->L[ri];
-    size_t last = ri + r->block_depth, Bmax = n->d.batch_size; (void)Bmax;
+    size_t last = ri + r->block_depth, Bmax = n->d.batch_size;
     for (size_t li = ri + 1; li <= last; ++li) fwd_residual_fc_layer(n, li, B);
-    const float *blk = layer_outputs(n, last);
+    float *blk = layer_outputs(n, last);
     size_t nb = n->L[last].H, na = n->L[o->prev].H;
     if (layer_uses_norm(r)) {
         int renorm = r->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
         if (n->state >= MYEA_STATE_TRAINING) fwd_bn_training(n, renorm, 0, B, nb, blk, scale_ptr(n, n->parameters, ri), shift_ptr(n, n->parameters, ri), o);
         else fwd_bn_inference(n, 0, B, nb, blk, scale_ptr(n, n->parameters, ri), shift_ptr(n, n->parameters, ri), o);
         blk = o->normalizes;
+    }
+    /* ShakeDrop on the block's output, in place (Forward_Pass__Residual__Block, NN/Neural_Network__Forward_Pass__Loop.cpp:4053-4078;
+     * Forward_Pass__Dropout__ShakeDrop :5016-5045): strictly in the training state an example is perturbed with probability
+     * dropout_values[0], each of its values then times its own U(-1, 1) draw; otherwise every value times 1 - dropout_values[0].
+     * Draws as supplied: [mask per example][forward draws][backward draws]. */
+    if (r->type_dropout == MYEA_DROPOUT_SHAKEDROP) {
+        const float *mask = o->noise, *alpha = o->noise + Bmax;
+        for (size_t b = 0; b < B; ++b)
+            for (size_t j = 0; j < nb; ++j) {
+                if (n->state == MYEA_STATE_TRAINING) { if (mask[b] != 0.f) blk[b * nb + j] *= alpha[b * nb + j]; }
+                else blk[b * nb + j] *= 1.f - r->dropout_values[0];
+            }
     }
     const float *a = layer_outputs(n, o->prev);
     for (size_t b = 0; b < B; ++b) {
@@ -1424,6 +1439,14 @@ static void bwd_residual_block_to_last(myea_oracle_net *n, size_t ri, size_t B, 
     float *tmp = dst;
     if (layer_uses_norm(r)) { tmp = o->norm_errors; memset(tmp, 0, Bmax * D * sizeof(float)); }
     bwd_residual_shortcut(n, B, o->H, D, o->pad, o->af_errors, tmp);
+    /* Backward_Pass__Dropout__ShakeDrop (NN/Neural_Network__Backward_Pass__Loop.cpp:433-443, 1050-1078): the perturbed examples'
+     * deltas times fresh U(0, 1) draws, one per value */
+    if (r->type_dropout == MYEA_DROPOUT_SHAKEDROP) {
+        const float *mask = o->noise, *beta = o->noise + Bmax + Bmax * D;
+        for (size_t b = 0; b < B; ++b)
+            if (mask[b] != 0.f)
+                for (size_t j = 0; j < D; ++j) tmp[b * D + j] *= beta[b * D + j];
+    }
     if (layer_uses_norm(r)) {
         int renorm = r->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
         bwd_bn(n, renorm, ri, 0, B, D, layer_outputs(n, ri + r->block_depth), tmp, o->norm_errors);
@@ -1782,7 +1805,7 @@ const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t 
     case MYEA_TENSOR_SUMMATIONS: p = o->summations; break;
     case MYEA_TENSOR_ERRORS: p = (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL || is_pooling(&n->d.layers[li])) ? o->af_errors : o->neuron_errors; break;
     case MYEA_TENSOR_NORM_HATS: p = o->hats; c = T * n->d.batch_size * o->NH; break;
-    case MYEA_TENSOR_DROPOUT_NOISE: p = o->noise; break;
+    case MYEA_TENSOR_DROPOUT_NOISE: p = o->noise; if (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) c = n->d.batch_size * (1 + 2 * o->NH); break;
     case MYEA_TENSOR_INPUT_SIDE_ERRORS:
         if (o->group == 2) p = layer_uses_norm(&n->d.layers[li]) ? o->norm_errors : o->af_errors;
         else if (o->group == 1 && layer_uses_norm(&n->d.layers[li])) p = o->norm_errors;
