@@ -418,6 +418,11 @@ int myea_hip_get_loss(myea_hip_net *net, myea_loss_state *out_state);
 int myea_hip_download_gradient(myea_hip_net *net, float *host_gradient, size_t count);
 int myea_hip_upload_gradient(myea_hip_net *net, const float *host_gradient, size_t count);
 int myea_hip_download_tensor(myea_hip_net *net, size_t layer_index, int kind, float *host, size_t count);
+/* The running statistics of a normalised layer are network state that outlives a training run (the reference keeps them in
+ * Normalized_unit::ptr_mean_average / ptr_variance_average and writes them into its dimension file, Neural_Network__Save.cpp:678-712).
+ * `kind` = MYEA_TENSOR_NORM_MEANS_AVERAGES or MYEA_TENSOR_NORM_VARIANCES_AVERAGES, `count` = T x the layer's normalised units,
+ * [T][units] as myea_hip_download_tensor returns them. */
+int myea_hip_upload_tensor(myea_hip_net *net, size_t layer_index, int kind, const float *host, size_t count);
 
 /* ---- profiling taps for the benchmark ---- */
 /* When enabled, every dense-contraction (GEMM) launch is bracketed by HIP events on the net's stream;

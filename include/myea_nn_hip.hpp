@@ -14,6 +14,7 @@
 #include <cfloat>
 #include <cmath>
 #include <cstring>
+#include <string>
 #include <vector>
 
 #include "myea_hip.h"
@@ -49,6 +50,8 @@ public:
     T_ optimizer_time_step = 0.f, epoch_time_step = 1.f, adam_previous_beta2 = 0.f;
     T_ loss_rprop = FLT_MAX, previous_loss_rprop = FLT_MAX;
     T_ warm_restarts_maximum_learning_rate = 1.f, warm_restarts_T_i = 1.f;
+    // the values a warm-restart schedule starts from; these are what the checkpoint keeps (Neural_Network__Save.cpp:85-88)
+    T_ warm_restarts_initial_maximum_learning_rate = 1.f, warm_restarts_initial_T_i = 1.f;
     unsigned int type_optimizer_function = MYEA_OPTIMIZER_NONE, type_loss_function = MYEA_LOSS_NONE;
     unsigned int type_accuracy_function = MYEA_ACCURACY_DISTANCE;
     unsigned int type_state_propagation = MYEA_STATE_INFERENCE;
@@ -245,8 +248,21 @@ public:
         if (!use_hip) { if (net_) { myea_hip_destroy(net_); net_ = nullptr; } return true; }
         if (net_) { myea_hip_destroy(net_); net_ = nullptr; }
         if (myea_hip_create(&desc_, &net_) != MYEA_OK) return Fail("Set__HIP", myea_hip_last_error());
+        // running statistics a checkpoint brought along (Load)
+        for (size_t li = 0; li < norm_means_averages_.size() && li < desc_.n_layers; ++li) {
+            if (norm_means_averages_[li].empty()) continue;
+            if (!Ok("Set__HIP", myea_hip_upload_tensor(net_, li, MYEA_TENSOR_NORM_MEANS_AVERAGES, norm_means_averages_[li].data(), norm_means_averages_[li].size())) ||
+                !Ok("Set__HIP", myea_hip_upload_tensor(net_, li, MYEA_TENSOR_NORM_VARIANCES_AVERAGES, norm_variances_averages_[li].data(), norm_variances_averages_[li].size()))) return false;
+        }
         return Copy__Parameters__Host_To_Device() && Copy__Dropout_Mask__Host_To_Device();
     }
+    // The reference's checkpoint: Save_General_Parameters / Save_Dimension_Parameters (Neural_Network__Save.cpp:23-624) write the
+    // two text files, Load (Neural_Network__Load.cpp:2323) reads them back; see myea_nn_hip_io.hpp.  Saving with a device object
+    // first pulls the parameters and the normalisation running statistics from the device; after Load the caller picks the batch
+    // size (Update__Batch_Size) and calls Set__HIP(true).
+    bool Save_General_Parameters(std::string const &path);
+    bool Save_Dimension_Parameters(std::string const &path);
+    bool Load(std::string const &path_dimension, std::string const &path_parameters, size_t maximum_allowable_memory = 0);
     bool Use__HIP() const { return net_ != nullptr; }
 
     // Data.hpp:3119-3189
@@ -407,6 +423,7 @@ private:
     myea_net_desc desc_;
     myea_hip_net *net_ = nullptr;
     std::vector<T_> rows_;
+    std::vector<std::vector<T_>> norm_means_averages_, norm_variances_averages_;   // per layer [T][units], from a checkpoint
     T_ r_mean_desired_ = 0.f, r_mean_predicted_ = 0.f;
 
     static bool Fail(const char *fn, const char *what) { std::printf("%s: ERROR: %s.\n", fn, what); return false; }
@@ -424,6 +441,7 @@ private:
         if (net_) { myea_hip_destroy(net_); net_ = nullptr; }
         delete[] ptr_array_parameters; ptr_array_parameters = nullptr;
         delete[] ptr_array_units_mask_dropout_bernoulli; ptr_array_units_mask_dropout_bernoulli = nullptr;
+        norm_means_averages_.clear(); norm_variances_averages_.clear();
     }
     bool Relayout(const char *fn)
     {
@@ -487,3 +505,6 @@ private:
 };
 
 }  // namespace MyEA_HIP
+
+#include "myea_nn_hip_io.hpp"
+

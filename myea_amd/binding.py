@@ -102,7 +102,7 @@ ABI_SYMBOLS = [
     "myea_hip_upload_zoneout_masks", "myea_hip_set_dropout_seed", "myea_hip_upload_dropout_noise", "myea_hip_compute_loss", "myea_hip_compute_accuracy_r", "myea_hip_gather_examples", "myea_hip_device_buffer_create", "myea_hip_device_buffer_destroy",
     "myea_hip_clear_training_arrays", "myea_hip_forward_pass", "myea_hip_compute_error", "myea_hip_backward_pass",
     "myea_hip_update_derivative_weight", "myea_hip_update_parameter", "myea_hip_reset_loss", "myea_hip_get_loss",
-    "myea_hip_download_gradient", "myea_hip_upload_gradient", "myea_hip_download_tensor",
+    "myea_hip_download_gradient", "myea_hip_upload_gradient", "myea_hip_download_tensor", "myea_hip_upload_tensor",
     "myea_hip_profile_enable", "myea_hip_profile_read", "myea_hip_gemm_f32", "myea_hip_optimizer_update",
 ]
 
@@ -158,6 +158,7 @@ def load_library(path=LIB_PATH):
     lib.myea_hip_device_buffer_create.argtypes = [sz, vp, P(vp)]
     lib.myea_hip_device_buffer_destroy.argtypes = [vp]
     lib.myea_hip_download_tensor.argtypes = [vp, sz, i32, vp, sz]
+    lib.myea_hip_upload_tensor.argtypes = [vp, sz, i32, vp, sz]
     lib.myea_hip_profile_enable.argtypes = [vp, i32]
     lib.myea_hip_profile_read.argtypes = [vp, i32, P(C.c_uint64), P(C.c_double), P(C.c_double)]
     lib.myea_hip_gemm_f32.argtypes = [vp, i32, i32, i32, sz, sz, sz, vp, sz, vp, sz, vp, sz]
@@ -338,6 +339,11 @@ class HipNetwork:
         out = np.empty(count, dtype=np.float32)
         self._check(self.lib.myea_hip_download_tensor(self.handle, layer, kind, _ptr(out), out.size))
         return out
+
+    def upload_tensor(self, layer, kind, values):
+        """running means / variances of a normalised layer, [T][units]"""
+        v = np.ascontiguousarray(values, dtype=np.float32)
+        self._check(self.lib.myea_hip_upload_tensor(self.handle, layer, kind, _ptr(v), v.size))
 
     def set_dropout_seed(self, seed):
         self._check(self.lib.myea_hip_set_dropout_seed(self.handle, seed))

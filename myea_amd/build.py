@@ -42,7 +42,7 @@ def build(verbose=False):
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
     # the C++ adaptor's check programs (host code only; link the C ABI)
     root = os.path.dirname(HERE)
-    for name in ("adaptor_check", "dataset_check"):
+    for name in ("adaptor_check", "dataset_check", "checkpoint_check"):
         _run(["g++", "-O2", "-std=c++17", "-Wall", os.path.join(root, "tests", "cpp", name + ".cpp"), "-o",
               os.path.join(root, "tests", "cpp", name), "-L" + CSRC, "-lmyea_hip", "-Wl,-rpath," + CSRC,
               "-Wl,-rpath,$ORIGIN/../../myea_amd/csrc"])
