@@ -326,6 +326,15 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
     __syncthreads();
 
     int cur = 0;   // stage holding step kt
+    // Fragments are double buffered in registers: the LDS reads of group g + 1 are in flight while the MFMAs of group g
+    // issue.  The barrier that publishes the next stage sits in front of the LAST group of a step - its fragments are
+    // already in registers by then - so the first fragments of the next step are read behind that group's MFMAs
+    // instead of in front of an idle matrix pipe.
+    f32x4 fa[2][TM], fb[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[0][i] = PA::frag(smem, wave_m + i * 32, 0, lane32, half);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[0][j] = PB::frag(smem + PA::kFloats, wave_n + j * 32, 0, lane32, half);
     for (int kt = 0; kt < nk; ++kt) {
         const int ahead = NS - 1;                       // how many steps ahead the fill runs
         const bool more = kt + ahead < nk;
@@ -336,13 +345,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
             moveB.fill(next + PA::kFloats, k_begin + (kt + ahead) * kBK, k_end);
         }
         const float *la = smem + cur * kStage, *lb = la + PA::kFloats;
-        // Fragments are double buffered in registers: the LDS reads of group g + 1 are in flight while the MFMAs of
-        // group g issue, so that a wavefront does not sit out the LDS latency between groups.
-        f32x4 fa[2][TM], fb[2][TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fa[0][i] = PA::frag(la, wave_m + i * 32, 0, lane32, half);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) fb[0][j] = PB::frag(lb, wave_n + j * 32, 0, lane32, half);
+        const int following = cur + 1 == NS ? 0 : cur + 1;   // stage of step kt + 1
 #pragma unroll
         for (int g = 0; g < kBK / 8; ++g) {
             const int cb = g & 1, nb = cb ^ 1;
@@ -351,6 +354,22 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
                 for (int i = 0; i < TM; ++i) fa[nb][i] = PA::frag(la, wave_m + i * 32, g + 1, lane32, half);
 #pragma unroll
                 for (int j = 0; j < TN; ++j) fb[nb][j] = PB::frag(lb, wave_n + j * 32, g + 1, lane32, half);
+            } else {
+                if (more) {
+                    moveA.commit(next);
+                    moveB.commit(next + PA::kFloats);
+                }
+                // step kt + 1 must have landed; with three stages the fill of step kt + 2 may stay in flight
+                if (NS == 3 && more) PA::Mover::template wait<kInFlight>();
+                else PA::Mover::template wait<0>();
+                __syncthreads();
+                if (kt + 1 < nk) {
+                    const float *na = smem + following * kStage, *nbp = na + PA::kFloats;
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) fa[nb][i] = PA::frag(na, wave_m + i * 32, 0, lane32, half);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) fb[nb][j] = PB::frag(nbp, wave_n + j * 32, 0, lane32, half);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of this group's MFMAs (the scheduler sinks it otherwise)
 #pragma unroll
@@ -361,14 +380,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
                     for (int j = 0; j < TN; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][i][s], fb[cb][j][s], acc[i][j], 0, 0, 0);
         }
-        if (more) {
-            moveA.commit(next);
-            moveB.commit(next + PA::kFloats);
-        }
-        if (NS == 3 && more) PA::Mover::template wait<kInFlight>();
-        else PA::Mover::template wait<0>();
-        __syncthreads();
-        cur = cur + 1 == NS ? 0 : cur + 1;
+        cur = following;
     }
 
     // Epilogue.  A lane owns one column of each accumulator, so per-column operands are read once.
@@ -396,8 +408,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
                     if (p.aux_out) p.aux_out[o] = af_fire_fused(p.act, v) * cs;
                 } else if (p.epilogue == EPI_FC_DERIVE) {
                     p.C[o] = v * af_derive_fused(p.act, p.pre[o], p.steep, p.val[o]);
+                } else if (p.accumulate) {
+                    // C += v without reading C back: one hardware add per element, performed at the L2.  Every element is
+                    // owned by exactly one lane of one workgroup, so the result is the C + v a load / add / store gives,
+                    // and the epilogue no longer waits for a tile of C to come in.
+                    unsafeAtomicAdd(&p.C[o], v);
                 } else {
-                    if (p.accumulate) v += p.C[o];
                     p.C[o] = v;
                 }
             }
