@@ -420,6 +420,8 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
         prof_end(2.0 * (double)rows * (double)q.G * (double)q.In);
     }
     const LstmGeom geom = geom_of(q);
+    // One pair of timing events brackets the whole time loop: a pair per step costs more than the 10 us steps it would time.
+    if (T > 1) prof_begin(0);
     for (size_t s = 0; s < T; ++s) {
         const size_t t = q.reverse ? T - 1 - s : s, tp = q.reverse ? t + 1 : t - 1;  // tp: the step processed before t
         float *acts_t = q.acts + t * Bmax * q.G;
@@ -434,9 +436,7 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
             f.acts = acts_t; f.c_prev = q.c + tp * Bmax * q.C;
             f.c = q.c + t * Bmax * q.C; f.ca = q.ca + t * Bmax * q.C; f.h = q.h + t * Bmax * q.C;
             f.zone_state = zs; f.zone_output = zo;
-            prof_begin(0);
             MYEA_TRY(launch_lstm_fused_forward(stream, f));
-            prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
             continue;
         }
         if (s > 0) {
@@ -447,15 +447,14 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
             g.M = (int)B; g.N = (int)q.G; g.K = (int)q.C;
             nparts = gemm_split_k(g.M, g.N, g.K);
             g.split_k = nparts; g.split_k_slab = (long)(B * q.G);
-            prof_begin(0);
             MYEA_TRY(launch_gemm(stream, g));
-            prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
         }
         hipLaunchKernelGGL(lstm_forward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, (int)(s == 0), bias, q.peep,
                            acts_t, s ? q.c + tp * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, q.h + t * Bmax * q.C,
                            q.part, nparts, s ? q.h + tp * Bmax * q.C : nullptr, zs, zo);
         MYEA_HIP_TRY(hipGetLastError());
     }
+    if (T > 1) prof_end(2.0 * (double)(T - 1) * (double)B * (double)q.G * (double)q.C, T - 1);   // the recurrent contractions of steps 1 .. T-1
     return MYEA_OK;
 }
 
@@ -477,6 +476,7 @@ int Net::lstm_backward_direction(LstmLayer &q, size_t B)
 {
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
     const LstmGeom geom = geom_of(q);
+    if (T > 1) prof_begin(1);   // one pair of timing events for the whole time loop
     for (size_t s = T; s-- > 0;) {
         // tn / tp: the steps processed after / before t in the direction's own order
         const size_t t = q.reverse ? T - 1 - s : s, tn = q.reverse ? t - 1 : t + 1, tp = q.reverse ? t + 1 : t - 1;
@@ -490,9 +490,7 @@ int Net::lstm_backward_direction(LstmLayer &q, size_t B)
             f.acts = q.acts + t * Bmax * q.G; f.acts_next = q.acts + tn * Bmax * q.G;
             f.c_prev = first ? nullptr : q.c + tp * Bmax * q.C; f.ca = q.ca + t * Bmax * q.C;
             f.dh = dh_t; f.dG = q.dG + t * Bmax * q.G; f.dc = q.dc + t * Bmax * q.C; f.dc_next = q.dc + tn * Bmax * q.C;
-            prof_begin(1);
             MYEA_TRY(launch_lstm_fused_backward(stream, f));
-            prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
             continue;
         }
         if (!last) {  // Backward_Pass__LSTM_Derivative__Output, recurrent part (:1174-1226)
@@ -503,9 +501,7 @@ int Net::lstm_backward_direction(LstmLayer &q, size_t B)
             g.M = (int)B; g.N = (int)q.C; g.K = (int)q.G;
             nparts = gemm_split_k(g.M, g.N, g.K);
             g.split_k = nparts; g.split_k_slab = (long)(B * q.C);
-            prof_begin(1);
             MYEA_TRY(launch_gemm(stream, g));
-            prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
         }
         const int mode = (first && last) ? 0 : (last ? 1 : (first ? 3 : 2));
         hipLaunchKernelGGL(lstm_backward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, mode, q.peep,
@@ -514,6 +510,7 @@ int Net::lstm_backward_direction(LstmLayer &q, size_t B)
                            q.dc + t * Bmax * q.C, last ? nullptr : q.dc + tn * Bmax * q.C, q.part, nparts);
         MYEA_HIP_TRY(hipGetLastError());
     }
+    if (T > 1) prof_end(2.0 * (double)(T - 1) * (double)B * (double)q.G * (double)q.C, T - 1);
     return MYEA_OK;
 }
 

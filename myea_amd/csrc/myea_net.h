@@ -46,6 +46,7 @@ struct ProfEvent {
     hipEvent_t start = nullptr, stop = nullptr;
     int family = 0;
     double work = 0;
+    uint64_t launches = 1;   // launches between the two events (a recurrent layer's time loop is bracketed as a whole)
 };
 
 bool layer_is_pooling(const myea_layer_desc &l);
@@ -98,7 +99,7 @@ struct Net {
     float *scale_ptr(float *base, size_t li);
     float *shift_ptr(float *base, size_t li);
     void prof_begin(int family);
-    void prof_end(double work);
+    void prof_end(double work, uint64_t launches = 1);
 
     int refresh_colscale(size_t li, bool *active);
     int forward_fc_layer(size_t li, size_t B);

@@ -87,11 +87,12 @@ void Net::prof_begin(int family)
     open_event = true;
 }
 
-void Net::prof_end(double work)
+void Net::prof_end(double work, uint64_t launches)
 {
     if (!profiling || !open_event) return;
     ProfEvent &ev = pending.back();
     ev.work = work;
+    ev.launches = launches;
     (void)hipEventRecord(ev.stop, stream);
     open_event = false;
 }
@@ -1419,7 +1420,7 @@ int myea_hip_profile_read(myea_hip_net *n, int family, uint64_t *launches, doubl
         if (hipEventElapsedTime(&t, e.start, e.stop) == hipSuccess) {
             n->net.prof_ms[e.family] += t;
             n->net.prof_work[e.family] += e.work;
-            n->net.prof_launches[e.family] += 1;
+            n->net.prof_launches[e.family] += e.launches;
         }
         n->net.free_events.push_back(e);
     }
