@@ -14,7 +14,13 @@
  * Parts of the behaviour that are reference quirks rather than mathematics (listed at each
  * function) are pinned only by reading: "parity unpinned" for
  *   - the LSTM bias index overrun (Prepare__Bias__LSTM),
- *   - the RNN head `pre` pointer quirk (RNN__Compute__Error).
+ *   - the RNN head `pre` pointer quirk (RNN__Compute__Error),
+ *   - the Nesterov update sign, ELU' / SELU' as written, the backward pass having no dropout, zoneout, k-sparse or
+ *     noise-dropout operator (each restated as written, with a test that shows where it leaves the textbook form),
+ *   - which of several EQUAL values stays at a k-sparse filter's cut (std::sort's order in the reference; the lower
+ *     index here),
+ *   - the random draws of Gaussian / Uout dropout and ShakeDrop: an INPUT of this restatement (the reference draws them
+ *     from its host generators inside the pass).
  *
  * Summation order is the serial order of the reference's __Loop variants; the __OpenMP variants
  * differ only in the order of the per-thread partial sums.
