@@ -23,7 +23,7 @@ if ROOT not in sys.path:
 # HBM bytes per contraction launch (mean over the launches of one step) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of this script, scaled by what the same counters read for copies of known size (FETCH_SIZE x2, WRITE_SIZE x1);
 # the per-kernel figures are in profiles/hbm_traffic__*__pmc.txt.  None where no counter run has been made.
-PMC_TRAFFIC_BYTES_PER_GEMM_LAUNCH = {"fc4096x4_b1024_adam": 2880900 * 1024 / 14}
+PMC_TRAFFIC_BYTES_PER_GEMM_LAUNCH = {"fc4096x4_b1024_adam": 2896189 * 1024 / 10}
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
@@ -180,8 +180,7 @@ def main():
     def step():
         net.Forward_Pass(B, xd, on_device=True)
         net.Compute__Error(B, yd, on_device=True)
-        net.Backward_Pass(B)
-        net.Update_Derivative_Weight(B)
+        net.Backward_Pass__Update_Derivative_Weight(B)     # the two calls of Train_Batch_BP as one entry point
         net.Update_Parameter(B, B)
 
     for _ in range(args.warmup):
@@ -196,17 +195,20 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    fam = {name: net.profile_read(i) for i, name in enumerate(("forward", "dx", "dw", "update"))}
+    fam = {name: net.profile_read(i) for i, name in enumerate(("forward", "dx", "dw", "update", "dx_dw_pair"))}
+    GEMM_FAMILIES = ("forward", "dx", "dw", "dx_dw_pair")   # dx_dw_pair: a layer's dX and dW contractions in one launch
     net.profile_enable(False)
     loss = net.get_loss()
 
-    g_launch = sum(fam[k][0] for k in ("forward", "dx", "dw"))
-    g_ms = sum(fam[k][1] for k in ("forward", "dx", "dw"))
-    g_flop = sum(fam[k][2] for k in ("forward", "dx", "dw"))
+    g_launch = sum(fam[k][0] for k in GEMM_FAMILIES)
+    g_ms = sum(fam[k][1] for k in GEMM_FAMILIES)
+    g_flop = sum(fam[k][2] for k in GEMM_FAMILIES)
     achieved = g_flop / (g_ms * 1e-3) / 1e12 if g_ms > 0 else 0.0
     kernels = {}
-    for k in ("forward", "dx", "dw"):
+    for k in GEMM_FAMILIES:
         n, ms, work = fam[k]
+        if n == 0:
+            continue
         kernels["gemm_" + k] = dict(launches=n, avg_ms=ms / max(n, 1), tflops=work / max(ms * 1e-3, 1e-12) / 1e12,
                                     frac_mfma_peak=work / max(ms * 1e-3, 1e-12) / 1e12 / PEAK_FP32_MFMA_TFLOPS)
     n, ms, work = fam["update"]
@@ -226,7 +228,7 @@ def main():
                    "gemm_flops_per_step": gemm_flops_per_step(wl["layers"], B, wl.get("depth", 1))},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": PMC_TRAFFIC_BYTES_PER_GEMM_LAUNCH.get(args.workload),
-                     "kernel": "gemm_f32_mfma_kernel (forward + dX + dW launches)", "launches": g_launch,
+                     "kernel": "gemm_f32_mfma_kernel / gemm_pair_kernel (forward, dX, dW and paired dX + dW launches)", "launches": g_launch,
                      "avg_launch_ms": g_ms / max(g_launch, 1), "flops_per_launch": g_flop / max(g_launch, 1),
                      "gemm_ms_per_step": g_ms / args.steps},
         "kernels": kernels,

@@ -120,13 +120,15 @@ enum {
  * way `Neural_Network::Compile` does for callers that have no host object. */
 typedef struct myea_layer_desc {
     uint32_t type_layer;               /* MYEA_LAYER_* */
-    uint32_t n_units;                  /* FC: neurons.  LSTM: blocks per direction.  Input layer: inputs. */
+    uint32_t n_units;                  /* FC / independently recurrent: neurons.  LSTM: blocks per direction.  Input layer: inputs.
+                                        * Pooling: written by myea_net_desc_layout.  Residual: unused (block_depth). */
     uint32_t n_cells_per_block;        /* LSTM only, >= 1 (Layer_Parameters::unit_parameters[1]) */
     uint32_t use_bidirectional;        /* LSTM only */
-    uint32_t type_activation_function; /* FC only; MYEA_AF_* (whole layer, Set__Layer_Activation_Function) */
-    float    activation_steepness;     /* FC only; Set__Layer_Activation_Steepness, default 1 */
+    uint32_t type_activation_function; /* FC and independently recurrent layers; MYEA_AF_* (whole layer, Set__Layer_Activation_Function) */
+    float    activation_steepness;     /* same layers; Set__Layer_Activation_Steepness, default 1 */
     uint32_t type_dropout;             /* MYEA_DROPOUT_* */
-    float    dropout_values[2];        /* [0] = retention probability */
+    float    dropout_values[2];        /* [0]: Bernoulli = retention probability, Gaussian = p / (1 - p), Uout = beta, ShakeDrop = probability,
+                                        * zoneout = cell-state probability; [1]: zoneout = cell-output probability */
     uint32_t type_normalization;       /* MYEA_NORMALIZATION_* */
     uint32_t use_layer_normalization_before_activation;
     uint32_t block_depth;              /* residual only: layers inside the block */
@@ -140,7 +142,7 @@ typedef struct myea_layer_desc {
      * Compute__Regularization__Constraint_Recurrent_Weight__Default, :33-75) */
     float    constraint_recurrent_weight_lower_bound;
     float    constraint_recurrent_weight_upper_bound;
-    /* k-sparse filter on the layer's outputs (hidden fully-connected layers, also inside residual blocks): after the dropout
+    /* k-sparse filter on the layer's outputs (hidden fully-connected layers outside residual blocks): after the dropout
      * only the k_sparsity largest values of an example's row stay, the others become 0; at inference
      * size_t(alpha_sparsity * k_sparsity) stay.  0 = no filter (Layer::k_sparsity / ::alpha_sparsity, Data.hpp:733-734;
      * Sparse_K_Filter, NN/Neural_Network__K_Sparse.cpp:268-339; the backward pass does not look at the filter). */
@@ -377,6 +379,12 @@ int myea_hip_backward_pass(myea_hip_net *net, size_t batch_size_received);
 /* Neural_Network::Update_Derivative_Weight (Data.hpp:2199) over layers
  * [first_layer_index, end_layer_index); the reference's callers pass (layers + 1, last). */
 int myea_hip_update_derivative_weight(myea_hip_net *net, size_t batch_size_received, size_t first_layer_index, size_t end_layer_index);
+/* Backward_Pass immediately followed by Update_Derivative_Weight(batch, 1, total_layers) - the two calls Dataset::Train_Batch_BP
+ * issues back to back (Neural_Network/Dataset.cpp:645-658) - as one entry point.  Results are those of the two calls; knowing
+ * that the weight gradients are wanted lets the library send a layer's `dW += delta^T X` along in the same launch as the
+ * `dX = delta W` that hands its delta down (two 128 x 128-tiled contractions sharing the CUs keep the matrix pipe busier than
+ * either alone when the batch is about a thousand rows). */
+int myea_hip_backward_pass_and_update_derivative_weight(myea_hip_net *net, size_t batch_size);
 
 /* Neural_Network::Update_Parameter (Data.hpp:849; Neural_Network.cpp:4719-4908): clip-by-global-norm
  * then the fused optimizer; zeroes the gradient. */

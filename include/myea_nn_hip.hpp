@@ -312,6 +312,11 @@ public:
         Ok("Compute__Error", myea_hip_compute_error(net_, batch_size_received, rows_.data(), 0));
     }
     void Backward_Pass(size_t batch_size_received) { if (Need("Backward_Pass") && PushFields("Backward_Pass")) Ok("Backward_Pass", myea_hip_backward_pass(net_, batch_size_received)); }
+    // Backward_Pass and Update_Derivative_Weight(batch, 1, total_layers) of Train_Batch_BP (Dataset.cpp:645-658) as one call
+    void Backward_Pass__Update_Derivative_Weight(size_t batch_size_received)
+    {
+        if (Need("Backward_Pass") && PushFields("Backward_Pass")) Ok("Backward_Pass", myea_hip_backward_pass_and_update_derivative_weight(net_, batch_size_received));
+    }
     // the reference's callers pass (ptr_array_layers + 1, ptr_last_layer); here as layer indices
     void Update_Derivative_Weight(size_t batch_size_received, size_t first_layer_index = 1, size_t end_layer_index = 0)
     {

@@ -264,21 +264,21 @@ struct GemmDev {
     long slab;
 };
 
+// One workgroup's share of a contraction: tile number `block` of problem `p`, staged through `smem`.
 template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
-__global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
+__device__ __forceinline__ void gemm_tile(const GemmDev &p, const int block, float *smem)
 {
     constexpr int TM = BM / 64, TN = BN / 64;  // 32x32 accumulators per wavefront along m / n
     using PA = OperandPath<BM, A_KC, VEC>;
     using PB = OperandPath<BN, B_KC, VEC>;
-    extern __shared__ __attribute__((aligned(16))) float smem[];
     constexpr int kStage = PA::kFloats + PB::kFloats;  // one LDS stage = A tile then B tile
 
     // Workgroup -> tile.  Consecutive workgroup ids land on different XCDs (8 of them, each with its own
     // L2), so give every XCD a contiguous run of tile ids, and walk tiles in bands of 8 m-tiles so that a
     // run shares its B columns and a small set of A rows.
     const int nblocks = p.nbm * p.nbn;
-    const int split = blockIdx.x / nblocks;   // split-K slab of this workgroup
-    int pid = blockIdx.x - split * nblocks;
+    const int split = block / nblocks;   // split-K slab of this workgroup
+    int pid = block - split * nblocks;
     if ((nblocks & 7) == 0) pid = (pid & 7) * (nblocks >> 3) + (pid >> 3);
     const int k_begin = split * p.kchunk, k_end = min(p.K, k_begin + p.kchunk);
     constexpr int kBand = 8;
@@ -422,6 +422,26 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
 }
 
 template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
+__global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
+{
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    gemm_tile<BM, BN, A_KC, B_KC, VEC>(p, (int)blockIdx.x, smem);
+}
+
+// Two independent contractions in one launch, 128 x 128 tiles each: workgroups [0, first_blocks) work on `a` (A k-contiguous,
+// B n-contiguous: dX = delta W), the others on `b` (both operands k-strided: dW += delta^T X).  A batch of 1024 gives dX only
+// 256 such tiles - one workgroup per CU, one wavefront per SIMD, too little to keep the matrix pipe busy - while dW has
+// four times as many, quarter as long.  Launched together, a CU holds one long dX workgroup next to a succession of
+// dW workgroups: two wavefronts per SIMD throughout, and the dW tiles' stores fall at different moments behind
+// the dX workgroup's MFMAs instead of all at once.
+__global__ __launch_bounds__(kThreads, 2) void gemm_pair_kernel(GemmDev a, GemmDev b, int first_blocks)
+{
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    if ((int)blockIdx.x < first_blocks) gemm_tile<128, 128, true, false, true>(a, (int)blockIdx.x, smem);
+    else gemm_tile<128, 128, false, false, true>(b, (int)blockIdx.x - first_blocks, smem);
+}
+
+template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
 int launch_one(hipStream_t stream, GemmDev d)
 {
     constexpr size_t lds_bytes = ((VEC && BM * BN < 128 * 128) ? 3 : 2) * (OperandPath<BM, A_KC, VEC>::kFloats + OperandPath<BN, B_KC, VEC>::kFloats) * sizeof(float);
@@ -498,7 +518,8 @@ bool gemm_can_fuse_activation(int act)
            act == MYEA_AF_TANH || act == MYEA_AF_SIGMOID;
 }
 
-int launch_gemm(hipStream_t stream, const GemmParams &p)
+// checks a problem and fills the kernel's argument block; *vec: operands take the direct (16-byte aligned) path
+static int prepare_gemm(const GemmParams &p, GemmDev &d, bool *vec)
 {
     if (p.M <= 0 || p.N <= 0 || p.K < 0) { set_last_error("gemm: bad shape M=%d N=%d K=%d", p.M, p.N, p.K); return MYEA_E_INVALID; }
     if (!p.A || !p.B || !p.C) { set_last_error("gemm: null operand"); return MYEA_E_INVALID; }
@@ -508,7 +529,6 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     if (p.epilogue == EPI_FC_DERIVE && !gemm_can_fuse_activation(p.act)) { set_last_error("gemm: activation %d cannot be fused", p.act); return MYEA_E_INVALID; }
     if (p.epilogue == EPI_FC_FORWARD && p.aux_out && !gemm_can_fuse_activation(p.act)) { set_last_error("gemm: activation %d cannot be fused", p.act); return MYEA_E_INVALID; }
 
-    GemmDev d;
     d.A = p.A; d.B = p.B; d.C = p.C;
     d.M = p.M; d.N = p.N; d.K = p.K;
     d.lda = p.lda; d.ldb = p.ldb; d.ldc = p.ldc;
@@ -532,7 +552,18 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     auto aligned = [](const float *ptr, long ld, long contiguous_extent) {
         return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0 && (ld & 3) == 0 && (contiguous_extent & 3) == 0;
     };
-    const bool vec = aligned(p.A, p.lda, p.a_k_contiguous ? p.K : p.M) && aligned(p.B, p.ldb, p.b_k_contiguous ? p.K : p.N);
+    *vec = aligned(p.A, p.lda, p.a_k_contiguous ? p.K : p.M) && aligned(p.B, p.ldb, p.b_k_contiguous ? p.K : p.N);
+    return MYEA_OK;
+}
+
+int launch_gemm(hipStream_t stream, const GemmParams &p)
+{
+    GemmDev d;
+    bool vec = false;
+    {
+        const int rc = prepare_gemm(p, d, &vec);
+        if (rc != MYEA_OK) return rc;
+    }
     const bool a_kc = p.a_k_contiguous != 0, b_kc = p.b_k_contiguous != 0;
 
     if (!vec || (!a_kc && b_kc)) return launch_layout_scalar(stream, d, a_kc, b_kc);
@@ -543,6 +574,37 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     if (tiles_128 * 2 * d.ksplit < 256) return launch_layout_vec_small(stream, d, a_kc, b_kc);
     if (p.M <= p.N) return launch_layout_vec<64, 128>(stream, d, a_kc, b_kc);
     return launch_layout_vec<128, 64>(stream, d, a_kc, b_kc);
+}
+
+// `a` = (A k-contiguous, B n-contiguous), `b` = (both k-strided), neither split along k, 16-byte aligned operands, and `a`
+// no more than about one 128 x 128 tile per CU: both in ONE launch (gemm_pair_kernel).  Returns MYEA_OK when launched,
+// 1 when the pair form does not apply (the caller launches the two one after the other), a negative code on an error.
+int launch_gemm_pair(hipStream_t stream, const GemmParams &a, const GemmParams &b)
+{
+    if (!a.a_k_contiguous || a.b_k_contiguous || b.a_k_contiguous || b.b_k_contiguous || a.split_k > 1 || b.split_k > 1) return 1;
+    GemmDev da, db;
+    bool va = false, vb = false;
+    int rc = prepare_gemm(a, da, &va);
+    if (rc != MYEA_OK) return rc;
+    rc = prepare_gemm(b, db, &vb);
+    if (rc != MYEA_OK) return rc;
+    if (!va || !vb) return 1;
+    da.nbm = (a.M + 127) / 128; da.nbn = (a.N + 127) / 128;
+    db.nbm = (b.M + 127) / 128; db.nbn = (b.N + 127) / 128;
+    const long na = (long)da.nbm * da.nbn, nb = (long)db.nbm * db.nbn;
+    // worth it when `a` alone would leave the CUs with one workgroup each and `b` brings at least as much work in shorter pieces
+    if (na < 128 || na > 256 || (na & 7) || nb < na || (double)a.K * (double)na > 2.0 * (double)b.K * (double)nb || (double)b.K * (double)nb > 2.0 * (double)a.K * (double)na) return 1;
+    constexpr size_t lds_a = 2 * (OperandPath<128, true, true>::kFloats + OperandPath<128, false, true>::kFloats) * sizeof(float);
+    constexpr size_t lds_b = 2 * (OperandPath<128, false, true>::kFloats + OperandPath<128, false, true>::kFloats) * sizeof(float);
+    constexpr size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
+    static bool attr_done = false;
+    if (!attr_done) {
+        MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pair_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(gemm_pair_kernel, dim3((unsigned)(na + nb)), dim3(kThreads), lds_bytes, stream, da, db, (int)na);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
 }
 
 }  // namespace myea

@@ -53,6 +53,9 @@ struct GemmParams {
 
 int gemm_split_k(int M, int N, int K);
 int launch_gemm(hipStream_t stream, const GemmParams &p);
+// dX = delta W (`a`) and dW += delta^T X (`b`) in one launch when their shapes suit it; MYEA_OK = launched, 1 = does not
+// apply (launch them one after the other), negative = error
+int launch_gemm_pair(hipStream_t stream, const GemmParams &a, const GemmParams &b);
 // activations the FC_FORWARD / FC_DERIVE epilogues can apply (the others run as a separate kernel)
 bool gemm_can_fuse_activation(int act);
 

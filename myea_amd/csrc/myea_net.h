@@ -41,7 +41,7 @@ struct DevLayer {
     LstmLayer *lstm = nullptr, *lstm2 = nullptr;  // lstm2: the time-reversed direction of a bidirectional layer
 };
 
-constexpr int kProfFamilies = 4;
+constexpr int kProfFamilies = 5;   // forward, dX, dW, update, dX + dW launched as a pair
 struct ProfEvent {
     hipEvent_t start = nullptr, stop = nullptr;
     int family = 0;
@@ -80,8 +80,8 @@ struct Net {
 
     bool profiling = false, open_event = false;
     std::vector<ProfEvent> pending, free_events;
-    uint64_t prof_launches[kProfFamilies] = {0, 0, 0, 0};
-    double prof_ms[kProfFamilies] = {0, 0, 0, 0}, prof_work[kProfFamilies] = {0, 0, 0, 0};
+    uint64_t prof_launches[kProfFamilies] = {};
+    double prof_ms[kProfFamilies] = {}, prof_work[kProfFamilies] = {};
 
     ~Net();
     int create(const myea_net_desc &desc);
@@ -100,6 +100,7 @@ struct Net {
     float *shift_ptr(float *base, size_t li);
     void prof_begin(int family);
     void prof_end(double work, uint64_t launches = 1);
+    void prof_cancel();
 
     int refresh_colscale(size_t li, bool *active);
     int forward_fc_layer(size_t li, size_t B);
@@ -112,6 +113,12 @@ struct Net {
     int forward_pass(size_t B, const float *inputs, int on_device);
     int compute_error(size_t B, const float *desired, int on_device);
     int backward_pass(size_t B);
+    // Backward_Pass followed by Update_Derivative_Weight over all layers, with a layer's weight gradient riding in the
+    // launch that sends its delta down wherever the two contractions suit each other
+    int backward_pass_and_update_derivative_weight(size_t B);
+    bool pairing = false;              // inside the call above
+    std::vector<char> dw_done;         // per layer: the weight contraction already ran in this pass
+    bool fc_dw_params(size_t li, size_t B, GemmParams *g);   // false: the layer's weight gradient is not one plain contraction
     int update_derivative_weight(size_t B, size_t first, size_t end);
     int update_parameter(size_t B, size_t training_size);
     int set_unit_activations(size_t li, const uint32_t *types, const float *steep, size_t count);

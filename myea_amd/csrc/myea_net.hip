@@ -87,6 +87,15 @@ void Net::prof_begin(int family)
     open_event = true;
 }
 
+// drops the pair opened by prof_begin when nothing was launched after all
+void Net::prof_cancel()
+{
+    if (!profiling || !open_event) return;
+    free_events.push_back(pending.back());
+    pending.pop_back();
+    open_event = false;
+}
+
 void Net::prof_end(double work, uint64_t launches)
 {
     if (!profiling || !open_event) return;
@@ -765,9 +774,21 @@ int Net::backward_into_layer(size_t li, size_t B)
             g.epilogue = EPI_NONE;
         }
         if (have_gemm) {
-            prof_begin(1);
-            MYEA_TRY(launch_gemm(stream, g));
-            prof_end(2.0 * (double)rows * (double)H * (double)Out);
+            bool paired = false;
+            GemmParams w{};
+            if (pairing && chunks == 1 && !second_direction && next.type_layer == MYEA_LAYER_FULLY_CONNECTED && on.group == 0 && fc_dw_params(gi, B, &w)) {
+                prof_begin(4);
+                const int rc = launch_gemm_pair(stream, g, w);
+                if (rc < 0) return rc;
+                paired = rc == MYEA_OK;
+                if (paired) { prof_end(2.0 * (double)rows * (double)H * (double)Out + 2.0 * (double)w.M * (double)w.N * (double)w.K); dw_done[gi] = 1; }
+                else prof_cancel();
+            }
+            if (!paired) {
+                prof_begin(1);
+                MYEA_TRY(launch_gemm(stream, g));
+                prof_end(2.0 * (double)rows * (double)H * (double)Out);
+            }
         } else if (pool_consumer) {
             MYEA_TRY(launch_pool_backward(stream, pool_params(gi, rows), on.neuron_errors + roff * on.H, on.pool_index ? on.pool_index + roff * on.H : nullptr, g.C));
         } else {
@@ -874,6 +895,19 @@ int Net::bn_backward(size_t li, size_t t, size_t rows, const float *x, const flo
     return launch_bn_backward(stream, p, scratch);
 }
 
+int Net::backward_pass_and_update_derivative_weight(size_t B)
+{
+    dw_done.assign(d.n_layers, 0);
+    // MYEA_GEMM_PAIR=0 in the environment keeps the two passes as separate launches (for A / B timing on one machine)
+    static const bool pair_off = [] { const char *e = std::getenv("MYEA_GEMM_PAIR"); return e && e[0] == '0'; }();
+    pairing = !pair_off;
+    int rc = backward_pass(B);
+    pairing = false;
+    if (rc == MYEA_OK) rc = update_derivative_weight(B, 1, d.n_layers);
+    dw_done.assign(d.n_layers, 0);
+    return rc;
+}
+
 int Net::backward_pass(size_t B)
 {
     if (B == 0 || B > d.batch_size) { set_last_error("Backward_Pass: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
@@ -900,6 +934,29 @@ static int fc_dw_slabs(size_t H, size_t In, size_t rows, size_t first_connection
 {
     if (((H * In) & 3) || (first_connection_index & 3) || rows > 0x7fffffffu) return 1;   // the slab sum works on aligned quads
     return gemm_split_k((int)H, (int)In, (int)rows);
+}
+
+// the weight gradient of fully-connected layer li as one accumulating contraction dW += delta^T X (false when it takes the
+// per-time-step or the split-K form instead)
+bool Net::fc_dw_params(size_t li, size_t B, GemmParams *out)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, In = o.In, H = o.H;
+    if (T > 1 && B != Bmax) return false;
+    const size_t rows = T > 1 ? T * B : B;
+    if (dw_slabs && fc_dw_slabs(H, In, rows, l.first_connection_index) > 1) return false;
+    const float *x = layer_outputs(o.prev);
+    if (o.group == 2) x = o.values;
+    else if (o.group == 1 && layer_uses_norm(l)) x = o.normalizes;
+    GemmParams g{};
+    g.A = o.neuron_errors; g.lda = (long)H; g.a_k_contiguous = 0;
+    g.B = x; g.ldb = (long)In; g.b_k_contiguous = 0;
+    g.C = gradient + l.first_connection_index; g.ldc = (long)In;
+    g.M = (int)H; g.N = (int)In; g.K = (int)rows;
+    g.accumulate = 1; g.epilogue = EPI_NONE;
+    *out = g;
+    return true;
 }
 
 int Net::update_derivative_weight(size_t B, size_t first, size_t end)
@@ -929,10 +986,13 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
             g.accumulate = 1; g.epilogue = EPI_NONE;
             const int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
             if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
-            prof_begin(2);
-            MYEA_TRY(launch_gemm(stream, g));
-            if (slabs > 1) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
-            prof_end(2.0 * (double)rows * (double)H * (double)In);
+            const bool done = li < dw_done.size() && dw_done[li];   // rode along with the delta's contraction in this pass
+            if (!done) {
+                prof_begin(2);
+                MYEA_TRY(launch_gemm(stream, g));
+                if (slabs > 1) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
+                prof_end(2.0 * (double)rows * (double)H * (double)In);
+            }
             if (layer_uses_bias(l)) MYEA_TRY(launch_column_sum(stream, rows, H, o.neuron_errors + roff * H, gradient + l.first_bias_connection_index, 1, scratch));
         }
         if (layer_is_ind_rnn(l))
@@ -1324,6 +1384,7 @@ int myea_hip_device_buffer_destroy(float *device)
 }
 int myea_hip_backward_pass(myea_hip_net *n, size_t B) { NET_OR_FAIL(n); return n->net.backward_pass(B); }
 int myea_hip_update_derivative_weight(myea_hip_net *n, size_t B, size_t first, size_t end) { NET_OR_FAIL(n); return n->net.update_derivative_weight(B, first, end); }
+int myea_hip_backward_pass_and_update_derivative_weight(myea_hip_net *n, size_t B) { NET_OR_FAIL(n); return n->net.backward_pass_and_update_derivative_weight(B); }
 int myea_hip_update_parameter(myea_hip_net *n, size_t B, size_t ts) { NET_OR_FAIL(n); return n->net.update_parameter(B, ts); }
 
 int myea_hip_reset_loss(myea_hip_net *n)
