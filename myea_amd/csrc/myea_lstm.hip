@@ -301,6 +301,13 @@ bool fused_lstm_disabled()
     return e && e[0] == '0';
 }
 
+// MYEA_LSTM_CONCURRENT=0 keeps both directions of a bidirectional layer on the caller's stream (for A/B timing)
+bool concurrent_directions_disabled()
+{
+    const char *e = std::getenv("MYEA_LSTM_CONCURRENT");
+    return e && e[0] == '0';
+}
+
 }  // namespace
 
 int Net::lstm_create_layer(size_t li)
@@ -312,6 +319,7 @@ int Net::lstm_create_layer(size_t li)
     if (l.n_cells_per_block == 0) { set_last_error("layer %zu: LSTM needs at least one cell per block", li); return MYEA_E_INVALID; }
     const size_t T = d.number_recurrent_depth, B = d.batch_size;
     const size_t dirs = l.use_bidirectional ? 2 : 1;
+    if (dirs == 2 && !concurrent_directions_disabled()) MYEA_TRY(side_stream_create());
     MYEA_TRY(dev_alloc_zero(&o.neuron_errors, T * B * (size_t)l.n_units * l.n_cells_per_block));  // delta of the layer's output (ptr_delta_cell_output)
     // Two directions (contract of this library: the reference overlays its two directions' buffers and has no behaviour to
     // follow): direction 1 owns the second half of the layer's blocks and the second [G] slice of its biases and walks time
@@ -458,16 +466,36 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
     return MYEA_OK;
 }
 
+int Net::side_stream_create()
+{
+    if (side_stream) return MYEA_OK;
+    MYEA_HIP_TRY(hipStreamCreateWithFlags(&side_stream, hipStreamNonBlocking));
+    MYEA_HIP_TRY(hipEventCreateWithFlags(&fork_event, hipEventDisableTiming));
+    MYEA_HIP_TRY(hipEventCreateWithFlags(&join_event, hipEventDisableTiming));
+    return MYEA_OK;
+}
+
+int Net::side_stream_join()
+{
+    if (side_stream) MYEA_HIP_TRY(hipStreamWaitEvent(stream, join_event, 0));
+    return MYEA_OK;
+}
+
 int Net::lstm_forward_layer(size_t li, size_t B)
 {
     DevLayer &o = L[li];
-    MYEA_TRY(lstm_forward_direction(li, *o.lstm, B));
     if (o.lstm2) {
-        MYEA_TRY(lstm_forward_direction(li, *o.lstm2, B));
+        {   // the second direction beside the first (on the same stream, in this order, without a side stream)
+            SideStreamScope side(*this);
+            MYEA_TRY(lstm_forward_direction(li, *o.lstm2, B));
+        }
+        MYEA_TRY(lstm_forward_direction(li, *o.lstm, B));
+        MYEA_TRY(side_stream_join());
         const size_t rows = (size_t)d.number_recurrent_depth * d.batch_size;
         MYEA_TRY(launch_padded_add(stream, rows, o.H, o.lstm->h, o.H, 0, o.lstm2->h, o.H, 0, o.values));  // output = h_forward + h_backward
+        return MYEA_OK;
     }
-    return MYEA_OK;
+    return lstm_forward_direction(li, *o.lstm, B);
 }
 
 // Recurrent__Backward_Pass__Gradient__LSTM (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:440-862), time
@@ -517,13 +545,20 @@ int Net::lstm_backward_direction(LstmLayer &q, size_t B)
 int Net::lstm_backward_layer(size_t li, size_t B)
 {
     DevLayer &o = L[li];
-    for (LstmLayer *q : {o.lstm, o.lstm2}) {
-        if (!q) continue;
-        if (q->own_h)  // both directions start from the same delta of the layer's output
-            MYEA_HIP_TRY(hipMemcpyAsync(q->dh, o.neuron_errors, (size_t)d.number_recurrent_depth * d.batch_size * q->C * sizeof(float), hipMemcpyDeviceToDevice, stream));
-        MYEA_TRY(lstm_backward_direction(*q, B));
+    auto one = [&](LstmLayer &q) -> int {
+        if (q.own_h)  // both directions start from the same delta of the layer's output
+            MYEA_HIP_TRY(hipMemcpyAsync(q.dh, o.neuron_errors, (size_t)d.number_recurrent_depth * d.batch_size * q.C * sizeof(float), hipMemcpyDeviceToDevice, stream));
+        return lstm_backward_direction(q, B);
+    };
+    if (o.lstm2) {
+        {
+            SideStreamScope side(*this);
+            MYEA_TRY(one(*o.lstm2));
+        }
+        MYEA_TRY(one(*o.lstm));
+        return side_stream_join();
     }
-    return MYEA_OK;
+    return one(*o.lstm);
 }
 
 // the operands of "delta of the layer below = dG Win" (Backward_Pass__LSTM, :1024-1120), handed to the shared driver

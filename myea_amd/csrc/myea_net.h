@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <utility>
 #include <vector>
 
 #include "../../include/myea_hip.h"
@@ -62,6 +63,10 @@ struct Net {
     myea_hyper h{};
     uint32_t state = MYEA_STATE_INFERENCE;
     hipStream_t stream = nullptr;
+    // The two directions of a bidirectional LSTM layer are independent until their outputs are added: the second one's
+    // launches go to a stream of the library's own (default priority), forked from and joined to `stream` by events.
+    hipStream_t side_stream = nullptr;
+    hipEvent_t fork_event = nullptr, join_event = nullptr;
     float *parameters = nullptr, *gradient = nullptr, *opt[MYEA_STATE_KINDS] = {};
     uint8_t *masks = nullptr;
     unsigned long long dropout_seed = 0x9E3779B97F4A7C15ull, dropout_stream = 0;   // device generator: key and the next stream id
@@ -131,12 +136,34 @@ struct Net {
     int lstm_backward_layer(size_t li, size_t B);       // BPTT inside LSTM layer li
     // delta / weight operands an LSTM consumer gi offers to the layer below: delta [T][Bmax][width], weights [width][fan-in]
     void lstm_delta_source(size_t gi, int direction, const float **delta, size_t *width, const float **weights);
+    int side_stream_create();
+    int side_stream_join();            // `stream` waits for what the last SideStreamScope enqueued
     int lstm_forward_direction(size_t li, LstmLayer &q, size_t B);
     int lstm_backward_direction(LstmLayer &q, size_t B);
     int lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t B);
     size_t lstm_scratch_floats() const;
     int lstm_update_derivative_weight(size_t li, size_t B);
     const float *lstm_tensor(size_t li, int kind, size_t *count);
+};
+
+// Launches made while the scope lives go to the side stream, ordered behind everything `stream` held when it opened.
+struct SideStreamScope {
+    Net &net;
+    bool active = false;
+    explicit SideStreamScope(Net &n) : net(n)
+    {
+        if (!n.side_stream || hipEventRecord(n.fork_event, n.stream) != hipSuccess || hipStreamWaitEvent(n.side_stream, n.fork_event, 0) != hipSuccess) return;
+        std::swap(n.stream, n.side_stream);
+        active = true;
+    }
+    ~SideStreamScope()
+    {
+        if (!active) return;
+        std::swap(net.stream, net.side_stream);
+        (void)hipEventRecord(net.join_event, net.side_stream);
+    }
+    SideStreamScope(const SideStreamScope &) = delete;
+    SideStreamScope &operator=(const SideStreamScope &) = delete;
 };
 
 }  // namespace myea

@@ -335,6 +335,12 @@ int Net::create(const myea_net_desc &desc)
 
 Net::~Net()
 {
+    if (side_stream) {
+        (void)hipStreamSynchronize(side_stream);
+        (void)hipStreamDestroy(side_stream);
+        (void)hipEventDestroy(fork_event);
+        (void)hipEventDestroy(join_event);
+    }
     auto fr = [](void *p) { if (p) (void)hipFree(p); };
     fr(parameters); fr(gradient);
     for (int k = 0; k < MYEA_STATE_KINDS; ++k) fr(opt[k]);
