@@ -301,10 +301,10 @@ bool fused_lstm_disabled()
     return e && e[0] == '0';
 }
 
-// MYEA_LSTM_CONCURRENT=0 keeps both directions of a bidirectional layer on the caller's stream (for A/B timing)
-bool concurrent_directions_disabled()
+// MYEA_SIDE_STREAM=0 keeps every launch on the caller's stream (for A/B timing)
+bool side_stream_disabled()
 {
-    const char *e = std::getenv("MYEA_LSTM_CONCURRENT");
+    const char *e = std::getenv("MYEA_SIDE_STREAM");
     return e && e[0] == '0';
 }
 
@@ -319,7 +319,6 @@ int Net::lstm_create_layer(size_t li)
     if (l.n_cells_per_block == 0) { set_last_error("layer %zu: LSTM needs at least one cell per block", li); return MYEA_E_INVALID; }
     const size_t T = d.number_recurrent_depth, B = d.batch_size;
     const size_t dirs = l.use_bidirectional ? 2 : 1;
-    if (dirs == 2 && !concurrent_directions_disabled()) MYEA_TRY(side_stream_create());
     MYEA_TRY(dev_alloc_zero(&o.neuron_errors, T * B * (size_t)l.n_units * l.n_cells_per_block));  // delta of the layer's output (ptr_delta_cell_output)
     // Two directions (contract of this library: the reference overlays its two directions' buffers and has no behaviour to
     // follow): direction 1 owns the second half of the layer's blocks and the second [G] slice of its biases and walks time
@@ -468,7 +467,7 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
 
 int Net::side_stream_create()
 {
-    if (side_stream) return MYEA_OK;
+    if (side_stream || side_stream_disabled()) return MYEA_OK;
     MYEA_HIP_TRY(hipStreamCreateWithFlags(&side_stream, hipStreamNonBlocking));
     MYEA_HIP_TRY(hipEventCreateWithFlags(&fork_event, hipEventDisableTiming));
     MYEA_HIP_TRY(hipEventCreateWithFlags(&join_event, hipEventDisableTiming));
@@ -572,10 +571,16 @@ void Net::lstm_delta_source(size_t gi, int direction, const float **delta, size_
 
 // Recurrent__Update_Derivative_Weight__LSTM (NN/Neural_Network__Recurrent_Update_Derivative_Weight__OpenMP.cpp:492-728)
 // and __LSTM__Bias (:730-776).
-int Net::lstm_update_derivative_weight(size_t li, size_t B)
+// The weight gradients of an LSTM layer come in two independent parts that write different slots of the gradient:
+// the contractions (input and recurrent weights, matrix-pipe bound) and the column reductions (peepholes and biases,
+// memory bound).  `reductions` selects the part; the caller runs the reductions of all layers beside the contractions.
+int Net::lstm_update_derivative_weight(size_t li, size_t B, bool reductions)
 {
-    MYEA_TRY(lstm_update_derivative_weight_direction(li, *L[li].lstm, B));
-    if (L[li].lstm2) MYEA_TRY(lstm_update_derivative_weight_direction(li, *L[li].lstm2, B));
+    for (LstmLayer *q : {L[li].lstm, L[li].lstm2}) {
+        if (!q) continue;
+        if (reductions) MYEA_TRY(lstm_update_derivative_weight_reductions(*q, B));
+        else MYEA_TRY(lstm_update_derivative_weight_direction(li, *q, B));
+    }
     return MYEA_OK;
 }
 
@@ -642,6 +647,13 @@ int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t
     hipLaunchKernelGGL(lstm_scatter_add_kernel, dim3(grid_for(q.G * (q.In + q.C), kBlock, 4096)), dim3(kBlock), 0, stream, geom, gradient, q.gWin, s_in,
                        q.gWrec, s_rec);
     MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int Net::lstm_update_derivative_weight_reductions(LstmLayer &q, size_t B)
+{
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
+    const LstmGeom geom = geom_of(q);
     // peepholes
     {
         size_t S, chunk;

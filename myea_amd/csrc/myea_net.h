@@ -63,8 +63,9 @@ struct Net {
     myea_hyper h{};
     uint32_t state = MYEA_STATE_INFERENCE;
     hipStream_t stream = nullptr;
-    // The two directions of a bidirectional LSTM layer are independent until their outputs are added: the second one's
-    // launches go to a stream of the library's own (default priority), forked from and joined to `stream` by events.
+    // A stream of the library's own (default priority), forked from and joined to `stream` by events, for work that is
+    // independent of what `stream` is busy with: the second direction of a bidirectional LSTM layer, and the bias /
+    // peephole column reductions of the weight-gradient phase beside its contractions.
     hipStream_t side_stream = nullptr;
     hipEvent_t fork_event = nullptr, join_event = nullptr;
     float *parameters = nullptr, *gradient = nullptr, *opt[MYEA_STATE_KINDS] = {};
@@ -142,7 +143,8 @@ struct Net {
     int lstm_backward_direction(LstmLayer &q, size_t B);
     int lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t B);
     size_t lstm_scratch_floats() const;
-    int lstm_update_derivative_weight(size_t li, size_t B);
+    int lstm_update_derivative_weight(size_t li, size_t B, bool reductions);
+    int lstm_update_derivative_weight_reductions(LstmLayer &q, size_t B);
     const float *lstm_tensor(size_t li, int kind, size_t *count);
 };
 

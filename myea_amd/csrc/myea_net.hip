@@ -303,6 +303,7 @@ int Net::create(const myea_net_desc &desc)
             MYEA_TRY(launch_fill(0, o.variances_averages, T * o.NH, 1.f));  // NN/Neural_Network__Allocate.cpp:2612-2615
         }
     }
+    MYEA_TRY(side_stream_create());
     MYEA_TRY(dev_alloc(&tmp1, T * B * max_h));
     MYEA_TRY(dev_alloc(&tmp2, T * B * max_h));
     {
@@ -970,42 +971,70 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
     if (first < 1 || end > d.n_layers || first > end) { set_last_error("Update_Derivative_Weight: layer range [%zu, %zu) invalid", first, end); return MYEA_E_INVALID; }
     if (B == 0 || B > d.batch_size) { set_last_error("Update_Derivative_Weight: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
-    for (size_t li = first; li < end; ++li) {
-        const myea_layer_desc &l = d.layers[li];
-        if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_update_derivative_weight(li, B)); continue; }
-        if (l.type_layer == MYEA_LAYER_RESIDUAL || layer_is_pooling(l)) continue;  // own no connection (:31-36)
-        DevLayer &o = L[li];
-        const size_t In = o.In, H = o.H;
-        // Layer::ptr_array_pre_summations: the operand the weights were applied to (NN/Neural_Network__Ordered.cpp:96-141)
-        const float *x = layer_outputs(o.prev);
-        if (o.group == 2) x = o.values;
-        else if (o.group == 1 && layer_uses_norm(l)) x = o.normalizes;
-        const bool per_t = T > 1 && B != Bmax;
-        const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
-        for (size_t c = 0; c < chunks; ++c) {
-            const size_t roff = c * Bmax;
-            GemmParams g{};
-            g.A = o.neuron_errors + roff * H; g.lda = (long)H; g.a_k_contiguous = 0;
-            g.B = x + roff * In; g.ldb = (long)In; g.b_k_contiguous = 0;
-            g.C = gradient + l.first_connection_index; g.ldc = (long)In;
-            g.M = (int)H; g.N = (int)In; g.K = (int)rows;
-            g.accumulate = 1; g.epilogue = EPI_NONE;
-            const int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
-            if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
-            const bool done = li < dw_done.size() && dw_done[li];   // rode along with the delta's contraction in this pass
-            if (!done) {
+    const bool per_t = T > 1 && B != Bmax;
+    const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
+    // The column reductions (biases, LSTM peepholes, self weights of independently recurrent layers) read deltas that
+    // are complete before this call and write gradient slots no contraction touches; slots shared between layers (the
+    // LSTM bias addressing reaches into the next layers' biases) are added to in the layers' order, on one stream.
+    auto reductions = [&]() -> int {
+        for (size_t li = first; li < end; ++li) {
+            const myea_layer_desc &l = d.layers[li];
+            if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_update_derivative_weight(li, B, true)); continue; }
+            if (!layer_is_dense(l)) continue;
+            DevLayer &o = L[li];
+            if (layer_uses_bias(l))
+                for (size_t c = 0; c < chunks; ++c)
+                    MYEA_TRY(launch_column_sum(stream, rows, o.H, o.neuron_errors + c * Bmax * o.H, gradient + l.first_bias_connection_index, 1, scratch));
+            if (layer_is_ind_rnn(l))
+                MYEA_TRY(launch_ind_rnn_self_weight_gradient(stream, T, B, Bmax, o.H, o.values, o.dafs_own ? o.dafs_own : o.neuron_errors,
+                                                             gradient + l.first_connection_index + o.H * o.In, scratch));
+        }
+        return MYEA_OK;
+    };
+    auto contractions = [&]() -> int {
+        for (size_t li = first; li < end; ++li) {
+            const myea_layer_desc &l = d.layers[li];
+            if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_update_derivative_weight(li, B, false)); continue; }
+            if (l.type_layer == MYEA_LAYER_RESIDUAL || layer_is_pooling(l)) continue;  // own no connection (:31-36)
+            if (li < dw_done.size() && dw_done[li]) continue;   // rode along with the delta's contraction in this pass
+            DevLayer &o = L[li];
+            const size_t In = o.In, H = o.H;
+            // Layer::ptr_array_pre_summations: the operand the weights were applied to (NN/Neural_Network__Ordered.cpp:96-141)
+            const float *x = layer_outputs(o.prev);
+            if (o.group == 2) x = o.values;
+            else if (o.group == 1 && layer_uses_norm(l)) x = o.normalizes;
+            for (size_t c = 0; c < chunks; ++c) {
+                const size_t roff = c * Bmax;
+                GemmParams g{};
+                g.A = o.neuron_errors + roff * H; g.lda = (long)H; g.a_k_contiguous = 0;
+                g.B = x + roff * In; g.ldb = (long)In; g.b_k_contiguous = 0;
+                g.C = gradient + l.first_connection_index; g.ldc = (long)In;
+                g.M = (int)H; g.N = (int)In; g.K = (int)rows;
+                g.accumulate = 1; g.epilogue = EPI_NONE;
+                const int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
+                if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
                 prof_begin(2);
                 MYEA_TRY(launch_gemm(stream, g));
                 if (slabs > 1) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
                 prof_end(2.0 * (double)rows * (double)H * (double)In);
             }
-            if (layer_uses_bias(l)) MYEA_TRY(launch_column_sum(stream, rows, H, o.neuron_errors + roff * H, gradient + l.first_bias_connection_index, 1, scratch));
         }
-        if (layer_is_ind_rnn(l))
-            MYEA_TRY(launch_ind_rnn_self_weight_gradient(stream, T, B, Bmax, H, o.values, o.dafs_own ? o.dafs_own : o.neuron_errors,
-                                                         gradient + l.first_connection_index + H * In, scratch));
+        return MYEA_OK;
+    };
+    bool any_lstm = false;
+    for (size_t li = 1; li < d.n_layers; ++li) any_lstm = any_lstm || d.layers[li].type_layer == MYEA_LAYER_LSTM;
+    if (any_lstm || !side_stream) {
+        // beside the split-K contractions of LSTM layers the long reductions over T x batch rows were measured to cost
+        // more than they hide: one stream, contractions first
+        MYEA_TRY(contractions());
+        return reductions();
     }
-    return MYEA_OK;
+    {   // memory-bound reductions on the side stream beside the matrix-pipe-bound contractions
+        SideStreamScope side(*this);
+        MYEA_TRY(reductions());
+    }
+    MYEA_TRY(contractions());
+    return side_stream_join();
 }
 
 // Per-unit activation arrays (struct AF_unit: ptr_type_activation_function / ptr_activation_steepness).  With them the
