@@ -90,28 +90,31 @@ __device__ __forceinline__ float tanh_f(float s) { return 2.f / (1.f + expf(-2.f
 __device__ __forceinline__ f32x4 ld4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
 
 // ---- forward -------------------------------------------------------------------------------------------------
-// Tile: 32 examples x 16 cells (64 gate columns z | i | f | o).  Wavefront w sums the k groups w, w + 4, w + 8, ...
+// Tile: 32 examples x CELLS cells (4 CELLS gate columns z | i | f | o), CELLS = 16, or 8 where 16 would leave half of the
+// compute units without a workgroup (small batches).  Wavefront w sums the k groups w, w + 4, w + 8, ...
 // Gate math: Forward_Pass__LSTM__Gates_CIF_AF_State (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:1042-1191),
 // __States_AF (:1547-1582), __Output (:1351-1418), for a step that has a previous step.
-constexpr int kFwdStride = 72;   // floats per row of a wavefront's partial tile in LDS
-
+template <int CELLS>
 __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedForward p)
 {
+    constexpr int NB = 4 * CELLS;               // rows of the weight tile = gate columns of the output tile
+    constexpr int PAIRS = 32 * CELLS / kThreads;   // (example, cell) pairs per lane
+    constexpr int kFwdStride = NB + 8;          // floats per row of a wavefront's partial tile in LDS
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lane32 = lane & 31, half = lane >> 5;
     const int C = (int)p.C, B = (int)p.B;
     int tile_c, tile_r;
-    tile_of(blockIdx.x, C / 16, tile_c, tile_r);
-    const int c0 = tile_c * 16, r0 = tile_r * 32;
+    tile_of(blockIdx.x, C / CELLS, tile_c, tile_r);
+    const int c0 = tile_c * CELLS, r0 = tile_r * 32;
     const int ng = (C / 32 - wave + 3) / 4;          // this wavefront's groups of 32 k: wave, wave + 4, wave + 8, ...
-    constexpr int kStage = (32 + 64) * 32;           // floats: A tile 32 x 32, then B tile 64 x 32
+    constexpr int kStage = (32 + NB) * 32;           // floats: A tile 32 x 32, then B tile NB x 32
     float *stage0 = smem + wave * kFwdStages * kStage;
 
-    // what the gate math of this lane's two (example, cell) pairs reads does not depend on the contraction: fetch it now
-    float e_in[2][4], e_bias[2][4], e_peep[2][3], e_cp[2];
+    // what the gate math of this lane's (example, cell) pairs reads does not depend on the contraction: fetch it now
+    float e_in[PAIRS][4], e_bias[PAIRS][4], e_peep[PAIRS][3], e_cp[PAIRS];
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        const int pair = threadIdx.x + q * kThreads, row = pair >> 4, cell = pair & 15;
+    for (int q = 0; q < PAIRS; ++q) {
+        const int pair = threadIdx.x + q * kThreads, row = pair / CELLS, cell = pair % CELLS;
         const int b = min(r0 + row, B - 1), k = c0 + cell;
         const float *arow = p.acts + (size_t)b * 4 * C;
 #pragma unroll
@@ -126,10 +129,10 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
     for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
     if (ng > 0) {
         WaveTile<32> ta;
-        WaveTile<64> tb;
+        WaveTile<NB> tb;
         ta.init(p.h_prev, (size_t)C, (size_t)wave * 32, [&](int r) { return (size_t)min(r0 + r, B - 1); });
-        // tile row j of B is gate j / 16 of cell c0 + j % 16: row gate * C + cell of the packed matrix
-        tb.init(p.Wrec, (size_t)C, (size_t)wave * 32, [&](int r) { return (size_t)(r >> 4) * C + c0 + (r & 15); });
+        // tile row j of B is gate j / CELLS of cell c0 + j % CELLS: row gate * C + cell of the packed matrix
+        tb.init(p.Wrec, (size_t)C, (size_t)wave * 32, [&](int r) { return (size_t)(r / CELLS) * C + c0 + (r % CELLS); });
         ta.fill(stage0, 128);
         tb.fill(stage0 + 32 * 32, 128);
         for (int g = 0; g < ng; ++g) {
@@ -138,7 +141,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
                 float *nxt = stage0 + ((g + 1) & 1) * kStage;
                 ta.fill(nxt, 128);
                 tb.fill(nxt + 32 * 32, 128);
-                wait_loads<12>();
+                wait_loads<4 + NB / 8>();   // the loads just issued may stay in flight
             } else {
                 wait_loads<0>();
             }
@@ -146,21 +149,21 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
             // fragments of k group kg + 1 are read while the MFMAs of group kg issue
             f32x4 fa[2], fb0[2], fb1[2];
             fa[0] = WaveTile<32>::chunk(la, lane32, half);
-            fb0[0] = WaveTile<64>::chunk(lb, lane32, half);
-            fb1[0] = WaveTile<64>::chunk(lb, 32 + lane32, half);
+            fb0[0] = WaveTile<NB>::chunk(lb, lane32, half);
+            if constexpr (NB == 64) fb1[0] = WaveTile<NB>::chunk(lb, 32 + lane32, half);
 #pragma unroll
             for (int kg = 0; kg < 4; ++kg) {
                 const int cb = kg & 1, nb = cb ^ 1;
                 if (kg + 1 < 4) {
                     fa[nb] = WaveTile<32>::chunk(la, lane32, (kg + 1) * 2 + half);
-                    fb0[nb] = WaveTile<64>::chunk(lb, lane32, (kg + 1) * 2 + half);
-                    fb1[nb] = WaveTile<64>::chunk(lb, 32 + lane32, (kg + 1) * 2 + half);
+                    fb0[nb] = WaveTile<NB>::chunk(lb, lane32, (kg + 1) * 2 + half);
+                    if constexpr (NB == 64) fb1[nb] = WaveTile<NB>::chunk(lb, 32 + lane32, (kg + 1) * 2 + half);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
                     acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][s], fb0[cb][s], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][s], fb1[cb][s], acc1, 0, 0, 0);
+                    if constexpr (NB == 64) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][s], fb1[cb][s], acc1, 0, 0, 0);
                 }
             }
         }
@@ -172,13 +175,13 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
     for (int r = 0; r < 16; ++r) {
         const int row = (r >> 2) * 8 + half * 4 + (r & 3);
         mine[row * kFwdStride + lane32] = acc0[r];
-        mine[row * kFwdStride + 32 + lane32] = acc1[r];
+        if constexpr (NB == 64) mine[row * kFwdStride + 32 + lane32] = acc1[r];
     }
     __syncthreads();
-    // 32 x 16 (example, cell) pairs, two per lane
+    // 32 x CELLS (example, cell) pairs
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        const int pair = threadIdx.x + q * kThreads, row = pair >> 4, cell = pair & 15;
+    for (int q = 0; q < PAIRS; ++q) {
+        const int pair = threadIdx.x + q * kThreads, row = pair / CELLS, cell = pair % CELLS;
         const int b = r0 + row;
         if (b >= B) continue;
         float rec[4];
@@ -186,7 +189,7 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
         for (int gate = 0; gate < 4; ++gate) {
             float v = 0.f;
 #pragma unroll
-            for (int w = 0; w < 4; ++w) v += part[(w * 32 + row) * kFwdStride + gate * 16 + cell];
+            for (int w = 0; w < 4; ++w) v += part[(w * 32 + row) * kFwdStride + gate * CELLS + cell];
             rec[gate] = v;
         }
         const int k = c0 + cell;
@@ -213,29 +216,33 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_forward_kernel(LstmFusedF
 
 // ---- backward ------------------------------------------------------------------------------------------------
 // dh[t] += dG[t'] Wrec (t' = the step processed after t), then the gate deltas of step t.
-// Tile: 32 examples x 16 cells; wavefront w sums the k range of gate w (k = gate * C + cell of dG[t']), reading the
-// transposed packed matrix WrecT [C][4C] so that both operands are k-contiguous.
+// Tile: ROWS examples x 16 cells (ROWS = 32, or 16 for small batches, as in the forward step); wavefront w sums the k
+// range of gate w (k = gate * C + cell of dG[t']), reading the transposed packed matrix WrecT [C][4C] so that both
+// operands are k-contiguous.
 // Gate math: Backward_Pass__LSTM_Derivative__Output (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:1228-1240),
 // __Cell_State_AF (:1275-1327), __Gates_CIF_AF_State (:1329-1604) for a step that has a following step; `first_step`:
 // the sequence's first step writes no forget-gate delta (:1460-1534).
 constexpr int kBwdStride = 17;
 
+template <int ROWS>
 __global__ __launch_bounds__(kThreads) void lstm_fused_backward_kernel(LstmFusedBackward p)
 {
+    constexpr int PAIRS = ROWS * 16 / kThreads;   // (example, cell) pairs per lane
+    constexpr int kLoads = ROWS / 8 + 2;          // direct loads per stage and wavefront
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lane16 = lane & 15, quad = lane >> 4;
     const int C = (int)p.C, B = (int)p.B, G = 4 * C;
     int tile_c, tile_r;
     tile_of(blockIdx.x, C / 16, tile_c, tile_r);
-    const int c0 = tile_c * 16, r0 = tile_r * 32;
+    const int c0 = tile_c * 16, r0 = tile_r * ROWS;
     const int ng = C / 32;   // groups of 32 k in this wavefront's range of C
-    constexpr int kStage = (32 + 16) * 32;   // floats: A tile 32 x 32 (rows of dG[t']), then B tile 16 x 32 (rows of WrecT)
+    constexpr int kStage = (ROWS + 16) * 32;   // floats: A tile ROWS x 32 (rows of dG[t']), then B tile 16 x 32 (rows of WrecT)
     float *stage0 = smem + wave * kBwdStages * kStage;
 
-    // operands of the gate math of this lane's two (example, cell) pairs, fetched ahead of the contraction
-    float e_dh[2], e_act[2][4], e_ca[2], e_din[2], e_dfn[2], e_fn[2], e_peep[2][3], e_dcn[2], e_cp[2];
+    // operands of the gate math of this lane's (example, cell) pairs, fetched ahead of the contraction
+    float e_dh[PAIRS], e_act[PAIRS][4], e_ca[PAIRS], e_din[PAIRS], e_dfn[PAIRS], e_fn[PAIRS], e_peep[PAIRS][3], e_dcn[PAIRS], e_cp[PAIRS];
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+    for (int q = 0; q < PAIRS; ++q) {
         const int pair = threadIdx.x + q * kThreads, row = pair >> 4, cell = pair & 15;
         const int b = min(r0 + row, B - 1), k = c0 + cell;
         const size_t ci = (size_t)b * C + k, gi_ = (size_t)b * G;
@@ -251,34 +258,34 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_backward_kernel(LstmFused
     }
 
     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-    WaveTile<32> ta;
+    WaveTile<ROWS> ta;
     WaveTile<16> tb;
     ta.init(p.dG_next, (size_t)G, (size_t)wave * C, [&](int r) { return (size_t)min(r0 + r, B - 1); });
     tb.init(p.WrecT, (size_t)G, (size_t)wave * C, [&](int r) { return (size_t)(c0 + r); });
     // stages g + 1 .. g + 3 are in flight while group g computes
 #pragma unroll
     for (int u = 0; u < kBwdStages - 1; ++u)
-        if (u < ng) { ta.fill(stage0 + u * kStage, 32); tb.fill(stage0 + u * kStage + 32 * 32, 32); }
+        if (u < ng) { ta.fill(stage0 + u * kStage, 32); tb.fill(stage0 + u * kStage + ROWS * 32, 32); }
     for (int g = 0; g < ng; ++g) {
         const float *cur = stage0 + (g & (kBwdStages - 1)) * kStage;
         if (g + kBwdStages - 1 < ng) {   // that stage was last read by the MFMAs of group g - 1
             float *nxt = stage0 + ((g + kBwdStages - 1) & (kBwdStages - 1)) * kStage;
             ta.fill(nxt, 32);
-            tb.fill(nxt + 32 * 32, 32);
-            wait_loads<18>();
+            tb.fill(nxt + ROWS * 32, 32);
+            wait_loads<3 * kLoads>();
         } else if (g + 2 < ng) {
-            wait_loads<12>();
+            wait_loads<2 * kLoads>();
         } else if (g + 1 < ng) {
-            wait_loads<6>();
+            wait_loads<kLoads>();
         } else {
             wait_loads<0>();
         }
-        const float *la = cur, *lb = cur + 32 * 32;
+        const float *la = cur, *lb = cur + ROWS * 32;
         f32x4 fa0[2], fa1[2], fb[2];
 #pragma unroll
         for (int kg = 0; kg < 2; ++kg) {
-            fa0[kg] = WaveTile<32>::chunk(la, lane16, kg * 4 + quad);
-            fa1[kg] = WaveTile<32>::chunk(la, 16 + lane16, kg * 4 + quad);
+            fa0[kg] = WaveTile<ROWS>::chunk(la, lane16, kg * 4 + quad);
+            if constexpr (ROWS == 32) fa1[kg] = WaveTile<ROWS>::chunk(la, 16 + lane16, kg * 4 + quad);
             fb[kg] = WaveTile<16>::chunk(lb, lane16, kg * 4 + quad);
         }
 #pragma unroll
@@ -286,26 +293,26 @@ __global__ __launch_bounds__(kThreads) void lstm_fused_backward_kernel(LstmFused
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(fa0[kg][s], fb[kg][s], acc0, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(fa1[kg][s], fb[kg][s], acc1, 0, 0, 0);
+                if constexpr (ROWS == 32) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(fa1[kg][s], fb[kg][s], acc1, 0, 0, 0);
             }
     }
     __syncthreads();   // every wavefront is done with its stages: the partial tiles reuse the memory
     float *part = smem;
-    float *mine = part + wave * 32 * kBwdStride;
+    float *mine = part + wave * ROWS * kBwdStride;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         mine[(quad * 4 + r) * kBwdStride + lane16] = acc0[r];
-        mine[(16 + quad * 4 + r) * kBwdStride + lane16] = acc1[r];
+        if constexpr (ROWS == 32) mine[(16 + quad * 4 + r) * kBwdStride + lane16] = acc1[r];
     }
     __syncthreads();
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+    for (int q = 0; q < PAIRS; ++q) {
         const int pair = threadIdx.x + q * kThreads, row = pair >> 4, cell = pair & 15;
         const int b = r0 + row;
         if (b >= B) continue;
         float rec = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) rec += part[(w * 32 + row) * kBwdStride + cell];
+        for (int w = 0; w < 4; ++w) rec += part[(w * ROWS + row) * kBwdStride + cell];
         const int k = c0 + cell;
         const size_t ci = (size_t)b * C + k, gi_ = (size_t)b * G;
         const float dh = e_dh[q] + rec;
@@ -346,6 +353,27 @@ bool aligned16(const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) ==
 
 bool lstm_fused_supported(size_t C, size_t cells_per_block) { return cells_per_block == 1 && C >= 32 && C % 32 == 0 && C <= (1u << 20); }
 
+// Half-size tiles where the full-size tiling would give at most half of the 256 compute units a workgroup (small batches):
+// twice the workgroups, each with half the contraction work, and two of them fit a compute unit's LDS.
+static bool narrow_tiles(size_t B, size_t C) { return ((B + 31) / 32) * (C / 16) <= 128; }
+
+template <int CELLS>
+static int launch_forward(hipStream_t s, const LstmFusedForward &p)
+{
+    const size_t blocks = ((p.B + 31) / 32) * (p.C / CELLS);
+    if (blocks > 0x7fffffffu) { set_last_error("fused LSTM forward step: grid out of range"); return MYEA_E_INVALID; }
+    constexpr size_t lds = (size_t)4 * kFwdStages * (32 + 4 * CELLS) * 32 * sizeof(float);
+    static_assert(lds >= 4 * 32 * (4 * CELLS + 8) * sizeof(float), "the partial tiles reuse the stages");
+    static bool attr_done = false;
+    if (!attr_done) {
+        MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(lstm_fused_forward_kernel<CELLS>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(lstm_fused_forward_kernel<CELLS>, dim3((unsigned)blocks), dim3(kThreads), lds, s, p);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
 int launch_lstm_fused_forward(hipStream_t s, const LstmFusedForward &p)
 {
     if (p.B == 0) return MYEA_OK;
@@ -354,16 +382,22 @@ int launch_lstm_fused_forward(hipStream_t s, const LstmFusedForward &p)
         set_last_error("fused LSTM forward step: unsupported shape or operand (C = %zu)", p.C);
         return MYEA_E_INVALID;
     }
-    const size_t blocks = ((p.B + 31) / 32) * (p.C / 16);
-    if (blocks > 0x7fffffffu) { set_last_error("fused LSTM forward step: grid out of range"); return MYEA_E_INVALID; }
-    constexpr size_t lds = (size_t)4 * kFwdStages * (32 + 64) * 32 * sizeof(float);
-    static_assert(lds >= 4 * 32 * kFwdStride * sizeof(float), "the partial tiles reuse the stages");
+    return narrow_tiles(p.B, p.C) ? launch_forward<8>(s, p) : launch_forward<16>(s, p);
+}
+
+template <int ROWS>
+static int launch_backward(hipStream_t s, const LstmFusedBackward &p)
+{
+    const size_t blocks = ((p.B + ROWS - 1) / ROWS) * (p.C / 16);
+    if (blocks > 0x7fffffffu) { set_last_error("fused LSTM backward step: grid out of range"); return MYEA_E_INVALID; }
+    constexpr size_t lds = (size_t)4 * kBwdStages * (ROWS + 16) * 32 * sizeof(float);
+    static_assert(lds >= 4 * ROWS * kBwdStride * sizeof(float), "the partial tiles reuse the stages");
     static bool attr_done = false;
     if (!attr_done) {
-        MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(lstm_fused_forward_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(lstm_fused_backward_kernel<ROWS>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_done = true;
     }
-    hipLaunchKernelGGL(lstm_fused_forward_kernel, dim3((unsigned)blocks), dim3(kThreads), lds, s, p);
+    hipLaunchKernelGGL(lstm_fused_backward_kernel<ROWS>, dim3((unsigned)blocks), dim3(kThreads), lds, s, p);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
@@ -376,18 +410,7 @@ int launch_lstm_fused_backward(hipStream_t s, const LstmFusedBackward &p)
         set_last_error("fused LSTM backward step: unsupported shape or operand (C = %zu)", p.C);
         return MYEA_E_INVALID;
     }
-    const size_t blocks = ((p.B + 31) / 32) * (p.C / 16);
-    if (blocks > 0x7fffffffu) { set_last_error("fused LSTM backward step: grid out of range"); return MYEA_E_INVALID; }
-    constexpr size_t lds = (size_t)4 * kBwdStages * (32 + 16) * 32 * sizeof(float);
-    static_assert(lds >= 4 * 32 * kBwdStride * sizeof(float), "the partial tiles reuse the stages");
-    static bool attr_done = false;
-    if (!attr_done) {
-        MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(lstm_fused_backward_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_done = true;
-    }
-    hipLaunchKernelGGL(lstm_fused_backward_kernel, dim3((unsigned)blocks), dim3(kThreads), lds, s, p);
-    MYEA_HIP_TRY(hipGetLastError());
-    return MYEA_OK;
+    return narrow_tiles(p.B, p.C) ? launch_backward<16>(s, p) : launch_backward<32>(s, p);
 }
 
 int launch_transpose(hipStream_t s, size_t rows, size_t cols, const float *src, float *dst)
