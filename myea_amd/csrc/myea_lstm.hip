@@ -408,12 +408,11 @@ int Net::lstm_parameters_changed()
 
 // Recurrent__Forward_Pass__LSTM (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:448-471): time ascending, or
 // descending for the second direction (the "previous" step is then t + 1, :456-461).
-int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
+// Input sums of every time step in one contraction when the rows are contiguous.
+int Net::lstm_forward_inputs(size_t li, LstmLayer &q, size_t B)
 {
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
     const float *x = layer_outputs(L[li].prev);
-    const float *bias = parameters + q.bias;
-    // input sums of every time step in one contraction when the rows are contiguous
     const bool per_t = T > 1 && B != Bmax;
     const size_t chunks = per_t ? T : 1, rows = per_t ? B : T * B;
     for (size_t c = 0; c < chunks; ++c) {
@@ -426,42 +425,43 @@ int Net::lstm_forward_direction(size_t li, LstmLayer &q, size_t B)
         MYEA_TRY(launch_gemm(stream, g));
         prof_end(2.0 * (double)rows * (double)q.G * (double)q.In);
     }
-    const LstmGeom geom = geom_of(q);
-    // One pair of timing events brackets the whole time loop: a pair per step costs more than the 10 us steps it would time.
-    if (T > 1) prof_begin(0);
-    for (size_t s = 0; s < T; ++s) {
-        const size_t t = q.reverse ? T - 1 - s : s, tp = q.reverse ? t + 1 : t - 1;  // tp: the step processed before t
-        float *acts_t = q.acts + t * Bmax * q.G;
-        // zoneout acts strictly in the training state (NN/Neural_Network__Forward_Pass__Loop.cpp:2088-2092)
-        const bool zone = q.zone_state != nullptr && state == MYEA_STATE_TRAINING;
-        const uint8_t *zs = zone ? q.zone_state + t * q.zone_stride : nullptr, *zo = zone ? q.zone_output + t * q.zone_stride : nullptr;
-        int nparts = 0;
-        if (s > 0 && q.fused) {   // recurrent contraction and gate math of the step in one launch
-            LstmFusedForward f{};
-            f.B = B; f.C = q.C;
-            f.h_prev = q.h + tp * Bmax * q.C; f.Wrec = q.Wrec; f.bias = bias; f.peep = q.peep;
-            f.acts = acts_t; f.c_prev = q.c + tp * Bmax * q.C;
-            f.c = q.c + t * Bmax * q.C; f.ca = q.ca + t * Bmax * q.C; f.h = q.h + t * Bmax * q.C;
-            f.zone_state = zs; f.zone_output = zo;
-            MYEA_TRY(launch_lstm_fused_forward(stream, f));
-            continue;
-        }
-        if (s > 0) {
-            GemmParams g{};
-            g.A = q.h + tp * Bmax * q.C; g.lda = (long)q.C; g.a_k_contiguous = 1;
-            g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 1;
-            g.C = q.part; g.ldc = (long)q.G;
-            g.M = (int)B; g.N = (int)q.G; g.K = (int)q.C;
-            nparts = gemm_split_k(g.M, g.N, g.K);
-            g.split_k = nparts; g.split_k_slab = (long)(B * q.G);
-            MYEA_TRY(launch_gemm(stream, g));
-        }
-        hipLaunchKernelGGL(lstm_forward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, (int)(s == 0), bias, q.peep,
-                           acts_t, s ? q.c + tp * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, q.h + t * Bmax * q.C,
-                           q.part, nparts, s ? q.h + tp * Bmax * q.C : nullptr, zs, zo);
-        MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+// the s-th time step the direction processes
+int Net::lstm_forward_step(LstmLayer &q, size_t B, size_t s)
+{
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
+    const float *bias = parameters + q.bias;
+    const size_t t = q.reverse ? T - 1 - s : s, tp = q.reverse ? t + 1 : t - 1;  // tp: the step processed before t
+    float *acts_t = q.acts + t * Bmax * q.G;
+    // zoneout acts strictly in the training state (NN/Neural_Network__Forward_Pass__Loop.cpp:2088-2092)
+    const bool zone = q.zone_state != nullptr && state == MYEA_STATE_TRAINING;
+    const uint8_t *zs = zone ? q.zone_state + t * q.zone_stride : nullptr, *zo = zone ? q.zone_output + t * q.zone_stride : nullptr;
+    int nparts = 0;
+    if (s > 0 && q.fused) {   // recurrent contraction and gate math of the step in one launch
+        LstmFusedForward f{};
+        f.B = B; f.C = q.C;
+        f.h_prev = q.h + tp * Bmax * q.C; f.Wrec = q.Wrec; f.bias = bias; f.peep = q.peep;
+        f.acts = acts_t; f.c_prev = q.c + tp * Bmax * q.C;
+        f.c = q.c + t * Bmax * q.C; f.ca = q.ca + t * Bmax * q.C; f.h = q.h + t * Bmax * q.C;
+        f.zone_state = zs; f.zone_output = zo;
+        return launch_lstm_fused_forward(stream, f);
     }
-    if (T > 1) prof_end(2.0 * (double)(T - 1) * (double)B * (double)q.G * (double)q.C, T - 1);   // the recurrent contractions of steps 1 .. T-1
+    if (s > 0) {
+        GemmParams g{};
+        g.A = q.h + tp * Bmax * q.C; g.lda = (long)q.C; g.a_k_contiguous = 1;
+        g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 1;
+        g.C = q.part; g.ldc = (long)q.G;
+        g.M = (int)B; g.N = (int)q.G; g.K = (int)q.C;
+        nparts = gemm_split_k(g.M, g.N, g.K);
+        g.split_k = nparts; g.split_k_slab = (long)(B * q.G);
+        MYEA_TRY(launch_gemm(stream, g));
+    }
+    hipLaunchKernelGGL(lstm_forward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom_of(q), B, (int)(s == 0), bias, q.peep,
+                       acts_t, s ? q.c + tp * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, q.h + t * Bmax * q.C,
+                       q.part, nparts, s ? q.h + tp * Bmax * q.C : nullptr, zs, zo);
+    MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
 
@@ -480,84 +480,116 @@ int Net::side_stream_join()
     return MYEA_OK;
 }
 
+// One pair of timing events brackets a whole time loop: a pair per step costs more than the 10 us steps it would time.
+// Two directions: their steps are enqueued alternately, the second direction's on the side stream, so that neither
+// direction's launches wait behind the other's on the host; the event pair then brackets both loops.
 int Net::lstm_forward_layer(size_t li, size_t B)
 {
     DevLayer &o = L[li];
-    if (o.lstm2) {
-        {   // the second direction beside the first (on the same stream, in this order, without a side stream)
-            SideStreamScope side(*this);
-            MYEA_TRY(lstm_forward_direction(li, *o.lstm2, B));
-        }
-        MYEA_TRY(lstm_forward_direction(li, *o.lstm, B));
-        MYEA_TRY(side_stream_join());
-        const size_t rows = (size_t)d.number_recurrent_depth * d.batch_size;
-        MYEA_TRY(launch_padded_add(stream, rows, o.H, o.lstm->h, o.H, 0, o.lstm2->h, o.H, 0, o.values));  // output = h_forward + h_backward
+    const size_t T = d.number_recurrent_depth;
+    const double loop_work = 2.0 * (double)(T - 1) * (double)B * (double)o.lstm->G * (double)o.lstm->C;   // the recurrent contractions of steps 1 .. T-1
+    if (!o.lstm2) {
+        MYEA_TRY(lstm_forward_inputs(li, *o.lstm, B));
+        if (T > 1) prof_begin(0);
+        for (size_t s = 0; s < T; ++s) MYEA_TRY(lstm_forward_step(*o.lstm, B, s));
+        if (T > 1) prof_end(loop_work, T - 1);
         return MYEA_OK;
     }
-    return lstm_forward_direction(li, *o.lstm, B);
+    {
+        SideStreamScope side(*this);
+        MYEA_TRY(lstm_forward_inputs(li, *o.lstm2, B));
+        if (side.active) std::swap(stream, side_stream);   // back on the caller's stream while the scope stays open
+        int rc = lstm_forward_inputs(li, *o.lstm, B);
+        if (T > 1) prof_begin(0);
+        for (size_t s = 0; s < T && rc == MYEA_OK; ++s) {
+            if (side.active) std::swap(stream, side_stream);
+            rc = lstm_forward_step(*o.lstm2, B, s);
+            if (side.active) std::swap(stream, side_stream);
+            if (rc == MYEA_OK) rc = lstm_forward_step(*o.lstm, B, s);
+        }
+        if (side.active) std::swap(stream, side_stream);   // the scope's end expects the side stream in place
+        MYEA_TRY(rc);
+    }
+    MYEA_TRY(side_stream_join());
+    if (T > 1) prof_end(2.0 * loop_work, 2 * (T - 1));
+    const size_t rows = (size_t)d.number_recurrent_depth * d.batch_size;
+    return launch_padded_add(stream, rows, o.H, o.lstm->h, o.H, 0, o.lstm2->h, o.H, 0, o.values);  // output = h_forward + h_backward
 }
 
 // Recurrent__Backward_Pass__Gradient__LSTM (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:440-862), time
 // descending; o.neuron_errors (= delta of the cell outputs) already holds what the layers above sent down.
-int Net::lstm_backward_direction(LstmLayer &q, size_t B)
+// `s` counts down from T - 1: the s-th time step of the direction's own order.
+int Net::lstm_backward_step(LstmLayer &q, size_t B, size_t s)
 {
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
-    const LstmGeom geom = geom_of(q);
-    if (T > 1) prof_begin(1);   // one pair of timing events for the whole time loop
-    for (size_t s = T; s-- > 0;) {
-        // tn / tp: the steps processed after / before t in the direction's own order
-        const size_t t = q.reverse ? T - 1 - s : s, tn = q.reverse ? t - 1 : t + 1, tp = q.reverse ? t + 1 : t - 1;
-        float *dh_t = q.dh + t * Bmax * q.C;
-        const bool last = s == T - 1, first = s == 0;
-        int nparts = 0;
-        if (!last && q.fused) {   // dh[t] += dG[tn] Wrec and the gate deltas of step t in one launch
-            LstmFusedBackward f{};
-            f.B = B; f.C = q.C; f.first_step = first;
-            f.dG_next = q.dG + tn * Bmax * q.G; f.WrecT = q.WrecT; f.peep = q.peep;
-            f.acts = q.acts + t * Bmax * q.G; f.acts_next = q.acts + tn * Bmax * q.G;
-            f.c_prev = first ? nullptr : q.c + tp * Bmax * q.C; f.ca = q.ca + t * Bmax * q.C;
-            f.dh = dh_t; f.dG = q.dG + t * Bmax * q.G; f.dc = q.dc + t * Bmax * q.C; f.dc_next = q.dc + tn * Bmax * q.C;
-            MYEA_TRY(launch_lstm_fused_backward(stream, f));
-            continue;
-        }
-        if (!last) {  // Backward_Pass__LSTM_Derivative__Output, recurrent part (:1174-1226)
-            GemmParams g{};
-            g.A = q.dG + tn * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 1;
-            g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 0;
-            g.C = q.part; g.ldc = (long)q.C;
-            g.M = (int)B; g.N = (int)q.C; g.K = (int)q.G;
-            nparts = gemm_split_k(g.M, g.N, g.K);
-            g.split_k = nparts; g.split_k_slab = (long)(B * q.C);
-            MYEA_TRY(launch_gemm(stream, g));
-        }
-        const int mode = (first && last) ? 0 : (last ? 1 : (first ? 3 : 2));
-        hipLaunchKernelGGL(lstm_backward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom, B, mode, q.peep,
-                           q.acts + t * Bmax * q.G, last ? nullptr : q.acts + tn * Bmax * q.G, first ? nullptr : q.c + tp * Bmax * q.C,
-                           q.ca + t * Bmax * q.C, dh_t, q.dG + t * Bmax * q.G, last ? nullptr : q.dG + tn * Bmax * q.G,
-                           q.dc + t * Bmax * q.C, last ? nullptr : q.dc + tn * Bmax * q.C, q.part, nparts);
-        MYEA_HIP_TRY(hipGetLastError());
+    // tn / tp: the steps processed after / before t in the direction's own order
+    const size_t t = q.reverse ? T - 1 - s : s, tn = q.reverse ? t - 1 : t + 1, tp = q.reverse ? t + 1 : t - 1;
+    float *dh_t = q.dh + t * Bmax * q.C;
+    const bool last = s == T - 1, first = s == 0;
+    int nparts = 0;
+    if (!last && q.fused) {   // dh[t] += dG[tn] Wrec and the gate deltas of step t in one launch
+        LstmFusedBackward f{};
+        f.B = B; f.C = q.C; f.first_step = first;
+        f.dG_next = q.dG + tn * Bmax * q.G; f.WrecT = q.WrecT; f.peep = q.peep;
+        f.acts = q.acts + t * Bmax * q.G; f.acts_next = q.acts + tn * Bmax * q.G;
+        f.c_prev = first ? nullptr : q.c + tp * Bmax * q.C; f.ca = q.ca + t * Bmax * q.C;
+        f.dh = dh_t; f.dG = q.dG + t * Bmax * q.G; f.dc = q.dc + t * Bmax * q.C; f.dc_next = q.dc + tn * Bmax * q.C;
+        return launch_lstm_fused_backward(stream, f);
     }
-    if (T > 1) prof_end(2.0 * (double)(T - 1) * (double)B * (double)q.G * (double)q.C, T - 1);
+    if (!last) {  // Backward_Pass__LSTM_Derivative__Output, recurrent part (:1174-1226)
+        GemmParams g{};
+        g.A = q.dG + tn * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 1;
+        g.B = q.Wrec; g.ldb = (long)q.C; g.b_k_contiguous = 0;
+        g.C = q.part; g.ldc = (long)q.C;
+        g.M = (int)B; g.N = (int)q.C; g.K = (int)q.G;
+        nparts = gemm_split_k(g.M, g.N, g.K);
+        g.split_k = nparts; g.split_k_slab = (long)(B * q.C);
+        MYEA_TRY(launch_gemm(stream, g));
+    }
+    const int mode = (first && last) ? 0 : (last ? 1 : (first ? 3 : 2));
+    hipLaunchKernelGGL(lstm_backward_step_kernel, dim3(grid_for(B * q.K, kBlock, 8192)), dim3(kBlock), 0, stream, geom_of(q), B, mode, q.peep,
+                       q.acts + t * Bmax * q.G, last ? nullptr : q.acts + tn * Bmax * q.G, first ? nullptr : q.c + tp * Bmax * q.C,
+                       q.ca + t * Bmax * q.C, dh_t, q.dG + t * Bmax * q.G, last ? nullptr : q.dG + tn * Bmax * q.G,
+                       q.dc + t * Bmax * q.C, last ? nullptr : q.dc + tn * Bmax * q.C, q.part, nparts);
+    MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
 
 int Net::lstm_backward_layer(size_t li, size_t B)
 {
     DevLayer &o = L[li];
-    auto one = [&](LstmLayer &q) -> int {
-        if (q.own_h)  // both directions start from the same delta of the layer's output
+    const size_t T = d.number_recurrent_depth;
+    const double loop_work = 2.0 * (double)(T - 1) * (double)B * (double)o.lstm->G * (double)o.lstm->C;
+    auto seed = [&](LstmLayer &q) -> int {   // both directions start from the same delta of the layer's output
+        if (q.own_h)
             MYEA_HIP_TRY(hipMemcpyAsync(q.dh, o.neuron_errors, (size_t)d.number_recurrent_depth * d.batch_size * q.C * sizeof(float), hipMemcpyDeviceToDevice, stream));
-        return lstm_backward_direction(q, B);
+        return MYEA_OK;
     };
-    if (o.lstm2) {
-        {
-            SideStreamScope side(*this);
-            MYEA_TRY(one(*o.lstm2));
-        }
-        MYEA_TRY(one(*o.lstm));
-        return side_stream_join();
+    if (!o.lstm2) {
+        MYEA_TRY(seed(*o.lstm));
+        if (T > 1) prof_begin(1);
+        for (size_t s = T; s-- > 0;) MYEA_TRY(lstm_backward_step(*o.lstm, B, s));
+        if (T > 1) prof_end(loop_work, T - 1);
+        return MYEA_OK;
     }
-    return one(*o.lstm);
+    {
+        SideStreamScope side(*this);
+        MYEA_TRY(seed(*o.lstm2));
+        if (side.active) std::swap(stream, side_stream);
+        int rc = seed(*o.lstm);
+        if (T > 1) prof_begin(1);
+        for (size_t s = T; s-- > 0 && rc == MYEA_OK;) {
+            if (side.active) std::swap(stream, side_stream);
+            rc = lstm_backward_step(*o.lstm2, B, s);
+            if (side.active) std::swap(stream, side_stream);
+            if (rc == MYEA_OK) rc = lstm_backward_step(*o.lstm, B, s);
+        }
+        if (side.active) std::swap(stream, side_stream);
+        MYEA_TRY(rc);
+    }
+    MYEA_TRY(side_stream_join());
+    if (T > 1) prof_end(2.0 * loop_work, 2 * (T - 1));
+    return MYEA_OK;
 }
 
 // the operands of "delta of the layer below = dG Win" (Backward_Pass__LSTM, :1024-1120), handed to the shared driver

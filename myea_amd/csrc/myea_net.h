@@ -139,8 +139,9 @@ struct Net {
     void lstm_delta_source(size_t gi, int direction, const float **delta, size_t *width, const float **weights);
     int side_stream_create();
     int side_stream_join();            // `stream` waits for what the last SideStreamScope enqueued
-    int lstm_forward_direction(size_t li, LstmLayer &q, size_t B);
-    int lstm_backward_direction(LstmLayer &q, size_t B);
+    int lstm_forward_inputs(size_t li, LstmLayer &q, size_t B);
+    int lstm_forward_step(LstmLayer &q, size_t B, size_t s);
+    int lstm_backward_step(LstmLayer &q, size_t B, size_t s);
     int lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t B);
     size_t lstm_scratch_floats() const;
     int lstm_update_derivative_weight(size_t li, size_t B, bool reductions);
