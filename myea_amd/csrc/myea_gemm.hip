@@ -434,10 +434,13 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f32_mfma_kernel(GemmDev p)
 // four times as many, quarter as long.  Launched together, a CU holds one long dX workgroup next to a succession of
 // dW workgroups: two wavefronts per SIMD throughout, and the dW tiles' stores fall at different moments behind
 // the dX workgroup's MFMAs instead of all at once.
+// At a batch of 512 the same holds one size down: dX as 64 x 64 tiles (256 of them for 2048-wide layers) beside dW as
+// 128 x 128 tiles over the short k = batch, equal work per workgroup, one of each per CU.
+template <int BMA, int BNA>
 __global__ __launch_bounds__(kThreads, 2) void gemm_pair_kernel(GemmDev a, GemmDev b, int first_blocks)
 {
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    if ((int)blockIdx.x < first_blocks) gemm_tile<128, 128, true, false, true>(a, (int)blockIdx.x, smem);
+    if ((int)blockIdx.x < first_blocks) gemm_tile<BMA, BNA, true, false, true>(a, (int)blockIdx.x, smem);
     else gemm_tile<128, 128, false, false, true>(b, (int)blockIdx.x - first_blocks, smem);
 }
 
@@ -589,20 +592,41 @@ int launch_gemm_pair(hipStream_t stream, const GemmParams &a, const GemmParams &
     rc = prepare_gemm(b, db, &vb);
     if (rc != MYEA_OK) return rc;
     if (!va || !vb) return 1;
-    da.nbm = (a.M + 127) / 128; da.nbn = (a.N + 127) / 128;
     db.nbm = (b.M + 127) / 128; db.nbn = (b.N + 127) / 128;
-    const long na = (long)da.nbm * da.nbn, nb = (long)db.nbm * db.nbn;
-    // worth it when `a` alone would leave the CUs with one workgroup each and `b` brings at least as much work in shorter pieces
-    if (na < 128 || na > 256 || (na & 7) || nb < na || (double)a.K * (double)na > 2.0 * (double)b.K * (double)nb || (double)b.K * (double)nb > 2.0 * (double)a.K * (double)na) return 1;
-    constexpr size_t lds_a = 2 * (OperandPath<128, true, true>::kFloats + OperandPath<128, false, true>::kFloats) * sizeof(float);
+    const long nb = (long)db.nbm * db.nbn;
+    // Worth it when `a` alone would leave the CUs with one workgroup each and `b` brings about as much work in at least as
+    // many pieces: `a` as 128 x 128 tiles if that gives 128 .. 256 of them, else as 64 x 64 tiles under the same test.
+    auto fits = [&](int tile) {
+        const long na = (long)((a.M + tile - 1) / tile) * ((a.N + tile - 1) / tile);
+        const double wa = (double)a.K * tile * tile * (double)na, wb = (double)b.K * 128.0 * 128.0 * (double)nb;
+        return na >= 128 && na <= 256 && (na & 7) == 0 && nb >= na && wa <= 2.0 * wb && wb <= 2.0 * wa;
+    };
     constexpr size_t lds_b = 2 * (OperandPath<128, false, true>::kFloats + OperandPath<128, false, true>::kFloats) * sizeof(float);
-    constexpr size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
-    static bool attr_done = false;
-    if (!attr_done) {
-        MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pair_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        attr_done = true;
+    if (fits(128)) {
+        da.nbm = (a.M + 127) / 128; da.nbn = (a.N + 127) / 128;
+        const long na = (long)da.nbm * da.nbn;
+        constexpr size_t lds_a = 2 * (OperandPath<128, true, true>::kFloats + OperandPath<128, false, true>::kFloats) * sizeof(float);
+        constexpr size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
+        static bool attr_done = false;
+        if (!attr_done) {
+            MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pair_kernel<128, 128>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+            attr_done = true;
+        }
+        hipLaunchKernelGGL((gemm_pair_kernel<128, 128>), dim3((unsigned)(na + nb)), dim3(kThreads), lds_bytes, stream, da, db, (int)na);
+    } else if (fits(64)) {
+        da.nbm = (a.M + 63) / 64; da.nbn = (a.N + 63) / 64;
+        const long na = (long)da.nbm * da.nbn;
+        constexpr size_t lds_a = 3 * (OperandPath<64, true, true>::kFloats + OperandPath<64, false, true>::kFloats) * sizeof(float);
+        constexpr size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
+        static bool attr_done = false;
+        if (!attr_done) {
+            MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pair_kernel<64, 64>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+            attr_done = true;
+        }
+        hipLaunchKernelGGL((gemm_pair_kernel<64, 64>), dim3((unsigned)(na + nb)), dim3(kThreads), lds_bytes, stream, da, db, (int)na);
+    } else {
+        return 1;
     }
-    hipLaunchKernelGGL(gemm_pair_kernel, dim3((unsigned)(na + nb)), dim3(kThreads), lds_bytes, stream, da, db, (int)na);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

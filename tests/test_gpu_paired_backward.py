@@ -83,3 +83,20 @@ def test_one_call_equals_the_two_calls(name, specs, T, B, loss):
     with pytest.raises(mb.MyeaError):          # the error behaviour of Backward_Pass: not in the inference state
         b.set_state_propagation(mb.STATE_INFERENCE)
         b.Backward_Pass__Update_Derivative_Weight(B)
+
+
+def test_weight_gradient_rides_with_the_delta_at_batch_512():
+    """one size down: the delta's contraction as 64 x 64 tiles beside the weight gradient's 128 x 128 ones"""
+    specs = [dict(units=2048), dict(units=2048, activation="RELU"), dict(units=2048, activation="TANH"), dict(units=100, activation="SOFTMAX")]
+    B = 512
+    desc, (a, b), X, Y, w = _pair(specs, B, loss="CROSS_ENTROPY")
+    b.profile_enable(True)
+    for step in range(2):
+        _step(a, B, X, Y, fused=False)
+        _step(b, B, X, Y, fused=True)
+    pairs = b.profile_read(4)
+    b.profile_enable(False)
+    assert pairs[0] >= 2, "no paired launch happened: %r" % (pairs,)
+    assert np.array_equal(a.download_gradient(), b.download_gradient())
+    for li in range(1, desc.n_layers):
+        assert np.array_equal(a.download_tensor(li, mb.TENSOR["ERRORS"]), b.download_tensor(li, mb.TENSOR["ERRORS"]))
