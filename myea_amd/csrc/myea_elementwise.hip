@@ -337,7 +337,13 @@ __global__ __launch_bounds__(kBlock) void bn_forward_apply_kernel(size_t n, BnFo
         float s = (p.x[i] - p.mean[j]) / p.var[j];
         if (p.renorm) s = s * p.r_corr[j] + p.d_corr[j];
         p.hats[i] = s;
-        p.normalizes[i] = p.scale[j] * s + p.shift[j];
+        const float y = p.scale[j] * s + p.shift[j];
+        p.normalizes[i] = y;
+        if (p.act_out) {   // Forward_Pass__FC_AF and the Bernoulli applier, as activation_kernel does them
+            float v = af_fire(p.act, y);
+            if (p.colscale) v *= p.colscale[j];
+            p.act_out[i] = v;
+        }
     }
 }
 

@@ -91,6 +91,11 @@ struct BnForwardParams {
     float *hats, *normalizes;
     float epsilon, momentum, r_max, d_max;
     int renorm;
+    // optional: the activation (and the dropout column multiplier) of a layer normalised before its activation, applied
+    // to the normalised value in the same pass: act_out = af(normalizes) * colscale
+    float *act_out;
+    const float *colscale;
+    int act;
 };
 int launch_bn_forward_training(hipStream_t s, const BnForwardParams &p, float *scratch /* >= 128 * H floats */);
 int launch_bn_forward_inference(hipStream_t s, size_t rows, size_t H, const float *x, const float *scale, const float *shift,

@@ -30,6 +30,8 @@ struct DevLayer {
     float *means = nullptr, *variances = nullptr, *means_averages = nullptr, *variances_averages = nullptr;
     float *r_corrections = nullptr, *d_corrections = nullptr;
     float *colscale = nullptr;  // dropout multiplier per (t, unit)
+    unsigned long long colscale_epoch = 0;   // Net::mask_epoch the multipliers were derived at
+    bool colscale_active = false;
     unsigned *pool_index = nullptr;  // max pooling: padded position each output took its value from [T][Bmax][H]
     // independently recurrent layer: pre-activations [T][Bmax][H]; the delta of the pre-activations lives in neuron_errors
     // unless a normalisation sits between the summation and the activation (then in dafs_own)
@@ -70,6 +72,7 @@ struct Net {
     hipEvent_t fork_event = nullptr, join_event = nullptr;
     float *parameters = nullptr, *gradient = nullptr, *opt[MYEA_STATE_KINDS] = {};
     uint8_t *masks = nullptr;
+    unsigned long long mask_epoch = 1;   // advances whenever the masks or the propagation state change
     unsigned long long dropout_seed = 0x9E3779B97F4A7C15ull, dropout_stream = 0;   // device generator: key and the next stream id
     uint8_t *zoneout_masks = nullptr;   // [state | output] halves, per LSTM layer [T][cells]
     size_t zoneout_count = 0;
@@ -110,7 +113,8 @@ struct Net {
 
     int refresh_colscale(size_t li, bool *active);
     int forward_fc_layer(size_t li, size_t B);
-    int bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training);
+    // act_out != nullptr (training only): the layer's activation and dropout multiplier ride in the normalisation's last pass
+    int bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training, float *act_out = nullptr, const float *colscale = nullptr);
     int bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx);
     int backward_into_layer(size_t li, size_t B);
     int forward_residual_block(size_t ri, size_t B);

@@ -366,6 +366,7 @@ int Net::refresh_colscale(size_t li, bool *active)
     DevLayer &o = L[li];
     *active = false;
     if (!layer_uses_mask_dropout(l) || !o.colscale) return MYEA_OK;
+    if (o.colscale_epoch == mask_epoch) { *active = o.colscale_active; return MYEA_OK; }   // same masks, same state: still valid
     const size_t n = (size_t)d.number_recurrent_depth * o.AH;
     if (state == MYEA_STATE_TRAINING) {
         float on = 1.f;
@@ -376,6 +377,8 @@ int Net::refresh_colscale(size_t li, bool *active)
         MYEA_TRY(launch_fill(stream, o.colscale, n, l.dropout_values[0]));
         *active = true;
     }
+    o.colscale_epoch = mask_epoch;
+    o.colscale_active = *active;
     return MYEA_OK;
 }
 
@@ -416,13 +419,15 @@ int Net::forward_fc_layer(size_t li, size_t B)
         prof_end(2.0 * (double)rows * (double)H * (double)In);
 
         const float *cur = o.summations + roff * H;
+        // training: the activation of a layer normalised first rides in the normalisation's last pass
+        const bool af_in_bn = norm && before && training && !ind && !softmax && !o.unit_act;
         if (norm && before) {
-            MYEA_TRY(bn_forward(li, c, rows, cur, training));
+            MYEA_TRY(bn_forward(li, c, rows, cur, training, af_in_bn ? o.values + roff * H : nullptr, cs));
             cur = o.normalizes + roff * H;
         }
         if (ind) continue;   // the recurrence and the activation follow for the whole sequence
         if (softmax) MYEA_TRY(launch_softmax(stream, rows, H, cur, o.values + roff * H, norm ? nullptr : cs));
-        else if (!fuse_af) MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, rows, H, cur, o.values + roff * H, cs, o.unit_act));
+        else if (!fuse_af && !af_in_bn) MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, rows, H, cur, o.values + roff * H, cs, o.unit_act));
         if (norm && !before) {
             MYEA_TRY(bn_forward(li, c, rows, o.values + roff * H, training));
             if (cs) MYEA_TRY(launch_colscale(stream, rows, H, o.normalizes + roff * H, cs));
@@ -464,7 +469,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
     return MYEA_OK;
 }
 
-int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training)
+int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training, float *act_out, const float *colscale)
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
@@ -483,6 +488,7 @@ int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool train
     p.epsilon = h.normalization_epsilon; p.momentum = h.normalization_momentum_average;
     p.r_max = h.batch_renormalization_r_correction_maximum; p.d_max = h.batch_renormalization_d_correction_maximum;
     p.renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    p.act_out = act_out; p.colscale = colscale; p.act = (int)l.type_activation_function;
     return launch_bn_forward_training(stream, p, scratch);
 }
 
@@ -1300,6 +1306,7 @@ int myea_hip_set_state_propagation(myea_hip_net *n, uint32_t s)
     NET_OR_FAIL(n);
     if (s > MYEA_STATE_TRAINING) { myea::set_last_error("state propagation %u is not on this path", s); return MYEA_E_UNSUPPORTED; }
     n->net.state = s;
+    ++n->net.mask_epoch;   // the dropout multipliers depend on the state
     return MYEA_OK;
 }
 
@@ -1350,6 +1357,7 @@ int myea_hip_upload_masks(myea_hip_net *n, const uint8_t *m, size_t c)
     if (!m || c > n->net.d.total_mask_units) { myea::set_last_error("upload_masks: null or count %zu > %llu", c, (unsigned long long)n->net.d.total_mask_units); return MYEA_E_INVALID; }
     MYEA_HIP_TRY(hipMemcpyAsync(n->net.masks, m, c, hipMemcpyHostToDevice, n->net.stream));
     MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
+    ++n->net.mask_epoch;
     return MYEA_OK;
 }
 int myea_hip_upload_zoneout_masks(myea_hip_net *n, const uint8_t *m, size_t c)
