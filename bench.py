@@ -1,11 +1,11 @@
 #!/usr/bin/env python3
 """Benchmark of the training hot path on one MI355X.
 
-One "step" = Forward_Pass + Compute__Error + Backward_Pass + Update_Derivative_Weight + Update_Parameter on one
+One "step" = Forward_Pass + Compute__Error + Backward_Pass and Update_Derivative_Weight (as one call) + Update_Parameter on one
 batch of synthetic data already resident in HBM.  Default workload: BASELINE config 2, the deep fully-connected
 stack 4096-4096-4096-4096-4096-1000 (ReLU, softmax + cross-entropy, Adam) at batch 1024, fp32.
 
-Prints ONE JSON line (see README / DESIGN).  `roofline` covers the dominant kernel family — the FP32 MFMA
+Prints ONE JSON line.  `roofline` covers the dominant kernel family — the FP32 MFMA
 contractions (forward X W^T, dX = delta W, dW += delta^T X): algorithmic FLOPs of all their launches in the
 timed region over their summed HIP-event durations on the stream they run on.  `cpu_baseline` times the CPU
 restatement of the reference (oracle/, OpenMP) on this host on a bounded sample of the same workload.
