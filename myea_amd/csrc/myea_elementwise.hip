@@ -290,6 +290,7 @@ __global__ __launch_bounds__(kBlock) void column_sum_final_kernel(size_t H, size
     const size_t col = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (col >= H) return;
     double s = 0.0;
+#pragma unroll 8
     for (size_t y = 0; y < S; ++y) s += partial[y * H + col];
     out[col] = accumulate ? out[col] + (float)s : (float)s;
 }
@@ -308,6 +309,7 @@ __global__ __launch_bounds__(kBlock) void bn_forward_final_kernel(size_t H, size
     const size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (j >= H) return;
     double smd = 0.0, svd = 0.0;
+#pragma unroll 8
     for (size_t y = 0; y < S; ++y) { smd += partial[(y * 2 + 0) * H + j]; svd += partial[(y * 2 + 1) * H + j]; }
     const float sm = (float)smd, sv = (float)svd;
     const float bscale = 1.f / (float)rows;
@@ -380,6 +382,7 @@ __global__ __launch_bounds__(kBlock) void bn_backward_final_kernel(size_t H, siz
     const size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (j >= H) return;
     double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
+#pragma unroll 8
     for (size_t y = 0; y < S; ++y) {
         a0 += partial[(y * 4 + 0) * H + j];
         a1 += partial[(y * 4 + 1) * H + j];

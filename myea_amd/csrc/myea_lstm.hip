@@ -236,33 +236,37 @@ __global__ __launch_bounds__(kBlock) void lstm_backward_step_kernel(LstmGeom g, 
 //   dp_i += di[t+1] c[t], dp_f += df[t+1] c[t] for t < T-1;  dp_o += do[t] c[t] for all t.
 // rows of the reduction are (t, b) pairs; columns are cells.
 struct PeepF {
+    static constexpr int kUnroll = 1;   // four strided loads and a division per row already: more rows in flight cost registers and time
     LstmGeom g;
     size_t B, Bmax, T;
     const float *c, *dG;
     int reverse;   // the step processed after t is t - 1
     __device__ void operator()(size_t r, size_t col, double *acc) const
     {
-        const size_t t = r / B, b = r % B, k = col / g.cpb;
-        const size_t row = t * Bmax + b;
+        // (t, b) of the row in 32-bit arithmetic (the launcher holds T * B below 2^32)
+        const unsigned t = (unsigned)r / (unsigned)B, b = (unsigned)r - t * (unsigned)B;
+        const size_t k = col / g.cpb;
+        const size_t row = (size_t)t * Bmax + b;
         const float cs = c[row * g.C + col];
         acc[2] += dG[row * g.G + g.C + 2 * g.K + k] * cs;
         if (reverse ? t > 0 : t + 1 < T) {
-            const size_t nrow = (reverse ? t - 1 : t + 1) * Bmax + b;
+            const size_t nrow = (size_t)(reverse ? t - 1 : t + 1) * Bmax + b;
             acc[0] += dG[nrow * g.G + g.C + k] * cs;
             acc[1] += dG[nrow * g.G + g.C + g.K + k] * cs;
         }
     }
 };
 
+// one lane per (gate, cell): the three peephole vectors' partial sums folded in order
 __global__ __launch_bounds__(kBlock) void lstm_peep_final_kernel(LstmGeom g, size_t S, const float *partial, float *flat_gradient)
 {
-    const size_t c = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (c >= g.C) return;
-    for (size_t gate = 0; gate < 3; ++gate) {
-        double s = 0.0;
-        for (size_t y = 0; y < S; ++y) s += partial[(y * 3 + gate) * g.C + c];
-        flat_gradient[peep_index(g, gate, c)] += (float)s;
-    }
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= 3 * g.C) return;
+    const size_t gate = i / g.C, c = i % g.C;
+    double s = 0.0;
+#pragma unroll 8
+    for (size_t y = 0; y < S; ++y) s += partial[(y * 3 + gate) * g.C + c];
+    flat_gradient[peep_index(g, gate, c)] += (float)s;
 }
 
 // column sums over (t, b) rows of a [T][Bmax][W] tensor when B < Bmax (rows are not contiguous)
@@ -276,6 +280,7 @@ __global__ __launch_bounds__(kBlock) void lstm_colsum_final_kernel(size_t H, siz
     const size_t col = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (col >= H) return;
     double s = 0.0;
+#pragma unroll 8
     for (size_t y = 0; y < S; ++y) s += partial[y * H + col];
     out[col] += (float)s;
 }
@@ -686,6 +691,7 @@ int Net::lstm_update_derivative_weight_reductions(LstmLayer &q, size_t B)
 {
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
     const LstmGeom geom = geom_of(q);
+    if (T * B > 0xffffffffull) { set_last_error("LSTM weight gradients: %zu x %zu (time steps x batch) rows do not fit 32 bits", T, B); return MYEA_E_INVALID; }
     // peepholes
     {
         size_t S, chunk;
@@ -693,7 +699,7 @@ int Net::lstm_update_derivative_weight_reductions(LstmLayer &q, size_t B)
         PeepF f{geom, B, Bmax, T, q.c, q.dG, q.reverse ? 1 : 0};
         hipLaunchKernelGGL((column_partial_kernel<3, PeepF>), dim3((unsigned)((q.C + 63) / 64), (unsigned)S), dim3(kBlock), 0, stream, T * B, q.C, chunk, scratch, f);
         MYEA_HIP_TRY(hipGetLastError());
-        hipLaunchKernelGGL(lstm_peep_final_kernel, dim3(grid_for(q.C, kBlock)), dim3(kBlock), 0, stream, geom, S, scratch, gradient);
+        hipLaunchKernelGGL(lstm_peep_final_kernel, dim3(grid_for(3 * q.C, kBlock)), dim3(kBlock), 0, stream, geom, S, scratch, gradient);
         MYEA_HIP_TRY(hipGetLastError());
     }
     // the four bias vectors: one contiguous [G] slice in the order z | i | f | o

@@ -1,5 +1,6 @@
 // myea_reduce.h — launch helpers and the deterministic two-stage column reduction shared by the HBM-bound kernels.
 #pragma once
+#include <type_traits>
 
 #include <hip/hip_runtime.h>
 #include <stddef.h>
@@ -37,6 +38,10 @@ __device__ __forceinline__ float wave_max(float v)
 // Per-lane accumulation is in fp64 (the kernels are HBM-bound, the adds are free): sums like
 // E[x^2] - mean^2 lose most of their digits when |mean| >> sigma, and the fp32 result should then be the
 // correctly rounded one rather than depend on the summation order.
+// rows a lane keeps in flight at once: 4 unless the functor says otherwise (F::kUnroll)
+template <class F, class = void> struct unroll_of { static constexpr int value = 4; };
+template <class F> struct unroll_of<F, std::void_t<decltype(F::kUnroll)>> { static constexpr int value = F::kUnroll; };
+
 template <int NV, typename F>
 __global__ __launch_bounds__(kBlock) void column_partial_kernel(size_t rows, size_t H, size_t chunk, float *partial, F f)
 {
@@ -48,6 +53,8 @@ __global__ __launch_bounds__(kBlock) void column_partial_kernel(size_t rows, siz
     for (int v = 0; v < NV; ++v) acc[v] = 0.0;
     if (col < H) {
         const size_t r0 = (size_t)blockIdx.y * chunk, r1 = min(rows, r0 + chunk);
+        // several rows' loads in flight per lane: a lane's rows are independent until the adds
+#pragma unroll unroll_of<F>::value
         for (size_t r = r0 + rl; r < r1; r += 4) f(r, col, acc);
     }
 #pragma unroll
