@@ -269,6 +269,58 @@ __global__ __launch_bounds__(kBlock) void lstm_peep_final_kernel(LstmGeom g, siz
     flat_gradient[peep_index(g, gate, c)] += (float)s;
 }
 
+// One cell per block: the four bias sums and the three peephole sums of a cell come from the same five values per
+// (time step, example) - the cell's four gate deltas and its state - so one pass over dG and c gives all seven.  A lane
+// owns one cell and walks the time steps of its examples in the direction's processing order, carrying the cell state
+// of the step before (dp_i, dp_f pair the deltas of a step with the state of the step processed before it).
+// grid (ceil(C / 64), S); partial[(y * 7 + v) * C + cell], v = b_z, b_i, b_f, b_o, p_i, p_f, p_o.
+__global__ __launch_bounds__(kBlock) void lstm_bias_peep_partial_kernel(size_t C, size_t B, size_t Bmax, size_t T, size_t per_lane, int reverse,
+                                                                        const float *__restrict__ c, const float *__restrict__ dG, float *partial)
+{
+    __shared__ double red[7][4][64];
+    const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6;
+    const size_t col = (size_t)blockIdx.x * 64 + cl, G = 4 * C;
+    double acc[7];
+#pragma unroll
+    for (int v = 0; v < 7; ++v) acc[v] = 0.0;
+    if (col < C) {
+        const size_t b0 = ((size_t)blockIdx.y * 4 + rl) * per_lane, b1 = min(B, b0 + per_lane);
+        for (size_t b = b0; b < b1; ++b) {
+            float c_prev = 0.f;   // no step before the first: its two terms vanish
+#pragma unroll 4
+            for (size_t s = 0; s < T; ++s) {
+                const size_t t = reverse ? T - 1 - s : s, row = t * Bmax + b;
+                const float *d = dG + row * G + col;
+                const float dz = d[0], di = d[C], df = d[2 * C], dout = d[3 * C], cs = c[row * C + col];
+                acc[0] += dz; acc[1] += di; acc[2] += df; acc[3] += dout;
+                acc[4] += di * c_prev; acc[5] += df * c_prev; acc[6] += dout * cs;
+                c_prev = cs;
+            }
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < 7; ++v) red[v][rl][cl] = acc[v];
+    __syncthreads();
+    if (rl == 0 && col < C) {
+#pragma unroll
+        for (int v = 0; v < 7; ++v)
+            partial[((size_t)blockIdx.y * 7 + v) * C + col] = (float)(red[v][0][cl] + red[v][1][cl] + red[v][2][cl] + red[v][3][cl]);
+    }
+}
+
+// one lane per (sum, cell): partials folded in order into the bias slice (v < 4) and the peephole slots (v >= 4)
+__global__ __launch_bounds__(kBlock) void lstm_bias_peep_final_kernel(LstmGeom g, size_t S, const float *partial, float *bias_gradient, float *flat_gradient)
+{
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= 7 * g.C) return;
+    const size_t v = i / g.C, cell = i % g.C;
+    double s = 0.0;
+#pragma unroll 8
+    for (size_t y = 0; y < S; ++y) s += partial[(y * 7 + v) * g.C + cell];
+    if (v < 4) bias_gradient[v * g.C + cell] += (float)s;
+    else flat_gradient[peep_index(g, v - 4, cell)] += (float)s;
+}
+
 // column sums over (t, b) rows of a [T][Bmax][W] tensor when B < Bmax (rows are not contiguous)
 struct StridedSumF {
     size_t B, Bmax, W;
@@ -692,6 +744,20 @@ int Net::lstm_update_derivative_weight_reductions(LstmLayer &q, size_t B)
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
     const LstmGeom geom = geom_of(q);
     if (T * B > 0xffffffffull) { set_last_error("LSTM weight gradients: %zu x %zu (time steps x batch) rows do not fit 32 bits", T, B); return MYEA_E_INVALID; }
+    if (q.cpb == 1) {   // biases and peepholes in one pass over the gate deltas
+        const size_t colblocks = (q.C + 63) / 64;
+        size_t S = (512 + colblocks - 1) / colblocks;          // aim at >= 512 workgroups
+        if (S > (B + 3) / 4) S = (B + 3) / 4;
+        if (S > 64) S = 64;                                     // the scratch holds 64 x 7 x C partial sums
+        const size_t per_lane = (B + 4 * S - 1) / (4 * S);
+        S = (B + 4 * per_lane - 1) / (4 * per_lane);
+        hipLaunchKernelGGL(lstm_bias_peep_partial_kernel, dim3((unsigned)colblocks, (unsigned)S), dim3(kBlock), 0, stream, q.C, B, Bmax, T, per_lane, q.reverse ? 1 : 0,
+                           q.c, q.dG, scratch);
+        MYEA_HIP_TRY(hipGetLastError());
+        hipLaunchKernelGGL(lstm_bias_peep_final_kernel, dim3(grid_for(7 * q.C, kBlock)), dim3(kBlock), 0, stream, geom, S, scratch, gradient + q.bias, gradient);
+        MYEA_HIP_TRY(hipGetLastError());
+        return MYEA_OK;
+    }
     // peepholes
     {
         size_t S, chunk;
