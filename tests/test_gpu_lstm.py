@@ -64,6 +64,9 @@ CASES = [
     ("fused-step-32-cells", [dict(units=9), dict(type="lstm", units=32), dict(units=32, activation="LINEAR")], 5, 7, 7),
     ("fused-step-96-cells-partial-batch", [dict(units=20), dict(type="lstm", units=96), dict(units=96, activation="TANH")], 4, 37, 40),
     ("fused-step-160-cells-two-steps", [dict(units=6), dict(type="lstm", units=160), dict(units=160, activation="LINEAR")], 2, 33, 33),
+    # enough (row tile, cell tile) pairs for the full-size tiles of the one-launch-per-step kernels, last row tile ragged
+    ("fused-step-full-size-tiles-512-cells-ragged", [dict(units=12), dict(type="lstm", units=512), dict(units=512, activation="LINEAR")], 3, 130, 136),
+    ("fused-step-full-size-tiles-256-cells-ragged", [dict(units=7), dict(type="lstm", units=256), dict(units=256, activation="TANH")], 2, 270, 270),
     ("fused-step-stacked-on-generic", [dict(units=10), dict(type="lstm", units=24), dict(type="lstm", units=64), dict(type="lstm", units=32),
                                        dict(units=32, activation="LINEAR")], 3, 12, 16),
 ]
@@ -81,7 +84,8 @@ def test_lstm_parity_three_amsgrad_steps(name, specs, T, B, Bmax):
             run_step(n, B, X, Y, update=False)
         _compare(desc, gpu, cpu, B, T, what="step %d" % step)
         g_cpu = cpu.download_gradient()
-        assert_close(gpu.download_gradient(), g_cpu, REL, ABS, what="gradient step %d" % step)
+        # sums over T x B terms of either sign: the absolute floor follows the gradient's scale where that exceeds 1
+        assert_close(gpu.download_gradient(), g_cpu, REL, ABS * max(1.0, float(np.abs(g_cpu).max())), what="gradient step %d" % step)
         lg, lc = gpu.get_loss(), cpu.get_loss()
         assert lg.number_loss == lc.number_loss and lg.loss_values == pytest.approx(lc.loss_values, rel=1e-4)
         for n in (gpu, cpu):
