@@ -20,8 +20,8 @@ def _step(net, B, X, Y, fused):
         net.Update_Derivative_Weight(B)
 
 
-def _pair(specs, B, T=1, seed=3, loss="MSE"):
-    desc = mb.make_desc(specs, B, T)
+def _pair(specs, B, T=1, seed=3, loss="MSE", Bmax=None):
+    desc = mb.make_desc(specs, Bmax or B, T)
     h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["ADAM"], type_loss_function=mb.LOSS[loss])
     nets = [mb.HipNetwork(desc, h) for _ in range(2)]
     w = glorot_parameters(desc, seed, bias_range=0.3)
@@ -38,10 +38,10 @@ def _pair(specs, B, T=1, seed=3, loss="MSE"):
     return desc, nets, X, Y, w
 
 
-def test_weight_gradient_rides_with_the_delta_at_batch_1024():
+@pytest.mark.parametrize("B", [1024, 999])
+def test_weight_gradient_rides_with_the_delta_at_batch_1024(B):
     specs = [dict(units=2048), dict(units=2048, activation="RELU"), dict(units=2048, activation="TANH"), dict(units=2048, activation="RELU"), dict(units=1000, activation="SOFTMAX")]
-    B = 1024
-    desc, (a, b), X, Y, w = _pair(specs, B, loss="CROSS_ENTROPY")
+    desc, (a, b), X, Y, w = _pair(specs, B, loss="CROSS_ENTROPY", Bmax=1024)
     b.profile_enable(True)
     for step in range(2):                     # the second step accumulates onto a non-zero gradient
         _step(a, B, X, Y, fused=False)
@@ -55,8 +55,8 @@ def test_weight_gradient_rides_with_the_delta_at_batch_1024():
         assert np.array_equal(a.download_tensor(li, mb.TENSOR["ERRORS"]), b.download_tensor(li, mb.TENSOR["ERRORS"]))
     # and both agree with float64 on a slice of the largest layer's gradient: dW = delta^T X, accumulated twice
     l = desc.layers[2]
-    delta = a.download_tensor(2, mb.TENSOR["ERRORS"]).reshape(B, 2048).astype(np.float64)
-    x = a.download_tensor(1, mb.TENSOR["OUTPUTS"]).reshape(B, 2048).astype(np.float64)
+    delta = a.download_tensor(2, mb.TENSOR["ERRORS"]).reshape(1024, 2048)[:B].astype(np.float64)
+    x = a.download_tensor(1, mb.TENSOR["OUTPUTS"]).reshape(1024, 2048)[:B].astype(np.float64)
     want = 2.0 * (delta[:, :64].T @ x)
     got = ga[l.first_connection_index:l.first_connection_index + 64 * 2048].reshape(64, 2048)
     assert_close(got, want, 1e-4, 1e-5 * float(np.abs(want).max()), what="dW rows 0..63 of layer 2")
@@ -85,11 +85,12 @@ def test_one_call_equals_the_two_calls(name, specs, T, B, loss):
         b.Backward_Pass__Update_Derivative_Weight(B)
 
 
-def test_weight_gradient_rides_with_the_delta_at_batch_512():
-    """one size down: the delta's contraction as 64 x 64 tiles beside the weight gradient's 128 x 128 ones"""
+@pytest.mark.parametrize("B", [512, 500, 449])
+def test_weight_gradient_rides_with_the_delta_at_batch_512(B):
+    """one size down: the delta's contraction as 64 x 64 tiles beside the weight gradient's 128 x 128 ones; batches that leave
+    the last row tile ragged (500) and that end a k range off the step of 32 (449, also an odd row count)"""
     specs = [dict(units=2048), dict(units=2048, activation="RELU"), dict(units=2048, activation="TANH"), dict(units=100, activation="SOFTMAX")]
-    B = 512
-    desc, (a, b), X, Y, w = _pair(specs, B, loss="CROSS_ENTROPY")
+    desc, (a, b), X, Y, w = _pair(specs, B, loss="CROSS_ENTROPY", Bmax=512)
     b.profile_enable(True)
     for step in range(2):
         _step(a, B, X, Y, fused=False)
@@ -100,3 +101,10 @@ def test_weight_gradient_rides_with_the_delta_at_batch_512():
     assert np.array_equal(a.download_gradient(), b.download_gradient())
     for li in range(1, desc.n_layers):
         assert np.array_equal(a.download_tensor(li, mb.TENSOR["ERRORS"]), b.download_tensor(li, mb.TENSOR["ERRORS"]))
+    # and the gradient itself against float64 on a slice: dW = delta^T X over the B rows in use, accumulated twice
+    l = desc.layers[2]
+    delta = a.download_tensor(2, mb.TENSOR["ERRORS"]).reshape(512, 2048)[:B].astype(np.float64)
+    x = a.download_tensor(1, mb.TENSOR["OUTPUTS"]).reshape(512, 2048)[:B].astype(np.float64)
+    want = 2.0 * (delta[:, :48].T @ x)
+    got = a.download_gradient()[l.first_connection_index:l.first_connection_index + 48 * 2048].reshape(48, 2048)
+    assert_close(got, want, 1e-4, 1e-5 * float(np.abs(want).max()), what="dW rows 0..47 of layer 2")
