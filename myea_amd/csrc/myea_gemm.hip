@@ -264,6 +264,97 @@ struct GemmDev {
     long slab;
 };
 
+struct TilePlace {
+    int m0, n0, wave_m, wave_n, lane32, half;
+    long slab_offset;
+};
+
+// The accumulators of one wavefront go out: a lane owns one column of each 32 x 32 accumulator (rows
+// (r / 4) * 8 + half * 4 + r % 4), so per-column operands are read once.  The kind of epilogue, the class of the
+// activation and the presence of an addend are the same for every element of a launch, and whether a tile lies wholly
+// inside the matrix is the same for every element of the tile: all four are template parameters, decided once per tile,
+// and the element loop carries no test of them (it carried a dozen branches per element before, 5 - 10 us per tile).
+//   KIND 0 store | 3 add onto C (one hardware add per element, performed at the L2: every element is owned by exactly one
+//        lane of one workgroup, so the result is the C + v a load / add / store gives, and nothing waits for C to come in)
+//   KIND 1 forward: C = v + bias, aux_out = AF(C) * column multiplier; CLASS 0 no aux_out, 1 piecewise linear (linear, ReLU,
+//        leaky: s < 0 ? slope * s : s, ReLU's zero kept exact), 2 through exp (sigmoid, tanh: a / (1 + exp(k s)) - b)
+//   KIND 2 C = v * AF'(pre, steep, val); CLASS 1 piecewise (q < 0 ? steep * slope : steep), 2 smooth (tanh, sigmoid)
+// Edge tiles (WHOLE false) run the same arithmetic behind a bounds test per element, so an element's value does not
+// depend on the tile shape it was computed in.
+template <int KIND, int CLASS, bool ADDEND, bool WHOLE, int TM, int TN>
+__device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&acc)[TM][TN], const TilePlace &at)
+{
+    const bool relu = p.act == MYEA_AF_RELU, tanh_like = p.act == MYEA_AF_TANH;
+    const float slope = p.act == MYEA_AF_LINEAR ? 1.f : 0.01f;                       // piecewise classes (ReLU handled by `relu`)
+    const float ek = tanh_like ? -2.f : -1.f, ea = tanh_like ? 2.f : 1.f, eb = tanh_like ? 1.f : 0.f;
+    const float d_neg = relu ? 0.f : (p.act == MYEA_AF_LINEAR ? p.steep : p.steep * 0.01f);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int col = at.n0 + at.wave_n + j * 32 + at.lane32;
+        if (!WHOLE && col >= p.N) continue;
+        float bias = 0.f, cs = 1.f;
+        if (KIND == 1) {
+            if (p.bias) bias = p.bias[col];
+            if (CLASS != 0 && p.colscale) cs = p.colscale[col];
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int row0 = at.m0 + at.wave_m + i * 32 + at.half * 4;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = row0 + (r >> 2) * 8 + (r & 3);
+                if (!WHOLE && row >= p.M) continue;
+                const long o = (long)row * p.ldc + col + at.slab_offset;
+                float v = acc[i][j][r];
+                if (ADDEND) v += p.addend[(long)row * p.ld_addend + col];
+                if (KIND == 1) {
+                    v += bias;
+                    p.C[o] = v;
+                    if (CLASS == 1) {
+                        const float neg = slope * v;
+                        p.aux_out[o] = (v < 0.f ? (relu ? 0.f : neg) : v) * cs;
+                    } else if (CLASS == 2) {
+                        const float e = expf(ek * v);
+                        p.aux_out[o] = (ea / (1.f + e) - eb) * cs;
+                    }
+                } else if (KIND == 2) {
+                    float dv;
+                    if (CLASS == 1) {
+                        dv = p.pre[o] < 0.f ? d_neg : p.steep;
+                    } else {
+                        const float y = p.val[o];
+                        dv = tanh_like ? p.steep * (1.f - y * y) : p.steep * y * (1.f - y);
+                    }
+                    p.C[o] = v * dv;
+                } else if (KIND == 3) {
+                    unsafeAtomicAdd(&p.C[o], v);
+                } else {
+                    p.C[o] = v;
+                }
+            }
+        }
+    }
+}
+
+template <bool WHOLE, int TM, int TN>
+__device__ __forceinline__ void store_tile_kind(const GemmDev &p, const f32x16 (&acc)[TM][TN], const TilePlace &at)
+{
+    const bool smooth = p.act == MYEA_AF_TANH || p.act == MYEA_AF_SIGMOID;
+    if (p.epilogue == EPI_FC_FORWARD) {          // the launcher admits no addend on this kind nor on an accumulating launch
+        if (!p.aux_out) store_tile_as<1, 0, false, WHOLE, TM, TN>(p, acc, at);
+        else if (smooth) store_tile_as<1, 2, false, WHOLE, TM, TN>(p, acc, at);
+        else store_tile_as<1, 1, false, WHOLE, TM, TN>(p, acc, at);
+    } else if (p.epilogue == EPI_FC_DERIVE) {
+        if (p.addend) { if (smooth) store_tile_as<2, 2, true, WHOLE, TM, TN>(p, acc, at); else store_tile_as<2, 1, true, WHOLE, TM, TN>(p, acc, at); }
+        else { if (smooth) store_tile_as<2, 2, false, WHOLE, TM, TN>(p, acc, at); else store_tile_as<2, 1, false, WHOLE, TM, TN>(p, acc, at); }
+    } else if (p.accumulate) {
+        store_tile_as<3, 0, false, WHOLE, TM, TN>(p, acc, at);
+    } else {
+        if (p.addend) store_tile_as<0, 0, true, WHOLE, TM, TN>(p, acc, at);
+        else store_tile_as<0, 0, false, WHOLE, TM, TN>(p, acc, at);
+    }
+}
+
 // One workgroup's share of a contraction: tile number `block` of problem `p`, staged through `smem`.
 template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
 __device__ __forceinline__ void gemm_tile(const GemmDev &p, const int block, float *smem)
@@ -383,42 +474,11 @@ __device__ __forceinline__ void gemm_tile(const GemmDev &p, const int block, flo
         cur = following;
     }
 
-    // Epilogue.  A lane owns one column of each accumulator, so per-column operands are read once.
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int col = n0 + wave_n + j * 32 + lane32;
-        if (col >= p.N) continue;
-        float bias = 0.f, cs = 1.f;
-        if (p.epilogue == EPI_FC_FORWARD) {
-            if (p.bias) bias = p.bias[col];
-            if (p.colscale) cs = p.colscale[col];
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wave_m + i * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-                if (row >= p.M) continue;
-                const long o = (long)row * p.ldc + col + (long)split * p.slab;
-                float v = acc[i][j][r];
-                if (p.addend) v += p.addend[(long)row * p.ld_addend + col];
-                if (p.epilogue == EPI_FC_FORWARD) {
-                    v += bias;
-                    p.C[o] = v;
-                    if (p.aux_out) p.aux_out[o] = af_fire_fused(p.act, v) * cs;
-                } else if (p.epilogue == EPI_FC_DERIVE) {
-                    p.C[o] = v * af_derive_fused(p.act, p.pre[o], p.steep, p.val[o]);
-                } else if (p.accumulate) {
-                    // C += v without reading C back: one hardware add per element, performed at the L2.  Every element is
-                    // owned by exactly one lane of one workgroup, so the result is the C + v a load / add / store gives,
-                    // and the epilogue no longer waits for a tile of C to come in.
-                    unsafeAtomicAdd(&p.C[o], v);
-                } else {
-                    p.C[o] = v;
-                }
-            }
-        }
-    }
+    // Epilogue.  What kind it is, whether an addend joins and whether the tile lies wholly inside the matrix are the same
+    // for every element of the tile: they are decided once, and the element loops of whole tiles carry no such test.
+    const TilePlace at{m0, n0, wave_m, wave_n, lane32, half, (long)split * p.slab};
+    if (m0 + BM <= p.M && n0 + BN <= p.N) store_tile_kind<true, TM, TN>(p, acc, at);
+    else store_tile_kind<false, TM, TN>(p, acc, at);
 }
 
 template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
@@ -529,6 +589,7 @@ static int prepare_gemm(const GemmParams &p, GemmDev &d, bool *vec)
     const long a_min = p.a_k_contiguous ? p.K : p.M, b_min = p.b_k_contiguous ? p.K : p.N;
     if (p.lda < a_min || p.ldb < b_min || p.ldc < p.N) { set_last_error("gemm: leading dimension smaller than the row length"); return MYEA_E_INVALID; }
     if (p.epilogue == EPI_FC_DERIVE && (!p.pre || !p.val)) { set_last_error("gemm: derive epilogue without pre/val"); return MYEA_E_INVALID; }
+    if (p.addend && (p.epilogue == EPI_FC_FORWARD || p.accumulate)) { set_last_error("gemm: an addend goes with a plain or a derivative epilogue only"); return MYEA_E_INVALID; }
     if (p.epilogue == EPI_FC_DERIVE && !gemm_can_fuse_activation(p.act)) { set_last_error("gemm: activation %d cannot be fused", p.act); return MYEA_E_INVALID; }
     if (p.epilogue == EPI_FC_FORWARD && p.aux_out && !gemm_can_fuse_activation(p.act)) { set_last_error("gemm: activation %d cannot be fused", p.act); return MYEA_E_INVALID; }
 
