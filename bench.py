@@ -23,7 +23,7 @@ if ROOT not in sys.path:
 # HBM bytes per contraction launch (mean over the launches of one step) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of this script, scaled by what the same counters read for copies of known size (FETCH_SIZE x2, WRITE_SIZE x1);
 # the per-kernel figures are in profiles/hbm_traffic__*__pmc.txt.  None where no counter run has been made.
-PMC_TRAFFIC_BYTES_PER_GEMM_LAUNCH = {"fc4096x4_b1024_adam": 2896189 * 1024 / 10}
+PMC_TRAFFIC_BYTES_PER_GEMM_LAUNCH = {"fc4096x4_b1024_adam": 2886299 * 1024 / 10}
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
