@@ -379,6 +379,15 @@ int myea_hip_backward_pass(myea_hip_net *net, size_t batch_size_received);
 /* Neural_Network::Update_Derivative_Weight (Data.hpp:2199) over layers
  * [first_layer_index, end_layer_index); the reference's callers pass (layers + 1, last). */
 int myea_hip_update_derivative_weight(myea_hip_net *net, size_t batch_size_received, size_t first_layer_index, size_t end_layer_index);
+/* No counterpart in the reference.  myea_hip_update_derivative_weight for callers that cannot allocate device memory
+ * around the call or must not depend on buffers the library allocated (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments, same launches, same results, but every scratch buffer of
+ * its kernels - the column reductions' partial sums, the split-K slabs of narrow fully-connected layers, the packed
+ * weight-gradient slabs of LSTM layers - comes out of one static device array of 32 MiB that each GPU the library
+ * runs on holds until the process ends.  The call allocates and frees nothing.  A network whose kernels need more
+ * scratch than the array holds is rejected with MYEA_E_INVALID (the text names both sizes).  Every call on a GPU
+ * shares that GPU's array: calls that overlap on one GPU (two networks on two streams) race. */
+int myea_hip_update_derivative_weight_no_alloc(myea_hip_net *net, size_t batch_size_received, size_t first_layer_index, size_t end_layer_index);
 /* Backward_Pass immediately followed by Update_Derivative_Weight(batch, 1, total_layers) - the two calls Dataset::Train_Batch_BP
  * issues back to back (Neural_Network/Dataset.cpp:645-658) - as one entry point.  Results are those of the two calls; knowing
  * that the weight gradients are wanted lets the library send a layer's `dW += delta^T X` along in the same launch as the

@@ -37,6 +37,7 @@ struct LstmLayer {
     size_t zone_stride = 0;
     bool fused = false;     // one launch per time step (myea_lstm_fused.hip) instead of contraction + gate kernel
     float *gWin = nullptr, *gWrec = nullptr;                     // packed gradient scratch
+    float *gWin_own = nullptr, *gWrec_own = nullptr;             // the layer's own allocations behind the two pointers above
     float *acts = nullptr;  // [T][Bmax][G]: pre-activation sums, overwritten in place by z | i | f | o
     float *c = nullptr, *ca = nullptr;                           // [T][Bmax][C] cell state and tanh(cell state)
     float *dG = nullptr;    // [T][Bmax][G] deltas dz | di | df | do
@@ -414,6 +415,7 @@ int Net::lstm_create_layer(size_t li)
         if (q->fused) MYEA_TRY(dev_alloc_zero(&q->WrecT, q->C * q->G));
         MYEA_TRY(dev_alloc_zero(&q->gWin, kMaxSlabs * q->G * q->In));   // split-K slabs of the weight-gradient contractions
         MYEA_TRY(dev_alloc_zero(&q->gWrec, kMaxSlabs * q->G * q->C));
+        q->gWin_own = q->gWin; q->gWrec_own = q->gWrec;
         MYEA_TRY(dev_alloc_zero(&q->acts, T * B * q->G));
         MYEA_TRY(dev_alloc_zero(&q->c, T * B * q->C));
         MYEA_TRY(dev_alloc_zero(&q->ca, T * B * q->C));
@@ -433,7 +435,7 @@ void Net::lstm_destroy_layer(DevLayer &o)
     for (LstmLayer **slot : {&o.lstm, &o.lstm2}) {
         LstmLayer *q = *slot;
         if (!q) continue;
-        float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin, q->gWrec, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr};
+        float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin_own, q->gWrec_own, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr};
         for (float *p : all) if (p) (void)hipFree(p);
         delete q;
         *slot = nullptr;
@@ -446,6 +448,28 @@ size_t Net::lstm_scratch_floats() const
     for (const DevLayer &o : L)
         if (o.lstm) { const size_t n = 64 * 3 * o.lstm->C + 64 * o.lstm->G; if (n > need) need = n; }
     return need;
+}
+
+static size_t round_up_64(size_t n) { return (n + 63) / 64 * 64; }
+
+size_t Net::lstm_gradient_slab_floats() const
+{
+    size_t need = 0;
+    for (const DevLayer &o : L)
+        for (const LstmLayer *q : {o.lstm, o.lstm2})
+            if (q) need += round_up_64(kMaxSlabs * q->G * q->In) + round_up_64(kMaxSlabs * q->G * q->C);
+    return need;
+}
+
+void Net::lstm_bind_gradient_slabs(float *base)
+{
+    for (DevLayer &o : L)
+        for (LstmLayer *q : {o.lstm, o.lstm2}) {
+            if (!q) continue;
+            if (!base) { q->gWin = q->gWin_own; q->gWrec = q->gWrec_own; continue; }
+            q->gWin = base; base += round_up_64(kMaxSlabs * q->G * q->In);
+            q->gWrec = base; base += round_up_64(kMaxSlabs * q->G * q->C);
+        }
 }
 
 // packed copies <- flat vector; called after every parameter upload and every optimizer update

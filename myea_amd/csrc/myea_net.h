@@ -84,6 +84,8 @@ struct Net {
     std::vector<DevLayer> L;
     float *tmp1 = nullptr, *tmp2 = nullptr, *scratch = nullptr, *stage_in = nullptr, *stage_out = nullptr;
     float *dw_slabs = nullptr;   // split-K slabs of a fully-connected weight gradient whose M x N is small and k long
+    size_t scratch_floats = 0, dw_slab_floats = 0;   // sizes of the two buffers above
+    float *static_scratch = nullptr;   // this device's copy of the library's static scratch array (update_derivative_weight_no_alloc)
     double *loss_acc = nullptr;                  // 8 doubles, see ErrorParams::loss_acc
     unsigned long long *index_stage = nullptr;   // [Bmax] example indices of a gathered batch
 
@@ -130,6 +132,8 @@ struct Net {
     std::vector<char> dw_done;         // per layer: the weight contraction already ran in this pass
     bool fc_dw_params(size_t li, size_t B, GemmParams *g);   // false: the layer's weight gradient is not one plain contraction
     int update_derivative_weight(size_t B, size_t first, size_t end);
+    // the same call with every scratch buffer of its kernels taken from the library's static device array
+    int update_derivative_weight_no_alloc(size_t B, size_t first, size_t end);
     int update_parameter(size_t B, size_t training_size);
     int set_unit_activations(size_t li, const uint32_t *types, const float *steep, size_t count);
 
@@ -148,6 +152,10 @@ struct Net {
     int lstm_backward_step(LstmLayer &q, size_t B, size_t s);
     int lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t B);
     size_t lstm_scratch_floats() const;
+    // packed weight-gradient slabs of all LSTM directions: their total size (each rounded up to 64 floats), and
+    // re-pointing them into `base` (null: back to the layers' own buffers)
+    size_t lstm_gradient_slab_floats() const;
+    void lstm_bind_gradient_slabs(float *base);
     int lstm_update_derivative_weight(size_t li, size_t B, bool reductions);
     int lstm_update_derivative_weight_reductions(LstmLayer &q, size_t B);
     const float *lstm_tensor(size_t li, int kind, size_t *count);

@@ -9,6 +9,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -32,6 +33,35 @@ int hip_fail(hipError_t e, const char *what)
 {
     set_last_error("HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
     return MYEA_E_DEVICE;
+}
+
+// ---- static device scratch ------------------------------------------------------------------------------
+// Scratch memory of the allocation-free entry point (myea_hip_update_derivative_weight_no_alloc): partial sums of the
+// column reductions and split-K slabs live here instead of in buffers the library allocates.  Every device the
+// library runs on holds its own copy of the array, at its own address, until the process ends; in host code the
+// array's name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t kStaticScratchFloats = (size_t)8 << 20;   // 32 MiB
+static __device__ __align__(256) float static_scratch[kStaticScratchFloats];
+
+constexpr int kMaxDevices = 64;
+static float *g_static_scratch_address[kMaxDevices] = {};
+static std::mutex g_static_scratch_mutex;
+
+// the current device's copy of the array; resolved once per device
+static int static_scratch_address(float **out)
+{
+    int dev = -1;
+    MYEA_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) { set_last_error("static scratch: device ordinal %d out of range", dev); return MYEA_E_DEVICE; }
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (!g_static_scratch_address[dev]) {
+        void *p = nullptr;
+        MYEA_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch)));
+        if (!p) { set_last_error("static scratch: hipGetSymbolAddress returned a null address"); return MYEA_E_DEVICE; }
+        g_static_scratch_address[dev] = static_cast<float *>(p);
+    }
+    *out = g_static_scratch_address[dev];
+    return MYEA_OK;
 }
 
 // ---- small helpers ------------------------------------------------------------------------------------
@@ -310,6 +340,7 @@ int Net::create(const myea_net_desc &desc)
         size_t need = 258 * max_h + 2048;
         if (lstm_scratch_floats() > need) need = lstm_scratch_floats();
         MYEA_TRY(dev_alloc(&scratch, need));
+        scratch_floats = need;
     }
     {   // weight gradients of narrow layers over long T x batch row ranges run as split-K contractions into slabs
         size_t need = 0;
@@ -319,7 +350,9 @@ int Net::create(const myea_net_desc &desc)
             if (slabs > 1) need = std::max(need, (size_t)slabs * L[li].H * L[li].In);
         }
         if (need) MYEA_TRY(dev_alloc(&dw_slabs, need));
+        dw_slab_floats = need;
     }
+    MYEA_TRY(static_scratch_address(&static_scratch));   // set-up: this device's address of the static array
     MYEA_TRY(dev_alloc(&stage_in, T * B * L[0].H));
     MYEA_TRY(dev_alloc(&stage_out, T * B * L[d.n_layers - 1].H));
     {
@@ -1043,6 +1076,37 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
     return side_stream_join();
 }
 
+// Update_Derivative_Weight without any buffer of the library's own behind its kernels: the column reductions' partial
+// sums, the split-K slabs of narrow fully-connected layers and the packed weight-gradient slabs of the LSTM layers are
+// carved out of the static device array (in this order, each piece a multiple of 64 floats).  Same launches, same
+// results as update_derivative_weight.  Nothing is allocated or freed.  Every piece is written before it is read within
+// the call, so what an earlier call left in the array does not matter; calls that overlap on one device (two networks
+// on two streams) would share the array and race.
+int Net::update_derivative_weight_no_alloc(size_t B, size_t first, size_t end)
+{
+    auto round_up = [](size_t n) { return (n + 63) / 64 * 64; };
+    const size_t need = round_up(scratch_floats) + round_up(dw_slab_floats) + lstm_gradient_slab_floats();
+    if (need > kStaticScratchFloats) {
+        set_last_error("Update_Derivative_Weight (no allocation): this network's kernels need %zu bytes of scratch memory, the static buffer holds %zu",
+                       need * sizeof(float), kStaticScratchFloats * sizeof(float));
+        return MYEA_E_INVALID;
+    }
+    if (!static_scratch) { set_last_error("Update_Derivative_Weight (no allocation): the static buffer's address was not resolved"); return MYEA_E_DEVICE; }
+    float *const own_scratch = scratch, *const own_slabs = dw_slabs;
+    float *at = static_scratch;
+    scratch = at; at += round_up(scratch_floats);
+    if (own_slabs) dw_slabs = at;
+    at += round_up(dw_slab_floats);
+    lstm_bind_gradient_slabs(at);
+    const bool was_profiling = profiling;
+    profiling = false;   // the profiling taps create events on demand
+    const int rc = update_derivative_weight(B, first, end);
+    profiling = was_profiling;
+    scratch = own_scratch; dw_slabs = own_slabs;
+    lstm_bind_gradient_slabs(nullptr);
+    return rc;
+}
+
 // Per-unit activation arrays (struct AF_unit: ptr_type_activation_function / ptr_activation_steepness).  With them the
 // activation can no longer ride in a contraction's epilogue; it runs as its own kernel reading the arrays per column.
 int Net::set_unit_activations(size_t li, const uint32_t *types, const float *steep, size_t count)
@@ -1427,6 +1491,7 @@ int myea_hip_device_buffer_destroy(float *device)
 }
 int myea_hip_backward_pass(myea_hip_net *n, size_t B) { NET_OR_FAIL(n); return n->net.backward_pass(B); }
 int myea_hip_update_derivative_weight(myea_hip_net *n, size_t B, size_t first, size_t end) { NET_OR_FAIL(n); return n->net.update_derivative_weight(B, first, end); }
+int myea_hip_update_derivative_weight_no_alloc(myea_hip_net *n, size_t B, size_t first, size_t end) { NET_OR_FAIL(n); return n->net.update_derivative_weight_no_alloc(B, first, end); }
 int myea_hip_backward_pass_and_update_derivative_weight(myea_hip_net *n, size_t B) { NET_OR_FAIL(n); return n->net.backward_pass_and_update_derivative_weight(B); }
 int myea_hip_update_parameter(myea_hip_net *n, size_t B, size_t ts) { NET_OR_FAIL(n); return n->net.update_parameter(B, ts); }
 
