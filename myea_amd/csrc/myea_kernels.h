@@ -232,4 +232,34 @@ int launch_lstm_fused_forward(hipStream_t s, const LstmFusedForward &p);
 int launch_lstm_fused_backward(hipStream_t s, const LstmFusedBackward &p);
 int launch_transpose(hipStream_t s, size_t rows, size_t cols, const float *src, float *dst);
 
+// ---- LSTM time loop as one resident launch (one cell per block, C in {128, 256, 512, 1024}) --------------------------
+// one direction of a layer: packed parameters and the layer's [T][Bmax][..] tensors
+struct LstmResidentDir {
+    const float *Wrec;     // [4C][C] packed recurrent weights, rows z | i | f | o (forward)
+    const float *WrecT;    // [C][4C] their transpose (backward)
+    const float *bias;     // [4C]
+    const float *peep;     // [3][C]
+    float *acts;           // [T][Bmax][4C] in: input sums; out: the activations z, i, f, o
+    float *c, *ca, *h;     // [T][Bmax][C] cell state, tanh(cell state), cell output
+    float *dh, *dG, *dc;   // backward: [T][Bmax][C] delta of the outputs (in: from above; out: plus the recurrent term), [T][Bmax][4C], [T][Bmax][C]
+    const uint8_t *zone_state, *zone_output;   // zoneout masks [T][zone_stride] (1 = update) or null
+    size_t zone_stride;
+    int reverse;           // walks time from T - 1 down to 0
+};
+struct LstmResidentPlan {
+    bool ok = false;       // the resident form applies
+    bool agent = false;    // groups wider than one XCD: device-scope exchange
+    bool backward = false; // the backward loop has a resident form too
+    int cells = 0, members = 0, rs = 0, row_groups = 0, grid = 0, cus = 0;
+};
+int lstm_resident_plan(size_t C, size_t cells_per_block, size_t B, int dirs, LstmResidentPlan *plan);
+size_t lstm_resident_sync_words();
+// sync: lstm_resident_sync_words() unsigneds of device memory (cleared by the call); host_flag: a pinned host word the
+// kernel sets when a bounded wait gave up (1) or the members of a group did not share an XCD (2)
+int launch_lstm_resident_forward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
+                                 const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag);
+// dh must hold the delta from the layers above for every time step
+int launch_lstm_resident_backward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
+                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag);
+
 }  // namespace myea

@@ -564,11 +564,46 @@ int Net::side_stream_join()
 // One pair of timing events brackets a whole time loop: a pair per step costs more than the 10 us steps it would time.
 // Two directions: their steps are enqueued alternately, the second direction's on the side stream, so that neither
 // direction's launches wait behind the other's on the host; the event pair then brackets both loops.
+int Net::lstm_resident_dirs(DevLayer &o, LstmResidentDir *dirs)
+{
+    const bool zone = state == MYEA_STATE_TRAINING;   // zoneout acts strictly in the training state
+    int n = 0;
+    for (LstmLayer *q : {o.lstm, o.lstm2}) {
+        if (!q) continue;
+        LstmResidentDir r{};
+        r.Wrec = q->Wrec; r.WrecT = q->WrecT; r.bias = parameters + q->bias; r.peep = q->peep;
+        r.acts = q->acts; r.c = q->c; r.ca = q->ca; r.h = q->h;
+        r.dh = q->dh; r.dG = q->dG; r.dc = q->dc;
+        r.zone_state = zone ? q->zone_state : nullptr; r.zone_output = zone ? q->zone_output : nullptr; r.zone_stride = q->zone_stride;
+        r.reverse = q->reverse ? 1 : 0;
+        dirs[n++] = r;
+    }
+    return n;
+}
+
 int Net::lstm_forward_layer(size_t li, size_t B)
 {
     DevLayer &o = L[li];
     const size_t T = d.number_recurrent_depth;
     const double loop_work = 2.0 * (double)(T - 1) * (double)B * (double)o.lstm->G * (double)o.lstm->C;   // the recurrent contractions of steps 1 .. T-1
+    if (T > 1 && o.lstm->fused && !resident_off && resident_sync) {
+        // the whole time loop (both directions) as one launch when the layer's shape and the device allow it
+        LstmResidentPlan plan;
+        const int dirs = o.lstm2 ? 2 : 1;
+        MYEA_TRY(lstm_resident_plan(o.lstm->C, o.lstm->cpb, B, dirs, &plan));
+        if (plan.ok) {
+            MYEA_TRY(lstm_forward_inputs(li, *o.lstm, B));
+            if (o.lstm2) MYEA_TRY(lstm_forward_inputs(li, *o.lstm2, B));
+            LstmResidentDir rd[2];
+            lstm_resident_dirs(o, rd);
+            prof_begin(0);
+            MYEA_TRY(launch_lstm_resident_forward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag));
+            prof_end(dirs * loop_work, 1);
+            if (!o.lstm2) return MYEA_OK;
+            const size_t rows = (size_t)d.number_recurrent_depth * d.batch_size;
+            return launch_padded_add(stream, rows, o.H, o.lstm->h, o.H, 0, o.lstm2->h, o.H, 0, o.values);  // output = h_forward + h_backward
+        }
+    }
     if (!o.lstm2) {
         MYEA_TRY(lstm_forward_inputs(li, *o.lstm, B));
         if (T > 1) prof_begin(0);
@@ -646,6 +681,21 @@ int Net::lstm_backward_layer(size_t li, size_t B)
             MYEA_HIP_TRY(hipMemcpyAsync(q.dh, o.neuron_errors, (size_t)d.number_recurrent_depth * d.batch_size * q.C * sizeof(float), hipMemcpyDeviceToDevice, stream));
         return MYEA_OK;
     };
+    if (T > 1 && o.lstm->fused && !resident_off && resident_sync) {
+        LstmResidentPlan plan;
+        const int dirs = o.lstm2 ? 2 : 1;
+        MYEA_TRY(lstm_resident_plan(o.lstm->C, o.lstm->cpb, B, dirs, &plan));
+        if (plan.ok && plan.backward) {   // the whole backward time loop (both directions) as one launch
+            MYEA_TRY(seed(*o.lstm));
+            if (o.lstm2) MYEA_TRY(seed(*o.lstm2));
+            LstmResidentDir rd[2];
+            lstm_resident_dirs(o, rd);
+            prof_begin(1);
+            MYEA_TRY(launch_lstm_resident_backward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag));
+            prof_end(dirs * loop_work, 1);
+            return MYEA_OK;
+        }
+    }
     if (!o.lstm2) {
         MYEA_TRY(seed(*o.lstm));
         if (T > 1) prof_begin(1);

@@ -1,0 +1,975 @@
+// myea_lstm_resident.hip — the time loop of an LSTM layer as ONE launch: a workgroup stays on its compute unit for all
+// time steps, keeps its slice of the recurrent weights in registers, and meets the other workgroups that share its
+// examples at a bounded barrier between steps.
+//
+// Why: as one launch per time step (myea_lstm_fused.hip) every step pays a launch, the fill and drain of a kernel that
+// lives for 10 us, and a fresh fetch of the workgroup's 128 KB weight slice.  The recurrence only needs, per step, what
+// the previous step produced for the SAME examples: workgroups that own different examples never talk.
+//
+// Shape of the work (one cell per block, C cells, gate rows z | i | f | o of the packed matrices):
+//   * a workgroup owns CELLS cells (16, or 8 when C > 512).  Forward: the 4 CELLS gate columns of those cells, its four wavefronts split
+//     k = C into contiguous quarters; backward: the CELLS columns of dh, wavefront w takes the k range of gate w.  Either
+//     way a wavefront holds its [columns][k range] slice of Wrec (WrecT) in registers for the whole launch (at most 128
+//     registers per lane) in the operand layout of v_mfma_f32_16x16x4_f32;
+//   * a GROUP is the set of workgroups that cover all C cells for 2 x ROWS examples of one direction (ROWS = 16 RS):
+//     C / CELLS members.  A member is a workgroup of four wavefronts - one per SIMD - that lives for all T steps and keeps
+//     its slice of the recurrent matrix in registers.  It works on two independent CHAINS of ROWS examples in turn: a
+//     UNIT is one time step of one chain, and the units of the two chains alternate in program order.
+//   * A unit: the exchanged tensor of the chain's examples (h[t-1] forward, the gate deltas dG[t+1] backward) arrives in
+//     LDS (global -> LDS directly, every wavefront only its own k range); MFMAs against the register-resident weights; the
+//     four partial tiles meet in LDS; gate math of the lane's (example, cell) pair(s); stores.
+//   * On this device the fp32 MFMAs and ordinary vector instructions of a SIMD do not overlap, whichever wavefront they
+//     come from (measured), so a second wavefront per SIMD buys nothing; what can be hidden is latency.  The chain that
+//     is not computing is the one whose stores, barrier and tile loads are in flight:
+//       - a unit's arrival at its chain's counter is signalled a quarter into the NEXT unit's MFMAs, when its stores have
+//         long been acknowledged;
+//       - the counter is read three quarters into those MFMAs and is normally complete at their end;
+//       - the tiles of the unit after that are requested then, and land under the partial exchange and the gate math.
+//
+// Barriers and visibility.  Two protocols, chosen on the host:
+//   * LOCAL: every member of a group runs on the same XCD (workgroup ids that are equal mod 8 share an XCD; the host
+//     checks that with a probe launch once per process, and in every launch the members of a group compare their XCC
+//     ids).  The XCD's L2 is then the point of coherence: plain stores, a counter bumped by an atomic performed in L2 and
+//     polled with loads that bypass the compute unit's L1 (sc1), as do the loads of the exchanged tensor;
+//   * AGENT (groups wider than an XCD, C = 1024, forward only): device-scope stores of h, device-scope counter, sc1 loads.
+// A wavefront arrives once its own stores are complete (vmcnt(0)); the last of the four - counted in LDS - bumps the
+// chain's counter.  A wait is bounded: after `spin_polls` polls the waiting wavefront raises the give-up flag, every
+// wavefront sees it at its next poll and leaves, the kernel ends normally and the host reports MYEA_E_DEVICE.
+// The host only launches when every workgroup of the grid can be resident at once (one per compute unit).
+//
+// vmcnt: the loads and stores of a wavefront complete in issue order as far as the counter is concerned, so "at most N
+// outstanding" with N = the stores issued after a unit's tile loads says that the tiles have landed.  Every lane issues
+// the same stores: lanes whose example lies beyond the batch write to a scrap area.
+//
+// Gate math: Forward_Pass__LSTM__Gates_CIF_AF_State (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:1042-1191),
+// __States_AF (:1547-1582), __Output (:1351-1418); backward: Backward_Pass__LSTM_Derivative__Output
+// (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:1130-1273), __Cell_State_AF (:1275-1327),
+// __Gates_CIF_AF_State (:1329-1604).  NN/ = Neural_Network_Library_Windows/Source_Files/Neural_Network/.
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <type_traits>
+#include <vector>
+
+#include "myea_kernels.h"
+
+namespace myea {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;      // four wavefronts, one per SIMD
+constexpr int kSyncStride = 32;    // counters sit 128 bytes apart
+constexpr int kMaxGroups = 64;     // groups a network's counter block holds
+constexpr int kScrapWords = 8192;   // where lanes without an example put their stores: 4 gate rows of up to 1024 + 4 x 1024
+constexpr int kLocalAux = 16;      // cache policy of the LOCAL protocol's tile loads: sc1, served by L2, never by this compute unit's L1
+
+#define MYEA_SCOPE_AGENT __HIP_MEMORY_SCOPE_AGENT
+#define MYEA_SCOPE_WORKGROUP __HIP_MEMORY_SCOPE_WORKGROUP
+
+// LDS of a workgroup: every wavefront's tiles of one unit, and the partial tiles of the two chains
+constexpr size_t forward_lds(int kw, int cells, int rs) { return ((size_t)4 * (kw / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * (4 * cells + 8)) * sizeof(float); }
+constexpr size_t backward_lds(int c, int rs) { return ((size_t)4 * (c / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * 17) * sizeof(float); }
+
+template <int N>
+__device__ __forceinline__ void wait_vm() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }   // vmcnt(N)
+
+// Workgroup barrier for data exchanged through LDS only: waits for this wavefront's LDS operations, not for its global
+// loads and stores (the next unit's tiles are in flight across it).
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+}
+
+// exp2 and reciprocal instructions (1 ulp each) instead of the library's expf and an IEEE division: the error stays some
+// orders of magnitude below the tolerance the gate activations are held to, and the vector pipe is what a unit waits for
+__device__ __forceinline__ float sigmoid_f(float s) { return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896341f * s)); }
+__device__ __forceinline__ float tanh_f(float s) { return 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-2.88539008177792681f * s)) - 1.f; }  // AF_TANH_real
+
+// [ROWS][32 k] tile of one wavefront in LDS, 16-byte chunks XOR-swizzled by (row >> 1) & 7; one direct load brings 8 rows.
+// AUX = 16 (sc1): the load is served beyond this compute unit's L1 at device scope; AUX = 0: a plain load.
+template <int ROWS, int AUX>
+struct ATile {
+    const float *ptr[ROWS / 8];
+    template <class RowOf>
+    __device__ __forceinline__ void init(const float *base, size_t ld, size_t k0, RowOf row_of)
+    {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int q = 0; q < ROWS / 8; ++q) {
+            const int r = q * 8 + (lane >> 3);
+            const int chunk = (lane & 7) ^ ((r >> 1) & 7);
+            ptr[q] = base + row_of(r) * ld + k0 + chunk * 4;
+        }
+    }
+    // tile number `i` of the wavefront's k range
+    __device__ __forceinline__ void fill(float *tile, int i) const
+    {
+#pragma unroll
+        for (int q = 0; q < ROWS / 8; ++q)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(ptr[q] + i * 32),
+                                             (__attribute__((address_space(3))) void *)(tile + q * 256), 16, 0, AUX);
+    }
+    static __device__ __forceinline__ f32x4 chunk(const float *tile, int row, int c)
+    {
+        return *reinterpret_cast<const f32x4 *>(tile + row * 32 + ((c ^ ((row >> 1) & 7)) << 2));
+    }
+};
+
+struct SyncWords {
+    unsigned *counters;   // [(group * 2 + chain) * kSyncStride]
+    unsigned *give_up;    // device flag, polled; behind it one word per group: the XCC id its first member ran on (+ 1)
+    unsigned *host_flag;  // pinned host word, written once on give-up
+    float *scrap;         // kScrapWords floats nobody reads
+};
+
+// One lane per wavefront talks to the counters.  A wavefront arrives once its own stores are complete; the last of the
+// workgroup's four (counted in LDS; the four stay within one unit of each other, so the count never mixes two units)
+// bumps the group's counter: one atomic per workgroup and unit on that cache line.
+template <bool AGENT>
+__device__ __forceinline__ void wave_arrive(unsigned *counter, unsigned *lds_count)
+{
+    if ((threadIdx.x & 63) == 0) {
+        const unsigned before = __hip_atomic_fetch_add(lds_count, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_WORKGROUP);
+        if ((before & 3u) == 3u) {
+            if (AGENT) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+            else __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_WORKGROUP);
+        }
+    }
+}
+
+// Waits until the counter reaches `target`.  Returns (to every lane) 1 when it did, 0 when the wait gave up here or
+// elsewhere.  One lane polls; the poll is a load that bypasses this compute unit's L1 (many wavefronts read the line, few
+// write it: reads do not queue behind one another the way atomics on one address do).  The loop - poll, look at the
+// give-up flag, count down, raise the flag when the count runs out - is one block of assembly: written in C++, a loop
+// with loads in it makes the compiler's wait-count bookkeeping pessimistic for what follows (it drains all memory
+// operations in front of the first MFMA).  Only lane 0 is active in the block, so vcc holds just its compare result.
+__device__ __forceinline__ int wave_wait(const SyncWords &w, unsigned *counter, unsigned target, unsigned spin_polls)
+{
+    int ok = 1;
+    if ((threadIdx.x & 63) == 0) {
+        unsigned value, polls = spin_polls;
+        asm volatile(
+            "v_mov_b32 %[ok], 0\n"
+            "1:\n\t"
+            "global_load_dword %[value], %[counter], off sc1\n\t"
+            "s_waitcnt vmcnt(0)\n\t"
+            "v_sub_u32 %[value], %[value], %[target]\n\t"
+            "v_cmp_le_i32 vcc, 0, %[value]\n\t"
+            "s_cbranch_vccnz 2f\n\t"
+            "global_load_dword %[value], %[give_up], off sc1\n\t"
+            "s_waitcnt vmcnt(0)\n\t"
+            "v_cmp_ne_u32 vcc, 0, %[value]\n\t"
+            "s_cbranch_vccnz 3f\n\t"
+            "s_sleep 2\n\t"
+            "s_sub_u32 %[polls], %[polls], 1\n\t"
+            "s_cmp_lg_u32 %[polls], 0\n\t"
+            "s_cbranch_scc1 1b\n\t"
+            "v_mov_b32 %[value], 1\n\t"
+            "global_store_dword %[give_up], %[value], off sc1\n\t"
+            "global_store_dword %[host_flag], %[value], off sc0 sc1\n\t"
+            "s_waitcnt vmcnt(0)\n\t"
+            "s_branch 3f\n"
+            "2:\n\t"
+            "v_mov_b32 %[ok], 1\n"
+            "3:\n"
+            : [ok] "=&v"(ok), [value] "=&v"(value), [polls] "+s"(polls)
+            : [counter] "v"(counter), [give_up] "v"(w.give_up), [host_flag] "v"(w.host_flag), [target] "v"(target)
+            : "vcc", "scc", "memory");
+    }
+    return __builtin_amdgcn_readfirstlane(ok);
+}
+
+__device__ __forceinline__ unsigned xcc_id() { return __builtin_amdgcn_s_getreg(20 | (3 << 11)) & 15u; }   // HW_REG_XCC_ID[3:0]
+
+// workgroup id -> (group, member).  LOCAL: the XCD of ids = x (mod 8) hosts the groups x, x + 8, ...; AGENT: members of a
+// group are spread over the XCDs.  Returns false for a workgroup without work.
+template <bool AGENT>
+__device__ __forceinline__ bool place(unsigned id, int members, int groups, int &group, int &member)
+{
+    if (AGENT) { group = (int)(id % (unsigned)groups); member = (int)(id / (unsigned)groups); return member < members; }
+    const int xcd = (int)(id & 7), slot = (int)(id >> 3);
+    group = (slot / members) * 8 + xcd;
+    member = slot % members;
+    return group < groups;
+}
+
+// LOCAL: every member of the group must sit on the same XCD (which one depends on the hardware queue the launch went
+// through): the first member to get here writes its XCC id, the others compare.  A member elsewhere does not share the
+// group's L2: it stops everybody.
+__device__ __forceinline__ void check_same_xcd(const SyncWords &w, int group)
+{
+    if (threadIdx.x != 0) return;
+    unsigned *word = w.give_up + 1 + group;
+    const unsigned mine = xcc_id() + 1u;
+    unsigned seen = 0u;
+    if (!__hip_atomic_compare_exchange_strong(word, &seen, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT) && seen != mine) {
+        __hip_atomic_store(w.give_up, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+        __hip_atomic_store(w.host_flag, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
+}  // namespace
+
+struct ResidentGeometry {
+    int T, B, Bmax, C;
+    int dirs, row_groups;      // groups = dirs * row_groups; group g: direction g % dirs, examples from (g / dirs) * 2 ROWS
+    int members;               // workgroups per group = C / CELLS
+    unsigned spin_polls;       // polls after which a wait gives up
+};
+
+namespace {
+
+// ---- forward ---------------------------------------------------------------------------------------------------------
+// KW = C / 4: k's per wavefront.  Chain 0 holds the group's first ROWS examples, chain 1 the next ROWS.
+// Per lane the addresses of its (example, cell) pair(s) and of its tile rows are set up once and then stepped.
+using Chain0 = std::integral_constant<int, 0>;
+using Chain1 = std::integral_constant<int, 1>;
+
+template <int KW, int CELLS, int RS, bool AGENT>
+__global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(ResidentGeometry g, LstmResidentDir d0, LstmResidentDir d1, SyncWords w)
+{
+    constexpr int C = 4 * KW, G = 4 * C;
+    constexpr int NB = 4 * CELLS, NCT = NB / 16, ROWS = 16 * RS, NT = KW / 32;
+    constexpr int LPT = ROWS / 8;                 // direct loads per tile
+    constexpr int PAIRS = ROWS * CELLS / kThreads;
+    constexpr int NSTORE = 7 * PAIRS;             // stores of a unit
+    constexpr int A1 = NT >= 4 ? NT / 4 : 1;      // tiles whose MFMAs run before the previous unit's arrival is signalled
+    constexpr int P1 = NT >= 4 ? (3 * NT) / 4 : NT - 1;   // tile before which the next unit's counter is read
+    constexpr int kStride = NB + 8;               // floats per row of a wavefront's partial tile
+    constexpr int kStage = NT * ROWS * 32, kPart = 4 * ROWS * kStride;
+    constexpr int kAux = AGENT ? 16 : kLocalAux;
+    static_assert(PAIRS >= 1 && ROWS * CELLS % kThreads == 0, "every lane has the same number of pairs");
+    static_assert(NT * LPT + NSTORE < 64, "vmcnt has 6 bits");
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    __shared__ unsigned s_arrive[2];   // wavefronts that arrived, per chain
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col16 = lane & 15, quad = lane >> 4;
+
+    int group, member;
+    if (!place<AGENT>(blockIdx.x, g.members, g.dirs * g.row_groups, group, member)) return;
+    const int dir = group % g.dirs, rg = group / g.dirs;
+    const LstmResidentDir &d = dir ? d1 : d0;
+    const int c0 = member * CELLS, B = g.B, T = g.T;
+    const size_t Bmax = (size_t)g.Bmax;
+    unsigned *const counters = w.counters + (size_t)group * 2 * kSyncStride;   // chain c: counters + c * kSyncStride
+    const unsigned members = (unsigned)g.members;
+    if (!AGENT) check_same_xcd(w, group);
+    if (threadIdx.x < 2) s_arrive[threadIdx.x] = 0u;
+    __syncthreads();
+
+    float *const stage = smem + wave * kStage;   // this wavefront's tiles of the unit in flight
+    float *const parts = smem + 4 * kStage;      // [chain][4 wavefronts][ROWS][kStride]
+
+    // the weight slice: gate column j = ct * 16 + col16 of the workgroup is gate j / CELLS of cell c0 + j % CELLS
+    f32x4 breg[NT][2][NCT];
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct) {
+        const int j = ct * 16 + col16;
+        const float *row = d.Wrec + ((size_t)(j / CELLS) * C + c0 + (j % CELLS)) * C + wave * KW;
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) breg[i][h][ct] = *reinterpret_cast<const f32x4 *>(row + i * 32 + (h * 4 + quad) * 4);
+    }
+    const int t_first = d.reverse ? T - 1 : 0;
+    const ptrdiff_t t_step = d.reverse ? -1 : 1;
+    const ptrdiff_t step_g = t_step * (ptrdiff_t)(Bmax * G), step_c = t_step * (ptrdiff_t)(Bmax * C);
+    const ptrdiff_t zone_step = t_step * (ptrdiff_t)d.zone_stride;
+    // the lane's pairs: constants shared by the chains; per chain the state carried from step to step and the addresses
+    float e_bias[PAIRS][4], e_peep[PAIRS][3];
+    float c_prev[2][PAIRS], h_prev[2][PAIRS], e_in[PAIRS][4];
+    unsigned keep_c[PAIRS], keep_h[PAIRS];   // 0: a zoned-out cell keeps its previous state / output at this step
+    float *p_acts[2][PAIRS], *p_c[2][PAIRS], *p_ca[2][PAIRS], *p_h[2][PAIRS];
+    ptrdiff_t lane_step_c[2][PAIRS];   // 0 for a lane whose stores go to the scrap area
+    const unsigned char *p_zone_c[PAIRS], *p_zone_h[PAIRS];   // chain 0's step; chain 1 is at the same one or one behind
+    const float *p_tile[2][LPT];
+#pragma unroll
+    for (int q = 0; q < PAIRS; ++q) {
+        const int pair = threadIdx.x + q * kThreads, row = pair / CELLS, cell = pair % CELLS, k = c0 + cell;
+#pragma unroll
+        for (int gate = 0; gate < 4; ++gate) e_bias[q][gate] = d.bias[gate * C + k];
+#pragma unroll
+        for (int gate = 0; gate < 3; ++gate) e_peep[q][gate] = d.peep[gate * C + k];
+        p_zone_c[q] = d.zone_state ? d.zone_state + (size_t)t_first * d.zone_stride + k : nullptr;
+        p_zone_h[q] = d.zone_output ? d.zone_output + (size_t)t_first * d.zone_stride + k : nullptr;
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch) {
+            const int r = (rg * 2 + ch) * ROWS + row;
+            const bool valid = r < B;
+            const size_t at = (size_t)t_first * Bmax + min(r, B - 1);
+            float *scrap = w.scrap + 4096 + (ch * PAIRS + q) * kThreads + threadIdx.x;
+            p_acts[ch][q] = d.acts + at * G + k;   // the input sums; a lane without an example reads the batch's last example's
+            p_c[ch][q] = valid ? d.c + at * C + k : scrap;
+            p_ca[ch][q] = valid ? d.ca + at * C + k : scrap + 1024;
+            p_h[ch][q] = valid ? d.h + at * C + k : scrap + 2048;
+            lane_step_c[ch][q] = valid ? step_c : 0;
+            c_prev[ch][q] = 0.f; h_prev[ch][q] = 0.f;
+        }
+    }
+    // where the gate activations go: over the input sums, or for a lane without an example to the scrap area
+    float *p_acts_out[2][PAIRS];
+    ptrdiff_t lane_step_out[2][PAIRS];
+#pragma unroll
+    for (int q = 0; q < PAIRS; ++q)
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch) {
+            const int pair = threadIdx.x + q * kThreads, r = (rg * 2 + ch) * ROWS + pair / CELLS;
+            p_acts_out[ch][q] = r < B ? p_acts[ch][q] : w.scrap + (ch * PAIRS + q) * kThreads + threadIdx.x;
+            lane_step_out[ch][q] = r < B ? step_g : 0;
+        }
+    // rows of h the wavefront stages (clamped to the batch), at the direction's first step
+#pragma unroll
+    for (int ch = 0; ch < 2; ++ch)
+#pragma unroll
+        for (int q = 0; q < LPT; ++q) {
+            const int r = q * 8 + (lane >> 3), chunk = (lane & 7) ^ ((r >> 1) & 7);
+            p_tile[ch][q] = d.h + ((size_t)t_first * Bmax + min((rg * 2 + ch) * ROWS + r, B - 1)) * C + wave * KW + chunk * 4;
+        }
+
+    f32x4 acc[RS][NCT];
+    unsigned seen = 0;   // the next unit's counter as read during the MFMAs
+
+    auto load_inputs = [&](auto ch) {   // input sums (and zoneout masks) of the step the chain's pointers are at
+        constexpr int c = decltype(ch)::value;
+#pragma unroll
+        for (int q = 0; q < PAIRS; ++q) {
+#pragma unroll
+            for (int gate = 0; gate < 4; ++gate) e_in[q][gate] = p_acts[c][q][gate * C];
+            keep_c[q] = 1u; keep_h[q] = 1u;
+        }
+        if (d.zone_state) {
+#pragma unroll
+            for (int q = 0; q < PAIRS; ++q) keep_c[q] = p_zone_c[q][0];
+        }
+        if (d.zone_output) {
+#pragma unroll
+            for (int q = 0; q < PAIRS; ++q) keep_h[q] = p_zone_h[q][0];
+        }
+    };
+    auto load_tiles = [&](auto ch) {   // h of the step before the one the chain's pointers are at: p_tile is one step behind
+        constexpr int c = decltype(ch)::value;
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+#pragma unroll
+            for (int q = 0; q < LPT; ++q)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p_tile[c][q] + i * 32),
+                                                 (__attribute__((address_space(3))) void *)(stage + i * ROWS * 32 + q * 256), 16, 0, kAux);
+#pragma unroll
+        for (int q = 0; q < LPT; ++q) p_tile[c][q] += step_c;
+    };
+    auto mfma_tiles = [&](auto first, auto last) {
+#pragma unroll
+        for (int i = decltype(first)::value; i < decltype(last)::value; ++i) {
+            const float *tile = stage + i * ROWS * 32;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                f32x4 fa[RS];
+#pragma unroll
+                for (int rs = 0; rs < RS; ++rs) fa[rs] = ATile<ROWS, kAux>::chunk(tile, rs * 16 + col16, h * 4 + quad);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                        for (int rs = 0; rs < RS; ++rs)
+                            acc[rs][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[rs][e], breg[i][h][ct][e], acc[rs][ct], 0, 0, 0);
+            }
+        }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using IA = std::integral_constant<int, A1>;
+    using IP = std::integral_constant<int, (P1 > A1 ? P1 : A1)>;
+    using IN = std::integral_constant<int, NT>;
+
+    // The first part of a unit with a recurrent term: its tiles have landed when only the previous unit's stores can be
+    // outstanding; after a quarter of the MFMAs those stores are complete too and the previous unit - of the other chain -
+    // arrives.  all_landed: nothing may be outstanding (after the first units, whose requests were made in another order).
+    auto head = [&](auto ch, auto all_landed) {
+        constexpr int c = decltype(ch)::value;
+#pragma unroll
+        for (int rs = 0; rs < RS; ++rs)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct) acc[rs][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (decltype(all_landed)::value) wait_vm<0>(); else wait_vm<NSTORE>();
+        mfma_tiles(I0{}, IA{});
+        __builtin_amdgcn_sched_barrier(0);   // keeps the MFMAs above in front of the wait
+        wait_vm<0>();
+        wave_arrive<AGENT>(counters + (1 - c) * kSyncStride, &s_arrive[1 - c]);
+    };
+    // The rest of the unit.  FIRST: the chain's first step (no recurrent term, no forget gate, no peephole into the input
+    // gate).  wait_for: the other chain's units that must have arrived before its next unit's tiles are requested (0: that
+    // unit has no recurrent term, or there is none).  Returns false when a wait gave up.
+    auto tail = [&](auto ch, auto first_tag, unsigned wait_for) -> bool {
+        constexpr int c = decltype(ch)::value;
+        constexpr bool FIRST = decltype(first_tag)::value;
+        load_inputs(ch);
+        if (!FIRST) {
+            mfma_tiles(IA{}, IP{});
+            if (wait_for) seen = __hip_atomic_load(counters + (1 - c) * kSyncStride, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+            mfma_tiles(IP{}, IN{});
+            __builtin_amdgcn_sched_barrier(0);   // the counter's value is looked at after the MFMAs, not right behind its load
+        }
+        if (wait_for) {
+            const unsigned target = wait_for * members;
+            const bool there = !FIRST && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0;
+            if (!there && !wave_wait(w, counters + (1 - c) * kSyncStride, target, g.spin_polls)) return false;
+            load_tiles(std::integral_constant<int, 1 - c>{});   // every wavefront's reads of this unit's tiles have been issued and waited for by its MFMAs
+        }
+        float *part = parts + c * kPart;
+        if (!FIRST) {
+            float *to = part + wave * ROWS * kStride;
+#pragma unroll
+            for (int rs = 0; rs < RS; ++rs)
+#pragma unroll
+                for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) to[(rs * 16 + quad * 4 + r) * kStride + ct * 16 + col16] = acc[rs][ct][r];
+            lds_barrier();
+        }
+#pragma unroll
+        for (int q = 0; q < PAIRS; ++q) {
+            const int pair = threadIdx.x + q * kThreads, row = pair / CELLS, cell = pair % CELLS;
+            float rec[4] = {0.f, 0.f, 0.f, 0.f};
+            if (!FIRST) {
+#pragma unroll
+                for (int gate = 0; gate < 4; ++gate) {
+                    float v = 0.f;
+#pragma unroll
+                    for (int wv = 0; wv < 4; ++wv) v += part[(wv * ROWS + row) * kStride + gate * CELLS + cell];
+                    rec[gate] = v;
+                }
+            }
+            const float cp = c_prev[c][q];
+            float si = e_in[q][1] + rec[1] + e_bias[q][1];
+            float gf = 0.f;
+            if (!FIRST) {
+                float sf = e_in[q][2] + rec[2] + e_bias[q][2];
+                si += cp * e_peep[q][0];
+                sf += cp * e_peep[q][1];
+                gf = sigmoid_f(sf);
+            }
+            const float gi = sigmoid_f(si);
+            const float z = tanh_f(e_in[q][0] + rec[0] + e_bias[q][0]);
+            float cs = FIRST ? z * gi : z * gi + gf * cp;
+            cs = keep_c[q] ? cs : cp;   // a zoned-out cell state keeps the previous one (0 on the first step)
+            const float a = tanh_f(cs);
+            const float so = e_in[q][3] + rec[3] + e_bias[q][3] + cs * e_peep[q][2];
+            const float go = sigmoid_f(so);
+            float hv = a * go;
+            hv = keep_h[q] ? hv : h_prev[c][q];
+            c_prev[c][q] = cs; h_prev[c][q] = hv;
+            if (AGENT) __hip_atomic_store(p_h[c][q], hv, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+            else *p_h[c][q] = hv;
+            float *arow = p_acts_out[c][q];
+            arow[0] = z; arow[C] = gi; arow[2 * C] = gf; arow[3 * C] = go;
+            *p_c[c][q] = cs; *p_ca[c][q] = a;
+            p_h[c][q] += lane_step_c[c][q]; p_c[c][q] += lane_step_c[c][q]; p_ca[c][q] += lane_step_c[c][q];
+            p_acts[c][q] += step_g; p_acts_out[c][q] += lane_step_out[c][q];
+        }
+        if (c == 1) {   // both chains have used this step's masks
+#pragma unroll
+            for (int q = 0; q < PAIRS; ++q) { if (d.zone_state) p_zone_c[q] += zone_step; if (d.zone_output) p_zone_h[q] += zone_step; }
+        }
+        return true;
+    };
+    using First = std::true_type;
+    using Later = std::false_type;
+
+    // units in program order: (0,0) (1,0) (0,1) (1,1) ... ; unit (c, s) needs every member's h of unit (c, s - 1)
+    if (!tail(Chain0{}, First{}, 0u)) return;
+    wait_vm<0>();
+    wave_arrive<AGENT>(counters, &s_arrive[0]);          // unit (0, 0)
+    if (!tail(Chain1{}, First{}, 1u)) return;            // requests the tiles of unit (0, 1)
+    head(Chain0{}, std::true_type{});                    // signals unit (1, 0)
+    for (int s = 1; s + 1 < T; ++s) {
+        if (!tail(Chain0{}, Later{}, (unsigned)s)) return;          // chain 1 has arrived s times: tiles of unit (1, s)
+        head(Chain1{}, std::false_type{});                          // signals unit (0, s)
+        if (!tail(Chain1{}, Later{}, (unsigned)s + 1u)) return;     // tiles of unit (0, s + 1)
+        head(Chain0{}, std::false_type{});                          // signals unit (1, s)
+    }
+    if (!tail(Chain0{}, Later{}, (unsigned)(T - 1))) return;
+    head(Chain1{}, std::false_type{});
+    if (!tail(Chain1{}, Later{}, 0u)) return;
+}
+
+// ---- backward --------------------------------------------------------------------------------------------------------
+// dh[t] += dG[t'] Wrec (t' = the step processed before t in this pass), then the gate deltas of step t.  The workgroup owns
+// CELLS = 16 columns of dh; wavefront w contracts over the k range of gate w (k = gate * C + cell of dG[t']) against its
+// slice of the transposed packed matrix WrecT [C][4C].  j counts the steps of this pass: the direction's own step is
+// s = T - 1 - j.  j = 0 has no recurrent term and no terms from a later step; s = 0 writes no forget-gate delta.
+template <int CC, int RS>
+__global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(ResidentGeometry g, LstmResidentDir d0, LstmResidentDir d1, SyncWords w)
+{
+    constexpr int C = CC, G = 4 * C, CELLS = 16;
+    constexpr int ROWS = 16 * RS, NT = C / 32;    // tiles of 32 k in a gate's range
+    constexpr int LPT = ROWS / 8;
+    constexpr int PAIRS = ROWS * CELLS / kThreads;
+    constexpr int NSTORE = 6 * PAIRS;
+    constexpr int A1 = NT / 4, P1 = (3 * NT) / 4;
+    constexpr int kStride = 17;
+    constexpr int kStage = NT * ROWS * 32, kPart = 4 * ROWS * kStride;
+    constexpr int kAux = kLocalAux;
+    static_assert(NT >= 4 && NT * LPT + NSTORE < 64, "vmcnt has 6 bits");
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    __shared__ unsigned s_arrive[2];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col16 = lane & 15, quad = lane >> 4;
+
+    int group, member;
+    if (!place<false>(blockIdx.x, g.members, g.dirs * g.row_groups, group, member)) return;
+    const int dir = group % g.dirs, rg = group / g.dirs;
+    const LstmResidentDir &d = dir ? d1 : d0;
+    const int c0 = member * CELLS, B = g.B, T = g.T;
+    const size_t Bmax = (size_t)g.Bmax;
+    unsigned *const counters = w.counters + (size_t)group * 2 * kSyncStride;
+    const unsigned members = (unsigned)g.members;
+    check_same_xcd(w, group);
+    if (threadIdx.x < 2) s_arrive[threadIdx.x] = 0u;
+    __syncthreads();
+
+    float *const stage = smem + wave * kStage;
+    float *const parts = smem + 4 * kStage;
+
+    // WrecT rows c0 .. c0 + 15, the k range of gate `wave`
+    f32x4 breg[NT][2];
+    {
+        const float *row = d.WrecT + (size_t)(c0 + col16) * G + (size_t)wave * C;
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) breg[i][h] = *reinterpret_cast<const f32x4 *>(row + i * 32 + (h * 4 + quad) * 4);
+    }
+    // this pass walks the direction's steps from its last to its first: in time, forwards for the reversed direction
+    const int t_first = d.reverse ? 0 : T - 1;
+    const ptrdiff_t t_step = d.reverse ? 1 : -1;
+    const ptrdiff_t step_g = t_step * (ptrdiff_t)(Bmax * G), step_c = t_step * (ptrdiff_t)(Bmax * C);
+    float e_peep[PAIRS][3];
+    float n_di[2][PAIRS], n_df[2][PAIRS], n_f[2][PAIRS], n_dc[2][PAIRS];   // of the chain's step processed before: delta i, delta f, f, delta c
+    float e_act[PAIRS][4], e_ca[PAIRS], e_cp[PAIRS], e_dh[PAIRS];
+    const float *p_acts[2][PAIRS], *p_ca[2][PAIRS], *p_cp[2][PAIRS], *p_dh_in[2][PAIRS];   // read: the batch's last example for a lane without one
+    float *p_dh[2][PAIRS], *p_dG[2][PAIRS], *p_dc[2][PAIRS];                                  // written: the scrap area for such a lane
+    ptrdiff_t lane_step_g[2][PAIRS], lane_step_c[2][PAIRS];
+    const float *p_tile[2][LPT];
+#pragma unroll
+    for (int q = 0; q < PAIRS; ++q) {
+        const int pair = threadIdx.x + q * kThreads, row = pair >> 4, cell = pair & 15, k = c0 + cell;
+#pragma unroll
+        for (int gate = 0; gate < 3; ++gate) e_peep[q][gate] = d.peep[gate * C + k];
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch) {
+            const int r = (rg * 2 + ch) * ROWS + row;
+            const bool valid = r < B;
+            const size_t at = (size_t)t_first * Bmax + min(r, B - 1);
+            float *scrap = w.scrap + (ch * PAIRS + q) * kThreads + threadIdx.x;
+            p_acts[ch][q] = d.acts + at * G + k;
+            p_ca[ch][q] = d.ca + at * C + k;
+            p_cp[ch][q] = d.c + at * C + k + step_c;   // the cell state of the step before t in the direction's order: one step further along this pass
+            p_dh_in[ch][q] = d.dh + at * C + k;
+            p_dh[ch][q] = valid ? d.dh + at * C + k : scrap + 4096;
+            p_dG[ch][q] = valid ? d.dG + at * G + k : scrap;
+            p_dc[ch][q] = valid ? d.dc + at * C + k : scrap + 4096 + 1024;
+            lane_step_g[ch][q] = valid ? step_g : 0;
+            lane_step_c[ch][q] = valid ? step_c : 0;
+            n_di[ch][q] = 0.f; n_df[ch][q] = 0.f; n_f[ch][q] = 0.f; n_dc[ch][q] = 0.f;
+        }
+    }
+    // rows of dG the wavefront stages, the k range of its gate, at the pass's first step
+#pragma unroll
+    for (int ch = 0; ch < 2; ++ch)
+#pragma unroll
+        for (int q = 0; q < LPT; ++q) {
+            const int r = q * 8 + (lane >> 3), chunk = (lane & 7) ^ ((r >> 1) & 7);
+            p_tile[ch][q] = d.dG + ((size_t)t_first * Bmax + min((rg * 2 + ch) * ROWS + r, B - 1)) * G + (size_t)wave * C + chunk * 4;
+        }
+
+    f32x4 acc[RS][2];
+    unsigned seen = 0;
+
+    auto load_operands = [&](auto ch, bool with_cp) {   // of the step the chain's pointers are at; with_cp: not the direction's first step, which has no step before it
+        constexpr int c = decltype(ch)::value;
+#pragma unroll
+        for (int q = 0; q < PAIRS; ++q) {
+#pragma unroll
+            for (int gate = 0; gate < 4; ++gate) e_act[q][gate] = p_acts[c][q][gate * C];
+            e_ca[q] = *p_ca[c][q];
+            e_dh[q] = *p_dh_in[c][q];
+            e_cp[q] = with_cp ? *p_cp[c][q] : 0.f;
+        }
+    };
+    auto load_tiles = [&](auto ch) {   // dG of the chain's step processed before the one its pointers are at
+        constexpr int c = decltype(ch)::value;
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+#pragma unroll
+            for (int q = 0; q < LPT; ++q)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p_tile[c][q] + i * 32),
+                                                 (__attribute__((address_space(3))) void *)(stage + i * ROWS * 32 + q * 256), 16, 0, kAux);
+#pragma unroll
+        for (int q = 0; q < LPT; ++q) p_tile[c][q] += step_g;
+    };
+    auto mfma_tiles = [&](auto first, auto last) {
+#pragma unroll
+        for (int i = decltype(first)::value; i < decltype(last)::value; ++i) {
+            const float *tile = stage + i * ROWS * 32;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                f32x4 fa[RS];
+#pragma unroll
+                for (int rs = 0; rs < RS; ++rs) fa[rs] = ATile<ROWS, kAux>::chunk(tile, rs * 16 + col16, h * 4 + quad);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int rs = 0; rs < RS; ++rs)
+                        acc[rs][e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[rs][e], breg[i][h][e], acc[rs][e & 1], 0, 0, 0);
+            }
+        }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using IA = std::integral_constant<int, A1>;
+    using IP = std::integral_constant<int, P1>;
+    using IN = std::integral_constant<int, NT>;
+
+    auto head = [&](auto ch, auto all_landed) {
+        constexpr int c = decltype(ch)::value;
+#pragma unroll
+        for (int rs = 0; rs < RS; ++rs) { acc[rs][0] = f32x4{0.f, 0.f, 0.f, 0.f}; acc[rs][1] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+        if (decltype(all_landed)::value) wait_vm<0>(); else wait_vm<NSTORE>();
+        mfma_tiles(I0{}, IA{});
+        __builtin_amdgcn_sched_barrier(0);   // keeps the MFMAs above in front of the wait
+        wait_vm<0>();
+        wave_arrive<false>(counters + (1 - c) * kSyncStride, &s_arrive[1 - c]);
+    };
+    // FIRST: the pass's first step of the chain (no recurrent term, nothing from a later step); s: the direction's step
+    auto tail = [&](auto ch, auto first_tag, int s, unsigned wait_for) -> bool {
+        constexpr int c = decltype(ch)::value;
+        constexpr bool FIRST = decltype(first_tag)::value;
+        load_operands(ch, s > 0);
+        if (!FIRST) {
+            mfma_tiles(IA{}, IP{});
+            if (wait_for) seen = __hip_atomic_load(counters + (1 - c) * kSyncStride, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+            mfma_tiles(IP{}, IN{});
+            __builtin_amdgcn_sched_barrier(0);   // the counter's value is looked at after the MFMAs, not right behind its load
+        }
+        if (wait_for) {
+            const unsigned target = wait_for * members;
+            const bool there = !FIRST && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0;
+            if (!there && !wave_wait(w, counters + (1 - c) * kSyncStride, target, g.spin_polls)) return false;
+            load_tiles(std::integral_constant<int, 1 - c>{});
+        }
+        float *part = parts + c * kPart;
+        if (!FIRST) {
+            float *to = part + wave * ROWS * kStride;
+#pragma unroll
+            for (int rs = 0; rs < RS; ++rs)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) to[(rs * 16 + quad * 4 + r) * kStride + col16] = acc[rs][0][r] + acc[rs][1][r];
+            lds_barrier();
+        }
+#pragma unroll
+        for (int q = 0; q < PAIRS; ++q) {
+            const int pair = threadIdx.x + q * kThreads, row = pair >> 4, cell = pair & 15;
+            float rec = 0.f;
+            if (!FIRST) {
+#pragma unroll
+                for (int wv = 0; wv < 4; ++wv) rec += part[(wv * ROWS + row) * kStride + cell];
+            }
+            const float dh = e_dh[q] + rec;
+            const float z = e_act[q][0], gi = e_act[q][1], gf = e_act[q][2], go = e_act[q][3];
+            const float a = e_ca[q];
+            const float ddo = go * (1.f - go) * (dh * a);
+            float e = dh * go * (1.f - a * a);
+            e += e_peep[q][2] * ddo;
+            if (!FIRST) {
+                e += e_peep[q][0] * n_di[c][q];
+                e += e_peep[q][1] * n_df[c][q];
+                e += n_dc[c][q] * n_f[c][q];
+            }
+            const float dz = e * gi * (1.f - z * z);
+            const float di = (e * z) * (gi * (1.f - gi));
+            const float df = s > 0 ? (e * e_cp[q]) * (gf * (1.f - gf)) : 0.f;
+            n_di[c][q] = di; n_df[c][q] = df; n_f[c][q] = gf; n_dc[c][q] = e;
+            float *drow = p_dG[c][q];
+            drow[0] = dz; drow[C] = di; drow[2 * C] = df; drow[3 * C] = ddo;
+            *p_dh[c][q] = dh; *p_dc[c][q] = e;
+            p_acts[c][q] += step_g; p_ca[c][q] += step_c; p_cp[c][q] += step_c; p_dh_in[c][q] += step_c;
+            p_dG[c][q] += lane_step_g[c][q]; p_dh[c][q] += lane_step_c[c][q]; p_dc[c][q] += lane_step_c[c][q];
+        }
+        return true;
+    };
+    using First = std::true_type;
+    using Later = std::false_type;
+
+    // units in program order: (0,0) (1,0) (0,1) (1,1) ... (chain, step j of this pass); the direction's step is T - 1 - j
+    if (!tail(Chain0{}, First{}, T - 1, 0u)) return;
+    wait_vm<0>();
+    wave_arrive<false>(counters, &s_arrive[0]);
+    if (!tail(Chain1{}, First{}, T - 1, 1u)) return;
+    head(Chain0{}, std::true_type{});
+    for (int j = 1; j + 1 < T; ++j) {
+        if (!tail(Chain0{}, Later{}, T - 1 - j, (unsigned)j)) return;
+        head(Chain1{}, std::false_type{});
+        if (!tail(Chain1{}, Later{}, T - 1 - j, (unsigned)j + 1u)) return;
+        head(Chain0{}, std::false_type{});
+    }
+    if (!tail(Chain0{}, Later{}, 0, (unsigned)(T - 1))) return;
+    head(Chain1{}, std::false_type{});
+    if (!tail(Chain1{}, Later{}, 0, 0u)) return;
+}
+
+__global__ void resident_probe_kernel(unsigned *table)
+{
+    if (threadIdx.x == 0) table[blockIdx.x] = xcc_id();
+}
+
+__global__ void resident_clear_kernel(unsigned *words, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) words[i] = 0u;
+}
+
+// ---- host: what the device offers ---------------------------------------------------------------------------------------
+struct ResidentDevice {
+    bool probed = false;
+    bool usable = false;           // 8 XCDs, workgroup ids equal mod 8 share one
+    int cus = 0;
+};
+std::mutex g_resident_mutex;
+ResidentDevice g_resident_device[64];
+
+constexpr size_t kMaxLds = 160 * 1024;   // LDS of a compute unit
+
+// One probe launch per device and process: a grid of one workgroup per compute unit (made so by its LDS size) records the
+// XCC id every workgroup ran on.  LOCAL groups are only used when the ids of one residue class mod 8 all ran on one XCD and
+// the eight classes on eight different ones (which class lands on which XCD varies with the hardware queue).
+int probe_device(ResidentDevice **out)
+{
+    int dev = -1;
+    MYEA_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) { set_last_error("resident LSTM: device ordinal %d out of range", dev); return MYEA_E_DEVICE; }
+    std::lock_guard<std::mutex> lock(g_resident_mutex);
+    ResidentDevice &r = g_resident_device[dev];
+    *out = &r;
+    if (r.probed) return MYEA_OK;
+    hipDeviceProp_t prop;
+    MYEA_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    r.cus = prop.multiProcessorCount;
+    r.probed = true;
+    if (r.cus < 8 || r.cus % 8 != 0 || r.cus > 1024 || prop.sharedMemPerBlock < kMaxLds) return MYEA_OK;
+    unsigned *table = nullptr;
+    MYEA_HIP_TRY(hipMalloc(&table, (size_t)r.cus * sizeof(unsigned)));
+    std::vector<unsigned> host((size_t)r.cus);
+    const size_t lds = 96 * 1024;   // more than half of a compute unit's LDS: one workgroup per compute unit
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(resident_probe_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(resident_probe_kernel, dim3((unsigned)r.cus), dim3(64), lds, 0, table);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpy(host.data(), table, host.size() * sizeof(unsigned), hipMemcpyDeviceToHost);
+    (void)hipFree(table);
+    if (e != hipSuccess) return hip_fail(e, "resident LSTM probe");
+    bool ok = true;
+    for (int i = 0; i < r.cus && ok; ++i) ok = host[i] == host[i & 7] && host[i] < 16;
+    for (int a = 0; a < 8 && ok; ++a)
+        for (int b = a + 1; b < 8 && ok; ++b) ok = host[a] != host[b];
+    r.usable = ok;
+    return MYEA_OK;
+}
+
+// MYEA_LSTM_RESIDENT=0 keeps every layer on one launch per time step
+bool resident_disabled()
+{
+    const char *e = std::getenv("MYEA_LSTM_RESIDENT");
+    return e && e[0] == '0';
+}
+
+// A wait gives up after this many polls of its counter (a poll is a load served by L2 or memory plus a short sleep: about a
+// microsecond); MYEA_LSTM_RESIDENT_SPIN_POLLS overrides the default of 200 000 (a fifth of a second).
+unsigned spin_polls()
+{
+    const char *e = std::getenv("MYEA_LSTM_RESIDENT_SPIN_POLLS");
+    if (e && *e) { const unsigned long long v = std::strtoull(e, nullptr, 10); return v < 1 ? 1u : (v > 0x7fffffffull ? 0x7fffffffu : (unsigned)v); }
+    return 200000u;
+}
+
+// ---- host: the kernels on offer ------------------------------------------------------------------------------------------
+using ResidentKernel = void (*)(ResidentGeometry, LstmResidentDir, LstmResidentDir, SyncWords);
+struct KernelInfo {
+    ResidentKernel fn = nullptr;
+    size_t lds = 0;
+    int cells = 0;
+    bool ready = false;
+    hipError_t status = hipSuccess;
+    int per_cu = 0;   // workgroups of this kernel a compute unit can hold
+};
+
+template <int KW, int CELLS, int RS, bool AGENT>
+KernelInfo forward_info()
+{
+    KernelInfo k;
+    k.fn = lstm_resident_forward_kernel<KW, CELLS, RS, AGENT>;
+    k.lds = forward_lds(KW, CELLS, RS);
+    k.cells = CELLS;
+    return k;
+}
+template <int C, int RS>
+KernelInfo backward_info()
+{
+    KernelInfo k;
+    k.fn = lstm_resident_backward_kernel<C, RS>;
+    k.lds = backward_lds(C, RS);
+    k.cells = 16;
+    return k;
+}
+
+// [backward][C: 128, 256, 512, 1024][rs - 1]; an entry without a kernel has fn == nullptr
+KernelInfo g_kernels[2][4][2] = {
+    {{forward_info<32, 16, 1, false>(), forward_info<32, 16, 2, false>()},
+     {forward_info<64, 16, 1, false>(), forward_info<64, 16, 2, false>()},
+     {forward_info<128, 16, 1, false>(), forward_info<128, 16, 2, false>()},
+     {forward_info<256, 16, 1, true>(), KernelInfo{}}},
+    {{backward_info<128, 1>(), backward_info<128, 2>()},
+     {backward_info<256, 1>(), backward_info<256, 2>()},
+     {backward_info<512, 1>(), KernelInfo{}},
+     {KernelInfo{}, KernelInfo{}}},
+};
+
+// the kernel for (C, rs) with its LDS attribute set and its occupancy known, or nullptr
+KernelInfo *kernel_for(size_t C, int rs, bool backward)
+{
+    const int ci = C == 128 ? 0 : C == 256 ? 1 : C == 512 ? 2 : C == 1024 ? 3 : -1;
+    if (ci < 0 || rs < 1 || rs > 2) return nullptr;
+    KernelInfo &k = g_kernels[backward ? 1 : 0][ci][rs - 1];
+    if (!k.fn) return nullptr;
+    std::lock_guard<std::mutex> lock(g_resident_mutex);
+    if (!k.ready) {
+        k.status = hipFuncSetAttribute(reinterpret_cast<const void *>(k.fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)k.lds);
+        if (k.status == hipSuccess) k.status = hipOccupancyMaxActiveBlocksPerMultiprocessor(&k.per_cu, reinterpret_cast<const void *>(k.fn), kThreads, k.lds);
+        k.ready = true;
+    }
+    return k.status == hipSuccess && k.per_cu >= 1 ? &k : nullptr;
+}
+
+// Groups of ROWS examples onto the device: LOCAL - an XCD hosts whole groups, as many as its compute units hold members;
+// AGENT - the members of a group are spread over the device.  Every workgroup must be resident at once, or a wait between
+// time steps could never end.
+bool place_groups(const ResidentDevice &dev, const KernelInfo &k, int members, bool agent, int groups, int *grid)
+{
+    if (groups > kMaxGroups) return false;
+    if (agent) { *grid = groups * members; return *grid <= dev.cus * k.per_cu; }
+    const int per_xcd = (dev.cus / 8) * k.per_cu / members;   // groups one XCD can host
+    const int slots = (groups + 7) / 8;                        // groups on the fullest XCD
+    *grid = 8 * slots * members;
+    return slots <= per_xcd;
+}
+
+int fill_geometry(const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs, ResidentGeometry *g)
+{
+    if (!plan.ok) { set_last_error("resident LSTM: no plan for this layer"); return MYEA_E_INVALID; }
+    if (T < 2 || T > 0x7fffffffu / (unsigned)(plan.members ? plan.members : 1)) { set_last_error("resident LSTM: %zu time steps do not fit the barrier counters", T); return MYEA_E_INVALID; }
+    g->T = (int)T; g->B = (int)B; g->Bmax = (int)Bmax; g->C = (int)C;
+    g->dirs = dirs; g->row_groups = plan.row_groups; g->members = plan.members;
+    g->spin_polls = spin_polls();
+    return MYEA_OK;
+}
+
+// clears the counters and flags and lays the words out
+int prepare_sync(hipStream_t s, const LstmResidentPlan &plan, int dirs, unsigned *sync, unsigned *host_flag, SyncWords *w)
+{
+    const int groups = plan.row_groups * dirs;
+    if (groups > kMaxGroups) { set_last_error("resident LSTM: %d groups exceed the counter block", groups); return MYEA_E_INVALID; }
+    const int words = groups * 2 * kSyncStride + 1 + groups;
+    hipLaunchKernelGGL(resident_clear_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, sync, words);
+    MYEA_HIP_TRY(hipGetLastError());
+    w->counters = sync;
+    w->give_up = sync + (size_t)groups * 2 * kSyncStride;
+    w->host_flag = host_flag;
+    w->scrap = reinterpret_cast<float *>(sync + (size_t)kMaxGroups * 2 * kSyncStride + 1 + kMaxGroups);
+    return MYEA_OK;
+}
+
+int check_dirs(const LstmResidentDir *dir, int dirs, bool backward)
+{
+    for (int k = 0; k < dirs; ++k) {
+        const LstmResidentDir &d = dir[k];
+        const bool fwd_ok = d.Wrec && d.bias && d.peep && d.acts && d.c && d.ca && d.h && !(reinterpret_cast<uintptr_t>(d.Wrec) & 15u) && !(reinterpret_cast<uintptr_t>(d.h) & 15u);
+        const bool bwd_ok = d.WrecT && d.peep && d.acts && d.c && d.ca && d.dh && d.dG && d.dc && !(reinterpret_cast<uintptr_t>(d.WrecT) & 15u) && !(reinterpret_cast<uintptr_t>(d.dG) & 15u);
+        if (backward ? !bwd_ok : !fwd_ok) { set_last_error("resident LSTM: null or unaligned operand"); return MYEA_E_INVALID; }
+    }
+    return MYEA_OK;
+}
+
+int launch_resident(hipStream_t s, bool backward, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
+                    const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag)
+{
+    ResidentGeometry g;
+    SyncWords w;
+    int rc = fill_geometry(plan, T, B, Bmax, C, dirs, &g);
+    if (rc == MYEA_OK && backward && !plan.backward) { set_last_error("resident LSTM backward: no plan for this layer"); rc = MYEA_E_INVALID; }
+    if (rc == MYEA_OK) rc = check_dirs(dir, dirs, backward);
+    if (rc != MYEA_OK) return rc;
+    KernelInfo *k = kernel_for(C, plan.rs, backward);
+    ResidentDevice *dev = nullptr;
+    rc = probe_device(&dev);
+    if (rc != MYEA_OK) return rc;
+    int grid = 0;
+    if (!k || !dev->usable || !place_groups(*dev, *k, plan.members, plan.agent, plan.row_groups * dirs, &grid) || grid != plan.grid) {
+        set_last_error("resident LSTM: the plan does not fit the device (C = %zu, %d groups)", C, plan.row_groups * dirs);
+        return MYEA_E_UNSUPPORTED;
+    }
+    rc = prepare_sync(s, plan, dirs, sync, host_flag, &w);
+    if (rc != MYEA_OK) return rc;
+    hipLaunchKernelGGL(k->fn, dim3((unsigned)plan.grid), dim3(kThreads), k->lds, s, g, dir[0], dir[dirs > 1 ? 1 : 0], w);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+}  // namespace
+
+// How a layer of C cells (one per block) and B examples per direction maps onto the device, or plan.ok == false when the
+// resident form does not apply (other widths, more examples than the device can hold groups for, probe failed).
+// plan.backward: the backward loop has a resident form too (C <= 512).
+int lstm_resident_plan(size_t C, size_t cells_per_block, size_t B, int dirs, LstmResidentPlan *plan)
+{
+    *plan = LstmResidentPlan{};
+    if (resident_disabled() || cells_per_block != 1 || B == 0 || dirs < 1 || dirs > 2) return MYEA_OK;
+    ResidentDevice *dev = nullptr;
+    {
+        const int rc = probe_device(&dev);
+        if (rc != MYEA_OK) return rc;
+    }
+    if (!dev->usable) return MYEA_OK;
+    // groups of two chains of 16 examples, or of 32 when there are more examples than the device holds such groups for
+    for (int rs = 1; rs <= 2; ++rs) {
+        KernelInfo *fwd = kernel_for(C, rs, false);
+        if (!fwd) continue;
+        KernelInfo *bwd = kernel_for(C, rs, true);
+        const int members = (int)C / fwd->cells;
+        const bool agent = members > dev->cus / 8;
+        const int rows = 2 * 16 * rs, row_groups = (int)((B + rows - 1) / rows), groups = row_groups * dirs;
+        int grid = 0, grid_b = 0;
+        if (!place_groups(*dev, *fwd, members, agent, groups, &grid)) continue;
+        const bool backward = bwd && !agent && place_groups(*dev, *bwd, members, false, groups, &grid_b) && grid_b == grid;
+        plan->ok = true; plan->agent = agent; plan->backward = backward;
+        plan->cells = fwd->cells; plan->members = members; plan->rs = rs; plan->row_groups = row_groups; plan->grid = grid; plan->cus = dev->cus;
+        break;
+    }
+    return MYEA_OK;
+}
+
+// counters (one per group and chain, 128 bytes apart), the give-up flag, one XCC word per group, the scrap area
+size_t lstm_resident_sync_words() { return (size_t)kMaxGroups * 2 * kSyncStride + 1 + kMaxGroups + kScrapWords; }
+
+// sync: lstm_resident_sync_words() unsigneds of device memory (cleared by the call); host_flag: one pinned host word (0 = fine)
+int launch_lstm_resident_forward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
+                                 const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag)
+{
+    return launch_resident(s, false, plan, T, B, Bmax, C, dirs, dir, sync, host_flag);
+}
+
+int launch_lstm_resident_backward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
+                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag)
+{
+    return launch_resident(s, true, plan, T, B, Bmax, C, dirs, dir, sync, host_flag);
+}
+
+}  // namespace myea

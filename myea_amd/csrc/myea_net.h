@@ -87,6 +87,11 @@ struct Net {
     size_t scratch_floats = 0, dw_slab_floats = 0;   // sizes of the two buffers above
     float *static_scratch = nullptr;   // this device's copy of the library's static scratch array (update_derivative_weight_no_alloc)
     double *loss_acc = nullptr;                  // 8 doubles, see ErrorParams::loss_acc
+    // LSTM time loops as one resident launch (myea_lstm_resident.hip): barrier counters in device memory, and a pinned host
+    // word a kernel sets when one of its bounded waits gave up; resident_off: this network stays on one launch per time step
+    unsigned *resident_sync = nullptr, *resident_flag = nullptr;
+    bool resident_off = false;
+    int resident_check();   // MYEA_E_DEVICE (once) after a resident launch reported a give-up
     unsigned long long *index_stage = nullptr;   // [Bmax] example indices of a gathered batch
 
     bool profiling = false, open_event = false;
@@ -149,6 +154,7 @@ struct Net {
     int side_stream_join();            // `stream` waits for what the last SideStreamScope enqueued
     int lstm_forward_inputs(size_t li, LstmLayer &q, size_t B);
     int lstm_forward_step(LstmLayer &q, size_t B, size_t s);
+    int lstm_resident_dirs(DevLayer &o, LstmResidentDir *dirs);   // the layer's directions as the resident kernels take them
     int lstm_backward_step(LstmLayer &q, size_t B, size_t s);
     int lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t B);
     size_t lstm_scratch_floats() const;

@@ -334,6 +334,18 @@ int Net::create(const myea_net_desc &desc)
         }
     }
     MYEA_TRY(side_stream_create());
+    {
+        bool any_lstm = false;
+        for (size_t li = 1; li < d.n_layers; ++li) any_lstm = any_lstm || d.layers[li].type_layer == MYEA_LAYER_LSTM;
+        if (any_lstm) {   // counters and flags of the resident time loops
+            void *q = nullptr;
+            MYEA_HIP_TRY(hipMalloc(&q, lstm_resident_sync_words() * sizeof(unsigned)));
+            resident_sync = static_cast<unsigned *>(q);
+            MYEA_HIP_TRY(hipHostMalloc(&q, 64, hipHostMallocDefault));
+            resident_flag = static_cast<unsigned *>(q);
+            *resident_flag = 0u;
+        }
+    }
     MYEA_TRY(dev_alloc(&tmp1, T * B * max_h));
     MYEA_TRY(dev_alloc(&tmp2, T * B * max_h));
     {
@@ -385,6 +397,8 @@ Net::~Net()
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
+    fr(resident_sync);
+    if (resident_flag) (void)hipHostFree(resident_flag);
     fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc); fr(index_stage); fr(dw_slabs);
     for (ProfEvent &e : pending) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
     for (ProfEvent &e : free_events) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
@@ -525,10 +539,24 @@ int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool train
     return launch_bn_forward_training(stream, p, scratch);
 }
 
+// A resident LSTM launch whose bounded wait gave up has left the pass it belonged to incomplete.  Reported once, at the
+// next call that looks; the network then keeps to one launch per time step.
+int Net::resident_check()
+{
+    if (!resident_flag || *resident_flag == 0u) return MYEA_OK;
+    const unsigned code = *resident_flag;
+    *resident_flag = 0u;
+    resident_off = true;
+    set_last_error(code == 2u ? "resident LSTM time loop: the workgroups of a group did not share an XCD; the pass is incomplete, later passes use one launch per time step"
+                              : "resident LSTM time loop: a wait between time steps gave up (workgroups not resident together?); the pass is incomplete, later passes use one launch per time step");
+    return MYEA_E_DEVICE;
+}
+
 // FF__Forward_Pass_Batch (NN/Neural_Network__Forward_Pass__OpenMP.cpp:24-120) / RNN__Forward_Pass_Batch
 // (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:24-130): assign inputs, then layer by layer.
 int Net::forward_pass(size_t B, const float *inputs, int on_device)
 {
+    MYEA_TRY(resident_check());
     if (!inputs) { set_last_error("Forward_Pass: null inputs"); return MYEA_E_INVALID; }
     if (B == 0 || B > d.batch_size) { set_last_error("Forward_Pass: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
     const size_t T = d.number_recurrent_depth, In = L[0].H, Bmax = d.batch_size;
@@ -1347,7 +1375,7 @@ int myea_hip_destroy(myea_hip_net *n)
 }
 
 int myea_hip_set_stream(myea_hip_net *n, void *s) { NET_OR_FAIL(n); n->net.stream = static_cast<hipStream_t>(s); return MYEA_OK; }
-int myea_hip_synchronize(myea_hip_net *n) { NET_OR_FAIL(n); MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream)); return MYEA_OK; }
+int myea_hip_synchronize(myea_hip_net *n) { NET_OR_FAIL(n); MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream)); return n->net.resident_check(); }
 
 int myea_hip_set_hyper(myea_hip_net *n, const myea_hyper *h)
 {
@@ -1380,7 +1408,7 @@ static int copy_vec(myea_hip_net *n, float *dev, float *host_out, const float *h
     if (host_in) MYEA_HIP_TRY(hipMemcpyAsync(dev, host_in, count * sizeof(float), hipMemcpyHostToDevice, n->net.stream));
     else MYEA_HIP_TRY(hipMemcpyAsync(host_out, dev, count * sizeof(float), hipMemcpyDeviceToHost, n->net.stream));
     MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
-    return MYEA_OK;
+    return n->net.resident_check();
 }
 
 int myea_hip_upload_parameters(myea_hip_net *n, const float *p, size_t c)
@@ -1508,6 +1536,10 @@ int myea_hip_get_loss(myea_hip_net *n, myea_loss_state *s)
     double v[8];
     MYEA_HIP_TRY(hipMemcpyAsync(v, n->net.loss_acc, sizeof(v), hipMemcpyDeviceToHost, n->net.stream));
     MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
+    {
+        const int rc = n->net.resident_check();
+        if (rc != MYEA_OK) return rc;
+    }
     s->loss_values = v[0]; s->number_loss = (uint64_t)v[1]; s->accuracy_value = v[2]; s->number_bit_fail = (uint64_t)v[3];
     for (int k = 0; k < 4; ++k) s->accuracy_r[k] = v[4 + k];
     return MYEA_OK;
@@ -1555,7 +1587,7 @@ int myea_hip_download_tensor(myea_hip_net *n, size_t li, int kind, float *host, 
     if (count > c) { myea::set_last_error("download_tensor: count %zu > tensor length %zu", count, c); return MYEA_E_INVALID; }
     MYEA_HIP_TRY(hipMemcpyAsync(host, p, count * sizeof(float), hipMemcpyDeviceToHost, n->net.stream));
     MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
-    return MYEA_OK;
+    return n->net.resident_check();
 }
 
 int myea_hip_upload_tensor(myea_hip_net *n, size_t li, int kind, const float *host, size_t count)
