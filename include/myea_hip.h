@@ -445,7 +445,9 @@ int myea_hip_upload_tensor(myea_hip_net *net, size_t layer_index, int kind, cons
 /* When enabled, every dense-contraction (GEMM) launch is bracketed by HIP events on the net's stream;
  * myea_hip_profile_read() synchronises and returns accumulated launches / milliseconds / FLOPs per
  * family since the last reset.  family: 0 = forward (NT), 1 = dX (NN), 2 = dW (TN), 3 = optimizer
- * update (bytes instead of FLOPs). */
+ * update (bytes instead of FLOPs), 4 = a layer's dX and dW contractions in one launch, 5 = the recurrent
+ * contractions and gate math of an LSTM layer's forward time loop (steps 1 .. T-1; one launch per layer when the
+ * loop runs as a resident kernel, one per step otherwise), 6 = the same of its backward time loop. */
 int myea_hip_profile_enable(myea_hip_net *net, int enable);
 int myea_hip_profile_read(myea_hip_net *net, int family, uint64_t *launches, double *milliseconds, double *work);
 

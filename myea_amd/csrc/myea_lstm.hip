@@ -596,7 +596,7 @@ int Net::lstm_forward_layer(size_t li, size_t B)
             if (o.lstm2) MYEA_TRY(lstm_forward_inputs(li, *o.lstm2, B));
             LstmResidentDir rd[2];
             lstm_resident_dirs(o, rd);
-            prof_begin(0);
+            prof_begin(kProfLstmForwardLoop);
             MYEA_TRY(launch_lstm_resident_forward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag));
             prof_end(dirs * loop_work, 1);
             if (!o.lstm2) return MYEA_OK;
@@ -606,7 +606,7 @@ int Net::lstm_forward_layer(size_t li, size_t B)
     }
     if (!o.lstm2) {
         MYEA_TRY(lstm_forward_inputs(li, *o.lstm, B));
-        if (T > 1) prof_begin(0);
+        if (T > 1) prof_begin(kProfLstmForwardLoop);
         for (size_t s = 0; s < T; ++s) MYEA_TRY(lstm_forward_step(*o.lstm, B, s));
         if (T > 1) prof_end(loop_work, T - 1);
         return MYEA_OK;
@@ -616,7 +616,7 @@ int Net::lstm_forward_layer(size_t li, size_t B)
         MYEA_TRY(lstm_forward_inputs(li, *o.lstm2, B));
         if (side.active) std::swap(stream, side_stream);   // back on the caller's stream while the scope stays open
         int rc = lstm_forward_inputs(li, *o.lstm, B);
-        if (T > 1) prof_begin(0);
+        if (T > 1) prof_begin(kProfLstmForwardLoop);
         for (size_t s = 0; s < T && rc == MYEA_OK; ++s) {
             if (side.active) std::swap(stream, side_stream);
             rc = lstm_forward_step(*o.lstm2, B, s);
@@ -690,7 +690,7 @@ int Net::lstm_backward_layer(size_t li, size_t B)
             if (o.lstm2) MYEA_TRY(seed(*o.lstm2));
             LstmResidentDir rd[2];
             lstm_resident_dirs(o, rd);
-            prof_begin(1);
+            prof_begin(kProfLstmBackwardLoop);
             MYEA_TRY(launch_lstm_resident_backward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag));
             prof_end(dirs * loop_work, 1);
             return MYEA_OK;
@@ -698,7 +698,7 @@ int Net::lstm_backward_layer(size_t li, size_t B)
     }
     if (!o.lstm2) {
         MYEA_TRY(seed(*o.lstm));
-        if (T > 1) prof_begin(1);
+        if (T > 1) prof_begin(kProfLstmBackwardLoop);
         for (size_t s = T; s-- > 0;) MYEA_TRY(lstm_backward_step(*o.lstm, B, s));
         if (T > 1) prof_end(loop_work, T - 1);
         return MYEA_OK;
@@ -708,7 +708,7 @@ int Net::lstm_backward_layer(size_t li, size_t B)
         MYEA_TRY(seed(*o.lstm2));
         if (side.active) std::swap(stream, side_stream);
         int rc = seed(*o.lstm);
-        if (T > 1) prof_begin(1);
+        if (T > 1) prof_begin(kProfLstmBackwardLoop);
         for (size_t s = T; s-- > 0 && rc == MYEA_OK;) {
             if (side.active) std::swap(stream, side_stream);
             rc = lstm_backward_step(*o.lstm2, B, s);

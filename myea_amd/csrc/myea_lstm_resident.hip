@@ -216,6 +216,7 @@ struct ResidentGeometry {
     int T, B, Bmax, C;
     int dirs, row_groups;      // groups = dirs * row_groups; group g: direction g % dirs, examples from (g / dirs) * 2 ROWS
     int members;               // workgroups per group = C / CELLS
+    int arrivals;              // arrivals that complete a unit: members (one more under the test switch, so that no unit ever completes)
     unsigned spin_polls;       // polls after which a wait gives up
 };
 
@@ -253,7 +254,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
     const int c0 = member * CELLS, B = g.B, T = g.T;
     const size_t Bmax = (size_t)g.Bmax;
     unsigned *const counters = w.counters + (size_t)group * 2 * kSyncStride;   // chain c: counters + c * kSyncStride
-    const unsigned members = (unsigned)g.members;
+    const unsigned members = (unsigned)g.arrivals;
     if (!AGENT) check_same_xcd(w, group);
     if (threadIdx.x < 2) s_arrive[threadIdx.x] = 0u;
     __syncthreads();
@@ -522,7 +523,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
     const int c0 = member * CELLS, B = g.B, T = g.T;
     const size_t Bmax = (size_t)g.Bmax;
     unsigned *const counters = w.counters + (size_t)group * 2 * kSyncStride;
-    const unsigned members = (unsigned)g.members;
+    const unsigned members = (unsigned)g.arrivals;
     check_same_xcd(w, group);
     if (threadIdx.x < 2) s_arrive[threadIdx.x] = 0u;
     __syncthreads();
@@ -791,6 +792,15 @@ unsigned spin_polls()
     return 200000u;
 }
 
+// MYEA_LSTM_RESIDENT_TEST_ABSENT_MEMBER=1 makes every group expect one member more than it has: its first wait runs out of
+// polls, the kernel ends through its give-up path and the host reports it.  For tests of that path; every wavefront still
+// exits normally.
+bool absent_member_for_test()
+{
+    const char *e = std::getenv("MYEA_LSTM_RESIDENT_TEST_ABSENT_MEMBER");
+    return e && e[0] == '1';
+}
+
 // ---- host: the kernels on offer ------------------------------------------------------------------------------------------
 using ResidentKernel = void (*)(ResidentGeometry, LstmResidentDir, LstmResidentDir, SyncWords);
 struct KernelInfo {
@@ -865,9 +875,10 @@ bool place_groups(const ResidentDevice &dev, const KernelInfo &k, int members, b
 int fill_geometry(const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs, ResidentGeometry *g)
 {
     if (!plan.ok) { set_last_error("resident LSTM: no plan for this layer"); return MYEA_E_INVALID; }
-    if (T < 2 || T > 0x7fffffffu / (unsigned)(plan.members ? plan.members : 1)) { set_last_error("resident LSTM: %zu time steps do not fit the barrier counters", T); return MYEA_E_INVALID; }
+    if (T < 2 || T > 0x7fffffffu / (unsigned)(plan.members + 1)) { set_last_error("resident LSTM: %zu time steps do not fit the barrier counters", T); return MYEA_E_INVALID; }
     g->T = (int)T; g->B = (int)B; g->Bmax = (int)Bmax; g->C = (int)C;
     g->dirs = dirs; g->row_groups = plan.row_groups; g->members = plan.members;
+    g->arrivals = plan.members + (absent_member_for_test() ? 1 : 0);
     g->spin_polls = spin_polls();
     return MYEA_OK;
 }

@@ -44,7 +44,8 @@ struct DevLayer {
     LstmLayer *lstm = nullptr, *lstm2 = nullptr;  // lstm2: the time-reversed direction of a bidirectional layer
 };
 
-constexpr int kProfFamilies = 5;   // forward, dX, dW, update, dX + dW launched as a pair
+constexpr int kProfFamilies = 7;   // forward, dX, dW, update, dX + dW launched as a pair, LSTM time loop forward, backward
+constexpr int kProfLstmForwardLoop = 5, kProfLstmBackwardLoop = 6;
 struct ProfEvent {
     hipEvent_t start = nullptr, stop = nullptr;
     int family = 0;
