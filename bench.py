@@ -20,10 +20,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# HBM bytes per contraction launch (mean over the launches of one step) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of this script, scaled by what the same counters read for copies of known size (FETCH_SIZE x2, WRITE_SIZE x1);
-# the per-kernel figures are in profiles/hbm_traffic__*__pmc.txt.  None where no counter run has been made.
-PMC_TRAFFIC_BYTES_PER_GEMM_LAUNCH = {"fc4096x4_b1024_adam": 2886299 * 1024 / 10}
+# HBM bytes per contraction launch (mean over the launches of one step): NOT measured by this script's run.  Recorded
+# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same counters read for copies of
+# known size (FETCH_SIZE x2, WRITE_SIZE x1); the line names the file the figure comes from.
+RECORDED_TRAFFIC = {"fc4096x4_b1024_adam": dict(bytes_per_launch=2886299 * 1024 / 10,
+                                                source="recorded constant, not measured in this run: profiles/hbm_traffic__fc4096x4_b1024_adam__pmc.txt")}
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
@@ -112,7 +113,7 @@ def cpu_baseline(wl, sample_rows, threads):
     full parameter vector; samples/s = batch / (t_sample * batch / sample_rows + t_update)."""
     import numpy as np
     from myea_amd import binding as mb
-    from tests.common import glorot_parameters
+    from myea_amd.synthetic import glorot_parameters
     from tests.oracle_lib import OracleNetwork, load_oracle
     lib = load_oracle()
     desc = mb.make_desc(wl["layers"], sample_rows, wl.get("depth", 1), lib=lib)
@@ -144,26 +145,22 @@ def cpu_baseline(wl, sample_rows, threads):
                        % (sample_rows, wl["batch"], t_sample, reps, t_update))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="fc4096x4_b1024_adam", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-rows", type=int, default=0, help="examples in the CPU sample (default: sized for ~20 s)")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); no multi-GPU path exists")
+# profile families of the library (myea_hip_profile_read): name, what its `work` counts
+FAMILIES = (("forward", "flop"), ("dx", "flop"), ("dw", "flop"), ("update", "byte"), ("dx_dw_pair", "flop"),
+            ("lstm_forward_loop", "flop"), ("lstm_backward_loop", "flop"),
+            ("normalization", "byte"), ("bias_gradient", "byte"))
+KERNEL_NAMES = {"forward": "gemm_forward", "dx": "gemm_dx", "dw": "gemm_dw", "dx_dw_pair": "gemm_dx_dw_pair", "update": "optimizer_update"}
 
+
+def run_workload(name, steps, warmup):
+    """Times `steps` training steps of one workload on cuda:0 (inputs resident in HBM), with the library's per-family
+    HIP-event timers on.  Returns the measurements as a dict."""
     import numpy as np
     import torch
     from myea_amd import binding as mb
-    from tests.common import glorot_parameters
+    from myea_amd.synthetic import glorot_parameters
 
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible")
-    wl = WORKLOADS[args.workload]
+    wl = WORKLOADS[name]
     B = wl["batch"]
     desc = mb.make_desc(wl["layers"], B, wl.get("depth", 1))
     h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER[wl["optimizer"]], type_loss_function=mb.LOSS[wl["loss"]], **wl["hyper"])
@@ -183,57 +180,126 @@ def main():
         net.Backward_Pass__Update_Derivative_Weight(B)     # the two calls of Train_Batch_BP as one entry point
         net.Update_Parameter(B, B)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     net.profile_enable(True)
-    for f in range(4):
+    for f in range(len(FAMILIES)):
         net.profile_read(f)            # drop anything recorded so far
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    fam = {name: net.profile_read(i) for i, name in enumerate(("forward", "dx", "dw", "update", "dx_dw_pair"))}
-    GEMM_FAMILIES = ("forward", "dx", "dw", "dx_dw_pair")   # dx_dw_pair: a layer's dX and dW contractions in one launch
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    fam = {fname: net.profile_read(i) for i, (fname, _) in enumerate(FAMILIES)}
     net.profile_enable(False)
     loss = net.get_loss()
+    net.close()
 
-    g_launch = sum(fam[k][0] for k in GEMM_FAMILIES)
-    g_ms = sum(fam[k][1] for k in GEMM_FAMILIES)
-    g_flop = sum(fam[k][2] for k in GEMM_FAMILIES)
-    achieved = g_flop / (g_ms * 1e-3) / 1e12 if g_ms > 0 else 0.0
     kernels = {}
-    for k in GEMM_FAMILIES:
-        n, ms, work = fam[k]
+    for fname, unit in FAMILIES:
+        n, ms, work = fam[fname]
         if n == 0:
             continue
-        kernels["gemm_" + k] = dict(launches=n, avg_ms=ms / max(n, 1), tflops=work / max(ms * 1e-3, 1e-12) / 1e12,
-                                    frac_mfma_peak=work / max(ms * 1e-3, 1e-12) / 1e12 / PEAK_FP32_MFMA_TFLOPS)
-    n, ms, work = fam["update"]
-    kernels["optimizer_update"] = dict(launches=n, avg_ms=ms / max(n, 1), gbs=work / max(ms * 1e-3, 1e-12) / 1e9,
-                                       frac_hbm_peak=work / max(ms * 1e-3, 1e-12) / 1e9 / PEAK_HBM_GBS)
+        rate = work / max(ms * 1e-3, 1e-12)
+        entry = dict(launches=n, avg_ms=ms / n, ms_per_step=ms / steps)
+        if unit == "flop":
+            entry.update(tflops=rate / 1e12, frac_mfma_peak=rate / 1e12 / PEAK_FP32_MFMA_TFLOPS)
+        else:
+            entry.update(gbs=rate / 1e9, frac_hbm_peak=rate / 1e9 / PEAK_HBM_GBS)
+        kernels[KERNEL_NAMES.get(fname, fname)] = entry
+
+    def mfma_aggregate(names):
+        n = sum(fam[k][0] for k in names)
+        ms = sum(fam[k][1] for k in names)
+        flop = sum(fam[k][2] for k in names)
+        achieved = flop / (ms * 1e-3) / 1e12 if ms > 0 else 0.0
+        return dict(bound="mfma", achieved=achieved, peak=PEAK_FP32_MFMA_TFLOPS, unit="TFLOP/s", frac=achieved / PEAK_FP32_MFMA_TFLOPS,
+                    launches=n, avg_launch_ms=ms / max(n, 1), flops_per_launch=flop / max(n, 1), ms_per_step=ms / steps)
+
+    return dict(workload=name, wl=wl, desc_parameters=int(desc.total_parameters), batch=B, ms_per_step=ms_per_step, value=B / (ms_per_step * 1e-3),
+                kernels=kernels, loss_per_output=loss.loss_values / max(loss.number_loss, 1),
+                contractions=mfma_aggregate(("forward", "dx", "dw", "dx_dw_pair")),
+                time_loops=mfma_aggregate(("lstm_forward_loop", "lstm_backward_loop")))
+
+
+def config_of(r):
+    wl = r["wl"]
+    return {"workload": r["workload"], "batch": r["batch"], "sequence_length": wl.get("depth", 1),
+            "layers": ["res%d" % l["block_depth"] if l.get("type") == "residual" else
+                       ("bilstm%d" if l.get("bidirectional") else "lstm%d" if l.get("type") == "lstm" else "fc%d") % l["units"] for l in wl["layers"]],
+            "optimizer": wl["optimizer"], "parameters": r["desc_parameters"],
+            "gemm_flops_per_step": gemm_flops_per_step(wl["layers"], r["batch"], wl.get("depth", 1))}
+
+
+SECONDARY = "lstm512x2_t64_b256_amsgrad"   # the metric's other half
+
+
+def measured_ceilings():
+    """What this device reaches on a kernel of nothing but FP32 MFMAs and on a streaming triad, beside the published peaks."""
+    import ctypes as C
+    import torch
+    from myea_amd import binding as mb
+    lib = mb.load_library()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    tf, gb = C.c_double(), C.c_double()
+    if lib.myea_hip_ceiling_mfma_f32(stream, 20000, 3, C.byref(tf)) != 0 or lib.myea_hip_ceiling_hbm_triad(stream, 1 << 30, 5, C.byref(gb)) != 0:
+        raise RuntimeError((lib.myea_hip_last_error() or b"").decode())
+    return {"mfma_f32_tflops": tf.value, "mfma_f32_published": PEAK_FP32_MFMA_TFLOPS, "hbm_triad_gbs": gb.value, "hbm_published": PEAK_HBM_GBS,
+            "how": "myea_hip_ceiling_mfma_f32 (independent v_mfma_f32_32x32x2_f32, 2 wavefronts per SIMD) and myea_hip_ceiling_hbm_triad (3 x 1 GiB)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="fc4096x4_b1024_adam", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true", help="skip the LSTM-512 leg the default workload's line also carries")
+    ap.add_argument("--no-ceilings", action="store_true", help="skip the measured MFMA / HBM ceilings")
+    ap.add_argument("--cpu-sample-rows", type=int, default=0, help="examples in the CPU sample (default: sized for ~20 s)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on one GPU only (--gpus 1); no multi-GPU path exists")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    r = run_workload(args.workload, args.steps, args.warmup)
+    wl, B = r["wl"], r["batch"]
+    has_loops = r["time_loops"]["launches"] > 0
+    roofline = dict(r["contractions"])
+    roofline["kernel"] = "gemm_f32_mfma_kernel / gemm_pair_kernel (forward, dX, dW and paired dX + dW launches)"
+    roofline["gemm_ms_per_step"] = roofline.pop("ms_per_step")
+    traffic = RECORDED_TRAFFIC.get(args.workload)
+    roofline["traffic"] = traffic["bytes_per_launch"] if traffic else None
+    if traffic:
+        roofline["traffic_source"] = traffic["source"]
 
     out = {
         "metric": "train samples/s (fwd+bwd+Adam) FC-4096x4 & LSTM-512; % FP32 MFMA/HBM peak",
-        "value": B / (ms_per_step * 1e-3),
+        "value": r["value"],
         "unit": "samples/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": args.workload, "batch": B, "sequence_length": wl.get("depth", 1),
-                   "layers": ["res%d" % l["block_depth"] if l.get("type") == "residual" else
-                              ("bilstm%d" if l.get("bidirectional") else "lstm%d" if l.get("type") == "lstm" else "fc%d") % l["units"] for l in wl["layers"]],
-                   "optimizer": wl["optimizer"], "parameters": int(desc.total_parameters),
-                   "gemm_flops_per_step": gemm_flops_per_step(wl["layers"], B, wl.get("depth", 1))},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": PMC_TRAFFIC_BYTES_PER_GEMM_LAUNCH.get(args.workload),
-                     "kernel": "gemm_f32_mfma_kernel / gemm_pair_kernel (forward, dX, dW and paired dX + dW launches)", "launches": g_launch,
-                     "avg_launch_ms": g_ms / max(g_launch, 1), "flops_per_launch": g_flop / max(g_launch, 1),
-                     "gemm_ms_per_step": g_ms / args.steps},
-        "kernels": kernels,
-        "loss_per_output": loss.loss_values / max(loss.number_loss, 1),
+        "config": config_of(r),
+        "roofline": roofline,
+        "kernels": r["kernels"],
+        "loss_per_output": r["loss_per_output"],
     }
+    if has_loops:
+        out["time_loops"] = dict(r["time_loops"], kernel="lstm_resident_forward_kernel / lstm_resident_backward_kernel (or one lstm_fused_* launch per step)")
+    if args.workload != SECONDARY and args.workload == "fc4096x4_b1024_adam" and not args.no_secondary:
+        s = run_workload(SECONDARY, max(5, args.steps // 3), max(2, args.warmup // 2))
+        loops = dict(s["time_loops"], kernel="lstm_resident_forward_kernel + lstm_resident_backward_kernel: the recurrent contractions and gate math of steps 1 .. T-1, one launch per layer and pass")
+        out["secondary"] = {"workload": SECONDARY, "value": s["value"], "unit": "samples/s", "ms_per_step": s["ms_per_step"],
+                            "steps": max(5, args.steps // 3), "config": config_of(s), "roofline": loops,
+                            "contractions": s["contractions"], "kernels": s["kernels"], "loss_per_output": s["loss_per_output"]}
+    if not args.no_ceilings:
+        out["ceilings"] = measured_ceilings()
     if not args.no_cpu_baseline:
         threads = min(16, os.cpu_count() or 1)
         rows = args.cpu_sample_rows

@@ -447,7 +447,9 @@ int myea_hip_upload_tensor(myea_hip_net *net, size_t layer_index, int kind, cons
  * family since the last reset.  family: 0 = forward (NT), 1 = dX (NN), 2 = dW (TN), 3 = optimizer
  * update (bytes instead of FLOPs), 4 = a layer's dX and dW contractions in one launch, 5 = the recurrent
  * contractions and gate math of an LSTM layer's forward time loop (steps 1 .. T-1; one launch per layer when the
- * loop runs as a resident kernel, one per step otherwise), 6 = the same of its backward time loop. */
+ * loop runs as a resident kernel, one per step otherwise), 6 = the same of its backward time loop, 7 = batch
+ * (re)normalisation forward and backward (bytes: every activation read or written once), 8 = column sums of the
+ * deltas for the bias gradients (bytes). */
 int myea_hip_profile_enable(myea_hip_net *net, int enable);
 int myea_hip_profile_read(myea_hip_net *net, int family, uint64_t *launches, double *milliseconds, double *work);
 
@@ -471,6 +473,14 @@ int myea_hip_gemm_f32(void *stream, int a_k_contiguous, int b_k_contiguous, int 
 int myea_hip_optimizer_update(void *stream, const myea_hyper *hyper, size_t count, size_t weight_count,
                               float gradient_scale, float *parameters, float *gradient,
                               float *state0, float *state1, float *state2);
+
+/* ---- measured ceilings (no counterpart in the reference: figures for a benchmark's roofline) ----
+ * myea_hip_ceiling_mfma_f32: a kernel of nothing but independent v_mfma_f32_32x32x2_f32, two wavefronts per SIMD,
+ * `iterations` x 16 MFMAs per wavefront; best of `repeats` launches, in TFLOP/s.
+ * myea_hip_ceiling_hbm_triad: a[i] = b[i] + s * c[i] over three arrays of `bytes_per_array` (allocated and freed by
+ * the call; choose them well beyond the caches); best of `repeats`, in GB/s of the 3 x bytes_per_array moved. */
+int myea_hip_ceiling_mfma_f32(void *stream, int iterations, int repeats, double *tflops);
+int myea_hip_ceiling_hbm_triad(void *stream, size_t bytes_per_array, int repeats, double *gigabytes_per_second);
 
 #ifdef __cplusplus
 }

@@ -104,6 +104,7 @@ ABI_SYMBOLS = [
     "myea_hip_update_derivative_weight", "myea_hip_update_derivative_weight_no_alloc", "myea_hip_backward_pass_and_update_derivative_weight", "myea_hip_update_parameter", "myea_hip_reset_loss", "myea_hip_get_loss",
     "myea_hip_download_gradient", "myea_hip_upload_gradient", "myea_hip_download_tensor", "myea_hip_upload_tensor",
     "myea_hip_profile_enable", "myea_hip_profile_read", "myea_hip_gemm_f32", "myea_hip_optimizer_update",
+    "myea_hip_ceiling_mfma_f32", "myea_hip_ceiling_hbm_triad",
 ]
 
 _lib = None
@@ -165,6 +166,8 @@ def load_library(path=LIB_PATH):
     lib.myea_hip_profile_read.argtypes = [vp, i32, P(C.c_uint64), P(C.c_double), P(C.c_double)]
     lib.myea_hip_gemm_f32.argtypes = [vp, i32, i32, i32, sz, sz, sz, vp, sz, vp, sz, vp, sz]
     lib.myea_hip_optimizer_update.argtypes = [vp, P(Hyper), sz, sz, C.c_float, vp, vp, vp, vp, vp]
+    lib.myea_hip_ceiling_mfma_f32.argtypes = [vp, i32, i32, P(C.c_double)]
+    lib.myea_hip_ceiling_hbm_triad.argtypes = [vp, sz, i32, P(C.c_double)]
     for name in ABI_SYMBOLS:
         if name not in ("myea_hyper_default", "myea_hip_last_error"):
             getattr(lib, name).restype = i32

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(CSRC, "libmyea_hip.so")
-HIP_SOURCES = ["myea_gemm.hip", "myea_elementwise.hip", "myea_lstm.hip", "myea_lstm_fused.hip", "myea_lstm_resident.hip", "myea_net.hip"]
+HIP_SOURCES = ["myea_gemm.hip", "myea_elementwise.hip", "myea_lstm.hip", "myea_lstm_fused.hip", "myea_lstm_resident.hip", "myea_ceilings.hip", "myea_net.hip"]
 C_SOURCES = ["myea_layout.c"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed-FP32 instructions are switched off for every device TU

@@ -44,8 +44,8 @@ struct DevLayer {
     LstmLayer *lstm = nullptr, *lstm2 = nullptr;  // lstm2: the time-reversed direction of a bidirectional layer
 };
 
-constexpr int kProfFamilies = 7;   // forward, dX, dW, update, dX + dW launched as a pair, LSTM time loop forward, backward
-constexpr int kProfLstmForwardLoop = 5, kProfLstmBackwardLoop = 6;
+constexpr int kProfFamilies = 9;   // forward, dX, dW, update, dX + dW launched as a pair, LSTM time loop forward, backward, normalisation, bias gradients
+constexpr int kProfLstmForwardLoop = 5, kProfLstmBackwardLoop = 6, kProfNormalization = 7, kProfBiasGradient = 8;
 struct ProfEvent {
     hipEvent_t start = nullptr, stop = nullptr;
     int family = 0;

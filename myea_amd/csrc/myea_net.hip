@@ -536,7 +536,11 @@ int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool train
     p.r_max = h.batch_renormalization_r_correction_maximum; p.d_max = h.batch_renormalization_d_correction_maximum;
     p.renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
     p.act_out = act_out; p.colscale = colscale; p.act = (int)l.type_activation_function;
-    return launch_bn_forward_training(stream, p, scratch);
+    // algorithmic bytes: x read once, the normalised values (x-hat) and the scaled and shifted output written once
+    prof_begin(kProfNormalization);
+    const int rc = launch_bn_forward_training(stream, p, scratch);
+    prof_end((double)rows * (double)H * sizeof(float) * (act_out ? 4.0 : 3.0));
+    return rc;
 }
 
 // A resident LSTM launch whose bounded wait gave up has left the pass it belonged to incomplete.  Reported once, at the
@@ -966,7 +970,11 @@ int Net::bn_backward(size_t li, size_t t, size_t rows, const float *x, const flo
     p.dscale = scale_ptr(gradient, li); p.dshift = shift_ptr(gradient, li);
     p.dx = dx;
     p.renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
-    return launch_bn_backward(stream, p, scratch);
+    // algorithmic bytes: dy and x-hat read once, dx written once
+    prof_begin(kProfNormalization);
+    const int rc = launch_bn_backward(stream, p, scratch);
+    prof_end((double)rows * (double)H * sizeof(float) * 3.0);
+    return rc;
 }
 
 int Net::backward_pass_and_update_derivative_weight(size_t B)
@@ -1050,8 +1058,11 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
             if (!layer_is_dense(l)) continue;
             DevLayer &o = L[li];
             if (layer_uses_bias(l))
-                for (size_t c = 0; c < chunks; ++c)
+                for (size_t c = 0; c < chunks; ++c) {
+                    prof_begin(kProfBiasGradient);
                     MYEA_TRY(launch_column_sum(stream, rows, o.H, o.neuron_errors + c * Bmax * o.H, gradient + l.first_bias_connection_index, 1, scratch));
+                    prof_end((double)rows * (double)o.H * sizeof(float));
+                }
             if (layer_is_ind_rnn(l))
                 MYEA_TRY(launch_ind_rnn_self_weight_gradient(stream, T, B, Bmax, o.H, o.values, o.dafs_own ? o.dafs_own : o.neuron_errors,
                                                              gradient + l.first_connection_index + o.H * o.In, scratch));
