@@ -831,6 +831,14 @@ int launch_column_sum(hipStream_t s, size_t rows, size_t H, const float *x, floa
     return MYEA_OK;
 }
 
+int launch_column_sum_final(hipStream_t s, size_t H, size_t S, const float *partial, float *out, int accumulate)
+{
+    if (H == 0) return MYEA_OK;
+    hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, kBlock)), dim3(kBlock), 0, s, H, S, partial, out, accumulate);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
 int launch_dropout_noise(hipStream_t s, size_t n, float *noise, int normal, float a, float b, unsigned long long seed, unsigned long long stream_id)
 {
     if (n == 0) return MYEA_OK;

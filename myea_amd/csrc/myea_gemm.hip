@@ -25,6 +25,8 @@
 //
 // Accumulator layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
 //   C[(r / 4) * 8 + (l / 32) * 4 + (r % 4)][l % 32].
+#include <mutex>
+
 #include "myea_device_af.h"
 #include "myea_kernels.h"
 
@@ -259,6 +261,7 @@ struct GemmDev {
     float steep;
     const float *addend;
     long ld_addend;
+    float *col_partials;
     int nbm, nbn;
     int ksplit, kchunk;   // split-K: number of slabs and k's per slab (multiple of BK); slab s writes C + s * slab
     long slab;
@@ -278,7 +281,9 @@ struct TilePlace {
 //        lane of one workgroup, so the result is the C + v a load / add / store gives, and nothing waits for C to come in)
 //   KIND 1 forward: C = v + bias, aux_out = AF(C) * column multiplier; CLASS 0 no aux_out, 1 piecewise linear (linear, ReLU,
 //        leaky: s < 0 ? slope * s : s, ReLU's zero kept exact), 2 through exp (sigmoid, tanh: a / (1 + exp(k s)) - b)
-//   KIND 2 C = v * AF'(pre, steep, val); CLASS 1 piecewise (q < 0 ? steep * slope : steep), 2 smooth (tanh, sigmoid)
+//   KIND 2 C = v * AF'(pre, steep, val); CLASS 1 piecewise (q < 0 ? steep * slope : steep), 2 smooth (tanh, sigmoid);
+//        with col_partials, the sum of each 32-row accumulator's column goes out too: 16 values per lane, the two lanes
+//        of a column combined, one store per (32-row block, column) - the bias gradient needs no pass of its own over C
 // Edge tiles (WHOLE false) run the same arithmetic behind a bounds test per element, so an element's value does not
 // depend on the tile shape it was computed in.
 template <int KIND, int CLASS, bool ADDEND, bool WHOLE, int TM, int TN>
@@ -300,6 +305,7 @@ __device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&a
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int row0 = at.m0 + at.wave_m + i * 32 + at.half * 4;
+            float column_sum = 0.f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = row0 + (r >> 2) * 8 + (r & 3);
@@ -325,12 +331,22 @@ __device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&a
                         const float y = p.val[o];
                         dv = tanh_like ? p.steep * (1.f - y * y) : p.steep * y * (1.f - y);
                     }
-                    p.C[o] = v * dv;
+                    {
+#pragma clang fp contract(off)   // the sum takes the stored, rounded product - never a fused multiply-add - so every tile shape gives the same bits
+                        const float out = v * dv;
+                        p.C[o] = out;
+                        column_sum = column_sum + out;
+                    }
                 } else if (KIND == 3) {
                     unsafeAtomicAdd(&p.C[o], v);
                 } else {
                     p.C[o] = v;
                 }
+            }
+            if (KIND == 2 && p.col_partials) {
+                const float both = column_sum + __shfl_xor(column_sum, 32);   // the column's other 16 rows of this accumulator
+                const int block_row = at.m0 + at.wave_m + i * 32;
+                if (at.half == 0 && (WHOLE || block_row < p.M)) p.col_partials[(long)(block_row >> 5) * p.N + col] = both;
             }
         }
     }
@@ -509,11 +525,10 @@ int launch_one(hipStream_t stream, GemmDev d)
 {
     constexpr size_t lds_bytes = ((VEC && BM * BN < 128 * 128) ? 3 : 2) * (OperandPath<BM, A_KC, VEC>::kFloats + OperandPath<BN, B_KC, VEC>::kFloats) * sizeof(float);
     auto kern = gemm_f32_mfma_kernel<BM, BN, A_KC, B_KC, VEC>;
-    static bool attr_done = false;  // per instantiation
-    if (!attr_done) {
-        MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        attr_done = true;
-    }
+    static std::once_flag attr_once;  // per instantiation; launches may come from several host threads
+    static hipError_t attr_status = hipSuccess;
+    std::call_once(attr_once, [&] { attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes); });
+    if (attr_status != hipSuccess) return hip_fail(attr_status, "hipFuncSetAttribute(gemm_f32_mfma_kernel)");
     d.nbm = (d.M + BM - 1) / BM;
     d.nbn = (d.N + BN - 1) / BN;
     const long nblocks = (long)d.nbm * d.nbn * d.ksplit;
@@ -600,6 +615,8 @@ static int prepare_gemm(const GemmParams &p, GemmDev &d, bool *vec)
     d.bias = p.bias; d.aux_out = p.aux_out; d.colscale = p.colscale;
     d.pre = p.pre; d.val = p.val; d.act = p.act; d.steep = p.steep;
     d.addend = p.addend; d.ld_addend = p.ld_addend;
+    d.col_partials = p.col_partials;
+    if (p.col_partials && p.epilogue != EPI_FC_DERIVE) { set_last_error("gemm: column partial sums go with the derivative epilogue only"); return MYEA_E_INVALID; }
     if (p.addend && (p.epilogue == EPI_FC_FORWARD || p.ld_addend < p.N)) { set_last_error("gemm: addend needs EPI_NONE / EPI_FC_DERIVE and ld_addend >= N"); return MYEA_E_INVALID; }
     d.nbm = d.nbn = 0;
     d.ksplit = 1; d.kchunk = p.K > 0 ? p.K : 1; d.slab = 0;
@@ -668,22 +685,20 @@ int launch_gemm_pair(hipStream_t stream, const GemmParams &a, const GemmParams &
         const long na = (long)da.nbm * da.nbn;
         constexpr size_t lds_a = 2 * (OperandPath<128, true, true>::kFloats + OperandPath<128, false, true>::kFloats) * sizeof(float);
         constexpr size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
-        static bool attr_done = false;
-        if (!attr_done) {
-            MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pair_kernel<128, 128>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-            attr_done = true;
-        }
+        static std::once_flag attr_once;
+        static hipError_t attr_status = hipSuccess;
+        std::call_once(attr_once, [&] { attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pair_kernel<128, 128>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes); });
+        if (attr_status != hipSuccess) return hip_fail(attr_status, "hipFuncSetAttribute(gemm_pair_kernel)");
         hipLaunchKernelGGL((gemm_pair_kernel<128, 128>), dim3((unsigned)(na + nb)), dim3(kThreads), lds_bytes, stream, da, db, (int)na);
     } else if (fits(64)) {
         da.nbm = (a.M + 63) / 64; da.nbn = (a.N + 63) / 64;
         const long na = (long)da.nbm * da.nbn;
         constexpr size_t lds_a = 3 * (OperandPath<64, true, true>::kFloats + OperandPath<64, false, true>::kFloats) * sizeof(float);
         constexpr size_t lds_bytes = lds_a > lds_b ? lds_a : lds_b;
-        static bool attr_done = false;
-        if (!attr_done) {
-            MYEA_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pair_kernel<64, 64>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-            attr_done = true;
-        }
+        static std::once_flag attr_once;
+        static hipError_t attr_status = hipSuccess;
+        std::call_once(attr_once, [&] { attr_status = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pair_kernel<64, 64>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes); });
+        if (attr_status != hipSuccess) return hip_fail(attr_status, "hipFuncSetAttribute(gemm_pair_kernel)");
         hipLaunchKernelGGL((gemm_pair_kernel<64, 64>), dim3((unsigned)(na + nb)), dim3(kThreads), lds_bytes, stream, da, db, (int)na);
     } else {
         return 1;

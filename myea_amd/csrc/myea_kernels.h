@@ -45,6 +45,9 @@ struct GemmParams {
     // gradient of a residual block arriving at the same destination); may be null
     const float *addend;
     long ld_addend;
+    // EPI_FC_DERIVE: when not null, [ceil(M / 32)][N] - the column sums of C over each block of 32 rows (the bias gradient's
+    // partial sums, taken from the accumulators on their way out; fixed order, so repeatable); the consumer sums the blocks
+    float *col_partials;
     // split-K (deterministic): slab s of the K range writes its partial product to C + s * split_k_slab; the consumer
     // sums the slabs in order.  Requires EPI_NONE and accumulate == 0.  0 / 1 = off.
     int split_k;
@@ -81,6 +84,8 @@ int launch_colscale(hipStream_t s, size_t rows, size_t H, float *y, const float 
 int launch_mask_to_scale(hipStream_t s, size_t n, const uint8_t *mask, float on, float *colscale);
 // out[j] (+)= sum_r x[r][j]; scratch >= 64 * H floats
 int launch_column_sum(hipStream_t s, size_t rows, size_t H, const float *x, float *out, int accumulate, float *scratch);
+// out[col] (+)= sum over the S rows of partial[S][H], in row order
+int launch_column_sum_final(hipStream_t s, size_t H, size_t S, const float *partial, float *out, int accumulate);
 
 // batch-normalisation forward (training): statistics, running averages, r/d corrections, hats, normalizes
 struct BnForwardParams {

@@ -26,6 +26,11 @@ struct DevLayer {
     // [T][Bmax][H] (summations, neuron_errors), [T][Bmax][AH] (values), [T][Bmax][NH] (hats, normalizes)
     float *summations = nullptr, *values = nullptr, *hats = nullptr, *normalizes = nullptr, *neuron_errors = nullptr;
     float *in_errors = nullptr;  // normalised first member of a block: delta reduced to its input side [Bmax][In]
+    // column sums of neuron_errors per block of 32 rows [ceil(T Bmax / 32)][H], left by the contraction that wrote the errors
+    // (the bias gradient then sums the blocks instead of the rows); bias_partial_rows = blocks valid for a batch of
+    // bias_partial_batch examples, 0 = the errors were written some other way
+    float *bias_partials = nullptr;
+    size_t bias_partial_rows = 0, bias_partial_batch = 0;
     // [T][NH]
     float *means = nullptr, *variances = nullptr, *means_averages = nullptr, *variances_averages = nullptr;
     float *r_corrections = nullptr, *d_corrections = nullptr;

@@ -309,6 +309,7 @@ int Net::create(const myea_net_desc &desc)
             MYEA_HIP_TRY(hipMemset(o.summations, 0, sz * sizeof(float)));
         }
         MYEA_TRY(dev_alloc(&o.neuron_errors, sz));  // residual layer: its basic units' errors
+        if (layer_is_dense(l) && layer_uses_bias(l) && li + 1 < d.n_layers) MYEA_TRY(dev_alloc(&o.bias_partials, (T * B + 31) / 32 * o.H));
         MYEA_HIP_TRY(hipMemset(o.neuron_errors, 0, sz * sizeof(float)));
         if (layer_is_ind_rnn(l)) {
             MYEA_TRY(dev_alloc(&o.pre_afs, sz));
@@ -393,7 +394,7 @@ Net::~Net()
     fr(seg_first); fr(seg_len);
     fr(masks); fr(zoneout_masks);
     for (DevLayer &o : L) {
-        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index); fr(o.pre_afs); fr(o.dafs_own); fr(o.noise);
+        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.bias_partials); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index); fr(o.pre_afs); fr(o.dafs_own); fr(o.noise);
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
@@ -844,6 +845,8 @@ int Net::backward_into_layer(size_t li, size_t B)
         } else if (!norm) {
             g.C = (fuse ? o.neuron_errors : tmp1) + roff * H;
             g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.summations + roff * H; g.val = o.values + roff * H;
+            // this launch writes the layer's final errors: their column sums (the bias gradient's) come out with them
+            if (fuse && chunks == 1 && o.bias_partials) { g.col_partials = o.bias_partials; o.bias_partial_rows = (rows + 31) / 32; o.bias_partial_batch = B; }
         } else if (before) {
             g.C = tmp1 + roff * H;
             g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.normalizes + roff * H; g.val = o.values + roff * H;
@@ -994,6 +997,7 @@ int Net::backward_pass(size_t B)
 {
     if (B == 0 || B > d.batch_size) { set_last_error("Backward_Pass: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
     if (state != MYEA_STATE_TRAINING) { set_last_error("Backward_Pass: can not back propagate gradient in inference mode"); return MYEA_E_STATE; }
+    for (DevLayer &o : L) o.bias_partial_rows = 0;   // set again by the contractions that leave column sums with a layer's errors
     // the walk of FF__Backward_Pass_Batch: from a consumer gi to its producer li = previous_connected_layers[0]; once a
     // residual layer's block is done it resumes from the residual layer itself (:117-120)
     for (size_t gi = d.n_layers - 1; gi != 1; --gi) {
@@ -1060,8 +1064,13 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
             if (layer_uses_bias(l))
                 for (size_t c = 0; c < chunks; ++c) {
                     prof_begin(kProfBiasGradient);
-                    MYEA_TRY(launch_column_sum(stream, rows, o.H, o.neuron_errors + c * Bmax * o.H, gradient + l.first_bias_connection_index, 1, scratch));
-                    prof_end((double)rows * (double)o.H * sizeof(float));
+                    if (chunks == 1 && o.bias_partial_rows == (rows + 31) / 32 && o.bias_partial_batch == B) {
+                        MYEA_TRY(launch_column_sum_final(stream, o.H, o.bias_partial_rows, o.bias_partials, gradient + l.first_bias_connection_index, 1));
+                        prof_end((double)o.bias_partial_rows * (double)o.H * sizeof(float));
+                    } else {
+                        MYEA_TRY(launch_column_sum(stream, rows, o.H, o.neuron_errors + c * Bmax * o.H, gradient + l.first_bias_connection_index, 1, scratch));
+                        prof_end((double)rows * (double)o.H * sizeof(float));
+                    }
                 }
             if (layer_is_ind_rnn(l))
                 MYEA_TRY(launch_ind_rnn_self_weight_gradient(stream, T, B, Bmax, o.H, o.values, o.dafs_own ? o.dafs_own : o.neuron_errors,
