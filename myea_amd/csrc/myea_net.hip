@@ -1320,9 +1320,8 @@ int Net::update_parameter(size_t B, size_t training_size)
     } else {
         const float lr = scale * h.adam_learning_rate;
         p.beta1 = h.adam_beta1; p.beta2 = h.adam_beta2; p.eps = h.adam_epsilon;
-        p.lr_t = h.use_adam_bias_correction
-                     ? (float)(lr * std::sqrt(1.0 - std::pow((double)h.adam_beta2, (double)ts)) / (1.0 - std::pow((double)h.adam_beta1, (double)ts)))
-                     : lr;
+        // in float throughout, as NN/Neural_Network__Adam.cpp:58 evaluates it with T_ = float
+        p.lr_t = h.use_adam_bias_correction ? lr * std::sqrt(1.f - std::pow(h.adam_beta2, ts)) / (1.f - std::pow(h.adam_beta1, ts)) : lr;
         p.lower = scale * h.learning_rate_final * (1.f - 1.f / (h.learning_gamma * ts + 1.f));
         p.upper = scale * h.learning_rate_final * (1.f + 1.f / (h.learning_gamma * ts));
         if (kind == MYEA_OPTIMIZER_NOSADAM) {
@@ -1667,9 +1666,7 @@ int myea_hip_optimizer_update(void *stream, const myea_hyper *h, size_t count, s
     p.lr = h->learning_rate; p.mu = h->learning_momentum;
     p.variant = h->learning_momentum != 0.f ? (h->use_Nesterov ? 2 : 1) : 0;
     p.beta1 = h->adam_beta1; p.beta2 = h->adam_beta2; p.eps = h->adam_epsilon;
-    p.lr_t = h->use_adam_bias_correction
-                 ? (float)(h->adam_learning_rate * std::sqrt(1.0 - std::pow((double)h->adam_beta2, (double)ts)) / (1.0 - std::pow((double)h->adam_beta1, (double)ts)))
-                 : h->adam_learning_rate;
+    p.lr_t = h->use_adam_bias_correction ? h->adam_learning_rate * std::sqrt(1.f - std::pow(h->adam_beta2, ts)) / (1.f - std::pow(h->adam_beta1, ts)) : h->adam_learning_rate;
     p.lower = h->learning_rate_final * (1.f - 1.f / (h->learning_gamma * ts + 1.f));
     p.upper = h->learning_rate_final * (1.f + 1.f / (h->learning_gamma * ts));
     return myea::launch_update(static_cast<hipStream_t>(stream), p);

@@ -1723,7 +1723,8 @@ int myea_oracle_update_parameter(myea_oracle_net *n, size_t B, size_t training_s
          * NN/Neural_Network__AMSBound.cpp:43-110, NN/Neural_Network__NosAdam.cpp:43-100 */
         uint32_t kind = h->type_optimizer_function;
         float lr = scale * h->adam_learning_rate, b1 = h->adam_beta1, b2 = h->adam_beta2, eps = h->adam_epsilon, ts = h->optimizer_time_step;
-        float lr_t = h->use_adam_bias_correction ? (float)(lr * sqrt(1.0 - pow(b2, ts)) / (1.0 - pow(b1, ts))) : lr;
+        /* every operand is a T_ = float there (NN/Neural_Network__Adam.cpp:58): float pow and sqrt, product first, then the quotient */
+        float lr_t = h->use_adam_bias_correction ? lr * sqrtf(1.f - powf(b2, ts)) / (1.f - powf(b1, ts)) : lr;
         float lo = scale * h->learning_rate_final * (1.f - 1.f / (h->learning_gamma * ts + 1.f));
         float hi = scale * h->learning_rate_final * (1.f + 1.f / (h->learning_gamma * ts));
         float b2v = b2;   /* the decay applied to the second moment */

@@ -148,3 +148,41 @@ def test_clip_gradient_global_norm():
     assert_close(_run(net, w0, [g2])[0], -g2.astype(np.float64))
     g3 = np.zeros(P, dtype=np.float32); g3[3] = 2.0                         # norm == clip: scaled by exactly 1
     assert_close(_run(net, w0, [g3])[0], -g3.astype(np.float64))
+
+
+def test_adam_bias_corrected_rate_is_evaluated_in_float():
+    """The reference evaluates lr_t = lr * sqrt(1 - beta2^t) / (1 - beta1^t) with every operand a float
+    (NN/Neural_Network__Adam.cpp:58, T_ = float).  With a gradient of constant sign and m = v = 0 at the start, step t moves
+    a weight by lr_t * m_t / (sqrt(v_t) + eps): restated here in numpy float32 it must match the oracle bit for bit, and the
+    same restatement with lr_t evaluated in double and rounded once must NOT (it differs in the last bits at some t <= 10) -
+    the check a double-precision lr_t fails."""
+    f = np.float32
+    lr, b1, b2, eps = f(1e-3), f(0.9), f(0.999), f(1e-8)
+    desc, net = _net(type_optimizer_function=mb.OPTIMIZER["ADAM"], adam_learning_rate=float(lr), adam_beta1=float(b1), adam_beta2=float(b2),
+                     adam_epsilon=float(eps), use_adam_bias_correction=1)
+    P = desc.total_parameters
+    rng = np.random.default_rng(11)
+    w0 = rng.normal(0, 1, P).astype(f)
+    grads = [rng.normal(0, 0.5, P).astype(f) for _ in range(10)]
+    got = [g.astype(f) for g in _run(net, w0, grads)]
+
+    def restate(rate_in_double):
+        w, m, v, out = w0.copy(), np.zeros(P, f), np.zeros(P, f), []
+        for k, g in enumerate(grads):
+            t = f(k + 1)
+            m = b1 * m + (f(1) - b1) * g
+            v = b2 * v + (f(1) - b2) * g * g
+            if rate_in_double:
+                lr_t = f(float(lr) * np.sqrt(1.0 - float(b2) ** float(t)) / (1.0 - float(b1) ** float(t)))
+            else:
+                # powf as the C library gives it: the correctly rounded float power (numpy's float32 power is a different routine)
+                p2, p1 = f(float(b2) ** float(t)), f(float(b1) ** float(t))
+                lr_t = f(lr * np.sqrt(f(1) - p2, dtype=f)) / (f(1) - p1)
+            w = w - lr_t * m / (np.sqrt(v, dtype=f) + eps)
+            out.append(w.astype(f))
+        return out
+
+    in_float, in_double = restate(False), restate(True)
+    assert any(not np.array_equal(a, b) for a, b in zip(in_float, in_double)), "float and double rates coincide on this data: the test pins nothing"
+    for k in range(10):
+        assert np.array_equal(got[k], in_float[k]), "step %d: the oracle's rate is not the float expression" % (k + 1)
