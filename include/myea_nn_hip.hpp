@@ -14,6 +14,7 @@
 #include <cfloat>
 #include <cmath>
 #include <cstring>
+#include <random>
 #include <string>
 #include <vector>
 
@@ -30,6 +31,15 @@ struct Layer_Parameters {
     // [0] FC: neurons, LSTM: blocks, RESIDUAL: block depth.  [1] LSTM: cells per block.
     // pooling layers: [0] kernel size, [1] stride, [2] padding, [3] dilation, [4] ceil mode.
     size_t unit_parameters[5u] = {0};
+};
+
+// The reference's callers hand `struct Layer` pointers to Update_Derivative_Weight (Dataset.cpp:655-657:
+// ptr_array_layers + 1, ptr_last_layer).  Here a Layer is a read-only view of one descriptor entry; what matters to the
+// step functions is its position in ptr_array_layers.
+struct Layer {
+    unsigned int type_layer = MYEA_LAYER_NONE, type_dropout = MYEA_DROPOUT_NONE;
+    bool use_bidirectional = false;
+    T_ dropout_values[3] = {0.f, 0.f, 0.f};
 };
 
 class Neural_Network_HIP {
@@ -60,6 +70,9 @@ public:
     // public host copies, written by the caller like the reference's members and pushed with the Copy__* calls
     T_ *ptr_array_parameters = nullptr;                      // [total_parameters]
     bool *ptr_array_units_mask_dropout_bernoulli = nullptr;  // [(sum of AF units) * T], all true after Compile
+    struct Layer *ptr_array_layers = nullptr;                // [total_layers], refreshed by Compile and the Set__* calls
+    struct Layer const *ptr_last_layer = nullptr;            // ptr_array_layers + total_layers
+    size_t total_layers = 0;
 
     Neural_Network_HIP() { std::memset(&desc_, 0, sizeof(desc_)); }
     ~Neural_Network_HIP() { Deallocate(); }
@@ -245,6 +258,7 @@ public:
     // descriptor and uploads parameters and masks.
     bool Set__HIP(bool use_hip)
     {
+        pushed_valid_ = false;
         if (!use_hip) { if (net_) { myea_hip_destroy(net_); net_ = nullptr; } return true; }
         if (net_) { myea_hip_destroy(net_); net_ = nullptr; }
         if (myea_hip_create(&desc_, &net_) != MYEA_OK) return Fail("Set__HIP", myea_hip_last_error());
@@ -297,38 +311,94 @@ public:
     void Reset__Loss() { if (Need("Reset__Loss")) Ok("Reset__Loss", myea_hip_reset_loss(net_)); }
 
     // ---- the five step entry points (Data.hpp:2896, 1033, 1709, 2199, 849) ----
-    void Forward_Pass(size_t batch_size_received, T_ const *const *ptr_array_inputs)
+    // The reference's training loop calls them from inside `#pragma omp parallel` (Dataset.cpp:645-658): every thread of the
+    // team makes the same call and the work is shared inside.  Here one thread - the master - makes the device call, between
+    // two barriers, so the unchanged loop may keep its parallel region; outside a parallel region the barriers do nothing.
+    // input_layer_index / output_layer_index: only the defaults (the whole network) are on this path.
+    void Forward_Pass(size_t batch_size_received, T_ const *const *ptr_array_inputs, long long int input_layer_index_received = -1ll,
+                      long long int output_layer_index_received = -1ll)
     {
-        if (!Need("Forward_Pass") || !PushFields("Forward_Pass")) return;
-        const size_t row = (size_t)desc_.layers[0].n_units * desc_.number_recurrent_depth;
-        if (!Flatten("Forward_Pass", batch_size_received, ptr_array_inputs, row)) return;
-        Ok("Forward_Pass", myea_hip_forward_pass(net_, batch_size_received, rows_.data(), 0));
+        Solo([&] {
+            if (input_layer_index_received != -1ll || output_layer_index_received != -1ll) { Fail("Forward_Pass", "a forward pass over a range of layers is not on this path"); return; }
+            if (!Need("Forward_Pass") || !PushFields("Forward_Pass")) return;
+            const size_t row = (size_t)desc_.layers[0].n_units * desc_.number_recurrent_depth;
+            if (!Flatten("Forward_Pass", batch_size_received, ptr_array_inputs, row)) return;
+            Ok("Forward_Pass", myea_hip_forward_pass(net_, batch_size_received, rows_.data(), 0));
+        });
     }
     void Compute__Error(size_t batch_size_received, T_ const *const *ptr_array_desireds_outputs)
     {
-        if (!Need("Compute__Error") || !PushFields("Compute__Error")) return;
-        const size_t row = (size_t)desc_.layers[desc_.n_layers - 1].n_units * desc_.number_recurrent_depth;
-        if (!Flatten("Compute__Error", batch_size_received, ptr_array_desireds_outputs, row)) return;
-        Ok("Compute__Error", myea_hip_compute_error(net_, batch_size_received, rows_.data(), 0));
+        Solo([&] {
+            if (!Need("Compute__Error") || !PushFields("Compute__Error")) return;
+            const size_t row = (size_t)desc_.layers[desc_.n_layers - 1].n_units * desc_.number_recurrent_depth;
+            if (!Flatten("Compute__Error", batch_size_received, ptr_array_desireds_outputs, row)) return;
+            Ok("Compute__Error", myea_hip_compute_error(net_, batch_size_received, rows_.data(), 0));
+        });
     }
-    void Backward_Pass(size_t batch_size_received) { if (Need("Backward_Pass") && PushFields("Backward_Pass")) Ok("Backward_Pass", myea_hip_backward_pass(net_, batch_size_received)); }
+    void Backward_Pass(size_t batch_size_received)
+    {
+        Solo([&] { if (Need("Backward_Pass") && PushFields("Backward_Pass")) Ok("Backward_Pass", myea_hip_backward_pass(net_, batch_size_received)); });
+    }
     // Backward_Pass and Update_Derivative_Weight(batch, 1, total_layers) of Train_Batch_BP (Dataset.cpp:645-658) as one call
     void Backward_Pass__Update_Derivative_Weight(size_t batch_size_received)
     {
-        if (Need("Backward_Pass") && PushFields("Backward_Pass")) Ok("Backward_Pass", myea_hip_backward_pass_and_update_derivative_weight(net_, batch_size_received));
+        Solo([&] { if (Need("Backward_Pass") && PushFields("Backward_Pass")) Ok("Backward_Pass", myea_hip_backward_pass_and_update_derivative_weight(net_, batch_size_received)); });
     }
-    // the reference's callers pass (ptr_array_layers + 1, ptr_last_layer); here as layer indices
+    // Data.hpp:2199: the layers [ptr_layer_it_received, ptr_layer_end_received) of ptr_array_layers
+    void Update_Derivative_Weight(size_t batch_size_received, struct Layer *const ptr_layer_it_received, struct Layer const *const ptr_layer_end_received)
+    {
+        if (ptr_array_layers == nullptr || ptr_layer_it_received < ptr_array_layers || ptr_layer_end_received > ptr_last_layer || ptr_layer_it_received > ptr_layer_end_received) {
+            Solo([&] { Fail("Update_Derivative_Weight", "the layer pointers do not lie in ptr_array_layers"); });
+            return;
+        }
+        Update_Derivative_Weight(batch_size_received, (size_t)(ptr_layer_it_received - ptr_array_layers), (size_t)(ptr_layer_end_received - ptr_array_layers));
+    }
+    // the same with layer indices; end_layer_index 0 = the last layer
     void Update_Derivative_Weight(size_t batch_size_received, size_t first_layer_index = 1, size_t end_layer_index = 0)
     {
-        if (!Need("Update_Derivative_Weight")) return;
-        Ok("Update_Derivative_Weight", myea_hip_update_derivative_weight(net_, batch_size_received, first_layer_index, end_layer_index ? end_layer_index : desc_.n_layers));
+        Solo([&] {
+            if (!Need("Update_Derivative_Weight")) return;
+            Ok("Update_Derivative_Weight", myea_hip_update_derivative_weight(net_, batch_size_received, first_layer_index, end_layer_index ? end_layer_index : desc_.n_layers));
+        });
     }
     void Update_Parameter(size_t batch_size_received, size_t training_size_received)
     {
-        if (!Need("Update_Parameter") || !PushFields("Update_Parameter")) return;
-        Ok("Update_Parameter", myea_hip_update_parameter(net_, batch_size_received, training_size_received));
-        PullState();
+        Solo([&] {
+            if (!Need("Update_Parameter") || !PushFields("Update_Parameter")) return;
+            Ok("Update_Parameter", myea_hip_update_parameter(net_, batch_size_received, training_size_received));
+            PullState();
+        });
     }
+
+    // Dropout_Bernoulli (Data.hpp:944; Neural_Network__Dropout__Bernoulli__Loop.cpp:33-97): new keep / drop draws for the
+    // layers whose dropout is BERNOULLI - never BERNOULLI_INVERTED, which has its own function there - in layer order (the
+    // input layer first, the output layer never), per layer [time step][unit], one std::bernoulli_distribution(retention
+    // probability) draw from a std::mt19937 each (Common_Library Random/Bernoulli.hpp); a retention probability of 0 clears
+    // the layer's masks.  The masks then go to the device when there is one.
+    void Dropout_Bernoulli(void)
+    {
+        Solo([&] {
+            bool any = false;
+            for (size_t li = 0; li + 1 < desc_.n_layers; ++li) {
+                const myea_layer_desc &l = desc_.layers[li];
+                if (l.type_dropout != MYEA_DROPOUT_BERNOULLI) continue;
+                const size_t first = l.first_mask_index;
+                const size_t end = li + 1 < desc_.n_layers ? desc_.layers[li + 1].first_mask_index : desc_.total_mask_units;
+                if (end == first) { if (li != 0) Fail("Dropout_Bernoulli", "the layer type is not managed (no activation unit)"); continue; }
+                any = true;
+                const T_ keep = l.dropout_values[0];
+                if (keep != 0.f) {
+                    if (bernoulli_probability_ != keep) { bernoulli_probability_ = keep; bernoulli_.param(std::bernoulli_distribution::param_type(keep)); }
+                    for (size_t i = first; i < end; ++i) ptr_array_units_mask_dropout_bernoulli[i] = bernoulli_(bernoulli_generator_);
+                } else {
+                    for (size_t i = first; i < end; ++i) ptr_array_units_mask_dropout_bernoulli[i] = false;
+                }
+            }
+            if (any && net_) Copy__Dropout_Mask__Host_To_Device();
+        });
+    }
+    // Base::Seed of the reference's generator classes
+    void Set__Seed__Dropout_Bernoulli(unsigned int seed) { bernoulli_generator_.seed(seed); bernoulli_.reset(); }
 
     // Compute__Loss (Neural_Network__Compute__Loss__Loop.cpp:22): loss / accuracy of the last forward pass, no delta
     void Compute__Loss(size_t batch_size_received, T_ const *const *ptr_array_desireds_outputs)
@@ -427,6 +497,39 @@ public:
 private:
     myea_net_desc desc_;
     myea_hip_net *net_ = nullptr;
+    std::vector<Layer> layers_;
+    std::mt19937 bernoulli_generator_{5489u};
+    std::bernoulli_distribution bernoulli_{0.5};
+    T_ bernoulli_probability_ = 0.5f;
+    myea_hyper pushed_;              // what the device object last received from the public fields
+    bool pushed_valid_ = false;
+    unsigned int pushed_state_ = 0;
+
+    // one thread of the calling team runs f, the others wait for it (see the step entry points)
+    template <class F>
+    static void Solo(F &&f)
+    {
+#ifdef _OPENMP
+#pragma omp barrier
+#pragma omp master
+        f();
+#pragma omp barrier
+#else
+        f();
+#endif
+    }
+    void RefreshLayers()
+    {
+        layers_.assign(desc_.n_layers, Layer());
+        for (size_t i = 0; i < desc_.n_layers; ++i) {
+            const myea_layer_desc &l = desc_.layers[i];
+            layers_[i].type_layer = l.type_layer; layers_[i].type_dropout = l.type_dropout; layers_[i].use_bidirectional = l.use_bidirectional != 0;
+            for (int k = 0; k < 3; ++k) layers_[i].dropout_values[k] = l.dropout_values[k];
+        }
+        total_layers = desc_.n_layers;
+        ptr_array_layers = layers_.empty() ? nullptr : layers_.data();
+        ptr_last_layer = ptr_array_layers ? ptr_array_layers + total_layers : nullptr;
+    }
     std::vector<T_> rows_;
     std::vector<std::vector<T_>> norm_means_averages_, norm_variances_averages_;   // per layer [T][units], from a checkpoint
     T_ r_mean_desired_ = 0.f, r_mean_predicted_ = 0.f;
@@ -440,13 +543,14 @@ private:
         return true;
     }
     // a structural change after Set__HIP needs a new device object, as a changed Layer does in the reference's CUDA path
-    bool Dirty() { if (net_) { myea_hip_destroy(net_); net_ = nullptr; } return true; }
+    bool Dirty() { if (net_) { myea_hip_destroy(net_); net_ = nullptr; } pushed_valid_ = false; RefreshLayers(); return true; }
     void Deallocate()
     {
         if (net_) { myea_hip_destroy(net_); net_ = nullptr; }
         delete[] ptr_array_parameters; ptr_array_parameters = nullptr;
         delete[] ptr_array_units_mask_dropout_bernoulli; ptr_array_units_mask_dropout_bernoulli = nullptr;
         norm_means_averages_.clear(); norm_variances_averages_.clear();
+        layers_.clear(); ptr_array_layers = nullptr; ptr_last_layer = nullptr; total_layers = 0; pushed_valid_ = false;
     }
     bool Relayout(const char *fn)
     {
@@ -464,6 +568,7 @@ private:
         delete[] ptr_array_units_mask_dropout_bernoulli;
         ptr_array_units_mask_dropout_bernoulli = new bool[desc_.total_mask_units ? desc_.total_mask_units : 1];
         for (size_t i = 0; i < desc_.total_mask_units; ++i) ptr_array_units_mask_dropout_bernoulli[i] = true;
+        RefreshLayers();
         return true;
     }
     void PullState()
@@ -473,11 +578,12 @@ private:
         optimizer_time_step = h.optimizer_time_step; epoch_time_step = h.epoch_time_step; adam_previous_beta2 = h.adam_previous_beta2;
         loss_rprop = h.loss_rprop; previous_loss_rprop = h.previous_loss_rprop;
         warm_restarts_maximum_learning_rate = h.warm_restarts_maximum_learning_rate; warm_restarts_T_i = h.warm_restarts_T_i;
+        // the device object and the public fields agree again: nothing to push until the caller writes a field
+        if (pushed_valid_) { std::memset(&pushed_, 0, sizeof(pushed_)); AssignFields(pushed_); }
     }
-    bool PushFields(const char *fn)
+    // the public fields written into a myea_hyper
+    void AssignFields(myea_hyper &h) const
     {
-        myea_hyper h;
-        if (myea_hip_get_hyper(net_, &h) != MYEA_OK) return Fail(fn, myea_hip_last_error());
         h.type_optimizer_function = type_optimizer_function; h.type_loss_function = type_loss_function; h.type_accuracy_function = type_accuracy_function;
         h.use_Nesterov = use_Nesterov; h.use_adam_bias_correction = use_adam_bias_correction; h.use_clip_gradient = use_clip_gradient;
         h.learning_rate = learning_rate; h.learning_rate_final = learning_rate_final; h.learning_momentum = learning_momentum; h.learning_gamma = learning_gamma;
@@ -496,8 +602,28 @@ private:
         h.optimizer_time_step = optimizer_time_step; h.epoch_time_step = epoch_time_step; h.adam_previous_beta2 = adam_previous_beta2;
         h.loss_rprop = loss_rprop; h.previous_loss_rprop = previous_loss_rprop;
         h.warm_restarts_maximum_learning_rate = warm_restarts_maximum_learning_rate; h.warm_restarts_T_i = warm_restarts_T_i;
-        if (myea_hip_set_hyper(net_, &h) != MYEA_OK) return Fail(fn, myea_hip_last_error());
-        return Ok(fn, myea_hip_set_state_propagation(net_, type_state_propagation));
+    }
+    // The public fields go to the device object when one of them differs from what it last received (a step function is
+    // called four times per batch; the fields change between epochs at most).  Fields of the library's state that this class
+    // does not hold are read back first, so a push never overwrites them.
+    bool PushFields(const char *fn)
+    {
+        myea_hyper want;
+        std::memset(&want, 0, sizeof(want));
+        AssignFields(want);
+        if (!pushed_valid_ || std::memcmp(&want, &pushed_, sizeof(want)) != 0) {
+            myea_hyper h;
+            if (myea_hip_get_hyper(net_, &h) != MYEA_OK) return Fail(fn, myea_hip_last_error());
+            AssignFields(h);
+            if (myea_hip_set_hyper(net_, &h) != MYEA_OK) return Fail(fn, myea_hip_last_error());
+            pushed_ = want;
+        }
+        if (!pushed_valid_ || pushed_state_ != type_state_propagation) {
+            if (!Ok(fn, myea_hip_set_state_propagation(net_, type_state_propagation))) return false;
+            pushed_state_ = type_state_propagation;
+        }
+        pushed_valid_ = true;
+        return true;
     }
     bool Flatten(const char *fn, size_t B, T_ const *const *rows, size_t row)
     {

@@ -43,7 +43,7 @@ def build(verbose=False):
     # the C++ adaptor's check programs (host code only; link the C ABI)
     root = os.path.dirname(HERE)
     for name in ("adaptor_check", "dataset_check", "checkpoint_check"):
-        _run(["g++", "-O2", "-std=c++17", "-Wall", os.path.join(root, "tests", "cpp", name + ".cpp"), "-o",
+        _run(["g++", "-O2", "-std=c++17", "-Wall", "-fopenmp", os.path.join(root, "tests", "cpp", name + ".cpp"), "-o",
               os.path.join(root, "tests", "cpp", name), "-L" + CSRC, "-lmyea_hip", "-Wl,-rpath," + CSRC,
               "-Wl,-rpath,$ORIGIN/../../myea_amd/csrc"])
     return LIB

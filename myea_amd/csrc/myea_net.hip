@@ -1416,8 +1416,8 @@ int myea_hip_set_state_propagation(myea_hip_net *n, uint32_t s)
 {
     NET_OR_FAIL(n);
     if (s > MYEA_STATE_TRAINING) { myea::set_last_error("state propagation %u is not on this path", s); return MYEA_E_UNSUPPORTED; }
+    if (n->net.state != s) ++n->net.mask_epoch;   // the dropout multipliers depend on the state
     n->net.state = s;
-    ++n->net.mask_epoch;   // the dropout multipliers depend on the state
     return MYEA_OK;
 }
 

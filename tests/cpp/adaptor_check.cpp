@@ -2,9 +2,13 @@
 // `Neural_Network` (Compile -> Set__* -> Set__HIP -> the 4-call step loop + Update_Parameter, cf.
 // Neural_Network_Launcher_Windows/Source_Files/debug.cpp:481-1555 and Neural_Network/Dataset.cpp:645-658).
 // usage: adaptor_check <dir> <kind>   reads <dir>/{w,x,y,mask}.bin, writes <dir>/{params,grad}.bin and prints the loss.
+//        adaptor_check <dir> dropout  host only: Dropout_Bernoulli's draws against the same draws made here.
+// The step loop runs inside `#pragma omp parallel`, every thread of the team calling the step members, as the reference's
+// Dataset::Train_Batch_BP does (Dataset.cpp:645-658); built with -fopenmp.
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <random>
 #include <string>
 #include <vector>
 
@@ -37,6 +41,40 @@ int main(int argc, char **argv)
     const std::string dir = argv[1], kind = argv[2];
     Neural_Network_HIP nn;
     size_t B, T, n_in, n_out, steps = 3;
+    if (kind == "dropout") {
+        // FC 10 (Bernoulli .8 on the inputs) -> 12 (Bernoulli .6) -> 9 (inverted .5) -> 7 (Bernoulli, retention 0) -> 4, T = 3
+        Layer_Parameters layers[5];
+        for (auto &l : layers) l.type_layer = MYEA_LAYER_FULLY_CONNECTED;
+        const size_t units[5] = {10, 12, 9, 7, 4};
+        for (int i = 0; i < 5; ++i) layers[i].unit_parameters[0] = units[i];
+        T = 3;
+        if (!nn.Update__Batch_Size(2) || !nn.Compile(5, T, MYEA_NETWORK_RECURRENT, layers)) return 1;
+        T_ k0[2] = {0.8f, 0.f}, k1[2] = {0.6f, 0.f}, k2[2] = {0.5f, 0.f}, k3[2] = {0.f, 0.f};
+        if (!nn.Set__Dropout(0, MYEA_DROPOUT_BERNOULLI, k0) || !nn.Set__Dropout(1, MYEA_DROPOUT_BERNOULLI, k1) ||
+            !nn.Set__Dropout(2, MYEA_DROPOUT_BERNOULLI_INVERTED, k2) || !nn.Set__Dropout(3, MYEA_DROPOUT_BERNOULLI, k3)) return 1;
+        if (nn.total_layers != 5 || nn.ptr_last_layer != nn.ptr_array_layers + 5 || nn.ptr_array_layers[2].type_dropout != MYEA_DROPOUT_BERNOULLI_INVERTED) return 1;
+        const size_t total = (10 + 12 + 9 + 7 + 4) * T;
+        if (nn.Get__Descriptor().total_mask_units != total) { std::printf("mask units %llu\n", (unsigned long long)nn.Get__Descriptor().total_mask_units); return 1; }
+        nn.Set__Seed__Dropout_Bernoulli(1234u);
+        nn.Dropout_Bernoulli();
+        // the same draws, made here: layer order, [time step][unit], the distribution re-parameterised when the probability changes
+        std::mt19937 gen(1234u);
+        std::bernoulli_distribution dist(0.5);
+        std::vector<bool> want(total, true);
+        dist.param(std::bernoulli_distribution::param_type(0.8f));
+        for (size_t i = 0; i < 10 * T; ++i) want[i] = dist(gen);
+        dist.param(std::bernoulli_distribution::param_type(0.6f));
+        for (size_t i = 0; i < 12 * T; ++i) want[10 * T + i] = dist(gen);
+        for (size_t i = 0; i < 7 * T; ++i) want[(10 + 12 + 9) * T + i] = false;     // retention 0: all dropped, no draw
+        size_t kept0 = 0;
+        for (size_t i = 0; i < total; ++i) {
+            if (nn.ptr_array_units_mask_dropout_bernoulli[i] != want[i]) { std::printf("mask %zu differs\n", i); return 1; }
+            if (i < 10 * T && want[i]) ++kept0;
+        }
+        if (kept0 == 0 || kept0 == 10 * T) return 1;
+        std::printf("dropout ok\n");
+        return 0;
+    }
     if (kind == "mlp") {  // FC 20 -> 32 (BN before, ReLU, inverted dropout .5) -> 24 tanh -> 6 softmax, Nesterov
         B = 16; T = 1; n_in = 20; n_out = 6;
         Layer_Parameters layers[4];
@@ -98,16 +136,26 @@ int main(int argc, char **argv)
     std::vector<const float *> xr(B), yr(B);
     for (size_t b = 0; b < B; ++b) { xr[b] = x.data() + b * T * n_in; yr[b] = y.data() + b * T * n_out; }
     std::vector<float> grad(nn.total_parameters);
+    int failed = 0;
+    // every thread of the team walks the loop and makes the calls; the class lets one of them through
+#pragma omp parallel num_threads(3)
     for (size_t s = 0; s < steps; ++s) {
+#pragma omp barrier
+#pragma omp master
         nn.Reset__Loss();
         nn.Forward_Pass(B, xr.data());
         nn.Compute__Error(B, yr.data());
         nn.Backward_Pass(B);
-        nn.Update_Derivative_Weight(B);
-        if (s + 1 == steps && !nn.Copy__Derivatives_Parameters__Device_To_Host(grad.data())) return 1;
-        std::printf("step %zu loss %.9g\n", s, (double)nn.Get__Loss());
+        nn.Update_Derivative_Weight(B, nn.ptr_array_layers + 1, nn.ptr_last_layer);
+#pragma omp barrier
+#pragma omp master
+        {
+            if (s + 1 == steps && !nn.Copy__Derivatives_Parameters__Device_To_Host(grad.data())) failed = 1;
+            std::printf("step %zu loss %.9g\n", s, (double)nn.Get__Loss());
+        }
         nn.Update_Parameter(B, B);
     }
+    if (failed) return 1;
     if (!nn.Copy__Parameters__Device_To_Host()) return 1;
     write_f32(dir + "/params.bin", nn.ptr_array_parameters, nn.total_parameters);
     write_f32(dir + "/grad.bin", grad.data(), grad.size());

@@ -170,3 +170,16 @@ def test_struct_sizes_match_the_header():
     d = oracle_desc([dict(units=3)] + [dict(units=2, activation="TANH")] * 63, 1)
     assert d.n_layers == 64 and d.layers[63].first_bias_connection_index == d.total_weights + 2 * 62
     assert C.sizeof(mb.LayerDesc) == 128 and C.sizeof(mb.Hyper) == 42 * 4 and C.sizeof(mb.LossState) == 64
+
+
+def test_adaptor_dropout_bernoulli_draws_on_the_host():
+    """Neural_Network_HIP::Dropout_Bernoulli (host only, no device object): BERNOULLI layers get new draws in the reference's
+    order from a std::mt19937 / std::bernoulli_distribution pair, BERNOULLI_INVERTED layers keep their masks, a retention
+    probability of 0 clears the layer (NN/Neural_Network__Dropout__Bernoulli__Loop.cpp:33-97).  The check program makes the same
+    draws itself and compares."""
+    import subprocess
+    binary = os.path.join(ROOT, "tests", "cpp", "adaptor_check")
+    if not os.path.exists(binary):
+        pytest.skip("tests/cpp/adaptor_check is not built (python -m myea_amd.build)")
+    out = subprocess.run([binary, "/tmp", "dropout"], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0 and "dropout ok" in out.stdout, out.stdout + out.stderr
