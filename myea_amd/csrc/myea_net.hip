@@ -1186,17 +1186,42 @@ int Net::set_unit_activations(size_t li, const uint32_t *types, const float *ste
 // Update_Parameter__OpenMP (NN/Neural_Network.cpp:4727-4828): [merge: one accumulator here] -> clip by global norm
 // over all P (NN/Neural_Network__Clip_Gradient.cpp:81-94) -> optimizer.  The clip scale is applied inside the
 // optimizer's gradient read instead of a separate pass over the gradient.
-// Clear_Optimizer (NN/Train.cpp:128-263): state vectors to zero (iRPROP steps to rprop_delta_zero, its two losses to the
-// largest float, NosAdam's running sum to 0), optimizer_time_step = 0, epoch_time_step = 1.
+// Clear_Optimizer (NN/Train.cpp:128-263): the state of the CURRENT optimizer only - gradient descent its previous deltas when
+// it has a momentum; iRPROP+ its two losses (to the largest float), previous derivatives, steps (to rprop_delta_zero) and
+// deltas; Adam and AdaBound the two moments, AMSGrad and AMSBound the maximum too, NosAdam the moments and its running sum -
+// then optimizer_time_step = 0, epoch_time_step = 1 whatever the optimizer.
 int Net::clear_optimizer()
 {
     const size_t P = d.total_parameters;
-    for (int k = 0; k < MYEA_STATE_KINDS; ++k)
-        if (k != MYEA_STATE_PREVIOUS_STEPS) MYEA_HIP_TRY(hipMemsetAsync(opt[k], 0, P * sizeof(float), stream));
-    MYEA_TRY(launch_fill(stream, opt[MYEA_STATE_PREVIOUS_STEPS], P, h.rprop_delta_zero));
-    h.loss_rprop = FLT_MAX;
-    h.previous_loss_rprop = FLT_MAX;
-    h.adam_previous_beta2 = 0.f;
+    auto zero = [&](int kind) -> int { MYEA_HIP_TRY(hipMemsetAsync(opt[kind], 0, P * sizeof(float), stream)); return MYEA_OK; };
+    switch (h.type_optimizer_function) {
+    case MYEA_OPTIMIZER_NONE: break;
+    case MYEA_OPTIMIZER_GD:
+        if (h.learning_momentum != 0.f) MYEA_TRY(zero(MYEA_STATE_PREVIOUS_DELTA));
+        break;
+    case MYEA_OPTIMIZER_IRPROP_PLUS:
+        h.loss_rprop = FLT_MAX;
+        h.previous_loss_rprop = FLT_MAX;
+        MYEA_TRY(zero(MYEA_STATE_PREVIOUS_DERIVATIVES));
+        MYEA_TRY(launch_fill(stream, opt[MYEA_STATE_PREVIOUS_STEPS], P, h.rprop_delta_zero));
+        MYEA_TRY(zero(MYEA_STATE_PREVIOUS_DELTA));
+        break;
+    case MYEA_OPTIMIZER_AMSBOUND:
+    case MYEA_OPTIMIZER_AMSGRAD:
+        MYEA_TRY(zero(MYEA_STATE_FIRST_MOMENT)); MYEA_TRY(zero(MYEA_STATE_SECOND_MOMENT)); MYEA_TRY(zero(MYEA_STATE_SECOND_MOMENT_HAT));
+        break;
+    case MYEA_OPTIMIZER_ADABOUND:
+    case MYEA_OPTIMIZER_ADAM:
+        MYEA_TRY(zero(MYEA_STATE_FIRST_MOMENT)); MYEA_TRY(zero(MYEA_STATE_SECOND_MOMENT));
+        break;
+    case MYEA_OPTIMIZER_NOSADAM:
+        MYEA_TRY(zero(MYEA_STATE_FIRST_MOMENT)); MYEA_TRY(zero(MYEA_STATE_SECOND_MOMENT));
+        h.adam_previous_beta2 = 0.f;
+        break;
+    default:
+        std::fprintf(stderr, "Clear_Optimizer: ERROR: Can not reset the optimizer parameters with (%u) as the current optimizer.\n", h.type_optimizer_function);
+        break;
+    }
     h.optimizer_time_step = 0.f;
     h.epoch_time_step = 1.f;
     return MYEA_OK;

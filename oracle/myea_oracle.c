@@ -253,6 +253,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
     n->parameters = zalloc(P);
     n->gradient = zalloc(P);
     for (int k = 0; k < MYEA_STATE_KINDS; ++k) n->opt[k] = zalloc(P);
+    for (size_t i = 0; i < P; ++i) n->opt[MYEA_STATE_PREVIOUS_STEPS][i] = n->h.rprop_delta_zero;   /* the iRPROP steps start at delta zero */
     n->masks = (uint8_t *)malloc(desc->total_mask_units ? desc->total_mask_units : 1);
     memset(n->masks, 1, desc->total_mask_units ? desc->total_mask_units : 1); /* NN/Neural_Network__Allocate.cpp:386-410: all true */
     /* scales start at 1, shifts at 0 (NN/Neural_Network__Allocate.cpp:2395-2401 and the scale fill) */
@@ -438,16 +439,41 @@ float *myea_oracle_dropout_noise(myea_oracle_net *n, size_t li, size_t *count)
 uint8_t *myea_oracle_zoneout_masks(myea_oracle_net *n, size_t *count) { if (count) *count = n->zoneout_count; return n->zoneout; }
 uint8_t *myea_oracle_masks(myea_oracle_net *n) { return n->masks; }
 
-/* Clear_Optimizer NN/Train.cpp:128-263: state vectors to zero (iRPROP steps to rprop_delta_zero, its two losses to the
- * largest float, NosAdam's running beta2 sum to 0), optimizer_time_step = 0, epoch_time_step = 1 */
+/* Clear_Optimizer NN/Train.cpp:128-263: a switch on the current optimizer - only ITS state is cleared (:134-258) - then
+ * optimizer_time_step = 0, epoch_time_step = 1 for all (:260-261) */
 static void clear_optimizer(myea_oracle_net *n)
 {
-    size_t P = n->d.total_parameters;
-    for (int k = 0; k < MYEA_STATE_KINDS; ++k) memset(n->opt[k], 0, P * sizeof(float));
-    for (size_t i = 0; i < P; ++i) n->opt[MYEA_STATE_PREVIOUS_STEPS][i] = n->h.rprop_delta_zero;
-    n->h.loss_rprop = FLT_MAX;
-    n->h.previous_loss_rprop = FLT_MAX;
-    n->h.adam_previous_beta2 = 0.f;
+    size_t P = n->d.total_parameters, bytes = P * sizeof(float);
+    switch (n->h.type_optimizer_function) {
+    case MYEA_OPTIMIZER_NONE: break;
+    case MYEA_OPTIMIZER_GD:                                    /* :136-143 */
+        if (n->h.learning_momentum != 0.f) memset(n->opt[MYEA_STATE_PREVIOUS_DELTA], 0, bytes);
+        break;
+    case MYEA_OPTIMIZER_IRPROP_PLUS:                           /* :166-198 */
+        n->h.loss_rprop = FLT_MAX;
+        n->h.previous_loss_rprop = FLT_MAX;
+        memset(n->opt[MYEA_STATE_PREVIOUS_DERIVATIVES], 0, bytes);
+        for (size_t i = 0; i < P; ++i) n->opt[MYEA_STATE_PREVIOUS_STEPS][i] = n->h.rprop_delta_zero;
+        memset(n->opt[MYEA_STATE_PREVIOUS_DELTA], 0, bytes);
+        break;
+    case MYEA_OPTIMIZER_AMSBOUND:
+    case MYEA_OPTIMIZER_AMSGRAD:                               /* :201-223 */
+        memset(n->opt[MYEA_STATE_FIRST_MOMENT], 0, bytes);
+        memset(n->opt[MYEA_STATE_SECOND_MOMENT], 0, bytes);
+        memset(n->opt[MYEA_STATE_SECOND_MOMENT_HAT], 0, bytes);
+        break;
+    case MYEA_OPTIMIZER_ADABOUND:
+    case MYEA_OPTIMIZER_ADAM:                                  /* :224-240 */
+        memset(n->opt[MYEA_STATE_FIRST_MOMENT], 0, bytes);
+        memset(n->opt[MYEA_STATE_SECOND_MOMENT], 0, bytes);
+        break;
+    case MYEA_OPTIMIZER_NOSADAM:                               /* :241-257 */
+        memset(n->opt[MYEA_STATE_FIRST_MOMENT], 0, bytes);
+        memset(n->opt[MYEA_STATE_SECOND_MOMENT], 0, bytes);
+        n->h.adam_previous_beta2 = 0.f;
+        break;
+    default: break;
+    }
     n->h.optimizer_time_step = 0.f;
     n->h.epoch_time_step = 1.f;
 }

@@ -165,3 +165,12 @@ def test_normalized_weight_decay_needs_the_training_set_size():
     assert gpu.get_hyper().optimizer_time_step == 0
     gpu.Update_Parameter(4, 4)
     assert gpu.get_hyper().optimizer_time_step == 1
+
+
+def test_clear_optimizer_touches_the_current_optimizers_state_only_on_the_gpu():
+    from tests.test_oracle_optimizers import SPECS, check_clear_optimizer_touches_the_current_optimizers_state_only
+
+    def make(**kw):
+        desc = mb.make_desc(SPECS, 2)
+        return desc, mb.HipNetwork(desc, mb.default_hyper(**kw))
+    check_clear_optimizer_touches_the_current_optimizers_state_only(make)

@@ -186,3 +186,39 @@ def test_adam_bias_corrected_rate_is_evaluated_in_float():
     assert any(not np.array_equal(a, b) for a, b in zip(in_float, in_double)), "float and double rates coincide on this data: the test pins nothing"
     for k in range(10):
         assert np.array_equal(got[k], in_float[k]), "step %d: the oracle's rate is not the float expression" % (k + 1)
+
+
+def check_clear_optimizer_touches_the_current_optimizers_state_only(make_net):
+    """Clear_Optimizer (NN/Train.cpp:128-263) switches on the optimizer: gradient descent with a momentum clears its previous
+    deltas and nothing else; NosAdam its two moments and its running sum; iRPROP+ its losses, derivatives, steps and deltas.
+    The step counters restart for all."""
+    S = mb.OPT_STATE
+    for kind, kw, cleared, kept in (
+            ("GD", dict(learning_momentum=0.9), ["PREVIOUS_DELTA"], ["FIRST_MOMENT", "SECOND_MOMENT", "SECOND_MOMENT_HAT", "PREVIOUS_DERIVATIVES"]),
+            ("GD", dict(learning_momentum=0.0), [], ["PREVIOUS_DELTA", "FIRST_MOMENT"]),
+            ("ADAM", {}, ["FIRST_MOMENT", "SECOND_MOMENT"], ["SECOND_MOMENT_HAT", "PREVIOUS_DELTA"]),
+            ("AMSGRAD", {}, ["FIRST_MOMENT", "SECOND_MOMENT", "SECOND_MOMENT_HAT"], ["PREVIOUS_DELTA", "PREVIOUS_DERIVATIVES"]),
+            ("NOSADAM", {}, ["FIRST_MOMENT", "SECOND_MOMENT"], ["SECOND_MOMENT_HAT"]),
+            ("IRPROP_PLUS", dict(rprop_delta_zero=0.07), ["PREVIOUS_DERIVATIVES", "PREVIOUS_DELTA"], ["FIRST_MOMENT", "SECOND_MOMENT"])):
+        desc, net = make_net(type_optimizer_function=mb.OPTIMIZER[kind], **kw)
+        P = desc.total_parameters
+        for name in S:
+            net.upload_optimizer_state(S[name], np.full(P, 2.0, dtype=np.float32))
+        h = net.get_hyper()
+        h.loss_rprop, h.previous_loss_rprop, h.adam_previous_beta2, h.optimizer_time_step, h.epoch_time_step = 3.0, 4.0, 5.0, 6.0, 7.0
+        net.set_hyper(h)
+        net.Clear_Training_Arrays()
+        for name in cleared:
+            assert np.all(net.download_optimizer_state(S[name]) == 0), (kind, name)
+        for name in kept:
+            assert np.all(net.download_optimizer_state(S[name]) == 2.0), (kind, name)
+        steps = net.download_optimizer_state(S["PREVIOUS_STEPS"])
+        assert np.all(steps == (np.float32(0.07) if kind == "IRPROP_PLUS" else 2.0)), kind
+        h = net.get_hyper()
+        assert (h.optimizer_time_step, h.epoch_time_step) == (0.0, 1.0)
+        assert (h.loss_rprop, h.previous_loss_rprop) == ((np.finfo(np.float32).max,) * 2 if kind == "IRPROP_PLUS" else (3.0, 4.0)), kind
+        assert h.adam_previous_beta2 == (0.0 if kind == "NOSADAM" else 5.0), kind
+
+
+def test_clear_optimizer_touches_the_current_optimizers_state_only():
+    check_clear_optimizer_touches_the_current_optimizers_state_only(_net)
