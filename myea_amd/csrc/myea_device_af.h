@@ -77,8 +77,9 @@ __device__ __forceinline__ float af_derive(int type, float q, float st, float v)
     case MYEA_AF_ELLIOT_SYMMETRIC: return st / ((1.f + fabsf(q)) * (1.f + fabsf(q)));
     case MYEA_AF_GAUSSIAN: return -2.f * q * v * st * st;
     case MYEA_AF_GAUSSIAN_SYMMETRIC: return -2.f * q * (v + 1.f) * st * st;
-    case MYEA_AF_ISRU: { float r = v / q; return st * (r * r * r); }
-    case MYEA_AF_ISRLU: { float r = v / q; return q < 0.f ? st * (r * r * r) : st; }
+    // pow(float, 3u) there promotes to double and the cube is rounded to float once (Activation_Functions.hpp:86, 90)
+    case MYEA_AF_ISRU: { const double r = (double)(v / q); return st * (float)(r * r * r); }
+    case MYEA_AF_ISRLU: { const double r = (double)(v / q); return q < 0.f ? st * (float)(r * r * r) : st; }
     case MYEA_AF_LINEAR:
     case MYEA_AF_LINEAR_PIECE:
     case MYEA_AF_LINEAR_PIECE_SYMMETRIC: return st;

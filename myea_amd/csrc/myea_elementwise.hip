@@ -5,6 +5,8 @@
 // batch are two-stage and deterministic (per-chunk partial sums in a fixed order, no float atomics).
 //
 // NN/ = Neural_Network_Library_Windows/Source_Files/Neural_Network/.
+#include <initializer_list>
+
 #include "myea_device_af.h"
 #include "myea_kernels.h"
 #include "myea_reduce.h"
@@ -346,6 +348,142 @@ __global__ __launch_bounds__(kBlock) void bn_forward_apply_kernel(size_t n, BnFo
             if (p.colscale) v *= p.colscale[j];
             p.act_out[i] = v;
         }
+    }
+}
+
+// The "Average" and "Activation function" loops in one launch, from the sums the producing contraction left per block
+// of 32 rows: sums[blk][0][j] = sum of x, sums[blk][1][j] = sum of x * x.  A workgroup owns 64 x V columns (a lane V
+// consecutive ones: V = 4 when H is a multiple of 4) and a slice of the rows; every workgroup finishes the statistics of
+// its columns for itself (a few dozen loads), the workgroups of the first slice store them and move the running averages.
+template <int V>
+__global__ __launch_bounds__(kBlock) void bn_forward_from_sums_kernel(size_t blocks, size_t rows_per_slice, const float *sums, BnForwardParams p)
+{
+    const size_t j0 = ((size_t)blockIdx.x * 64 + (threadIdx.x & 63)) * V;
+    const bool live = j0 < p.H;
+    // every wavefront sums a quarter of the row blocks of the workgroup's columns; the four meet in LDS
+    constexpr int kWaves = kBlock / 64;
+    __shared__ double s_sum[kWaves][64 * V], s_sq[kWaves][64 * V];
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
+    {
+        double smd[V], svd[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) { smd[v] = 0.0; svd[v] = 0.0; }
+        if (live) {
+            for (size_t y = w; y < blocks; y += kWaves) {
+                float a[V], b[V];
+                if (V == 4) { *reinterpret_cast<float4 *>(a) = *reinterpret_cast<const float4 *>(sums + (y * 2 + 0) * p.H + j0); *reinterpret_cast<float4 *>(b) = *reinterpret_cast<const float4 *>(sums + (y * 2 + 1) * p.H + j0); }
+                else { a[0] = sums[(y * 2 + 0) * p.H + j0]; b[0] = sums[(y * 2 + 1) * p.H + j0]; }
+#pragma unroll
+                for (int v = 0; v < V; ++v) { smd[v] += a[v]; svd[v] += b[v]; }
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < V; ++v) { s_sum[w][l * V + v] = smd[v]; s_sq[w][l * V + v] = svd[v]; }
+    }
+    __syncthreads();
+    if (!live) return;
+    float mean[V], var[V], scale[V], shift[V], cs[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const size_t j = j0 + v;
+        double smd = 0.0, svd = 0.0;
+#pragma unroll
+        for (int k = 0; k < kWaves; ++k) { smd += s_sum[k][l * V + v]; svd += s_sq[k][l * V + v]; }   // in wavefront order: every lane gets the same bits
+        const float sm = (float)smd, sv = (float)svd;
+        const float bscale = 1.f / (float)p.rows;
+        mean[v] = sm * bscale;
+        var[v] = sqrtf(sv * bscale - mean[v] * mean[v] + p.epsilon);
+        if (blockIdx.y == 0 && w == 0) {
+            float mavg = p.mean_avg[j];
+            mavg += p.momentum * (mean[v] - mavg);
+            p.mean_avg[j] = mavg;
+            float vavg = p.var_avg[j];
+            vavg += p.momentum * (var[v] - vavg);
+            p.var_avg[j] = vavg;
+            p.mean[j] = mean[v];
+            p.var[j] = var[v];
+        }
+        scale[v] = p.scale[j]; shift[v] = p.shift[j];
+        cs[v] = (p.act_out && p.colscale) ? p.colscale[j] : 1.f;
+    }
+    const size_t r0 = (size_t)blockIdx.y * rows_per_slice, r1 = r0 + rows_per_slice < p.rows ? r0 + rows_per_slice : p.rows;
+    for (size_t r = r0 + (threadIdx.x >> 6); r < r1; r += kBlock / 64) {
+        const size_t i = r * p.H + j0;
+        float x[V], hat[V], y[V], a[V];
+        if (V == 4) *reinterpret_cast<float4 *>(x) = *reinterpret_cast<const float4 *>(p.x + i); else x[0] = p.x[i];
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            hat[v] = (x[v] - mean[v]) / var[v];
+            y[v] = scale[v] * hat[v] + shift[v];
+            a[v] = p.act_out ? af_fire(p.act, y[v]) * cs[v] : 0.f;
+        }
+        if (V == 4) {
+            *reinterpret_cast<float4 *>(p.hats + i) = *reinterpret_cast<const float4 *>(hat);
+            *reinterpret_cast<float4 *>(p.normalizes + i) = *reinterpret_cast<const float4 *>(y);
+            if (p.act_out) *reinterpret_cast<float4 *>(p.act_out + i) = *reinterpret_cast<const float4 *>(a);
+        } else {
+            p.hats[i] = hat[0]; p.normalizes[i] = y[0];
+            if (p.act_out) p.act_out[i] = a[0];
+        }
+    }
+}
+
+// The backward pass's three loops in one launch, from sums[blk][0][j] = sum of dy * hats and sums[blk][1][j] = sum of dy:
+// with hats = (x - mean) / sigma the two other sums of the first loop are these two times -scale / sigma.
+template <int V>
+__global__ __launch_bounds__(kBlock) void bn_backward_from_sums_kernel(size_t blocks, size_t rows_per_slice, const float *sums, BnBackwardParams p)
+{
+    const size_t j0 = ((size_t)blockIdx.x * 64 + (threadIdx.x & 63)) * V;
+    const bool live = j0 < p.H;
+    constexpr int kWaves = kBlock / 64;
+    __shared__ double s_a0[kWaves][64 * V], s_a1[kWaves][64 * V];
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
+    {
+        double a0[V], a1[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) { a0[v] = 0.0; a1[v] = 0.0; }
+        if (live) {
+            for (size_t y = w; y < blocks; y += kWaves) {
+                float a[V], b[V];
+                if (V == 4) { *reinterpret_cast<float4 *>(a) = *reinterpret_cast<const float4 *>(sums + (y * 2 + 0) * p.H + j0); *reinterpret_cast<float4 *>(b) = *reinterpret_cast<const float4 *>(sums + (y * 2 + 1) * p.H + j0); }
+                else { a[0] = sums[(y * 2 + 0) * p.H + j0]; b[0] = sums[(y * 2 + 1) * p.H + j0]; }
+#pragma unroll
+                for (int v = 0; v < V; ++v) { a0[v] += a[v]; a1[v] += b[v]; }
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < V; ++v) { s_a0[w][l * V + v] = a0[v]; s_a1[w][l * V + v] = a1[v]; }
+    }
+    __syncthreads();
+    if (!live) return;
+    float vb[V], scale[V], mean[V], dmean[V], dvar[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const size_t j = j0 + v;
+        double a0 = 0.0, a1 = 0.0;
+#pragma unroll
+        for (int k = 0; k < kWaves; ++k) { a0 += s_a0[k][l * V + v]; a1 += s_a1[k][l * V + v]; }
+        if (blockIdx.y == 0 && w == 0) { p.dscale[j] += (float)a0; p.dshift[j] += (float)a1; }
+        vb[v] = p.var[j]; scale[v] = p.scale[j]; mean[v] = p.mean[j];
+        dmean[v] = (float)a1 * scale[v] * (-1.f / vb[v]);
+        dvar[v] = (float)a0 * scale[v] * (-1.f / vb[v]);
+    }
+    const float bsz = (float)p.rows, bscale = 1.f / (float)p.rows;
+    const size_t r0 = (size_t)blockIdx.y * rows_per_slice, r1 = r0 + rows_per_slice < p.rows ? r0 + rows_per_slice : p.rows;
+    for (size_t r = r0 + (threadIdx.x >> 6); r < r1; r += kBlock / 64) {
+        const size_t i = r * p.H + j0;
+        float dy[V], x[V], dx[V];
+        if (V == 4) { *reinterpret_cast<float4 *>(dy) = *reinterpret_cast<const float4 *>(p.dy + i); *reinterpret_cast<float4 *>(x) = *reinterpret_cast<const float4 *>(p.x + i); }
+        else { dy[0] = p.dy[i]; x[0] = p.x[i]; }
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            float e = dy[v] * scale[v];
+            e *= 1.f / vb[v];
+            e += dvar[v] * ((x[v] - mean[v]) / (bsz * vb[v]));
+            e += dmean[v] * bscale;
+            dx[v] = e;
+        }
+        if (V == 4) *reinterpret_cast<float4 *>(p.dx + i) = *reinterpret_cast<const float4 *>(dx); else p.dx[i] = dx[0];
     }
 }
 
@@ -931,6 +1069,48 @@ int launch_bn_forward_training(hipStream_t s, const BnForwardParams &p, float *s
     MYEA_HIP_TRY(hipGetLastError());
     const size_t n = p.rows * p.H;
     hipLaunchKernelGGL(bn_forward_apply_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, n, p);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+// rows per slice so that the grid has about a thousand workgroups, at least 8 rows each
+static size_t bn_rows_per_slice(size_t rows, size_t colblocks)
+{
+    size_t slices = (1024 + colblocks - 1) / colblocks;
+    if (slices > (rows + 7) / 8) slices = (rows + 7) / 8;
+    if (slices < 1) slices = 1;
+    return (rows + slices - 1) / slices;
+}
+static bool rows_of_float4(size_t H, std::initializer_list<const void *> tensors)
+{
+    if (H % 4) return false;
+    for (const void *t : tensors) if (t && (reinterpret_cast<uintptr_t>(t) & 15u)) return false;
+    return true;
+}
+
+int launch_bn_forward_training_from_sums(hipStream_t s, const BnForwardParams &p, const float *sums, size_t blocks)
+{
+    if (p.H == 0 || p.rows == 0) return MYEA_OK;
+    if (p.renorm || !sums || blocks == 0) { set_last_error("bn_forward_training_from_sums: plain batch normalisation with its column sums only"); return MYEA_E_INVALID; }
+    static_assert(kBlock % 64 == 0, "64 lanes of columns per workgroup");
+    const bool wide = rows_of_float4(p.H, {p.x, p.hats, p.normalizes, p.act_out});
+    const size_t colblocks = (p.H + (wide ? 255 : 63)) / (wide ? 256 : 64), per = bn_rows_per_slice(p.rows, colblocks);
+    const dim3 grid((unsigned)colblocks, (unsigned)((p.rows + per - 1) / per));
+    if (wide) hipLaunchKernelGGL(bn_forward_from_sums_kernel<4>, grid, dim3(kBlock), 0, s, blocks, per, sums, p);
+    else hipLaunchKernelGGL(bn_forward_from_sums_kernel<1>, grid, dim3(kBlock), 0, s, blocks, per, sums, p);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_bn_backward_from_sums(hipStream_t s, const BnBackwardParams &p, const float *sums, size_t blocks)
+{
+    if (p.H == 0 || p.rows == 0) return MYEA_OK;
+    if (p.renorm || !sums || blocks == 0) { set_last_error("bn_backward_from_sums: plain batch normalisation with its column sums only"); return MYEA_E_INVALID; }
+    const bool wide = rows_of_float4(p.H, {p.x, p.dy, p.dx});
+    const size_t colblocks = (p.H + (wide ? 255 : 63)) / (wide ? 256 : 64), per = bn_rows_per_slice(p.rows, colblocks);
+    const dim3 grid((unsigned)colblocks, (unsigned)((p.rows + per - 1) / per));
+    if (wide) hipLaunchKernelGGL(bn_backward_from_sums_kernel<4>, grid, dim3(kBlock), 0, s, blocks, per, sums, p);
+    else hipLaunchKernelGGL(bn_backward_from_sums_kernel<1>, grid, dim3(kBlock), 0, s, blocks, per, sums, p);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

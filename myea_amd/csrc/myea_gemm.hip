@@ -262,6 +262,7 @@ struct GemmDev {
     const float *addend;
     long ld_addend;
     float *col_partials;
+    const float *hats;
     int nbm, nbn;
     int ksplit, kchunk;   // split-K: number of slabs and k's per slab (multiple of BK); slab s writes C + s * slab
     long slab;
@@ -305,7 +306,7 @@ __device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&a
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int row0 = at.m0 + at.wave_m + i * 32 + at.half * 4;
-            float column_sum = 0.f;
+            float column_sum = 0.f, column_sum2 = 0.f;   // per kind: see col_partials
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = row0 + (r >> 2) * 8 + (r & 3);
@@ -316,6 +317,11 @@ __device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&a
                 if (KIND == 1) {
                     v += bias;
                     p.C[o] = v;
+                    {
+#pragma clang fp contract(off)   // as for the derivative's sums below: the same bits from every tile shape
+                        column_sum = column_sum + v;
+                        column_sum2 = column_sum2 + v * v;
+                    }
                     if (CLASS == 1) {
                         const float neg = slope * v;
                         p.aux_out[o] = (v < 0.f ? (relu ? 0.f : neg) : v) * cs;
@@ -336,6 +342,7 @@ __device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&a
                         const float out = v * dv;
                         p.C[o] = out;
                         column_sum = column_sum + out;
+                        if (p.hats) column_sum2 = column_sum2 + out * p.hats[o];
                     }
                 } else if (KIND == 3) {
                     unsafeAtomicAdd(&p.C[o], v);
@@ -343,10 +350,19 @@ __device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&a
                     p.C[o] = v;
                 }
             }
-            if (KIND == 2 && p.col_partials) {
+            if ((KIND == 1 || KIND == 2) && p.col_partials) {
                 const float both = column_sum + __shfl_xor(column_sum, 32);   // the column's other 16 rows of this accumulator
+                const float both2 = column_sum2 + __shfl_xor(column_sum2, 32);
                 const int block_row = at.m0 + at.wave_m + i * 32;
-                if (at.half == 0 && (WHOLE || block_row < p.M)) p.col_partials[(long)(block_row >> 5) * p.N + col] = both;
+                if (at.half == 0 && (WHOLE || block_row < p.M)) {
+                    if (KIND == 2 && !p.hats) {
+                        p.col_partials[(long)(block_row >> 5) * p.N + col] = both;
+                    } else {   // pairs: forward (sum, sum of squares); derivative with hats (sum of C * hats, sum of C)
+                        float *pair = p.col_partials + (long)(block_row >> 5) * 2 * p.N + col;
+                        pair[0] = KIND == 1 ? both : both2;
+                        pair[p.N] = KIND == 1 ? both2 : both;
+                    }
+                }
             }
         }
     }
@@ -615,8 +631,9 @@ static int prepare_gemm(const GemmParams &p, GemmDev &d, bool *vec)
     d.bias = p.bias; d.aux_out = p.aux_out; d.colscale = p.colscale;
     d.pre = p.pre; d.val = p.val; d.act = p.act; d.steep = p.steep;
     d.addend = p.addend; d.ld_addend = p.ld_addend;
-    d.col_partials = p.col_partials;
-    if (p.col_partials && p.epilogue != EPI_FC_DERIVE) { set_last_error("gemm: column partial sums go with the derivative epilogue only"); return MYEA_E_INVALID; }
+    d.col_partials = p.col_partials; d.hats = p.hats;
+    if (p.col_partials && p.epilogue == EPI_NONE) { set_last_error("gemm: column partial sums go with the forward and the derivative epilogue only"); return MYEA_E_INVALID; }
+    if (p.hats && (p.epilogue != EPI_FC_DERIVE || !p.col_partials)) { set_last_error("gemm: hats go with the derivative epilogue's column sums"); return MYEA_E_INVALID; }
     if (p.addend && (p.epilogue == EPI_FC_FORWARD || p.ld_addend < p.N)) { set_last_error("gemm: addend needs EPI_NONE / EPI_FC_DERIVE and ld_addend >= N"); return MYEA_E_INVALID; }
     d.nbm = d.nbn = 0;
     d.ksplit = 1; d.kchunk = p.K > 0 ? p.K : 1; d.slab = 0;

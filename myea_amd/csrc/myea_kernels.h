@@ -45,9 +45,14 @@ struct GemmParams {
     // gradient of a residual block arriving at the same destination); may be null
     const float *addend;
     long ld_addend;
-    // EPI_FC_DERIVE: when not null, [ceil(M / 32)][N] - the column sums of C over each block of 32 rows (the bias gradient's
-    // partial sums, taken from the accumulators on their way out; fixed order, so repeatable); the consumer sums the blocks
+    // When not null, column sums over each block of 32 rows, taken from the accumulators on their way out (fixed order,
+    // so repeatable); the consumer sums the blocks.
+    //   EPI_FC_DERIVE without `hats`: [ceil(M / 32)][N], the sums of C (the bias gradient's partial sums);
+    //   EPI_FC_DERIVE with `hats` ([M][ldc], the normalised values of a batch-normalised layer): [ceil(M / 32)][2][N],
+    //     the sums of C * hats and of C (what the normalisation's backward pass reduces first);
+    //   EPI_FC_FORWARD: [ceil(M / 32)][2][N], the sums of C and of C * C (the batch statistics of a normalisation that follows)
     float *col_partials;
+    const float *hats;
     // split-K (deterministic): slab s of the K range writes its partial product to C + s * split_k_slab; the consumer
     // sums the slabs in order.  Requires EPI_NONE and accumulate == 0.  0 / 1 = off.
     int split_k;
@@ -103,6 +108,9 @@ struct BnForwardParams {
     int act;
 };
 int launch_bn_forward_training(hipStream_t s, const BnForwardParams &p, float *scratch /* >= 128 * H floats */);
+// the same from column sums the producing contraction left ([blocks][2][H]: sums of x and of x * x per block of rows): one
+// launch that finishes the statistics and applies them; plain batch normalisation only (p.renorm == 0)
+int launch_bn_forward_training_from_sums(hipStream_t s, const BnForwardParams &p, const float *sums, size_t blocks);
 int launch_bn_forward_inference(hipStream_t s, size_t rows, size_t H, const float *x, const float *scale, const float *shift,
                                 const float *mean_avg, const float *var_avg, float *normalizes);
 struct BnBackwardParams {
@@ -114,6 +122,9 @@ struct BnBackwardParams {
     int renorm;
 };
 int launch_bn_backward(hipStream_t s, const BnBackwardParams &p, float *scratch /* >= 258 * H floats */);
+// the same from column sums the producing contraction left ([blocks][2][H]: sums of dy * hats and of dy per block of rows);
+// plain batch normalisation only
+int launch_bn_backward_from_sums(hipStream_t s, const BnBackwardParams &p, const float *sums, size_t blocks);
 
 // output-layer delta + loss / accuracy accumulation
 struct ErrorParams {

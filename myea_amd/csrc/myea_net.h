@@ -31,6 +31,9 @@ struct DevLayer {
     // bias_partial_batch examples, 0 = the errors were written some other way
     float *bias_partials = nullptr;
     size_t bias_partial_rows = 0, bias_partial_batch = 0;
+    // a batch-normalised dense layer: [ceil(Bmax / 32)][2][H] column sums a contraction leaves for the normalisation's forward
+    // (sum of x, of x * x) and backward pass (sum of dy * hats, of dy); consumed by the launch that follows it
+    float *norm_partials = nullptr;
     // [T][NH]
     float *means = nullptr, *variances = nullptr, *means_averages = nullptr, *variances_averages = nullptr;
     float *r_corrections = nullptr, *d_corrections = nullptr;
@@ -127,8 +130,10 @@ struct Net {
     int refresh_colscale(size_t li, bool *active);
     int forward_fc_layer(size_t li, size_t B);
     // act_out != nullptr (training only): the layer's activation and dropout multiplier ride in the normalisation's last pass
-    int bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training, float *act_out = nullptr, const float *colscale = nullptr);
-    int bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx);
+    // sums / sum_blocks: column sums the contraction that produced x (forward) or dy (backward) left per block of 32 rows
+    int bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training, float *act_out = nullptr, const float *colscale = nullptr,
+                   const float *sums = nullptr, size_t sum_blocks = 0);
+    int bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx, const float *sums = nullptr, size_t sum_blocks = 0);
     int backward_into_layer(size_t li, size_t B);
     int forward_residual_block(size_t ri, size_t B);
     int backward_residual_block(size_t ri, size_t B);

@@ -310,6 +310,7 @@ int Net::create(const myea_net_desc &desc)
         }
         MYEA_TRY(dev_alloc(&o.neuron_errors, sz));  // residual layer: its basic units' errors
         if (layer_is_dense(l) && layer_uses_bias(l) && li + 1 < d.n_layers) MYEA_TRY(dev_alloc(&o.bias_partials, (T * B + 31) / 32 * o.H));
+        if (layer_is_dense(l) && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION) MYEA_TRY(dev_alloc(&o.norm_partials, (B + 31) / 32 * 2 * (o.H > o.NH ? o.H : o.NH)));
         MYEA_HIP_TRY(hipMemset(o.neuron_errors, 0, sz * sizeof(float)));
         if (layer_is_ind_rnn(l)) {
             MYEA_TRY(dev_alloc(&o.pre_afs, sz));
@@ -394,7 +395,7 @@ Net::~Net()
     fr(seg_first); fr(seg_len);
     fr(masks); fr(zoneout_masks);
     for (DevLayer &o : L) {
-        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.bias_partials); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index); fr(o.pre_afs); fr(o.dafs_own); fr(o.noise);
+        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.bias_partials); fr(o.norm_partials); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index); fr(o.pre_afs); fr(o.dafs_own); fr(o.noise);
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
@@ -462,6 +463,9 @@ int Net::forward_fc_layer(size_t li, size_t B)
         const bool fuse_af = !ind && !softmax && !(norm && before) && !o.unit_act && gemm_can_fuse_activation((int)l.type_activation_function);
         g.aux_out = fuse_af ? o.values + roff * H : nullptr;
         g.colscale = (fuse_af && !norm) ? cs : nullptr;
+        // a batch normalisation in front of the activation, training: its column sums leave with the contraction's tiles
+        const bool sums_from_gemm = norm && before && training && o.norm_partials && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H;
+        if (sums_from_gemm) g.col_partials = o.norm_partials;
         prof_begin(0);
         MYEA_TRY(launch_gemm(stream, g));
         prof_end(2.0 * (double)rows * (double)H * (double)In);
@@ -470,7 +474,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
         // training: the activation of a layer normalised first rides in the normalisation's last pass
         const bool af_in_bn = norm && before && training && !ind && !softmax && !o.unit_act;
         if (norm && before) {
-            MYEA_TRY(bn_forward(li, c, rows, cur, training, af_in_bn ? o.values + roff * H : nullptr, cs));
+            MYEA_TRY(bn_forward(li, c, rows, cur, training, af_in_bn ? o.values + roff * H : nullptr, cs, sums_from_gemm ? o.norm_partials : nullptr, (rows + 31) / 32));
             cur = o.normalizes + roff * H;
         }
         if (ind) continue;   // the recurrence and the activation follow for the whole sequence
@@ -517,7 +521,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
     return MYEA_OK;
 }
 
-int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training, float *act_out, const float *colscale)
+int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training, float *act_out, const float *colscale, const float *sums, size_t sum_blocks)
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
@@ -539,7 +543,7 @@ int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool train
     p.act_out = act_out; p.colscale = colscale; p.act = (int)l.type_activation_function;
     // algorithmic bytes: x read once, the normalised values (x-hat) and the scaled and shifted output written once
     prof_begin(kProfNormalization);
-    const int rc = launch_bn_forward_training(stream, p, scratch);
+    const int rc = (sums && !p.renorm) ? launch_bn_forward_training_from_sums(stream, p, sums, sum_blocks) : launch_bn_forward_training(stream, p, scratch);
     prof_end((double)rows * (double)H * sizeof(float) * (act_out ? 4.0 : 3.0));
     return rc;
 }
@@ -850,6 +854,10 @@ int Net::backward_into_layer(size_t li, size_t B)
         } else if (before) {
             g.C = tmp1 + roff * H;
             g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.normalizes + roff * H; g.val = o.values + roff * H;
+            // the sums the normalisation's backward pass starts with leave with the contraction's tiles
+            if (fuse && o.norm_partials && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H) {
+                g.col_partials = o.norm_partials; g.hats = o.hats + roff * H;
+            }
         } else {
             g.C = tmp1 + roff * H;
             g.epilogue = EPI_NONE;
@@ -884,7 +892,8 @@ int Net::backward_into_layer(size_t li, size_t B)
                                               o.unit_act, o.unit_steep, H));
         }
         if (norm && before) {
-            MYEA_TRY(bn_backward(li, c, rows, o.summations + roff * H, tmp1 + roff * H, o.neuron_errors + roff * H));
+            const bool sums_from_gemm = have_gemm && g.col_partials == o.norm_partials && g.col_partials != nullptr;
+            MYEA_TRY(bn_backward(li, c, rows, o.summations + roff * H, tmp1 + roff * H, o.neuron_errors + roff * H, sums_from_gemm ? o.norm_partials : nullptr, (rows + 31) / 32));
         } else if (norm) {
             MYEA_TRY(bn_backward(li, c, rows, o.values + roff * H, tmp1 + roff * H, tmp2 + roff * H));
             MYEA_TRY(launch_activation_derive(stream, (int)l.type_activation_function, l.activation_steepness, rows * H,
@@ -962,7 +971,7 @@ int Net::backward_residual_block(size_t ri, size_t B)
     return MYEA_OK;
 }
 
-int Net::bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx)
+int Net::bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx, const float *sums, size_t sum_blocks)
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
@@ -975,7 +984,7 @@ int Net::bn_backward(size_t li, size_t t, size_t rows, const float *x, const flo
     p.renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
     // algorithmic bytes: dy and x-hat read once, dx written once
     prof_begin(kProfNormalization);
-    const int rc = launch_bn_backward(stream, p, scratch);
+    const int rc = (sums && !p.renorm) ? launch_bn_backward_from_sums(stream, p, sums, sum_blocks) : launch_bn_backward(stream, p, scratch);
     prof_end((double)rows * (double)H * sizeof(float) * 3.0);
     return rc;
 }

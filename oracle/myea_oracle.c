@@ -163,8 +163,9 @@ float myea_oracle_activation_derive(uint32_t type, float q, float st, float v)
     case MYEA_AF_ELLIOT_SYMMETRIC: return st * 1.f / ((1.f + fabsf(q)) * (1.f + fabsf(q)));
     case MYEA_AF_GAUSSIAN: return -2.f * q * v * st * st;
     case MYEA_AF_GAUSSIAN_SYMMETRIC: return -2.f * q * (v + 1.f) * st * st;
-    case MYEA_AF_ISRU: { float r = v / q; return st * (r * r * r); }
-    case MYEA_AF_ISRLU: { float r = v / q; return q < 0.f ? st * (r * r * r) : st; }
+    /* static_cast<T_>(pow(value / summation, 3u)): the float quotient is cubed in double and rounded once (Activation_Functions.hpp:86, 90) */
+    case MYEA_AF_ISRU: { float r = v / q; return st * (float)pow((double)r, 3.0); }
+    case MYEA_AF_ISRLU: { float r = v / q; return q < 0.f ? st * (float)pow((double)r, 3.0) : st; }
     case MYEA_AF_LINEAR:
     case MYEA_AF_LINEAR_PIECE:
     case MYEA_AF_LINEAR_PIECE_SYMMETRIC: return st;
