@@ -524,7 +524,7 @@ private:
         for (size_t i = 0; i < desc_.n_layers; ++i) {
             const myea_layer_desc &l = desc_.layers[i];
             layers_[i].type_layer = l.type_layer; layers_[i].type_dropout = l.type_dropout; layers_[i].use_bidirectional = l.use_bidirectional != 0;
-            for (int k = 0; k < 3; ++k) layers_[i].dropout_values[k] = l.dropout_values[k];
+            for (int k = 0; k < 2; ++k) layers_[i].dropout_values[k] = l.dropout_values[k];
         }
         total_layers = desc_.n_layers;
         ptr_array_layers = layers_.empty() ? nullptr : layers_.data();

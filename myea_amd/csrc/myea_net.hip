@@ -143,7 +143,7 @@ static int check_desc(const myea_net_desc &d)
     if (d.total_parameters != d.total_weights + d.total_bias + 2 * d.total_normalized_units) { set_last_error("descriptor: total_parameters inconsistent"); return MYEA_E_INVALID; }
     if (d.layers[0].type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("descriptor: the input layer must be a fully-connected (unit) layer"); return MYEA_E_INVALID; }
     // residual blocks: members are the block_depth fully-connected layers after the residual layer, a consumer follows
-    bool any_residual = false, any_lstm = false, any_pool = false;
+    bool any_residual = false, any_lstm = false, any_pool = false, any_shakedrop = false;
     uint32_t block_end = 0;  // index of the last member of the block being walked, 0 outside
     std::vector<int> group(d.n_layers, 0);
     for (uint32_t li = 0; li < d.n_layers; ++li) {
@@ -188,12 +188,14 @@ static int check_desc(const myea_net_desc &d)
             if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_SHAKEDROP) { set_last_error("layer %u: a residual layer's dropout is ShakeDrop or none", li); return MYEA_E_UNSUPPORTED; }
             if (l.type_dropout == MYEA_DROPOUT_SHAKEDROP && !(l.dropout_values[0] >= 0.f && l.dropout_values[0] <= 1.f)) { set_last_error("layer %u: ShakeDrop probability %g", li, (double)l.dropout_values[0]); return MYEA_E_INVALID; }
             any_residual = true;
+            if (l.type_dropout == MYEA_DROPOUT_SHAKEDROP) any_shakedrop = true;
             block_end = li + l.block_depth;
         }
         if (l.type_layer == MYEA_LAYER_LSTM) any_lstm = true;
     }
     if (any_pool && any_lstm) { set_last_error("descriptor: pooling layers are on this path for stacks without LSTM layers"); return MYEA_E_UNSUPPORTED; }
-    if (any_residual && (any_lstm || d.number_recurrent_depth != 1)) { set_last_error("descriptor: residual blocks are on this path for feed-forward stacks only"); return MYEA_E_UNSUPPORTED; }
+    if (any_residual && any_lstm) { set_last_error("descriptor: residual blocks are on this path for stacks without LSTM layers"); return MYEA_E_UNSUPPORTED; }
+    if (any_shakedrop && d.number_recurrent_depth != 1) { set_last_error("descriptor: ShakeDrop is on this path for feed-forward stacks only"); return MYEA_E_UNSUPPORTED; }
     for (uint32_t li = 0; li < d.n_layers; ++li) {
         const myea_layer_desc &l = d.layers[li];
         if (l.type_layer == MYEA_LAYER_RESIDUAL) {
@@ -434,6 +436,13 @@ int Net::refresh_colscale(size_t li, bool *active)
 // ---- forward ----------------------------------------------------------------------------------------------
 // Forward_Pass__FC (layer driver), NN/Neural_Network__Forward_Pass__OpenMP.cpp:256-698:
 // GEMM -> bias -> [BN before] -> activation / softmax -> [BN after] -> dropout.
+// MYEA_BN_SUMS_FROM_GEMM=0 in the environment keeps the normalisation's column sums in kernels of their own (for A / B runs)
+static bool bn_sums_from_gemm()
+{
+    static const bool off = [] { const char *e = std::getenv("MYEA_BN_SUMS_FROM_GEMM"); return e && e[0] == '0'; }();
+    return !off;
+}
+
 int Net::forward_fc_layer(size_t li, size_t B)
 {
     const myea_layer_desc &l = d.layers[li];
@@ -464,7 +473,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
         g.aux_out = fuse_af ? o.values + roff * H : nullptr;
         g.colscale = (fuse_af && !norm) ? cs : nullptr;
         // a batch normalisation in front of the activation, training: its column sums leave with the contraction's tiles
-        const bool sums_from_gemm = norm && before && training && o.norm_partials && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H;
+        const bool sums_from_gemm = norm && before && training && o.norm_partials && bn_sums_from_gemm() && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H;
         if (sums_from_gemm) g.col_partials = o.norm_partials;
         prof_begin(0);
         MYEA_TRY(launch_gemm(stream, g));
@@ -628,75 +637,81 @@ int Net::forward_pool_layer(size_t li, size_t B)
 int Net::forward_residual_block(size_t ri, size_t B)
 {
     const myea_layer_desc &r = d.layers[ri];
-    const size_t last = ri + r.block_depth;
+    const size_t last = ri + r.block_depth, T = d.number_recurrent_depth, Bmax = d.batch_size;
     const bool training = state >= MYEA_STATE_TRAINING;
-    bool values_ready = false;  // the member's activation values were written by the previous contraction
-    for (size_t m = ri + 1; m <= last; ++m) {
-        const myea_layer_desc &l = d.layers[m];
-        DevLayer &o = L[m];
-        const size_t In = o.In, H = o.H;
-        const float *cur = layer_outputs(o.prev);
-        if (layer_uses_norm(l)) {
-            MYEA_TRY(bn_forward(m, 0, B, cur, training));
-            cur = o.normalizes;
-        }
-        if (o.group == 2) {
-            if (!values_ready) {
-                bool drop = false;
-                MYEA_TRY(refresh_colscale(m, &drop));
-                MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, B, In, cur, o.values, drop ? o.colscale : nullptr, o.unit_act));
+    // the dropout multipliers of the members, once for all time steps
+    std::vector<char> drops(last + 2, 0);
+    for (size_t m = ri + 1; m <= last; ++m)
+        if (L[m].group == 2) { bool drop = false; MYEA_TRY(refresh_colscale(m, &drop)); drops[m] = drop ? 1 : 0; }
+    // With a recurrent depth the block runs time step by time step on the [T][Bmax][width] tensors (Recurrent__Forward_Pass__Residual,
+    // NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:563-817): every normalisation has its own statistics per time step.
+    for (size_t t = 0; t < T; ++t) {
+        const size_t roff = t * Bmax;
+        bool values_ready = false;  // the member's activation values were written by the previous contraction
+        for (size_t m = ri + 1; m <= last; ++m) {
+            const myea_layer_desc &l = d.layers[m];
+            DevLayer &o = L[m];
+            const size_t In = o.In, H = o.H;
+            const float *cur = layer_outputs(o.prev) + roff * In;
+            if (layer_uses_norm(l)) {
+                MYEA_TRY(bn_forward(m, t, B, cur, training));
+                cur = o.normalizes + roff * In;
             }
-            cur = o.values;
+            if (o.group == 2) {
+                if (!values_ready)
+                    MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, B, In, cur, o.values + roff * In, drops[m] ? o.colscale + t * o.AH : nullptr, o.unit_act));
+                cur = o.values + roff * In;
+            }
+            GemmParams g{};
+            g.A = cur; g.lda = (long)In; g.a_k_contiguous = 1;
+            g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 1;
+            g.C = o.summations + roff * H; g.ldc = (long)H;
+            g.M = (int)B; g.N = (int)H; g.K = (int)In;
+            g.epilogue = EPI_FC_FORWARD;
+            g.bias = layer_uses_bias(l) ? parameters + l.first_bias_connection_index : nullptr;
+            values_ready = false;
+            if (m < last) {
+                const myea_layer_desc &nx = d.layers[m + 1];
+                if (!layer_uses_norm(nx) && !L[m + 1].unit_act && gemm_can_fuse_activation((int)nx.type_activation_function)) {
+                    g.act = (int)nx.type_activation_function;
+                    g.aux_out = L[m + 1].values + roff * H;
+                    g.colscale = drops[m + 1] ? L[m + 1].colscale + t * L[m + 1].AH : nullptr;
+                    values_ready = true;
+                }
+            }
+            prof_begin(0);
+            MYEA_TRY(launch_gemm(stream, g));
+            prof_end(2.0 * (double)B * (double)H * (double)In);
         }
-        GemmParams g{};
-        g.A = cur; g.lda = (long)In; g.a_k_contiguous = 1;
-        g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 1;
-        g.C = o.summations; g.ldc = (long)H;
-        g.M = (int)B; g.N = (int)H; g.K = (int)In;
-        g.epilogue = EPI_FC_FORWARD;
-        g.bias = layer_uses_bias(l) ? parameters + l.first_bias_connection_index : nullptr;
-        values_ready = false;
-        if (m < last) {
-            const myea_layer_desc &nx = d.layers[m + 1];
-            if (!layer_uses_norm(nx) && !L[m + 1].unit_act && gemm_can_fuse_activation((int)nx.type_activation_function)) {
-                bool drop = false;
-                MYEA_TRY(refresh_colscale(m + 1, &drop));
-                g.act = (int)nx.type_activation_function;
-                g.aux_out = L[m + 1].values;
-                g.colscale = drop ? L[m + 1].colscale : nullptr;
-                values_ready = true;
+        DevLayer &o = L[ri];
+        const float *blk = L[last].summations + roff * L[last].H;
+        if (layer_uses_norm(r)) {
+            MYEA_TRY(bn_forward(ri, t, B, blk, training));
+            blk = o.normalizes + roff * o.NH;
+        }
+        // ShakeDrop on the block's output, in place (NN/Neural_Network__Forward_Pass__Loop.cpp:4053-4078); feed-forward stacks only
+        if (r.type_dropout == MYEA_DROPOUT_SHAKEDROP) {
+            const size_t W = o.NH;
+            float *out = const_cast<float *>(blk);
+            if (state == MYEA_STATE_TRAINING) {
+                if (!o.noise_uploaded) {   // masks, forward and backward draws of this pass
+                    MYEA_TRY(launch_dropout_noise(stream, Bmax, o.noise, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
+                    MYEA_TRY(launch_threshold(stream, Bmax, o.noise, r.dropout_values[0]));
+                    MYEA_TRY(launch_dropout_noise(stream, Bmax * W, o.noise + Bmax, 0, -1.f, 1.f, dropout_seed, dropout_stream++));
+                    MYEA_TRY(launch_dropout_noise(stream, Bmax * W, o.noise + Bmax + Bmax * W, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
+                }
+                MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, o.noise, o.noise + Bmax, 1.f));
+            } else {
+                MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, nullptr, nullptr, 1.f - r.dropout_values[0]));
             }
         }
-        prof_begin(0);
-        MYEA_TRY(launch_gemm(stream, g));
-        prof_end(2.0 * (double)B * (double)H * (double)In);
+        const size_t na = o.In, nb = o.NH;
+        const float *src = layer_outputs(o.prev) + roff * na;
+        float *out = o.values + roff * o.H;
+        if (na >= nb) MYEA_TRY(launch_padded_add(stream, B, o.H, src, na, 0, blk, nb, -(long)o.pad, out));
+        else MYEA_TRY(launch_padded_add(stream, B, o.H, blk, nb, 0, src, na, -(long)o.pad, out));
     }
-    DevLayer &o = L[ri];
-    const float *blk = L[last].summations;
-    if (layer_uses_norm(r)) {
-        MYEA_TRY(bn_forward(ri, 0, B, blk, training));
-        blk = o.normalizes;
-    }
-    // ShakeDrop on the block's output, in place (NN/Neural_Network__Forward_Pass__Loop.cpp:4053-4078)
-    if (r.type_dropout == MYEA_DROPOUT_SHAKEDROP) {
-        const size_t Bmax = d.batch_size, W = o.NH;
-        float *out = const_cast<float *>(blk);
-        if (state == MYEA_STATE_TRAINING) {
-            if (!o.noise_uploaded) {   // masks, forward and backward draws of this pass
-                MYEA_TRY(launch_dropout_noise(stream, Bmax, o.noise, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
-                MYEA_TRY(launch_threshold(stream, Bmax, o.noise, r.dropout_values[0]));
-                MYEA_TRY(launch_dropout_noise(stream, Bmax * W, o.noise + Bmax, 0, -1.f, 1.f, dropout_seed, dropout_stream++));
-                MYEA_TRY(launch_dropout_noise(stream, Bmax * W, o.noise + Bmax + Bmax * W, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
-            }
-            MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, o.noise, o.noise + Bmax, 1.f));
-        } else {
-            MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, nullptr, nullptr, 1.f - r.dropout_values[0]));
-        }
-    }
-    const float *src = layer_outputs(o.prev);
-    const size_t na = o.In, nb = o.NH;
-    if (na >= nb) return launch_padded_add(stream, B, o.H, src, na, 0, blk, nb, -(long)o.pad, o.values);
-    return launch_padded_add(stream, B, o.H, blk, nb, 0, src, na, -(long)o.pad, o.values);
+    return MYEA_OK;
 }
 
 // ---- Compute__Error -------------------------------------------------------------------------------------------
@@ -818,7 +833,7 @@ int Net::backward_into_layer(size_t li, size_t B)
         g.B = weights; g.ldb = (long)H; g.b_k_contiguous = 0;
         g.M = (int)rows; g.N = (int)H; g.K = (int)Out;
         g.ldc = (long)H;
-        g.addend = addend; g.ld_addend = ld_addend;
+        g.addend = addend ? addend + roff * (size_t)ld_addend : nullptr; g.ld_addend = ld_addend;
         if (second_direction) {  // the time-reversed direction's share dG2 Win2 first; it joins the main contraction as its addend
             const float *delta2, *weights2;
             size_t out2;
@@ -835,7 +850,7 @@ int Net::backward_into_layer(size_t li, size_t B)
             g.C = o.neuron_errors + roff * H;
             g.epilogue = EPI_NONE;
             if (pool_consumer) { MYEA_TRY(launch_pool_backward(stream, pool_params(gi, rows), on.neuron_errors + roff * on.H, on.pool_index ? on.pool_index + roff * on.H : nullptr, g.C)); continue; }
-            if (!have_gemm) { MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors, shortcut->H, crop, identity, H, 0, g.C)); continue; }
+            if (!have_gemm) { MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors + roff * shortcut->H, shortcut->H, crop, identity + roff * H, H, 0, g.C)); continue; }
             prof_begin(1);
             MYEA_TRY(launch_gemm(stream, g));
             prof_end(2.0 * (double)rows * (double)H * (double)Out);
@@ -855,7 +870,7 @@ int Net::backward_into_layer(size_t li, size_t B)
             g.C = tmp1 + roff * H;
             g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.normalizes + roff * H; g.val = o.values + roff * H;
             // the sums the normalisation's backward pass starts with leave with the contraction's tiles
-            if (fuse && o.norm_partials && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H) {
+            if (fuse && o.norm_partials && bn_sums_from_gemm() && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H) {
                 g.col_partials = o.norm_partials; g.hats = o.hats + roff * H;
             }
         } else {
@@ -881,7 +896,7 @@ int Net::backward_into_layer(size_t li, size_t B)
         } else if (pool_consumer) {
             MYEA_TRY(launch_pool_backward(stream, pool_params(gi, rows), on.neuron_errors + roff * on.H, on.pool_index ? on.pool_index + roff * on.H : nullptr, g.C));
         } else {
-            MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors, shortcut->H, crop, identity, H, 0, g.C));
+            MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors + roff * shortcut->H, shortcut->H, crop, identity + roff * H, H, 0, g.C));
         }
         if (ind) {   // the recurrence follows for the whole sequence
             if (norm && !before) MYEA_TRY(bn_backward(li, c, rows, o.values + roff * H, tmp1 + roff * H, tmp2 + roff * H));
@@ -927,46 +942,54 @@ int Net::backward_residual_block(size_t ri, size_t B)
 {
     const myea_layer_desc &r = d.layers[ri];
     DevLayer &ro = L[ri];
-    const size_t last = ri + r.block_depth;
+    const size_t last = ri + r.block_depth, T = d.number_recurrent_depth, Bmax = d.batch_size;
     const long crop = ro.H > ro.NH ? (long)ro.pad : 0;
     // the perturbed examples' deltas times the backward draws (NN/Neural_Network__Backward_Pass__Loop.cpp:433-443)
     const bool shake = r.type_dropout == MYEA_DROPOUT_SHAKEDROP;
     const float *beta = shake ? ro.noise + d.batch_size + d.batch_size * ro.NH : nullptr;
-    if (layer_uses_norm(r)) {
-        MYEA_TRY(launch_padded_add(stream, B, ro.NH, ro.neuron_errors, ro.H, crop, nullptr, 0, 0, tmp1));
-        if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, tmp1, ro.noise, beta, 1.f));
-        MYEA_TRY(bn_backward(ri, 0, B, L[last].summations, tmp1, L[last].neuron_errors));
-    } else {
-        MYEA_TRY(launch_padded_add(stream, B, ro.NH, ro.neuron_errors, ro.H, crop, nullptr, 0, 0, L[last].neuron_errors));
-        if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, L[last].neuron_errors, ro.noise, beta, 1.f));
-    }
-    for (size_t m = last; m > ri; --m) {
-        const myea_layer_desc &l = d.layers[m];
-        DevLayer &o = L[m];
-        const bool norm = layer_uses_norm(l);
-        if (o.group == 1 && !norm) break;
-        const size_t In = o.In, H = o.H;
-        float *dst = o.group == 2 ? L[m - 1].neuron_errors : o.in_errors;
-        const float *prev_out = layer_outputs(o.prev);
-        GemmParams g{};
-        g.A = o.neuron_errors; g.lda = (long)H; g.a_k_contiguous = 1;
-        g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 0;
-        g.C = norm ? tmp1 : dst; g.ldc = (long)In;
-        g.M = (int)B; g.N = (int)In; g.K = (int)H;
-        g.epilogue = EPI_NONE;
-        bool derive_pending = false;
-        if (o.group == 2) {
-            g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
-            g.pre = norm ? o.normalizes : prev_out;   // Layer::ptr_array_pre_activation_functions
-            g.val = o.values;
-            if (!o.unit_act && !o.unit_steep && gemm_can_fuse_activation(g.act)) g.epilogue = EPI_FC_DERIVE;
-            else derive_pending = true;
+    // time steps in descending order, as the dense layers of a recurrent network are walked; each is on its own
+    for (size_t t = T; t-- > 0;) {
+        const size_t roff = t * Bmax;
+        const float *res_errors = ro.neuron_errors + roff * ro.H;
+        float *last_errors = L[last].neuron_errors + roff * L[last].H;
+        if (layer_uses_norm(r)) {
+            float *tmp = tmp1 + roff * ro.NH;
+            MYEA_TRY(launch_padded_add(stream, B, ro.NH, res_errors, ro.H, crop, nullptr, 0, 0, tmp));
+            if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, tmp, ro.noise, beta, 1.f));
+            MYEA_TRY(bn_backward(ri, t, B, L[last].summations + roff * L[last].H, tmp, last_errors));
+        } else {
+            MYEA_TRY(launch_padded_add(stream, B, ro.NH, res_errors, ro.H, crop, nullptr, 0, 0, last_errors));
+            if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, last_errors, ro.noise, beta, 1.f));
         }
-        prof_begin(1);
-        MYEA_TRY(launch_gemm(stream, g));
-        prof_end(2.0 * (double)B * (double)H * (double)In);
-        if (derive_pending) MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, B * In, g.pre, g.val, g.C, g.C, o.unit_act, o.unit_steep, In));
-        if (norm) MYEA_TRY(bn_backward(m, 0, B, prev_out, tmp1, dst));
+        for (size_t m = last; m > ri; --m) {
+            const myea_layer_desc &l = d.layers[m];
+            DevLayer &o = L[m];
+            const bool norm = layer_uses_norm(l);
+            if (o.group == 1 && !norm) break;
+            const size_t In = o.In, H = o.H;
+            float *dst = (o.group == 2 ? L[m - 1].neuron_errors : o.in_errors) + roff * In;
+            float *tmp = tmp1 + roff * In;
+            const float *prev_out = layer_outputs(o.prev) + roff * In;
+            GemmParams g{};
+            g.A = o.neuron_errors + roff * H; g.lda = (long)H; g.a_k_contiguous = 1;
+            g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 0;
+            g.C = norm ? tmp : dst; g.ldc = (long)In;
+            g.M = (int)B; g.N = (int)In; g.K = (int)H;
+            g.epilogue = EPI_NONE;
+            bool derive_pending = false;
+            if (o.group == 2) {
+                g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
+                g.pre = norm ? o.normalizes + roff * In : prev_out;   // Layer::ptr_array_pre_activation_functions
+                g.val = o.values + roff * In;
+                if (!o.unit_act && !o.unit_steep && gemm_can_fuse_activation(g.act)) g.epilogue = EPI_FC_DERIVE;
+                else derive_pending = true;
+            }
+            prof_begin(1);
+            MYEA_TRY(launch_gemm(stream, g));
+            prof_end(2.0 * (double)B * (double)H * (double)In);
+            if (derive_pending) MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, B * In, g.pre, g.val, g.C, g.C, o.unit_act, o.unit_steep, In));
+            if (norm) MYEA_TRY(bn_backward(m, t, B, prev_out, tmp, dst));
+        }
     }
     return MYEA_OK;
 }

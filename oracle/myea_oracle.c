@@ -275,7 +275,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
                 if (block != 0) { o->group = seen == 0 ? 1 : 2; ++seen; }
             }
             if (l->type_layer == MYEA_LAYER_RESIDUAL) {
-                if (block != 0 || T != 1 || l->block_depth == 0 || li + l->block_depth + 1 >= desc->n_layers || (l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_SHAKEDROP)) { free(n); return MYEA_E_UNSUPPORTED; }
+                if (block != 0 || (T != 1 && l->type_dropout == MYEA_DROPOUT_SHAKEDROP) || l->block_depth == 0 || li + l->block_depth + 1 >= desc->n_layers || (l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_SHAKEDROP)) { free(n); return MYEA_E_UNSUPPORTED; }
                 block = li; seen = 0;
             }
         }
@@ -711,7 +711,7 @@ static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
 /* Forward_Pass__Residual__FC: NN/Neural_Network__Forward_Pass__OpenMP.cpp:4039-4433.  Pre-activation order on the
  * layer's INPUT (fan-in wide): [BN] -> (not for the block's first layer: activation -> dropout) -> weights -> bias.
  * The layer's output is its summation. */
-static void fwd_residual_fc_layer(myea_oracle_net *n, size_t li, size_t B)
+static void fwd_residual_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
 {
     const myea_layer_desc *l = &n->d.layers[li];
     olayer *o = &n->L[li];
@@ -720,36 +720,40 @@ static void fwd_residual_fc_layer(myea_oracle_net *n, size_t li, size_t B)
     int training = n->state >= MYEA_STATE_TRAINING;
     int renorm = l->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
     if (layer_uses_norm(l)) {
-        if (training) fwd_bn_training(n, renorm, 0, B, In, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
-        else fwd_bn_inference(n, 0, B, In, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
+        if (training) fwd_bn_training(n, renorm, t, B, In, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
+        else fwd_bn_inference(n, t, B, In, cur, scale_ptr(n, n->parameters, li), shift_ptr(n, n->parameters, li), o);
         cur = o->normalizes;
     }
     if (o->group == 2) {
-        fwd_af(n, 0, B, In, l->type_activation_function, o->unit_af, cur, o->values);
-        fwd_dropout(n, l, 0, B, In, o->values);
+        fwd_af(n, t, B, In, l->type_activation_function, o->unit_af, cur, o->values);
+        fwd_dropout(n, l, t, B, In, o->values);
         cur = o->values;
     }
-    fwd_fc(n, 0, B, In, H, cur, n->parameters + l->first_connection_index, o->summations);
-    if (layer_uses_bias(l)) fwd_bias(n, 0, B, H, n->parameters + l->first_bias_connection_index, o->summations);
+    fwd_fc(n, t, B, In, H, cur, n->parameters + l->first_connection_index, o->summations);
+    if (layer_uses_bias(l)) fwd_bias(n, t, B, H, n->parameters + l->first_bias_connection_index, o->summations);
 }
 
 /* Forward_Pass__Residual: :3861-3997 (block members, then [block-level BN] on the last member's output, then the
  * shortcut); Forward_Pass__Zero_Padded_Identity: :5158-5240 (A = shortcut source, B = block output; the narrower one is
  * added into the wider one at offset `padding`). */
-static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t B)
+/* With a recurrent depth T > 1 every member and the shortcut run time step by time step on the [T][Bmax][width] tensors
+ * (Recurrent__Forward_Pass__Residual / __Residual__FC / __Zero_Padded_Identity,
+ * NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:563-817: loops over the time steps around the same functions). */
+static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t t, size_t B)
 {
     const myea_layer_desc *r = &n->d.layers[ri];
     olayer *o = &n->L[ri];
     size_t last = ri + r->block_depth, Bmax = n->d.batch_size;
-    for (size_t li = ri + 1; li <= last; ++li) fwd_residual_fc_layer(n, li, B);
+    for (size_t li = ri + 1; li <= last; ++li) fwd_residual_fc_layer(n, li, t, B);
     float *blk = layer_outputs(n, last);
     size_t nb = n->L[last].H, na = n->L[o->prev].H;
     if (layer_uses_norm(r)) {
         int renorm = r->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
-        if (n->state >= MYEA_STATE_TRAINING) fwd_bn_training(n, renorm, 0, B, nb, blk, scale_ptr(n, n->parameters, ri), shift_ptr(n, n->parameters, ri), o);
-        else fwd_bn_inference(n, 0, B, nb, blk, scale_ptr(n, n->parameters, ri), shift_ptr(n, n->parameters, ri), o);
+        if (n->state >= MYEA_STATE_TRAINING) fwd_bn_training(n, renorm, t, B, nb, blk, scale_ptr(n, n->parameters, ri), shift_ptr(n, n->parameters, ri), o);
+        else fwd_bn_inference(n, t, B, nb, blk, scale_ptr(n, n->parameters, ri), shift_ptr(n, n->parameters, ri), o);
         blk = o->normalizes;
     }
+    blk += t * Bmax * nb;   /* the time step's rows, from here on */
     /* ShakeDrop on the block's output, in place (Forward_Pass__Residual__Block, NN/Neural_Network__Forward_Pass__Loop.cpp:4053-4078;
      * Forward_Pass__Dropout__ShakeDrop :5016-5045): strictly in the training state an example is perturbed with probability
      * dropout_values[0], each of its values then times its own U(-1, 1) draw; otherwise every value times 1 - dropout_values[0].
@@ -762,18 +766,19 @@ static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t B)
                 else blk[b * nb + j] *= 1.f - r->dropout_values[0];
             }
     }
-    const float *a = layer_outputs(n, o->prev);
+    const float *a = layer_outputs(n, o->prev) + t * Bmax * na;
+    float *values = o->values + t * Bmax * o->H;
     for (size_t b = 0; b < B; ++b) {
         const float *ar = a + b * na, *br = blk + b * nb;
         if (o->pad == 0) {
-            float *y = o->values + b * na;
+            float *y = values + b * na;
             for (size_t j = 0; j < na; ++j) y[j] = ar[j] + br[j];
         } else if (na > nb) {
-            float *y = o->values + b * na;
+            float *y = values + b * na;
             for (size_t j = 0; j < na; ++j) y[j] = ar[j];
             for (size_t j = 0; j < nb; ++j) y[j + o->pad] += br[j];
         } else {
-            float *y = o->values + b * nb;
+            float *y = values + b * nb;
             for (size_t j = 0; j < nb; ++j) y[j] = br[j];
             for (size_t j = 0; j < na; ++j) y[j + o->pad] += ar[j];
         }
@@ -1159,7 +1164,7 @@ int myea_oracle_forward_pass(myea_oracle_net *n, size_t B, const float *inputs)
         } else if (l->type_layer == MYEA_LAYER_LSTM) {
             fwd_lstm_layer(n, li, B);
         } else if (l->type_layer == MYEA_LAYER_RESIDUAL) {
-            fwd_residual_block(n, li, B);
+            for (size_t t = 0; t < T; ++t) fwd_residual_block(n, li, t, B);
             li += l->block_depth; /* the iterator is left on the block's last member, :3884-3885 */
         } else if (is_pooling(l)) {
             for (size_t t = 0; t < T; ++t) fwd_pooling(n, li, t, B);
@@ -1411,9 +1416,10 @@ static void bwd_gradient_fc(myea_oracle_net *n, size_t li, size_t t, size_t B)
 
 /* Backward_Pass__Residual (7-arg): NN/Neural_Network__Backward_Pass__OpenMP.cpp:1155-1215.  Shortcut gradient:
  * dst (width D) += the residual layer's errors (width R >= D), cropped at `pad` when R > D. */
-static void bwd_residual_shortcut(myea_oracle_net *n, size_t B, size_t R, size_t D, size_t pad, const float *err, float *dst)
+static void bwd_residual_shortcut(myea_oracle_net *n, size_t t, size_t B, size_t R, size_t D, size_t pad, const float *err, float *dst)
 {
-    (void)n;
+    err += t * n->d.batch_size * R;
+    dst += t * n->d.batch_size * D;
     for (size_t b = 0; b < B; ++b) {
         const float *e = err + b * R;
         float *d = dst + b * D;
@@ -1427,22 +1433,22 @@ static void bwd_residual_shortcut(myea_oracle_net *n, size_t B, size_t R, size_t
  * first layer has already reduced its delta to its input side (Backward_Pass__Gradient__Residual__FC), so the producer
  * receives a COPY of those errors; the block's first layer ADDS (its producer also receives the shortcut): its
  * normalisation errors when it is normalised, delta * W otherwise. */
-static void bwd_residual_fc_to_previous(myea_oracle_net *n, size_t gi, size_t B, float *dst)
+static void bwd_residual_fc_to_previous(myea_oracle_net *n, size_t gi, size_t t, size_t B, float *dst)
 {
     const myea_layer_desc *g = &n->d.layers[gi];
     olayer *q = &n->L[gi];
-    size_t Bmax = n->d.batch_size, D = q->In;
-    if (q->group == 2) memcpy(dst, layer_uses_norm(g) ? q->norm_errors : q->af_errors, Bmax * D * sizeof(float));
+    size_t Bmax = n->d.batch_size, D = q->In, at = t * Bmax * D;
+    if (q->group == 2) memcpy(dst + at, (layer_uses_norm(g) ? q->norm_errors : q->af_errors) + at, Bmax * D * sizeof(float));
     else if (layer_uses_norm(g)) {
         for (size_t b = 0; b < B; ++b)
-            for (size_t j = 0; j < D; ++j) dst[b * D + j] += q->norm_errors[b * D + j]; /* Backward_Pass__Identity, :1084-1108 */
-    } else bwd_fc(n, 0, B, q->H, D, q->neuron_errors, n->parameters + g->first_connection_index, dst);
+            for (size_t j = 0; j < D; ++j) dst[at + b * D + j] += q->norm_errors[at + b * D + j]; /* Backward_Pass__Identity, :1084-1108 */
+    } else bwd_fc(n, t, B, q->H, D, q->neuron_errors, n->parameters + g->first_connection_index, dst);
 }
 
 /* Backward_Pass__Gradient__Residual__FC: :822-950 - delta of the summation -> input side: dX = delta * W into the
  * activation errors (block's first layer: into the normalisation errors, or nothing when it is not normalised),
  * then act' on the input-side activation, then [BN backward] over the fan-in wide normalised units. */
-static void bwd_gradient_residual_fc(myea_oracle_net *n, size_t li, size_t B)
+static void bwd_gradient_residual_fc(myea_oracle_net *n, size_t li, size_t t, size_t B)
 {
     const myea_layer_desc *l = &n->d.layers[li];
     olayer *o = &n->L[li];
@@ -1452,26 +1458,26 @@ static void bwd_gradient_residual_fc(myea_oracle_net *n, size_t li, size_t B)
     if (o->group == 2) din = o->af_errors;
     else if (layer_uses_norm(l)) din = o->norm_errors;
     else return;
-    memset(din, 0, Bmax * In * sizeof(float));
-    bwd_fc(n, 0, B, o->H, In, o->neuron_errors, n->parameters + l->first_connection_index, din);
+    memset(din + t * Bmax * In, 0, Bmax * In * sizeof(float));
+    bwd_fc(n, t, B, o->H, In, o->neuron_errors, n->parameters + l->first_connection_index, din);
     const float *prev_out = layer_outputs(n, o->prev);
     if (o->group == 2) {
         const float *pre_af = layer_uses_norm(l) ? o->normalizes : prev_out; /* ptr_array_pre_activation_functions */
-        bwd_df(n, 0, B, In, l->type_activation_function, l->activation_steepness, o->unit_af, o->unit_steep, pre_af, o->values, din, o->af_errors);
+        bwd_df(n, t, B, In, l->type_activation_function, l->activation_steepness, o->unit_af, o->unit_steep, pre_af, o->values, din, o->af_errors);
     }
-    if (layer_uses_norm(l)) bwd_bn(n, renorm, li, 0, B, In, prev_out /* ptr_array_pre_normalization */, din, o->norm_errors);
+    if (layer_uses_norm(l)) bwd_bn(n, renorm, li, t, B, In, prev_out /* ptr_array_pre_normalization */, din, o->norm_errors);
 }
 
 /* Backward_Pass__Residual__Block: :351-452 - the residual layer's errors reach the block's last member through the
  * (cropped) shortcut add, then [block-level BN backward], copied into the member's delta. */
-static void bwd_residual_block_to_last(myea_oracle_net *n, size_t ri, size_t B, float *dst)
+static void bwd_residual_block_to_last(myea_oracle_net *n, size_t ri, size_t t, size_t B, float *dst)
 {
     const myea_layer_desc *r = &n->d.layers[ri];
     olayer *o = &n->L[ri];
-    size_t D = o->NH, Bmax = n->d.batch_size;
+    size_t D = o->NH, Bmax = n->d.batch_size, at = t * Bmax * D;
     float *tmp = dst;
-    if (layer_uses_norm(r)) { tmp = o->norm_errors; memset(tmp, 0, Bmax * D * sizeof(float)); }
-    bwd_residual_shortcut(n, B, o->H, D, o->pad, o->af_errors, tmp);
+    if (layer_uses_norm(r)) { tmp = o->norm_errors; memset(tmp + at, 0, Bmax * D * sizeof(float)); }
+    bwd_residual_shortcut(n, t, B, o->H, D, o->pad, o->af_errors, tmp);
     /* Backward_Pass__Dropout__ShakeDrop (NN/Neural_Network__Backward_Pass__Loop.cpp:433-443, 1050-1078): the perturbed examples'
      * deltas times fresh U(0, 1) draws, one per value */
     if (r->type_dropout == MYEA_DROPOUT_SHAKEDROP) {
@@ -1482,8 +1488,8 @@ static void bwd_residual_block_to_last(myea_oracle_net *n, size_t ri, size_t B, 
     }
     if (layer_uses_norm(r)) {
         int renorm = r->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
-        bwd_bn(n, renorm, ri, 0, B, D, layer_outputs(n, ri + r->block_depth), tmp, o->norm_errors);
-        memcpy(dst, o->norm_errors, Bmax * D * sizeof(float));
+        bwd_bn(n, renorm, ri, t, B, D, layer_outputs(n, ri + r->block_depth), tmp, o->norm_errors);
+        memcpy(dst + at, o->norm_errors + at, Bmax * D * sizeof(float));
     }
 }
 
@@ -1492,13 +1498,15 @@ static void bwd_residual_block_to_last(myea_oracle_net *n, size_t ri, size_t B, 
 static void bwd_gradient_residual(myea_oracle_net *n, size_t ri, size_t B)
 {
     const myea_layer_desc *r = &n->d.layers[ri];
-    size_t Bmax = n->d.batch_size, last = ri + r->block_depth;
+    size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, last = ri + r->block_depth;
     for (size_t li = last; li > ri; --li) {
         olayer *o = &n->L[li];
-        memset(o->neuron_errors, 0, Bmax * o->H * sizeof(float));
-        if (li == last) bwd_residual_block_to_last(n, ri, B, o->neuron_errors);
-        else bwd_residual_fc_to_previous(n, li + 1, B, o->neuron_errors);
-        bwd_gradient_residual_fc(n, li, B);
+        memset(o->neuron_errors, 0, T * Bmax * o->H * sizeof(float));
+        for (size_t t = T; t-- > 0;) {   /* time steps in descending order, like every dense layer of a recurrent network */
+            if (li == last) bwd_residual_block_to_last(n, ri, t, B, o->neuron_errors);
+            else bwd_residual_fc_to_previous(n, li + 1, t, B, o->neuron_errors);
+            bwd_gradient_residual_fc(n, li, t, B);
+        }
     }
 }
 
@@ -1528,13 +1536,13 @@ int myea_oracle_backward_pass(myea_oracle_net *n, size_t B)
             size_t ci = consumers[c];
             const myea_layer_desc *next = &n->d.layers[ci];
             if (is_dense(next)) {
-                if (n->L[ci].group) bwd_residual_fc_to_previous(n, ci, B, dst);
+                if (n->L[ci].group) for (size_t tt = T; tt-- > 0;) bwd_residual_fc_to_previous(n, ci, tt, B, dst);
                 else for (size_t tt = T; tt-- > 0;)
                     bwd_fc(n, tt, B, n->L[ci].H, o->H, n->L[ci].neuron_errors, n->parameters + next->first_connection_index, dst);
             } else if (next->type_layer == MYEA_LAYER_LSTM) {
                 for (size_t tt = 0; tt < T; ++tt) bwd_lstm_to_previous(n, ci, tt, B, dst);
             } else if (next->type_layer == MYEA_LAYER_RESIDUAL) {
-                bwd_residual_shortcut(n, B, n->L[ci].H, o->H, n->L[ci].pad, n->L[ci].af_errors, dst);
+                for (size_t tt = T; tt-- > 0;) bwd_residual_shortcut(n, tt, B, n->L[ci].H, o->H, n->L[ci].pad, n->L[ci].af_errors, dst);
             } else if (is_pooling(next)) {
                 for (size_t tt = 0; tt < T; ++tt) bwd_pooling_to_previous(n, ci, tt, B, dst);
             } else return MYEA_E_UNSUPPORTED;

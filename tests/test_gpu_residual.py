@@ -101,9 +101,69 @@ def test_residual_inference_forward_matches_oracle():
 
 def test_unsupported_residual_shapes_are_refused():
     B = 4
-    for specs, T in (([fc(4), res(1), fc(4), fc(2)], 3),                                                 # recurrent depth
+    for specs, T in (([fc(4), res(1, dropout="SHAKEDROP", keep=0.5), fc(4), fc(2)], 3),                  # ShakeDrop with a recurrent depth
                      ([fc(4), res(1, dropout="BERNOULLI", keep=0.5), fc(4), fc(2)], 1),                  # block-level dropout
                      ([fc(4), res(2), fc(4), fc(4, "SOFTMAX"), fc(2)], 1)):                              # softmax inside a block
         desc = mb.make_desc(specs, B, T, network=mb.NETWORK_FEEDFORWARD)
         with pytest.raises(mb.MyeaError):
             mb.HipNetwork(desc)
+
+
+def _mostly_close(a, b, what, fraction=0.01):
+    """rel 1e-4 / abs 1e-5, except that up to 1 % of the entries may be off by up to 1 %: a batch normalisation over a few
+    dozen examples subtracts nearly equal terms on its way back and amplifies the fp32 rounding of its statistics on either
+    side.  (The feed-forward cases above have a float64 arbiter for such entries; the time-step-by-time-step check against the
+    library's own feed-forward path holds every entry to 1e-4.)"""
+    a, b = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+    err = np.abs(a - b)
+    bad = err > REL * np.abs(b) + ABS
+    assert bad.mean() <= fraction, "%s: %d / %d out of tolerance" % (what, int(bad.sum()), a.size)
+    assert np.all(err[bad] <= 1e-2 * np.abs(b[bad]) + 1e-4), "%s: an entry is off by more than rounding can explain" % what
+
+
+def test_recurrent_depth_is_the_block_time_step_by_time_step_on_the_gpu():
+    """residual blocks with a recurrent depth: against T feed-forward runs of the same library, then against the oracle"""
+    from tests.test_oracle_residual import RECURRENT_SPECS, check_recurrent_depth_is_the_block_time_step_by_time_step
+    check_recurrent_depth_is_the_block_time_step_by_time_step(
+        lambda desc: mb.HipNetwork(desc, mb.default_hyper(type_loss_function=mb.LOSS["MSE"])), lambda specs, B, T: mb.make_desc(specs, B, T), rel=1e-4, abs_=1e-5)
+    T, B, Bmax = 4, 29, 32   # enough examples for well-conditioned batch statistics
+    desc = mb.make_desc(RECURRENT_SPECS, Bmax, T)
+    h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["ADAM"], type_loss_function=mb.LOSS["MSE"])
+    gpu, cpu = mb.HipNetwork(desc, h), OracleNetwork(desc, h)
+    w = glorot_parameters(desc, 23, bias_range=0.3)
+    rng = np.random.default_rng(23)
+    masks = (rng.uniform(0, 1, desc.total_mask_units) < 0.6).astype(np.uint8)
+    X = rng.normal(0, 1, (B, T * 5)).astype(np.float32)
+    Y = rng.normal(0, 1, (B, T * 3)).astype(np.float32)
+    for n in (gpu, cpu):
+        n.set_state_propagation(mb.STATE_TRAINING)
+        n.upload_parameters(w)
+        n.upload_masks(masks)
+        n.Clear_Training_Arrays()
+    for step in range(2):
+        for n in (gpu, cpu):
+            n.Reset__Loss()
+            run_step(n, B, X, Y, update=False)
+        for li in range(1, desc.n_layers):
+            for kind in ("OUTPUTS", "ERRORS"):
+                a, b = gpu.download_tensor(li, mb.TENSOR[kind]), cpu.download_tensor(li, mb.TENSOR[kind])
+                W = len(a) // (T * Bmax)
+                _mostly_close(np.asarray(a).reshape(T, Bmax, W)[:, :B], np.asarray(b).reshape(T, Bmax, W)[:, :B], "step %d layer %d %s" % (step, li, kind))
+        # The bias of block 1's last member feeds the block's normalisation, which removes any constant: its gradient is zero
+        # in exact arithmetic, and what either side holds there is the rounding of a sum that cancels.
+        gg, gc = gpu.download_gradient(), cpu.download_gradient()
+        b4 = desc.layers[4].first_bias_connection_index
+        assert np.all(np.abs(gg[b4:b4 + 8]) < 5e-3) and np.all(np.abs(gc[b4:b4 + 8]) < 5e-3)
+        keep = np.ones(len(gg), dtype=bool)
+        keep[b4:b4 + 8] = False
+        _mostly_close(gg[keep], gc[keep], "gradient step %d" % step, fraction=0.02)   # sums of T x B terms of either sign
+        for n in (gpu, cpu):
+            n.Update_Parameter(B, B)
+        gpu.upload_parameters(cpu.download_parameters())
+    # inference: the running averages of each time step
+    for n in (gpu, cpu):
+        n.set_state_propagation(mb.STATE_INFERENCE)
+        n.Forward_Pass(B, X)
+    last = desc.n_layers - 1
+    assert_close(np.asarray(gpu.download_tensor(last, mb.TENSOR["OUTPUTS"])).reshape(T, Bmax, 3)[:, :B],
+                 np.asarray(cpu.download_tensor(last, mb.TENSOR["OUTPUTS"])).reshape(T, Bmax, 3)[:, :B], 1e-4, 1e-5, what="inference")

@@ -341,12 +341,73 @@ def test_member_dropout_acts_on_the_input_side_and_is_not_replayed_backward():
     assert_close(g[l4.first_connection_index:l4.last_connection_index].reshape(8, 7), d4.T @ v, 2e-4, 2e-6)
 
 
-def test_residual_needs_a_feed_forward_net_and_plain_members():
+def test_shakedrop_blocks_need_a_feed_forward_net():
     B = 2
     lib = load_oracle()
-    d = mb.make_desc([fc(4), res(1), fc(4), fc(2)], B, 3, lib=lib)         # recurrent depth 3
+    d = mb.make_desc([fc(4), res(1, dropout="SHAKEDROP", keep=0.5), fc(4), fc(2)], B, 3, lib=lib)         # recurrent depth 3
     with pytest.raises(Exception):
         OracleNetwork(d, oracle_hyper())
+
+
+RECURRENT_SPECS = [fc(5), fc(6, "TANH", normalization="BATCH_NORMALIZATION", norm_before=True),
+                   res(2, normalization="BATCH_NORMALIZATION"),
+                   fc(7, "TANH", normalization="BATCH_NORMALIZATION"), fc(8, "SIGMOID", dropout="BERNOULLI_INVERTED", keep=0.5),
+                   res(1), fc(8, "TANH"),
+                   fc(3, "LINEAR")]
+
+
+def check_recurrent_depth_is_the_block_time_step_by_time_step(make_net, make_desc, rel=2e-5, abs_=2e-6):
+    """A stack of dense layers and residual blocks has no recurrence: with a recurrent depth T every layer, every batch
+    normalisation (its own statistics and running averages per time step) and every dropout mask (its own per time step) works
+    on the time steps one by one (Recurrent__Forward_Pass__Residual*, NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:563-817;
+    the backward walks them in descending order).  So time step t of the T-deep network IS the feed-forward network on
+    the t-th slice of the inputs, targets, masks and normalisation parameters, and the weight gradients are the sums over the
+    time steps - the feed-forward path is pinned by float64 differentiation above."""
+    T, B, Bmax = 3, 5, 6
+    specs = RECURRENT_SPECS
+    deep, flat = make_desc(specs, Bmax, T), make_desc(specs, Bmax, 1)
+    rng = np.random.default_rng(17)
+    X = rng.normal(0, 1, (B, T, 5)).astype(np.float32)
+    Y = rng.normal(0, 1, (B, T, 3)).astype(np.float32)
+    w = glorot_parameters(deep, 17, bias_range=0.3)
+    masks = (rng.uniform(0, 1, deep.total_mask_units) < 0.6).astype(np.uint8)
+    assert deep.total_parameters == flat.total_parameters and deep.total_mask_units == T * flat.total_mask_units
+    net = make_net(deep)
+    net.set_state_propagation(mb.STATE_TRAINING)
+    net.upload_parameters(w)
+    net.upload_masks(masks)
+    net.Clear_Training_Arrays()
+    run_step(net, B, X.reshape(B, T * 5), Y.reshape(B, T * 3), update=False)
+    g_deep = net.download_gradient().astype(np.float64)
+    g_sum = np.zeros_like(g_deep)
+    last = deep.n_layers - 1
+    out = net.download_tensor(last, mb.TENSOR["OUTPUTS"]).reshape(T, Bmax, 3)
+    for t in range(T):
+        m = np.ones(flat.total_mask_units, dtype=np.uint8)
+        for li in range(flat.n_layers):
+            a0 = flat.layers[li].first_mask_index
+            a1 = flat.layers[li + 1].first_mask_index if li + 1 < flat.n_layers else flat.total_mask_units
+            u = a1 - a0
+            m[a0:a1] = masks[deep.layers[li].first_mask_index + t * u:deep.layers[li].first_mask_index + (t + 1) * u]
+        one = make_net(flat)
+        one.set_state_propagation(mb.STATE_TRAINING)
+        one.upload_parameters(w)
+        one.upload_masks(m)
+        one.Clear_Training_Arrays()
+        run_step(one, B, X[:, t], Y[:, t], update=False)
+        assert_close(out[t, :B], one.download_tensor(last, mb.TENSOR["OUTPUTS"]).reshape(Bmax, 3)[:B], rel, abs_, what="outputs of time step %d" % t)
+        for li in (1, 2, 3):   # the running averages of time step t are the feed-forward network's
+            nh = deep.layers[li + 1].first_normalized_unit_index - deep.layers[li].first_normalized_unit_index
+            for kind in ("NORM_MEANS_AVERAGES", "NORM_VARIANCES_AVERAGES"):
+                assert_close(net.download_tensor(li, mb.TENSOR[kind], T * nh).reshape(T, nh)[t], one.download_tensor(li, mb.TENSOR[kind], nh).reshape(nh), rel, abs_,
+                             what="layer %d %s at time step %d" % (li, kind, t))
+        g_sum += one.download_gradient().astype(np.float64)
+    assert_close(g_deep, g_sum, 10 * rel, 10 * abs_, what="gradient = sum over the time steps")
+
+
+def test_recurrent_depth_is_the_block_time_step_by_time_step():
+    check_recurrent_depth_is_the_block_time_step_by_time_step(
+        lambda desc: OracleNetwork(desc, oracle_hyper(type_loss_function=mb.LOSS["MSE"])), oracle_desc)
 
 
 def test_float64_model_reproduces_the_dropout_and_renormalisation_cases_of_the_oracle():
