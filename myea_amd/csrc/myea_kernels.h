@@ -266,6 +266,7 @@ struct LstmResidentPlan {
     bool ok = false;       // the resident form applies
     bool agent = false;    // groups wider than one XCD: device-scope exchange
     bool backward = false; // the backward loop has a resident form too
+    bool ksplit = false;   // ... and it is the one split along k, which needs the exchange buffer
     int cells = 0, members = 0, rs = 0, row_groups = 0, grid = 0, cus = 0;
 };
 int lstm_resident_plan(size_t C, size_t cells_per_block, size_t B, int dirs, LstmResidentPlan *plan);
@@ -274,8 +275,10 @@ size_t lstm_resident_sync_words();
 // kernel sets when a bounded wait gave up (1) or the members of a group did not share an XCD (2)
 int launch_lstm_resident_forward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag);
-// dh must hold the delta from the layers above for every time step
+// dh must hold the delta from the layers above for every time step.  exchange: device memory of at least
+// lstm_resident_exchange_floats(C, B, dirs) floats, 16-byte aligned, when plan.ksplit (its contents do not matter); else unused
+size_t lstm_resident_exchange_floats(size_t C, size_t B, int dirs);
 int launch_lstm_resident_backward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
-                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag);
+                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, float *exchange, size_t exchange_floats);
 
 }  // namespace myea

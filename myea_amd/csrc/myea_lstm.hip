@@ -427,6 +427,9 @@ int Net::lstm_create_layer(size_t li)
             MYEA_TRY(dev_alloc_zero(&q->dh, T * B * q->C));
         } else { q->h = o.values; q->dh = o.neuron_errors; }
     }
+    // the widest layer sizes the buffer the members of a resident backward loop hand each other partial sums through
+    if (o.lstm->fused && o.lstm->cpb == 1)
+        resident_exchange_floats = std::max(resident_exchange_floats, lstm_resident_exchange_floats(o.lstm->C, B, (int)dirs));
     return MYEA_OK;
 }
 
@@ -691,7 +694,7 @@ int Net::lstm_backward_layer(size_t li, size_t B)
             LstmResidentDir rd[2];
             lstm_resident_dirs(o, rd);
             prof_begin(kProfLstmBackwardLoop);
-            MYEA_TRY(launch_lstm_resident_backward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag));
+            MYEA_TRY(launch_lstm_resident_backward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag, resident_exchange, resident_exchange_floats));
             prof_end(dirs * loop_work, 1);
             return MYEA_OK;
         }

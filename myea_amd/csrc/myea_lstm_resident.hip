@@ -10,7 +10,9 @@
 //   * a workgroup owns CELLS cells (16, or 8 when C > 512).  Forward: the 4 CELLS gate columns of those cells, its four wavefronts split
 //     k = C into contiguous quarters; backward: the CELLS columns of dh, wavefront w takes the k range of gate w.  Either
 //     way a wavefront holds its [columns][k range] slice of Wrec (WrecT) in registers for the whole launch (at most 128
-//     registers per lane) in the operand layout of v_mfma_f32_16x16x4_f32;
+//     registers per lane) in the operand layout of v_mfma_f32_16x16x4_f32.  The backward loop has a second form, split
+//     along k instead of along the columns (described at its kernel), which is the one taken when the layer leaves half of
+//     the compute units or more idle;
 //   * a GROUP is the set of workgroups that cover all C cells for 2 x ROWS examples of one direction (ROWS = 16 RS):
 //     C / CELLS members.  A member is a workgroup of four wavefronts - one per SIMD - that lives for all T steps and keeps
 //     its slice of the recurrent matrix in registers.  It works on two independent CHAINS of ROWS examples in turn: a
@@ -57,6 +59,7 @@ namespace myea {
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;      // four wavefronts, one per SIMD
 constexpr int kSyncStride = 32;    // counters sit 128 bytes apart
@@ -122,6 +125,7 @@ struct SyncWords {
     unsigned *give_up;    // device flag, polled; behind it one word per group: the XCC id its first member ran on (+ 1)
     unsigned *host_flag;  // pinned host word, written once on give-up
     float *scrap;         // kScrapWords floats nobody reads
+    float *exchange;      // backward, split along k: per group 2 chains x 2 buffers x members^2 tiles of 1 KiB
 };
 
 // One lane per wavefront talks to the counters.  A wavefront arrives once its own stores are complete; the last of the
@@ -717,6 +721,233 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
     if (!tail(Chain1{}, Later{}, 0, 0u)) return;
 }
 
+// ---- backward, the contraction split along k ------------------------------------------------------------------------
+// dh[t] += dG[t'] Wrec with every member contracting over ITS OWN 64 k's: the gate deltas of its 16 cells, which it has
+// just computed and keeps in LDS - no member reads another's gate deltas.  What it owes the others is its share of every
+// column of dh: per unit a [16 examples][C] slab of partial sums, left in an exchange buffer as 1 KiB tiles
+// [consumer][producer][16 examples][16 columns]; a member's recurrent term is the sum of the `members` tiles addressed to
+// it, taken in a fixed order (repeatable).  Per unit and workgroup that is members KiB read and C / 16 KiB written
+// (C = 512: 32 + 32 KiB, register to register) against the 128 KiB of gate deltas the form above brings into LDS, whose
+// load instructions - bound by the compute unit's address path, hidden behind nothing - are a third of its time.
+// The slice of Wrec a member keeps is [its 64 gate rows][C]: 16 C / 64 registers per lane.
+//
+// A unit (chain c, step j of the pass): sum the tiles of (c, j) [requested during the other chain's unit] -> gate deltas
+// of step j -> own k's to LDS -> MFMAs for step j + 1 (the transposed product: an accumulator holds four consecutive
+// columns of one example, one 16-byte store per lane and tile) -> tiles out.  The other chain's tiles are requested
+// three quarters into the MFMAs, when its counter is normally complete; a chain's arrival is signalled behind the NEXT
+// unit's gate stores, by which time its tile stores have long been acknowledged.  The tiles of a chain alternate between
+// two buffers: a member overwrites a tile two steps later, which it can only reach after every member has arrived for
+// the step in between, that is after every member has summed the tiles of the step before that.
+// Tiles travel through buffer instructions (the compiler keeps count of them, unlike of inline assembly): loads with sc1
+// (served beyond this compute unit's L1), plain stores; a group shares one XCD's L2, as in the form above.
+constexpr unsigned kBufferWord3 = 0x00020000u;   // raw buffer of dwords
+constexpr int kAuxSc1 = 16;
+
+template <int CC>
+__global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_ksplit_kernel(ResidentGeometry g, LstmResidentDir d0, LstmResidentDir d1, SyncWords w)
+{
+    constexpr int C = CC, G = 4 * C, CELLS = 16, ROWS = 16;
+    constexpr int NQ = C / 4;               // columns of dh per wavefront
+    constexpr int NCT = NQ / 16;            // tiles of 16 columns per wavefront = consumers it writes to
+    constexpr int MEMBERS = C / CELLS;
+    constexpr int NIN = MEMBERS / 4;        // producers whose tiles a wavefront sums
+    constexpr int NSTORE = 6;               // stores of a unit's gate math, every lane the same (scrap for lanes without an example)
+    constexpr int kRow = 68;                // floats per example of the own gate deltas in LDS: [k & 3][k >> 2], padded
+    constexpr int kRead = 7, kCheck = 11;   // k steps (of 16) at which the other chain's counter is read and looked at
+    constexpr unsigned kTileBytes = ROWS * CELLS * sizeof(float);
+    constexpr unsigned kParityBytes = (unsigned)MEMBERS * MEMBERS * kTileBytes;   // one chain's tiles of one step
+    static_assert(NCT >= 1 && NIN == NCT, "16 cells per member");
+    __shared__ __attribute__((aligned(16))) float s_own[2][ROWS * kRow];      // per chain: its gate deltas of this member's cells
+    __shared__ __attribute__((aligned(16))) float s_sum[2][4][ROWS][CELLS];   // per chain and wavefront: the sum of its producers' tiles
+    __shared__ unsigned s_arrive[2];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col16 = lane & 15, quad = lane >> 4;
+
+    int group, member;
+    if (!place<false>(blockIdx.x, g.members, g.dirs * g.row_groups, group, member)) return;
+    const int dir = group % g.dirs, rg = group / g.dirs;
+    const LstmResidentDir &d = dir ? d1 : d0;
+    const int c0 = member * CELLS, B = g.B, T = g.T;
+    const size_t Bmax = (size_t)g.Bmax;
+    unsigned *const counters = w.counters + (size_t)group * 2 * kSyncStride;
+    const unsigned arrivals = (unsigned)g.arrivals;
+    check_same_xcd(w, group);
+    if (threadIdx.x < 2) s_arrive[threadIdx.x] = 0u;
+    __syncthreads();
+
+    // the weights of the member's 64 k's (k = gate * 16 + cell: row gate * C + c0 + cell of Wrec [4C][C]) against the
+    // wavefront's columns, as the A operand of the transposed product: lane (col16, quad) holds Wrec[k = 4 ks + quad][16 ct + col16]
+    float breg[16][NCT];
+#pragma unroll
+    for (int ks = 0; ks < 16; ++ks) {
+        const int k = ks * 4 + quad;
+        const float *wrow = d.Wrec + ((size_t)(k >> 4) * C + c0 + (k & 15)) * C + wave * NQ + col16;
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct) breg[ks][ct] = wrow[ct * 16];
+    }
+    // this pass walks the direction's steps from its last to its first: in time, forwards for the reversed direction
+    const int t_first = d.reverse ? 0 : T - 1;
+    const ptrdiff_t t_step = d.reverse ? 1 : -1;
+    const ptrdiff_t step_g = t_step * (ptrdiff_t)(Bmax * G), step_c = t_step * (ptrdiff_t)(Bmax * C);
+    const int row = threadIdx.x >> 4, cell = threadIdx.x & 15, kcell = c0 + cell;   // the lane's (example, cell) pair
+    float e_peep[3];
+#pragma unroll
+    for (int gate = 0; gate < 3; ++gate) e_peep[gate] = d.peep[gate * C + kcell];
+    float n_di[2], n_df[2], n_f[2], n_dc[2];   // of the chain's step processed before: delta i, delta f, f, delta c
+    float e_act[4], e_ca, e_cp, e_dh;
+    const float *p_acts[2], *p_ca[2], *p_cp[2], *p_dh_in[2];   // read: the batch's last example for a lane without one
+    float *p_dh[2], *p_dG[2], *p_dc[2];                          // written: the scrap area for such a lane
+    ptrdiff_t lane_step_g[2], lane_step_c[2];
+#pragma unroll
+    for (int ch = 0; ch < 2; ++ch) {
+        const int r = (rg * 2 + ch) * ROWS + row;
+        const bool valid = r < B;
+        const size_t at = (size_t)t_first * Bmax + min(r, B - 1);
+        float *scrap = w.scrap + ch * kThreads + threadIdx.x;
+        p_acts[ch] = d.acts + at * G + kcell;
+        p_ca[ch] = d.ca + at * C + kcell;
+        p_cp[ch] = d.c + at * C + kcell + step_c;   // the cell state of the step before t in the direction's order: one step further along this pass
+        p_dh_in[ch] = d.dh + at * C + kcell;
+        p_dh[ch] = valid ? d.dh + at * C + kcell : scrap + 4096;
+        p_dG[ch] = valid ? d.dG + at * G + kcell : scrap;
+        p_dc[ch] = valid ? d.dc + at * C + kcell : scrap + 4096 + 1024;
+        lane_step_g[ch] = valid ? step_g : 0;
+        lane_step_c[ch] = valid ? step_c : 0;
+        n_di[ch] = 0.f; n_df[ch] = 0.f; n_f[ch] = 0.f; n_dc[ch] = 0.f;
+    }
+    // the group's part of the exchange buffer: [chain][buffer][consumer][producer][16 examples][16 columns]
+    const __amdgpu_buffer_rsrc_t exchange =
+        __builtin_amdgcn_make_buffer_rsrc(w.exchange + (size_t)group * (4 * (size_t)kParityBytes / sizeof(float)), 0, (int)(4 * kParityBytes), (int)kBufferWord3);
+    // byte offsets within one chain's buffer: the tiles addressed to this member from the wavefront's producers, and this
+    // member's tiles to the wavefront's consumers
+    const unsigned in_lane = ((unsigned)member * MEMBERS + (unsigned)wave * NIN) * kTileBytes + (unsigned)lane * 16u;
+    const unsigned out_lane = ((unsigned)(wave * NCT) * MEMBERS + (unsigned)member) * kTileBytes + (unsigned)(col16 * CELLS + quad * 4) * 4u;
+
+    u32x4 tiles[NIN];
+    unsigned seen = 0;
+
+    auto load_operands = [&](auto ch, bool with_cp) {   // of the step the chain's pointers are at; with_cp: not the direction's first step, which has no step before it
+        constexpr int c = decltype(ch)::value;
+#pragma unroll
+        for (int gate = 0; gate < 4; ++gate) e_act[gate] = p_acts[c][gate * C];
+        e_ca = *p_ca[c];
+        e_dh = *p_dh_in[c];
+        e_cp = *(with_cp ? p_cp[c] : p_ca[c]);   // no step before the direction's first: any finite value, the forget gate's delta is zero there
+    };
+    auto load_tiles = [&](auto ch, int buffer) {
+        constexpr int c = decltype(ch)::value;
+        const unsigned from = (unsigned)(c * 2 + buffer) * kParityBytes + in_lane;
+#pragma unroll
+        for (int i = 0; i < NIN; ++i) tiles[i] = __builtin_amdgcn_raw_buffer_load_b128(exchange, (int)(from + (unsigned)i * kTileBytes), 0, kAuxSc1);
+    };
+
+    // One unit: step j of the pass for chain c (s: the direction's step).  FIRST: j = 0, no recurrent term and nothing from a
+    // later step.  LAST: no step j + 1 follows.  other_target: arrivals of the other chain that complete the tiles of ITS next
+    // unit (unused when it has none, or that one is a first step); other_with_cp: that unit is not at the direction's first
+    // step.  Returns false when a wait gave up.  Which loads a unit issues depends on its compile-time kind only: a load under
+    // a run-time condition would have the compiler wait for it where the two paths meet.
+    auto unit = [&](auto ch, auto first_tag, auto last_tag, int j, int s, unsigned other_target, bool other_with_cp) -> bool {
+        constexpr int c = decltype(ch)::value;
+        constexpr bool FIRST = decltype(first_tag)::value, LAST = decltype(last_tag)::value;
+        constexpr bool REQUEST = !(FIRST && c == 0) && !(LAST && c == 1);   // the other chain's next unit exists and sums tiles
+        using Other = std::integral_constant<int, 1 - c>;
+        const int other_buffer = (j + c) & 1;   // the other chain's next unit is step j (c == 0) or j + 1 (c == 1)
+        float rec = 0.f;
+        if (!FIRST) {
+            f32x4 sum = __builtin_bit_cast(f32x4, tiles[0]);
+#pragma unroll
+            for (int i = 1; i < NIN; ++i) sum += __builtin_bit_cast(f32x4, tiles[i]);
+            *reinterpret_cast<f32x4 *>(&s_sum[c][wave][lane >> 2][(lane & 3) * 4]) = sum;
+            lds_barrier();
+#pragma unroll
+            for (int wv = 0; wv < 4; ++wv) rec += s_sum[c][wv][row][cell];
+        }
+        const float dh = e_dh + rec;
+        const float z = e_act[0], gi = e_act[1], gf = e_act[2], go = e_act[3];
+        const float a = e_ca;
+        const float ddo = go * (1.f - go) * (dh * a);
+        float e = dh * go * (1.f - a * a);
+        e += e_peep[2] * ddo;
+        if (!FIRST) {
+            e += e_peep[0] * n_di[c];
+            e += e_peep[1] * n_df[c];
+            e += n_dc[c] * n_f[c];
+        }
+        const float dz = e * gi * (1.f - z * z);
+        const float di = (e * z) * (gi * (1.f - gi));
+        const float df = s > 0 ? (e * e_cp) * (gf * (1.f - gf)) : 0.f;
+        n_di[c] = di; n_df[c] = df; n_f[c] = gf; n_dc[c] = e;
+        float *drow = p_dG[c];
+        drow[0] = dz; drow[C] = di; drow[2 * C] = df; drow[3 * C] = ddo;
+        *p_dh[c] = dh; *p_dc[c] = e;
+        p_acts[c] += step_g; p_ca[c] += step_c; p_cp[c] += step_c; p_dh_in[c] += step_c;
+        p_dG[c] += lane_step_g[c]; p_dh[c] += lane_step_c[c]; p_dc[c] += lane_step_c[c];
+        if (!(FIRST && c == 0)) {
+            // the tiles the other chain stored at the end of its unit are older than these six stores: they are complete
+            // once at most six operations are outstanding, and with them the other chain has arrived
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<NSTORE>();
+            wave_arrive<false>(counters + (1 - c) * kSyncStride, &s_arrive[1 - c]);
+        }
+        if (LAST) {
+            // the pass's last step: no MFMAs to hide the other chain's requests behind
+            if (REQUEST) {
+                load_operands(Other{}, other_with_cp);
+                if (!wave_wait(w, counters + (1 - c) * kSyncStride, other_target, g.spin_polls)) return false;
+                load_tiles(Other{}, other_buffer);
+            }
+            return true;
+        }
+        // own k's for the MFMAs: k = gate * 16 + cell sits at [example][(k & 3) * 16 + (k >> 2)]
+        {
+            float *own = s_own[c] + row * kRow + (cell & 3) * 16 + (cell >> 2);
+            own[0] = dz; own[4] = di; own[8] = df; own[12] = ddo;
+        }
+        lds_barrier();
+        // the next unit in program order is the other chain's: its operands now, its tiles when its counter is complete
+        load_operands(Other{}, other_with_cp);
+        f32x4 bf[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bf[q] = *reinterpret_cast<const f32x4 *>(s_own[c] + col16 * kRow + quad * 16 + q * 4);
+        f32x4 acc[NCT];
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct) acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < 16; ++ks) {
+#pragma unroll
+            for (int ct = 0; ct < NCT; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(breg[ks][ct], bf[ks >> 2][ks & 3], acc[ct], 0, 0, 0);
+            if (ks == kRead && REQUEST) seen = __hip_atomic_load(counters + (1 - c) * kSyncStride, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+            if (ks == kCheck && REQUEST) {
+                __builtin_amdgcn_sched_barrier(0);   // the counter's value is looked at here, not right behind its load
+                if ((int)(__builtin_amdgcn_readfirstlane(seen) - other_target) < 0 && !wave_wait(w, counters + (1 - c) * kSyncStride, other_target, g.spin_polls)) return false;
+                load_tiles(Other{}, other_buffer);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // tiles out: accumulator ct holds, for example col16, the columns 16 ct + 4 quad .. + 3 of the wavefront's range,
+        // which belong to consumer wave * NCT + ct
+        const unsigned to = (unsigned)(c * 2 + ((j + 1) & 1)) * kParityBytes + out_lane;
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[ct]), exchange, (int)(to + (unsigned)ct * MEMBERS * kTileBytes), 0, 0);
+        return true;
+    };
+    using First = std::true_type;
+    using Later = std::false_type;
+
+    // units in program order: (0,0) (1,0) (0,1) (1,1) ...; unit (c, j), j >= 1, sums the tiles every member stored at the end
+    // of unit (c, j - 1).  Chain 1's arrivals are signalled in chain 0's units and the other way round: before unit (0, j)'s
+    // MFMAs chain 1 has arrived j times, before unit (1, j)'s chain 0 has arrived j + 1 times.
+    load_operands(Chain0{}, true);
+    if (!unit(Chain0{}, First{}, Later{}, 0, T - 1, 0u, true)) return;
+    if (!unit(Chain1{}, First{}, Later{}, 0, T - 1, arrivals, T > 2)) return;
+    for (int j = 1; j + 1 < T; ++j) {
+        if (!unit(Chain0{}, Later{}, Later{}, j, T - 1 - j, (unsigned)j * arrivals, true)) return;
+        if (!unit(Chain1{}, Later{}, Later{}, j, T - 1 - j, (unsigned)(j + 1) * arrivals, T - 2 - j > 0)) return;
+    }
+    if (!unit(Chain0{}, Later{}, First{}, T - 1, 0, (unsigned)(T - 1) * arrivals, false)) return;
+    unit(Chain1{}, Later{}, First{}, T - 1, 0, 0u, false);
+}
+
 __global__ void resident_probe_kernel(unsigned *table)
 {
     if (threadIdx.x == 0) table[blockIdx.x] = xcc_id();
@@ -792,6 +1023,18 @@ unsigned spin_polls()
     return 200000u;
 }
 
+// Which resident form the backward loop takes.  Measured on this device (T = 64, microseconds per launch, split along k
+// against split along the columns of dh): with every compute unit busy the column form wins (512 cells x 256 examples: 594
+// against 523; 256 x 512: 405 against 392), with half of them or fewer the k form does (512 x 64: 408 against 450;
+// 256 x 128: 236 against 267; 128 x 256: 179 against 190) - its exchange is lighter, but what bounds both under full load
+// is the tail latency of the operands streamed from memory, which stalls a group at one more barrier per step in the k form.
+// MYEA_LSTM_BACKWARD_KSPLIT=0 / 1 forces the column form / the k form wherever it exists.
+int ksplit_choice()   // -1: by occupancy, 0: never, 1: always
+{
+    const char *e = std::getenv("MYEA_LSTM_BACKWARD_KSPLIT");
+    return !e || !*e ? -1 : e[0] == '0' ? 0 : 1;
+}
+
 // MYEA_LSTM_RESIDENT_TEST_ABSENT_MEMBER=1 makes every group expect one member more than it has: its first wait runs out of
 // polls, the kernel ends through its give-up path and the host reports it.  For tests of that path; every wavefront still
 // exits normally.
@@ -831,6 +1074,16 @@ KernelInfo backward_info()
     return k;
 }
 
+template <int C>
+KernelInfo ksplit_info()
+{
+    KernelInfo k;
+    k.fn = lstm_resident_backward_ksplit_kernel<C>;
+    k.lds = 0;   // its LDS is static
+    k.cells = 16;
+    return k;
+}
+
 // [backward][C: 128, 256, 512, 1024][rs - 1]; an entry without a kernel has fn == nullptr
 KernelInfo g_kernels[2][4][2] = {
     {{forward_info<32, 16, 1, false>(), forward_info<32, 16, 2, false>()},
@@ -843,16 +1096,19 @@ KernelInfo g_kernels[2][4][2] = {
      {KernelInfo{}, KernelInfo{}}},
 };
 
+// the backward loop split along k, [C: 128, 256, 512, 1024]: two chains of 16 examples only, groups within one XCD
+KernelInfo g_ksplit[4] = {ksplit_info<128>(), ksplit_info<256>(), ksplit_info<512>(), KernelInfo{}};
+
 // the kernel for (C, rs) with its LDS attribute set and its occupancy known, or nullptr
-KernelInfo *kernel_for(size_t C, int rs, bool backward)
+KernelInfo *kernel_for(size_t C, int rs, bool backward, bool ksplit = false)
 {
     const int ci = C == 128 ? 0 : C == 256 ? 1 : C == 512 ? 2 : C == 1024 ? 3 : -1;
-    if (ci < 0 || rs < 1 || rs > 2) return nullptr;
-    KernelInfo &k = g_kernels[backward ? 1 : 0][ci][rs - 1];
+    if (ci < 0 || rs < 1 || rs > 2 || (ksplit && (rs != 1 || !backward))) return nullptr;
+    KernelInfo &k = ksplit ? g_ksplit[ci] : g_kernels[backward ? 1 : 0][ci][rs - 1];
     if (!k.fn) return nullptr;
     std::lock_guard<std::mutex> lock(g_resident_mutex);
     if (!k.ready) {
-        k.status = hipFuncSetAttribute(reinterpret_cast<const void *>(k.fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)k.lds);
+        k.status = k.lds ? hipFuncSetAttribute(reinterpret_cast<const void *>(k.fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)k.lds) : hipSuccess;
         if (k.status == hipSuccess) k.status = hipOccupancyMaxActiveBlocksPerMultiprocessor(&k.per_cu, reinterpret_cast<const void *>(k.fn), kThreads, k.lds);
         k.ready = true;
     }
@@ -886,6 +1142,7 @@ int fill_geometry(const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax,
 // clears the counters and flags and lays the words out
 int prepare_sync(hipStream_t s, const LstmResidentPlan &plan, int dirs, unsigned *sync, unsigned *host_flag, SyncWords *w)
 {
+    w->exchange = nullptr;
     const int groups = plan.row_groups * dirs;
     if (groups > kMaxGroups) { set_last_error("resident LSTM: %d groups exceed the counter block", groups); return MYEA_E_INVALID; }
     const int words = groups * 2 * kSyncStride + 1 + groups;
@@ -910,15 +1167,25 @@ int check_dirs(const LstmResidentDir *dir, int dirs, bool backward)
 }
 
 int launch_resident(hipStream_t s, bool backward, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
-                    const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag)
+                    const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, float *exchange = nullptr, size_t exchange_floats = 0)
 {
+    const bool ksplit = backward && plan.ksplit;
     ResidentGeometry g;
     SyncWords w;
     int rc = fill_geometry(plan, T, B, Bmax, C, dirs, &g);
     if (rc == MYEA_OK && backward && !plan.backward) { set_last_error("resident LSTM backward: no plan for this layer"); rc = MYEA_E_INVALID; }
     if (rc == MYEA_OK) rc = check_dirs(dir, dirs, backward);
     if (rc != MYEA_OK) return rc;
-    KernelInfo *k = kernel_for(C, plan.rs, backward);
+    if (ksplit) {
+        for (int q = 0; q < dirs; ++q)
+            if (!dir[q].Wrec) { set_last_error("resident LSTM backward: null operand"); return MYEA_E_INVALID; }
+        const size_t need = lstm_resident_exchange_floats(C, B, dirs);
+        if (!exchange || (reinterpret_cast<uintptr_t>(exchange) & 15u) || exchange_floats < need) {
+            set_last_error("resident LSTM backward: the exchange buffer holds %zu floats, the layer needs %zu", exchange ? exchange_floats : (size_t)0, need);
+            return MYEA_E_INVALID;
+        }
+    }
+    KernelInfo *k = kernel_for(C, plan.rs, backward, ksplit);
     ResidentDevice *dev = nullptr;
     rc = probe_device(&dev);
     if (rc != MYEA_OK) return rc;
@@ -929,6 +1196,7 @@ int launch_resident(hipStream_t s, bool backward, const LstmResidentPlan &plan, 
     }
     rc = prepare_sync(s, plan, dirs, sync, host_flag, &w);
     if (rc != MYEA_OK) return rc;
+    w.exchange = ksplit ? exchange : nullptr;
     hipLaunchKernelGGL(k->fn, dim3((unsigned)plan.grid), dim3(kThreads), k->lds, s, g, dir[0], dir[dirs > 1 ? 1 : 0], w);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
@@ -959,12 +1227,26 @@ int lstm_resident_plan(size_t C, size_t cells_per_block, size_t B, int dirs, Lst
         const int rows = 2 * 16 * rs, row_groups = (int)((B + rows - 1) / rows), groups = row_groups * dirs;
         int grid = 0, grid_b = 0;
         if (!place_groups(*dev, *fwd, members, agent, groups, &grid)) continue;
-        const bool backward = bwd && !agent && place_groups(*dev, *bwd, members, false, groups, &grid_b) && grid_b == grid;
-        plan->ok = true; plan->agent = agent; plan->backward = backward;
+        bool backward = bwd && !agent && place_groups(*dev, *bwd, members, false, groups, &grid_b) && grid_b == grid;
+        const int choice = ksplit_choice();
+        KernelInfo *split = choice == 0 ? nullptr : kernel_for(C, rs, true, true);
+        bool ksplit = split && !agent && fwd->cells == 16 && place_groups(*dev, *split, members, agent, groups, &grid_b) && grid_b == grid;
+        if (ksplit && backward && choice < 0) ksplit = 2 * groups * members <= dev->cus;
+        backward = backward || ksplit;
+        plan->ok = true; plan->agent = agent; plan->backward = backward; plan->ksplit = ksplit;
         plan->cells = fwd->cells; plan->members = members; plan->rs = rs; plan->row_groups = row_groups; plan->grid = grid; plan->cus = dev->cus;
         break;
     }
     return MYEA_OK;
+}
+
+// Floats of exchange buffer the backward loop split along k needs for a layer of C cells and up to B examples per direction:
+// per group of 32 examples and direction, 2 chains x 2 buffers x (C / 16)^2 tiles of 256 floats.  0 for other widths.
+size_t lstm_resident_exchange_floats(size_t C, size_t B, int dirs)
+{
+    if ((C != 128 && C != 256 && C != 512) || B == 0 || dirs < 1) return 0;
+    const size_t members = C / 16, groups = (B + 31) / 32 * (size_t)dirs;
+    return groups * 4 * members * members * 256;
 }
 
 // counters (one per group and chain, 128 bytes apart), the give-up flag, one XCC word per group, the scrap area
@@ -978,9 +1260,9 @@ int launch_lstm_resident_forward(hipStream_t s, const LstmResidentPlan &plan, si
 }
 
 int launch_lstm_resident_backward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
-                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag)
+                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, float *exchange, size_t exchange_floats)
 {
-    return launch_resident(s, true, plan, T, B, Bmax, C, dirs, dir, sync, host_flag);
+    return launch_resident(s, true, plan, T, B, Bmax, C, dirs, dir, sync, host_flag, exchange, exchange_floats);
 }
 
 }  // namespace myea

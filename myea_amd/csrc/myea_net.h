@@ -99,6 +99,8 @@ struct Net {
     // LSTM time loops as one resident launch (myea_lstm_resident.hip): barrier counters in device memory, and a pinned host
     // word a kernel sets when one of its bounded waits gave up; resident_off: this network stays on one launch per time step
     unsigned *resident_sync = nullptr, *resident_flag = nullptr;
+    float *resident_exchange = nullptr;   // partial sums the members of a group hand each other in the backward loop
+    size_t resident_exchange_floats = 0;
     bool resident_off = false;
     int resident_check();   // MYEA_E_DEVICE (once) after a resident launch reported a give-up
     unsigned long long *index_stage = nullptr;   // [Bmax] example indices of a gathered batch

@@ -348,6 +348,7 @@ int Net::create(const myea_net_desc &desc)
             MYEA_HIP_TRY(hipHostMalloc(&q, 64, hipHostMallocDefault));
             resident_flag = static_cast<unsigned *>(q);
             *resident_flag = 0u;
+            if (resident_exchange_floats) MYEA_TRY(dev_alloc(&resident_exchange, resident_exchange_floats));
         }
     }
     MYEA_TRY(dev_alloc(&tmp1, T * B * max_h));
@@ -402,6 +403,7 @@ Net::~Net()
         lstm_destroy_layer(o);
     }
     fr(resident_sync);
+    fr(resident_exchange);
     if (resident_flag) (void)hipHostFree(resident_flag);
     fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc); fr(index_stage); fr(dw_slabs);
     for (ProfEvent &e : pending) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }

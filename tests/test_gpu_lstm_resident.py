@@ -93,8 +93,11 @@ def _loop_launches(net):
     return net.profile_read(FORWARD_LOOP)[0], net.profile_read(BACKWARD_LOOP)[0]
 
 
+# the backward loop has two resident forms: split along k (members exchange partial sums; the default) and split along the
+# columns of dh (members read each other's gate deltas; MYEA_LSTM_BACKWARD_KSPLIT=0)
+@pytest.mark.parametrize("ksplit", ["1", "0"], ids=["backward-split-along-k", "backward-split-along-columns"])
 @pytest.mark.parametrize("name,specs,T,B,Bmax,backward", CASES, ids=[c[0] for c in CASES])
-def test_resident_loop_matches_one_launch_per_step_and_the_oracle(name, specs, T, B, Bmax, backward):
+def test_resident_loop_matches_one_launch_per_step_and_the_oracle(name, specs, T, B, Bmax, backward, ksplit):
     desc, h, w, masks, X, Y = _setup(specs, T, B, Bmax, seed=21)
     resident = _net(desc, h, w, masks)
     stepwise = _net(desc, h, w, masks)
@@ -108,11 +111,12 @@ def test_resident_loop_matches_one_launch_per_step_and_the_oracle(name, specs, T
     wide = [l for l in layers]   # every LSTM layer of these cases has a resident form
     per_step = sum((2 if l.use_bidirectional else 1) * (T - 1) for l in layers)
     for step in range(2):
-        resident.profile_enable(True)
-        resident.Reset__Loss()
-        run_step(resident, B, X, Y, update=False)
-        fwd, bwd = _loop_launches(resident)
-        resident.profile_enable(False)
+        with environment(MYEA_LSTM_BACKWARD_KSPLIT=ksplit):
+            resident.profile_enable(True)
+            resident.Reset__Loss()
+            run_step(resident, B, X, Y, update=False)
+            fwd, bwd = _loop_launches(resident)
+            resident.profile_enable(False)
         assert fwd == len(wide), "the forward time loops did not run as one launch per layer"
         if backward:
             assert bwd == len(wide), "the backward time loops did not run as one launch per layer"
@@ -178,3 +182,30 @@ def test_a_wait_that_gives_up_is_reported_once_and_the_network_carries_on_per_st
     assert _loop_launches(gpu) == (T - 1, T - 1), "after a give-up the time loops run one launch per step"
     gpu.profile_enable(False)
     _compare(desc, gpu, cpu, B, T, "after the give-up")
+
+
+@pytest.mark.parametrize("ksplit", ["1", "0"], ids=["backward-split-along-k", "backward-split-along-columns"])
+def test_a_backward_wait_that_gives_up_is_reported_too(ksplit):
+    """the same forced give-up in the backward loop, in either of its forms: the forward pass runs normally, the backward
+    loop's first wait between steps runs out of polls and every wavefront leaves"""
+    specs = [dict(units=8), lstm(128), dict(units=128, activation="LINEAR")]
+    T, B = 5, 32
+    desc, h, w, masks, X, Y = _setup(specs, T, B, B, seed=9)
+    gpu = _net(desc, h, w, None)
+    gpu.Forward_Pass(B, X)
+    gpu.Compute__Error(B, Y)
+    gpu.synchronize()
+    with environment(MYEA_LSTM_RESIDENT_TEST_ABSENT_MEMBER=1, MYEA_LSTM_RESIDENT_SPIN_POLLS=64, MYEA_LSTM_BACKWARD_KSPLIT=ksplit):
+        gpu.Backward_Pass(B)
+        with pytest.raises(mb.MyeaError) as e:
+            gpu.synchronize()
+    assert e.value.code == mb.E_DEVICE and "gave up" in str(e.value)
+    cpu = OracleNetwork(desc, h)
+    cpu.set_state_propagation(mb.STATE_TRAINING)
+    cpu.upload_parameters(w)
+    cpu.Clear_Training_Arrays()
+    for n in (gpu, cpu):
+        n.Clear_Training_Arrays()
+        n.Reset__Loss()
+        run_step(n, B, X, Y, update=False)
+    _compare(desc, gpu, cpu, B, T, "after the backward give-up")
