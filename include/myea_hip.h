@@ -276,6 +276,13 @@ enum {
                                               bidirectional layer is the delta of the summed output, from above only) */
     MYEA_TENSOR_DIRECTION_BACKWARD = 0x100 /* OR-ed onto an LSTM kind: the time-reversed direction of a bidirectional layer */
 };
+/* A normalised LSTM layer owns nine groups of normalised units (Neural_Network__Allocate.cpp:2710-2790): 0 block input
+ * from below, 1 block input recurrent, 2 cell state, 3 / 4 input gate, 5 / 6 forget gate, 7 / 8 output gate (from below /
+ * recurrent).  (group + 1) << MYEA_TENSOR_LSTM_NORM_GROUP_SHIFT OR-ed onto NORM_HATS / NORM_MEANS / NORM_VARIANCES /
+ * NORM_MEANS_AVERAGES / NORM_VARIANCES_AVERAGES selects the group's tensor ([T][Bmax][units] or [T][units]); onto ERRORS,
+ * the delta of the group's input after the backward pass through its normalisation. */
+#define MYEA_TENSOR_LSTM_NORM_GROUP_SHIFT 12
+#define MYEA_TENSOR_LSTM_NORM_GROUP(g) (((g) + 1) << MYEA_TENSOR_LSTM_NORM_GROUP_SHIFT)
 
 /* ---- host-side descriptor helpers (no GPU needed) ---- */
 

@@ -37,6 +37,12 @@ TENSOR = dict(OUTPUTS=0, SUMMATIONS=1, ERRORS=2, NORM_HATS=3, NORM_MEANS=4, NORM
               LSTM_OUTPUT_GATE=20, LSTM_DELTA_CELL_INPUT=21, LSTM_DELTA_CELL_STATE=22,
               LSTM_DELTA_INPUT_GATE=23, LSTM_DELTA_FORGET_GATE=24, LSTM_DELTA_OUTPUT_GATE=25, LSTM_CELL_OUTPUT=26, LSTM_DELTA_CELL_OUTPUT=27,
               DIRECTION_BACKWARD=0x100)
+
+
+def TENSOR_LSTM_NORM_GROUP(group):
+    """OR-ed onto a NORM_* kind (or ERRORS) of a normalised LSTM layer: one of its nine groups of normalised units, 0 block
+    input from below, 1 block input recurrent, 2 cell state, 3 / 4 input gate, 5 / 6 forget gate, 7 / 8 output gate"""
+    return (group + 1) << 12
 E_INVALID, E_UNSUPPORTED, E_BATCH, E_STATE, E_NOMEM, E_DEVICE = -1, -2, -3, -4, -5, -6
 
 

@@ -49,7 +49,20 @@ typedef struct olstm {
     float *sum_in_z, *sum_rec_z, *sum_z, *z, *c, *ca;          /* cells */
     float *sum_in_i, *sum_in_f, *sum_in_o, *sum_rec_i, *sum_rec_f, *sum_rec_o, *sum_i, *sum_f, *sum_o, *gi, *gf, *go; /* blocks */
     float *dz, *dc, *di, *df, *dgo;                              /* deltas */
+    /* normalised layer (NN/Neural_Network__Allocate.cpp:2710-2790, one cell per block): nine groups of normalised units,
+     * 0 block input from below, 1 block input recurrent, 2 cell state, 3 / 4 input gate, 5 / 6 forget gate, 7 / 8 output gate
+     * (from below / recurrent), each with its own statistics per time step; and the deltas of the eight sums after the
+     * backward pass through their normalisation */
+    int norm;
+    struct obn {
+        size_t H, param;   /* width; flat index of the group's first scale (the shift sits total_normalized_units further) */
+        float *means, *variances, *means_averages, *variances_averages, *r_corrections, *d_corrections;   /* [T][H] */
+        float *derivatives_means, *derivatives_variances;
+        float *hats, *normalizes;   /* [T][Bmax][H] */
+    } nrm[9];
+    float *dz_in, *dz_rec, *di_in, *di_rec, *df_in, *df_rec, *do_in, *do_rec;
 } olstm;
+typedef struct obn obn;
 
 typedef struct olayer {
     size_t H;            /* *ptr_number_outputs */
@@ -305,7 +318,11 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
         const myea_layer_desc *l = &desc->layers[li];
         olayer *o = &n->L[li];
         if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED) { free(n); return MYEA_E_UNSUPPORTED; }
-        if (l->type_layer == MYEA_LAYER_LSTM && (layer_uses_norm(l) || (l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_ZONEOUT))) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (l->type_layer == MYEA_LAYER_LSTM && l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_ZONEOUT) { free(n); return MYEA_E_UNSUPPORTED; }
+        /* with more cells per block the reference's indices [3] .. [8] into the layer's normalised units (NN/Neural_Network.cpp:4498-4613)
+         * land on the second cell's units instead of the block's (the units are laid out per block: 3 per cell, then 6,
+         * NN/Neural_Network__Ordered.cpp:937-966): no behaviour to follow */
+        if (l->type_layer == MYEA_LAYER_LSTM && layer_uses_norm(l) && l->n_cells_per_block != 1) { free(n); return MYEA_E_UNSUPPORTED; }
         if (l->type_layer != MYEA_LAYER_LSTM && l->type_dropout == MYEA_DROPOUT_ZONEOUT) { free(n); return MYEA_E_UNSUPPORTED; }
         if (is_ind_rnn(l) && l->type_activation_function == MYEA_AF_SOFTMAX) { free(n); return MYEA_E_UNSUPPORTED; }
         size_t sz = T * B * o->H;
@@ -337,6 +354,25 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
                 for (size_t a = 0; a < sizeof(blocks) / sizeof(blocks[0]); ++a) *blocks[a] = zalloc(sk);
                 if (dirs == 2) { q->h = zalloc(sc); q->dh = zalloc(sc); }
                 else { q->h = o->values; q->dh = o->af_errors; }
+                q->norm = layer_uses_norm(l);
+                if (q->norm) {
+                    /* scales of the layer: per direction [3 groups of C | 6 groups of K] in group order (Allocate: the scale
+                     * iterator advances group by group, :2718-2776) */
+                    size_t at = desc->total_weights + desc->total_bias + l->first_normalized_unit_index + dir * (3 * q->C + 6 * q->K);
+                    for (int g = 0; g < 9; ++g) {
+                        obn *bn = &q->nrm[g];
+                        bn->H = g < 3 ? q->C : q->K;
+                        bn->param = at; at += bn->H;
+                        float **small[] = {&bn->means, &bn->variances, &bn->means_averages, &bn->variances_averages, &bn->r_corrections, &bn->d_corrections,
+                                           &bn->derivatives_means, &bn->derivatives_variances};
+                        for (size_t a = 0; a < sizeof(small) / sizeof(small[0]); ++a) *small[a] = zalloc(T * bn->H);
+                        for (size_t a = 0; a < T * bn->H; ++a) bn->variances_averages[a] = 1.f;   /* NN/Neural_Network__Allocate.cpp:2612-2615 */
+                        bn->hats = zalloc(T * B * bn->H); bn->normalizes = zalloc(T * B * bn->H);
+                    }
+                    float **dc_[] = {&q->dz_in, &q->dz_rec}, **dk_[] = {&q->di_in, &q->di_rec, &q->df_in, &q->df_rec, &q->do_in, &q->do_rec};
+                    for (size_t a = 0; a < 2; ++a) *dc_[a] = zalloc(sc);
+                    for (size_t a = 0; a < 6; ++a) *dk_[a] = zalloc(sk);
+                }
             }
             o->lstm = qq;
             zone_at += T * qq[0].zone_stride;
@@ -399,6 +435,16 @@ int myea_oracle_destroy(myea_oracle_net *n)
                 float *all[] = {q->sum_in_z, q->sum_rec_z, q->sum_z, q->z, q->c, q->ca, q->dz, q->dc, q->sum_in_i, q->sum_in_f, q->sum_in_o, q->sum_rec_i,
                                 q->sum_rec_f, q->sum_rec_o, q->sum_i, q->sum_f, q->sum_o, q->gi, q->gf, q->go, q->di, q->df, q->dgo};
                 for (size_t a = 0; a < sizeof(all) / sizeof(all[0]); ++a) free(all[a]);
+                if (q->norm) {
+                    for (int g = 0; g < 9; ++g) {
+                        obn *bn = &q->nrm[g];
+                        float *bns[] = {bn->means, bn->variances, bn->means_averages, bn->variances_averages, bn->r_corrections, bn->d_corrections,
+                                        bn->derivatives_means, bn->derivatives_variances, bn->hats, bn->normalizes};
+                        for (size_t a = 0; a < sizeof(bns) / sizeof(bns[0]); ++a) free(bns[a]);
+                    }
+                    float *ds[] = {q->dz_in, q->dz_rec, q->di_in, q->di_rec, q->df_in, q->df_rec, q->do_in, q->do_rec};
+                    for (size_t a = 0; a < 8; ++a) free(ds[a]);
+                }
                 if (q->h != o->values) free(q->h);
                 if (q->dh != o->af_errors) free(q->dh);
             }
@@ -786,6 +832,80 @@ static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t t, size_t B
 }
 
 /* ------------------------------------------------------------------------------------------- */
+/* The same normalisation on one group of an LSTM layer's normalised units: training (:4591-4701 / :4703-4837), inference
+ * (:4559-4589), and the backward pass WITHOUT a shift gradient that the LSTM path calls
+ * (NN/Neural_Network__Backward_Pass__OpenMP.cpp:1469-1584, renormalised :1711-1829; dy and dx may be the same array). */
+static void lstm_bn_forward(myea_oracle_net *n, int renorm, obn *bn, size_t t, size_t B, const float *x)
+{
+    size_t Bmax = n->d.batch_size, H = bn->H, off = Bmax * H * t;
+    const float *scale = n->parameters + bn->param, *shift = scale + n->d.total_normalized_units;
+    const float *xt = x + off;
+    float *hat = bn->hats + off, *nor = bn->normalizes + off;
+    float *mavg = bn->means_averages + t * H, *vavg = bn->variances_averages + t * H;
+    if (n->state < MYEA_STATE_TRAINING) {
+        for (size_t b = 0; b < B; ++b)
+            for (size_t j = 0; j < H; ++j) nor[b * H + j] = scale[j] * ((xt[b * H + j] - mavg[j]) / vavg[j]) + shift[j];
+        return;
+    }
+    float *mean = bn->means + t * H, *var = bn->variances + t * H, *rc = bn->r_corrections + t * H, *dc = bn->d_corrections + t * H;
+    float bscale = 1.f / (float)B, eps = n->h.normalization_epsilon, mom = n->h.normalization_momentum_average;
+    float rmax = n->h.batch_renormalization_r_correction_maximum, dmax = n->h.batch_renormalization_d_correction_maximum;
+    for (size_t j = 0; j < H; ++j) { mean[j] = 0.f; var[j] = 0.f; }
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) { float v = xt[b * H + j]; mean[j] += v; var[j] += v * v; }
+    for (size_t j = 0; j < H; ++j) {
+        mean[j] *= bscale;
+        mavg[j] += mom * (mean[j] - mavg[j]);
+        var[j] = sqrtf(var[j] * bscale - mean[j] * mean[j] + eps);
+        vavg[j] += mom * (var[j] - vavg[j]);
+        if (renorm) {
+            float g = var[j] / vavg[j], lo = 1.f / rmax;
+            rc[j] = g < lo ? lo : (g > rmax ? rmax : g);
+            float dd = (mean[j] - mavg[j]) / vavg[j];
+            dc[j] = dd < -dmax ? -dmax : (dd > dmax ? dmax : dd);
+        }
+    }
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            float v = xt[b * H + j];
+            if (renorm) v = (v - mean[j]) / var[j] * rc[j] + dc[j];
+            else v = (v - mean[j]) / var[j];
+            hat[b * H + j] = v;
+            nor[b * H + j] = scale[j] * v + shift[j];
+        }
+}
+
+static void lstm_bn_backward(myea_oracle_net *n, int renorm, obn *bn, size_t t, size_t B, const float *x, float *d)
+{
+    size_t Bmax = n->d.batch_size, H = bn->H, off = Bmax * H * t;
+    const float *mean = bn->means + t * H, *var = bn->variances + t * H, *rc = bn->r_corrections + t * H;
+    const float *scale = n->parameters + bn->param;
+    float *dscale = n->gradient + bn->param;
+    float *dmean = bn->derivatives_means + t * H, *dvar = bn->derivatives_variances + t * H;
+    float bscale = 1.f / (float)B;
+    for (size_t j = 0; j < H; ++j) { dmean[j] = 0.f; dvar[j] = 0.f; }
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            size_t k = off + b * H + j;
+            float e = d[k], vb = var[j], r = renorm ? rc[j] : 1.f;
+            dscale[j] += e * bn->hats[k];
+            e *= scale[j];
+            dmean[j] += e * (-r / vb);
+            dvar[j] += e * (x[k] - mean[j]) * (-r / (vb * vb));
+            d[k] = e;
+        }
+    for (size_t b = 0; b < B; ++b)
+        for (size_t j = 0; j < H; ++j) {
+            size_t k = off + b * H + j;
+            float e = d[k], vb = var[j], r = renorm ? rc[j] : 1.f;
+            e *= r / vb;
+            e += dvar[j] * ((x[k] - mean[j]) / ((float)B * vb));
+            e += dmean[j] * bscale;
+            d[k] = e;
+        }
+}
+
+/* ------------------------------------------------------------------------------------------- */
 /* LSTM with peepholes (one direction, time ascending) */
 
 /* parameter offsets inside the layer's slice, NN/Neural_Network__Prepare_Connections.cpp:82-222: per block
@@ -888,6 +1008,95 @@ static void fwd_lstm_step(myea_oracle_net *n, size_t li, int dir, size_t t, size
     }
 }
 
+/* Forward_Pass__LSTM (NN/Neural_Network__Forward_Pass__OpenMP.cpp:1769-2340) of a normalised layer, one cell per block.
+ * The eight sums of Gates_CIFO are normalised group by group and the gate functions take the normalised values
+ * (Layer::Get__Array_Summations__*__Activation, NN/Neural_Network.cpp:4498-4613); the cell state is normalised before its
+ * activation, while the recurrence, the peepholes and the forget path keep the raw cell state.  At the direction's first
+ * step only groups 0, 3, 2 and 7 run (:1801-1829, :2014-2032, :2058-2074). */
+static void fwd_lstm_step_norm(myea_oracle_net *n, size_t li, int dir, size_t t, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    olstm *q = &o->lstm[dir];
+    size_t Bmax = n->d.batch_size, K = q->K, C = q->C, In = q->In;
+    const float *x = layer_outputs(n, n->L[li].prev), *w = n->parameters;
+    const float *bz = w + q->bias, *bi = bz + C, *bf = bi + K, *bo = bf + K;
+    size_t tp = q->reverse ? t + 1 : t - 1;
+    int first = q->reverse ? t == n->d.number_recurrent_depth - 1 : t == 0;
+    int zone = l->type_dropout == MYEA_DROPOUT_ZONEOUT && n->state == MYEA_STATE_TRAINING;
+    int renorm = l->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    long b;
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+    for (b = 0; b < (long)B; ++b) {   /* Gates_CIFO */
+        size_t kb = (size_t)b * K + Bmax * K * t, cp = (size_t)b * C + Bmax * C * tp;
+        const float *xi = x + (size_t)b * In + Bmax * In * t;
+        const float *hp = first ? NULL : q->h + cp;
+        for (size_t k = 0; k < K; ++k) {
+            float *in4[4] = {q->sum_in_z, q->sum_in_i, q->sum_in_f, q->sum_in_o}, *rec4[4] = {q->sum_rec_z, q->sum_rec_i, q->sum_rec_f, q->sum_rec_o};
+            for (int g = 0; g < 4; ++g) {
+                const float *wi = w + (g == 0 ? lstm_z_in(l, q, k, 0) : lstm_gate_in(l, q, k, g - 1));
+                float v = 0.f;
+                for (size_t a = 0; a < In; ++a) v += xi[a] * wi[a];
+                in4[g][kb + k] = v;
+                if (first) continue;
+                const float *wr = w + (g == 0 ? lstm_z_rec(l, q, k, 0) : lstm_gate_rec(l, q, k, g - 1));
+                v = 0.f;
+                for (size_t a = 0; a < C; ++a) v += hp[a] * wr[a];
+                rec4[g][kb + k] = v;
+            }
+        }
+    }
+    lstm_bn_forward(n, renorm, &q->nrm[0], t, B, q->sum_in_z);
+    lstm_bn_forward(n, renorm, &q->nrm[3], t, B, q->sum_in_i);
+    if (!first) {
+        lstm_bn_forward(n, renorm, &q->nrm[5], t, B, q->sum_in_f);
+        lstm_bn_forward(n, renorm, &q->nrm[1], t, B, q->sum_rec_z);
+        lstm_bn_forward(n, renorm, &q->nrm[4], t, B, q->sum_rec_i);
+        lstm_bn_forward(n, renorm, &q->nrm[6], t, B, q->sum_rec_f);
+    }
+    for (size_t bb = 0; bb < B; ++bb) {   /* Gates_CIF_AF_State on the normalised sums */
+        size_t kb = bb * K + Bmax * K * t, cp = bb * C + Bmax * C * tp;
+        for (size_t k = 0; k < K; ++k) {
+            const float *pi = w + lstm_peep(l, q, k, 0), *pf = w + lstm_peep(l, q, k, 1);
+            size_t c = kb + k;
+            if (!first) {
+                float si = q->nrm[3].normalizes[c] + q->nrm[4].normalizes[c] + bi[k];
+                float sf = q->nrm[5].normalizes[c] + q->nrm[6].normalizes[c] + bf[k];
+                si += q->c[cp + k] * pi[0]; sf += q->c[cp + k] * pf[0];
+                q->sum_i[c] = si; q->sum_f[c] = sf;
+                q->gi[c] = sigmoid_f(si); q->gf[c] = sigmoid_f(sf);
+            } else {
+                float si = q->nrm[3].normalizes[c] + bi[k];
+                q->sum_i[c] = si;
+                q->gi[c] = sigmoid_f(si);
+            }
+            float sz = first ? q->nrm[0].normalizes[c] + bz[k] : q->nrm[0].normalizes[c] + q->nrm[1].normalizes[c] + bz[k];
+            q->sum_z[c] = sz;
+            q->z[c] = tanh_f(sz);
+            q->c[c] = first ? q->z[c] * q->gi[c] : q->z[c] * q->gi[c] + q->gf[c] * q->c[cp + k];
+            if (zone && !q->zone_state[t * q->zone_stride + k]) q->c[c] = first ? 0.f : q->c[cp + k];
+        }
+    }
+    lstm_bn_forward(n, renorm, &q->nrm[2], t, B, q->c);
+    for (size_t bb = 0; bb < B; ++bb)   /* States_AF on the normalised cell state */
+        for (size_t k = 0; k < C; ++k) { size_t c = bb * C + Bmax * C * t + k; q->ca[c] = tanh_f(q->nrm[2].normalizes[c]); }
+    lstm_bn_forward(n, renorm, &q->nrm[7], t, B, q->sum_in_o);
+    if (!first) lstm_bn_forward(n, renorm, &q->nrm[8], t, B, q->sum_rec_o);
+    for (size_t bb = 0; bb < B; ++bb) {   /* Output */
+        size_t kb = bb * K + Bmax * K * t, cp = bb * C + Bmax * C * tp;
+        for (size_t k = 0; k < K; ++k) {
+            const float *po = w + lstm_peep(l, q, k, 2);
+            size_t c = kb + k;
+            float so = q->nrm[7].normalizes[c] + (first ? 0.f : q->nrm[8].normalizes[c]) + bo[k];
+            so += q->c[c] * po[0];
+            q->sum_o[c] = so;
+            q->go[c] = sigmoid_f(so);
+            q->h[c] = q->ca[c] * q->go[c];
+            if (zone && !q->zone_output[t * q->zone_stride + k]) q->h[c] = first ? 0.f : q->h[cp + k];
+        }
+    }
+}
+
 /* Backward_Pass__LSTM (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:1024-1120): delta to the layer below,
  * dst[t][b][:] += dz_c Wz_in[c][:] + di_k Wi_in[k][:] + df_k Wf_in[k][:] + do_k Wo_in[k][:] */
 static void bwd_lstm_to_previous_dir(myea_oracle_net *n, size_t gi, int dir, size_t t, size_t B, float *dst)
@@ -901,13 +1110,16 @@ static void bwd_lstm_to_previous_dir(myea_oracle_net *n, size_t gi, int dir, siz
     for (b = 0; b < (long)B; ++b) {
         size_t kb = (size_t)b * K + Bmax * K * t, cb = (size_t)b * C + Bmax * C * t;
         float *dx = dst + (size_t)b * In + Bmax * In * t;
+        /* a normalised layer hands down the deltas of its sums from below, after their normalisation's backward pass
+         * (Layer::Get__Array_Deltas__*__Input, NN/Neural_Network.cpp:4615-4717) */
+        const float *dzs = q->norm ? q->dz_in : q->dz;
         for (size_t k = 0; k < K; ++k) {
             for (size_t j = 0; j < cpb; ++j) {
-                float e = q->dz[cb + k * cpb + j];
+                float e = dzs[cb + k * cpb + j];
                 const float *wr = w + lstm_z_in(l, q, k, j);
                 for (size_t a = In; a--;) dx[a] += e * wr[a];
             }
-            const float *d3[3] = {q->di, q->df, q->dgo};
+            const float *d3[3] = {q->norm ? q->di_in : q->di, q->norm ? q->df_in : q->df, q->norm ? q->do_in : q->dgo};
             for (int g = 0; g < 3; ++g) {
                 float e = d3[g][kb + k];
                 const float *wr = w + lstm_gate_in(l, q, k, g);
@@ -941,14 +1153,15 @@ static void bwd_lstm_step(myea_oracle_net *n, size_t li, int dir, size_t t, size
         size_t kb = (size_t)b * K + Bmax * K * t, cb = (size_t)b * C + Bmax * C * t;
         size_t kn = (size_t)b * K + Bmax * K * tn, cn = (size_t)b * C + Bmax * C * tn, cp = (size_t)b * C + Bmax * C * tp;
         float *dh = q->dh + cb;
-        if (!last) { /* recurrent delta from t + 1 */
+        if (!last) { /* recurrent delta from t + 1: of the recurrent sums when the layer is normalised (Get__Array_Deltas__*__Recurrent) */
+            const float *rz = q->norm ? q->dz_rec : q->dz, *ri = q->norm ? q->di_rec : q->di, *rf = q->norm ? q->df_rec : q->df, *ro = q->norm ? q->do_rec : q->dgo;
             for (size_t c = 0; c < C; ++c) {
-                float e = q->dz[cn + c];
+                float e = rz[cn + c];
                 const float *wr = w + lstm_z_rec(l, q, c / cpb, c % cpb);
                 for (size_t a = 0; a < C; ++a) dh[a] += e * wr[a];
             }
             for (size_t k = 0; k < K; ++k) {
-                float ei = q->di[kn + k], ef = q->df[kn + k], eo = q->dgo[kn + k];
+                float ei = ri[kn + k], ef = rf[kn + k], eo = ro[kn + k];
                 const float *wi = w + lstm_gate_rec(l, q, k, 0), *wf = w + lstm_gate_rec(l, q, k, 1), *wo = w + lstm_gate_rec(l, q, k, 2);
                 for (size_t a = C; a--;) { float e = ei * wi[a]; e += ef * wf[a]; e += eo * wo[a]; dh[a] += e; }
             }
@@ -992,6 +1205,93 @@ static void bwd_lstm_step(myea_oracle_net *n, size_t li, int dir, size_t t, size
     }
 }
 
+/* The same time step of a normalised layer (one cell per block), NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:476-862:
+ * Output -> [output gate's delta copied to its two sums' deltas, each through its normalisation] -> Cell_State_AF ->
+ * [cell state's delta through its normalisation, in place] -> Gates_CIF_AF_State -> [block input, input gate and forget
+ * gate deltas copied to their sums' deltas, each through its normalisation].  The recurrent sums have no delta at the
+ * direction's first step, and there the forget gate's sum from below is copied but not passed through (:650-664, :706-741). */
+static void bwd_lstm_step_norm(myea_oracle_net *n, size_t li, int dir, size_t t, size_t B)
+{
+    const myea_layer_desc *l = &n->d.layers[li];
+    olayer *o = &n->L[li];
+    olstm *q = &o->lstm[dir];
+    size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, K = q->K, C = q->C;
+    const float *w = n->parameters;
+    size_t tn = q->reverse ? t - 1 : t + 1, tp = q->reverse ? t + 1 : t - 1;
+    int last = q->reverse ? t == 0 : t == T - 1, first = q->reverse ? t == T - 1 : t == 0;
+    int renorm = l->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    size_t row0 = Bmax * K * t, bytes = B * K * sizeof(float);
+    long b;
+#pragma omp parallel for schedule(static) num_threads(n->threads)
+    for (b = 0; b < (long)B; ++b) {
+        size_t kb = (size_t)b * K + row0, kn = (size_t)b * K + Bmax * K * tn;
+        float *dh = q->dh + kb;
+        if (!last) {
+            for (size_t c = 0; c < C; ++c) {
+                float e = q->dz_rec[kn + c];
+                const float *wr = w + lstm_z_rec(l, q, c, 0);
+                for (size_t a = 0; a < C; ++a) dh[a] += e * wr[a];
+            }
+            for (size_t k = 0; k < K; ++k) {
+                float ei = q->di_rec[kn + k], ef = q->df_rec[kn + k], eo = q->do_rec[kn + k];
+                const float *wi = w + lstm_gate_rec(l, q, k, 0), *wf = w + lstm_gate_rec(l, q, k, 1), *wo = w + lstm_gate_rec(l, q, k, 2);
+                for (size_t a = C; a--;) { float e = ei * wi[a]; e += ef * wf[a]; e += eo * wo[a]; dh[a] += e; }
+            }
+        }
+        for (size_t k = 0; k < K; ++k) {
+            float a = q->go[kb + k];
+            q->dgo[kb + k] = (1.f * a * (1.f - a)) * (dh[k] * q->ca[kb + k]);
+        }
+    }
+    memcpy(q->do_in + row0, q->dgo + row0, bytes);
+    lstm_bn_backward(n, renorm, &q->nrm[7], t, B, q->sum_in_o, q->do_in);
+    if (!first) {
+        memcpy(q->do_rec + row0, q->dgo + row0, bytes);
+        lstm_bn_backward(n, renorm, &q->nrm[8], t, B, q->sum_rec_o, q->do_rec);
+    }
+    for (size_t bb = 0; bb < B; ++bb)
+        for (size_t k = 0; k < K; ++k) {
+            size_t c = bb * K + row0 + k;
+            q->dc[c] = q->dh[c] * q->go[c] * (1.f * (1.f - q->ca[c] * q->ca[c]));
+        }
+    lstm_bn_backward(n, renorm, &q->nrm[2], t, B, q->c, q->dc);
+    if (!(first && last))
+        for (size_t bb = 0; bb < B; ++bb) {
+            size_t kb = bb * K + row0, kn = bb * K + Bmax * K * tn, cp = bb * C + Bmax * C * tp;
+            for (size_t k = 0; k < K; ++k) {
+                const float *pi = w + lstm_peep(l, q, k, 0), *pf = w + lstm_peep(l, q, k, 1), *po = w + lstm_peep(l, q, k, 2);
+                float gi_ = q->gi[kb + k];
+                float e = q->dc[kb + k];
+                e += po[0] * q->dgo[kb + k];
+                if (!last) {
+                    e += pi[0] * q->di[kn + k];
+                    e += pf[0] * q->df[kn + k];
+                    e += q->dc[kn + k] * q->gf[kn + k];
+                }
+                q->dc[kb + k] = e;
+                q->dz[kb + k] = e * gi_ * (1.f * (1.f - q->z[kb + k] * q->z[kb + k]));
+                q->di[kb + k] = (e * q->z[kb + k]) * (1.f * gi_ * (1.f - gi_));
+                if (!first) { float f = q->gf[kb + k]; q->df[kb + k] = (e * q->c[cp + k]) * (1.f * f * (1.f - f)); }
+            }
+        }
+    memcpy(q->dz_in + row0, q->dz + row0, bytes);
+    memcpy(q->di_in + row0, q->di + row0, bytes);
+    memcpy(q->df_in + row0, q->df + row0, bytes);
+    if (!first) {
+        memcpy(q->dz_rec + row0, q->dz + row0, bytes);
+        memcpy(q->di_rec + row0, q->di + row0, bytes);
+        memcpy(q->df_rec + row0, q->df + row0, bytes);
+    }
+    lstm_bn_backward(n, renorm, &q->nrm[0], t, B, q->sum_in_z, q->dz_in);
+    lstm_bn_backward(n, renorm, &q->nrm[3], t, B, q->sum_in_i, q->di_in);
+    if (!first) {
+        lstm_bn_backward(n, renorm, &q->nrm[5], t, B, q->sum_in_f, q->df_in);
+        lstm_bn_backward(n, renorm, &q->nrm[1], t, B, q->sum_rec_z, q->dz_rec);
+        lstm_bn_backward(n, renorm, &q->nrm[4], t, B, q->sum_rec_i, q->di_rec);
+        lstm_bn_backward(n, renorm, &q->nrm[6], t, B, q->sum_rec_f, q->df_rec);
+    }
+}
+
 /* Recurrent__Update_Derivative_Weight__LSTM (NN/Neural_Network__Recurrent_Update_Derivative_Weight__OpenMP.cpp:492-728)
  * and __LSTM__Bias (:730-776). */
 static void dw_lstm_dir(myea_oracle_net *n, size_t li, int dir, size_t B)
@@ -1003,6 +1303,14 @@ static void dw_lstm_dir(myea_oracle_net *n, size_t li, int dir, size_t B)
     const float *x = layer_outputs(n, n->L[li].prev);
     float *g = n->gradient;
     long kk;
+    /* a normalised layer: the weights from below take the deltas of the sums from below, the recurrent weights those of the
+     * recurrent sums, each after its normalisation's backward pass; the input and forget peepholes take the RECURRENT sums'
+     * deltas of the next step and the output peephole the delta of the output gate's sum FROM BELOW (the variables the
+     * reference's loop happens to hold at that point, :601-617, :688-696); the biases take the gates' own deltas (:730-776) */
+    const float *z_in = q->norm ? q->dz_in : q->dz, *z_rec = q->norm ? q->dz_rec : q->dz;
+    const float *i_in = q->norm ? q->di_in : q->di, *i_rec = q->norm ? q->di_rec : q->di;
+    const float *f_in = q->norm ? q->df_in : q->df, *f_rec = q->norm ? q->df_rec : q->df;
+    const float *o_in = q->norm ? q->do_in : q->dgo, *o_rec = q->norm ? q->do_rec : q->dgo;
     /* parallel over blocks: every parameter belongs to one block, so the per-parameter summation order (b, then t)
      * is the serial one */
 #pragma omp parallel for schedule(static) num_threads(n->threads)
@@ -1016,23 +1324,23 @@ static void dw_lstm_dir(myea_oracle_net *n, size_t li, int dir, size_t B)
                 const float *xi = x + b * In + Bmax * In * t, *h = q->h + cb;
                 for (size_t j = 0; j < cpb; ++j) {
                     size_t c = k * cpb + j;
-                    float e = q->dz[cb + c];
+                    float e = z_in[cb + c];
                     float *gw = g + lstm_z_in(l, q, k, j);
                     for (size_t a = 0; a < In; ++a) gw[a] += e * xi[a];
                     if (!last) {
-                        e = q->dz[cn + c];
+                        e = z_rec[cn + c];
                         gw = g + lstm_z_rec(l, q, k, j);
                         for (size_t a = 0; a < C; ++a) gw[a] += e * h[a];
                     }
                 }
-                float ei = q->di[kb + k], ef = q->df[kb + k], eo = q->dgo[kb + k];
+                float ei = i_in[kb + k], ef = f_in[kb + k], eo = o_in[kb + k];
                 float *gi_ = g + lstm_gate_in(l, q, k, 0), *gf_ = g + lstm_gate_in(l, q, k, 1), *go_ = g + lstm_gate_in(l, q, k, 2);
                 for (size_t a = 0; a < In; ++a) { gi_[a] += ei * xi[a]; gf_[a] += ef * xi[a]; go_[a] += eo * xi[a]; }
                 float *pi = g + lstm_peep(l, q, k, 0), *pf = g + lstm_peep(l, q, k, 1), *po = g + lstm_peep(l, q, k, 2);
                 if (!last) {
-                    ei = q->di[kn + k]; ef = q->df[kn + k];
+                    ei = i_rec[kn + k]; ef = f_rec[kn + k];
                     for (size_t j = 0; j < cpb; ++j) { float cs = q->c[cb + k * cpb + j]; pi[j] += ei * cs; pf[j] += ef * cs; po[j] += eo * cs; }
-                    eo = q->dgo[kn + k];
+                    eo = o_rec[kn + k];
                     gi_ = g + lstm_gate_rec(l, q, k, 0); gf_ = g + lstm_gate_rec(l, q, k, 1); go_ = g + lstm_gate_rec(l, q, k, 2);
                     for (size_t a = 0; a < C; ++a) { gi_[a] += ei * h[a]; gf_[a] += ef * h[a]; go_[a] += eo * h[a]; }
                 } else {
@@ -1065,7 +1373,7 @@ static void fwd_lstm_layer(myea_oracle_net *n, size_t li, size_t B)
     olayer *o = &n->L[li];
     size_t T = n->d.number_recurrent_depth, dirs = n->d.layers[li].use_bidirectional ? 2 : 1;
     for (size_t dir = 0; dir < dirs; ++dir)
-        for (size_t s = 0; s < T; ++s) fwd_lstm_step(n, li, (int)dir, dir ? T - 1 - s : s, B);
+        for (size_t s = 0; s < T; ++s) (o->lstm[dir].norm ? fwd_lstm_step_norm : fwd_lstm_step)(n, li, (int)dir, dir ? T - 1 - s : s, B);
     if (dirs == 2) {
         size_t cnt = T * n->d.batch_size * o->H;
         for (size_t i = 0; i < cnt; ++i) o->values[i] = o->lstm[0].h[i] + o->lstm[1].h[i];
@@ -1078,7 +1386,7 @@ static void bwd_lstm_layer(myea_oracle_net *n, size_t li, size_t B)
     size_t T = n->d.number_recurrent_depth, dirs = n->d.layers[li].use_bidirectional ? 2 : 1;
     for (size_t dir = 0; dir < dirs; ++dir) {
         if (dirs == 2) memcpy(o->lstm[dir].dh, o->af_errors, T * n->d.batch_size * o->H * sizeof(float));
-        for (size_t s = T; s-- > 0;) bwd_lstm_step(n, li, (int)dir, dir ? T - 1 - s : s, B);
+        for (size_t s = T; s-- > 0;) (o->lstm[dir].norm ? bwd_lstm_step_norm : bwd_lstm_step)(n, li, (int)dir, dir ? T - 1 - s : s, B);
     }
 }
 
@@ -1865,6 +2173,27 @@ const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t 
         olstm *q = &o->lstm[backward];
         kind &= ~MYEA_TENSOR_DIRECTION_BACKWARD;
         size_t cc = T * n->d.batch_size * q->C, kk = T * n->d.batch_size * q->K;
+        int group = (kind >> MYEA_TENSOR_LSTM_NORM_GROUP_SHIFT) & 15;   /* 1 + the group of normalised units, or 0 */
+        kind &= ~(15 << MYEA_TENSOR_LSTM_NORM_GROUP_SHIFT);
+        if (group) {
+            p = NULL;
+            if (q->norm && group <= 9) {
+                obn *bn = &q->nrm[group - 1];
+                float *deltas[9] = {q->dz_in, q->dz_rec, q->dc, q->di_in, q->di_rec, q->df_in, q->df_rec, q->do_in, q->do_rec};
+                size_t full_g = T * n->d.batch_size * bn->H, th_g = T * bn->H;
+                switch (kind) {
+                case MYEA_TENSOR_NORM_HATS: p = bn->hats; c = full_g; break;
+                case MYEA_TENSOR_NORM_MEANS: p = bn->means; c = th_g; break;
+                case MYEA_TENSOR_NORM_VARIANCES: p = bn->variances; c = th_g; break;
+                case MYEA_TENSOR_NORM_MEANS_AVERAGES: p = bn->means_averages; c = th_g; break;
+                case MYEA_TENSOR_NORM_VARIANCES_AVERAGES: p = bn->variances_averages; c = th_g; break;
+                case MYEA_TENSOR_ERRORS: p = deltas[group - 1]; c = full_g; break;
+                default: break;
+                }
+            }
+            if (count) *count = p ? c : 0;
+            return p;
+        }
         switch (kind) {
         case MYEA_TENSOR_LSTM_CELL_OUTPUT: p = q->h; c = cc; break;
         case MYEA_TENSOR_ERRORS: p = o->af_errors; c = cc; break;
