@@ -43,6 +43,20 @@ struct LstmLayer {
     float *dG = nullptr;    // [T][Bmax][G] deltas dz | di | df | do
     float *dc = nullptr;    // [T][Bmax][C]
     float *part = nullptr;  // split-K slabs of the per-step recurrent contractions, 16 x [Bmax][G]
+    // Normalised layer (one cell per block).  The eight gate sums and the cell state pass through their own normalisation at
+    // every time step (NN/Neural_Network__Forward_Pass__OpenMP.cpp:1769-2340): nine groups of normalised units, 0 block input
+    // from below, 1 block input recurrent, 2 cell state, 3 / 4 input gate, 5 / 6 forget gate, 7 / 8 output gate (from below /
+    // recurrent).  The sums stay packed as rows of [G] in the order z | i | f | o, separately for what comes from below and
+    // what is recurrent, as do their normalised values, their x-hats and - in the backward pass - their deltas; a group is a
+    // band of C columns of one of those tensors.  `acts` then holds the activations only.
+    bool norm = false, renorm = false;
+    size_t norm_param = 0;                   // flat index of the direction's first scale: [3 groups of C | 6 groups of K] in group order
+    float *sin = nullptr, *srec = nullptr;   // [T][Bmax][G] sums from below / recurrent sums
+    float *nin = nullptr, *nrec = nullptr;   // ... normalised
+    float *hin = nullptr, *hrec = nullptr;   // ... their x-hats
+    float *din = nullptr, *drec = nullptr;   // ... their deltas, after the backward pass through the normalisation
+    float *nc = nullptr, *hc = nullptr;      // [T][Bmax][C] normalised cell state and its x-hat
+    float *stats[9] = {};                    // per group 8 x [T][H]: mean, sigma, their running averages, r, d, d mean, d sigma
 };
 
 namespace {
@@ -275,8 +289,12 @@ __global__ __launch_bounds__(kBlock) void lstm_peep_final_kernel(LstmGeom g, siz
 // owns one cell and walks the time steps of its examples in the direction's processing order, carrying the cell state
 // of the step before (dp_i, dp_f pair the deltas of a step with the state of the step processed before it).
 // grid (ceil(C / 64), S); partial[(y * 7 + v) * C + cell], v = b_z, b_i, b_f, b_o, p_i, p_f, p_o.
+// A normalised layer takes the bias sums from the gates' own deltas (dG), the input and forget peepholes from the deltas of
+// the gates' recurrent sums (d_rec) and the output peephole from the delta of the output gate's sum from below (d_in); a plain
+// layer passes dG three times.
 __global__ __launch_bounds__(kBlock) void lstm_bias_peep_partial_kernel(size_t C, size_t B, size_t Bmax, size_t T, size_t per_lane, int reverse,
-                                                                        const float *__restrict__ c, const float *__restrict__ dG, float *partial)
+                                                                        const float *__restrict__ c, const float *__restrict__ dG,
+                                                                        const float *__restrict__ d_rec, const float *__restrict__ d_in, float *partial)
 {
     __shared__ double red[7][4][64];
     const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6;
@@ -294,7 +312,7 @@ __global__ __launch_bounds__(kBlock) void lstm_bias_peep_partial_kernel(size_t C
                 const float *d = dG + row * G + col;
                 const float dz = d[0], di = d[C], df = d[2 * C], dout = d[3 * C], cs = c[row * C + col];
                 acc[0] += dz; acc[1] += di; acc[2] += df; acc[3] += dout;
-                acc[4] += di * c_prev; acc[5] += df * c_prev; acc[6] += dout * cs;
+                acc[4] += d_rec[row * G + C + col] * c_prev; acc[5] += d_rec[row * G + 2 * C + col] * c_prev; acc[6] += d_in[row * G + 3 * C + col] * cs;
                 c_prev = cs;
             }
         }
@@ -338,6 +356,215 @@ __global__ __launch_bounds__(kBlock) void lstm_colsum_final_kernel(size_t H, siz
     out[col] += (float)s;
 }
 
+// ---- normalised layer ------------------------------------------------------------------------------------------------
+// One group of normalised units at one time step: a band of H columns of row-major tensors.  Forward_Pass__Batch_
+// Normalization__Training / __Batch_Renormalization__Training (NN/Neural_Network__Forward_Pass__OpenMP.cpp:4591-4837),
+// __Inference (:4559-4589); backward without a shift gradient, as the LSTM path calls it
+// (NN/Neural_Network__Backward_Pass__OpenMP.cpp:1469-1584, :1711-1829).
+struct NormBand {
+    const float *x; size_t ldx;            // what is normalised
+    float *hat, *nor; size_t ldo;          // x-hat and scale * x-hat + shift
+    float *d; size_t ldd;                  // backward: the delta, replaced in place
+    const float *scale, *shift;
+    float *dscale;                         // backward: accumulated
+    float *mean, *sigma, *mean_avg, *sigma_avg, *r, *dd, *dmean, *dsigma;   // [H] of the time step
+    int H;
+};
+constexpr int kMaxBands = 8;
+struct NormBands { NormBand g[kMaxBands]; int n; };
+struct NormHyper { float epsilon, momentum, r_max, d_max; int renorm; };
+
+// grid (ceil(H / 64), bands): column sums over the batch in double, four row lanes folded in a fixed order
+__global__ __launch_bounds__(kBlock) void lstm_norm_statistics_kernel(NormBands bands, size_t B, NormHyper hy)
+{
+    __shared__ double red[2][4][64];
+    const NormBand &g = bands.g[blockIdx.y];
+    const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6, col = blockIdx.x * 64 + cl;
+    double s1 = 0.0, s2 = 0.0;
+    if (col < g.H)
+        for (size_t b = rl; b < B; b += 4) { const float v = g.x[b * g.ldx + col]; s1 += v; s2 += (double)v * v; }
+    red[0][rl][cl] = s1; red[1][rl][cl] = s2;
+    __syncthreads();
+    if (rl != 0 || col >= g.H) return;
+    s1 = red[0][0][cl] + red[0][1][cl] + red[0][2][cl] + red[0][3][cl];
+    s2 = red[1][0][cl] + red[1][1][cl] + red[1][2][cl] + red[1][3][cl];
+    const float bscale = 1.f / (float)B;
+    const float mean = (float)s1 * bscale;
+    const float mavg = g.mean_avg[col] + hy.momentum * (mean - g.mean_avg[col]);
+    const float sigma = sqrtf((float)s2 * bscale - mean * mean + hy.epsilon);
+    const float vavg = g.sigma_avg[col] + hy.momentum * (sigma - g.sigma_avg[col]);
+    g.mean[col] = mean; g.sigma[col] = sigma; g.mean_avg[col] = mavg; g.sigma_avg[col] = vavg;
+    if (hy.renorm) {
+        const float q = sigma / vavg, lo = 1.f / hy.r_max;
+        g.r[col] = q < lo ? lo : (q > hy.r_max ? hy.r_max : q);
+        const float e = (mean - mavg) / vavg;
+        g.dd[col] = e < -hy.d_max ? -hy.d_max : (e > hy.d_max ? hy.d_max : e);
+    }
+}
+
+// grid (x, bands); training: x-hat and the normalised value from the batch statistics; inference: from the running averages
+__global__ __launch_bounds__(kBlock) void lstm_norm_apply_kernel(NormBands bands, size_t B, int training, int renorm)
+{
+    const NormBand &g = bands.g[blockIdx.y];
+    const size_t n = B * (size_t)g.H;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t b = i / g.H, col = i % g.H;
+        float v = g.x[b * g.ldx + col];
+        if (!training) { g.nor[b * g.ldo + col] = g.scale[col] * ((v - g.mean_avg[col]) / g.sigma_avg[col]) + g.shift[col]; continue; }
+        if (renorm) v = (v - g.mean[col]) / g.sigma[col] * g.r[col] + g.dd[col];
+        else v = (v - g.mean[col]) / g.sigma[col];
+        g.hat[b * g.ldo + col] = v;
+        g.nor[b * g.ldo + col] = g.scale[col] * v + g.shift[col];
+    }
+}
+
+// grid (ceil(H / 64), bands): the three column sums of the backward pass; the scale gradient accumulates
+__global__ __launch_bounds__(kBlock) void lstm_norm_backward_sums_kernel(NormBands bands, size_t B, int renorm)
+{
+    __shared__ double red[3][4][64];
+    const NormBand &g = bands.g[blockIdx.y];
+    const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6, col = blockIdx.x * 64 + cl;
+    double a1 = 0.0, a2 = 0.0, a3 = 0.0;
+    if (col < g.H) {
+        const float vb = g.sigma[col], r = renorm ? g.r[col] : 1.f, sc = g.scale[col], mean = g.mean[col];
+        const float k2 = -r / vb, k3 = -r / (vb * vb);
+        for (size_t b = rl; b < B; b += 4) {
+            float e = g.d[b * g.ldd + col];
+            a1 += e * g.hat[b * g.ldo + col];
+            e *= sc;
+            a2 += e * k2;
+            a3 += e * (g.x[b * g.ldx + col] - mean) * k3;
+        }
+    }
+    red[0][rl][cl] = a1; red[1][rl][cl] = a2; red[2][rl][cl] = a3;
+    __syncthreads();
+    if (rl != 0 || col >= g.H) return;
+    g.dscale[col] += (float)(red[0][0][cl] + red[0][1][cl] + red[0][2][cl] + red[0][3][cl]);
+    g.dmean[col] = (float)(red[1][0][cl] + red[1][1][cl] + red[1][2][cl] + red[1][3][cl]);
+    g.dsigma[col] = (float)(red[2][0][cl] + red[2][1][cl] + red[2][2][cl] + red[2][3][cl]);
+}
+
+__global__ __launch_bounds__(kBlock) void lstm_norm_backward_apply_kernel(NormBands bands, size_t B, int renorm)
+{
+    const NormBand &g = bands.g[blockIdx.y];
+    const size_t n = B * (size_t)g.H;
+    const float bscale = 1.f / (float)B;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        const size_t b = i / g.H, col = i % g.H;
+        const float vb = g.sigma[col], r = renorm ? g.r[col] : 1.f;
+        float e = g.d[b * g.ldd + col] * g.scale[col];
+        e *= r / vb;
+        e += g.dsigma[col] * ((g.x[b * g.ldx + col] - g.mean[col]) / ((float)B * vb));
+        e += g.dmean[col] * bscale;
+        g.d[b * g.ldd + col] = e;
+    }
+}
+
+// One lane per (example, cell), one cell per block.  Gates_CIF_AF_State on the normalised sums
+// (NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:1042-1191 with the operands of Layer::Get__Array_Summations__*__
+// Activation, NN/Neural_Network.cpp:4498-4613): the recurrence and the peepholes keep the raw cell state.
+__global__ __launch_bounds__(kBlock) void lstm_norm_gates_kernel(size_t C, size_t B, int first, const float *bias, const float *peep, const float *nin,
+                                                                 const float *nrec, const float *c_prev, float *acts, float *c, const uint8_t *zone_state)
+{
+    const size_t n = B * C, G = 4 * C;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < n; idx += (size_t)gridDim.x * kBlock) {
+        const size_t b = idx / C, k = idx % C;
+        const float *a = nin + b * G, *r = nrec + b * G;
+        float *row = acts + b * G;
+        float gi, gf = 0.f, sz;
+        if (!first) {
+            const float cp = c_prev[b * C + k];
+            float si = a[C + k] + r[C + k] + bias[C + k];
+            float sf = a[2 * C + k] + r[2 * C + k] + bias[2 * C + k];
+            si += cp * peep[k]; sf += cp * peep[C + k];
+            gi = sigmoid_f(si); gf = sigmoid_f(sf);
+            sz = a[k] + r[k] + bias[k];
+        } else {
+            gi = sigmoid_f(a[C + k] + bias[C + k]);
+            sz = a[k] + bias[k];
+        }
+        const float z = tanh_f(sz);
+        row[k] = z; row[C + k] = gi; row[2 * C + k] = gf;
+        float cs = first ? z * gi : z * gi + gf * c_prev[b * C + k];
+        if (zone_state && !zone_state[k]) cs = first ? 0.f : c_prev[b * C + k];
+        c[b * C + k] = cs;
+    }
+}
+
+// States_AF on the normalised cell state (:1547-1582) and Output (:1351-1418): the output gate peeps at the raw c[t]
+__global__ __launch_bounds__(kBlock) void lstm_norm_output_kernel(size_t C, size_t B, int first, const float *bias, const float *peep, const float *nin,
+                                                                  const float *nrec, const float *nc, const float *c, float *acts, float *ca, float *h,
+                                                                  const float *h_prev, const uint8_t *zone_output)
+{
+    const size_t n = B * C, G = 4 * C;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < n; idx += (size_t)gridDim.x * kBlock) {
+        const size_t b = idx / C, k = idx % C;
+        const float a = tanh_f(nc[b * C + k]);
+        ca[b * C + k] = a;
+        float so = nin[b * G + 3 * C + k] + (first ? 0.f : nrec[b * G + 3 * C + k]) + bias[3 * C + k];
+        so += c[b * C + k] * peep[2 * C + k];
+        const float go = sigmoid_f(so);
+        acts[b * G + 3 * C + k] = go;
+        float hv = a * go;
+        if (zone_output && !zone_output[k]) hv = first ? 0.f : h_prev[b * C + k];
+        h[b * C + k] = hv;
+    }
+}
+
+// Backward_Pass__LSTM_Derivative__Output (elementwise part) and __Cell_State_AF: the output gate's delta, copied to its two
+// sums' deltas, and the cell state's delta through tanh (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:476-575)
+__global__ __launch_bounds__(kBlock) void lstm_norm_backward_output_kernel(size_t C, size_t B, int first, const float *acts, const float *ca, float *dh,
+                                                                           const float *part, int nparts, float *dG, float *din, float *drec, float *dc)
+{
+    const size_t n = B * C, G = 4 * C;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < n; idx += (size_t)gridDim.x * kBlock) {
+        const size_t b = idx / C, k = idx % C;
+        float v = dh[b * C + k];
+        for (int s = 0; s < nparts; ++s) v += part[((size_t)s * B + b) * C + k];
+        if (nparts > 0) dh[b * C + k] = v;
+        const float go = acts[b * G + 3 * C + k], a = ca[b * C + k];
+        const float ddo = (go * (1.f - go)) * (v * a);
+        dG[b * G + 3 * C + k] = ddo;
+        din[b * G + 3 * C + k] = ddo;
+        if (!first) drec[b * G + 3 * C + k] = ddo;
+        dc[b * C + k] = v * go * (1.f - a * a);
+    }
+}
+
+// Backward_Pass__LSTM_Derivative__Gates_CIF_AF_State (:1329-1604) on the cell state's delta as its normalisation's backward
+// pass left it, then the copies to the sums' deltas (:612-664).  compute == 0 (a single time step): no branch of the
+// reference matches, the gate deltas keep their values and only the copies happen.
+__global__ __launch_bounds__(kBlock) void lstm_norm_backward_gates_kernel(size_t C, size_t B, int compute, int first, int last, const float *peep,
+                                                                          const float *acts, const float *acts_next, const float *c_prev, float *dG,
+                                                                          const float *dG_next, float *dc, const float *dc_next, float *din, float *drec)
+{
+    const size_t n = B * C, G = 4 * C;
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < n; idx += (size_t)gridDim.x * kBlock) {
+        const size_t b = idx / C, k = idx % C;
+        float *drow = dG + b * G;
+        if (compute) {
+            const float *row = acts + b * G;
+            const float z = row[k], gi = row[C + k];
+            float e = dc[b * C + k];
+            e += peep[2 * C + k] * drow[3 * C + k];
+            if (!last) {
+                e += peep[k] * dG_next[b * G + C + k];
+                e += peep[C + k] * dG_next[b * G + 2 * C + k];
+                e += dc_next[b * C + k] * acts_next[b * G + 2 * C + k];
+            }
+            dc[b * C + k] = e;
+            drow[k] = e * gi * (1.f - z * z);
+            drow[C + k] = (e * z) * (gi * (1.f - gi));
+            if (!first) { const float gf = row[2 * C + k]; drow[2 * C + k] = (e * c_prev[b * C + k]) * (gf * (1.f - gf)); }
+        }
+        for (int gate = 0; gate < 3; ++gate) {
+            const float v = drow[gate * C + k];
+            din[b * G + gate * C + k] = v;
+            if (!first) drec[b * G + gate * C + k] = v;
+        }
+    }
+}
+
 int dev_alloc_zero(float **p, size_t count)
 {
     void *q = nullptr;
@@ -372,7 +599,9 @@ int Net::lstm_create_layer(size_t li)
 {
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
-    if (layer_uses_norm(l)) { set_last_error("layer %zu: normalisation inside an LSTM layer is not on this path", li); return MYEA_E_UNSUPPORTED; }
+    // with more cells per block the reference's indices [3] .. [8] into the layer's normalised units (NN/Neural_Network.cpp:4498-4613)
+    // land on the second cell's units, not on the block's (they are laid out per block, NN/Neural_Network__Ordered.cpp:937-966)
+    if (layer_uses_norm(l) && l.n_cells_per_block != 1) { set_last_error("layer %zu: a normalised LSTM layer needs one cell per block", li); return MYEA_E_UNSUPPORTED; }
     if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_ZONEOUT) { set_last_error("layer %zu: dropout type %u on an LSTM layer is not on this path", li, l.type_dropout); return MYEA_E_UNSUPPORTED; }
     if (l.n_cells_per_block == 0) { set_last_error("layer %zu: LSTM needs at least one cell per block", li); return MYEA_E_INVALID; }
     const size_t T = d.number_recurrent_depth, B = d.batch_size;
@@ -411,7 +640,9 @@ int Net::lstm_create_layer(size_t li)
         MYEA_TRY(dev_alloc_zero(&q->Win, q->G * q->In));
         MYEA_TRY(dev_alloc_zero(&q->Wrec, q->G * q->C));
         MYEA_TRY(dev_alloc_zero(&q->peep, 3 * q->C));
-        q->fused = lstm_fused_supported(q->C, q->cpb) && !fused_lstm_disabled();
+        q->norm = layer_uses_norm(l);
+        q->renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+        q->fused = !q->norm && lstm_fused_supported(q->C, q->cpb) && !fused_lstm_disabled();
         if (q->fused) MYEA_TRY(dev_alloc_zero(&q->WrecT, q->C * q->G));
         MYEA_TRY(dev_alloc_zero(&q->gWin, kMaxSlabs * q->G * q->In));   // split-K slabs of the weight-gradient contractions
         MYEA_TRY(dev_alloc_zero(&q->gWrec, kMaxSlabs * q->G * q->C));
@@ -426,6 +657,17 @@ int Net::lstm_create_layer(size_t li)
             MYEA_TRY(dev_alloc_zero(&q->h, T * B * q->C));
             MYEA_TRY(dev_alloc_zero(&q->dh, T * B * q->C));
         } else { q->h = o.values; q->dh = o.neuron_errors; }
+        if (q->norm) {
+            q->norm_param = d.total_weights + d.total_bias + l.first_normalized_unit_index + dir * (3 * q->C + 6 * q->K);
+            if (l.first_normalized_unit_index + dirs * (3 * q->C + 6 * q->K) > d.total_normalized_units) { set_last_error("layer %zu: scale/shift slice leaves its region", li); return MYEA_E_INVALID; }
+            for (float **p : {&q->sin, &q->srec, &q->nin, &q->nrec, &q->hin, &q->hrec, &q->din, &q->drec}) MYEA_TRY(dev_alloc_zero(p, T * B * q->G));
+            for (float **p : {&q->nc, &q->hc}) MYEA_TRY(dev_alloc_zero(p, T * B * q->C));
+            for (int g = 0; g < 9; ++g) {
+                MYEA_TRY(dev_alloc_zero(&q->stats[g], 8 * T * q->C));
+                MYEA_TRY(launch_fill(0, q->stats[g] + 3 * T * q->C, T * q->C, 1.f));   // running sigma starts at 1, NN/Neural_Network__Allocate.cpp:2612-2615
+            }
+            MYEA_HIP_TRY(hipDeviceSynchronize());
+        }
     }
     // the widest layer sizes the buffer the members of a resident backward loop hand each other partial sums through
     if (o.lstm->fused && o.lstm->cpb == 1)
@@ -438,8 +680,10 @@ void Net::lstm_destroy_layer(DevLayer &o)
     for (LstmLayer **slot : {&o.lstm, &o.lstm2}) {
         LstmLayer *q = *slot;
         if (!q) continue;
-        float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin_own, q->gWrec_own, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr};
+        float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin_own, q->gWrec_own, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr,
+                        q->sin, q->srec, q->nin, q->nrec, q->hin, q->hrec, q->din, q->drec, q->nc, q->hc};
         for (float *p : all) if (p) (void)hipFree(p);
+        for (float *p : q->stats) if (p) (void)hipFree(p);
         delete q;
         *slot = nullptr;
     }
@@ -503,7 +747,7 @@ int Net::lstm_forward_inputs(size_t li, LstmLayer &q, size_t B)
         GemmParams g{};
         g.A = x + c * Bmax * q.In; g.lda = (long)q.In; g.a_k_contiguous = 1;
         g.B = q.Win; g.ldb = (long)q.In; g.b_k_contiguous = 1;
-        g.C = q.acts + c * Bmax * q.G; g.ldc = (long)q.G;
+        g.C = (q.norm ? q.sin : q.acts) + c * Bmax * q.G; g.ldc = (long)q.G;
         g.M = (int)rows; g.N = (int)q.G; g.K = (int)q.In;
         prof_begin(0);
         MYEA_TRY(launch_gemm(stream, g));
@@ -546,6 +790,128 @@ int Net::lstm_forward_step(LstmLayer &q, size_t B, size_t s)
                        acts_t, s ? q.c + tp * Bmax * q.C : nullptr, q.c + t * Bmax * q.C, q.ca + t * Bmax * q.C, q.h + t * Bmax * q.C,
                        q.part, nparts, s ? q.h + tp * Bmax * q.C : nullptr, zs, zo);
     MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+// the band of group `g` (0 .. 8) of a normalised layer at time step t
+static NormBand norm_band(const LstmLayer &q, float *parameters, float *gradient, size_t total_norm, int g, size_t t, size_t T, size_t Bmax)
+{
+    NormBand b{};
+    const size_t C = q.C, G = q.G, rows = t * Bmax;
+    const bool below = g == 0 || g == 3 || g == 5 || g == 7;
+    const size_t col = g == 2 ? 0 : (g < 2 ? 0 : (size_t)((g - 1) / 2) * C);   // z | i | f | o bands of the packed rows
+    if (g == 2) {
+        b.x = q.c + rows * C; b.ldx = C; b.hat = q.hc + rows * C; b.nor = q.nc + rows * C; b.ldo = C; b.d = q.dc + rows * C; b.ldd = C;
+    } else {
+        b.x = (below ? q.sin : q.srec) + rows * G + col; b.ldx = G;
+        b.hat = (below ? q.hin : q.hrec) + rows * G + col; b.nor = (below ? q.nin : q.nrec) + rows * G + col; b.ldo = G;
+        b.d = (below ? q.din : q.drec) + rows * G + col; b.ldd = G;
+    }
+    const size_t at = q.norm_param + (g < 3 ? (size_t)g * C : 3 * C + (size_t)(g - 3) * q.K);
+    b.scale = parameters + at; b.shift = parameters + at + total_norm; b.dscale = gradient + at;
+    float *st = q.stats[g] + t * C;
+    const size_t TH = T * C;
+    b.mean = st; b.sigma = st + TH; b.mean_avg = st + 2 * TH; b.sigma_avg = st + 3 * TH; b.r = st + 4 * TH; b.dd = st + 5 * TH; b.dmean = st + 6 * TH; b.dsigma = st + 7 * TH;
+    b.H = (int)C;
+    return b;
+}
+
+int Net::lstm_norm_forward_groups(LstmLayer &q, size_t B, size_t t, std::initializer_list<int> groups)
+{
+    NormBands bands{};
+    for (int g : groups) bands.g[bands.n++] = norm_band(q, parameters, gradient, d.total_normalized_units, g, t, d.number_recurrent_depth, d.batch_size);
+    if (bands.n == 0 || B == 0) return MYEA_OK;
+    const bool training = state >= MYEA_STATE_TRAINING;
+    const NormHyper hy{h.normalization_epsilon, h.normalization_momentum_average, h.batch_renormalization_r_correction_maximum,
+                       h.batch_renormalization_d_correction_maximum, q.renorm ? 1 : 0};
+    prof_begin(kProfNormalization);
+    if (training) {
+        hipLaunchKernelGGL(lstm_norm_statistics_kernel, dim3((unsigned)((q.C + 63) / 64), (unsigned)bands.n), dim3(kBlock), 0, stream, bands, B, hy);
+        MYEA_HIP_TRY(hipGetLastError());
+    }
+    hipLaunchKernelGGL(lstm_norm_apply_kernel, dim3(grid_for(B * q.C, kBlock, 2048), (unsigned)bands.n), dim3(kBlock), 0, stream, bands, B, training ? 1 : 0, q.renorm ? 1 : 0);
+    MYEA_HIP_TRY(hipGetLastError());
+    prof_end((double)bands.n * (double)B * (double)q.C * sizeof(float) * 3.0);
+    return MYEA_OK;
+}
+
+int Net::lstm_norm_backward_groups(LstmLayer &q, size_t B, size_t t, std::initializer_list<int> groups)
+{
+    NormBands bands{};
+    for (int g : groups) bands.g[bands.n++] = norm_band(q, parameters, gradient, d.total_normalized_units, g, t, d.number_recurrent_depth, d.batch_size);
+    if (bands.n == 0 || B == 0) return MYEA_OK;
+    prof_begin(kProfNormalization);
+    hipLaunchKernelGGL(lstm_norm_backward_sums_kernel, dim3((unsigned)((q.C + 63) / 64), (unsigned)bands.n), dim3(kBlock), 0, stream, bands, B, q.renorm ? 1 : 0);
+    MYEA_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(lstm_norm_backward_apply_kernel, dim3(grid_for(B * q.C, kBlock, 2048), (unsigned)bands.n), dim3(kBlock), 0, stream, bands, B, q.renorm ? 1 : 0);
+    MYEA_HIP_TRY(hipGetLastError());
+    prof_end((double)bands.n * (double)B * (double)q.C * sizeof(float) * 5.0);
+    return MYEA_OK;
+}
+
+// The s-th time step of a normalised layer: Forward_Pass__LSTM (NN/Neural_Network__Forward_Pass__OpenMP.cpp:1769-2340).
+// The output gate's two sums are normalised together with the others (they depend on nothing the step computes); at the
+// direction's first step only groups 0, 3, 2 and 7 run.
+int Net::lstm_forward_step_norm(LstmLayer &q, size_t B, size_t s)
+{
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, C = q.C, G = q.G;
+    const float *bias = parameters + q.bias;
+    const size_t t = q.reverse ? T - 1 - s : s, tp = q.reverse ? t + 1 : t - 1;
+    const bool first = s == 0;
+    const bool zone = q.zone_state != nullptr && state == MYEA_STATE_TRAINING;
+    const uint8_t *zs = zone ? q.zone_state + t * q.zone_stride : nullptr, *zo = zone ? q.zone_output + t * q.zone_stride : nullptr;
+    if (!first) {   // recurrent sums h[tp] Wrec^T
+        GemmParams g{};
+        g.A = q.h + tp * Bmax * C; g.lda = (long)C; g.a_k_contiguous = 1;
+        g.B = q.Wrec; g.ldb = (long)C; g.b_k_contiguous = 1;
+        g.C = q.srec + t * Bmax * G; g.ldc = (long)G;
+        g.M = (int)B; g.N = (int)G; g.K = (int)C;
+        MYEA_TRY(launch_gemm(stream, g));
+        MYEA_TRY(lstm_norm_forward_groups(q, B, t, {0, 3, 5, 1, 4, 6, 7, 8}));
+    } else {
+        MYEA_TRY(lstm_norm_forward_groups(q, B, t, {0, 3, 7}));
+    }
+    const unsigned grid = grid_for(B * C, kBlock, 8192);
+    hipLaunchKernelGGL(lstm_norm_gates_kernel, dim3(grid), dim3(kBlock), 0, stream, C, B, first ? 1 : 0, bias, q.peep, q.nin + t * Bmax * G, q.nrec + t * Bmax * G,
+                       first ? nullptr : q.c + tp * Bmax * C, q.acts + t * Bmax * G, q.c + t * Bmax * C, zs);
+    MYEA_HIP_TRY(hipGetLastError());
+    MYEA_TRY(lstm_norm_forward_groups(q, B, t, {2}));
+    hipLaunchKernelGGL(lstm_norm_output_kernel, dim3(grid), dim3(kBlock), 0, stream, C, B, first ? 1 : 0, bias, q.peep, q.nin + t * Bmax * G, q.nrec + t * Bmax * G,
+                       q.nc + t * Bmax * C, q.c + t * Bmax * C, q.acts + t * Bmax * G, q.ca + t * Bmax * C, q.h + t * Bmax * C,
+                       first ? nullptr : q.h + tp * Bmax * C, zo);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+// The same time step of the backward pass (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:476-862); s counts down.
+int Net::lstm_backward_step_norm(LstmLayer &q, size_t B, size_t s)
+{
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, C = q.C, G = q.G;
+    const size_t t = q.reverse ? T - 1 - s : s, tn = q.reverse ? t - 1 : t + 1, tp = q.reverse ? t + 1 : t - 1;
+    const bool last = s == T - 1, first = s == 0;
+    int nparts = 0;
+    if (!last) {   // dh[t] += (deltas of the recurrent sums of step tn) Wrec
+        GemmParams g{};
+        g.A = q.drec + tn * Bmax * G; g.lda = (long)G; g.a_k_contiguous = 1;
+        g.B = q.Wrec; g.ldb = (long)C; g.b_k_contiguous = 0;
+        g.C = q.part; g.ldc = (long)C;
+        g.M = (int)B; g.N = (int)C; g.K = (int)G;
+        nparts = gemm_split_k(g.M, g.N, g.K);
+        g.split_k = nparts; g.split_k_slab = (long)(B * C);
+        MYEA_TRY(launch_gemm(stream, g));
+    }
+    const unsigned grid = grid_for(B * C, kBlock, 8192);
+    hipLaunchKernelGGL(lstm_norm_backward_output_kernel, dim3(grid), dim3(kBlock), 0, stream, C, B, first ? 1 : 0, q.acts + t * Bmax * G, q.ca + t * Bmax * C,
+                       q.dh + t * Bmax * C, q.part, nparts, q.dG + t * Bmax * G, q.din + t * Bmax * G, q.drec + t * Bmax * G, q.dc + t * Bmax * C);
+    MYEA_HIP_TRY(hipGetLastError());
+    if (first) MYEA_TRY(lstm_norm_backward_groups(q, B, t, {7, 2}));
+    else MYEA_TRY(lstm_norm_backward_groups(q, B, t, {7, 8, 2}));
+    hipLaunchKernelGGL(lstm_norm_backward_gates_kernel, dim3(grid), dim3(kBlock), 0, stream, C, B, (first && last) ? 0 : 1, first ? 1 : 0, last ? 1 : 0, q.peep,
+                       q.acts + t * Bmax * G, last ? nullptr : q.acts + tn * Bmax * G, first ? nullptr : q.c + tp * Bmax * C, q.dG + t * Bmax * G,
+                       last ? nullptr : q.dG + tn * Bmax * G, q.dc + t * Bmax * C, last ? nullptr : q.dc + tn * Bmax * C, q.din + t * Bmax * G, q.drec + t * Bmax * G);
+    MYEA_HIP_TRY(hipGetLastError());
+    if (first) MYEA_TRY(lstm_norm_backward_groups(q, B, t, {0, 3}));
+    else MYEA_TRY(lstm_norm_backward_groups(q, B, t, {0, 3, 5, 1, 4, 6}));
     return MYEA_OK;
 }
 
@@ -606,6 +972,15 @@ int Net::lstm_forward_layer(size_t li, size_t B)
             const size_t rows = (size_t)d.number_recurrent_depth * d.batch_size;
             return launch_padded_add(stream, rows, o.H, o.lstm->h, o.H, 0, o.lstm2->h, o.H, 0, o.values);  // output = h_forward + h_backward
         }
+    }
+    if (o.lstm->norm) {   // a normalised layer: every step is a sequence of launches; the directions run one after the other
+        for (LstmLayer *q : {o.lstm, o.lstm2}) {
+            if (!q) continue;
+            MYEA_TRY(lstm_forward_inputs(li, *q, B));
+            for (size_t s = 0; s < T; ++s) MYEA_TRY(lstm_forward_step_norm(*q, B, s));
+        }
+        if (!o.lstm2) return MYEA_OK;
+        return launch_padded_add(stream, (size_t)d.number_recurrent_depth * d.batch_size, o.H, o.lstm->h, o.H, 0, o.lstm2->h, o.H, 0, o.values);
     }
     if (!o.lstm2) {
         MYEA_TRY(lstm_forward_inputs(li, *o.lstm, B));
@@ -699,6 +1074,14 @@ int Net::lstm_backward_layer(size_t li, size_t B)
             return MYEA_OK;
         }
     }
+    if (o.lstm->norm) {
+        for (LstmLayer *q : {o.lstm, o.lstm2}) {
+            if (!q) continue;
+            MYEA_TRY(seed(*q));
+            for (size_t s = T; s-- > 0;) MYEA_TRY(lstm_backward_step_norm(*q, B, s));
+        }
+        return MYEA_OK;
+    }
     if (!o.lstm2) {
         MYEA_TRY(seed(*o.lstm));
         if (T > 1) prof_begin(kProfLstmBackwardLoop);
@@ -730,7 +1113,7 @@ int Net::lstm_backward_layer(size_t li, size_t B)
 void Net::lstm_delta_source(size_t gi, int direction, const float **delta, size_t *width, const float **weights)
 {
     LstmLayer &q = direction ? *L[gi].lstm2 : *L[gi].lstm;
-    *delta = q.dG;
+    *delta = q.norm ? q.din : q.dG;   // a normalised layer hands down the deltas of its sums from below (Layer::Get__Array_Deltas__*__Input)
     *width = q.G;
     *weights = q.Win;
 }
@@ -759,10 +1142,13 @@ int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t
     // input weights: dG^T X over every (t, b).  M x N is small and K = T*B is long: split K into slabs so that the
     // launch fills the chip; the scatter kernel sums the slabs in order.
     int s_in = 1, s_rec = 0;
+    // a normalised layer: the weights from below take the deltas of the sums from below, the recurrent weights those of the
+    // recurrent sums (:563-598)
+    const float *d_below = q.norm ? q.din : q.dG, *d_rec = q.norm ? q.drec : q.dG;
     if (!per_t) {
         const size_t rows = T * B;
         GemmParams g{};
-        g.A = q.dG; g.lda = (long)q.G; g.a_k_contiguous = 0;
+        g.A = d_below; g.lda = (long)q.G; g.a_k_contiguous = 0;
         g.B = x; g.ldb = (long)q.In; g.b_k_contiguous = 0;
         g.C = q.gWin; g.ldc = (long)q.In;
         g.M = (int)q.G; g.N = (int)q.In; g.K = (int)rows;
@@ -774,7 +1160,7 @@ int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t
     } else {
         for (size_t c = 0; c < T; ++c) {
             GemmParams g{};
-            g.A = q.dG + c * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
+            g.A = d_below + c * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
             g.B = x + c * Bmax * q.In; g.ldb = (long)q.In; g.b_k_contiguous = 0;
             g.C = q.gWin; g.ldc = (long)q.In; g.accumulate = c > 0;
             g.M = (int)q.G; g.N = (int)q.In; g.K = (int)B;
@@ -788,7 +1174,7 @@ int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t
     if (T > 1 && !per_t) {
         const size_t rows = (T - 1) * B;
         GemmParams g{};
-        g.A = q.dG + dg_shift * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
+        g.A = d_rec + dg_shift * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
         g.B = q.h + h_shift * Bmax * q.C; g.ldb = (long)q.C; g.b_k_contiguous = 0;
         g.C = q.gWrec; g.ldc = (long)q.C;
         g.M = (int)q.G; g.N = (int)q.C; g.K = (int)rows;
@@ -801,7 +1187,7 @@ int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t
         s_rec = 1;
         for (size_t c = 0; c + 1 < T; ++c) {
             GemmParams g{};
-            g.A = q.dG + (c + dg_shift) * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
+            g.A = d_rec + (c + dg_shift) * Bmax * q.G; g.lda = (long)q.G; g.a_k_contiguous = 0;
             g.B = q.h + (c + h_shift) * Bmax * q.C; g.ldb = (long)q.C; g.b_k_contiguous = 0;
             g.C = q.gWrec; g.ldc = (long)q.C; g.accumulate = c > 0;
             g.M = (int)q.G; g.N = (int)q.C; g.K = (int)B;
@@ -829,7 +1215,7 @@ int Net::lstm_update_derivative_weight_reductions(LstmLayer &q, size_t B)
         const size_t per_lane = (B + 4 * S - 1) / (4 * S);
         S = (B + 4 * per_lane - 1) / (4 * per_lane);
         hipLaunchKernelGGL(lstm_bias_peep_partial_kernel, dim3((unsigned)colblocks, (unsigned)S), dim3(kBlock), 0, stream, q.C, B, Bmax, T, per_lane, q.reverse ? 1 : 0,
-                           q.c, q.dG, scratch);
+                           q.c, q.dG, q.norm ? q.drec : q.dG, q.norm ? q.din : q.dG, scratch);
         MYEA_HIP_TRY(hipGetLastError());
         hipLaunchKernelGGL(lstm_bias_peep_final_kernel, dim3(grid_for(7 * q.C, kBlock)), dim3(kBlock), 0, stream, geom, S, scratch, gradient + q.bias, gradient);
         MYEA_HIP_TRY(hipGetLastError());
@@ -869,6 +1255,26 @@ const float *Net::lstm_tensor(size_t li, int kind, size_t *count)
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, rows = T * Bmax;
     const float *src = nullptr;
     size_t width = 0, offset = 0, ld = 0;
+    const int group = (kind >> MYEA_TENSOR_LSTM_NORM_GROUP_SHIFT) & 15;   // 1 + the group of normalised units, or 0
+    kind &= ~(15 << MYEA_TENSOR_LSTM_NORM_GROUP_SHIFT);
+    if (group) {
+        if (!q->norm || group > 9) return nullptr;
+        const int g = group - 1;
+        const NormBand b = norm_band(*q, parameters, gradient, d.total_normalized_units, g, 0, T, Bmax);
+        const size_t TH = T * q->C;
+        switch (kind) {
+        case MYEA_TENSOR_NORM_MEANS: if (count) *count = TH; return b.mean;
+        case MYEA_TENSOR_NORM_VARIANCES: if (count) *count = TH; return b.sigma;
+        case MYEA_TENSOR_NORM_MEANS_AVERAGES: if (count) *count = TH; return b.mean_avg;
+        case MYEA_TENSOR_NORM_VARIANCES_AVERAGES: if (count) *count = TH; return b.sigma_avg;
+        case MYEA_TENSOR_NORM_HATS: src = b.hat; ld = b.ldo; break;
+        case MYEA_TENSOR_ERRORS: src = b.d; ld = b.ldd; break;
+        default: return nullptr;
+        }
+        if (hipMemcpy2DAsync(tmp1, q->C * sizeof(float), src, ld * sizeof(float), q->C * sizeof(float), rows, hipMemcpyDeviceToDevice, stream) != hipSuccess) return nullptr;
+        if (count) *count = rows * q->C;
+        return tmp1;
+    }
     switch (kind) {
     case MYEA_TENSOR_LSTM_CELL_OUTPUT: if (count) *count = rows * q->C; return q->h;
     case MYEA_TENSOR_LSTM_DELTA_CELL_OUTPUT: if (count) *count = rows * q->C; return q->dh;
@@ -889,6 +1295,23 @@ const float *Net::lstm_tensor(size_t li, int kind, size_t *count)
     if (hipMemcpy2DAsync(tmp1, width * sizeof(float), src + offset, ld * sizeof(float), width * sizeof(float), rows, hipMemcpyDeviceToDevice, stream) != hipSuccess) return nullptr;
     if (count) *count = rows * width;
     return tmp1;
+}
+
+// the running mean / sigma of one group of a normalised layer, writable (a checkpoint restores them)
+float *Net::lstm_norm_statistics(size_t li, int kind, size_t *count)
+{
+    if (count) *count = 0;
+    const bool backward = (kind & MYEA_TENSOR_DIRECTION_BACKWARD) != 0;
+    kind &= ~MYEA_TENSOR_DIRECTION_BACKWARD;
+    LstmLayer *q = backward ? L[li].lstm2 : L[li].lstm;
+    const int group = (kind >> MYEA_TENSOR_LSTM_NORM_GROUP_SHIFT) & 15;
+    kind &= ~(15 << MYEA_TENSOR_LSTM_NORM_GROUP_SHIFT);
+    if (!q || !q->norm || group < 1 || group > 9) return nullptr;
+    const size_t TH = d.number_recurrent_depth * q->C;
+    if (count) *count = TH;
+    if (kind == MYEA_TENSOR_NORM_MEANS_AVERAGES) return q->stats[group - 1] + 2 * TH;
+    if (kind == MYEA_TENSOR_NORM_VARIANCES_AVERAGES) return q->stats[group - 1] + 3 * TH;
+    return nullptr;
 }
 
 }  // namespace myea

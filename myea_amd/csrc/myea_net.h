@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <utility>
+#include <initializer_list>
 #include <vector>
 
 #include "../../include/myea_hip.h"
@@ -169,6 +170,12 @@ struct Net {
     int lstm_forward_step(LstmLayer &q, size_t B, size_t s);
     int lstm_resident_dirs(DevLayer &o, LstmResidentDir *dirs);   // the layer's directions as the resident kernels take them
     int lstm_backward_step(LstmLayer &q, size_t B, size_t s);
+    // a normalised layer's time steps, and the normalisation of a list of its nine groups of normalised units at one step
+    int lstm_forward_step_norm(LstmLayer &q, size_t B, size_t s);
+    int lstm_backward_step_norm(LstmLayer &q, size_t B, size_t s);
+    int lstm_norm_forward_groups(LstmLayer &q, size_t B, size_t t, std::initializer_list<int> groups);
+    int lstm_norm_backward_groups(LstmLayer &q, size_t B, size_t t, std::initializer_list<int> groups);
+    float *lstm_norm_statistics(size_t li, int kind, size_t *count);   // running averages of one group (kind carries the group)
     int lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t B);
     size_t lstm_scratch_floats() const;
     // packed weight-gradient slabs of all LSTM directions: their total size (each rounded up to 64 floats), and

@@ -1674,7 +1674,8 @@ int myea_hip_upload_tensor(myea_hip_net *n, size_t li, int kind, const float *ho
     if (!host || li >= n->net.d.n_layers) { myea::set_last_error("upload_tensor: null or layer %zu out of range", li); return MYEA_E_INVALID; }
     myea::DevLayer &o = n->net.L[li];
     float *p = kind == MYEA_TENSOR_NORM_MEANS_AVERAGES ? o.means_averages : (kind == MYEA_TENSOR_NORM_VARIANCES_AVERAGES ? o.variances_averages : nullptr);
-    const size_t want = (size_t)n->net.d.number_recurrent_depth * o.NH;
+    size_t want = (size_t)n->net.d.number_recurrent_depth * o.NH;
+    if (!p && o.lstm) p = n->net.lstm_norm_statistics(li, kind, &want);   // one group of a normalised LSTM layer
     if (!p) { myea::set_last_error("upload_tensor: layer %zu has no running statistics of kind %d", li, kind); return MYEA_E_INVALID; }
     if (count != want) { myea::set_last_error("upload_tensor: count %zu != %zu (T x normalised units)", count, want); return MYEA_E_INVALID; }
     MYEA_HIP_TRY(hipMemcpyAsync(p, host, count * sizeof(float), hipMemcpyHostToDevice, n->net.stream));

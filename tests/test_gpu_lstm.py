@@ -162,7 +162,8 @@ def test_lstm_error_paths():
         mb.HipNetwork(mb.make_desc([dict(units=3), dict(type="lstm", units=6), dict(units=2, activation="LINEAR")], 2, 3))
     assert e.value.code == mb.E_INVALID and "bias" in str(e.value)
     with pytest.raises(mb.MyeaError) as e:
-        mb.HipNetwork(mb.make_desc([dict(units=3), dict(type="lstm", units=2, normalization="BATCH_NORMALIZATION"), dict(units=8, activation="LINEAR")], 2, 3))
+        # a normalised layer with more than one cell per block: the reference's own indexing of the normalised units breaks there
+        mb.HipNetwork(mb.make_desc([dict(units=3), dict(type="lstm", units=2, cells_per_block=2, normalization="BATCH_NORMALIZATION"), dict(units=8, activation="LINEAR")], 2, 3))
     assert e.value.code == mb.E_UNSUPPORTED
 
 
