@@ -265,6 +265,15 @@ public:
         // running statistics a checkpoint brought along (Load)
         for (size_t li = 0; li < norm_means_averages_.size() && li < desc_.n_layers; ++li) {
             if (norm_means_averages_[li].empty()) continue;
+            if (desc_.layers[li].type_layer == MYEA_LAYER_LSTM) {   // held as [direction][group][T][K], uploaded group by group
+                const size_t per = (size_t)desc_.number_recurrent_depth * desc_.layers[li].n_units;
+                for (size_t dg = 0; dg * per < norm_means_averages_[li].size(); ++dg) {
+                    const int sel = MYEA_TENSOR_LSTM_NORM_GROUP((int)(dg % 9)) | (dg >= 9 ? MYEA_TENSOR_DIRECTION_BACKWARD : 0);
+                    if (!Ok("Set__HIP", myea_hip_upload_tensor(net_, li, MYEA_TENSOR_NORM_MEANS_AVERAGES | sel, norm_means_averages_[li].data() + dg * per, per)) ||
+                        !Ok("Set__HIP", myea_hip_upload_tensor(net_, li, MYEA_TENSOR_NORM_VARIANCES_AVERAGES | sel, norm_variances_averages_[li].data() + dg * per, per))) return false;
+                }
+                continue;
+            }
             if (!Ok("Set__HIP", myea_hip_upload_tensor(net_, li, MYEA_TENSOR_NORM_MEANS_AVERAGES, norm_means_averages_[li].data(), norm_means_averages_[li].size())) ||
                 !Ok("Set__HIP", myea_hip_upload_tensor(net_, li, MYEA_TENSOR_NORM_VARIANCES_AVERAGES, norm_variances_averages_[li].data(), norm_variances_averages_[li].size()))) return false;
         }
@@ -531,7 +540,7 @@ private:
         ptr_last_layer = ptr_array_layers ? ptr_array_layers + total_layers : nullptr;
     }
     std::vector<T_> rows_;
-    std::vector<std::vector<T_>> norm_means_averages_, norm_variances_averages_;   // per layer [T][units], from a checkpoint
+    std::vector<std::vector<T_>> norm_means_averages_, norm_variances_averages_;   // per layer [T][units] ([direction][group][T][K] for an LSTM layer), from a checkpoint
     T_ r_mean_desired_ = 0.f, r_mean_predicted_ = 0.f;
 
     static bool Fail(const char *fn, const char *what) { std::printf("%s: ERROR: %s.\n", fn, what); return false; }

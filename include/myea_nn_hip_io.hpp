@@ -177,9 +177,21 @@ inline bool Neural_Network_HIP::Save_Dimension_Parameters(std::string const &pat
     std::vector<size_t> first_norm(L, 0);
     for (size_t li = 0; li < L; ++li) {
         first_norm[li] = norm_at; norm_at += norm_units[li];
-        if (desc_.layers[li].type_normalization == MYEA_NORMALIZATION_NONE || desc_.layers[li].type_layer == MYEA_LAYER_LSTM) continue;
+        if (desc_.layers[li].type_normalization == MYEA_NORMALIZATION_NONE) continue;
         mean[li].assign(T * norm_units[li], 0.f); var[li].assign(T * norm_units[li], 1.f);
         if (li < norm_means_averages_.size() && norm_means_averages_[li].size() == mean[li].size()) { mean[li] = norm_means_averages_[li]; var[li] = norm_variances_averages_[li]; }
+        if (desc_.layers[li].type_layer == MYEA_LAYER_LSTM) {
+            // a normalised LSTM layer (one cell per block): nine groups of K units per direction, held as [direction][group][T][K]
+            if (desc_.layers[li].n_cells_per_block != 1) return Fail("Save_Dimension_Parameters", "a normalised LSTM layer needs one cell per block");
+            const size_t K = desc_.layers[li].n_units;
+            for (size_t dg = 0; net_ && dg < 9 * dirs(li); ++dg) {
+                const int sel = MYEA_TENSOR_LSTM_NORM_GROUP((int)(dg % 9)) | (dg >= 9 ? MYEA_TENSOR_DIRECTION_BACKWARD : 0);
+                if (myea_hip_download_tensor(net_, li, MYEA_TENSOR_NORM_MEANS_AVERAGES | sel, mean[li].data() + dg * T * K, T * K) != MYEA_OK ||
+                    myea_hip_download_tensor(net_, li, MYEA_TENSOR_NORM_VARIANCES_AVERAGES | sel, var[li].data() + dg * T * K, T * K) != MYEA_OK)
+                    return Fail("Save_Dimension_Parameters", myea_hip_last_error());
+            }
+            continue;
+        }
         if (net_ && (myea_hip_download_tensor(net_, li, MYEA_TENSOR_NORM_MEANS_AVERAGES, mean[li].data(), mean[li].size()) != MYEA_OK ||
                      myea_hip_download_tensor(net_, li, MYEA_TENSOR_NORM_VARIANCES_AVERAGES, var[li].data(), var[li].size()) != MYEA_OK))
             return Fail("Save_Dimension_Parameters", myea_hip_last_error());
@@ -216,11 +228,21 @@ inline bool Neural_Network_HIP::Save_Dimension_Parameters(std::string const &pat
         for (size_t u = 0; u < norm_units[li]; ++u) {
             s += "        NormU["; s += str(u); s += "]\n";
             const bool held = total_norm != 0 && !mean[li].empty();
-            line("          ", "scale", TS(held ? P[scale_at + l.first_normalized_unit_index + u] : 1.f));
-            line("          ", "shift", TS(held ? P[scale_at + total_norm + l.first_normalized_unit_index + u] : 0.f));
+            // where unit u keeps its scale, and its statistics of step t.  An LSTM layer's units are written block by block, the
+            // cell's three then the block's six (Neural_Network__Ordered.cpp:937-966), while their parameters and statistics are
+            // held group by group; the [t] entries carry the group's own statistics of step t (the reference's writer steps through
+            // them with the layer's unit count instead of the group's, Neural_Network__Save.cpp:695, so that for t > 0 its own file
+            // does not hold what its forward pass used: nothing to follow there).
+            size_t slot = u, stat0 = u, stat_stride = norm_units[li];
+            if (l.type_layer == MYEA_LAYER_LSTM) {
+                const size_t K = l.n_units, dir = u / (9 * K), k = (u % (9 * K)) / 9, g = u % 9;
+                slot = dir * 9 * K + g * K + k; stat0 = (dir * 9 + g) * T * K + k; stat_stride = K;
+            }
+            line("          ", "scale", TS(held ? P[scale_at + l.first_normalized_unit_index + slot] : 1.f));
+            line("          ", "shift", TS(held ? P[scale_at + total_norm + l.first_normalized_unit_index + slot] : 0.f));
             for (size_t t = 0; t < T; ++t) {
-                line("          ", "mean_average[" + str(t) + "]", TS(held ? mean[li][t * norm_units[li] + u] : 0.f));
-                line("          ", "variance_average[" + str(t) + "]", TS(held ? var[li][t * norm_units[li] + u] : 1.f));
+                line("          ", "mean_average[" + str(t) + "]", TS(held ? mean[li][t * stat_stride + stat0] : 0.f));
+                line("          ", "variance_average[" + str(t) + "]", TS(held ? var[li][t * stat_stride + stat0] : 1.f));
             }
         }
     };
@@ -542,6 +564,20 @@ inline bool Neural_Network_HIP::Load(std::string const &path_dimension, std::str
         const myea_layer_desc &l = desc_.layers[li];
         const size_t at = desc_.total_weights + desc_.total_bias + l.first_normalized_unit_index;
         if (desc_.total_normalized_units == 0 || l.first_normalized_unit_index + n.scale.size() > desc_.total_normalized_units) return Fail(fn, "dimension parameters: normalised units overflow");
+        if (l.type_layer == MYEA_LAYER_LSTM) {   // units written block by block, held group by group: see the writer
+            if (l.n_cells_per_block != 1) return Fail(fn, "dimension parameters: a normalised LSTM layer needs one cell per block");
+            const size_t K = l.n_units, units = n.scale.size();
+            norm_means_averages_[li].assign(T * units, 0.f); norm_variances_averages_[li].assign(T * units, 1.f);
+            for (size_t u = 0; u < units; ++u) {
+                const size_t dir = u / (9 * K), k = (u % (9 * K)) / 9, g = u % 9, slot = dir * 9 * K + g * K + k;
+                ptr_array_parameters[at + slot] = n.scale[u]; ptr_array_parameters[at + desc_.total_normalized_units + slot] = n.shift[u];
+                for (size_t t = 0; t < T; ++t) {
+                    norm_means_averages_[li][((dir * 9 + g) * T + t) * K + k] = n.mean[t * units + u];
+                    norm_variances_averages_[li][((dir * 9 + g) * T + t) * K + k] = n.var[t * units + u];
+                }
+            }
+            continue;
+        }
         for (size_t k = 0; k < n.scale.size(); ++k) { ptr_array_parameters[at + k] = n.scale[k]; ptr_array_parameters[at + desc_.total_normalized_units + k] = n.shift[k]; }
         norm_means_averages_[li] = n.mean; norm_variances_averages_[li] = n.var;
     }

@@ -1,7 +1,7 @@
 // Host program for the checkpoint tests: builds a network through the adaptor, optionally trains it for two steps on the
 // device, writes the reference's two text files, reads them into a second object, writes them again and compares - the
 // files byte for byte, and with a device the inference outputs of both objects bit for bit.
-// usage: checkpoint_check <dir> <kind> [device]      kinds: mlp, recurrent, residual
+// usage: checkpoint_check <dir> <kind> [device]      kinds: mlp, recurrent, normalised, residual
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -61,6 +61,16 @@ static bool build(Neural_Network_HIP &nn, const std::string &kind, size_t B, siz
         nn.learning_rate = 0.02f; nn.learning_momentum = 0.5f; nn.use_Nesterov = true; nn.Set__Clip_Gradient(true); nn.clip_gradient = 2.5f;
         nn.use_Warm_Restarts = true; nn.warm_restarts_initial_maximum_learning_rate = nn.warm_restarts_maximum_learning_rate = 0.5f;
         nn.warm_restarts_initial_T_i = nn.warm_restarts_T_i = 8.f; nn.warm_restarts_multiplier = 3.f; nn.regularization__max_norm_constraints = 4.f;
+    } else if (kind == "normalised") {   // 5 -> LSTM 6 blocks of one cell, batch renormalisation -> 6 linear, T = 3
+        *T = 3; *n_in = 5; *n_out = 6;
+        Layer_Parameters layers[3];
+        layers[0].type_layer = MYEA_LAYER_FULLY_CONNECTED; layers[0].unit_parameters[0] = 5;
+        layers[1].type_layer = MYEA_LAYER_LSTM; layers[1].unit_parameters[0] = 6; layers[1].unit_parameters[1] = 1;
+        layers[2].type_layer = MYEA_LAYER_FULLY_CONNECTED; layers[2].unit_parameters[0] = 6;
+        if (!nn.Compile(3, *T, MYEA_NETWORK_RECURRENT, layers)) return false;
+        if (!nn.Set__Layer_Activation_Function(2, MYEA_AF_LINEAR) || !nn.Set__Layer_Normalization(1, MYEA_NORMALIZATION_BATCH_RENORMALIZATION)) return false;
+        nn.Set__Loss_Function(MYEA_LOSS_MSE); nn.Set__Optimizer_Function(MYEA_OPTIMIZER_ADAM);
+        nn.normalization_momentum_average = 0.5f; nn.batch_renormalization_r_correction_maximum = 2.f; nn.batch_renormalization_d_correction_maximum = 1.f;
     } else {   // 8 -> 12 tanh -> residual block of 2 (block BN, ShakeDrop; members 10 and 14: wider than the shortcut) -> 4 linear
         *T = 1; *n_in = 8; *n_out = 4;
         Layer_Parameters layers[6];

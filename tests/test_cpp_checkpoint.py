@@ -71,6 +71,17 @@ def _check_files(tmp_path, kind):
         assert "          connected_to_cell 0" in lines and "        connected_to_AF_Ind_R 0" in lines and "    number_block_units 4" in lines and "    number_cell_units 8" in lines
         assert "    constraint_recurrent_weight_upper_bound 0.75" in lines and "number_time_delays 1" in lines
         assert "    number_bias_parameters 12" in lines              # an LSTM layer writes its 3 x blocks gate biases
+    if kind == "normalised":
+        # 6 blocks of one cell: 54 normalised units, written block by block (the cell's three, then the block's six)
+        assert "      number_normalized_units 54" in lines and "        NormU[53]" in lines and sum(l.split()[:1] == ["mean_average[2]"] for l in lines) == 54
+        at = lines.index("        NormU[0]")
+        p = np.fromfile(str(tmp_path / "params.bin"), dtype=np.float32)
+        head = [l.split() for l in lines if l.startswith("total_weights") or l.startswith("total_bias")]
+        base = int(head[0][1]) + int(head[1][1]) + 5   # the input layer's five units come first in the scale region
+        scales = [np.float32(l.split()[1]) for l in lines[at:] if l.split()[:1] == ["scale"]]
+        assert len(scales) == 54
+        for u, v in enumerate(scales):   # unit u = 9 * block + group keeps its scale at group * 6 + block
+            assert v == p[base + (u % 9) * 6 + u // 9], u
     if kind == "residual":
         assert "    block_depth 2" in lines and "    padding 1" in lines and "    number_basic_units 14" in lines and "          connected_to_basic 0" in lines
     # every weight line carries its flat index: the values are the parameters at those indices
@@ -85,14 +96,14 @@ def _check_files(tmp_path, kind):
     assert seen > 100
 
 
-@pytest.mark.parametrize("kind", ["mlp", "recurrent", "residual"])
+@pytest.mark.parametrize("kind", ["mlp", "recurrent", "normalised", "residual"])
 def test_checkpoint_round_trip_on_the_host(tmp_path, kind):
     _run(tmp_path, kind, device=False)
     _check_files(tmp_path, kind)
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kind", ["mlp", "recurrent", "residual"])
+@pytest.mark.parametrize("kind", ["mlp", "recurrent", "normalised", "residual"])
 def test_checkpoint_round_trip_through_the_device(tmp_path, kind):
     out = _run(tmp_path, kind, device=True)
     assert "inference outputs" in out and "differing 0 magnitude" in out
