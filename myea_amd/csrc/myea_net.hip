@@ -438,11 +438,12 @@ int Net::refresh_colscale(size_t li, bool *active)
 // ---- forward ----------------------------------------------------------------------------------------------
 // Forward_Pass__FC (layer driver), NN/Neural_Network__Forward_Pass__OpenMP.cpp:256-698:
 // GEMM -> bias -> [BN before] -> activation / softmax -> [BN after] -> dropout.
-// MYEA_BN_SUMS_FROM_GEMM=0 in the environment keeps the normalisation's column sums in kernels of their own (for A / B runs)
-static bool bn_sums_from_gemm()
+// MYEA_BN_SUMS_FROM_GEMM=0 in the environment keeps the normalisation's column sums in kernels of their own, =f / =b takes them
+// from the contraction in the forward / backward pass only (for A / B runs)
+static bool bn_sums_from_gemm(bool backward = false)
 {
-    static const bool off = [] { const char *e = std::getenv("MYEA_BN_SUMS_FROM_GEMM"); return e && e[0] == '0'; }();
-    return !off;
+    static const int mode = [] { const char *e = std::getenv("MYEA_BN_SUMS_FROM_GEMM"); return !e || !*e ? 3 : e[0] == '0' ? 0 : e[0] == 'f' ? 1 : e[0] == 'b' ? 2 : 3; }();
+    return (mode & (backward ? 2 : 1)) != 0;
 }
 
 int Net::forward_fc_layer(size_t li, size_t B)
@@ -872,7 +873,7 @@ int Net::backward_into_layer(size_t li, size_t B)
             g.C = tmp1 + roff * H;
             g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.normalizes + roff * H; g.val = o.values + roff * H;
             // the sums the normalisation's backward pass starts with leave with the contraction's tiles
-            if (fuse && o.norm_partials && bn_sums_from_gemm() && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H) {
+            if (fuse && o.norm_partials && bn_sums_from_gemm(true) && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H) {
                 g.col_partials = o.norm_partials; g.hats = o.hats + roff * H;
             }
         } else {
