@@ -267,6 +267,7 @@ struct LstmResidentPlan {
     bool agent = false;    // groups wider than one XCD: device-scope exchange
     bool backward = false; // the backward loop has a resident form too
     bool ksplit = false;   // ... and it is the one split along k, which needs the exchange buffer
+    bool ksplit_available = false;   // the k form exists for this layer (a caller may set ksplit when other work shares the device)
     int cells = 0, members = 0, rs = 0, row_groups = 0, grid = 0, cus = 0;
 };
 int lstm_resident_plan(size_t C, size_t cells_per_block, size_t B, int dirs, LstmResidentPlan *plan);

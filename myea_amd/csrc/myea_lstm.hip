@@ -1064,6 +1064,8 @@ int Net::lstm_backward_layer(size_t li, size_t B)
         const int dirs = o.lstm2 ? 2 : 1;
         MYEA_TRY(lstm_resident_plan(o.lstm->C, o.lstm->cpb, B, dirs, &plan));
         if (plan.ok && plan.backward) {   // the whole backward time loop (both directions) as one launch
+            // weight contractions are about to run beside this loop: the form that leaves them room in LDS
+            if (loop_shares_device && plan.ksplit_available) plan.ksplit = true;
             MYEA_TRY(seed(*o.lstm));
             if (o.lstm2) MYEA_TRY(seed(*o.lstm2));
             LstmResidentDir rd[2];

@@ -773,6 +773,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_ksplit_ker
     check_same_xcd(w, group);
     if (threadIdx.x < 2) s_arrive[threadIdx.x] = 0u;
     __syncthreads();
+    __builtin_amdgcn_s_setprio(3);   // ahead of the wavefronts of a contraction that shares the compute unit: the loop is the critical path
 
     // the weights of the member's 64 k's (k = gate * 16 + cell: row gate * C + c0 + cell of Wrec [4C][C]) against the
     // wavefront's columns, as the A operand of the transposed product: lane (col16, quad) holds Wrec[k = 4 ks + quad][16 ct + col16]
@@ -1028,6 +1029,8 @@ unsigned spin_polls()
 // against 523; 256 x 512: 405 against 392), with half of them or fewer the k form does (512 x 64: 408 against 450;
 // 256 x 128: 236 against 267; 128 x 256: 179 against 190) - its exchange is lighter, but what bounds both under full load
 // is the tail latency of the operands streamed from memory, which stalls a group at one more barrier per step in the k form.
+// The k form needs 17 KB of LDS where the column form needs 140: it is also the one a contraction's workgroups fit beside
+// on a compute unit, so a caller that runs weight contractions next to the loop asks for it (plan.ksplit_available).
 // MYEA_LSTM_BACKWARD_KSPLIT=0 / 1 forces the column form / the k form wherever it exists.
 int ksplit_choice()   // -1: by occupancy, 0: never, 1: always
 {
@@ -1231,9 +1234,10 @@ int lstm_resident_plan(size_t C, size_t cells_per_block, size_t B, int dirs, Lst
         const int choice = ksplit_choice();
         KernelInfo *split = choice == 0 ? nullptr : kernel_for(C, rs, true, true);
         bool ksplit = split && !agent && fwd->cells == 16 && place_groups(*dev, *split, members, agent, groups, &grid_b) && grid_b == grid;
+        const bool ksplit_available = ksplit;
         if (ksplit && backward && choice < 0) ksplit = 2 * groups * members <= dev->cus;
         backward = backward || ksplit;
-        plan->ok = true; plan->agent = agent; plan->backward = backward; plan->ksplit = ksplit;
+        plan->ok = true; plan->agent = agent; plan->backward = backward; plan->ksplit = ksplit; plan->ksplit_available = ksplit_available && choice != 0;
         plan->cells = fwd->cells; plan->members = members; plan->rs = rs; plan->row_groups = row_groups; plan->grid = grid; plan->cus = dev->cus;
         break;
     }

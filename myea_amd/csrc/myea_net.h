@@ -151,6 +151,10 @@ struct Net {
     std::vector<char> dw_done;         // per layer: the weight contraction already ran in this pass
     bool fc_dw_params(size_t li, size_t B, GemmParams *g);   // false: the layer's weight gradient is not one plain contraction
     int update_derivative_weight(size_t B, size_t first, size_t end);
+    int update_derivative_weight_contraction(size_t li, size_t B);   // the weight contraction(s) of one layer
+    bool dw_beside_loop_allowed(size_t gi, size_t li, size_t B);
+    bool dw_beside_loop = false;       // this pass put weight contractions on the side stream beside a time loop: join before returning
+    bool loop_shares_device = false;   // set around a time loop that weight contractions will run beside
     // the same call with every scratch buffer of its kernels taken from the library's static device array
     int update_derivative_weight_no_alloc(size_t B, size_t first, size_t end);
     int update_parameter(size_t B, size_t training_size);

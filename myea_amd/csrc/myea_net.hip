@@ -1024,6 +1024,8 @@ int Net::backward_pass_and_update_derivative_weight(size_t B)
     int rc = backward_pass(B);
     pairing = false;
     if (rc == MYEA_OK) rc = update_derivative_weight(B, 1, d.n_layers);
+    if (rc == MYEA_OK && dw_beside_loop) rc = side_stream_join();
+    dw_beside_loop = false;
     dw_done.assign(d.n_layers, 0);
     return rc;
 }
@@ -1038,8 +1040,27 @@ int Net::backward_pass(size_t B)
     for (size_t gi = d.n_layers - 1; gi != 1; --gi) {
         const size_t li = L[gi].prev;
         MYEA_TRY(backward_into_layer(li, B));
-        if (d.layers[li].type_layer == MYEA_LAYER_LSTM) MYEA_TRY(lstm_backward_layer(li, B));
-        else if (d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) {
+        if (d.layers[li].type_layer == MYEA_LAYER_LSTM) {
+            // The weight contractions of the consumer above need nothing the time loop of this layer produces, and the loop leaves
+            // most of the matrix pipe idle: in the combined call they go to the side stream, enqueued right behind the loop so that
+            // its workgroups are placed first.  MYEA_DW_BESIDE_LOOP=0 keeps them behind the loop on the one stream.
+            const bool beside = pairing && dw_beside_loop_allowed(gi, li, B);
+            if (beside) MYEA_HIP_TRY(hipEventRecord(fork_event, stream));
+            loop_shares_device = beside;
+            const int loop_rc = lstm_backward_layer(li, B);
+            loop_shares_device = false;
+            MYEA_TRY(loop_rc);
+            if (beside) {
+                MYEA_HIP_TRY(hipStreamWaitEvent(side_stream, fork_event, 0));
+                std::swap(stream, side_stream);
+                const int rc = update_derivative_weight_contraction(gi, B);
+                std::swap(stream, side_stream);
+                MYEA_HIP_TRY(hipEventRecord(join_event, side_stream));
+                dw_beside_loop = true;
+                MYEA_TRY(rc);
+                dw_done[gi] = 1;
+            }
+        } else if (d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) {
             MYEA_TRY(backward_residual_block(li, B));
             gi = li + 1;
         }
@@ -1080,6 +1101,53 @@ bool Net::fc_dw_params(size_t li, size_t B, GemmParams *out)
     return true;
 }
 
+// the weight contraction(s) of layer li: dW += delta^T X (:178-216); LSTM layers: their input and recurrent weights
+int Net::update_derivative_weight_contraction(size_t li, size_t B)
+{
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
+    const bool per_t = T > 1 && B != Bmax;
+    const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
+    const myea_layer_desc &l = d.layers[li];
+    if (li < dw_done.size() && dw_done[li]) return MYEA_OK;   // rode along with the delta's contraction, or ran beside a time loop, in this pass
+    if (l.type_layer == MYEA_LAYER_LSTM) return lstm_update_derivative_weight(li, B, false);
+    if (l.type_layer == MYEA_LAYER_RESIDUAL || layer_is_pooling(l)) return MYEA_OK;  // own no connection (:31-36)
+    DevLayer &o = L[li];
+    const size_t In = o.In, H = o.H;
+    // Layer::ptr_array_pre_summations: the operand the weights were applied to (NN/Neural_Network__Ordered.cpp:96-141)
+    const float *x = layer_outputs(o.prev);
+    if (o.group == 2) x = o.values;
+    else if (o.group == 1 && layer_uses_norm(l)) x = o.normalizes;
+    for (size_t c = 0; c < chunks; ++c) {
+        const size_t roff = c * Bmax;
+        GemmParams g{};
+        g.A = o.neuron_errors + roff * H; g.lda = (long)H; g.a_k_contiguous = 0;
+        g.B = x + roff * In; g.ldb = (long)In; g.b_k_contiguous = 0;
+        g.C = gradient + l.first_connection_index; g.ldc = (long)In;
+        g.M = (int)H; g.N = (int)In; g.K = (int)rows;
+        g.accumulate = 1; g.epilogue = EPI_NONE;
+        const int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
+        if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
+        prof_begin(2);
+        MYEA_TRY(launch_gemm(stream, g));
+        if (slabs > 1) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
+        prof_end(2.0 * (double)rows * (double)H * (double)In);
+    }
+
+    return MYEA_OK;
+}
+
+// May the weight contractions of layer gi run on the side stream beside the backward time loop of LSTM layer li?  Where nothing
+// is shared and it was measured to pay: a one-direction loop (a two-direction layer uses the side stream itself) under an
+// LSTM consumer, whose two long contractions write packed slabs of their own.  (A dense consumer's single contraction hides
+// less than the loop loses by sharing the device: 3.93 against 3.90 ms per step on 2 x LSTM-512.)
+bool Net::dw_beside_loop_allowed(size_t gi, size_t li, size_t B)
+{
+    static const bool off = [] { const char *e = std::getenv("MYEA_DW_BESIDE_LOOP"); return e && e[0] == '0'; }();
+    if (off || !side_stream || d.number_recurrent_depth < 2 || B != d.batch_size) return false;
+    if (L[li].lstm2 || L[gi].lstm2 || (gi < dw_done.size() && dw_done[gi])) return false;
+    return d.layers[gi].type_layer == MYEA_LAYER_LSTM;
+}
+
 int Net::update_derivative_weight(size_t B, size_t first, size_t end)
 {
     if (first < 1 || end > d.n_layers || first > end) { set_last_error("Update_Derivative_Weight: layer range [%zu, %zu) invalid", first, end); return MYEA_E_INVALID; }
@@ -1114,33 +1182,7 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
         return MYEA_OK;
     };
     auto contractions = [&]() -> int {
-        for (size_t li = first; li < end; ++li) {
-            const myea_layer_desc &l = d.layers[li];
-            if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_update_derivative_weight(li, B, false)); continue; }
-            if (l.type_layer == MYEA_LAYER_RESIDUAL || layer_is_pooling(l)) continue;  // own no connection (:31-36)
-            if (li < dw_done.size() && dw_done[li]) continue;   // rode along with the delta's contraction in this pass
-            DevLayer &o = L[li];
-            const size_t In = o.In, H = o.H;
-            // Layer::ptr_array_pre_summations: the operand the weights were applied to (NN/Neural_Network__Ordered.cpp:96-141)
-            const float *x = layer_outputs(o.prev);
-            if (o.group == 2) x = o.values;
-            else if (o.group == 1 && layer_uses_norm(l)) x = o.normalizes;
-            for (size_t c = 0; c < chunks; ++c) {
-                const size_t roff = c * Bmax;
-                GemmParams g{};
-                g.A = o.neuron_errors + roff * H; g.lda = (long)H; g.a_k_contiguous = 0;
-                g.B = x + roff * In; g.ldb = (long)In; g.b_k_contiguous = 0;
-                g.C = gradient + l.first_connection_index; g.ldc = (long)In;
-                g.M = (int)H; g.N = (int)In; g.K = (int)rows;
-                g.accumulate = 1; g.epilogue = EPI_NONE;
-                const int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
-                if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
-                prof_begin(2);
-                MYEA_TRY(launch_gemm(stream, g));
-                if (slabs > 1) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
-                prof_end(2.0 * (double)rows * (double)H * (double)In);
-            }
-        }
+        for (size_t li = first; li < end; ++li) MYEA_TRY(update_derivative_weight_contraction(li, B));
         return MYEA_OK;
     };
     bool any_lstm = false;

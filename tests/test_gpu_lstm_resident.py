@@ -209,3 +209,32 @@ def test_a_backward_wait_that_gives_up_is_reported_too(ksplit):
         n.Reset__Loss()
         run_step(n, B, X, Y, update=False)
     _compare(desc, gpu, cpu, B, T, "after the backward give-up")
+
+
+def test_weight_contractions_beside_the_backward_loop_change_nothing():
+    """the combined backward + weight-gradient call runs the weight contractions of the layer above on a second stream beside an
+    LSTM layer's backward time loop (and picks the loop's form that leaves them room): same gradient as the two separate calls
+    within the tolerance the two resident forms are held to, and the same as the oracle"""
+    specs = [dict(units=16), lstm(128), lstm(128), dict(units=128, activation="LINEAR")]
+    T, B = 6, 64
+    desc, h, w, masks, X, Y = _setup(specs, T, B, B, seed=13)
+    combined, separate = _net(desc, h, w, None), _net(desc, h, w, None)
+    cpu = OracleNetwork(desc, h)
+    cpu.set_state_propagation(mb.STATE_TRAINING)
+    cpu.upload_parameters(w)
+    cpu.Clear_Training_Arrays()
+    for step in range(2):
+        combined.Forward_Pass(B, X)
+        combined.Compute__Error(B, Y)
+        combined.Backward_Pass__Update_Derivative_Weight(B)
+        run_step(separate, B, X, Y, update=False)
+        run_step(cpu, B, X, Y, update=False)
+        g = cpu.download_gradient()
+        tol = ABS * max(1.0, float(np.abs(g).max()))
+        assert_close(combined.download_gradient(), separate.download_gradient(), REL, tol, what="step %d: combined against separate calls" % step)
+        assert_close(combined.download_gradient(), g, REL, tol, what="step %d: combined against the oracle" % step)
+        for n in (combined, separate, cpu):
+            n.Update_Parameter(B, B)
+        wc = cpu.download_parameters()
+        combined.upload_parameters(wc)
+        separate.upload_parameters(wc)
