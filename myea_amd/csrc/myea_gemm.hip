@@ -25,6 +25,7 @@
 //
 // Accumulator layout of v_mfma_f32_32x32x2_f32: register r of lane l holds
 //   C[(r / 4) * 8 + (l / 32) * 4 + (r % 4)][l % 32].
+#include <cstdlib>
 #include <mutex>
 
 #include "myea_device_af.h"
@@ -266,6 +267,8 @@ struct GemmDev {
     int nbm, nbn;
     int ksplit, kchunk;   // split-K: number of slabs and k's per slab (multiple of BK); slab s writes C + s * slab
     long slab;
+    float *pair_partials;    // not null: ksplit == 2 and the two workgroups of a tile combine their halves in the launch
+    unsigned *pair_tickets;
 };
 
 struct TilePlace {
@@ -506,6 +509,45 @@ __device__ __forceinline__ void gemm_tile(const GemmDev &p, const int block, flo
         cur = following;
     }
 
+    if (BM == 64 && BN == 64 && p.pair_partials) {   // only the 64 x 64 launches are split this way
+        // Two workgroups share this tile, one per half of k (their ids are equal mod 8: the same XCD).  Whoever is done first
+        // leaves its accumulators and goes; the other adds them and carries on to the epilogue.  The sum is half 0 + half 1
+        // either way.  The wait below is for a workgroup that has nothing left to do but store 16 KB and raise its flag.
+        __shared__ unsigned s_ticket;
+        const int tile = block - split * nblocks;
+        unsigned *ticket = p.pair_tickets + 2 * tile, *flag = ticket + 1;
+        float *partial = p.pair_partials + (size_t)tile * (BM * BN);
+        if (threadIdx.x == 0) s_ticket = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (s_ticket == 0u) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        __hip_atomic_store(partial + ((i * TN + j) * 16 + r) * kThreads + threadIdx.x, acc[i][j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's stores are complete
+            __syncthreads();
+            if (threadIdx.x == 0) __hip_atomic_store(flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+        if (threadIdx.x == 0) {
+            for (unsigned polls = 0; polls < (1u << 24) && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u; ++polls) __builtin_amdgcn_s_sleep(1);
+            __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects them
+            __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float other = __hip_atomic_load(partial + ((i * TN + j) * 16 + r) * kThreads + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    acc[i][j][r] = split == 0 ? acc[i][j][r] + other : other + acc[i][j][r];
+                }
+    }
     // Epilogue.  What kind it is, whether an addend joins and whether the tile lies wholly inside the matrix are the same
     // for every element of the tile: they are decided once, and the element loops of whole tiles carry no such test.
     const TilePlace at{m0, n0, wave_m, wave_n, lane32, half, (long)split * p.slab};
@@ -637,6 +679,7 @@ static int prepare_gemm(const GemmParams &p, GemmDev &d, bool *vec)
     if (p.addend && (p.epilogue == EPI_FC_FORWARD || p.ld_addend < p.N)) { set_last_error("gemm: addend needs EPI_NONE / EPI_FC_DERIVE and ld_addend >= N"); return MYEA_E_INVALID; }
     d.nbm = d.nbn = 0;
     d.ksplit = 1; d.kchunk = p.K > 0 ? p.K : 1; d.slab = 0;
+    d.pair_partials = nullptr; d.pair_tickets = nullptr;
     if (p.split_k > 1) {
         if (p.epilogue != EPI_NONE || p.accumulate || p.addend) { set_last_error("gemm: split-K writes plain partial slabs"); return MYEA_E_INVALID; }
         const int chunk = ((p.K + p.split_k - 1) / p.split_k + kBK - 1) / kBK * kBK;
@@ -669,6 +712,17 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     // 64-row tiles to keep the chip filled for short-M / short-N problems.
     const long tiles_128 = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
     if (tiles_128 >= 512) return launch_layout_vec<128, 128>(stream, d, a_kc, b_kc);
+    // At most one 64 x 64 tile per compute unit and a k worth splitting: two workgroups per tile, half of k each, combined in
+    // the launch - a second wavefront per SIMD to fill the first one's waits, which such a launch otherwise lacks.
+    // MYEA_GEMM_PAIR_K=0 keeps one workgroup per tile.
+    static const bool pair_k_off = [] { const char *e = std::getenv("MYEA_GEMM_PAIR_K"); return e && e[0] == '0'; }();
+    const long tiles_64 = (long)((p.M + 63) / 64) * ((p.N + 63) / 64);
+    if (p.pair_partials && p.pair_tickets && !pair_k_off && d.ksplit == 1 && tiles_64 <= kGemmPairTiles && tiles_64 % 8 == 0 && tiles_64 >= 128 && p.K >= 512) {
+        d.ksplit = 2;
+        d.kchunk = ((p.K + 1) / 2 + kBK - 1) / kBK * kBK;
+        d.pair_partials = p.pair_partials; d.pair_tickets = p.pair_tickets;
+        return launch_layout_vec_small(stream, d, a_kc, b_kc);
+    }
     if (tiles_128 * 2 * d.ksplit < 256) return launch_layout_vec_small(stream, d, a_kc, b_kc);
     if (p.M <= p.N) return launch_layout_vec<64, 128>(stream, d, a_kc, b_kc);
     return launch_layout_vec<128, 64>(stream, d, a_kc, b_kc);

@@ -57,7 +57,15 @@ struct GemmParams {
     // sums the slabs in order.  Requires EPI_NONE and accumulate == 0.  0 / 1 = off.
     int split_k;
     long split_k_slab;
+    // Two-way split along k INSIDE the launch, any epilogue: when the problem has too few tiles to give every compute unit two
+    // workgroups, two workgroups share a tile, each contracting over half of k; the first to finish leaves its accumulators in
+    // `pair_partials`, the second adds them to its own (half 0 + half 1: the same sum whichever finishes first) and runs the
+    // epilogue.  pair_partials: at least 256 x 4096 floats; pair_tickets: 2 x 256 words, zero before the first use (a launch
+    // leaves them zero).  One launch at a time may use a given pair of buffers.  Null = off; the launcher decides per problem.
+    float *pair_partials;
+    unsigned *pair_tickets;
 };
+constexpr int kGemmPairTiles = 256;   // tiles the two buffers above serve
 
 int gemm_split_k(int M, int N, int K);
 int launch_gemm(hipStream_t stream, const GemmParams &p);

@@ -100,6 +100,8 @@ struct Net {
     // LSTM time loops as one resident launch (myea_lstm_resident.hip): barrier counters in device memory, and a pinned host
     // word a kernel sets when one of its bounded waits gave up; resident_off: this network stays on one launch per time step
     unsigned *resident_sync = nullptr, *resident_flag = nullptr;
+    float *gemm_pair_partials = nullptr;       // scratch of the contractions that split a tile's k between two workgroups
+    unsigned *gemm_pair_tickets = nullptr;
     float *resident_exchange = nullptr;   // partial sums the members of a group hand each other in the backward loop
     size_t resident_exchange_floats = 0;
     bool resident_off = false;

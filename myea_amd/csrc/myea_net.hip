@@ -338,6 +338,13 @@ int Net::create(const myea_net_desc &desc)
         }
     }
     MYEA_TRY(side_stream_create());
+    {   // forward contractions of few tiles split each tile's k between two workgroups: their meeting place
+        MYEA_TRY(dev_alloc(&gemm_pair_partials, (size_t)kGemmPairTiles * 64 * 64));
+        void *q = nullptr;
+        MYEA_HIP_TRY(hipMalloc(&q, 2 * kGemmPairTiles * sizeof(unsigned)));
+        MYEA_HIP_TRY(hipMemset(q, 0, 2 * kGemmPairTiles * sizeof(unsigned)));
+        gemm_pair_tickets = static_cast<unsigned *>(q);
+    }
     {
         bool any_lstm = false;
         for (size_t li = 1; li < d.n_layers; ++li) any_lstm = any_lstm || d.layers[li].type_layer == MYEA_LAYER_LSTM;
@@ -404,6 +411,7 @@ Net::~Net()
     }
     fr(resident_sync);
     fr(resident_exchange);
+    fr(gemm_pair_partials); fr(gemm_pair_tickets);
     if (resident_flag) (void)hipHostFree(resident_flag);
     fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc); fr(index_stage); fr(dw_slabs);
     for (ProfEvent &e : pending) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
@@ -478,6 +486,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
         // a batch normalisation in front of the activation, training: its column sums leave with the contraction's tiles
         const bool sums_from_gemm = norm && before && training && o.norm_partials && bn_sums_from_gemm() && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H;
         if (sums_from_gemm) g.col_partials = o.norm_partials;
+        g.pair_partials = gemm_pair_partials; g.pair_tickets = gemm_pair_tickets;   // forward contractions run one at a time on this stream
         prof_begin(0);
         MYEA_TRY(launch_gemm(stream, g));
         prof_end(2.0 * (double)rows * (double)H * (double)In);

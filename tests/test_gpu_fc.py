@@ -312,3 +312,30 @@ def test_device_resident_inputs_match_host_inputs():
     gpu.Update_Derivative_Weight(B)
     run_step(cpu, B, X, Y, update=False)
     assert_close(gpu.download_gradient(), cpu.download_gradient(), REL, ABS)
+
+
+def test_forward_contraction_that_splits_a_tile_between_two_workgroups():
+    """A forward contraction with at most one 64 x 64 tile per compute unit (here 512 x 1024 outputs over k = 512 and 1024) splits
+    each tile's k between two workgroups that combine their halves inside the launch: against the oracle, and bit for bit
+    the same from run to run (the combined sum is half 0 + half 1 whichever workgroup finishes first)."""
+    specs = [dict(units=512), dict(units=1024, activation="TANH"), dict(units=1024, activation="SIGMOID", normalization="BATCH_NORMALIZATION"),
+             dict(units=64, activation="LINEAR")]
+    B = 512
+    desc = mb.make_desc(specs, B, 1)
+    h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["GD"], type_loss_function=mb.LOSS["MSE"])
+    w = glorot_parameters(desc, 5)
+    rng = np.random.default_rng(5)
+    X = rng.normal(0, 1, (B, 512)).astype(np.float32)
+    Y = rng.normal(0, 1, (B, 64)).astype(np.float32)
+    outs = []
+    for cls in (mb.HipNetwork, mb.HipNetwork, OracleNetwork):
+        n = cls(desc, h)
+        n.set_state_propagation(mb.STATE_TRAINING)
+        n.upload_parameters(w)
+        n.Clear_Training_Arrays()
+        run_step(n, B, X, Y, update=False)
+        outs.append([n.download_tensor(li, mb.TENSOR["OUTPUTS"], B * desc.layers[li].n_units) for li in (1, 2, 3)] + [n.download_gradient()])
+    for a, b in zip(outs[0], outs[1]):
+        assert np.array_equal(a, b)
+    for k, (a, b) in enumerate(zip(outs[0], outs[2])):
+        assert_close(a, b, 1e-4, 1e-5 * max(1.0, float(np.abs(b).max())), what="tensor %d" % k)
