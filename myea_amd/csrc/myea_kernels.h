@@ -266,6 +266,8 @@ struct LstmResidentDir {
     float *acts;           // [T][Bmax][4C] in: input sums; out: the activations z, i, f, o
     float *c, *ca, *h;     // [T][Bmax][C] cell state, tanh(cell state), cell output
     float *dh, *dG, *dc;   // backward: [T][Bmax][C] delta of the outputs (in: from above; out: plus the recurrent term), [T][Bmax][4C], [T][Bmax][C]
+    float *sums;           // backward, or null: [plan.row_groups][7][C] sums over the group's examples and all time steps of
+                           // dz, di, df, do (the bias gradients) and di c[step before], df c[step before], do c (the peepholes')
     const uint8_t *zone_state, *zone_output;   // zoneout masks [T][zone_stride] (1 = update) or null
     size_t zone_stride;
     int reverse;           // walks time from T - 1 down to 0

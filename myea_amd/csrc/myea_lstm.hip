@@ -43,6 +43,10 @@ struct LstmLayer {
     float *dG = nullptr;    // [T][Bmax][G] deltas dz | di | df | do
     float *dc = nullptr;    // [T][Bmax][C]
     float *part = nullptr;  // split-K slabs of the per-step recurrent contractions, 16 x [Bmax][G]
+    // [ceil(Bmax / 32)][7][C]: what the resident backward loop sums of its gate deltas as it goes (bias and peephole gradients
+    // per group of examples); sums_groups > 0 while they belong to the deltas in dG, of a pass over sums_batch examples
+    float *sums = nullptr;
+    size_t sums_groups = 0, sums_batch = 0;
     // Normalised layer (one cell per block).  The eight gate sums and the cell state pass through their own normalisation at
     // every time step (NN/Neural_Network__Forward_Pass__OpenMP.cpp:1769-2340): nine groups of normalised units, 0 block input
     // from below, 1 block input recurrent, 2 cell state, 3 / 4 input gate, 5 / 6 forget gate, 7 / 8 output gate (from below /
@@ -644,6 +648,7 @@ int Net::lstm_create_layer(size_t li)
         q->renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
         q->fused = !q->norm && lstm_fused_supported(q->C, q->cpb) && !fused_lstm_disabled();
         if (q->fused) MYEA_TRY(dev_alloc_zero(&q->WrecT, q->C * q->G));
+        if (q->fused) MYEA_TRY(dev_alloc_zero(&q->sums, (B + 31) / 32 * 7 * q->C));
         MYEA_TRY(dev_alloc_zero(&q->gWin, kMaxSlabs * q->G * q->In));   // split-K slabs of the weight-gradient contractions
         MYEA_TRY(dev_alloc_zero(&q->gWrec, kMaxSlabs * q->G * q->C));
         q->gWin_own = q->gWin; q->gWrec_own = q->gWrec;
@@ -680,7 +685,7 @@ void Net::lstm_destroy_layer(DevLayer &o)
     for (LstmLayer **slot : {&o.lstm, &o.lstm2}) {
         LstmLayer *q = *slot;
         if (!q) continue;
-        float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin_own, q->gWrec_own, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr,
+        float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin_own, q->gWrec_own, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->sums, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr,
                         q->sin, q->srec, q->nin, q->nrec, q->hin, q->hrec, q->din, q->drec, q->nc, q->hc};
         for (float *p : all) if (p) (void)hipFree(p);
         for (float *p : q->stats) if (p) (void)hipFree(p);
@@ -942,7 +947,7 @@ int Net::lstm_resident_dirs(DevLayer &o, LstmResidentDir *dirs)
         LstmResidentDir r{};
         r.Wrec = q->Wrec; r.WrecT = q->WrecT; r.bias = parameters + q->bias; r.peep = q->peep;
         r.acts = q->acts; r.c = q->c; r.ca = q->ca; r.h = q->h;
-        r.dh = q->dh; r.dG = q->dG; r.dc = q->dc;
+        r.dh = q->dh; r.dG = q->dG; r.dc = q->dc; r.sums = q->sums;
         r.zone_state = zone ? q->zone_state : nullptr; r.zone_output = zone ? q->zone_output : nullptr; r.zone_stride = q->zone_stride;
         r.reverse = q->reverse ? 1 : 0;
         dirs[n++] = r;
@@ -1059,6 +1064,8 @@ int Net::lstm_backward_layer(size_t li, size_t B)
             MYEA_HIP_TRY(hipMemcpyAsync(q.dh, o.neuron_errors, (size_t)d.number_recurrent_depth * d.batch_size * q.C * sizeof(float), hipMemcpyDeviceToDevice, stream));
         return MYEA_OK;
     };
+    for (LstmLayer *q : {o.lstm, o.lstm2})
+        if (q) q->sums_groups = 0;   // the gate deltas are about to change
     if (T > 1 && o.lstm->fused && !resident_off && resident_sync) {
         LstmResidentPlan plan;
         const int dirs = o.lstm2 ? 2 : 1;
@@ -1073,6 +1080,8 @@ int Net::lstm_backward_layer(size_t li, size_t B)
             prof_begin(kProfLstmBackwardLoop);
             MYEA_TRY(launch_lstm_resident_backward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag, resident_exchange, resident_exchange_floats));
             prof_end(dirs * loop_work, 1);
+            for (LstmLayer *q : {o.lstm, o.lstm2})
+                if (q && q->sums) { q->sums_groups = (size_t)plan.row_groups; q->sums_batch = B; }
             return MYEA_OK;
         }
     }
@@ -1204,11 +1213,23 @@ int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t
     return MYEA_OK;
 }
 
+// MYEA_LSTM_RESIDENT_SUMS=0: the bias and peephole gradients always come from their own pass over the gate deltas
+static bool resident_sums_allowed()
+{
+    const char *e = std::getenv("MYEA_LSTM_RESIDENT_SUMS");   // read at every call: a test compares the two ways in one process
+    return !(e && e[0] == '0');
+}
+
 int Net::lstm_update_derivative_weight_reductions(LstmLayer &q, size_t B)
 {
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
     const LstmGeom geom = geom_of(q);
     if (T * B > 0xffffffffull) { set_last_error("LSTM weight gradients: %zu x %zu (time steps x batch) rows do not fit 32 bits", T, B); return MYEA_E_INVALID; }
+    if (q.sums_groups && q.sums_batch == B && resident_sums_allowed()) {   // the backward time loop summed them as it went
+        hipLaunchKernelGGL(lstm_bias_peep_final_kernel, dim3(grid_for(7 * q.C, kBlock)), dim3(kBlock), 0, stream, geom, q.sums_groups, q.sums, gradient + q.bias, gradient);
+        MYEA_HIP_TRY(hipGetLastError());
+        return MYEA_OK;
+    }
     if (q.cpb == 1) {   // biases and peepholes in one pass over the gate deltas
         const size_t colblocks = (q.C + 63) / 64;
         size_t S = (512 + colblocks - 1) / colblocks;          // aim at >= 512 workgroups

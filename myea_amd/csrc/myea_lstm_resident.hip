@@ -499,6 +499,28 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
 }
 
 // ---- backward --------------------------------------------------------------------------------------------------------
+// The seven sums every lane of a backward workgroup has gathered over its examples (lane = 16 * example + cell within a
+// wavefront's 64) folded over the workgroup's examples in a fixed order and left at out[(row_group * 7 + v) * C + c0 + cell]:
+// what the weight-gradient pass otherwise reads the gate deltas and cell states once more for.
+__device__ __forceinline__ void store_column_sums(const double (&sums)[7], float *out, int row_group, int C, int c0)
+{
+    if (!out) return;
+    __shared__ double s_fold[4][7][16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int v = 0; v < 7; ++v) {
+        double x = sums[v];
+        x += __shfl_xor(x, 16);
+        x += __shfl_xor(x, 32);
+        if (lane < 16) s_fold[wave][v][lane] = x;
+    }
+    __syncthreads();
+    if (threadIdx.x < 7 * 16) {
+        const int v = threadIdx.x >> 4, cell = threadIdx.x & 15;
+        out[((size_t)row_group * 7 + v) * C + c0 + cell] = (float)(((s_fold[0][v][cell] + s_fold[1][v][cell]) + s_fold[2][v][cell]) + s_fold[3][v][cell]);
+    }
+}
+
 // dh[t] += dG[t'] Wrec (t' = the step processed before t in this pass), then the gate deltas of step t.  The workgroup owns
 // CELLS = 16 columns of dh; wavefront w contracts over the k range of gate w (k = gate * C + cell of dG[t']) against its
 // slice of the transposed packed matrix WrecT [C][4C].  j counts the steps of this pass: the direction's own step is
@@ -550,7 +572,8 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
     const ptrdiff_t step_g = t_step * (ptrdiff_t)(Bmax * G), step_c = t_step * (ptrdiff_t)(Bmax * C);
     float e_peep[PAIRS][3];
     float n_di[2][PAIRS], n_df[2][PAIRS], n_f[2][PAIRS], n_dc[2][PAIRS];   // of the chain's step processed before: delta i, delta f, f, delta c
-    float e_act[PAIRS][4], e_ca[PAIRS], e_cp[PAIRS], e_dh[PAIRS];
+    float e_act[PAIRS][4], e_ca[PAIRS], e_cp[PAIRS], e_cs[PAIRS], e_dh[PAIRS];
+    double sums[7] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};   // over the lane's examples and steps: dz, di, df, do, di c', df c', do c (c': the state of the step before)
     const float *p_acts[2][PAIRS], *p_ca[2][PAIRS], *p_cp[2][PAIRS], *p_dh_in[2][PAIRS];   // read: the batch's last example for a lane without one
     float *p_dh[2][PAIRS], *p_dG[2][PAIRS], *p_dc[2][PAIRS];                                  // written: the scrap area for such a lane
     ptrdiff_t lane_step_g[2][PAIRS], lane_step_c[2][PAIRS];
@@ -599,6 +622,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
             e_ca[q] = *p_ca[c][q];
             e_dh[q] = *p_dh_in[c][q];
             e_cp[q] = with_cp ? *p_cp[c][q] : 0.f;
+            e_cs[q] = p_cp[c][q][-step_c];
         }
     };
     auto load_tiles = [&](auto ch) {   // dG of the chain's step processed before the one its pointers are at
@@ -693,6 +717,10 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
             const float di = (e * z) * (gi * (1.f - gi));
             const float df = s > 0 ? (e * e_cp[q]) * (gf * (1.f - gf)) : 0.f;
             n_di[c][q] = di; n_df[c][q] = df; n_f[c][q] = gf; n_dc[c][q] = e;
+            if (lane_step_g[c][q] != 0) {   // the lane has an example in this chain
+                sums[0] += dz; sums[1] += di; sums[2] += df; sums[3] += ddo;
+                sums[4] += di * e_cp[q]; sums[5] += df * e_cp[q]; sums[6] += ddo * e_cs[q];
+            }
             float *drow = p_dG[c][q];
             drow[0] = dz; drow[C] = di; drow[2 * C] = df; drow[3 * C] = ddo;
             *p_dh[c][q] = dh; *p_dc[c][q] = e;
@@ -719,6 +747,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
     if (!tail(Chain0{}, Later{}, 0, (unsigned)(T - 1))) return;
     head(Chain1{}, std::false_type{});
     if (!tail(Chain1{}, Later{}, 0, 0u)) return;
+    store_column_sums(sums, d.sums, rg, C, c0);
 }
 
 // ---- backward, the contraction split along k ------------------------------------------------------------------------
@@ -794,7 +823,8 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_ksplit_ker
 #pragma unroll
     for (int gate = 0; gate < 3; ++gate) e_peep[gate] = d.peep[gate * C + kcell];
     float n_di[2], n_df[2], n_f[2], n_dc[2];   // of the chain's step processed before: delta i, delta f, f, delta c
-    float e_act[4], e_ca, e_cp, e_dh;
+    float e_act[4], e_ca, e_cp, e_cs, e_dh;
+    double sums[7] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};   // over the lane's examples and steps: dz, di, df, do, di c', df c', do c (c': the state of the step before)
     const float *p_acts[2], *p_ca[2], *p_cp[2], *p_dh_in[2];   // read: the batch's last example for a lane without one
     float *p_dh[2], *p_dG[2], *p_dc[2];                          // written: the scrap area for such a lane
     ptrdiff_t lane_step_g[2], lane_step_c[2];
@@ -833,6 +863,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_ksplit_ker
         e_ca = *p_ca[c];
         e_dh = *p_dh_in[c];
         e_cp = *(with_cp ? p_cp[c] : p_ca[c]);   // no step before the direction's first: any finite value, the forget gate's delta is zero there
+        e_cs = p_cp[c][-step_c];
     };
     auto load_tiles = [&](auto ch, int buffer) {
         constexpr int c = decltype(ch)::value;
@@ -877,6 +908,10 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_ksplit_ker
         const float di = (e * z) * (gi * (1.f - gi));
         const float df = s > 0 ? (e * e_cp) * (gf * (1.f - gf)) : 0.f;
         n_di[c] = di; n_df[c] = df; n_f[c] = gf; n_dc[c] = e;
+        if (lane_step_g[c] != 0) {   // the lane has an example in this chain
+            sums[0] += dz; sums[1] += di; sums[2] += df; sums[3] += ddo;
+            sums[4] += s > 0 ? di * e_cp : 0.f; sums[5] += df * e_cp; sums[6] += ddo * e_cs;
+        }
         float *drow = p_dG[c];
         drow[0] = dz; drow[C] = di; drow[2 * C] = df; drow[3 * C] = ddo;
         *p_dh[c] = dh; *p_dc[c] = e;
@@ -946,7 +981,8 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_ksplit_ker
         if (!unit(Chain1{}, Later{}, Later{}, j, T - 1 - j, (unsigned)(j + 1) * arrivals, T - 2 - j > 0)) return;
     }
     if (!unit(Chain0{}, Later{}, First{}, T - 1, 0, (unsigned)(T - 1) * arrivals, false)) return;
-    unit(Chain1{}, Later{}, First{}, T - 1, 0, 0u, false);
+    if (!unit(Chain1{}, Later{}, First{}, T - 1, 0, 0u, false)) return;
+    store_column_sums(sums, d.sums, rg, C, c0);
 }
 
 __global__ void resident_probe_kernel(unsigned *table)

@@ -138,6 +138,30 @@ def test_resident_loop_matches_one_launch_per_step_and_the_oracle(name, specs, T
         stepwise.upload_parameters(wc)
 
 
+@pytest.mark.parametrize("ksplit", ["1", "0"], ids=["backward-split-along-k", "backward-split-along-columns"])
+def test_bias_and_peephole_gradients_summed_inside_the_backward_loop(ksplit):
+    """the resident backward loop sums the bias and peephole gradients of its layer as it goes; MYEA_LSTM_RESIDENT_SUMS=0 has the
+    weight-gradient pass read the gate deltas once more instead: the same gradient either way, with examples missing from the last
+    group, in both directions, and when a smaller batch follows a larger one"""
+    specs = [dict(units=12), lstm(256, bidirectional=True), lstm(128), dict(units=128, activation="LINEAR")]
+    T, Bmax = 7, 80
+    desc, h, w, masks, X, Y = _setup(specs, T, Bmax, Bmax, seed=33)
+    inside, apart = _net(desc, h, w, None), _net(desc, h, w, None)
+    for B in (80, 45):
+        with environment(MYEA_LSTM_BACKWARD_KSPLIT=ksplit):
+            inside.profile_enable(True)
+            run_step(inside, B, X[:B], Y[:B], update=False)
+            assert _loop_launches(inside)[1] == 2, "the backward time loops did not run as one launch per layer"
+            inside.profile_enable(False)
+            with environment(MYEA_LSTM_RESIDENT_SUMS="0"):
+                run_step(apart, B, X[:B], Y[:B], update=False)
+        g = apart.download_gradient()
+        assert np.abs(g).max() > 0
+        assert_close(inside.download_gradient(), g, 2e-5, 2e-6 * float(np.abs(g).max()), what="batch %d: sums inside the loop against the separate pass" % B)
+        for n in (inside, apart):
+            n.Update_Parameter(B, B)
+
+
 def test_a_smaller_batch_after_a_larger_one():
     """rows beyond the batch keep what the larger batch left there; the rows of the batch do not depend on them"""
     specs = [dict(units=8), lstm(128), dict(units=128, activation="LINEAR")]
