@@ -1,8 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the training hot path on one MI355X.
 
-One "step" = Forward_Pass + Compute__Error + Backward_Pass and Update_Derivative_Weight (as one call) + Update_Parameter on one
-batch of synthetic data already resident in HBM.  Default workload: BASELINE config 2, the deep fully-connected
+One "step" = Forward_Pass + Compute__Error + Backward_Pass, Update_Derivative_Weight and Update_Parameter (the last three as
+one call; --separate-update: Update_Parameter as a call of its own) on one batch of synthetic data already resident in HBM.  Default workload: BASELINE config 2, the deep fully-connected
 stack 4096-4096-4096-4096-4096-1000 (ReLU, softmax + cross-entropy, Adam) at batch 1024, fp32.
 
 Prints ONE JSON line.  `value` comes from exactly `steps` timed steps.  `roofline` covers the dominant kernel family — the
@@ -153,7 +153,7 @@ FAMILIES = (("forward", "flop"), ("dx", "flop"), ("dw", "flop"), ("update", "byt
 KERNEL_NAMES = {"forward": "gemm_forward", "dx": "gemm_dx", "dw": "gemm_dw", "dx_dw_pair": "gemm_dx_dw_pair", "update": "optimizer_update"}
 
 
-def run_workload(name, steps, warmup):
+def run_workload(name, steps, warmup, separate_update=False):
     """Times `steps` training steps of one workload on cuda:0 (inputs resident in HBM): that is the throughput.  Then runs
     `steps` more with the library's per-family HIP-event timers on for the per-kernel figures - a pair of timing events around
     every launch keeps launches from overlapping their neighbours' tails and costs 3 % (the wide dense stack) to 16 % (the
@@ -178,11 +178,14 @@ def run_workload(name, steps, warmup):
     X, Y = make_inputs(np, wl, 2)
     xd, yd = torch.from_numpy(X).cuda(), torch.from_numpy(Y).cuda()   # inputs resident in HBM before the timed region
 
-    def step():
+    def step(separate=separate_update):
         net.Forward_Pass(B, xd, on_device=True)
         net.Compute__Error(B, yd, on_device=True)
-        net.Backward_Pass__Update_Derivative_Weight(B)     # the two calls of Train_Batch_BP as one entry point
-        net.Update_Parameter(B, B)
+        if separate:
+            net.Backward_Pass__Update_Derivative_Weight(B)     # the two calls of Train_Batch_BP as one entry point
+            net.Update_Parameter(B, B)
+        else:   # and the update that follows them: a layer's weights step as soon as their gradient is complete
+            net.Backward_Pass__Update_Derivative_Weight__Update_Parameter(B, B)
 
     for _ in range(warmup):
         step()
@@ -203,6 +206,17 @@ def run_workload(name, steps, warmup):
     t3 = time.perf_counter()
     ms_per_step_events = (t3 - t2) * 1e3 / steps
     fam = {fname: net.profile_read(i) for i, (fname, _) in enumerate(FAMILIES)}
+    # When layers took their update beside the contractions below them (more update launches than steps), the contractions'
+    # durations above include what the update took from them: a third pass with Update_Parameter as a call of its own times
+    # the contractions alone on the device.
+    fam_alone, ms_per_step_alone = None, None
+    if not separate_update and fam["update"][0] > steps:
+        t4 = time.perf_counter()
+        for _ in range(steps):
+            step(separate=True)
+        torch.cuda.synchronize()
+        ms_per_step_alone = (time.perf_counter() - t4) * 1e3 / steps
+        fam_alone = {fname: net.profile_read(i) for i, (fname, _) in enumerate(FAMILIES)}
     net.profile_enable(False)
     loss = net.get_loss()
     net.close()
@@ -220,7 +234,7 @@ def run_workload(name, steps, warmup):
             entry.update(gbs=rate / 1e9, frac_hbm_peak=rate / 1e9 / PEAK_HBM_GBS)
         kernels[KERNEL_NAMES.get(fname, fname)] = entry
 
-    def mfma_aggregate(names):
+    def mfma_aggregate(names, fam=fam):
         n = sum(fam[k][0] for k in names)
         ms = sum(fam[k][1] for k in names)
         flop = sum(fam[k][2] for k in names)
@@ -232,6 +246,8 @@ def run_workload(name, steps, warmup):
                 ms_per_step_events=ms_per_step_events,
                 kernels=kernels, loss_per_output=loss.loss_values / max(loss.number_loss, 1),
                 contractions=mfma_aggregate(("forward", "dx", "dw", "dx_dw_pair")),
+                contractions_alone=mfma_aggregate(("forward", "dx", "dw", "dx_dw_pair"), fam_alone) if fam_alone else None,
+                ms_per_step_events_alone=ms_per_step_alone,
                 time_loops=mfma_aggregate(("lstm_forward_loop", "lstm_backward_loop")))
 
 
@@ -270,6 +286,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the LSTM-512 leg the default workload's line also carries")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the measured MFMA / HBM ceilings")
+    ap.add_argument("--separate-update", action="store_true", help="Update_Parameter as a call of its own behind the backward pass")
     ap.add_argument("--cpu-sample-rows", type=int, default=0, help="examples in the CPU sample (default: sized for ~20 s)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -279,13 +296,21 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
-    r = run_workload(args.workload, args.steps, args.warmup)
+    r = run_workload(args.workload, args.steps, args.warmup, args.separate_update)
     wl, B = r["wl"], r["batch"]
     has_loops = r["time_loops"]["launches"] > 0
-    roofline = dict(r["contractions"])
+    alone = r["contractions_alone"]
+    roofline = dict(alone or r["contractions"])
     roofline["kernel"] = "gemm_f32_mfma_kernel / gemm_pair_kernel (forward, dX, dW and paired dX + dW launches)"
     roofline["gemm_ms_per_step"] = roofline.pop("ms_per_step")
     roofline["measured_in"] = "events_pass"
+    if alone:
+        # the timed steps run the optimizer update of a layer on a second stream beside the contractions of the layers below it;
+        # what a contraction's events then span includes the update's share of the device.  The figures above are the
+        # contractions alone (Update_Parameter as a call of its own); these are the same launches beside the update.
+        roofline["measured_in"] = "events_pass_update_apart"
+        roofline["beside_update"] = {k: r["contractions"][k] for k in ("achieved", "frac", "avg_launch_ms")}
+        roofline["beside_update"]["gemm_ms_per_step"] = r["contractions"]["ms_per_step"]
     traffic = RECORDED_TRAFFIC.get(args.workload)
     roofline["traffic"] = traffic["bytes_per_launch"] if traffic else None
     if traffic:
@@ -303,12 +328,15 @@ def main():
         # the per-kernel figures (roofline, kernels, time_loops) come from a second pass of `steps` steps with a pair of HIP timing
         # events around every launch; those events slow the step itself, so `value` is from the pass without them
         "events_pass": {"steps": args.steps, "ms_per_step": r["ms_per_step_events"]},
+        "update": "separate call" if args.separate_update else "with the backward pass (one call)",
         "loss_per_output": r["loss_per_output"],
     }
+    if alone:
+        out["events_pass_update_apart"] = {"steps": args.steps, "ms_per_step": r["ms_per_step_events_alone"]}
     if has_loops:
         out["time_loops"] = dict(r["time_loops"], kernel="lstm_resident_forward_kernel / lstm_resident_backward_kernel (or one lstm_fused_* launch per step)")
     if args.workload != SECONDARY and args.workload == "fc4096x4_b1024_adam" and not args.no_secondary:
-        s = run_workload(SECONDARY, max(5, args.steps // 3), max(2, args.warmup // 2))
+        s = run_workload(SECONDARY, max(5, args.steps // 3), max(2, args.warmup // 2), args.separate_update)
         loops = dict(s["time_loops"], kernel="lstm_resident_forward_kernel + lstm_resident_backward_kernel: the recurrent contractions and gate math of steps 1 .. T-1, one launch per layer and pass")
         out["secondary"] = {"workload": SECONDARY, "value": s["value"], "unit": "samples/s", "ms_per_step": s["ms_per_step"],
                             "steps": max(5, args.steps // 3), "events_pass": {"steps": max(5, args.steps // 3), "ms_per_step": s["ms_per_step_events"]}, "config": config_of(s), "roofline": loops,

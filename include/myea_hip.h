@@ -405,6 +405,16 @@ int myea_hip_backward_pass_and_update_derivative_weight(myea_hip_net *net, size_
 /* Neural_Network::Update_Parameter (Data.hpp:849; Neural_Network.cpp:4719-4908): clip-by-global-norm
  * then the fused optimizer; zeroes the gradient. */
 int myea_hip_update_parameter(myea_hip_net *net, size_t batch_size_received, size_t training_size_received);
+/* Backward_Pass, Update_Derivative_Weight(batch, 1, total_layers) and Update_Parameter(batch, training size) as one entry
+ * point: the tail of Train_Batch_BP (Neural_Network/Dataset.cpp:645-658) and the Update_Parameter that Dataset::Training_OpenMP
+ * issues right behind it (Dataset.cpp:7652-7658).  Dataset_Mini_Batch::Training_OpenMP measures the batch's accuracy between the
+ * two (Dataset__Mini_Batch.cpp:353-372): a caller of this entry point takes that measurement, which reads the weights, first.
+ * Results are those of the three calls.
+ * Knowing that the update follows lets the library give the weights of a fully-connected layer their optimizer step as soon as
+ * their gradient is complete and the pass has no reader of them left: the memory-bound update then runs on a second stream
+ * beside the matrix-pipe-bound contractions of the layers below instead of behind all of them.  That needs an update whose
+ * scalars are known up front: with clipping by the gradient's global norm or iRPROP+ the three calls simply run in turn. */
+int myea_hip_backward_pass_update_derivative_weight_and_update_parameter(myea_hip_net *net, size_t batch_size, size_t training_size);
 
 /* Neural_Network::Compute__Loss (Neural_Network__Compute__Loss__Loop.cpp:22-140, Neural_Network__Recurrent_Compute__Loss__Loop.cpp:20-140):
  * the evaluation twin of Compute__Error - the same loss and accuracy accumulation over the output layer's values, no

@@ -378,6 +378,16 @@ public:
             PullState();
         });
     }
+    // Backward_Pass, Update_Derivative_Weight(batch, 1, total_layers) and Update_Parameter as one call (Dataset.cpp:645-658 and
+    // :7652-7658): the update of a layer's weights may then run beside the contractions of the layers below it
+    void Backward_Pass__Update_Derivative_Weight__Update_Parameter(size_t batch_size_received, size_t training_size_received)
+    {
+        Solo([&] {
+            if (!Need("Backward_Pass") || !PushFields("Backward_Pass")) return;
+            Ok("Backward_Pass", myea_hip_backward_pass_update_derivative_weight_and_update_parameter(net_, batch_size_received, training_size_received));
+            PullState();
+        });
+    }
 
     // Dropout_Bernoulli (Data.hpp:944; Neural_Network__Dropout__Bernoulli__Loop.cpp:33-97): new keep / drop draws for the
     // layers whose dropout is BERNOULLI - never BERNOULLI_INVERTED, which has its own function there - in layer order (the

@@ -107,7 +107,8 @@ ABI_SYMBOLS = [
     "myea_hip_upload_optimizer_state", "myea_hip_download_optimizer_state", "myea_hip_upload_masks", "myea_hip_set_unit_activations",
     "myea_hip_upload_zoneout_masks", "myea_hip_set_dropout_seed", "myea_hip_upload_dropout_noise", "myea_hip_compute_loss", "myea_hip_compute_accuracy_r", "myea_hip_gather_examples", "myea_hip_device_buffer_create", "myea_hip_device_buffer_destroy",
     "myea_hip_clear_training_arrays", "myea_hip_forward_pass", "myea_hip_compute_error", "myea_hip_backward_pass",
-    "myea_hip_update_derivative_weight", "myea_hip_update_derivative_weight_no_alloc", "myea_hip_backward_pass_and_update_derivative_weight", "myea_hip_update_parameter", "myea_hip_reset_loss", "myea_hip_get_loss",
+    "myea_hip_update_derivative_weight", "myea_hip_update_derivative_weight_no_alloc", "myea_hip_backward_pass_and_update_derivative_weight", "myea_hip_update_parameter",
+    "myea_hip_backward_pass_update_derivative_weight_and_update_parameter", "myea_hip_reset_loss", "myea_hip_get_loss",
     "myea_hip_download_gradient", "myea_hip_upload_gradient", "myea_hip_download_tensor", "myea_hip_upload_tensor",
     "myea_hip_profile_enable", "myea_hip_profile_read", "myea_hip_gemm_f32", "myea_hip_optimizer_update",
     "myea_hip_ceiling_mfma_f32", "myea_hip_ceiling_hbm_triad",
@@ -153,6 +154,7 @@ def load_library(path=LIB_PATH):
     lib.myea_hip_compute_error.argtypes = [vp, sz, vp, i32]
     lib.myea_hip_backward_pass.argtypes = [vp, sz]
     lib.myea_hip_backward_pass_and_update_derivative_weight.argtypes = [vp, sz]
+    lib.myea_hip_backward_pass_update_derivative_weight_and_update_parameter.argtypes = [vp, sz, sz]
     lib.myea_hip_update_derivative_weight.argtypes = [vp, sz, sz, sz]
     lib.myea_hip_update_derivative_weight_no_alloc.argtypes = [vp, sz, sz, sz]
     lib.myea_hip_update_parameter.argtypes = [vp, sz, sz]
@@ -410,6 +412,10 @@ class HipNetwork:
     def Backward_Pass__Update_Derivative_Weight(self, batch_size):
         """Backward_Pass then Update_Derivative_Weight over all layers, as one call"""
         self._check(self.lib.myea_hip_backward_pass_and_update_derivative_weight(self.handle, batch_size))
+
+    def Backward_Pass__Update_Derivative_Weight__Update_Parameter(self, batch_size, training_size):
+        """Backward_Pass, Update_Derivative_Weight over all layers and Update_Parameter, as one call"""
+        self._check(self.lib.myea_hip_backward_pass_update_derivative_weight_and_update_parameter(self.handle, batch_size, training_size))
 
     def Update_Derivative_Weight(self, batch_size, first_layer=1, end_layer=None):
         end_layer = self.desc.n_layers if end_layer is None else end_layer

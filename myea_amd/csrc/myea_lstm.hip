@@ -926,6 +926,7 @@ int Net::side_stream_create()
     MYEA_HIP_TRY(hipStreamCreateWithFlags(&side_stream, hipStreamNonBlocking));
     MYEA_HIP_TRY(hipEventCreateWithFlags(&fork_event, hipEventDisableTiming));
     MYEA_HIP_TRY(hipEventCreateWithFlags(&join_event, hipEventDisableTiming));
+    MYEA_HIP_TRY(hipEventCreateWithFlags(&update_event, hipEventDisableTiming));
     return MYEA_OK;
 }
 

@@ -79,7 +79,7 @@ struct Net {
     // independent of what `stream` is busy with: the second direction of a bidirectional LSTM layer, and the bias /
     // peephole column reductions of the weight-gradient phase beside its contractions.
     hipStream_t side_stream = nullptr;
-    hipEvent_t fork_event = nullptr, join_event = nullptr;
+    hipEvent_t fork_event = nullptr, join_event = nullptr, update_event = nullptr;
     float *parameters = nullptr, *gradient = nullptr, *opt[MYEA_STATE_KINDS] = {};
     uint8_t *masks = nullptr;
     unsigned long long mask_epoch = 1;   // advances whenever the masks or the propagation state change
@@ -160,6 +160,20 @@ struct Net {
     // the same call with every scratch buffer of its kernels taken from the library's static device array
     int update_derivative_weight_no_alloc(size_t B, size_t first, size_t end);
     int update_parameter(size_t B, size_t training_size);
+    // Update_Parameter in three parts: the step's scalars (advances the optimizer's time step), the elementwise update of a
+    // range of the flat vectors, and what follows the update (constraints, repacking)
+    int update_prepare(size_t B, size_t training_size, UpdateParams *p, double *bytes_per_param);
+    int update_range(const UpdateParams &p, size_t first, size_t count, double bytes_per_param);
+    int update_finish();
+    // Backward_Pass, Update_Derivative_Weight over all layers and Update_Parameter as one call: the weights of a
+    // fully-connected layer take their step on the side stream as soon as their gradient is complete and nothing reads them
+    // any more in this pass, beside the contractions of the layers below
+    int backward_pass_update_derivative_weight_and_update_parameter(size_t B, size_t training_size);
+    bool early_update_allowed() const;
+    int early_update_layer(size_t li);
+    const UpdateParams *early_update = nullptr;              // inside the call above, when it updates early
+    double early_bytes_per_param = 0;
+    std::vector<std::pair<size_t, size_t>> early_ranges;     // [first, end) of the flat vectors updated so far in this call
     int set_unit_activations(size_t li, const uint32_t *types, const float *steep, size_t count);
 
     // LSTM-with-peephole layers (myea_lstm.hip)
