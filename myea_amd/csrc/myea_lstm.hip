@@ -72,6 +72,7 @@ namespace {
     } while (0)
 
 constexpr size_t kMaxSlabs = 16;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 struct LstmGeom {
     size_t K, cpb, C, G, In, per_block, base;
@@ -94,33 +95,55 @@ __device__ __forceinline__ size_t peep_index(const LstmGeom &g, size_t gate, siz
     return g.base + k * g.per_block + g.cpb * (g.In + g.C) + 3 * g.In + 3 * g.C + gate * g.cpb + j;
 }
 
+// One workgroup per packed row (the index arithmetic of the flat layout once per row, on the scalar unit; lanes walk the row's
+// columns, which are consecutive in both layouts); the last workgroup takes the peepholes.
 __global__ __launch_bounds__(kBlock) void lstm_gather_kernel(LstmGeom g, const float *flat, float *Win, float *Wrec, float *peep)
 {
-    const size_t n_in = g.G * g.In, n_rec = g.G * g.C, n_peep = 3 * g.C, n = n_in + n_rec + n_peep;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-        if (i < n_in) Win[i] = flat[flat_index(g, i / g.In, i % g.In, false)];
-        else if (i < n_in + n_rec) { const size_t q = i - n_in; Wrec[q] = flat[flat_index(g, q / g.C, q % g.C, true)]; }
-        else { const size_t q = i - n_in - n_rec; peep[q] = flat[peep_index(g, q / g.C, q % g.C)]; }
+    const size_t r = blockIdx.x;
+    if (r == g.G) {
+        for (size_t q = threadIdx.x; q < 3 * g.C; q += kBlock) peep[q] = flat[peep_index(g, q / g.C, q % g.C)];
+        return;
     }
+    const float *from_in = flat + flat_index(g, r, 0, false), *from_rec = flat + flat_index(g, r, 0, true);
+    float *win = Win + r * g.In, *wrec = Wrec + r * g.C;
+    for (size_t a = threadIdx.x; a < g.In; a += kBlock) win[a] = from_in[a];
+    for (size_t a = threadIdx.x; a < g.C; a += kBlock) wrec[a] = from_rec[a];
 }
 
 // flat gradient += packed gradient (every flat slot is owned by exactly one packed element: no atomics)
-// gWin / gWrec hold s_in / s_rec split-K slabs, summed in slab order.
+// gWin / gWrec hold s_in / s_rec split-K slabs, summed in slab order.  One workgroup per packed row, as above; a lane takes
+// four consecutive columns when the widths allow (the slabs as 16-byte loads; the flat rows start at any dword).
 __global__ __launch_bounds__(kBlock) void lstm_scatter_add_kernel(LstmGeom g, float *flat, const float *gWin, int s_in, const float *gWrec, int s_rec)
 {
-    const size_t n_in = g.G * g.In, n_rec = s_rec > 0 ? g.G * g.C : 0, n = n_in + n_rec;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-        if (i < n_in) {
-            float v = 0.f;
-            for (int s = 0; s < s_in; ++s) v += gWin[(size_t)s * n_in + i];
-            flat[flat_index(g, i / g.In, i % g.In, false)] += v;
-        } else {
-            const size_t q = i - n_in;
-            float v = 0.f;
-            for (int s = 0; s < s_rec; ++s) v += gWrec[(size_t)s * n_rec + q];
-            flat[flat_index(g, q / g.C, q % g.C, true)] += v;
+    const size_t r = blockIdx.x, n_in = g.G * g.In, n_rec = g.G * g.C;
+    float *to_in = flat + flat_index(g, r, 0, false), *to_rec = flat + flat_index(g, r, 0, true);
+    const float *win = gWin + r * g.In, *wrec = gWrec + r * g.C;
+    if (((g.In | g.C) & 3) == 0) {
+        const size_t q_in = g.In / 4, q_all = q_in + (s_rec > 0 ? g.C / 4 : 0);
+        for (size_t q = threadIdx.x; q < q_all; q += kBlock) {
+            const bool rec = q >= q_in;
+            const size_t a = (rec ? q - q_in : q) * 4, slab = rec ? n_rec : n_in;
+            const float *from = (rec ? wrec : win) + a;
+            const int slabs = rec ? s_rec : s_in;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < slabs; ++s) v += *reinterpret_cast<const f32x4 *>(from + (size_t)s * slab);
+            float *to = (rec ? to_rec : to_in) + a;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) to[e] += v[e];
         }
+        return;
     }
+    for (size_t a = threadIdx.x; a < g.In; a += kBlock) {
+        float v = 0.f;
+        for (int s = 0; s < s_in; ++s) v += win[(size_t)s * n_in + a];
+        to_in[a] += v;
+    }
+    if (s_rec > 0)
+        for (size_t a = threadIdx.x; a < g.C; a += kBlock) {
+            float v = 0.f;
+            for (int s = 0; s < s_rec; ++s) v += wrec[(size_t)s * n_rec + a];
+            to_rec[a] += v;
+        }
 }
 
 __device__ __forceinline__ float sigmoid_f(float s) { return 1.f / (1.f + expf(-s)); }
@@ -730,8 +753,7 @@ int Net::lstm_parameters_changed()
     for (size_t li = 1; li < L.size(); ++li) {
         for (LstmLayer *q : {L[li].lstm, L[li].lstm2}) {
             if (!q) continue;
-            const size_t n = q->G * (q->In + q->C) + 3 * q->C;
-            hipLaunchKernelGGL(lstm_gather_kernel, dim3(grid_for(n, kBlock, 4096)), dim3(kBlock), 0, stream, geom_of(*q), parameters, q->Win, q->Wrec, q->peep);
+            hipLaunchKernelGGL(lstm_gather_kernel, dim3((unsigned)q->G + 1u), dim3(kBlock), 0, stream, geom_of(*q), parameters, q->Win, q->Wrec, q->peep);
             MYEA_HIP_TRY(hipGetLastError());
             if (q->WrecT) MYEA_TRY(launch_transpose(stream, q->G, q->C, q->Wrec, q->WrecT));
         }
@@ -1208,8 +1230,7 @@ int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t
             prof_end(2.0 * (double)B * (double)q.G * (double)q.C);
         }
     }
-    hipLaunchKernelGGL(lstm_scatter_add_kernel, dim3(grid_for(q.G * (q.In + q.C), kBlock, 4096)), dim3(kBlock), 0, stream, geom, gradient, q.gWin, s_in,
-                       q.gWrec, s_rec);
+    hipLaunchKernelGGL(lstm_scatter_add_kernel, dim3((unsigned)q.G), dim3(kBlock), 0, stream, geom, gradient, q.gWin, s_in, q.gWrec, s_rec);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
