@@ -116,6 +116,35 @@ def test_second_pass_doubles_the_gradient_then_adam_follows_its_closed_form(trai
     assert_close(net.download_optimizer_state(mb.OPT_STATE["SECOND_MOMENT"])[sel], v, 1e-5, 1e-20, what="second moment")
 
 
+def test_the_one_call_step_updates_the_wide_layers_early_and_equals_the_separate_calls(trained):
+    """Backward_Pass + Update_Derivative_Weight + Update_Parameter as one call: the four 4096 x 4096 layers take their Adam step on
+    the second stream beside the contractions below them (five update launches a step: four layers, then the head with the
+    biases), and parameters and moments equal those of the separate calls bit for bit"""
+    desc, h, w, X, Y = (trained[k] for k in ("desc", "h", "w", "X", "Y"))
+    nets = [mb.HipNetwork(desc, h) for _ in range(2)]
+    for n in nets:
+        n.set_state_propagation(mb.STATE_TRAINING)
+        n.upload_parameters(w)
+        n.Clear_Training_Arrays()
+    apart, one = nets
+    one.profile_enable(True)
+    for step in range(2):
+        for n in nets:
+            n.Forward_Pass(B, X)
+            n.Compute__Error(B, Y)
+        apart.Backward_Pass__Update_Derivative_Weight(B)
+        apart.Update_Parameter(B, 8 * B)
+        one.Backward_Pass__Update_Derivative_Weight__Update_Parameter(B, 8 * B)
+    assert one.profile_read(3)[0] == 2 * 5
+    one.profile_enable(False)
+    assert np.array_equal(apart.download_parameters(), one.download_parameters())
+    for kind in ("FIRST_MOMENT", "SECOND_MOMENT"):
+        assert np.array_equal(apart.download_optimizer_state(mb.OPT_STATE[kind]), one.download_optimizer_state(mb.OPT_STATE[kind])), kind
+    assert not one.download_gradient().any()
+    for n in nets:
+        n.close()
+
+
 def test_config5_full_size_sampled_examples_and_batch_additivity():
     """Bidirectional LSTM, 1024 cells per direction, input 256, T = 512, batch 64, per-step 32-class softmax (the largest
     recurrent configuration).  Without normalisation an example's forward values and deltas do not depend on the rest of
