@@ -555,6 +555,8 @@ __global__ __launch_bounds__(kBlock) void bn_backward_apply_kernel(size_t n, BnB
 
 __device__ __forceinline__ float sign_f(float v) { return v > 0.f ? 1.f : (v < 0.f ? -1.f : 0.f); }
 
+// V: elements per lane and trip (4: rows whose width is a multiple of 4, 16-byte loads and stores; 1 otherwise)
+template <int V>
 __global__ __launch_bounds__(kBlock) void compute_error_kernel(ErrorParams p)
 {
     __shared__ float red[5][kBlock / 64];
@@ -586,8 +588,22 @@ __global__ __launch_bounds__(kBlock) void compute_error_kernel(ErrorParams p)
             if (want == 0xffffffffu) want = (unsigned)p.H;
             if (lane == 0) acc += (want == got) ? 1.f : 0.f;
         }
-        for (size_t j = lane; j < p.H; j += 64) {
-            const float yo = y[j], de = d[j], diff = yo - de;
+        for (size_t j0 = (size_t)lane * V; j0 < p.H; j0 += 64 * V) {
+            float y_v[V], d_v[V], pre_v[V], err_v[V];
+            if (V == 4) {
+                const f32x4 y4 = *reinterpret_cast<const f32x4 *>(y + j0), d4 = *reinterpret_cast<const f32x4 *>(d + j0);
+                f32x4 q4 = {0.f, 0.f, 0.f, 0.f};
+                if (p.write_delta && !p.rnn_pre_quirk) q4 = *reinterpret_cast<const f32x4 *>(pre + j0);
+#pragma unroll
+                for (int e = 0; e < V; ++e) { y_v[e] = y4[e]; d_v[e] = d4[e]; pre_v[e] = q4[e]; }
+            } else {
+                y_v[0] = y[j0]; d_v[0] = d[j0]; pre_v[0] = (p.write_delta && !p.rnn_pre_quirk) ? pre[j0] : 0.f;
+            }
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+            const size_t j = j0 + v;
+            const float yo = y_v[v], de = d_v[v], diff = yo - de;
+            err_v[v] = 0.f;
             float e = 0.f; bool counted = true;
             switch (p.loss) {
             case MYEA_LOSS_ME:
@@ -620,8 +636,13 @@ __global__ __launch_bounds__(kBlock) void compute_error_kernel(ErrorParams p)
             default: break;
             }
             if (!p.write_delta) continue;  // Compute__Loss: the same accumulation, no delta
-            const float q = p.rnn_pre_quirk ? pre[0] : pre[j];
-            err[j] = af_derive(p.unit_act ? p.unit_act[j] : p.act, q, p.unit_steep ? p.unit_steep[j] : p.steep, yo) * diff;
+            const float q = p.rnn_pre_quirk ? pre[0] : pre_v[v];
+            err_v[v] = af_derive(p.unit_act ? p.unit_act[j] : p.act, q, p.unit_steep ? p.unit_steep[j] : p.steep, yo) * diff;
+            }
+            if (p.write_delta) {
+                if (V == 4) *reinterpret_cast<f32x4 *>(err + j0) = f32x4{err_v[0], err_v[1], err_v[2], err_v[3]};
+                else err[j0] = err_v[0];
+            }
         }
     }
     loss = wave_sum(loss); cnt = wave_sum(cnt); acc = wave_sum(acc); bits = wave_sum(bits); sum_y = wave_sum(sum_y);
@@ -1148,7 +1169,10 @@ int launch_compute_error(hipStream_t s, const ErrorParams &p)
 {
     if (p.T <= p.first_t || p.B == 0 || p.H == 0) return MYEA_OK;
     const size_t nrows = (p.T - p.first_t) * p.B;
-    hipLaunchKernelGGL(compute_error_kernel, dim3(grid_for(nrows, kBlock / 64, 1024)), dim3(kBlock), 0, s, p);
+    auto aligned = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    const bool vec = (p.H & 3) == 0 && aligned(p.values) && aligned(p.desired) && aligned(p.pre) && aligned(p.errors);
+    if (vec) hipLaunchKernelGGL(compute_error_kernel<4>, dim3(grid_for(nrows, kBlock / 64, 2048)), dim3(kBlock), 0, s, p);
+    else hipLaunchKernelGGL(compute_error_kernel<1>, dim3(grid_for(nrows, kBlock / 64, 1024)), dim3(kBlock), 0, s, p);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
