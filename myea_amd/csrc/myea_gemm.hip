@@ -509,10 +509,10 @@ __device__ __forceinline__ void gemm_tile(const GemmDev &p, const int block, flo
         cur = following;
     }
 
-    if (BM == 64 && BN == 64 && p.pair_partials) {   // only the 64 x 64 launches are split this way
+    if (BM == BN && p.pair_partials) {   // only launches of square tiles are split this way
         // Two workgroups share this tile, one per half of k (their ids are equal mod 8: the same XCD).  Whoever is done first
         // leaves its accumulators and goes; the other adds them and carries on to the epilogue.  The sum is half 0 + half 1
-        // either way.  The wait below is for a workgroup that has nothing left to do but store 16 KB and raise its flag.
+        // either way.  The wait below is for a workgroup that has nothing left to do but store its tile and raise its flag.
         __shared__ unsigned s_ticket;
         const int tile = block - split * nblocks;
         unsigned *ticket = p.pair_tickets + 2 * tile, *flag = ticket + 1;
@@ -715,7 +715,17 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     // At most one 64 x 64 tile per compute unit and a k worth splitting: two workgroups per tile, half of k each, combined in
     // the launch - a second wavefront per SIMD to fill the first one's waits, which such a launch otherwise lacks.
     // MYEA_GEMM_PAIR_K=0 keeps one workgroup per tile.
-    static const bool pair_k_off = [] { const char *e = std::getenv("MYEA_GEMM_PAIR_K"); return e && e[0] == '0'; }();
+    static const int pair_k = [] { const char *e = std::getenv("MYEA_GEMM_PAIR_K"); return e ? std::atoi(e) : 3; }();   // bit 0: 64 x 64 tiles, bit 1: 128 x 128
+    const bool pair_k_off = !(pair_k & 1);
+    // The same one size up: at most one 128 x 128 tile per compute unit (a batch of 1024 in front of 4096 units) would run as 64 x
+    // 128 tiles to put two workgroups on every compute unit; two workgroups sharing a 128 x 128 tile's k do that with the larger
+    // tile's operand reuse.
+    if ((pair_k & 2) && p.pair_partials && p.pair_tickets && d.ksplit == 1 && tiles_128 <= kGemmPairTiles && tiles_128 % 8 == 0 && tiles_128 >= 128 && p.K >= 2048) {
+        d.ksplit = 2;
+        d.kchunk = ((p.K + 1) / 2 + kBK - 1) / kBK * kBK;
+        d.pair_partials = p.pair_partials; d.pair_tickets = p.pair_tickets;
+        return launch_layout_vec<128, 128>(stream, d, a_kc, b_kc);
+    }
     const long tiles_64 = (long)((p.M + 63) / 64) * ((p.N + 63) / 64);
     if (p.pair_partials && p.pair_tickets && !pair_k_off && d.ksplit == 1 && tiles_64 <= kGemmPairTiles && tiles_64 % 8 == 0 && tiles_64 >= 128 && p.K >= 512) {
         d.ksplit = 2;

@@ -60,7 +60,7 @@ struct GemmParams {
     // Two-way split along k INSIDE the launch, any epilogue: when the problem has too few tiles to give every compute unit two
     // workgroups, two workgroups share a tile, each contracting over half of k; the first to finish leaves its accumulators in
     // `pair_partials`, the second adds them to its own (half 0 + half 1: the same sum whichever finishes first) and runs the
-    // epilogue.  pair_partials: at least 256 x 4096 floats; pair_tickets: 2 x 256 words, zero before the first use (a launch
+    // epilogue.  pair_partials: at least 256 x 16384 floats (256 tiles of up to 128 x 128); pair_tickets: 2 x 256 words, zero before the first use (a launch
     // leaves them zero).  One launch at a time may use a given pair of buffers.  Null = off; the launcher decides per problem.
     float *pair_partials;
     unsigned *pair_tickets;

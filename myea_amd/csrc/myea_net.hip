@@ -339,7 +339,7 @@ int Net::create(const myea_net_desc &desc)
     }
     MYEA_TRY(side_stream_create());
     {   // forward contractions of few tiles split each tile's k between two workgroups: their meeting place
-        MYEA_TRY(dev_alloc(&gemm_pair_partials, (size_t)kGemmPairTiles * 64 * 64));
+        MYEA_TRY(dev_alloc(&gemm_pair_partials, (size_t)kGemmPairTiles * 128 * 128));
         void *q = nullptr;
         MYEA_HIP_TRY(hipMalloc(&q, 2 * kGemmPairTiles * sizeof(unsigned)));
         MYEA_HIP_TRY(hipMemset(q, 0, 2 * kGemmPairTiles * sizeof(unsigned)));

@@ -339,3 +339,33 @@ def test_forward_contraction_that_splits_a_tile_between_two_workgroups():
         assert np.array_equal(a, b)
     for k, (a, b) in enumerate(zip(outs[0], outs[2])):
         assert_close(a, b, 1e-4, 1e-5 * max(1.0, float(np.abs(b).max())), what="tensor %d" % k)
+
+
+def test_forward_contraction_that_splits_a_128_tile_between_two_workgroups():
+    """One size up: at most one 128 x 128 tile per compute unit and k >= 2048 (here 1024 x 2048 outputs over k = 2048; the layer
+    behind it has half the tiles and takes the 64 x 64 form): outputs held against float64 on sampled entries - the oracle
+    would take minutes at this size - and bit for bit the same from run to run."""
+    specs = [dict(units=2048), dict(units=2048, activation="TANH"), dict(units=1024, activation="RELU"), dict(units=16, activation="LINEAR")]
+    B = 1024
+    desc = mb.make_desc(specs, B, 1)
+    h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["GD"], type_loss_function=mb.LOSS["MSE"])
+    w = glorot_parameters(desc, 8, bias_range=0.2)
+    rng = np.random.default_rng(8)
+    X = rng.normal(0, 1, (B, 2048)).astype(np.float32)
+    runs = []
+    for _ in range(2):
+        n = mb.HipNetwork(desc, h)
+        n.set_state_propagation(mb.STATE_TRAINING)
+        n.upload_parameters(w)
+        n.Forward_Pass(B, X)
+        runs.append([n.download_tensor(li, mb.TENSOR["OUTPUTS"], B * desc.layers[li].n_units) for li in (1, 2)])
+        n.close()
+    for a, b in zip(*runs):
+        assert np.array_equal(a, b)
+    l = desc.layers[1]
+    W = w[l.first_connection_index:l.first_connection_index + 2048 * 2048].reshape(2048, 2048).astype(np.float64)
+    bias = w[l.first_bias_connection_index:l.first_bias_connection_index + 2048].astype(np.float64)
+    rows, cols = rng.integers(0, B, 256), rng.integers(0, 2048, 256)
+    want = np.tanh(np.einsum("sk,sk->s", X[rows].astype(np.float64), W[cols]) + bias[cols])
+    got = runs[0][0].reshape(B, 2048)[rows, cols]
+    assert_close(got, want, 1e-4, 1e-5, what="outputs of the split 128 x 128 tiles")
