@@ -24,7 +24,7 @@ if ROOT not in sys.path:
 # HBM bytes per contraction launch (mean over the launches of one step): NOT measured by this script's run.  Recorded
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same counters read for copies of
 # known size (FETCH_SIZE x2, WRITE_SIZE x1); the line names the file the figure comes from.
-RECORDED_TRAFFIC = {"fc4096x4_b1024_adam": dict(bytes_per_launch=2886299 * 1024 / 10,
+RECORDED_TRAFFIC = {"fc4096x4_b1024_adam": dict(bytes_per_launch=2944490 * 1024 / 10,
                                                 source="recorded constant, not measured in this run: profiles/hbm_traffic__fc4096x4_b1024_adam__pmc.txt")}
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
