@@ -33,6 +33,7 @@ struct GemmParams {
     long lda, ldb, ldc;
     int a_k_contiguous, b_k_contiguous;
     int accumulate;
+    int c_is_zero;          // with accumulate: C is known to hold zeros, so the launch may store its product instead of adding it (same values)
     int epilogue;
     const float *bias;      // EPI_FC_FORWARD, may be null
     float *aux_out;         // EPI_FC_FORWARD, [M][ldc], may be null

@@ -151,6 +151,11 @@ struct Net {
     int backward_pass_and_update_derivative_weight(size_t B);
     bool pairing = false;              // inside the call above
     std::vector<char> dw_done;         // per layer: the weight contraction already ran in this pass
+    // per layer: the layer's slice of the gradient is known to be zero (the update zeroes what it reads), so its next weight
+    // contraction may store its product instead of adding it element by element at the L2.  MYEA_DW_STORE=0: always add.
+    std::vector<char> dw_zero;
+    void gradient_known_zero(bool zero) { dw_zero.assign(d.n_layers, zero ? 1 : 0); }
+    bool dw_may_store(size_t li) const;
     bool fc_dw_params(size_t li, size_t B, GemmParams *g);   // false: the layer's weight gradient is not one plain contraction
     int update_derivative_weight(size_t B, size_t first, size_t end);
     int update_derivative_weight_contraction(size_t li, size_t B);   // the weight contraction(s) of one layer

@@ -248,6 +248,7 @@ int Net::create(const myea_net_desc &desc)
     for (int k = 0; k < MYEA_STATE_KINDS; ++k) MYEA_TRY(dev_alloc(&opt[k], P));
     MYEA_HIP_TRY(hipMemset(parameters, 0, P * sizeof(float)));
     MYEA_HIP_TRY(hipMemset(gradient, 0, P * sizeof(float)));
+    gradient_known_zero(true);
     for (int k = 0; k < MYEA_STATE_KINDS; ++k) MYEA_HIP_TRY(hipMemset(opt[k], 0, P * sizeof(float)));
     MYEA_TRY(launch_fill(0, opt[MYEA_STATE_PREVIOUS_STEPS], P, h.rprop_delta_zero));
     if (d.total_normalized_units) MYEA_TRY(launch_fill(0, parameters + d.total_weights + d.total_bias, d.total_normalized_units, 1.f));
@@ -901,6 +902,7 @@ int Net::backward_into_layer(size_t li, size_t B)
                 if (paired) {
                     prof_end(2.0 * (double)rows * (double)H * (double)Out + 2.0 * (double)w.M * (double)w.N * (double)w.K);
                     dw_done[gi] = 1;
+                    if (gi < dw_zero.size()) dw_zero[gi] = 0;
                     if (early_update) MYEA_TRY(early_update_layer(gi));   // that launch was the last reader of the layer's weights in this pass
                 } else prof_cancel();
             }
@@ -1109,9 +1111,15 @@ bool Net::fc_dw_params(size_t li, size_t B, GemmParams *out)
     g.B = x; g.ldb = (long)In; g.b_k_contiguous = 0;
     g.C = gradient + l.first_connection_index; g.ldc = (long)In;
     g.M = (int)H; g.N = (int)In; g.K = (int)rows;
-    g.accumulate = 1; g.epilogue = EPI_NONE;
+    g.accumulate = 1; g.c_is_zero = dw_may_store(li) ? 1 : 0; g.epilogue = EPI_NONE;
     *out = g;
     return true;
+}
+
+bool Net::dw_may_store(size_t li) const
+{
+    static const bool off = [] { const char *e = std::getenv("MYEA_DW_STORE"); return e && e[0] == '0'; }();
+    return !off && li < dw_zero.size() && dw_zero[li];
 }
 
 // the weight contraction(s) of layer li: dW += delta^T X (:178-216); LSTM layers: their input and recurrent weights
@@ -1137,9 +1145,10 @@ int Net::update_derivative_weight_contraction(size_t li, size_t B)
         g.B = x + roff * In; g.ldb = (long)In; g.b_k_contiguous = 0;
         g.C = gradient + l.first_connection_index; g.ldc = (long)In;
         g.M = (int)H; g.N = (int)In; g.K = (int)rows;
-        g.accumulate = 1; g.epilogue = EPI_NONE;
+        g.accumulate = 1; g.c_is_zero = dw_may_store(li) ? 1 : 0; g.epilogue = EPI_NONE;
         const int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
-        if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
+        if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.c_is_zero = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
+        else if (li < dw_zero.size()) dw_zero[li] = 0;   // from here on the slice holds this product
         prof_begin(2);
         MYEA_TRY(launch_gemm(stream, g));
         if (slabs > 1) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
@@ -1475,6 +1484,7 @@ int Net::update_range(const UpdateParams &whole, size_t first, size_t count, dou
 
 int Net::update_finish()
 {
+    gradient_known_zero(true);   // the update zeroed every element it read
     if (h.regularization__max_norm_constraints != 0.f) {
         MYEA_TRY(build_max_norm_segments());
         MYEA_TRY(launch_max_norm(stream, n_segments, seg_first, seg_len, longest_segment, h.regularization__max_norm_constraints, parameters));
@@ -1718,6 +1728,7 @@ int myea_hip_clear_training_arrays(myea_hip_net *n)
     NET_OR_FAIL(n);
     const size_t bytes = n->net.d.total_parameters * sizeof(float);
     MYEA_HIP_TRY(hipMemsetAsync(n->net.gradient, 0, bytes, n->net.stream));
+    n->net.gradient_known_zero(true);
     return n->net.clear_optimizer();
 }
 
@@ -1791,6 +1802,7 @@ int myea_hip_upload_gradient(myea_hip_net *n, const float *g, size_t c)
 {
     NET_OR_FAIL(n);
     if (!g) { myea::set_last_error("upload_gradient: null"); return MYEA_E_INVALID; }
+    n->net.gradient_known_zero(false);
     return copy_vec(n, n->net.gradient, nullptr, g, c, "upload_gradient");
 }
 
