@@ -166,7 +166,8 @@ static int check_desc(const myea_net_desc &d)
             // between fully-connected / pooling layers of a stack without blocks around it; the width must be the one
             // Assign__Post__Layer computes (NN/Neural_Network__Compile.cpp:250-271) - the kernels index with it
             any_pool = true;
-            if (li == 0 || li + 1 >= d.n_layers || block_end != 0) { set_last_error("layer %u: a pooling layer sits between the input and the output layer, outside residual blocks", li); return MYEA_E_UNSUPPORTED; }
+            if (li == 0 || li + 1 >= d.n_layers) { set_last_error("layer %u: a pooling layer sits between the input and the output layer", li); return MYEA_E_UNSUPPORTED; }
+            if (block_end != 0 && d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) { set_last_error("layer %u: a pooling layer may be any member of a residual block but the first", li); return MYEA_E_UNSUPPORTED; }
             const myea_layer_desc &pl = d.layers[li - 1], &nl = d.layers[li + 1];
             if ((pl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(pl)) || (nl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(nl))) {
                 set_last_error("layer %u: pooling layers connect to fully-connected or pooling layers on this path", li);
@@ -180,8 +181,8 @@ static int check_desc(const myea_net_desc &d)
             if (l.type_dropout != MYEA_DROPOUT_NONE || l.type_normalization != MYEA_NORMALIZATION_NONE) { set_last_error("layer %u: a pooling layer carries no dropout or normalization", li); return MYEA_E_UNSUPPORTED; }
         }
         if (block_end != 0) {
-            if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("layer %u: only fully-connected layers may sit inside a residual block", li); return MYEA_E_UNSUPPORTED; }
-            group[li] = (d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) ? 1 : 2;
+            if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(l)) { set_last_error("layer %u: only fully-connected and pooling layers may sit inside a residual block", li); return MYEA_E_UNSUPPORTED; }
+            group[li] = layer_is_pooling(l) ? 3 : ((d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) ? 1 : 2);
             if (li == block_end) block_end = 0;
         } else if (l.type_layer == MYEA_LAYER_RESIDUAL) {
             if (l.block_depth == 0 || (uint64_t)li + l.block_depth + 1 >= d.n_layers) { set_last_error("layer %u: residual block of depth %u does not fit in front of a consumer", li, l.block_depth); return MYEA_E_INVALID; }
@@ -277,14 +278,17 @@ int Net::create(const myea_net_desc &desc)
         if (li > 1 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             if (d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) o.group = 1;
             else if (L[li - 1].group != 0 && o.prev == li - 1) o.group = 2;  // the first layer after a block connects to the residual layer
+        } else if (li > 1 && layer_is_pooling(l) && L[li - 1].group != 0 && o.prev == li - 1) {
+            o.group = 3;   // a pooling member of a block: basic units as wide as the layer, no activation or normalised units
         }
         if (l.type_layer == MYEA_LAYER_RESIDUAL) {
             o.NH = (size_t)myea_net_desc_number_outputs(&d, (uint32_t)(li + l.block_depth));
             o.AH = o.H;
             o.pad = ((o.In > o.NH ? o.In - o.NH : o.NH - o.In) + 1) / 2;  // Assign__Post__Layer, NN/Neural_Network__Compile.cpp:277
         } else {
-            o.AH = o.group == 0 ? o.H : (o.group == 1 ? 0 : o.In);
-            o.NH = o.group == 0 ? o.H : o.In;
+            const bool own_width = o.group == 0 || o.group == 3;
+            o.AH = own_width ? o.H : (o.group == 1 ? 0 : o.In);
+            o.NH = own_width ? o.H : o.In;
         }
         if (o.H > max_h) max_h = o.H;
         const size_t sz = T * B * o.H, sa = T * B * o.AH, sn = T * B * o.NH;
@@ -667,6 +671,11 @@ int Net::forward_residual_block(size_t ri, size_t B)
             DevLayer &o = L[m];
             const size_t In = o.In, H = o.H;
             const float *cur = layer_outputs(o.prev) + roff * In;
+            if (layer_is_pooling(l)) {   // a pooling member (Forward_Pass__Residual__Layer, :4005-4030): windows over the member before it
+                MYEA_TRY(launch_pool_forward(stream, pool_params(m, B), cur, o.values + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr));
+                values_ready = false;
+                continue;
+            }
             if (layer_uses_norm(l)) {
                 MYEA_TRY(bn_forward(m, t, B, cur, training));
                 cur = o.normalizes + roff * In;
@@ -686,7 +695,7 @@ int Net::forward_residual_block(size_t ri, size_t B)
             values_ready = false;
             if (m < last) {
                 const myea_layer_desc &nx = d.layers[m + 1];
-                if (!layer_uses_norm(nx) && !L[m + 1].unit_act && gemm_can_fuse_activation((int)nx.type_activation_function)) {
+                if (layer_is_dense(nx) && !layer_uses_norm(nx) && !L[m + 1].unit_act && gemm_can_fuse_activation((int)nx.type_activation_function)) {
                     g.act = (int)nx.type_activation_function;
                     g.aux_out = L[m + 1].values + roff * H;
                     g.colscale = drops[m + 1] ? L[m + 1].colscale + t * L[m + 1].AH : nullptr;
@@ -698,7 +707,7 @@ int Net::forward_residual_block(size_t ri, size_t B)
             prof_end(2.0 * (double)B * (double)H * (double)In);
         }
         DevLayer &o = L[ri];
-        const float *blk = L[last].summations + roff * L[last].H;
+        const float *blk = layer_outputs(last) + roff * L[last].H;   // a dense member's sums, a pooling member's values
         if (layer_uses_norm(r)) {
             MYEA_TRY(bn_forward(ri, t, B, blk, training));
             blk = o.normalizes + roff * o.NH;
@@ -974,7 +983,7 @@ int Net::backward_residual_block(size_t ri, size_t B)
             float *tmp = tmp1 + roff * ro.NH;
             MYEA_TRY(launch_padded_add(stream, B, ro.NH, res_errors, ro.H, crop, nullptr, 0, 0, tmp));
             if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, tmp, ro.noise, beta, 1.f));
-            MYEA_TRY(bn_backward(ri, t, B, L[last].summations + roff * L[last].H, tmp, last_errors));
+            MYEA_TRY(bn_backward(ri, t, B, layer_outputs(last) + roff * L[last].H, tmp, last_errors));
         } else {
             MYEA_TRY(launch_padded_add(stream, B, ro.NH, res_errors, ro.H, crop, nullptr, 0, 0, last_errors));
             if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, last_errors, ro.noise, beta, 1.f));
@@ -985,6 +994,11 @@ int Net::backward_residual_block(size_t ri, size_t B)
             const bool norm = layer_uses_norm(l);
             if (o.group == 1 && !norm) break;
             const size_t In = o.In, H = o.H;
+            if (layer_is_pooling(l)) {   // hands its delta down through its windows (Backward_Pass__Gradient__Residual__Layer, :753-772), nothing else
+                MYEA_TRY(launch_pool_backward(stream, pool_params(m, B), o.neuron_errors + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr,
+                                              L[m - 1].neuron_errors + roff * In));
+                continue;
+            }
             float *dst = (o.group == 2 ? L[m - 1].neuron_errors : o.in_errors) + roff * In;
             float *tmp = tmp1 + roff * In;
             const float *prev_out = layer_outputs(o.prev) + roff * In;

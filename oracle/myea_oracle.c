@@ -304,7 +304,8 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
                 o->NH = b;
             } else o->H = layer_width(l);
             o->In = li ? n->L[o->prev].H : 0;
-            if (l->type_layer != MYEA_LAYER_RESIDUAL) { o->AH = o->group ? (o->group == 1 ? 0 : o->In) : o->H; o->NH = o->group ? o->In : o->H; }
+            if (is_pooling(l)) { o->AH = o->H; o->NH = o->H; }   /* basic units: as wide as the layer, inside a block too */
+            else if (l->type_layer != MYEA_LAYER_RESIDUAL) { o->AH = o->group ? (o->group == 1 ? 0 : o->In) : o->H; o->NH = o->group ? o->In : o->H; }
             else o->AH = o->H;
         }
     }
@@ -317,7 +318,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
     for (size_t li = 0; li < desc->n_layers; ++li) {
         const myea_layer_desc *l = &desc->layers[li];
         olayer *o = &n->L[li];
-        if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED && !(o->group == 2 && is_pooling(l))) { free(n); return MYEA_E_UNSUPPORTED; }
         if (l->type_layer == MYEA_LAYER_LSTM && l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_ZONEOUT) { free(n); return MYEA_E_UNSUPPORTED; }
         /* with more cells per block the reference's indices [3] .. [8] into the layer's normalised units (NN/Neural_Network.cpp:4498-4613)
          * land on the second cell's units instead of the block's (the units are laid out per block: 3 per cell, then 6,
@@ -754,6 +755,8 @@ static void fwd_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_t B)
         fwd_k_sparse(n, t, B, H, n->state == MYEA_STATE_TRAINING ? (size_t)l->k_sparsity : (size_t)(l->alpha_sparsity * (float)l->k_sparsity), out);
 }
 
+static void fwd_pooling(myea_oracle_net *n, size_t li, size_t t, size_t B);
+
 /* Forward_Pass__Residual__FC: NN/Neural_Network__Forward_Pass__OpenMP.cpp:4039-4433.  Pre-activation order on the
  * layer's INPUT (fan-in wide): [BN] -> (not for the block's first layer: activation -> dropout) -> weights -> bias.
  * The layer's output is its summation. */
@@ -790,7 +793,11 @@ static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t t, size_t B
     const myea_layer_desc *r = &n->d.layers[ri];
     olayer *o = &n->L[ri];
     size_t last = ri + r->block_depth, Bmax = n->d.batch_size;
-    for (size_t li = ri + 1; li <= last; ++li) fwd_residual_fc_layer(n, li, t, B);
+    /* Forward_Pass__Residual__Layer, :3999-4036: fully-connected and pooling members */
+    for (size_t li = ri + 1; li <= last; ++li) {
+        if (is_pooling(&n->d.layers[li])) fwd_pooling(n, li, t, B);
+        else fwd_residual_fc_layer(n, li, t, B);
+    }
     float *blk = layer_outputs(n, last);
     size_t nb = n->L[last].H, na = n->L[o->prev].H;
     if (layer_uses_norm(r)) {
@@ -1809,11 +1816,14 @@ static void bwd_gradient_residual(myea_oracle_net *n, size_t ri, size_t B)
     size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, last = ri + r->block_depth;
     for (size_t li = last; li > ri; --li) {
         olayer *o = &n->L[li];
-        memset(o->neuron_errors, 0, T * Bmax * o->H * sizeof(float));
+        const int pooling = is_pooling(&n->d.layers[li]);
+        float *delta = pooling ? o->af_errors : o->neuron_errors;   /* Layer::ptr_array_derivative_outputs of the member */
+        memset(delta, 0, T * Bmax * o->H * sizeof(float));
         for (size_t t = T; t-- > 0;) {   /* time steps in descending order, like every dense layer of a recurrent network */
-            if (li == last) bwd_residual_block_to_last(n, ri, t, B, o->neuron_errors);
-            else bwd_residual_fc_to_previous(n, li + 1, t, B, o->neuron_errors);
-            bwd_gradient_residual_fc(n, li, t, B);
+            if (li == last) bwd_residual_block_to_last(n, ri, t, B, delta);
+            else if (is_pooling(&n->d.layers[li + 1])) bwd_pooling_to_previous(n, li + 1, t, B, delta);   /* :753-758, :767-772 */
+            else bwd_residual_fc_to_previous(n, li + 1, t, B, delta);
+            if (!pooling) bwd_gradient_residual_fc(n, li, t, B);   /* a pooling member has nothing of its own to reduce (:802-804) */
         }
     }
 }

@@ -20,6 +20,10 @@ EXTRA = {
     "relu_bn_dropout_blocks": ([fc(64), fc(96, "RELU")] + sum(([res(2), fc(96, "RELU", normalization="BATCH_NORMALIZATION"),
                                 fc(96, "RELU", normalization="BATCH_NORMALIZATION", dropout="BERNOULLI_INVERTED", keep=0.5)] for _ in range(4)), [])
                                + [fc(20, "SOFTMAX")], 64),
+    # pooling members at a width the tiled kernels see: a dilated max pooling (96 -> 47) between normalised dense members, dropout behind it
+    "pooling_member_wide": ([fc(48), fc(64, "RELU"), res(3, normalization="BATCH_NORMALIZATION"), fc(96, "RELU", normalization="BATCH_NORMALIZATION"),
+                             dict(type="max_pooling", kernel=3, stride=2, padding=1, dilation=2), fc(64, "TANH", dropout="BERNOULLI_INVERTED", keep=0.5),
+                             fc(10, "SOFTMAX")], 32),
     # odd widths: guarded scalar-load contraction path, shortcut wider and narrower in consecutive blocks
     "odd_widths": ([fc(19), res(2), fc(31, "TANH"), fc(27, "LEAKY_RELU"), res(1), fc(13, "SIGMOID"), fc(7, "LINEAR")], 11),
 }
@@ -123,9 +127,11 @@ def _mostly_close(a, b, what, fraction=0.01):
 
 def test_recurrent_depth_is_the_block_time_step_by_time_step_on_the_gpu():
     """residual blocks with a recurrent depth: against T feed-forward runs of the same library, then against the oracle"""
-    from tests.test_oracle_residual import RECURRENT_SPECS, check_recurrent_depth_is_the_block_time_step_by_time_step
-    check_recurrent_depth_is_the_block_time_step_by_time_step(
-        lambda desc: mb.HipNetwork(desc, mb.default_hyper(type_loss_function=mb.LOSS["MSE"])), lambda specs, B, T: mb.make_desc(specs, B, T), rel=1e-4, abs_=1e-5)
+    from tests.test_oracle_residual import RECURRENT_POOLING_SPECS, RECURRENT_SPECS, check_recurrent_depth_is_the_block_time_step_by_time_step
+    for specs in (None, RECURRENT_POOLING_SPECS):   # the normalised stack, then one with pooling members
+        check_recurrent_depth_is_the_block_time_step_by_time_step(
+            lambda desc: mb.HipNetwork(desc, mb.default_hyper(type_loss_function=mb.LOSS["MSE"])), lambda specs, B, T: mb.make_desc(specs, B, T), rel=1e-4, abs_=1e-5,
+            specs=specs)
     T, B, Bmax = 4, 29, 32   # enough examples for well-conditioned batch statistics
     desc = mb.make_desc(RECURRENT_SPECS, Bmax, T)
     h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["ADAM"], type_loss_function=mb.LOSS["MSE"])

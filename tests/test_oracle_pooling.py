@@ -92,11 +92,11 @@ def test_average_pooling_with_dilation_follows_the_reference_window():
     assert_close(net.download_tensor(2, mb.TENSOR["OUTPUTS"], 4), np.array(want), rel=1e-6)
 
 
-def test_pooling_layers_are_refused_where_the_reference_has_no_path():
+def test_pooling_layers_are_refused_where_this_path_has_none():
     with pytest.raises(ValueError):    # as the output layer
         oracle_desc([dict(units=6), dict(units=8, activation="TANH"), dict(type="max_pooling", kernel=2, stride=2)], 2)
     with pytest.raises(ValueError):    # window larger than the padded input
         oracle_desc([dict(units=6), dict(units=3, activation="TANH"), dict(type="average_pooling", kernel=9, stride=1), dict(units=2, activation="LINEAR")], 2)
-    with pytest.raises(ValueError):    # inside a residual block
-        oracle_desc([dict(units=6), dict(type="residual", block_depth=2), dict(units=6, activation="RELU"), dict(type="max_pooling", kernel=2, stride=1, padding=1),
+    with pytest.raises(ValueError):    # as the first member of a residual block (any other member may be a pooling layer)
+        oracle_desc([dict(units=6), dict(type="residual", block_depth=2), dict(type="max_pooling", kernel=2, stride=1, padding=1), dict(units=6, activation="RELU"),
                      dict(units=3, activation="LINEAR")], 2)

@@ -11,6 +11,7 @@ import torch
 from myea_amd import binding as mb
 from tests.common import assert_close, glorot_parameters, one_hot, oracle_desc, oracle_hyper, run_step
 from tests.oracle_lib import OracleNetwork, load_oracle
+from tests.test_oracle_pooling import _torch_pool
 
 T64 = torch.float64
 
@@ -165,6 +166,11 @@ class TorchResidualNet:
                 u = x
                 for k in range(1, sp["block_depth"] + 1):
                     m = li + k
+                    if specs[m].get("type", "").endswith("pooling"):   # a pooling member: windows over the member before it
+                        u, _ = _torch_pool(specs[m], u)
+                        u.retain_grad()
+                        self.taps[m] = u
+                        continue
                     if specs[m].get("normalization", "NONE") != "NONE":
                         u = self._bn(m, u)
                     if k > 1:
@@ -222,6 +228,16 @@ CASES = {
                              res(1, normalization="BATCH_NORMALIZATION"), fc(13, "TANH"), fc(5, "SINE_SYMMETRIC"), fc(4, "SOFTMAX")], 8),
     # odd difference of one: offset (1 + 1) // 2 = 1, so the narrower operand lands on the LAST column
     "difference_of_one": ([fc(4), fc(5, "TANH"), res(1), fc(6, "TANH"), fc(2, "LINEAR")], 5),
+    # pooling members (Forward_Pass__Residual__Layer's switch, NN/Neural_Network__Forward_Pass__OpenMP.cpp:4005-4030): an average
+    # pooling between two dense members (12 -> 6), a normalised member behind it
+    "average_pooling_member": ([fc(6), fc(8, "TANH"), res(3), fc(12, "TANH"), dict(type="average_pooling", kernel=2, stride=2),
+                                fc(8, "SIGMOID", normalization="BATCH_NORMALIZATION"), fc(4, "SOFTMAX")], 7),
+    # a max pooling as the block's LAST member (11 -> 6 with padding: narrower than the 9-wide shortcut) under a block-level
+    # normalisation, and two pooling members in a row
+    "max_pooling_last_member": ([fc(5), fc(9, "TANH"), res(2, normalization="BATCH_NORMALIZATION"), fc(11, "TANH"),
+                                 dict(type="max_pooling", kernel=3, stride=2, padding=1), fc(3, "LINEAR")], 6),
+    "two_pooling_members": ([fc(5), fc(7, "SIGMOID"), res(4), fc(16, "TANH"), dict(type="max_pooling", kernel=2, stride=2),
+                             dict(type="average_pooling", kernel=3, stride=1, padding=1), fc(7, "TANH"), fc(2, "LINEAR")], 6),
 }
 
 
@@ -356,7 +372,13 @@ RECURRENT_SPECS = [fc(5), fc(6, "TANH", normalization="BATCH_NORMALIZATION", nor
                    fc(3, "LINEAR")]
 
 
-def check_recurrent_depth_is_the_block_time_step_by_time_step(make_net, make_desc, rel=2e-5, abs_=2e-6):
+# the same with pooling members: a max pooling between two dense members (10 -> 5), an average pooling as the last one (6 -> 7)
+RECURRENT_POOLING_SPECS = [fc(5), fc(6, "TANH"), res(4), fc(10, "TANH"), dict(type="max_pooling", kernel=2, stride=2),
+                           fc(6, "SIGMOID", dropout="BERNOULLI_INVERTED", keep=0.5), dict(type="average_pooling", kernel=2, stride=1, padding=1),
+                           fc(3, "LINEAR")]
+
+
+def check_recurrent_depth_is_the_block_time_step_by_time_step(make_net, make_desc, rel=2e-5, abs_=2e-6, specs=None):
     """A stack of dense layers and residual blocks has no recurrence: with a recurrent depth T every layer, every batch
     normalisation (its own statistics and running averages per time step) and every dropout mask (its own per time step) works
     on the time steps one by one (Recurrent__Forward_Pass__Residual*, NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:563-817;
@@ -364,7 +386,7 @@ def check_recurrent_depth_is_the_block_time_step_by_time_step(make_net, make_des
     the t-th slice of the inputs, targets, masks and normalisation parameters, and the weight gradients are the sums over the
     time steps - the feed-forward path is pinned by float64 differentiation above."""
     T, B, Bmax = 3, 5, 6
-    specs = RECURRENT_SPECS
+    specs = specs or RECURRENT_SPECS
     deep, flat = make_desc(specs, Bmax, T), make_desc(specs, Bmax, 1)
     rng = np.random.default_rng(17)
     X = rng.normal(0, 1, (B, T, 5)).astype(np.float32)
@@ -397,6 +419,8 @@ def check_recurrent_depth_is_the_block_time_step_by_time_step(make_net, make_des
         run_step(one, B, X[:, t], Y[:, t], update=False)
         assert_close(out[t, :B], one.download_tensor(last, mb.TENSOR["OUTPUTS"]).reshape(Bmax, 3)[:B], rel, abs_, what="outputs of time step %d" % t)
         for li in (1, 2, 3):   # the running averages of time step t are the feed-forward network's
+            if specs[li].get("normalization", "NONE") == "NONE":
+                continue
             nh = deep.layers[li + 1].first_normalized_unit_index - deep.layers[li].first_normalized_unit_index
             for kind in ("NORM_MEANS_AVERAGES", "NORM_VARIANCES_AVERAGES"):
                 assert_close(net.download_tensor(li, mb.TENSOR[kind], T * nh).reshape(T, nh)[t], one.download_tensor(li, mb.TENSOR[kind], nh).reshape(nh), rel, abs_,
@@ -408,6 +432,11 @@ def check_recurrent_depth_is_the_block_time_step_by_time_step(make_net, make_des
 def test_recurrent_depth_is_the_block_time_step_by_time_step():
     check_recurrent_depth_is_the_block_time_step_by_time_step(
         lambda desc: OracleNetwork(desc, oracle_hyper(type_loss_function=mb.LOSS["MSE"])), oracle_desc)
+
+
+def test_recurrent_depth_with_pooling_members_is_the_block_time_step_by_time_step():
+    check_recurrent_depth_is_the_block_time_step_by_time_step(
+        lambda desc: OracleNetwork(desc, oracle_hyper(type_loss_function=mb.LOSS["MSE"])), oracle_desc, specs=RECURRENT_POOLING_SPECS)
 
 
 def test_float64_model_reproduces_the_dropout_and_renormalisation_cases_of_the_oracle():
