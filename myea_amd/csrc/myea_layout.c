@@ -140,9 +140,8 @@ int myea_net_desc_layout(myea_net_desc *d)
     for (uint32_t li = 1; li < d->n_layers; ++li) {
         myea_layer_desc *l = &d->layers[li];
         if (!is_pooling(l)) continue;
-        /* inside a residual block a pooling layer may be any member but the first (Assign__Post__Residual_Layer,
-         * NN/Neural_Network__Compile.cpp:352-376, computes its width by the same formulas) */
-        { const uint32_t r = enclosing_block(d, li); if (r != 0 && li == r + 1) return MYEA_E_UNSUPPORTED; }
+        /* inside a residual block too (Assign__Post__Residual_Layer, NN/Neural_Network__Compile.cpp:352-376, computes a member's
+         * width by the same formulas) */
         const double in = (double)number_outputs(d, previous_layer(d, li));
         const double kernel = l->pooling_values[0], stride = l->pooling_values[1], padding = l->pooling_values[2], dilation = l->pooling_values[3];
         const double span = l->type_layer == MYEA_LAYER_AVERAGE_POOLING ? in + 2.0 * padding - kernel : in + 2.0 * padding - dilation * (kernel - 1.0) - 1.0;
@@ -158,7 +157,7 @@ int myea_net_desc_layout(myea_net_desc *d)
         if (l->type_layer != MYEA_LAYER_RESIDUAL) continue;
         if (l->block_depth == 0 || (uint64_t)li + l->block_depth + 1 >= d->n_layers) return MYEA_E_INVALID;
         for (uint32_t k = 1; k <= l->block_depth; ++k)
-            if ((d->layers[li + k].type_layer != MYEA_LAYER_FULLY_CONNECTED && !(k > 1 && is_pooling(&d->layers[li + k]))) || d->layers[li + k].k_sparsity != 0) return MYEA_E_UNSUPPORTED;
+            if ((d->layers[li + k].type_layer != MYEA_LAYER_FULLY_CONNECTED && !is_pooling(&d->layers[li + k])) || d->layers[li + k].k_sparsity != 0) return MYEA_E_UNSUPPORTED;
         li += l->block_depth;
     }
 

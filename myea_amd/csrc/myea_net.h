@@ -140,6 +140,7 @@ struct Net {
                    const float *sums = nullptr, size_t sum_blocks = 0);
     int bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx, const float *sums = nullptr, size_t sum_blocks = 0);
     int backward_into_layer(size_t li, size_t B);
+    int pool_backward_with_shortcut(size_t gi, size_t rows, size_t roff, const DevLayer *shortcut, long crop, float *dst);
     int forward_residual_block(size_t ri, size_t B);
     int backward_residual_block(size_t ri, size_t B);
 

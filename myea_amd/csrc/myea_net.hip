@@ -167,13 +167,13 @@ static int check_desc(const myea_net_desc &d)
             // Assign__Post__Layer computes (NN/Neural_Network__Compile.cpp:250-271) - the kernels index with it
             any_pool = true;
             if (li == 0 || li + 1 >= d.n_layers) { set_last_error("layer %u: a pooling layer sits between the input and the output layer", li); return MYEA_E_UNSUPPORTED; }
-            if (block_end != 0 && d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) { set_last_error("layer %u: a pooling layer may be any member of a residual block but the first", li); return MYEA_E_UNSUPPORTED; }
             const myea_layer_desc &pl = d.layers[li - 1], &nl = d.layers[li + 1];
-            if ((pl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(pl)) || (nl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(nl))) {
+            const bool first_member = pl.type_layer == MYEA_LAYER_RESIDUAL && block_end != 0;   // then the layer in front of the block feeds it
+            if ((pl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(pl) && !first_member) || (nl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(nl))) {
                 set_last_error("layer %u: pooling layers connect to fully-connected or pooling layers on this path", li);
                 return MYEA_E_UNSUPPORTED;
             }
-            const double in = (double)myea_net_desc_number_outputs(&d, li - 1), k = l.pooling_values[0], st = l.pooling_values[1], pad = l.pooling_values[2], dil = l.pooling_values[3];
+            const double in = (double)myea_net_desc_number_outputs(&d, myea_net_desc_previous_layer(&d, li)), k = l.pooling_values[0], st = l.pooling_values[1], pad = l.pooling_values[2], dil = l.pooling_values[3];
             if (k < 1 || st < 1) { set_last_error("layer %u: pooling kernel and stride must be >= 1", li); return MYEA_E_INVALID; }
             const double span = l.type_layer == MYEA_LAYER_AVERAGE_POOLING ? in + 2 * pad - k : in + 2 * pad - dil * (k - 1) - 1;
             const double out = span < 0 ? 0 : (l.pooling_values[4] == 0 ? std::floor(span / st + 1.0) : std::ceil(span / st + 1.0));
@@ -278,7 +278,7 @@ int Net::create(const myea_net_desc &desc)
         if (li > 1 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) {
             if (d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) o.group = 1;
             else if (L[li - 1].group != 0 && o.prev == li - 1) o.group = 2;  // the first layer after a block connects to the residual layer
-        } else if (li > 1 && layer_is_pooling(l) && L[li - 1].group != 0 && o.prev == li - 1) {
+        } else if (li > 1 && layer_is_pooling(l) && (d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL || (L[li - 1].group != 0 && o.prev == li - 1))) {
             o.group = 3;   // a pooling member of a block: basic units as wide as the layer, no activation or normalised units
         }
         if (l.type_layer == MYEA_LAYER_RESIDUAL) {
@@ -808,6 +808,18 @@ int Net::gather_examples(float *dst, const float *src, size_t examples, size_t r
 }
 
 // ---- backward ---------------------------------------------------------------------------------------------------
+// What pooling layer gi hands down to its producer's `rows` rows at row offset roff, into dst; when gi is the first member of
+// a residual block, plus the shortcut's share (the residual layer's errors, cropped at the padding offset).
+int Net::pool_backward_with_shortcut(size_t gi, size_t rows, size_t roff, const DevLayer *shortcut, long crop, float *dst)
+{
+    DevLayer &on = L[gi];
+    const size_t In = on.In;
+    float *through = shortcut ? tmp2 + roff * In : dst;
+    MYEA_TRY(launch_pool_backward(stream, pool_params(gi, rows), on.neuron_errors + roff * on.H, on.pool_index ? on.pool_index + roff * on.H : nullptr, through));
+    if (shortcut) MYEA_TRY(launch_padded_add(stream, rows, In, shortcut->neuron_errors + roff * shortcut->H, shortcut->H, crop, through, In, 0, dst));
+    return MYEA_OK;
+}
+
 // FF__Backward_Pass_Batch (NN/Neural_Network__Backward_Pass__OpenMP.cpp:24-155): for every layer below the
 // output layer, dX = delta_next * W_next (Backward_Pass__FC, :1044-1082) and then
 // Backward_Pass__Gradient__FC (:544-709): [BN after] -> act' -> [BN before].  The act' multiply is fused
@@ -872,7 +884,7 @@ int Net::backward_into_layer(size_t li, size_t B)
         if (!is_fc) {  // an LSTM layer receives the plain delta of its cell outputs (BPTT follows), a residual layer that of its units
             g.C = o.neuron_errors + roff * H;
             g.epilogue = EPI_NONE;
-            if (pool_consumer) { MYEA_TRY(launch_pool_backward(stream, pool_params(gi, rows), on.neuron_errors + roff * on.H, on.pool_index ? on.pool_index + roff * on.H : nullptr, g.C)); continue; }
+            if (pool_consumer) { MYEA_TRY(pool_backward_with_shortcut(gi, rows, roff, shortcut, crop, g.C)); continue; }
             if (!have_gemm) { MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors + roff * shortcut->H, shortcut->H, crop, identity + roff * H, H, 0, g.C)); continue; }
             prof_begin(1);
             MYEA_TRY(launch_gemm(stream, g));
@@ -921,7 +933,7 @@ int Net::backward_into_layer(size_t li, size_t B)
                 prof_end(2.0 * (double)rows * (double)H * (double)Out);
             }
         } else if (pool_consumer) {
-            MYEA_TRY(launch_pool_backward(stream, pool_params(gi, rows), on.neuron_errors + roff * on.H, on.pool_index ? on.pool_index + roff * on.H : nullptr, g.C));
+            MYEA_TRY(pool_backward_with_shortcut(gi, rows, roff, shortcut, crop, g.C));
         } else {
             MYEA_TRY(launch_padded_add(stream, rows, H, shortcut->neuron_errors + roff * shortcut->H, shortcut->H, crop, identity + roff * H, H, 0, g.C));
         }
@@ -995,6 +1007,7 @@ int Net::backward_residual_block(size_t ri, size_t B)
             if (o.group == 1 && !norm) break;
             const size_t In = o.In, H = o.H;
             if (layer_is_pooling(l)) {   // hands its delta down through its windows (Backward_Pass__Gradient__Residual__Layer, :753-772), nothing else
+                if (m == ri + 1) break;   // the first member: the layer in front of the block pulls it, together with the shortcut's share
                 MYEA_TRY(launch_pool_backward(stream, pool_params(m, B), o.neuron_errors + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr,
                                               L[m - 1].neuron_errors + roff * In));
                 continue;

@@ -318,7 +318,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
     for (size_t li = 0; li < desc->n_layers; ++li) {
         const myea_layer_desc *l = &desc->layers[li];
         olayer *o = &n->L[li];
-        if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED && !(o->group == 2 && is_pooling(l))) { free(n); return MYEA_E_UNSUPPORTED; }
+        if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED && !is_pooling(l)) { free(n); return MYEA_E_UNSUPPORTED; }
         if (l->type_layer == MYEA_LAYER_LSTM && l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_ZONEOUT) { free(n); return MYEA_E_UNSUPPORTED; }
         /* with more cells per block the reference's indices [3] .. [8] into the layer's normalised units (NN/Neural_Network.cpp:4498-4613)
          * land on the second cell's units instead of the block's (the units are laid out per block: 3 per cell, then 6,

@@ -97,6 +97,3 @@ def test_pooling_layers_are_refused_where_this_path_has_none():
         oracle_desc([dict(units=6), dict(units=8, activation="TANH"), dict(type="max_pooling", kernel=2, stride=2)], 2)
     with pytest.raises(ValueError):    # window larger than the padded input
         oracle_desc([dict(units=6), dict(units=3, activation="TANH"), dict(type="average_pooling", kernel=9, stride=1), dict(units=2, activation="LINEAR")], 2)
-    with pytest.raises(ValueError):    # as the first member of a residual block (any other member may be a pooling layer)
-        oracle_desc([dict(units=6), dict(type="residual", block_depth=2), dict(type="max_pooling", kernel=2, stride=1, padding=1), dict(units=6, activation="RELU"),
-                     dict(units=3, activation="LINEAR")], 2)

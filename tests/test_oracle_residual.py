@@ -168,8 +168,9 @@ class TorchResidualNet:
                     m = li + k
                     if specs[m].get("type", "").endswith("pooling"):   # a pooling member: windows over the member before it
                         u, _ = _torch_pool(specs[m], u)
-                        u.retain_grad()
-                        self.taps[m] = u
+                        if u.requires_grad:   # not when the block hangs on the input layer and this is its first member
+                            u.retain_grad()
+                            self.taps[m] = u
                         continue
                     if specs[m].get("normalization", "NONE") != "NONE":
                         u = self._bn(m, u)
@@ -236,6 +237,10 @@ CASES = {
     # normalisation, and two pooling members in a row
     "max_pooling_last_member": ([fc(5), fc(9, "TANH"), res(2, normalization="BATCH_NORMALIZATION"), fc(11, "TANH"),
                                  dict(type="max_pooling", kernel=3, stride=2, padding=1), fc(3, "LINEAR")], 6),
+    # a pooling layer as the block's FIRST member: the layer in front of the block receives its share and the shortcut's
+    "pooling_first_member": ([fc(6), fc(12, "TANH"), res(2), dict(type="average_pooling", kernel=2, stride=2), fc(9, "TANH"), fc(3, "LINEAR")], 6),
+    "max_pooling_first_member_on_the_input": ([fc(10), res(3), dict(type="max_pooling", kernel=3, stride=1, padding=1),
+                                               fc(7, "SIGMOID"), fc(12, "TANH"), fc(4, "SOFTMAX")], 7),
     "two_pooling_members": ([fc(5), fc(7, "SIGMOID"), res(4), fc(16, "TANH"), dict(type="max_pooling", kernel=2, stride=2),
                              dict(type="average_pooling", kernel=3, stride=1, padding=1), fc(7, "TANH"), fc(2, "LINEAR")], 6),
 }
