@@ -72,7 +72,7 @@ constexpr int kLocalAux = 16;      // cache policy of the LOCAL protocol's tile 
 
 // LDS of a workgroup: every wavefront's tiles of one unit, and the partial tiles of the two chains
 constexpr size_t forward_lds(int kw, int cells, int rs) { return ((size_t)4 * (kw / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * (4 * cells + 8)) * sizeof(float); }
-constexpr size_t backward_lds(int c, int rs) { return ((size_t)4 * (c / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * 17) * sizeof(float); }
+constexpr size_t backward_lds(int c, int rs) { return ((size_t)4 * (c > 512 ? 16 : c / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * 17) * sizeof(float); }
 
 template <int N>
 __device__ __forceinline__ void wait_vm() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }   // vmcnt(N)
@@ -535,22 +535,29 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
     constexpr int NSTORE = 6 * PAIRS;
     constexpr int A1 = NT / 4, P1 = (3 * NT) / 4;
     constexpr int kStride = 17;
-    constexpr int kStage = NT * ROWS * 32, kPart = 4 * ROWS * kStride;
-    constexpr int kAux = kLocalAux;
-    static_assert(NT >= 4 && NT * LPT + NSTORE < 64, "vmcnt has 6 bits");
+    // WIDE (C = 1024): a unit's gate deltas (16 examples x 4096 k = 256 KiB) do not fit LDS at once.  They pass through two
+    // half buffers of NT / 4 tiles per wavefront in four groups: while group g is contracted, group g + 2 lands in the half
+    // that group g has just left.  Its 64 members span two XCDs: device-scope stores of the gate deltas, device-scope
+    // counter, tile loads served beyond the XCD's L2 (as in the forward loop of this width).
+    constexpr bool WIDE = C > 512, AGENT = WIDE;
+    constexpr int SLOTS = WIDE ? NT / 2 : NT, NG = NT / 4;   // tiles of LDS per wavefront; tiles per group
+    constexpr int kStage = SLOTS * ROWS * 32, kPart = 4 * ROWS * kStride;
+    constexpr int kAux = AGENT ? 16 : kLocalAux;
+    static_assert(!WIDE || RS == 1, "the wide form has one set of rows per chain");
+    static_assert(NT >= 4 && (WIDE ? 3 * NG * LPT + 9 : NT * LPT) + NSTORE < 64, "vmcnt has 6 bits");
     extern __shared__ __attribute__((aligned(16))) float smem[];
     __shared__ unsigned s_arrive[2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col16 = lane & 15, quad = lane >> 4;
 
     int group, member;
-    if (!place<false>(blockIdx.x, g.members, g.dirs * g.row_groups, group, member)) return;
+    if (!place<AGENT>(blockIdx.x, g.members, g.dirs * g.row_groups, group, member)) return;
     const int dir = group % g.dirs, rg = group / g.dirs;
     const LstmResidentDir &d = dir ? d1 : d0;
     const int c0 = member * CELLS, B = g.B, T = g.T;
     const size_t Bmax = (size_t)g.Bmax;
     unsigned *const counters = w.counters + (size_t)group * 2 * kSyncStride;
     const unsigned members = (unsigned)g.arrivals;
-    check_same_xcd(w, group);
+    if (!AGENT) check_same_xcd(w, group);
     if (threadIdx.x < 2) s_arrive[threadIdx.x] = 0u;
     __syncthreads();
 
@@ -625,21 +632,28 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
             e_cs[q] = p_cp[c][q][-step_c];
         }
     };
-    auto load_tiles = [&](auto ch) {   // dG of the chain's step processed before the one its pointers are at
+    // tiles [first, last) of the chain's step into their LDS slots (tile i lives in slot i mod SLOTS); `advance`: these were
+    // the step's last tiles, the pointers move on to the next step
+    auto load_tile_range = [&](auto ch, auto first, auto last, auto advance) {
         constexpr int c = decltype(ch)::value;
 #pragma unroll
-        for (int i = 0; i < NT; ++i)
+        for (int i = decltype(first)::value; i < decltype(last)::value; ++i)
 #pragma unroll
             for (int q = 0; q < LPT; ++q)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p_tile[c][q] + i * 32),
-                                                 (__attribute__((address_space(3))) void *)(stage + i * ROWS * 32 + q * 256), 16, 0, kAux);
+                                                 (__attribute__((address_space(3))) void *)(stage + (i % SLOTS) * ROWS * 32 + q * 256), 16, 0, kAux);
+        if (decltype(advance)::value) {
 #pragma unroll
-        for (int q = 0; q < LPT; ++q) p_tile[c][q] += step_g;
+            for (int q = 0; q < LPT; ++q) p_tile[c][q] += step_g;
+        }
+    };
+    auto load_tiles = [&](auto ch) {   // dG of the chain's step processed before the one its pointers are at: all of it, or (WIDE) its first two groups
+        load_tile_range(ch, std::integral_constant<int, 0>{}, std::integral_constant<int, SLOTS>{}, std::integral_constant<bool, !WIDE>{});
     };
     auto mfma_tiles = [&](auto first, auto last) {
 #pragma unroll
         for (int i = decltype(first)::value; i < decltype(last)::value; ++i) {
-            const float *tile = stage + i * ROWS * 32;
+            const float *tile = stage + (i % SLOTS) * ROWS * 32;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 f32x4 fa[RS];
@@ -666,14 +680,34 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
         mfma_tiles(I0{}, IA{});
         __builtin_amdgcn_sched_barrier(0);   // keeps the MFMAs above in front of the wait
         wait_vm<0>();
-        wave_arrive<false>(counters + (1 - c) * kSyncStride, &s_arrive[1 - c]);
+        wave_arrive<AGENT>(counters + (1 - c) * kSyncStride, &s_arrive[1 - c]);
+        if (WIDE) {   // the third group into the half the first one has left - here, not wherever the scheduler would sink it
+            __builtin_amdgcn_sched_barrier(0);
+            load_tile_range(ch, std::integral_constant<int, 2 * NG>{}, std::integral_constant<int, 3 * NG>{}, std::false_type{});
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
     // FIRST: the pass's first step of the chain (no recurrent term, nothing from a later step); s: the direction's step
     auto tail = [&](auto ch, auto first_tag, int s, unsigned wait_for) -> bool {
         constexpr int c = decltype(ch)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
         load_operands(ch, s > 0);
-        if (!FIRST) {
+        if (!FIRST && WIDE) {
+            using I2 = std::integral_constant<int, 2 * NG>;
+            __builtin_amdgcn_sched_barrier(0);                                         // the operands' loads stay in front of the MFMAs
+            mfma_tiles(IA{}, I2{});                                                    // group 1, from the second half
+            __builtin_amdgcn_sched_barrier(0);
+            load_tile_range(ch, IP{}, IN{}, std::true_type{});                         // group 3 into that half
+            // all but group 3's loads have landed: group 2 and the operands (how many loads those are depends on the unit's kind,
+            // so they cannot be left out of the count)
+            wait_vm<NG * LPT>();
+            mfma_tiles(I2{}, IP{});
+            __builtin_amdgcn_sched_barrier(0);
+            if (wait_for) { seen = __hip_atomic_load(counters + (1 - c) * kSyncStride, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT); wait_vm<1>(); }
+            else wait_vm<0>();                                                         // group 3 is here
+            mfma_tiles(IP{}, IN{});
+            __builtin_amdgcn_sched_barrier(0);
+        } else if (!FIRST) {
             mfma_tiles(IA{}, IP{});
             if (wait_for) seen = __hip_atomic_load(counters + (1 - c) * kSyncStride, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
             mfma_tiles(IP{}, IN{});
@@ -722,7 +756,12 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
                 sums[4] += di * e_cp[q]; sums[5] += df * e_cp[q]; sums[6] += ddo * e_cs[q];
             }
             float *drow = p_dG[c][q];
-            drow[0] = dz; drow[C] = di; drow[2 * C] = df; drow[3 * C] = ddo;
+            if (AGENT) {   // read by members on another XCD
+                __hip_atomic_store(drow, dz, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT); __hip_atomic_store(drow + C, di, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+                __hip_atomic_store(drow + 2 * C, df, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT); __hip_atomic_store(drow + 3 * C, ddo, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+            } else {
+                drow[0] = dz; drow[C] = di; drow[2 * C] = df; drow[3 * C] = ddo;
+            }
             *p_dh[c][q] = dh; *p_dc[c][q] = e;
             p_acts[c][q] += step_g; p_ca[c][q] += step_c; p_cp[c][q] += step_c; p_dh_in[c][q] += step_c;
             p_dG[c][q] += lane_step_g[c][q]; p_dh[c][q] += lane_step_c[c][q]; p_dc[c][q] += lane_step_c[c][q];
@@ -735,7 +774,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
     // units in program order: (0,0) (1,0) (0,1) (1,1) ... (chain, step j of this pass); the direction's step is T - 1 - j
     if (!tail(Chain0{}, First{}, T - 1, 0u)) return;
     wait_vm<0>();
-    wave_arrive<false>(counters, &s_arrive[0]);
+    wave_arrive<AGENT>(counters, &s_arrive[0]);
     if (!tail(Chain1{}, First{}, T - 1, 1u)) return;
     head(Chain0{}, std::true_type{});
     for (int j = 1; j + 1 < T; ++j) {
@@ -1132,7 +1171,7 @@ KernelInfo g_kernels[2][4][2] = {
     {{backward_info<128, 1>(), backward_info<128, 2>()},
      {backward_info<256, 1>(), backward_info<256, 2>()},
      {backward_info<512, 1>(), KernelInfo{}},
-     {KernelInfo{}, KernelInfo{}}},
+     {backward_info<1024, 1>(), KernelInfo{}}},
 };
 
 // the backward loop split along k, [C: 128, 256, 512, 1024]: two chains of 16 examples only, groups within one XCD
@@ -1266,7 +1305,8 @@ int lstm_resident_plan(size_t C, size_t cells_per_block, size_t B, int dirs, Lst
         const int rows = 2 * 16 * rs, row_groups = (int)((B + rows - 1) / rows), groups = row_groups * dirs;
         int grid = 0, grid_b = 0;
         if (!place_groups(*dev, *fwd, members, agent, groups, &grid)) continue;
-        bool backward = bwd && !agent && place_groups(*dev, *bwd, members, false, groups, &grid_b) && grid_b == grid;
+        // the backward kernel of 1024 cells is the device-scope one, the narrower ones keep a group on one XCD
+        bool backward = bwd && agent == (C > 512) && place_groups(*dev, *bwd, members, agent, groups, &grid_b) && grid_b == grid;
         const int choice = ksplit_choice();
         KernelInfo *split = choice == 0 ? nullptr : kernel_for(C, rs, true, true);
         bool ksplit = split && !agent && fwd->cells == 16 && place_groups(*dev, *split, members, agent, groups, &grid_b) && grid_b == grid;

@@ -42,7 +42,8 @@ CASES = [
     ("128-cells-second-chain-empty", [dict(units=8), lstm(128), dict(units=128, activation="LINEAR")], 5, 13, 16, True),
     ("256-cells-two-directions", [dict(units=12), lstm(256, bidirectional=True), dict(units=256, activation="TANH")], 5, 33, 40, True),
     ("512-cells-zoneout-stacked", [dict(units=16), zone(512), lstm(128), dict(units=128, activation="LINEAR")], 4, 48, 48, True),
-    ("1024-cells-forward-only-two-directions", [dict(units=10), lstm(1024, bidirectional=True), dict(units=1024, activation="LINEAR")], 3, 40, 40, False),
+    ("1024-cells-two-directions", [dict(units=10), lstm(1024, bidirectional=True), dict(units=1024, activation="LINEAR")], 3, 40, 40, True),
+    ("1024-cells-ragged-seven-steps", [dict(units=6), lstm(1024), dict(units=1024, activation="LINEAR")], 7, 45, 48, True),
     ("two-steps", [dict(units=6), lstm(256), dict(units=256, activation="LINEAR")], 2, 32, 32, True),
 ]
 
