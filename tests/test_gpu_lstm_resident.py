@@ -209,11 +209,13 @@ def test_a_wait_that_gives_up_is_reported_once_and_the_network_carries_on_per_st
     _compare(desc, gpu, cpu, B, T, "after the give-up")
 
 
-@pytest.mark.parametrize("ksplit", ["1", "0"], ids=["backward-split-along-k", "backward-split-along-columns"])
-def test_a_backward_wait_that_gives_up_is_reported_too(ksplit):
-    """the same forced give-up in the backward loop, in either of its forms: the forward pass runs normally, the backward
-    loop's first wait between steps runs out of polls and every wavefront leaves"""
-    specs = [dict(units=8), lstm(128), dict(units=128, activation="LINEAR")]
+@pytest.mark.parametrize("cells,ksplit", [(128, "1"), (128, "0"), (1024, "0")],
+                         ids=["backward-split-along-k", "backward-split-along-columns", "1024-cells-across-two-xcds"])
+def test_a_backward_wait_that_gives_up_is_reported_too(cells, ksplit):
+    """the same forced give-up in the backward loop, in each of its forms (at 1024 cells with tile loads into LDS in flight
+    when the wait begins): the forward pass runs normally, the backward loop's first wait between steps runs out of polls and
+    every wavefront leaves"""
+    specs = [dict(units=8), lstm(cells), dict(units=cells, activation="LINEAR")]
     T, B = 5, 32
     desc, h, w, masks, X, Y = _setup(specs, T, B, B, seed=9)
     gpu = _net(desc, h, w, None)
