@@ -261,6 +261,7 @@ def config_of(r):
 
 
 SECONDARY = "lstm512x2_t64_b256_amsgrad"   # the metric's other half
+OTHERS = ("fc2048x8_bn_relu_dropout_b512_nesterov", "bilstm1024_t512_b64_adabound")
 
 
 def measured_ceilings():
@@ -284,7 +285,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="fc4096x4_b1024_adam", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-secondary", action="store_true", help="skip the LSTM-512 leg the default workload's line also carries")
+    ap.add_argument("--no-secondary", action="store_true", help="skip the LSTM-512 leg and the two short legs of the other configurations that the default workload's line also carries")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the measured MFMA / HBM ceilings")
     ap.add_argument("--separate-update", action="store_true", help="Update_Parameter as a call of its own behind the backward pass")
     ap.add_argument("--cpu-sample-rows", type=int, default=0, help="examples in the CPU sample (default: sized for ~20 s)")
@@ -336,11 +337,21 @@ def main():
     if has_loops:
         out["time_loops"] = dict(r["time_loops"], kernel="lstm_resident_forward_kernel / lstm_resident_backward_kernel (or one lstm_fused_* launch per step)")
     if args.workload != SECONDARY and args.workload == "fc4096x4_b1024_adam" and not args.no_secondary:
-        s = run_workload(SECONDARY, max(5, args.steps // 3), max(2, args.warmup // 2), args.separate_update)
+        sec_steps = max(5, 2 * args.steps // 3)
+        s = run_workload(SECONDARY, sec_steps, max(2, args.warmup), args.separate_update)
         loops = dict(s["time_loops"], kernel="lstm_resident_forward_kernel + lstm_resident_backward_kernel: the recurrent contractions and gate math of steps 1 .. T-1, one launch per layer and pass")
         out["secondary"] = {"workload": SECONDARY, "value": s["value"], "unit": "samples/s", "ms_per_step": s["ms_per_step"],
-                            "steps": max(5, args.steps // 3), "events_pass": {"steps": max(5, args.steps // 3), "ms_per_step": s["ms_per_step_events"]}, "config": config_of(s), "roofline": loops,
+                            "steps": sec_steps, "events_pass": {"steps": sec_steps, "ms_per_step": s["ms_per_step_events"]}, "config": config_of(s), "roofline": loops,
                             "contractions": s["contractions"], "kernels": s["kernels"], "loss_per_output": s["loss_per_output"]}
+        # the other two configurations of the baseline that are timed on the GPU, a few steps each, so that one run records all four
+        out["other_configurations"] = []
+        for name in OTHERS:
+            o = run_workload(name, max(5, args.steps // 3), max(2, args.warmup // 2), args.separate_update)
+            leg = {"workload": name, "value": o["value"], "unit": "samples/s", "ms_per_step": o["ms_per_step"], "steps": max(5, args.steps // 3),
+                   "config": config_of(o), "contractions": o["contractions_alone"] or o["contractions"], "loss_per_output": o["loss_per_output"]}
+            if o["time_loops"]["launches"] > 0:
+                leg["time_loops"] = o["time_loops"]
+            out["other_configurations"].append(leg)
     if not args.no_ceilings:
         out["ceilings"] = measured_ceilings()
     if not args.no_cpu_baseline:
