@@ -648,6 +648,12 @@ int gemm_split_k(int M, int N, int K)
     return (K + chunk - 1) / chunk;
 }
 
+bool gemm_pair_k_128(int M, int N, int K)
+{
+    const long tiles_128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    return tiles_128 <= kGemmPairTiles && tiles_128 % 8 == 0 && tiles_128 >= 128 && K >= 2048;
+}
+
 bool gemm_can_fuse_activation(int act)
 {
     return act == MYEA_AF_LINEAR || act == MYEA_AF_RELU || act == MYEA_AF_LEAKY_RELU || act == MYEA_AF_PARAMETRIC_RELU ||
@@ -720,7 +726,7 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     // The same one size up: at most one 128 x 128 tile per compute unit (a batch of 1024 in front of 4096 units) would run as 64 x
     // 128 tiles to put two workgroups on every compute unit; two workgroups sharing a 128 x 128 tile's k do that with the larger
     // tile's operand reuse.
-    if ((pair_k & 2) && p.pair_partials && p.pair_tickets && d.ksplit == 1 && tiles_128 <= kGemmPairTiles && tiles_128 % 8 == 0 && tiles_128 >= 128 && p.K >= 2048) {
+    if ((pair_k & 2) && p.pair_partials && p.pair_tickets && d.ksplit == 1 && gemm_pair_k_128(p.M, p.N, p.K)) {
         d.ksplit = 2;
         d.kchunk = ((p.K + 1) / 2 + kBK - 1) / kBK * kBK;
         d.pair_partials = p.pair_partials; d.pair_tickets = p.pair_tickets;

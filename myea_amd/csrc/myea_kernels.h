@@ -69,6 +69,9 @@ struct GemmParams {
 constexpr int kGemmPairTiles = 256;   // tiles the two buffers above serve
 
 int gemm_split_k(int M, int N, int K);
+// true when launch_gemm, handed pair_partials / pair_tickets, would share every 128 x 128 tile's k between two workgroups
+// (at most one such tile per compute unit, a k worth halving): callers size their pair buffers by it
+bool gemm_pair_k_128(int M, int N, int K);
 int launch_gemm(hipStream_t stream, const GemmParams &p);
 // dX = delta W (`a`) and dW += delta^T X (`b`) in one launch when their shapes suit it; MYEA_OK = launched, 1 = does not
 // apply (launch them one after the other), negative = error

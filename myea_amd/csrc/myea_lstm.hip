@@ -38,6 +38,10 @@ struct LstmLayer {
     bool fused = false;     // one launch per time step (myea_lstm_fused.hip) instead of contraction + gate kernel
     float *gWin = nullptr, *gWrec = nullptr;                     // packed gradient scratch
     float *gWin_own = nullptr, *gWrec_own = nullptr;             // the layer's own allocations behind the two pointers above
+    // the recurrent weights' contraction over all time steps, when it is one 128 x 128 tile per compute unit (1024 cells): two
+    // workgroups share a tile's k and meet here (the layer's own buffers: the contractions of two layers may run beside each
+    // other on two streams); pair_tickets: 2 x 256 words, zero between launches
+    float *pair_partials = nullptr, *pair_tickets = nullptr;
     float *acts = nullptr;  // [T][Bmax][G]: pre-activation sums, overwritten in place by z | i | f | o
     float *c = nullptr, *ca = nullptr;                           // [T][Bmax][C] cell state and tanh(cell state)
     float *dG = nullptr;    // [T][Bmax][G] deltas dz | di | df | do
@@ -675,6 +679,10 @@ int Net::lstm_create_layer(size_t li)
         MYEA_TRY(dev_alloc_zero(&q->gWin, kMaxSlabs * q->G * q->In));   // split-K slabs of the weight-gradient contractions
         MYEA_TRY(dev_alloc_zero(&q->gWrec, kMaxSlabs * q->G * q->C));
         q->gWin_own = q->gWin; q->gWrec_own = q->gWrec;
+        if (T > 1 && gemm_pair_k_128((int)q->G, (int)q->C, (int)((T - 1) * B))) {
+            MYEA_TRY(dev_alloc_zero(&q->pair_partials, (size_t)kGemmPairTiles * 128 * 128));
+            MYEA_TRY(dev_alloc_zero(&q->pair_tickets, 2 * kGemmPairTiles));
+        }
         MYEA_TRY(dev_alloc_zero(&q->acts, T * B * q->G));
         MYEA_TRY(dev_alloc_zero(&q->c, T * B * q->C));
         MYEA_TRY(dev_alloc_zero(&q->ca, T * B * q->C));
@@ -708,7 +716,7 @@ void Net::lstm_destroy_layer(DevLayer &o)
     for (LstmLayer **slot : {&o.lstm, &o.lstm2}) {
         LstmLayer *q = *slot;
         if (!q) continue;
-        float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin_own, q->gWrec_own, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->sums, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr,
+        float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin_own, q->gWrec_own, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->sums, q->pair_partials, q->pair_tickets, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr,
                         q->sin, q->srec, q->nin, q->nrec, q->hin, q->hrec, q->din, q->drec, q->nc, q->hc};
         for (float *p : all) if (p) (void)hipFree(p);
         for (float *p : q->stats) if (p) (void)hipFree(p);
@@ -1214,6 +1222,7 @@ int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t
         g.M = (int)q.G; g.N = (int)q.C; g.K = (int)rows;
         s_rec = gemm_split_k(g.M, g.N, g.K);
         g.split_k = s_rec; g.split_k_slab = (long)(q.G * q.C);
+        if (q.pair_partials && s_rec == 1) { g.pair_partials = q.pair_partials; g.pair_tickets = reinterpret_cast<unsigned *>(q.pair_tickets); }
         prof_begin(2);
         MYEA_TRY(launch_gemm(stream, g));
         prof_end(2.0 * (double)rows * (double)q.G * (double)q.C);
