@@ -135,7 +135,11 @@ template <bool AGENT>
 __device__ __forceinline__ void wave_arrive(unsigned *counter, unsigned *lds_count)
 {
     if ((threadIdx.x & 63) == 0) {
-        const unsigned before = __hip_atomic_fetch_add(lds_count, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_WORKGROUP);
+        // as assembly: in front of an LDS atomic the compiler drains every load still on its way into LDS (it cannot tell that
+        // they go elsewhere), which would stall a unit that has just requested its next tiles
+        unsigned before;
+        const unsigned at = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned *)lds_count, one = 1u;
+        asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=v"(before) : "v"(at), "v"(one) : "memory");
         if ((before & 3u) == 3u) {
             if (AGENT) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
             else __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_WORKGROUP);
@@ -189,6 +193,16 @@ __device__ __forceinline__ unsigned xcc_id() { return __builtin_amdgcn_s_getreg(
 
 // workgroup id -> (group, member).  LOCAL: the XCD of ids = x (mod 8) hosts the groups x, x + 8, ...; AGENT: members of a
 // group are spread over the XCDs.  Returns false for a workgroup without work.
+// f(integral_constant<int, I>{}) for I = FIRST .. LAST - 1, unrolled
+template <int FIRST, int LAST, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (FIRST < LAST) {
+        f(std::integral_constant<int, FIRST>{});
+        static_for<FIRST + 1, LAST>(f);
+    }
+}
+
 template <bool AGENT>
 __device__ __forceinline__ bool place(unsigned id, int members, int groups, int &group, int &member)
 {
@@ -628,7 +642,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
             for (int gate = 0; gate < 4; ++gate) e_act[q][gate] = p_acts[c][q][gate * C];
             e_ca[q] = *p_ca[c][q];
             e_dh[q] = *p_dh_in[c][q];
-            e_cp[q] = with_cp ? *p_cp[c][q] : 0.f;
+            e_cp[q] = p_cp[c][q][with_cp ? 0 : -step_c];   // without a step before: any valid address, the value is not used
             e_cs[q] = p_cp[c][q][-step_c];
         }
     };
@@ -647,8 +661,20 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
             for (int q = 0; q < LPT; ++q) p_tile[c][q] += step_g;
         }
     };
-    auto load_tiles = [&](auto ch) {   // dG of the chain's step processed before the one its pointers are at: all of it, or (WIDE) its first two groups
-        load_tile_range(ch, std::integral_constant<int, 0>{}, std::integral_constant<int, SLOTS>{}, std::integral_constant<bool, !WIDE>{});
+    auto load_tiles = [&](auto ch) {   // dG of the chain's step processed before the one its pointers are at: all of it, or (WIDE) its first group
+        load_tile_range(ch, std::integral_constant<int, 0>{}, std::integral_constant<int, WIDE ? NG : SLOTS>{}, std::integral_constant<bool, !WIDE>{});
+    };
+    // WIDE: one tile at a time, the next tile's operand read from LDS while this one's MFMAs run
+    auto read_tile = [&](auto i, f32x4 (&fa)[2]) {
+        const float *tile = stage + (decltype(i)::value % SLOTS) * ROWS * 32;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) fa[h] = ATile<ROWS, kAux>::chunk(tile, col16, h * 4 + quad);
+    };
+    auto mfma_tile = [&](auto i, const f32x4 (&fa)[2]) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[0][e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[h][e], breg[decltype(i)::value][h][e], acc[0][e & 1], 0, 0, 0);
     };
     auto mfma_tiles = [&](auto first, auto last) {
 #pragma unroll
@@ -676,44 +702,87 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
         constexpr int c = decltype(ch)::value;
 #pragma unroll
         for (int rs = 0; rs < RS; ++rs) { acc[rs][0] = f32x4{0.f, 0.f, 0.f, 0.f}; acc[rs][1] = f32x4{0.f, 0.f, 0.f, 0.f}; }
-        if (decltype(all_landed)::value) wait_vm<0>(); else wait_vm<NSTORE>();
-        mfma_tiles(I0{}, IA{});
-        __builtin_amdgcn_sched_barrier(0);   // keeps the MFMAs above in front of the wait
-        wait_vm<0>();
-        wave_arrive<AGENT>(counters + (1 - c) * kSyncStride, &s_arrive[1 - c]);
-        if (WIDE) {   // the third group into the half the first one has left - here, not wherever the scheduler would sink it
+        if (decltype(all_landed)::value) wait_vm<0>(); else wait_vm<NSTORE>();   // the unit's first group has landed
+        if constexpr (WIDE) {
+            // The loads of a tile are issued one tile at a time between the MFMAs, never as a burst: a compute unit's address path
+            // takes 16 clocks per 1 KiB load instruction, and a wavefront that issues sixteen of them in a row stands still for
+            // as long as sixty-four MFMAs take.  Here: the second group into the second half, which the other chain has left.
+            f32x4 fa[2][2];
+            read_tile(I0{}, fa[0]);
+            static_for<0, NG>([&](auto i) {
+                constexpr int I = decltype(i)::value;
+                __builtin_amdgcn_sched_barrier(0);
+                if (I + 1 < NG) read_tile(std::integral_constant<int, I + 1>{}, fa[(I + 1) & 1]);
+                mfma_tile(i, fa[I & 1]);
+                load_tile_range(ch, std::integral_constant<int, I + NG>{}, std::integral_constant<int, I + NG + 1>{}, std::false_type{});
+            });
             __builtin_amdgcn_sched_barrier(0);
-            load_tile_range(ch, std::integral_constant<int, 2 * NG>{}, std::integral_constant<int, 3 * NG>{}, std::false_type{});
-            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<NG * LPT>();             // the stores of the unit before are older than the second group's loads
+        } else {
+            mfma_tiles(I0{}, IA{});
+            __builtin_amdgcn_sched_barrier(0);   // keeps the MFMAs above in front of the wait
+            wait_vm<0>();
         }
+        wave_arrive<AGENT>(counters + (1 - c) * kSyncStride, &s_arrive[1 - c]);
     };
     // FIRST: the pass's first step of the chain (no recurrent term, nothing from a later step); s: the direction's step
     auto tail = [&](auto ch, auto first_tag, int s, unsigned wait_for) -> bool {
         constexpr int c = decltype(ch)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
+        // WIDE: every unit must issue the same number of loads, the waits count them - where `s` is a literal zero the compiler
+        // would drop the load of the state before it
+        if (WIDE) asm volatile("" : "+s"(s));
         load_operands(ch, s > 0);
-        if (!FIRST && WIDE) {
-            using I2 = std::integral_constant<int, 2 * NG>;
-            __builtin_amdgcn_sched_barrier(0);                                         // the operands' loads stay in front of the MFMAs
-            mfma_tiles(IA{}, I2{});                                                    // group 1, from the second half
+        if constexpr (!FIRST && WIDE) {
+            // tile i's MFMAs, then the loads of the tile that takes a slot no longer read: i + 8 of this unit (two groups ahead
+            // of its use minus one), or - the last group - tile i - 24 of the other chain's next unit, if that chain's step is
+            // complete by then.  The waits count what was issued behind the tile they wait for (two loads per tile, the eight
+            // operands, the counter's value, in program order).
+            constexpr int kOps = 8 * PAIRS;
+            const unsigned target = wait_for * members;
+            f32x4 fa[2][2];
             __builtin_amdgcn_sched_barrier(0);
-            load_tile_range(ch, IP{}, IN{}, std::true_type{});                         // group 3 into that half
-            // all but group 3's loads have landed: group 2 and the operands (how many loads those are depends on the unit's kind,
-            // so they cannot be left out of the count)
-            wait_vm<NG * LPT>();
-            mfma_tiles(I2{}, IP{});
+            wait_vm<(NG - 1) * LPT + kOps>();
+            read_tile(IA{}, fa[NG & 1]);
+            static_for<NG, 3 * NG>([&](auto i) {
+                constexpr int I = decltype(i)::value;
+                __builtin_amdgcn_sched_barrier(0);
+                wait_vm<(I + 1 < 2 * NG ? (NG - 2) * LPT + kOps : (I <= 2 * NG + 1 ? (NG - 2) * LPT : (NG - 2) * LPT + 1))>();
+                read_tile(std::integral_constant<int, I + 1>{}, fa[(I + 1) & 1]);
+                mfma_tile(i, fa[I & 1]);
+                if (I == 2 * NG + 1)   // the other chain's counter, as assembly: the compiler would wait for ALL loads where the value is used
+                    asm volatile("global_load_dword %0, %1, off sc1" : "=v"(seen) : "v"(counters + (1 - c) * kSyncStride) : "memory");
+                load_tile_range(ch, std::integral_constant<int, I + NG>{}, std::integral_constant<int, I + NG + 1>{}, std::integral_constant<bool, I + 1 == 3 * NG>{});
+            });
             __builtin_amdgcn_sched_barrier(0);
-            if (wait_for) { seen = __hip_atomic_load(counters + (1 - c) * kSyncStride, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT); wait_vm<1>(); }
-            else wait_vm<0>();                                                         // group 3 is here
-            mfma_tiles(IP{}, IN{});
-            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<(NG - 2) * LPT>();       // tile 3 NG + 1 has landed, and the counter's value before it
+            asm volatile("" : "+v"(seen));      // the value is looked at behind the wait, not before
+            if (wait_for && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0) {
+                static_for<3 * NG, NT>([&](auto i) {
+                    constexpr int I = decltype(i)::value;
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (I > 3 * NG && I + 1 < NT) wait_vm<(NG - 2) * LPT>();
+                    if (I + 1 < NT) read_tile(std::integral_constant<int, I + 1>{}, fa[(I + 1) & 1]);
+                    mfma_tile(i, fa[I & 1]);
+                    load_tile_range(std::integral_constant<int, 1 - c>{}, std::integral_constant<int, I - 3 * NG>{}, std::integral_constant<int, I - 3 * NG + 1>{}, std::false_type{});
+                });
+                __builtin_amdgcn_sched_barrier(0);
+            } else {   // the other chain is late (or has no further unit): this unit's last group first, then the wait, then its tiles in a row
+                wait_vm<0>();
+                mfma_tiles(IP{}, IN{});
+                __builtin_amdgcn_sched_barrier(0);
+                if (wait_for) {
+                    if (!wave_wait(w, counters + (1 - c) * kSyncStride, target, g.spin_polls)) return false;
+                    load_tiles(std::integral_constant<int, 1 - c>{});
+                }
+            }
         } else if (!FIRST) {
             mfma_tiles(IA{}, IP{});
             if (wait_for) seen = __hip_atomic_load(counters + (1 - c) * kSyncStride, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
             mfma_tiles(IP{}, IN{});
             __builtin_amdgcn_sched_barrier(0);   // the counter's value is looked at after the MFMAs, not right behind its load
         }
-        if (wait_for) {
+        if (wait_for && (FIRST || !WIDE)) {
             const unsigned target = wait_for * members;
             const bool there = !FIRST && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0;
             if (!there && !wave_wait(w, counters + (1 - c) * kSyncStride, target, g.spin_polls)) return false;
@@ -753,7 +822,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
             n_di[c][q] = di; n_df[c][q] = df; n_f[c][q] = gf; n_dc[c][q] = e;
             if (lane_step_g[c][q] != 0) {   // the lane has an example in this chain
                 sums[0] += dz; sums[1] += di; sums[2] += df; sums[3] += ddo;
-                sums[4] += di * e_cp[q]; sums[5] += df * e_cp[q]; sums[6] += ddo * e_cs[q];
+                sums[4] += s > 0 ? di * e_cp[q] : 0.f; sums[5] += df * e_cp[q]; sums[6] += ddo * e_cs[q];
             }
             float *drow = p_dG[c][q];
             if (AGENT) {   // read by members on another XCD
