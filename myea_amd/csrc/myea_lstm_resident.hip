@@ -259,6 +259,9 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
     constexpr int kStride = NB + 8;               // floats per row of a wavefront's partial tile
     constexpr int kStage = NT * ROWS * 32, kPart = 4 * ROWS * kStride;
     constexpr int kAux = AGENT ? 16 : kLocalAux;
+    constexpr bool DB = AGENT;                    // the other chain's tiles are requested during this chain's last MFMAs, into the slots those have left
+    constexpr int S1 = (5 * NT) / 8, X1 = (3 * NT) / 4;   // DB: tile behind which the other chain's counter is read / behind which its value is looked at
+    static_assert(!DB || (NT >= 8 && X1 > S1 && X1 < NT && X1 % (NT - X1) == 0), "tiles left to spread the requests over");
     static_assert(PAIRS >= 1 && ROWS * CELLS % kThreads == 0, "every lane has the same number of pairs");
     static_assert(NT * LPT + NSTORE < 64, "vmcnt has 6 bits");
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -366,18 +369,23 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
             for (int q = 0; q < PAIRS; ++q) keep_h[q] = p_zone_h[q][0];
         }
     };
-    auto load_tiles = [&](auto ch) {   // h of the step before the one the chain's pointers are at: p_tile is one step behind
+    // tiles [first, last) of h of the step before the one the chain's pointers are at (p_tile is one step behind);
+    // `advance`: these were the step's last tiles
+    auto load_tile_range = [&](auto ch, auto first, auto last, auto advance) {
         constexpr int c = decltype(ch)::value;
 #pragma unroll
-        for (int i = 0; i < NT; ++i)
+        for (int i = decltype(first)::value; i < decltype(last)::value; ++i)
 #pragma unroll
             for (int q = 0; q < LPT; ++q)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p_tile[c][q] + i * 32),
                                                  (__attribute__((address_space(3))) void *)(stage + i * ROWS * 32 + q * 256), 16, 0, kAux);
+        if (decltype(advance)::value) {
 #pragma unroll
-        for (int q = 0; q < LPT; ++q) p_tile[c][q] += step_c;
+            for (int q = 0; q < LPT; ++q) p_tile[c][q] += step_c;
+        }
     };
-    auto mfma_tiles = [&](auto first, auto last) {
+    auto load_tiles = [&](auto ch) { load_tile_range(ch, std::integral_constant<int, 0>{}, std::integral_constant<int, NT>{}, std::true_type{}); };
+    auto mfma_tiles = [&](auto ch, auto first, auto last) {
 #pragma unroll
         for (int i = decltype(first)::value; i < decltype(last)::value; ++i) {
             const float *tile = stage + i * ROWS * 32;
@@ -411,7 +419,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
 #pragma unroll
             for (int ct = 0; ct < NCT; ++ct) acc[rs][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (decltype(all_landed)::value) wait_vm<0>(); else wait_vm<NSTORE>();
-        mfma_tiles(I0{}, IA{});
+        mfma_tiles(ch, I0{}, IA{});
         __builtin_amdgcn_sched_barrier(0);   // keeps the MFMAs above in front of the wait
         wait_vm<0>();
         wave_arrive<AGENT>(counters + (1 - c) * kSyncStride, &s_arrive[1 - c]);
@@ -423,15 +431,48 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
         constexpr int c = decltype(ch)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
         load_inputs(ch);
-        if (!FIRST) {
-            mfma_tiles(IA{}, IP{});
+        bool requested = false;   // DB: the other chain's tiles are on their way already
+        if constexpr (!FIRST && DB) {
+            // The other chain's counter is read five eighths into the MFMAs, when its step is normally complete, and looked at an
+            // eighth later; its tiles are then requested between the last quarter's MFMAs, into the slots whose tiles those
+            // MFMAs no longer need (a tile's own slot right behind its MFMAs) - they have those MFMAs and the gate math to
+            // arrive, and the requests do not come as one burst (a compute unit's address path takes 16 clocks per 1 KiB load
+            // instruction; a wavefront that issues sixteen in a row stands still meanwhile).
+            using IS = std::integral_constant<int, S1>;
+            using IX = std::integral_constant<int, X1>;
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_tiles(ch, IA{}, IS{});
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("global_load_dword %0, %1, off sc1" : "=v"(seen) : "v"(counters + (1 - c) * kSyncStride) : "memory");
+            mfma_tiles(ch, IS{}, IX{});
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<0>();                          // the unit's inputs (requested long ago) and the counter's value
+            asm volatile("" : "+v"(seen));         // looked at behind the wait, not before
+            if (wait_for && (int)(__builtin_amdgcn_readfirstlane(seen) - wait_for * members) >= 0) {
+                constexpr int kEach = X1 / (NT - X1);   // free slots filled per tile of MFMAs
+                static_for<X1, NT>([&](auto i) {
+                    constexpr int I = decltype(i)::value;
+                    __builtin_amdgcn_sched_barrier(0);
+                    mfma_tiles(ch, i, std::integral_constant<int, I + 1>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_tile_range(std::integral_constant<int, 1 - c>{}, std::integral_constant<int, (I - X1) * kEach>{},
+                                    std::integral_constant<int, (I - X1 + 1) * kEach>{}, std::false_type{});
+                    load_tile_range(std::integral_constant<int, 1 - c>{}, i, std::integral_constant<int, I + 1>{}, std::integral_constant<bool, I + 1 == NT>{});
+                });
+                requested = true;
+            } else {
+                mfma_tiles(ch, IX{}, IN{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        } else if (!FIRST) {
+            mfma_tiles(ch, IA{}, IP{});
             if (wait_for) seen = __hip_atomic_load(counters + (1 - c) * kSyncStride, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
-            mfma_tiles(IP{}, IN{});
+            mfma_tiles(ch, IP{}, IN{});
             __builtin_amdgcn_sched_barrier(0);   // the counter's value is looked at after the MFMAs, not right behind its load
         }
-        if (wait_for) {
+        if (wait_for && !requested) {
             const unsigned target = wait_for * members;
-            const bool there = !FIRST && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0;
+            const bool there = !FIRST && !DB && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0;
             if (!there && !wave_wait(w, counters + (1 - c) * kSyncStride, target, g.spin_polls)) return false;
             load_tiles(std::integral_constant<int, 1 - c>{});   // every wavefront's reads of this unit's tiles have been issued and waited for by its MFMAs
         }
