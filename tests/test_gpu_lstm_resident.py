@@ -44,6 +44,8 @@ CASES = [
     ("512-cells-zoneout-stacked", [dict(units=16), zone(512), lstm(128), dict(units=128, activation="LINEAR")], 4, 48, 48, True),
     ("1024-cells-two-directions", [dict(units=10), lstm(1024, bidirectional=True), dict(units=1024, activation="LINEAR")], 3, 40, 40, True),
     ("1024-cells-ragged-seven-steps", [dict(units=6), lstm(1024), dict(units=1024, activation="LINEAR")], 7, 45, 48, True),
+    ("1024-cells-two-steps", [dict(units=5), lstm(1024), dict(units=1024, activation="LINEAR")], 2, 33, 33, True),
+    ("1024-cells-twelve-steps-zoneout", [dict(units=7), zone(1024, bidirectional=True), dict(units=1024, activation="LINEAR")], 12, 64, 64, True),
     ("two-steps", [dict(units=6), lstm(256), dict(units=256, activation="LINEAR")], 2, 32, 32, True),
 ]
 
