@@ -950,6 +950,15 @@ int Net::lstm_backward_step_norm(LstmLayer &q, size_t B, size_t s)
     return MYEA_OK;
 }
 
+bool Net::lstm_backward_loop_leaves_room(size_t li, size_t B)
+{
+    const DevLayer &o = L[li];
+    if (!o.lstm) return false;
+    LstmResidentPlan plan;
+    if (lstm_resident_plan(o.lstm->C, o.lstm->cpb, B, o.lstm2 ? 2 : 1, &plan) != MYEA_OK || !plan.ok || !plan.backward) return false;
+    return 2 * plan.grid <= plan.cus;
+}
+
 int Net::side_stream_create()
 {
     if (side_stream || side_stream_disabled()) return MYEA_OK;

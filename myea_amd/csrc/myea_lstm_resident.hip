@@ -72,7 +72,7 @@ constexpr int kLocalAux = 16;      // cache policy of the LOCAL protocol's tile 
 
 // LDS of a workgroup: every wavefront's tiles of one unit, and the partial tiles of the two chains
 constexpr size_t forward_lds(int kw, int cells, int rs) { return ((size_t)4 * (kw / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * (4 * cells + 8)) * sizeof(float); }
-constexpr size_t backward_lds(int c, int rs) { return ((size_t)4 * (c > 512 ? 16 : c / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * 17) * sizeof(float); }
+constexpr size_t backward_lds(int c, int rs) { return ((size_t)4 * (c >= 512 && rs == 1 ? c / 64 : c / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * 17) * sizeof(float); }
 
 template <int N>
 __device__ __forceinline__ void wait_vm() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }   // vmcnt(N)
@@ -594,7 +594,8 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
     // half buffers of NT / 4 tiles per wavefront in four groups: while group g is contracted, group g + 2 lands in the half
     // that group g has just left.  Its 64 members span two XCDs: device-scope stores of the gate deltas, device-scope
     // counter, tile loads served beyond the XCD's L2 (as in the forward loop of this width).
-    constexpr bool WIDE = C > 512, AGENT = WIDE;
+    constexpr bool AGENT = C > 512;               // 64 members: the group spans two XCDs
+    constexpr bool WIDE = C >= 512 && RS == 1;    // a unit's tiles pass through half as many LDS slots, requested a quarter of the unit ahead
     constexpr int SLOTS = WIDE ? NT / 2 : NT, NG = NT / 4;   // tiles of LDS per wavefront; tiles per group
     constexpr int kStage = SLOTS * ROWS * 32, kPart = 4 * ROWS * kStride;
     constexpr int kAux = AGENT ? 16 : kLocalAux;

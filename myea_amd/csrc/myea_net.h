@@ -190,6 +190,7 @@ struct Net {
     int lstm_backward_layer(size_t li, size_t B);       // BPTT inside LSTM layer li
     // delta / weight operands an LSTM consumer gi offers to the layer below: delta [T][Bmax][width], weights [width][fan-in]
     void lstm_delta_source(size_t gi, int direction, const float **delta, size_t *width, const float **weights);
+    bool lstm_backward_loop_leaves_room(size_t li, size_t B);   // the layer's resident backward loop occupies at most half of the compute units
     int side_stream_create();
     int side_stream_join();            // `stream` waits for what the last SideStreamScope enqueued
     int lstm_forward_inputs(size_t li, LstmLayer &q, size_t B);

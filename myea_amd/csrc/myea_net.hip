@@ -1194,7 +1194,11 @@ bool Net::dw_beside_loop_allowed(size_t gi, size_t li, size_t B)
     static const bool off = [] { const char *e = std::getenv("MYEA_DW_BESIDE_LOOP"); return e && e[0] == '0'; }();
     if (off || !side_stream || d.number_recurrent_depth < 2 || B != d.batch_size) return false;
     if (L[li].lstm2 || L[gi].lstm2 || (gi < dw_done.size() && dw_done[gi])) return false;
-    return d.layers[gi].type_layer == MYEA_LAYER_LSTM;
+    if (d.layers[gi].type_layer != MYEA_LAYER_LSTM || !L[li].lstm) return false;
+    // ... and a loop that leaves at least half of the compute units without a workgroup.  One that fills the device is faster
+    // alone in its column form than in the k form beside the contractions, by more than those then hide (2 x LSTM-512 at a
+    // batch of 256: 3.66 against 3.70 ms per step).
+    return lstm_backward_loop_leaves_room(li, B);
 }
 
 int Net::update_derivative_weight(size_t B, size_t first, size_t end)
