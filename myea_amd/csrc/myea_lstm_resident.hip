@@ -71,7 +71,7 @@ constexpr int kLocalAux = 16;      // cache policy of the LOCAL protocol's tile 
 #define MYEA_SCOPE_WORKGROUP __HIP_MEMORY_SCOPE_WORKGROUP
 
 // LDS of a workgroup: every wavefront's tiles of one unit, and the partial tiles of the two chains
-constexpr size_t forward_lds(int kw, int cells, int rs) { return ((size_t)4 * (kw / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * (4 * cells + 8)) * sizeof(float); }
+constexpr size_t forward_lds(int kw, int cells, int rs) { return ((size_t)4 * (kw == 128 && rs == 1 ? 2 : kw / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * (4 * cells + 8)) * sizeof(float); }
 constexpr size_t backward_lds(int c, int rs) { return ((size_t)4 * (c >= 512 && rs == 1 ? c / 64 : c / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * 17) * sizeof(float); }
 
 template <int N>
@@ -257,7 +257,9 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
     constexpr int A1 = NT >= 4 ? NT / 4 : 1;      // tiles whose MFMAs run before the previous unit's arrival is signalled
     constexpr int P1 = NT >= 4 ? (3 * NT) / 4 : NT - 1;   // tile before which the next unit's counter is read
     constexpr int kStride = NB + 8;               // floats per row of a wavefront's partial tile
-    constexpr int kStage = NT * ROWS * 32, kPart = 4 * ROWS * kStride;
+    constexpr bool HALF = !AGENT && NT == 4 && RS == 1;   // 512 cells: two LDS slots for a unit's four tiles, each requested two tiles ahead
+    constexpr int SLOTS = HALF ? NT / 2 : NT;
+    constexpr int kStage = SLOTS * ROWS * 32, kPart = 4 * ROWS * kStride;
     constexpr int kAux = AGENT ? 16 : kLocalAux;
     constexpr bool DB = AGENT;                    // the other chain's tiles are requested during this chain's last MFMAs, into the slots those have left
     constexpr int S1 = (5 * NT) / 8, X1 = (3 * NT) / 4;   // DB: tile behind which the other chain's counter is read / behind which its value is looked at
@@ -378,17 +380,17 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
 #pragma unroll
             for (int q = 0; q < LPT; ++q)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p_tile[c][q] + i * 32),
-                                                 (__attribute__((address_space(3))) void *)(stage + i * ROWS * 32 + q * 256), 16, 0, kAux);
+                                                 (__attribute__((address_space(3))) void *)(stage + (i % SLOTS) * ROWS * 32 + q * 256), 16, 0, kAux);
         if (decltype(advance)::value) {
 #pragma unroll
             for (int q = 0; q < LPT; ++q) p_tile[c][q] += step_c;
         }
     };
-    auto load_tiles = [&](auto ch) { load_tile_range(ch, std::integral_constant<int, 0>{}, std::integral_constant<int, NT>{}, std::true_type{}); };
+    auto load_tiles = [&](auto ch) { load_tile_range(ch, std::integral_constant<int, 0>{}, std::integral_constant<int, SLOTS>{}, std::integral_constant<bool, !HALF>{}); };
     auto mfma_tiles = [&](auto ch, auto first, auto last) {
 #pragma unroll
         for (int i = decltype(first)::value; i < decltype(last)::value; ++i) {
-            const float *tile = stage + i * ROWS * 32;
+            const float *tile = stage + (i % SLOTS) * ROWS * 32;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 f32x4 fa[RS];
@@ -421,7 +423,13 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
         if (decltype(all_landed)::value) wait_vm<0>(); else wait_vm<NSTORE>();
         mfma_tiles(ch, I0{}, IA{});
         __builtin_amdgcn_sched_barrier(0);   // keeps the MFMAs above in front of the wait
-        wait_vm<0>();
+        if constexpr (HALF) {   // the third tile into the slot the first has left; the stores of the unit before are older
+            load_tile_range(ch, std::integral_constant<int, 2>{}, std::integral_constant<int, 3>{}, std::false_type{});
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<LPT>();
+        } else {
+            wait_vm<0>();
+        }
         wave_arrive<AGENT>(counters + (1 - c) * kSyncStride, &s_arrive[1 - c]);
     };
     // The rest of the unit.  FIRST: the chain's first step (no recurrent term, no forget gate, no peephole into the input
@@ -431,8 +439,44 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
         constexpr int c = decltype(ch)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
         load_inputs(ch);
-        bool requested = false;   // DB: the other chain's tiles are on their way already
-        if constexpr (!FIRST && DB) {
+        bool requested = false;   // the other chain's tiles are on their way already
+        if constexpr (!FIRST && HALF) {
+            // Two slots for four tiles: tile i + 2 is requested behind tile i's MFMAs (a unit's first two behind the last two
+            // MFMA tiles of the unit before, if the chain's counter is complete by then), so a wavefront never issues more than
+            // two loads in a row - eight in a row, four wavefronts at once, keep the compute unit's address path busy for 512
+            // clocks during which the issuing wavefronts stand still.  The first wait counts what was issued behind the tile it
+            // waits for; the unit's inputs are counted as four loads, the fewest there can be (two more with zoneout masks: it
+            // then asks for a little more than it needs).  The second leaves nothing in flight - the inputs too, requested two
+            // tiles of MFMAs ago - so that the compiler has no load left to wait for in front of the gate math: it would
+            // wait for everything there, the next unit's tiles included.
+            constexpr int kIn = 4 * PAIRS;
+            using I1 = std::integral_constant<int, 1>;
+            using I2 = std::integral_constant<int, 2>;
+            using I3 = std::integral_constant<int, 3>;
+            using Other = std::integral_constant<int, 1 - c>;
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_tiles(ch, I1{}, I2{});
+            __builtin_amdgcn_sched_barrier(0);
+            load_tile_range(ch, I3{}, IN{}, std::true_type{});   // the fourth tile into the second's slot
+            asm volatile("global_load_dword %0, %1, off sc1" : "=v"(seen) : "v"(counters + (1 - c) * kSyncStride) : "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<LPT + 1 + kIn>();              // the third tile has landed: behind it came the inputs, the fourth tile, the counter
+            mfma_tiles(ch, I2{}, I3{});
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<0>();                          // the fourth, the counter's value, the inputs
+            asm volatile("" : "+v"(seen));         // looked at behind the wait, not before
+            if (wait_for && (int)(__builtin_amdgcn_readfirstlane(seen) - wait_for * members) >= 0) {
+                load_tile_range(Other{}, I0{}, I1{}, std::false_type{});
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_tiles(ch, I3{}, IN{});
+                __builtin_amdgcn_sched_barrier(0);
+                load_tile_range(Other{}, I1{}, I2{}, std::false_type{});
+                requested = true;
+            } else {
+                mfma_tiles(ch, I3{}, IN{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        } else if constexpr (!FIRST && DB) {
             // The other chain's counter is read five eighths into the MFMAs, when its step is normally complete, and looked at an
             // eighth later; its tiles are then requested between the last quarter's MFMAs, into the slots whose tiles those
             // MFMAs no longer need (a tile's own slot right behind its MFMAs) - they have those MFMAs and the gate math to
@@ -472,7 +516,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
         }
         if (wait_for && !requested) {
             const unsigned target = wait_for * members;
-            const bool there = !FIRST && !DB && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0;
+            const bool there = !FIRST && !DB && !HALF && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0;
             if (!there && !wave_wait(w, counters + (1 - c) * kSyncStride, target, g.spin_polls)) return false;
             load_tiles(std::integral_constant<int, 1 - c>{});   // every wavefront's reads of this unit's tiles have been issued and waited for by its MFMAs
         }
