@@ -717,7 +717,7 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     // Tile choice: 128 x 128 when that still yields at least two workgroups per CU (256 CUs), else
     // 64-row tiles to keep the chip filled for short-M / short-N problems.
     const long tiles_128 = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
-    if (tiles_128 >= 512) return launch_layout_vec<128, 128>(stream, d, a_kc, b_kc);
+    if (tiles_128 * d.ksplit >= 512) return launch_layout_vec<128, 128>(stream, d, a_kc, b_kc);   // slabs of a split k count: they fill the chip like tiles do
     // At most one 64 x 64 tile per compute unit and a k worth splitting: two workgroups per tile, half of k each, combined in
     // the launch - a second wavefront per SIMD to fill the first one's waits, which such a launch otherwise lacks.
     // MYEA_GEMM_PAIR_K=0 keeps one workgroup per tile.

@@ -1804,8 +1804,8 @@ int myea_hip_backward_pass_update_derivative_weight_and_update_parameter(myea_hi
 int myea_hip_reset_loss(myea_hip_net *n)
 {
     NET_OR_FAIL(n);
-    MYEA_HIP_TRY(hipMemsetAsync(n->net.loss_acc, 0, 8 * sizeof(double), n->net.stream));
-    return MYEA_OK;
+    // a fill kernel, not a memset: callers may capture their step in a graph
+    return myea::launch_fill(n->net.stream, reinterpret_cast<float *>(n->net.loss_acc), 8 * sizeof(double) / sizeof(float), 0.f);
 }
 int myea_hip_get_loss(myea_hip_net *n, myea_loss_state *s)
 {
