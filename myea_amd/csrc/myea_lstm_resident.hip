@@ -236,6 +236,7 @@ struct ResidentGeometry {
     int members;               // workgroups per group = C / CELLS
     int arrivals;              // arrivals that complete a unit: members (one more under the test switch, so that no unit ever completes)
     unsigned spin_polls;       // polls after which a wait gives up
+    int never_early;           // test switch: the look at the other chain's counter during a unit's MFMAs always says "not yet"
 };
 
 namespace {
@@ -465,7 +466,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
             __builtin_amdgcn_sched_barrier(0);
             wait_vm<0>();                          // the fourth, the counter's value, the inputs
             asm volatile("" : "+v"(seen));         // looked at behind the wait, not before
-            if (wait_for && (int)(__builtin_amdgcn_readfirstlane(seen) - wait_for * members) >= 0) {
+            if (wait_for && !g.never_early && (int)(__builtin_amdgcn_readfirstlane(seen) - wait_for * members) >= 0) {
                 load_tile_range(Other{}, I0{}, I1{}, std::false_type{});
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_tiles(ch, I3{}, IN{});
@@ -492,7 +493,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
             __builtin_amdgcn_sched_barrier(0);
             wait_vm<0>();                          // the unit's inputs (requested long ago) and the counter's value
             asm volatile("" : "+v"(seen));         // looked at behind the wait, not before
-            if (wait_for && (int)(__builtin_amdgcn_readfirstlane(seen) - wait_for * members) >= 0) {
+            if (wait_for && !g.never_early && (int)(__builtin_amdgcn_readfirstlane(seen) - wait_for * members) >= 0) {
                 constexpr int kEach = X1 / (NT - X1);   // free slots filled per tile of MFMAs
                 static_for<X1, NT>([&](auto i) {
                     constexpr int I = decltype(i)::value;
@@ -843,7 +844,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
             __builtin_amdgcn_sched_barrier(0);
             wait_vm<(NG - 2) * LPT>();       // tile 3 NG + 1 has landed, and the counter's value before it
             asm volatile("" : "+v"(seen));      // the value is looked at behind the wait, not before
-            if (wait_for && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0) {
+            if (wait_for && !g.never_early && (int)(__builtin_amdgcn_readfirstlane(seen) - target) >= 0) {
                 static_for<3 * NG, NT>([&](auto i) {
                     constexpr int I = decltype(i)::value;
                     __builtin_amdgcn_sched_barrier(0);
@@ -1277,6 +1278,15 @@ bool absent_member_for_test()
     return e && e[0] == '1';
 }
 
+// MYEA_LSTM_RESIDENT_TEST_NEVER_EARLY=1: a unit never finds the other chain's counter complete while its own MFMAs run, so
+// the next unit's first tiles are always requested behind them (the path a late group takes).  For tests: which of the two
+// paths a unit takes otherwise depends on timing.
+bool never_early_for_test()
+{
+    const char *e = std::getenv("MYEA_LSTM_RESIDENT_TEST_NEVER_EARLY");
+    return e && e[0] == '1';
+}
+
 // ---- host: the kernels on offer ------------------------------------------------------------------------------------------
 using ResidentKernel = void (*)(ResidentGeometry, LstmResidentDir, LstmResidentDir, SyncWords);
 struct KernelInfo {
@@ -1368,6 +1378,7 @@ int fill_geometry(const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax,
     g->T = (int)T; g->B = (int)B; g->Bmax = (int)Bmax; g->C = (int)C;
     g->dirs = dirs; g->row_groups = plan.row_groups; g->members = plan.members;
     g->arrivals = plan.members + (absent_member_for_test() ? 1 : 0);
+    g->never_early = never_early_for_test() ? 1 : 0;
     g->spin_polls = spin_polls();
     return MYEA_OK;
 }

@@ -165,6 +165,33 @@ def test_bias_and_peephole_gradients_summed_inside_the_backward_loop(ksplit):
             n.Update_Parameter(B, B)
 
 
+@pytest.mark.parametrize("name,specs,T,B,Bmax", [(c[0], c[1], c[2], c[3], c[4]) for c in CASES if "512-cells" in c[0] or "1024-cells" in c[0]],
+                         ids=[c[0] for c in CASES if "512-cells" in c[0] or "1024-cells" in c[0]])
+def test_the_path_of_a_late_group(name, specs, T, B, Bmax):
+    """At 512 and 1024 cells a unit requests the next unit's first tiles between its own last MFMAs if the other chain's
+    counter is complete by then, behind them if not; which of the two happens depends on timing.  Here the second is forced
+    (every unit is told "not yet") and held against the oracle."""
+    desc, h, w, masks, X, Y = _setup(specs, T, B, Bmax, seed=23)
+    zone_masks = masks if any(s.get("dropout") == "ZONEOUT" for s in specs) else None
+    gpu = _net(desc, h, w, zone_masks)
+    cpu = OracleNetwork(desc, h)
+    cpu.set_state_propagation(mb.STATE_TRAINING)
+    cpu.upload_parameters(w)
+    if zone_masks is not None:
+        cpu.upload_zoneout_masks(zone_masks)
+    cpu.Clear_Training_Arrays()
+    with environment(MYEA_LSTM_RESIDENT_TEST_NEVER_EARLY=1, MYEA_LSTM_BACKWARD_KSPLIT=0):   # the backward form that stages tiles
+        gpu.profile_enable(True)
+        for n in (gpu, cpu):
+            n.Reset__Loss()
+            run_step(n, B, X[:B], Y[:B], update=False)
+        fwd, bwd = _loop_launches(gpu)
+        gpu.profile_enable(False)
+    layers = sum(1 for i in range(desc.n_layers) if desc.layers[i].type_layer == mb.LAYER_LSTM)
+    assert fwd == layers and bwd == layers, "the time loops did not run as one launch per layer"
+    _compare(desc, gpu, cpu, B, T, "late path")
+
+
 def test_a_smaller_batch_after_a_larger_one():
     """rows beyond the batch keep what the larger batch left there; the rows of the batch do not depend on them"""
     specs = [dict(units=8), lstm(128), dict(units=128, activation="LINEAR")]
