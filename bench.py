@@ -5,7 +5,8 @@ One "step" = Forward_Pass + Compute__Error + Backward_Pass, Update_Derivative_We
 one call; --separate-update: Update_Parameter as a call of its own) on one batch of synthetic data already resident in HBM.  Default workload: BASELINE config 2, the deep fully-connected
 stack 4096-4096-4096-4096-4096-1000 (ReLU, softmax + cross-entropy, Adam) at batch 1024, fp32.
 
-Prints ONE JSON line.  `value` comes from exactly `steps` timed steps.  `roofline` covers the dominant kernel family — the
+Prints ONE JSON line.  The timed block of exactly `steps` steps is run `--repeats` times; `value` and `ms_per_step` are the
+median block's, every block's figure is listed (`ms_per_step_blocks`).  `roofline` covers the dominant kernel family — the
 FP32 MFMA contractions (forward X W^T, dX = delta W, dW += delta^T X): algorithmic FLOPs of all their launches over their
 summed HIP-event durations on the stream they run on, taken in a second pass of `steps` steps (`events_pass`), because a
 pair of timing events around every launch slows the step it measures.  `cpu_baseline` times the CPU restatement of the
@@ -25,7 +26,10 @@ if ROOT not in sys.path:
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same counters read for copies of
 # known size (FETCH_SIZE x2, WRITE_SIZE x1); the line names the file the figure comes from.
 RECORDED_TRAFFIC = {"fc4096x4_b1024_adam": dict(bytes_per_launch=2944490 * 1024 / 10,
-                                                source="recorded constant, not measured in this run: profiles/hbm_traffic__fc4096x4_b1024_adam__pmc.txt")}
+                                                source="recorded constant, not measured in this run: profiles/hbm_traffic__fc4096x4_b1024_adam__pmc.txt"),
+                    # the two resident time loops of one layer (forward + backward launch), mean per launch
+                    "lstm512x2_t64_b256_amsgrad": dict(bytes_per_launch=(299.0e6 + 400.0e6) / 2,
+                                                       source="recorded constant, not measured in this run: profiles/lstm_resident__lstm512x2_t64_b256_amsgrad__pmc.txt")}
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
@@ -149,11 +153,11 @@ def cpu_baseline(wl, sample_rows, threads):
 # profile families of the library (myea_hip_profile_read): name, what its `work` counts
 FAMILIES = (("forward", "flop"), ("dx", "flop"), ("dw", "flop"), ("update", "byte"), ("dx_dw_pair", "flop"),
             ("lstm_forward_loop", "flop"), ("lstm_backward_loop", "flop"),
-            ("normalization", "byte"), ("bias_gradient", "byte"))
+            ("normalization", "byte"), ("bias_gradient", "byte"), ("output_error", "byte"), ("softmax", "byte"))
 KERNEL_NAMES = {"forward": "gemm_forward", "dx": "gemm_dx", "dw": "gemm_dw", "dx_dw_pair": "gemm_dx_dw_pair", "update": "optimizer_update"}
 
 
-def run_workload(name, steps, warmup, separate_update=False):
+def run_workload(name, steps, warmup, separate_update=False, repeats=1):
     """Times `steps` training steps of one workload on cuda:0 (inputs resident in HBM): that is the throughput.  Then runs
     `steps` more with the library's per-family HIP-event timers on for the per-kernel figures - a pair of timing events around
     every launch keeps launches from overlapping their neighbours' tails and costs 3 % (the wide dense stack) to 16 % (the
@@ -189,13 +193,15 @@ def run_workload(name, steps, warmup, separate_update=False):
 
     for _ in range(warmup):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / steps
+    blocks = []
+    for _ in range(max(1, repeats)):      # every block: exactly `steps` steps between two synchronisations
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        blocks.append((time.perf_counter() - t0) * 1e3 / steps)
+    ms_per_step = sorted(blocks)[(len(blocks) - 1) // 2]   # the median block (the lower middle one of an even count)
     net.profile_enable(True)
     for f in range(len(FAMILIES)):
         net.profile_read(f)            # drop anything recorded so far
@@ -243,6 +249,7 @@ def run_workload(name, steps, warmup, separate_update=False):
                     launches=n, avg_launch_ms=ms / max(n, 1), flops_per_launch=flop / max(n, 1), ms_per_step=ms / steps)
 
     return dict(workload=name, wl=wl, desc_parameters=int(desc.total_parameters), batch=B, ms_per_step=ms_per_step, value=B / (ms_per_step * 1e-3),
+                ms_per_step_blocks=blocks,
                 ms_per_step_events=ms_per_step_events,
                 kernels=kernels, loss_per_output=loss.loss_values / max(loss.number_loss, 1),
                 contractions=mfma_aggregate(("forward", "dx", "dw", "dx_dw_pair")),
@@ -264,6 +271,50 @@ SECONDARY = "lstm512x2_t64_b256_amsgrad"   # the metric's other half
 OTHERS = ("fc2048x8_bn_relu_dropout_b512_nesterov", "bilstm1024_t512_b64_adabound")
 
 
+def timed_blocks(stream_call):
+    """stream_call() enqueues one launch on torch's current stream; returns the mean duration in ms of a launch inside a block
+    of 20 back-to-back launches between two events on that stream (best of 3 blocks, after a warm-up launch)"""
+    import torch
+    stream_call()
+    best = None
+    for _ in range(3):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(20):
+            stream_call()
+        b.record()
+        b.synchronize()
+        ms = a.elapsed_time(b) / 20
+        best = ms if best is None or ms < best else best
+    return best
+
+
+def optimizer_update_alone(parameters):
+    """myea_hip_optimizer_update alone on the device over `parameters` floats (the headline configuration's vector), per
+    optimizer: algorithmic bytes (every vector the update reads or writes, once) over the launch's duration."""
+    import ctypes as C
+    import torch
+    from myea_amd import binding as mb
+    lib = mb.load_library()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    vec = [torch.zeros(parameters, dtype=torch.float32, device="cuda") for _ in range(5)]
+    vec[1].normal_(0, 1e-2)
+    legs = {}
+    for name, kw, bytes_per in (("adam", dict(type_optimizer_function=mb.OPTIMIZER["ADAM"]), 32), ("amsgrad", dict(type_optimizer_function=mb.OPTIMIZER["AMSGRAD"]), 40),
+                                ("adabound", dict(type_optimizer_function=mb.OPTIMIZER["ADABOUND"]), 32),
+                                ("nesterov", dict(type_optimizer_function=mb.OPTIMIZER["GD"], use_Nesterov=1, learning_momentum=0.9), 24)):
+        h = mb.default_hyper(optimizer_time_step=1.0, **kw)
+
+        def call():
+            rc = lib.myea_hip_optimizer_update(stream, C.byref(h), parameters, parameters, 1.0, *(C.c_void_p(v.data_ptr()) for v in vec))
+            if rc != 0:
+                raise RuntimeError((lib.myea_hip_last_error() or b"").decode())
+        ms = timed_blocks(call)
+        gbs = bytes_per * parameters / (ms * 1e-3) / 1e9
+        legs[name] = dict(avg_ms=ms, bytes_per_parameter=bytes_per, gbs=gbs, frac_hbm_peak=gbs / PEAK_HBM_GBS)
+    return dict(kernel="update_kernel (myea_hip_optimizer_update alone on the device)", parameters=parameters, optimizers=legs)
+
+
 def measured_ceilings():
     """What this device reaches on a kernel of nothing but FP32 MFMAs and on a streaming triad, beside the published peaks."""
     import ctypes as C
@@ -283,6 +334,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--repeats", type=int, default=10, help="timed blocks of exactly --steps steps; value = the median block")
     ap.add_argument("--workload", default="fc4096x4_b1024_adam", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the LSTM-512 leg and the two short legs of the other configurations that the default workload's line also carries")
@@ -297,7 +349,7 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
-    r = run_workload(args.workload, args.steps, args.warmup, args.separate_update)
+    r = run_workload(args.workload, args.steps, args.warmup, args.separate_update, args.repeats)
     wl, B = r["wl"], r["batch"]
     has_loops = r["time_loops"]["launches"] > 0
     alone = r["contractions_alone"]
@@ -322,6 +374,10 @@ def main():
         "value": r["value"],
         "unit": "samples/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms_per_step"],
+        # the timed block (exactly `steps` steps between two synchronisations) was run `repeats` times: value and ms_per_step are the
+        # median block's, the others are listed
+        "repeats": len(r["ms_per_step_blocks"]), "ms_per_step_blocks": [round(x, 4) for x in r["ms_per_step_blocks"]],
+        "ms_per_step_spread": {"min": min(r["ms_per_step_blocks"]), "max": max(r["ms_per_step_blocks"])},
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": config_of(r),
         "roofline": roofline,
@@ -338,9 +394,14 @@ def main():
         out["time_loops"] = dict(r["time_loops"], kernel="lstm_resident_forward_kernel / lstm_resident_backward_kernel (or one lstm_fused_* launch per step)")
     if args.workload != SECONDARY and args.workload == "fc4096x4_b1024_adam" and not args.no_secondary:
         sec_steps = max(5, 2 * args.steps // 3)
-        s = run_workload(SECONDARY, sec_steps, max(2, args.warmup), args.separate_update)
+        s = run_workload(SECONDARY, sec_steps, max(2, args.warmup), args.separate_update, args.repeats)
         loops = dict(s["time_loops"], kernel="lstm_resident_forward_kernel + lstm_resident_backward_kernel: the recurrent contractions and gate math of steps 1 .. T-1, one launch per layer and pass")
+        sec_traffic = RECORDED_TRAFFIC.get(SECONDARY)
+        loops["traffic"] = sec_traffic["bytes_per_launch"] if sec_traffic else None
+        if sec_traffic:
+            loops["traffic_source"] = sec_traffic["source"]
         out["secondary"] = {"workload": SECONDARY, "value": s["value"], "unit": "samples/s", "ms_per_step": s["ms_per_step"],
+                            "repeats": len(s["ms_per_step_blocks"]), "ms_per_step_blocks": [round(x, 4) for x in s["ms_per_step_blocks"]],
                             "steps": sec_steps, "events_pass": {"steps": sec_steps, "ms_per_step": s["ms_per_step_events"]}, "config": config_of(s), "roofline": loops,
                             "contractions": s["contractions"], "kernels": s["kernels"], "loss_per_output": s["loss_per_output"]}
         # the other two configurations of the baseline that are timed on the GPU, a few steps each, so that one run records all four
@@ -348,10 +409,12 @@ def main():
         for name in OTHERS:
             o = run_workload(name, max(5, args.steps // 3), max(2, args.warmup // 2), args.separate_update)
             leg = {"workload": name, "value": o["value"], "unit": "samples/s", "ms_per_step": o["ms_per_step"], "steps": max(5, args.steps // 3),
-                   "config": config_of(o), "contractions": o["contractions_alone"] or o["contractions"], "loss_per_output": o["loss_per_output"]}
+                   "config": config_of(o), "contractions": o["contractions_alone"] or o["contractions"], "kernels": o["kernels"], "loss_per_output": o["loss_per_output"]}
             if o["time_loops"]["launches"] > 0:
                 leg["time_loops"] = o["time_loops"]
             out["other_configurations"].append(leg)
+        # the memory-bound update alone on the device, per optimizer, over the headline configuration's parameter vector
+        out["optimizer_update_alone"] = optimizer_update_alone(r["desc_parameters"])
     if not args.no_ceilings:
         out["ceilings"] = measured_ceilings()
     if not args.no_cpu_baseline:
@@ -363,6 +426,12 @@ def main():
             rows = int(max(4, min(B, 20.0 * threads * 15.0e9 / flop_per_row)))
             rows = max(threads, rows - rows % threads)
         out["cpu_baseline"] = cpu_baseline(wl, rows, threads)
+        if "secondary" in out:   # the metric's other half on the same host cores: whole sequences through the oracle
+            swl = WORKLOADS[SECONDARY]
+            flop_per_row = gemm_flops_per_step(swl["layers"], 1, swl.get("depth", 1))
+            rows = int(max(4, min(swl["batch"], 20.0 * threads * 15.0e9 / flop_per_row)))
+            rows = max(threads, rows - rows % threads)
+            out["secondary"]["cpu_baseline"] = cpu_baseline(swl, min(rows, swl["batch"]), threads)
     print(json.dumps(out))
 
 

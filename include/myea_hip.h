@@ -65,6 +65,8 @@ enum {
 enum {
     MYEA_OPTIMIZER_NONE = 0, MYEA_OPTIMIZER_ADABOUND = 1, MYEA_OPTIMIZER_ADAM = 2,
     MYEA_OPTIMIZER_AMSBOUND = 4, MYEA_OPTIMIZER_AMSGRAD = 5, MYEA_OPTIMIZER_GD = 6,
+    MYEA_OPTIMIZER_IRPROP_MINUS = 7,   /* myea_hip_optimizer_update only: the reference's Update_Parameter has no case for it
+                                        * (Neural_Network.cpp:4770-4821) and neither has myea_hip_update_parameter */
     MYEA_OPTIMIZER_IRPROP_PLUS = 8, MYEA_OPTIMIZER_NOSADAM = 9
 };
 
@@ -107,7 +109,16 @@ enum {
     MYEA_E_BATCH = -3,        /* batch_size_received > batch_size (Forward_Pass__OpenMP.cpp:33-43) */
     MYEA_E_STATE = -4,        /* e.g. backward in inference mode (Backward_Pass__OpenMP.cpp:41-51) */
     MYEA_E_NOMEM = -5,
-    MYEA_E_DEVICE = -6        /* HIP runtime error; text in myea_hip_last_error() */
+    MYEA_E_DEVICE = -6        /* HIP runtime error; text in myea_hip_last_error().  Also reported, once, by the next call that
+                               * looks (Forward_Pass, synchronize, get_loss, any download or upload) after a kernel's bounded wait
+                               * for another workgroup gave up - a resident LSTM time loop, a contraction whose tiles two
+                               * workgroups share.  The pass that kernel belonged to is incomplete.  State the caller is left in:
+                               * no Update_Parameter enqueued behind that kernel has changed parameters or optimizer vectors
+                               * (the update kernels see a device-side flag), the optimizer's time step and the other scalars an
+                               * update advances are back at their values before the first such update, the gradient is zero,
+                               * and the network uses the plain form of that kernel from then on (one launch per time step, one
+                               * workgroup per tile).  Repeat the mini-batch.  Only an optimizer clearing by a warm restart that
+                               * fell on a skipped update is not taken back. */
 };
 
 /* ---- network descriptor ---- */
@@ -318,8 +329,13 @@ int myea_hip_synchronize(myea_hip_net *net);
 const char *myea_hip_last_error(void);
 
 /* ---- public-field setters: replace the `Set__*` forwarding in Train.cpp:28-90 ---- */
+/* set_hyper replaces EVERY field, the ones the library itself advances included: optimizer_time_step (every update),
+ * adam_previous_beta2 (NosAdam's running sum), epoch_time_step, warm_restarts_T_i and warm_restarts_maximum_learning_rate
+ * (a warm restart), loss_rprop / previous_loss_rprop (Clear_Training_Arrays).  A caller that changes a setting between
+ * steps starts from get_hyper, changes that field and hands the struct back - as the reference's setters change one public
+ * field of the object and leave the others alone; a struct built from myea_hyper_default() would reset the optimizer's clock. */
 int myea_hip_set_hyper(myea_hip_net *net, const myea_hyper *hyper);
-int myea_hip_get_hyper(myea_hip_net *net, myea_hyper *hyper);  /* reads back optimizer_time_step */
+int myea_hip_get_hyper(myea_hip_net *net, myea_hyper *hyper);
 /* `type_state_propagation` (Data.hpp, Enum_Type_State_Propagation.hpp) */
 int myea_hip_set_state_propagation(myea_hip_net *net, uint32_t type_state_propagation);
 
@@ -466,7 +482,8 @@ int myea_hip_upload_tensor(myea_hip_net *net, size_t layer_index, int kind, cons
  * contractions and gate math of an LSTM layer's forward time loop (steps 1 .. T-1; one launch per layer when the
  * loop runs as a resident kernel, one per step otherwise), 6 = the same of its backward time loop, 7 = batch
  * (re)normalisation forward and backward (bytes: every activation read or written once), 8 = column sums of the
- * deltas for the bias gradients (bytes). */
+ * deltas for the bias gradients (bytes), 9 = Compute__Error's output delta + loss kernel (bytes: outputs and desired values
+ * read, delta written), 10 = the output layer's softmax (bytes: sums read, values written). */
 int myea_hip_profile_enable(myea_hip_net *net, int enable);
 int myea_hip_profile_read(myea_hip_net *net, int family, uint64_t *launches, double *milliseconds, double *work);
 
@@ -482,11 +499,15 @@ int myea_hip_gemm_f32(void *stream, int a_k_contiguous, int b_k_contiguous, int 
                       size_t M, size_t N, size_t K,
                       const float *A, size_t lda, const float *B, size_t ldb, float *C, size_t ldc);
 
-/* Fused weight update over [0, count): Update_Parameters__{Adam,AMSGrad,AdaBound} and
- * Update_Parameter__Gradient_Descent{,_Momentum}, _Nesterov_Accelerated_Gradient.  `hyper` supplies
- * every scalar; optimizer_time_step is the value *after* the increment.  `gradient_scale` multiplies
+/* Fused weight update over [0, count): Update_Parameters__{Adam,AMSGrad,AdaBound,AMSBound} and
+ * Update_Parameter__Gradient_Descent{,_Momentum}, _Nesterov_Accelerated_Gradient, __iRPROP_plus, __iRPROP_minus.  `hyper`
+ * supplies every scalar; optimizer_time_step is the value *after* the increment.  `gradient_scale` multiplies
  * the gradient on read (clip-by-norm fused; pass 1).  Unused state pointers may be NULL.
- * weight decay applies to indices < weight_count. */
+ * weight decay applies to indices < weight_count.
+ * state0 / state1 / state2: gradient descent: previous deltas, -, -; the Adam family: first moment, second moment, its running
+ * maximum (AMSGrad, AMSBound); iRPROP+: previous deltas, previous steps, previous derivatives (the step back is taken when
+ * hyper->loss_rprop > hyper->previous_loss_rprop); iRPROP- (Neural_Network__iRPROP_minus.cpp:21-67): -, previous steps,
+ * previous derivatives. */
 int myea_hip_optimizer_update(void *stream, const myea_hyper *hyper, size_t count, size_t weight_count,
                               float gradient_scale, float *parameters, float *gradient,
                               float *state0, float *state1, float *state2);
@@ -495,7 +516,8 @@ int myea_hip_optimizer_update(void *stream, const myea_hyper *hyper, size_t coun
  * myea_hip_ceiling_mfma_f32: a kernel of nothing but independent v_mfma_f32_32x32x2_f32, two wavefronts per SIMD,
  * `iterations` x 16 MFMAs per wavefront; best of `repeats` launches, in TFLOP/s.
  * myea_hip_ceiling_hbm_triad: a[i] = b[i] + s * c[i] over three arrays of `bytes_per_array` (allocated and freed by
- * the call; choose them well beyond the caches); best of `repeats`, in GB/s of the 3 x bytes_per_array moved. */
+ * the call; choose them well beyond the caches), one 16-byte element per lane and non-temporal stores as the optimizer
+ * update has them; best of `repeats`, in GB/s of the 3 x bytes_per_array moved. */
 int myea_hip_ceiling_mfma_f32(void *stream, int iterations, int repeats, double *tflops);
 int myea_hip_ceiling_hbm_triad(void *stream, size_t bytes_per_array, int repeats, double *gigabytes_per_second);
 

@@ -24,7 +24,7 @@ AF = dict(NONE=0, COSINE=1, COSINE_SYMMETRIC=2, ELU=3, ELLIOT=4, ELLIOT_SYMMETRI
           LINEAR_PIECE_SYMMETRIC=13, LEAKY_RELU=14, PARAMETRIC_RELU=15, RELU=16, SELU=17, SIGMOID=18,
           SINE=19, SIGMOID_STEPWISE=20, SINE_SYMMETRIC=21, SOFTMAX=22, TANH=23, TANH_STEPWISE=24,
           THRESHOLD=25, THRESHOLD_SYMMETRIC=26)
-OPTIMIZER = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP_PLUS=8, NOSADAM=9)
+OPTIMIZER = dict(NONE=0, ADABOUND=1, ADAM=2, AMSBOUND=4, AMSGRAD=5, GD=6, IRPROP_MINUS=7, IRPROP_PLUS=8, NOSADAM=9)
 DROPOUT = dict(NONE=0, BERNOULLI=2, BERNOULLI_INVERTED=3, GAUSSIAN=4, SHAKEDROP=5, UOUT=6, ZONEOUT=7)
 NORMALIZATION = dict(NONE=0, BATCH_NORMALIZATION=1, BATCH_RENORMALIZATION=2)
 LOSS = dict(NONE=0, BIT=1, CROSS_ENTROPY=2, L1=3, L2=4, MAE=5, MAPE=6, ME=9, MSE=10, RMSE=11, SMAPE=12)

@@ -737,6 +737,8 @@ struct UpdateDev {
     float lr, mu, lr_t, beta1, beta2, eps, lower, upper, wd;
     const float *norm_sq;
     float clip, grad_scale;
+    const unsigned *fault;
+    unsigned long long *applied;
 };
 
 // One element of Update_Parameters__Adam (NN/Neural_Network__Adam.cpp:43-97), __AMSGrad
@@ -748,12 +750,23 @@ struct UpdateDev {
 // NosAdam (NN/Neural_Network__NosAdam.cpp:43-100) is KIND 3 with the host's beta2 at time t.
 // KIND: 0 GD, 1 momentum, 2 Nesterov, 3 Adam, 4 AMSGrad, 5 AdaBound, 6 AMSBound,
 //       7 iRPROP+ (a = previous delta, b = previous step, c = previous slope; lr / mu = increase / decrease factor,
-//         lower / upper = smallest / largest step, beta1 != 0 when the loss got worse).
+//         lower / upper = smallest / largest step, beta1 != 0 when the loss got worse),
+//       8 iRPROP- (NN/Neural_Network__iRPROP_minus.cpp:21-67; b, c and the scalars as for iRPROP+; a slope that changed sign
+//         is forgotten and, the sign of zero being zero, leaves the weight where it is).
 template <int KIND, bool WD>
 __device__ __forceinline__ void update_one(const UpdateDev &p, float gs, float &w, float g, float &a, float &b, float &c, bool is_weight)
 {
     g *= gs;
     float step;
+    if (KIND == 8) {
+        const float same = c * g;
+        float d = b;
+        if (same > 0.f) b = d = fminf(b * p.lr, p.upper);
+        else if (same < 0.f) { b = d = fmaxf(b * p.mu, p.lower); g = 0.f; }
+        w += -(g > 0.f ? 1.f : (g < 0.f ? -1.f : 0.f)) * d;
+        c = g;
+        return;
+    }
     if (KIND == 7) {
         const float sg = g > 0.f ? 1.f : (g < 0.f ? -1.f : 0.f), same = c * g;
         if (same > 0.f) {
@@ -799,12 +812,16 @@ __device__ __forceinline__ void update_one(const UpdateDev &p, float gs, float &
 template <int KIND, bool WD>
 __global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
 {
+    // A kernel of an earlier pass whose bounded wait gave up has left that pass incomplete and raised this word: the
+    // update then changes nothing (weights, optimizer vectors and gradient stay as they are) until the host has dealt with it.
+    if (p.fault && __hip_atomic_load(p.fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return;
+    if (p.applied && blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(p.applied, 1ull);   // the launch that completes a whole update counts it
     float gs = p.grad_scale;
     if (p.norm_sq) {  // Clip_Gradient: scale when norm >= clip (NN/Neural_Network__Clip_Gradient.cpp:81-94)
         const float norm = sqrtf(p.norm_sq[0]);
         if (norm >= p.clip) gs = p.clip / norm;
     }
-    constexpr bool kA = KIND >= 1, kB = KIND >= 3, kC = KIND == 4 || KIND >= 6;
+    constexpr bool kA = KIND >= 1 && KIND != 8, kB = KIND >= 3, kC = KIND == 4 || KIND >= 6;
     const size_t n4 = p.n / 4;
     f32x4 *w4 = reinterpret_cast<f32x4 *>(p.w), *g4 = reinterpret_cast<f32x4 *>(p.g);
     f32x4 *a4 = reinterpret_cast<f32x4 *>(p.s0), *b4 = reinterpret_cast<f32x4 *>(p.s1), *c4 = reinterpret_cast<f32x4 *>(p.s2);
@@ -884,7 +901,7 @@ __global__ __launch_bounds__(kBlock) void max_norm_kernel(size_t nseg, const uns
 template <int KIND>
 int launch_update_kind(hipStream_t s, const UpdateDev &d, bool wd)
 {
-    const unsigned grid = grid_for(d.n / 4 + 1, kBlock, 0x7fffffffu);
+    const unsigned grid = grid_for(d.n / 4 + 1, kBlock, 0x7fffffffu);   // at least one workgroup, also for an empty range that only counts
     if (wd) hipLaunchKernelGGL((update_kernel<KIND, true>), dim3(grid), dim3(kBlock), 0, s, d);
     else hipLaunchKernelGGL((update_kernel<KIND, false>), dim3(grid), dim3(kBlock), 0, s, d);
     MYEA_HIP_TRY(hipGetLastError());
@@ -1323,13 +1340,14 @@ int launch_max_norm(hipStream_t s, size_t nseg, const unsigned long long *first,
 
 int launch_update(hipStream_t s, const UpdateParams &p)
 {
-    if (p.n == 0) return MYEA_OK;
+    if (p.n == 0 && !p.applied) return MYEA_OK;
     UpdateDev d;
     d.n = p.n; d.n_weights = p.n_weights;
     d.w = p.w; d.g = p.g; d.s0 = p.s0; d.s1 = p.s1; d.s2 = p.s2;
     d.lr = p.lr; d.mu = p.mu; d.lr_t = p.lr_t; d.beta1 = p.beta1; d.beta2 = p.beta2; d.eps = p.eps;
     d.lower = p.lower; d.upper = p.upper; d.wd = p.wd;
     d.norm_sq = p.norm_sq; d.clip = p.clip; d.grad_scale = p.grad_scale;
+    d.fault = p.fault; d.applied = p.applied;
     const bool wd = p.wd != 0.f;
     auto need = [&](float *ptr, const char *name) { if (!ptr) { set_last_error("optimizer update: %s state is null", name); return false; } return true; };
     // the vector path needs 16-byte aligned bases
@@ -1358,6 +1376,9 @@ int launch_update(hipStream_t s, const UpdateParams &p)
     case MYEA_OPTIMIZER_IRPROP_PLUS:
         if (!need(p.s0, "previous delta") || !need(p.s1, "previous steps") || !need(p.s2, "previous slopes")) return MYEA_E_INVALID;
         return launch_update_kind<7>(s, d, false);
+    case MYEA_OPTIMIZER_IRPROP_MINUS:
+        if (!need(p.s1, "previous steps") || !need(p.s2, "previous slopes")) return MYEA_E_INVALID;
+        return launch_update_kind<8>(s, d, false);
     default:
         set_last_error("optimizer %d is not on this path", p.optimizer);
         return MYEA_E_UNSUPPORTED;

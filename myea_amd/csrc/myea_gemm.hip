@@ -269,6 +269,8 @@ struct GemmDev {
     long slab;
     float *pair_partials;    // not null: ksplit == 2 and the two workgroups of a tile combine their halves in the launch
     unsigned *pair_tickets;
+    unsigned *pair_fault, *pair_host_flag;   // raised when the wait for the tile's other half runs out of polls
+    unsigned pair_polls;
 };
 
 struct TilePlace {
@@ -529,15 +531,32 @@ __device__ __forceinline__ void gemm_tile(const GemmDev &p, const int block, flo
                         __hip_atomic_store(partial + ((i * TN + j) * 16 + r) * kThreads + threadIdx.x, acc[i][j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's stores are complete
             __syncthreads();
-            if (threadIdx.x == 0) __hip_atomic_store(flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (threadIdx.x == 0) __hip_atomic_store(flag, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);   // publishes the tile stored above
             return;
         }
+        // The wait is bounded.  When it runs out the other half is not there to add: this workgroup raises the network's fault
+        // words (a device word the update kernels look at, a pinned host word the next call that looks reports) and leaves
+        // without storing its tile.  Ticket and flag stay as they are - a late partner still raises its flag - and the host
+        // clears both before these buffers serve another launch.
+        __shared__ unsigned s_there;
         if (threadIdx.x == 0) {
-            for (unsigned polls = 0; polls < (1u << 24) && __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u; ++polls) __builtin_amdgcn_s_sleep(1);
-            __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects them
-            __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned there = 0u;
+            for (unsigned polls = 0; polls < p.pair_polls; ++polls) {
+                there = __hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+                if (there != 0u) break;
+                __builtin_amdgcn_s_sleep(1);
+            }
+            if (there != 0u) {
+                __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // as the next launch expects them
+                __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                if (p.pair_fault) __hip_atomic_store(p.pair_fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (p.pair_host_flag) __hip_atomic_store(p.pair_host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+            s_there = there;
         }
         __syncthreads();
+        if (s_there == 0u) return;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -648,6 +667,13 @@ int gemm_split_k(int M, int N, int K)
     return (K + chunk - 1) / chunk;
 }
 
+unsigned gemm_pair_polls()
+{
+    const char *e = std::getenv("MYEA_GEMM_PAIR_SPIN_POLLS");
+    if (e && *e) { const unsigned long long v = std::strtoull(e, nullptr, 10); return v > 0xffffffffull ? 0xffffffffu : (unsigned)v; }
+    return 1u << 24;
+}
+
 bool gemm_pair_k_128(int M, int N, int K)
 {
     const long tiles_128 = (long)((M + 127) / 128) * ((N + 127) / 128);
@@ -686,6 +712,7 @@ static int prepare_gemm(const GemmParams &p, GemmDev &d, bool *vec)
     d.nbm = d.nbn = 0;
     d.ksplit = 1; d.kchunk = p.K > 0 ? p.K : 1; d.slab = 0;
     d.pair_partials = nullptr; d.pair_tickets = nullptr;
+    d.pair_fault = p.pair_fault; d.pair_host_flag = p.pair_host_flag; d.pair_polls = p.pair_polls;
     if (p.split_k > 1) {
         if (p.epilogue != EPI_NONE || p.accumulate || p.addend) { set_last_error("gemm: split-K writes plain partial slabs"); return MYEA_E_INVALID; }
         const int chunk = ((p.K + p.split_k - 1) / p.split_k + kBK - 1) / kBK * kBK;

@@ -65,10 +65,18 @@ struct GemmParams {
     // leaves them zero).  One launch at a time may use a given pair of buffers.  Null = off; the launcher decides per problem.
     float *pair_partials;
     unsigned *pair_tickets;
+    // The second workgroup's wait for the first one's half is bounded by pair_polls polls (gemm_pair_polls()).  When they run out
+    // it stores nothing and raises *pair_fault (device memory) and *pair_host_flag (pinned host memory), either may be null; the
+    // product is then incomplete, ticket and flag words are left as they are and must be cleared before the buffers' next use.
+    unsigned *pair_fault, *pair_host_flag;
+    unsigned pair_polls;
 };
 constexpr int kGemmPairTiles = 256;   // tiles the two buffers above serve
 
 int gemm_split_k(int M, int N, int K);
+// polls a tile's second workgroup waits for the first: 2^24 (seconds), or MYEA_GEMM_PAIR_SPIN_POLLS (0: give up at once, for tests
+// of that path; read at every call)
+unsigned gemm_pair_polls();
 // true when launch_gemm, handed pair_partials / pair_tickets, would share every 128 x 128 tile's k between two workgroups
 // (at most one such tile per compute unit, a k worth halving): callers size their pair buffers by it
 bool gemm_pair_k_128(int M, int N, int K);
@@ -207,6 +215,8 @@ struct UpdateParams {
     const float *norm_sq;  // device scalar: sum of squares of g, or null (no clipping)
     float clip;
     float grad_scale;      // host-side multiplier (used when norm_sq is null)
+    const unsigned *fault;          // device word or null: while it is not 0 the launch changes nothing
+    unsigned long long *applied;    // device counter or null: incremented by a launch that found `fault` clear
 };
 int launch_update(hipStream_t s, const UpdateParams &p);
 // every segment w[first[i] .. first[i] + len[i]) whose Euclidean norm is >= max_norm is scaled onto that norm;
@@ -287,13 +297,14 @@ struct LstmResidentPlan {
 int lstm_resident_plan(size_t C, size_t cells_per_block, size_t B, int dirs, LstmResidentPlan *plan);
 size_t lstm_resident_sync_words();
 // sync: lstm_resident_sync_words() unsigneds of device memory (cleared by the call); host_flag: a pinned host word the
-// kernel sets when a bounded wait gave up (1) or the members of a group did not share an XCD (2)
+// kernel sets when a bounded wait gave up (1) or the members of a group did not share an XCD (2); fault: a device word set
+// to 1 on the same occasions and never cleared by these calls (null: none)
 int launch_lstm_resident_forward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
-                                 const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag);
+                                 const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, unsigned *fault);
 // dh must hold the delta from the layers above for every time step.  exchange: device memory of at least
 // lstm_resident_exchange_floats(C, B, dirs) floats, 16-byte aligned, when plan.ksplit (its contents do not matter); else unused
 size_t lstm_resident_exchange_floats(size_t C, size_t B, int dirs);
 int launch_lstm_resident_backward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
-                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, float *exchange, size_t exchange_floats);
+                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, unsigned *fault, float *exchange, size_t exchange_floats);
 
 }  // namespace myea

@@ -755,6 +755,14 @@ void Net::lstm_bind_gradient_slabs(float *base)
         }
 }
 
+int Net::lstm_pair_words_clear()
+{
+    for (size_t li = 1; li < L.size(); ++li)
+        for (LstmLayer *q : {L[li].lstm, L[li].lstm2})
+            if (q && q->pair_tickets) MYEA_HIP_TRY(hipMemset(q->pair_tickets, 0, 2 * kGemmPairTiles * sizeof(unsigned)));
+    return MYEA_OK;
+}
+
 // packed copies <- flat vector; called after every parameter upload and every optimizer update
 int Net::lstm_parameters_changed()
 {
@@ -1011,7 +1019,7 @@ int Net::lstm_forward_layer(size_t li, size_t B)
             LstmResidentDir rd[2];
             lstm_resident_dirs(o, rd);
             prof_begin(kProfLstmForwardLoop);
-            MYEA_TRY(launch_lstm_resident_forward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag));
+            MYEA_TRY(launch_lstm_resident_forward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag, fault));
             prof_end(dirs * loop_work, 1);
             if (!o.lstm2) return MYEA_OK;
             const size_t rows = (size_t)d.number_recurrent_depth * d.batch_size;
@@ -1118,7 +1126,7 @@ int Net::lstm_backward_layer(size_t li, size_t B)
             LstmResidentDir rd[2];
             lstm_resident_dirs(o, rd);
             prof_begin(kProfLstmBackwardLoop);
-            MYEA_TRY(launch_lstm_resident_backward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag, resident_exchange, resident_exchange_floats));
+            MYEA_TRY(launch_lstm_resident_backward(stream, plan, T, B, d.batch_size, o.lstm->C, dirs, rd, resident_sync, resident_flag, fault, resident_exchange, resident_exchange_floats));
             prof_end(dirs * loop_work, 1);
             for (LstmLayer *q : {o.lstm, o.lstm2})
                 if (q && q->sums) { q->sums_groups = (size_t)plan.row_groups; q->sums_batch = B; }
@@ -1231,7 +1239,7 @@ int Net::lstm_update_derivative_weight_direction(size_t li, LstmLayer &q, size_t
         g.M = (int)q.G; g.N = (int)q.C; g.K = (int)rows;
         s_rec = gemm_split_k(g.M, g.N, g.K);
         g.split_k = s_rec; g.split_k_slab = (long)(q.G * q.C);
-        if (q.pair_partials && s_rec == 1) { g.pair_partials = q.pair_partials; g.pair_tickets = reinterpret_cast<unsigned *>(q.pair_tickets); }
+        if (q.pair_partials && s_rec == 1) pair_buffers(&g, q.pair_partials, reinterpret_cast<unsigned *>(q.pair_tickets));
         prof_begin(2);
         MYEA_TRY(launch_gemm(stream, g));
         prof_end(2.0 * (double)rows * (double)q.G * (double)q.C);

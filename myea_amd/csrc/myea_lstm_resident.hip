@@ -124,6 +124,7 @@ struct SyncWords {
     unsigned *counters;   // [(group * 2 + chain) * kSyncStride]
     unsigned *give_up;    // device flag, polled; behind it one word per group: the XCC id its first member ran on (+ 1)
     unsigned *host_flag;  // pinned host word, written once on give-up
+    unsigned *fault;      // device word the launch never clears, written on give-up like the two above (a scrap word when the caller has none)
     float *scrap;         // kScrapWords floats nobody reads
     float *exchange;      // backward, split along k: per group 2 chains x 2 buffers x members^2 tiles of 1 KiB
 };
@@ -177,13 +178,14 @@ __device__ __forceinline__ int wave_wait(const SyncWords &w, unsigned *counter, 
             "v_mov_b32 %[value], 1\n\t"
             "global_store_dword %[give_up], %[value], off sc1\n\t"
             "global_store_dword %[host_flag], %[value], off sc0 sc1\n\t"
+            "global_store_dword %[fault], %[value], off sc1\n\t"
             "s_waitcnt vmcnt(0)\n\t"
             "s_branch 3f\n"
             "2:\n\t"
             "v_mov_b32 %[ok], 1\n"
             "3:\n"
             : [ok] "=&v"(ok), [value] "=&v"(value), [polls] "+s"(polls)
-            : [counter] "v"(counter), [give_up] "v"(w.give_up), [host_flag] "v"(w.host_flag), [target] "v"(target)
+            : [counter] "v"(counter), [give_up] "v"(w.give_up), [host_flag] "v"(w.host_flag), [fault] "v"(w.fault), [target] "v"(target)
             : "vcc", "scc", "memory");
     }
     return __builtin_amdgcn_readfirstlane(ok);
@@ -225,6 +227,7 @@ __device__ __forceinline__ void check_same_xcd(const SyncWords &w, int group)
     if (!__hip_atomic_compare_exchange_strong(word, &seen, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT) && seen != mine) {
         __hip_atomic_store(w.give_up, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
         __hip_atomic_store(w.host_flag, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(w.fault, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
     }
 }
 
@@ -1384,7 +1387,7 @@ int fill_geometry(const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax,
 }
 
 // clears the counters and flags and lays the words out
-int prepare_sync(hipStream_t s, const LstmResidentPlan &plan, int dirs, unsigned *sync, unsigned *host_flag, SyncWords *w)
+int prepare_sync(hipStream_t s, const LstmResidentPlan &plan, int dirs, unsigned *sync, unsigned *host_flag, unsigned *fault, SyncWords *w)
 {
     w->exchange = nullptr;
     const int groups = plan.row_groups * dirs;
@@ -1396,6 +1399,7 @@ int prepare_sync(hipStream_t s, const LstmResidentPlan &plan, int dirs, unsigned
     w->give_up = sync + (size_t)groups * 2 * kSyncStride;
     w->host_flag = host_flag;
     w->scrap = reinterpret_cast<float *>(sync + (size_t)kMaxGroups * 2 * kSyncStride + 1 + kMaxGroups);
+    w->fault = fault ? fault : reinterpret_cast<unsigned *>(w->scrap);
     return MYEA_OK;
 }
 
@@ -1411,7 +1415,7 @@ int check_dirs(const LstmResidentDir *dir, int dirs, bool backward)
 }
 
 int launch_resident(hipStream_t s, bool backward, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
-                    const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, float *exchange = nullptr, size_t exchange_floats = 0)
+                    const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, unsigned *fault, float *exchange = nullptr, size_t exchange_floats = 0)
 {
     const bool ksplit = backward && plan.ksplit;
     ResidentGeometry g;
@@ -1438,7 +1442,7 @@ int launch_resident(hipStream_t s, bool backward, const LstmResidentPlan &plan, 
         set_last_error("resident LSTM: the plan does not fit the device (C = %zu, %d groups)", C, plan.row_groups * dirs);
         return MYEA_E_UNSUPPORTED;
     }
-    rc = prepare_sync(s, plan, dirs, sync, host_flag, &w);
+    rc = prepare_sync(s, plan, dirs, sync, host_flag, fault, &w);
     if (rc != MYEA_OK) return rc;
     w.exchange = ksplit ? exchange : nullptr;
     hipLaunchKernelGGL(k->fn, dim3((unsigned)plan.grid), dim3(kThreads), k->lds, s, g, dir[0], dir[dirs > 1 ? 1 : 0], w);
@@ -1500,15 +1504,15 @@ size_t lstm_resident_sync_words() { return (size_t)kMaxGroups * 2 * kSyncStride 
 
 // sync: lstm_resident_sync_words() unsigneds of device memory (cleared by the call); host_flag: one pinned host word (0 = fine)
 int launch_lstm_resident_forward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
-                                 const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag)
+                                 const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, unsigned *fault)
 {
-    return launch_resident(s, false, plan, T, B, Bmax, C, dirs, dir, sync, host_flag);
+    return launch_resident(s, false, plan, T, B, Bmax, C, dirs, dir, sync, host_flag, fault);
 }
 
 int launch_lstm_resident_backward(hipStream_t s, const LstmResidentPlan &plan, size_t T, size_t B, size_t Bmax, size_t C, int dirs,
-                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, float *exchange, size_t exchange_floats)
+                                  const LstmResidentDir *dir, unsigned *sync, unsigned *host_flag, unsigned *fault, float *exchange, size_t exchange_floats)
 {
-    return launch_resident(s, true, plan, T, B, Bmax, C, dirs, dir, sync, host_flag, exchange, exchange_floats);
+    return launch_resident(s, true, plan, T, B, Bmax, C, dirs, dir, sync, host_flag, fault, exchange, exchange_floats);
 }
 
 }  // namespace myea

@@ -53,8 +53,8 @@ struct DevLayer {
     LstmLayer *lstm = nullptr, *lstm2 = nullptr;  // lstm2: the time-reversed direction of a bidirectional layer
 };
 
-constexpr int kProfFamilies = 9;   // forward, dX, dW, update, dX + dW launched as a pair, LSTM time loop forward, backward, normalisation, bias gradients
-constexpr int kProfLstmForwardLoop = 5, kProfLstmBackwardLoop = 6, kProfNormalization = 7, kProfBiasGradient = 8;
+constexpr int kProfFamilies = 11;   // forward, dX, dW, update, dX + dW launched as a pair, LSTM time loop forward, backward, normalisation, bias gradients, output error, softmax
+constexpr int kProfLstmForwardLoop = 5, kProfLstmBackwardLoop = 6, kProfNormalization = 7, kProfBiasGradient = 8, kProfOutputError = 9, kProfSoftmax = 10;
 struct ProfEvent {
     hipEvent_t start = nullptr, stop = nullptr;
     int family = 0;
@@ -100,6 +100,18 @@ struct Net {
     // LSTM time loops as one resident launch (myea_lstm_resident.hip): barrier counters in device memory, and a pinned host
     // word a kernel sets when one of its bounded waits gave up; resident_off: this network stays on one launch per time step
     unsigned *resident_sync = nullptr, *resident_flag = nullptr;
+    // Bounded waits inside kernels (the time loops' barriers, the meeting of two workgroups that share a contraction's tile):
+    // one that gives up raises resident_flag[0] (time loop) or resident_flag[1] (contraction) in pinned host memory and
+    // `fault` in device memory.  While `fault` is set the update kernels change nothing, so no Update_Parameter enqueued behind
+    // the incomplete pass steps the weights; the host word is reported by the next call that looks (resident_check()).
+    unsigned *fault = nullptr;
+    unsigned long long *updates_applied = nullptr;   // device counter: whole-vector updates that ran with `fault` clear
+    // the optimizer's host-side scalars as they were before each update enqueued and not yet known to have run
+    struct UpdateSnapshot { unsigned long long sequence; myea_hyper h; };
+    std::vector<UpdateSnapshot> update_history;
+    unsigned long long updates_enqueued = 0;
+    bool gemm_pair_off = false;            // after a contraction's give-up: one workgroup per tile from then on
+    void pair_buffers(GemmParams *g, float *partials, unsigned *tickets) const;   // a contraction's meeting place and fault words
     float *gemm_pair_partials = nullptr;       // scratch of the contractions that split a tile's k between two workgroups
     unsigned *gemm_pair_tickets = nullptr;
     float *resident_exchange = nullptr;   // partial sums the members of a group hand each other in the backward loop
@@ -169,7 +181,7 @@ struct Net {
     // Update_Parameter in three parts: the step's scalars (advances the optimizer's time step), the elementwise update of a
     // range of the flat vectors, and what follows the update (constraints, repacking)
     int update_prepare(size_t B, size_t training_size, UpdateParams *p, double *bytes_per_param);
-    int update_range(const UpdateParams &p, size_t first, size_t count, double bytes_per_param);
+    int update_range(const UpdateParams &p, size_t first, size_t count, double bytes_per_param, bool last);   // last: the range that completes the update
     int update_finish();
     // Backward_Pass, Update_Derivative_Weight over all layers and Update_Parameter as one call: the weights of a
     // fully-connected layer take their step on the side stream as soon as their gradient is complete and nothing reads them
@@ -186,6 +198,7 @@ struct Net {
     int lstm_create_layer(size_t li);
     void lstm_destroy_layer(DevLayer &o);
     int lstm_parameters_changed();
+    int lstm_pair_words_clear();   // the meeting words of the LSTM layers' shared-tile contractions back to zero
     int lstm_forward_layer(size_t li, size_t B);
     int lstm_backward_layer(size_t li, size_t B);       // BPTT inside LSTM layer li
     // delta / weight operands an LSTM consumer gi offers to the layer below: delta [T][Bmax][width], weights [width][fan-in]

@@ -349,6 +349,15 @@ int Net::create(const myea_net_desc &desc)
         MYEA_HIP_TRY(hipMalloc(&q, 2 * kGemmPairTiles * sizeof(unsigned)));
         MYEA_HIP_TRY(hipMemset(q, 0, 2 * kGemmPairTiles * sizeof(unsigned)));
         gemm_pair_tickets = static_cast<unsigned *>(q);
+        // what a kernel's bounded wait raises when it gives up: a device word the update kernels look at (behind it, 8 bytes on,
+        // the count of updates that ran) and two pinned host words the next call that looks reports
+        MYEA_HIP_TRY(hipMalloc(&q, 16));
+        MYEA_HIP_TRY(hipMemset(q, 0, 16));
+        fault = static_cast<unsigned *>(q);
+        updates_applied = reinterpret_cast<unsigned long long *>(fault + 2);
+        MYEA_HIP_TRY(hipHostMalloc(&q, 64, hipHostMallocDefault));
+        resident_flag = static_cast<unsigned *>(q);
+        resident_flag[0] = resident_flag[1] = 0u;
     }
     {
         bool any_lstm = false;
@@ -357,9 +366,6 @@ int Net::create(const myea_net_desc &desc)
             void *q = nullptr;
             MYEA_HIP_TRY(hipMalloc(&q, lstm_resident_sync_words() * sizeof(unsigned)));
             resident_sync = static_cast<unsigned *>(q);
-            MYEA_HIP_TRY(hipHostMalloc(&q, 64, hipHostMallocDefault));
-            resident_flag = static_cast<unsigned *>(q);
-            *resident_flag = 0u;
             if (resident_exchange_floats) MYEA_TRY(dev_alloc(&resident_exchange, resident_exchange_floats));
         }
     }
@@ -417,7 +423,7 @@ Net::~Net()
     }
     fr(resident_sync);
     fr(resident_exchange);
-    fr(gemm_pair_partials); fr(gemm_pair_tickets);
+    fr(gemm_pair_partials); fr(gemm_pair_tickets); fr(fault);
     if (resident_flag) (void)hipHostFree(resident_flag);
     fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc); fr(index_stage); fr(dw_slabs);
     for (ProfEvent &e : pending) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
@@ -492,7 +498,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
         // a batch normalisation in front of the activation, training: its column sums leave with the contraction's tiles
         const bool sums_from_gemm = norm && before && training && o.norm_partials && bn_sums_from_gemm() && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H;
         if (sums_from_gemm) g.col_partials = o.norm_partials;
-        g.pair_partials = gemm_pair_partials; g.pair_tickets = gemm_pair_tickets;   // forward contractions run one at a time on this stream
+        pair_buffers(&g, gemm_pair_partials, gemm_pair_tickets);   // forward contractions run one at a time on this stream
         prof_begin(0);
         MYEA_TRY(launch_gemm(stream, g));
         prof_end(2.0 * (double)rows * (double)H * (double)In);
@@ -505,7 +511,11 @@ int Net::forward_fc_layer(size_t li, size_t B)
             cur = o.normalizes + roff * H;
         }
         if (ind) continue;   // the recurrence and the activation follow for the whole sequence
-        if (softmax) MYEA_TRY(launch_softmax(stream, rows, H, cur, o.values + roff * H, norm ? nullptr : cs));
+        if (softmax) {
+            prof_begin(kProfSoftmax);
+            MYEA_TRY(launch_softmax(stream, rows, H, cur, o.values + roff * H, norm ? nullptr : cs));
+            prof_end((double)rows * (double)H * sizeof(float) * 2.0);   // sums read once, values written once
+        }
         else if (!fuse_af && !af_in_bn) MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, rows, H, cur, o.values + roff * H, cs, o.unit_act));
         if (norm && !before) {
             MYEA_TRY(bn_forward(li, c, rows, o.values + roff * H, training));
@@ -575,17 +585,57 @@ int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool train
     return rc;
 }
 
-// A resident LSTM launch whose bounded wait gave up has left the pass it belonged to incomplete.  Reported once, at the
-// next call that looks; the network then keeps to one launch per time step.
+// A kernel whose bounded wait gave up - a resident LSTM time loop, or a contraction whose tiles two workgroups share - has left
+// the pass it belonged to incomplete.  From that kernel on the device-side fault word is set and every update kernel behind
+// it has changed nothing.  The next call that looks reports it, once: everything enqueued runs to its end, the host-side
+// optimizer scalars go back to what they were before the first update that did not run, the gradient is cleared, the fault
+// words and the contractions' meeting words are reset, and the network keeps to the plain forms (one launch per time step,
+// one workgroup per tile) from then on.  The caller repeats the mini-batch.
 int Net::resident_check()
 {
-    if (!resident_flag || *resident_flag == 0u) return MYEA_OK;
-    const unsigned code = *resident_flag;
-    *resident_flag = 0u;
-    resident_off = true;
-    set_last_error(code == 2u ? "resident LSTM time loop: the workgroups of a group did not share an XCD; the pass is incomplete, later passes use one launch per time step"
-                              : "resident LSTM time loop: a wait between time steps gave up (workgroups not resident together?); the pass is incomplete, later passes use one launch per time step");
+    if (!resident_flag || (resident_flag[0] == 0u && resident_flag[1] == 0u)) return MYEA_OK;
+    MYEA_HIP_TRY(hipStreamSynchronize(stream));
+    if (side_stream) MYEA_HIP_TRY(hipStreamSynchronize(side_stream));
+    const unsigned loop_code = resident_flag[0], pair_code = resident_flag[1];
+    resident_flag[0] = resident_flag[1] = 0u;
+    if (loop_code) resident_off = true;
+    if (pair_code) gemm_pair_off = true;
+    unsigned long long applied = 0;
+    MYEA_HIP_TRY(hipMemcpy(&applied, updates_applied, sizeof(applied), hipMemcpyDeviceToHost));
+    bool rolled_back = applied == updates_enqueued;
+    for (const UpdateSnapshot &snap : update_history) {
+        if (snap.sequence != applied) continue;
+        // the scalars an update advances (update_prepare, warm_restarts_decay, clear_optimizer); what the caller set stays
+        h.optimizer_time_step = snap.h.optimizer_time_step; h.adam_previous_beta2 = snap.h.adam_previous_beta2;
+        h.epoch_time_step = snap.h.epoch_time_step; h.warm_restarts_T_i = snap.h.warm_restarts_T_i;
+        h.warm_restarts_maximum_learning_rate = snap.h.warm_restarts_maximum_learning_rate;
+        h.loss_rprop = snap.h.loss_rprop; h.previous_loss_rprop = snap.h.previous_loss_rprop;
+        rolled_back = true;
+        break;
+    }
+    const unsigned long long skipped = updates_enqueued - applied;
+    updates_enqueued = applied;
+    update_history.clear();
+    MYEA_HIP_TRY(hipMemset(fault, 0, sizeof(unsigned)));
+    MYEA_HIP_TRY(hipMemset(gemm_pair_tickets, 0, 2 * kGemmPairTiles * sizeof(unsigned)));
+    MYEA_HIP_TRY(hipMemset(gradient, 0, d.total_parameters * sizeof(float)));
+    gradient_known_zero(true);
+    MYEA_TRY(lstm_pair_words_clear());
+    const char *what = loop_code == 2u ? "resident LSTM time loop: the workgroups of a group did not share an XCD"
+                       : loop_code    ? "resident LSTM time loop: a wait between time steps gave up (workgroups not resident together?)"
+                                      : "contraction with tiles shared by two workgroups: the wait for a tile's other half gave up";
+    set_last_error("%s; the pass is incomplete, %llu update(s) enqueued behind it changed nothing%s, the gradient is cleared; later passes use %s",
+                   what, skipped, rolled_back ? "" : " (the optimizer's time step could not be taken back)",
+                   loop_code ? "one launch per time step" : "one workgroup per tile");
     return MYEA_E_DEVICE;
+}
+
+void Net::pair_buffers(GemmParams *g, float *partials, unsigned *tickets) const
+{
+    if (gemm_pair_off) return;
+    g->pair_partials = partials; g->pair_tickets = tickets;
+    g->pair_fault = fault; g->pair_host_flag = resident_flag ? resident_flag + 1 : nullptr;
+    g->pair_polls = gemm_pair_polls();
 }
 
 // FF__Forward_Pass_Batch (NN/Neural_Network__Forward_Pass__OpenMP.cpp:24-120) / RNN__Forward_Pass_Batch
@@ -774,7 +824,11 @@ int Net::compute_error(size_t B, const float *desired, int on_device)
 {
     ErrorParams p;
     MYEA_TRY(output_error_params(B, desired, on_device, "Compute__Error", &p));
-    return launch_compute_error(stream, p);
+    // algorithmic bytes: the outputs and the desired values read once, the delta written once
+    prof_begin(kProfOutputError);
+    const int rc = launch_compute_error(stream, p);
+    prof_end((double)B * (double)p.T * (double)p.H * sizeof(float) * 3.0);
+    return rc;
 }
 
 // Compute__Loss (NN/Neural_Network__Compute__Loss__Loop.cpp:22-140): loss and accuracy of the values the last forward pass left
@@ -1175,7 +1229,7 @@ int Net::update_derivative_weight_contraction(size_t li, size_t B)
         g.accumulate = 1; g.c_is_zero = dw_may_store(li) ? 1 : 0; g.epilogue = EPI_NONE;
         const int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
         if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.c_is_zero = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
-        else if (li < dw_zero.size()) dw_zero[li] = 0;   // from here on the slice holds this product
+        if (li < dw_zero.size()) dw_zero[li] = 0;   // from here on the slice holds this product, stored or added from the slabs
         prof_begin(2);
         MYEA_TRY(launch_gemm(stream, g));
         if (slabs > 1) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
@@ -1440,11 +1494,15 @@ int Net::update_prepare(size_t B, size_t training_size, UpdateParams *out, doubl
         set_last_error("Update_Parameter: normalized weight decay needs the training-set size");
         return MYEA_E_INVALID;
     }
+    // the scalars as they are before this update, until it is known to have run (resident_check)
+    if (update_history.size() >= 1024) update_history.erase(update_history.begin(), update_history.begin() + 512);
+    update_history.push_back(UpdateSnapshot{updates_enqueued++, h});
     UpdateParams p{};
     p.optimizer = (int)kind;
     p.n = d.total_parameters; p.n_weights = d.total_weights;
     p.w = parameters; p.g = gradient;
     p.grad_scale = 1.f;
+    p.fault = fault;
     if (h.use_clip_gradient) { p.norm_sq = scratch; p.clip = h.clip_gradient; }   // the caller leaves the gradient's sum of squares there
     const bool rprop = kind == MYEA_OPTIMIZER_IRPROP_PLUS, gd = kind == MYEA_OPTIMIZER_GD;
     float scale = 1.f;
@@ -1497,10 +1555,11 @@ int Net::update_prepare(size_t B, size_t training_size, UpdateParams *out, doubl
 }
 
 // the elementwise update of [first, first + count) of the flat vectors; first a multiple of 4 (the kernels move 16 bytes per lane)
-int Net::update_range(const UpdateParams &whole, size_t first, size_t count, double bytes_per_param)
+int Net::update_range(const UpdateParams &whole, size_t first, size_t count, double bytes_per_param, bool last)
 {
-    if (count == 0) return MYEA_OK;
+    if (count == 0 && !last) return MYEA_OK;
     UpdateParams p = whole;
+    p.applied = last ? updates_applied : nullptr;   // the range that completes the update counts it
     p.n = count;
     p.n_weights = whole.n_weights > first ? std::min(count, whole.n_weights - first) : 0;
     p.w += first; p.g += first;
@@ -1537,7 +1596,7 @@ int Net::update_parameter(size_t B, size_t training_size)
     double bytes_per_param = 0;
     MYEA_TRY(update_prepare(B, training_size, &p, &bytes_per_param));
     if (h.use_clip_gradient) MYEA_TRY(launch_sum_squares(stream, p.n, gradient, scratch + 16, scratch));
-    MYEA_TRY(update_range(p, 0, p.n, bytes_per_param));
+    MYEA_TRY(update_range(p, 0, p.n, bytes_per_param, true));
     return update_finish();
 }
 
@@ -1547,7 +1606,9 @@ int Net::update_parameter(size_t B, size_t training_size)
 bool Net::early_update_allowed() const
 {
     static const bool off = [] { const char *e = std::getenv("MYEA_EARLY_UPDATE"); return e && e[0] == '0'; }();
-    return !off && side_stream && !h.use_clip_gradient && h.type_optimizer_function != MYEA_OPTIMIZER_IRPROP_PLUS;
+    // ... and no resident time loop in the pass: one that gives up after a layer above it has taken its step would leave the
+    // network half updated; without LSTM layers only a forward contraction can give up, before any update of its step
+    return !off && side_stream && !resident_sync && !h.use_clip_gradient && h.type_optimizer_function != MYEA_OPTIMIZER_IRPROP_PLUS;
 }
 
 // The weights of fully-connected layer li: gradient complete, no reader left in this pass.  Their update goes to the side
@@ -1566,7 +1627,7 @@ int Net::early_update_layer(size_t li)
     MYEA_HIP_TRY(hipEventRecord(update_event, stream));
     MYEA_HIP_TRY(hipStreamWaitEvent(side_stream, update_event, 0));
     std::swap(stream, side_stream);
-    const int rc = update_range(*early_update, first, count, early_bytes_per_param);
+    const int rc = update_range(*early_update, first, count, early_bytes_per_param, false);
     std::swap(stream, side_stream);
     MYEA_TRY(rc);
     early_ranges.emplace_back(first, first + count);
@@ -1598,10 +1659,10 @@ int Net::backward_pass_update_derivative_weight_and_update_parameter(size_t B, s
     std::sort(early_ranges.begin(), early_ranges.end());
     size_t at = 0;
     for (const auto &r : early_ranges) {
-        MYEA_TRY(update_range(p, at, r.first - at, early_bytes_per_param));
+        MYEA_TRY(update_range(p, at, r.first - at, early_bytes_per_param, false));
         at = r.second;
     }
-    MYEA_TRY(update_range(p, at, p.n - at, early_bytes_per_param));
+    MYEA_TRY(update_range(p, at, p.n - at, early_bytes_per_param, true));
     early_ranges.clear();
     return update_finish();
 }
@@ -1930,6 +1991,12 @@ int myea_hip_optimizer_update(void *stream, const myea_hyper *h, size_t count, s
     p.lr_t = h->use_adam_bias_correction ? h->adam_learning_rate * std::sqrt(1.f - std::pow(h->adam_beta2, ts)) / (1.f - std::pow(h->adam_beta1, ts)) : h->adam_learning_rate;
     p.lower = h->learning_rate_final * (1.f - 1.f / (h->learning_gamma * ts + 1.f));
     p.upper = h->learning_rate_final * (1.f + 1.f / (h->learning_gamma * ts));
+    if (p.optimizer == MYEA_OPTIMIZER_IRPROP_PLUS || p.optimizer == MYEA_OPTIMIZER_IRPROP_MINUS) {   // as Net::update_prepare hands them over
+        p.lr = h->rprop_increase_factor; p.mu = h->rprop_decrease_factor;
+        p.lower = h->rprop_delta_min; p.upper = h->rprop_delta_max;
+        p.beta1 = h->loss_rprop > h->previous_loss_rprop ? 1.f : 0.f;
+        p.wd = 0.f;
+    }
     return myea::launch_update(static_cast<hipStream_t>(stream), p);
 }
 

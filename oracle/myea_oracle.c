@@ -1944,6 +1944,29 @@ int myea_oracle_update_derivative_weight(myea_oracle_net *n, size_t B, size_t fi
     return MYEA_OK;
 }
 
+/* Update_Parameter__iRPROP_minus__Loop: NN/Neural_Network__iRPROP_minus.cpp:21-67.  Same slope sign: the step grows (capped) and
+ * is taken; opposite sign: the step shrinks (floored), the slope is forgotten and - the sign of a forgotten slope being 0 - the
+ * weight stays; otherwise the step is taken as it is. */
+static float irprop_sign(float x) { return x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f); }
+
+void myea_oracle_irprop_minus(const myea_hyper *h, size_t count, float *w, float *g, float *steps, float *slopes)
+{
+    for (size_t i = 0; i < count; ++i) {
+        float gi = g[i], d;
+        if (slopes[i] * gi > 0.f) {
+            d = steps[i] * h->rprop_increase_factor;
+            steps[i] = d = d < h->rprop_delta_max ? d : h->rprop_delta_max;
+        } else if (slopes[i] * gi < 0.f) {
+            d = steps[i] * h->rprop_decrease_factor;
+            steps[i] = d = d > h->rprop_delta_min ? d : h->rprop_delta_min;
+            gi = 0.f;
+        } else d = steps[i];
+        w[i] += -irprop_sign(gi) * d;
+        slopes[i] = gi;
+        g[i] = 0.f;
+    }
+}
+
 /* ------------------------------------------------------------------------------------------- */
 /* Update_Parameter: NN/Neural_Network.cpp:4719-4908 (merge is a no-op with one accumulator) */
 

@@ -49,6 +49,11 @@ int myea_oracle_get_loss(myea_oracle_net *net, myea_loss_state *out_state);
 /* pointer to a layer tensor (same kinds as myea_hip_download_tensor); *count receives its length */
 const float *myea_oracle_tensor(myea_oracle_net *net, size_t layer_index, int kind, size_t *count);
 
+/* Update_Parameter__iRPROP_minus__Loop (Neural_Network__iRPROP_minus.cpp:21-67) over [0, count): the reference's own
+ * Update_Parameter never dispatches it (its switch, Neural_Network.cpp:4770-4821, has no such case), so it stands alone here as
+ * it does there.  previous_steps / previous_derivatives are the two vectors of that name; the gradient is zeroed. */
+void myea_oracle_irprop_minus(const myea_hyper *hyper, size_t count, float *parameters, float *gradient, float *previous_steps, float *previous_derivatives);
+
 /* scalar pieces, exported so the tests can pin them one by one */
 float myea_oracle_activation(uint32_t type_activation_function, float summation);
 float myea_oracle_activation_derive(uint32_t type_activation_function, float summation, float steepness, float value);

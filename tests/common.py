@@ -1,11 +1,28 @@
 """Shared builders for the parity tests: seeded synthetic nets and data in the reference's layouts."""
 import ctypes as C
+import os
+from contextlib import contextmanager
 
 import numpy as np
 
 from myea_amd import binding as mb
 from myea_amd.synthetic import glorot_parameters, one_hot   # noqa: F401 (re-exported for the tests)
 from tests.oracle_lib import load_oracle
+
+
+@contextmanager
+def environment(**kw):
+    """environment variables for the library's switches, restored afterwards"""
+    old = {k: os.environ.get(k) for k in kw}
+    os.environ.update({k: str(v) for k, v in kw.items()})
+    try:
+        yield
+    finally:
+        for k, v in old.items():
+            if v is None:
+                del os.environ[k]
+            else:
+                os.environ[k] = v
 
 
 def oracle_desc(layers, batch_size, recurrent_depth=1):

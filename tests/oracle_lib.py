@@ -57,6 +57,8 @@ def load_oracle():
     lib.myea_oracle_activation.restype = C.c_float
     lib.myea_oracle_activation_derive.argtypes = [C.c_uint32, C.c_float, C.c_float, C.c_float]
     lib.myea_oracle_activation_derive.restype = C.c_float
+    lib.myea_oracle_irprop_minus.argtypes = [P(mb.Hyper), sz, vp, vp, vp, vp]
+    lib.myea_oracle_irprop_minus.restype = None
     lib.myea_hyper_default.argtypes = [P(mb.Hyper)]
     lib.myea_hyper_default.restype = None
     lib.myea_net_desc_layout.argtypes = [P(mb.NetDesc)]

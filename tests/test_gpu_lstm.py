@@ -168,25 +168,33 @@ def test_lstm_error_paths():
 
 
 def test_config3_full_size_one_step():
-    """BASELINE config 3 at full size: 2 x LSTM-512 (peephole), input 128, T = 64, batch 256, linear FC-512 head,
-    MSE, AMSGrad; one step on both sides (the oracle runs on the host's cores)."""
+    """BASELINE config 3 at full size: 2 x LSTM-512 (peephole), input 128, T = 64, batch 256, linear FC-512 head, MSE,
+    AMSGrad; one whole step on both sides (the oracle runs on the host's cores): outputs, deltas and every LSTM tap of all
+    layers at every time step, the whole gradient - entries outside the tolerance of the oracle go to a float64 sum of their
+    16384 products (tests/full_size_support.py) - then the AMSGrad-stepped parameters and the three optimizer vectors."""
+    from tests.full_size_support import GradientTerms, assert_first_adam_type_step_matches, assert_sums_match
     T, B = 64, 256
     specs = [dict(units=128), dict(type="lstm", units=512), dict(type="lstm", units=512), dict(units=512, activation="LINEAR")]
     threads = min(16, os.cpu_count() or 1)
-    desc, gpu, cpu = _pair(specs, B, T, dict(type_optimizer_function=mb.OPTIMIZER["AMSGRAD"], type_loss_function=mb.LOSS["MSE"]), seed=3, threads=threads)
+    hyper = dict(type_optimizer_function=mb.OPTIMIZER["AMSGRAD"], type_loss_function=mb.LOSS["MSE"])
+    desc, gpu, cpu = _pair(specs, B, T, hyper, seed=3, threads=threads)
+    twin = OracleNetwork(desc, mb.default_hyper(**hyper), threads=threads)
+    w = gpu.download_parameters()
+    twin.set_state_propagation(mb.STATE_TRAINING)
+    twin.upload_parameters(w)
+    twin.Clear_Training_Arrays()
     rng = np.random.default_rng(3)
     X = rng.normal(0, 1, (B, T * 128)).astype(np.float32)
     Y = rng.normal(0, 1, (B, T * 512)).astype(np.float32)
     for n in (gpu, cpu):
+        n.Reset__Loss()
         run_step(n, B, X, Y, update=False)
-    for li in (1, 2, 3):
-        a = gpu.download_tensor(li, mb.TENSOR["OUTPUTS"], T * B * 512)
-        b = cpu.download_tensor(li, mb.TENSOR["OUTPUTS"], T * B * 512)
-        assert_close(a, b, REL, ABS, what="outputs layer %d" % li)
+    _compare(desc, gpu, cpu, B, T, what="full size")
+    lg, lc = gpu.get_loss(), cpu.get_loss()
+    assert lg.number_loss == lc.number_loss and lg.loss_values == pytest.approx(lc.loss_values, rel=1e-5)
     g_gpu, g_cpu = gpu.download_gradient(), cpu.download_gradient()
-    # gradients here are sums of 16384 terms of either sign (up to ~1e3 in magnitude): the tolerance is taken relative
-    # to the scale of each parameter class' gradient, as fp32 summation in any order would require
-    scale = np.abs(g_cpu).max()
-    assert np.max(np.abs(g_gpu.astype(np.float64) - g_cpu)) <= 1e-4 * scale + 1e-5
-    off = np.abs(g_gpu.astype(np.float64) - g_cpu) > (ABS + REL * np.abs(g_cpu))
-    assert off.mean() < 0.05
+    report = {}
+    assert_sums_match(g_gpu, g_cpu, GradientTerms(desc, cpu, X, B).exact, "gradient", report=report)
+    print("config 3 gradient:", report["gradient"])
+    print("config 3 update:", assert_first_adam_type_step_matches(gpu, cpu, twin, w, g_gpu, g_cpu, B, mb.default_hyper(**hyper),
+                                                                  ("FIRST_MOMENT", "SECOND_MOMENT", "SECOND_MOMENT_HAT"), "AMSGrad step"))

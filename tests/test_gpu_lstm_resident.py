@@ -3,13 +3,12 @@ C ABI: against the same library with one launch per time step (MYEA_LSTM_RESIDEN
 bounded wait's give-up path.  Tolerance rel 1e-4 / abs 1e-5 (the resident kernels use the exp2 and reciprocal
 instructions in the gate functions, the per-step kernels expf and a division: a few ulp apart)."""
 import os
-from contextlib import contextmanager
 
 import numpy as np
 import pytest
 
 from myea_amd import binding as mb
-from tests.common import assert_close, glorot_parameters, run_step
+from tests.common import assert_close, environment, glorot_parameters, run_step
 from tests.oracle_lib import OracleNetwork
 from tests.test_gpu_lstm import LSTM_TAPS, _rows, _width
 
@@ -17,20 +16,6 @@ pytestmark = pytest.mark.gpu
 REL, ABS = 1e-4, 1e-5
 BACK = mb.TENSOR["DIRECTION_BACKWARD"]
 FORWARD_LOOP, BACKWARD_LOOP = 5, 6   # profile families of the time loops
-
-
-@contextmanager
-def environment(**kw):
-    old = {k: os.environ.get(k) for k in kw}
-    os.environ.update({k: str(v) for k, v in kw.items()})
-    try:
-        yield
-    finally:
-        for k, v in old.items():
-            if v is None:
-                del os.environ[k]
-            else:
-                os.environ[k] = v
 
 
 lstm = lambda units, **kw: dict(type="lstm", units=units, **kw)

@@ -174,3 +174,40 @@ def test_clear_optimizer_touches_the_current_optimizers_state_only_on_the_gpu():
         desc = mb.make_desc(SPECS, 2)
         return desc, mb.HipNetwork(desc, mb.default_hyper(**kw))
     check_clear_optimizer_touches_the_current_optimizers_state_only(make)
+
+
+def test_irprop_minus_through_the_kernel_level_entry_is_bit_exact():
+    """iRPROP- (Neural_Network__iRPROP_minus.cpp:21-67) has no case in the reference's Update_Parameter, so it is reached the way
+    the reference leaves it reachable: as a function of its own, myea_hip_optimizer_update on raw device vectors, against the
+    oracle's restatement fed the same gradients (sign changes, zeros, steps at the cap and at the floor; a length that is not a
+    multiple of four)."""
+    import ctypes as C
+    import torch
+    from tests.oracle_lib import load_oracle
+    lib, olib = mb.load_library(), load_oracle()
+    n = 100003
+    h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["IRPROP_MINUS"], rprop_delta_max=0.4, rprop_delta_min=0.02)
+    rng = np.random.default_rng(12)
+    w = rng.normal(0, 1, n).astype(np.float32)
+    steps, slopes = np.full(n, 0.1, np.float32), np.zeros(n, np.float32)
+    dev = [torch.from_numpy(a.copy()).cuda() for a in (w, np.zeros(n, np.float32), steps, slopes)]
+    for k in range(8):
+        g = rng.normal(0, 1, n).astype(np.float32) * (rng.uniform(0, 1, n) > 0.1)    # a tenth exact zeros
+        if k % 3 == 2:
+            g = np.abs(g) * np.sign(slopes + (slopes == 0))                           # mostly the sign of before: steps reach the cap
+        dev[1].copy_(torch.from_numpy(g))
+        gc = g.copy()
+        olib.myea_oracle_irprop_minus(C.byref(h), n, *(C.c_void_p(a.ctypes.data) for a in (w, gc, steps, slopes)))
+        rc = lib.myea_hip_optimizer_update(None, C.byref(h), n, n, 1.0, C.c_void_p(dev[0].data_ptr()), C.c_void_p(dev[1].data_ptr()), None,
+                                           C.c_void_p(dev[2].data_ptr()), C.c_void_p(dev[3].data_ptr()))
+        assert rc == 0, lib.myea_hip_last_error()
+        torch.cuda.synchronize()
+        assert np.array_equal(dev[0].cpu().numpy(), w), "weights, update %d" % k
+        assert np.array_equal(dev[2].cpu().numpy(), steps) and np.array_equal(dev[3].cpu().numpy(), slopes)
+        assert not dev[1].cpu().numpy().any()
+    assert steps.max() == np.float32(0.4) and steps.min() == np.float32(0.02)
+    # the network-level update refuses it, as the reference's switch does
+    desc, gpu, cpu = _pair(FC, dict(type_optimizer_function=mb.OPTIMIZER["IRPROP_MINUS"]))
+    with pytest.raises(mb.MyeaError) as e:
+        gpu.Update_Parameter(4, 4)
+    assert e.value.code == mb.E_UNSUPPORTED
