@@ -6,13 +6,15 @@ in different orders agree to rel 1e-4 / abs 1e-5 wherever the sum is not much sm
 holds more digits than the terms allow, the reference's own path under another number of OpenMP threads included.  So an
 entry outside the tolerance of the oracle is taken to float64: the exact sum of the very products (from the oracle's own
 delta and input tensors) and the sum of their magnitudes.  It passes when it is within the tolerance of the exact sum, or
-at least as near to it as the oracle's entry is, or within one fp32 unit in the last place (2^-23) of the sum of
-magnitudes.  No share of entries is exempt."""
+at least as near to it as the oracle's entry is, or within four fp32 units in the last place (2^-21) of the sum of
+magnitudes - the products themselves are built from fp32 deltas and activations that agree between the two sides to a unit
+or two in the last place, so no summation, however exact, can agree more closely than that.  No share of entries is
+exempt."""
 import numpy as np
 
 from myea_amd import binding as mb
 
-ULP32 = 2.0 ** -23
+ULPS = 4 * 2.0 ** -23   # of the sum of the terms' magnitudes
 
 
 def assert_sums_match(got, oracle, exact, what, rel=1e-4, abs_=1e-5, report=None):
@@ -26,7 +28,7 @@ def assert_sums_match(got, oracle, exact, what, rel=1e-4, abs_=1e-5, report=None
         eg, eo = np.abs(got[off] - truth), np.abs(oracle[off] - truth)
         within = eg <= abs_ + rel * np.abs(truth)
         nearer = eg <= eo
-        ulp = eg <= ULP32 * mags
+        ulp = eg <= ULPS * mags
         counts.update(within_exact=int(within.sum()), nearer_than_oracle=int((~within & nearer).sum()), within_ulp_of_magnitudes=int((~within & ~nearer & ulp).sum()))
         bad = ~(within | nearer | ulp)
         if bad.any():
@@ -141,7 +143,9 @@ def assert_first_adam_type_step_matches(gpu, cpu, twin, w, g_gpu, g_cpu, B, h, k
     gradient g_gpu), the oracle (its own gradient g_cpu) and a second oracle network `twin` that is handed the device's
     gradient.
     (a) Device against twin - the same gradient on both sides, so the update arithmetic alone: every parameter and every
-        entry of the optimizer vectors `kinds`, rel 1e-5.
+        entry of the optimizer vectors `kinds`, rel 1e-5; with clipping by the global norm rel 1e-4 / abs 1e-5, since the norm
+        is an fp32 sum over all parameters (ten million squares here) whose rounding depends on the order of summation - the
+        reference's own with its thread count - and scales every step.
     (b) Device against oracle, each from its own gradient: parameters within rel / abs and the optimizer vectors within the
         tolerance the gradient's own tolerance turns into (first moment (1 - beta1) s g, second moment (1 - beta2) (s g)^2,
         s the clipping factor), wherever the two gradients agree within rel / abs and the gradient is not below its own
@@ -152,7 +156,8 @@ def assert_first_adam_type_step_matches(gpu, cpu, twin, w, g_gpu, g_cpu, B, h, k
         n.Update_Parameter(B, B)
     wg, wc, wt = (n.download_parameters().astype(np.float64) for n in (gpu, cpu, twin))
     e = np.abs(wg - wt)
-    assert not (e > 1e-7 + 1e-5 * np.abs(wt)).any(), "%s: update arithmetic: %d parameters differ, worst %.3g" % (what, int((e > 1e-7 + 1e-5 * np.abs(wt)).sum()), float(e.max()))
+    arel, aabs = (rel, abs_) if h.use_clip_gradient else (1e-5, 1e-7)
+    assert not (e > aabs + arel * np.abs(wt)).any(), "%s: update arithmetic: %d parameters differ, worst %.3g" % (what, int((e > aabs + arel * np.abs(wt)).sum()), float(e.max()))
     gg, gc = np.asarray(g_gpu, np.float64), np.asarray(g_cpu, np.float64)
     agree = np.abs(gg - gc) <= abs_ + rel * np.abs(gc)
     strict = (agree & (np.abs(gc) >= abs_)) | ((gg == 0) & (gc == 0))
@@ -167,7 +172,7 @@ def assert_first_adam_type_step_matches(gpu, cpu, twin, w, g_gpu, g_cpu, B, h, k
     for kind in kinds:
         a, b, t = (n.download_optimizer_state(mb.OPT_STATE[kind]).astype(np.float64) for n in (gpu, cpu, twin))
         e = np.abs(a - t)
-        assert not (e > 1e-30 + 1e-5 * np.abs(t)).any(), "%s: update arithmetic: optimizer vector %s: %d entries differ" % (what, kind, int((e > 1e-30 + 1e-5 * np.abs(t)).sum()))
+        assert not (e > 1e-30 + arel * np.abs(t)).any(), "%s: update arithmetic: optimizer vector %s: %d entries differ" % (what, kind, int((e > 1e-30 + arel * np.abs(t)).sum()))
         if kind == "FIRST_MOMENT":
             tol = 1.1 * rel * np.abs(b) + (1.0 - b1) * s * 1.1 * abs_
         else:

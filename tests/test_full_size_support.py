@@ -36,7 +36,7 @@ def test_listed_products_add_up_to_the_oracles_gradient(name, specs, T, B, Bmax)
 def test_the_three_clauses():
     oracle = np.array([1.0, 2.0, 3.0, 4.0, 5.0])
     exact = lambda idx: (np.array([1.0, 2.5, 3.0, 4.0, 5.0])[idx], np.array([1.0, 1.0, 1e6, 1.0, 1.0])[idx])
-    got = np.array([1.00005, 2.4, 3.05, 4.0, 5.0])       # inside the oracle's tolerance; nearer to the exact sum; within an ulp of 1e6
+    got = np.array([1.00005, 2.4, 3.05, 4.0, 5.0])       # inside the oracle's tolerance; nearer to the exact sum; within four ulps of 1e6
     counts = assert_sums_match(got, oracle, exact, "clauses")
     assert counts["outside_oracle_tolerance"] == 2 and counts["nearer_than_oracle"] == 1 and counts["within_ulp_of_magnitudes"] == 1
     with pytest.raises(AssertionError):

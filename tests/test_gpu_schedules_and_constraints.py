@@ -4,6 +4,7 @@ gradient sequence.  Tolerance: rel 1e-4 / abs 1e-5 on weights and optimizer stat
 must agree bit for bit; the scalar state the update advances (time steps, cycle length, running sums) exactly."""
 import numpy as np
 import pytest
+import torch   # before the library first touches the device: imported later, torch finds no GPU in this process
 
 from myea_amd import binding as mb
 from tests.common import assert_close, glorot_parameters
@@ -182,11 +183,10 @@ def test_irprop_minus_through_the_kernel_level_entry_is_bit_exact():
     oracle's restatement fed the same gradients (sign changes, zeros, steps at the cap and at the floor; a length that is not a
     multiple of four)."""
     import ctypes as C
-    import torch
     from tests.oracle_lib import load_oracle
     lib, olib = mb.load_library(), load_oracle()
     n = 100003
-    h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["IRPROP_MINUS"], rprop_delta_max=0.4, rprop_delta_min=0.02)
+    h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["IRPROP_MINUS"], rprop_delta_max=0.15, rprop_delta_min=0.02)
     rng = np.random.default_rng(12)
     w = rng.normal(0, 1, n).astype(np.float32)
     steps, slopes = np.full(n, 0.1, np.float32), np.zeros(n, np.float32)
@@ -205,7 +205,7 @@ def test_irprop_minus_through_the_kernel_level_entry_is_bit_exact():
         assert np.array_equal(dev[0].cpu().numpy(), w), "weights, update %d" % k
         assert np.array_equal(dev[2].cpu().numpy(), steps) and np.array_equal(dev[3].cpu().numpy(), slopes)
         assert not dev[1].cpu().numpy().any()
-    assert steps.max() == np.float32(0.4) and steps.min() == np.float32(0.02)
+    assert steps.max() == np.float32(0.15) and steps.min() == np.float32(0.02)
     # the network-level update refuses it, as the reference's switch does
     desc, gpu, cpu = _pair(FC, dict(type_optimizer_function=mb.OPTIMIZER["IRPROP_MINUS"]))
     with pytest.raises(mb.MyeaError) as e:
