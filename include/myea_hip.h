@@ -375,10 +375,12 @@ int myea_hip_upload_zoneout_masks(myea_hip_net *net, const uint8_t *host_masks, 
  *    width), used by every following forward pass until the call is repeated with NULL / 0.  A caller that draws with the
  *    reference's generators in the reference's order gets the reference's numbers.
  * Either way MYEA_TENSOR_DROPOUT_NOISE reads back what the last forward pass used.
+ * Inside a residual block the draws belong to a member's input-side activation units: [T][Bmax][fan-in].
  * ShakeDrop on a residual layer (Forward_Pass__Dropout__ShakeDrop :5016-5045, Backward_Pass__Dropout__ShakeDrop
- * Neural_Network__Backward_Pass__Loop.cpp:1050-1078) uses the same two sources; its tensor is
- * [batch_size masks as 0 / 1][batch_size x width forward draws][batch_size x width backward draws] with `width` the block's
- * last layer's, `count` = batch_size x (1 + 2 x width).  The device generator draws all three in the forward pass. */
+ * Neural_Network__Backward_Pass__Loop.cpp:1050-1078; one mask per (time step, example),
+ * Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:367-386) uses the same two sources; its tensor is
+ * [T x batch_size masks as 0 / 1][T x batch_size x width forward draws][T x batch_size x width backward draws] with `width`
+ * the block's last layer's, `count` = T x batch_size x (1 + 2 x width).  The device generator draws all three in the forward pass. */
 int myea_hip_set_dropout_seed(myea_hip_net *net, uint64_t seed);
 int myea_hip_upload_dropout_noise(myea_hip_net *net, size_t layer_index, const float *noise, size_t count, int noise_on_device);
 /* Clear_Training_Arrays (Train.cpp:93-126) + Clear_Optimizer (Train.cpp:128-263): zero the gradient

@@ -812,10 +812,11 @@ __device__ __forceinline__ void update_one(const UpdateDev &p, float gs, float &
 template <int KIND, bool WD>
 __global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
 {
-    // A kernel of an earlier pass whose bounded wait gave up has left that pass incomplete and raised this word: the
-    // update then changes nothing (weights, optimizer vectors and gradient stay as they are) until the host has dealt with it.
-    if (p.fault && __hip_atomic_load(p.fault, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return;
-    if (p.applied && blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(p.applied, 1ull);   // the launch that completes a whole update counts it
+    // A kernel of an earlier pass whose bounded wait gave up has left that pass incomplete and raised this word (earlier in
+    // stream order: a plain load sees it): the update then changes nothing - weights, optimizer vectors and gradient stay as
+    // they are - until the host has dealt with it.  The word is fetched with the operands and looked at in front of the stores,
+    // so that no wavefront waits for it before it has its own loads in flight.
+    const unsigned faulted = p.fault ? *p.fault : 0u;
     float gs = p.grad_scale;
     if (p.norm_sq) {  // Clip_Gradient: scale when norm >= clip (NN/Neural_Network__Clip_Gradient.cpp:81-94)
         const float norm = sqrtf(p.norm_sq[0]);
@@ -835,6 +836,7 @@ __global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
         if (kA) av = a4[i];
         if (kB) bv = b4[i];
         if (kC) cv = c4[i];
+        if (faulted) return;
         float w[4], a[4], b[4], c[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -847,6 +849,8 @@ __global__ __launch_bounds__(kBlock) void update_kernel(UpdateDev p)
         if (kC) __builtin_nontemporal_store(f32x4{c[0], c[1], c[2], c[3]}, &c4[i]);
         __builtin_nontemporal_store(f32x4{0.f, 0.f, 0.f, 0.f}, &g4[i]);
     }
+    if (faulted) return;
+    if (p.applied && blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(p.applied, 1ull);   // the launch that completes a whole update counts it
     if (blockIdx.x == 0 && threadIdx.x < (p.n & 3)) {
         const size_t i = n4 * 4 + threadIdx.x;
         float w = p.w[i], a = kA ? p.s0[i] : 0.f, b = kB ? p.s1[i] : 0.f, c = kC ? p.s2[i] : 0.f;
@@ -1274,6 +1278,7 @@ __global__ __launch_bounds__(kBlock) void pool_backward_kernel(PoolParams p, con
         for (unsigned kk = p.kernel; kk-- > 0;) {
             const size_t off = (size_t)kk * p.dilation;
             if (off > pos) continue;
+            if (p.is_max && p.dilation == 0 && kk != 0) continue;   // every tap of such a window is the one position: its window hands down once
             const size_t q = pos - off;
             if (q % p.stride) continue;
             const size_t j = q / p.stride;

@@ -150,14 +150,15 @@ int myea_net_desc_layout(myea_net_desc *d)
         if (out < 1.0 || out > 4294967295.0) return MYEA_E_INVALID;
         l->n_units = (uint32_t)out;
     }
-    /* residual blocks: depth >= 1, wholly inside the stack, followed by at least one layer, fully-connected and
-     * pooling members (what Forward_Pass__Residual__Layer's switch knows), no block inside a block */
+    /* residual blocks: depth >= 1, wholly inside the stack, followed by at least one layer; fully-connected, independently
+     * recurrent, LSTM and pooling members (what Recurrent__Forward_Pass__Residual__Layer's switch knows,
+     * NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:711-771), no block inside a block */
     for (uint32_t li = 1; li < d->n_layers; ++li) {
         const myea_layer_desc *l = &d->layers[li];
         if (l->type_layer != MYEA_LAYER_RESIDUAL) continue;
         if (l->block_depth == 0 || (uint64_t)li + l->block_depth + 1 >= d->n_layers) return MYEA_E_INVALID;
         for (uint32_t k = 1; k <= l->block_depth; ++k)
-            if ((d->layers[li + k].type_layer != MYEA_LAYER_FULLY_CONNECTED && !is_pooling(&d->layers[li + k])) || d->layers[li + k].k_sparsity != 0) return MYEA_E_UNSUPPORTED;
+            if (d->layers[li + k].type_layer == MYEA_LAYER_RESIDUAL) return MYEA_E_UNSUPPORTED;
         li += l->block_depth;
     }
 
@@ -169,7 +170,12 @@ int myea_net_desc_layout(myea_net_desc *d)
         uint64_t fan_in = number_outputs(d, previous_layer(d, li));
         l->first_connection_index = total_weights;
         if (is_dense(l)) {
-            total_weights += fan_in * l->n_units + (is_ind_rnn(l) ? l->n_units : 0u);
+            /* one self weight per recurrent activation unit: as many as the layer has units; inside a residual block they sit on
+             * the layer's input side - fan-in many, none for the block's first layer (Assign__Post__Residual_Layer,
+             * NN/Neural_Network__Compile.cpp:385-392) */
+            const uint32_t r = enclosing_block(d, li);
+            const uint64_t recurrent_units = !is_ind_rnn(l) ? 0u : (r == 0 ? l->n_units : (li == r + 1 ? 0u : fan_in));
+            total_weights += fan_in * l->n_units + recurrent_units;
         } else { /* LSTM */
             uint64_t dirs = l->use_bidirectional ? 2u : 1u;
             uint64_t cpb = l->n_cells_per_block, cells_per_layer = (uint64_t)l->n_units * cpb;

@@ -142,8 +142,9 @@ static int check_desc(const myea_net_desc &d)
     if (d.batch_size == 0 || d.number_recurrent_depth == 0) { set_last_error("descriptor: batch_size and number_recurrent_depth must be >= 1"); return MYEA_E_INVALID; }
     if (d.total_parameters != d.total_weights + d.total_bias + 2 * d.total_normalized_units) { set_last_error("descriptor: total_parameters inconsistent"); return MYEA_E_INVALID; }
     if (d.layers[0].type_layer != MYEA_LAYER_FULLY_CONNECTED) { set_last_error("descriptor: the input layer must be a fully-connected (unit) layer"); return MYEA_E_INVALID; }
-    // residual blocks: members are the block_depth fully-connected layers after the residual layer, a consumer follows
-    bool any_residual = false, any_lstm = false, any_pool = false, any_shakedrop = false;
+    // residual blocks: members are the block_depth layers after the residual layer, a consumer follows.  group: 0 outside a
+    // block, 1 a dense first member, 2 another dense member, 3 a pooling member, 4 an LSTM member
+    bool any_lstm = false;
     uint32_t block_end = 0;  // index of the last member of the block being walked, 0 outside
     std::vector<int> group(d.n_layers, 0);
     for (uint32_t li = 0; li < d.n_layers; ++li) {
@@ -152,27 +153,42 @@ static int check_desc(const myea_net_desc &d)
             set_last_error("layer %u: type %u is not on this path", li, l.type_layer);
             return MYEA_E_UNSUPPORTED;
         }
+        if (block_end != 0) {
+            if (l.type_layer == MYEA_LAYER_RESIDUAL) { set_last_error("layer %u: a residual block inside a residual block is not on this path", li); return MYEA_E_UNSUPPORTED; }
+            group[li] = layer_is_pooling(l) ? 3 : (l.type_layer == MYEA_LAYER_LSTM ? 4 : ((d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) ? 1 : 2));
+            if (li == block_end) block_end = 0;
+        } else if (l.type_layer == MYEA_LAYER_RESIDUAL) {
+            if (l.block_depth == 0 || (uint64_t)li + l.block_depth + 1 >= d.n_layers) { set_last_error("layer %u: residual block of depth %u does not fit in front of a consumer", li, l.block_depth); return MYEA_E_INVALID; }
+            if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_SHAKEDROP) { set_last_error("layer %u: a residual layer's dropout is ShakeDrop or none", li); return MYEA_E_UNSUPPORTED; }
+            if (l.type_dropout == MYEA_DROPOUT_SHAKEDROP && !(l.dropout_values[0] >= 0.f && l.dropout_values[0] <= 1.f)) { set_last_error("layer %u: ShakeDrop probability %g", li, (double)l.dropout_values[0]); return MYEA_E_INVALID; }
+            block_end = li + l.block_depth;
+        }
+        if (l.type_layer == MYEA_LAYER_LSTM) any_lstm = true;
+    }
+    (void)any_lstm;
+    for (uint32_t li = 0; li < d.n_layers; ++li) {
+        const myea_layer_desc &l = d.layers[li];
         if (l.k_sparsity != 0) {
+            // hidden fully-connected layers; inside a residual block on the member's input-side activation units (none on a first member)
             const float scaled = (float)l.k_sparsity * l.alpha_sparsity;
-            if (li == 0 || li + 1 >= d.n_layers || l.type_layer != MYEA_LAYER_FULLY_CONNECTED || block_end != 0) { set_last_error("layer %u: the k-sparse filter is on this path for hidden fully-connected layers outside residual blocks", li); return MYEA_E_UNSUPPORTED; }
-            if (l.k_sparsity > l.n_units || !(l.alpha_sparsity >= 0.f) || !(scaled >= 1.f) || (uint64_t)scaled > l.n_units) { set_last_error("layer %u: k-sparse filter: k %u, alpha %g do not fit %u units", li, l.k_sparsity, (double)l.alpha_sparsity, l.n_units); return MYEA_E_INVALID; }
+            const size_t width = group[li] == 2 ? (size_t)myea_net_desc_number_outputs(&d, myea_net_desc_previous_layer(&d, li)) : l.n_units;
+            if (li == 0 || li + 1 >= d.n_layers || l.type_layer != MYEA_LAYER_FULLY_CONNECTED || group[li] == 1) { set_last_error("layer %u: the k-sparse filter is on this path for hidden fully-connected layers that own activation units", li); return MYEA_E_UNSUPPORTED; }
+            if (l.k_sparsity > width || !(l.alpha_sparsity >= 0.f) || !(scaled >= 1.f) || (uint64_t)scaled > width) { set_last_error("layer %u: k-sparse filter: k %u, alpha %g do not fit %zu units", li, l.k_sparsity, (double)l.alpha_sparsity, width); return MYEA_E_INVALID; }
         }
         if (layer_is_ind_rnn(l)) {
             if (li == 0 || li + 1 >= d.n_layers) { set_last_error("layer %u: an independently recurrent layer is a hidden layer", li); return MYEA_E_INVALID; }
             if (l.type_activation_function == MYEA_AF_SOFTMAX) { set_last_error("layer %u: softmax belongs to the output layer only", li); return MYEA_E_UNSUPPORTED; }
             if (l.constraint_recurrent_weight_lower_bound > l.constraint_recurrent_weight_upper_bound) { set_last_error("layer %u: recurrent weight bounds out of order", li); return MYEA_E_INVALID; }
-        }
-        if (layer_is_pooling(l)) {
-            // between fully-connected / pooling layers of a stack without blocks around it; the width must be the one
-            // Assign__Post__Layer computes (NN/Neural_Network__Compile.cpp:250-271) - the kernels index with it
-            any_pool = true;
-            if (li == 0 || li + 1 >= d.n_layers) { set_last_error("layer %u: a pooling layer sits between the input and the output layer", li); return MYEA_E_UNSUPPORTED; }
-            const myea_layer_desc &pl = d.layers[li - 1], &nl = d.layers[li + 1];
-            const bool first_member = pl.type_layer == MYEA_LAYER_RESIDUAL && block_end != 0;   // then the layer in front of the block feeds it
-            if ((pl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(pl) && !first_member) || (nl.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(nl))) {
-                set_last_error("layer %u: pooling layers connect to fully-connected or pooling layers on this path", li);
+            // inside a block the recurrence sits on the member's input side, fan-in wide; the reference's backward pass walks it with
+            // the member's output width (NN/Neural_Network__Backward_Pass__OpenMP.cpp:867-877), which only addresses it when the two are equal
+            if (group[li] == 2 && myea_net_desc_number_outputs(&d, myea_net_desc_previous_layer(&d, li)) != l.n_units) {
+                set_last_error("layer %u: an independently recurrent member of a residual block is as wide as its input on this path (as in the reference's own indexing)", li);
                 return MYEA_E_UNSUPPORTED;
             }
+        }
+        if (layer_is_pooling(l)) {
+            // the width must be the one Assign__Post__Layer computes (NN/Neural_Network__Compile.cpp:250-271) - the kernels index with it
+            if (li == 0 || li + 1 >= d.n_layers) { set_last_error("layer %u: a pooling layer sits between the input and the output layer", li); return MYEA_E_UNSUPPORTED; }
             const double in = (double)myea_net_desc_number_outputs(&d, myea_net_desc_previous_layer(&d, li)), k = l.pooling_values[0], st = l.pooling_values[1], pad = l.pooling_values[2], dil = l.pooling_values[3];
             if (k < 1 || st < 1) { set_last_error("layer %u: pooling kernel and stride must be >= 1", li); return MYEA_E_INVALID; }
             const double span = l.type_layer == MYEA_LAYER_AVERAGE_POOLING ? in + 2 * pad - k : in + 2 * pad - dil * (k - 1) - 1;
@@ -180,23 +196,7 @@ static int check_desc(const myea_net_desc &d)
             if (out < 1 || (double)l.n_units != out) { set_last_error("layer %u: pooling width %u does not follow from its parameters (%.0f)", li, l.n_units, out); return MYEA_E_INVALID; }
             if (l.type_dropout != MYEA_DROPOUT_NONE || l.type_normalization != MYEA_NORMALIZATION_NONE) { set_last_error("layer %u: a pooling layer carries no dropout or normalization", li); return MYEA_E_UNSUPPORTED; }
         }
-        if (block_end != 0) {
-            if (l.type_layer != MYEA_LAYER_FULLY_CONNECTED && !layer_is_pooling(l)) { set_last_error("layer %u: only fully-connected and pooling layers may sit inside a residual block", li); return MYEA_E_UNSUPPORTED; }
-            group[li] = layer_is_pooling(l) ? 3 : ((d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) ? 1 : 2);
-            if (li == block_end) block_end = 0;
-        } else if (l.type_layer == MYEA_LAYER_RESIDUAL) {
-            if (l.block_depth == 0 || (uint64_t)li + l.block_depth + 1 >= d.n_layers) { set_last_error("layer %u: residual block of depth %u does not fit in front of a consumer", li, l.block_depth); return MYEA_E_INVALID; }
-            if (l.type_dropout != MYEA_DROPOUT_NONE && l.type_dropout != MYEA_DROPOUT_SHAKEDROP) { set_last_error("layer %u: a residual layer's dropout is ShakeDrop or none", li); return MYEA_E_UNSUPPORTED; }
-            if (l.type_dropout == MYEA_DROPOUT_SHAKEDROP && !(l.dropout_values[0] >= 0.f && l.dropout_values[0] <= 1.f)) { set_last_error("layer %u: ShakeDrop probability %g", li, (double)l.dropout_values[0]); return MYEA_E_INVALID; }
-            any_residual = true;
-            if (l.type_dropout == MYEA_DROPOUT_SHAKEDROP) any_shakedrop = true;
-            block_end = li + l.block_depth;
-        }
-        if (l.type_layer == MYEA_LAYER_LSTM) any_lstm = true;
     }
-    if (any_pool && any_lstm) { set_last_error("descriptor: pooling layers are on this path for stacks without LSTM layers"); return MYEA_E_UNSUPPORTED; }
-    if (any_residual && any_lstm) { set_last_error("descriptor: residual blocks are on this path for stacks without LSTM layers"); return MYEA_E_UNSUPPORTED; }
-    if (any_shakedrop && d.number_recurrent_depth != 1) { set_last_error("descriptor: ShakeDrop is on this path for feed-forward stacks only"); return MYEA_E_UNSUPPORTED; }
     for (uint32_t li = 0; li < d.n_layers; ++li) {
         const myea_layer_desc &l = d.layers[li];
         if (l.type_layer == MYEA_LAYER_RESIDUAL) {
@@ -210,8 +210,8 @@ static int check_desc(const myea_net_desc &d)
         if (l.type_dropout == MYEA_DROPOUT_ZONEOUT && l.type_layer == MYEA_LAYER_LSTM) {
             // masks per (time step, cell), uploaded with myea_hip_upload_zoneout_masks
         } else if (layer_uses_noise_dropout(l)) {
-            // one draw per (time step, example, unit): hidden / output fully-connected layers outside residual blocks
-            if (li == 0 || l.type_layer != MYEA_LAYER_FULLY_CONNECTED || group[li] != 0) { set_last_error("layer %u: Gaussian / Uout dropout is on this path for fully-connected layers outside residual blocks", li); return MYEA_E_UNSUPPORTED; }
+            // one draw per (time step, example, activation unit): hidden / output fully-connected layers; a block's first member owns no such unit
+            if (li == 0 || l.type_layer != MYEA_LAYER_FULLY_CONNECTED || group[li] == 1) { set_last_error("layer %u: Gaussian / Uout dropout is on this path for fully-connected layers that own activation units", li); return MYEA_E_UNSUPPORTED; }
             if (!(l.dropout_values[0] >= 0.f)) { set_last_error("layer %u: dropout value %g", li, (double)l.dropout_values[0]); return MYEA_E_INVALID; }
         } else if (l.type_dropout != MYEA_DROPOUT_NONE && !layer_uses_mask_dropout(l)) {
             set_last_error("layer %u: dropout type %u is not on this path", li, l.type_dropout);
@@ -224,7 +224,7 @@ static int check_desc(const myea_net_desc &d)
             if (group[li] == 2 && l.type_activation_function == MYEA_AF_SOFTMAX) { set_last_error("layer %u: softmax belongs to the output layer only", li); return MYEA_E_UNSUPPORTED; }
             const size_t fan_in = (size_t)myea_net_desc_number_outputs(&d, myea_net_desc_previous_layer(&d, li));
             const size_t units_af = group[li] == 0 ? l.n_units : (group[li] == 1 ? 0 : fan_in), units_norm = group[li] == 0 ? l.n_units : fan_in;
-            if (l.first_connection_index + fan_in * l.n_units + (layer_is_ind_rnn(l) ? l.n_units : 0u) > d.total_weights) { set_last_error("layer %u: weight slice leaves the weight region", li); return MYEA_E_INVALID; }
+            if (l.first_connection_index + fan_in * l.n_units + (layer_is_ind_rnn(l) ? units_af : 0u) > d.total_weights) { set_last_error("layer %u: weight slice leaves the weight region", li); return MYEA_E_INVALID; }
             if (layer_uses_bias(l) && l.first_bias_connection_index + l.n_units > d.total_weights + d.total_bias) { set_last_error("layer %u: bias slice leaves the bias region", li); return MYEA_E_INVALID; }
             if (layer_uses_norm(l) && l.first_normalized_unit_index + units_norm > d.total_normalized_units) { set_last_error("layer %u: scale/shift slice leaves its region", li); return MYEA_E_INVALID; }
             if (l.type_dropout != MYEA_DROPOUT_NONE && l.first_mask_index + (uint64_t)units_af * d.number_recurrent_depth > d.total_mask_units) { set_last_error("layer %u: mask slice leaves the mask buffer", li); return MYEA_E_INVALID; }
@@ -275,18 +275,21 @@ int Net::create(const myea_net_desc &desc)
         o.prev = myea_net_desc_previous_layer(&d, (uint32_t)li);
         o.In = li ? (size_t)myea_net_desc_number_outputs(&d, (uint32_t)o.prev) : 0;
         o.group = 0;
-        if (li > 1 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) {
-            if (d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) o.group = 1;
-            else if (L[li - 1].group != 0 && o.prev == li - 1) o.group = 2;  // the first layer after a block connects to the residual layer
-        } else if (li > 1 && layer_is_pooling(l) && (d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL || (L[li - 1].group != 0 && o.prev == li - 1))) {
-            o.group = 3;   // a pooling member of a block: basic units as wide as the layer, no activation or normalised units
+        {   // inside a residual block: the layer right behind a residual layer, and every layer up to the block's depth
+            bool member = false;
+            for (size_t r = 1; r < li && !member; ++r) member = d.layers[r].type_layer == MYEA_LAYER_RESIDUAL && li <= r + d.layers[r].block_depth;
+            if (member) {
+                if (layer_is_dense(l)) o.group = d.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL ? 1 : 2;
+                else if (layer_is_pooling(l)) o.group = 3;   // basic units as wide as the layer, no activation or normalised units
+                else if (l.type_layer == MYEA_LAYER_LSTM) o.group = 4;   // the layer as it is outside a block
+            }
         }
         if (l.type_layer == MYEA_LAYER_RESIDUAL) {
             o.NH = (size_t)myea_net_desc_number_outputs(&d, (uint32_t)(li + l.block_depth));
             o.AH = o.H;
             o.pad = ((o.In > o.NH ? o.In - o.NH : o.NH - o.In) + 1) / 2;  // Assign__Post__Layer, NN/Neural_Network__Compile.cpp:277
         } else {
-            const bool own_width = o.group == 0 || o.group == 3;
+            const bool own_width = o.group == 0 || o.group >= 3;
             o.AH = own_width ? o.H : (o.group == 1 ? 0 : o.In);
             o.NH = own_width ? o.H : o.In;
         }
@@ -295,13 +298,13 @@ int Net::create(const myea_net_desc &desc)
         MYEA_TRY(dev_alloc(&o.values, sa));
         MYEA_HIP_TRY(hipMemset(o.values, 0, (sa ? sa : 1) * sizeof(float)));
         if (layer_uses_mask_dropout(l) && layer_is_dense(l)) MYEA_TRY(dev_alloc(&o.colscale, T * o.AH));
-        if (l.type_layer == MYEA_LAYER_RESIDUAL && l.type_dropout == MYEA_DROPOUT_SHAKEDROP) {   // [masks][forward draws][backward draws]
-            MYEA_TRY(dev_alloc(&o.noise, B + 2 * B * o.NH));
-            MYEA_HIP_TRY(hipMemset(o.noise, 0, (B + 2 * B * o.NH) * sizeof(float)));
+        if (l.type_layer == MYEA_LAYER_RESIDUAL && l.type_dropout == MYEA_DROPOUT_SHAKEDROP) {   // [T][B] masks, [T][B][NH] forward draws, [T][B][NH] backward draws
+            MYEA_TRY(dev_alloc(&o.noise, T * (B + 2 * B * o.NH)));
+            MYEA_HIP_TRY(hipMemset(o.noise, 0, T * (B + 2 * B * o.NH) * sizeof(float)));
         }
-        if (layer_uses_noise_dropout(l)) {
-            MYEA_TRY(dev_alloc(&o.noise, sz));
-            MYEA_TRY(launch_fill(0, o.noise, sz, l.type_dropout == MYEA_DROPOUT_GAUSSIAN ? 1.f : 0.f));   // neutral until a pass draws
+        if (layer_uses_noise_dropout(l)) {   // one draw per activation unit
+            MYEA_TRY(dev_alloc(&o.noise, sa));
+            MYEA_TRY(launch_fill(0, o.noise, sa, l.type_dropout == MYEA_DROPOUT_GAUSSIAN ? 1.f : 0.f));   // neutral until a pass draws
         }
         if (li == 0) continue;
         if (l.type_layer == MYEA_LAYER_LSTM) { MYEA_TRY(lstm_create_layer(li)); continue; }
@@ -319,13 +322,15 @@ int Net::create(const myea_net_desc &desc)
         if (layer_is_dense(l) && layer_uses_bias(l) && li + 1 < d.n_layers) MYEA_TRY(dev_alloc(&o.bias_partials, (T * B + 31) / 32 * o.H));
         if (layer_is_dense(l) && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION) MYEA_TRY(dev_alloc(&o.norm_partials, (B + 31) / 32 * 2 * (o.H > o.NH ? o.H : o.NH)));
         MYEA_HIP_TRY(hipMemset(o.neuron_errors, 0, sz * sizeof(float)));
-        if (layer_is_ind_rnn(l)) {
-            MYEA_TRY(dev_alloc(&o.pre_afs, sz));
-            MYEA_HIP_TRY(hipMemset(o.pre_afs, 0, sz * sizeof(float)));
-            // the delta of the pre-activations IS the neuron errors unless a normalisation sits between the two
-            if (layer_uses_norm(l) && l.use_layer_normalization_before_activation) {
-                MYEA_TRY(dev_alloc(&o.dafs_own, sz));
-                MYEA_HIP_TRY(hipMemset(o.dafs_own, 0, sz * sizeof(float)));
+        if (layer_is_ind_rnn(l) && o.group != 1) {   // a block's first member owns no recurrent unit: a plain member
+            const size_t su = o.group ? sa : sz;     // inside a block the recurrent units sit on the input side
+            MYEA_TRY(dev_alloc(&o.pre_afs, su));
+            MYEA_HIP_TRY(hipMemset(o.pre_afs, 0, su * sizeof(float)));
+            // the delta of the pre-activations IS the neuron errors unless a normalisation sits between the two; a block member
+            // always keeps its own (what it hands to the member before it may be changed by that member afterwards)
+            if (o.group || (layer_uses_norm(l) && l.use_layer_normalization_before_activation)) {
+                MYEA_TRY(dev_alloc(&o.dafs_own, su));
+                MYEA_HIP_TRY(hipMemset(o.dafs_own, 0, su * sizeof(float)));
             }
         }
         if (layer_uses_norm(l)) {
@@ -698,42 +703,83 @@ int Net::forward_pool_layer(size_t li, size_t B)
 }
 
 // Forward_Pass__Residual (NN/Neural_Network__Forward_Pass__OpenMP.cpp:3861-3997) over pre-activation members
-// (Forward_Pass__Residual__FC, :4039-4433): on the member's INPUT [BN] -> (not the first member: activation -> dropout),
-// then weights and bias; the member's output is its summation.  The activation (+ dropout) of member m+1 is applied by
-// the epilogue of member m's contraction whenever nothing (a normalisation) sits between them.  After the last
-// member: [block-level BN], then the zero-padded identity shortcut (:5158-5240).
+// (Forward_Pass__Residual__FC, :4039-4433): on the member's INPUT [BN] -> (not the first member: [+ u * AF[t-1]] -> activation ->
+// dropout -> k-sparse filter), then weights and bias; the member's output is its summation.  The activation (+ Bernoulli
+// dropout) of member m+1 is applied by the epilogue of member m's contraction whenever nothing else sits between them.
+// After the last member: [block-level BN], [ShakeDrop], then the zero-padded identity shortcut (:5158-5240).
+// With a recurrent depth the members run one after the other, each over all of its time steps
+// (Recurrent__Forward_Pass__Residual / __Residual__Layer, NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:563-771): a
+// dense or pooling member time step by time step (every normalisation has its own statistics per time step), an
+// independently recurrent member's recurrence and an LSTM member's time loop as the layers of that kind outside a block.
 int Net::forward_residual_block(size_t ri, size_t B)
 {
     const myea_layer_desc &r = d.layers[ri];
     const size_t last = ri + r.block_depth, T = d.number_recurrent_depth, Bmax = d.batch_size;
     const bool training = state >= MYEA_STATE_TRAINING;
-    // the dropout multipliers of the members, once for all time steps
-    std::vector<char> drops(last + 2, 0);
-    for (size_t m = ri + 1; m <= last; ++m)
-        if (L[m].group == 2) { bool drop = false; MYEA_TRY(refresh_colscale(m, &drop)); drops[m] = drop ? 1 : 0; }
-    // With a recurrent depth the block runs time step by time step on the [T][Bmax][width] tensors (Recurrent__Forward_Pass__Residual,
-    // NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:563-817): every normalisation has its own statistics per time step.
-    for (size_t t = 0; t < T; ++t) {
-        const size_t roff = t * Bmax;
-        bool values_ready = false;  // the member's activation values were written by the previous contraction
-        for (size_t m = ri + 1; m <= last; ++m) {
-            const myea_layer_desc &l = d.layers[m];
-            DevLayer &o = L[m];
-            const size_t In = o.In, H = o.H;
-            const float *cur = layer_outputs(o.prev) + roff * In;
-            if (layer_is_pooling(l)) {   // a pooling member (Forward_Pass__Residual__Layer, :4005-4030): windows over the member before it
-                MYEA_TRY(launch_pool_forward(stream, pool_params(m, B), cur, o.values + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr));
-                values_ready = false;
-                continue;
+    bool values_ready = false;  // the member's activation values were written by the previous member's contractions
+    for (size_t m = ri + 1; m <= last; ++m) {
+        const myea_layer_desc &l = d.layers[m];
+        DevLayer &o = L[m];
+        const size_t In = o.In, H = o.H;
+        const float *x = layer_outputs(o.prev);
+        if (l.type_layer == MYEA_LAYER_LSTM) {
+            MYEA_TRY(lstm_forward_layer(m, B));
+            values_ready = false;
+            continue;
+        }
+        if (layer_is_pooling(l)) {   // a pooling member (Forward_Pass__Residual__Layer, :4005-4030): windows over the member before it
+            for (size_t t = 0; t < T; ++t) {
+                const size_t roff = t * Bmax;
+                MYEA_TRY(launch_pool_forward(stream, pool_params(m, B), x + roff * In, o.values + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr));
             }
-            if (layer_uses_norm(l)) {
-                MYEA_TRY(bn_forward(m, t, B, cur, training));
-                cur = o.normalizes + roff * In;
-            }
+            values_ready = false;
+            continue;
+        }
+        bool drop = false;
+        if (o.group == 2) MYEA_TRY(refresh_colscale(m, &drop));
+        const bool norm = layer_uses_norm(l), ind = o.group == 2 && layer_is_ind_rnn(l);
+        if (norm)
+            for (size_t t = 0; t < T; ++t) MYEA_TRY(bn_forward(m, t, B, x + t * Bmax * In, training));
+        const float *in = norm ? o.normalizes : x;
+        if (ind) {   // the recurrence and the activation over the whole sequence; Bernoulli dropout in place on what the next step reads
+            IndRnnParams p{};
+            p.T = T; p.B = B; p.Bmax = Bmax; p.H = In;
+            p.u = parameters + l.first_connection_index + H * In;
+            p.act = (int)l.type_activation_function; p.unit_act = o.unit_act;
+            p.in = in; p.pre_afs = o.pre_afs; p.afs = o.values;
+            p.colscale = drop ? o.colscale : nullptr;
+            MYEA_TRY(launch_ind_rnn_forward(stream, p));
+        }
+        // what the contractions of this member leave for the next one: its activation values, when only an activation and a
+        // Bernoulli multiplier stand between the two
+        bool feeds_next = false;
+        if (m < last) {
+            const myea_layer_desc &nx = d.layers[m + 1];
+            feeds_next = nx.type_layer == MYEA_LAYER_FULLY_CONNECTED && !layer_uses_norm(nx) && !L[m + 1].unit_act && !L[m + 1].noise && nx.k_sparsity == 0 &&
+                         gemm_can_fuse_activation((int)nx.type_activation_function);
+        }
+        bool next_drop = false;
+        if (feeds_next) MYEA_TRY(refresh_colscale(m + 1, &next_drop));
+        for (size_t t = 0; t < T; ++t) {
+            const size_t roff = t * Bmax;
+            const float *cur = in + roff * In;
             if (o.group == 2) {
-                if (!values_ready)
-                    MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, B, In, cur, o.values + roff * In, drops[m] ? o.colscale + t * o.AH : nullptr, o.unit_act));
-                cur = o.values + roff * In;
+                float *vals = o.values + roff * In;
+                if (!ind && !values_ready)
+                    MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, B, In, cur, vals, drop ? o.colscale + t * o.AH : nullptr, o.unit_act));
+                // Gaussian / Uout dropout, strictly in the training state, then the k-sparse filter (:4197-4274)
+                if (o.noise && state == MYEA_STATE_TRAINING) {
+                    if (t == 0 && !o.noise_uploaded) {
+                        const bool normal = l.type_dropout == MYEA_DROPOUT_GAUSSIAN;
+                        MYEA_TRY(launch_dropout_noise(stream, T * Bmax * In, o.noise, normal ? 1 : 0, normal ? 1.f : -l.dropout_values[0], l.dropout_values[0], dropout_seed, dropout_stream++));
+                    }
+                    MYEA_TRY(launch_dropout_noise_apply(stream, B * In, vals, o.noise + roff * In, l.type_dropout == MYEA_DROPOUT_UOUT));
+                }
+                if (l.k_sparsity != 0) {
+                    const size_t k = state == MYEA_STATE_TRAINING ? (size_t)l.k_sparsity : (size_t)(l.alpha_sparsity * (float)l.k_sparsity);
+                    MYEA_TRY(launch_k_sparse(stream, B, In, k, vals));
+                }
+                cur = vals;
             }
             GemmParams g{};
             g.A = cur; g.lda = (long)In; g.a_k_contiguous = 1;
@@ -742,38 +788,38 @@ int Net::forward_residual_block(size_t ri, size_t B)
             g.M = (int)B; g.N = (int)H; g.K = (int)In;
             g.epilogue = EPI_FC_FORWARD;
             g.bias = layer_uses_bias(l) ? parameters + l.first_bias_connection_index : nullptr;
-            values_ready = false;
-            if (m < last) {
-                const myea_layer_desc &nx = d.layers[m + 1];
-                if (layer_is_dense(nx) && !layer_uses_norm(nx) && !L[m + 1].unit_act && gemm_can_fuse_activation((int)nx.type_activation_function)) {
-                    g.act = (int)nx.type_activation_function;
-                    g.aux_out = L[m + 1].values + roff * H;
-                    g.colscale = drops[m + 1] ? L[m + 1].colscale + t * L[m + 1].AH : nullptr;
-                    values_ready = true;
-                }
+            if (feeds_next) {
+                g.act = (int)d.layers[m + 1].type_activation_function;
+                g.aux_out = L[m + 1].values + roff * H;
+                g.colscale = next_drop ? L[m + 1].colscale + t * L[m + 1].AH : nullptr;
             }
             prof_begin(0);
             MYEA_TRY(launch_gemm(stream, g));
             prof_end(2.0 * (double)B * (double)H * (double)In);
         }
-        DevLayer &o = L[ri];
-        const float *blk = layer_outputs(last) + roff * L[last].H;   // a dense member's sums, a pooling member's values
+        values_ready = feeds_next;
+    }
+    DevLayer &o = L[ri];
+    for (size_t t = 0; t < T; ++t) {
+        const size_t roff = t * Bmax;
+        const float *blk = layer_outputs(last) + roff * L[last].H;   // a dense member's sums, a pooling member's values, an LSTM member's outputs
         if (layer_uses_norm(r)) {
             MYEA_TRY(bn_forward(ri, t, B, blk, training));
             blk = o.normalizes + roff * o.NH;
         }
-        // ShakeDrop on the block's output, in place (NN/Neural_Network__Forward_Pass__Loop.cpp:4053-4078); feed-forward stacks only
+        // ShakeDrop on the block's output, in place (NN/Neural_Network__Forward_Pass__Loop.cpp:4053-4078): one mask per (time step,
+        // example), one draw per value (Recurrent__Forward_Pass__Dropout__ShakeDrop, NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:367-386)
         if (r.type_dropout == MYEA_DROPOUT_SHAKEDROP) {
             const size_t W = o.NH;
             float *out = const_cast<float *>(blk);
             if (state == MYEA_STATE_TRAINING) {
-                if (!o.noise_uploaded) {   // masks, forward and backward draws of this pass
-                    MYEA_TRY(launch_dropout_noise(stream, Bmax, o.noise, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
-                    MYEA_TRY(launch_threshold(stream, Bmax, o.noise, r.dropout_values[0]));
-                    MYEA_TRY(launch_dropout_noise(stream, Bmax * W, o.noise + Bmax, 0, -1.f, 1.f, dropout_seed, dropout_stream++));
-                    MYEA_TRY(launch_dropout_noise(stream, Bmax * W, o.noise + Bmax + Bmax * W, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
+                if (t == 0 && !o.noise_uploaded) {   // masks, forward and backward draws of this pass, all time steps
+                    MYEA_TRY(launch_dropout_noise(stream, T * Bmax, o.noise, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
+                    MYEA_TRY(launch_threshold(stream, T * Bmax, o.noise, r.dropout_values[0]));
+                    MYEA_TRY(launch_dropout_noise(stream, T * Bmax * W, o.noise + T * Bmax, 0, -1.f, 1.f, dropout_seed, dropout_stream++));
+                    MYEA_TRY(launch_dropout_noise(stream, T * Bmax * W, o.noise + T * Bmax + T * Bmax * W, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
                 }
-                MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, o.noise, o.noise + Bmax, 1.f));
+                MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, o.noise + roff, o.noise + T * Bmax + roff * W, 1.f));
             } else {
                 MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, nullptr, nullptr, 1.f - r.dropout_values[0]));
             }
@@ -929,7 +975,7 @@ int Net::backward_into_layer(size_t li, size_t B)
             lstm_delta_source(gi, 1, &delta2, &out2, &weights2);
             GemmParams g2 = g;
             g2.A = delta2 + roff * out2; g2.lda = (long)out2; g2.B = weights2; g2.K = (int)out2;
-            g2.C = tmp2 + roff * H; g2.epilogue = EPI_NONE; g2.addend = nullptr;
+            g2.C = tmp2 + roff * H; g2.epilogue = EPI_NONE;   // (a shortcut's share, when there is one, rides along as this launch's addend)
             prof_begin(1);
             MYEA_TRY(launch_gemm(stream, g2));
             prof_end(2.0 * (double)rows * (double)H * (double)out2);
@@ -1025,12 +1071,16 @@ int Net::backward_into_layer(size_t li, size_t B)
 }
 
 // Backward_Pass__Gradient__Residual (NN/Neural_Network__Backward_Pass__OpenMP.cpp:711-950) with
-// Backward_Pass__Residual__Block (:351-452) and Backward_Pass__Residual__FC (:454-534), members from the last to the first.
+// Backward_Pass__Residual__Block (:351-452) and Backward_Pass__Residual__FC (:454-534), members from the last to the first,
+// each over all of its time steps before the member in front of it (Recurrent__Backward_Pass__Gradient__Residual__Layer,
+// NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:885-1001).
 // The last member's delta is the residual layer's errors (cropped to its width), through the block-level BN backward when
-// there is one.  A member reduces its delta to its input side: dX = delta * W, times act' of its input-side activation,
-// through its BN backward; that result IS the delta of the member before it (the reference copies it there), so it is
-// written straight into that member's buffer.  A normalised first member keeps its input-side errors for the shortcut
-// source; an un-normalised one contributes delta * W there directly (backward_into_layer).
+// there is one.  A dense member reduces its delta to its input side: dX = delta * W, times act' of its input-side activation
+// (an independently recurrent member: through its recurrence over the time steps), through its BN backward; that result IS
+// the delta of the member before it (the reference copies it there), so it is written straight into that member's buffer.
+// An LSTM member runs its time loop backwards and hands the member before it dG * Win.  A normalised first member keeps its
+// input-side errors for the shortcut source; an un-normalised one, or an LSTM, contributes its contraction there directly
+// (backward_into_layer).
 int Net::backward_residual_block(size_t ri, size_t B)
 {
     const myea_layer_desc &r = d.layers[ri];
@@ -1039,44 +1089,78 @@ int Net::backward_residual_block(size_t ri, size_t B)
     const long crop = ro.H > ro.NH ? (long)ro.pad : 0;
     // the perturbed examples' deltas times the backward draws (NN/Neural_Network__Backward_Pass__Loop.cpp:433-443)
     const bool shake = r.type_dropout == MYEA_DROPOUT_SHAKEDROP;
-    const float *beta = shake ? ro.noise + d.batch_size + d.batch_size * ro.NH : nullptr;
     // time steps in descending order, as the dense layers of a recurrent network are walked; each is on its own
     for (size_t t = T; t-- > 0;) {
         const size_t roff = t * Bmax;
         const float *res_errors = ro.neuron_errors + roff * ro.H;
+        const float *mask = shake ? ro.noise + roff : nullptr, *beta = shake ? ro.noise + T * Bmax + T * Bmax * ro.NH + roff * ro.NH : nullptr;
         float *last_errors = L[last].neuron_errors + roff * L[last].H;
         if (layer_uses_norm(r)) {
             float *tmp = tmp1 + roff * ro.NH;
             MYEA_TRY(launch_padded_add(stream, B, ro.NH, res_errors, ro.H, crop, nullptr, 0, 0, tmp));
-            if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, tmp, ro.noise, beta, 1.f));
+            if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, tmp, mask, beta, 1.f));
             MYEA_TRY(bn_backward(ri, t, B, layer_outputs(last) + roff * L[last].H, tmp, last_errors));
         } else {
             MYEA_TRY(launch_padded_add(stream, B, ro.NH, res_errors, ro.H, crop, nullptr, 0, 0, last_errors));
-            if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, last_errors, ro.noise, beta, 1.f));
+            if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, last_errors, mask, beta, 1.f));
         }
-        for (size_t m = last; m > ri; --m) {
-            const myea_layer_desc &l = d.layers[m];
-            DevLayer &o = L[m];
-            const bool norm = layer_uses_norm(l);
-            if (o.group == 1 && !norm) break;
-            const size_t In = o.In, H = o.H;
-            if (layer_is_pooling(l)) {   // hands its delta down through its windows (Backward_Pass__Gradient__Residual__Layer, :753-772), nothing else
-                if (m == ri + 1) break;   // the first member: the layer in front of the block pulls it, together with the shortcut's share
+    }
+    for (size_t m = last; m > ri; --m) {
+        const myea_layer_desc &l = d.layers[m];
+        DevLayer &o = L[m];
+        const bool norm = layer_uses_norm(l), first = m == ri + 1;
+        const size_t In = o.In, H = o.H;
+        if (l.type_layer == MYEA_LAYER_LSTM) {
+            MYEA_TRY(lstm_backward_layer(m, B));
+            if (first) break;   // the layer in front of the block pulls dG * Win together with the shortcut's share
+            // what the member before it receives: dG * Win of every time step (both directions of a two-direction member)
+            const bool per_t = T > 1 && B != Bmax;
+            const size_t chunks = per_t ? T : 1, rows = per_t ? B : T * B;
+            for (size_t c = 0; c < chunks; ++c) {
+                const size_t roff = c * Bmax;
+                for (int direction = o.lstm2 ? 1 : 0; direction >= 0; --direction) {
+                    const float *delta, *weights;
+                    size_t out;
+                    lstm_delta_source(m, direction, &delta, &out, &weights);
+                    GemmParams g{};
+                    g.A = delta + roff * out; g.lda = (long)out; g.a_k_contiguous = 1;
+                    g.B = weights; g.ldb = (long)In; g.b_k_contiguous = 0;
+                    g.M = (int)rows; g.N = (int)In; g.K = (int)out;
+                    g.ldc = (long)In; g.epilogue = EPI_NONE;
+                    g.C = (direction == 1 ? tmp2 : L[m - 1].neuron_errors) + roff * In;
+                    if (direction == 0 && o.lstm2) { g.addend = tmp2 + roff * In; g.ld_addend = (long)In; }
+                    prof_begin(1);
+                    MYEA_TRY(launch_gemm(stream, g));
+                    prof_end(2.0 * (double)rows * (double)In * (double)out);
+                }
+            }
+            continue;
+        }
+        if (layer_is_pooling(l)) {   // hands its delta down through its windows (Backward_Pass__Gradient__Residual__Layer, :753-772), nothing else
+            if (first) break;   // the first member: the layer in front of the block pulls it, together with the shortcut's share
+            for (size_t t = T; t-- > 0;) {
+                const size_t roff = t * Bmax;
                 MYEA_TRY(launch_pool_backward(stream, pool_params(m, B), o.neuron_errors + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr,
                                               L[m - 1].neuron_errors + roff * In));
-                continue;
             }
-            float *dst = (o.group == 2 ? L[m - 1].neuron_errors : o.in_errors) + roff * In;
-            float *tmp = tmp1 + roff * In;
-            const float *prev_out = layer_outputs(o.prev) + roff * In;
+            continue;
+        }
+        if (o.group == 1 && !norm) break;
+        const bool ind = o.group == 2 && layer_is_ind_rnn(l);
+        const float *prev_all = layer_outputs(o.prev);
+        float *dst_all = o.group == 2 ? L[m - 1].neuron_errors : o.in_errors;
+        for (size_t t = T; t-- > 0;) {
+            const size_t roff = t * Bmax;
+            float *dst = dst_all + roff * In, *tmp = tmp1 + roff * In;
+            const float *prev_out = prev_all + roff * In;
             GemmParams g{};
             g.A = o.neuron_errors + roff * H; g.lda = (long)H; g.a_k_contiguous = 1;
             g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 0;
-            g.C = norm ? tmp : dst; g.ldc = (long)In;
+            g.C = (norm || ind) ? tmp : dst; g.ldc = (long)In;
             g.M = (int)B; g.N = (int)In; g.K = (int)H;
             g.epilogue = EPI_NONE;
             bool derive_pending = false;
-            if (o.group == 2) {
+            if (o.group == 2 && !ind) {
                 g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
                 g.pre = norm ? o.normalizes + roff * In : prev_out;   // Layer::ptr_array_pre_activation_functions
                 g.val = o.values + roff * In;
@@ -1087,7 +1171,23 @@ int Net::backward_residual_block(size_t ri, size_t B)
             MYEA_TRY(launch_gemm(stream, g));
             prof_end(2.0 * (double)B * (double)H * (double)In);
             if (derive_pending) MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, B * In, g.pre, g.val, g.C, g.C, o.unit_act, o.unit_steep, In));
-            if (norm) MYEA_TRY(bn_backward(m, t, B, prev_out, tmp, dst));
+            if (norm && !ind) MYEA_TRY(bn_backward(m, t, B, prev_out, tmp, dst));
+        }
+        if (ind) {
+            // Backward_Pass__FC__DF_Ind_RNN over the whole sequence (:865-880): what the member hands on is the delta of its
+            // pre-activations, through the input-side normalisation when there is one
+            IndRnnParams p{};
+            p.T = T; p.B = B; p.Bmax = Bmax; p.H = In;
+            p.u = parameters + l.first_connection_index + H * In;
+            p.act = (int)l.type_activation_function; p.steep = l.activation_steepness; p.unit_act = o.unit_act; p.unit_steep = o.unit_steep;
+            p.pre_afs = o.pre_afs; p.afs = o.values;
+            p.dy = tmp1; p.dafs = o.dafs_own;
+            MYEA_TRY(launch_ind_rnn_backward(stream, p));
+            if (norm) {
+                for (size_t t = T; t-- > 0;) MYEA_TRY(bn_backward(m, t, B, prev_all + t * Bmax * In, o.dafs_own + t * Bmax * In, dst_all + t * Bmax * In));
+            } else {
+                MYEA_HIP_TRY(hipMemcpyAsync(dst_all, o.dafs_own, T * Bmax * In * sizeof(float), hipMemcpyDeviceToDevice, stream));
+            }
         }
     }
     return MYEA_OK;
@@ -1282,8 +1382,9 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
                         prof_end((double)rows * (double)o.H * sizeof(float));
                     }
                 }
-            if (layer_is_ind_rnn(l))
-                MYEA_TRY(launch_ind_rnn_self_weight_gradient(stream, T, B, Bmax, o.H, o.values, o.dafs_own ? o.dafs_own : o.neuron_errors,
+            // the self weights: as many as the layer has recurrent units - its width, a block member's fan-in, none for a block's first member
+            if (layer_is_ind_rnn(l) && o.group != 1)
+                MYEA_TRY(launch_ind_rnn_self_weight_gradient(stream, T, B, Bmax, o.group ? o.AH : o.H, o.values, o.dafs_own ? o.dafs_own : o.neuron_errors,
                                                              gradient + l.first_connection_index + o.H * o.In, scratch));
         }
         return MYEA_OK;
@@ -1583,8 +1684,8 @@ int Net::update_finish()
     // 289-333): the self weights of the independently recurrent hidden layers clipped to their bounds
     for (size_t li = 1; li + 1 < d.n_layers; ++li) {
         const myea_layer_desc &l = d.layers[li];
-        if (!layer_is_ind_rnn(l) || (l.constraint_recurrent_weight_lower_bound == 0.f && l.constraint_recurrent_weight_upper_bound == 0.f)) continue;
-        MYEA_TRY(launch_clip_range(stream, L[li].H, parameters + l.first_connection_index + L[li].H * L[li].In,
+        if (!layer_is_ind_rnn(l) || L[li].group == 1 || (l.constraint_recurrent_weight_lower_bound == 0.f && l.constraint_recurrent_weight_upper_bound == 0.f)) continue;
+        MYEA_TRY(launch_clip_range(stream, L[li].group ? L[li].AH : L[li].H, parameters + l.first_connection_index + L[li].H * L[li].In,
                                    l.constraint_recurrent_weight_lower_bound, l.constraint_recurrent_weight_upper_bound));
     }
     return lstm_parameters_changed();  // refresh the packed gate matrices
@@ -1808,8 +1909,9 @@ int myea_hip_upload_dropout_noise(myea_hip_net *n, size_t li, const float *noise
     myea::DevLayer &o = n->net.L[li];
     if (!noise && count == 0) { o.noise_uploaded = false; return MYEA_OK; }   // back to the device generator
     const bool shake = n->net.d.layers[li].type_layer == MYEA_LAYER_RESIDUAL;
-    const size_t want = shake ? (size_t)n->net.d.batch_size * (1 + 2 * o.NH) : (size_t)n->net.d.number_recurrent_depth * n->net.d.batch_size * o.H;
-    if (!noise || count != want) { myea::set_last_error("upload_dropout_noise: null or count %zu != %zu (%s)", count, want, shake ? "batch_size x (1 + 2 x block width)" : "T x batch_size x width"); return MYEA_E_INVALID; }
+    const size_t TB = (size_t)n->net.d.number_recurrent_depth * n->net.d.batch_size;
+    const size_t want = shake ? TB * (1 + 2 * o.NH) : TB * o.AH;
+    if (!noise || count != want) { myea::set_last_error("upload_dropout_noise: null or count %zu != %zu (%s)", count, want, shake ? "T x batch_size x (1 + 2 x block width)" : "T x batch_size x activation units"); return MYEA_E_INVALID; }
     MYEA_HIP_TRY(hipMemcpyAsync(o.noise, noise, count * sizeof(float), on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, n->net.stream));
     MYEA_HIP_TRY(hipStreamSynchronize(n->net.stream));
     o.noise_uploaded = true;
@@ -1911,9 +2013,9 @@ int myea_hip_download_tensor(myea_hip_net *n, size_t li, int kind, float *host, 
     case MYEA_TENSOR_SUMMATIONS: p = o.summations; break;
     case MYEA_TENSOR_ERRORS: p = o.neuron_errors; break;
     case MYEA_TENSOR_NORM_HATS: p = o.hats; c = T * n->net.d.batch_size * o.NH; break;
-    case MYEA_TENSOR_DROPOUT_NOISE: p = o.noise; if (n->net.d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) c = n->net.d.batch_size * (1 + 2 * o.NH); break;
+    case MYEA_TENSOR_DROPOUT_NOISE: p = o.noise; c = n->net.d.layers[li].type_layer == MYEA_LAYER_RESIDUAL ? T * n->net.d.batch_size * (1 + 2 * o.NH) : T * n->net.d.batch_size * o.AH; break;
     case MYEA_TENSOR_INPUT_SIDE_ERRORS:
-        if (o.group == 2) p = n->net.L[li - 1].neuron_errors;
+        if (o.group == 2) p = n->net.L[li - 1].neuron_errors;   // what the member handed to the one before it (an LSTM there adds its recurrent terms to it afterwards)
         else if (o.group == 1) p = o.in_errors;
         c = T * n->net.d.batch_size * o.In;
         break;

@@ -37,3 +37,27 @@ def one_hot(labels, n):
     y = np.zeros((len(labels), n), dtype=np.float32)
     y[np.arange(len(labels)), labels] = 1.0
     return y
+
+
+def simple_debug_layers(inputs=28, outputs=10, units=32, blocks_per_group=3, block_depth=3, widening=-9, normalization="BATCH_NORMALIZATION"):
+    """The network the reference's worked example builds (Neural_Network_Launcher_Windows/Source_Files/debug.cpp:81-87, 727-1075):
+    an independently recurrent first hidden layer, then three groups of residual blocks whose members are independently recurrent
+    layers, a max pooling (kernel 2, stride 2, dilation 0) between the groups, every block `widening / (3 * blocks_per_group)`
+    units wider than the one before; ISRLU members, batch normalisation on every hidden and residual layer (before the
+    activation), a softmax head.  sMNIST rows: 28 inputs per time step."""
+    norm = dict(normalization=normalization, norm_before=True) if normalization != "NONE" else {}
+    member = lambda n: dict(type="ind_rnn", units=int(n), activation="ISRLU", **norm)
+    layers = [dict(units=inputs), member(units)]
+    width, step = float(units), widening / (3.0 * blocks_per_group)
+    for group in range(3):
+        if group:
+            layers.append(dict(type="max_pooling", kernel=2, stride=2, padding=0, dilation=0))
+        for _ in range(blocks_per_group):
+            width += step
+            block = dict(type="residual", block_depth=block_depth)
+            if normalization != "NONE":
+                block["normalization"] = normalization
+            layers.append(block)
+            layers += [member(width)] * block_depth
+    layers.append(dict(units=outputs, activation="SOFTMAX"))
+    return layers

@@ -288,7 +288,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
                 if (block != 0) { o->group = seen == 0 ? 1 : 2; ++seen; }
             }
             if (l->type_layer == MYEA_LAYER_RESIDUAL) {
-                if (block != 0 || (T != 1 && l->type_dropout == MYEA_DROPOUT_SHAKEDROP) || l->block_depth == 0 || li + l->block_depth + 1 >= desc->n_layers || (l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_SHAKEDROP)) { free(n); return MYEA_E_UNSUPPORTED; }
+                if (block != 0 || l->block_depth == 0 || li + l->block_depth + 1 >= desc->n_layers || (l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_SHAKEDROP)) { free(n); return MYEA_E_UNSUPPORTED; }
                 block = li; seen = 0;
             }
         }
@@ -304,7 +304,7 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
                 o->NH = b;
             } else o->H = layer_width(l);
             o->In = li ? n->L[o->prev].H : 0;
-            if (is_pooling(l)) { o->AH = o->H; o->NH = o->H; }   /* basic units: as wide as the layer, inside a block too */
+            if (is_pooling(l) || l->type_layer == MYEA_LAYER_LSTM) { o->AH = o->H; o->NH = o->H; }   /* basic units / cells: as wide as the layer, inside a block too */
             else if (l->type_layer != MYEA_LAYER_RESIDUAL) { o->AH = o->group ? (o->group == 1 ? 0 : o->In) : o->H; o->NH = o->group ? o->In : o->H; }
             else o->AH = o->H;
         }
@@ -318,7 +318,13 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
     for (size_t li = 0; li < desc->n_layers; ++li) {
         const myea_layer_desc *l = &desc->layers[li];
         olayer *o = &n->L[li];
-        if (o->group && l->type_layer != MYEA_LAYER_FULLY_CONNECTED && !is_pooling(l)) { free(n); return MYEA_E_UNSUPPORTED; }
+        /* members of a residual block: fully-connected, independently recurrent, LSTM and pooling layers (the recurrent member
+         * switch, NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:711-771).  An independently recurrent member that is not
+         * the block's first carries its recurrence on its input side, fan-in wide; the reference's backward pass walks those
+         * units with the member's OUTPUT width (NN/Neural_Network__Backward_Pass__OpenMP.cpp:867-877 hands tmp_output_size to
+         * Backward_Pass__FC__DF_Ind_RNN), which addresses them correctly only when the two widths are equal: other shapes have no
+         * behaviour to follow */
+        if (o->group == 2 && is_ind_rnn(l) && o->In != o->H) { free(n); return MYEA_E_UNSUPPORTED; }
         if (l->type_layer == MYEA_LAYER_LSTM && l->type_dropout != MYEA_DROPOUT_NONE && l->type_dropout != MYEA_DROPOUT_ZONEOUT) { free(n); return MYEA_E_UNSUPPORTED; }
         /* with more cells per block the reference's indices [3] .. [8] into the layer's normalised units (NN/Neural_Network.cpp:4498-4613)
          * land on the second cell's units instead of the block's (the units are laid out per block: 3 per cell, then 6,
@@ -388,13 +394,15 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
             o->summations = zalloc(sz);
             o->neuron_errors = zalloc(sz);
         }
-        if (is_ind_rnn(l)) { o->pre_afs = zalloc(sz); o->dafs = zalloc(sz); }
-        if (l->type_layer == MYEA_LAYER_RESIDUAL && l->type_dropout == MYEA_DROPOUT_SHAKEDROP) o->noise = zalloc(B + 2 * B * o->NH);   /* all masks false */
+        if (is_ind_rnn(l)) { o->pre_afs = zalloc(o->group ? T * B * o->AH : sz); o->dafs = zalloc(o->group ? T * B * o->AH : sz); }
+        if (l->type_layer == MYEA_LAYER_RESIDUAL && l->type_dropout == MYEA_DROPOUT_SHAKEDROP) o->noise = zalloc(T * (B + 2 * B * o->NH));   /* all masks false */
         if (l->type_layer != MYEA_LAYER_RESIDUAL && l->type_dropout == MYEA_DROPOUT_SHAKEDROP) { free(n); return MYEA_E_UNSUPPORTED; }
         if (l->type_dropout == MYEA_DROPOUT_GAUSSIAN || l->type_dropout == MYEA_DROPOUT_UOUT) {
-            if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED || o->group) { free(n); return MYEA_E_UNSUPPORTED; }
-            o->noise = zalloc(sz);
-            if (l->type_dropout == MYEA_DROPOUT_GAUSSIAN) for (size_t i = 0; i < sz; ++i) o->noise[i] = 1.f;
+            /* one draw per activation unit: the layer's own width, or a block member's fan-in (none for a block's first member) */
+            if (l->type_layer != MYEA_LAYER_FULLY_CONNECTED || o->group == 1) { free(n); return MYEA_E_UNSUPPORTED; }
+            size_t sa = T * B * o->AH;
+            o->noise = zalloc(sa);
+            if (l->type_dropout == MYEA_DROPOUT_GAUSSIAN) for (size_t i = 0; i < sa; ++i) o->noise[i] = 1.f;
         }
         if (layer_uses_norm(l)) {
             size_t sn = T * B * o->NH, tn = T * o->NH;
@@ -480,8 +488,8 @@ float *myea_oracle_optimizer_state(myea_oracle_net *n, int k) { return (k >= 0 &
 float *myea_oracle_dropout_noise(myea_oracle_net *n, size_t li, size_t *count)
 {
     if (!n || li >= n->d.n_layers || !n->L[li].noise) { if (count) *count = 0; return NULL; }
-    if (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) { if (count) *count = (size_t)n->d.batch_size * (1 + 2 * n->L[li].NH); return n->L[li].noise; }
-    if (count) *count = (size_t)n->d.number_recurrent_depth * n->d.batch_size * n->L[li].H;
+    if (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) { if (count) *count = (size_t)n->d.number_recurrent_depth * n->d.batch_size * (1 + 2 * n->L[li].NH); return n->L[li].noise; }
+    if (count) *count = (size_t)n->d.number_recurrent_depth * n->d.batch_size * n->L[li].AH;
     return n->L[li].noise;
 }
 uint8_t *myea_oracle_zoneout_masks(myea_oracle_net *n, size_t *count) { if (count) *count = n->zoneout_count; return n->zoneout; }
@@ -774,8 +782,14 @@ static void fwd_residual_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_
         cur = o->normalizes;
     }
     if (o->group == 2) {
+        if (is_ind_rnn(l)) {   /* the recurrence sits on the member's input side too (:4108-4150): self weights behind the [H][In] matrix */
+            fwd_ind_rnn(n, t, B, In, n->parameters + l->first_connection_index + H * In, o->values, cur, o->pre_afs);
+            cur = o->pre_afs;
+        }
         fwd_af(n, t, B, In, l->type_activation_function, o->unit_af, cur, o->values);
-        fwd_dropout(n, l, t, B, In, o->values);
+        fwd_dropout(n, l, t, B, In, o->values);   /* Bernoulli (training masks, inference scaling), Gaussian, Uout: :4197-4232, :4253-4262 */
+        if (l->k_sparsity != 0)                   /* :4234-4245, :4264-4274 */
+            fwd_k_sparse(n, t, B, In, n->state == MYEA_STATE_TRAINING ? (size_t)l->k_sparsity : (size_t)(l->alpha_sparsity * (float)l->k_sparsity), o->values);
         cur = o->values;
     }
     fwd_fc(n, t, B, In, H, cur, n->parameters + l->first_connection_index, o->summations);
@@ -788,16 +802,28 @@ static void fwd_residual_fc_layer(myea_oracle_net *n, size_t li, size_t t, size_
 /* With a recurrent depth T > 1 every member and the shortcut run time step by time step on the [T][Bmax][width] tensors
  * (Recurrent__Forward_Pass__Residual / __Residual__FC / __Zero_Padded_Identity,
  * NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:563-817: loops over the time steps around the same functions). */
+static void fwd_lstm_layer(myea_oracle_net *n, size_t li, size_t B);
+
+/* the members, one after the other, each over all of its time steps (Recurrent__Forward_Pass__Residual__Layer,
+ * NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:711-771; feed-forward: Forward_Pass__Residual__Layer, :3999-4036) */
+static void fwd_residual_members(myea_oracle_net *n, size_t ri, size_t B)
+{
+    size_t last = ri + n->d.layers[ri].block_depth, T = n->d.number_recurrent_depth;
+    for (size_t li = ri + 1; li <= last; ++li) {
+        const myea_layer_desc *l = &n->d.layers[li];
+        if (l->type_layer == MYEA_LAYER_LSTM) fwd_lstm_layer(n, li, B);
+        else for (size_t t = 0; t < T; ++t) {
+            if (is_pooling(l)) fwd_pooling(n, li, t, B);
+            else fwd_residual_fc_layer(n, li, t, B);
+        }
+    }
+}
+
 static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t t, size_t B)
 {
     const myea_layer_desc *r = &n->d.layers[ri];
     olayer *o = &n->L[ri];
     size_t last = ri + r->block_depth, Bmax = n->d.batch_size;
-    /* Forward_Pass__Residual__Layer, :3999-4036: fully-connected and pooling members */
-    for (size_t li = ri + 1; li <= last; ++li) {
-        if (is_pooling(&n->d.layers[li])) fwd_pooling(n, li, t, B);
-        else fwd_residual_fc_layer(n, li, t, B);
-    }
     float *blk = layer_outputs(n, last);
     size_t nb = n->L[last].H, na = n->L[o->prev].H;
     if (layer_uses_norm(r)) {
@@ -812,7 +838,11 @@ static void fwd_residual_block(myea_oracle_net *n, size_t ri, size_t t, size_t B
      * dropout_values[0], each of its values then times its own U(-1, 1) draw; otherwise every value times 1 - dropout_values[0].
      * Draws as supplied: [mask per example][forward draws][backward draws]. */
     if (r->type_dropout == MYEA_DROPOUT_SHAKEDROP) {
-        const float *mask = o->noise, *alpha = o->noise + Bmax;
+        /* one mask per (time step, example), one draw per (time step, example, value): [T][Bmax] masks, then the forward
+         * draws [T][Bmax][width], then the backward draws (Recurrent__Forward_Pass__Dropout__ShakeDrop,
+         * NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:367-386, indexes the mask with batch_size x time step + example) */
+        const size_t T = n->d.number_recurrent_depth;
+        const float *mask = o->noise + t * Bmax, *alpha = o->noise + T * Bmax + t * Bmax * nb;
         for (size_t b = 0; b < B; ++b)
             for (size_t j = 0; j < nb; ++j) {
                 if (n->state == MYEA_STATE_TRAINING) { if (mask[b] != 0.f) blk[b * nb + j] *= alpha[b * nb + j]; }
@@ -1479,6 +1509,7 @@ int myea_oracle_forward_pass(myea_oracle_net *n, size_t B, const float *inputs)
         } else if (l->type_layer == MYEA_LAYER_LSTM) {
             fwd_lstm_layer(n, li, B);
         } else if (l->type_layer == MYEA_LAYER_RESIDUAL) {
+            fwd_residual_members(n, li, B);
             for (size_t t = 0; t < T; ++t) fwd_residual_block(n, li, t, B);
             li += l->block_depth; /* the iterator is left on the block's last member, :3884-3885 */
         } else if (is_pooling(l)) {
@@ -1753,7 +1784,7 @@ static void bwd_residual_fc_to_previous(myea_oracle_net *n, size_t gi, size_t t,
     const myea_layer_desc *g = &n->d.layers[gi];
     olayer *q = &n->L[gi];
     size_t Bmax = n->d.batch_size, D = q->In, at = t * Bmax * D;
-    if (q->group == 2) memcpy(dst + at, (layer_uses_norm(g) ? q->norm_errors : q->af_errors) + at, Bmax * D * sizeof(float));
+    if (q->group == 2) memcpy(dst + at, (layer_uses_norm(g) ? q->norm_errors : (is_ind_rnn(g) ? q->dafs : q->af_errors)) + at, Bmax * D * sizeof(float));
     else if (layer_uses_norm(g)) {
         for (size_t b = 0; b < B; ++b)
             for (size_t j = 0; j < D; ++j) dst[at + b * D + j] += q->norm_errors[at + b * D + j]; /* Backward_Pass__Identity, :1084-1108 */
@@ -1776,7 +1807,13 @@ static void bwd_gradient_residual_fc(myea_oracle_net *n, size_t li, size_t t, si
     memset(din + t * Bmax * In, 0, Bmax * In * sizeof(float));
     bwd_fc(n, t, B, o->H, In, o->neuron_errors, n->parameters + l->first_connection_index, din);
     const float *prev_out = layer_outputs(n, o->prev);
-    if (o->group == 2) {
+    if (o->group == 2 && is_ind_rnn(l)) {
+        /* :865-880: through the recurrence; what the member hands on is its dAFs (the AF errors keep the step's own share).
+         * Nothing undoes the dropout or the k-sparse filter on the way back. */
+        bwd_df_ind_rnn(n, t, B, In, n->parameters + l->first_connection_index + o->H * In, l->type_activation_function, l->activation_steepness,
+                       o->unit_af, o->unit_steep, o->pre_afs, o->values, din, o->dafs, o->af_errors);
+        din = o->dafs;
+    } else if (o->group == 2) {
         const float *pre_af = layer_uses_norm(l) ? o->normalizes : prev_out; /* ptr_array_pre_activation_functions */
         bwd_df(n, t, B, In, l->type_activation_function, l->activation_steepness, o->unit_af, o->unit_steep, pre_af, o->values, din, o->af_errors);
     }
@@ -1796,10 +1833,11 @@ static void bwd_residual_block_to_last(myea_oracle_net *n, size_t ri, size_t t, 
     /* Backward_Pass__Dropout__ShakeDrop (NN/Neural_Network__Backward_Pass__Loop.cpp:433-443, 1050-1078): the perturbed examples'
      * deltas times fresh U(0, 1) draws, one per value */
     if (r->type_dropout == MYEA_DROPOUT_SHAKEDROP) {
-        const float *mask = o->noise, *beta = o->noise + Bmax + Bmax * D;
+        const size_t T = n->d.number_recurrent_depth;
+        const float *mask = o->noise + t * Bmax, *beta = o->noise + T * Bmax + T * Bmax * D + t * Bmax * D;
         for (size_t b = 0; b < B; ++b)
             if (mask[b] != 0.f)
-                for (size_t j = 0; j < D; ++j) tmp[b * D + j] *= beta[b * D + j];
+                for (size_t j = 0; j < D; ++j) tmp[at + b * D + j] *= beta[b * D + j];
     }
     if (layer_uses_norm(r)) {
         int renorm = r->type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
@@ -1814,17 +1852,24 @@ static void bwd_gradient_residual(myea_oracle_net *n, size_t ri, size_t B)
 {
     const myea_layer_desc *r = &n->d.layers[ri];
     size_t Bmax = n->d.batch_size, T = n->d.number_recurrent_depth, last = ri + r->block_depth;
+    /* Recurrent__Backward_Pass__Gradient__Residual__Layer (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:885-1001): the
+     * member's delta is pulled from its consumer over all time steps first (descending for dense, pooling and residual
+     * consumers, ascending for an LSTM consumer), then the member reduces it */
     for (size_t li = last; li > ri; --li) {
         olayer *o = &n->L[li];
-        const int pooling = is_pooling(&n->d.layers[li]);
-        float *delta = pooling ? o->af_errors : o->neuron_errors;   /* Layer::ptr_array_derivative_outputs of the member */
+        const myea_layer_desc *l = &n->d.layers[li];
+        const int pooling = is_pooling(l), lstm = l->type_layer == MYEA_LAYER_LSTM;
+        float *delta = (pooling || lstm) ? o->af_errors : o->neuron_errors;   /* Layer::ptr_array_derivative_outputs of the member */
         memset(delta, 0, T * Bmax * o->H * sizeof(float));
-        for (size_t t = T; t-- > 0;) {   /* time steps in descending order, like every dense layer of a recurrent network */
+        if (li != last && n->d.layers[li + 1].type_layer == MYEA_LAYER_LSTM) {
+            for (size_t t = 0; t < T; ++t) bwd_lstm_to_previous(n, li + 1, t, B, delta);
+        } else for (size_t t = T; t-- > 0;) {
             if (li == last) bwd_residual_block_to_last(n, ri, t, B, delta);
             else if (is_pooling(&n->d.layers[li + 1])) bwd_pooling_to_previous(n, li + 1, t, B, delta);   /* :753-758, :767-772 */
             else bwd_residual_fc_to_previous(n, li + 1, t, B, delta);
-            if (!pooling) bwd_gradient_residual_fc(n, li, t, B);   /* a pooling member has nothing of its own to reduce (:802-804) */
         }
+        if (lstm) bwd_lstm_layer(n, li, B);
+        else if (!pooling) for (size_t t = T; t-- > 0;) bwd_gradient_residual_fc(n, li, t, B);   /* a pooling member has nothing of its own to reduce (:802-804) */
     }
 }
 
@@ -1933,9 +1978,9 @@ int myea_oracle_update_derivative_weight(myea_oracle_net *n, size_t B, size_t fi
             if (layer_uses_bias(l)) dw_bias(n, t, B, o->H, o->neuron_errors, n->gradient + l->first_bias_connection_index);
             /* Update_Derivative_Weight__FC_Ind_RNN (NN/Neural_Network__Recurrent_Update_Derivative_Weight__Loop.cpp:461-483),
              * from the second time step on: du += AF[t-1] * dAF[t] */
-            if (t != 0 && is_ind_rnn(l)) {
-                size_t Bmax = n->d.batch_size, H = o->H;
-                float *du = n->gradient + l->first_connection_index + H * o->In;
+            if (t != 0 && is_ind_rnn(l) && o->group != 1) {   /* a block's first member owns no recurrent unit (tmp_AF_size == 0) */
+                size_t Bmax = n->d.batch_size, H = o->group ? o->AH : o->H;
+                float *du = n->gradient + l->first_connection_index + o->H * o->In;
                 for (size_t b = 0; b < B; ++b)
                     for (size_t j = 0; j < H; ++j) du[j] += o->values[Bmax * H * (t - 1) + b * H + j] * o->dafs[Bmax * H * t + b * H + j];
             }
@@ -2167,9 +2212,9 @@ int myea_oracle_update_parameter(myea_oracle_net *n, size_t B, size_t training_s
      * 289-333): hidden layers only; the self weights of an independently recurrent layer clipped to its bounds */
     for (size_t li = 1; li + 1 < n->d.n_layers; ++li) {
         const myea_layer_desc *l = &n->d.layers[li];
-        if (!is_ind_rnn(l) || (l->constraint_recurrent_weight_lower_bound == 0.f && l->constraint_recurrent_weight_upper_bound == 0.f)) continue;
-        float *u = n->parameters + l->first_connection_index + n->L[li].H * n->L[li].In;
-        for (size_t j = 0; j < n->L[li].H; ++j) u[j] = clipf(u[j], l->constraint_recurrent_weight_lower_bound, l->constraint_recurrent_weight_upper_bound);
+        if (!is_ind_rnn(l) || n->L[li].group == 1 || (l->constraint_recurrent_weight_lower_bound == 0.f && l->constraint_recurrent_weight_upper_bound == 0.f)) continue;
+        float *u = n->parameters + l->first_connection_index + n->L[li].H * n->L[li].In;   /* one per recurrent activation unit */
+        for (size_t j = 0; j < (n->L[li].group ? n->L[li].AH : n->L[li].H); ++j) u[j] = clipf(u[j], l->constraint_recurrent_weight_lower_bound, l->constraint_recurrent_weight_upper_bound);
     }
     return MYEA_OK;
 }
@@ -2188,9 +2233,13 @@ const float *myea_oracle_tensor(myea_oracle_net *n, size_t li, int kind, size_t 
     case MYEA_TENSOR_SUMMATIONS: p = o->summations; break;
     case MYEA_TENSOR_ERRORS: p = (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL || is_pooling(&n->d.layers[li])) ? o->af_errors : o->neuron_errors; break;
     case MYEA_TENSOR_NORM_HATS: p = o->hats; c = T * n->d.batch_size * o->NH; break;
-    case MYEA_TENSOR_DROPOUT_NOISE: p = o->noise; if (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) c = n->d.batch_size * (1 + 2 * o->NH); break;
+    case MYEA_TENSOR_DROPOUT_NOISE:
+        p = o->noise;
+        if (n->d.layers[li].type_layer == MYEA_LAYER_RESIDUAL) c = T * n->d.batch_size * (1 + 2 * o->NH);
+        else c = T * n->d.batch_size * o->AH;
+        break;
     case MYEA_TENSOR_INPUT_SIDE_ERRORS:
-        if (o->group == 2) p = layer_uses_norm(&n->d.layers[li]) ? o->norm_errors : o->af_errors;
+        if (o->group == 2) p = layer_uses_norm(&n->d.layers[li]) ? o->norm_errors : (is_ind_rnn(&n->d.layers[li]) ? o->dafs : o->af_errors);
         else if (o->group == 1 && layer_uses_norm(&n->d.layers[li])) p = o->norm_errors;
         c = T * n->d.batch_size * o->In;
         break;

@@ -138,27 +138,51 @@ class GradientTerms:
         return sums, mags
 
 
+def _clip_factor(first_moment, gradient, beta1):
+    """the factor s a clipped update applied, read back from its first moment m = (1 - beta1) s g on the entries with the
+    largest gradients"""
+    top = np.argsort(np.abs(gradient))[-4096:]
+    return float(np.median(first_moment[top] / ((1.0 - beta1) * gradient[top])))
+
+
 def assert_first_adam_type_step_matches(gpu, cpu, twin, w, g_gpu, g_cpu, B, h, kinds, what, rel=1e-4, abs_=1e-5):
     """Update_Parameter from cleared optimizer state on three networks that hold the same parameters `w`: the device (its own
     gradient g_gpu), the oracle (its own gradient g_cpu) and a second oracle network `twin` that is handed the device's
     gradient.
     (a) Device against twin - the same gradient on both sides, so the update arithmetic alone: every parameter and every
-        entry of the optimizer vectors `kinds`, rel 1e-5; with clipping by the global norm rel 1e-4 / abs 1e-5, since the norm
-        is an fp32 sum over all parameters (ten million squares here) whose rounding depends on the order of summation - the
-        reference's own with its thread count - and scales every step.
+        entry of the optimizer vectors `kinds`, rel 1e-5.
     (b) Device against oracle, each from its own gradient: parameters within rel / abs and the optimizer vectors within the
         tolerance the gradient's own tolerance turns into (first moment (1 - beta1) s g, second moment (1 - beta2) (s g)^2,
         s the clipping factor), wherever the two gradients agree within rel / abs and the gradient is not below its own
         absolute tolerance.  An Adam-type step has the size lr whatever |g| is, so where |g| < abs_ - rounding noise of
-        either side - the step's direction is noise too: those parameters are held to the step's bound, 2.1 lr."""
+        either side - the step's direction is noise too: those parameters are held to the step's bound, 2.1 lr.
+    With clipping by the global norm every step carries one more scalar, s = clip / |g|, and |g| is an fp32 sum over all
+    parameters: the reference's serial loop over ten million squares stops taking in addends below half a unit in the last
+    place of its running sum (its OpenMP build, which sums per thread, lands elsewhere again), so its s is off in the fourth
+    digit.  The factor is therefore held on its own - the device's must be at least as near to clip / (the float64 norm) as
+    the oracle's, or within 1e-6 of it - and taken out of the entrywise comparisons of the optimizer vectors; the
+    parameters are compared as they are (an Adam-type step barely depends on the gradient's scale) and, in (a), also
+    against the float64 closed form of the step from the device's own optimizer vectors."""
     twin.upload_gradient(g_gpu)
     for n in (gpu, cpu, twin):
         n.Update_Parameter(B, B)
     wg, wc, wt = (n.download_parameters().astype(np.float64) for n in (gpu, cpu, twin))
-    e = np.abs(wg - wt)
-    arel, aabs = (rel, abs_) if h.use_clip_gradient else (1e-5, 1e-7)
-    assert not (e > aabs + arel * np.abs(wt)).any(), "%s: update arithmetic: %d parameters differ, worst %.3g" % (what, int((e > aabs + arel * np.abs(wt)).sum()), float(e.max()))
     gg, gc = np.asarray(g_gpu, np.float64), np.asarray(g_cpu, np.float64)
+    b1, b2 = float(h.adam_beta1), float(h.adam_beta2)
+    states = {kind: tuple(n.download_optimizer_state(mb.OPT_STATE[kind]).astype(np.float64) for n in (gpu, cpu, twin)) for kind in kinds}
+    clipped = bool(h.use_clip_gradient)
+    s_gpu = s_cpu = s_twin = 1.0
+    report = {}
+    if clipped:
+        m = states["FIRST_MOMENT"]
+        s_gpu, s_cpu, s_twin = _clip_factor(m[0], gg, b1), _clip_factor(m[1], gc, b1), _clip_factor(m[2], gg, b1)
+        exact = min(1.0, float(h.clip_gradient) / float(np.sqrt((gg * gg).sum())))
+        err_gpu, err_twin = abs(s_gpu / exact - 1.0), abs(s_twin / exact - 1.0)
+        assert err_gpu <= max(1e-6, err_twin), "%s: clipping factor %.9g, exact %.9g, oracle %.9g" % (what, s_gpu, exact, s_twin)
+        report.update(clip_factor_error=err_gpu, oracle_clip_factor_error=err_twin)
+    e = np.abs(wg - wt)
+    arel, aabs = (rel, abs_) if clipped else (1e-5, 1e-7)
+    assert not (e > aabs + arel * np.abs(wt)).any(), "%s: update arithmetic: %d parameters differ, worst %.3g" % (what, int((e > aabs + arel * np.abs(wt)).sum()), float(e.max()))
     agree = np.abs(gg - gc) <= abs_ + rel * np.abs(gc)
     strict = (agree & (np.abs(gc) >= abs_)) | ((gg == 0) & (gc == 0))
     e = np.abs(wg - wc)
@@ -166,17 +190,27 @@ def assert_first_adam_type_step_matches(gpu, cpu, twin, w, g_gpu, g_cpu, B, h, k
     assert not bad.any(), "%s: %d parameters differ from the oracle's, worst %.3g" % (what, int(bad.sum()), float(e[bad].max()))
     lr = float(h.adam_learning_rate)
     assert float(np.abs(wg - w)[~strict].max(initial=0.0)) <= 2.1 * lr, "%s: a parameter with a noise-level gradient moved by more than a step" % what
-    norm = float(np.sqrt((gc * gc).sum()))
-    s = min(1.0, float(h.clip_gradient) / norm) if h.use_clip_gradient and norm > 0 else 1.0
-    b1, b2 = float(h.adam_beta1), float(h.adam_beta2)
     for kind in kinds:
-        a, b, t = (n.download_optimizer_state(mb.OPT_STATE[kind]).astype(np.float64) for n in (gpu, cpu, twin))
+        a, b, t = states[kind]
+        power = 1 if kind == "FIRST_MOMENT" else 2
+        t = t * (s_gpu / s_twin) ** power     # the clipping factors taken out (1 without clipping)
+        b = b * (s_gpu / s_cpu) ** power
         e = np.abs(a - t)
-        assert not (e > 1e-30 + arel * np.abs(t)).any(), "%s: update arithmetic: optimizer vector %s: %d entries differ" % (what, kind, int((e > 1e-30 + arel * np.abs(t)).sum()))
+        assert not (e > 1e-30 + 1e-5 * np.abs(t)).any(), "%s: update arithmetic: optimizer vector %s: %d entries differ" % (what, kind, int((e > 1e-30 + 1e-5 * np.abs(t)).sum()))
         if kind == "FIRST_MOMENT":
-            tol = 1.1 * rel * np.abs(b) + (1.0 - b1) * s * 1.1 * abs_
+            tol = 1.1 * rel * np.abs(b) + (1.0 - b1) * s_gpu * 1.1 * abs_
         else:
-            tol = 2.2 * rel * np.abs(b) + (1.0 - b2) * s * s * (2.1 * np.abs(gc) * abs_ + abs_ * abs_)
+            tol = 2.2 * rel * np.abs(b) + (1.0 - b2) * s_gpu * s_gpu * (2.1 * np.abs(gc) * abs_ + abs_ * abs_)
         bad = agree & (np.abs(a - b) > tol)
         assert not bad.any(), "%s: optimizer vector %s: %d entries differ from the oracle's" % (what, kind, int(bad.sum()))
-    return dict(parameters=int(wg.size), compared_strictly=int(strict.sum()), noise_level_or_disagreeing_gradients=int((~strict).sum()))
+    if clipped and h.type_optimizer_function == mb.OPTIMIZER["ADABOUND"]:
+        # Update_Parameters__AdaBound (NN/Neural_Network__AdaBound.cpp:43-110), first step, from the device's own vectors
+        m, v = states["FIRST_MOMENT"][0], states["SECOND_MOMENT"][0]
+        lr_t = lr * np.sqrt(1.0 - b2) / (1.0 - b1) if h.use_adam_bias_correction else lr
+        lo = float(h.learning_rate_final) * (1.0 - 1.0 / (float(h.learning_gamma) + 1.0))
+        hi = float(h.learning_rate_final) * (1.0 + 1.0 / float(h.learning_gamma))
+        want = w - np.clip(lr_t / (np.sqrt(v) + float(h.adam_epsilon)), lo, hi) * m
+        e = np.abs(wg - want)
+        assert not (e > 1e-7 + 1e-5 * np.abs(want)).any(), "%s: parameters against the closed form of the step: %d differ, worst %.3g" % (what, int((e > 1e-7 + 1e-5 * np.abs(want)).sum()), float(e.max()))
+    report.update(parameters=int(wg.size), compared_strictly=int(strict.sum()), noise_level_or_disagreeing_gradients=int((~strict).sum()))
+    return report

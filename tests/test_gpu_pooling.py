@@ -95,6 +95,3 @@ def test_pooling_error_paths():
     with pytest.raises(mb.MyeaError) as e:
         mb.HipNetwork(desc)
     assert e.value.code == mb.E_INVALID and "pooling width" in str(e.value)
-    with pytest.raises(mb.MyeaError) as e:    # next to an LSTM layer
-        mb.HipNetwork(mb.make_desc([dict(units=6), dict(type="lstm", units=8), avg(kernel=2, stride=2), dict(units=8, activation="LINEAR")], 2, 3))
-    assert e.value.code == mb.E_UNSUPPORTED

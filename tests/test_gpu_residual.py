@@ -105,8 +105,7 @@ def test_residual_inference_forward_matches_oracle():
 
 def test_unsupported_residual_shapes_are_refused():
     B = 4
-    for specs, T in (([fc(4), res(1, dropout="SHAKEDROP", keep=0.5), fc(4), fc(2)], 3),                  # ShakeDrop with a recurrent depth
-                     ([fc(4), res(1, dropout="BERNOULLI", keep=0.5), fc(4), fc(2)], 1),                  # block-level dropout
+    for specs, T in (([fc(4), res(1, dropout="BERNOULLI", keep=0.5), fc(4), fc(2)], 1),                  # block-level dropout
                      ([fc(4), res(2), fc(4), fc(4, "SOFTMAX"), fc(2)], 1)):                              # softmax inside a block
         desc = mb.make_desc(specs, B, T, network=mb.NETWORK_FEEDFORWARD)
         with pytest.raises(mb.MyeaError):

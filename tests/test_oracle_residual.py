@@ -362,14 +362,6 @@ def test_member_dropout_acts_on_the_input_side_and_is_not_replayed_backward():
     assert_close(g[l4.first_connection_index:l4.last_connection_index].reshape(8, 7), d4.T @ v, 2e-4, 2e-6)
 
 
-def test_shakedrop_blocks_need_a_feed_forward_net():
-    B = 2
-    lib = load_oracle()
-    d = mb.make_desc([fc(4), res(1, dropout="SHAKEDROP", keep=0.5), fc(4), fc(2)], B, 3, lib=lib)         # recurrent depth 3
-    with pytest.raises(Exception):
-        OracleNetwork(d, oracle_hyper())
-
-
 RECURRENT_SPECS = [fc(5), fc(6, "TANH", normalization="BATCH_NORMALIZATION", norm_before=True),
                    res(2, normalization="BATCH_NORMALIZATION"),
                    fc(7, "TANH", normalization="BATCH_NORMALIZATION"), fc(8, "SIGMOID", dropout="BERNOULLI_INVERTED", keep=0.5),
