@@ -30,6 +30,8 @@ RECORDED_TRAFFIC = {"fc4096x4_b1024_adam": dict(bytes_per_launch=2944490 * 1024 
                     # the two resident time loops of one layer (forward + backward launch), mean per launch
                     "lstm512x2_t64_b256_amsgrad": dict(bytes_per_launch=(299.0e6 + 400.0e6) / 2,
                                                        source="recorded constant, not measured in this run: profiles/lstm_resident__lstm512x2_t64_b256_amsgrad__pmc.txt")}
+from myea_amd.synthetic import simple_debug_layers  # noqa: E402  (no device is touched by the import)
+
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
@@ -68,30 +70,41 @@ WORKLOADS = {
                + [dict(units=100, activation="SOFTMAX")],
         batch=512, head="SOFTMAX", optimizer="GD", loss="CROSS_ENTROPY", data="normal",
         hyper=dict(learning_rate=0.01, learning_momentum=0.9, use_Nesterov=1)),
+    # the reference's worked example (Neural_Network_Launcher_Windows/Source_Files/debug.cpp:36-1555): sMNIST rows (28 inputs x 28
+    # time steps, the label read at the last one), residual blocks of independently recurrent ISRLU members with batch
+    # normalisation, max pooling between the groups, softmax head, AMSGrad at 1e-3, max-norm constraint 8
+    "resindrnn_smnist28_t28_b256_amsgrad": dict(
+        layers=simple_debug_layers(), batch=256, depth=28, head="SOFTMAX", optimizer="AMSGRAD", loss="CROSS_ENTROPY", data="uniform",
+        hyper=dict(adam_learning_rate=1e-3, regularization__max_norm_constraints=8.0, normalization_momentum_average=1.0,
+                   normalization_epsilon=0.1, number_time_delays=27)),
 }
 
 
 def gemm_flops_per_step(layers, batch, depth=1):
-    """2*M*N*K of forward, dX (layers 2..) and dW; LSTM layers: 4 gate rows per cell, input contraction at every
-    step, recurrent contraction at T-1 steps."""
-    w = [l.get("units", 0) * l.get("cells_per_block", 1) for l in layers]
+    """2*M*N*K of forward, dX (every layer whose producer is not the input layer) and dW; LSTM layers: 4 gate rows per cell, input
+    contraction at every step, recurrent contraction at T-1 steps.  Widths come from the laid-out description (pooling layers
+    and residual blocks change them and own no contraction)."""
+    from myea_amd import binding as mb
+    lib = mb.load_library()
+    desc = mb.make_desc(layers, batch, depth)
     fwd = dx = 0.0
-    prev = 0   # index of the producer (residual layers own no weights and keep the block's width here: equal widths)
-    for i in range(1, len(w)):
-        if layers[i].get("type") == "residual":
-            w[i] = w[prev]
+    for i in range(1, desc.n_layers):
+        l = desc.layers[i]
+        if l.type_layer in (mb.LAYER_RESIDUAL, mb.LAYER_AVERAGE_POOLING, mb.LAYER_MAX_POOLING):
             continue
-        if layers[i].get("type") == "lstm":
-            dirs = 2 if layers[i].get("bidirectional") else 1
-            gates = w[i] + 3 * layers[i]["units"]
-            f_in, f_rec = 2.0 * dirs * batch * depth * gates * w[prev], 2.0 * dirs * batch * (depth - 1) * gates * w[i]
+        prev = lib.myea_net_desc_previous_layer(desc, i)
+        fan_in, width = lib.myea_net_desc_number_outputs(desc, prev), lib.myea_net_desc_number_outputs(desc, i)
+        if l.type_layer == mb.LAYER_LSTM:
+            dirs = 2 if l.use_bidirectional else 1
+            cells = l.n_units * l.n_cells_per_block
+            gates = cells + 3 * l.n_units
+            f_in, f_rec = 2.0 * dirs * batch * depth * gates * fan_in, 2.0 * dirs * batch * (depth - 1) * gates * cells
             fwd += f_in + f_rec
-            dx += f_rec + (f_in if i >= 2 else 0.0)
+            dx += f_rec + (f_in if prev != 0 else 0.0)
         else:
-            f = 2.0 * batch * depth * w[i] * w[prev]
+            f = 2.0 * batch * depth * width * fan_in
             fwd += f
-            dx += f if i >= 2 else 0.0
-        prev = i
+            dx += f if prev != 0 else 0.0
     return fwd + dx + fwd
 
 
@@ -262,7 +275,9 @@ def config_of(r):
     wl = r["wl"]
     return {"workload": r["workload"], "batch": r["batch"], "sequence_length": wl.get("depth", 1),
             "layers": ["res%d" % l["block_depth"] if l.get("type") == "residual" else
-                       ("bilstm%d" if l.get("bidirectional") else "lstm%d" if l.get("type") == "lstm" else "fc%d") % l["units"] for l in wl["layers"]],
+                       "%s_k%d_s%d" % (l["type"], l["kernel"], l["stride"]) if "pooling" in l.get("type", "") else
+                       ("bilstm%d" if l.get("bidirectional") else "lstm%d" if l.get("type") == "lstm" else
+                        "indrnn%d" if l.get("type") == "ind_rnn" else "fc%d") % l["units"] for l in wl["layers"]],
             "optimizer": wl["optimizer"], "parameters": r["desc_parameters"],
             "gemm_flops_per_step": gemm_flops_per_step(wl["layers"], r["batch"], wl.get("depth", 1))}
 

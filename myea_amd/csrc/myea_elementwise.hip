@@ -1158,6 +1158,172 @@ int launch_bn_backward_from_sums(hipStream_t s, const BnBackwardParams &p, const
     return MYEA_OK;
 }
 
+// Every time step of a [T][Bmax][H] tensor in one launch.  Each time step has statistics of its own (the reference runs the
+// layer's normalisation once per time step); workgroup (column block, t) owns 64 columns of time step t over all of its rows:
+// the column sums meet in LDS (four row lanes), one lane per column finishes the statistics exactly as bn_forward_final_kernel
+// does, then the workgroup applies them as bn_forward_apply_kernel does.  p's per-time-step vectors (mean, var, averages,
+// corrections, colscale) are those of time step 0, H apart from one step to the next; its tensors those of time step 0,
+// Bmax * H apart.  training == 0: the running averages of each time step, nothing written but the output.
+template <int CW>   // columns per workgroup: 64, or 16 for narrow layers (more row lanes, shorter loops)
+__global__ __launch_bounds__(kBlock) void bn_forward_sequence_kernel(BnForwardParams p, size_t Bmax, int training)
+{
+    constexpr int kLanes = kBlock / CW;
+    __shared__ double s_sum[kLanes][CW], s_sq[kLanes][CW];
+    __shared__ float s_stat[4][CW];
+    const int c = threadIdx.x % CW, rl = threadIdx.x / CW;
+    const size_t t = blockIdx.y, j = (size_t)blockIdx.x * CW + c;
+    const bool live = j < p.H;
+    const size_t base = t * Bmax * p.H, sj = t * p.H + j;
+    if (training) {
+        double sm = 0.0, sv = 0.0;
+        if (live) {
+#pragma unroll 8
+            for (size_t r = rl; r < p.rows; r += kLanes) { const double v = p.x[base + r * p.H + j]; sm += v; sv += v * v; }
+        }
+        s_sum[rl][c] = sm; s_sq[rl][c] = sv;
+        __syncthreads();
+        if (rl == 0 && live) {
+            double smd = 0.0, svd = 0.0;
+#pragma unroll
+            for (int k = 0; k < kLanes; ++k) { smd += s_sum[k][c]; svd += s_sq[k][c]; }
+            const float bscale = 1.f / (float)p.rows;
+            const float mean = (float)smd * bscale;
+            float mavg = p.mean_avg[sj];
+            mavg += p.momentum * (mean - mavg);
+            p.mean_avg[sj] = mavg;
+            const float var = sqrtf((float)svd * bscale - mean * mean + p.epsilon);
+            float vavg = p.var_avg[sj];
+            vavg += p.momentum * (var - vavg);
+            p.var_avg[sj] = vavg;
+            p.mean[sj] = mean;
+            p.var[sj] = var;
+            float rc = 1.f, dc = 0.f;
+            if (p.renorm) {
+                const float g = var / vavg, lo = 1.f / p.r_max;
+                rc = g < lo ? lo : (g > p.r_max ? p.r_max : g);
+                const float d = (mean - mavg) / vavg;
+                dc = d < -p.d_max ? -p.d_max : (d > p.d_max ? p.d_max : d);
+                p.r_corr[sj] = rc; p.d_corr[sj] = dc;
+            }
+            s_stat[0][c] = mean; s_stat[1][c] = var; s_stat[2][c] = rc; s_stat[3][c] = dc;
+        }
+        __syncthreads();
+    }
+    if (!live) return;
+    const float scale = p.scale[j], shift = p.shift[j];
+    if (!training) {
+        const float mavg = p.mean_avg[sj], vavg = p.var_avg[sj];
+        for (size_t r = rl; r < p.rows; r += kLanes) {
+            const size_t i = base + r * p.H + j;
+            p.normalizes[i] = scale * ((p.x[i] - mavg) / vavg) + shift;
+        }
+        return;
+    }
+    const float mean = s_stat[0][c], var = s_stat[1][c], rc = s_stat[2][c], dc = s_stat[3][c];
+    const float cs = p.colscale ? p.colscale[sj] : 1.f;
+#pragma unroll 4
+    for (size_t r = rl; r < p.rows; r += kLanes) {
+        const size_t i = base + r * p.H + j;
+        float h = (p.x[i] - mean) / var;
+        if (p.renorm) h = h * rc + dc;
+        p.hats[i] = h;
+        const float y = scale * h + shift;
+        p.normalizes[i] = y;
+        if (p.act_out) {
+            float v = af_fire(p.act, y);
+            if (p.colscale) v *= cs;
+            p.act_out[i] = v;
+        }
+    }
+}
+
+int launch_bn_forward_sequence(hipStream_t s, const BnForwardParams &p, size_t T, size_t Bmax, int training)
+{
+    if (p.H == 0 || p.rows == 0 || T == 0) return MYEA_OK;
+    if (p.rows > Bmax || T > 65535) { set_last_error("bn_forward_sequence: %zu rows of %zu, %zu time steps", p.rows, Bmax, T); return MYEA_E_INVALID; }
+    if (p.H <= 32) hipLaunchKernelGGL(bn_forward_sequence_kernel<16>, dim3((unsigned)((p.H + 15) / 16), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, training);
+    else hipLaunchKernelGGL(bn_forward_sequence_kernel<64>, dim3((unsigned)((p.H + 63) / 64), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, training);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+// The backward pass of the same, every time step in one launch: the four column sums of BnBackF in LDS, the last loop of
+// bn_backward_apply_kernel behind them.  The shares of the scale's and the shift's gradient - one per time step, all onto the
+// same two vectors - go to `partial` ([T][2][H]) and are added by bn_backward_sequence_final_kernel in descending time-step
+// order, the order the launches per time step add them in.
+template <int CW>
+__global__ __launch_bounds__(kBlock) void bn_backward_sequence_kernel(BnBackwardParams p, size_t Bmax, float *__restrict__ partial)
+{
+    constexpr int kLanes = kBlock / CW;
+    __shared__ double s_acc[4][kLanes][CW];
+    __shared__ float s_d[2][CW];
+    const int c = threadIdx.x % CW, rl = threadIdx.x / CW;
+    const size_t t = blockIdx.y, j = (size_t)blockIdx.x * CW + c;
+    const bool live = j < p.H;
+    const size_t base = t * Bmax * p.H, sj = t * p.H + j;
+    float vb = 1.f, rc = 1.f, mean = 0.f, scale = 0.f;
+    if (live) { vb = p.var[sj]; rc = p.renorm ? p.r_corr[sj] : 1.f; mean = p.mean[sj]; scale = p.scale[j]; }
+    double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
+    if (live) {
+#pragma unroll 4
+        for (size_t r = rl; r < p.rows; r += kLanes) {
+            const size_t k = base + r * p.H + j;
+            float e = p.dy[k];
+            a0 += e * p.hats[k];
+            a1 += e;
+            e *= scale;
+            a2 += e * (-rc / vb);
+            a3 += e * (p.x[k] - mean) * (-rc / (vb * vb));
+        }
+    }
+    s_acc[0][rl][c] = a0; s_acc[1][rl][c] = a1; s_acc[2][rl][c] = a2; s_acc[3][rl][c] = a3;
+    __syncthreads();
+    if (rl == 0 && live) {
+        double b[4] = {0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int k = 0; k < kLanes; ++k) b[q] += s_acc[q][k][c];
+        partial[(t * 2 + 0) * p.H + j] = (float)b[0];
+        partial[(t * 2 + 1) * p.H + j] = (float)b[1];
+        s_d[0][c] = (float)b[2]; s_d[1][c] = (float)b[3];
+    }
+    __syncthreads();
+    if (!live) return;
+    const float dmean = s_d[0][c], dvar = s_d[1][c];
+    const float bsz = (float)p.rows, bscale = 1.f / (float)p.rows;
+#pragma unroll 4
+    for (size_t r = rl; r < p.rows; r += kLanes) {
+        const size_t i = base + r * p.H + j;
+        float e = p.dy[i] * scale;
+        e *= rc / vb;
+        e += dvar * ((p.x[i] - mean) / (bsz * vb));
+        e += dmean * bscale;
+        p.dx[i] = e;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void bn_backward_sequence_final_kernel(size_t H, size_t T, const float *__restrict__ partial, float *dscale, float *dshift)
+{
+    const size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (j >= H) return;
+    float a = dscale[j], b = dshift[j];
+    for (size_t t = T; t-- > 0;) { a += partial[(t * 2 + 0) * H + j]; b += partial[(t * 2 + 1) * H + j]; }
+    dscale[j] = a; dshift[j] = b;
+}
+
+int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t T, size_t Bmax, float *scratch)
+{
+    if (p.H == 0 || p.rows == 0 || T == 0) return MYEA_OK;
+    if (p.rows > Bmax || T > 65535) { set_last_error("bn_backward_sequence: %zu rows of %zu, %zu time steps", p.rows, Bmax, T); return MYEA_E_INVALID; }
+    if (p.H <= 32) hipLaunchKernelGGL(bn_backward_sequence_kernel<16>, dim3((unsigned)((p.H + 15) / 16), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, scratch);
+    else hipLaunchKernelGGL(bn_backward_sequence_kernel<64>, dim3((unsigned)((p.H + 63) / 64), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, scratch);
+    MYEA_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(bn_backward_sequence_final_kernel, dim3(grid_for(p.H, kBlock)), dim3(kBlock), 0, s, p.H, T, scratch, p.dscale, p.dshift);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
 int launch_bn_forward_inference(hipStream_t s, size_t rows, size_t H, const float *x, const float *scale, const float *shift,
                                 const float *mean_avg, const float *var_avg, float *normalizes)
 {
@@ -1324,11 +1490,23 @@ __global__ __launch_bounds__(kBlock) void slab_sum_add_kernel(size_t n, int nsla
     }
 }
 
+// the same value by value, for slices that are no aligned multiple of four floats
+__global__ __launch_bounds__(kBlock) void slab_sum_add_scalar_kernel(size_t n, int nslab, const float *__restrict__ slabs, float *__restrict__ dst)
+{
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+        float v = slabs[i];
+        for (int s = 1; s < nslab; ++s) v += slabs[(size_t)s * n + i];
+        dst[i] += v;
+    }
+}
+
 int launch_slab_sum_add(hipStream_t s, size_t n, int nslab, const float *slabs, float *dst)
 {
     if (n == 0 || nslab <= 0) return MYEA_OK;
-    if ((n & 3) || (reinterpret_cast<uintptr_t>(slabs) & 15u) || (reinterpret_cast<uintptr_t>(dst) & 15u)) { set_last_error("slab sum: operands must be 16-byte aligned multiples of 4"); return MYEA_E_INVALID; }
-    hipLaunchKernelGGL(slab_sum_add_kernel, dim3(grid_for(n / 4, kBlock, 8192)), dim3(kBlock), 0, s, n, nslab, slabs, dst);
+    if ((n & 3) || (reinterpret_cast<uintptr_t>(slabs) & 15u) || (reinterpret_cast<uintptr_t>(dst) & 15u))
+        hipLaunchKernelGGL(slab_sum_add_scalar_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, n, nslab, slabs, dst);
+    else
+        hipLaunchKernelGGL(slab_sum_add_kernel, dim3(grid_for(n / 4, kBlock, 8192)), dim3(kBlock), 0, s, n, nslab, slabs, dst);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }

@@ -653,7 +653,10 @@ int gemm_split_k(int M, int N, int K)
         // long k (weight gradients over T x batch rows): enough slabs for ~1000 workgroups of 128 x 64, each slab at least
         // 1024 k's deep - the larger tile's operand reuse is worth more than the pass over the slabs that sums them
         want = (512 + tiles_128 - 1) / tiles_128;
-        if (want > K / 1024) want = K / 1024;
+        // (a product no larger than one 64 x 64 tile has no operand reuse to protect: slabs 256 k's deep, up to 32 of them)
+        const long depth = (M <= 64 && N <= 64) ? 256 : 1024;
+        if (want > K / depth) want = K / depth;
+        if (depth == 256) { if (want > 32) want = 32; if (want < 1) want = 1; const int c = (int)(((K + want - 1) / want + kBK - 1) / kBK * kBK); return (K + c - 1) / c; }
     } else {
         const long tiles_64 = (long)((M + 63) / 64) * ((N + 63) / 64);
         want = (256 + tiles_64 - 1) / tiles_64;

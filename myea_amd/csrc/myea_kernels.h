@@ -145,6 +145,10 @@ int launch_bn_backward(hipStream_t s, const BnBackwardParams &p, float *scratch 
 // the same from column sums the producing contraction left ([blocks][2][H]: sums of dy * hats and of dy per block of rows);
 // plain batch normalisation only
 int launch_bn_backward_from_sums(hipStream_t s, const BnBackwardParams &p, const float *sums, size_t blocks);
+// every time step of a [T][Bmax][H] tensor in one launch (statistics per time step): p's tensors and per-time-step vectors are
+// those of time step 0; p.rows <= Bmax rows of each time step take part.  scratch: 2 * T * H floats
+int launch_bn_forward_sequence(hipStream_t s, const BnForwardParams &p, size_t T, size_t Bmax, int training);
+int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t T, size_t Bmax, float *scratch);
 
 // output-layer delta + loss / accuracy accumulation
 struct ErrorParams {

@@ -151,6 +151,9 @@ struct Net {
     int bn_forward(size_t li, size_t t, size_t rows, const float *x, bool training, float *act_out = nullptr, const float *colscale = nullptr,
                    const float *sums = nullptr, size_t sum_blocks = 0);
     int bn_backward(size_t li, size_t t, size_t rows, const float *x, const float *dy, float *dx, const float *sums = nullptr, size_t sum_blocks = 0);
+    // the normalisation of layer li over all time steps of [T][batch_size][width] tensors
+    int bn_forward_all(size_t li, size_t B, const float *x, bool training, float *act_out = nullptr, const float *colscale = nullptr);
+    int bn_backward_all(size_t li, size_t B, const float *x, const float *dy, float *dx);
     int backward_into_layer(size_t li, size_t B);
     int pool_backward_with_shortcut(size_t gi, size_t rows, size_t roff, const DevLayer *shortcut, long crop, float *dst);
     int forward_residual_block(size_t ri, size_t B);

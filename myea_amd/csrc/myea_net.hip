@@ -378,6 +378,7 @@ int Net::create(const myea_net_desc &desc)
     MYEA_TRY(dev_alloc(&tmp2, T * B * max_h));
     {
         size_t need = 258 * max_h + 2048;
+        if (2 * T * max_h > need) need = 2 * T * max_h;   // a sequence's normalisation: the scale / shift gradient shares per time step
         if (lstm_scratch_floats() > need) need = lstm_scratch_floats();
         MYEA_TRY(dev_alloc(&scratch, need));
         scratch_floats = need;
@@ -471,6 +472,14 @@ static bool bn_sums_from_gemm(bool backward = false)
     return (mode & (backward ? 2 : 1)) != 0;
 }
 
+// The normalisation of every time step of a [T][Bmax][width] tensor: one launch for the whole sequence (each time step keeps
+// statistics of its own); MYEA_BN_SEQUENCE=0 in the environment keeps one set of launches per time step (for A / B runs).
+static bool bn_sequence_allowed()
+{
+    static const bool on = [] { const char *e = std::getenv("MYEA_BN_SEQUENCE"); return !(e && e[0] == '0'); }();
+    return on;
+}
+
 int Net::forward_fc_layer(size_t li, size_t B)
 {
     const myea_layer_desc &l = d.layers[li];
@@ -483,8 +492,11 @@ int Net::forward_fc_layer(size_t li, size_t B)
     const bool ind = layer_is_ind_rnn(l);
     bool drop = false;
     MYEA_TRY(refresh_colscale(li, &drop));
-    // all time steps in one launch when the rows are contiguous and nothing is per time step
-    const bool per_t = T > 1 && (B != Bmax || norm || (drop && !ind));
+    // all time steps in one launch when the rows are contiguous and nothing is per time step; a normalisation in front of the
+    // activation has its own statistics per time step inside one launch (with the activation and the dropout multiplier of each)
+    const bool af_in_bn_ok = training && !ind && !softmax && !o.unit_act;
+    const bool seq_bn = T > 1 && norm && before && B == Bmax && bn_sequence_allowed() && 2 * T * H <= scratch_floats && (ind || !drop || af_in_bn_ok);
+    const bool per_t = T > 1 && !seq_bn && (B != Bmax || norm || (drop && !ind));
     const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
     for (size_t c = 0; c < chunks; ++c) {
         const size_t roff = c * Bmax;  // first row of the chunk
@@ -501,7 +513,7 @@ int Net::forward_fc_layer(size_t li, size_t B)
         g.aux_out = fuse_af ? o.values + roff * H : nullptr;
         g.colscale = (fuse_af && !norm) ? cs : nullptr;
         // a batch normalisation in front of the activation, training: its column sums leave with the contraction's tiles
-        const bool sums_from_gemm = norm && before && training && o.norm_partials && bn_sums_from_gemm() && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H;
+        const bool sums_from_gemm = !seq_bn && norm && before && training && o.norm_partials && bn_sums_from_gemm() && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H;
         if (sums_from_gemm) g.col_partials = o.norm_partials;
         pair_buffers(&g, gemm_pair_partials, gemm_pair_tickets);   // forward contractions run one at a time on this stream
         prof_begin(0);
@@ -512,7 +524,8 @@ int Net::forward_fc_layer(size_t li, size_t B)
         // training: the activation of a layer normalised first rides in the normalisation's last pass
         const bool af_in_bn = norm && before && training && !ind && !softmax && !o.unit_act;
         if (norm && before) {
-            MYEA_TRY(bn_forward(li, c, rows, cur, training, af_in_bn ? o.values + roff * H : nullptr, cs, sums_from_gemm ? o.norm_partials : nullptr, (rows + 31) / 32));
+            if (seq_bn) MYEA_TRY(bn_forward_all(li, B, cur, training, af_in_bn ? o.values : nullptr, cs));
+            else MYEA_TRY(bn_forward(li, c, rows, cur, training, af_in_bn ? o.values + roff * H : nullptr, cs, sums_from_gemm ? o.norm_partials : nullptr, (rows + 31) / 32));
             cur = o.normalizes + roff * H;
         }
         if (ind) continue;   // the recurrence and the activation follow for the whole sequence
@@ -587,6 +600,53 @@ int Net::bn_forward(size_t li, size_t t, size_t rows, const float *x, bool train
     prof_begin(kProfNormalization);
     const int rc = (sums && !p.renorm) ? launch_bn_forward_training_from_sums(stream, p, sums, sum_blocks) : launch_bn_forward_training(stream, p, scratch);
     prof_end((double)rows * (double)H * sizeof(float) * (act_out ? 4.0 : 3.0));
+    return rc;
+}
+
+int Net::bn_forward_all(size_t li, size_t B, const float *x, bool training, float *act_out, const float *colscale)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, H = o.NH;
+    if (T == 1 || !bn_sequence_allowed() || 2 * T * H > scratch_floats) {
+        for (size_t t = 0; t < T; ++t)
+            MYEA_TRY(bn_forward(li, t, B, x + t * Bmax * H, training, act_out ? act_out + t * Bmax * H : nullptr, colscale ? colscale + t * H : nullptr));
+        return MYEA_OK;
+    }
+    BnForwardParams p{};
+    p.rows = B; p.H = H; p.x = x;
+    p.scale = scale_ptr(parameters, li); p.shift = shift_ptr(parameters, li);
+    p.mean = o.means; p.var = o.variances; p.mean_avg = o.means_averages; p.var_avg = o.variances_averages;
+    p.r_corr = o.r_corrections; p.d_corr = o.d_corrections;
+    p.hats = o.hats; p.normalizes = o.normalizes;
+    p.epsilon = h.normalization_epsilon; p.momentum = h.normalization_momentum_average;
+    p.r_max = h.batch_renormalization_r_correction_maximum; p.d_max = h.batch_renormalization_d_correction_maximum;
+    p.renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    p.act_out = act_out; p.colscale = colscale; p.act = (int)l.type_activation_function;
+    prof_begin(kProfNormalization);
+    const int rc = launch_bn_forward_sequence(stream, p, T, Bmax, training ? 1 : 0);
+    prof_end((double)T * (double)B * (double)H * sizeof(float) * (training ? (act_out ? 4.0 : 3.0) : 2.0));
+    return rc;
+}
+
+int Net::bn_backward_all(size_t li, size_t B, const float *x, const float *dy, float *dx)
+{
+    const myea_layer_desc &l = d.layers[li];
+    DevLayer &o = L[li];
+    const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, H = o.NH;
+    if (T == 1 || !bn_sequence_allowed() || 2 * T * H > scratch_floats) {
+        for (size_t t = T; t-- > 0;) MYEA_TRY(bn_backward(li, t, B, x + t * Bmax * H, dy + t * Bmax * H, dx + t * Bmax * H));
+        return MYEA_OK;
+    }
+    BnBackwardParams p{};
+    p.rows = B; p.H = H; p.x = x; p.hats = o.hats; p.dy = dy;
+    p.mean = o.means; p.var = o.variances; p.scale = scale_ptr(parameters, li); p.r_corr = o.r_corrections;
+    p.dscale = scale_ptr(gradient, li); p.dshift = shift_ptr(gradient, li);
+    p.dx = dx;
+    p.renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
+    prof_begin(kProfNormalization);
+    const int rc = launch_bn_backward_sequence(stream, p, T, Bmax, scratch);
+    prof_end((double)T * (double)B * (double)H * sizeof(float) * 3.0);
     return rc;
 }
 
@@ -716,6 +776,14 @@ int Net::forward_residual_block(size_t ri, size_t B)
     const myea_layer_desc &r = d.layers[ri];
     const size_t last = ri + r.block_depth, T = d.number_recurrent_depth, Bmax = d.batch_size;
     const bool training = state >= MYEA_STATE_TRAINING;
+    // Launches that treat every row alike cover the whole sequence when the batch fills the network's rows (the time steps are
+    // then contiguous); one per time step otherwise, or when something differs from one time step to the next (by_step)
+    auto chunked = [&](bool by_step, auto &&launch) -> int {
+        const bool split = T > 1 && (by_step || B != Bmax);
+        const size_t n = split ? T : 1, rows = split ? B : T * B;
+        for (size_t c = 0; c < n; ++c) MYEA_TRY(launch(c, c * Bmax, rows));
+        return MYEA_OK;
+    };
     bool values_ready = false;  // the member's activation values were written by the previous member's contractions
     for (size_t m = ri + 1; m <= last; ++m) {
         const myea_layer_desc &l = d.layers[m];
@@ -728,18 +796,16 @@ int Net::forward_residual_block(size_t ri, size_t B)
             continue;
         }
         if (layer_is_pooling(l)) {   // a pooling member (Forward_Pass__Residual__Layer, :4005-4030): windows over the member before it
-            for (size_t t = 0; t < T; ++t) {
-                const size_t roff = t * Bmax;
-                MYEA_TRY(launch_pool_forward(stream, pool_params(m, B), x + roff * In, o.values + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr));
-            }
+            MYEA_TRY(chunked(false, [&](size_t, size_t roff, size_t rows) {
+                return launch_pool_forward(stream, pool_params(m, rows), x + roff * In, o.values + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr);
+            }));
             values_ready = false;
             continue;
         }
         bool drop = false;
         if (o.group == 2) MYEA_TRY(refresh_colscale(m, &drop));
         const bool norm = layer_uses_norm(l), ind = o.group == 2 && layer_is_ind_rnn(l);
-        if (norm)
-            for (size_t t = 0; t < T; ++t) MYEA_TRY(bn_forward(m, t, B, x + t * Bmax * In, training));
+        if (norm) MYEA_TRY(bn_forward_all(m, B, x, training));
         const float *in = norm ? o.normalizes : x;
         if (ind) {   // the recurrence and the activation over the whole sequence; Bernoulli dropout in place on what the next step reads
             IndRnnParams p{};
@@ -749,6 +815,27 @@ int Net::forward_residual_block(size_t ri, size_t B)
             p.in = in; p.pre_afs = o.pre_afs; p.afs = o.values;
             p.colscale = drop ? o.colscale : nullptr;
             MYEA_TRY(launch_ind_rnn_forward(stream, p));
+        }
+        if (o.group == 2) {
+            if (!ind && !values_ready)
+                MYEA_TRY(chunked(drop, [&](size_t t, size_t roff, size_t rows) {
+                    return launch_activation(stream, (int)l.type_activation_function, rows, In, in + roff * In, o.values + roff * In, drop ? o.colscale + t * o.AH : nullptr, o.unit_act);
+                }));
+            // Gaussian / Uout dropout, strictly in the training state, then the k-sparse filter (:4197-4274)
+            if (o.noise && state == MYEA_STATE_TRAINING) {
+                if (!o.noise_uploaded) {
+                    const bool normal = l.type_dropout == MYEA_DROPOUT_GAUSSIAN;
+                    MYEA_TRY(launch_dropout_noise(stream, T * Bmax * In, o.noise, normal ? 1 : 0, normal ? 1.f : -l.dropout_values[0], l.dropout_values[0], dropout_seed, dropout_stream++));
+                }
+                MYEA_TRY(chunked(false, [&](size_t, size_t roff, size_t rows) {
+                    return launch_dropout_noise_apply(stream, rows * In, o.values + roff * In, o.noise + roff * In, l.type_dropout == MYEA_DROPOUT_UOUT);
+                }));
+            }
+            if (l.k_sparsity != 0) {
+                const size_t k = state == MYEA_STATE_TRAINING ? (size_t)l.k_sparsity : (size_t)(l.alpha_sparsity * (float)l.k_sparsity);
+                MYEA_TRY(chunked(false, [&](size_t, size_t roff, size_t rows) { return launch_k_sparse(stream, rows, In, k, o.values + roff * In); }));
+            }
+            in = o.values;
         }
         // what the contractions of this member leave for the next one: its activation values, when only an activation and a
         // Bernoulli multiplier stand between the two
@@ -760,32 +847,12 @@ int Net::forward_residual_block(size_t ri, size_t B)
         }
         bool next_drop = false;
         if (feeds_next) MYEA_TRY(refresh_colscale(m + 1, &next_drop));
-        for (size_t t = 0; t < T; ++t) {
-            const size_t roff = t * Bmax;
-            const float *cur = in + roff * In;
-            if (o.group == 2) {
-                float *vals = o.values + roff * In;
-                if (!ind && !values_ready)
-                    MYEA_TRY(launch_activation(stream, (int)l.type_activation_function, B, In, cur, vals, drop ? o.colscale + t * o.AH : nullptr, o.unit_act));
-                // Gaussian / Uout dropout, strictly in the training state, then the k-sparse filter (:4197-4274)
-                if (o.noise && state == MYEA_STATE_TRAINING) {
-                    if (t == 0 && !o.noise_uploaded) {
-                        const bool normal = l.type_dropout == MYEA_DROPOUT_GAUSSIAN;
-                        MYEA_TRY(launch_dropout_noise(stream, T * Bmax * In, o.noise, normal ? 1 : 0, normal ? 1.f : -l.dropout_values[0], l.dropout_values[0], dropout_seed, dropout_stream++));
-                    }
-                    MYEA_TRY(launch_dropout_noise_apply(stream, B * In, vals, o.noise + roff * In, l.type_dropout == MYEA_DROPOUT_UOUT));
-                }
-                if (l.k_sparsity != 0) {
-                    const size_t k = state == MYEA_STATE_TRAINING ? (size_t)l.k_sparsity : (size_t)(l.alpha_sparsity * (float)l.k_sparsity);
-                    MYEA_TRY(launch_k_sparse(stream, B, In, k, vals));
-                }
-                cur = vals;
-            }
+        MYEA_TRY(chunked(next_drop, [&](size_t t, size_t roff, size_t rows) {
             GemmParams g{};
-            g.A = cur; g.lda = (long)In; g.a_k_contiguous = 1;
+            g.A = in + roff * In; g.lda = (long)In; g.a_k_contiguous = 1;
             g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 1;
             g.C = o.summations + roff * H; g.ldc = (long)H;
-            g.M = (int)B; g.N = (int)H; g.K = (int)In;
+            g.M = (int)rows; g.N = (int)H; g.K = (int)In;
             g.epilogue = EPI_FC_FORWARD;
             g.bias = layer_uses_bias(l) ? parameters + l.first_bias_connection_index : nullptr;
             if (feeds_next) {
@@ -794,43 +861,46 @@ int Net::forward_residual_block(size_t ri, size_t B)
                 g.colscale = next_drop ? L[m + 1].colscale + t * L[m + 1].AH : nullptr;
             }
             prof_begin(0);
-            MYEA_TRY(launch_gemm(stream, g));
-            prof_end(2.0 * (double)B * (double)H * (double)In);
-        }
+            const int rc = launch_gemm(stream, g);
+            prof_end(2.0 * (double)rows * (double)H * (double)In);
+            return rc;
+        }));
         values_ready = feeds_next;
     }
     DevLayer &o = L[ri];
-    for (size_t t = 0; t < T; ++t) {
-        const size_t roff = t * Bmax;
-        const float *blk = layer_outputs(last) + roff * L[last].H;   // a dense member's sums, a pooling member's values, an LSTM member's outputs
-        if (layer_uses_norm(r)) {
-            MYEA_TRY(bn_forward(ri, t, B, blk, training));
-            blk = o.normalizes + roff * o.NH;
-        }
-        // ShakeDrop on the block's output, in place (NN/Neural_Network__Forward_Pass__Loop.cpp:4053-4078): one mask per (time step,
-        // example), one draw per value (Recurrent__Forward_Pass__Dropout__ShakeDrop, NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:367-386)
-        if (r.type_dropout == MYEA_DROPOUT_SHAKEDROP) {
-            const size_t W = o.NH;
-            float *out = const_cast<float *>(blk);
-            if (state == MYEA_STATE_TRAINING) {
-                if (t == 0 && !o.noise_uploaded) {   // masks, forward and backward draws of this pass, all time steps
-                    MYEA_TRY(launch_dropout_noise(stream, T * Bmax, o.noise, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
-                    MYEA_TRY(launch_threshold(stream, T * Bmax, o.noise, r.dropout_values[0]));
-                    MYEA_TRY(launch_dropout_noise(stream, T * Bmax * W, o.noise + T * Bmax, 0, -1.f, 1.f, dropout_seed, dropout_stream++));
-                    MYEA_TRY(launch_dropout_noise(stream, T * Bmax * W, o.noise + T * Bmax + T * Bmax * W, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
-                }
-                MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, o.noise + roff, o.noise + T * Bmax + roff * W, 1.f));
-            } else {
-                MYEA_TRY(launch_shakedrop_apply(stream, B, W, out, nullptr, nullptr, 1.f - r.dropout_values[0]));
-            }
-        }
-        const size_t na = o.In, nb = o.NH;
-        const float *src = layer_outputs(o.prev) + roff * na;
-        float *out = o.values + roff * o.H;
-        if (na >= nb) MYEA_TRY(launch_padded_add(stream, B, o.H, src, na, 0, blk, nb, -(long)o.pad, out));
-        else MYEA_TRY(launch_padded_add(stream, B, o.H, blk, nb, 0, src, na, -(long)o.pad, out));
+    const float *blk = layer_outputs(last);   // a dense member's sums, a pooling member's values, an LSTM member's outputs
+    if (layer_uses_norm(r)) {
+        MYEA_TRY(bn_forward_all(ri, B, blk, training));
+        blk = o.normalizes;
     }
-    return MYEA_OK;
+    // ShakeDrop on the block's output, in place (NN/Neural_Network__Forward_Pass__Loop.cpp:4053-4078): one mask per (time step,
+    // example), one draw per value (Recurrent__Forward_Pass__Dropout__ShakeDrop, NN/Neural_Network__Recurrent_Forward_Pass__OpenMP.cpp:367-386)
+    if (r.type_dropout == MYEA_DROPOUT_SHAKEDROP) {
+        const size_t W = o.NH;
+        float *out = const_cast<float *>(blk);
+        if (state == MYEA_STATE_TRAINING) {
+            if (!o.noise_uploaded) {   // masks, forward and backward draws of this pass, all time steps
+                MYEA_TRY(launch_dropout_noise(stream, T * Bmax, o.noise, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
+                MYEA_TRY(launch_threshold(stream, T * Bmax, o.noise, r.dropout_values[0]));
+                MYEA_TRY(launch_dropout_noise(stream, T * Bmax * W, o.noise + T * Bmax, 0, -1.f, 1.f, dropout_seed, dropout_stream++));
+                MYEA_TRY(launch_dropout_noise(stream, T * Bmax * W, o.noise + T * Bmax + T * Bmax * W, 0, 0.f, 1.f, dropout_seed, dropout_stream++));
+            }
+            MYEA_TRY(chunked(false, [&](size_t, size_t roff, size_t rows) {
+                return launch_shakedrop_apply(stream, rows, W, out + roff * W, o.noise + roff, o.noise + T * Bmax + roff * W, 1.f);
+            }));
+        } else {
+            MYEA_TRY(chunked(false, [&](size_t, size_t roff, size_t rows) {
+                return launch_shakedrop_apply(stream, rows, W, out + roff * W, nullptr, nullptr, 1.f - r.dropout_values[0]);
+            }));
+        }
+    }
+    const size_t na = o.In, nb = o.NH;
+    const float *src = layer_outputs(o.prev);
+    return chunked(false, [&](size_t, size_t roff, size_t rows) {
+        float *out = o.values + roff * o.H;
+        if (na >= nb) return launch_padded_add(stream, rows, o.H, src + roff * na, na, 0, blk + roff * nb, nb, -(long)o.pad, out);
+        return launch_padded_add(stream, rows, o.H, blk + roff * nb, nb, 0, src + roff * na, na, -(long)o.pad, out);
+    });
 }
 
 // ---- Compute__Error -------------------------------------------------------------------------------------------
@@ -959,7 +1029,8 @@ int Net::backward_into_layer(size_t li, size_t B)
     const bool second_direction = next.type_layer == MYEA_LAYER_LSTM && on.lstm2 != nullptr;
     const bool is_fc = layer_is_dense(l), ind = layer_is_ind_rnn(l);
     const bool norm = is_fc && layer_uses_norm(l), before = l.use_layer_normalization_before_activation != 0;
-    const bool per_t = T > 1 && (B != Bmax || norm);
+    const bool seq_bn = T > 1 && norm && before && B == Bmax && bn_sequence_allowed() && 2 * T * H <= scratch_floats;
+    const bool per_t = T > 1 && !seq_bn && (B != Bmax || norm);
     const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
     for (size_t c = 0; c < chunks; ++c) {
         const size_t roff = c * Bmax;
@@ -1005,7 +1076,7 @@ int Net::backward_into_layer(size_t li, size_t B)
             g.C = tmp1 + roff * H;
             g.epilogue = fuse ? EPI_FC_DERIVE : EPI_NONE; g.pre = o.normalizes + roff * H; g.val = o.values + roff * H;
             // the sums the normalisation's backward pass starts with leave with the contraction's tiles
-            if (fuse && o.norm_partials && bn_sums_from_gemm(true) && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H) {
+            if (!seq_bn && fuse && o.norm_partials && bn_sums_from_gemm(true) && l.type_normalization == MYEA_NORMALIZATION_BATCH_NORMALIZATION && o.NH == H) {
                 g.col_partials = o.norm_partials; g.hats = o.hats + roff * H;
             }
         } else {
@@ -1045,7 +1116,9 @@ int Net::backward_into_layer(size_t li, size_t B)
             MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, rows * H, g.pre, g.val, tmp1 + roff * H, (norm ? tmp1 : o.neuron_errors) + roff * H,
                                               o.unit_act, o.unit_steep, H));
         }
-        if (norm && before) {
+        if (norm && before && seq_bn) {
+            MYEA_TRY(bn_backward_all(li, B, o.summations, tmp1, o.neuron_errors));
+        } else if (norm && before) {
             const bool sums_from_gemm = have_gemm && g.col_partials == o.norm_partials && g.col_partials != nullptr;
             MYEA_TRY(bn_backward(li, c, rows, o.summations + roff * H, tmp1 + roff * H, o.neuron_errors + roff * H, sums_from_gemm ? o.norm_partials : nullptr, (rows + 31) / 32));
         } else if (norm) {
@@ -1064,8 +1137,7 @@ int Net::backward_into_layer(size_t li, size_t B)
         p.dy = (norm && !before) ? tmp2 : tmp1;
         p.dafs = o.dafs_own ? o.dafs_own : o.neuron_errors;
         MYEA_TRY(launch_ind_rnn_backward(stream, p));
-        if (norm && before)
-            for (size_t t = T; t-- > 0;) MYEA_TRY(bn_backward(li, t, B, o.summations + t * Bmax * H, o.dafs_own + t * Bmax * H, o.neuron_errors + t * Bmax * H));
+        if (norm && before) MYEA_TRY(bn_backward_all(li, B, o.summations, o.dafs_own, o.neuron_errors));
     }
     return MYEA_OK;
 }
@@ -1087,23 +1159,26 @@ int Net::backward_residual_block(size_t ri, size_t B)
     DevLayer &ro = L[ri];
     const size_t last = ri + r.block_depth, T = d.number_recurrent_depth, Bmax = d.batch_size;
     const long crop = ro.H > ro.NH ? (long)ro.pad : 0;
+    // the whole sequence in one launch when the batch fills the network's rows, one launch per time step otherwise (the time
+    // steps are on their own in everything that is not a recurrence)
+    auto chunked = [&](auto &&launch) -> int {
+        const bool split = T > 1 && B != Bmax;
+        const size_t n = split ? T : 1, rows = split ? B : T * B;
+        for (size_t c = n; c-- > 0;) MYEA_TRY(launch(c * Bmax, rows));
+        return MYEA_OK;
+    };
     // the perturbed examples' deltas times the backward draws (NN/Neural_Network__Backward_Pass__Loop.cpp:433-443)
     const bool shake = r.type_dropout == MYEA_DROPOUT_SHAKEDROP;
-    // time steps in descending order, as the dense layers of a recurrent network are walked; each is on its own
-    for (size_t t = T; t-- > 0;) {
-        const size_t roff = t * Bmax;
-        const float *res_errors = ro.neuron_errors + roff * ro.H;
-        const float *mask = shake ? ro.noise + roff : nullptr, *beta = shake ? ro.noise + T * Bmax + T * Bmax * ro.NH + roff * ro.NH : nullptr;
-        float *last_errors = L[last].neuron_errors + roff * L[last].H;
-        if (layer_uses_norm(r)) {
-            float *tmp = tmp1 + roff * ro.NH;
-            MYEA_TRY(launch_padded_add(stream, B, ro.NH, res_errors, ro.H, crop, nullptr, 0, 0, tmp));
-            if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, tmp, mask, beta, 1.f));
-            MYEA_TRY(bn_backward(ri, t, B, layer_outputs(last) + roff * L[last].H, tmp, last_errors));
-        } else {
-            MYEA_TRY(launch_padded_add(stream, B, ro.NH, res_errors, ro.H, crop, nullptr, 0, 0, last_errors));
-            if (shake) MYEA_TRY(launch_shakedrop_apply(stream, B, ro.NH, last_errors, mask, beta, 1.f));
-        }
+    {
+        const bool norm = layer_uses_norm(r);
+        float *to = norm ? tmp1 : L[last].neuron_errors;
+        const size_t W = norm ? ro.NH : L[last].H;   // (the same width: the block's last member's)
+        MYEA_TRY(chunked([&](size_t roff, size_t rows) -> int {
+            MYEA_TRY(launch_padded_add(stream, rows, ro.NH, ro.neuron_errors + roff * ro.H, ro.H, crop, nullptr, 0, 0, to + roff * W));
+            if (shake) MYEA_TRY(launch_shakedrop_apply(stream, rows, ro.NH, to + roff * W, ro.noise + roff, ro.noise + T * Bmax + T * Bmax * ro.NH + roff * ro.NH, 1.f));
+            return MYEA_OK;
+        }));
+        if (norm) MYEA_TRY(bn_backward_all(ri, B, layer_outputs(last), tmp1, L[last].neuron_errors));
     }
     for (size_t m = last; m > ri; --m) {
         const myea_layer_desc &l = d.layers[m];
@@ -1114,10 +1189,7 @@ int Net::backward_residual_block(size_t ri, size_t B)
             MYEA_TRY(lstm_backward_layer(m, B));
             if (first) break;   // the layer in front of the block pulls dG * Win together with the shortcut's share
             // what the member before it receives: dG * Win of every time step (both directions of a two-direction member)
-            const bool per_t = T > 1 && B != Bmax;
-            const size_t chunks = per_t ? T : 1, rows = per_t ? B : T * B;
-            for (size_t c = 0; c < chunks; ++c) {
-                const size_t roff = c * Bmax;
+            MYEA_TRY(chunked([&](size_t roff, size_t rows) -> int {
                 for (int direction = o.lstm2 ? 1 : 0; direction >= 0; --direction) {
                     const float *delta, *weights;
                     size_t out;
@@ -1133,46 +1205,43 @@ int Net::backward_residual_block(size_t ri, size_t B)
                     MYEA_TRY(launch_gemm(stream, g));
                     prof_end(2.0 * (double)rows * (double)In * (double)out);
                 }
-            }
+                return MYEA_OK;
+            }));
             continue;
         }
         if (layer_is_pooling(l)) {   // hands its delta down through its windows (Backward_Pass__Gradient__Residual__Layer, :753-772), nothing else
             if (first) break;   // the first member: the layer in front of the block pulls it, together with the shortcut's share
-            for (size_t t = T; t-- > 0;) {
-                const size_t roff = t * Bmax;
-                MYEA_TRY(launch_pool_backward(stream, pool_params(m, B), o.neuron_errors + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr,
-                                              L[m - 1].neuron_errors + roff * In));
-            }
+            MYEA_TRY(chunked([&](size_t roff, size_t rows) -> int {
+                return launch_pool_backward(stream, pool_params(m, rows), o.neuron_errors + roff * H, o.pool_index ? o.pool_index + roff * H : nullptr,
+                                            L[m - 1].neuron_errors + roff * In);
+            }));
             continue;
         }
         if (o.group == 1 && !norm) break;
         const bool ind = o.group == 2 && layer_is_ind_rnn(l);
         const float *prev_all = layer_outputs(o.prev);
         float *dst_all = o.group == 2 ? L[m - 1].neuron_errors : o.in_errors;
-        for (size_t t = T; t-- > 0;) {
-            const size_t roff = t * Bmax;
-            float *dst = dst_all + roff * In, *tmp = tmp1 + roff * In;
-            const float *prev_out = prev_all + roff * In;
+        MYEA_TRY(chunked([&](size_t roff, size_t rows) -> int {
             GemmParams g{};
             g.A = o.neuron_errors + roff * H; g.lda = (long)H; g.a_k_contiguous = 1;
             g.B = parameters + l.first_connection_index; g.ldb = (long)In; g.b_k_contiguous = 0;
-            g.C = (norm || ind) ? tmp : dst; g.ldc = (long)In;
-            g.M = (int)B; g.N = (int)In; g.K = (int)H;
+            g.C = ((norm || ind) ? tmp1 : dst_all) + roff * In; g.ldc = (long)In;
+            g.M = (int)rows; g.N = (int)In; g.K = (int)H;
             g.epilogue = EPI_NONE;
             bool derive_pending = false;
             if (o.group == 2 && !ind) {
                 g.act = (int)l.type_activation_function; g.steep = l.activation_steepness;
-                g.pre = norm ? o.normalizes + roff * In : prev_out;   // Layer::ptr_array_pre_activation_functions
+                g.pre = (norm ? o.normalizes : prev_all) + roff * In;   // Layer::ptr_array_pre_activation_functions
                 g.val = o.values + roff * In;
                 if (!o.unit_act && !o.unit_steep && gemm_can_fuse_activation(g.act)) g.epilogue = EPI_FC_DERIVE;
                 else derive_pending = true;
             }
             prof_begin(1);
             MYEA_TRY(launch_gemm(stream, g));
-            prof_end(2.0 * (double)B * (double)H * (double)In);
-            if (derive_pending) MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, B * In, g.pre, g.val, g.C, g.C, o.unit_act, o.unit_steep, In));
-            if (norm && !ind) MYEA_TRY(bn_backward(m, t, B, prev_out, tmp, dst));
-        }
+            prof_end(2.0 * (double)rows * (double)H * (double)In);
+            if (derive_pending) MYEA_TRY(launch_activation_derive(stream, g.act, g.steep, rows * In, g.pre, g.val, g.C, g.C, o.unit_act, o.unit_steep, In));
+            return MYEA_OK;
+        }));
         if (ind) {
             // Backward_Pass__FC__DF_Ind_RNN over the whole sequence (:865-880): what the member hands on is the delta of its
             // pre-activations, through the input-side normalisation when there is one
@@ -1183,11 +1252,10 @@ int Net::backward_residual_block(size_t ri, size_t B)
             p.pre_afs = o.pre_afs; p.afs = o.values;
             p.dy = tmp1; p.dafs = o.dafs_own;
             MYEA_TRY(launch_ind_rnn_backward(stream, p));
-            if (norm) {
-                for (size_t t = T; t-- > 0;) MYEA_TRY(bn_backward(m, t, B, prev_all + t * Bmax * In, o.dafs_own + t * Bmax * In, dst_all + t * Bmax * In));
-            } else {
-                MYEA_HIP_TRY(hipMemcpyAsync(dst_all, o.dafs_own, T * Bmax * In * sizeof(float), hipMemcpyDeviceToDevice, stream));
-            }
+            if (norm) MYEA_TRY(bn_backward_all(m, B, prev_all, o.dafs_own, dst_all));
+            else MYEA_HIP_TRY(hipMemcpyAsync(dst_all, o.dafs_own, T * Bmax * In * sizeof(float), hipMemcpyDeviceToDevice, stream));
+        } else if (norm) {
+            MYEA_TRY(bn_backward_all(m, B, prev_all, tmp1, dst_all));
         }
     }
     return MYEA_OK;
@@ -1270,7 +1338,8 @@ int Net::backward_pass(size_t B)
 // slabs of the split-K form of a fully-connected layer's weight gradient; 1 = the plain accumulating contraction
 static int fc_dw_slabs(size_t H, size_t In, size_t rows, size_t first_connection_index)
 {
-    if (((H * In) & 3) || (first_connection_index & 3) || rows > 0x7fffffffu) return 1;   // the slab sum works on aligned quads
+    (void)first_connection_index;
+    if (rows > 0x7fffffffu) return 1;
     return gemm_split_k((int)H, (int)In, (int)rows);
 }
 
