@@ -70,6 +70,11 @@ WORKLOADS = {
                + [dict(units=100, activation="SOFTMAX")],
         batch=512, head="SOFTMAX", optimizer="GD", loss="CROSS_ENTROPY", data="normal",
         hyper=dict(learning_rate=0.01, learning_momentum=0.9, use_Nesterov=1)),
+    # LSTM layers normalised inside (batch normalisation of the eight gate sums and of the cell state at every time step)
+    "lstm256x2_bn_t32_b128_adam": dict(
+        layers=[dict(units=64), dict(type="lstm", units=256, normalization="BATCH_NORMALIZATION"),
+                dict(type="lstm", units=256, normalization="BATCH_NORMALIZATION"), dict(units=256, activation="LINEAR")],
+        batch=128, depth=32, head="LINEAR", optimizer="ADAM", loss="MSE", data="normal", hyper={}),
     # the reference's worked example (Neural_Network_Launcher_Windows/Source_Files/debug.cpp:36-1555): sMNIST rows (28 inputs x 28
     # time steps, the label read at the last one), residual blocks of independently recurrent ISRLU members with batch
     # normalisation, max pooling between the groups, softmax head, AMSGrad at 1e-3, max-norm constraint 8

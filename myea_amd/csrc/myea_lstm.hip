@@ -596,6 +596,359 @@ __global__ __launch_bounds__(kBlock) void lstm_norm_backward_gates_kernel(size_t
     }
 }
 
+// ---- a normalised layer's time step in one launch -----------------------------------------------------------------------
+// Everything a time step does behind its recurrent contraction touches one cell's column of a few tensors over the batch: the
+// statistics are sums over the batch of that column, the gate math combines the normalised sums of the same cell.  A workgroup
+// therefore owns CW cells and ALL examples, with kBlock / CW row lanes: the column sums of every group meet in LDS, one lane
+// per (group, cell) finishes the statistics as lstm_norm_statistics_kernel does, and the lanes go over their rows again to
+// apply them and to run the gates; a lane meets the same (example, cell) pairs in every pass, so what it wrote it may read back.
+struct NormStep { NormBand g[9]; };   // indexed by group: 0 z, 3 i, 5 f, 7 o from below; 1, 4, 6, 8 recurrent; 2 the cell state
+constexpr int kNormThreads = 1024, kNormWaves = kNormThreads / 64;
+constexpr int kNormBackThreads = 512;   // the backward pass keeps more per lane: 256 registers a lane instead of 128
+
+// a wavefront holds 64 / CW rows of the workgroup's CW columns (lane = CW * row + column): those rows' values of a column, summed
+template <int CW>
+__device__ __forceinline__ double norm_fold_rows(double v)
+{
+#pragma unroll
+    for (int m = CW; m < 64; m <<= 1) v += __shfl_xor(v, m);
+    return v;
+}
+
+__device__ __forceinline__ void norm_finish_statistics(const NormBand &g, size_t col, double s1, double s2, size_t B, const NormHyper &hy, float *st)
+{
+    const float bscale = 1.f / (float)B;
+    const float mean = (float)s1 * bscale;
+    const float mavg = g.mean_avg[col] + hy.momentum * (mean - g.mean_avg[col]);
+    const float sigma = sqrtf((float)s2 * bscale - mean * mean + hy.epsilon);
+    const float vavg = g.sigma_avg[col] + hy.momentum * (sigma - g.sigma_avg[col]);
+    g.mean[col] = mean; g.sigma[col] = sigma; g.mean_avg[col] = mavg; g.sigma_avg[col] = vavg;
+    float r = 1.f, dd = 0.f;
+    if (hy.renorm) {
+        const float q = sigma / vavg, lo = 1.f / hy.r_max;
+        r = q < lo ? lo : (q > hy.r_max ? hy.r_max : q);
+        const float e = (mean - mavg) / vavg;
+        dd = e < -hy.d_max ? -hy.d_max : (e > hy.d_max ? hy.d_max : e);
+        g.r[col] = r; g.dd[col] = dd;
+    }
+    st[0] = mean; st[1] = sigma; st[2] = r; st[3] = dd;
+}
+
+// Forward_Pass__LSTM of one time step behind the recurrent contraction (NN/Neural_Network__Forward_Pass__OpenMP.cpp:1769-2340):
+// the normalisations of the gate sums, Gates_CIF_AF_State, the cell state's normalisation, States_AF and Output - the kernels
+// lstm_norm_statistics / _apply / _gates / _output above in one launch.  grid: ceil(C / CW) workgroups of 16 wavefronts
+template <bool FIRST, int CW>   // FIRST: the direction's first time step (no recurrent sums, no forget gate); CW: cells per workgroup
+__global__ __launch_bounds__(kNormThreads) void lstm_norm_forward_fused_kernel(NormStep nb, size_t C, size_t B, int training, NormHyper hy, const float *bias,
+                                                                               const float *peep, const float *c_prev, float *acts, float *c, float *ca, float *h,
+                                                                               const float *h_prev, const uint8_t *zone_state, const uint8_t *zone_output)
+{
+    constexpr int RL = kNormThreads / CW, NW = kNormWaves;
+    __shared__ double red[8][2][NW][CW];
+    __shared__ float st[9][4][CW];
+    const int cl = threadIdx.x % CW, rl = threadIdx.x / CW, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const size_t k = (size_t)blockIdx.x * CW + cl, G = 4 * C;
+    const bool live = k < C;
+    constexpr bool first = FIRST;
+    constexpr int order[8] = {0, 3, FIRST ? 7 : 5, 1, 4, 6, 7, 8};
+    constexpr int n = FIRST ? 3 : 8;
+    if (training) {
+        double s1[n], s2[n];
+#pragma unroll
+        for (int i = 0; i < n; ++i) { s1[i] = 0.0; s2[i] = 0.0; }
+        if (live)
+            for (size_t b = rl; b < B; b += RL) {
+#pragma unroll
+                for (int i = 0; i < n; ++i) {
+                    const NormBand &g = nb.g[order[i]];
+                    const float v = g.x[b * g.ldx + k];
+                    s1[i] += v; s2[i] += (double)v * v;
+                }
+            }
+#pragma unroll
+        for (int i = 0; i < n; ++i) {
+            const double a = norm_fold_rows<CW>(s1[i]), q = norm_fold_rows<CW>(s2[i]);
+            if (lane < CW) { red[i][0][wave][cl] = a; red[i][1][wave][cl] = q; }
+        }
+        __syncthreads();
+        {   // one lane per (group, cell)
+            const int i = threadIdx.x / CW, col_l = threadIdx.x % CW;
+            const size_t col = (size_t)blockIdx.x * CW + col_l;
+            if (i < n && col < C) {
+                double a = 0.0, q = 0.0;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) { a += red[i][0][w][col_l]; q += red[i][1][w][col_l]; }
+                float out[4];
+                norm_finish_statistics(nb.g[order[i]], col, a, q, B, hy, out);
+                st[order[i]][0][col_l] = out[0]; st[order[i]][1][col_l] = out[1]; st[order[i]][2][col_l] = out[2]; st[order[i]][3][col_l] = out[3];
+            }
+        }
+    } else {
+        const int i = threadIdx.x / CW, col_l = threadIdx.x % CW;
+        const size_t col = (size_t)blockIdx.x * CW + col_l;
+        if (i < 9 && col < C) { st[i][0][col_l] = nb.g[i].mean_avg[col]; st[i][1][col_l] = nb.g[i].sigma_avg[col]; st[i][2][col_l] = 1.f; st[i][3][col_l] = 0.f; }
+    }
+    __syncthreads();
+    // the normalised sums of the lane's cell, the gates, the cell state; the cell state's column sums on the way
+    double c1 = 0.0, c2 = 0.0;
+    if (live) {
+        const float pi = peep[k], pf = peep[C + k];
+        const float bz = bias[k], bi = bias[C + k], bf = bias[2 * C + k];
+        float scale[n], shift[n];
+#pragma unroll
+        for (int i = 0; i < n; ++i) { scale[i] = nb.g[order[i]].scale[k]; shift[i] = nb.g[order[i]].shift[k]; }
+        for (size_t b = rl; b < B; b += RL) {
+            float nor[9];
+#pragma unroll
+            for (int i = 0; i < n; ++i) {
+                constexpr int dummy = 0; (void)dummy;
+                const int gi = order[i];
+                const NormBand &g = nb.g[gi];
+                float v = g.x[b * g.ldx + k];
+                v = (v - st[gi][0][cl]) / st[gi][1][cl];
+                if (training) {
+                    if (hy.renorm) v = v * st[gi][2][cl] + st[gi][3][cl];
+                    g.hat[b * g.ldo + k] = v;
+                }
+                v = scale[i] * v + shift[i];
+                g.nor[b * g.ldo + k] = v;
+                nor[gi] = v;
+            }
+            float *row = acts + b * G;
+            float gate_i, gate_f = 0.f, sz;
+            const float cp = first ? 0.f : c_prev[b * C + k];
+            if (!first) {
+                float si = nor[3] + nor[4] + bi;
+                float sf = nor[5] + nor[6] + bf;
+                si += cp * pi; sf += cp * pf;
+                gate_i = sigmoid_f(si); gate_f = sigmoid_f(sf);
+                sz = nor[0] + nor[1] + bz;
+            } else {
+                gate_i = sigmoid_f(nor[3] + bi);
+                sz = nor[0] + bz;
+            }
+            const float z = tanh_f(sz);
+            row[k] = z; row[C + k] = gate_i; row[2 * C + k] = gate_f;
+            float cs = first ? z * gate_i : z * gate_i + gate_f * cp;
+            if (zone_state && !zone_state[k]) cs = first ? 0.f : cp;
+            c[b * C + k] = cs;
+            c1 += cs; c2 += (double)cs * cs;
+        }
+    }
+    if (training) {
+        __syncthreads();   // every lane is through with red
+        const double a = norm_fold_rows<CW>(c1), q = norm_fold_rows<CW>(c2);
+        if (lane < CW) { red[0][0][wave][cl] = a; red[0][1][wave][cl] = q; }
+        __syncthreads();
+        if (rl == 0 && live) {
+            double sa = 0.0, sq = 0.0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) { sa += red[0][0][w][cl]; sq += red[0][1][w][cl]; }
+            float out[4];
+            norm_finish_statistics(nb.g[2], k, sa, sq, B, hy, out);
+            st[2][0][cl] = out[0]; st[2][1][cl] = out[1]; st[2][2][cl] = out[2]; st[2][3][cl] = out[3];
+        }
+        __syncthreads();
+    }
+    if (!live) return;
+    const NormBand &gc = nb.g[2];
+    const NormBand &g7 = nb.g[7], &g8 = nb.g[8];
+    const float po = peep[2 * C + k], bo = bias[3 * C + k], csc = gc.scale[k], csh = gc.shift[k];
+    for (size_t b = rl; b < B; b += RL) {
+        const float cs = c[b * C + k];
+        float v = (cs - st[2][0][cl]) / st[2][1][cl];
+        if (training) {
+            if (hy.renorm) v = v * st[2][2][cl] + st[2][3][cl];
+            gc.hat[b * gc.ldo + k] = v;
+        }
+        v = csc * v + csh;
+        gc.nor[b * gc.ldo + k] = v;
+        const float a = tanh_f(v);
+        ca[b * C + k] = a;
+        float so = g7.nor[b * g7.ldo + k] + (first ? 0.f : g8.nor[b * g8.ldo + k]) + bo;
+        so += cs * po;
+        const float go = sigmoid_f(so);
+        acts[b * G + 3 * C + k] = go;
+        float hv = a * go;
+        if (zone_output && !zone_output[k]) hv = first ? 0.f : h_prev[b * C + k];
+        h[b * C + k] = hv;
+    }
+}
+
+// the three column sums of a normalisation's backward pass for one (example, cell), as lstm_norm_backward_sums_kernel forms them
+struct NormBackColumn {
+    float vb, r, sc, mean, k2, k3;
+    __device__ __forceinline__ void load(const NormBand &g, size_t col, int renorm)
+    {
+        vb = g.sigma[col]; r = renorm ? g.r[col] : 1.f; sc = g.scale[col]; mean = g.mean[col];
+        k2 = -r / vb; k3 = -r / (vb * vb);
+    }
+    __device__ __forceinline__ void add(const NormBand &g, size_t b, size_t col, float e, double *a) const
+    {
+        a[0] += e * g.hat[b * g.ldo + col];
+        e *= sc;
+        a[1] += e * k2;
+        a[2] += e * (g.x[b * g.ldx + col] - mean) * k3;
+    }
+    // the last loop of the backward pass (lstm_norm_backward_apply_kernel)
+    __device__ __forceinline__ float apply(const NormBand &g, size_t b, size_t col, float d, float dmean, float dsigma, size_t B) const
+    {
+        float e = d * sc;
+        e *= r / vb;
+        e += dsigma * ((g.x[b * g.ldx + col] - mean) / ((float)B * vb));
+        e += dmean * (1.f / (float)B);
+        return e;
+    }
+};
+
+// The backward pass of one time step behind the recurrent contraction (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:476-862):
+// lstm_norm_backward_output, the backward normalisations of the output gate's sums and the cell state, lstm_norm_backward_gates and
+// the backward normalisations of the other gate sums in one launch.  grid: ceil(C / CW) workgroups of 8 wavefronts
+template <bool FIRST, int CW>
+__global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_kernel(NormStep nb, size_t C, size_t B, int last, int renorm, const float *peep,
+                                                                                const float *acts, const float *acts_next, const float *ca, const float *c_prev, float *dh,
+                                                                                const float *part, int nparts, float *dG, const float *dG_next, float *dc,
+                                                                                const float *dc_next, float *din, float *drec)
+{
+    constexpr int RL = kNormBackThreads / CW, NW = kNormBackThreads / 64;
+    __shared__ double red[6][3][NW][CW];
+    __shared__ float fin[6][2][CW];   // dmean, dsigma of the groups in flight
+    const int cl = threadIdx.x % CW, rl = threadIdx.x / CW, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const size_t k = (size_t)blockIdx.x * CW + cl, G = 4 * C;
+    const bool live = k < C;
+    constexpr bool first = FIRST;
+    const int compute = (first && last) ? 0 : 1;
+    // ---- the output gate's delta and the cell state's, their normalisations' sums: groups 7, 2 and, behind the first step, 8
+    constexpr int head[3] = {7, 2, 8};
+    constexpr int nh = FIRST ? 2 : 3;
+    NormBackColumn col[nh];
+    {
+        double a[nh][3];
+#pragma unroll
+        for (int i = 0; i < nh; ++i) { a[i][0] = a[i][1] = a[i][2] = 0.0; }
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < nh; ++i) col[i].load(nb.g[head[i]], k, renorm);
+            for (size_t b = rl; b < B; b += RL) {
+                float v = dh[b * C + k];
+                for (int s = 0; s < nparts; ++s) v += part[((size_t)s * B + b) * C + k];
+                if (nparts > 0) dh[b * C + k] = v;
+                const float go = acts[b * G + 3 * C + k], av = ca[b * C + k];
+                const float ddo = (go * (1.f - go)) * (v * av);
+                dG[b * G + 3 * C + k] = ddo;
+                din[b * G + 3 * C + k] = ddo;
+                if (!first) drec[b * G + 3 * C + k] = ddo;
+                const float dcv = v * go * (1.f - av * av);
+                dc[b * C + k] = dcv;
+                col[0].add(nb.g[7], b, k, ddo, a[0]);
+                col[1].add(nb.g[2], b, k, dcv, a[1]);
+                if (!first) col[nh - 1].add(nb.g[8], b, k, ddo, a[nh - 1]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < nh; ++i)
+#pragma unroll
+            for (int v = 0; v < 3; ++v) {
+                const double f = norm_fold_rows<CW>(a[i][v]);
+                if (lane < CW) red[i][v][wave][cl] = f;
+            }
+    }
+    __syncthreads();
+    {
+        const int i = threadIdx.x / CW, col_l = threadIdx.x % CW;
+        const size_t cc = (size_t)blockIdx.x * CW + col_l;
+        if (i < nh && cc < C) {
+            double q0 = 0.0, q1 = 0.0, q2 = 0.0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) { q0 += red[i][0][w][col_l]; q1 += red[i][1][w][col_l]; q2 += red[i][2][w][col_l]; }
+            const NormBand &g = nb.g[head[i]];
+            g.dscale[cc] += (float)q0; g.dmean[cc] = (float)q1; g.dsigma[cc] = (float)q2;
+            fin[i][0][col_l] = (float)q1; fin[i][1][col_l] = (float)q2;
+        }
+    }
+    __syncthreads();
+    // ---- those normalisations' last loop, the gates' deltas, the sums of the other groups: 0, 3 and, behind the first step, 5, 1, 4, 6
+    constexpr int tail[6] = {0, 3, 5, 1, 4, 6};
+    constexpr int nt = FIRST ? 2 : 6;
+    constexpr int tail_gate[6] = {0, 1, 2, 0, 1, 2};   // which gate's delta a group normalises
+    NormBackColumn tc[nt];
+    float dmean_head[nh], dsigma_head[nh];
+#pragma unroll
+    for (int i = 0; i < nh; ++i) { dmean_head[i] = fin[i][0][cl]; dsigma_head[i] = fin[i][1][cl]; }
+    {
+        double a[nt][3];
+#pragma unroll
+        for (int i = 0; i < nt; ++i) { a[i][0] = a[i][1] = a[i][2] = 0.0; }
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < nt; ++i) tc[i].load(nb.g[tail[i]], k, renorm);
+            const float p_i = peep[k], p_f = peep[C + k], p_o = peep[2 * C + k];
+            for (size_t b = rl; b < B; b += RL) {
+                const float ddo = dG[b * G + 3 * C + k];
+                din[b * G + 3 * C + k] = col[0].apply(nb.g[7], b, k, ddo, dmean_head[0], dsigma_head[0], B);
+                if (!first) drec[b * G + 3 * C + k] = col[nh - 1].apply(nb.g[8], b, k, ddo, dmean_head[nh - 1], dsigma_head[nh - 1], B);
+                float e = col[1].apply(nb.g[2], b, k, dc[b * C + k], dmean_head[1], dsigma_head[1], B);
+                float *drow = dG + b * G;
+                if (compute) {
+                    const float *row = acts + b * G;
+                    const float z = row[k], gi = row[C + k];
+                    e += p_o * ddo;
+                    if (!last) {
+                        e += p_i * dG_next[b * G + C + k];
+                        e += p_f * dG_next[b * G + 2 * C + k];
+                        e += dc_next[b * C + k] * acts_next[b * G + 2 * C + k];
+                    }
+                    dc[b * C + k] = e;
+                    drow[k] = e * gi * (1.f - z * z);
+                    drow[C + k] = (e * z) * (gi * (1.f - gi));
+                    if (!first) { const float gf = row[2 * C + k]; drow[2 * C + k] = (e * c_prev[b * C + k]) * (gf * (1.f - gf)); }
+                } else {
+                    dc[b * C + k] = e;
+                }
+                float gd[3];
+#pragma unroll
+                for (int gate = 0; gate < 3; ++gate) {
+                    gd[gate] = drow[gate * C + k];
+                    din[b * G + gate * C + k] = gd[gate];
+                    if (!first) drec[b * G + gate * C + k] = gd[gate];
+                }
+#pragma unroll
+                for (int i = 0; i < nt; ++i) tc[i].add(nb.g[tail[i]], b, k, gd[tail_gate[i]], a[i]);
+            }
+        }
+        __syncthreads();   // fin and red are free again
+#pragma unroll
+        for (int i = 0; i < nt; ++i)
+#pragma unroll
+            for (int v = 0; v < 3; ++v) {
+                const double f = norm_fold_rows<CW>(a[i][v]);
+                if (lane < CW) red[i][v][wave][cl] = f;
+            }
+    }
+    __syncthreads();
+    {
+        const int i = threadIdx.x / CW, col_l = threadIdx.x % CW;
+        const size_t cc = (size_t)blockIdx.x * CW + col_l;
+        if (i < nt && cc < C) {
+            double q0 = 0.0, q1 = 0.0, q2 = 0.0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) { q0 += red[i][0][w][col_l]; q1 += red[i][1][w][col_l]; q2 += red[i][2][w][col_l]; }
+            const NormBand &g = nb.g[tail[i]];
+            g.dscale[cc] += (float)q0; g.dmean[cc] = (float)q1; g.dsigma[cc] = (float)q2;
+            fin[i][0][col_l] = (float)q1; fin[i][1][col_l] = (float)q2;
+        }
+    }
+    __syncthreads();
+    if (!live) return;
+    for (size_t b = rl; b < B; b += RL) {
+#pragma unroll
+        for (int i = 0; i < nt; ++i) {
+            const NormBand &g = nb.g[tail[i]];
+            float *d = g.d + b * g.ldd + k;
+            *d = tc[i].apply(g, b, k, *d, fin[i][0][cl], fin[i][1][cl], B);
+        }
+    }
+}
+
 int dev_alloc_zero(float **p, size_t count)
 {
     void *q = nullptr;
@@ -615,6 +968,14 @@ bool fused_lstm_disabled()
 {
     const char *e = std::getenv("MYEA_LSTM_FUSED");
     return e && e[0] == '0';
+}
+
+// MYEA_LSTM_NORM_FUSED=0 keeps a normalised layer's time step as the sequence of statistics / apply / gate launches (read at
+// every call: a test runs both forms in one process)
+bool lstm_norm_fused_allowed()
+{
+    const char *e = std::getenv("MYEA_LSTM_NORM_FUSED");
+    return !(e && e[0] == '0');
 }
 
 // MYEA_SIDE_STREAM=0 keeps every launch on the caller's stream (for A/B timing)
@@ -910,6 +1271,28 @@ int Net::lstm_forward_step_norm(LstmLayer &q, size_t B, size_t s)
         g.C = q.srec + t * Bmax * G; g.ldc = (long)G;
         g.M = (int)B; g.N = (int)G; g.K = (int)C;
         MYEA_TRY(launch_gemm(stream, g));
+    }
+    if (lstm_norm_fused_allowed()) {   // everything behind the contraction in one launch
+        NormStep nb;
+        for (int gi = 0; gi < 9; ++gi) nb.g[gi] = norm_band(q, parameters, gradient, d.total_normalized_units, gi, t, T, Bmax);
+        const bool training = state >= MYEA_STATE_TRAINING;
+        const NormHyper hy{h.normalization_epsilon, h.normalization_momentum_average, h.batch_renormalization_r_correction_maximum,
+                           h.batch_renormalization_d_correction_maximum, q.renorm ? 1 : 0};
+        float *acts = q.acts + t * Bmax * G, *c = q.c + t * Bmax * C, *ca = q.ca + t * Bmax * C, *hh = q.h + t * Bmax * C;
+        const float *c_prev = first ? nullptr : q.c + tp * Bmax * C, *h_prev = first ? nullptr : q.h + tp * Bmax * C;
+        const int tr = training ? 1 : 0;
+        prof_begin(kProfNormalization);
+        // few cells a workgroup when the layer is narrow: the launch is a chain of memory round trips, shorter the more lanes share a column
+        auto launch = [&](auto kernel, int cw) {
+            hipLaunchKernelGGL(kernel, dim3((unsigned)((C + cw - 1) / cw)), dim3(kNormThreads), 0, stream, nb, C, B, tr, hy, bias, (const float *)q.peep, c_prev, acts, c, ca, hh, h_prev, zs, zo);
+        };
+        if (C >= 1024) { if (first) launch(lstm_norm_forward_fused_kernel<true, 16>, 16); else launch(lstm_norm_forward_fused_kernel<false, 16>, 16); }
+        else { if (first) launch(lstm_norm_forward_fused_kernel<true, 4>, 4); else launch(lstm_norm_forward_fused_kernel<false, 4>, 4); }
+        MYEA_HIP_TRY(hipGetLastError());
+        prof_end((double)(first ? 4 : 9) * (double)B * (double)C * sizeof(float) * 3.0);
+        return MYEA_OK;
+    }
+    if (!first) {
         MYEA_TRY(lstm_norm_forward_groups(q, B, t, {0, 3, 5, 1, 4, 6, 7, 8}));
     } else {
         MYEA_TRY(lstm_norm_forward_groups(q, B, t, {0, 3, 7}));
@@ -942,6 +1325,23 @@ int Net::lstm_backward_step_norm(LstmLayer &q, size_t B, size_t s)
         nparts = gemm_split_k(g.M, g.N, g.K);
         g.split_k = nparts; g.split_k_slab = (long)(B * C);
         MYEA_TRY(launch_gemm(stream, g));
+    }
+    if (lstm_norm_fused_allowed()) {
+        NormStep nb;
+        for (int gi = 0; gi < 9; ++gi) nb.g[gi] = norm_band(q, parameters, gradient, d.total_normalized_units, gi, t, T, Bmax);
+        const float *acts_next = last ? nullptr : q.acts + tn * Bmax * G, *c_prev = first ? nullptr : q.c + tp * Bmax * C;
+        const float *dG_next = last ? nullptr : q.dG + tn * Bmax * G, *dc_next = last ? nullptr : q.dc + tn * Bmax * C;
+        prof_begin(kProfNormalization);
+        auto launch = [&](auto kernel, int cw) {
+            hipLaunchKernelGGL(kernel, dim3((unsigned)((C + cw - 1) / cw)), dim3(kNormBackThreads), 0, stream, nb, C, B, last ? 1 : 0, q.renorm ? 1 : 0, (const float *)q.peep,
+                               (const float *)(q.acts + t * Bmax * G), acts_next, (const float *)(q.ca + t * Bmax * C), c_prev, q.dh + t * Bmax * C, (const float *)q.part, nparts,
+                               q.dG + t * Bmax * G, dG_next, q.dc + t * Bmax * C, dc_next, q.din + t * Bmax * G, q.drec + t * Bmax * G);
+        };
+        if (C >= 1024) { if (first) launch(lstm_norm_backward_fused_kernel<true, 16>, 16); else launch(lstm_norm_backward_fused_kernel<false, 16>, 16); }
+        else { if (first) launch(lstm_norm_backward_fused_kernel<true, 4>, 4); else launch(lstm_norm_backward_fused_kernel<false, 4>, 4); }
+        MYEA_HIP_TRY(hipGetLastError());
+        prof_end((double)(first ? 4 : 9) * (double)B * (double)C * sizeof(float) * 5.0);
+        return MYEA_OK;
     }
     const unsigned grid = grid_for(B * C, kBlock, 8192);
     hipLaunchKernelGGL(lstm_norm_backward_output_kernel, dim3(grid), dim3(kBlock), 0, stream, C, B, first ? 1 : 0, q.acts + t * Bmax * G, q.ca + t * Bmax * C,

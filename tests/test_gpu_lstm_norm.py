@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 from myea_amd import binding as mb
-from tests.common import assert_close, run_step
+from tests.common import assert_close, environment, run_step
 from tests.oracle_lib import OracleNetwork
 from tests.test_gpu_lstm import LSTM_TAPS, _rows, _width
 from tests.test_oracle_lstm_norm import lstm, parameters
@@ -80,6 +80,14 @@ CASES = [   # name, layers, T, B, Bmax
 ]
 
 
+@pytest.fixture(params=["one-launch-per-step", "launch-per-kernel"], autouse=True)
+def step_form(request):
+    """every test runs with a time step's work behind its recurrent contraction as one launch (the default) and as the sequence
+    of statistics / apply / gate launches"""
+    with environment(MYEA_LSTM_NORM_FUSED="1" if request.param == "one-launch-per-step" else "0"):
+        yield request.param
+
+
 @pytest.mark.parametrize("name,specs,T,B,Bmax", CASES, ids=[c[0] for c in CASES])
 def test_training_steps_match_the_oracle(name, specs, T, B, Bmax):
     hyper = dict(batch_renormalization_r_correction_maximum=2.0, batch_renormalization_d_correction_maximum=3.0, normalization_momentum_average=0.3)
@@ -136,3 +144,22 @@ def test_running_statistics_can_be_restored():
         n.set_state_propagation(mb.STATE_INFERENCE)
         n.Forward_Pass(B, X)
     _close(gpu.download_tensor(2, mb.TENSOR["OUTPUTS"], T * B * 12), cpu.download_tensor(2, mb.TENSOR["OUTPUTS"], T * B * 12), "outputs from restored statistics")
+
+
+def test_a_time_step_is_two_launches_per_pass(step_form):
+    """behind its recurrent contraction a time step's normalisations and gate math are one launch (forward and backward); as
+    separate kernels the same step takes six resp. six launches, which the library's own launch counter shows"""
+    specs = [dict(units=8), lstm(32), dict(units=32, activation="LINEAR")]
+    T, B = 6, 16
+    desc, gpu, cpu = _pair(specs, B, T, 53)
+    rng = np.random.default_rng(4)
+    X = rng.normal(0, 1, (B, T * 8)).astype(np.float32)
+    Y = rng.normal(0, 1, (B, T * 32)).astype(np.float32)
+    gpu.profile_enable(True)
+    run_step(gpu, B, X, Y, update=False)
+    launches = gpu.profile_read(7)[0]       # the normalisation family's timed regions: one per launch group
+    gpu.profile_enable(False)
+    if step_form == "one-launch-per-step":
+        assert launches == 2 * T
+    else:
+        assert launches > 2 * T
