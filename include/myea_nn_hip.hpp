@@ -173,9 +173,12 @@ public:
         Compute__Regularization__Constraint_Recurrent_Weight__Default(index_layer, &lo, &hi);
         return Set__Regularization__Constraint_Recurrent_Weight(index_layer, lo, hi);
     }
+    // Train.cpp:676-720: a steepness in [0, 1], any layer of the network (the example program walks all of them, the input layer,
+    // residual and pooling layers included: those have no activation to steepen and the value means nothing there)
     bool Set__Layer_Activation_Steepness(size_t index_layer, T_ activation_steepness)
     {
-        if (!CheckLayer("Set__Layer_Activation_Steepness", index_layer)) return false;
+        if (activation_steepness < 0.f || activation_steepness > 1.f) return Fail("Set__Layer_Activation_Steepness", "activation steepness outside [0, 1]");
+        if (index_layer >= desc_.n_layers) return Fail("Set__Layer_Activation_Steepness", "layer index overflow");
         desc_.layers[index_layer].activation_steepness = activation_steepness;
         return Dirty();
     }
@@ -235,6 +238,13 @@ public:
         clip_gradient = value;
         for (size_t i = 0; i < desc_.n_layers; ++i)
             if (follows[i] && !Set__Regularization__Constraint_Recurrent_Weight__Default(i)) return false;
+        return true;
+    }
+    // Neural_Network__Regularization__Max_Norm_Constraints.cpp:24-46: a negative bound prints and returns false
+    bool Set__Regularization__Max_Norm_Constraints(T_ v)
+    {
+        if (v < 0.f) return Fail("Set__Regularization__Max_Norm_Constraints", "max-norm constraints less than zero");
+        regularization__max_norm_constraints = v;
         return true;
     }
     bool Set__Accurancy_Variance(T_ v) { accuracy_variance = v; return true; }

@@ -194,7 +194,9 @@ static int check_desc(const myea_net_desc &d)
             const double span = l.type_layer == MYEA_LAYER_AVERAGE_POOLING ? in + 2 * pad - k : in + 2 * pad - dil * (k - 1) - 1;
             const double out = span < 0 ? 0 : (l.pooling_values[4] == 0 ? std::floor(span / st + 1.0) : std::ceil(span / st + 1.0));
             if (out < 1 || (double)l.n_units != out) { set_last_error("layer %u: pooling width %u does not follow from its parameters (%.0f)", li, l.n_units, out); return MYEA_E_INVALID; }
-            if (l.type_dropout != MYEA_DROPOUT_NONE || l.type_normalization != MYEA_NORMALIZATION_NONE) { set_last_error("layer %u: a pooling layer carries no dropout or normalization", li); return MYEA_E_UNSUPPORTED; }
+            // (a normalisation type on a pooling layer is accepted and means nothing: the reference's setter takes any hidden layer,
+            // NN/Neural_Network__Layer_Normalization.cpp:217-288, the layer owns no normalised unit and its passes never look at the field)
+            if (l.type_dropout != MYEA_DROPOUT_NONE) { set_last_error("layer %u: a pooling layer carries no dropout", li); return MYEA_E_UNSUPPORTED; }
         }
     }
     for (uint32_t li = 0; li < d.n_layers; ++li) {
@@ -242,6 +244,8 @@ int Net::create(const myea_net_desc &desc)
 {
     MYEA_TRY(check_desc(desc));
     d = desc;
+    for (uint32_t li = 0; li < d.n_layers; ++li)   // see check_desc: the field means nothing on a pooling layer
+        if (layer_is_pooling(d.layers[li])) d.layers[li].type_normalization = MYEA_NORMALIZATION_NONE;
     myea_hyper_default(&h);
     const size_t P = d.total_parameters, T = d.number_recurrent_depth, B = d.batch_size;
     MYEA_TRY(dev_alloc(&parameters, P));

@@ -261,6 +261,12 @@ int myea_oracle_create(const myea_net_desc *desc, myea_oracle_net **out)
     myea_oracle_net *n = (myea_oracle_net *)calloc(1, sizeof(*n));
     if (!n) return MYEA_E_NOMEM;
     n->d = *desc;
+    /* a pooling layer may carry a normalisation type (the reference's setter takes any hidden layer, Neural_Network__Layer_
+     * Normalization.cpp:217-288; its example program sets one on every hidden layer): the layer owns no normalised unit and
+     * its passes never look at the field, so this copy of the description drops it */
+    for (size_t li = 0; li < n->d.n_layers; ++li)
+        if (n->d.layers[li].type_layer == MYEA_LAYER_AVERAGE_POOLING || n->d.layers[li].type_layer == MYEA_LAYER_MAX_POOLING) n->d.layers[li].type_normalization = MYEA_NORMALIZATION_NONE;
+    desc = &n->d;
     myea_hyper_default(&n->h);
     n->threads = 1;
     size_t P = desc->total_parameters, T = desc->number_recurrent_depth, B = desc->batch_size;

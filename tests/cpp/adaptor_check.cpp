@@ -111,6 +111,45 @@ int main(int argc, char **argv)
         if (!nn.Set__Layer_Activation_Function(3, MYEA_AF_LINEAR)) return 1;
         nn.Set__Loss_Function(MYEA_LOSS_MSE);
         nn.Set__Optimizer_Function(MYEA_OPTIMIZER_GD);
+    } else if (kind == "example") {
+        // The network of the reference's worked example, built with its sequence of calls (Neural_Network_Launcher_Windows/Source_Files/
+        // debug.cpp:693-1075 the layer list, :1160-1230 time delays and activations, :1317 the constraint, :1503-1520 the normalisation of
+        // EVERY hidden layer - residual and pooling layers included): sMNIST rows, an independently recurrent first hidden layer, three
+        // groups of three residual blocks of three independently recurrent members, 9 units narrower in all over the nine blocks, a max
+        // pooling (kernel 2, stride 2, dilation 0) between the groups, ISRLU, softmax head, AMSGrad, max-norm constraint 8
+        B = 12; T = 5; n_in = 28; n_out = 10;
+        std::vector<Layer_Parameters> lp;
+        Layer_Parameters l;
+        l.type_layer = MYEA_LAYER_FULLY_CONNECTED; l.unit_parameters[0] = 28; lp.push_back(l);
+        l.type_layer = MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT; l.unit_parameters[0] = 32; lp.push_back(l);
+        double width = 32.0;
+        const double widening = -9.0 / 9.0;
+        for (int group = 0; group < 3; ++group) {
+            if (group) {
+                l.type_layer = MYEA_LAYER_MAX_POOLING;
+                l.unit_parameters[0] = 2; l.unit_parameters[1] = 2; l.unit_parameters[2] = 0; l.unit_parameters[3] = 0; l.unit_parameters[4] = 0;
+                lp.push_back(l);
+            }
+            for (int block = 0; block < 3; ++block) {
+                l.type_layer = MYEA_LAYER_RESIDUAL; l.unit_parameters[0] = 3; lp.push_back(l);
+                width += widening;
+                l.type_layer = MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT; l.unit_parameters[0] = (size_t)width;
+                for (int member = 0; member < 3; ++member) lp.push_back(l);
+            }
+        }
+        l.type_layer = MYEA_LAYER_FULLY_CONNECTED; l.unit_parameters[0] = 10; lp.push_back(l);
+        if (!nn.Update__Batch_Size(B)) return 1;
+        if (!nn.Compile(lp.size(), T, MYEA_NETWORK_FEEDFORWARD, lp.data())) return 1;
+        if (!nn.Set__Number_Time_Delays(T - 1)) return 1;
+        for (size_t i = 0; i < lp.size(); ++i) if (!nn.Set__Layer_Activation_Steepness(i, 1.f)) return 1;
+        for (size_t i = 1; i + 1 < lp.size(); ++i) if (!nn.Set__Layer_Activation_Function(i, MYEA_AF_ISRLU)) return 1;
+        if (!nn.Set__Layer_Activation_Function(lp.size() - 1, MYEA_AF_SOFTMAX)) return 1;
+        nn.Set__Loss_Function(MYEA_LOSS_CROSS_ENTROPY);
+        nn.Set__Accuracy_Function(MYEA_ACCURACY_CROSS_ENTROPY);
+        nn.Set__Optimizer_Function(MYEA_OPTIMIZER_AMSGRAD);
+        if (!nn.Set__Regularization__Max_Norm_Constraints(8.f)) return 1;
+        for (size_t i = 1; i + 1 < lp.size(); ++i) if (!nn.Set__Layer_Normalization(i, MYEA_NORMALIZATION_BATCH_NORMALIZATION, true)) return 1;
+        if (!nn.Set__Normalization_Momentum_Average(1.f) || !nn.Set__Normalization_Epsilon(0.1f)) return 1;
     } else {  // LSTM 8 -> 2 x LSTM-12 -> FC-12 linear, AMSGrad, clip 1.0
         B = 6; T = 5; n_in = 8; n_out = 12;
         Layer_Parameters layers[4];

@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 BIN = os.path.join(HERE, "cpp", "adaptor_check")
 
 
-def _run(tmp_path, kind, specs, B, T, hyper, X, Y, masks, seed):
+def _run(tmp_path, kind, specs, B, T, hyper, X, Y, masks, seed, gradient_close=None):
     desc = mb.make_desc(specs, B, T)
     w = glorot_parameters(desc, seed, bias_range=0.3)
     for name, arr in (("w", w), ("x", X), ("y", Y), ("mask", masks.astype(np.float32))):
@@ -37,7 +37,7 @@ def _run(tmp_path, kind, specs, B, T, hyper, X, Y, masks, seed):
     got_losses = [float(l.split()[-1]) for l in out.stdout.splitlines() if l.startswith("step ")]
     assert got_losses == pytest.approx(losses, rel=1e-4)
     assert "time step 3.0" in out.stdout and "ERROR" in out.stdout     # the oversized batch printed and returned
-    assert_close(np.fromfile(str(tmp_path / "grad.bin"), dtype=np.float32), g, 1e-4, 1e-5, what="gradient")
+    (gradient_close or (lambda a, b: assert_close(a, b, 1e-4, 1e-5, what="gradient")))(np.fromfile(str(tmp_path / "grad.bin"), dtype=np.float32), g)
     return np.fromfile(str(tmp_path / "params.bin"), dtype=np.float32), cpu.download_parameters(), g
 
 
@@ -88,3 +88,30 @@ def test_adaptor_ind_rnn_default_bounds_and_clip(tmp_path):
     l = desc.layers[2]
     u = got[l.last_connection_index - 12:l.last_connection_index]
     assert u.min() >= -0.5 and u.max() <= 0.75
+
+
+def test_adaptor_builds_and_trains_the_reference_example_network(tmp_path):
+    """The host program makes the calls of the reference's worked example in its order (residual blocks of independently
+    recurrent members, pooling between the groups, normalisation set on every hidden layer, AMSGrad, max-norm constraint, the
+    label read at the last time step); the description it arrives at must be the builder's, its three steps the oracle's."""
+    from myea_amd.synthetic import simple_debug_layers
+    specs = simple_debug_layers()
+    B, T = 12, 5
+    rng = np.random.default_rng(5)
+    X = rng.uniform(0, 1, (B, T * 28)).astype(np.float32)
+    Y = np.zeros((B, T, 10), np.float32)
+    np.put_along_axis(Y, rng.integers(0, 10, (B, T))[..., None], 1.0, axis=2)
+    Y = Y.reshape(B, T * 10)
+    desc = mb.make_desc(specs, B, T, network=mb.NETWORK_FEEDFORWARD)
+    masks = np.ones(max(1, desc.total_mask_units), dtype=np.uint8)[:desc.total_mask_units]
+    hyper = dict(type_optimizer_function=mb.OPTIMIZER["AMSGRAD"], type_loss_function=mb.LOSS["CROSS_ENTROPY"], type_accuracy_function=mb.ACCURACY["CROSS_ENTROPY"],
+                 regularization__max_norm_constraints=8.0, normalization_momentum_average=1.0, normalization_epsilon=0.1, number_time_delays=T - 1)
+    def mostly_close(a, b):
+        """rel 1e-4 / abs 1e-5, up to 1 % of the entries off by up to 1 %: 28 normalisations over 12 examples amplify fp32 rounding"""
+        err = np.abs(a.astype(np.float64) - b)
+        bad = err > 1e-4 * np.abs(b) + 1e-5
+        assert bad.mean() <= 0.01 and np.all(err[bad] <= 1e-2 * np.abs(b[bad]) + 1e-4), "gradient: %d / %d out of tolerance" % (int(bad.sum()), a.size)
+    got, want, _ = _run(tmp_path, "example", specs, B, T, hyper, X, Y, masks, seed=5, gradient_close=mostly_close)
+    # three AMSGrad steps without re-synchronisation: entries driven by rounding-noise gradients may move by up to lr per step
+    close = np.abs(got.astype(np.float64) - want) <= 1e-5 + 1e-4 * np.abs(want)
+    assert close.mean() > 0.98 and np.max(np.abs(got.astype(np.float64) - want)) <= 3 * 2.1e-3
