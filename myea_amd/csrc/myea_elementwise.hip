@@ -58,6 +58,9 @@ __global__ __launch_bounds__(kBlock) void activation_derive_kernel(int act, floa
 // Forward_Pass__FC_Ind_RNN (NN/Neural_Network__Recurrent_Forward_Pass__Loop.cpp:813-866): pre_AF[t] = input[t] + u * AF[t-1]
 // (a copy at t = 0), then Forward_Pass__FC_AF and, for an un-normalised layer, the Bernoulli applier in place on AF - the
 // value the next time step reads.
+// (The operands of kChunk time steps are requested together, ahead of the chain of dependent steps that consumes them: the
+// chain then waits for memory once per chunk instead of once per step.)
+constexpr int kIndRnnChunk = 32;
 __global__ __launch_bounds__(kBlock) void ind_rnn_forward_kernel(IndRnnParams p)
 {
     const size_t n = p.B * p.H, step = p.Bmax * p.H;
@@ -66,15 +69,25 @@ __global__ __launch_bounds__(kBlock) void ind_rnn_forward_kernel(IndRnnParams p)
         const float u = p.u[j];
         const int act = p.unit_act ? p.unit_act[j] : p.act;
         float h = 0.f;
-        size_t k = i;
-#pragma unroll 4
-        for (size_t t = 0; t < p.T; ++t, k += step) {
-            float pre = p.in[k];
-            if (t) pre = __fadd_rn(pre, __fmul_rn(u, h));
-            p.pre_afs[k] = pre;
-            h = af_fire(act, pre);
-            if (p.colscale) h *= p.colscale[t * p.H + j];
-            p.afs[k] = h;
+        for (size_t t0 = 0; t0 < p.T; t0 += kIndRnnChunk) {
+            const size_t k0 = i + t0 * step;
+            const int m = (int)(p.T - t0 < (size_t)kIndRnnChunk ? p.T - t0 : (size_t)kIndRnnChunk);
+            float x[kIndRnnChunk], cs[kIndRnnChunk];
+#pragma unroll
+            for (int s = 0; s < kIndRnnChunk; ++s) {
+                x[s] = s < m ? p.in[k0 + s * step] : 0.f;
+                cs[s] = (p.colscale && s < m) ? p.colscale[(t0 + s) * p.H + j] : 1.f;
+            }
+#pragma unroll
+            for (int s = 0; s < kIndRnnChunk; ++s) {
+                if (s >= m) break;
+                float pre = x[s];
+                if (t0 + s) pre = __fadd_rn(pre, __fmul_rn(u, h));
+                p.pre_afs[k0 + s * step] = pre;
+                h = af_fire(act, pre);
+                if (p.colscale) h *= cs[s];
+                p.afs[k0 + s * step] = h;
+            }
         }
     }
 }
@@ -89,15 +102,25 @@ __global__ __launch_bounds__(kBlock) void ind_rnn_backward_kernel(IndRnnParams p
         const float u = p.u[j], steep = p.unit_steep ? p.unit_steep[j] : p.steep;
         const int act = p.unit_act ? p.unit_act[j] : p.act;
         float next = 0.f;
-        size_t k = i + (p.T - 1) * step;
-#pragma unroll 4
-        for (size_t t = p.T; t-- > 0; k -= step) {
-            const float daf = af_derive(act, p.pre_afs[k], steep, p.afs[k]);
-            const float e = __fmul_rn(p.dy[k], daf);
-            const float r = (t + 1 == p.T) ? e : __fadd_rn(e, __fmul_rn(__fmul_rn(u, daf), next));
-            p.dafs[k] = r;
-            next = r;
-            if (t == 0) break;
+        for (size_t done = 0; done < p.T; done += kIndRnnChunk) {   // time steps T-1-done, T-2-done, ...
+            const int m = (int)(p.T - done < (size_t)kIndRnnChunk ? p.T - done : (size_t)kIndRnnChunk);
+            const size_t top = p.T - 1 - done;
+            float pre[kIndRnnChunk], val[kIndRnnChunk], dy[kIndRnnChunk];
+#pragma unroll
+            for (int s = 0; s < kIndRnnChunk; ++s) {
+                const size_t k = i + (top - (s < m ? s : 0)) * step;
+                pre[s] = p.pre_afs[k]; val[s] = p.afs[k]; dy[s] = p.dy[k];
+            }
+#pragma unroll
+            for (int s = 0; s < kIndRnnChunk; ++s) {
+                if (s >= m) break;
+                const size_t t = top - s;
+                const float daf = af_derive(act, pre[s], steep, val[s]);
+                const float e = __fmul_rn(dy[s], daf);
+                const float r = (t + 1 == p.T) ? e : __fadd_rn(e, __fmul_rn(__fmul_rn(u, daf), next));
+                p.dafs[i + t * step] = r;
+                next = r;
+            }
         }
     }
 }
@@ -1237,11 +1260,22 @@ __global__ __launch_bounds__(kBlock) void bn_forward_sequence_kernel(BnForwardPa
     }
 }
 
+static int sequence_columns(size_t H, size_t T)
+{
+    for (int cw : {64, 16})
+        if ((H + cw - 1) / cw * T >= 256) return cw;
+    return 4;
+}
+
 int launch_bn_forward_sequence(hipStream_t s, const BnForwardParams &p, size_t T, size_t Bmax, int training)
 {
     if (p.H == 0 || p.rows == 0 || T == 0) return MYEA_OK;
     if (p.rows > Bmax || T > 65535) { set_last_error("bn_forward_sequence: %zu rows of %zu, %zu time steps", p.rows, Bmax, T); return MYEA_E_INVALID; }
-    if (p.H <= 32) hipLaunchKernelGGL(bn_forward_sequence_kernel<16>, dim3((unsigned)((p.H + 15) / 16), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, training);
+    // the widest column block that still gives the device a workgroup per compute unit: a launch is a chain of memory round trips,
+    // shorter the more row lanes share a column
+    const int cw = sequence_columns(p.H, T);
+    if (cw == 4) hipLaunchKernelGGL(bn_forward_sequence_kernel<4>, dim3((unsigned)((p.H + 3) / 4), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, training);
+    else if (cw == 16) hipLaunchKernelGGL(bn_forward_sequence_kernel<16>, dim3((unsigned)((p.H + 15) / 16), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, training);
     else hipLaunchKernelGGL(bn_forward_sequence_kernel<64>, dim3((unsigned)((p.H + 63) / 64), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, training);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
@@ -1316,9 +1350,14 @@ int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t
 {
     if (p.H == 0 || p.rows == 0 || T == 0) return MYEA_OK;
     if (p.rows > Bmax || T > 65535) { set_last_error("bn_backward_sequence: %zu rows of %zu, %zu time steps", p.rows, Bmax, T); return MYEA_E_INVALID; }
-    if (p.H <= 32) hipLaunchKernelGGL(bn_backward_sequence_kernel<16>, dim3((unsigned)((p.H + 15) / 16), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, scratch);
-    else hipLaunchKernelGGL(bn_backward_sequence_kernel<64>, dim3((unsigned)((p.H + 63) / 64), (unsigned)T), dim3(kBlock), 0, s, p, Bmax, scratch);
+    const int cw = sequence_columns(p.H, T);
+    const size_t blocks = (p.H + cw - 1) / cw;
+    if (cw == 4) hipLaunchKernelGGL(bn_backward_sequence_kernel<4>, dim3((unsigned)blocks, (unsigned)T), dim3(kBlock), 0, s, p, Bmax, scratch);
+    else if (cw == 16) hipLaunchKernelGGL(bn_backward_sequence_kernel<16>, dim3((unsigned)blocks, (unsigned)T), dim3(kBlock), 0, s, p, Bmax, scratch);
+    else hipLaunchKernelGGL(bn_backward_sequence_kernel<64>, dim3((unsigned)blocks, (unsigned)T), dim3(kBlock), 0, s, p, Bmax, scratch);
     MYEA_HIP_TRY(hipGetLastError());
+    // (the shares are added by a launch of their own: a column block's last workgroup could add them itself, but the release of its
+    // stores to the other XCDs' workgroups costs more than the launch - 38 against 9 + 8 us measured)
     hipLaunchKernelGGL(bn_backward_sequence_final_kernel, dim3(grid_for(p.H, kBlock)), dim3(kBlock), 0, s, p.H, T, scratch, p.dscale, p.dshift);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
