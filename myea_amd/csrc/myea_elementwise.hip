@@ -310,13 +310,23 @@ struct SumF {
     __device__ void operator()(size_t r, size_t col, double *acc) const { acc[0] += x[r * H + col]; }
 };
 
+// grid: ceil(H / 64) workgroups; four row lanes per column (lane r: slabs r, r + 4, ...) whose sums meet in LDS and are added in
+// lane order - the launch is a short chain of loads, shorter the more lanes share a column
 __global__ __launch_bounds__(kBlock) void column_sum_final_kernel(size_t H, size_t S, const float *partial, float *out, int accumulate)
 {
-    const size_t col = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (col >= H) return;
+    __shared__ double red[kBlock / 64][64];
+    const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6;
+    const size_t col = (size_t)blockIdx.x * 64 + cl;
     double s = 0.0;
+    if (col < H) {
 #pragma unroll 8
-    for (size_t y = 0; y < S; ++y) s += partial[y * H + col];
+        for (size_t y = rl; y < S; y += kBlock / 64) s += partial[y * H + col];
+    }
+    red[rl][cl] = s;
+    __syncthreads();
+    if (rl != 0 || col >= H) return;
+#pragma unroll
+    for (int r = 1; r < kBlock / 64; ++r) s += red[r][cl];
     out[col] = accumulate ? out[col] + (float)s : (float)s;
 }
 
@@ -1030,7 +1040,7 @@ int launch_column_sum(hipStream_t s, size_t rows, size_t H, const float *x, floa
     SumF f{x, H};
     hipLaunchKernelGGL((column_partial_kernel<1, SumF>), dim3((unsigned)((H + 63) / 64), (unsigned)S), dim3(kBlock), 0, s, rows, H, chunk, scratch, f);
     MYEA_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, kBlock)), dim3(kBlock), 0, s, H, S, scratch, out, accumulate);
+    hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, 64)), dim3(kBlock), 0, s, H, S, scratch, out, accumulate);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
@@ -1038,7 +1048,7 @@ int launch_column_sum(hipStream_t s, size_t rows, size_t H, const float *x, floa
 int launch_column_sum_final(hipStream_t s, size_t H, size_t S, const float *partial, float *out, int accumulate)
 {
     if (H == 0) return MYEA_OK;
-    hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, kBlock)), dim3(kBlock), 0, s, H, S, partial, out, accumulate);
+    hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, 64)), dim3(kBlock), 0, s, H, S, partial, out, accumulate);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
@@ -1110,7 +1120,7 @@ int launch_ind_rnn_self_weight_gradient(hipStream_t s, size_t T, size_t B, size_
     IndRnnDotF f{afs, dafs, H, B, Bmax};
     hipLaunchKernelGGL((column_partial_kernel<1, IndRnnDotF>), dim3((unsigned)((H + 63) / 64), (unsigned)S), dim3(kBlock), 0, s, rows, H, chunk, scratch, f);
     MYEA_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, kBlock)), dim3(kBlock), 0, s, H, S, scratch, du, 1);
+    hipLaunchKernelGGL(column_sum_final_kernel, dim3(grid_for(H, 64)), dim3(kBlock), 0, s, H, S, scratch, du, 1);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
@@ -1397,6 +1407,8 @@ int launch_compute_error(hipStream_t s, const ErrorParams &p)
     const size_t nrows = (p.T - p.first_t) * p.B;
     auto aligned = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     const bool vec = (p.H & 3) == 0 && aligned(p.values) && aligned(p.desired) && aligned(p.pre) && aligned(p.errors);
+    // 2048 workgroups: fewer leave long queues of rows behind each wavefront (512: 66 us for config-3-sized 16 384 rows of 512 against 54),
+    // more lengthen the queue of fp64 atomics every workgroup ends with (8192: 69 us, and 113 against 52 on 32 768 rows of 32)
     if (vec) hipLaunchKernelGGL(compute_error_kernel<4>, dim3(grid_for(nrows, kBlock / 64, 2048)), dim3(kBlock), 0, s, p);
     else hipLaunchKernelGGL(compute_error_kernel<1>, dim3(grid_for(nrows, kBlock / 64, 1024)), dim3(kBlock), 0, s, p);
     MYEA_HIP_TRY(hipGetLastError());
