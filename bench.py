@@ -25,10 +25,10 @@ if ROOT not in sys.path:
 # HBM bytes per contraction launch (mean over the launches of one step): NOT measured by this script's run.  Recorded
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same counters read for copies of
 # known size (FETCH_SIZE x2, WRITE_SIZE x1); the line names the file the figure comes from.
-RECORDED_TRAFFIC = {"fc4096x4_b1024_adam": dict(bytes_per_launch=2944490 * 1024 / 10,
+RECORDED_TRAFFIC = {"fc4096x4_b1024_adam": dict(bytes_per_launch=2951372 * 1024 / 10,
                                                 source="recorded constant, not measured in this run: profiles/hbm_traffic__fc4096x4_b1024_adam__pmc.txt"),
                     # the two resident time loops of one layer (forward + backward launch), mean per launch
-                    "lstm512x2_t64_b256_amsgrad": dict(bytes_per_launch=(299.0e6 + 400.0e6) / 2,
+                    "lstm512x2_t64_b256_amsgrad": dict(bytes_per_launch=(2 * 98047.4 + 230411.9 + 2 * 195875.0 + 197752.0) * 1024 / 2,
                                                        source="recorded constant, not measured in this run: profiles/lstm_resident__lstm512x2_t64_b256_amsgrad__pmc.txt")}
 from myea_amd.synthetic import simple_debug_layers  # noqa: E402  (no device is touched by the import)
 

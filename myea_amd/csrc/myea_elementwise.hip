@@ -1407,7 +1407,7 @@ int launch_compute_error(hipStream_t s, const ErrorParams &p)
     const size_t nrows = (p.T - p.first_t) * p.B;
     auto aligned = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     const bool vec = (p.H & 3) == 0 && aligned(p.values) && aligned(p.desired) && aligned(p.pre) && aligned(p.errors);
-    // 2048 workgroups: fewer leave long queues of rows behind each wavefront (512: 66 us for config-3-sized 16 384 rows of 512 against 54),
+    // 2048 workgroups: fewer leave long queues of rows behind each wavefront (512: 66 us for 16 384 rows of 512 against 54),
     // more lengthen the queue of fp64 atomics every workgroup ends with (8192: 69 us, and 113 against 52 on 32 768 rows of 32)
     if (vec) hipLaunchKernelGGL(compute_error_kernel<4>, dim3(grid_for(nrows, kBlock / 64, 2048)), dim3(kBlock), 0, s, p);
     else hipLaunchKernelGGL(compute_error_kernel<1>, dim3(grid_for(nrows, kBlock / 64, 1024)), dim3(kBlock), 0, s, p);
