@@ -153,16 +153,20 @@ inline bool Neural_Network_HIP::Save_Dimension_Parameters(std::string const &pat
     size_t n_basic = 0, n_indice = 0, n_neuron = 0, n_af = 0, n_ind = 0, n_block = 0, n_cell = 0, n_norm = 0;
     for (size_t li = 0; li < L; ++li) {
         const myea_layer_desc &l = desc_.layers[li];
-        if (li > 1 && l.type_layer == MYEA_LAYER_FULLY_CONNECTED) {
-            if (desc_.layers[li - 1].type_layer == MYEA_LAYER_RESIDUAL) group[li] = 1;
-            else if (group[li - 1] != 0 && myea_net_desc_previous_layer(&desc_, (uint32_t)li) == li - 1) group[li] = 2;
-        }
+        // a residual block's dense members (fully-connected or independently recurrent) keep their activation, recurrent and
+        // normalised units on their input side: none on the block's first member, fan-in many on the others
+        // (Assign__Post__Residual_Layer, Neural_Network__Compile.cpp:283-376)
+        if (l.type_layer == MYEA_LAYER_RESIDUAL)
+            for (size_t m = li + 1; m <= li + l.block_depth && m < L; ++m)
+                if (desc_.layers[m].type_layer == MYEA_LAYER_FULLY_CONNECTED || desc_.layers[m].type_layer == MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT)
+                    group[m] = m == li + 1 ? 1 : 2;
         const size_t H = width(li), In = li ? width(myea_net_desc_previous_layer(&desc_, (uint32_t)li)) : 0;
         neuron_at[li] = n_neuron; cell_at[li] = n_cell; basic_at[li] = n_basic; indice_at[li] = n_indice; ind_at[li] = n_ind;
         switch (l.type_layer) {
         case MYEA_LAYER_FULLY_CONNECTED:
             n_neuron += H; af_units[li] = group[li] == 0 ? H : (group[li] == 1 ? 0 : In); n_af += af_units[li]; norm_units[li] = group[li] == 0 ? H : In; break;
-        case MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT: n_neuron += H; n_ind += H; norm_units[li] = H; break;
+        case MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT:
+            n_neuron += H; af_units[li] = group[li] == 0 ? H : (group[li] == 1 ? 0 : In); n_ind += af_units[li]; norm_units[li] = group[li] == 0 ? H : In; break;
         case MYEA_LAYER_LSTM: n_block += (size_t)l.n_units * dirs(li); n_cell += H * dirs(li); norm_units[li] = (3 * H + 6 * l.n_units) * dirs(li); break;
         case MYEA_LAYER_RESIDUAL: n_basic += H; norm_units[li] = width(li + l.block_depth); break;
         case MYEA_LAYER_AVERAGE_POOLING: n_basic += H; break;
@@ -307,8 +311,8 @@ inline bool Neural_Network_HIP::Save_Dimension_Parameters(std::string const &pat
             if (l.type_layer == MYEA_LAYER_FULLY_CONNECTED) af(li);
             else {   // Information__Layer__AF_Ind_Recurrent, :844-863
                 const size_t H = width(li), u0 = l.first_connection_index + H * width(myea_net_desc_previous_layer(&desc_, (uint32_t)li));
-                line("    ", "number_AF_Ind_recurrent_units", str(H));
-                for (size_t u = 0; u < H; ++u) {
+                line("    ", "number_AF_Ind_recurrent_units", str(af_units[li]));
+                for (size_t u = 0; u < af_units[li]; ++u) {
                     s += "      AF_Ind_R["; s += str(u); s += "]\n";
                     line("        ", "activation_steepness", TS(l.activation_steepness)); line("        ", "activation_function", str(l.type_activation_function));
                     line("        ", "connected_to_AF_Ind_R", str(ind_at[li] + u)); weight("        ", u0 + u);

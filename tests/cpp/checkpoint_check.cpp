@@ -71,6 +71,25 @@ static bool build(Neural_Network_HIP &nn, const std::string &kind, size_t B, siz
         if (!nn.Set__Layer_Activation_Function(2, MYEA_AF_LINEAR) || !nn.Set__Layer_Normalization(1, MYEA_NORMALIZATION_BATCH_RENORMALIZATION)) return false;
         nn.Set__Loss_Function(MYEA_LOSS_MSE); nn.Set__Optimizer_Function(MYEA_OPTIMIZER_ADAM);
         nn.normalization_momentum_average = 0.5f; nn.batch_renormalization_r_correction_maximum = 2.f; nn.batch_renormalization_d_correction_maximum = 1.f;
+    } else if (kind == "recurrent_residual") {
+        // 6 -> IndRNN-8 tanh (BN before) -> residual block of 3 (block BN; members: IndRNN-8, IndRNN-8 with BN, LSTM 8 blocks of one cell)
+        //   -> max pooling (kernel 2, stride 2, dilation 0) -> 4 linear, T = 3
+        *T = 3; *n_in = 6; *n_out = 4;
+        Layer_Parameters layers[8];
+        layers[0].type_layer = MYEA_LAYER_FULLY_CONNECTED; layers[0].unit_parameters[0] = 6;
+        layers[1].type_layer = MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT; layers[1].unit_parameters[0] = 8;
+        layers[2].type_layer = MYEA_LAYER_RESIDUAL; layers[2].unit_parameters[0] = 3;
+        layers[3].type_layer = layers[4].type_layer = MYEA_LAYER_FULLY_CONNECTED_INDEPENDENTLY_RECURRENT; layers[3].unit_parameters[0] = layers[4].unit_parameters[0] = 8;
+        layers[5].type_layer = MYEA_LAYER_LSTM; layers[5].unit_parameters[0] = 8; layers[5].unit_parameters[1] = 1;
+        layers[6].type_layer = MYEA_LAYER_MAX_POOLING; layers[6].unit_parameters[0] = 2; layers[6].unit_parameters[1] = 2;
+        layers[7].type_layer = MYEA_LAYER_FULLY_CONNECTED; layers[7].unit_parameters[0] = 8;   // >= the LSTM member's cells: its bias vectors reach into these slots
+        if (!nn.Compile(8, *T, MYEA_NETWORK_RECURRENT, layers)) return false;
+        *n_out = 8;
+        if (!nn.Set__Layer_Activation_Function(1, MYEA_AF_TANH) || !nn.Set__Layer_Activation_Function(3, MYEA_AF_TANH) || !nn.Set__Layer_Activation_Function(4, MYEA_AF_ISRLU) ||
+            !nn.Set__Layer_Activation_Function(7, MYEA_AF_LINEAR) || !nn.Set__Layer_Normalization(1, MYEA_NORMALIZATION_BATCH_NORMALIZATION) ||
+            !nn.Set__Layer_Normalization(2, MYEA_NORMALIZATION_BATCH_NORMALIZATION) || !nn.Set__Layer_Normalization(4, MYEA_NORMALIZATION_BATCH_NORMALIZATION) ||
+            !nn.Set__Layer_Normalization(6, MYEA_NORMALIZATION_BATCH_NORMALIZATION)) return false;   // on a pooling layer: taken, means nothing
+        nn.Set__Loss_Function(MYEA_LOSS_MSE); nn.Set__Optimizer_Function(MYEA_OPTIMIZER_AMSGRAD);
     } else {   // 8 -> 12 tanh -> residual block of 2 (block BN, ShakeDrop; members 10 and 14: wider than the shortcut) -> 4 linear
         *T = 1; *n_in = 8; *n_out = 4;
         Layer_Parameters layers[6];

@@ -82,6 +82,9 @@ def _check_files(tmp_path, kind):
         assert len(scales) == 54
         for u, v in enumerate(scales):   # unit u = 9 * block + group keeps its scale at group * 6 + block
             assert v == p[base + (u % 9) * 6 + u // 9], u
+    if kind == "recurrent_residual":
+        # a member's recurrent units sit on its input side; the block's first member owns none
+        assert "    block_depth 3" in lines and "    number_block_units 8" in lines and sum(l.strip().startswith("connected_to_AF_Ind_R") for l in lines) >= 8
     if kind == "residual":
         assert "    block_depth 2" in lines and "    padding 1" in lines and "    number_basic_units 14" in lines and "          connected_to_basic 0" in lines
     # every weight line carries its flat index: the values are the parameters at those indices
@@ -96,14 +99,14 @@ def _check_files(tmp_path, kind):
     assert seen > 100
 
 
-@pytest.mark.parametrize("kind", ["mlp", "recurrent", "normalised", "residual"])
+@pytest.mark.parametrize("kind", ["mlp", "recurrent", "normalised", "residual", "recurrent_residual"])
 def test_checkpoint_round_trip_on_the_host(tmp_path, kind):
     _run(tmp_path, kind, device=False)
     _check_files(tmp_path, kind)
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kind", ["mlp", "recurrent", "normalised", "residual"])
+@pytest.mark.parametrize("kind", ["mlp", "recurrent", "normalised", "residual", "recurrent_residual"])
 def test_checkpoint_round_trip_through_the_device(tmp_path, kind):
     out = _run(tmp_path, kind, device=True)
     assert "inference outputs" in out and "differing 0 magnitude" in out
