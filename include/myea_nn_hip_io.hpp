@@ -181,7 +181,7 @@ inline bool Neural_Network_HIP::Save_Dimension_Parameters(std::string const &pat
     std::vector<size_t> first_norm(L, 0);
     for (size_t li = 0; li < L; ++li) {
         first_norm[li] = norm_at; norm_at += norm_units[li];
-        if (desc_.layers[li].type_normalization == MYEA_NORMALIZATION_NONE) continue;
+        if (desc_.layers[li].type_normalization == MYEA_NORMALIZATION_NONE || norm_units[li] == 0) continue;   // (a pooling layer owns no normalised unit, whatever its type says)
         mean[li].assign(T * norm_units[li], 0.f); var[li].assign(T * norm_units[li], 1.f);
         if (li < norm_means_averages_.size() && norm_means_averages_[li].size() == mean[li].size()) { mean[li] = norm_means_averages_[li]; var[li] = norm_variances_averages_[li]; }
         if (desc_.layers[li].type_layer == MYEA_LAYER_LSTM) {
