@@ -289,6 +289,7 @@ def config_of(r):
 
 SECONDARY = "lstm512x2_t64_b256_amsgrad"   # the metric's other half
 OTHERS = ("fc2048x8_bn_relu_dropout_b512_nesterov", "bilstm1024_t512_b64_adabound")
+EXAMPLE = "resindrnn_smnist28_t28_b256_amsgrad"   # the reference's own worked example: a leg of the default line too
 
 
 def timed_blocks(stream_call):
@@ -426,7 +427,7 @@ def main():
                             "contractions": s["contractions"], "kernels": s["kernels"], "loss_per_output": s["loss_per_output"]}
         # the other two configurations of the baseline that are timed on the GPU, a few steps each, so that one run records all four
         out["other_configurations"] = []
-        for name in OTHERS:
+        for name in OTHERS + (EXAMPLE,):
             o = run_workload(name, max(5, args.steps // 3), max(2, args.warmup // 2), args.separate_update)
             leg = {"workload": name, "value": o["value"], "unit": "samples/s", "ms_per_step": o["ms_per_step"], "steps": max(5, args.steps // 3),
                    "config": config_of(o), "contractions": o["contractions_alone"] or o["contractions"], "kernels": o["kernels"], "loss_per_output": o["loss_per_output"]}
@@ -452,6 +453,9 @@ def main():
             rows = int(max(4, min(swl["batch"], 20.0 * threads * 15.0e9 / flop_per_row)))
             rows = max(threads, rows - rows % threads)
             out["secondary"]["cpu_baseline"] = cpu_baseline(swl, min(rows, swl["batch"]), threads)
+            for leg in out.get("other_configurations", []):   # the example network is small enough to walk whole on the host
+                if leg["workload"] == EXAMPLE:
+                    leg["cpu_baseline"] = cpu_baseline(WORKLOADS[EXAMPLE], WORKLOADS[EXAMPLE]["batch"], threads)
     print(json.dumps(out))
 
 
