@@ -1293,8 +1293,7 @@ int launch_bn_forward_sequence(hipStream_t s, const BnForwardParams &p, size_t T
 
 // The backward pass of the same, every time step in one launch: the four column sums of BnBackF in LDS, the last loop of
 // bn_backward_apply_kernel behind them.  The shares of the scale's and the shift's gradient - one per time step, all onto the
-// same two vectors - go to `partial` ([T][2][H]) and are added by bn_backward_sequence_final_kernel in descending time-step
-// order, the order the launches per time step add them in.
+// same two vectors - go to `partial` ([T][2][H]) and are added by bn_backward_sequence_final_kernel in a fixed order.
 template <int CW>
 __global__ __launch_bounds__(kBlock) void bn_backward_sequence_kernel(BnBackwardParams p, size_t Bmax, float *__restrict__ partial)
 {
@@ -1347,13 +1346,26 @@ __global__ __launch_bounds__(kBlock) void bn_backward_sequence_kernel(BnBackward
     }
 }
 
+// grid: ceil(H / 64); four lanes per column (lane q: time steps T-1-q, T-5-q, ...), their sums added in lane order onto the gradient
 __global__ __launch_bounds__(kBlock) void bn_backward_sequence_final_kernel(size_t H, size_t T, const float *__restrict__ partial, float *dscale, float *dshift)
 {
-    const size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (j >= H) return;
-    float a = dscale[j], b = dshift[j];
-    for (size_t t = T; t-- > 0;) { a += partial[(t * 2 + 0) * H + j]; b += partial[(t * 2 + 1) * H + j]; }
-    dscale[j] = a; dshift[j] = b;
+    __shared__ float red[2][kBlock / 64][64];
+    const int cl = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const size_t j = (size_t)blockIdx.x * 64 + cl;
+    float a = 0.f, b = 0.f;
+    if (j < H) {
+#pragma unroll 8
+        for (size_t k = q; k < T; k += kBlock / 64) {
+            const size_t t = T - 1 - k;
+            a += partial[(t * 2 + 0) * H + j]; b += partial[(t * 2 + 1) * H + j];
+        }
+    }
+    red[0][q][cl] = a; red[1][q][cl] = b;
+    __syncthreads();
+    if (q != 0 || j >= H) return;
+#pragma unroll
+    for (int r = 1; r < kBlock / 64; ++r) { a += red[0][r][cl]; b += red[1][r][cl]; }
+    dscale[j] += a; dshift[j] += b;
 }
 
 int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t T, size_t Bmax, float *scratch)
@@ -1368,7 +1380,7 @@ int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t
     MYEA_HIP_TRY(hipGetLastError());
     // (the shares are added by a launch of their own: a column block's last workgroup could add them itself, but the release of its
     // stores to the other XCDs' workgroups costs more than the launch - 38 against 9 + 8 us measured)
-    hipLaunchKernelGGL(bn_backward_sequence_final_kernel, dim3(grid_for(p.H, kBlock)), dim3(kBlock), 0, s, p.H, T, scratch, p.dscale, p.dshift);
+    hipLaunchKernelGGL(bn_backward_sequence_final_kernel, dim3(grid_for(p.H, 64)), dim3(kBlock), 0, s, p.H, T, scratch, p.dscale, p.dshift);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
@@ -1531,6 +1543,7 @@ __global__ __launch_bounds__(kBlock) void slab_sum_add_kernel(size_t n, int nsla
     const size_t n4 = n / 4;
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += (size_t)gridDim.x * kBlock) {
         f32x4 v = reinterpret_cast<const f32x4 *>(slabs)[i];
+#pragma unroll 8
         for (int s = 1; s < nslab; ++s) {
             const f32x4 w = reinterpret_cast<const f32x4 *>(slabs + (size_t)s * n)[i];
             v[0] += w[0]; v[1] += w[1]; v[2] += w[2]; v[3] += w[3];
@@ -1541,21 +1554,32 @@ __global__ __launch_bounds__(kBlock) void slab_sum_add_kernel(size_t n, int nsla
     }
 }
 
-// the same value by value, for slices that are no aligned multiple of four floats
+// the same value by value, for slices that are no aligned multiple of four floats; 64 values a workgroup, four lanes per value
+// (lane q: slabs q, q + 4, ...), their sums added in lane order: few values and many slabs make the launch a chain of loads,
+// shorter the more lanes share a value
 __global__ __launch_bounds__(kBlock) void slab_sum_add_scalar_kernel(size_t n, int nslab, const float *__restrict__ slabs, float *__restrict__ dst)
 {
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-        float v = slabs[i];
-        for (int s = 1; s < nslab; ++s) v += slabs[(size_t)s * n + i];
-        dst[i] += v;
+    __shared__ float red[kBlock / 64][64];
+    const int cl = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const size_t i = (size_t)blockIdx.x * 64 + cl;
+    float v = 0.f;
+    if (i < n) {
+#pragma unroll 8
+        for (int s = q; s < nslab; s += kBlock / 64) v += slabs[(size_t)s * n + i];
     }
+    red[q][cl] = v;
+    __syncthreads();
+    if (q != 0 || i >= n) return;
+#pragma unroll
+    for (int r = 1; r < kBlock / 64; ++r) v += red[r][cl];
+    dst[i] += v;
 }
 
 int launch_slab_sum_add(hipStream_t s, size_t n, int nslab, const float *slabs, float *dst)
 {
     if (n == 0 || nslab <= 0) return MYEA_OK;
     if ((n & 3) || (reinterpret_cast<uintptr_t>(slabs) & 15u) || (reinterpret_cast<uintptr_t>(dst) & 15u))
-        hipLaunchKernelGGL(slab_sum_add_scalar_kernel, dim3(grid_for(n, kBlock, 8192)), dim3(kBlock), 0, s, n, nslab, slabs, dst);
+        hipLaunchKernelGGL(slab_sum_add_scalar_kernel, dim3(grid_for(n, 64)), dim3(kBlock), 0, s, n, nslab, slabs, dst);
     else
         hipLaunchKernelGGL(slab_sum_add_kernel, dim3(grid_for(n / 4, kBlock, 8192)), dim3(kBlock), 0, s, n, nslab, slabs, dst);
     MYEA_HIP_TRY(hipGetLastError());
