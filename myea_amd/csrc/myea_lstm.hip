@@ -17,6 +17,7 @@
 //
 // NN/ = Neural_Network_Library_Windows/Source_Files/Neural_Network/.
 #include <cstdlib>
+#include <type_traits>
 
 #include "myea_device_af.h"
 #include "myea_kernels.h"
@@ -599,202 +600,294 @@ __global__ __launch_bounds__(kBlock) void lstm_norm_backward_gates_kernel(size_t
 // ---- a normalised layer's time step in one launch -----------------------------------------------------------------------
 // Everything a time step does behind its recurrent contraction touches one cell's column of a few tensors over the batch: the
 // statistics are sums over the batch of that column, the gate math combines the normalised sums of the same cell.  A workgroup
-// therefore owns CW cells and ALL examples, with kBlock / CW row lanes: the column sums of every group meet in LDS, one lane
-// per (group, cell) finishes the statistics as lstm_norm_statistics_kernel does, and the lanes go over their rows again to
-// apply them and to run the gates; a lane meets the same (example, cell) pairs in every pass, so what it wrote it may read back.
-struct NormStep { NormBand g[9]; };   // indexed by group: 0 z, 3 i, 5 f, 7 o from below; 1, 4, 6, 8 recurrent; 2 the cell state
-constexpr int kNormThreads = 1024, kNormWaves = kNormThreads / 64;
+// therefore owns CW cells and ALL examples, with lanes / CW row lanes: the column sums of every group meet in LDS, a wavefront
+// per group finishes the statistics as lstm_norm_statistics_kernel does, and the lanes go over their rows again to apply them
+// and to run the gates; a lane meets the same (example, cell) pairs in every pass, so what it wrote it may read back.
+//
+// What bounds such a launch is not traffic but the chain of things that wait for each other, so the kernels keep that chain short:
+//  - the arguments are a few base pointers (two cache lines) and a group's tensors are computed from them; nine bands of
+//    pointers would be fetched piecewise, each piece a trip to memory before the first operand can be asked for;
+//  - a lane asks for its column's parameters and for its FIRST row's operands before anything waits, and keeps what it computed
+//    of that row in registers for the later passes (with B <= lanes / CW no pass but the first reads a tensor);
+//  - every address is a base plus one of two 32-bit offsets (rows of G = 4C floats, rows of C floats): the host keeps B * G
+//    below 2^32;
+//  - a column's sum over the lanes goes through the LDS unit, which all wavefronts share, as little as possible: lanes of a
+//    16-lane row combine with row rotations in the vector unit, one partial per row (or per wavefront) is written, and the
+//    finishing lane adds the partials in a fixed order.
+// Groups: 0 z, 3 i, 5 f, 7 o from below; 1, 4, 6, 8 the recurrent sums of the same gates; 2 the cell state.
+struct NormStepArgs {
+    float *sum[2], *hat[2], *nor[2], *delta[2];   // [0] from below, [1] recurrent, at this time step: rows of 4C floats, z | i | f | o
+    float *c, *hc, *nc, *dc;                      // the cell state's group at this time step: rows of C floats
+    const float *scale, *shift;                   // of group 0; group g's at g * C
+    float *dscale;
+    float *stats;                                 // group 0's statistics at this time step; field f of group g at (8 g + f) * field
+    unsigned cells, field;                        // C; T * C
+    enum Field { kMean = 0, kSigma, kMeanAvg, kSigmaAvg, kR, kD, kDMean, kDSigma };
+    __device__ __forceinline__ static int side(int g) { return (g == 0 || g == 3 || g == 5 || g == 7) ? 0 : 1; }
+    __device__ __forceinline__ unsigned band(int g) const { return (unsigned)((g - 1) / 2) * cells; }   // g >= 3; 0 for groups 0 and 1
+    __device__ __forceinline__ const float *x_of(int g) const { return g == 2 ? c : (g < 2 ? sum[side(g)] : sum[side(g)] + band(g)); }
+    __device__ __forceinline__ float *hat_of(int g) const { return g == 2 ? hc : (g < 2 ? hat[side(g)] : hat[side(g)] + band(g)); }
+    __device__ __forceinline__ float *nor_of(int g) const { return g == 2 ? nc : (g < 2 ? nor[side(g)] : nor[side(g)] + band(g)); }
+    __device__ __forceinline__ float *delta_of(int g) const { return g == 2 ? dc : (g < 2 ? delta[side(g)] : delta[side(g)] + band(g)); }
+    __device__ __forceinline__ float *stat(int g, int f) const { return stats + (size_t)(8 * g + f) * field; }
+};
 constexpr int kNormBackThreads = 512;   // the backward pass keeps more per lane: 256 registers a lane instead of 128
 
-// a wavefront holds 64 / CW rows of the workgroup's CW columns (lane = CW * row + column): those rows' values of a column, summed
-template <int CW>
-__device__ __forceinline__ double norm_fold_rows(double v)
+// lane j of a 16-lane row takes the value of lane j - N (mod 16) of its row
+template <int N>
+__device__ __forceinline__ double norm_row_rotate(double v)
 {
-#pragma unroll
-    for (int m = CW; m < 64; m <<= 1) v += __shfl_xor(v, m);
-    return v;
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_mov_dpp(lo, 0x120 + N, 0xf, 0xf, false);
+    hi = __builtin_amdgcn_mov_dpp(hi, 0x120 + N, 0xf, 0xf, false);
+    return __hiloint2double(hi, lo);
 }
 
-__device__ __forceinline__ void norm_finish_statistics(const NormBand &g, size_t col, double s1, double s2, size_t B, const NormHyper &hy, float *st)
+// A wavefront holds 64 / CW rows of the workgroup's CW columns (lane = CW * row + column).  With CW < 16 the lanes of each
+// 16-lane row that share a column add up in place: four partials a wavefront.  With CW == 16 a 16-lane row is one batch row and
+// the four of them add up across the wavefront: one partial.
+template <int CW> constexpr int kNormPartials = CW < 16 ? 4 : 1;
+template <int CW>
+__device__ __forceinline__ double norm_fold_partial(double v)
+{
+    if (CW <= 1) v += norm_row_rotate<1>(v);
+    if (CW <= 2) v += norm_row_rotate<2>(v);
+    if (CW <= 4) v += norm_row_rotate<4>(v);
+    if (CW <= 8) v += norm_row_rotate<8>(v);
+    if (CW == 16) { v += __shfl_xor(v, 16); v += __shfl_xor(v, 32); }
+    return v;
+}
+// which lanes hold a partial, and where it goes among the workgroup's NW * kNormPartials<CW>
+template <int CW> __device__ __forceinline__ bool norm_partial_holder(int lane) { return CW < 16 ? (lane & 15) < CW : lane < 16; }
+template <int CW> __device__ __forceinline__ int norm_partial_index(int wave, int lane) { return CW < 16 ? wave * 4 + (lane >> 4) : wave; }
+
+// st: the group's statistics at this time step, fields `field` floats apart; mean_avg_old, sigma_avg_old: the running averages as
+// they stood before this step (the caller asked for them early)
+__device__ __forceinline__ void norm_finish_statistics(float *st, unsigned field, unsigned col, double s1, double s2, size_t B, const NormHyper &hy, float mean_avg_old,
+                                                       float sigma_avg_old, float *out)
 {
     const float bscale = 1.f / (float)B;
     const float mean = (float)s1 * bscale;
-    const float mavg = g.mean_avg[col] + hy.momentum * (mean - g.mean_avg[col]);
+    const float mavg = mean_avg_old + hy.momentum * (mean - mean_avg_old);
     const float sigma = sqrtf((float)s2 * bscale - mean * mean + hy.epsilon);
-    const float vavg = g.sigma_avg[col] + hy.momentum * (sigma - g.sigma_avg[col]);
-    g.mean[col] = mean; g.sigma[col] = sigma; g.mean_avg[col] = mavg; g.sigma_avg[col] = vavg;
+    const float vavg = sigma_avg_old + hy.momentum * (sigma - sigma_avg_old);
+    st[NormStepArgs::kMean * field + col] = mean; st[NormStepArgs::kSigma * field + col] = sigma;
+    st[NormStepArgs::kMeanAvg * field + col] = mavg; st[NormStepArgs::kSigmaAvg * field + col] = vavg;
     float r = 1.f, dd = 0.f;
     if (hy.renorm) {
         const float q = sigma / vavg, lo = 1.f / hy.r_max;
         r = q < lo ? lo : (q > hy.r_max ? hy.r_max : q);
         const float e = (mean - mavg) / vavg;
         dd = e < -hy.d_max ? -hy.d_max : (e > hy.d_max ? hy.d_max : e);
-        g.r[col] = r; g.dd[col] = dd;
+        st[NormStepArgs::kR * field + col] = r; st[NormStepArgs::kD * field + col] = dd;
     }
-    st[0] = mean; st[1] = sigma; st[2] = r; st[3] = dd;
+    out[0] = mean; out[1] = sigma; out[2] = r; out[3] = dd;
 }
 
 // Forward_Pass__LSTM of one time step behind the recurrent contraction (NN/Neural_Network__Forward_Pass__OpenMP.cpp:1769-2340):
 // the normalisations of the gate sums, Gates_CIF_AF_State, the cell state's normalisation, States_AF and Output - the kernels
-// lstm_norm_statistics / _apply / _gates / _output above in one launch.  grid: ceil(C / CW) workgroups of 16 wavefronts
-template <bool FIRST, int CW>   // FIRST: the direction's first time step (no recurrent sums, no forget gate); CW: cells per workgroup
-__global__ __launch_bounds__(kNormThreads) void lstm_norm_forward_fused_kernel(NormStep nb, size_t C, size_t B, int training, NormHyper hy, const float *bias,
-                                                                               const float *peep, const float *c_prev, float *acts, float *c, float *ca, float *h,
-                                                                               const float *h_prev, const uint8_t *zone_state, const uint8_t *zone_output)
+// lstm_norm_statistics / _apply / _gates / _output above in one launch.  grid: ceil(C / CW) workgroups of NT lanes.
+template <bool FIRST, int CW, int NT>   // FIRST: the direction's first time step (no recurrent sums, no forget gate); CW: cells per workgroup; NT: lanes
+__global__ __launch_bounds__(NT) void lstm_norm_forward_fused_kernel(NormStepArgs ns, size_t B, int training, NormHyper hy, const float *bias,
+                                                                     const float *peep, const float *c_prev, float *acts, float *c, float *ca, float *h,
+                                                                     const float *h_prev, const uint8_t *zone_state, const uint8_t *zone_output)
 {
-    constexpr int RL = kNormThreads / CW, NW = kNormWaves;
-    __shared__ double red[8][2][NW][CW];
+    constexpr int RL = NT / CW, NW = NT / 64, NP = NW * kNormPartials<CW>;
+    __shared__ double red[8][2][NP][CW];
     __shared__ float st[9][4][CW];
     const int cl = threadIdx.x % CW, rl = threadIdx.x / CW, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const size_t k = (size_t)blockIdx.x * CW + cl, G = 4 * C;
-    const bool live = k < C;
+    const unsigned Cu = ns.cells, Gu = 4 * Cu, Bu = (unsigned)B, k = blockIdx.x * CW + cl;
+    const bool live = k < Cu;
+    const bool row0 = live && (unsigned)rl < Bu;   // the lane has a first row
+    const bool finisher = live && lane < CW;       // lanes 0 .. CW-1 of a wavefront: its group's statistics of column cl
+    const bool holder = norm_partial_holder<CW>(lane);
+    const int slot = norm_partial_index<CW>(wave, lane);
     constexpr bool first = FIRST;
     constexpr int order[8] = {0, 3, FIRST ? 7 : 5, 1, 4, 6, 7, 8};
     constexpr int n = FIRST ? 3 : 8;
+    static_assert(NW >= 8, "a wavefront per group finishes the statistics");
+    static_assert(16 % CW == 0, "a 16-lane row holds whole batch rows");
+    // offset of (row b, this lane's cell) in a tensor with rows of G floats / of C floats
+    auto at_g = [&](unsigned b) { return b * Gu + k; };
+    auto at_c = [&](unsigned b) { return b * Cu + k; };
+    // ---- everything that does not depend on another lane
+    float x0[n], scale[n], shift[n];
+    float pi = 0.f, pf = 0.f, po = 0.f, bz = 0.f, bi = 0.f, bf = 0.f, bo = 0.f, csc = 0.f, csh = 0.f, cp0 = 0.f;
+    float avg_mean = 0.f, avg_sigma = 0.f, avg_mean_c = 0.f, avg_sigma_c = 0.f;   // the running averages a finishing lane updates
+    bool keep_state = false, keep_output = false;   // zoneout holds this cell's state / output at its previous value
+#pragma unroll
+    for (int i = 0; i < n; ++i) { x0[i] = 0.f; scale[i] = 0.f; shift[i] = 0.f; }
+    if (row0) {
+#pragma unroll
+        for (int i = 0; i < n; ++i) x0[i] = ns.x_of(order[i])[at_g(rl)];
+        if (!first) cp0 = c_prev[at_c(rl)];
+    }
+    if (live) {
+        pi = peep[k]; pf = peep[Cu + k]; po = peep[2 * Cu + k];
+        bz = bias[k]; bi = bias[Cu + k]; bf = bias[2 * Cu + k]; bo = bias[3 * Cu + k];
+        csc = ns.scale[2 * Cu + k]; csh = ns.shift[2 * Cu + k];
+#pragma unroll
+        for (int i = 0; i < n; ++i) { scale[i] = ns.scale[order[i] * Cu + k]; shift[i] = ns.shift[order[i] * Cu + k]; }
+        if (zone_state) keep_state = !zone_state[k];
+        if (zone_output) keep_output = !zone_output[k];
+    }
+    if (training && finisher) {
+#pragma unroll
+        for (int i = 0; i < n; ++i)
+            if (wave == i) { avg_mean = ns.stat(order[i], NormStepArgs::kMeanAvg)[k]; avg_sigma = ns.stat(order[i], NormStepArgs::kSigmaAvg)[k]; }
+        if (wave == 0) { avg_mean_c = ns.stat(2, NormStepArgs::kMeanAvg)[k]; avg_sigma_c = ns.stat(2, NormStepArgs::kSigmaAvg)[k]; }
+    }
+    // ---- the statistics of the gate sums
     if (training) {
         double s1[n], s2[n];
 #pragma unroll
         for (int i = 0; i < n; ++i) { s1[i] = 0.0; s2[i] = 0.0; }
+        if (row0) {
+#pragma unroll
+            for (int i = 0; i < n; ++i) { const float v = x0[i]; s1[i] += v; s2[i] += (double)v * v; }
+        }
         if (live)
-            for (size_t b = rl; b < B; b += RL) {
+            for (unsigned b = rl + RL; b < Bu; b += RL) {
 #pragma unroll
                 for (int i = 0; i < n; ++i) {
-                    const NormBand &g = nb.g[order[i]];
-                    const float v = g.x[b * g.ldx + k];
+                    const float v = ns.x_of(order[i])[at_g(b)];
                     s1[i] += v; s2[i] += (double)v * v;
                 }
             }
 #pragma unroll
         for (int i = 0; i < n; ++i) {
-            const double a = norm_fold_rows<CW>(s1[i]), q = norm_fold_rows<CW>(s2[i]);
-            if (lane < CW) { red[i][0][wave][cl] = a; red[i][1][wave][cl] = q; }
+            const double a = norm_fold_partial<CW>(s1[i]), q = norm_fold_partial<CW>(s2[i]);
+            if (holder) { red[i][0][slot][cl] = a; red[i][1][slot][cl] = q; }
         }
         __syncthreads();
-        {   // one lane per (group, cell)
-            const int i = threadIdx.x / CW, col_l = threadIdx.x % CW;
-            const size_t col = (size_t)blockIdx.x * CW + col_l;
-            if (i < n && col < C) {
+#pragma unroll
+        for (int i = 0; i < n; ++i)
+            if (wave == i && finisher) {
                 double a = 0.0, q = 0.0;
 #pragma unroll
-                for (int w = 0; w < NW; ++w) { a += red[i][0][w][col_l]; q += red[i][1][w][col_l]; }
+                for (int w = 0; w < NP; ++w) { a += red[i][0][w][cl]; q += red[i][1][w][cl]; }
                 float out[4];
-                norm_finish_statistics(nb.g[order[i]], col, a, q, B, hy, out);
-                st[order[i]][0][col_l] = out[0]; st[order[i]][1][col_l] = out[1]; st[order[i]][2][col_l] = out[2]; st[order[i]][3][col_l] = out[3];
+                norm_finish_statistics(ns.stat(order[i], 0), ns.field, k, a, q, B, hy, avg_mean, avg_sigma, out);
+                st[order[i]][0][cl] = out[0]; st[order[i]][1][cl] = out[1]; st[order[i]][2][cl] = out[2]; st[order[i]][3][cl] = out[3];
             }
-        }
     } else {
-        const int i = threadIdx.x / CW, col_l = threadIdx.x % CW;
-        const size_t col = (size_t)blockIdx.x * CW + col_l;
-        if (i < 9 && col < C) { st[i][0][col_l] = nb.g[i].mean_avg[col]; st[i][1][col_l] = nb.g[i].sigma_avg[col]; st[i][2][col_l] = 1.f; st[i][3][col_l] = 0.f; }
+#pragma unroll
+        for (int i = 0; i < 9; ++i)
+            if (wave == i % NW && finisher) {
+                st[i][0][cl] = ns.stat(i, NormStepArgs::kMeanAvg)[k]; st[i][1][cl] = ns.stat(i, NormStepArgs::kSigmaAvg)[k];
+                st[i][2][cl] = 1.f; st[i][3][cl] = 0.f;
+            }
     }
     __syncthreads();
-    // the normalised sums of the lane's cell, the gates, the cell state; the cell state's column sums on the way
+    // ---- the normalised sums of the lane's cell, the gates, the cell state; the cell state's column sums on the way
     double c1 = 0.0, c2 = 0.0;
-    if (live) {
-        const float pi = peep[k], pf = peep[C + k];
-        const float bz = bias[k], bi = bias[C + k], bf = bias[2 * C + k];
-        float scale[n], shift[n];
+    float cs0 = 0.f, n7_0 = 0.f, n8_0 = 0.f;   // of the first row, for the last pass
+    auto gates_row = [&](unsigned b, auto cached) {
+        constexpr bool kCached = decltype(cached)::value;
+        const unsigned og = at_g(b), oc = at_c(b);
+        float nor[9];
 #pragma unroll
-        for (int i = 0; i < n; ++i) { scale[i] = nb.g[order[i]].scale[k]; shift[i] = nb.g[order[i]].shift[k]; }
-        for (size_t b = rl; b < B; b += RL) {
-            float nor[9];
-#pragma unroll
-            for (int i = 0; i < n; ++i) {
-                constexpr int dummy = 0; (void)dummy;
-                const int gi = order[i];
-                const NormBand &g = nb.g[gi];
-                float v = g.x[b * g.ldx + k];
-                v = (v - st[gi][0][cl]) / st[gi][1][cl];
-                if (training) {
-                    if (hy.renorm) v = v * st[gi][2][cl] + st[gi][3][cl];
-                    g.hat[b * g.ldo + k] = v;
-                }
-                v = scale[i] * v + shift[i];
-                g.nor[b * g.ldo + k] = v;
-                nor[gi] = v;
+        for (int i = 0; i < n; ++i) {
+            const int gi = order[i];
+            float v = kCached ? x0[i] : ns.x_of(gi)[og];
+            v = (v - st[gi][0][cl]) / st[gi][1][cl];
+            if (training) {
+                if (hy.renorm) v = v * st[gi][2][cl] + st[gi][3][cl];
+                ns.hat_of(gi)[og] = v;
             }
-            float *row = acts + b * G;
-            float gate_i, gate_f = 0.f, sz;
-            const float cp = first ? 0.f : c_prev[b * C + k];
-            if (!first) {
-                float si = nor[3] + nor[4] + bi;
-                float sf = nor[5] + nor[6] + bf;
-                si += cp * pi; sf += cp * pf;
-                gate_i = sigmoid_f(si); gate_f = sigmoid_f(sf);
-                sz = nor[0] + nor[1] + bz;
-            } else {
-                gate_i = sigmoid_f(nor[3] + bi);
-                sz = nor[0] + bz;
-            }
-            const float z = tanh_f(sz);
-            row[k] = z; row[C + k] = gate_i; row[2 * C + k] = gate_f;
-            float cs = first ? z * gate_i : z * gate_i + gate_f * cp;
-            if (zone_state && !zone_state[k]) cs = first ? 0.f : cp;
-            c[b * C + k] = cs;
-            c1 += cs; c2 += (double)cs * cs;
+            v = scale[i] * v + shift[i];
+            ns.nor_of(gi)[og] = v;
+            nor[gi] = v;
         }
-    }
+        float *row = acts + og;
+        float gate_i, gate_f = 0.f, sz;
+        const float cp = first ? 0.f : (kCached ? cp0 : c_prev[oc]);
+        if (!first) {
+            float si = nor[3] + nor[4] + bi;
+            float sf = nor[5] + nor[6] + bf;
+            si += cp * pi; sf += cp * pf;
+            gate_i = sigmoid_f(si); gate_f = sigmoid_f(sf);
+            sz = nor[0] + nor[1] + bz;
+        } else {
+            gate_i = sigmoid_f(nor[3] + bi);
+            sz = nor[0] + bz;
+        }
+        const float z = tanh_f(sz);
+        row[0] = z; row[Cu] = gate_i; row[2 * Cu] = gate_f;
+        float cs = first ? z * gate_i : z * gate_i + gate_f * cp;
+        if (keep_state) cs = first ? 0.f : cp;
+        c[oc] = cs;
+        c1 += cs; c2 += (double)cs * cs;
+        if (kCached) { cs0 = cs; n7_0 = nor[7]; n8_0 = first ? 0.f : nor[8]; }
+    };
+    if (row0) gates_row(rl, std::true_type{});
+    if (live)
+        for (unsigned b = rl + RL; b < Bu; b += RL) gates_row(b, std::false_type{});
     if (training) {
         __syncthreads();   // every lane is through with red
-        const double a = norm_fold_rows<CW>(c1), q = norm_fold_rows<CW>(c2);
-        if (lane < CW) { red[0][0][wave][cl] = a; red[0][1][wave][cl] = q; }
+        const double a = norm_fold_partial<CW>(c1), q = norm_fold_partial<CW>(c2);
+        if (holder) { red[0][0][slot][cl] = a; red[0][1][slot][cl] = q; }
         __syncthreads();
-        if (rl == 0 && live) {
+        if (wave == 0 && finisher) {
             double sa = 0.0, sq = 0.0;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) { sa += red[0][0][w][cl]; sq += red[0][1][w][cl]; }
+            for (int w = 0; w < NP; ++w) { sa += red[0][0][w][cl]; sq += red[0][1][w][cl]; }
             float out[4];
-            norm_finish_statistics(nb.g[2], k, sa, sq, B, hy, out);
+            norm_finish_statistics(ns.stat(2, 0), ns.field, k, sa, sq, B, hy, avg_mean_c, avg_sigma_c, out);
             st[2][0][cl] = out[0]; st[2][1][cl] = out[1]; st[2][2][cl] = out[2]; st[2][3][cl] = out[3];
         }
         __syncthreads();
     }
     if (!live) return;
-    const NormBand &gc = nb.g[2];
-    const NormBand &g7 = nb.g[7], &g8 = nb.g[8];
-    const float po = peep[2 * C + k], bo = bias[3 * C + k], csc = gc.scale[k], csh = gc.shift[k];
-    for (size_t b = rl; b < B; b += RL) {
-        const float cs = c[b * C + k];
+    // ---- the cell state's normalisation, States_AF, the output gate and the cell's output
+    auto output_row = [&](unsigned b, auto cached) {
+        constexpr bool kCached = decltype(cached)::value;
+        const unsigned og = at_g(b), oc = at_c(b);
+        const float cs = kCached ? cs0 : c[oc];
         float v = (cs - st[2][0][cl]) / st[2][1][cl];
         if (training) {
             if (hy.renorm) v = v * st[2][2][cl] + st[2][3][cl];
-            gc.hat[b * gc.ldo + k] = v;
+            ns.hc[oc] = v;
         }
         v = csc * v + csh;
-        gc.nor[b * gc.ldo + k] = v;
+        ns.nc[oc] = v;
         const float a = tanh_f(v);
-        ca[b * C + k] = a;
-        float so = g7.nor[b * g7.ldo + k] + (first ? 0.f : g8.nor[b * g8.ldo + k]) + bo;
+        ca[oc] = a;
+        float so = kCached ? n7_0 + n8_0 + bo : ns.nor_of(7)[og] + (first ? 0.f : ns.nor_of(8)[og]) + bo;
         so += cs * po;
         const float go = sigmoid_f(so);
-        acts[b * G + 3 * C + k] = go;
+        acts[og + 3 * Cu] = go;
         float hv = a * go;
-        if (zone_output && !zone_output[k]) hv = first ? 0.f : h_prev[b * C + k];
-        h[b * C + k] = hv;
-    }
+        if (keep_output) hv = first ? 0.f : h_prev[oc];
+        h[oc] = hv;
+    };
+    if (row0) output_row(rl, std::true_type{});
+    for (unsigned b = rl + RL; b < Bu; b += RL) output_row(b, std::false_type{});
 }
 
 // the three column sums of a normalisation's backward pass for one (example, cell), as lstm_norm_backward_sums_kernel forms them
 struct NormBackColumn {
     float vb, r, sc, mean, k2, k3;
-    __device__ __forceinline__ void load(const NormBand &g, size_t col, int renorm)
+    __device__ __forceinline__ void load(const NormStepArgs &ns, int g, unsigned col, int renorm)
     {
-        vb = g.sigma[col]; r = renorm ? g.r[col] : 1.f; sc = g.scale[col]; mean = g.mean[col];
-        k2 = -r / vb; k3 = -r / (vb * vb);
+        vb = ns.stat(g, NormStepArgs::kSigma)[col]; r = renorm ? ns.stat(g, NormStepArgs::kR)[col] : 1.f;
+        sc = ns.scale[g * ns.cells + col]; mean = ns.stat(g, NormStepArgs::kMean)[col];
     }
-    __device__ __forceinline__ void add(const NormBand &g, size_t b, size_t col, float e, double *a) const
+    __device__ __forceinline__ void derive() { k2 = -r / vb; k3 = -r / (vb * vb); }
+    // hat, x: the normalisation's forward values of this (example, cell); e: its delta
+    __device__ __forceinline__ void add(float hat, float x, float e, double *a) const
     {
-        a[0] += e * g.hat[b * g.ldo + col];
+        a[0] += e * hat;
         e *= sc;
         a[1] += e * k2;
-        a[2] += e * (g.x[b * g.ldx + col] - mean) * k3;
+        a[2] += e * (x - mean) * k3;
     }
     // the last loop of the backward pass (lstm_norm_backward_apply_kernel)
-    __device__ __forceinline__ float apply(const NormBand &g, size_t b, size_t col, float d, float dmean, float dsigma, size_t B) const
+    __device__ __forceinline__ float apply(float x, float d, float dmean, float dsigma, size_t B) const
     {
         float e = d * sc;
         e *= r / vb;
-        e += dsigma * ((g.x[b * g.ldx + col] - mean) / ((float)B * vb));
+        e += dsigma * ((x - mean) / ((float)B * vb));
         e += dmean * (1.f / (float)B);
         return e;
     }
@@ -802,151 +895,226 @@ struct NormBackColumn {
 
 // The backward pass of one time step behind the recurrent contraction (NN/Neural_Network__Recurrent_Backward_Pass__OpenMP.cpp:476-862):
 // lstm_norm_backward_output, the backward normalisations of the output gate's sums and the cell state, lstm_norm_backward_gates and
-// the backward normalisations of the other gate sums in one launch.  grid: ceil(C / CW) workgroups of 8 wavefronts
+// the backward normalisations of the other gate sums in one launch.  grid: ceil(C / CW) workgroups of 8 wavefronts.
 template <bool FIRST, int CW>
-__global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_kernel(NormStep nb, size_t C, size_t B, int last, int renorm, const float *peep,
+__global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_kernel(NormStepArgs ns, size_t B, int last, int renorm, const float *peep,
                                                                                 const float *acts, const float *acts_next, const float *ca, const float *c_prev, float *dh,
                                                                                 const float *part, int nparts, float *dG, const float *dG_next, float *dc,
                                                                                 const float *dc_next, float *din, float *drec)
 {
-    constexpr int RL = kNormBackThreads / CW, NW = kNormBackThreads / 64;
-    __shared__ double red[6][3][NW][CW];
+    constexpr int RL = kNormBackThreads / CW, NW = kNormBackThreads / 64, NP = NW * kNormPartials<CW>;
+    __shared__ double red[6][3][NP][CW];
     __shared__ float fin[6][2][CW];   // dmean, dsigma of the groups in flight
     const int cl = threadIdx.x % CW, rl = threadIdx.x / CW, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const size_t k = (size_t)blockIdx.x * CW + cl, G = 4 * C;
-    const bool live = k < C;
+    const unsigned Cu = ns.cells, Gu = 4 * Cu, Bu = (unsigned)B, k = blockIdx.x * CW + cl;
+    const bool live = k < Cu;
+    const bool row0 = live && (unsigned)rl < Bu;
+    const bool finisher = live && lane < CW;   // lanes 0 .. CW-1 of a wavefront: its group's column sums of column cl
+    const bool holder = norm_partial_holder<CW>(lane);
+    const int slot = norm_partial_index<CW>(wave, lane);
     constexpr bool first = FIRST;
     const int compute = (first && last) ? 0 : 1;
-    // ---- the output gate's delta and the cell state's, their normalisations' sums: groups 7, 2 and, behind the first step, 8
-    constexpr int head[3] = {7, 2, 8};
+    constexpr int head[3] = {7, 2, 8};   // the output gate's sums from below, the cell state, the output gate's recurrent sums
     constexpr int nh = FIRST ? 2 : 3;
-    NormBackColumn col[nh];
+    constexpr int tail[6] = {0, 3, 5, 1, 4, 6};
+    constexpr int nt = FIRST ? 2 : 6;
+    constexpr int tail_gate[6] = {0, 1, 2, 0, 1, 2};   // which gate's delta a group normalises
+    static_assert(NW >= 6, "a wavefront per group finishes the column sums");
+    static_assert(16 % CW == 0, "a 16-lane row holds whole batch rows");
+    // offset of (row b, this lane's cell) in a tensor with rows of G floats / of C floats; the cell state's group (2) has rows
+    // of C floats, every other group rows of G floats
+    auto at_g = [&](unsigned b) { return b * Gu + k; };
+    auto at_c = [&](unsigned b) { return b * Cu + k; };
+    // ---- everything that does not depend on another lane
+    NormBackColumn col[nh], tc[nt];
+    float p_i = 0.f, p_f = 0.f, p_o = 0.f;
+    float dscale_head = 0.f, dscale_tail = 0.f;   // the scale's derivative a finishing lane adds to
+    float dh0 = 0.f, go0 = 0.f, av0 = 0.f, z0 = 0.f, gi0 = 0.f, gf0 = 0.f, cp0 = 0.f, next_i0 = 0.f, next_f0 = 0.f, next_c0 = 0.f, next_gf0 = 0.f;
+    float hat_head[nh], x_head[nh], hat_tail[nt], x_tail[nt], held0[3];
+#pragma unroll
+    for (int i = 0; i < nh; ++i) { hat_head[i] = 0.f; x_head[i] = 0.f; }
+#pragma unroll
+    for (int i = 0; i < nt; ++i) { hat_tail[i] = 0.f; x_tail[i] = 0.f; }
+    held0[0] = held0[1] = held0[2] = 0.f;
+    if (row0) {
+        const unsigned og = at_g(rl), oc = at_c(rl);
+        dh0 = dh[oc]; go0 = acts[og + 3 * Cu]; av0 = ca[oc];
+#pragma unroll
+        for (int i = 0; i < nh; ++i) { const unsigned o = head[i] == 2 ? oc : og; hat_head[i] = ns.hat_of(head[i])[o]; x_head[i] = ns.x_of(head[i])[o]; }
+#pragma unroll
+        for (int i = 0; i < nt; ++i) { hat_tail[i] = ns.hat_of(tail[i])[og]; x_tail[i] = ns.x_of(tail[i])[og]; }
+        if (compute) {
+            z0 = acts[og]; gi0 = acts[og + Cu];
+            if (!first) { gf0 = acts[og + 2 * Cu]; cp0 = c_prev[oc]; }
+            if (!last) { next_i0 = dG_next[og + Cu]; next_f0 = dG_next[og + 2 * Cu]; next_c0 = dc_next[oc]; next_gf0 = acts_next[og + 2 * Cu]; }
+        } else {
+#pragma unroll
+            for (int gate = 0; gate < 3; ++gate) held0[gate] = dG[og + gate * Cu];
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < nh; ++i) col[i].load(ns, head[i], k, renorm);
+#pragma unroll
+        for (int i = 0; i < nt; ++i) tc[i].load(ns, tail[i], k, renorm);
+        p_i = peep[k]; p_f = peep[Cu + k]; p_o = peep[2 * Cu + k];
+    }
+    if (finisher) {
+#pragma unroll
+        for (int i = 0; i < nh; ++i)
+            if (wave == i) dscale_head = ns.dscale[head[i] * Cu + k];
+#pragma unroll
+        for (int i = 0; i < nt; ++i)
+            if (wave == i) dscale_tail = ns.dscale[tail[i] * Cu + k];
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < nh; ++i) col[i].derive();
+#pragma unroll
+        for (int i = 0; i < nt; ++i) tc[i].derive();
+    }
+    // ---- the output gate's delta and the cell state's, their normalisations' sums: groups 7, 2 and, behind the first step, 8
+    float ddo0 = 0.f, dcv0 = 0.f;   // of the first row, for the next pass
     {
         double a[nh][3];
 #pragma unroll
         for (int i = 0; i < nh; ++i) { a[i][0] = a[i][1] = a[i][2] = 0.0; }
-        if (live) {
+        auto output_row = [&](unsigned b, auto cached) {
+            constexpr bool kCached = decltype(cached)::value;
+            const unsigned og = at_g(b), oc = at_c(b);
+            float v = kCached ? dh0 : dh[oc];
+            for (int s = 0; s < nparts; ++s) v += part[((size_t)s * B + b) * Cu + k];
+            if (nparts > 0) dh[oc] = v;
+            const float go = kCached ? go0 : acts[og + 3 * Cu], av = kCached ? av0 : ca[oc];
+            const float ddo = (go * (1.f - go)) * (v * av);
+            dG[og + 3 * Cu] = ddo;
+            din[og + 3 * Cu] = ddo;
+            if (!first) drec[og + 3 * Cu] = ddo;
+            const float dcv = v * go * (1.f - av * av);
+            dc[oc] = dcv;
 #pragma unroll
-            for (int i = 0; i < nh; ++i) col[i].load(nb.g[head[i]], k, renorm);
-            for (size_t b = rl; b < B; b += RL) {
-                float v = dh[b * C + k];
-                for (int s = 0; s < nparts; ++s) v += part[((size_t)s * B + b) * C + k];
-                if (nparts > 0) dh[b * C + k] = v;
-                const float go = acts[b * G + 3 * C + k], av = ca[b * C + k];
-                const float ddo = (go * (1.f - go)) * (v * av);
-                dG[b * G + 3 * C + k] = ddo;
-                din[b * G + 3 * C + k] = ddo;
-                if (!first) drec[b * G + 3 * C + k] = ddo;
-                const float dcv = v * go * (1.f - av * av);
-                dc[b * C + k] = dcv;
-                col[0].add(nb.g[7], b, k, ddo, a[0]);
-                col[1].add(nb.g[2], b, k, dcv, a[1]);
-                if (!first) col[nh - 1].add(nb.g[8], b, k, ddo, a[nh - 1]);
+            for (int i = 0; i < nh; ++i) {
+                const unsigned o = head[i] == 2 ? oc : og;
+                const float hat = kCached ? hat_head[i] : ns.hat_of(head[i])[o], x = kCached ? x_head[i] : ns.x_of(head[i])[o];
+                col[i].add(hat, x, i == 1 ? dcv : ddo, a[i]);
             }
-        }
+            if (kCached) { ddo0 = ddo; dcv0 = dcv; }
+        };
+        if (row0) output_row(rl, std::true_type{});
+        if (live)
+            for (unsigned b = rl + RL; b < Bu; b += RL) output_row(b, std::false_type{});
 #pragma unroll
         for (int i = 0; i < nh; ++i)
 #pragma unroll
             for (int v = 0; v < 3; ++v) {
-                const double f = norm_fold_rows<CW>(a[i][v]);
-                if (lane < CW) red[i][v][wave][cl] = f;
+                const double f = norm_fold_partial<CW>(a[i][v]);
+                if (holder) red[i][v][slot][cl] = f;
             }
     }
     __syncthreads();
-    {
-        const int i = threadIdx.x / CW, col_l = threadIdx.x % CW;
-        const size_t cc = (size_t)blockIdx.x * CW + col_l;
-        if (i < nh && cc < C) {
+#pragma unroll
+    for (int i = 0; i < nh; ++i)
+        if (wave == i && finisher) {
             double q0 = 0.0, q1 = 0.0, q2 = 0.0;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) { q0 += red[i][0][w][col_l]; q1 += red[i][1][w][col_l]; q2 += red[i][2][w][col_l]; }
-            const NormBand &g = nb.g[head[i]];
-            g.dscale[cc] += (float)q0; g.dmean[cc] = (float)q1; g.dsigma[cc] = (float)q2;
-            fin[i][0][col_l] = (float)q1; fin[i][1][col_l] = (float)q2;
+            for (int w = 0; w < NP; ++w) { q0 += red[i][0][w][cl]; q1 += red[i][1][w][cl]; q2 += red[i][2][w][cl]; }
+            ns.dscale[head[i] * Cu + k] = dscale_head + (float)q0;
+            ns.stat(head[i], NormStepArgs::kDMean)[k] = (float)q1; ns.stat(head[i], NormStepArgs::kDSigma)[k] = (float)q2;
+            fin[i][0][cl] = (float)q1; fin[i][1][cl] = (float)q2;
         }
-    }
     __syncthreads();
     // ---- those normalisations' last loop, the gates' deltas, the sums of the other groups: 0, 3 and, behind the first step, 5, 1, 4, 6
-    constexpr int tail[6] = {0, 3, 5, 1, 4, 6};
-    constexpr int nt = FIRST ? 2 : 6;
-    constexpr int tail_gate[6] = {0, 1, 2, 0, 1, 2};   // which gate's delta a group normalises
-    NormBackColumn tc[nt];
     float dmean_head[nh], dsigma_head[nh];
 #pragma unroll
     for (int i = 0; i < nh; ++i) { dmean_head[i] = fin[i][0][cl]; dsigma_head[i] = fin[i][1][cl]; }
+    float gd0[3] = {0.f, 0.f, 0.f};   // the first row's gate deltas, for the last pass
     {
         double a[nt][3];
 #pragma unroll
         for (int i = 0; i < nt; ++i) { a[i][0] = a[i][1] = a[i][2] = 0.0; }
-        if (live) {
-#pragma unroll
-            for (int i = 0; i < nt; ++i) tc[i].load(nb.g[tail[i]], k, renorm);
-            const float p_i = peep[k], p_f = peep[C + k], p_o = peep[2 * C + k];
-            for (size_t b = rl; b < B; b += RL) {
-                const float ddo = dG[b * G + 3 * C + k];
-                din[b * G + 3 * C + k] = col[0].apply(nb.g[7], b, k, ddo, dmean_head[0], dsigma_head[0], B);
-                if (!first) drec[b * G + 3 * C + k] = col[nh - 1].apply(nb.g[8], b, k, ddo, dmean_head[nh - 1], dsigma_head[nh - 1], B);
-                float e = col[1].apply(nb.g[2], b, k, dc[b * C + k], dmean_head[1], dsigma_head[1], B);
-                float *drow = dG + b * G;
-                if (compute) {
-                    const float *row = acts + b * G;
-                    const float z = row[k], gi = row[C + k];
-                    e += p_o * ddo;
-                    if (!last) {
-                        e += p_i * dG_next[b * G + C + k];
-                        e += p_f * dG_next[b * G + 2 * C + k];
-                        e += dc_next[b * C + k] * acts_next[b * G + 2 * C + k];
-                    }
-                    dc[b * C + k] = e;
-                    drow[k] = e * gi * (1.f - z * z);
-                    drow[C + k] = (e * z) * (gi * (1.f - gi));
-                    if (!first) { const float gf = row[2 * C + k]; drow[2 * C + k] = (e * c_prev[b * C + k]) * (gf * (1.f - gf)); }
+        auto gates_row = [&](unsigned b, auto cached) {
+            constexpr bool kCached = decltype(cached)::value;
+            const unsigned og = at_g(b), oc = at_c(b);
+            const float ddo = kCached ? ddo0 : dG[og + 3 * Cu];
+            din[og + 3 * Cu] = col[0].apply(kCached ? x_head[0] : ns.x_of(7)[og], ddo, dmean_head[0], dsigma_head[0], B);
+            if (!first) drec[og + 3 * Cu] = col[nh - 1].apply(kCached ? x_head[nh - 1] : ns.x_of(8)[og], ddo, dmean_head[nh - 1], dsigma_head[nh - 1], B);
+            float e = col[1].apply(kCached ? x_head[1] : ns.c[oc], kCached ? dcv0 : dc[oc], dmean_head[1], dsigma_head[1], B);
+            float *drow = dG + og;
+            float gd[3];
+            if (compute) {
+                const float *row = acts + og;
+                const float z = kCached ? z0 : row[0], gi = kCached ? gi0 : row[Cu];
+                e += p_o * ddo;
+                if (!last) {
+                    e += p_i * (kCached ? next_i0 : dG_next[og + Cu]);
+                    e += p_f * (kCached ? next_f0 : dG_next[og + 2 * Cu]);
+                    e += (kCached ? next_c0 : dc_next[oc]) * (kCached ? next_gf0 : acts_next[og + 2 * Cu]);
+                }
+                dc[oc] = e;
+                gd[0] = e * gi * (1.f - z * z);
+                gd[1] = (e * z) * (gi * (1.f - gi));
+                drow[0] = gd[0]; drow[Cu] = gd[1];
+                if (!first) {
+                    const float gf = kCached ? gf0 : row[2 * Cu];
+                    gd[2] = (e * (kCached ? cp0 : c_prev[oc])) * (gf * (1.f - gf));
+                    drow[2 * Cu] = gd[2];
                 } else {
-                    dc[b * C + k] = e;
+                    gd[2] = drow[2 * Cu];   // the first step has no forget gate: its delta keeps its value
                 }
-                float gd[3];
+            } else {
+                dc[oc] = e;
 #pragma unroll
-                for (int gate = 0; gate < 3; ++gate) {
-                    gd[gate] = drow[gate * C + k];
-                    din[b * G + gate * C + k] = gd[gate];
-                    if (!first) drec[b * G + gate * C + k] = gd[gate];
-                }
-#pragma unroll
-                for (int i = 0; i < nt; ++i) tc[i].add(nb.g[tail[i]], b, k, gd[tail_gate[i]], a[i]);
+                for (int gate = 0; gate < 3; ++gate) gd[gate] = kCached ? held0[gate] : drow[gate * Cu];
             }
-        }
+#pragma unroll
+            for (int gate = 0; gate < 3; ++gate) {
+                din[og + gate * Cu] = gd[gate];
+                if (!first) drec[og + gate * Cu] = gd[gate];
+            }
+#pragma unroll
+            for (int i = 0; i < nt; ++i) {
+                const float hat = kCached ? hat_tail[i] : ns.hat_of(tail[i])[og], x = kCached ? x_tail[i] : ns.x_of(tail[i])[og];
+                tc[i].add(hat, x, gd[tail_gate[i]], a[i]);
+            }
+            if (kCached) { gd0[0] = gd[0]; gd0[1] = gd[1]; gd0[2] = gd[2]; }
+        };
+        if (row0) gates_row(rl, std::true_type{});
+        if (live)
+            for (unsigned b = rl + RL; b < Bu; b += RL) gates_row(b, std::false_type{});
         __syncthreads();   // fin and red are free again
 #pragma unroll
         for (int i = 0; i < nt; ++i)
 #pragma unroll
             for (int v = 0; v < 3; ++v) {
-                const double f = norm_fold_rows<CW>(a[i][v]);
-                if (lane < CW) red[i][v][wave][cl] = f;
+                const double f = norm_fold_partial<CW>(a[i][v]);
+                if (holder) red[i][v][slot][cl] = f;
             }
     }
     __syncthreads();
-    {
-        const int i = threadIdx.x / CW, col_l = threadIdx.x % CW;
-        const size_t cc = (size_t)blockIdx.x * CW + col_l;
-        if (i < nt && cc < C) {
+#pragma unroll
+    for (int i = 0; i < nt; ++i)
+        if (wave == i && finisher) {
             double q0 = 0.0, q1 = 0.0, q2 = 0.0;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) { q0 += red[i][0][w][col_l]; q1 += red[i][1][w][col_l]; q2 += red[i][2][w][col_l]; }
-            const NormBand &g = nb.g[tail[i]];
-            g.dscale[cc] += (float)q0; g.dmean[cc] = (float)q1; g.dsigma[cc] = (float)q2;
-            fin[i][0][col_l] = (float)q1; fin[i][1][col_l] = (float)q2;
+            for (int w = 0; w < NP; ++w) { q0 += red[i][0][w][cl]; q1 += red[i][1][w][cl]; q2 += red[i][2][w][cl]; }
+            ns.dscale[tail[i] * Cu + k] = dscale_tail + (float)q0;
+            ns.stat(tail[i], NormStepArgs::kDMean)[k] = (float)q1; ns.stat(tail[i], NormStepArgs::kDSigma)[k] = (float)q2;
+            fin[i][0][cl] = (float)q1; fin[i][1][cl] = (float)q2;
         }
-    }
     __syncthreads();
     if (!live) return;
-    for (size_t b = rl; b < B; b += RL) {
+    // ---- the last loop of the other groups' normalisations, on the deltas this lane left in din and drec
+    auto apply_row = [&](unsigned b, auto cached) {
+        constexpr bool kCached = decltype(cached)::value;
+        const unsigned og = at_g(b);
 #pragma unroll
         for (int i = 0; i < nt; ++i) {
-            const NormBand &g = nb.g[tail[i]];
-            float *d = g.d + b * g.ldd + k;
-            *d = tc[i].apply(g, b, k, *d, fin[i][0][cl], fin[i][1][cl], B);
+            float *d = ns.delta_of(tail[i]) + og;
+            *d = tc[i].apply(kCached ? x_tail[i] : ns.x_of(tail[i])[og], kCached ? gd0[tail_gate[i]] : *d, fin[i][0][cl], fin[i][1][cl], B);
         }
-    }
+    };
+    if (row0) apply_row(rl, std::true_type{});
+    for (unsigned b = rl + RL; b < Bu; b += RL) apply_row(b, std::false_type{});
 }
 
 int dev_alloc_zero(float **p, size_t count)
@@ -972,10 +1140,12 @@ bool fused_lstm_disabled()
 
 // MYEA_LSTM_NORM_FUSED=0 keeps a normalised layer's time step as the sequence of statistics / apply / gate launches (read at
 // every call: a test runs both forms in one process)
-bool lstm_norm_fused_allowed()
+// The one-launch kernels address with 32-bit offsets into a time step's tensors and into a statistics field over all time
+// steps: rows * (4 * cells) and steps * cells have to stay below 2^32.
+bool lstm_norm_fused_allowed(size_t rows, size_t cells, size_t steps)
 {
     const char *e = std::getenv("MYEA_LSTM_NORM_FUSED");
-    return !(e && e[0] == '0');
+    return !(e && e[0] == '0') && rows * 4 * cells < ((size_t)1 << 32) && steps * cells < ((size_t)1 << 32);
 }
 
 // MYEA_SIDE_STREAM=0 keeps every launch on the caller's stream (for A/B timing)
@@ -1059,8 +1229,9 @@ int Net::lstm_create_layer(size_t li)
             if (l.first_normalized_unit_index + dirs * (3 * q->C + 6 * q->K) > d.total_normalized_units) { set_last_error("layer %zu: scale/shift slice leaves its region", li); return MYEA_E_INVALID; }
             for (float **p : {&q->sin, &q->srec, &q->nin, &q->nrec, &q->hin, &q->hrec, &q->din, &q->drec}) MYEA_TRY(dev_alloc_zero(p, T * B * q->G));
             for (float **p : {&q->nc, &q->hc}) MYEA_TRY(dev_alloc_zero(p, T * B * q->C));
+            MYEA_TRY(dev_alloc_zero(&q->stats[0], 9 * 8 * T * q->C));   // one block: the one-launch kernels reach every group from the first
             for (int g = 0; g < 9; ++g) {
-                MYEA_TRY(dev_alloc_zero(&q->stats[g], 8 * T * q->C));
+                q->stats[g] = q->stats[0] + (size_t)g * 8 * T * q->C;
                 MYEA_TRY(launch_fill(0, q->stats[g] + 3 * T * q->C, T * q->C, 1.f));   // running sigma starts at 1, NN/Neural_Network__Allocate.cpp:2612-2615
             }
             MYEA_HIP_TRY(hipDeviceSynchronize());
@@ -1080,7 +1251,7 @@ void Net::lstm_destroy_layer(DevLayer &o)
         float *all[] = {q->Win, q->Wrec, q->WrecT, q->peep, q->gWin_own, q->gWrec_own, q->acts, q->c, q->ca, q->dG, q->dc, q->part, q->sums, q->pair_partials, q->pair_tickets, q->own_h ? q->h : nullptr, q->own_h ? q->dh : nullptr,
                         q->sin, q->srec, q->nin, q->nrec, q->hin, q->hrec, q->din, q->drec, q->nc, q->hc};
         for (float *p : all) if (p) (void)hipFree(p);
-        for (float *p : q->stats) if (p) (void)hipFree(p);
+        if (q->stats[0]) (void)hipFree(q->stats[0]);   // the nine groups share one block
         delete q;
         *slot = nullptr;
     }
@@ -1220,6 +1391,20 @@ static NormBand norm_band(const LstmLayer &q, float *parameters, float *gradient
     return b;
 }
 
+// the tensors of a normalised layer at time step t, for the one-launch kernels
+static NormStepArgs norm_step_args(const LstmLayer &q, float *parameters, float *gradient, size_t total_norm, size_t t, size_t T, size_t Bmax)
+{
+    NormStepArgs a{};
+    const size_t rg = t * Bmax * q.G, rc = t * Bmax * q.C;
+    a.sum[0] = q.sin + rg; a.sum[1] = q.srec + rg; a.hat[0] = q.hin + rg; a.hat[1] = q.hrec + rg;
+    a.nor[0] = q.nin + rg; a.nor[1] = q.nrec + rg; a.delta[0] = q.din + rg; a.delta[1] = q.drec + rg;
+    a.c = q.c + rc; a.hc = q.hc + rc; a.nc = q.nc + rc; a.dc = q.dc + rc;
+    a.scale = parameters + q.norm_param; a.shift = a.scale + total_norm; a.dscale = gradient + q.norm_param;
+    a.stats = q.stats[0] + t * q.C;   // the groups' statistics are one block, 8 fields of [T][C] a group
+    a.cells = (unsigned)q.C; a.field = (unsigned)(T * q.C);
+    return a;
+}
+
 int Net::lstm_norm_forward_groups(LstmLayer &q, size_t B, size_t t, std::initializer_list<int> groups)
 {
     NormBands bands{};
@@ -1272,9 +1457,8 @@ int Net::lstm_forward_step_norm(LstmLayer &q, size_t B, size_t s)
         g.M = (int)B; g.N = (int)G; g.K = (int)C;
         MYEA_TRY(launch_gemm(stream, g));
     }
-    if (lstm_norm_fused_allowed()) {   // everything behind the contraction in one launch
-        NormStep nb;
-        for (int gi = 0; gi < 9; ++gi) nb.g[gi] = norm_band(q, parameters, gradient, d.total_normalized_units, gi, t, T, Bmax);
+    if (lstm_norm_fused_allowed(B, C, T)) {   // everything behind the contraction in one launch
+        const NormStepArgs ns = norm_step_args(q, parameters, gradient, d.total_normalized_units, t, T, Bmax);
         const bool training = state >= MYEA_STATE_TRAINING;
         const NormHyper hy{h.normalization_epsilon, h.normalization_momentum_average, h.batch_renormalization_r_correction_maximum,
                            h.batch_renormalization_d_correction_maximum, q.renorm ? 1 : 0};
@@ -1282,12 +1466,20 @@ int Net::lstm_forward_step_norm(LstmLayer &q, size_t B, size_t s)
         const float *c_prev = first ? nullptr : q.c + tp * Bmax * C, *h_prev = first ? nullptr : q.h + tp * Bmax * C;
         const int tr = training ? 1 : 0;
         prof_begin(kProfNormalization);
-        // few cells a workgroup when the layer is narrow: the launch is a chain of memory round trips, shorter the more lanes share a column
-        auto launch = [&](auto kernel, int cw) {
-            hipLaunchKernelGGL(kernel, dim3((unsigned)((C + cw - 1) / cw)), dim3(kNormThreads), 0, stream, nb, C, B, tr, hy, bias, (const float *)q.peep, c_prev, acts, c, ca, hh, h_prev, zs, zo);
+        // few cells a workgroup when the layer is narrow (more workgroups), and no more lanes than the batch has rows for them:
+        // a lane without a row still takes part in every fold
+        auto launch = [&](auto kernel, int cw, int lanes) {
+            hipLaunchKernelGGL(kernel, dim3((unsigned)((C + cw - 1) / cw)), dim3(lanes), 0, stream, ns, B, tr, hy, bias, (const float *)q.peep, c_prev, acts, c, ca, hh, h_prev, zs, zo);
         };
-        if (C >= 1024) { if (first) launch(lstm_norm_forward_fused_kernel<true, 16>, 16); else launch(lstm_norm_forward_fused_kernel<false, 16>, 16); }
-        else { if (first) launch(lstm_norm_forward_fused_kernel<true, 4>, 4); else launch(lstm_norm_forward_fused_kernel<false, 4>, 4); }
+        auto pick = [&](auto first_step) {
+            constexpr bool kFirst = decltype(first_step)::value;
+            if (C >= 1024) {
+                if (B * 16 <= 512) launch(lstm_norm_forward_fused_kernel<kFirst, 16, 512>, 16, 512); else launch(lstm_norm_forward_fused_kernel<kFirst, 16, 1024>, 16, 1024);
+            } else {
+                if (B * 4 <= 512) launch(lstm_norm_forward_fused_kernel<kFirst, 4, 512>, 4, 512); else launch(lstm_norm_forward_fused_kernel<kFirst, 4, 1024>, 4, 1024);
+            }
+        };
+        if (first) pick(std::true_type{}); else pick(std::false_type{});
         MYEA_HIP_TRY(hipGetLastError());
         prof_end((double)(first ? 4 : 9) * (double)B * (double)C * sizeof(float) * 3.0);
         return MYEA_OK;
@@ -1326,14 +1518,13 @@ int Net::lstm_backward_step_norm(LstmLayer &q, size_t B, size_t s)
         g.split_k = nparts; g.split_k_slab = (long)(B * C);
         MYEA_TRY(launch_gemm(stream, g));
     }
-    if (lstm_norm_fused_allowed()) {
-        NormStep nb;
-        for (int gi = 0; gi < 9; ++gi) nb.g[gi] = norm_band(q, parameters, gradient, d.total_normalized_units, gi, t, T, Bmax);
+    if (lstm_norm_fused_allowed(B, C, T)) {
+        const NormStepArgs ns = norm_step_args(q, parameters, gradient, d.total_normalized_units, t, T, Bmax);
         const float *acts_next = last ? nullptr : q.acts + tn * Bmax * G, *c_prev = first ? nullptr : q.c + tp * Bmax * C;
         const float *dG_next = last ? nullptr : q.dG + tn * Bmax * G, *dc_next = last ? nullptr : q.dc + tn * Bmax * C;
         prof_begin(kProfNormalization);
         auto launch = [&](auto kernel, int cw) {
-            hipLaunchKernelGGL(kernel, dim3((unsigned)((C + cw - 1) / cw)), dim3(kNormBackThreads), 0, stream, nb, C, B, last ? 1 : 0, q.renorm ? 1 : 0, (const float *)q.peep,
+            hipLaunchKernelGGL(kernel, dim3((unsigned)((C + cw - 1) / cw)), dim3(kNormBackThreads), 0, stream, ns, B, last ? 1 : 0, q.renorm ? 1 : 0, (const float *)q.peep,
                                (const float *)(q.acts + t * Bmax * G), acts_next, (const float *)(q.ca + t * Bmax * C), c_prev, q.dh + t * Bmax * C, (const float *)q.part, nparts,
                                q.dG + t * Bmax * G, dG_next, q.dc + t * Bmax * C, dc_next, q.din + t * Bmax * G, q.drec + t * Bmax * G);
         };
