@@ -633,15 +633,20 @@ struct NormStepArgs {
 };
 constexpr int kNormBackThreads = 512;   // the backward pass keeps more per lane: 256 registers a lane instead of 128
 
-// lane j of a 16-lane row takes the value of lane j - N (mod 16) of its row
-template <int N>
-__device__ __forceinline__ double norm_row_rotate(double v)
+// the value of another lane of the 16-lane row, chosen by a data-parallel-primitive control word: a move inside the vector unit
+template <int CTRL>
+__device__ __forceinline__ double norm_dpp(double v)
 {
     int lo = __double2loint(v), hi = __double2hiint(v);
-    lo = __builtin_amdgcn_mov_dpp(lo, 0x120 + N, 0xf, 0xf, false);
-    hi = __builtin_amdgcn_mov_dpp(hi, 0x120 + N, 0xf, 0xf, false);
+    lo = __builtin_amdgcn_mov_dpp(lo, CTRL, 0xf, 0xf, false);
+    hi = __builtin_amdgcn_mov_dpp(hi, CTRL, 0xf, 0xf, false);
     return __hiloint2double(hi, lo);
 }
+// lane j of a 16-lane row takes the value of lane j - N (mod 16) of its row
+template <int N> __device__ __forceinline__ double norm_row_rotate(double v) { return norm_dpp<0x120 + N>(v); }
+// lane j takes the value of lane j ^ 1 resp. j ^ 2
+__device__ __forceinline__ double norm_quad_xor1(double v) { return norm_dpp<0xB1>(v); }
+__device__ __forceinline__ double norm_quad_xor2(double v) { return norm_dpp<0x4E>(v); }
 
 // A wavefront holds 64 / CW rows of the workgroup's CW columns (lane = CW * row + column).  With CW < 16 the lanes of each
 // 16-lane row that share a column add up in place: four partials a wavefront.  With CW == 16 a 16-lane row is one batch row and
@@ -660,6 +665,24 @@ __device__ __forceinline__ double norm_fold_partial(double v)
 // which lanes hold a partial, and where it goes among the workgroup's NW * kNormPartials<CW>
 template <int CW> __device__ __forceinline__ bool norm_partial_holder(int lane) { return CW < 16 ? (lane & 15) < CW : lane < 16; }
 template <int CW> __device__ __forceinline__ int norm_partial_index(int wave, int lane) { return CW < 16 ? wave * 4 + (lane >> 4) : wave; }
+
+// The finishing wavefront adds up a column's NP partials with 64 / CW lanes a column (lane = column * lanes + j takes the
+// partials j, j + lanes, ...; the lanes of a column then add up inside their 16-lane row): every lane returns its column's total.
+template <int CW, int NP>
+__device__ __forceinline__ double norm_sum_partials(const double (&p)[NP][CW], int lane)
+{
+    constexpr int LPC = 64 / CW;
+    static_assert(LPC == 4 || LPC == 16, "a column's lanes are a quad or a 16-lane row");
+    static_assert(NP % LPC == 0, "every lane of a column takes the same number of partials");
+    const int column = lane / LPC, j = lane % LPC;
+    double v = 0.0;
+#pragma unroll
+    for (int w = 0; w < NP / LPC; ++w) v += p[w * LPC + j][column];
+    v += norm_quad_xor1(v);
+    v += norm_quad_xor2(v);
+    if (LPC == 16) { v += norm_row_rotate<4>(v); v += norm_row_rotate<8>(v); }
+    return v;
+}
 
 // st: the group's statistics at this time step, fields `field` floats apart; mean_avg_old, sigma_avg_old: the running averages as
 // they stood before this step (the caller asked for them early)
@@ -699,7 +722,10 @@ __global__ __launch_bounds__(NT) void lstm_norm_forward_fused_kernel(NormStepArg
     const unsigned Cu = ns.cells, Gu = 4 * Cu, Bu = (unsigned)B, k = blockIdx.x * CW + cl;
     const bool live = k < Cu;
     const bool row0 = live && (unsigned)rl < Bu;   // the lane has a first row
-    const bool finisher = live && lane < CW;       // lanes 0 .. CW-1 of a wavefront: its group's statistics of column cl
+    // a wavefront finishes its group's statistics with 64 / CW lanes a column; the first of them keeps the result: column fc
+    const int fc = lane / (64 / CW);
+    const unsigned fk = blockIdx.x * CW + fc;
+    const bool finisher = lane % (64 / CW) == 0 && fk < Cu;
     const bool holder = norm_partial_holder<CW>(lane);
     const int slot = norm_partial_index<CW>(wave, lane);
     constexpr bool first = FIRST;
@@ -734,8 +760,8 @@ __global__ __launch_bounds__(NT) void lstm_norm_forward_fused_kernel(NormStepArg
     if (training && finisher) {
 #pragma unroll
         for (int i = 0; i < n; ++i)
-            if (wave == i) { avg_mean = ns.stat(order[i], NormStepArgs::kMeanAvg)[k]; avg_sigma = ns.stat(order[i], NormStepArgs::kSigmaAvg)[k]; }
-        if (wave == 0) { avg_mean_c = ns.stat(2, NormStepArgs::kMeanAvg)[k]; avg_sigma_c = ns.stat(2, NormStepArgs::kSigmaAvg)[k]; }
+            if (wave == i) { avg_mean = ns.stat(order[i], NormStepArgs::kMeanAvg)[fk]; avg_sigma = ns.stat(order[i], NormStepArgs::kSigmaAvg)[fk]; }
+        if (wave == 0) { avg_mean_c = ns.stat(2, NormStepArgs::kMeanAvg)[fk]; avg_sigma_c = ns.stat(2, NormStepArgs::kSigmaAvg)[fk]; }
     }
     // ---- the statistics of the gate sums
     if (training) {
@@ -762,20 +788,20 @@ __global__ __launch_bounds__(NT) void lstm_norm_forward_fused_kernel(NormStepArg
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < n; ++i)
-            if (wave == i && finisher) {
-                double a = 0.0, q = 0.0;
-#pragma unroll
-                for (int w = 0; w < NP; ++w) { a += red[i][0][w][cl]; q += red[i][1][w][cl]; }
-                float out[4];
-                norm_finish_statistics(ns.stat(order[i], 0), ns.field, k, a, q, B, hy, avg_mean, avg_sigma, out);
-                st[order[i]][0][cl] = out[0]; st[order[i]][1][cl] = out[1]; st[order[i]][2][cl] = out[2]; st[order[i]][3][cl] = out[3];
+            if (wave == i) {
+                const double a = norm_sum_partials<CW, NP>(red[i][0], lane), q = norm_sum_partials<CW, NP>(red[i][1], lane);
+                if (finisher) {
+                    float out[4];
+                    norm_finish_statistics(ns.stat(order[i], 0), ns.field, fk, a, q, B, hy, avg_mean, avg_sigma, out);
+                    st[order[i]][0][fc] = out[0]; st[order[i]][1][fc] = out[1]; st[order[i]][2][fc] = out[2]; st[order[i]][3][fc] = out[3];
+                }
             }
     } else {
 #pragma unroll
         for (int i = 0; i < 9; ++i)
             if (wave == i % NW && finisher) {
-                st[i][0][cl] = ns.stat(i, NormStepArgs::kMeanAvg)[k]; st[i][1][cl] = ns.stat(i, NormStepArgs::kSigmaAvg)[k];
-                st[i][2][cl] = 1.f; st[i][3][cl] = 0.f;
+                st[i][0][fc] = ns.stat(i, NormStepArgs::kMeanAvg)[fk]; st[i][1][fc] = ns.stat(i, NormStepArgs::kSigmaAvg)[fk];
+                st[i][2][fc] = 1.f; st[i][3][fc] = 0.f;
             }
     }
     __syncthreads();
@@ -828,13 +854,13 @@ __global__ __launch_bounds__(NT) void lstm_norm_forward_fused_kernel(NormStepArg
         const double a = norm_fold_partial<CW>(c1), q = norm_fold_partial<CW>(c2);
         if (holder) { red[0][0][slot][cl] = a; red[0][1][slot][cl] = q; }
         __syncthreads();
-        if (wave == 0 && finisher) {
-            double sa = 0.0, sq = 0.0;
-#pragma unroll
-            for (int w = 0; w < NP; ++w) { sa += red[0][0][w][cl]; sq += red[0][1][w][cl]; }
-            float out[4];
-            norm_finish_statistics(ns.stat(2, 0), ns.field, k, sa, sq, B, hy, avg_mean_c, avg_sigma_c, out);
-            st[2][0][cl] = out[0]; st[2][1][cl] = out[1]; st[2][2][cl] = out[2]; st[2][3][cl] = out[3];
+        if (wave == 0) {
+            const double sa = norm_sum_partials<CW, NP>(red[0][0], lane), sq = norm_sum_partials<CW, NP>(red[0][1], lane);
+            if (finisher) {
+                float out[4];
+                norm_finish_statistics(ns.stat(2, 0), ns.field, fk, sa, sq, B, hy, avg_mean_c, avg_sigma_c, out);
+                st[2][0][fc] = out[0]; st[2][1][fc] = out[1]; st[2][2][fc] = out[2]; st[2][3][fc] = out[3];
+            }
         }
         __syncthreads();
     }
@@ -909,7 +935,10 @@ __global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_ker
     const unsigned Cu = ns.cells, Gu = 4 * Cu, Bu = (unsigned)B, k = blockIdx.x * CW + cl;
     const bool live = k < Cu;
     const bool row0 = live && (unsigned)rl < Bu;
-    const bool finisher = live && lane < CW;   // lanes 0 .. CW-1 of a wavefront: its group's column sums of column cl
+    // a wavefront finishes its group's column sums with 64 / CW lanes a column; the first of them keeps the result: column fc
+    const int fc = lane / (64 / CW);
+    const unsigned fk = blockIdx.x * CW + fc;
+    const bool finisher = lane % (64 / CW) == 0 && fk < Cu;
     const bool holder = norm_partial_holder<CW>(lane);
     const int slot = norm_partial_index<CW>(wave, lane);
     constexpr bool first = FIRST;
@@ -931,6 +960,15 @@ __global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_ker
     float dscale_head = 0.f, dscale_tail = 0.f;   // the scale's derivative a finishing lane adds to
     float dh0 = 0.f, go0 = 0.f, av0 = 0.f, z0 = 0.f, gi0 = 0.f, gf0 = 0.f, cp0 = 0.f, next_i0 = 0.f, next_f0 = 0.f, next_c0 = 0.f, next_gf0 = 0.f;
     float hat_head[nh], x_head[nh], hat_tail[nt], x_tail[nt], held0[3];
+    constexpr int kSlabs = 16;   // at most this many partial products of the recurrent contraction (gemm_split_k's limit)
+    float slab0[kSlabs];
+    // the slabs of row b, asked for together: a loop that adds them one by one waits for memory once a slab
+    auto load_slabs = [&](unsigned b, float *v) {
+#pragma unroll
+        for (int s = 0; s < kSlabs; ++s) v[s] = s < nparts ? part[((size_t)s * B + b) * Cu + k] : 0.f;
+    };
+#pragma unroll
+    for (int s = 0; s < kSlabs; ++s) slab0[s] = 0.f;
 #pragma unroll
     for (int i = 0; i < nh; ++i) { hat_head[i] = 0.f; x_head[i] = 0.f; }
 #pragma unroll
@@ -939,6 +977,7 @@ __global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_ker
     if (row0) {
         const unsigned og = at_g(rl), oc = at_c(rl);
         dh0 = dh[oc]; go0 = acts[og + 3 * Cu]; av0 = ca[oc];
+        load_slabs(rl, slab0);
 #pragma unroll
         for (int i = 0; i < nh; ++i) { const unsigned o = head[i] == 2 ? oc : og; hat_head[i] = ns.hat_of(head[i])[o]; x_head[i] = ns.x_of(head[i])[o]; }
 #pragma unroll
@@ -962,10 +1001,10 @@ __global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_ker
     if (finisher) {
 #pragma unroll
         for (int i = 0; i < nh; ++i)
-            if (wave == i) dscale_head = ns.dscale[head[i] * Cu + k];
+            if (wave == i) dscale_head = ns.dscale[head[i] * Cu + fk];
 #pragma unroll
         for (int i = 0; i < nt; ++i)
-            if (wave == i) dscale_tail = ns.dscale[tail[i] * Cu + k];
+            if (wave == i) dscale_tail = ns.dscale[tail[i] * Cu + fk];
     }
     if (live) {
 #pragma unroll
@@ -983,7 +1022,15 @@ __global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_ker
             constexpr bool kCached = decltype(cached)::value;
             const unsigned og = at_g(b), oc = at_c(b);
             float v = kCached ? dh0 : dh[oc];
-            for (int s = 0; s < nparts; ++s) v += part[((size_t)s * B + b) * Cu + k];
+            if (kCached) {
+#pragma unroll
+                for (int s = 0; s < kSlabs; ++s) if (s < nparts) v += slab0[s];
+            } else {
+                float slab[kSlabs];
+                load_slabs(b, slab);
+#pragma unroll
+                for (int s = 0; s < kSlabs; ++s) if (s < nparts) v += slab[s];
+            }
             if (nparts > 0) dh[oc] = v;
             const float go = kCached ? go0 : acts[og + 3 * Cu], av = kCached ? av0 : ca[oc];
             const float ddo = (go * (1.f - go)) * (v * av);
@@ -1014,13 +1061,13 @@ __global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_ker
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < nh; ++i)
-        if (wave == i && finisher) {
-            double q0 = 0.0, q1 = 0.0, q2 = 0.0;
-#pragma unroll
-            for (int w = 0; w < NP; ++w) { q0 += red[i][0][w][cl]; q1 += red[i][1][w][cl]; q2 += red[i][2][w][cl]; }
-            ns.dscale[head[i] * Cu + k] = dscale_head + (float)q0;
-            ns.stat(head[i], NormStepArgs::kDMean)[k] = (float)q1; ns.stat(head[i], NormStepArgs::kDSigma)[k] = (float)q2;
-            fin[i][0][cl] = (float)q1; fin[i][1][cl] = (float)q2;
+        if (wave == i) {
+            const double q0 = norm_sum_partials<CW, NP>(red[i][0], lane), q1 = norm_sum_partials<CW, NP>(red[i][1], lane), q2 = norm_sum_partials<CW, NP>(red[i][2], lane);
+            if (finisher) {
+                ns.dscale[head[i] * Cu + fk] = dscale_head + (float)q0;
+                ns.stat(head[i], NormStepArgs::kDMean)[fk] = (float)q1; ns.stat(head[i], NormStepArgs::kDSigma)[fk] = (float)q2;
+                fin[i][0][fc] = (float)q1; fin[i][1][fc] = (float)q2;
+            }
         }
     __syncthreads();
     // ---- those normalisations' last loop, the gates' deltas, the sums of the other groups: 0, 3 and, behind the first step, 5, 1, 4, 6
@@ -1093,13 +1140,13 @@ __global__ __launch_bounds__(kNormBackThreads) void lstm_norm_backward_fused_ker
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < nt; ++i)
-        if (wave == i && finisher) {
-            double q0 = 0.0, q1 = 0.0, q2 = 0.0;
-#pragma unroll
-            for (int w = 0; w < NP; ++w) { q0 += red[i][0][w][cl]; q1 += red[i][1][w][cl]; q2 += red[i][2][w][cl]; }
-            ns.dscale[tail[i] * Cu + k] = dscale_tail + (float)q0;
-            ns.stat(tail[i], NormStepArgs::kDMean)[k] = (float)q1; ns.stat(tail[i], NormStepArgs::kDSigma)[k] = (float)q2;
-            fin[i][0][cl] = (float)q1; fin[i][1][cl] = (float)q2;
+        if (wave == i) {
+            const double q0 = norm_sum_partials<CW, NP>(red[i][0], lane), q1 = norm_sum_partials<CW, NP>(red[i][1], lane), q2 = norm_sum_partials<CW, NP>(red[i][2], lane);
+            if (finisher) {
+                ns.dscale[tail[i] * Cu + fk] = dscale_tail + (float)q0;
+                ns.stat(tail[i], NormStepArgs::kDMean)[fk] = (float)q1; ns.stat(tail[i], NormStepArgs::kDSigma)[fk] = (float)q2;
+                fin[i][0][fc] = (float)q1; fin[i][1][fc] = (float)q2;
+            }
         }
     __syncthreads();
     if (!live) return;
@@ -1515,6 +1562,7 @@ int Net::lstm_backward_step_norm(LstmLayer &q, size_t B, size_t s)
         g.C = q.part; g.ldc = (long)C;
         g.M = (int)B; g.N = (int)C; g.K = (int)G;
         nparts = gemm_split_k(g.M, g.N, g.K);
+        if (nparts > 16) nparts = 16;   // what the slab buffer holds and the kernels below read
         g.split_k = nparts; g.split_k_slab = (long)(B * C);
         MYEA_TRY(launch_gemm(stream, g));
     }
