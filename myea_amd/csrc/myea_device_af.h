@@ -9,6 +9,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "../../include/myea_hip.h"
 
 namespace myea {
@@ -98,6 +100,29 @@ __device__ __forceinline__ float af_derive(int type, float q, float st, float v)
     }
 }
 
+
+// af_fire and af_derive take the layer's activation type as a run-time value.  Inlined into a loop body the whole switch - its
+// sines, exponentials and tables - sits in that loop, and a chain unrolled over time steps carries a copy per step: the lanes
+// then fetch and branch through kilobytes of code for a handful of instructions.  af_with(type, f) calls f with the type as a
+// compile-time constant for the types the hot paths meet and with the run-time value for the others; inside f (a generic
+// lambda that reads its argument as an int) the switch folds to its one case.
+template <int TYPE> using AfConst = std::integral_constant<int, TYPE>;
+template <class F>
+__device__ __forceinline__ void af_with(int type, F &&f)
+{
+    switch (type) {
+    case MYEA_AF_LINEAR: f(AfConst<MYEA_AF_LINEAR>{}); break;
+    case MYEA_AF_SIGMOID: f(AfConst<MYEA_AF_SIGMOID>{}); break;
+    case MYEA_AF_TANH: f(AfConst<MYEA_AF_TANH>{}); break;
+    case MYEA_AF_RELU: f(AfConst<MYEA_AF_RELU>{}); break;
+    case MYEA_AF_LEAKY_RELU: f(AfConst<MYEA_AF_LEAKY_RELU>{}); break;
+    case MYEA_AF_ISRU: f(AfConst<MYEA_AF_ISRU>{}); break;
+    case MYEA_AF_ISRLU: f(AfConst<MYEA_AF_ISRLU>{}); break;
+    case MYEA_AF_ELU: f(AfConst<MYEA_AF_ELU>{}); break;
+    case MYEA_AF_SELU: f(AfConst<MYEA_AF_SELU>{}); break;
+    default: f(type); break;
+    }
+}
 
 // Activations cheap enough to live in a contraction's epilogue (no table, at most one exp).
 __device__ __forceinline__ bool af_is_fusable(int type)

@@ -28,11 +28,15 @@ __global__ __launch_bounds__(kBlock) void fill_kernel(float *p, size_t n, float 
 // appliers (:4907-4990) through a per-column multiplier.
 __global__ __launch_bounds__(kBlock) void activation_kernel(int act, const int *unit_act, size_t n, size_t H, const float *x, float *y, const float *colscale)
 {
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-        float v = af_fire(unit_act ? unit_act[i % H] : act, x[i]);
-        if (colscale) v *= colscale[i % H];
-        y[i] = v;
-    }
+    auto all = [&](auto activation) {
+        const int shared = activation;
+        for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+            float v = af_fire(unit_act ? unit_act[i % H] : shared, x[i]);
+            if (colscale) v *= colscale[i % H];
+            y[i] = v;
+        }
+    };
+    if (unit_act) all(act); else af_with(act, all);
 }
 
 __global__ __launch_bounds__(kBlock) void colscale_kernel(size_t n, size_t H, float *y, const float *colscale)
@@ -49,8 +53,12 @@ __global__ __launch_bounds__(kBlock) void mask_to_scale_kernel(size_t n, const u
 __global__ __launch_bounds__(kBlock) void activation_derive_kernel(int act, float steep, const int *unit_act, const float *unit_steep, size_t H, size_t n,
                                                                    const float *pre, const float *val, const float *dy, float *dx)
 {
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
-        dx[i] = dy[i] * af_derive(unit_act ? unit_act[i % H] : act, pre[i], unit_steep ? unit_steep[i % H] : steep, val[i]);
+    auto all = [&](auto activation) {
+        const int shared = activation;
+        for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock)
+            dx[i] = dy[i] * af_derive(unit_act ? unit_act[i % H] : shared, pre[i], unit_steep ? unit_steep[i % H] : steep, val[i]);
+    };
+    if (unit_act) all(act); else af_with(act, all);
 }
 
 // Independently recurrent layer, the whole sequence in one launch: a thread owns one (example, unit) pair and walks the
@@ -58,70 +66,104 @@ __global__ __launch_bounds__(kBlock) void activation_derive_kernel(int act, floa
 // Forward_Pass__FC_Ind_RNN (NN/Neural_Network__Recurrent_Forward_Pass__Loop.cpp:813-866): pre_AF[t] = input[t] + u * AF[t-1]
 // (a copy at t = 0), then Forward_Pass__FC_AF and, for an un-normalised layer, the Bernoulli applier in place on AF - the
 // value the next time step reads.
-// (The operands of kChunk time steps are requested together, ahead of the chain of dependent steps that consumes them: the
-// chain then waits for memory once per chunk instead of once per step.)
+// Two things bound such a launch: trips to memory inside the chain of dependent steps, and the code of the chain itself - a
+// loop unrolled over the time steps is kilobytes of instructions that every wavefront fetches once and runs once, and that
+// fetch was measured to cost more than the arithmetic.  So the operands of kIndRnnChunk time steps are requested together,
+// ahead of the chain, straight into LDS (a lane's words of LDS are its own: no barrier), and the chain is a loop of a few dozen
+// instructions that reads them from there, with the layer's activation as a compile-time constant where af_with knows it.
 constexpr int kIndRnnChunk = 32;
-__global__ __launch_bounds__(kBlock) void ind_rnn_forward_kernel(IndRnnParams p)
+constexpr int kIndRnnLanes = 128;
+// operand number `which` of the lane's time step `s` of the chunk: [which][s][lane]
+template <int N>
+struct IndRnnStage {
+    float w[N][kIndRnnChunk][kIndRnnLanes];
+    // the load of every lane of the wavefront: global address of the lane's own element, LDS slot of the lane
+    __device__ __forceinline__ void request(int which, int s, const float *from)
+    {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)from,
+                                         (__attribute__((address_space(3))) void *)&w[which][s][threadIdx.x & ~63u], 4, 0, 0);
+    }
+    __device__ __forceinline__ float at(int which, int s) const { return w[which][s][threadIdx.x]; }
+};
+// every request of this wavefront has written its LDS words: vmcnt(0), and nothing that reads them moves above the wait
+__device__ __forceinline__ void ind_rnn_requests_landed()
 {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" ::: "memory");
+}
+
+__global__ __launch_bounds__(kIndRnnLanes) void ind_rnn_forward_kernel(IndRnnParams p)
+{
+    __shared__ IndRnnStage<1> stage;
     const size_t n = p.B * p.H, step = p.Bmax * p.H;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    for (size_t i0 = (size_t)blockIdx.x * kIndRnnLanes; i0 < n; i0 += (size_t)gridDim.x * kIndRnnLanes) {
+        const size_t i = i0 + threadIdx.x;
+        if (i >= n) continue;
         const size_t j = i % p.H;
         const float u = p.u[j];
-        const int act = p.unit_act ? p.unit_act[j] : p.act;
-        float h = 0.f;
-        for (size_t t0 = 0; t0 < p.T; t0 += kIndRnnChunk) {
-            const size_t k0 = i + t0 * step;
-            const int m = (int)(p.T - t0 < (size_t)kIndRnnChunk ? p.T - t0 : (size_t)kIndRnnChunk);
-            float x[kIndRnnChunk], cs[kIndRnnChunk];
-#pragma unroll
-            for (int s = 0; s < kIndRnnChunk; ++s) {
-                x[s] = s < m ? p.in[k0 + s * step] : 0.f;
-                cs[s] = (p.colscale && s < m) ? p.colscale[(t0 + s) * p.H + j] : 1.f;
+        auto walk = [&](auto activation) {
+            const int act = activation;
+            float h = 0.f;
+            for (size_t t0 = 0; t0 < p.T; t0 += kIndRnnChunk) {
+                const size_t k0 = i + t0 * step;
+                const int m = (int)(p.T - t0 < (size_t)kIndRnnChunk ? p.T - t0 : (size_t)kIndRnnChunk);
+                for (int s = 0; s < m; ++s) stage.request(0, s, p.in + k0 + s * step);
+                ind_rnn_requests_landed();
+                float x = stage.at(0, 0), cs = p.colscale ? p.colscale[t0 * p.H + j] : 1.f;
+                for (int s = 0; s < m; ++s) {
+                    const float x_next = s + 1 < m ? stage.at(0, s + 1) : 0.f;
+                    const float cs_next = (p.colscale && s + 1 < m) ? p.colscale[(t0 + s + 1) * p.H + j] : 1.f;
+                    float pre = x;
+                    if (t0 + s) pre = __fadd_rn(pre, __fmul_rn(u, h));
+                    p.pre_afs[k0 + s * step] = pre;
+                    h = af_fire(act, pre);
+                    if (p.colscale) h *= cs;
+                    p.afs[k0 + s * step] = h;
+                    x = x_next; cs = cs_next;
+                }
             }
-#pragma unroll
-            for (int s = 0; s < kIndRnnChunk; ++s) {
-                if (s >= m) break;
-                float pre = x[s];
-                if (t0 + s) pre = __fadd_rn(pre, __fmul_rn(u, h));
-                p.pre_afs[k0 + s * step] = pre;
-                h = af_fire(act, pre);
-                if (p.colscale) h *= cs[s];
-                p.afs[k0 + s * step] = h;
-            }
-        }
+        };
+        if (p.unit_act) walk(p.unit_act[j]); else af_with(p.act, walk);
     }
 }
 
 // Backward_Pass__FC__DF_Ind_RNN (NN/Neural_Network__Backward_Pass__Loop.cpp:1296-1390), time steps from the last to the
 // first: errors = dY AF'(t); dAF(t) = errors + u AF'(t) dAF(t+1), without the second term at the last step.
-__global__ __launch_bounds__(kBlock) void ind_rnn_backward_kernel(IndRnnParams p)
+__global__ __launch_bounds__(kIndRnnLanes) void ind_rnn_backward_kernel(IndRnnParams p)
 {
+    __shared__ IndRnnStage<3> stage;   // pre-activations, activations, the deltas from above
     const size_t n = p.B * p.H, step = p.Bmax * p.H;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+    for (size_t i0 = (size_t)blockIdx.x * kIndRnnLanes; i0 < n; i0 += (size_t)gridDim.x * kIndRnnLanes) {
+        const size_t i = i0 + threadIdx.x;
+        if (i >= n) continue;
         const size_t j = i % p.H;
         const float u = p.u[j], steep = p.unit_steep ? p.unit_steep[j] : p.steep;
-        const int act = p.unit_act ? p.unit_act[j] : p.act;
-        float next = 0.f;
-        for (size_t done = 0; done < p.T; done += kIndRnnChunk) {   // time steps T-1-done, T-2-done, ...
-            const int m = (int)(p.T - done < (size_t)kIndRnnChunk ? p.T - done : (size_t)kIndRnnChunk);
-            const size_t top = p.T - 1 - done;
-            float pre[kIndRnnChunk], val[kIndRnnChunk], dy[kIndRnnChunk];
-#pragma unroll
-            for (int s = 0; s < kIndRnnChunk; ++s) {
-                const size_t k = i + (top - (s < m ? s : 0)) * step;
-                pre[s] = p.pre_afs[k]; val[s] = p.afs[k]; dy[s] = p.dy[k];
+        auto walk = [&](auto activation) {
+            const int act = activation;
+            float next = 0.f;
+            for (size_t done = 0; done < p.T; done += kIndRnnChunk) {   // time steps T-1-done, T-2-done, ...
+                const int m = (int)(p.T - done < (size_t)kIndRnnChunk ? p.T - done : (size_t)kIndRnnChunk);
+                const size_t top = p.T - 1 - done;
+                for (int s = 0; s < m; ++s) {
+                    const size_t k = i + (top - s) * step;
+                    stage.request(0, s, p.pre_afs + k); stage.request(1, s, p.afs + k); stage.request(2, s, p.dy + k);
+                }
+                ind_rnn_requests_landed();
+                float pre = stage.at(0, 0), val = stage.at(1, 0), dy = stage.at(2, 0);
+                for (int s = 0; s < m; ++s) {
+                    const int sn = s + 1 < m ? s + 1 : s;
+                    const float pre_next = stage.at(0, sn), val_next = stage.at(1, sn), dy_next = stage.at(2, sn);
+                    const size_t t = top - s;
+                    const float daf = af_derive(act, pre, steep, val);
+                    const float e = __fmul_rn(dy, daf);
+                    const float r = (t + 1 == p.T) ? e : __fadd_rn(e, __fmul_rn(__fmul_rn(u, daf), next));
+                    p.dafs[i + t * step] = r;
+                    next = r;
+                    pre = pre_next; val = val_next; dy = dy_next;
+                }
             }
-#pragma unroll
-            for (int s = 0; s < kIndRnnChunk; ++s) {
-                if (s >= m) break;
-                const size_t t = top - s;
-                const float daf = af_derive(act, pre[s], steep, val[s]);
-                const float e = __fmul_rn(dy[s], daf);
-                const float r = (t + 1 == p.T) ? e : __fadd_rn(e, __fmul_rn(__fmul_rn(u, daf), next));
-                p.dafs[i + t * step] = r;
-                next = r;
-            }
-        }
+        };
+        if (p.unit_act) walk(p.unit_act[j]); else af_with(p.act, walk);
     }
 }
 
@@ -369,19 +411,22 @@ __global__ __launch_bounds__(kBlock) void bn_forward_final_kernel(size_t H, size
 // "Activation function" loop of the same functions (:4677-4700, :4815-4836)
 __global__ __launch_bounds__(kBlock) void bn_forward_apply_kernel(size_t n, BnForwardParams p)
 {
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
-        const size_t j = i % p.H;
-        float s = (p.x[i] - p.mean[j]) / p.var[j];
-        if (p.renorm) s = s * p.r_corr[j] + p.d_corr[j];
-        p.hats[i] = s;
-        const float y = p.scale[j] * s + p.shift[j];
-        p.normalizes[i] = y;
-        if (p.act_out) {   // Forward_Pass__FC_AF and the Bernoulli applier, as activation_kernel does them
-            float v = af_fire(p.act, y);
-            if (p.colscale) v *= p.colscale[j];
-            p.act_out[i] = v;
+    af_with(p.act, [&](auto activation) {
+        const int act = activation;
+        for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) {
+            const size_t j = i % p.H;
+            float s = (p.x[i] - p.mean[j]) / p.var[j];
+            if (p.renorm) s = s * p.r_corr[j] + p.d_corr[j];
+            p.hats[i] = s;
+            const float y = p.scale[j] * s + p.shift[j];
+            p.normalizes[i] = y;
+            if (p.act_out) {   // Forward_Pass__FC_AF and the Bernoulli applier, as activation_kernel does them
+                float v = af_fire(act, y);
+                if (p.colscale) v *= p.colscale[j];
+                p.act_out[i] = v;
+            }
         }
-    }
+    });
 }
 
 // The "Average" and "Activation function" loops in one launch, from the sums the producing contraction left per block
@@ -440,29 +485,37 @@ __global__ __launch_bounds__(kBlock) void bn_forward_from_sums_kernel(size_t blo
         cs[v] = (p.act_out && p.colscale) ? p.colscale[j] : 1.f;
     }
     const size_t r0 = (size_t)blockIdx.y * rows_per_slice, r1 = r0 + rows_per_slice < p.rows ? r0 + rows_per_slice : p.rows;
-    for (size_t r = r0 + (threadIdx.x >> 6); r < r1; r += kBlock / 64) {
-        const size_t i = r * p.H + j0;
-        float x[V], hat[V], y[V], a[V];
-        if (V == 4) *reinterpret_cast<float4 *>(x) = *reinterpret_cast<const float4 *>(p.x + i); else x[0] = p.x[i];
+    af_with(p.act, [&](auto activation) {
+        const int act = activation;
+        for (size_t r = r0 + (threadIdx.x >> 6); r < r1; r += kBlock / 64) {
+            const size_t i = r * p.H + j0;
+            float x[V], hat[V], y[V], a[V];
+            if (V == 4) *reinterpret_cast<float4 *>(x) = *reinterpret_cast<const float4 *>(p.x + i); else x[0] = p.x[i];
 #pragma unroll
-        for (int v = 0; v < V; ++v) {
-            hat[v] = (x[v] - mean[v]) / var[v];
-            y[v] = scale[v] * hat[v] + shift[v];
-            a[v] = p.act_out ? af_fire(p.act, y[v]) * cs[v] : 0.f;
+            for (int v = 0; v < V; ++v) {
+                hat[v] = (x[v] - mean[v]) / var[v];
+                y[v] = scale[v] * hat[v] + shift[v];
+                a[v] = p.act_out ? af_fire(act, y[v]) * cs[v] : 0.f;
+            }
+            if (V == 4) {
+                *reinterpret_cast<float4 *>(p.hats + i) = *reinterpret_cast<const float4 *>(hat);
+                *reinterpret_cast<float4 *>(p.normalizes + i) = *reinterpret_cast<const float4 *>(y);
+                if (p.act_out) *reinterpret_cast<float4 *>(p.act_out + i) = *reinterpret_cast<const float4 *>(a);
+            } else {
+                p.hats[i] = hat[0]; p.normalizes[i] = y[0];
+                if (p.act_out) p.act_out[i] = a[0];
+            }
         }
-        if (V == 4) {
-            *reinterpret_cast<float4 *>(p.hats + i) = *reinterpret_cast<const float4 *>(hat);
-            *reinterpret_cast<float4 *>(p.normalizes + i) = *reinterpret_cast<const float4 *>(y);
-            if (p.act_out) *reinterpret_cast<float4 *>(p.act_out + i) = *reinterpret_cast<const float4 *>(a);
-        } else {
-            p.hats[i] = hat[0]; p.normalizes[i] = y[0];
-            if (p.act_out) p.act_out[i] = a[0];
-        }
-    }
+    });
 }
 
 // The backward pass's three loops in one launch, from sums[blk][0][j] = sum of dy * hats and sums[blk][1][j] = sum of dy:
 // with hats = (x - mean) / sigma the two other sums of the first loop are these two times -scale / sigma.
+// The launch is a chain - the blocks' sums, the column terms, the rows - and each link that asks memory for something only when
+// its turn comes adds a round trip: a lane asks for its share of the sums, its columns' statistics and its first kBnHeld rows
+// before it waits for anything; rows beyond those are read in the loop.  (The forward kernel measured no faster that way: it
+// writes three tensors for each one it reads and is bound by those.)
+constexpr int kBnHeld = 4;
 template <int V>
 __global__ __launch_bounds__(kBlock) void bn_backward_from_sums_kernel(size_t blocks, size_t rows_per_slice, const float *sums, BnBackwardParams p)
 {
@@ -471,17 +524,50 @@ __global__ __launch_bounds__(kBlock) void bn_backward_from_sums_kernel(size_t bl
     constexpr int kWaves = kBlock / 64;
     __shared__ double s_a0[kWaves][64 * V], s_a1[kWaves][64 * V];
     const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
+    const bool keeper = blockIdx.y == 0 && w == 0;   // adds the column sums to the scale's and the shift's derivatives
+    const size_t r0 = (size_t)blockIdx.y * rows_per_slice, r1 = r0 + rows_per_slice < p.rows ? r0 + rows_per_slice : p.rows;
+    float held_dy[kBnHeld][V], held_x[kBnHeld][V], vb[V], scale[V], mean[V], dscale_old[V], dshift_old[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) { vb[v] = 1.f; scale[v] = 0.f; mean[v] = 0.f; dscale_old[v] = 0.f; dshift_old[v] = 0.f; }
     {
         double a0[V], a1[V];
 #pragma unroll
         for (int v = 0; v < V; ++v) { a0[v] = 0.0; a1[v] = 0.0; }
         if (live) {
-            for (size_t y = w; y < blocks; y += kWaves) {
-                float a[V], b[V];
-                if (V == 4) { *reinterpret_cast<float4 *>(a) = *reinterpret_cast<const float4 *>(sums + (y * 2 + 0) * p.H + j0); *reinterpret_cast<float4 *>(b) = *reinterpret_cast<const float4 *>(sums + (y * 2 + 1) * p.H + j0); }
-                else { a[0] = sums[(y * 2 + 0) * p.H + j0]; b[0] = sums[(y * 2 + 1) * p.H + j0]; }
 #pragma unroll
-                for (int v = 0; v < V; ++v) { a0[v] += a[v]; a1[v] += b[v]; }
+            for (int h = 0; h < kBnHeld; ++h) {
+                const size_t r = r0 + w + (size_t)h * kWaves;
+#pragma unroll
+                for (int v = 0; v < V; ++v) { held_dy[h][v] = 0.f; held_x[h][v] = 0.f; }
+                if (r < r1) {
+                    if (V == 4) { *reinterpret_cast<float4 *>(held_dy[h]) = *reinterpret_cast<const float4 *>(p.dy + r * p.H + j0); *reinterpret_cast<float4 *>(held_x[h]) = *reinterpret_cast<const float4 *>(p.x + r * p.H + j0); }
+                    else { held_dy[h][0] = p.dy[r * p.H + j0]; held_x[h][0] = p.x[r * p.H + j0]; }
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                vb[v] = p.var[j0 + v]; scale[v] = p.scale[j0 + v]; mean[v] = p.mean[j0 + v];
+                if (keeper) { dscale_old[v] = p.dscale[j0 + v]; dshift_old[v] = p.dshift[j0 + v]; }
+            }
+            constexpr int kAhead = 4;   // blocks a wavefront asks for at once
+            for (size_t y0 = w; y0 < blocks; y0 += kAhead * kWaves) {
+                float a[kAhead][V], b[kAhead][V];
+#pragma unroll
+                for (int u = 0; u < kAhead; ++u) {
+                    const size_t y = y0 + (size_t)u * kWaves;
+#pragma unroll
+                    for (int v = 0; v < V; ++v) { a[u][v] = 0.f; b[u][v] = 0.f; }
+                    if (y < blocks) {
+                        if (V == 4) { *reinterpret_cast<float4 *>(a[u]) = *reinterpret_cast<const float4 *>(sums + (y * 2 + 0) * p.H + j0); *reinterpret_cast<float4 *>(b[u]) = *reinterpret_cast<const float4 *>(sums + (y * 2 + 1) * p.H + j0); }
+                        else { a[u][0] = sums[(y * 2 + 0) * p.H + j0]; b[u][0] = sums[(y * 2 + 1) * p.H + j0]; }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kAhead; ++u)
+                    if (y0 + (size_t)u * kWaves < blocks) {
+#pragma unroll
+                        for (int v = 0; v < V; ++v) { a0[v] += a[u][v]; a1[v] += b[u][v]; }
+                    }
             }
         }
 #pragma unroll
@@ -489,24 +575,30 @@ __global__ __launch_bounds__(kBlock) void bn_backward_from_sums_kernel(size_t bl
     }
     __syncthreads();
     if (!live) return;
-    float vb[V], scale[V], mean[V], dmean[V], dvar[V];
+    float dmean[V], dvar[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
         const size_t j = j0 + v;
         double a0 = 0.0, a1 = 0.0;
 #pragma unroll
         for (int k = 0; k < kWaves; ++k) { a0 += s_a0[k][l * V + v]; a1 += s_a1[k][l * V + v]; }
-        if (blockIdx.y == 0 && w == 0) { p.dscale[j] += (float)a0; p.dshift[j] += (float)a1; }
-        vb[v] = p.var[j]; scale[v] = p.scale[j]; mean[v] = p.mean[j];
+        if (keeper) { p.dscale[j] = dscale_old[v] + (float)a0; p.dshift[j] = dshift_old[v] + (float)a1; }
         dmean[v] = (float)a1 * scale[v] * (-1.f / vb[v]);
         dvar[v] = (float)a0 * scale[v] * (-1.f / vb[v]);
     }
     const float bsz = (float)p.rows, bscale = 1.f / (float)p.rows;
-    const size_t r0 = (size_t)blockIdx.y * rows_per_slice, r1 = r0 + rows_per_slice < p.rows ? r0 + rows_per_slice : p.rows;
-    for (size_t r = r0 + (threadIdx.x >> 6); r < r1; r += kBlock / 64) {
+    int h = 0;
+    for (size_t r = r0 + (threadIdx.x >> 6); r < r1; r += kBlock / 64, ++h) {
         const size_t i = r * p.H + j0;
         float dy[V], x[V], dx[V];
-        if (V == 4) { *reinterpret_cast<float4 *>(dy) = *reinterpret_cast<const float4 *>(p.dy + i); *reinterpret_cast<float4 *>(x) = *reinterpret_cast<const float4 *>(p.x + i); }
+        if (h < kBnHeld) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                dy[v] = held_dy[0][v]; x[v] = held_x[0][v];
+#pragma unroll
+                for (int u = 1; u < kBnHeld; ++u) if (h == u) { dy[v] = held_dy[u][v]; x[v] = held_x[u][v]; }
+            }
+        } else if (V == 4) { *reinterpret_cast<float4 *>(dy) = *reinterpret_cast<const float4 *>(p.dy + i); *reinterpret_cast<float4 *>(x) = *reinterpret_cast<const float4 *>(p.x + i); }
         else { dy[0] = p.dy[i]; x[0] = p.x[i]; }
 #pragma unroll
         for (int v = 0; v < V; ++v) {
@@ -1097,7 +1189,7 @@ int launch_k_sparse(hipStream_t s, size_t rows, size_t H, size_t k, float *x)
 int launch_ind_rnn_forward(hipStream_t s, const IndRnnParams &p)
 {
     if (p.B * p.H == 0 || p.T == 0) return MYEA_OK;
-    hipLaunchKernelGGL(ind_rnn_forward_kernel, dim3(grid_for(p.B * p.H, kBlock)), dim3(kBlock), 0, s, p);
+    hipLaunchKernelGGL(ind_rnn_forward_kernel, dim3(grid_for(p.B * p.H, kIndRnnLanes)), dim3(kIndRnnLanes), 0, s, p);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
@@ -1105,7 +1197,7 @@ int launch_ind_rnn_forward(hipStream_t s, const IndRnnParams &p)
 int launch_ind_rnn_backward(hipStream_t s, const IndRnnParams &p)
 {
     if (p.B * p.H == 0 || p.T == 0) return MYEA_OK;
-    hipLaunchKernelGGL(ind_rnn_backward_kernel, dim3(grid_for(p.B * p.H, kBlock)), dim3(kBlock), 0, s, p);
+    hipLaunchKernelGGL(ind_rnn_backward_kernel, dim3(grid_for(p.B * p.H, kIndRnnLanes)), dim3(kIndRnnLanes), 0, s, p);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
@@ -1149,11 +1241,11 @@ int launch_bn_forward_training(hipStream_t s, const BnForwardParams &p, float *s
     return MYEA_OK;
 }
 
-// rows per slice so that the grid has about a thousand workgroups, at least 8 rows each
-static size_t bn_rows_per_slice(size_t rows, size_t colblocks)
+// rows per slice so that the grid has about a thousand workgroups, at least `least` rows each
+static size_t bn_rows_per_slice(size_t rows, size_t colblocks, size_t least)
 {
     size_t slices = (1024 + colblocks - 1) / colblocks;
-    if (slices > (rows + 7) / 8) slices = (rows + 7) / 8;
+    if (slices > (rows + least - 1) / least) slices = (rows + least - 1) / least;
     if (slices < 1) slices = 1;
     return (rows + slices - 1) / slices;
 }
@@ -1170,7 +1262,9 @@ int launch_bn_forward_training_from_sums(hipStream_t s, const BnForwardParams &p
     if (p.renorm || !sums || blocks == 0) { set_last_error("bn_forward_training_from_sums: plain batch normalisation with its column sums only"); return MYEA_E_INVALID; }
     static_assert(kBlock % 64 == 0, "64 lanes of columns per workgroup");
     const bool wide = rows_of_float4(p.H, {p.x, p.hats, p.normalizes, p.act_out});
-    const size_t colblocks = (p.H + (wide ? 255 : 63)) / (wide ? 256 : 64), per = bn_rows_per_slice(p.rows, colblocks);
+    // a row a wavefront where the batch allows: the launch's time is its row loop, a memory round trip an iteration (512 x 2048:
+    // 10.1 us at 4 rows a slice, 10.5 at 8, 12.1 at 16)
+    const size_t colblocks = (p.H + (wide ? 255 : 63)) / (wide ? 256 : 64), per = bn_rows_per_slice(p.rows, colblocks, 4);
     const dim3 grid((unsigned)colblocks, (unsigned)((p.rows + per - 1) / per));
     if (wide) hipLaunchKernelGGL(bn_forward_from_sums_kernel<4>, grid, dim3(kBlock), 0, s, blocks, per, sums, p);
     else hipLaunchKernelGGL(bn_forward_from_sums_kernel<1>, grid, dim3(kBlock), 0, s, blocks, per, sums, p);
@@ -1183,7 +1277,7 @@ int launch_bn_backward_from_sums(hipStream_t s, const BnBackwardParams &p, const
     if (p.H == 0 || p.rows == 0) return MYEA_OK;
     if (p.renorm || !sums || blocks == 0) { set_last_error("bn_backward_from_sums: plain batch normalisation with its column sums only"); return MYEA_E_INVALID; }
     const bool wide = rows_of_float4(p.H, {p.x, p.dy, p.dx});
-    const size_t colblocks = (p.H + (wide ? 255 : 63)) / (wide ? 256 : 64), per = bn_rows_per_slice(p.rows, colblocks);
+    const size_t colblocks = (p.H + (wide ? 255 : 63)) / (wide ? 256 : 64), per = bn_rows_per_slice(p.rows, colblocks, 4 * kBnHeld);
     const dim3 grid((unsigned)colblocks, (unsigned)((p.rows + per - 1) / per));
     if (wide) hipLaunchKernelGGL(bn_backward_from_sums_kernel<4>, grid, dim3(kBlock), 0, s, blocks, per, sums, p);
     else hipLaunchKernelGGL(bn_backward_from_sums_kernel<1>, grid, dim3(kBlock), 0, s, blocks, per, sums, p);
@@ -1254,20 +1348,23 @@ __global__ __launch_bounds__(kBlock) void bn_forward_sequence_kernel(BnForwardPa
     }
     const float mean = s_stat[0][c], var = s_stat[1][c], rc = s_stat[2][c], dc = s_stat[3][c];
     const float cs = p.colscale ? p.colscale[sj] : 1.f;
+    af_with(p.act, [&](auto activation) {
+        const int act = activation;
 #pragma unroll 4
-    for (size_t r = rl; r < p.rows; r += kLanes) {
-        const size_t i = base + r * p.H + j;
-        float h = (p.x[i] - mean) / var;
-        if (p.renorm) h = h * rc + dc;
-        p.hats[i] = h;
-        const float y = scale * h + shift;
-        p.normalizes[i] = y;
-        if (p.act_out) {
-            float v = af_fire(p.act, y);
-            if (p.colscale) v *= cs;
-            p.act_out[i] = v;
+        for (size_t r = rl; r < p.rows; r += kLanes) {
+            const size_t i = base + r * p.H + j;
+            float h = (p.x[i] - mean) / var;
+            if (p.renorm) h = h * rc + dc;
+            p.hats[i] = h;
+            const float y = scale * h + shift;
+            p.normalizes[i] = y;
+            if (p.act_out) {
+                float v = af_fire(act, y);
+                if (p.colscale) v *= cs;
+                p.act_out[i] = v;
+            }
         }
-    }
+    });
 }
 
 static int sequence_columns(size_t H, size_t T)

@@ -640,6 +640,56 @@ int launch_layout_scalar(hipStream_t stream, const GemmDev &d, bool a_kc, bool b
     return launch_one<64, 64, false, true, false>(stream, d);
 }
 
+
+// ---- the weight gradient of a narrow layer ------------------------------------------------------------------------------
+// dW = delta^T X with at most 32 outputs (columns of delta) and at most 32 inputs (columns of X) over many rows - a layer of an
+// independently recurrent stack over T x batch rows.  Two rows of delta and of X, as they lie in memory, ARE the operands of
+// v_mfma_f32_32x32x2f32 (lane l: column l % 32 of row l / 32): a wavefront walks its share of the rows with two coalesced
+// loads and one matrix instruction per pair of rows, no LDS, no tile edges to test; a loop of a few dozen instructions.
+// The wavefronts of a workgroup add their 32 x 32 accumulators in wavefront order and store one slab [H][In]; the slabs
+// are added by launch_slab_sum_add, as the slabs of a split-K launch are.  (The tiled kernel spends its time on such a
+// shape in its set-up, its predicated scalar loads of operands whose rows are not 16-byte multiples, and its epilogue.)
+constexpr int kNarrowAhead = 16;   // pairs of rows a wavefront asks for at once: its whole share when the launch is not capped
+constexpr int kNarrowWaves = 8;    // wavefronts a workgroup: fewer slabs to add afterwards
+__global__ __launch_bounds__(64 * kNarrowWaves) void narrow_dw_kernel(const float *__restrict__ delta, const float *__restrict__ x, float *__restrict__ slabs,
+                                                             int H, int In, long rows, long rows_per_wave)
+{
+    __shared__ float handed[kNarrowWaves - 1][16][64];   // the accumulators of the wavefronts behind the first
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 31, half = lane >> 5;
+    const long first = ((long)blockIdx.x * kNarrowWaves + wave) * rows_per_wave;
+    const long last = first + rows_per_wave < rows ? first + rows_per_wave : rows;
+    const bool in_delta = col < H, in_x = col < In;
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (long r0 = first; r0 < last; r0 += 2 * kNarrowAhead) {
+        float a[kNarrowAhead], b[kNarrowAhead];
+#pragma unroll
+        for (int u = 0; u < kNarrowAhead; ++u) {
+            const long row = r0 + 2 * u + half;
+            a[u] = (in_delta && row < last) ? delta[row * H + col] : 0.f;
+            b[u] = (in_x && row < last) ? x[row * In + col] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < kNarrowAhead; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+    }
+    if (wave) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) handed[wave - 1][r][lane] = acc[r];
+    }
+    __syncthreads();
+    if (wave || !in_x) return;
+    float *slab = slabs + (size_t)blockIdx.x * H * In;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m = (r >> 2) * 8 + half * 4 + (r & 3);   // the accumulator's row of this lane's column
+        float v = acc[r];
+#pragma unroll
+        for (int w = 0; w < kNarrowWaves - 1; ++w) v += handed[w][r][lane];
+        if (m < H) slab[m * In + col] = v;
+    }
+}
+
 }  // namespace
 
 // Number of K slabs for a contraction whose M x N alone does not fill the chip; 1 when the plain launch already does.
@@ -730,6 +780,29 @@ static int prepare_gemm(const GemmParams &p, GemmDev &d, bool *vec)
         return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0 && (ld & 3) == 0 && (contiguous_extent & 3) == 0;
     };
     *vec = aligned(p.A, p.lda, p.a_k_contiguous ? p.K : p.M) && aligned(p.B, p.ldb, p.b_k_contiguous ? p.K : p.N);
+    return MYEA_OK;
+}
+
+// Slabs the narrow weight-gradient kernel writes for these shapes: 0 when the shape is not its own (the tiled kernel takes it).
+// A wavefront gets at least 32 rows (one round of loads), a launch at most 128 workgroups.
+int narrow_dw_slabs(size_t H, size_t In, size_t rows)
+{
+    if (H == 0 || In == 0 || H > 32 || In > 32 || rows < 512 || rows > 0x7fffffffu) return 0;
+    static const bool off = [] { const char *e = std::getenv("MYEA_NARROW_DW"); return e && e[0] == '0'; }();
+    if (off) return 0;
+    size_t per_wave = 2 * kNarrowAhead;
+    while ((rows + kNarrowWaves * per_wave - 1) / (kNarrowWaves * per_wave) > 128) per_wave *= 2;
+    return (int)((rows + kNarrowWaves * per_wave - 1) / (kNarrowWaves * per_wave));
+}
+
+// delta [rows][H], x [rows][In], both dense; slabs: narrow_dw_slabs(H, In, rows) x [H][In]
+int launch_narrow_dw(hipStream_t stream, const float *delta, const float *x, float *slabs, size_t H, size_t In, size_t rows)
+{
+    const int S = narrow_dw_slabs(H, In, rows);
+    if (S <= 0 || !delta || !x || !slabs) { set_last_error("narrow weight gradient: %zu x %zu over %zu rows is not its shape", H, In, rows); return MYEA_E_INVALID; }
+    const long per_wave = (long)(((rows + (size_t)S * kNarrowWaves - 1) / ((size_t)S * kNarrowWaves) + 1) / 2 * 2);   // even: a matrix instruction takes a pair of rows
+    hipLaunchKernelGGL(narrow_dw_kernel, dim3((unsigned)S), dim3(64 * kNarrowWaves), 0, stream, delta, x, slabs, (int)H, (int)In, (long)rows, per_wave);
+    MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
 

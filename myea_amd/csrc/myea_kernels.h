@@ -81,6 +81,10 @@ unsigned gemm_pair_polls();
 // (at most one such tile per compute unit, a k worth halving): callers size their pair buffers by it
 bool gemm_pair_k_128(int M, int N, int K);
 int launch_gemm(hipStream_t stream, const GemmParams &p);
+// The weight gradient delta^T X of a layer with at most 32 outputs and 32 inputs over many rows, as slabs [H][In] to be added:
+// narrow_dw_slabs gives their number (0: not this kernel's shape), launch_narrow_dw writes them.
+int narrow_dw_slabs(size_t H, size_t In, size_t rows);
+int launch_narrow_dw(hipStream_t stream, const float *delta, const float *x, float *slabs, size_t H, size_t In, size_t rows);
 // dX = delta W (`a`) and dW += delta^T X (`b`) in one launch when their shapes suit it; MYEA_OK = launched, 1 = does not
 // apply (launch them one after the other), negative = error
 int launch_gemm_pair(hipStream_t stream, const GemmParams &a, const GemmParams &b);

@@ -1344,6 +1344,8 @@ static int fc_dw_slabs(size_t H, size_t In, size_t rows, size_t first_connection
 {
     (void)first_connection_index;
     if (rows > 0x7fffffffu) return 1;
+    const int narrow = narrow_dw_slabs(H, In, rows);   // a narrow layer's kernel of its own: always through slabs
+    if (narrow > 0) return narrow > 1 ? narrow : 2;    // (room for two, so that "more than one slab" still says "through slabs")
     return gemm_split_k((int)H, (int)In, (int)rows);
 }
 
@@ -1400,12 +1402,14 @@ int Net::update_derivative_weight_contraction(size_t li, size_t B)
         g.C = gradient + l.first_connection_index; g.ldc = (long)In;
         g.M = (int)H; g.N = (int)In; g.K = (int)rows;
         g.accumulate = 1; g.c_is_zero = dw_may_store(li) ? 1 : 0; g.epilogue = EPI_NONE;
-        const int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
+        int slabs = dw_slabs ? fc_dw_slabs(H, In, rows, l.first_connection_index) : 1;
+        const int narrow = dw_slabs ? narrow_dw_slabs(H, In, rows) : 0;
         if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.c_is_zero = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
         if (li < dw_zero.size()) dw_zero[li] = 0;   // from here on the slice holds this product, stored or added from the slabs
         prof_begin(2);
-        MYEA_TRY(launch_gemm(stream, g));
-        if (slabs > 1) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
+        if (narrow > 0) { slabs = narrow; MYEA_TRY(launch_narrow_dw(stream, g.A, g.B, dw_slabs, H, In, rows)); }
+        else MYEA_TRY(launch_gemm(stream, g));
+        if (slabs > 1 || narrow > 0) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
         prof_end(2.0 * (double)rows * (double)H * (double)In);
     }
 
