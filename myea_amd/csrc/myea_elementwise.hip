@@ -1286,60 +1286,81 @@ int launch_bn_backward_from_sums(hipStream_t s, const BnBackwardParams &p, const
 }
 
 // Every time step of a [T][Bmax][H] tensor in one launch.  Each time step has statistics of its own (the reference runs the
-// layer's normalisation once per time step); workgroup (column block, t) owns 64 columns of time step t over all of its rows:
-// the column sums meet in LDS (four row lanes), one lane per column finishes the statistics exactly as bn_forward_final_kernel
-// does, then the workgroup applies them as bn_forward_apply_kernel does.  p's per-time-step vectors (mean, var, averages,
+// layer's normalisation once per time step); workgroup (column block, t) owns CW columns of time step t over all of its rows:
+// the column sums meet in LDS, one lane per column finishes the statistics with bn_forward_final_kernel's arithmetic, then the
+// workgroup applies them as bn_forward_apply_kernel does.  p's per-time-step vectors (mean, var, averages,
 // corrections, colscale) are those of time step 0, H apart from one step to the next; its tensors those of time step 0,
 // Bmax * H apart.  training == 0: the running averages of each time step, nothing written but the output.
-template <int CW>   // columns per workgroup: 64, or 16 for narrow layers (more row lanes, shorter loops)
+// A launch is a chain of passes that wait for each other, so a lane asks for its first kSeqHeld rows and its column's parameters
+// before anything waits and keeps those rows in registers for the second pass; the column sums take the two-stage form of
+// norm_fold_partial / norm_sum_partials.
+constexpr int kSeqHeld = 4;
+template <int CW>   // columns per workgroup: 64, or 16 / 4 for narrow layers (more row lanes, shorter loops)
 __global__ __launch_bounds__(kBlock) void bn_forward_sequence_kernel(BnForwardParams p, size_t Bmax, int training)
 {
-    constexpr int kLanes = kBlock / CW;
-    __shared__ double s_sum[kLanes][CW], s_sq[kLanes][CW];
+    constexpr int kLanes = kBlock / CW, NW = kBlock / 64, NP = NW * kNormPartials<CW>;
+    __shared__ double red[2][NP][CW];
     __shared__ float s_stat[4][CW];
-    const int c = threadIdx.x % CW, rl = threadIdx.x / CW;
+    const int c = threadIdx.x % CW, rl = threadIdx.x / CW, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const size_t t = blockIdx.y, j = (size_t)blockIdx.x * CW + c;
     const bool live = j < p.H;
     const size_t base = t * Bmax * p.H, sj = t * p.H + j;
+    // the lanes of wavefront 0 that finish the statistics: column fc of the workgroup
+    const int fc = norm_finish_column<CW>(lane);
+    const size_t fj = (size_t)blockIdx.x * CW + fc, sfj = t * p.H + fj;
+    const bool keeper = wave == 0 && norm_finish_keeper<CW>(lane) && fj < p.H;
+    float held[kSeqHeld], scale = 0.f, shift = 0.f, cs = 1.f, mavg = 0.f, vavg = 1.f;
+#pragma unroll
+    for (int h = 0; h < kSeqHeld; ++h) held[h] = 0.f;
+    if (live) {
+#pragma unroll
+        for (int h = 0; h < kSeqHeld; ++h) {
+            const size_t r = rl + (size_t)h * kLanes;
+            if (r < p.rows) held[h] = p.x[base + r * p.H + j];
+        }
+        scale = p.scale[j]; shift = p.shift[j];
+        if (p.colscale) cs = p.colscale[sj];
+        if (!training) { mavg = p.mean_avg[sj]; vavg = p.var_avg[sj]; }
+    }
+    if (training && keeper) { mavg = p.mean_avg[sfj]; vavg = p.var_avg[sfj]; }
     if (training) {
         double sm = 0.0, sv = 0.0;
         if (live) {
-#pragma unroll 8
-            for (size_t r = rl; r < p.rows; r += kLanes) { const double v = p.x[base + r * p.H + j]; sm += v; sv += v * v; }
-        }
-        s_sum[rl][c] = sm; s_sq[rl][c] = sv;
-        __syncthreads();
-        if (rl == 0 && live) {
-            double smd = 0.0, svd = 0.0;
 #pragma unroll
-            for (int k = 0; k < kLanes; ++k) { smd += s_sum[k][c]; svd += s_sq[k][c]; }
-            const float bscale = 1.f / (float)p.rows;
-            const float mean = (float)smd * bscale;
-            float mavg = p.mean_avg[sj];
-            mavg += p.momentum * (mean - mavg);
-            p.mean_avg[sj] = mavg;
-            const float var = sqrtf((float)svd * bscale - mean * mean + p.epsilon);
-            float vavg = p.var_avg[sj];
-            vavg += p.momentum * (var - vavg);
-            p.var_avg[sj] = vavg;
-            p.mean[sj] = mean;
-            p.var[sj] = var;
-            float rc = 1.f, dc = 0.f;
-            if (p.renorm) {
-                const float g = var / vavg, lo = 1.f / p.r_max;
-                rc = g < lo ? lo : (g > p.r_max ? p.r_max : g);
-                const float d = (mean - mavg) / vavg;
-                dc = d < -p.d_max ? -p.d_max : (d > p.d_max ? p.d_max : d);
-                p.r_corr[sj] = rc; p.d_corr[sj] = dc;
+            for (int h = 0; h < kSeqHeld; ++h)
+                if (rl + (size_t)h * kLanes < p.rows) { const double v = held[h]; sm += v; sv += v * v; }
+            for (size_t r = rl + (size_t)kSeqHeld * kLanes; r < p.rows; r += kLanes) { const double v = p.x[base + r * p.H + j]; sm += v; sv += v * v; }
+        }
+        sm = norm_fold_partial<CW>(sm); sv = norm_fold_partial<CW>(sv);
+        if (norm_partial_holder<CW>(lane)) { const int slot = norm_partial_index<CW>(wave, lane); red[0][slot][c] = sm; red[1][slot][c] = sv; }
+        __syncthreads();
+        if (wave == 0) {
+            const double smd = norm_sum_partials<CW, NP>(red[0], lane), svd = norm_sum_partials<CW, NP>(red[1], lane);
+            if (keeper) {
+                const float bscale = 1.f / (float)p.rows;
+                const float mean = (float)smd * bscale;
+                mavg += p.momentum * (mean - mavg);
+                p.mean_avg[sfj] = mavg;
+                const float var = sqrtf((float)svd * bscale - mean * mean + p.epsilon);
+                vavg += p.momentum * (var - vavg);
+                p.var_avg[sfj] = vavg;
+                p.mean[sfj] = mean;
+                p.var[sfj] = var;
+                float rc = 1.f, dc = 0.f;
+                if (p.renorm) {
+                    const float g = var / vavg, lo = 1.f / p.r_max;
+                    rc = g < lo ? lo : (g > p.r_max ? p.r_max : g);
+                    const float d = (mean - mavg) / vavg;
+                    dc = d < -p.d_max ? -p.d_max : (d > p.d_max ? p.d_max : d);
+                    p.r_corr[sfj] = rc; p.d_corr[sfj] = dc;
+                }
+                s_stat[0][fc] = mean; s_stat[1][fc] = var; s_stat[2][fc] = rc; s_stat[3][fc] = dc;
             }
-            s_stat[0][c] = mean; s_stat[1][c] = var; s_stat[2][c] = rc; s_stat[3][c] = dc;
         }
         __syncthreads();
     }
     if (!live) return;
-    const float scale = p.scale[j], shift = p.shift[j];
     if (!training) {
-        const float mavg = p.mean_avg[sj], vavg = p.var_avg[sj];
         for (size_t r = rl; r < p.rows; r += kLanes) {
             const size_t i = base + r * p.H + j;
             p.normalizes[i] = scale * ((p.x[i] - mavg) / vavg) + shift;
@@ -1347,13 +1368,11 @@ __global__ __launch_bounds__(kBlock) void bn_forward_sequence_kernel(BnForwardPa
         return;
     }
     const float mean = s_stat[0][c], var = s_stat[1][c], rc = s_stat[2][c], dc = s_stat[3][c];
-    const float cs = p.colscale ? p.colscale[sj] : 1.f;
     af_with(p.act, [&](auto activation) {
         const int act = activation;
-#pragma unroll 4
-        for (size_t r = rl; r < p.rows; r += kLanes) {
+        auto row = [&](size_t r, float x) {
             const size_t i = base + r * p.H + j;
-            float h = (p.x[i] - mean) / var;
+            float h = (x - mean) / var;
             if (p.renorm) h = h * rc + dc;
             p.hats[i] = h;
             const float y = scale * h + shift;
@@ -1363,7 +1382,11 @@ __global__ __launch_bounds__(kBlock) void bn_forward_sequence_kernel(BnForwardPa
                 if (p.colscale) v *= cs;
                 p.act_out[i] = v;
             }
-        }
+        };
+#pragma unroll
+        for (int h = 0; h < kSeqHeld; ++h)
+            if (rl + (size_t)h * kLanes < p.rows) row(rl + (size_t)h * kLanes, held[h]);
+        for (size_t r = rl + (size_t)kSeqHeld * kLanes; r < p.rows; r += kLanes) row(r, p.x[base + r * p.H + j]);
     });
 }
 
@@ -1394,52 +1417,76 @@ int launch_bn_forward_sequence(hipStream_t s, const BnForwardParams &p, size_t T
 template <int CW>
 __global__ __launch_bounds__(kBlock) void bn_backward_sequence_kernel(BnBackwardParams p, size_t Bmax, float *__restrict__ partial)
 {
-    constexpr int kLanes = kBlock / CW;
-    __shared__ double s_acc[4][kLanes][CW];
+    constexpr int kLanes = kBlock / CW, NW = kBlock / 64, NP = NW * kNormPartials<CW>;
+    static_assert(NW == 4, "a wavefront finishes each of the four column sums");
+    __shared__ double red[4][NP][CW];
     __shared__ float s_d[2][CW];
-    const int c = threadIdx.x % CW, rl = threadIdx.x / CW;
+    const int c = threadIdx.x % CW, rl = threadIdx.x / CW, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const size_t t = blockIdx.y, j = (size_t)blockIdx.x * CW + c;
     const bool live = j < p.H;
     const size_t base = t * Bmax * p.H, sj = t * p.H + j;
+    const int fc = norm_finish_column<CW>(lane);
+    const size_t fj = (size_t)blockIdx.x * CW + fc;
+    const bool keeper = norm_finish_keeper<CW>(lane) && fj < p.H;
     float vb = 1.f, rc = 1.f, mean = 0.f, scale = 0.f;
-    if (live) { vb = p.var[sj]; rc = p.renorm ? p.r_corr[sj] : 1.f; mean = p.mean[sj]; scale = p.scale[j]; }
+    float held_dy[kSeqHeld], held_x[kSeqHeld], held_hat[kSeqHeld];
+#pragma unroll
+    for (int h = 0; h < kSeqHeld; ++h) { held_dy[h] = 0.f; held_x[h] = 0.f; held_hat[h] = 0.f; }
+    if (live) {
+#pragma unroll
+        for (int h = 0; h < kSeqHeld; ++h) {
+            const size_t r = rl + (size_t)h * kLanes;
+            if (r < p.rows) { const size_t k = base + r * p.H + j; held_dy[h] = p.dy[k]; held_hat[h] = p.hats[k]; held_x[h] = p.x[k]; }
+        }
+        vb = p.var[sj]; rc = p.renorm ? p.r_corr[sj] : 1.f; mean = p.mean[sj]; scale = p.scale[j];
+    }
     double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
     if (live) {
-#pragma unroll 4
-        for (size_t r = rl; r < p.rows; r += kLanes) {
-            const size_t k = base + r * p.H + j;
-            float e = p.dy[k];
-            a0 += e * p.hats[k];
+        auto row = [&](float e, float hat, float x) {
+            a0 += e * hat;
             a1 += e;
             e *= scale;
             a2 += e * (-rc / vb);
-            a3 += e * (p.x[k] - mean) * (-rc / (vb * vb));
+            a3 += e * (x - mean) * (-rc / (vb * vb));
+        };
+#pragma unroll
+        for (int h = 0; h < kSeqHeld; ++h)
+            if (rl + (size_t)h * kLanes < p.rows) row(held_dy[h], held_hat[h], held_x[h]);
+        for (size_t r = rl + (size_t)kSeqHeld * kLanes; r < p.rows; r += kLanes) {
+            const size_t k = base + r * p.H + j;
+            row(p.dy[k], p.hats[k], p.x[k]);
         }
     }
-    s_acc[0][rl][c] = a0; s_acc[1][rl][c] = a1; s_acc[2][rl][c] = a2; s_acc[3][rl][c] = a3;
+    a0 = norm_fold_partial<CW>(a0); a1 = norm_fold_partial<CW>(a1); a2 = norm_fold_partial<CW>(a2); a3 = norm_fold_partial<CW>(a3);
+    if (norm_partial_holder<CW>(lane)) {
+        const int slot = norm_partial_index<CW>(wave, lane);
+        red[0][slot][c] = a0; red[1][slot][c] = a1; red[2][slot][c] = a2; red[3][slot][c] = a3;
+    }
     __syncthreads();
-    if (rl == 0 && live) {
-        double b[4] = {0.0, 0.0, 0.0, 0.0};
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-            for (int k = 0; k < kLanes; ++k) b[q] += s_acc[q][k][c];
-        partial[(t * 2 + 0) * p.H + j] = (float)b[0];
-        partial[(t * 2 + 1) * p.H + j] = (float)b[1];
-        s_d[0][c] = (float)b[2]; s_d[1][c] = (float)b[3];
+    {   // wavefront q finishes sum q: the scale's and the shift's shares of this time step go out, the two others to the second pass
+        const double total = norm_sum_partials<CW, NP>(red[wave], lane);
+        if (keeper) {
+            if (wave < 2) partial[(t * 2 + wave) * p.H + fj] = (float)total;
+            else s_d[wave - 2][fc] = (float)total;
+        }
     }
     __syncthreads();
     if (!live) return;
     const float dmean = s_d[0][c], dvar = s_d[1][c];
     const float bsz = (float)p.rows, bscale = 1.f / (float)p.rows;
-#pragma unroll 4
-    for (size_t r = rl; r < p.rows; r += kLanes) {
-        const size_t i = base + r * p.H + j;
-        float e = p.dy[i] * scale;
+    auto apply = [&](size_t r, float dy, float x) {
+        float e = dy * scale;
         e *= rc / vb;
-        e += dvar * ((p.x[i] - mean) / (bsz * vb));
+        e += dvar * ((x - mean) / (bsz * vb));
         e += dmean * bscale;
-        p.dx[i] = e;
+        p.dx[base + r * p.H + j] = e;
+    };
+#pragma unroll
+    for (int h = 0; h < kSeqHeld; ++h)
+        if (rl + (size_t)h * kLanes < p.rows) apply(rl + (size_t)h * kLanes, held_dy[h], held_x[h]);
+    for (size_t r = rl + (size_t)kSeqHeld * kLanes; r < p.rows; r += kLanes) {
+        const size_t i = base + r * p.H + j;
+        apply(r, p.dy[i], p.x[i]);
     }
 }
 

@@ -633,57 +633,6 @@ struct NormStepArgs {
 };
 constexpr int kNormBackThreads = 512;   // the backward pass keeps more per lane: 256 registers a lane instead of 128
 
-// the value of another lane of the 16-lane row, chosen by a data-parallel-primitive control word: a move inside the vector unit
-template <int CTRL>
-__device__ __forceinline__ double norm_dpp(double v)
-{
-    int lo = __double2loint(v), hi = __double2hiint(v);
-    lo = __builtin_amdgcn_mov_dpp(lo, CTRL, 0xf, 0xf, false);
-    hi = __builtin_amdgcn_mov_dpp(hi, CTRL, 0xf, 0xf, false);
-    return __hiloint2double(hi, lo);
-}
-// lane j of a 16-lane row takes the value of lane j - N (mod 16) of its row
-template <int N> __device__ __forceinline__ double norm_row_rotate(double v) { return norm_dpp<0x120 + N>(v); }
-// lane j takes the value of lane j ^ 1 resp. j ^ 2
-__device__ __forceinline__ double norm_quad_xor1(double v) { return norm_dpp<0xB1>(v); }
-__device__ __forceinline__ double norm_quad_xor2(double v) { return norm_dpp<0x4E>(v); }
-
-// A wavefront holds 64 / CW rows of the workgroup's CW columns (lane = CW * row + column).  With CW < 16 the lanes of each
-// 16-lane row that share a column add up in place: four partials a wavefront.  With CW == 16 a 16-lane row is one batch row and
-// the four of them add up across the wavefront: one partial.
-template <int CW> constexpr int kNormPartials = CW < 16 ? 4 : 1;
-template <int CW>
-__device__ __forceinline__ double norm_fold_partial(double v)
-{
-    if (CW <= 1) v += norm_row_rotate<1>(v);
-    if (CW <= 2) v += norm_row_rotate<2>(v);
-    if (CW <= 4) v += norm_row_rotate<4>(v);
-    if (CW <= 8) v += norm_row_rotate<8>(v);
-    if (CW == 16) { v += __shfl_xor(v, 16); v += __shfl_xor(v, 32); }
-    return v;
-}
-// which lanes hold a partial, and where it goes among the workgroup's NW * kNormPartials<CW>
-template <int CW> __device__ __forceinline__ bool norm_partial_holder(int lane) { return CW < 16 ? (lane & 15) < CW : lane < 16; }
-template <int CW> __device__ __forceinline__ int norm_partial_index(int wave, int lane) { return CW < 16 ? wave * 4 + (lane >> 4) : wave; }
-
-// The finishing wavefront adds up a column's NP partials with 64 / CW lanes a column (lane = column * lanes + j takes the
-// partials j, j + lanes, ...; the lanes of a column then add up inside their 16-lane row): every lane returns its column's total.
-template <int CW, int NP>
-__device__ __forceinline__ double norm_sum_partials(const double (&p)[NP][CW], int lane)
-{
-    constexpr int LPC = 64 / CW;
-    static_assert(LPC == 4 || LPC == 16, "a column's lanes are a quad or a 16-lane row");
-    static_assert(NP % LPC == 0, "every lane of a column takes the same number of partials");
-    const int column = lane / LPC, j = lane % LPC;
-    double v = 0.0;
-#pragma unroll
-    for (int w = 0; w < NP / LPC; ++w) v += p[w * LPC + j][column];
-    v += norm_quad_xor1(v);
-    v += norm_quad_xor2(v);
-    if (LPC == 16) { v += norm_row_rotate<4>(v); v += norm_row_rotate<8>(v); }
-    return v;
-}
-
 // st: the group's statistics at this time step, fields `field` floats apart; mean_avg_old, sigma_avg_old: the running averages as
 // they stood before this step (the caller asked for them early)
 __device__ __forceinline__ void norm_finish_statistics(float *st, unsigned field, unsigned col, double s1, double s2, size_t B, const NormHyper &hy, float mean_avg_old,

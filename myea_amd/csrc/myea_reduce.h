@@ -31,6 +31,71 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
+// ---- column sums inside a workgroup of (row lane, column) lanes ---------------------------------
+// For kernels in which a workgroup owns CW columns and all rows of a tensor: lane = CW * row lane + column, CW in {4, 16, 64},
+// so a wavefront holds 64 / CW row lanes of every column.  What each lane summed over its rows becomes the column's sum in
+// two stages.  Stage one runs in every wavefront and costs the LDS unit (which all wavefronts share) as little as possible:
+// with CW < 16 the lanes of a 16-lane row that share a column add up by row rotations inside the vector unit and the row's
+// first CW lanes write one partial each (four partials a wavefront); with CW == 16 the four 16-lane rows add up across the
+// wavefront (one partial); with CW == 64 a lane's value is the partial.  Stage two runs in ONE wavefront per quantity: its
+// lanes share out the column's partials, 64 / CW lanes a column, and add up inside their quad or 16-lane row.  Every sum is
+// taken in a fixed order: the same bits in every run.
+// the value of another lane of the 16-lane row, chosen by a data-parallel-primitive control word: a move inside the vector unit
+template <int CTRL>
+__device__ __forceinline__ double norm_dpp(double v)
+{
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_mov_dpp(lo, CTRL, 0xf, 0xf, false);
+    hi = __builtin_amdgcn_mov_dpp(hi, CTRL, 0xf, 0xf, false);
+    return __hiloint2double(hi, lo);
+}
+// lane j of a 16-lane row takes the value of lane j - N (mod 16) of its row
+template <int N> __device__ __forceinline__ double norm_row_rotate(double v) { return norm_dpp<0x120 + N>(v); }
+// lane j takes the value of lane j ^ 1 resp. j ^ 2
+__device__ __forceinline__ double norm_quad_xor1(double v) { return norm_dpp<0xB1>(v); }
+__device__ __forceinline__ double norm_quad_xor2(double v) { return norm_dpp<0x4E>(v); }
+
+template <int CW> constexpr int kNormPartials = CW < 16 ? 4 : 1;   // partials a wavefront leaves per column
+template <int CW>
+__device__ __forceinline__ double norm_fold_partial(double v)
+{
+    static_assert(CW == 1 || CW == 2 || CW == 4 || CW == 8 || CW == 16 || CW == 64, "columns per workgroup");
+    if (CW <= 1) v += norm_row_rotate<1>(v);
+    if (CW <= 2) v += norm_row_rotate<2>(v);
+    if (CW <= 4) v += norm_row_rotate<4>(v);
+    if (CW <= 8) v += norm_row_rotate<8>(v);
+    if (CW == 16) { v += __shfl_xor(v, 16); v += __shfl_xor(v, 32); }
+    return v;
+}
+// which lanes hold a partial, and where it goes among the workgroup's (wavefronts) * kNormPartials<CW>
+template <int CW> __device__ __forceinline__ bool norm_partial_holder(int lane) { return CW < 16 ? (lane & 15) < CW : (CW == 16 ? lane < 16 : true); }
+template <int CW> __device__ __forceinline__ int norm_partial_index(int wave, int lane) { return CW < 16 ? wave * 4 + (lane >> 4) : wave; }
+// The finishing wavefront's lanes: lane -> the column it works for, and whether it is the one that keeps the column's total
+template <int CW> __device__ __forceinline__ int norm_finish_column(int lane) { return CW >= 64 ? lane : lane / (64 / CW); }
+template <int CW> __device__ __forceinline__ bool norm_finish_keeper(int lane) { return CW >= 64 ? true : lane % (64 / CW) == 0; }
+// every lane of the finishing wavefront returns its column's total
+template <int CW, int NP>
+__device__ __forceinline__ double norm_sum_partials(const double (&p)[NP][CW], int lane)
+{
+    if (CW >= 64) {
+        double v = 0.0;
+#pragma unroll
+        for (int w = 0; w < NP; ++w) v += p[w][lane % CW];
+        return v;
+    }
+    constexpr int LPC = CW >= 64 ? 4 : 64 / CW;
+    static_assert(CW >= 64 || LPC == 4 || LPC == 16, "a column's lanes are a quad or a 16-lane row");
+    static_assert(CW >= 64 || NP % LPC == 0, "every lane of a column takes the same number of partials");
+    const int column = lane / LPC, j = lane % LPC;
+    double v = 0.0;
+#pragma unroll
+    for (int w = 0; w < NP / LPC; ++w) v += p[w * LPC + j][column % CW];
+    v += norm_quad_xor1(v);
+    v += norm_quad_xor2(v);
+    if (LPC == 16) { v += norm_row_rotate<4>(v); v += norm_row_rotate<8>(v); }
+    return v;
+}
+
 // ---- two-stage column reductions -----------------------------------------------------------------
 // Stage 1: grid (ceil(H/64), S); a workgroup is 64 columns x 4 row lanes and owns rows
 // [y*chunk, (y+1)*chunk).  It writes NV partial sums per column to partial[(y*NV + v)*H + col].
