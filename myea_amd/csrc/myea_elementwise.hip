@@ -1512,7 +1512,40 @@ __global__ __launch_bounds__(kBlock) void bn_backward_sequence_final_kernel(size
     dscale[j] += a; dshift[j] += b;
 }
 
-int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t T, size_t Bmax, float *scratch)
+// the same for one layer of a table of them: grid (ceil(widest H / 64), layers)
+__global__ __launch_bounds__(kBlock) void bn_share_fold_kernel(const BnFoldJob *__restrict__ jobs)
+{
+    __shared__ float red[2][kBlock / 64][64];
+    const BnFoldJob job = jobs[blockIdx.y];
+    if ((size_t)blockIdx.x * 64 >= job.H) return;
+    const int cl = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const size_t j = (size_t)blockIdx.x * 64 + cl, H = job.H, T = job.T;
+    float a = 0.f, b = 0.f;
+    if (j < H) {
+#pragma unroll 8
+        for (size_t k = q; k < T; k += kBlock / 64) {
+            const size_t t = T - 1 - k;
+            a += job.shares[(t * 2 + 0) * H + j]; b += job.shares[(t * 2 + 1) * H + j];
+        }
+    }
+    red[0][q][cl] = a; red[1][q][cl] = b;
+    __syncthreads();
+    if (q != 0 || j >= H) return;
+#pragma unroll
+    for (int r = 1; r < kBlock / 64; ++r) { a += red[0][r][cl]; b += red[1][r][cl]; }
+    job.dscale[j] += a; job.dshift[j] += b;
+}
+
+int launch_bn_share_folds(hipStream_t s, const BnFoldJob *jobs, size_t count, size_t widest)
+{
+    if (count == 0 || widest == 0) return MYEA_OK;
+    if (count > 65535) { set_last_error("bn_share_folds: %zu layers in one launch", count); return MYEA_E_INVALID; }
+    hipLaunchKernelGGL(bn_share_fold_kernel, dim3(grid_for(widest, 64), (unsigned)count), dim3(kBlock), 0, s, jobs);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t T, size_t Bmax, float *scratch, bool fold_now)
 {
     if (p.H == 0 || p.rows == 0 || T == 0) return MYEA_OK;
     if (p.rows > Bmax || T > 65535) { set_last_error("bn_backward_sequence: %zu rows of %zu, %zu time steps", p.rows, Bmax, T); return MYEA_E_INVALID; }
@@ -1524,6 +1557,7 @@ int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t
     MYEA_HIP_TRY(hipGetLastError());
     // (the shares are added by a launch of their own: a column block's last workgroup could add them itself, but the release of its
     // stores to the other XCDs' workgroups costs more than the launch - 38 against 9 + 8 us measured)
+    if (!fold_now) return MYEA_OK;
     hipLaunchKernelGGL(bn_backward_sequence_final_kernel, dim3(grid_for(p.H, 64)), dim3(kBlock), 0, s, p.H, T, scratch, p.dscale, p.dshift);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;

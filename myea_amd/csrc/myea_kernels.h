@@ -150,9 +150,14 @@ int launch_bn_backward(hipStream_t s, const BnBackwardParams &p, float *scratch 
 // plain batch normalisation only
 int launch_bn_backward_from_sums(hipStream_t s, const BnBackwardParams &p, const float *sums, size_t blocks);
 // every time step of a [T][Bmax][H] tensor in one launch (statistics per time step): p's tensors and per-time-step vectors are
-// those of time step 0; p.rows <= Bmax rows of each time step take part.  scratch: 2 * T * H floats
+// those of time step 0; p.rows <= Bmax rows of each time step take part.  shares: 2 * T * H floats, the scale's and the shift's
+// gradient of every time step; fold_now: a second launch adds them onto p.dscale / p.dshift, otherwise the caller does that
+// later (launch_bn_share_folds: the shares of many layers in one launch)
 int launch_bn_forward_sequence(hipStream_t s, const BnForwardParams &p, size_t T, size_t Bmax, int training);
-int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t T, size_t Bmax, float *scratch);
+int launch_bn_backward_sequence(hipStream_t s, const BnBackwardParams &p, size_t T, size_t Bmax, float *shares, bool fold_now);
+struct BnFoldJob { const float *shares; float *dscale, *dshift; unsigned H, T; };
+// jobs: device memory; widest: the largest H among them
+int launch_bn_share_folds(hipStream_t s, const BnFoldJob *jobs, size_t count, size_t widest);
 
 // output-layer delta + loss / accuracy accumulation
 struct ErrorParams {

@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "../../include/myea_hip.h"
+#include "myea_kernels.h"
 
 namespace myea {
 
@@ -95,6 +96,14 @@ struct Net {
     float *tmp1 = nullptr, *tmp2 = nullptr, *scratch = nullptr, *stage_in = nullptr, *stage_out = nullptr;
     float *dw_slabs = nullptr;   // split-K slabs of a fully-connected weight gradient whose M x N is small and k long
     size_t scratch_floats = 0, dw_slab_floats = 0;   // sizes of the two buffers above
+    // A sequence normalisation's backward launch leaves the scale's and the shift's gradient as shares per time step in the layer's
+    // slice of bn_shares; ONE launch at the end of the backward pass adds the shares of every such layer onto the gradient
+    // (flush_bn_shares).  bn_jobs: the table that launch reads, uploaded when the set of layers changes.
+    float *bn_shares = nullptr;
+    std::vector<size_t> bn_share_at;           // per layer: its slice's offset in floats, SIZE_MAX without one
+    BnFoldJob *bn_jobs = nullptr, *bn_jobs_staging = nullptr;   // device; pinned host
+    std::vector<BnFoldJob> bn_jobs_pending, bn_jobs_uploaded;
+    int flush_bn_shares();
     float *static_scratch = nullptr;   // this device's copy of the library's static scratch array (update_derivative_weight_no_alloc)
     double *loss_acc = nullptr;                  // 8 doubles, see ErrorParams::loss_acc
     // LSTM time loops as one resident launch (myea_lstm_resident.hip): barrier counters in device memory, and a pinned host

@@ -380,6 +380,20 @@ int Net::create(const myea_net_desc &desc)
     }
     MYEA_TRY(dev_alloc(&tmp1, T * B * max_h));
     MYEA_TRY(dev_alloc(&tmp2, T * B * max_h));
+    bn_share_at.assign(d.n_layers, SIZE_MAX);
+    if (T > 1) {   // a slice per normalised dense layer or block for the per-time-step shares of its scale / shift gradient
+        size_t need = 0, count = 0;
+        for (size_t li = 1; li < d.n_layers; ++li)
+            if (layer_uses_norm(d.layers[li]) && d.layers[li].type_layer != MYEA_LAYER_LSTM && L[li].NH) { bn_share_at[li] = need; need += (2 * T * L[li].NH + 63) / 64 * 64; ++count; }
+        if (count) {
+            MYEA_TRY(dev_alloc(&bn_shares, need));
+            void *q = nullptr;
+            MYEA_HIP_TRY(hipMalloc(&q, count * sizeof(BnFoldJob)));
+            bn_jobs = static_cast<BnFoldJob *>(q);
+            MYEA_HIP_TRY(hipHostMalloc(&q, count * sizeof(BnFoldJob), hipHostMallocDefault));
+            bn_jobs_staging = static_cast<BnFoldJob *>(q);
+        }
+    }
     {
         size_t need = 258 * max_h + 2048;
         if (2 * T * max_h > need) need = 2 * T * max_h;   // a sequence's normalisation: the scale / shift gradient shares per time step
@@ -435,6 +449,8 @@ Net::~Net()
     fr(resident_exchange);
     fr(gemm_pair_partials); fr(gemm_pair_tickets); fr(fault);
     if (resident_flag) (void)hipHostFree(resident_flag);
+    fr(bn_shares); fr(bn_jobs);
+    if (bn_jobs_staging) (void)hipHostFree(bn_jobs_staging);
     fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc); fr(index_stage); fr(dw_slabs);
     for (ProfEvent &e : pending) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
     for (ProfEvent &e : free_events) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
@@ -638,7 +654,7 @@ int Net::bn_backward_all(size_t li, size_t B, const float *x, const float *dy, f
     const myea_layer_desc &l = d.layers[li];
     DevLayer &o = L[li];
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size, H = o.NH;
-    if (T == 1 || !bn_sequence_allowed() || 2 * T * H > scratch_floats) {
+    if (T == 1 || !bn_sequence_allowed() || 2 * T * H > scratch_floats || bn_share_at[li] == SIZE_MAX) {
         for (size_t t = T; t-- > 0;) MYEA_TRY(bn_backward(li, t, B, x + t * Bmax * H, dy + t * Bmax * H, dx + t * Bmax * H));
         return MYEA_OK;
     }
@@ -649,8 +665,34 @@ int Net::bn_backward_all(size_t li, size_t B, const float *x, const float *dy, f
     p.dx = dx;
     p.renorm = l.type_normalization == MYEA_NORMALIZATION_BATCH_RENORMALIZATION;
     prof_begin(kProfNormalization);
-    const int rc = launch_bn_backward_sequence(stream, p, T, Bmax, scratch);
+    // the shares of the scale's and the shift's gradient stay in the layer's slice until the end of the pass: flush_bn_shares
+    float *shares = bn_shares + bn_share_at[li];
+    const int rc = launch_bn_backward_sequence(stream, p, T, Bmax, shares, false);
     prof_end((double)T * (double)B * (double)H * sizeof(float) * 3.0);
+    if (rc == MYEA_OK) bn_jobs_pending.push_back(BnFoldJob{shares, p.dscale, p.dshift, (unsigned)H, (unsigned)T});
+    return rc;
+}
+
+// The shares every sequence normalisation of this backward pass left are added onto the gradient: one launch for all layers.
+int Net::flush_bn_shares()
+{
+    if (bn_jobs_pending.empty()) return MYEA_OK;
+    const size_t count = bn_jobs_pending.size();
+    bool same = bn_jobs_uploaded.size() == count;
+    for (size_t i = 0; same && i < count; ++i) same = std::memcmp(&bn_jobs_pending[i], &bn_jobs_uploaded[i], sizeof(BnFoldJob)) == 0;
+    if (!same) {   // the first pass, or one over other layers than the last (another batch size): the table goes up again
+        MYEA_HIP_TRY(hipStreamSynchronize(stream));   // no earlier launch still reads the table
+        std::memcpy(bn_jobs_staging, bn_jobs_pending.data(), count * sizeof(BnFoldJob));
+        MYEA_HIP_TRY(hipMemcpyAsync(bn_jobs, bn_jobs_staging, count * sizeof(BnFoldJob), hipMemcpyHostToDevice, stream));
+        MYEA_HIP_TRY(hipStreamSynchronize(stream));   // the staging words are free again
+        bn_jobs_uploaded = bn_jobs_pending;
+    }
+    size_t widest = 0;
+    for (const BnFoldJob &j : bn_jobs_pending) widest = std::max(widest, (size_t)j.H);
+    bn_jobs_pending.clear();
+    prof_begin(kProfNormalization);
+    const int rc = launch_bn_share_folds(stream, bn_jobs, count, widest);
+    prof_end(0.0);
     return rc;
 }
 
@@ -1303,6 +1345,7 @@ int Net::backward_pass(size_t B)
     if (B == 0 || B > d.batch_size) { set_last_error("Backward_Pass: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
     if (state != MYEA_STATE_TRAINING) { set_last_error("Backward_Pass: can not back propagate gradient in inference mode"); return MYEA_E_STATE; }
     for (DevLayer &o : L) o.bias_partial_rows = 0;   // set again by the contractions that leave column sums with a layer's errors
+    bn_jobs_pending.clear();
     // the walk of FF__Backward_Pass_Batch: from a consumer gi to its producer li = previous_connected_layers[0]; once a
     // residual layer's block is done it resumes from the residual layer itself (:117-120)
     for (size_t gi = d.n_layers - 1; gi != 1; --gi) {
@@ -1333,7 +1376,7 @@ int Net::backward_pass(size_t B)
             gi = li + 1;
         }
     }
-    return MYEA_OK;
+    return flush_bn_shares();
 }
 
 // ---- Update_Derivative_Weight -----------------------------------------------------------------------------------
