@@ -141,6 +141,7 @@ __global__ __launch_bounds__(kIndRnnLanes) void ind_rnn_backward_kernel(IndRnnPa
         auto walk = [&](auto activation) {
             const int act = activation;
             float next = 0.f;
+            double du = 0.0;   // this (example, unit)'s share of the self weight's gradient: the sum over t >= 1 of AF[t-1] dAF[t]
             for (size_t done = 0; done < p.T; done += kIndRnnChunk) {   // time steps T-1-done, T-2-done, ...
                 const int m = (int)(p.T - done < (size_t)kIndRnnChunk ? p.T - done : (size_t)kIndRnnChunk);
                 const size_t top = p.T - 1 - done;
@@ -154,6 +155,7 @@ __global__ __launch_bounds__(kIndRnnLanes) void ind_rnn_backward_kernel(IndRnnPa
                     const int sn = s + 1 < m ? s + 1 : s;
                     const float pre_next = stage.at(0, sn), val_next = stage.at(1, sn), dy_next = stage.at(2, sn);
                     const size_t t = top - s;
+                    if (t + 1 != p.T) du += (double)val * (double)next;   // next: dAF[t+1]
                     const float daf = af_derive(act, pre, steep, val);
                     const float e = __fmul_rn(dy, daf);
                     const float r = (t + 1 == p.T) ? e : __fadd_rn(e, __fmul_rn(__fmul_rn(u, daf), next));
@@ -162,6 +164,7 @@ __global__ __launch_bounds__(kIndRnnLanes) void ind_rnn_backward_kernel(IndRnnPa
                     pre = pre_next; val = val_next; dy = dy_next;
                 }
             }
+            if (p.du_rows) p.du_rows[i] = (float)du;
         };
         if (p.unit_act) walk(p.unit_act[j]); else af_with(p.act, walk);
     }
@@ -1217,6 +1220,25 @@ int launch_ind_rnn_self_weight_gradient(hipStream_t s, size_t T, size_t B, size_
     return MYEA_OK;
 }
 
+// grid (ceil(longest / 256), ranges)
+__global__ __launch_bounds__(kBlock) void clip_ranges_kernel(const ClipRange *__restrict__ ranges, float *w)
+{
+    const ClipRange r = ranges[blockIdx.y];
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= r.count) return;
+    const float v = w[r.first + i];
+    w[r.first + i] = v < r.lo ? r.lo : (v > r.hi ? r.hi : v);
+}
+
+int launch_clip_ranges(hipStream_t s, const ClipRange *ranges, size_t count, size_t longest, float *w)
+{
+    if (count == 0 || longest == 0) return MYEA_OK;
+    if (count > 65535) { set_last_error("clip_ranges: %zu ranges in one launch", count); return MYEA_E_INVALID; }
+    hipLaunchKernelGGL(clip_ranges_kernel, dim3(grid_for(longest, kBlock), (unsigned)count), dim3(kBlock), 0, s, ranges, w);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
 int launch_clip_range(hipStream_t s, size_t n, float *w, float lo, float hi)
 {
     if (n == 0) return MYEA_OK;
@@ -1753,10 +1775,41 @@ __global__ __launch_bounds__(kBlock) void slab_sum_add_scalar_kernel(size_t n, i
     dst[i] += v;
 }
 
-int launch_slab_sum_add(hipStream_t s, size_t n, int nslab, const float *slabs, float *dst)
+// grid (ceil(widest n / 64), jobs)
+__global__ __launch_bounds__(kBlock) void slab_fold_jobs_kernel(const SlabFoldJob *__restrict__ jobs)
+{
+    __shared__ float red[kBlock / 64][64];
+    const SlabFoldJob job = jobs[blockIdx.y];
+    if ((size_t)blockIdx.x * 64 >= job.n) return;
+    const int cl = threadIdx.x & 63, q = threadIdx.x >> 6;
+    const size_t i = (size_t)blockIdx.x * 64 + cl, n = job.n;
+    float v = 0.f;
+    if (i < n) {
+#pragma unroll 8
+        for (unsigned s = q; s < job.nslab; s += kBlock / 64) v += job.slabs[(size_t)s * n + i];
+    }
+    red[q][cl] = v;
+    __syncthreads();
+    if (q != 0 || i >= n) return;
+#pragma unroll
+    for (int r = 1; r < kBlock / 64; ++r) v += red[r][cl];
+    job.dst[i] += v;
+}
+
+int launch_slab_fold_jobs(hipStream_t s, const SlabFoldJob *jobs, size_t count, size_t widest)
+{
+    if (count == 0 || widest == 0) return MYEA_OK;
+    if (count > 65535) { set_last_error("slab_fold_jobs: %zu sums in one launch", count); return MYEA_E_INVALID; }
+    hipLaunchKernelGGL(slab_fold_jobs_kernel, dim3(grid_for(widest, 64), (unsigned)count), dim3(kBlock), 0, s, jobs);
+    MYEA_HIP_TRY(hipGetLastError());
+    return MYEA_OK;
+}
+
+// value_by_value: the value-by-value form (and its order of additions) whatever the alignment
+int launch_slab_sum_add(hipStream_t s, size_t n, int nslab, const float *slabs, float *dst, bool value_by_value)
 {
     if (n == 0 || nslab <= 0) return MYEA_OK;
-    if ((n & 3) || (reinterpret_cast<uintptr_t>(slabs) & 15u) || (reinterpret_cast<uintptr_t>(dst) & 15u))
+    if (value_by_value || (n & 3) || (reinterpret_cast<uintptr_t>(slabs) & 15u) || (reinterpret_cast<uintptr_t>(dst) & 15u))
         hipLaunchKernelGGL(slab_sum_add_scalar_kernel, dim3(grid_for(n, 64)), dim3(kBlock), 0, s, n, nslab, slabs, dst);
     else
         hipLaunchKernelGGL(slab_sum_add_kernel, dim3(grid_for(n / 4, kBlock, 8192)), dim3(kBlock), 0, s, n, nslab, slabs, dst);

@@ -207,12 +207,16 @@ struct IndRnnParams {
     const float *colscale;     // forward: optional dropout multiplier [T][H] applied in place on the activations
     const float *dy;           // backward: delta of the layer's activations
     float *dafs;               // backward: delta of the pre-activations (the recurrence runs through it)
+    float *du_rows;            // backward, optional: [B][H], the sum over t >= 1 of AF[t-1] dAF[t] of every (example, unit)
 };
 int launch_ind_rnn_forward(hipStream_t s, const IndRnnParams &p);
 int launch_ind_rnn_backward(hipStream_t s, const IndRnnParams &p);
 // du[j] += sum over t >= 1 and the batch of AF[t-1] dAF[t]; scratch: 64 * H floats
 int launch_ind_rnn_self_weight_gradient(hipStream_t s, size_t T, size_t B, size_t Bmax, size_t H, const float *afs, const float *dafs, float *du, float *scratch);
 int launch_clip_range(hipStream_t s, size_t n, float *w, float lo, float hi);
+// the same for a table of ranges of one vector in one launch (ranges: device memory; longest: the largest count among them)
+struct ClipRange { unsigned long long first; unsigned count; float lo, hi; };
+int launch_clip_ranges(hipStream_t s, const ClipRange *ranges, size_t count, size_t longest, float *w);
 
 // [B][T][W] (example rows) -> [T][Bmax][W]
 int launch_scatter_time_major(hipStream_t s, size_t B, size_t T, size_t W, size_t Bmax, const float *src, float *dst);
@@ -249,7 +253,11 @@ int launch_pool_forward(hipStream_t s, const PoolParams &p, const float *x, floa
 // dx [rows][In] <- dy [rows][H] (overwrites dx)
 int launch_pool_backward(hipStream_t s, const PoolParams &p, const float *dy, const unsigned *index, float *dx);
 // dst[0..n) += sum over the nslab slabs of n floats each, in slab order (n % 4 == 0, 16-byte aligned)
-int launch_slab_sum_add(hipStream_t s, size_t n, int nslab, const float *slabs, float *dst);
+int launch_slab_sum_add(hipStream_t s, size_t n, int nslab, const float *slabs, float *dst, bool value_by_value = false);
+// the same for a table of such sums in one launch (jobs: device memory; widest: the largest n among them); every sum in the
+// order of the value-by-value form: four lanes a value, lane q the slabs q, q + 4, ..., the lanes' sums added in lane order
+struct SlabFoldJob { const float *slabs; float *dst; unsigned n, nslab; };
+int launch_slab_fold_jobs(hipStream_t s, const SlabFoldJob *jobs, size_t count, size_t widest);
 
 // ---- fused LSTM time step (one cell per block, C % 32 == 0) ---------------------------------------------------
 // all tensors are the rows of ONE time step: [B][C] (stride C) or [B][4C] gate rows z | i | f | o (stride 4C)

@@ -33,6 +33,10 @@ struct DevLayer {
     // bias_partial_batch examples, 0 = the errors were written some other way
     float *bias_partials = nullptr;
     size_t bias_partial_rows = 0, bias_partial_batch = 0;
+    // an independently recurrent layer: [Bmax][recurrent units], every example's share of the self weights' gradient (the sum over
+    // the time steps of AF[t-1] dAF[t]), left by the backward time loop for du_rows_batch examples (0: not left in this pass)
+    float *du_rows = nullptr;
+    size_t du_rows_batch = 0;
     // a batch-normalised dense layer: [ceil(Bmax / 32)][2][H] column sums a contraction leaves for the normalisation's forward
     // (sum of x, of x * x) and backward pass (sum of dy * hats, of dy); consumed by the launch that follows it
     float *norm_partials = nullptr;
@@ -104,6 +108,19 @@ struct Net {
     BnFoldJob *bn_jobs = nullptr, *bn_jobs_staging = nullptr;   // device; pinned host
     std::vector<BnFoldJob> bn_jobs_pending, bn_jobs_uploaded;
     int flush_bn_shares();
+    // The same for the weight gradients of narrow layers (narrow_dw_slabs): a layer's slabs stay in its slice of narrow_slabs
+    // until ONE launch at the end of Update_Derivative_Weight adds every layer's onto the gradient (flush_slab_folds).
+    float *narrow_slabs = nullptr;
+    size_t narrow_slab_floats = 0;
+    std::vector<size_t> narrow_slab_at;        // per layer, SIZE_MAX without a slice
+    SlabFoldJob *fold_jobs = nullptr, *fold_jobs_staging = nullptr;   // device; pinned host
+    std::vector<SlabFoldJob> fold_pending, fold_uploaded;
+    int flush_slab_folds();
+    // the bounds of the independently recurrent layers' self weights, clipped behind every update in one launch; built at the first update
+    ClipRange *clip_ranges = nullptr;
+    size_t n_clip_ranges = 0, longest_clip_range = 0;
+    bool clip_ranges_built = false;
+    bool defer_folds = true;   // false: every layer's slabs are added right behind its contraction (a call that may not wait for the stream)
     float *static_scratch = nullptr;   // this device's copy of the library's static scratch array (update_derivative_weight_no_alloc)
     double *loss_acc = nullptr;                  // 8 doubles, see ErrorParams::loss_acc
     // LSTM time loops as one resident launch (myea_lstm_resident.hip): barrier counters in device memory, and a pinned host

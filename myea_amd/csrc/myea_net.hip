@@ -330,6 +330,7 @@ int Net::create(const myea_net_desc &desc)
             const size_t su = o.group ? sa : sz;     // inside a block the recurrent units sit on the input side
             MYEA_TRY(dev_alloc(&o.pre_afs, su));
             MYEA_HIP_TRY(hipMemset(o.pre_afs, 0, su * sizeof(float)));
+            if (T > 1) MYEA_TRY(dev_alloc(&o.du_rows, su / T));   // [Bmax][recurrent units]
             // the delta of the pre-activations IS the neuron errors unless a normalisation sits between the two; a block member
             // always keeps its own (what it hands to the member before it may be changed by that member afterwards)
             if (o.group || (layer_uses_norm(l) && l.use_layer_normalization_before_activation)) {
@@ -410,6 +411,24 @@ int Net::create(const myea_net_desc &desc)
         }
         if (need) MYEA_TRY(dev_alloc(&dw_slabs, need));
         dw_slab_floats = need;
+        // the narrow ones among them keep their slabs until the end of the call: a slice each
+        narrow_slab_at.assign(d.n_layers, SIZE_MAX);
+        size_t pool = 0, count = 0;
+        for (size_t li = 1; li < d.n_layers; ++li) {
+            if (!layer_is_dense(d.layers[li])) continue;
+            const int slabs = narrow_dw_slabs(L[li].H, L[li].In, T * B);
+            if (slabs > 0) { narrow_slab_at[li] = pool; pool += ((size_t)slabs * L[li].H * L[li].In + 63) / 64 * 64; ++count; }
+            if (L[li].du_rows) ++count;   // the shares of an independently recurrent layer's self weights go through the same table
+        }
+        narrow_slab_floats = pool;
+        if (count) {
+            if (pool) MYEA_TRY(dev_alloc(&narrow_slabs, pool));
+            void *q = nullptr;
+            MYEA_HIP_TRY(hipMalloc(&q, count * sizeof(SlabFoldJob)));
+            fold_jobs = static_cast<SlabFoldJob *>(q);
+            MYEA_HIP_TRY(hipHostMalloc(&q, count * sizeof(SlabFoldJob), hipHostMallocDefault));
+            fold_jobs_staging = static_cast<SlabFoldJob *>(q);
+        }
     }
     MYEA_TRY(static_scratch_address(&static_scratch));   // set-up: this device's address of the static array
     MYEA_TRY(dev_alloc(&stage_in, T * B * L[0].H));
@@ -441,7 +460,7 @@ Net::~Net()
     fr(seg_first); fr(seg_len);
     fr(masks); fr(zoneout_masks);
     for (DevLayer &o : L) {
-        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.bias_partials); fr(o.norm_partials); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index); fr(o.pre_afs); fr(o.dafs_own); fr(o.noise);
+        fr(o.summations); fr(o.values); fr(o.hats); fr(o.normalizes); fr(o.neuron_errors); fr(o.in_errors); fr(o.bias_partials); fr(o.norm_partials); fr(o.colscale); fr(o.unit_act); fr(o.unit_steep); fr(o.pool_index); fr(o.pre_afs); fr(o.dafs_own); fr(o.du_rows); fr(o.noise);
         fr(o.means); fr(o.variances); fr(o.means_averages); fr(o.variances_averages); fr(o.r_corrections); fr(o.d_corrections);
         lstm_destroy_layer(o);
     }
@@ -449,7 +468,8 @@ Net::~Net()
     fr(resident_exchange);
     fr(gemm_pair_partials); fr(gemm_pair_tickets); fr(fault);
     if (resident_flag) (void)hipHostFree(resident_flag);
-    fr(bn_shares); fr(bn_jobs);
+    fr(bn_shares); fr(bn_jobs); fr(narrow_slabs); fr(fold_jobs); fr(clip_ranges);
+    if (fold_jobs_staging) (void)hipHostFree(fold_jobs_staging);
     if (bn_jobs_staging) (void)hipHostFree(bn_jobs_staging);
     fr(tmp1); fr(tmp2); fr(scratch); fr(stage_in); fr(stage_out); fr(loss_acc); fr(index_stage); fr(dw_slabs);
     for (ProfEvent &e : pending) { (void)hipEventDestroy(e.start); (void)hipEventDestroy(e.stop); }
@@ -670,6 +690,29 @@ int Net::bn_backward_all(size_t li, size_t B, const float *x, const float *dy, f
     const int rc = launch_bn_backward_sequence(stream, p, T, Bmax, shares, false);
     prof_end((double)T * (double)B * (double)H * sizeof(float) * 3.0);
     if (rc == MYEA_OK) bn_jobs_pending.push_back(BnFoldJob{shares, p.dscale, p.dshift, (unsigned)H, (unsigned)T});
+    return rc;
+}
+
+// The slabs the narrow layers' weight gradients of this call left are added onto the gradient: one launch for all layers.
+int Net::flush_slab_folds()
+{
+    if (fold_pending.empty()) return MYEA_OK;
+    const size_t count = fold_pending.size();
+    bool same = fold_uploaded.size() == count;
+    for (size_t i = 0; same && i < count; ++i) same = std::memcmp(&fold_pending[i], &fold_uploaded[i], sizeof(SlabFoldJob)) == 0;
+    if (!same) {   // the first call, or one over other layers or buffers than the last: the table goes up again
+        MYEA_HIP_TRY(hipStreamSynchronize(stream));   // no earlier launch still reads the table
+        std::memcpy(fold_jobs_staging, fold_pending.data(), count * sizeof(SlabFoldJob));
+        MYEA_HIP_TRY(hipMemcpyAsync(fold_jobs, fold_jobs_staging, count * sizeof(SlabFoldJob), hipMemcpyHostToDevice, stream));
+        MYEA_HIP_TRY(hipStreamSynchronize(stream));   // the staging words are free again
+        fold_uploaded = fold_pending;
+    }
+    size_t widest = 0;
+    for (const SlabFoldJob &j : fold_pending) widest = std::max(widest, (size_t)j.n);
+    fold_pending.clear();
+    prof_begin(2);
+    const int rc = launch_slab_fold_jobs(stream, fold_jobs, count, widest);
+    prof_end(0.0);
     return rc;
 }
 
@@ -1182,7 +1225,9 @@ int Net::backward_into_layer(size_t li, size_t B)
         p.pre_afs = o.pre_afs; p.afs = o.values;
         p.dy = (norm && !before) ? tmp2 : tmp1;
         p.dafs = o.dafs_own ? o.dafs_own : o.neuron_errors;
+        p.du_rows = o.du_rows;
         MYEA_TRY(launch_ind_rnn_backward(stream, p));
+        o.du_rows_batch = o.du_rows ? B : 0;
         if (norm && before) MYEA_TRY(bn_backward_all(li, B, o.summations, o.dafs_own, o.neuron_errors));
     }
     return MYEA_OK;
@@ -1297,7 +1342,9 @@ int Net::backward_residual_block(size_t ri, size_t B)
             p.act = (int)l.type_activation_function; p.steep = l.activation_steepness; p.unit_act = o.unit_act; p.unit_steep = o.unit_steep;
             p.pre_afs = o.pre_afs; p.afs = o.values;
             p.dy = tmp1; p.dafs = o.dafs_own;
+            p.du_rows = o.du_rows;
             MYEA_TRY(launch_ind_rnn_backward(stream, p));
+            o.du_rows_batch = o.du_rows ? B : 0;
             if (norm) MYEA_TRY(bn_backward_all(m, B, prev_all, o.dafs_own, dst_all));
             else MYEA_HIP_TRY(hipMemcpyAsync(dst_all, o.dafs_own, T * Bmax * In * sizeof(float), hipMemcpyDeviceToDevice, stream));
         } else if (norm) {
@@ -1344,7 +1391,7 @@ int Net::backward_pass(size_t B)
 {
     if (B == 0 || B > d.batch_size) { set_last_error("Backward_Pass: batch size (%zu) > maximum batch size (%u)", B, d.batch_size); return MYEA_E_BATCH; }
     if (state != MYEA_STATE_TRAINING) { set_last_error("Backward_Pass: can not back propagate gradient in inference mode"); return MYEA_E_STATE; }
-    for (DevLayer &o : L) o.bias_partial_rows = 0;   // set again by the contractions that leave column sums with a layer's errors
+    for (DevLayer &o : L) { o.bias_partial_rows = 0; o.du_rows_batch = 0; }   // set again by the launches that leave such sums
     bn_jobs_pending.clear();
     // the walk of FF__Backward_Pass_Batch: from a consumer gi to its producer li = previous_connected_layers[0]; once a
     // residual layer's block is done it resumes from the residual layer itself (:117-120)
@@ -1450,9 +1497,13 @@ int Net::update_derivative_weight_contraction(size_t li, size_t B)
         if (slabs > 1) { g.C = dw_slabs; g.accumulate = 0; g.c_is_zero = 0; g.split_k = slabs; g.split_k_slab = (long)(H * In); }
         if (li < dw_zero.size()) dw_zero[li] = 0;   // from here on the slice holds this product, stored or added from the slabs
         prof_begin(2);
-        if (narrow > 0) { slabs = narrow; MYEA_TRY(launch_narrow_dw(stream, g.A, g.B, dw_slabs, H, In, rows)); }
+        // a narrow layer over all of its rows: the slabs wait in the layer's slice for the one launch that adds every layer's
+        const bool later = defer_folds && narrow > 0 && chunks == 1 && narrow_slabs && narrow_slab_at[li] != SIZE_MAX;
+        float *const slabs_at = later ? narrow_slabs + narrow_slab_at[li] : dw_slabs;
+        if (narrow > 0) { slabs = narrow; MYEA_TRY(launch_narrow_dw(stream, g.A, g.B, slabs_at, H, In, rows)); }
         else MYEA_TRY(launch_gemm(stream, g));
-        if (slabs > 1 || narrow > 0) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index));
+        if (later) fold_pending.push_back(SlabFoldJob{slabs_at, gradient + l.first_connection_index, (unsigned)(H * In), (unsigned)slabs});
+        else if (slabs > 1 || narrow > 0) MYEA_TRY(launch_slab_sum_add(stream, H * In, slabs, dw_slabs, gradient + l.first_connection_index, narrow > 0));
         prof_end(2.0 * (double)rows * (double)H * (double)In);
     }
 
@@ -1482,6 +1533,7 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
     const size_t T = d.number_recurrent_depth, Bmax = d.batch_size;
     const bool per_t = T > 1 && B != Bmax;
     const size_t chunks = per_t ? T : 1, rows = per_t ? B : (T > 1 ? T * B : B);
+    fold_pending.clear();
     // The column reductions (biases, LSTM peepholes, self weights of independently recurrent layers) read deltas that
     // are complete before this call and write gradient slots no contraction touches; slots shared between layers (the
     // LSTM bias addressing reaches into the next layers' biases) are added to in the layers' order, on one stream.
@@ -1503,16 +1555,33 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
                     }
                 }
             // the self weights: as many as the layer has recurrent units - its width, a block member's fan-in, none for a block's first member
-            if (layer_is_ind_rnn(l) && o.group != 1)
-                MYEA_TRY(launch_ind_rnn_self_weight_gradient(stream, T, B, Bmax, o.group ? o.AH : o.H, o.values, o.dafs_own ? o.dafs_own : o.neuron_errors,
-                                                             gradient + l.first_connection_index + o.H * o.In, scratch));
+            if (layer_is_ind_rnn(l) && o.group != 1) {
+                const size_t units = o.group ? o.AH : o.H;
+                float *du = gradient + l.first_connection_index + o.H * o.In;
+                // the backward time loop left every example's share: they are added with the narrow layers' slabs, one launch for all
+                if (defer_folds && fold_jobs && o.du_rows && o.du_rows_batch == B && T > 1) fold_pending.push_back(SlabFoldJob{o.du_rows, du, (unsigned)units, (unsigned)B});
+                else MYEA_TRY(launch_ind_rnn_self_weight_gradient(stream, T, B, Bmax, units, o.values, o.dafs_own ? o.dafs_own : o.neuron_errors, du, scratch));
+            }
         }
         return MYEA_OK;
     };
-    auto contractions = [&]() -> int {
+    // alternate: narrow layers, whose slabs wait in slices of their own, take turns on the two streams - each is a launch of a few
+    // dozen workgroups and a chain of them on one stream leaves most of the device idle
+    auto contractions = [&](bool alternate) -> int {
+        bool on_side = false;
         for (size_t li = first; li < end; ++li) {
             const bool done_before = li < dw_done.size() && dw_done[li];
-            MYEA_TRY(update_derivative_weight_contraction(li, B));
+            const bool own_slice = alternate && !done_before && chunks == 1 && defer_folds && narrow_slabs && li < narrow_slab_at.size() &&
+                                   narrow_slab_at[li] != SIZE_MAX && layer_is_dense(d.layers[li]) && narrow_dw_slabs(L[li].H, L[li].In, rows) > 0;
+            if (own_slice && on_side) {
+                std::swap(stream, side_stream);
+                const int rc = update_derivative_weight_contraction(li, B);
+                std::swap(stream, side_stream);
+                MYEA_TRY(rc);
+            } else {
+                MYEA_TRY(update_derivative_weight_contraction(li, B));
+            }
+            if (own_slice) on_side = !on_side;
             // the combined call: every delta has been handed down by now, so the layer's weights may take their step beside the
             // contractions of the layers that follow
             if (early_update && !done_before) MYEA_TRY(early_update_layer(li));
@@ -1524,21 +1593,30 @@ int Net::update_derivative_weight(size_t B, size_t first, size_t end)
     if (any_lstm || !side_stream) {
         // beside the split-K contractions of LSTM layers the long reductions over T x batch rows were measured to cost
         // more than they hide: one stream, contractions first
-        MYEA_TRY(contractions());
-        return reductions();
-    }
-    {   // memory-bound reductions on the side stream beside the matrix-pipe-bound contractions
-        SideStreamScope side(*this);
+        MYEA_TRY(contractions(false));
         MYEA_TRY(reductions());
+        return flush_slab_folds();
     }
-    MYEA_TRY(contractions());
-    return side_stream_join();
+    // memory-bound reductions on the side stream beside the matrix-pipe-bound contractions, and every other narrow contraction
+    MYEA_HIP_TRY(hipEventRecord(fork_event, stream));
+    MYEA_HIP_TRY(hipStreamWaitEvent(side_stream, fork_event, 0));
+    std::swap(stream, side_stream);
+    int rc = reductions();
+    std::swap(stream, side_stream);
+    if (rc == MYEA_OK) rc = contractions(true);
+    const hipError_t e = hipEventRecord(join_event, side_stream);   // the main stream goes on behind the side stream, whatever else happened
+    const int joined = e == hipSuccess ? side_stream_join() : MYEA_E_DEVICE;
+    if (e != hipSuccess && rc == MYEA_OK) set_last_error("hipEventRecord: %s", hipGetErrorString(e));
+    MYEA_TRY(rc);
+    MYEA_TRY(joined);
+    return flush_slab_folds();
 }
 
 // Update_Derivative_Weight without any buffer of the library's own behind its kernels: the column reductions' partial
 // sums, the split-K slabs of narrow fully-connected layers and the packed weight-gradient slabs of the LSTM layers are
-// carved out of the static device array (in this order, each piece a multiple of 64 floats).  Same launches, same
-// results as update_derivative_weight.  Nothing is allocated or freed.  Every piece is written before it is read within
+// carved out of the static device array (in this order, each piece a multiple of 64 floats).  Same results as
+// update_derivative_weight (the same additions in the same order; a narrow layer's slabs are added by a launch of the layer's own
+// instead of one launch for all layers).  Nothing is allocated or freed, and the call never waits for the stream.  Every piece is written before it is read within
 // the call, so what an earlier call left in the array does not matter; calls that overlap on one device (two networks
 // on two streams) would share the array and race.
 int Net::update_derivative_weight_no_alloc(size_t B, size_t first, size_t end)
@@ -1556,12 +1634,13 @@ int Net::update_derivative_weight_no_alloc(size_t B, size_t first, size_t end)
     scratch = at; at += round_up(scratch_floats);
     if (own_slabs) dw_slabs = at;
     at += round_up(dw_slab_floats);
+    defer_folds = false;   // a narrow layer's slabs are added right behind its contraction: no table to upload, no wait for the stream
     lstm_bind_gradient_slabs(at);
     const bool was_profiling = profiling;
     profiling = false;   // the profiling taps create events on demand
     const int rc = update_derivative_weight(B, first, end);
     profiling = was_profiling;
-    scratch = own_scratch; dw_slabs = own_slabs;
+    scratch = own_scratch; dw_slabs = own_slabs; defer_folds = true;
     lstm_bind_gradient_slabs(nullptr);
     return rc;
 }
@@ -1802,12 +1881,26 @@ int Net::update_finish()
     }
     // Update_Weight_Regularization__Constraint_Recurrent_Weight (NN/Neural_Network__Regularization__Constraint_Recurrent_Weight.cpp:
     // 289-333): the self weights of the independently recurrent hidden layers clipped to their bounds
-    for (size_t li = 1; li + 1 < d.n_layers; ++li) {
-        const myea_layer_desc &l = d.layers[li];
-        if (!layer_is_ind_rnn(l) || L[li].group == 1 || (l.constraint_recurrent_weight_lower_bound == 0.f && l.constraint_recurrent_weight_upper_bound == 0.f)) continue;
-        MYEA_TRY(launch_clip_range(stream, L[li].group ? L[li].AH : L[li].H, parameters + l.first_connection_index + L[li].H * L[li].In,
-                                   l.constraint_recurrent_weight_lower_bound, l.constraint_recurrent_weight_upper_bound));
+    if (!clip_ranges_built) {   // the layers' bounds are part of the description: one table for the network's life
+        std::vector<ClipRange> ranges;
+        for (size_t li = 1; li + 1 < d.n_layers; ++li) {
+            const myea_layer_desc &l = d.layers[li];
+            if (!layer_is_ind_rnn(l) || L[li].group == 1 || (l.constraint_recurrent_weight_lower_bound == 0.f && l.constraint_recurrent_weight_upper_bound == 0.f)) continue;
+            const size_t units = L[li].group ? L[li].AH : L[li].H;
+            ranges.push_back(ClipRange{(unsigned long long)(l.first_connection_index + L[li].H * L[li].In), (unsigned)units,
+                                       l.constraint_recurrent_weight_lower_bound, l.constraint_recurrent_weight_upper_bound});
+            longest_clip_range = std::max(longest_clip_range, units);
+        }
+        n_clip_ranges = ranges.size();
+        if (n_clip_ranges) {
+            void *q = nullptr;
+            MYEA_HIP_TRY(hipMalloc(&q, n_clip_ranges * sizeof(ClipRange)));
+            clip_ranges = static_cast<ClipRange *>(q);
+            MYEA_HIP_TRY(hipMemcpy(clip_ranges, ranges.data(), n_clip_ranges * sizeof(ClipRange), hipMemcpyHostToDevice));
+        }
+        clip_ranges_built = true;
     }
+    MYEA_TRY(launch_clip_ranges(stream, clip_ranges, n_clip_ranges, longest_clip_range, parameters));
     return lstm_parameters_changed();  // refresh the packed gate matrices
 }
 
