@@ -24,6 +24,12 @@ CASES = [
     ("between-lstm-layers", [dict(units=8), dict(type="lstm", units=12), ind(20, "RELU"), dict(type="lstm", units=6), dict(units=12, activation="LINEAR")], 5, 6, 6),
     ("single-time-step", [dict(units=12), ind(16, "RELU"), dict(units=5, activation="LINEAR")], 1, 4, 4),
     ("wide", [dict(units=64), ind(512, "RELU"), ind(512, "RELU"), dict(units=10, activation="SOFTMAX")], 12, 64, 64),
+    # layers of at most 32 units over 640 rows: their weight gradients take the kernel that feeds the matrix unit from memory,
+    # the self weights' gradient comes from the shares the backward time loop leaves; T > 32: two rounds of staged operands
+    ("narrow-long", [dict(units=28), ind(31, "ISRLU", normalization="BATCH_NORMALIZATION", norm_before=True), ind(30, "ISRLU"), ind(17, "TANH"),
+                     dict(units=10, activation="SOFTMAX")], 8, 80, 80),
+    ("narrow-long-partial-batch", [dict(units=28), ind(31, "ISRLU"), ind(32, "RELU"), dict(units=10, activation="SOFTMAX")], 8, 70, 80),
+    ("narrow-many-steps", [dict(units=9), ind(24, "ISRLU"), ind(11, "SIGMOID"), dict(units=3, activation="LINEAR")], 40, 16, 16),
 ]
 
 
