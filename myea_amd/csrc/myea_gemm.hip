@@ -641,6 +641,43 @@ int launch_layout_scalar(hipStream_t stream, const GemmDev &d, bool a_kc, bool b
 }
 
 
+// ---- a narrow product ---------------------------------------------------------------------------------------------------
+// C [M][N] = A B with N <= 32 and K <= 64 - a layer of an independently recurrent stack over T x batch rows, forward or backward.
+// The tiled kernel spends such a launch on its set-up, its predicated scalar loads and its stages (rows of 31 floats are no
+// 16-byte multiples): a few microseconds of instructions fetched to be run once.  Here a wavefront owns 32 rows of C: the
+// lane's operands of v_mfma_f32_32x32x2f32 are asked for straight from memory, all of a round of 32 k's together (A: lane l
+// takes row l % 32 at k + l / 32; B: column l % 32), then the round's 16 matrix instructions; no LDS, one round or two.  The
+// accumulator has the layout of the tiled kernel's, so its epilogue (store_tile_kind) finishes the tile: every kind of
+// epilogue, the same arithmetic per element.
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kThreads) void narrow_gemm_kernel(GemmDev p)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lane32 = lane & 31, half = lane >> 5;
+    const int m0 = (int)blockIdx.x * 128, row = m0 + wave * 32 + lane32;
+    const bool in_m = row < p.M, in_n = lane32 < p.N;
+    f32x16 acc[1][1];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[0][0][r] = 0.f;
+    const float *a_at = A_KC ? p.A + (long)row * p.lda + half : p.A + (long)half * p.lda + row;
+    const float *b_at = B_KC ? p.B + (long)lane32 * p.ldb + half : p.B + (long)half * p.ldb + lane32;
+    const long a_step = A_KC ? 2 : 2 * p.lda, b_step = B_KC ? 2 : 2 * p.ldb;   // from one pair of k's to the next
+    for (int k0 = 0; k0 < p.K; k0 += 32) {
+        float a[16], b[16];
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+            const bool in_k = k0 + 2 * s + half < p.K;
+            a[s] = (in_m && in_k) ? a_at[s * a_step] : 0.f;
+            b[s] = (in_n && in_k) ? b_at[s * b_step] : 0.f;
+        }
+#pragma unroll
+        for (int s = 0; s < 16; ++s) acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc[0][0], 0, 0, 0);
+        a_at += 16 * a_step; b_at += 16 * b_step;
+    }
+    const TilePlace at{m0, 0, wave * 32, 0, lane32, half, 0L};
+    if (m0 + 128 <= p.M && p.N == 32) store_tile_kind<true, 1, 1>(p, acc, at);
+    else store_tile_kind<false, 1, 1>(p, acc, at);
+}
+
 // ---- the weight gradient of a narrow layer ------------------------------------------------------------------------------
 // dW = delta^T X with at most 32 outputs (columns of delta) and at most 32 inputs (columns of X) over many rows - a layer of an
 // independently recurrent stack over T x batch rows.  Two rows of delta and of X, as they lie in memory, ARE the operands of
@@ -816,6 +853,17 @@ int launch_gemm(hipStream_t stream, const GemmParams &p)
     }
     const bool a_kc = p.a_k_contiguous != 0, b_kc = p.b_k_contiguous != 0;
 
+    // a narrow product over many rows: the kernel that feeds the matrix unit straight from memory (MYEA_NARROW_GEMM=0: the tiled one)
+    static const bool narrow_off = [] { const char *e = std::getenv("MYEA_NARROW_GEMM"); return e && e[0] == '0'; }();
+    if (!narrow_off && p.N <= 32 && p.K <= 64 && p.M >= 256 && d.ksplit == 1) {
+        const dim3 grid((unsigned)((p.M + 127) / 128));
+        if (a_kc && b_kc) hipLaunchKernelGGL((narrow_gemm_kernel<true, true>), grid, dim3(kThreads), 0, stream, d);
+        else if (a_kc) hipLaunchKernelGGL((narrow_gemm_kernel<true, false>), grid, dim3(kThreads), 0, stream, d);
+        else if (b_kc) hipLaunchKernelGGL((narrow_gemm_kernel<false, true>), grid, dim3(kThreads), 0, stream, d);
+        else hipLaunchKernelGGL((narrow_gemm_kernel<false, false>), grid, dim3(kThreads), 0, stream, d);
+        MYEA_HIP_TRY(hipGetLastError());
+        return MYEA_OK;
+    }
     if (!vec || (!a_kc && b_kc)) return launch_layout_scalar(stream, d, a_kc, b_kc);
     // Tile choice: 128 x 128 when that still yields at least two workgroups per CU (256 CUs), else
     // 64-row tiles to keep the chip filled for short-M / short-N problems.
