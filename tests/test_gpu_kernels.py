@@ -24,7 +24,9 @@ def _gemm(lib, a_kc, b_kc, acc, M, N, K, A, B, Cc, lda=None, ldb=None, ldc=None)
 
 
 SHAPES = [(1, 1, 1), (3, 5, 7), (64, 64, 32), (65, 63, 33), (128, 256, 100), (130, 70, 257), (256, 128, 64),
-          (1000, 36, 20), (17, 1000, 520), (512, 1024, 96), (1024, 1000, 128)]
+          (1000, 36, 20), (17, 1000, 520), (512, 1024, 96), (1024, 1000, 128),
+          # at most 32 columns over at most 64 k's and 256 rows or more: the kernel that feeds the matrix unit straight from memory
+          (256, 32, 32), (300, 31, 31), (257, 10, 64), (7168, 23, 29), (1000, 1, 33)]
 
 
 @pytest.mark.parametrize("a_kc,b_kc", [(1, 1), (1, 0), (0, 0), (0, 1)])
