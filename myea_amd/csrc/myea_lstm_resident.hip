@@ -71,7 +71,7 @@ constexpr int kLocalAux = 16;      // cache policy of the LOCAL protocol's tile 
 #define MYEA_SCOPE_WORKGROUP __HIP_MEMORY_SCOPE_WORKGROUP
 
 // LDS of a workgroup: every wavefront's tiles of one unit, and the partial tiles of the two chains
-constexpr size_t forward_lds(int kw, int cells, int rs) { return ((size_t)4 * (kw == 128 && rs == 1 ? 2 : kw / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * (4 * cells + 8)) * sizeof(float); }
+constexpr size_t forward_lds(int kw, int cells, int rs) { return ((size_t)4 * (kw / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * (4 * cells + 8)) * sizeof(float); }
 constexpr size_t backward_lds(int c, int rs) { return ((size_t)4 * (c >= 512 && rs == 1 ? c / 64 : c / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * 17) * sizeof(float); }
 
 template <int N>
@@ -261,8 +261,9 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
     constexpr int A1 = NT >= 4 ? NT / 4 : 1;      // tiles whose MFMAs run before the previous unit's arrival is signalled
     constexpr int P1 = NT >= 4 ? (3 * NT) / 4 : NT - 1;   // tile before which the next unit's counter is read
     constexpr int kStride = NB + 8;               // floats per row of a wavefront's partial tile
-    constexpr bool HALF = !AGENT && NT == 4 && RS == 1;   // 512 cells: two LDS slots for a unit's four tiles, each requested two tiles ahead
-    constexpr int SLOTS = HALF ? NT / 2 : NT;
+    constexpr bool HALF = !AGENT && NT == 4 && RS == 1;   // 512 cells: a unit's four tiles are requested in two halves, each two tiles of MFMAs ahead
+    constexpr int SLOTS = NT;
+    constexpr int kAhead = HALF ? NT / 2 : NT;    // tiles of a unit that the other chain requests for it
     constexpr int kStage = SLOTS * ROWS * 32, kPart = 4 * ROWS * kStride;
     constexpr int kAux = AGENT ? 16 : kLocalAux;
     constexpr bool DB = AGENT;                    // the other chain's tiles are requested during this chain's last MFMAs, into the slots those have left
@@ -390,7 +391,7 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
             for (int q = 0; q < LPT; ++q) p_tile[c][q] += step_c;
         }
     };
-    auto load_tiles = [&](auto ch) { load_tile_range(ch, std::integral_constant<int, 0>{}, std::integral_constant<int, SLOTS>{}, std::integral_constant<bool, !HALF>{}); };
+    auto load_tiles = [&](auto ch) { load_tile_range(ch, std::integral_constant<int, 0>{}, std::integral_constant<int, kAhead>{}, std::integral_constant<bool, !HALF>{}); };
     auto mfma_tiles = [&](auto ch, auto first, auto last) {
 #pragma unroll
         for (int i = decltype(first)::value; i < decltype(last)::value; ++i) {
@@ -425,12 +426,17 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
 #pragma unroll
             for (int ct = 0; ct < NCT; ++ct) acc[rs][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (decltype(all_landed)::value) wait_vm<0>(); else wait_vm<NSTORE>();
-        mfma_tiles(ch, I0{}, IA{});
-        __builtin_amdgcn_sched_barrier(0);   // keeps the MFMAs above in front of the wait
-        if constexpr (HALF) {   // the third tile into the slot the first has left; the stores of the unit before are older
+        if constexpr (HALF) {   // the unit's second half: the third tile now, the fourth behind the first tile's MFMAs - two tiles of MFMAs ahead each
+            __builtin_amdgcn_sched_barrier(0);
             load_tile_range(ch, std::integral_constant<int, 2>{}, std::integral_constant<int, 3>{}, std::false_type{});
             __builtin_amdgcn_sched_barrier(0);
-            wait_vm<LPT>();
+        }
+        mfma_tiles(ch, I0{}, IA{});
+        __builtin_amdgcn_sched_barrier(0);   // keeps the MFMAs above in front of the wait
+        if constexpr (HALF) {   // the stores of the unit before are older than the two requests
+            load_tile_range(ch, std::integral_constant<int, 3>{}, IN{}, std::true_type{});
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<2 * LPT>();
         } else {
             wait_vm<0>();
         }
@@ -445,12 +451,13 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
         load_inputs(ch);
         bool requested = false;   // the other chain's tiles are on their way already
         if constexpr (!FIRST && HALF) {
-            // Two slots for four tiles: tile i + 2 is requested behind tile i's MFMAs (a unit's first two behind the last two
-            // MFMA tiles of the unit before, if the chain's counter is complete by then), so a wavefront never issues more than
-            // two loads in a row - eight in a row, four wavefronts at once, keep the compute unit's address path busy for 512
-            // clocks during which the issuing wavefronts stand still.  The first wait counts what was issued behind the tile it
-            // waits for; the unit's inputs are counted as four loads, the fewest there can be (two more with zoneout masks: it
-            // then asks for a little more than it needs).  The second leaves nothing in flight - the inputs too, requested two
+            // A unit's four tiles are requested two at a time (its first two behind the last two MFMA tiles of the unit before, if
+            // the chain's counter is complete by then; the third and the fourth in the unit's head, around its first tile's
+            // MFMAs), so a wavefront never issues more than two loads in a row - eight in a row, four wavefronts at once, keep
+            // the compute unit's address path busy for 512 clocks during which the issuing wavefronts stand still - and every tile
+            // has two tiles of MFMAs to arrive (with one, the wait for it cost 500 clocks a tile).  The first wait counts what
+            // was issued behind the tile it waits for: the fourth tile, the counter, and the unit's inputs, counted as four loads,
+            // the fewest there can be (two more with zoneout masks: it then asks for a little more than it needs).  The second leaves nothing in flight - the inputs too, requested two
             // tiles of MFMAs ago - so that the compiler has no load left to wait for in front of the gate math: it would
             // wait for everything there, the next unit's tiles included.
             constexpr int kIn = 4 * PAIRS;
@@ -461,7 +468,6 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_forward_kernel(Resi
             __builtin_amdgcn_sched_barrier(0);
             mfma_tiles(ch, I1{}, I2{});
             __builtin_amdgcn_sched_barrier(0);
-            load_tile_range(ch, I3{}, IN{}, std::true_type{});   // the fourth tile into the second's slot
             asm volatile("global_load_dword %0, %1, off sc1" : "=v"(seen) : "v"(counters + (1 - c) * kSyncStride) : "memory");
             __builtin_amdgcn_sched_barrier(0);
             wait_vm<LPT + 1 + kIn>();              // the third tile has landed: behind it came the inputs, the fourth tile, the counter
