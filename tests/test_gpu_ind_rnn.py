@@ -137,3 +137,34 @@ def test_refusals():
         mb.HipNetwork(mb.make_desc([dict(units=6), ind(8, "SOFTMAX"), dict(units=3, activation="LINEAR")], 4, 3))
     with pytest.raises(ValueError):        # as the output layer
         mb.make_desc([dict(units=6), ind(8, "TANH")], 4, 3)
+
+
+def test_gradient_sums_of_many_layers_follow_the_batch_size():
+    """A narrow normalised stack over 640 rows adds its per-layer partial results - the normalisations' per-time-step shares,
+    the narrow weight gradients' slabs, the self weights' per-example shares - in one launch per pass when the batch fills the
+    network's rows, and layer by layer when it does not: full, partial and full batches in turn give the oracle's gradient each
+    time."""
+    specs = [dict(units=20), ind(31, "ISRLU", normalization="BATCH_NORMALIZATION", norm_before=True),
+             ind(29, "TANH", normalization="BATCH_NORMALIZATION", norm_before=True), dict(units=7, activation="LINEAR")]
+    T, Bmax = 8, 80
+    desc = mb.make_desc(specs, Bmax, T)
+    h = mb.default_hyper(type_optimizer_function=mb.OPTIMIZER["GD"], learning_rate=1e-5, type_loss_function=mb.LOSS["MSE"])
+    gpu, cpu = mb.HipNetwork(desc, h), OracleNetwork(desc, h)
+    w = _self_weights(desc, glorot_parameters(desc, 21, bias_range=0.3), 21)
+    rng = np.random.default_rng(21)
+    for n in (gpu, cpu):
+        n.set_state_propagation(mb.STATE_TRAINING)
+        n.upload_parameters(w)
+        n.Clear_Training_Arrays()
+    for step, B in enumerate((80, 64, 80, 80, 33)):
+        X = rng.normal(0, 1, (B, T * 20)).astype(np.float32)
+        Y = rng.normal(0, 1, (B, T * 7)).astype(np.float32)
+        for n in (gpu, cpu):
+            n.Reset__Loss()
+            run_step(n, B, X, Y, update=False)
+        g, want = gpu.download_gradient(), cpu.download_gradient()
+        assert 1e-3 < float(np.abs(want).max()) < 1e4, "the steps stay small: the gradient is neither vacuous nor blown up"
+        assert_close(g, want, REL, ABS * max(1.0, float(np.abs(want).max())), what="gradient, step %d with %d examples" % (step, B))
+        for n in (gpu, cpu):
+            n.Update_Parameter(B, B)
+        gpu.upload_parameters(cpu.download_parameters())
