@@ -77,6 +77,8 @@ int gemm_split_k(int M, int N, int K);
 // polls a tile's second workgroup waits for the first: 2^24 (seconds), or MYEA_GEMM_PAIR_SPIN_POLLS (0: give up at once, for tests
 // of that path; read at every call)
 unsigned gemm_pair_polls();
+// true when workgroups whose ids are equal mod 8 run on one XCD of the current device (probed by one launch per device and process)
+bool device_groups_share_xcd();
 // true when launch_gemm, handed pair_partials / pair_tickets, would share every 128 x 128 tile's k between two workgroups
 // (at most one such tile per compute unit, a k worth halving): callers size their pair buffers by it
 bool gemm_pair_k_128(int M, int N, int K);

@@ -1248,6 +1248,16 @@ int probe_device(ResidentDevice **out)
     return MYEA_OK;
 }
 
+}  // namespace
+
+bool device_groups_share_xcd()
+{
+    ResidentDevice *dev = nullptr;
+    return probe_device(&dev) == MYEA_OK && dev && dev->usable;
+}
+
+namespace {
+
 // MYEA_LSTM_RESIDENT=0 keeps every layer on one launch per time step
 bool resident_disabled()
 {
