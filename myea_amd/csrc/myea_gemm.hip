@@ -315,13 +315,33 @@ __device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&a
         for (int i = 0; i < TM; ++i) {
             const int row0 = at.m0 + at.wave_m + i * 32 + at.half * 4;
             float column_sum = 0.f, column_sum2 = 0.f;   // per kind: see col_partials
+            // What an accumulator's elements read from other tensors - the addend, the pre-activation or the activation, x-hat -
+            // is asked for four elements at a time, ahead of their arithmetic: read where it is used, every load would sit behind
+            // the store of the element before it (the compiler may not move it across: the tensors could overlap) and cost its
+            // own trip to memory.  (All sixteen at once need 48 more registers than the 128 x 128 tile leaves.)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = row0 + (r >> 2) * 8 + (r & 3);
+            for (int rq = 0; rq < 4; ++rq) {
+            float addend_v[4], operand_v[4], hats_v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = row0 + rq * 8 + e;
+                addend_v[e] = 0.f; operand_v[e] = 0.f; hats_v[e] = 0.f;
+                if (!WHOLE && row >= p.M) continue;
+                const long o = (long)row * p.ldc + col + at.slab_offset;
+                if (ADDEND) addend_v[e] = p.addend[(long)row * p.ld_addend + col];
+                if (KIND == 2) {
+                    operand_v[e] = CLASS == 1 ? p.pre[o] : p.val[o];
+                    if (p.hats) hats_v[e] = p.hats[o];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int r = rq * 4 + e;
+                const int row = row0 + rq * 8 + e;
                 if (!WHOLE && row >= p.M) continue;
                 const long o = (long)row * p.ldc + col + at.slab_offset;
                 float v = acc[i][j][r];
-                if (ADDEND) v += p.addend[(long)row * p.ld_addend + col];
+                if (ADDEND) v += addend_v[e];
                 if (KIND == 1) {
                     v += bias;
                     p.C[o] = v;
@@ -340,9 +360,9 @@ __device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&a
                 } else if (KIND == 2) {
                     float dv;
                     if (CLASS == 1) {
-                        dv = p.pre[o] < 0.f ? d_neg : p.steep;
+                        dv = operand_v[e] < 0.f ? d_neg : p.steep;
                     } else {
-                        const float y = p.val[o];
+                        const float y = operand_v[e];
                         dv = tanh_like ? p.steep * (1.f - y * y) : p.steep * y * (1.f - y);
                     }
                     {
@@ -350,13 +370,14 @@ __device__ __forceinline__ void store_tile_as(const GemmDev &p, const f32x16 (&a
                         const float out = v * dv;
                         p.C[o] = out;
                         column_sum = column_sum + out;
-                        if (p.hats) column_sum2 = column_sum2 + out * p.hats[o];
+                        if (p.hats) column_sum2 = column_sum2 + out * hats_v[e];
                     }
                 } else if (KIND == 3) {
                     unsafeAtomicAdd(&p.C[o], v);
                 } else {
                     p.C[o] = v;
                 }
+            }
             }
             if ((KIND == 1 || KIND == 2) && p.col_partials) {
                 const float both = column_sum + __shfl_xor(column_sum, 32);   // the column's other 16 rows of this accumulator
