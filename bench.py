@@ -428,8 +428,10 @@ def main():
         # the other two configurations of the baseline that are timed on the GPU, a few steps each, so that one run records all four
         out["other_configurations"] = []
         for name in OTHERS + (EXAMPLE,):
-            o = run_workload(name, max(5, args.steps // 3), max(2, args.warmup // 2), args.separate_update)
+            # timed like the headline: the same warm-up, the median of `repeats` blocks of exactly `steps` steps each
+            o = run_workload(name, max(5, args.steps // 3), max(2, args.warmup), args.separate_update, repeats=args.repeats)
             leg = {"workload": name, "value": o["value"], "unit": "samples/s", "ms_per_step": o["ms_per_step"], "steps": max(5, args.steps // 3),
+                   "warmup": max(2, args.warmup), "repeats": args.repeats, "ms_per_step_blocks": [round(x, 4) for x in o["ms_per_step_blocks"]],
                    "config": config_of(o), "contractions": o["contractions_alone"] or o["contractions"], "kernels": o["kernels"], "loss_per_output": o["loss_per_output"]}
             if o["time_loops"]["launches"] > 0:
                 leg["time_loops"] = o["time_loops"]
