@@ -72,6 +72,7 @@ constexpr int kLocalAux = 16;      // cache policy of the LOCAL protocol's tile 
 
 // LDS of a workgroup: every wavefront's tiles of one unit, and the partial tiles of the two chains
 constexpr size_t forward_lds(int kw, int cells, int rs) { return ((size_t)4 * (kw / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * (4 * cells + 8)) * sizeof(float); }
+constexpr size_t backward_sets_lds(int c) { return ((size_t)8 * (c / 32 < 8 ? c / 32 : 8) * 16 * 32 + (size_t)2 * 4 * 16 * 17) * sizeof(float); }
 constexpr size_t backward_lds(int c, int rs) { return ((size_t)4 * (c >= 512 && rs == 1 ? c / 64 : c / 32) * 16 * rs * 32 + (size_t)2 * 4 * 16 * rs * 17) * sizeof(float); }
 
 template <int N>
@@ -954,6 +955,334 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
     store_column_sums(sums, d.sums, rg, C, c0);
 }
 
+// ---- backward, one chain per set of four wavefronts --------------------------------------------------------------------
+// The same split along the columns of dh, the same group protocol (LOCAL) and the same arithmetic as the kernel above, with
+// the two chains of a member in two SETS of four wavefronts instead of alternating in one instruction stream: eight
+// wavefronts, two per SIMD, each set running the plain loop of its own chain - wait for the group, stream the gate deltas of
+// the step before through LDS into the MFMAs, exchange the partial tiles within the set, gate deltas, stores, arrive.
+// Why: a unit's tail - exchange, gate arithmetic, stores, their drain, the group's counter - has no MFMAs at all, and in one
+// instruction stream nothing else runs during it.  With a set per chain one chain's tail and waits run under the other's
+// MFMAs.  Both sets keep the member's slice of WrecT in registers (2 x C / 4 registers a lane: C <= 512).
+// What made it work (each measured at 512 cells x 256 examples, where the one-stream kernel takes 464 us a pass):
+//   - The tile loops take TURNS, in one fixed order (s_turn).  Left alone the two sets fall into step - both contracting at
+//     half speed, then both in their tails - and stay there: 1005 us.
+//   - Nobody polls a word the whole launch shares, and one wavefront per set polls the group's counter while the other three
+//     watch LDS.  A poll in flight to a busy line holds up everything else its compute unit asks of memory (a tile step of
+//     1000 clocks instead of 380, every load instruction a few hundred clocks to issue): 755 -> 438 us.
+//   - A short pause before the first poll (below): 414 us.
+// The four wavefronts of a set meet through a counter in LDS (s_barrier would tie the two chains together); every wait of
+// this kernel is bounded by the same count of polls and ends the wavefront through the give-up path.
+template <int CC>
+__global__ __launch_bounds__(2 * kThreads, 1) void lstm_resident_backward_sets_kernel(ResidentGeometry g, LstmResidentDir d0, LstmResidentDir d1, SyncWords w)
+{
+    constexpr int C = CC, G = 4 * C, CELLS = 16, ROWS = 16, NT = C / 32, LPT = ROWS / 8;
+    constexpr int SLOTS = NT < 8 ? NT : 8;             // tiles of LDS per wavefront
+    constexpr int AHEAD = NT <= 8 ? NT : SLOTS - 2;    // tiles requested ahead of the one being contracted
+    constexpr int kStride = 17, kStage = SLOTS * ROWS * 32, kPart = 4 * ROWS * kStride;
+    static_assert(NT >= 4 && C <= 512 && 2 * AHEAD + 8 < 64, "weights of both sets in registers; vmcnt has 6 bits");
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    __shared__ unsigned s_arrive[2], s_meet[2], s_go[2], s_turn;   // s_turn: how many tile loops the member has finished; loop number n is chain n % 2's
+    __shared__ double s_fold[8][7][16];
+    const int lane = threadIdx.x & 63, col16 = lane & 15, quad = lane >> 4;
+    const int wave8 = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), c = wave8 >> 2, wave = wave8 & 3;   // c: the set's chain
+    const int tid = (int)threadIdx.x & (kThreads - 1);
+
+    int group, member;
+    if (!place<false>(blockIdx.x, g.members, g.dirs * g.row_groups, group, member)) return;
+    const int dir = group % g.dirs, rg = group / g.dirs;
+    const LstmResidentDir &d = dir ? d1 : d0;
+    const int c0 = member * CELLS, B = g.B, T = g.T;
+    const size_t Bmax = (size_t)g.Bmax;
+    unsigned *const counter = w.counters + ((size_t)group * 2 + c) * kSyncStride;
+    const unsigned members = (unsigned)g.arrivals;
+    check_same_xcd(w, group);
+    if (threadIdx.x < 2) { s_arrive[threadIdx.x] = 0u; s_meet[threadIdx.x] = 0u; s_go[threadIdx.x] = 0u; }
+    if (threadIdx.x == 0) s_turn = 0u;
+    __syncthreads();
+
+    float *const stage = smem + wave8 * kStage;
+    float *const part = smem + 8 * kStage + c * kPart;
+
+    // WrecT rows c0 .. c0 + 15, the k range of gate `wave`
+    f32x4 breg[NT][2];
+    {
+        const float *row = d.WrecT + (size_t)(c0 + col16) * G + (size_t)wave * C;
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) breg[i][h] = *reinterpret_cast<const f32x4 *>(row + i * 32 + (h * 4 + quad) * 4);
+    }
+    // Offsets into the [T][Bmax][4C] and [T][Bmax][C] tensors as 32-bit unsigned numbers (the host only picks this kernel when
+    // they fit) that step by a wrapped-around amount: a uniform base plus one register per lane instead of a pointer each.
+    const int t_first = d.reverse ? 0 : T - 1;
+    const unsigned step_g = (unsigned)((d.reverse ? 1 : -1) * (int)(Bmax * G)), step_c = (unsigned)((d.reverse ? 1 : -1) * (int)(Bmax * C));
+    // the lane's (example, cell) pair of the set's chain
+    const int row = tid >> 4, cell = tid & 15, k = c0 + cell;
+    const int r = (rg * 2 + c) * ROWS + row;
+    const bool valid = r < B;   // a lane without an example reads the batch's last one and stores nothing
+    float e_peep[3];
+#pragma unroll
+    for (int gate = 0; gate < 3; ++gate) e_peep[gate] = d.peep[gate * C + k];
+    const unsigned at = (unsigned)t_first * (unsigned)Bmax + (unsigned)min(r, B - 1);
+    unsigned off_g = at * G + k, off_c = at * C + k;
+    float n_di = 0.f, n_df = 0.f, n_f = 0.f, n_dc = 0.f;   // of the step processed before: delta i, delta f, f, delta c
+    double sums[7] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+    // rows of dG the wavefront stages: the k range of its gate, at the step this pass processed before the current one
+    unsigned off_tile[LPT];
+#pragma unroll
+    for (int q = 0; q < LPT; ++q) {
+        const int tr = q * 8 + (lane >> 3), chunk = (lane & 7) ^ ((tr >> 1) & 7);
+        off_tile[q] = ((unsigned)t_first * (unsigned)Bmax + (unsigned)min((rg * 2 + c) * ROWS + tr, B - 1)) * G + (unsigned)wave * C + chunk * 4;
+    }
+    auto request_tile = [&](auto i) {
+        constexpr int I = decltype(i)::value;
+#pragma unroll
+        for (int q = 0; q < LPT; ++q)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(d.dG + off_tile[q] + I * 32),
+                                             (__attribute__((address_space(3))) void *)(stage + (I % SLOTS) * ROWS * 32 + q * 256), 16, 0, kLocalAux);
+    };
+    // The set's four wavefronts meet: `target` arrivals in the set's LDS word.  Bounded like every wait here.
+    auto meet = [&](unsigned target) -> bool {
+        int ok = 1;
+        if (lane == 0) {
+            const unsigned word = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned *)&s_meet[c], one = 1u;
+            const unsigned turn_at = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned *)&s_turn;
+            unsigned value, polls = g.spin_polls;
+            asm volatile(
+                "s_waitcnt lgkmcnt(0)\n\t"
+                "ds_add_rtn_u32 %[value], %[word], %[one]\n\t"
+                "s_waitcnt lgkmcnt(0)\n\t"
+                "v_and_b32 %[value], 3, %[value]\n\t"
+                "v_cmp_ne_u32 vcc, 3, %[value]\n\t"
+                "s_cbranch_vccnz 1f\n\t"
+                "ds_add_u32 %[turn], %[one]\n"      // the set's last wavefront through its tiles hands the matrix units on
+                "1:\n\t"
+                "ds_read_b32 %[value], %[word]\n\t"
+                "s_waitcnt lgkmcnt(0)\n\t"
+                "v_sub_u32 %[value], %[value], %[target]\n\t"
+                "v_cmp_le_i32 vcc, 0, %[value]\n\t"
+                "s_cbranch_vccnz 2f\n\t"
+                "s_sleep 1\n\t"
+                "s_sub_u32 %[polls], %[polls], 1\n\t"
+                "s_cmp_lg_u32 %[polls], 0\n\t"
+                "s_cbranch_scc1 1b\n\t"
+                "v_mov_b32 %[ok], 0\n"
+                "2:\n"
+                : [ok] "+v"(ok), [value] "=&v"(value), [polls] "+s"(polls)
+                : [word] "v"(word), [one] "v"(one), [target] "v"(target), [turn] "v"(turn_at)
+                : "vcc", "scc", "memory");
+            if (!ok) {
+                __hip_atomic_store(w.give_up, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+                __hip_atomic_store(w.host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                __hip_atomic_store(w.fault, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+            }
+        }
+        return __builtin_amdgcn_readfirstlane(ok) != 0;
+    };
+
+    // The matrix units go to one set at a time, in one fixed order for every member of every group: chain 0's unit, chain 1's,
+    // chain 0's next ...  Two sets contracting at once run at half speed each, end together and sit through their tails together -
+    // and stay in step; members that took their turns in different orders would hold up both chains of their group.  In turns,
+    // a set's exchange, gate arithmetic, stores and waits run under the other's MFMAs.  `number`: which tile loop of the member
+    // this is; the set's last wavefront through the tiles counts it as done (in meet()).
+    auto take_turn = [&](unsigned number) -> bool {
+        int ok = 1;
+        if (lane == 0) {
+            const unsigned turn_at = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned *)&s_turn;
+            unsigned value, polls = g.spin_polls;
+            asm volatile(
+                "1:\n\t"
+                "ds_read_b32 %[value], %[turn]\n\t"
+                "s_waitcnt lgkmcnt(0)\n\t"
+                "v_cmp_eq_u32 vcc, %[number], %[value]\n\t"
+                "s_cbranch_vccnz 2f\n\t"
+                "s_sleep 1\n\t"
+                "s_sub_u32 %[polls], %[polls], 1\n\t"
+                "s_cmp_lg_u32 %[polls], 0\n\t"
+                "s_cbranch_scc1 1b\n\t"
+                "v_mov_b32 %[ok], 0\n"
+                "2:\n"
+                : [ok] "+v"(ok), [value] "=&v"(value), [polls] "+s"(polls)
+                : [turn] "v"(turn_at), [number] "v"(number)
+                : "vcc", "scc", "memory");
+            if (!ok) {
+                __hip_atomic_store(w.give_up, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+                __hip_atomic_store(w.host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                __hip_atomic_store(w.fault, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+            }
+        }
+        return __builtin_amdgcn_readfirstlane(ok) != 0;
+    };
+
+    // The group's counter has reached `target`: the set's first wavefront asks memory (the counter's line only - a word that
+    // every wavefront of the launch polls is a queue at one L2 channel, and everything else this compute unit asks of memory
+    // waits behind its polls), the other three watch a word in LDS.  Bounded; 0 when the wait gave up here or elsewhere.
+    auto group_wait = [&](unsigned target) -> bool {
+        int ok = 1;
+        if (lane == 0) {
+            const unsigned go_at = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned *)&s_go[c];
+            unsigned value, polls = g.spin_polls;
+            if (wave == 0) {
+                asm volatile(
+                    "1:\n\t"
+                    "global_load_dword %[value], %[counter], off sc1\n\t"
+                    "s_waitcnt vmcnt(0)\n\t"
+                    "v_sub_u32 %[value], %[value], %[target]\n\t"
+                    "v_cmp_le_i32 vcc, 0, %[value]\n\t"
+                    "s_cbranch_vccnz 2f\n\t"
+                    "s_sleep 4\n\t"
+                    "s_sub_u32 %[polls], %[polls], 1\n\t"
+                    "s_cmp_lg_u32 %[polls], 0\n\t"
+                    "s_cbranch_scc1 1b\n\t"
+                    "v_mov_b32 %[ok], 0\n\t"
+                    "s_branch 3f\n"
+                    "2:\n\t"
+                    "ds_write_b32 %[go], %[target]\n"
+                    "3:\n"
+                    : [ok] "+v"(ok), [value] "=&v"(value), [polls] "+s"(polls)
+                    : [counter] "v"(counter), [target] "v"(target), [go] "v"(go_at)
+                    : "vcc", "scc", "memory");
+            } else {
+                asm volatile(
+                    "1:\n\t"
+                    "ds_read_b32 %[value], %[go]\n\t"
+                    "s_waitcnt lgkmcnt(0)\n\t"
+                    "v_sub_u32 %[value], %[value], %[target]\n\t"
+                    "v_cmp_le_i32 vcc, 0, %[value]\n\t"
+                    "s_cbranch_vccnz 2f\n\t"
+                    "s_sleep 2\n\t"
+                    "s_sub_u32 %[polls], %[polls], 1\n\t"
+                    "s_cmp_lg_u32 %[polls], 0\n\t"
+                    "s_cbranch_scc1 1b\n\t"
+                    "v_mov_b32 %[ok], 0\n"
+                    "2:\n"
+                    : [ok] "+v"(ok), [value] "=&v"(value), [polls] "+s"(polls)
+                    : [target] "v"(target), [go] "v"(go_at)
+                    : "vcc", "scc", "memory");
+            }
+            if (!ok) {
+                __hip_atomic_store(w.give_up, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+                __hip_atomic_store(w.host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                __hip_atomic_store(w.fault, 1u, __ATOMIC_RELAXED, MYEA_SCOPE_AGENT);
+            }
+        }
+        return __builtin_amdgcn_readfirstlane(ok) != 0;
+    };
+
+    // the operands of the unit at hand: asked for inside the unit's tile loop, behind its last tile request (the pass's first
+    // unit, which has no tiles, asks for them up front)
+    float e_act[4], e_ca, e_dh, e_cp, e_cs;
+    auto load_operands = [&](int s) {   // s: the direction's step the offsets stand at
+#pragma unroll
+        for (int gate = 0; gate < 4; ++gate) e_act[gate] = d.acts[off_g + gate * C];
+        e_ca = d.ca[off_c]; e_dh = d.dh[off_c];
+        e_cp = d.c[s > 0 ? off_c + step_c : off_c];   // the cell state of the step before in the direction's order (without one: any valid address, the value is not used)
+        e_cs = d.c[off_c];
+    };
+    load_operands(T - 1);
+    bool alive = true;
+    for (int j = 0; j < T && alive; ++j) {
+        const int s = T - 1 - j;   // the direction's step
+        float rec = 0.f;
+        if (j > 0) {
+            // every member's gate deltas of the step before are in memory
+            // A pause of about 2 k clocks in front of the first look at the counter: the group is never complete earlier, and a set
+            // that starts to poll right behind its arrival slows the other set's tiles and stores by more than the pause costs
+            // (measured at 512 cells x 256 examples: 414 us a pass with it, 720 without; 16, 48 and 80 x 64 clocks: 420, 417, 457)
+            __builtin_amdgcn_s_sleep(32);
+            if (!group_wait((unsigned)j * members)) { alive = false; break; }
+            static_for<0, AHEAD>([&](auto i) { request_tile(i); });   // on their way while the set waits for its turn
+            if constexpr (AHEAD == NT) {   // every tile has been asked for: the operands right behind them
+                __builtin_amdgcn_sched_barrier(0);
+                load_operands(s);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (!take_turn(2u * (unsigned)(j - 1) + (unsigned)c)) { alive = false; break; }
+            f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+            static_for<0, NT>([&](auto i) {
+                constexpr int I = decltype(i)::value;
+                // loads requested behind tile I's: the tiles after it and, once the last tile has been asked for, this unit's own
+                // eight operands (the unit before could not ask for them without standing between its arrival and this wait)
+                constexpr int kBehind = (I + AHEAD < NT ? AHEAD - 1 : NT - 1 - I) * LPT + (I + AHEAD >= NT ? 8 : 0);
+                __builtin_amdgcn_sched_barrier(0);
+                wait_vm<kBehind>();
+                const float *tile = stage + (I % SLOTS) * ROWS * 32;
+                f32x4 fa[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) fa[h] = ATile<ROWS, kLocalAux>::chunk(tile, col16, h * 4 + quad);
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[h][e], breg[I][h][e], acc[e & 1], 0, 0, 0);
+                asm volatile("" : "+v"(acc[0]), "+v"(acc[1]));   // keeps the tile's MFMAs here: without a side effect of their own they would all sink behind the last tile
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (I + AHEAD < NT) request_tile(std::integral_constant<int, I + AHEAD>{});
+                if constexpr (I + AHEAD + 1 == NT) {
+                    load_operands(s);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < LPT; ++q) off_tile[q] += step_g;
+            float *to = part + wave * ROWS * kStride;
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) to[(quad * 4 + rr) * kStride + col16] = acc[0][rr] + acc[1][rr];
+            if (!meet(4u * (unsigned)j)) { alive = false; break; }
+#pragma unroll
+            for (int wv = 0; wv < 4; ++wv) rec += part[(wv * ROWS + row) * kStride + cell];
+        }
+        const float dh = e_dh + rec;
+        const float z = e_act[0], gi = e_act[1], gf = e_act[2], go = e_act[3];
+        const float a = e_ca;
+        const float ddo = go * (1.f - go) * (dh * a);
+        float e = dh * go * (1.f - a * a);
+        e += e_peep[2] * ddo;
+        if (j > 0) {
+            e += e_peep[0] * n_di;
+            e += e_peep[1] * n_df;
+            e += n_dc * n_f;
+        }
+        const float dz = e * gi * (1.f - z * z);
+        const float di = (e * z) * (gi * (1.f - gi));
+        const float df = s > 0 ? (e * e_cp) * (gf * (1.f - gf)) : 0.f;
+        n_di = di; n_df = df; n_f = gf; n_dc = e;
+        if (valid) {
+            sums[0] += dz; sums[1] += di; sums[2] += df; sums[3] += ddo;
+            sums[4] += s > 0 ? di * e_cp : 0.f; sums[5] += df * e_cp; sums[6] += ddo * e_cs;
+        }
+        if (valid) {
+            float *drow = d.dG + off_g;
+            drow[0] = dz; drow[C] = di; drow[2 * C] = df; drow[3 * C] = ddo;
+            d.dh[off_c] = dh; d.dc[off_c] = e;
+        }
+        off_g += step_g; off_c += step_c;
+        if (j + 1 < T) {
+            wait_vm<0>();
+            wave_arrive<false>(counter, &s_arrive[c]);
+        }
+    }
+    // the seven sums over the member's examples of both chains, in a fixed order; every wavefront takes part, also one
+    // that gave up (its sums are not used: the launch is reported as failed)
+    if (d.sums) {
+#pragma unroll
+        for (int v = 0; v < 7; ++v) {
+            double x = sums[v];
+            x += __shfl_xor(x, 16);
+            x += __shfl_xor(x, 32);
+            if (lane < 16) s_fold[wave8][v][lane] = x;
+        }
+    }
+    __syncthreads();
+    if (d.sums && threadIdx.x < 7 * 16) {
+        const int v = threadIdx.x >> 4, cl = threadIdx.x & 15;
+        double x = s_fold[0][v][cl];
+#pragma unroll
+        for (int wv = 1; wv < 8; ++wv) x += s_fold[wv][v][cl];
+        d.sums[((size_t)rg * 7 + v) * C + c0 + cl] = (float)x;
+    }
+}
+
 // ---- backward, the contraction split along k ------------------------------------------------------------------------
 // dh[t] += dG[t'] Wrec with every member contracting over ITS OWN 64 k's: the gate deltas of its 16 cells, which it has
 // just computed and keeps in LDS - no member reads another's gate deltas.  What it owes the others is its share of every
@@ -1312,6 +1641,7 @@ struct KernelInfo {
     ResidentKernel fn = nullptr;
     size_t lds = 0;
     int cells = 0;
+    int threads = kThreads;
     bool ready = false;
     hipError_t status = hipSuccess;
     int per_cu = 0;   // workgroups of this kernel a compute unit can hold
@@ -1333,6 +1663,17 @@ KernelInfo backward_info()
     k.fn = lstm_resident_backward_kernel<C, RS>;
     k.lds = backward_lds(C, RS);
     k.cells = 16;
+    return k;
+}
+
+template <int C>
+KernelInfo sets_info()
+{
+    KernelInfo k;
+    k.fn = lstm_resident_backward_sets_kernel<C>;
+    k.lds = backward_sets_lds(C);
+    k.cells = 16;
+    k.threads = 2 * kThreads;
     return k;
 }
 
@@ -1361,17 +1702,28 @@ KernelInfo g_kernels[2][4][2] = {
 // the backward loop split along k, [C: 128, 256, 512, 1024]: two chains of 16 examples only, groups within one XCD
 KernelInfo g_ksplit[4] = {ksplit_info<128>(), ksplit_info<256>(), ksplit_info<512>(), KernelInfo{}};
 
+// the backward loop with one chain per set of four wavefronts, [C: 128, 256, 512, 1024]: two chains of 16 examples, groups
+// within one XCD
+KernelInfo g_sets[4] = {KernelInfo{}, KernelInfo{}, sets_info<512>(), KernelInfo{}};
+
+// MYEA_LSTM_BACKWARD_SETS=0 keeps the backward loop's two chains in one instruction stream
+bool sets_disabled()
+{
+    const char *e = std::getenv("MYEA_LSTM_BACKWARD_SETS");
+    return e && e[0] == '0';
+}
+
 // the kernel for (C, rs) with its LDS attribute set and its occupancy known, or nullptr
-KernelInfo *kernel_for(size_t C, int rs, bool backward, bool ksplit = false)
+KernelInfo *kernel_for(size_t C, int rs, bool backward, bool ksplit = false, bool sets = false)
 {
     const int ci = C == 128 ? 0 : C == 256 ? 1 : C == 512 ? 2 : C == 1024 ? 3 : -1;
-    if (ci < 0 || rs < 1 || rs > 2 || (ksplit && (rs != 1 || !backward))) return nullptr;
-    KernelInfo &k = ksplit ? g_ksplit[ci] : g_kernels[backward ? 1 : 0][ci][rs - 1];
+    if (ci < 0 || rs < 1 || rs > 2 || ((ksplit || sets) && (rs != 1 || !backward))) return nullptr;
+    KernelInfo &k = sets ? g_sets[ci] : ksplit ? g_ksplit[ci] : g_kernels[backward ? 1 : 0][ci][rs - 1];
     if (!k.fn) return nullptr;
     std::lock_guard<std::mutex> lock(g_resident_mutex);
     if (!k.ready) {
         k.status = k.lds ? hipFuncSetAttribute(reinterpret_cast<const void *>(k.fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)k.lds) : hipSuccess;
-        if (k.status == hipSuccess) k.status = hipOccupancyMaxActiveBlocksPerMultiprocessor(&k.per_cu, reinterpret_cast<const void *>(k.fn), kThreads, k.lds);
+        if (k.status == hipSuccess) k.status = hipOccupancyMaxActiveBlocksPerMultiprocessor(&k.per_cu, reinterpret_cast<const void *>(k.fn), k.threads, k.lds);
         k.ready = true;
     }
     return k.status == hipSuccess && k.per_cu >= 1 ? &k : nullptr;
@@ -1454,6 +1806,11 @@ int launch_resident(hipStream_t s, bool backward, const LstmResidentPlan &plan, 
     rc = probe_device(&dev);
     if (rc != MYEA_OK) return rc;
     int grid = 0;
+    if (backward && !ksplit && !plan.agent && plan.rs == 1 && !sets_disabled() && dev->usable && (unsigned long long)T * Bmax * 4ull * C < (1ull << 30)) {   // its offsets are 32-bit byte counts
+        // the column form with a set of wavefronts per chain, where it exists and maps onto the device like the plan's kernel
+        KernelInfo *sets = kernel_for(C, plan.rs, true, false, true);
+        if (sets && place_groups(*dev, *sets, plan.members, false, plan.row_groups * dirs, &grid) && grid == plan.grid) k = sets;
+    }
     if (!k || !dev->usable || !place_groups(*dev, *k, plan.members, plan.agent, plan.row_groups * dirs, &grid) || grid != plan.grid) {
         set_last_error("resident LSTM: the plan does not fit the device (C = %zu, %d groups)", C, plan.row_groups * dirs);
         return MYEA_E_UNSUPPORTED;
@@ -1461,7 +1818,7 @@ int launch_resident(hipStream_t s, bool backward, const LstmResidentPlan &plan, 
     rc = prepare_sync(s, plan, dirs, sync, host_flag, fault, &w);
     if (rc != MYEA_OK) return rc;
     w.exchange = ksplit ? exchange : nullptr;
-    hipLaunchKernelGGL(k->fn, dim3((unsigned)plan.grid), dim3(kThreads), k->lds, s, g, dir[0], dir[dirs > 1 ? 1 : 0], w);
+    hipLaunchKernelGGL(k->fn, dim3((unsigned)plan.grid), dim3((unsigned)k->threads), k->lds, s, g, dir[0], dir[dirs > 1 ? 1 : 0], w);
     MYEA_HIP_TRY(hipGetLastError());
     return MYEA_OK;
 }
