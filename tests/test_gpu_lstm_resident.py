@@ -82,10 +82,15 @@ def _loop_launches(net):
 
 
 # the backward loop has two resident forms: split along k (members exchange partial sums; the default) and split along the
-# columns of dh (members read each other's gate deltas; MYEA_LSTM_BACKWARD_KSPLIT=0)
-@pytest.mark.parametrize("ksplit", ["1", "0"], ids=["backward-split-along-k", "backward-split-along-columns"])
-@pytest.mark.parametrize("name,specs,T,B,Bmax,backward", CASES, ids=[c[0] for c in CASES])
-def test_resident_loop_matches_one_launch_per_step_and_the_oracle(name, specs, T, B, Bmax, backward, ksplit):
+# columns of dh (members read each other's gate deltas; MYEA_LSTM_BACKWARD_KSPLIT=0); at 512 cells the column form runs a
+# member's two chains in two sets of wavefronts, or (MYEA_LSTM_BACKWARD_SETS=0) in one instruction stream as at other widths
+FORMS = [("backward-split-along-k", "1", "1"), ("backward-split-along-columns", "0", "1")]
+LOOP_CASES = [c + f[1:] for c in CASES for f in FORMS] + [c + ("0", "0") for c in CASES if "512-cells" in c[0]]
+LOOP_IDS = ["%s-%s" % (f[0], c[0]) for c in CASES for f in FORMS] + ["backward-split-along-columns-one-stream-" + c[0] for c in CASES if "512-cells" in c[0]]
+
+
+@pytest.mark.parametrize("name,specs,T,B,Bmax,backward,ksplit,sets", LOOP_CASES, ids=LOOP_IDS)
+def test_resident_loop_matches_one_launch_per_step_and_the_oracle(name, specs, T, B, Bmax, backward, ksplit, sets):
     desc, h, w, masks, X, Y = _setup(specs, T, B, Bmax, seed=21)
     resident = _net(desc, h, w, masks)
     stepwise = _net(desc, h, w, masks)
@@ -99,7 +104,7 @@ def test_resident_loop_matches_one_launch_per_step_and_the_oracle(name, specs, T
     wide = [l for l in layers]   # every LSTM layer of these cases has a resident form
     per_step = sum((2 if l.use_bidirectional else 1) * (T - 1) for l in layers)
     for step in range(2):
-        with environment(MYEA_LSTM_BACKWARD_KSPLIT=ksplit):
+        with environment(MYEA_LSTM_BACKWARD_KSPLIT=ksplit, MYEA_LSTM_BACKWARD_SETS=sets):
             resident.profile_enable(True)
             resident.Reset__Loss()
             run_step(resident, B, X, Y, update=False)
@@ -165,7 +170,8 @@ def test_the_path_of_a_late_group(name, specs, T, B, Bmax):
     if zone_masks is not None:
         cpu.upload_zoneout_masks(zone_masks)
     cpu.Clear_Training_Arrays()
-    with environment(MYEA_LSTM_RESIDENT_TEST_NEVER_EARLY=1, MYEA_LSTM_BACKWARD_KSPLIT=0):   # the backward form that stages tiles
+    # the backward form that stages tiles, with a member's two chains in one instruction stream (the form that has the two paths)
+    with environment(MYEA_LSTM_RESIDENT_TEST_NEVER_EARLY=1, MYEA_LSTM_BACKWARD_KSPLIT=0, MYEA_LSTM_BACKWARD_SETS=0):
         gpu.profile_enable(True)
         for n in (gpu, cpu):
             n.Reset__Loss()
@@ -223,11 +229,12 @@ def test_a_wait_that_gives_up_is_reported_once_and_the_network_carries_on_per_st
     _compare(desc, gpu, cpu, B, T, "after the give-up")
 
 
-@pytest.mark.parametrize("cells,ksplit", [(128, "1"), (128, "0"), (1024, "0")],
-                         ids=["backward-split-along-k", "backward-split-along-columns", "1024-cells-across-two-xcds"])
+@pytest.mark.parametrize("cells,ksplit", [(128, "1"), (128, "0"), (512, "0"), (1024, "0")],
+                         ids=["backward-split-along-k", "backward-split-along-columns", "512-cells-a-set-of-wavefronts-per-chain", "1024-cells-across-two-xcds"])
 def test_a_backward_wait_that_gives_up_is_reported_too(cells, ksplit):
     """the same forced give-up in the backward loop, in each of its forms (at 1024 cells with tile loads into LDS in flight
-    when the wait begins): the forward pass runs normally, the backward loop's first wait between steps runs out of polls and
+    when the wait begins; at 512 cells every wait of the two sets of wavefronts - for the group, for the turn, for each other -
+    runs out on its own): the forward pass runs normally, the backward loop's first wait between steps runs out of polls and
     every wavefront leaves"""
     specs = [dict(units=8), lstm(cells), dict(units=cells, activation="LINEAR")]
     T, B = 5, 32
