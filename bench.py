@@ -28,7 +28,7 @@ if ROOT not in sys.path:
 RECORDED_TRAFFIC = {"fc4096x4_b1024_adam": dict(bytes_per_launch=2951372 * 1024 / 10,
                                                 source="recorded constant, not measured in this run: profiles/hbm_traffic__fc4096x4_b1024_adam__pmc.txt"),
                     # the two resident time loops of one layer (forward + backward launch), mean per launch
-                    "lstm512x2_t64_b256_amsgrad": dict(bytes_per_launch=(2 * 98047.4 + 230411.9 + 2 * 195875.0 + 197752.0) * 1024 / 2,
+                    "lstm512x2_t64_b256_amsgrad": dict(bytes_per_launch=(2 * 98055.1 + 230411.5 + 2 * 203936.9 + 197795.6) * 1024 / 2,
                                                        source="recorded constant, not measured in this run: profiles/lstm_resident__lstm512x2_t64_b256_amsgrad__pmc.txt")}
 from myea_amd.synthetic import simple_debug_layers  # noqa: E402  (no device is touched by the import)
 
