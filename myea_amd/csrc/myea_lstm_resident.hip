@@ -21,8 +21,10 @@
 //     LDS (global -> LDS directly, every wavefront only its own k range); MFMAs against the register-resident weights; the
 //     four partial tiles meet in LDS; gate math of the lane's (example, cell) pair(s); stores.
 //   * On this device the fp32 MFMAs and ordinary vector instructions of a SIMD do not overlap, whichever wavefront they
-//     come from (measured), so a second wavefront per SIMD buys nothing; what can be hidden is latency.  The chain that
-//     is not computing is the one whose stores, barrier and tile loads are in flight:
+//     come from (measured), so a second wavefront per SIMD buys no issue slots; what can be hidden is latency.  (The 512-cell
+//     backward loop does give each chain its own set of four wavefronts - lstm_resident_backward_sets_kernel - because its
+//     tail is mostly latency: described there.)  In one instruction stream the chain that is not computing is the one whose
+//     stores, barrier and tile loads are in flight:
 //       - a unit's arrival at its chain's counter is signalled a quarter into the NEXT unit's MFMAs, when its stores have
 //         long been acknowledged;
 //       - the counter is read three quarters into those MFMAs and is normally complete at their end;
