@@ -27,6 +27,7 @@ CASES = [
     ("128-cells-second-chain-empty", [dict(units=8), lstm(128), dict(units=128, activation="LINEAR")], 5, 13, 16, True),
     ("256-cells-two-directions", [dict(units=12), lstm(256, bidirectional=True), dict(units=256, activation="TANH")], 5, 33, 40, True),
     ("512-cells-zoneout-stacked", [dict(units=16), zone(512), lstm(128), dict(units=128, activation="LINEAR")], 4, 48, 48, True),
+    ("512-cells-two-directions-ragged", [dict(units=9), lstm(512, bidirectional=True), dict(units=512, activation="LINEAR")], 4, 41, 44, True),
     ("1024-cells-two-directions", [dict(units=10), lstm(1024, bidirectional=True), dict(units=1024, activation="LINEAR")], 3, 40, 40, True),
     ("1024-cells-ragged-seven-steps", [dict(units=6), lstm(1024), dict(units=1024, activation="LINEAR")], 7, 45, 48, True),
     ("1024-cells-two-steps", [dict(units=5), lstm(1024), dict(units=1024, activation="LINEAR")], 2, 33, 33, True),
