@@ -968,9 +968,9 @@ __global__ __launch_bounds__(kThreads, 1) void lstm_resident_backward_kernel(Res
 // What made it work (each measured at 512 cells x 256 examples, where the one-stream kernel takes 464 us a pass):
 //   - The tile loops take TURNS, in one fixed order (s_turn).  Left alone the two sets fall into step - both contracting at
 //     half speed, then both in their tails - and stay there: 1005 us.
-//   - Nobody polls a word the whole launch shares, and one wavefront per set polls the group's counter while the other three
-//     watch LDS.  A poll in flight to a busy line holds up everything else its compute unit asks of memory (a tile step of
-//     1000 clocks instead of 380, every load instruction a few hundred clocks to issue): 755 -> 438 us.
+//   - One wavefront per set polls the group's counter while the other three watch LDS.  Polls that queue at a busy line hold
+//     up everything else their compute units ask of memory (a tile step of 1000 clocks instead of 380, every load
+//     instruction a few hundred clocks to issue): 755 -> 438 us (524 -> 418 in the final form).
 //   - A short pause before the first poll (below): 414 us.
 // The four wavefronts of a set meet through a counter in LDS (s_barrier would tie the two chains together); every wait of
 // this kernel is bounded by the same count of polls and ends the wavefront through the give-up path.
@@ -1116,9 +1116,10 @@ __global__ __launch_bounds__(2 * kThreads, 1) void lstm_resident_backward_sets_k
         return __builtin_amdgcn_readfirstlane(ok) != 0;
     };
 
-    // The group's counter has reached `target`: the set's first wavefront asks memory (the counter's line only - a word that
-    // every wavefront of the launch polls is a queue at one L2 channel, and everything else this compute unit asks of memory
-    // waits behind its polls), the other three watch a word in LDS.  Bounded; 0 when the wait gave up here or elsewhere.
+    // The group's counter has reached `target`: the set's first wavefront asks memory, the other three watch a word in LDS.
+    // With all four polling - 128 wavefronts on the line that the group's 32 arrivals are added to - a pass took 524 us instead
+    // of 418: the polls queue at the line, and what else their compute units ask of memory queues behind them (a tile step of
+    // 1000 clocks instead of 380, a few hundred clocks to issue any load).  Bounded; 0 when the wait gave up here or elsewhere.
     auto group_wait = [&](unsigned target) -> bool {
         int ok = 1;
         if (lane == 0) {
@@ -1132,17 +1133,22 @@ __global__ __launch_bounds__(2 * kThreads, 1) void lstm_resident_backward_sets_k
                     "v_sub_u32 %[value], %[value], %[target]\n\t"
                     "v_cmp_le_i32 vcc, 0, %[value]\n\t"
                     "s_cbranch_vccnz 2f\n\t"
+                    "global_load_dword %[value], %[give_up], off sc1\n\t"   // somebody else of the launch gave up
+                    "s_waitcnt vmcnt(0)\n\t"
+                    "v_cmp_ne_u32 vcc, 0, %[value]\n\t"
+                    "s_cbranch_vccnz 4f\n\t"
                     "s_sleep 4\n\t"
                     "s_sub_u32 %[polls], %[polls], 1\n\t"
                     "s_cmp_lg_u32 %[polls], 0\n\t"
-                    "s_cbranch_scc1 1b\n\t"
+                    "s_cbranch_scc1 1b\n"
+                    "4:\n\t"
                     "v_mov_b32 %[ok], 0\n\t"
                     "s_branch 3f\n"
                     "2:\n\t"
                     "ds_write_b32 %[go], %[target]\n"
                     "3:\n"
                     : [ok] "+v"(ok), [value] "=&v"(value), [polls] "+s"(polls)
-                    : [counter] "v"(counter), [target] "v"(target), [go] "v"(go_at)
+                    : [counter] "v"(counter), [target] "v"(target), [go] "v"(go_at), [give_up] "v"(w.give_up)
                     : "vcc", "scc", "memory");
             } else {
                 asm volatile(
